@@ -1,0 +1,139 @@
+/*
+ * libjigsaw_hip — C ABI of the MI355X (gfx950) kernels that sit underneath the
+ * per-rank hot path of RAI-SCC/jigsaw's domain- and sequence-parallel layers.
+ *
+ * Conventions
+ *   - Every pointer is a device pointer owned by the caller unless it is
+ *     documented as a host pointer. The library never allocates, frees or keeps
+ *     a pointer past the call.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream). Calls
+ *     only enqueue work; they never synchronise the device.
+ *   - Return value: JG_OK (0) or a negative jg_status. jg_last_error() returns
+ *     the message of the last failure on the calling host thread.
+ *   - Tensors are dense and row-major ("contiguous" in torch terms) in the
+ *     layout named per function.
+ *   - All functions are re-entrant and may be called from any host thread.
+ *
+ * The reference has no FFI: its boundary is Python callables held on per-layer
+ * config objects. Each entry point cites the reference code it stands in for
+ * (paths relative to the reference checkout).
+ */
+#ifndef JIGSAW_HIP_H
+#define JIGSAW_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { JG_F32 = 0, JG_BF16 = 1, JG_F16 = 2 } jg_dtype;
+
+typedef enum {
+  JG_OK = 0,
+  JG_ERR_BAD_ARG = -1,     /* a shape / pointer / size argument is invalid        */
+  JG_ERR_UNSUPPORTED = -2, /* valid request the kernels do not cover              */
+  JG_ERR_LAUNCH = -3,      /* the HIP runtime refused the launch                  */
+  JG_ERR_WORKSPACE = -4    /* workspace too small (see the *_workspace query)     */
+} jg_status;
+
+/* Message of the most recent failure on this host thread ("" if none). */
+const char* jg_last_error(void);
+/* ABI version, bumped on any signature change. */
+int jg_abi_version(void);
+
+/* ------------------------------------------------------------------------- *
+ * Halo movement (bit-exact copies / fixed-order adds; HBM-bound)
+ *
+ * Geometry of one rank's tile. Spatial axes are (D, H, W); a 2-D tile has
+ * size[0] = 1 and lo[0] = hi[0] = 0. `planes` = batch * channels (the tensors
+ * are channels-first, so each plane is one contiguous (D, H, W) block).
+ * lo / hi are the halo widths in front of / behind the interior on each axis:
+ * for jigsaw's span [lo_g, lo_g + need) of needed_input_span
+ * (jigsaw/modules/convolution/_conv/halo.py:9-63) they are
+ * lo = r*n - lo_g and hi = lo_g + need - (r+1)*n.
+ *
+ * Neighbour tables have 27 slots indexed (dd+1)*9 + (dh+1)*3 + (dw+1) for the
+ * neighbour at offset (dd, dh, dw) in {-1,0,1}^3; slot 13 is this rank. A NULL
+ * slot is a neighbour outside the global domain (its halo is zero on assemble,
+ * contributes nothing on fold, is skipped on pack). The 2-D entry points take
+ * 9 slots indexed (dh+1)*3 + (dw+1), slot 4 = this rank.
+ *
+ * Strip shapes: the strip of neighbour (dd, dh, dw) is dense
+ * (planes, ed, eh, ew) where, per axis and for the three verbs:
+ *                      offset -1      offset 0     offset +1
+ *   assemble (recv)      lo           size          hi     <- fills my halo
+ *   pack_fwd (send)      hi           size          lo     <- their halo of me
+ *   pack_bwd (send)      lo           size          hi     <- my halo's grads
+ *   fold     (recv)      hi           size          lo     <- their halo of me
+ * ------------------------------------------------------------------------- */
+typedef struct {
+  int64_t planes;
+  int32_t size[3];
+  int32_t lo[3];
+  int32_t hi[3];
+} jg_halo_geom;
+
+/* x_aug (planes, D+lo+hi, H+lo+hi, W+lo+hi) <- own tile src[13] + 26 strips.
+ * One pass over the destination: every element is written exactly once (copied
+ * or zero), which replaces new_zeros + narrow().copy_() per split axis in
+ * halo_gather (jigsaw/modules/convolution/_conv/halo.py:66-156) and the
+ * all_to_all staging of exchange_along_axis (_common/halo.py:7-63).
+ * elem_size is 2 or 4 bytes; bytes are moved untouched (-0.0 and NaN payloads
+ * survive). */
+int jg_halo_assemble_3d(void* x_aug, const void* const src[27],
+                        const jg_halo_geom* geom, int elem_size, void* stream);
+int jg_halo_assemble_2d(void* x_aug, const void* const src[9], int64_t planes,
+                        int H, int W, int lo_h, int hi_h, int lo_w, int hi_w,
+                        int elem_size, void* stream);
+
+/* Cut the strips this rank sends. from_padded = 0: `src` is the own tile
+ * (planes, D, H, W) and strip (dd,dh,dw) is the edge block that neighbour needs
+ * for its halo (forward; the x.narrow(axis, col, sn) sends of halo.py:134-147).
+ * from_padded = 1: `src` is a padded tensor (planes, D+.., H+.., W+..) and strip
+ * (dd,dh,dw) is the halo block that neighbour owns (backward; the
+ * g_x_need.narrow sends of halo.py:222-226). NULL slots are skipped. */
+int jg_halo_pack_3d(void* const strips[27], const void* src,
+                    const jg_halo_geom* geom, int from_padded, int elem_size,
+                    void* stream);
+int jg_halo_pack_2d(void* const strips[9], const void* src, int64_t planes,
+                    int H, int W, int lo_h, int hi_h, int lo_w, int hi_w,
+                    int from_padded, int elem_size, void* stream);
+
+/* gx (planes, D, H, W) <- fold of the padded gradient gx_aug and the strips the
+ * neighbours sent back. Restates halo_scatter_add (halo.py:159-251) applied in
+ * reverse axis order W, H, D (distributed.py:378-389) with its exact
+ * association: per axis acc = 0; acc += lower neighbour; acc += own;
+ * acc += upper neighbour, each add rounded to `dtype`; the W fold is innermost.
+ * Needs lo <= size and hi <= size on every axis. */
+int jg_halo_fold_3d(void* gx, const void* gx_aug, const void* const strips[27],
+                    const jg_halo_geom* geom, int dtype, void* stream);
+int jg_halo_fold_2d(void* gx, const void* gx_aug, const void* const strips[9],
+                    int64_t planes, int H, int W, int lo_h, int hi_h, int lo_w,
+                    int hi_w, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------- *
+ * DistributedRoll (pure copies; HBM-bound)
+ * ------------------------------------------------------------------------- */
+
+/* dst = torch.roll(src, shifts, dims) for a dense tensor of `ndim` <= 6 axes
+ * (jigsaw/modules/roll/_distributed_roll.py:99). shifts[i] is the shift of axis
+ * i (0 = not rolled), any sign, taken modulo sizes[i]. dst must not alias src. */
+int jg_roll(void* dst, const void* src, int ndim, const int64_t* sizes,
+            const int64_t* shifts, int elem_size, void* stream);
+
+/* The wrapped slab of exchange_halo_1d (_distributed_roll.py:44-48, 59): with
+ * window > 0 the leading `window` entries of `axis`, else the trailing
+ * |window|. jg_roll_pack copies that slab of x into the dense `strip`
+ * (x[sl].contiguous()); jg_roll_unpack writes a dense strip into that slab of x
+ * in place (x[sl] = recv). */
+int jg_roll_pack(void* strip, const void* x, int ndim, const int64_t* sizes,
+                 int axis, int64_t window, int elem_size, void* stream);
+int jg_roll_unpack(void* x, const void* strip, int ndim, const int64_t* sizes,
+                   int axis, int64_t window, int elem_size, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* JIGSAW_HIP_H */

@@ -1,0 +1,161 @@
+"""ctypes binding of ``libjigsaw_hip.so``.
+
+The library is plain C ABI (pointers, sizes, a ``hipStream_t``); torch is used
+here only to obtain device pointers and the current stream. ``torch`` is imported
+first so that the library binds to the HIP runtime torch already loaded.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import threading
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int32, c_int64, c_size_t, c_void_p
+from pathlib import Path
+
+import torch
+
+_LIB_PATH = Path(__file__).resolve().parent / "lib" / "libjigsaw_hip.so"
+_lock = threading.Lock()
+_lib: ctypes.CDLL | None = None
+
+JG_F32, JG_BF16, JG_F16 = 0, 1, 2
+_DTYPES = {torch.float32: JG_F32, torch.bfloat16: JG_BF16, torch.float16: JG_F16}
+
+
+class LibraryMissing(RuntimeError):
+    """``libjigsaw_hip.so`` is not built; there is no fallback path."""
+
+
+class KernelError(RuntimeError):
+    """A C-ABI call returned a negative status."""
+
+
+class HaloGeom(ctypes.Structure):
+    """``jg_halo_geom`` of ``include/jigsaw_hip.h``."""
+
+    _fields_ = [
+        ("planes", c_int64),
+        ("size", c_int32 * 3),
+        ("lo", c_int32 * 3),
+        ("hi", c_int32 * 3),
+    ]
+
+
+VoidP27 = c_void_p * 27
+VoidP9 = c_void_p * 9
+
+# name -> (restype, argtypes); kept next to include/jigsaw_hip.h by test_abi.py
+SIGNATURES: dict[str, tuple] = {
+    "jg_last_error": (c_char_p, []),
+    "jg_abi_version": (c_int, []),
+    "jg_halo_assemble_3d": (c_int, [c_void_p, POINTER(c_void_p), POINTER(HaloGeom), c_int, c_void_p]),
+    "jg_halo_assemble_2d": (
+        c_int,
+        [c_void_p, POINTER(c_void_p), c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    ),
+    "jg_halo_pack_3d": (c_int, [POINTER(c_void_p), c_void_p, POINTER(HaloGeom), c_int, c_int, c_void_p]),
+    "jg_halo_pack_2d": (
+        c_int,
+        [POINTER(c_void_p), c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    ),
+    "jg_halo_fold_3d": (c_int, [c_void_p, c_void_p, POINTER(c_void_p), POINTER(HaloGeom), c_int, c_void_p]),
+    "jg_halo_fold_2d": (
+        c_int,
+        [c_void_p, c_void_p, POINTER(c_void_p), c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    ),
+    "jg_roll": (c_int, [c_void_p, c_void_p, c_int, POINTER(c_int64), POINTER(c_int64), c_int, c_void_p]),
+    "jg_roll_pack": (c_int, [c_void_p, c_void_p, c_int, POINTER(c_int64), c_int, c_int64, c_int, c_void_p]),
+    "jg_roll_unpack": (c_int, [c_void_p, c_void_p, c_int, POINTER(c_int64), c_int, c_int64, c_int, c_void_p]),
+}
+
+
+def lib_path() -> Path:
+    """Path the built library is expected at."""
+    return _LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    """Load the library once and declare every entry point's signature."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not _LIB_PATH.exists():
+            raise LibraryMissing(
+                f"{_LIB_PATH} is not built. Run `python -m jigsaw_amd.build` "
+                "(needs hipcc); there is no CPU or PyTorch fallback for these operators."
+            )
+        lib = ctypes.CDLL(str(_LIB_PATH))
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def abi_version() -> int:
+    return int(load().jg_abi_version())
+
+
+def check(rc: int, what: str = "") -> None:
+    """Raise on a negative status, with the library's own message."""
+    if rc == 0:
+        return
+    msg = load().jg_last_error().decode("utf-8", "replace")
+    exc = {-1: ValueError, -2: NotImplementedError}.get(rc, KernelError)
+    raise exc(f"{what or 'libjigsaw_hip'}: {msg} (status {rc})")
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise NotImplementedError(f"dtype {dtype} is not supported by the HIP kernels") from None
+
+
+def require_gpu(*tensors: torch.Tensor) -> None:
+    """Operators only run on HIP device tensors; say so instead of falling back."""
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "jigsaw_amd operators run on the GPU only (got a tensor on "
+                f"{t.device}); there is no CPU path in this package."
+            )
+
+
+def ptr(t: torch.Tensor | None) -> c_void_p:
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def stream_ptr(device: torch.device | None = None) -> c_void_p:
+    return c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def i64_array(values) -> ctypes.Array:
+    vals = [int(v) for v in values]
+    return (c_int64 * len(vals))(*vals)
+
+
+__all__ = [
+    "HaloGeom",
+    "KernelError",
+    "LibraryMissing",
+    "SIGNATURES",
+    "VoidP27",
+    "VoidP9",
+    "abi_version",
+    "check",
+    "dtype_code",
+    "i64_array",
+    "lib_path",
+    "load",
+    "ptr",
+    "require_gpu",
+    "stream_ptr",
+    "c_float",
+    "c_double",
+    "c_size_t",
+]

@@ -1,0 +1,579 @@
+// Halo movement for the halo-exchange convolution: assemble (own tile + up to
+// 26 neighbour strips -> zero-padded tile), pack (cut the strips a rank sends)
+// and fold (padded gradient + neighbour strips -> owned gradient, in the
+// reference's association order). All three are destination-driven single
+// passes: every output element is produced exactly once, stores are 16-byte
+// vectors, and the work is pure HBM traffic (no LDS, no MFMA).
+//
+// Reference behaviour restated here:
+//   jigsaw/modules/convolution/_conv/halo.py:66-156   (halo_gather)
+//   jigsaw/modules/convolution/_conv/halo.py:159-251  (halo_scatter_add)
+//   jigsaw/modules/convolution/_conv/distributed.py:264-275, 378-389 (axis order)
+#include "jg_common.h"
+
+namespace {
+
+struct Geom {
+  long long planes;
+  int n[3];   // interior D, H, W
+  int lo[3];  // halo before
+  int hi[3];  // halo after
+};
+
+struct Table {
+  const void* p[27];
+};
+
+struct MutTable {
+  void* p[27];
+};
+
+// 16-byte vector of raw bits.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+template <typename T>
+struct Bits;
+template <>
+struct Bits<uint16_t> {
+  static constexpr int V = 8;
+};
+template <>
+struct Bits<uint32_t> {
+  static constexpr int V = 4;
+};
+
+// Load 16 bytes from an address that is only sizeof(T)-aligned.
+template <typename T>
+__device__ __forceinline__ u32x4 load16_unaligned(const T* s);
+
+template <>
+__device__ __forceinline__ u32x4 load16_unaligned<uint32_t>(const uint32_t* s) {
+  return *reinterpret_cast<const u32x4_a4*>(s);
+}
+
+template <>
+__device__ __forceinline__ u32x4 load16_unaligned<uint16_t>(const uint16_t* s) {
+  uintptr_t a = reinterpret_cast<uintptr_t>(s);
+  if ((a & 3) == 0) return *reinterpret_cast<const u32x4_a4*>(s);
+  // 2-byte phase: read the five dwords that cover the 16 bytes and funnel-shift.
+  const uint32_t* q = reinterpret_cast<const uint32_t*>(a - 2);
+  u32x4_a4 lo4 = *reinterpret_cast<const u32x4_a4*>(q);
+  uint32_t d4 = q[4];
+  u32x4 r;
+  r.x = (lo4.x >> 16) | (lo4.y << 16);
+  r.y = (lo4.y >> 16) | (lo4.z << 16);
+  r.z = (lo4.z >> 16) | (lo4.w << 16);
+  r.w = (lo4.w >> 16) | (d4 << 16);
+  return r;
+}
+
+// Region of a padded coordinate: 0 = lower halo, 1 = interior, 2 = upper halo.
+__device__ __forceinline__ void region(int x, int lo, int n, int hi, int& r, int& c,
+                                       int& ext) {
+  if (x < lo) {
+    r = 0; c = x; ext = lo;
+  } else if (x < lo + n) {
+    r = 1; c = x - lo; ext = n;
+  } else {
+    r = 2; c = x - lo - n; ext = hi;
+  }
+}
+
+// ------------------------------------------------------------------ assemble
+template <typename T>
+__device__ __forceinline__ T assemble_fetch(const Table& tab, const Geom& g, long long p,
+                                            int da, int ha, int wa) {
+  int rd, cd, ed, rh, ch, eh, rw, cw, ew;
+  region(da, g.lo[0], g.n[0], g.hi[0], rd, cd, ed);
+  region(ha, g.lo[1], g.n[1], g.hi[1], rh, ch, eh);
+  region(wa, g.lo[2], g.n[2], g.hi[2], rw, cw, ew);
+  const T* s = static_cast<const T*>(tab.p[rd * 9 + rh * 3 + rw]);
+  if (s == nullptr) return T(0);
+  long long off = ((p * ed + cd) * eh + ch) * (long long)ew + cw;
+  return s[off];
+}
+
+template <typename T, typename I>
+__global__ __launch_bounds__(256) void assemble_kernel(T* __restrict__ dst, Table tab,
+                                                       Geom g, I total) {
+  constexpr int V = Bits<T>::V;
+  const I nvec = (total + V - 1) / V;
+  const int Da = g.lo[0] + g.n[0] + g.hi[0];
+  const int Ha = g.lo[1] + g.n[1] + g.hi[1];
+  const int Wa = g.lo[2] + g.n[2] + g.hi[2];
+  for (I v = (I)blockIdx.x * 256 + threadIdx.x; v < nvec; v += (I)gridDim.x * 256) {
+    const I e0 = v * V;
+    I row = e0 / (I)Wa;
+    int wa = (int)(e0 - row * (I)Wa);
+    I t = row / (I)Ha;
+    int ha = (int)(row - t * (I)Ha);
+    I pp = t / (I)Da;
+    int da = (int)(t - pp * (I)Da);
+    long long p = (long long)pp;
+
+    bool fast = (wa + V <= Wa) && (e0 + V <= total);
+    int rw = 0, cw = 0, ew = 0;
+    if (fast) {
+      int rw2, cw2, ew2;
+      region(wa, g.lo[2], g.n[2], g.hi[2], rw, cw, ew);
+      region(wa + V - 1, g.lo[2], g.n[2], g.hi[2], rw2, cw2, ew2);
+      fast = (rw == rw2);
+    }
+    if (fast) {
+      int rd, cd, ed, rh, ch, eh;
+      region(da, g.lo[0], g.n[0], g.hi[0], rd, cd, ed);
+      region(ha, g.lo[1], g.n[1], g.hi[1], rh, ch, eh);
+      const T* s = static_cast<const T*>(tab.p[rd * 9 + rh * 3 + rw]);
+      u32x4 val = {0u, 0u, 0u, 0u};
+      if (s != nullptr) {
+        long long off = ((p * ed + cd) * eh + ch) * (long long)ew + cw;
+        val = load16_unaligned<T>(s + off);
+      }
+      *reinterpret_cast<u32x4*>(dst + e0) = val;
+    } else {
+      T tmp[V];
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        tmp[i] = T(0);
+        if (e0 + i < total) tmp[i] = assemble_fetch<T>(tab, g, p, da, ha, wa);
+        if (++wa == Wa) {
+          wa = 0;
+          if (++ha == Ha) {
+            ha = 0;
+            if (++da == Da) {
+              da = 0;
+              ++p;
+            }
+          }
+        }
+      }
+      if (e0 + V <= total) {
+        u32x4 val;
+        __builtin_memcpy(&val, tmp, 16);
+        *reinterpret_cast<u32x4*>(dst + e0) = val;
+      } else {
+        for (int i = 0; i < V && e0 + i < total; ++i) dst[e0 + i] = tmp[i];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------- pack
+struct Box {
+  int org[3];  // origin in the source, per axis
+  int ext[3];  // extent, per axis
+};
+struct PackArgs {
+  void* dst[27];
+  Box box[27];
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void pack_kernel(PackArgs a, const T* __restrict__ src,
+                                                   long long planes, int Sd, int Sh,
+                                                   int Sw) {
+  const int slot = blockIdx.y;
+  T* d = static_cast<T*>(a.dst[slot]);
+  if (d == nullptr) return;
+  const Box b = a.box[slot];
+  const long long per_plane = (long long)b.ext[0] * b.ext[1] * b.ext[2];
+  const long long total = planes * per_plane;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total;
+       i += (long long)gridDim.x * 256) {
+    long long r = i / b.ext[2];
+    int cw = (int)(i - r * b.ext[2]);
+    long long r2 = r / b.ext[1];
+    int ch = (int)(r - r2 * b.ext[1]);
+    long long p = r2 / b.ext[0];
+    int cd = (int)(r2 - p * b.ext[0]);
+    long long so = ((p * Sd + (b.org[0] + cd)) * Sh + (b.org[1] + ch)) * (long long)Sw +
+                   (b.org[2] + cw);
+    d[i] = src[so];
+  }
+}
+
+// ---------------------------------------------------------------------- fold
+// Arithmetic of one `acc += v` in the tensor dtype (what Tensor.add_ does).
+template <int DT>
+struct Arith;
+template <>
+struct Arith<JG_F32> {
+  typedef uint32_t T;
+  __device__ static __forceinline__ float up(uint32_t b) { return __uint_as_float(b); }
+  __device__ static __forceinline__ uint32_t down(float f) { return __float_as_uint(f); }
+};
+template <>
+struct Arith<JG_BF16> {
+  typedef uint16_t T;
+  __device__ static __forceinline__ float up(uint16_t b) { return jg::bf16_to_f32(b); }
+  __device__ static __forceinline__ uint16_t down(float f) { return jg::f32_to_bf16(f); }
+};
+template <>
+struct Arith<JG_F16> {
+  typedef uint16_t T;
+  __device__ static __forceinline__ float up(uint16_t b) {
+    _Float16 h;
+    __builtin_memcpy(&h, &b, 2);
+    return (float)h;
+  }
+  __device__ static __forceinline__ uint16_t down(float f) {
+    _Float16 h = (_Float16)f;
+    uint16_t b;
+    __builtin_memcpy(&b, &h, 2);
+    return b;
+  }
+};
+
+// Which neighbour offsets reach interior coordinate x of an axis, and where in
+// that neighbour's strip. o = -1: the lower neighbour's upper halo covers
+// [0, hi); o = +1: the upper neighbour's lower halo covers [n - lo, n).
+__device__ __forceinline__ bool reach(int o, int x, int lo, int n, int hi, int& c,
+                                      int& ext) {
+  if (o < 0) {
+    c = x; ext = hi;
+    return x < hi;
+  }
+  if (o == 0) {
+    c = x; ext = n;
+    return true;
+  }
+  c = x - (n - lo); ext = lo;
+  return x >= n - lo;
+}
+
+template <int DT>
+__device__ __forceinline__ typename Arith<DT>::T fold_one(
+    const typename Arith<DT>::T* __restrict__ own, const Table& tab, const Geom& g,
+    long long p, int d, int h, int w) {
+  typedef typename Arith<DT>::T T;
+  const int Ha = g.lo[1] + g.n[1] + g.hi[1];
+  const int Wa = g.lo[2] + g.n[2] + g.hi[2];
+  const int Da = g.lo[0] + g.n[0] + g.hi[0];
+  float acc_d = 0.0f;
+  for (int od = -1; od <= 1; ++od) {
+    int cd, ed;
+    if (!reach(od, d, g.lo[0], g.n[0], g.hi[0], cd, ed)) continue;
+    float acc_h = 0.0f;
+    for (int oh = -1; oh <= 1; ++oh) {
+      int ch, eh;
+      if (!reach(oh, h, g.lo[1], g.n[1], g.hi[1], ch, eh)) continue;
+      float acc_w = 0.0f;
+      for (int ow = -1; ow <= 1; ++ow) {
+        int cw, ew;
+        if (!reach(ow, w, g.lo[2], g.n[2], g.hi[2], cw, ew)) continue;
+        T bits;
+        if (od == 0 && oh == 0 && ow == 0) {
+          long long off = ((p * Da + (d + g.lo[0])) * Ha + (h + g.lo[1])) * (long long)Wa +
+                          (w + g.lo[2]);
+          bits = own[off];
+        } else {
+          const T* s = static_cast<const T*>(tab.p[(od + 1) * 9 + (oh + 1) * 3 + (ow + 1)]);
+          if (s == nullptr) continue;
+          long long off = ((p * ed + cd) * eh + ch) * (long long)ew + cw;
+          bits = s[off];
+        }
+        acc_w = Arith<DT>::up(Arith<DT>::down(acc_w + Arith<DT>::up(bits)));
+      }
+      acc_h = Arith<DT>::up(Arith<DT>::down(acc_h + acc_w));
+    }
+    acc_d = Arith<DT>::up(Arith<DT>::down(acc_d + acc_h));
+  }
+  return Arith<DT>::down(acc_d);
+}
+
+template <int DT, typename I>
+__global__ __launch_bounds__(256) void fold_kernel(typename Arith<DT>::T* __restrict__ dst,
+                                                   const typename Arith<DT>::T* __restrict__ own,
+                                                   Table tab, Geom g, I total) {
+  typedef typename Arith<DT>::T T;
+  constexpr int V = Bits<T>::V;
+  constexpr T ABS = (T)(~(T(1) << (sizeof(T) * 8 - 1)));
+  const I nvec = (total + V - 1) / V;
+  const int D = g.n[0], H = g.n[1], W = g.n[2];
+  const int Ha = g.lo[1] + H + g.hi[1];
+  const int Wa = g.lo[2] + W + g.hi[2];
+  const int Da = g.lo[0] + D + g.hi[0];
+  for (I v = (I)blockIdx.x * 256 + threadIdx.x; v < nvec; v += (I)gridDim.x * 256) {
+    const I e0 = v * V;
+    I row = e0 / (I)W;
+    int w = (int)(e0 - row * (I)W);
+    I t = row / (I)H;
+    int h = (int)(row - t * (I)H);
+    I pp = t / (I)D;
+    int d = (int)(t - pp * (I)D);
+    long long p = (long long)pp;
+
+    // Interior of the tile: nothing but `0 + own`, which only clears the sign
+    // of a zero.
+    bool fast = (e0 + V <= total) && (w >= g.hi[2]) && (w + V <= W - g.lo[2]) &&
+                (h >= g.hi[1]) && (h < H - g.lo[1]) && (d >= g.hi[0]) && (d < D - g.lo[0]);
+    if (fast) {
+      long long off = ((p * Da + (d + g.lo[0])) * Ha + (h + g.lo[1])) * (long long)Wa +
+                      (w + g.lo[2]);
+      u32x4 val = load16_unaligned<T>(own + off);
+      T tmp[V];
+      __builtin_memcpy(tmp, &val, 16);
+#pragma unroll
+      for (int i = 0; i < V; ++i)
+        if ((tmp[i] & ABS) == 0) tmp[i] = 0;
+      __builtin_memcpy(&val, tmp, 16);
+      *reinterpret_cast<u32x4*>(dst + e0) = val;
+    } else {
+      T tmp[V];
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        tmp[i] = T(0);
+        if (e0 + i < total) tmp[i] = fold_one<DT>(own, tab, g, p, d, h, w);
+        if (++w == W) {
+          w = 0;
+          if (++h == H) {
+            h = 0;
+            if (++d == D) {
+              d = 0;
+              ++p;
+            }
+          }
+        }
+      }
+      if (e0 + V <= total) {
+        u32x4 val;
+        __builtin_memcpy(&val, tmp, 16);
+        *reinterpret_cast<u32x4*>(dst + e0) = val;
+      } else {
+        for (int i = 0; i < V && e0 + i < total; ++i) dst[e0 + i] = tmp[i];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- host side
+int check_geom(const jg_halo_geom* g, const char* who, bool adjacent_only) {
+  JG_REQUIRE(g != nullptr, "%s: geom is NULL", who);
+  JG_REQUIRE(g->planes >= 0, "%s: planes < 0", who);
+  for (int a = 0; a < 3; ++a) {
+    JG_REQUIRE(g->size[a] >= 1, "%s: size[%d] = %d must be >= 1", who, a, g->size[a]);
+    JG_REQUIRE(g->lo[a] >= 0 && g->hi[a] >= 0, "%s: negative halo on axis %d", who, a);
+    if (adjacent_only)
+      JG_REQUIRE(g->lo[a] <= g->size[a] && g->hi[a] <= g->size[a],
+                 "%s: halo (%d, %d) wider than the tile (%d) on axis %d: strips would "
+                 "come from non-adjacent ranks",
+                 who, g->lo[a], g->hi[a], g->size[a], a);
+  }
+  return JG_OK;
+}
+
+Geom to_geom(const jg_halo_geom* g) {
+  Geom r;
+  r.planes = g->planes;
+  for (int a = 0; a < 3; ++a) {
+    r.n[a] = g->size[a];
+    r.lo[a] = g->lo[a];
+    r.hi[a] = g->hi[a];
+  }
+  return r;
+}
+
+int grid_for(unsigned long long nvec) {
+  unsigned long long blocks = (nvec + 255) / 256;
+  // Enough to cover the chip many times over; the kernels grid-stride beyond it.
+  const unsigned long long cap = 1u << 20;
+  if (blocks > cap) blocks = cap;
+  if (blocks == 0) blocks = 1;
+  return (int)blocks;
+}
+
+void expand9(const void* const in[9], const void* out[27]) {
+  for (int i = 0; i < 27; ++i) out[i] = nullptr;
+  for (int i = 0; i < 9; ++i) out[9 + i] = in[i];
+}
+
+jg_halo_geom geom2d(int64_t planes, int H, int W, int lo_h, int hi_h, int lo_w, int hi_w) {
+  jg_halo_geom g;
+  g.planes = planes;
+  g.size[0] = 1; g.size[1] = H; g.size[2] = W;
+  g.lo[0] = 0; g.lo[1] = lo_h; g.lo[2] = lo_w;
+  g.hi[0] = 0; g.hi[1] = hi_h; g.hi[2] = hi_w;
+  return g;
+}
+
+}  // namespace
+
+extern "C" int jg_halo_assemble_3d(void* x_aug, const void* const src[27],
+                                   const jg_halo_geom* geom, int elem_size, void* stream) {
+  int rc = check_geom(geom, "jg_halo_assemble_3d", true);
+  if (rc) return rc;
+  JG_REQUIRE(x_aug != nullptr && src != nullptr, "jg_halo_assemble_3d: NULL pointer");
+  JG_REQUIRE(src[13] != nullptr, "jg_halo_assemble_3d: slot 13 (own tile) is NULL");
+  JG_REQUIRE(elem_size == 2 || elem_size == 4,
+             "jg_halo_assemble_3d: elem_size %d not in {2, 4}", elem_size);
+  JG_REQUIRE((reinterpret_cast<uintptr_t>(x_aug) & 15) == 0,
+             "jg_halo_assemble_3d: x_aug must be 16-byte aligned");
+  Table tab;
+  for (int i = 0; i < 27; ++i) {
+    tab.p[i] = src[i];
+    JG_REQUIRE((reinterpret_cast<uintptr_t>(src[i]) & (elem_size - 1)) == 0,
+               "jg_halo_assemble_3d: slot %d is not element aligned", i);
+  }
+  Geom g = to_geom(geom);
+  unsigned long long total = (unsigned long long)g.planes;
+  for (int a = 0; a < 3; ++a) total *= (unsigned long long)(g.lo[a] + g.n[a] + g.hi[a]);
+  if (total == 0) return JG_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool wide = total >= (1ull << 31);
+  if (elem_size == 2) {
+    int grid = grid_for((total + 7) / 8);
+    if (wide)
+      assemble_kernel<uint16_t, unsigned long long><<<grid, 256, 0, s>>>(
+          static_cast<uint16_t*>(x_aug), tab, g, total);
+    else
+      assemble_kernel<uint16_t, uint32_t><<<grid, 256, 0, s>>>(
+          static_cast<uint16_t*>(x_aug), tab, g, (uint32_t)total);
+  } else {
+    int grid = grid_for((total + 3) / 4);
+    if (wide)
+      assemble_kernel<uint32_t, unsigned long long><<<grid, 256, 0, s>>>(
+          static_cast<uint32_t*>(x_aug), tab, g, total);
+    else
+      assemble_kernel<uint32_t, uint32_t><<<grid, 256, 0, s>>>(
+          static_cast<uint32_t*>(x_aug), tab, g, (uint32_t)total);
+  }
+  JG_CHECK_LAUNCH("jg_halo_assemble_3d");
+  return JG_OK;
+}
+
+extern "C" int jg_halo_assemble_2d(void* x_aug, const void* const src[9], int64_t planes,
+                                   int H, int W, int lo_h, int hi_h, int lo_w, int hi_w,
+                                   int elem_size, void* stream) {
+  JG_REQUIRE(src != nullptr, "jg_halo_assemble_2d: src is NULL");
+  const void* t[27];
+  expand9(src, t);
+  jg_halo_geom g = geom2d(planes, H, W, lo_h, hi_h, lo_w, hi_w);
+  return jg_halo_assemble_3d(x_aug, t, &g, elem_size, stream);
+}
+
+extern "C" int jg_halo_pack_3d(void* const strips[27], const void* src,
+                               const jg_halo_geom* geom, int from_padded, int elem_size,
+                               void* stream) {
+  int rc = check_geom(geom, "jg_halo_pack_3d", true);
+  if (rc) return rc;
+  JG_REQUIRE(strips != nullptr && src != nullptr, "jg_halo_pack_3d: NULL pointer");
+  JG_REQUIRE(elem_size == 2 || elem_size == 4, "jg_halo_pack_3d: elem_size %d not in {2, 4}",
+             elem_size);
+  Geom g = to_geom(geom);
+  PackArgs a;
+  long long biggest = 0;
+  for (int od = -1; od <= 1; ++od)
+    for (int oh = -1; oh <= 1; ++oh)
+      for (int ow = -1; ow <= 1; ++ow) {
+        const int slot = (od + 1) * 9 + (oh + 1) * 3 + (ow + 1);
+        const int o[3] = {od, oh, ow};
+        a.dst[slot] = (slot == 13) ? nullptr : strips[slot];
+        for (int ax = 0; ax < 3; ++ax) {
+          int org, ext;
+          if (!from_padded) {
+            // forward: the block of my tile that lies in that neighbour's halo
+            if (o[ax] < 0) { org = 0; ext = g.hi[ax]; }
+            else if (o[ax] == 0) { org = 0; ext = g.n[ax]; }
+            else { org = g.n[ax] - g.lo[ax]; ext = g.lo[ax]; }
+          } else {
+            // backward: the block of my padded gradient that neighbour owns
+            if (o[ax] < 0) { org = 0; ext = g.lo[ax]; }
+            else if (o[ax] == 0) { org = g.lo[ax]; ext = g.n[ax]; }
+            else { org = g.lo[ax] + g.n[ax]; ext = g.hi[ax]; }
+          }
+          a.box[slot].org[ax] = org;
+          a.box[slot].ext[ax] = ext;
+        }
+        long long cnt = g.planes * (long long)a.box[slot].ext[0] * a.box[slot].ext[1] *
+                        a.box[slot].ext[2];
+        if (cnt == 0) a.dst[slot] = nullptr;
+        if (a.dst[slot] != nullptr && cnt > biggest) biggest = cnt;
+      }
+  if (biggest == 0) return JG_OK;
+  int Sd = g.n[0], Sh = g.n[1], Sw = g.n[2];
+  if (from_padded) {
+    Sd += g.lo[0] + g.hi[0];
+    Sh += g.lo[1] + g.hi[1];
+    Sw += g.lo[2] + g.hi[2];
+  }
+  long long bx = (biggest + 255) / 256;
+  if (bx > 4096) bx = 4096;
+  dim3 grid((unsigned)bx, 27, 1);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (elem_size == 2)
+    pack_kernel<uint16_t><<<grid, 256, 0, s>>>(a, static_cast<const uint16_t*>(src), g.planes,
+                                               Sd, Sh, Sw);
+  else
+    pack_kernel<uint32_t><<<grid, 256, 0, s>>>(a, static_cast<const uint32_t*>(src), g.planes,
+                                               Sd, Sh, Sw);
+  JG_CHECK_LAUNCH("jg_halo_pack_3d");
+  return JG_OK;
+}
+
+extern "C" int jg_halo_pack_2d(void* const strips[9], const void* src, int64_t planes, int H,
+                               int W, int lo_h, int hi_h, int lo_w, int hi_w, int from_padded,
+                               int elem_size, void* stream) {
+  JG_REQUIRE(strips != nullptr, "jg_halo_pack_2d: strips is NULL");
+  void* t[27];
+  for (int i = 0; i < 27; ++i) t[i] = nullptr;
+  for (int i = 0; i < 9; ++i) t[9 + i] = strips[i];
+  jg_halo_geom g = geom2d(planes, H, W, lo_h, hi_h, lo_w, hi_w);
+  return jg_halo_pack_3d(t, src, &g, from_padded, elem_size, stream);
+}
+
+extern "C" int jg_halo_fold_3d(void* gx, const void* gx_aug, const void* const strips[27],
+                               const jg_halo_geom* geom, int dtype, void* stream) {
+  int rc = check_geom(geom, "jg_halo_fold_3d", true);
+  if (rc) return rc;
+  JG_REQUIRE(gx != nullptr && gx_aug != nullptr && strips != nullptr,
+             "jg_halo_fold_3d: NULL pointer");
+  JG_REQUIRE(dtype == JG_F32 || dtype == JG_BF16 || dtype == JG_F16,
+             "jg_halo_fold_3d: unknown dtype %d", dtype);
+  JG_REQUIRE((reinterpret_cast<uintptr_t>(gx) & 15) == 0,
+             "jg_halo_fold_3d: gx must be 16-byte aligned");
+  const int es = (int)jg::dtype_size(dtype);
+  Table tab;
+  for (int i = 0; i < 27; ++i) {
+    tab.p[i] = (i == 13) ? nullptr : strips[i];
+    JG_REQUIRE((reinterpret_cast<uintptr_t>(tab.p[i]) & (es - 1)) == 0,
+               "jg_halo_fold_3d: slot %d is not element aligned", i);
+  }
+  JG_REQUIRE((reinterpret_cast<uintptr_t>(gx_aug) & (es - 1)) == 0,
+             "jg_halo_fold_3d: gx_aug is not element aligned");
+  Geom g = to_geom(geom);
+  unsigned long long total = (unsigned long long)g.planes * g.n[0] * g.n[1] * g.n[2];
+  unsigned long long total_aug = (unsigned long long)g.planes;
+  for (int a = 0; a < 3; ++a) total_aug *= (unsigned long long)(g.lo[a] + g.n[a] + g.hi[a]);
+  if (total == 0) return JG_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool wide = total_aug >= (1ull << 31);
+  const int V = 16 / es;
+  int grid = grid_for((total + V - 1) / V);
+#define JG_FOLD(DT)                                                                         \
+  do {                                                                                      \
+    typedef Arith<DT>::T T;                                                                 \
+    if (wide)                                                                               \
+      fold_kernel<DT, unsigned long long><<<grid, 256, 0, s>>>(                             \
+          static_cast<T*>(gx), static_cast<const T*>(gx_aug), tab, g, total);               \
+    else                                                                                    \
+      fold_kernel<DT, uint32_t><<<grid, 256, 0, s>>>(                                       \
+          static_cast<T*>(gx), static_cast<const T*>(gx_aug), tab, g, (uint32_t)total);     \
+  } while (0)
+  if (dtype == JG_F32) JG_FOLD(JG_F32);
+  else if (dtype == JG_BF16) JG_FOLD(JG_BF16);
+  else JG_FOLD(JG_F16);
+#undef JG_FOLD
+  JG_CHECK_LAUNCH("jg_halo_fold_3d");
+  return JG_OK;
+}
+
+extern "C" int jg_halo_fold_2d(void* gx, const void* gx_aug, const void* const strips[9],
+                               int64_t planes, int H, int W, int lo_h, int hi_h, int lo_w,
+                               int hi_w, int dtype, void* stream) {
+  JG_REQUIRE(strips != nullptr, "jg_halo_fold_2d: strips is NULL");
+  const void* t[27];
+  expand9(strips, t);
+  jg_halo_geom g = geom2d(planes, H, W, lo_h, hi_h, lo_w, hi_w);
+  return jg_halo_fold_3d(gx, gx_aug, t, &g, dtype, stream);
+}

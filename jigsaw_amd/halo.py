@@ -1,0 +1,305 @@
+"""Halo pack / assemble / fold of the halo-exchange convolution on the GPU.
+
+Host-side mirror of jigsaw/modules/convolution/_conv/halo.py. The reference
+pads one split axis at a time through an uneven all-to-all (``halo_gather``,
+halo.py:66-156) and folds gradients back the same way (``halo_scatter_add``,
+halo.py:159-251). Here the exchange is expressed once for all axes: a rank cuts
+up to 8 (2-D) / 26 (3-D) strips for its neighbours (``halo_pack``), and builds
+its padded tile from its own tile plus the strips it received in one pass
+(``halo_assemble``); the backward direction cuts the halo blocks of the padded
+gradient and folds the received ones in the reference's association order
+(``halo_fold``). What travels between ranks is outside this module.
+"""
+
+from __future__ import annotations
+
+import itertools
+from dataclasses import dataclass
+from typing import Mapping, Sequence
+
+import torch
+
+from . import _lib
+from ._lib import HaloGeom, VoidP27
+
+Offset = tuple  # one entry in {-1, 0, 1} per spatial axis
+
+
+def needed_input_span(
+    rank: int,
+    group_size: int,
+    local_in_size: int,
+    kernel: int,
+    stride: int,
+    padding: int,
+    dilation: int,
+) -> tuple[int, int, int, int]:
+    """Return ``(lo, hi, need_size, out_local)`` of a rank's output block.
+
+    Same contract as ``needed_input_span`` of
+    jigsaw/modules/convolution/_conv/halo.py:9-63, including the
+    ``NotImplementedError`` when the global output size does not divide by the
+    group size.
+    """
+    extent = dilation * (kernel - 1) + 1
+    global_out = (group_size * local_in_size + 2 * padding - extent) // stride + 1
+    if global_out % group_size != 0:
+        raise NotImplementedError(
+            "Distributed convolution with a halo exchange needs the global "
+            f"output size along the split axis ({global_out}) to be divisible by "
+            f"the spatial group size ({group_size})."
+        )
+    out_local = global_out // group_size
+    lo = rank * out_local * stride - padding
+    need_size = (out_local - 1) * stride + extent
+    return lo, lo + need_size, need_size, out_local
+
+
+def halo_widths(
+    rank: int, group_size: int, local_in_size: int, kernel: int, stride: int, padding: int, dilation: int
+) -> tuple[int, int, int]:
+    """``(lo_width, hi_width, out_local)`` of the need span around the owned rows.
+
+    Only the regime all fused kernels handle is accepted: the span starts at most
+    one tile before and ends at most one tile after the owned rows, it covers the
+    owned rows completely, and its offset is the same on every rank (so every
+    strip comes from an adjacent rank). Anything else raises
+    ``NotImplementedError``.
+    """
+    n = local_in_size
+    lo, hi, _, out_local = needed_input_span(rank, group_size, n, kernel, stride, padding, dilation)
+    lo_w = rank * n - lo
+    hi_w = hi - (rank + 1) * n
+    if out_local * stride != n:
+        raise NotImplementedError(
+            f"need span drifts across ranks (out_local*stride = {out_local * stride} != local size {n}); "
+            "strips would come from non-adjacent ranks"
+        )
+    if lo_w < 0 or hi_w < 0:
+        raise NotImplementedError(
+            f"need span ({lo}, {hi}) does not cover the owned rows [{rank * n}, {(rank + 1) * n})"
+        )
+    if lo_w > n or hi_w > n:
+        raise NotImplementedError(f"halo ({lo_w}, {hi_w}) wider than the tile ({n})")
+    return lo_w, hi_w, out_local
+
+
+def slot(offset: Sequence[int]) -> int:
+    """Index of a neighbour offset in the 27-entry table of the C ABI."""
+    o = (0,) * (3 - len(offset)) + tuple(int(v) for v in offset)
+    if len(o) != 3 or any(v not in (-1, 0, 1) for v in o):
+        raise ValueError(f"bad neighbour offset {tuple(offset)}")
+    return (o[0] + 1) * 9 + (o[1] + 1) * 3 + (o[2] + 1)
+
+
+@dataclass(frozen=True)
+class HaloGeometry:
+    """Tile size and halo widths of one rank (1 to 3 spatial axes)."""
+
+    size: tuple  # interior extent per spatial axis
+    lo: tuple  # halo in front of the interior
+    hi: tuple  # halo behind the interior
+
+    def __post_init__(self) -> None:
+        ns = len(self.size)
+        if not 1 <= ns <= 3 or len(self.lo) != ns or len(self.hi) != ns:
+            raise ValueError("HaloGeometry needs 1 to 3 spatial axes with matching lo / hi")
+
+    @property
+    def n_spatial(self) -> int:
+        return len(self.size)
+
+    @property
+    def padded(self) -> tuple:
+        return tuple(l + n + h for l, n, h in zip(self.lo, self.size, self.hi))
+
+    def offsets(self) -> list:
+        """All neighbour offsets except the rank itself."""
+        return [o for o in itertools.product((-1, 0, 1), repeat=self.n_spatial) if any(o)]
+
+    def strip_extent(self, offset: Sequence[int], verb: str) -> tuple:
+        """Spatial extent of the strip of ``offset`` for ``verb``.
+
+        ``assemble`` / ``pack_bwd``: (lo, size, hi) for offset (-1, 0, +1);
+        ``fold`` / ``pack_fwd``: (hi, size, lo).
+        """
+        if verb in ("assemble", "pack_bwd"):
+            pick = lambda a, o: (self.lo[a], self.size[a], self.hi[a])[o + 1]  # noqa: E731
+        elif verb in ("fold", "pack_fwd"):
+            pick = lambda a, o: (self.hi[a], self.size[a], self.lo[a])[o + 1]  # noqa: E731
+        else:
+            raise ValueError(f"unknown verb {verb!r}")
+        return tuple(pick(a, o) for a, o in enumerate(offset))
+
+    def c_geom(self, planes: int) -> HaloGeom:
+        pad = 3 - self.n_spatial
+        g = HaloGeom()
+        g.planes = planes
+        for a in range(3):
+            if a < pad:
+                g.size[a], g.lo[a], g.hi[a] = 1, 0, 0
+            else:
+                g.size[a], g.lo[a], g.hi[a] = self.size[a - pad], self.lo[a - pad], self.hi[a - pad]
+        return g
+
+    @classmethod
+    def for_conv(
+        cls,
+        local_in_spatial: Sequence[int],
+        kernel: Sequence[int],
+        stride: Sequence[int],
+        padding: Sequence[int],
+        dilation: Sequence[int],
+        ranks: Sequence[int],
+        group_sizes: Sequence[int],
+    ) -> "HaloGeometry":
+        """Geometry of a rank's need span; axes with a group of one are not padded
+        (the local conv pads them itself, spatial_split.py:75-82)."""
+        lo, hi = [], []
+        for a, n in enumerate(local_in_spatial):
+            if group_sizes[a] <= 1:
+                lo.append(0)
+                hi.append(0)
+                continue
+            l, h, _ = halo_widths(ranks[a], group_sizes[a], n, kernel[a], stride[a], padding[a], dilation[a])
+            lo.append(l)
+            hi.append(h)
+        return cls(tuple(int(n) for n in local_in_spatial), tuple(lo), tuple(hi))
+
+
+def _check_tile(x: torch.Tensor, spatial: tuple, what: str) -> int:
+    ns = len(spatial)
+    if x.dim() < ns + 1:
+        raise ValueError(f"{what}: expected (..., C, {', '.join('S' * ns)}) but got shape {tuple(x.shape)}")
+    if tuple(x.shape[-ns:]) != tuple(spatial):
+        raise ValueError(f"{what}: spatial shape {tuple(x.shape[-ns:])} != expected {tuple(spatial)}")
+    if not x.is_contiguous():
+        raise ValueError(f"{what}: tensor must be contiguous")
+    planes = 1
+    for s in x.shape[:-ns]:
+        planes *= int(s)
+    return planes
+
+
+def _table(
+    strips: Mapping[Offset, torch.Tensor | None],
+    geom: HaloGeometry,
+    verb: str,
+    lead: tuple,
+    like: torch.Tensor,
+    own: torch.Tensor | None,
+) -> VoidP27:
+    tab = VoidP27()
+    for o in geom.offsets():
+        t = strips.get(o)
+        if t is None:
+            continue
+        want = lead + geom.strip_extent(o, verb)
+        if tuple(t.shape) != want:
+            raise ValueError(f"strip {o}: shape {tuple(t.shape)} != expected {want}")
+        if t.dtype != like.dtype or t.device != like.device or not t.is_contiguous():
+            raise ValueError(f"strip {o}: must be contiguous, {like.dtype}, on {like.device}")
+        if t.numel():
+            tab[slot(o)] = t.data_ptr()
+    if own is not None:
+        tab[13] = own.data_ptr()
+    return tab
+
+
+def halo_assemble(
+    x: torch.Tensor,
+    strips: Mapping[Offset, torch.Tensor | None],
+    geom: HaloGeometry,
+    out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Padded tile from the own tile and the strips received from the neighbours.
+
+    A missing / ``None`` strip is a neighbour outside the domain and reads as
+    zero (halo.py:77). Bit-exact copy, one pass over the destination.
+    """
+    _lib.require_gpu(x)
+    planes = _check_tile(x, geom.size, "halo_assemble")
+    lead = tuple(x.shape[: -geom.n_spatial])
+    if out is None:
+        out = torch.empty(lead + geom.padded, dtype=x.dtype, device=x.device)
+    elif tuple(out.shape) != lead + geom.padded or out.dtype != x.dtype or not out.is_contiguous():
+        raise ValueError("halo_assemble: `out` has the wrong shape / dtype / layout")
+    tab = _table(strips, geom, "assemble", lead, x, x)
+    cg = geom.c_geom(planes)
+    rc = _lib.load().jg_halo_assemble_3d(_lib.ptr(out), tab, cg, x.element_size(), _lib.stream_ptr(x.device))
+    _lib.check(rc, "jg_halo_assemble_3d")
+    return out
+
+
+def halo_pack(
+    src: torch.Tensor,
+    geom: HaloGeometry,
+    *,
+    from_padded: bool,
+    present: Sequence[Offset] | None = None,
+) -> dict:
+    """Cut the strips this rank sends, keyed by the neighbour's offset.
+
+    ``from_padded=False``: ``src`` is the own tile, strips are the edge blocks the
+    neighbours need for their halos (forward). ``from_padded=True``: ``src`` is a
+    padded tensor (the dgrad of the padded tile) and strips are its halo blocks,
+    owned by the neighbours (backward). ``present`` limits the offsets to the
+    neighbours that exist.
+    """
+    _lib.require_gpu(src)
+    spatial = geom.padded if from_padded else geom.size
+    planes = _check_tile(src, spatial, "halo_pack")
+    lead = tuple(src.shape[: -geom.n_spatial])
+    verb = "pack_bwd" if from_padded else "pack_fwd"
+    offs = geom.offsets() if present is None else [tuple(o) for o in present]
+    out: dict = {}
+    tab = VoidP27()
+    for o in offs:
+        t = torch.empty(lead + geom.strip_extent(o, verb), dtype=src.dtype, device=src.device)
+        out[o] = t
+        if t.numel():
+            tab[slot(o)] = t.data_ptr()
+    cg = geom.c_geom(planes)
+    rc = _lib.load().jg_halo_pack_3d(
+        tab, _lib.ptr(src), cg, int(from_padded), src.element_size(), _lib.stream_ptr(src.device)
+    )
+    _lib.check(rc, "jg_halo_pack_3d")
+    return out
+
+
+def halo_fold(
+    gx_aug: torch.Tensor,
+    strips: Mapping[Offset, torch.Tensor | None],
+    geom: HaloGeometry,
+    out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Owned gradient from the padded gradient and the neighbours' halo blocks.
+
+    Same result, bit for bit, as ``halo_scatter_add`` (halo.py:159-251) applied
+    per split axis in reverse order (distributed.py:378-389).
+    """
+    _lib.require_gpu(gx_aug)
+    planes = _check_tile(gx_aug, geom.padded, "halo_fold")
+    lead = tuple(gx_aug.shape[: -geom.n_spatial])
+    if out is None:
+        out = torch.empty(lead + geom.size, dtype=gx_aug.dtype, device=gx_aug.device)
+    elif tuple(out.shape) != lead + geom.size or out.dtype != gx_aug.dtype or not out.is_contiguous():
+        raise ValueError("halo_fold: `out` has the wrong shape / dtype / layout")
+    tab = _table(strips, geom, "fold", lead, gx_aug, None)
+    cg = geom.c_geom(planes)
+    rc = _lib.load().jg_halo_fold_3d(
+        _lib.ptr(out), _lib.ptr(gx_aug), tab, cg, _lib.dtype_code(gx_aug.dtype), _lib.stream_ptr(gx_aug.device)
+    )
+    _lib.check(rc, "jg_halo_fold_3d")
+    return out
+
+
+__all__ = [
+    "HaloGeometry",
+    "halo_assemble",
+    "halo_fold",
+    "halo_pack",
+    "halo_widths",
+    "needed_input_span",
+    "slot",
+]

@@ -1,0 +1,66 @@
+"""Shared helpers of the parity tests (seeded meshes of tiles, bit comparisons)."""
+
+from __future__ import annotations
+
+import itertools
+
+import torch
+
+from jigsaw_amd.halo import HaloGeometry
+
+
+def bits(t: torch.Tensor) -> torch.Tensor:
+    """Reinterpret a float tensor as integers so that equality is bit equality."""
+    t = t.detach().contiguous().cpu()
+    return t.view({2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()])
+
+
+def assert_bit_equal(got: torch.Tensor, want: torch.Tensor, what: str = "") -> None:
+    assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} != {tuple(want.shape)}"
+    assert got.dtype == want.dtype, f"{what}: dtype {got.dtype} != {want.dtype}"
+    g, w = bits(got), bits(want)
+    if not torch.equal(g, w):
+        bad = (g != w).nonzero()
+        raise AssertionError(f"{what}: {bad.shape[0]} elements differ bitwise; first at {bad[0].tolist()}")
+
+
+def rel_l2(got: torch.Tensor, want: torch.Tensor) -> float:
+    g = got.detach().double().cpu()
+    w = want.detach().double().cpu()
+    den = w.norm().item()
+    return (g - w).norm().item() / (den if den > 0 else 1.0)
+
+
+def mesh_coords(mesh_shape):
+    return list(itertools.product(*[range(s) for s in mesh_shape]))
+
+
+def neighbour(coord, offset, mesh_shape):
+    """Mesh coordinate of the neighbour at ``offset`` or None outside the mesh.
+
+    Axes with a group of one have no neighbours (offset must be 0 there).
+    """
+    out = []
+    for c, o, s in zip(coord, offset, mesh_shape):
+        if s <= 1 and o != 0:
+            return None
+        v = c + o
+        if v < 0 or v >= s:
+            return None
+        out.append(v)
+    return tuple(out)
+
+
+def conv_geometry(local_spatial, mesh_shape, coord, kernel, stride, padding, dilation) -> HaloGeometry:
+    return HaloGeometry.for_conv(local_spatial, kernel, stride, padding, dilation, coord, mesh_shape)
+
+
+def special_values_(t: torch.Tensor) -> torch.Tensor:
+    """Sprinkle -0.0, +0.0 and a denormal into a tensor (bit-exactness probes)."""
+    flat = t.view(-1)
+    n = flat.numel()
+    if n >= 16:
+        flat[::7] = -0.0
+        flat[3::11] = 0.0
+        flat[5::13] = 1e-39 if t.dtype == torch.float32 else 1e-39
+    return t

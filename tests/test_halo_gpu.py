@@ -1,0 +1,129 @@
+"""HIP halo assemble / pack / fold against the oracle: bit-exact (GPU)."""
+
+import itertools
+
+import pytest
+import torch
+
+from helpers import assert_bit_equal, conv_geometry, mesh_coords, neighbour, special_values_
+from jigsaw_amd.halo import HaloGeometry, halo_assemble, halo_fold, halo_pack
+from oracle import halo as oh
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # mesh, local spatial, kernel, padding, dilation
+    ((2, 2), (16, 24), (3, 3), (1, 1), (1, 1)),
+    ((3, 3), (8, 9), (3, 3), (1, 1), (1, 1)),
+    ((3, 3), (7, 5), (5, 5), (2, 2), (1, 1)),
+    ((2, 3), (9, 8), (3, 5), (1, 2), (1, 1)),
+    ((3, 2), (8, 8), (3, 3), (2, 2), (2, 2)),
+    ((2, 1), (8, 10), (3, 3), (1, 1), (1, 1)),
+    ((1, 3), (8, 10), (3, 3), (1, 1), (1, 1)),
+    ((3, 3), (4, 4), (4, 2), (2, 1), (1, 1)),  # asymmetric halo: lo 2, hi 1 / lo 1, hi 0
+    ((2, 2, 2), (6, 5, 8), (3, 3, 3), (1, 1, 1), (1, 1, 1)),
+    ((3, 3, 3), (4, 5, 6), (3, 3, 3), (1, 1, 1), (1, 1, 1)),
+    ((3, 1, 3), (4, 5, 6), (5, 3, 3), (2, 1, 1), (1, 1, 1)),
+]
+
+
+def _case_id(c):
+    return "mesh{}_n{}_k{}_p{}_d{}".format(*["x".join(map(str, v)) for v in c])
+
+
+def gpu_strips(tiles_gpu, geoms, coord, mesh, from_padded):
+    """Strips rank `coord` receives: each neighbour packs, the slot facing us is kept."""
+    ns = len(mesh)
+    out = {}
+    for o in itertools.product((-1, 0, 1), repeat=ns):
+        if not any(o):
+            continue
+        nb = neighbour(coord, o, mesh)
+        if nb is None:
+            continue
+        back = tuple(-v for v in o)
+        out[o] = halo_pack(tiles_gpu[nb], geoms[nb], from_padded=from_padded, present=[back])[back]
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", CASES, ids=_case_id)
+def test_assemble_matches_oracle_bitwise(case, dtype, dev):
+    mesh, n, k, p, d = case
+    ns = len(mesh)
+    s = (1,) * ns
+    torch.manual_seed(0)
+    gshape = tuple(a * b for a, b in zip(n, mesh))
+    x = special_values_(torch.randn(2, 3, *gshape)).to(dtype)
+    tiles = oh.split_global(x, mesh)
+    want = oh.gather_mesh(tiles, mesh, k, s, p, d)
+    tiles_gpu = {c: t.to(dev) for c, t in tiles.items()}
+    geoms = {c: conv_geometry(n, mesh, c, k, s, p, d) for c in tiles}
+    for c in mesh_coords(mesh):
+        strips = gpu_strips(tiles_gpu, geoms, c, mesh, from_padded=False)
+        got = halo_assemble(tiles_gpu[c], strips, geoms[c])
+        assert_bit_equal(got, want[c], f"rank {c}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", CASES, ids=_case_id)
+def test_fold_matches_oracle_bitwise(case, dtype, dev):
+    mesh, n, k, p, d = case
+    ns = len(mesh)
+    s = (1,) * ns
+    torch.manual_seed(1)
+    geoms = {c: conv_geometry(n, mesh, c, k, s, p, d) for c in mesh_coords(mesh)}
+    # magnitudes spread over many binades so that the association order matters
+    grads = {}
+    for c, g in geoms.items():
+        t = torch.randn(2, 3, *g.padded) * torch.exp2(torch.randint(-12, 12, (2, 3, *g.padded)).float())
+        grads[c] = special_values_(t).to(dtype)
+    want = oh.scatter_add_mesh(grads, mesh, k, s, p, d, n)
+    grads_gpu = {c: t.to(dev) for c, t in grads.items()}
+    for c in mesh_coords(mesh):
+        strips = gpu_strips(grads_gpu, geoms, c, mesh, from_padded=True)
+        got = halo_fold(grads_gpu[c], strips, geoms[c])
+        assert_bit_equal(got, want[c], f"rank {c}")
+
+
+def test_assemble_rejects_wrong_shapes(dev):
+    g = HaloGeometry((8, 8), (1, 1), (1, 1))
+    x = torch.zeros(1, 2, 8, 8, device=dev)
+    with pytest.raises(ValueError):
+        halo_assemble(x, {(0, 1): torch.zeros(1, 2, 8, 2, device=dev)}, g)
+    with pytest.raises(ValueError):
+        halo_assemble(torch.zeros(1, 2, 8, 7, device=dev), {}, g)
+    with pytest.raises(RuntimeError):
+        halo_assemble(torch.zeros(1, 2, 8, 8), {}, g)
+
+
+def test_geometry_rejects_drifting_spans():
+    # kernel 3, stride 2, padding 1 on 8 rows per rank is fine; padding 0 drifts
+    HaloGeometry.for_conv((8,), (3,), (2,), (1,), (1,), (1,), (2,))
+    with pytest.raises(NotImplementedError):
+        HaloGeometry.for_conv((9,), (3,), (1,), (0,), (1,), (1,), (2,))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_assemble_fold_full_size_properties(dtype, dev):
+    """Config-2-like tile (reduced batch): window identity and adjoint identity on device."""
+    torch.manual_seed(3)
+    n, mesh, c = (1024, 1024), (3, 3), (1, 1)
+    geom = HaloGeometry(n, (1, 1), (1, 1))
+    lead = (2, 64)
+    x = torch.randn(*lead, *n, device=dev).to(dtype)
+    strips = {o: torch.randn(*lead, *geom.strip_extent(o, "assemble"), device=dev).to(dtype) for o in geom.offsets()}
+    aug = halo_assemble(x, strips, geom)
+    assert torch.equal(aug[..., 1:-1, 1:-1], x)
+    assert torch.equal(aug[..., 0:1, 1:-1], strips[(-1, 0)])
+    assert torch.equal(aug[..., 1:-1, -1:], strips[(0, 1)])
+    assert torch.equal(aug[..., -1:, 0:1], strips[(1, -1)])
+    # a rank with no neighbours: the halo is zero and fold(assemble(x)) == x + 0
+    alone = halo_assemble(x, {}, geom)
+    assert alone[..., 0, :].abs().max().item() == 0 and alone[..., :, -1].abs().max().item() == 0
+    back = halo_fold(alone, {}, geom)
+    assert torch.equal(back, x + 0.0)
+    # pack_bwd of the padded tensor returns exactly the strips that went in
+    cut = halo_pack(aug, geom, from_padded=True)
+    for o, t in strips.items():
+        assert torch.equal(cut[o], t), o
