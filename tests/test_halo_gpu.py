@@ -12,23 +12,24 @@ from oracle import halo as oh
 pytestmark = pytest.mark.gpu
 
 CASES = [
-    # mesh, local spatial, kernel, padding, dilation
-    ((2, 2), (16, 24), (3, 3), (1, 1), (1, 1)),
-    ((3, 3), (8, 9), (3, 3), (1, 1), (1, 1)),
-    ((3, 3), (7, 5), (5, 5), (2, 2), (1, 1)),
-    ((2, 3), (9, 8), (3, 5), (1, 2), (1, 1)),
-    ((3, 2), (8, 8), (3, 3), (2, 2), (2, 2)),
-    ((2, 1), (8, 10), (3, 3), (1, 1), (1, 1)),
-    ((1, 3), (8, 10), (3, 3), (1, 1), (1, 1)),
-    ((3, 3), (4, 4), (4, 2), (2, 1), (1, 1)),  # asymmetric halo: lo 2, hi 1 / lo 1, hi 0
-    ((2, 2, 2), (6, 5, 8), (3, 3, 3), (1, 1, 1), (1, 1, 1)),
-    ((3, 3, 3), (4, 5, 6), (3, 3, 3), (1, 1, 1), (1, 1, 1)),
-    ((3, 1, 3), (4, 5, 6), (5, 3, 3), (2, 1, 1), (1, 1, 1)),
+    # mesh, local spatial, kernel, stride, padding, dilation
+    ((2, 2), (16, 24), (3, 3), (1, 1), (1, 1), (1, 1)),
+    ((3, 3), (8, 9), (3, 3), (1, 1), (1, 1), (1, 1)),
+    ((3, 3), (7, 5), (5, 5), (1, 1), (2, 2), (1, 1)),
+    ((2, 3), (9, 8), (3, 5), (1, 1), (1, 2), (1, 1)),
+    ((3, 2), (8, 8), (3, 3), (1, 1), (2, 2), (2, 2)),
+    ((2, 1), (8, 10), (3, 3), (1, 1), (1, 1), (1, 1)),
+    ((1, 3), (8, 10), (3, 3), (1, 1), (1, 1), (1, 1)),
+    ((3, 3), (4, 6), (3, 5), (2, 2), (1, 2), (1, 1)),  # strided: halo (lo 1, hi 0) and (lo 2, hi 1)
+    ((3, 3), (2, 2), (5, 5), (1, 1), (2, 2), (1, 1)),  # halo as wide as the tile
+    ((2, 2, 2), (6, 5, 8), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+    ((3, 3, 3), (4, 5, 6), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+    ((3, 1, 3), (4, 5, 6), (5, 3, 3), (1, 1, 1), (2, 1, 1), (1, 1, 1)),
 ]
 
 
 def _case_id(c):
-    return "mesh{}_n{}_k{}_p{}_d{}".format(*["x".join(map(str, v)) for v in c])
+    return "mesh{}_n{}_k{}_s{}_p{}_d{}".format(*["x".join(map(str, v)) for v in c])
 
 
 def gpu_strips(tiles_gpu, geoms, coord, mesh, from_padded):
@@ -49,9 +50,7 @@ def gpu_strips(tiles_gpu, geoms, coord, mesh, from_padded):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("case", CASES, ids=_case_id)
 def test_assemble_matches_oracle_bitwise(case, dtype, dev):
-    mesh, n, k, p, d = case
-    ns = len(mesh)
-    s = (1,) * ns
+    mesh, n, k, s, p, d = case
     torch.manual_seed(0)
     gshape = tuple(a * b for a, b in zip(n, mesh))
     x = special_values_(torch.randn(2, 3, *gshape)).to(dtype)
@@ -68,9 +67,7 @@ def test_assemble_matches_oracle_bitwise(case, dtype, dev):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("case", CASES, ids=_case_id)
 def test_fold_matches_oracle_bitwise(case, dtype, dev):
-    mesh, n, k, p, d = case
-    ns = len(mesh)
-    s = (1,) * ns
+    mesh, n, k, s, p, d = case
     torch.manual_seed(1)
     geoms = {c: conv_geometry(n, mesh, c, k, s, p, d) for c in mesh_coords(mesh)}
     # magnitudes spread over many binades so that the association order matters
