@@ -133,6 +133,61 @@ int jg_roll_pack(void* strip, const void* x, int ndim, const int64_t* sizes,
 int jg_roll_unpack(void* x, const void* strip, int ndim, const int64_t* sizes,
                    int axis, int64_t window, int elem_size, void* stream);
 
+/* ------------------------------------------------------------------------- *
+ * Sharded LayerNorm (last axis split over the channel group; HBM-bound)
+ *
+ * x is (rows, cols) dense with cols = the LOCAL width. Statistics are fp32.
+ * The two all-reduces between partial statistics and apply stay with the
+ * caller (jigsaw/modules/normalization/_functional.py:49-53, 160-171).
+ * ------------------------------------------------------------------------- */
+
+/* Per row: mean[r] = mean(x[r,:]), var[r] = biased variance of x[r,:]
+ * (local_mean / local_var of _functional.py:46-47). */
+int jg_ln_partial_fwd(float* mean, float* var, const void* x, int64_t rows,
+                      int64_t cols, int x_dtype, void* stream);
+
+/* x_hat = (x - mean) / sqrt(var + eps);  y = w * x_hat + b  (_functional.py:55-58)
+ * with the COMBINED statistics. Also writes std[r] = sqrt(var[r] + eps), the
+ * tensor the backward saves (_functional.py:75). w, b, y, x_hat have dtype
+ * out_dtype; b may be NULL; x_hat may be NULL (inference). */
+int jg_ln_apply(void* y, void* x_hat, float* std_out, const void* x,
+                const float* mean, const float* var, const void* w, const void* b,
+                int64_t rows, int64_t cols, float eps, int x_dtype, int out_dtype,
+                void* stream);
+
+/* Backward partials (_functional.py:150-168), one pass over g and x_hat:
+ *   mean_gxn[r] = mean_c(g*w), dot_gxn_xhat[r] = sum_c(g*w*x_hat)   (per row)
+ *   gw[c] = sum_r g*x_hat,      gb[c] = sum_r g                     (per column)
+ * gw / gb are fp32 (cols,); either may be NULL. workspace: device scratch of
+ * jg_ln_bwd_workspace_bytes(rows, cols) bytes (deterministic two-stage column
+ * reduction, no atomics). g, x_hat, w share `dtype`. */
+size_t jg_ln_bwd_workspace_bytes(int64_t rows, int64_t cols);
+int jg_ln_partial_bwd(float* mean_gxn, float* dot_gxn_xhat, float* gw, float* gb,
+                      const void* g, const void* x_hat, const void* w, int64_t rows,
+                      int64_t cols, int dtype, void* workspace, size_t workspace_bytes,
+                      void* stream);
+
+/* gx = (1/std) * (g*w - mean_gxn - x_hat * dot_gxn_xhat / n_global) with the
+ * COMBINED row terms (_functional.py:173-175). */
+int jg_ln_bwd_apply(void* gx, const void* g, const void* x_hat, const void* w,
+                    const float* mean_gxn, const float* dot_gxn_xhat,
+                    const float* std, int64_t rows, int64_t cols, int64_t n_global,
+                    int dtype, void* stream);
+
+/* ------------------------------------------------------------------------- *
+ * Online-softmax / log-sum-exp merge of ring attention (HBM-bound)
+ * ------------------------------------------------------------------------- */
+
+/* In place on o1:  w = sigmoid(l2 - l1);  o1 += w * (o2 - o1);
+ * l_new = max(l1,l2) + log(1 + exp(-|l1 - l2|)).
+ * Stands in for the Triton kernel behind fused_online_softmax_merge_
+ * (jigsaw/modules/attention/_functional/_merge_kernel.py:37-82, 88-172).
+ * o1 / o2: (b, h, n, d) when bshd == 0, (b, n, h, d) when bshd != 0;
+ * l1, l2, l_new: fp32 (b, h, n). l_new must not alias l1 or l2. */
+int jg_lse_merge(void* o1, const float* l1, const void* o2, const float* l2,
+                 float* l_new, int64_t b, int64_t h, int64_t n, int64_t d, int bshd,
+                 int o1_dtype, int o2_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

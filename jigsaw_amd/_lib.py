@@ -66,6 +66,28 @@ SIGNATURES: dict[str, tuple] = {
     "jg_roll": (c_int, [c_void_p, c_void_p, c_int, POINTER(c_int64), POINTER(c_int64), c_int, c_void_p]),
     "jg_roll_pack": (c_int, [c_void_p, c_void_p, c_int, POINTER(c_int64), c_int, c_int64, c_int, c_void_p]),
     "jg_roll_unpack": (c_int, [c_void_p, c_void_p, c_int, POINTER(c_int64), c_int, c_int64, c_int, c_void_p]),
+    "jg_ln_partial_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
+    "jg_ln_apply": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_float,
+         c_int, c_int, c_void_p],
+    ),
+    "jg_ln_bwd_workspace_bytes": (c_size_t, [c_int64, c_int64]),
+    "jg_ln_partial_bwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p,
+         c_size_t, c_void_p],
+    ),
+    "jg_ln_bwd_apply": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int,
+         c_void_p],
+    ),
+    "jg_lse_merge": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int,
+         c_void_p],
+    ),
 }
 
 

@@ -1,0 +1,445 @@
+// Sharded LayerNorm: partial statistics, apply, and the backward partials.
+// One wavefront owns one row at a time; lanes stride the columns in 16-byte (or
+// 8-byte) vectors so every global access is coalesced; row reductions are
+// wavefront butterflies (no LDS), column reductions are per-lane registers plus
+// a deterministic two-stage tree (no atomics). Everything is HBM-bound.
+//
+// Reference behaviour restated here:
+//   jigsaw/modules/normalization/_functional.py:45-58   (forward)
+//   jigsaw/modules/normalization/_functional.py:141-175 (backward)
+#include "jg_common.h"
+
+namespace {
+
+constexpr int kWave = 64;
+constexpr int kWavesPerBlock = 4;
+constexpr int kThreads = kWave * kWavesPerBlock;
+constexpr int kVec = 4;        // elements per lane per step
+constexpr int kMaxChunks = 8;  // column chunks a lane can own in the backward
+
+template <int DT>
+struct Elem;
+template <>
+struct Elem<JG_F32> {
+  typedef float T;
+  __device__ static __forceinline__ float up(float v) { return v; }
+  __device__ static __forceinline__ float down(float v) { return v; }
+};
+template <>
+struct Elem<JG_BF16> {
+  typedef uint16_t T;
+  __device__ static __forceinline__ float up(uint16_t v) { return jg::bf16_to_f32(v); }
+  __device__ static __forceinline__ uint16_t down(float v) { return jg::f32_to_bf16(v); }
+};
+template <>
+struct Elem<JG_F16> {
+  typedef _Float16 T;
+  __device__ static __forceinline__ float up(_Float16 v) { return (float)v; }
+  __device__ static __forceinline__ _Float16 down(float v) { return (_Float16)v; }
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+
+// Load up to kVec consecutive elements of a row starting at column c (c % kVec == 0).
+template <int DT>
+__device__ __forceinline__ void load_vec(const typename Elem<DT>::T* row, long long c,
+                                         long long cols, bool vec_ok, float out[kVec]) {
+  typedef typename Elem<DT>::T T;
+  if (vec_ok && c + kVec <= cols) {
+    struct alignas(sizeof(T) * kVec) Pack { T v[kVec]; };
+    Pack p = *reinterpret_cast<const Pack*>(row + c);
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) out[i] = Elem<DT>::up(p.v[i]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) out[i] = (c + i < cols) ? Elem<DT>::up(row[c + i]) : 0.0f;
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void store_vec(typename Elem<DT>::T* row, long long c, long long cols,
+                                          bool vec_ok, const float in[kVec]) {
+  typedef typename Elem<DT>::T T;
+  if (vec_ok && c + kVec <= cols) {
+    struct alignas(sizeof(T) * kVec) Pack { T v[kVec]; };
+    Pack p;
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) p.v[i] = Elem<DT>::down(in[i]);
+    *reinterpret_cast<Pack*>(row + c) = p;
+  } else {
+#pragma unroll
+    for (int i = 0; i < kVec; ++i)
+      if (c + i < cols) row[c + i] = Elem<DT>::down(in[i]);
+  }
+}
+
+// ---------------------------------------------------------- partial statistics
+template <int DT>
+__global__ __launch_bounds__(kThreads) void ln_partial_fwd_kernel(
+    float* __restrict__ mean, float* __restrict__ var, const typename Elem<DT>::T* __restrict__ x,
+    long long rows, long long cols, bool vec_ok) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const float inv = 1.0f / (float)cols;
+  for (long long r = (long long)blockIdx.x * kWavesPerBlock + wave; r < rows;
+       r += (long long)gridDim.x * kWavesPerBlock) {
+    const typename Elem<DT>::T* row = x + r * cols;
+    float s = 0.0f;
+    for (long long c = (long long)lane * kVec; c < cols; c += kWave * kVec) {
+      float v[kVec];
+      load_vec<DT>(row, c, cols, vec_ok, v);
+#pragma unroll
+      for (int i = 0; i < kVec; ++i) s += v[i];
+    }
+    const float m = wave_sum(s) * inv;
+    float q = 0.0f;
+    for (long long c = (long long)lane * kVec; c < cols; c += kWave * kVec) {
+      float v[kVec];
+      load_vec<DT>(row, c, cols, vec_ok, v);
+#pragma unroll
+      for (int i = 0; i < kVec; ++i) {
+        float d = (c + i < cols) ? v[i] - m : 0.0f;
+        q += d * d;
+      }
+    }
+    q = wave_sum(q) * inv;
+    if (lane == 0) {
+      mean[r] = m;
+      var[r] = q;
+    }
+  }
+}
+
+// ----------------------------------------------------------------------- apply
+template <int XDT, int ODT>
+__global__ __launch_bounds__(kThreads) void ln_apply_kernel(
+    typename Elem<ODT>::T* __restrict__ y, typename Elem<ODT>::T* __restrict__ x_hat,
+    float* __restrict__ std_out, const typename Elem<XDT>::T* __restrict__ x,
+    const float* __restrict__ mean, const float* __restrict__ var,
+    const typename Elem<ODT>::T* __restrict__ w, const typename Elem<ODT>::T* __restrict__ b,
+    long long rows, long long cols, float eps, bool vx_ok, bool vo_ok, bool vw_ok) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  for (long long r = (long long)blockIdx.x * kWavesPerBlock + wave; r < rows;
+       r += (long long)gridDim.x * kWavesPerBlock) {
+    const float m = mean[r];
+    const float sd = sqrtf(var[r] + eps);
+    if (lane == 0 && std_out != nullptr) std_out[r] = sd;
+    for (long long c = (long long)lane * kVec; c < cols; c += kWave * kVec) {
+      float v[kVec], wv[kVec], bv[kVec], xh[kVec], out[kVec];
+      load_vec<XDT>(x + r * cols, c, cols, vx_ok, v);
+      load_vec<ODT>(w, c, cols, vw_ok, wv);
+      if (b != nullptr) load_vec<ODT>(b, c, cols, vw_ok, bv);
+#pragma unroll
+      for (int i = 0; i < kVec; ++i) {
+        // x_hat is rounded to the output dtype before the affine map, as the
+        // reference materialises x_norm in that dtype and then multiplies.
+        xh[i] = Elem<ODT>::up(Elem<ODT>::down((v[i] - m) / sd));
+        out[i] = wv[i] * xh[i] + (b != nullptr ? bv[i] : 0.0f);
+      }
+      if (x_hat != nullptr) store_vec<ODT>(x_hat + r * cols, c, cols, vo_ok, xh);
+      store_vec<ODT>(y + r * cols, c, cols, vo_ok, out);
+    }
+  }
+}
+
+// ------------------------------------------------------------ backward partials
+// Stage 1: block `blk` walks rows blk*kWavesPerBlock + wave + k*gridDim*kWavesPerBlock.
+// Each lane keeps column partials for the columns it touches; they are reduced
+// across the block's waves in LDS and written to part[blk][which][col].
+template <int DT, int CH>
+__global__ __launch_bounds__(kThreads) void ln_partial_bwd_kernel(
+    float* __restrict__ mean_gxn, float* __restrict__ dot, float* __restrict__ part,
+    const typename Elem<DT>::T* __restrict__ g, const typename Elem<DT>::T* __restrict__ x_hat,
+    const typename Elem<DT>::T* __restrict__ w, long long rows, long long cols, bool vec_ok,
+    bool vw_ok, bool want_cols) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const float inv = 1.0f / (float)cols;
+  float wv[CH][kVec];
+  float agw[CH][kVec], agb[CH][kVec];
+#pragma unroll
+  for (int k = 0; k < CH; ++k) {
+    long long c = ((long long)k * kWave + lane) * kVec;
+    if (c < cols) load_vec<DT>(w, c, cols, vw_ok, wv[k]);
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) {
+      agw[k][i] = 0.0f;
+      agb[k][i] = 0.0f;
+      if (c >= cols) wv[k][i] = 0.0f;
+    }
+  }
+  for (long long r = (long long)blockIdx.x * kWavesPerBlock + wave; r < rows;
+       r += (long long)gridDim.x * kWavesPerBlock) {
+    float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+      long long c = ((long long)k * kWave + lane) * kVec;
+      if (c < cols) {
+        float gv[kVec], xh[kVec];
+        load_vec<DT>(g + r * cols, c, cols, vec_ok, gv);
+        load_vec<DT>(x_hat + r * cols, c, cols, vec_ok, xh);
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) {
+          // grad_x_norm = g * w is materialised in the tensor dtype by the reference
+          float gxn = Elem<DT>::up(Elem<DT>::down(gv[i] * wv[k][i]));
+          s1 += gxn;
+          s2 += gxn * xh[i];
+          agw[k][i] += gv[i] * xh[i];
+          agb[k][i] += gv[i];
+        }
+      }
+    }
+    s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    if (lane == 0) {
+      mean_gxn[r] = s1 * inv;
+      dot[r] = s2;
+    }
+  }
+  if (!want_cols) return;
+  __shared__ float red[kWavesPerBlock][2][CH * kWave * kVec];
+#pragma unroll
+  for (int k = 0; k < CH; ++k)
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) {
+      red[wave][0][(k * kWave + lane) * kVec + i] = agw[k][i];
+      red[wave][1][(k * kWave + lane) * kVec + i] = agb[k][i];
+    }
+  __syncthreads();
+  for (long long c = threadIdx.x; c < cols; c += kThreads) {
+    float a = 0.0f, b2 = 0.0f;
+#pragma unroll
+    for (int wv2 = 0; wv2 < kWavesPerBlock; ++wv2) {
+      a += red[wv2][0][c];
+      b2 += red[wv2][1][c];
+    }
+    part[((long long)blockIdx.x * 2 + 0) * cols + c] = a;
+    part[((long long)blockIdx.x * 2 + 1) * cols + c] = b2;
+  }
+}
+
+// Stage 2: one thread per column sums the block partials in block order.
+__global__ __launch_bounds__(256) void ln_colreduce_kernel(float* __restrict__ gw,
+                                                           float* __restrict__ gb,
+                                                           const float* __restrict__ part,
+                                                           int nblocks, long long cols) {
+  long long c = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (c >= cols) return;
+  float a = 0.0f, b = 0.0f;
+  for (int k = 0; k < nblocks; ++k) {
+    a += part[((long long)k * 2 + 0) * cols + c];
+    b += part[((long long)k * 2 + 1) * cols + c];
+  }
+  if (gw != nullptr) gw[c] = a;
+  if (gb != nullptr) gb[c] = b;
+}
+
+template <int DT>
+__global__ __launch_bounds__(kThreads) void ln_bwd_apply_kernel(
+    typename Elem<DT>::T* __restrict__ gx, const typename Elem<DT>::T* __restrict__ g,
+    const typename Elem<DT>::T* __restrict__ x_hat, const typename Elem<DT>::T* __restrict__ w,
+    const float* __restrict__ mean_gxn, const float* __restrict__ dot,
+    const float* __restrict__ stdv, long long rows, long long cols, float inv_n, bool vec_ok,
+    bool vw_ok) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  for (long long r = (long long)blockIdx.x * kWavesPerBlock + wave; r < rows;
+       r += (long long)gridDim.x * kWavesPerBlock) {
+    const float m = mean_gxn[r];
+    const float dn = dot[r] * inv_n;
+    const float rs = 1.0f / stdv[r];
+    for (long long c = (long long)lane * kVec; c < cols; c += kWave * kVec) {
+      float gv[kVec], xh[kVec], wv[kVec], out[kVec];
+      load_vec<DT>(g + r * cols, c, cols, vec_ok, gv);
+      load_vec<DT>(x_hat + r * cols, c, cols, vec_ok, xh);
+      load_vec<DT>(w, c, cols, vw_ok, wv);
+#pragma unroll
+      for (int i = 0; i < kVec; ++i) {
+        float gxn = Elem<DT>::up(Elem<DT>::down(gv[i] * wv[i]));
+        out[i] = rs * (gxn - m - xh[i] * dn);
+      }
+      store_vec<DT>(gx + r * cols, c, cols, vec_ok, out);
+    }
+  }
+}
+
+int row_grid(long long rows) {
+  long long b = (rows + kWavesPerBlock - 1) / kWavesPerBlock;
+  if (b > 65536) b = 65536;
+  if (b < 1) b = 1;
+  return (int)b;
+}
+
+int bwd_blocks(long long rows) {
+  long long b = (rows + kWavesPerBlock - 1) / kWavesPerBlock;
+  if (b > 1024) b = 1024;  // 4 blocks per CU; bounds the stage-2 sum length
+  if (b < 1) b = 1;
+  return (int)b;
+}
+
+bool vec_aligned(const void* p, long long cols, int dtype) {
+  const size_t bytes = jg::dtype_size(dtype) * kVec;
+  return (reinterpret_cast<uintptr_t>(p) % bytes) == 0 && (cols % kVec) == 0;
+}
+
+bool known(int dt) { return dt == JG_F32 || dt == JG_BF16 || dt == JG_F16; }
+
+}  // namespace
+
+extern "C" int jg_ln_partial_fwd(float* mean, float* var, const void* x, int64_t rows,
+                                 int64_t cols, int x_dtype, void* stream) {
+  JG_REQUIRE(mean && var && x, "jg_ln_partial_fwd: NULL pointer");
+  JG_REQUIRE(rows >= 0 && cols >= 1, "jg_ln_partial_fwd: bad shape (%lld, %lld)",
+             (long long)rows, (long long)cols);
+  JG_REQUIRE(known(x_dtype), "jg_ln_partial_fwd: unknown dtype %d", x_dtype);
+  if (rows == 0) return JG_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool v = vec_aligned(x, cols, x_dtype);
+#define JG_GO(DT)                                                          \
+  ln_partial_fwd_kernel<DT><<<row_grid(rows), kThreads, 0, s>>>(           \
+      mean, var, static_cast<const Elem<DT>::T*>(x), rows, cols, v)
+  if (x_dtype == JG_F32) JG_GO(JG_F32);
+  else if (x_dtype == JG_BF16) JG_GO(JG_BF16);
+  else JG_GO(JG_F16);
+#undef JG_GO
+  JG_CHECK_LAUNCH("jg_ln_partial_fwd");
+  return JG_OK;
+}
+
+template <int XDT, int ODT>
+static void launch_apply(void* y, void* x_hat, float* std_out, const void* x, const float* mean,
+                         const float* var, const void* w, const void* b, int64_t rows,
+                         int64_t cols, float eps, hipStream_t s) {
+  typedef typename Elem<XDT>::T XT;
+  typedef typename Elem<ODT>::T OT;
+  const bool vx = vec_aligned(x, cols, XDT);
+  const bool vo = vec_aligned(y, cols, ODT) && (x_hat == nullptr || vec_aligned(x_hat, cols, ODT));
+  const bool vw = vec_aligned(w, cols, ODT) && (b == nullptr || vec_aligned(b, cols, ODT));
+  ln_apply_kernel<XDT, ODT><<<row_grid(rows), kThreads, 0, s>>>(
+      static_cast<OT*>(y), static_cast<OT*>(x_hat), std_out, static_cast<const XT*>(x), mean, var,
+      static_cast<const OT*>(w), static_cast<const OT*>(b), rows, cols, eps, vx, vo, vw);
+}
+
+extern "C" int jg_ln_apply(void* y, void* x_hat, float* std_out, const void* x,
+                           const float* mean, const float* var, const void* w, const void* b,
+                           int64_t rows, int64_t cols, float eps, int x_dtype, int out_dtype,
+                           void* stream) {
+  JG_REQUIRE(y && x && mean && var && w, "jg_ln_apply: NULL pointer");
+  JG_REQUIRE(rows >= 0 && cols >= 1, "jg_ln_apply: bad shape");
+  JG_REQUIRE(known(x_dtype) && known(out_dtype), "jg_ln_apply: unknown dtype");
+  if (rows == 0) return JG_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define JG_GO(X, O) launch_apply<X, O>(y, x_hat, std_out, x, mean, var, w, b, rows, cols, eps, s)
+  if (x_dtype == out_dtype) {
+    if (x_dtype == JG_F32) JG_GO(JG_F32, JG_F32);
+    else if (x_dtype == JG_BF16) JG_GO(JG_BF16, JG_BF16);
+    else JG_GO(JG_F16, JG_F16);
+  } else if (out_dtype == JG_F32) {
+    // autocast: low-precision input promoted to fp32 on the fly
+    if (x_dtype == JG_BF16) JG_GO(JG_BF16, JG_F32);
+    else JG_GO(JG_F16, JG_F32);
+  } else {
+    JG_FAIL(JG_ERR_UNSUPPORTED, "jg_ln_apply: x dtype %d with output dtype %d", x_dtype,
+            out_dtype);
+  }
+#undef JG_GO
+  JG_CHECK_LAUNCH("jg_ln_apply");
+  return JG_OK;
+}
+
+extern "C" size_t jg_ln_bwd_workspace_bytes(int64_t rows, int64_t cols) {
+  if (rows <= 0 || cols <= 0) return 0;
+  return (size_t)bwd_blocks(rows) * 2 * (size_t)cols * sizeof(float);
+}
+
+template <int DT>
+static int launch_partial_bwd(float* mean_gxn, float* dot, float* part, const void* g,
+                              const void* x_hat, const void* w, int64_t rows, int64_t cols,
+                              bool want_cols, hipStream_t s) {
+  typedef typename Elem<DT>::T T;
+  const bool v = vec_aligned(g, cols, DT) && vec_aligned(x_hat, cols, DT);
+  const bool vw = vec_aligned(w, cols, DT);
+  const int nb = bwd_blocks(rows);
+  const long long per = (long long)kWave * kVec;
+  const int ch = (int)((cols + per - 1) / per);
+#define JG_GO(CH)                                                                        \
+  ln_partial_bwd_kernel<DT, CH><<<nb, kThreads, 0, s>>>(                                 \
+      mean_gxn, dot, part, static_cast<const T*>(g), static_cast<const T*>(x_hat),       \
+      static_cast<const T*>(w), rows, cols, v, vw, want_cols)
+  if (ch <= 1) JG_GO(1);
+  else if (ch <= 2) JG_GO(2);
+  else if (ch <= 4) JG_GO(4);
+  else if (ch <= kMaxChunks) JG_GO(8);
+  else
+    JG_FAIL(JG_ERR_UNSUPPORTED, "jg_ln_partial_bwd: local width %lld exceeds %lld",
+            (long long)cols, (long long)(per * kMaxChunks));
+#undef JG_GO
+  return JG_OK;
+}
+
+extern "C" int jg_ln_partial_bwd(float* mean_gxn, float* dot_gxn_xhat, float* gw, float* gb,
+                                 const void* g, const void* x_hat, const void* w, int64_t rows,
+                                 int64_t cols, int dtype, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  JG_REQUIRE(mean_gxn && dot_gxn_xhat && g && x_hat && w, "jg_ln_partial_bwd: NULL pointer");
+  JG_REQUIRE(rows >= 0 && cols >= 1, "jg_ln_partial_bwd: bad shape");
+  JG_REQUIRE(known(dtype), "jg_ln_partial_bwd: unknown dtype %d", dtype);
+  if (rows == 0) return JG_OK;
+  const bool want_cols = gw != nullptr || gb != nullptr;
+  if (want_cols) {
+    JG_REQUIRE(workspace != nullptr, "jg_ln_partial_bwd: workspace is NULL");
+    if (workspace_bytes < jg_ln_bwd_workspace_bytes(rows, cols))
+      JG_FAIL(JG_ERR_WORKSPACE, "jg_ln_partial_bwd: workspace %zu < %zu bytes", workspace_bytes,
+              jg_ln_bwd_workspace_bytes(rows, cols));
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* part = static_cast<float*>(workspace);
+  int rc;
+  if (dtype == JG_F32)
+    rc = launch_partial_bwd<JG_F32>(mean_gxn, dot_gxn_xhat, part, g, x_hat, w, rows, cols, want_cols, s);
+  else if (dtype == JG_BF16)
+    rc = launch_partial_bwd<JG_BF16>(mean_gxn, dot_gxn_xhat, part, g, x_hat, w, rows, cols, want_cols, s);
+  else
+    rc = launch_partial_bwd<JG_F16>(mean_gxn, dot_gxn_xhat, part, g, x_hat, w, rows, cols, want_cols, s);
+  if (rc) return rc;
+  JG_CHECK_LAUNCH("jg_ln_partial_bwd");
+  if (want_cols) {
+    ln_colreduce_kernel<<<jg::cdiv(cols, 256), 256, 0, s>>>(gw, gb, part, bwd_blocks(rows), cols);
+    JG_CHECK_LAUNCH("jg_ln_partial_bwd(colreduce)");
+  }
+  return JG_OK;
+}
+
+extern "C" int jg_ln_bwd_apply(void* gx, const void* g, const void* x_hat, const void* w,
+                               const float* mean_gxn, const float* dot_gxn_xhat,
+                               const float* std, int64_t rows, int64_t cols, int64_t n_global,
+                               int dtype, void* stream) {
+  JG_REQUIRE(gx && g && x_hat && w && mean_gxn && dot_gxn_xhat && std,
+             "jg_ln_bwd_apply: NULL pointer");
+  JG_REQUIRE(rows >= 0 && cols >= 1 && n_global >= 1, "jg_ln_bwd_apply: bad shape");
+  JG_REQUIRE(known(dtype), "jg_ln_bwd_apply: unknown dtype %d", dtype);
+  if (rows == 0) return JG_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const float inv_n = 1.0f / (float)n_global;
+#define JG_GO(DT)                                                                          \
+  do {                                                                                     \
+    typedef Elem<DT>::T T;                                                                 \
+    const bool v = vec_aligned(g, cols, DT) && vec_aligned(x_hat, cols, DT) &&             \
+                   vec_aligned(gx, cols, DT);                                              \
+    const bool vw = vec_aligned(w, cols, DT);                                              \
+    ln_bwd_apply_kernel<DT><<<row_grid(rows), kThreads, 0, s>>>(                           \
+        static_cast<T*>(gx), static_cast<const T*>(g), static_cast<const T*>(x_hat),       \
+        static_cast<const T*>(w), mean_gxn, dot_gxn_xhat, std, rows, cols, inv_n, v, vw);  \
+  } while (0)
+  if (dtype == JG_F32) JG_GO(JG_F32);
+  else if (dtype == JG_BF16) JG_GO(JG_BF16);
+  else JG_GO(JG_F16);
+#undef JG_GO
+  JG_CHECK_LAUNCH("jg_ln_bwd_apply");
+  return JG_OK;
+}

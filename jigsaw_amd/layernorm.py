@@ -1,0 +1,155 @@
+"""Sharded LayerNorm on the GPU.
+
+Host-side mirror of ``_LayerNorm`` (jigsaw/modules/normalization/_functional.py:13-177):
+same call signature ``apply(x, weight, bias, channel_group, eps)`` and the same
+four outputs, so it can be assigned to ``DistributedLayerNorm.layernorm``
+(jigsaw/modules/normalization/_layer_norm.py:90-94). The partial statistics, the
+normalise + affine epilogue and the backward partials run in HIP kernels; the
+two all-reduces per direction over the channel group stay here.
+"""
+
+from __future__ import annotations
+
+from typing import Any
+
+import torch
+import torch.distributed as dist
+
+from . import _lib
+
+
+def _group_size(group: Any) -> int:
+    if group is None:
+        return 1
+    return int(group.size())
+
+
+def _all_reduce(t: torch.Tensor, op: str, group: Any) -> None:
+    """AVG / SUM all-reduce of ``t`` over the channel group, in place.
+
+    ``group`` is a ``torch.distributed`` process group, ``None`` (no sharding), or
+    any object with ``size()`` and ``all_reduce(tensor, op)`` (a single-process
+    stand-in that already holds the other shards' contributions).
+    """
+    if _group_size(group) == 1:
+        return
+    if hasattr(group, "all_reduce"):
+        group.all_reduce(t, op)
+        return
+    red = dist.ReduceOp.AVG if op == "avg" else dist.ReduceOp.SUM
+    dist.all_reduce(t, op=red, group=group)
+
+
+def partial_stats(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """fp32 ``(mean, biased var)`` over the last (local) axis, shape ``(..., 1)``."""
+    _lib.require_gpu(x)
+    x = x.contiguous()
+    cols = x.shape[-1]
+    rows = x.numel() // cols if cols else 0
+    mean = torch.empty(x.shape[:-1] + (1,), dtype=torch.float32, device=x.device)
+    var = torch.empty_like(mean)
+    rc = _lib.load().jg_ln_partial_fwd(
+        _lib.ptr(mean), _lib.ptr(var), _lib.ptr(x), rows, cols, _lib.dtype_code(x.dtype), _lib.stream_ptr(x.device)
+    )
+    _lib.check(rc, "jg_ln_partial_fwd")
+    return mean, var
+
+
+def _compute_dtype(x: torch.Tensor) -> torch.dtype:
+    # promote_to_fp32_under_autocast (jigsaw/_core/autocast.py:83-107): norms run in
+    # fp32 when autocast is on, otherwise in the input dtype.
+    if torch.is_autocast_enabled():
+        return torch.float32
+    return x.dtype
+
+
+class _LayerNorm(torch.autograd.Function):
+    """Autograd function of the distributed LayerNorm (HIP kernels inside)."""
+
+    @staticmethod
+    def forward(x, weight, bias, channel_group, eps):  # noqa: D102
+        _lib.require_gpu(x, weight, bias)
+        cdt = _compute_dtype(x)
+        x = x.contiguous()
+        w = weight.to(cdt).contiguous()
+        b = None if bias is None else bias.to(cdt).contiguous()
+        cols = x.shape[-1]
+        rows = x.numel() // cols
+        local_mean, local_var = partial_stats(x)
+
+        mean = local_mean.clone()
+        _all_reduce(mean, "avg", channel_group)
+        var = local_var + (local_mean - mean) ** 2 if _group_size(channel_group) > 1 else local_var
+        _all_reduce(var, "avg", channel_group)
+
+        y = torch.empty(x.shape, dtype=cdt, device=x.device)
+        x_norm = torch.empty_like(y)
+        rc = _lib.load().jg_ln_apply(
+            _lib.ptr(y), _lib.ptr(x_norm), None, _lib.ptr(x), _lib.ptr(mean), _lib.ptr(var),
+            _lib.ptr(w), _lib.ptr(b), rows, cols, float(eps),
+            _lib.dtype_code(x.dtype), _lib.dtype_code(cdt), _lib.stream_ptr(x.device),
+        )
+        _lib.check(rc, "jg_ln_apply")
+        return y, x_norm, w, (var + eps).to(cdt)
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):  # noqa: D102
+        x, weight, bias, channel_group, eps = inputs
+        _, x_norm, w, var = output
+        ctx.mark_non_differentiable(x_norm, w, var)
+        ctx.channel_group = channel_group
+        ctx.has_bias = bias is not None
+        ctx.param_dtypes = (weight.dtype, None if bias is None else bias.dtype)
+        ctx.in_dtype = x.dtype
+        # sqrt(var + eps), as the reference saves it (_functional.py:75); fp32 for the kernels
+        ctx.save_for_backward(x_norm, w, torch.sqrt(var.to(torch.float32)))
+
+    @staticmethod
+    def backward(ctx, grad_output, x_norm_grad, weight_grad, var_grad):  # noqa: D102
+        x_norm, w, std = ctx.saved_tensors
+        g = grad_output.to(x_norm.dtype).contiguous()
+        group = ctx.channel_group
+        cols = x_norm.shape[-1]
+        rows = x_norm.numel() // cols
+        n_global = cols * _group_size(group)
+        lib = _lib.load()
+        dev = g.device
+
+        mean_gxn = torch.empty_like(std)
+        dot = torch.empty_like(std)
+        need_w = ctx.needs_input_grad[1]
+        need_b = ctx.has_bias and ctx.needs_input_grad[2]
+        gw = torch.empty(cols, dtype=torch.float32, device=dev) if need_w else None
+        gb = torch.empty(cols, dtype=torch.float32, device=dev) if need_b else None
+        ws_bytes = int(lib.jg_ln_bwd_workspace_bytes(rows, cols)) if (need_w or need_b) else 0
+        ws = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=dev)
+        rc = lib.jg_ln_partial_bwd(
+            _lib.ptr(mean_gxn), _lib.ptr(dot), _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(g), _lib.ptr(x_norm),
+            _lib.ptr(w), rows, cols, _lib.dtype_code(g.dtype), _lib.ptr(ws), ws_bytes, _lib.stream_ptr(dev),
+        )
+        _lib.check(rc, "jg_ln_partial_bwd")
+
+        grad_x = None
+        if ctx.needs_input_grad[0]:
+            _all_reduce(mean_gxn, "avg", group)
+            _all_reduce(dot, "sum", group)
+            grad_x = torch.empty_like(g)
+            rc = lib.jg_ln_bwd_apply(
+                _lib.ptr(grad_x), _lib.ptr(g), _lib.ptr(x_norm), _lib.ptr(w), _lib.ptr(mean_gxn), _lib.ptr(dot),
+                _lib.ptr(std), rows, cols, n_global, _lib.dtype_code(g.dtype), _lib.stream_ptr(dev),
+            )
+            _lib.check(rc, "jg_ln_bwd_apply")
+            grad_x = grad_x.to(ctx.in_dtype)
+        wdt, bdt = ctx.param_dtypes
+        grad_w = gw.to(wdt) if need_w else None
+        grad_b = gb.to(bdt) if need_b else None
+        return grad_x, grad_w, grad_b, None, None
+
+
+def layer_norm(x, weight, bias, channel_group=None, eps: float = 1e-5) -> torch.Tensor:
+    """``DistributedLayerNorm.forward``'s call: ``_LayerNorm.apply(...)[0]``
+    (jigsaw/modules/normalization/_layer_norm.py:363-368)."""
+    return _LayerNorm.apply(x, weight, bias, channel_group, eps)[0]
+
+
+__all__ = ["_LayerNorm", "layer_norm", "partial_stats"]

@@ -1,0 +1,127 @@
+"""HIP sharded LayerNorm against the oracle and nn.LayerNorm (GPU).
+
+Tolerances: fp32 path atol 1e-5 / rtol 1e-5 (the reference's own test uses 1e-3,
+tests/modules/normalization/test_normalization.py); bf16 path rel-L2 2e-2.
+"""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import rel_l2
+from jigsaw_amd import layernorm as jl
+from oracle import layernorm as ol
+
+pytestmark = pytest.mark.gpu
+
+
+class ShardGroup:
+    """Channel group stand-in on one GPU: holds the other shards' statistics, in the
+    order the forward / backward ask for them."""
+
+    def __init__(self, size, others):
+        self._size = size
+        self.others = list(others)  # per all_reduce call: list of peer tensors
+        self.calls = []
+
+    def size(self):
+        return self._size
+
+    def all_reduce(self, t, op):
+        peers = self.others.pop(0)
+        self.calls.append(op)
+        total = t.clone()
+        for p in peers:
+            total += p.to(t.device, t.dtype)
+        t.copy_(total / self._size if op == "avg" else total)
+
+
+@pytest.mark.parametrize("rows,cols", [((4, 33), 256), ((2, 5, 7), 96), ((1, 4096), 256), ((3,), 1000), ((9,), 130)])
+def test_partial_stats(rows, cols, dev):
+    torch.manual_seed(0)
+    for dtype in (torch.float32, torch.bfloat16):
+        x = (torch.randn(*rows, cols) * 3 + 1.5).to(dtype)
+        m, v = jl.partial_stats(x.to(dev))
+        wm, wv = ol.partial_stats(x.double())
+        torch.testing.assert_close(m.cpu().double(), wm, atol=1e-5, rtol=1e-5)
+        torch.testing.assert_close(v.cpu().double(), wv, atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("G", [1, 2, 4])
+@pytest.mark.parametrize("bias", [True, False])
+def test_layernorm_forward_backward_fp32(G, bias, dev):
+    torch.manual_seed(1)
+    C, eps = 64 * G, 1e-5
+    x = torch.randn(2, 37, C)
+    w = 1 + 0.2 * torch.randn(C)
+    b = 0.2 * torch.randn(C) if bias else None
+    g = torch.randn(2, 37, C)
+    xs, ws, gs = (list(t.chunk(G, -1)) for t in (x, w, g))
+    bs = list(b.chunk(G, -1)) if bias else [None] * G
+    ys, xns, std = ol.forward([t.double() for t in xs], [t.double() for t in ws], [None if t is None else t.double() for t in bs], eps)
+    gxs, gws, gbs = ol.backward([t.double() for t in gs], xns, [t.double() for t in ws], std, has_bias=bias)
+    # full-width torch layer norm agrees with the oracle
+    torch.testing.assert_close(torch.cat(ys, -1), F.layer_norm(x.double(), (C,), w.double(), None if b is None else b.double(), eps), atol=1e-10, rtol=1e-8)
+
+    for r in range(G):
+        peers = [i for i in range(G) if i != r]
+        lm = [ol.partial_stats(xs[i]) for i in range(G)]
+        mean = torch.stack([m for m, _ in lm]).mean(0)
+        others = []
+        if G > 1:
+            others.append([lm[i][0] for i in peers])
+            others.append([lm[i][1] + (lm[i][0] - mean) ** 2 for i in peers])
+            gxn = [gs[i] * ws[i] for i in range(G)]
+            others.append([gxn[i].mean(-1, keepdim=True) for i in peers])
+            others.append([(gxn[i] * xns[i].float()).sum(-1, keepdim=True) for i in peers])
+        grp = ShardGroup(G, others)
+        xr = xs[r].to(dev).requires_grad_()
+        wr = ws[r].to(dev).requires_grad_()
+        br = bs[r].to(dev).requires_grad_() if bias else None
+        y, x_norm, w_out, var_eps = jl._LayerNorm.apply(xr, wr, br, grp, eps)
+        assert y.dtype == torch.float32 and not x_norm.requires_grad
+        torch.testing.assert_close(y.cpu().double(), ys[r], atol=1e-5, rtol=1e-5)
+        torch.testing.assert_close(x_norm.cpu().double(), xns[r], atol=1e-5, rtol=1e-5)
+        torch.testing.assert_close(var_eps.cpu().double(), std**2, atol=1e-6, rtol=1e-5)
+        y.backward(gs[r].to(dev))
+        torch.testing.assert_close(xr.grad.cpu().double(), gxs[r], atol=1e-5, rtol=1e-5)
+        torch.testing.assert_close(wr.grad.cpu().double(), gws[r], atol=1e-4, rtol=1e-5)
+        if bias:
+            torch.testing.assert_close(br.grad.cpu().double(), gbs[r], atol=1e-4, rtol=1e-5)
+        if G > 1:
+            assert grp.calls == ["avg", "avg", "avg", "sum"]
+
+
+def test_layernorm_under_autocast_returns_fp32_and_leaf_dtype_grad(dev):
+    """LayerNorm under autocast computes in fp32 (reference: tests/test_autocast.py:265-292)."""
+    torch.manual_seed(2)
+    C = 256
+    x = torch.randn(4, 128, C).bfloat16()
+    w, b = 1 + 0.2 * torch.randn(C), 0.2 * torch.randn(C)
+    want = F.layer_norm(x.float(), (C,), w, b, 1e-5)
+    xr = x.to(dev).requires_grad_()
+    wr, br = w.to(dev).requires_grad_(), b.to(dev).requires_grad_()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = jl.layer_norm(xr, wr, br, None, 1e-5)
+    assert y.dtype == torch.float32
+    torch.testing.assert_close(y.cpu(), want, atol=1e-4, rtol=1e-4)
+    y.backward(torch.randn_like(y))
+    assert xr.grad.dtype == torch.bfloat16 and wr.grad.dtype == torch.float32
+
+
+def test_layernorm_bf16_config4_shape(dev):
+    """Sharded-channel LayerNorm of config 4: dim 512, 256 local, 4096 tokens."""
+    torch.manual_seed(3)
+    C, G, eps = 512, 2, 1e-5
+    x = torch.randn(1, 4096, C)
+    w, b = 1 + 0.2 * torch.randn(C), 0.2 * torch.randn(C)
+    want = F.layer_norm(x, (C,), w, b, eps)
+    xs, ws, bs = (list(t.chunk(G, -1)) for t in (x, w, b))
+    lm = [ol.partial_stats(t) for t in xs]
+    mean = torch.stack([m for m, _ in lm]).mean(0)
+    for r in range(G):
+        o = 1 - r
+        grp = ShardGroup(G, [[lm[o][0]], [lm[o][1] + (lm[o][0] - mean) ** 2]])
+        y = jl.layer_norm(xs[r].bfloat16().to(dev), ws[r].bfloat16().to(dev), bs[r].bfloat16().to(dev), grp, eps)
+        assert y.dtype == torch.bfloat16
+        assert rel_l2(y, want.chunk(G, -1)[r]) < 2e-2
