@@ -90,7 +90,8 @@ class _LayerNorm(torch.autograd.Function):
             _lib.dtype_code(x.dtype), _lib.dtype_code(cdt), _lib.stream_ptr(x.device),
         )
         _lib.check(rc, "jg_ln_apply")
-        return y, x_norm, w, (var + eps).to(cdt)
+        # an input returned as-is cannot be saved by setup_context: hand out a view
+        return y, x_norm, (w.view_as(w) if w is weight else w), (var + eps).to(cdt)
 
     @staticmethod
     def setup_context(ctx, inputs, output):  # noqa: D102
