@@ -188,6 +188,65 @@ int jg_lse_merge(void* o1, const float* l1, const void* o2, const float* l2,
                  float* l_new, int64_t b, int64_t h, int64_t n, int64_t d, int bshd,
                  int o1_dtype, int o2_dtype, void* stream);
 
+/* ------------------------------------------------------------------------- *
+ * Local convolution on the halo-padded tile (MFMA-bound for bf16 / fp16 with
+ * wide channels, FMA otherwise)
+ *
+ * Layouts are torch's: x (N, Cin, *in), w (Cout, Cin, *kernel), y (N, Cout, *out),
+ * all dense, one dtype per call; accumulation is fp32. A 1-D / 2-D problem fills
+ * the LAST n_spatial entries of the per-axis arrays (leading entries ignored).
+ * `padding` is the LOCAL padding of the call: zero on split axes, whose halo is
+ * already in x (jigsaw/modules/convolution/_common/spatial_split.py:75-82).
+ * out = (in + 2*padding - dilation*(kernel-1) - 1) / stride + 1 per axis.
+ * groups must be 1.
+ *
+ * Workspace: query with jg_conv_workspace_bytes(desc, op, dtype) (op: 0 = fwd,
+ * 1 = dgrad, 2 = wgrad); may be 0, then `workspace` may be NULL. Contents are
+ * scratch; concurrent calls need distinct workspaces.
+ * ------------------------------------------------------------------------- */
+typedef struct {
+  int32_t n_spatial; /* 1, 2 or 3 */
+  int32_t groups;    /* 1 */
+  int64_t batch;
+  int32_t c_in;
+  int32_t c_out;
+  int32_t in_size[3];
+  int32_t kernel[3];
+  int32_t stride[3];
+  int32_t padding[3];
+  int32_t dilation[3];
+} jg_conv_desc;
+
+typedef enum { JG_CONV_FWD = 0, JG_CONV_DGRAD = 1, JG_CONV_WGRAD = 2 } jg_conv_op;
+
+size_t jg_conv_workspace_bytes(const jg_conv_desc* desc, int op, int dtype);
+
+/* y = conv(x, w) + bias  — F.conv{1,2,3}d as called at
+ * jigsaw/modules/convolution/_conv/channel_comm.py:155-158 (table config.py:27).
+ * bias (Cout,) may be NULL. */
+int jg_conv_fwd(void* y, const void* x, const void* w, const void* bias,
+                const jg_conv_desc* desc, int dtype, void* workspace,
+                size_t workspace_bytes, void* stream);
+
+/* gx (N, Cin, *in) = gradient of the PADDED tile — torch.nn.grad.conv*_input as
+ * called at jigsaw/modules/convolution/_conv/distributed.py:346-355. */
+int jg_conv_dgrad(void* gx, const void* w, const void* g, const jg_conv_desc* desc,
+                  int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* gw (Cout, Cin, *kernel) — torch.nn.grad.conv*_weight as called at
+ * jigsaw/modules/convolution/_conv/distributed.py:359-368. Deterministic
+ * (fixed-order two-stage reduction, no atomics). */
+int jg_conv_wgrad(void* gw, const void* x, const void* g, const jg_conv_desc* desc,
+                  int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* gb (C,) = sum of g (N, C, spatial...) over batch and spatial axes —
+ * _sum_grad_bias, jigsaw/modules/convolution/_conv/config.py:117-120.
+ * `spatial` = product of the spatial extents. */
+size_t jg_bias_grad_workspace_bytes(int64_t batch, int64_t channels, int64_t spatial);
+int jg_bias_grad(void* gb, const void* g, int64_t batch, int64_t channels,
+                 int64_t spatial, int dtype, void* workspace, size_t workspace_bytes,
+                 void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -41,6 +41,23 @@ class HaloGeom(ctypes.Structure):
     ]
 
 
+class ConvDesc(ctypes.Structure):
+    """``jg_conv_desc`` of ``include/jigsaw_hip.h``."""
+
+    _fields_ = [
+        ("n_spatial", c_int32),
+        ("groups", c_int32),
+        ("batch", c_int64),
+        ("c_in", c_int32),
+        ("c_out", c_int32),
+        ("in_size", c_int32 * 3),
+        ("kernel", c_int32 * 3),
+        ("stride", c_int32 * 3),
+        ("padding", c_int32 * 3),
+        ("dilation", c_int32 * 3),
+    ]
+
+
 VoidP27 = c_void_p * 27
 VoidP9 = c_void_p * 9
 
@@ -83,6 +100,15 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int,
          c_void_p],
     ),
+    "jg_conv_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int, c_int]),
+    "jg_conv_fwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, POINTER(ConvDesc), c_int, c_void_p, c_size_t, c_void_p],
+    ),
+    "jg_conv_dgrad": (c_int, [c_void_p, c_void_p, c_void_p, POINTER(ConvDesc), c_int, c_void_p, c_size_t, c_void_p]),
+    "jg_conv_wgrad": (c_int, [c_void_p, c_void_p, c_void_p, POINTER(ConvDesc), c_int, c_void_p, c_size_t, c_void_p]),
+    "jg_bias_grad_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
+    "jg_bias_grad": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p]),
     "jg_lse_merge": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int,
@@ -162,6 +188,7 @@ def i64_array(values) -> ctypes.Array:
 
 
 __all__ = [
+    "ConvDesc",
     "HaloGeom",
     "KernelError",
     "LibraryMissing",

@@ -1,0 +1,397 @@
+"""Local convolution and the halo-exchange convolution on the GPU.
+
+Host-side mirror of the callables the reference keeps on ``ConvNdConfig``
+(jigsaw/modules/convolution/_conv/config.py:82-95):
+
+* ``conv_fn`` / ``conv_input_fn`` / ``conv_weight_fn`` / ``grad_bias`` with the
+  signatures of ``F.conv{1,2,3}d``, ``torch.nn.grad.conv*_input``,
+  ``conv*_weight`` and ``_sum_grad_bias``;
+* ``dist_conv_fn`` / ``dist_conv_backward_fn`` with the signatures of
+  ``conv_halo_nway`` / ``conv_halo_nway_backward``
+  (jigsaw/modules/convolution/_conv/distributed.py:212-396);
+* ``_ConvNd`` (jigsaw/modules/convolution/_conv/functional.py:28-169).
+
+The reference pads one split axis at a time through a collective. Here a rank
+packs all its strips once, hands them to ``config.halo_exchange`` (the only part
+that talks to other ranks), and assembles the padded tile in one pass.
+"""
+
+from __future__ import annotations
+
+from collections.abc import Sequence
+from typing import Any, Protocol
+
+import torch
+
+from . import _lib
+from .halo import HaloGeometry, halo_assemble, halo_fold, halo_pack
+
+# --------------------------------------------------------------------------- #
+# local primitives
+# --------------------------------------------------------------------------- #
+
+
+def _tup(v: int | Sequence[int], n: int, name: str) -> tuple:
+    if isinstance(v, int):
+        return (v,) * n
+    v = tuple(int(i) for i in v)
+    if len(v) == 1:
+        return v * n
+    if len(v) != n:
+        raise ValueError(f"{name} must have {n} entries, got {v}")
+    return v
+
+
+def _desc(batch, c_in, c_out, in_spatial, kernel, stride, padding, dilation, groups) -> _lib.ConvDesc:
+    n = len(kernel)
+    d = _lib.ConvDesc()
+    d.n_spatial, d.groups, d.batch, d.c_in, d.c_out = n, groups, batch, c_in, c_out
+    lead = 3 - n
+    for a in range(3):
+        if a < lead:
+            d.in_size[a], d.kernel[a], d.stride[a], d.padding[a], d.dilation[a] = 1, 1, 1, 0, 1
+        else:
+            i = a - lead
+            d.in_size[a], d.kernel[a] = in_spatial[i], kernel[i]
+            d.stride[a], d.padding[a], d.dilation[a] = stride[i], padding[i], dilation[i]
+    return d
+
+
+def _out_spatial(in_spatial, kernel, stride, padding, dilation) -> tuple:
+    out = []
+    for i, k, s, p, d in zip(in_spatial, kernel, stride, padding, dilation):
+        span = i + 2 * p - d * (k - 1) - 1
+        if span < 0:
+            raise RuntimeError(
+                f"Calculated padded input size per channel: ({i + 2 * p}). Kernel size: ({d * (k - 1) + 1}). "
+                "Kernel size can't be greater than actual input size"
+            )
+        out.append(span // s + 1)
+    return tuple(out)
+
+
+def _workspace(desc: _lib.ConvDesc, op: int, dtype: torch.dtype, device) -> tuple[torch.Tensor | None, int]:
+    nbytes = int(_lib.load().jg_conv_workspace_bytes(desc, op, _lib.dtype_code(dtype)))
+    if nbytes == 0:
+        return None, 0
+    return torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes
+
+
+def _check_args(x_like, w, groups, padding):
+    if isinstance(padding, str):
+        raise NotImplementedError(f"string padding ({padding!r}) is not supported; pass per-axis integers")
+    if groups != 1:
+        raise NotImplementedError(f"groups = {groups}: only groups = 1 is covered by the HIP kernels")
+    n = w.dim() - 2
+    if n not in (1, 2, 3):
+        raise ValueError(f"weight must be (Cout, Cin, *kernel) with 1 to 3 spatial axes, got {tuple(w.shape)}")
+    return n
+
+
+def conv_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1) -> torch.Tensor:
+    """``F.conv{1,2,3}d(x, w, b, stride, padding, dilation, groups)`` on the HIP kernels."""
+    _lib.require_gpu(x, w, b)
+    n = _check_args(x, w, groups, padding)
+    if x.dim() != n + 2:
+        raise ValueError(f"expected a batched (N, C, *spatial) input with {n} spatial axes, got {tuple(x.shape)}")
+    if x.dtype != w.dtype or (b is not None and b.dtype != x.dtype):
+        raise RuntimeError(f"Input type ({x.dtype}) and weight / bias type ({w.dtype}) should be the same")
+    if x.shape[1] != w.shape[1]:
+        raise RuntimeError(f"expected input to have {w.shape[1]} channels, but got {x.shape[1]} channels instead")
+    stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
+    x, w = x.contiguous(), w.contiguous()
+    b = None if b is None else b.contiguous()
+    out_sp = _out_spatial(x.shape[2:], w.shape[2:], stride, padding, dilation)
+    y = torch.empty((x.shape[0], w.shape[0], *out_sp), dtype=x.dtype, device=x.device)
+    desc = _desc(x.shape[0], x.shape[1], w.shape[0], x.shape[2:], w.shape[2:], stride, padding, dilation, groups)
+    ws, nbytes = _workspace(desc, 0, x.dtype, x.device)
+    rc = _lib.load().jg_conv_fwd(
+        _lib.ptr(y), _lib.ptr(x), _lib.ptr(w), _lib.ptr(b), desc, _lib.dtype_code(x.dtype), _lib.ptr(ws), nbytes,
+        _lib.stream_ptr(x.device),
+    )
+    _lib.check(rc, "jg_conv_fwd")
+    return y
+
+
+def conv_nd_input(input_shape, w, g, *, stride=1, padding=0, dilation=1, groups=1) -> torch.Tensor:
+    """``torch.nn.grad.conv{1,2,3}d_input(input_shape, w, g, ...)`` on the HIP kernels."""
+    _lib.require_gpu(w, g)
+    n = _check_args(g, w, groups, padding)
+    input_shape = tuple(int(v) for v in input_shape)
+    if len(input_shape) != n + 2:
+        raise ValueError(f"input_shape must have {n + 2} entries, got {input_shape}")
+    if g.dtype != w.dtype:
+        raise RuntimeError(f"grad_output type ({g.dtype}) and weight type ({w.dtype}) should be the same")
+    stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
+    g, w = g.contiguous(), w.contiguous()
+    out_sp = _out_spatial(input_shape[2:], w.shape[2:], stride, padding, dilation)
+    if tuple(g.shape) != (input_shape[0], w.shape[0], *out_sp):
+        raise ValueError(
+            f"grad_output shape {tuple(g.shape)} does not match the convolution of an input of shape {input_shape} "
+            f"(expected {(input_shape[0], w.shape[0], *out_sp)})"
+        )
+    gx = torch.empty(input_shape, dtype=g.dtype, device=g.device)
+    desc = _desc(input_shape[0], input_shape[1], w.shape[0], input_shape[2:], w.shape[2:], stride, padding, dilation, groups)
+    ws, nbytes = _workspace(desc, 1, g.dtype, g.device)
+    rc = _lib.load().jg_conv_dgrad(
+        _lib.ptr(gx), _lib.ptr(w), _lib.ptr(g), desc, _lib.dtype_code(g.dtype), _lib.ptr(ws), nbytes,
+        _lib.stream_ptr(g.device),
+    )
+    _lib.check(rc, "jg_conv_dgrad")
+    return gx
+
+
+def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, groups=1) -> torch.Tensor:
+    """``torch.nn.grad.conv{1,2,3}d_weight(x, weight_shape, g, ...)`` on the HIP kernels."""
+    _lib.require_gpu(x, g)
+    weight_shape = tuple(int(v) for v in weight_shape)
+    n = len(weight_shape) - 2
+    if isinstance(padding, str):
+        raise NotImplementedError(f"string padding ({padding!r}) is not supported; pass per-axis integers")
+    if groups != 1:
+        raise NotImplementedError(f"groups = {groups}: only groups = 1 is covered by the HIP kernels")
+    if x.dtype != g.dtype:
+        raise RuntimeError(f"input type ({x.dtype}) and grad_output type ({g.dtype}) should be the same")
+    stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
+    x, g = x.contiguous(), g.contiguous()
+    out_sp = _out_spatial(x.shape[2:], weight_shape[2:], stride, padding, dilation)
+    if tuple(g.shape) != (x.shape[0], weight_shape[0], *out_sp) or x.shape[1] != weight_shape[1]:
+        raise ValueError(f"grad_output {tuple(g.shape)} / input {tuple(x.shape)} do not match weight {weight_shape}")
+    gw = torch.empty(weight_shape, dtype=x.dtype, device=x.device)
+    desc = _desc(x.shape[0], x.shape[1], weight_shape[0], x.shape[2:], weight_shape[2:], stride, padding, dilation, groups)
+    ws, nbytes = _workspace(desc, 2, x.dtype, x.device)
+    rc = _lib.load().jg_conv_wgrad(
+        _lib.ptr(gw), _lib.ptr(x), _lib.ptr(g), desc, _lib.dtype_code(x.dtype), _lib.ptr(ws), nbytes,
+        _lib.stream_ptr(x.device),
+    )
+    _lib.check(rc, "jg_conv_wgrad")
+    return gw
+
+
+def sum_grad_bias(g: torch.Tensor, n_spatial: int) -> torch.Tensor:
+    """``grad_output.sum`` over batch and spatial axes (config.py:117-120)."""
+    _lib.require_gpu(g)
+    if g.dim() != n_spatial + 2:
+        raise ValueError(f"expected (N, C, *spatial) with {n_spatial} spatial axes, got {tuple(g.shape)}")
+    g = g.contiguous()
+    batch, ch = g.shape[0], g.shape[1]
+    spatial = 1
+    for s in g.shape[2:]:
+        spatial *= int(s)
+    gb = torch.empty(ch, dtype=g.dtype, device=g.device)
+    lib = _lib.load()
+    nbytes = int(lib.jg_bias_grad_workspace_bytes(batch, ch, spatial))
+    ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=g.device)
+    rc = lib.jg_bias_grad(
+        _lib.ptr(gb), _lib.ptr(g), batch, ch, spatial, _lib.dtype_code(g.dtype), _lib.ptr(ws), nbytes,
+        _lib.stream_ptr(g.device),
+    )
+    _lib.check(rc, "jg_bias_grad")
+    return gb
+
+
+# --------------------------------------------------------------------------- #
+# the distributed convolution of one rank
+# --------------------------------------------------------------------------- #
+
+
+class TileGroup:
+    """One axis of the spatial mesh as seen from one rank: ``size()`` and ``rank()``,
+    the two members of a process group the halo geometry needs."""
+
+    def __init__(self, size: int, rank: int) -> None:
+        if not 0 <= rank < size:
+            raise ValueError(f"rank {rank} outside a group of {size}")
+        self._size, self._rank = int(size), int(rank)
+
+    def size(self) -> int:
+        return self._size
+
+    def rank(self) -> int:
+        return self._rank
+
+
+class HaloExchange(Protocol):
+    """What moves strips between ranks. ``send`` maps a neighbour offset to the strip
+    packed for it; the result maps the offset of each existing neighbour to the strip
+    received from it. One implementation per transport; none lives in this module."""
+
+    def forward(self, send: dict) -> dict: ...
+
+    def backward(self, send: dict) -> dict: ...
+
+
+def _mesh_position(spatial_groups) -> tuple[tuple, tuple]:
+    sizes = tuple(1 if g is None else int(g.size()) for g in spatial_groups)
+    ranks = tuple(0 if g is None else int(g.rank()) for g in spatial_groups)
+    return ranks, sizes
+
+
+def _present_offsets(geom: HaloGeometry, ranks, sizes) -> list:
+    out = []
+    for o in geom.offsets():
+        ok = True
+        for a, v in enumerate(o):
+            if v == 0:
+                continue
+            if sizes[a] <= 1 or not 0 <= ranks[a] + v < sizes[a]:
+                ok = False
+        if ok:
+            out.append(o)
+    return out
+
+
+def _local_padding(padding, sizes) -> tuple:
+    """Zero on split axes (jigsaw/modules/convolution/_common/spatial_split.py:75-82)."""
+    return tuple(0 if s > 1 else p for p, s in zip(padding, sizes))
+
+
+def _needs_halo(sizes, padding, dilation) -> bool:
+    return any(s > 1 and (p != 0 or d != 1) for s, p, d in zip(sizes, padding, dilation))
+
+
+def conv_halo_nway(x, w, b, stride, padding, dilation, spatial_groups, channel_group, config):
+    """Convolve with a halo exchange on every split axis; returns ``(y, x_aug)``.
+
+    Same contract as ``conv_halo_nway``
+    (jigsaw/modules/convolution/_conv/distributed.py:212-293) for a channel-local
+    layer: ``x_aug`` is the halo-padded tile kept for the backward pass.
+    """
+    if not isinstance(padding, tuple):
+        raise NotImplementedError(
+            "Distributed ConvNd with a halo exchange does not support "
+            f"string padding ({padding!r}); pass an explicit per-axis padding."
+        )
+    if channel_group is not None and channel_group.size() != 1:
+        raise NotImplementedError("channel-sharded convolution is outside this package (col must be 1)")
+    n = config.n_spatial
+    ranks, sizes = _mesh_position(spatial_groups)
+    x = x.contiguous()
+    geom = HaloGeometry.for_conv(x.shape[-n:], w.shape[-n:], stride, padding, dilation, ranks, sizes)
+    present = _present_offsets(geom, ranks, sizes)
+    send = halo_pack(x, geom, from_padded=False, present=present) if present else {}
+    recv = config.halo_exchange.forward(send) if present else {}
+    x_aug = halo_assemble(x, recv, geom)
+    kwargs = {"stride": stride, "padding": _local_padding(padding, sizes), "dilation": dilation, "groups": 1}
+    y = config.conv_fn(x_aug, w, b, **kwargs) if b is not None else config.conv_fn(x_aug, w, **kwargs)
+    return y, x_aug
+
+
+def conv_halo_nway_backward(
+    grad_output, x_aug, weight, stride, padding, dilation, local_in_spatial, spatial_groups, channel_group, config,
+    need=(True, True),
+):
+    """Gradients of the halo-exchange convolution; returns ``(g_x or None, g_w or None)``.
+
+    Same contract as ``conv_halo_nway_backward``
+    (jigsaw/modules/convolution/_conv/distributed.py:296-396): dgrad on the padded
+    shape, wgrad, then the halo gradients are folded onto their owners.
+    """
+    n = config.n_spatial
+    ranks, sizes = _mesh_position(spatial_groups)
+    local_padding = _local_padding(padding, sizes)
+    need_x, need_w = need
+    g = grad_output.to(weight.dtype)
+    kwargs = {"stride": stride, "padding": local_padding, "dilation": dilation, "groups": 1}
+    g_x_need = config.conv_input_fn(x_aug.shape, weight, g, **kwargs) if need_x else None
+    g_w = config.conv_weight_fn(x_aug, weight.shape, g, **kwargs) if need_w else None
+    if not need_x:
+        return None, g_w
+    geom = HaloGeometry.for_conv(local_in_spatial, weight.shape[-n:], stride, padding, dilation, ranks, sizes)
+    present = _present_offsets(geom, ranks, sizes)
+    send = halo_pack(g_x_need, geom, from_padded=True, present=present) if present else {}
+    recv = config.halo_exchange.backward(send) if present else {}
+    g_x = halo_fold(g_x_need, recv, geom)
+    return g_x, g_w
+
+
+class HipConvNdConfig:
+    """Kernel table of one distributed convolution layer, HIP edition.
+
+    Carries the attributes ``_ConvNd`` and the two ``dist_conv_*`` functions read
+    from the reference's ``ConvNdConfig`` (config.py:62-95): ``n_spatial``,
+    ``conv_fn``, ``conv_input_fn``, ``conv_weight_fn``, ``grad_bias``,
+    ``dist_conv_fn``, ``dist_conv_backward_fn``, plus ``halo_exchange``.
+    """
+
+    vmapped = False
+    channel_local = True
+    groups = 1
+    groups_local = 1
+
+    def __init__(self, n_spatial: int, bias: Any, halo_exchange: HaloExchange | None = None) -> None:
+        self.n_spatial = int(n_spatial)
+        self.halo_exchange = halo_exchange
+        self.conv_fn = conv_nd
+        self.native_conv_fn = conv_nd
+        self.conv_input_fn = conv_nd_input
+        self.conv_weight_fn = conv_nd_weight
+        self.grad_bias = self._no_bias if bias is None else self._sum_grad_bias
+        self.dist_conv_fn = conv_halo_nway
+        self.dist_conv_backward_fn = conv_halo_nway_backward
+
+    def _no_bias(self, *args: Any, **kwargs: Any) -> None:
+        return None
+
+    def _sum_grad_bias(self, grad_output: torch.Tensor) -> torch.Tensor:
+        return sum_grad_bias(grad_output, self.n_spatial)
+
+
+def _cast_to_autocast_dtype(*tensors):
+    """Matmul-family opt-in to autocast: cast down to the autocast dtype
+    (jigsaw/_core/autocast.py:44-66)."""
+    if not torch.is_autocast_enabled():
+        return tensors
+    dt = torch.get_autocast_gpu_dtype()
+    return tuple(t if t is None or not t.is_floating_point() else t.to(dt) for t in tensors)
+
+
+class _ConvNd(torch.autograd.Function):
+    """Autograd function of the distributed convolution
+    (jigsaw/modules/convolution/_conv/functional.py:28-169), HIP kernels inside."""
+
+    @staticmethod
+    def forward(x, weight, bias, stride, padding, dilation, spatial_groups, channel_group, config):  # noqa: D102
+        x, weight, bias = _cast_to_autocast_dtype(x, weight, bias)
+        return config.dist_conv_fn(
+            x, weight, bias, stride=stride, padding=padding, dilation=dilation, spatial_groups=spatial_groups,
+            channel_group=channel_group, config=config,
+        )
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):  # noqa: D102
+        x, weight, bias, stride, padding, dilation, spatial_groups, channel_group, config = inputs
+        _, x_aug = output
+        ctx.mark_non_differentiable(x_aug)
+        ctx.save_for_backward(x_aug, weight)
+        ctx.spatial_groups, ctx.channel_group = spatial_groups, channel_group
+        ctx.local_in_spatial = tuple(x.shape[-config.n_spatial :])
+        ctx.stride, ctx.padding, ctx.dilation, ctx.config = stride, padding, dilation, config
+        ctx.has_bias = bias is not None
+
+    @staticmethod
+    def backward(ctx, grad_output, grad_x_aug):  # noqa: D102
+        x_aug, weight = ctx.saved_tensors
+        config = ctx.config
+        x_aug = x_aug.to(weight.dtype)
+        need_x, need_w, need_b = ctx.needs_input_grad[:3]
+        g_b = config.grad_bias(grad_output.contiguous()) if (need_b and ctx.has_bias) else None
+        g_x, g_w = config.dist_conv_backward_fn(
+            grad_output, x_aug, weight, ctx.stride, ctx.padding, ctx.dilation, ctx.local_in_spatial,
+            ctx.spatial_groups, ctx.channel_group, config, need=(need_x, need_w),
+        )
+        return g_x, g_w, g_b, None, None, None, None, None, None
+
+
+__all__ = [
+    "HaloExchange",
+    "HipConvNdConfig",
+    "TileGroup",
+    "_ConvNd",
+    "conv_halo_nway",
+    "conv_halo_nway_backward",
+    "conv_nd",
+    "conv_nd_input",
+    "conv_nd_weight",
+    "sum_grad_bias",
+]

@@ -1,0 +1,94 @@
+// C entry points of the local convolution: validate, resolve the geometry and
+// route to the implicit-GEMM MFMA kernels when they cover the problem, to the
+// direct kernels otherwise.
+#include "conv_common.h"
+
+namespace jg {
+
+int resolve_conv(const jg_conv_desc* d, const char* who, ConvGeom* out) {
+  JG_REQUIRE(d != nullptr, "%s: desc is NULL", who);
+  JG_REQUIRE(d->n_spatial >= 1 && d->n_spatial <= 3, "%s: n_spatial %d not in 1..3", who,
+             d->n_spatial);
+  if (d->groups != 1) JG_FAIL(JG_ERR_UNSUPPORTED, "%s: groups = %d (only 1)", who, d->groups);
+  JG_REQUIRE(d->batch >= 0 && d->c_in >= 1 && d->c_out >= 1, "%s: bad batch / channels", who);
+  ConvGeom g;
+  g.batch = d->batch;
+  g.cin = d->c_in;
+  g.cout = d->c_out;
+  const int lead = 3 - d->n_spatial;
+  for (int a = 0; a < 3; ++a) {
+    if (a < lead) {
+      g.in[a] = 1; g.k[a] = 1; g.s[a] = 1; g.p[a] = 0; g.d[a] = 1;
+    } else {
+      g.in[a] = d->in_size[a]; g.k[a] = d->kernel[a]; g.s[a] = d->stride[a];
+      g.p[a] = d->padding[a]; g.d[a] = d->dilation[a];
+    }
+    JG_REQUIRE(g.in[a] >= 1 && g.k[a] >= 1 && g.s[a] >= 1 && g.p[a] >= 0 && g.d[a] >= 1,
+               "%s: bad geometry on axis %d (in %d, k %d, s %d, p %d, d %d)", who, a, g.in[a],
+               g.k[a], g.s[a], g.p[a], g.d[a]);
+    const int span = g.in[a] + 2 * g.p[a] - g.d[a] * (g.k[a] - 1) - 1;
+    JG_REQUIRE(span >= 0, "%s: kernel extent exceeds the padded input on axis %d", who, a);
+    g.out[a] = span / g.s[a] + 1;
+  }
+  *out = g;
+  return JG_OK;
+}
+
+}  // namespace jg
+
+namespace {
+bool known(int dt) { return dt == JG_F32 || dt == JG_BF16 || dt == JG_F16; }
+}  // namespace
+
+extern "C" size_t jg_conv_workspace_bytes(const jg_conv_desc* desc, int op, int dtype) {
+  jg::ConvGeom g;
+  if (jg::resolve_conv(desc, "jg_conv_workspace_bytes", &g) != JG_OK) return 0;
+  switch (op) {
+    case JG_CONV_FWD:
+      return jg::mfma_fwd_supported(g, dtype) ? jg::mfma_fwd_workspace(g) : 0;
+    case JG_CONV_DGRAD:
+      return jg::mfma_dgrad_supported(g, dtype) ? jg::mfma_dgrad_workspace(g) : 0;
+    case JG_CONV_WGRAD:
+      return jg::mfma_wgrad_supported(g, dtype) ? jg::mfma_wgrad_workspace(g)
+                                                : jg::direct_wgrad_workspace(g);
+    default:
+      return 0;
+  }
+}
+
+extern "C" int jg_conv_fwd(void* y, const void* x, const void* w, const void* bias,
+                           const jg_conv_desc* desc, int dtype, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+  jg::ConvGeom g;
+  int rc = jg::resolve_conv(desc, "jg_conv_fwd", &g);
+  if (rc) return rc;
+  JG_REQUIRE(y && x && w, "jg_conv_fwd: NULL pointer");
+  JG_REQUIRE(known(dtype), "jg_conv_fwd: unknown dtype %d", dtype);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (jg::mfma_fwd_supported(g, dtype)) return jg::mfma_fwd(y, x, w, bias, g, workspace, workspace_bytes, s);
+  return jg::direct_fwd(y, x, w, bias, g, dtype, s);
+}
+
+extern "C" int jg_conv_dgrad(void* gx, const void* w, const void* go, const jg_conv_desc* desc,
+                             int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  jg::ConvGeom g;
+  int rc = jg::resolve_conv(desc, "jg_conv_dgrad", &g);
+  if (rc) return rc;
+  JG_REQUIRE(gx && w && go, "jg_conv_dgrad: NULL pointer");
+  JG_REQUIRE(known(dtype), "jg_conv_dgrad: unknown dtype %d", dtype);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (jg::mfma_dgrad_supported(g, dtype)) return jg::mfma_dgrad(gx, w, go, g, workspace, workspace_bytes, s);
+  return jg::direct_dgrad(gx, w, go, g, dtype, s);
+}
+
+extern "C" int jg_conv_wgrad(void* gw, const void* x, const void* go, const jg_conv_desc* desc,
+                             int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  jg::ConvGeom g;
+  int rc = jg::resolve_conv(desc, "jg_conv_wgrad", &g);
+  if (rc) return rc;
+  JG_REQUIRE(gw && x && go, "jg_conv_wgrad: NULL pointer");
+  JG_REQUIRE(known(dtype), "jg_conv_wgrad: unknown dtype %d", dtype);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (jg::mfma_wgrad_supported(g, dtype)) return jg::mfma_wgrad(gw, x, go, g, workspace, workspace_bytes, s);
+  return jg::direct_wgrad(gw, x, go, g, dtype, workspace, workspace_bytes, s);
+}

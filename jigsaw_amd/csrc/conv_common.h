@@ -1,0 +1,43 @@
+// Geometry shared by the convolution kernels.
+#pragma once
+#include "jg_common.h"
+
+namespace jg {
+
+// Resolved geometry; 1-D and 2-D problems carry leading axes of extent 1.
+struct ConvGeom {
+  long long batch;
+  int cin, cout;
+  int in[3];   // input spatial extent (the padded tile)
+  int out[3];  // output spatial extent
+  int k[3], s[3], p[3], d[3];
+};
+
+// Validate a jg_conv_desc and resolve it. Returns JG_OK or a negative status.
+int resolve_conv(const jg_conv_desc* desc, const char* who, ConvGeom* out);
+
+// Direct kernels (conv_direct.hip).
+size_t direct_wgrad_workspace(const ConvGeom& g);
+int direct_fwd(void* y, const void* x, const void* w, const void* bias, const ConvGeom& g,
+               int dtype, hipStream_t s);
+int direct_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, int dtype,
+                 hipStream_t s);
+int direct_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, int dtype, void* ws,
+                 size_t ws_bytes, hipStream_t s);
+
+// Implicit-GEMM MFMA kernels (conv_mfma.hip). `*_supported` says whether a
+// geometry / dtype is covered; the workspace queries return bytes.
+bool mfma_fwd_supported(const ConvGeom& g, int dtype);
+bool mfma_dgrad_supported(const ConvGeom& g, int dtype);
+bool mfma_wgrad_supported(const ConvGeom& g, int dtype);
+size_t mfma_fwd_workspace(const ConvGeom& g);
+size_t mfma_dgrad_workspace(const ConvGeom& g);
+size_t mfma_wgrad_workspace(const ConvGeom& g);
+int mfma_fwd(void* y, const void* x, const void* w, const void* bias, const ConvGeom& g,
+             void* ws, size_t ws_bytes, hipStream_t s);
+int mfma_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, void* ws,
+               size_t ws_bytes, hipStream_t s);
+int mfma_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, void* ws,
+               size_t ws_bytes, hipStream_t s);
+
+}  // namespace jg

@@ -1,0 +1,212 @@
+"""HIP convolution kernels against the oracle (torch CPU operators in fp64) (GPU).
+
+Tolerances (rel-L2 of the whole tensor): fp32 tensors 1e-5, bf16 / fp16 tensors 2e-2,
+as the north-star states; the reference's own conv tests use atol/rtol 1e-4 for
+y / dx / db and a looser bound for dw (tests/modules/convolution/conv/test_conv2d_multi_spatial.py:207-233).
+"""
+
+import itertools
+
+import pytest
+import torch
+
+from helpers import conv_geometry, mesh_coords, neighbour, rel_l2
+from jigsaw_amd import conv as jc
+from jigsaw_amd.halo import halo_pack
+from oracle import conv as oc
+from oracle import halo as oh
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+
+PRIM_CASES = [
+    # (N, Cin, Cout, in spatial, kernel, stride, padding, dilation)
+    (2, 3, 16, (18, 18), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (2, 16, 3, (18, 20), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (1, 5, 7, (13, 11), (3, 2), (2, 1), (1, 0), (1, 2)),
+    (2, 4, 4, (9, 9), (1, 1), (1, 1), (0, 0), (1, 1)),
+    (2, 4, 6, (12, 12), (5, 5), (1, 1), (2, 2), (1, 1)),
+    (1, 3, 5, (40,), (3,), (1,), (1,), (1,)),
+    (1, 4, 6, (8, 9, 10), (3, 3, 3), (1, 1, 1), (0, 0, 0), (1, 1, 1)),
+    (2, 3, 4, (7, 8, 9), (3, 1, 2), (1, 2, 1), (1, 0, 1), (1, 1, 1)),
+    (2, 64, 64, (18, 34), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (1, 32, 32, (10, 10, 18), (3, 3, 3), (1, 1, 1), (0, 0, 0), (1, 1, 1)),
+    (1, 64, 64, (20, 70), (3, 3), (1, 1), (1, 1), (1, 1)),
+    (3, 64, 64, (37, 53), (3, 3), (1, 1), (0, 0), (1, 1)),
+]
+
+
+def _pid(c):
+    return "n{}_ci{}_co{}_in{}_k{}_s{}_p{}_d{}".format(c[0], c[1], c[2], *["x".join(map(str, v)) for v in c[3:]])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", PRIM_CASES, ids=_pid)
+def test_conv_primitives_match_oracle(case, dtype, dev):
+    N, cin, cout, insp, k, s, p, d = case
+    torch.manual_seed(0)
+    x = torch.randn(N, cin, *insp).to(dtype)
+    fan_in = cin * int(torch.tensor(k).prod())
+    w = ((torch.rand(cout, cin, *k) * 2 - 1) / fan_in**0.5).to(dtype)
+    b = (torch.randn(cout) * 0.1).to(dtype)
+    xd, wd, bd = x.double(), w.double(), b.double()
+    y_want = oc.forward(xd, wd, bd, s, p, d)
+    g = torch.randn_like(y_want).to(dtype)
+    gd = g.double()
+    gx_want = oc.dgrad(x.shape, wd, gd, s, p, d)
+    gw_want = oc.wgrad(xd, w.shape, gd, s, p, d)
+    gb_want = oc.grad_bias(gd, len(k))
+
+    xg, wg, bg, gg = x.to(dev), w.to(dev), b.to(dev), g.to(dev)
+    y = jc.conv_nd(xg, wg, bg, stride=s, padding=p, dilation=d)
+    assert y.dtype == dtype and y.shape == y_want.shape
+    assert rel_l2(y, y_want) < TOL[dtype], f"fwd rel-L2 {rel_l2(y, y_want):.3e}"
+    y0 = jc.conv_nd(xg, wg, None, stride=s, padding=p, dilation=d)
+    assert rel_l2(y0, oc.forward(xd, wd, None, s, p, d)) < TOL[dtype]
+    gx = jc.conv_nd_input(x.shape, wg, gg, stride=s, padding=p, dilation=d)
+    assert rel_l2(gx, gx_want) < TOL[dtype], f"dgrad rel-L2 {rel_l2(gx, gx_want):.3e}"
+    gw = jc.conv_nd_weight(xg, w.shape, gg, stride=s, padding=p, dilation=d)
+    assert gw.shape == w.shape
+    assert rel_l2(gw, gw_want) < TOL[dtype], f"wgrad rel-L2 {rel_l2(gw, gw_want):.3e}"
+    gb = jc.sum_grad_bias(gg, len(k))
+    assert rel_l2(gb, gb_want) < TOL[dtype], f"bias grad rel-L2 {rel_l2(gb, gb_want):.3e}"
+
+
+def test_conv_argument_errors(dev):
+    x = torch.zeros(1, 4, 8, 8, device=dev)
+    w = torch.zeros(4, 4, 3, 3, device=dev)
+    with pytest.raises(NotImplementedError):
+        jc.conv_nd(x, w, padding="same")
+    with pytest.raises(NotImplementedError):
+        jc.conv_nd(x, w, groups=2)
+    with pytest.raises(RuntimeError):
+        jc.conv_nd(x, w.bfloat16())
+    with pytest.raises(RuntimeError):
+        jc.conv_nd(x[:, :3], w)
+    with pytest.raises(RuntimeError):
+        jc.conv_nd(x.cpu(), w.cpu())
+    with pytest.raises(RuntimeError):
+        jc.conv_nd(x[:, :, :2, :2], w)
+
+
+class TableExchange:
+    """HaloExchange stand-in on one GPU: the strips the neighbours would send are
+    computed beforehand (by packing the neighbours' tensors) and handed over."""
+
+    def __init__(self, fwd, bwd):
+        self.fwd, self.bwd = fwd, bwd
+        self.sent_fwd = self.sent_bwd = None
+
+    def forward(self, send):
+        self.sent_fwd = send
+        return self.fwd
+
+    def backward(self, send):
+        self.sent_bwd = send
+        return self.bwd
+
+
+def _recv_tables(tensors, geoms, mesh, from_padded):
+    """For every rank: offset -> strip received from the neighbour at that offset."""
+    ns = len(mesh)
+    out = {}
+    for c in mesh_coords(mesh):
+        tab = {}
+        for o in itertools.product((-1, 0, 1), repeat=ns):
+            nb = neighbour(c, o, mesh) if any(o) else None
+            if nb is None:
+                continue
+            back = tuple(-v for v in o)
+            tab[o] = halo_pack(tensors[nb], geoms[nb], from_padded=from_padded, present=[back])[back]
+        out[c] = tab
+    return out
+
+
+DIST_CASES = [
+    # mesh, local spatial, N, Cin, Cout, kernel, padding, dtype
+    ((2, 2), (32, 32), 2, 3, 16, (3, 3), (1, 1), torch.float32),
+    ((2, 2), (32, 32), 2, 16, 3, (3, 3), (1, 1), torch.float32),
+    ((3, 3), (8, 12), 1, 4, 5, (5, 3), (2, 1), torch.float32),
+    ((2, 1), (16, 20), 2, 4, 4, (3, 3), (1, 1), torch.float32),
+    ((2, 2), (32, 64), 1, 64, 64, (3, 3), (1, 1), torch.bfloat16),
+    ((2, 2, 2), (8, 8, 16), 1, 32, 32, (3, 3, 3), (1, 1, 1), torch.bfloat16),
+    ((2, 2, 2), (6, 6, 6), 1, 3, 4, (3, 3, 3), (1, 1, 1), torch.float32),
+]
+
+
+@pytest.mark.parametrize("case", DIST_CASES, ids=lambda c: f"mesh{'x'.join(map(str, c[0]))}_{c[3]}to{c[4]}_{str(c[7]).split('.')[-1]}")
+def test_distributed_conv_matches_global_conv(case, dev):
+    """The reference's parity method: every rank's y / dx and the summed dw / db equal
+    the serial conv on the gathered tensor (test_conv2d_multi_spatial.py:73-233)."""
+    mesh, n, N, cin, cout, k, p, dtype = case
+    ns = len(mesh)
+    s, d = (1,) * ns, (1,) * ns
+    torch.manual_seed(0)
+    gshape = tuple(a * b for a, b in zip(n, mesh))
+    X = torch.randn(N, cin, *gshape).to(dtype)
+    fan_in = cin * int(torch.tensor(k).prod())
+    W = ((torch.rand(cout, cin, *k) * 2 - 1) / fan_in**0.5).to(dtype)
+    B = (torch.randn(cout) * 0.1).to(dtype)
+    Xd = X.double().requires_grad_()
+    Wd = W.double().requires_grad_()
+    Bd = B.double().requires_grad_()
+    Y = oc.forward(Xd, Wd, Bd, s, p, d)
+    G = torch.randn_like(Y).to(dtype)
+    Y.backward(G.double())
+
+    tiles = {c: t.to(dev) for c, t in oh.split_global(X, mesh).items()}
+    gtiles = {c: t.to(dev) for c, t in oh.split_global(G, mesh).items()}
+    geoms = {c: conv_geometry(n, mesh, c, k, s, p, d) for c in tiles}
+    fwd_tabs = _recv_tables(tiles, geoms, mesh, from_padded=False)
+    Wg, Bg = W.to(dev), B.to(dev)
+
+    # pass 1: forward of every rank, and the padded dgrad every rank will send from
+    cfgs, outs, leaves, gx_need = {}, {}, {}, {}
+    for c in mesh_coords(mesh):
+        cfgs[c] = jc.HipConvNdConfig(ns, Bg, TableExchange(fwd_tabs[c], None))
+        groups = tuple(jc.TileGroup(mesh[a], c[a]) for a in range(ns))
+        xl = tiles[c].clone().requires_grad_()
+        wl, bl = Wg.clone().requires_grad_(), Bg.clone().requires_grad_()
+        y, x_aug = jc._ConvNd.apply(xl, wl, bl, s, p, d, groups, None, cfgs[c])
+        outs[c], leaves[c] = y, (xl, wl, bl)
+        assert not x_aug.requires_grad
+        lp = oh.local_padding(p, mesh)
+        gx_need[c] = jc.conv_nd_input(x_aug.shape, Wg, gtiles[c], stride=s, padding=lp, dilation=d)
+    bwd_tabs = _recv_tables(gx_need, geoms, mesh, from_padded=True)
+
+    # pass 2: backward of every rank
+    gw_sum = torch.zeros_like(W, dtype=torch.float64)
+    gb_sum = torch.zeros_like(B, dtype=torch.float64)
+    tol = TOL[dtype]
+    for c in mesh_coords(mesh):
+        cfgs[c].halo_exchange.bwd = bwd_tabs[c]
+        outs[c].backward(gtiles[c])
+        xl, wl, bl = leaves[c]
+        sl = (slice(None), slice(None)) + tuple(slice(c[a] * n[a], (c[a] + 1) * n[a]) for a in range(ns))
+        assert rel_l2(outs[c], Y.detach()[sl]) < tol, f"y of rank {c}: {rel_l2(outs[c], Y.detach()[sl]):.3e}"
+        assert rel_l2(xl.grad, Xd.grad[sl]) < tol, f"dx of rank {c}: {rel_l2(xl.grad, Xd.grad[sl]):.3e}"
+        gw_sum += wl.grad.double().cpu()
+        gb_sum += bl.grad.double().cpu()
+    # replicated weights: gradients are summed over the spatial ranks (parallel/_sync.py:33-46)
+    assert rel_l2(gw_sum, Wd.grad) < tol, f"dw: {rel_l2(gw_sum, Wd.grad):.3e}"
+    assert rel_l2(gb_sum, Bd.grad) < tol, f"db: {rel_l2(gb_sum, Bd.grad):.3e}"
+
+
+def test_first_layer_skips_dgrad(dev):
+    """needs_input_grad gating (functional.py:131-148): no input grad -> no dgrad, no fold."""
+    cfg = jc.HipConvNdConfig(2, None, TableExchange({}, {}))
+    x = torch.randn(1, 3, 8, 8, device=dev)
+    w = torch.randn(4, 3, 3, 3, device=dev, requires_grad=True)
+    groups = (jc.TileGroup(1, 0), jc.TileGroup(1, 0))
+    y, _ = jc._ConvNd.apply(x, w, None, (1, 1), (1, 1), (1, 1), groups, None, cfg)
+    y.sum().backward()
+    assert w.grad is not None and cfg.halo_exchange.sent_bwd is None
+
+
+def test_string_padding_is_rejected(dev):
+    cfg = jc.HipConvNdConfig(2, None, TableExchange({}, {}))
+    x = torch.randn(1, 3, 8, 8, device=dev)
+    w = torch.randn(4, 3, 3, 3, device=dev)
+    with pytest.raises(NotImplementedError):
+        jc.conv_halo_nway(x, w, None, (1, 1), "same", (1, 1), (None, None), None, cfg)
