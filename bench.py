@@ -1,0 +1,267 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-rank hot path on one MI355X.
+
+One "step" is one pass of the halo-exchange convolution of BASELINE.json's
+configuration 2 for one rank: pack the 8 strips, assemble the padded tile from
+the (seeded, locally held) neighbour strips, convolution forward, then bias
+gradient, dgrad on the padded shape, wgrad, pack of the halo gradients and fold
+of the neighbours' halo gradients. All inputs are resident in HBM before the
+timed region. ``value`` is the convolution's algorithmic FLOPs (fwd + dgrad +
+wgrad) divided by the whole step time, halo movement included.
+
+Prints ONE JSON line (see the keys below). ``--gpus`` above 1 is refused: this
+build runs one rank's share on one GPU and has no collectives.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
+
+METRIC = "halo-conv fwd+bwd & ring-attn step TFLOP/s on 1 GPU; % MFMA peak; halo GB/s"
+
+# HBM bytes per launch of the forward conv kernel (FETCH_SIZE + WRITE_SIZE from
+# rocprofv3 --pmc, scaled by a copy kernel of known size); None until measured.
+CONV_FWD_TRAFFIC_BYTES = None
+
+
+def _events():
+    return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+
+def time_gpu(fn, iters: int, warmup: int = 2) -> float:
+    """Average milliseconds per call, HIP events on the stream the kernels run on
+    (the library launches on torch's current stream)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = _events()
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def build_conv2_workload(dev, batch=8, ch=64, tile=1024):
+    """Configuration 2: one rank's 1024x1024 tile of a 2048x2048 domain, batch 8,
+    64 -> 64 channels, 3x3, pad 1; bf16 N(0,1) activations, Kaiming-uniform weights.
+    The 8 neighbour strips (width 1) are seeded stand-ins for the neighbours' edges."""
+    from jigsaw_amd.halo import HaloGeometry
+
+    g = torch.Generator(device=dev).manual_seed(0)
+    geom = HaloGeometry((tile, tile), (1, 1), (1, 1))
+    lead = (batch, ch)
+    x = torch.randn(*lead, tile, tile, device=dev, generator=g).bfloat16()
+    bound = 1.0 / (ch * 9) ** 0.5
+    w = ((torch.rand(ch, ch, 3, 3, device=dev, generator=g) * 2 - 1) * bound).bfloat16()
+    b = ((torch.rand(ch, device=dev, generator=g) * 2 - 1) * bound).bfloat16()
+    gout = torch.randn(*lead, tile, tile, device=dev, generator=g).bfloat16()
+    strips_fwd = {
+        o: torch.randn(*lead, *geom.strip_extent(o, "assemble"), device=dev, generator=g).bfloat16()
+        for o in geom.offsets()
+    }
+    strips_bwd = {
+        o: torch.randn(*lead, *geom.strip_extent(o, "fold"), device=dev, generator=g).bfloat16()
+        for o in geom.offsets()
+    }
+    return {"geom": geom, "x": x, "w": w, "b": b, "g": gout, "strips_fwd": strips_fwd, "strips_bwd": strips_bwd}
+
+
+def conv_step(wl):
+    """The hot path of one rank for one batch (see the module docstring)."""
+    from jigsaw_amd import conv as jc
+    from jigsaw_amd.halo import halo_assemble, halo_fold, halo_pack
+
+    geom, x, w, b, g = wl["geom"], wl["x"], wl["w"], wl["b"], wl["g"]
+    halo_pack(x, geom, from_padded=False)  # strips this rank sends
+    x_aug = halo_assemble(x, wl["strips_fwd"], geom)
+    y = jc.conv_nd(x_aug, w, b)
+    gb = jc.sum_grad_bias(g, 2)
+    gx_aug = jc.conv_nd_input(x_aug.shape, w, g)
+    gw = jc.conv_nd_weight(x_aug, w.shape, g)
+    halo_pack(gx_aug, geom, from_padded=True)  # halo gradients this rank sends
+    gx = halo_fold(gx_aug, wl["strips_bwd"], geom)
+    return y, gx, gw, gb
+
+
+def cpu_baseline(seconds_budget: float = 30.0) -> dict:
+    """The oracle (the reference's torch CPU operators) timed on the host cores on a
+    bounded sample of the same workload: batch 1 of a 512x512, 64 -> 64 tile in fp32
+    (1/32 of the step's FLOPs), rank (0, 0) of a 2x2 mesh."""
+    from oracle import conv as oc
+    from oracle import halo as oh
+
+    cores = torch.get_num_threads()
+    batch, ch, tile = 1, 64, 512
+    torch.manual_seed(0)
+    # a 2x2 mesh so that the oracle's exchange-by-axis code runs; rank (0, 0) is timed
+    mesh, k, s, p, d = (2, 2), (3, 3), (1, 1), (1, 1), (1, 1)
+    glob = torch.randn(batch, ch, 2 * tile, 2 * tile)
+    w = (torch.rand(ch, ch, 3, 3) * 2 - 1) / 24
+    b = (torch.rand(ch) * 2 - 1) / 24
+    gout = torch.randn(batch, ch, tile, tile)
+    tiles = oh.split_global(glob, mesh)
+
+    def step():
+        aug = oh.gather_mesh(tiles, mesh, k, s, p, d)
+        lp = oh.local_padding(p, mesh)
+        y = oc.forward(aug[(0, 0)], w, b, s, lp, d)
+        gb = oc.grad_bias(gout, 2)
+        gx_aug = {c: oc.dgrad(aug[c].shape, w, gout, s, lp, d) if c == (0, 0) else torch.zeros_like(aug[c]) for c in aug}
+        gw = oc.wgrad(aug[(0, 0)], w.shape, gout, s, lp, d)
+        gx = oh.scatter_add_mesh(gx_aug, mesh, k, s, p, d, (tile, tile))
+        return y, gx, gw, gb
+
+    step()  # warm-up (thread pools, oneDNN primitive cache)
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        step()
+        reps += 1
+        if time.perf_counter() - t0 > seconds_budget / 3 or reps >= 3:
+            break
+    sec = (time.perf_counter() - t0) / reps
+    flop = 3 * 2 * batch * ch * ch * 9 * tile * tile
+    return {
+        "value": flop / sec / 1e12,
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"oracle halo gather + conv fwd/dgrad/wgrad/bias-grad + scatter-add, fp32, batch {batch} of a "
+        f"{tile}x{tile} 64->64 tile ({flop / 1e9:.1f} GFLOP of the step's 1855 GFLOP), {reps} reps, "
+        f"torch {torch.__version__} CPU, {cores} threads of {os.cpu_count()} logical cores",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
+    ns = ap.parse_args()
+    if ns.gpus != 1:
+        print(
+            "bench.py: this build runs one rank's share on ONE GPU and has no collectives; "
+            f"--gpus {ns.gpus} is not supported (use --gpus 1).",
+            file=sys.stderr,
+        )
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP kernels have no CPU fallback.", file=sys.stderr)
+        return 2
+
+    import jigsaw_amd
+    from jigsaw_amd import conv as jc
+    from jigsaw_amd.halo import halo_assemble, halo_fold
+
+    jigsaw_amd.load()  # fail loudly if the library is not built
+    dev = torch.device("cuda:0")
+    wl = build_conv2_workload(dev)
+    batch, ch, tile = wl["x"].shape[0], wl["x"].shape[1], wl["x"].shape[-1]
+    flop_one = 2 * batch * ch * ch * 9 * tile * tile  # fwd = dgrad = wgrad
+    flop_step = 3 * flop_one
+
+    # ---- the timed region: W warm-up steps, then exactly K steps
+    for _ in range(ns.warmup):
+        conv_step(wl)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0, e1 = _events()
+    e0.record()
+    for _ in range(ns.steps):
+        conv_step(wl)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / ns.steps
+    ms_per_step = e0.elapsed_time(e1) / ns.steps
+    ms_per_step = max(ms_per_step, wall_ms)  # host-side gaps count too
+    value = flop_step / (ms_per_step * 1e-3) / 1e12
+
+    # ---- per-kernel figures (HIP events around repeated launches of one operator)
+    geom = wl["geom"]
+    x_aug = halo_assemble(wl["x"], wl["strips_fwd"], geom)
+    gx_aug = jc.conv_nd_input(x_aug.shape, wl["w"], wl["g"])
+    it = max(5, ns.steps)
+    ms_fwd = time_gpu(lambda: jc.conv_nd(x_aug, wl["w"], wl["b"]), it)
+    ms_dgrad = time_gpu(lambda: jc.conv_nd_input(x_aug.shape, wl["w"], wl["g"]), it)
+    ms_wgrad = time_gpu(lambda: jc.conv_nd_weight(x_aug, wl["w"].shape, wl["g"]), it)
+    ms_asm = time_gpu(lambda: halo_assemble(wl["x"], wl["strips_fwd"], geom), it)
+    ms_fold = time_gpu(lambda: halo_fold(gx_aug, wl["strips_bwd"], geom), it)
+    es = wl["x"].element_size()
+    strip_bytes = sum(t.numel() for t in wl["strips_fwd"].values()) * es
+    halo_bytes = (wl["x"].numel() + x_aug.numel()) * es + strip_bytes  # read tile + strips, write padded tile
+    tf = lambda ms: flop_one / (ms * 1e-3) / 1e12  # noqa: E731
+    gbps = lambda ms: halo_bytes / (ms * 1e-3) / 1e9  # noqa: E731
+
+    roofline = {
+        "kernel": "conv3x3_mfma_kernel (forward, config 2)",
+        "bound": "mfma",
+        "achieved": tf(ms_fwd),
+        "peak": PEAK_BF16_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": tf(ms_fwd) / PEAK_BF16_TFLOPS,
+        "traffic": CONV_FWD_TRAFFIC_BYTES,
+    }
+    extra = {
+        "conv_fwd": {"ms": ms_fwd, "tflops": tf(ms_fwd), "frac_mfma_peak": tf(ms_fwd) / PEAK_BF16_TFLOPS},
+        "conv_dgrad": {"ms": ms_dgrad, "tflops": tf(ms_dgrad), "frac_mfma_peak": tf(ms_dgrad) / PEAK_BF16_TFLOPS},
+        "conv_wgrad": {"ms": ms_wgrad, "tflops": tf(ms_wgrad), "frac_mfma_peak": tf(ms_wgrad) / PEAK_BF16_TFLOPS},
+        "conv_fwd_bwd_kernels_only": {
+            "ms": ms_fwd + ms_dgrad + ms_wgrad,
+            "tflops": flop_step / ((ms_fwd + ms_dgrad + ms_wgrad) * 1e-3) / 1e12,
+            "frac_mfma_peak": flop_step / ((ms_fwd + ms_dgrad + ms_wgrad) * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+        },
+        "halo_assemble": {"ms": ms_asm, "GBps": gbps(ms_asm), "frac_hbm_peak": gbps(ms_asm) / PEAK_HBM_GBPS, "bytes": halo_bytes},
+        "halo_fold": {"ms": ms_fold, "GBps": gbps(ms_fold), "frac_hbm_peak": gbps(ms_fold) / PEAK_HBM_GBPS, "bytes": halo_bytes},
+    }
+    try:
+        from _bench_attention import attention_figures  # optional: ring-attention step figures
+
+        extra.update(attention_figures(dev, it))
+    except ImportError:
+        pass
+
+    line = {
+        "metric": METRIC,
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": ns.steps,
+        "warmup": ns.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "config 2: one rank's 1024x1024 tile of a 2048x2048 domain, batch 8, 64->64 ch, 3x3, pad 1; "
+            "halo pack + assemble + conv fwd + bias-grad + dgrad + wgrad + halo pack + fold",
+            "flop_per_step": flop_step,
+            "frac_mfma_peak": value / PEAK_BF16_TFLOPS,
+        },
+        "roofline": roofline,
+        "cpu_baseline": None if ns.no_cpu_baseline else cpu_baseline(),
+        "extra": extra,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -408,11 +408,9 @@ bool mfma_dgrad_supported(const ConvGeom& g, int dtype) {
   if (g.p[1] > KH - 1 || g.p[2] > KW - 1) return false;
   return shape_ok(g.cout, g.cin, g);
 }
-bool mfma_wgrad_supported(const ConvGeom&, int) { return false; }
 
 size_t mfma_fwd_workspace(const ConvGeom& g) { return prep_bytes(g.cin, g.cout); }
 size_t mfma_dgrad_workspace(const ConvGeom& g) { return prep_bytes(g.cout, g.cin); }
-size_t mfma_wgrad_workspace(const ConvGeom&) { return 0; }
 
 int mfma_fwd(void* y, const void* x, const void* w, const void* bias, const ConvGeom& g, void* ws,
              size_t ws_bytes, hipStream_t s) {
@@ -429,10 +427,6 @@ int mfma_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, void*
                      static_cast<uint16_t*>(gx), (int)g.batch, g.cout, g.cin, g.out[1], g.out[2],
                      g.in[1], g.in[2], KH - 1 - g.p[1], KW - 1 - g.p[2], 1, ws, ws_bytes, s,
                      "jg_conv_dgrad(mfma)");
-}
-
-int mfma_wgrad(void*, const void*, const void*, const ConvGeom&, void*, size_t, hipStream_t) {
-  JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_wgrad(mfma): not available");
 }
 
 }  // namespace jg

@@ -80,22 +80,34 @@ __device__ __forceinline__ void region(int x, int lo, int n, int hi, int& r, int
   }
 }
 
+// The neighbour table is the FIRST parameter of every kernel that looks it up
+// with a per-lane index: it is then read straight from the kernel-argument
+// segment (constant memory, offset 0) instead of being copied to scratch.
+__device__ __forceinline__ const void* table_entry(int idx) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const void* const* kt = (const void* const*)__builtin_amdgcn_kernarg_segment_ptr();
+  return kt[idx];
+#else  // host pass of hipcc: never called
+  (void)idx;
+  return nullptr;
+#endif
+}
+
 // ------------------------------------------------------------------ assemble
 template <typename T>
-__device__ __forceinline__ T assemble_fetch(const Table& tab, const Geom& g, long long p,
-                                            int da, int ha, int wa) {
+__device__ __forceinline__ T assemble_fetch(const Geom& g, long long p, int da, int ha, int wa) {
   int rd, cd, ed, rh, ch, eh, rw, cw, ew;
   region(da, g.lo[0], g.n[0], g.hi[0], rd, cd, ed);
   region(ha, g.lo[1], g.n[1], g.hi[1], rh, ch, eh);
   region(wa, g.lo[2], g.n[2], g.hi[2], rw, cw, ew);
-  const T* s = static_cast<const T*>(tab.p[rd * 9 + rh * 3 + rw]);
+  const T* s = static_cast<const T*>(table_entry(rd * 9 + rh * 3 + rw));
   if (s == nullptr) return T(0);
   long long off = ((p * ed + cd) * eh + ch) * (long long)ew + cw;
   return s[off];
 }
 
 template <typename T, typename I>
-__global__ __launch_bounds__(256) void assemble_kernel(T* __restrict__ dst, Table tab,
+__global__ __launch_bounds__(256) void assemble_kernel(Table tab, T* __restrict__ dst,
                                                        Geom g, I total) {
   constexpr int V = Bits<T>::V;
   const I nvec = (total + V - 1) / V;
@@ -124,7 +136,7 @@ __global__ __launch_bounds__(256) void assemble_kernel(T* __restrict__ dst, Tabl
       int rd, cd, ed, rh, ch, eh;
       region(da, g.lo[0], g.n[0], g.hi[0], rd, cd, ed);
       region(ha, g.lo[1], g.n[1], g.hi[1], rh, ch, eh);
-      const T* s = static_cast<const T*>(tab.p[rd * 9 + rh * 3 + rw]);
+      const T* s = static_cast<const T*>(table_entry(rd * 9 + rh * 3 + rw));
       u32x4 val = {0u, 0u, 0u, 0u};
       if (s != nullptr) {
         long long off = ((p * ed + cd) * eh + ch) * (long long)ew + cw;
@@ -136,7 +148,7 @@ __global__ __launch_bounds__(256) void assemble_kernel(T* __restrict__ dst, Tabl
 #pragma unroll
       for (int i = 0; i < V; ++i) {
         tmp[i] = T(0);
-        if (e0 + i < total) tmp[i] = assemble_fetch<T>(tab, g, p, da, ha, wa);
+        if (e0 + i < total) tmp[i] = assemble_fetch<T>(g, p, da, ha, wa);
         if (++wa == Wa) {
           wa = 0;
           if (++ha == Ha) {
@@ -425,18 +437,18 @@ extern "C" int jg_halo_assemble_3d(void* x_aug, const void* const src[27],
     int grid = grid_for((total + 7) / 8);
     if (wide)
       assemble_kernel<uint16_t, unsigned long long><<<grid, 256, 0, s>>>(
-          static_cast<uint16_t*>(x_aug), tab, g, total);
+          tab, static_cast<uint16_t*>(x_aug), g, total);
     else
       assemble_kernel<uint16_t, uint32_t><<<grid, 256, 0, s>>>(
-          static_cast<uint16_t*>(x_aug), tab, g, (uint32_t)total);
+          tab, static_cast<uint16_t*>(x_aug), g, (uint32_t)total);
   } else {
     int grid = grid_for((total + 3) / 4);
     if (wide)
       assemble_kernel<uint32_t, unsigned long long><<<grid, 256, 0, s>>>(
-          static_cast<uint32_t*>(x_aug), tab, g, total);
+          tab, static_cast<uint32_t*>(x_aug), g, total);
     else
       assemble_kernel<uint32_t, uint32_t><<<grid, 256, 0, s>>>(
-          static_cast<uint32_t*>(x_aug), tab, g, (uint32_t)total);
+          tab, static_cast<uint32_t*>(x_aug), g, (uint32_t)total);
   }
   JG_CHECK_LAUNCH("jg_halo_assemble_3d");
   return JG_OK;
