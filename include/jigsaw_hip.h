@@ -247,6 +247,45 @@ int jg_bias_grad(void* gb, const void* g, int64_t batch, int64_t channels,
                  int64_t spatial, int dtype, void* workspace, size_t workspace_bytes,
                  void* stream);
 
+/* ------------------------------------------------------------------------- *
+ * Attention core of the ring step (MFMA-bound for bf16, head size 64)
+ *
+ * q (batch, sq, d), k / v (batch, sk, d), dense, `batch` = all leading axes
+ * flattened (b*h for the "bhsd" layout of jigsaw's sdpa / math cores). One dtype
+ * per call; softmax and accumulation in fp32. Non-causal, no dropout.
+ * `bias` (optional, fp32): additive score bias / mask of shape
+ * (bias_period, sq, sk); batch entry i uses bias[i % bias_period]
+ * (windowed attention with a relative-position bias, examples/swin.py:146-151).
+ * ------------------------------------------------------------------------- */
+
+/* out = softmax(scale * q k^T + bias) v, lse = natural-log sum-exp of the scaled
+ * scores, (batch, sq) fp32 — cores/math.forward
+ * (jigsaw/modules/attention/_functional/cores/math.py:31-78) and the contract of
+ * cores/__init__.py:1-15.
+ * Fused ring merge: when out_acc (fp32, shape of out) and lse_acc (fp32,
+ * (batch, sq)) are given, this chunk's result is merged into them in place,
+ *   w = sigmoid(lse - lse_acc); out_acc += w*(out - out_acc); lse_acc = logaddexp,
+ * which is _online_softmax_merge_ (forward.py:23-61) without the round trip of
+ * out_j through HBM; `out` / `lse` may then be NULL. */
+int jg_attn_fwd(void* out, float* lse, const void* q, const void* k, const void* v,
+                int64_t batch, int64_t sq, int64_t sk, int64_t d, float scale,
+                const float* bias, int64_t bias_period, float* out_acc,
+                float* lse_acc, int dtype, void* stream);
+
+/* (dq, dk, dv) of one chunk from the GLOBAL out / lse of the ring
+ * (cores/math.backward, cores/math.py:81-149): p = exp(scale*q k^T + bias - lse),
+ * delta = rowsum(dout*out), ds = p*(dout v^T - delta)*scale, dq = ds k,
+ * dk = ds^T q, dv = p^T dout. dq/dk/dv have the dtype of the inputs.
+ * dbias (optional, fp32, (batch, sq, sk)) receives p*(dout v^T - delta), the
+ * gradient of the additive bias per batch entry.
+ * workspace: jg_attn_bwd_workspace_bytes(batch, sq, sk, d) bytes of scratch. */
+size_t jg_attn_bwd_workspace_bytes(int64_t batch, int64_t sq, int64_t sk, int64_t d);
+int jg_attn_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q,
+                const void* k, const void* v, const void* out, const float* lse,
+                int64_t batch, int64_t sq, int64_t sk, int64_t d, float scale,
+                const float* bias, int64_t bias_period, float* dbias, int dtype,
+                void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

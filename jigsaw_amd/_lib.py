@@ -109,6 +109,17 @@ SIGNATURES: dict[str, tuple] = {
     "jg_conv_wgrad": (c_int, [c_void_p, c_void_p, c_void_p, POINTER(ConvDesc), c_int, c_void_p, c_size_t, c_void_p]),
     "jg_bias_grad_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "jg_bias_grad": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p]),
+    "jg_attn_fwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float, c_void_p,
+         c_int64, c_void_p, c_void_p, c_int, c_void_p],
+    ),
+    "jg_attn_bwd_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
+    "jg_attn_bwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+         c_int64, c_int64, c_float, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_size_t, c_void_p],
+    ),
     "jg_lse_merge": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int,

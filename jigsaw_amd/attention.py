@@ -1,11 +1,24 @@
 """Ring-attention step on the GPU: attention core, log-sum-exp merge, ring loops.
 
-Host-side mirror of the attention-core contract
-(jigsaw/modules/attention/_functional/cores/__init__.py:1-15) and of the fused
-merge hook (jigsaw/modules/attention/_functional/_merge_kernel.py:88-172).
+Host-side mirror of
+
+* the attention-core contract ``forward(q, k, v, scale, dropout_p, seed=None, *,
+  layout) -> (out, logsumexp, rng_state)`` and ``backward(grad_out, q, k, v, out,
+  logsumexp, scale, *extra, ...) -> (dq, dk, dv)``
+  (jigsaw/modules/attention/_functional/cores/__init__.py:1-15), i.e. what
+  ``RingAttentionConfig.attn_core_forward_fn / attn_core_backward_fn`` hold
+  (jigsaw/modules/attention/_config.py:459-464);
+* the fused merge hook ``fused_online_softmax_merge_``
+  (jigsaw/modules/attention/_functional/_merge_kernel.py:88-172);
+* the per-rank loops of ``ring_forward`` / ``ring_backward``
+  (jigsaw/modules/attention/_functional/forward.py:160-199, backward.py:176-270)
+  over K/V chunks that are already local. Circulating the chunks between ranks is
+  outside this module.
 """
 
 from __future__ import annotations
+
+from collections.abc import Sequence
 
 import torch
 
@@ -14,6 +27,9 @@ from . import _lib
 _SUPPORTED_O = (torch.float16, torch.bfloat16, torch.float32)
 
 
+# --------------------------------------------------------------------------- #
+# merge hook
+# --------------------------------------------------------------------------- #
 def fused_online_softmax_merge_(o1, l1, o2, l2, layout):
     """HIP stand-in for the Triton merge: mutates ``o1``, returns ``(o1, l_new)``.
 
@@ -49,4 +65,210 @@ def fused_online_softmax_merge_(o1, l1, o2, l2, layout):
     return o1, l_new
 
 
-__all__ = ["fused_online_softmax_merge_"]
+# --------------------------------------------------------------------------- #
+# attention core
+# --------------------------------------------------------------------------- #
+def _flat(t: torch.Tensor) -> tuple[int, int, int]:
+    if t.dim() < 3:
+        raise ValueError(f"expected (..., s, d), got shape {tuple(t.shape)}")
+    batch = 1
+    for s in t.shape[:-2]:
+        batch *= int(s)
+    return batch, int(t.shape[-2]), int(t.shape[-1])
+
+
+def _check_qkv(q, k, v):
+    _lib.require_gpu(q, k, v)
+    if not (q.dtype == k.dtype == v.dtype):
+        raise RuntimeError(f"q, k, v must share a dtype, got {q.dtype}, {k.dtype}, {v.dtype}")
+    if k.shape != v.shape or q.shape[:-2] != k.shape[:-2] or q.shape[-1] != k.shape[-1]:
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
+
+
+def _bias_args(bias, batch, sq, sk):
+    if bias is None:
+        return None, 0
+    bias = bias.to(torch.float32).contiguous()
+    if bias.dim() < 2 or tuple(bias.shape[-2:]) != (sq, sk):
+        raise ValueError(f"bias must end in ({sq}, {sk}), got {tuple(bias.shape)}")
+    period = bias.numel() // (sq * sk)
+    if period == 0 or batch % period:
+        raise ValueError(f"bias with {period} matrices does not tile a batch of {batch}")
+    return bias, period
+
+
+def core_forward(q, k, v, scale, bias=None, out_acc=None, lse_acc=None, want_out=True):
+    """One attention core call; optionally merges into ``(out_acc, lse_acc)`` in place.
+
+    Returns ``(out, lse)`` (``None`` each when ``want_out`` is false).
+    """
+    _check_qkv(q, k, v)
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    batch, sq, d = _flat(q)
+    sk = int(k.shape[-2])
+    bias_t, period = _bias_args(bias, batch, sq, sk)
+    out = torch.empty_like(q) if want_out else None
+    lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device) if want_out else None
+    rc = _lib.load().jg_attn_fwd(
+        _lib.ptr(out), _lib.ptr(lse), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), batch, sq, sk, d, float(scale),
+        _lib.ptr(bias_t), period, _lib.ptr(out_acc), _lib.ptr(lse_acc), _lib.dtype_code(q.dtype),
+        _lib.stream_ptr(q.device),
+    )
+    _lib.check(rc, "jg_attn_fwd")
+    return out, lse
+
+
+def forward(q, k, v, scale=0.0, dropout_p=0.0, seed=None, *, layout="bhsd"):
+    """Attention core forward with the reference's signature
+    (cores/math.py:31-78, cores/sdpa.py:17-85): ``(out, logsumexp, rng_state)``."""
+    if layout != "bhsd":
+        raise NotImplementedError(f"the HIP core is bhsd-only; got layout={layout!r}")
+    if dropout_p != 0.0:
+        raise NotImplementedError("attention dropout is not supported by the HIP core")
+    scale = scale or (q.size(-1) ** -0.5)
+    out, lse = core_forward(q, k, v, scale)
+    return out, lse, None
+
+
+def core_backward(grad_out, q, k, v, out, logsumexp, scale, bias=None, want_dbias=False):
+    """``(dq, dk, dv[, dbias])`` of one chunk from the global ``out`` / ``logsumexp``."""
+    _check_qkv(q, k, v)
+    _lib.require_gpu(grad_out, out, logsumexp)
+    dt = q.dtype
+    grad_out, out = grad_out.to(dt).contiguous(), out.to(dt).contiguous()
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    lse = logsumexp.to(torch.float32).contiguous()
+    batch, sq, d = _flat(q)
+    sk = int(k.shape[-2])
+    bias_t, period = _bias_args(bias, batch, sq, sk)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dbias = torch.empty(q.shape[:-1] + (sk,), dtype=torch.float32, device=q.device) if want_dbias else None
+    lib = _lib.load()
+    nbytes = int(lib.jg_attn_bwd_workspace_bytes(batch, sq, sk, d))
+    ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=q.device)
+    rc = lib.jg_attn_bwd(
+        _lib.ptr(dq), _lib.ptr(dk), _lib.ptr(dv), _lib.ptr(grad_out), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v),
+        _lib.ptr(out), _lib.ptr(lse), batch, sq, sk, d, float(scale), _lib.ptr(bias_t), period, _lib.ptr(dbias),
+        _lib.dtype_code(dt), _lib.ptr(ws), nbytes, _lib.stream_ptr(q.device),
+    )
+    _lib.check(rc, "jg_attn_bwd")
+    if want_dbias:
+        return dq, dk, dv, dbias
+    return dq, dk, dv
+
+
+def backward(grad_out, q, k, v, out, logsumexp, scale, *args, dropout_p=0.0, seed=None, rng_state=None,
+             layout="bhsd", **kwargs):
+    """Attention core backward with the reference's signature
+    (cores/math.py:81-149, cores/sdpa.py:88-165): ``(dq, dk, dv)`` in ``grad_out.dtype``."""
+    if layout != "bhsd":
+        raise NotImplementedError(f"the HIP core is bhsd-only; got layout={layout!r}")
+    if dropout_p != 0.0:
+        raise NotImplementedError("attention dropout is not supported by the HIP core")
+    dq, dk, dv = core_backward(grad_out, q, k, v, out, logsumexp, scale)
+    gd = grad_out.dtype
+    return dq.to(gd), dk.to(gd), dv.to(gd)
+
+
+# --------------------------------------------------------------------------- #
+# per-rank ring loops over local chunks
+# --------------------------------------------------------------------------- #
+def _fused_ok(q, k) -> bool:
+    return (
+        q.dtype == torch.bfloat16 and q.shape[-1] == 64 and q.shape[-2] % 128 == 0 and k.shape[-2] % 128 == 0
+    )
+
+
+def attend_step_(q, kj, vj, scale, out, lse):
+    """One ring step: attend chunk ``(kj, vj)`` and merge into the running fp32
+    ``(out, lse)`` in place (``_attend_step``, forward.py:64-96). Uses the fused
+    kernel when it covers the shape, the core + merge kernels otherwise."""
+    kj, vj = kj.contiguous(), vj.contiguous()
+    if _fused_ok(q, kj) and out.dtype == torch.float32 and out.is_contiguous() and lse.is_contiguous():
+        core_forward(q, kj, vj, scale, out_acc=out, lse_acc=lse, want_out=False)
+        return out, lse
+    out_j, l_j = core_forward(q, kj, vj, scale)
+    fused = fused_online_softmax_merge_(out, lse, out_j, l_j, "bhsd")
+    if fused is None:
+        raise NotImplementedError("merge of these dtypes / layouts is not covered by the HIP kernel")
+    return fused
+
+
+def ring_forward(q, k_chunks: Sequence[torch.Tensor], v_chunks: Sequence[torch.Tensor], scale, rank: int = 0):
+    """``(out, lse)`` of one rank's queries over all P chunks, visited in ring order
+    ``(rank + step) % P`` (forward_chunk_provider.py:190-192). The accumulator is
+    fp32 and cast to ``q.dtype`` once at the end (forward.py:160-167, 199)."""
+    P = len(k_chunks)
+    acc = torch.promote_types(q.dtype, torch.float32)
+    out = torch.zeros(q.shape, device=q.device, dtype=acc)
+    lse = torch.full(q.shape[:-1], float("-inf"), device=q.device, dtype=acc)
+    for step in range(P):
+        j = (rank + step) % P
+        out, lse = attend_step_(q, k_chunks[j].to(q.dtype), v_chunks[j].to(q.dtype), scale, out, lse)
+    return out.to(q.dtype), lse
+
+
+def ring_backward(dout, q, out, lse, k_chunks, v_chunks, scale):
+    """``(dq, [dk_j], [dv_j])``: this rank's contribution to every chunk's gradient.
+
+    ``dq`` accumulates over the chunks (backward.py:184, 269; here in fp32, cast to
+    ``q.dtype`` at the end — the reference accumulates in ``q.dtype``); the sum of
+    dK/dV over the ranks that attended a chunk is the caller's collective."""
+    core = q.dtype
+    dout, out = dout.to(core), out.to(core)
+    dq = torch.zeros(q.shape, device=q.device, dtype=torch.float32)
+    dks, dvs = [], []
+    for kj, vj in zip(k_chunks, v_chunks):
+        dq_j, dk_j, dv_j = core_backward(dout, q, kj.to(core), vj.to(core), out, lse, scale)
+        dq += dq_j
+        dks.append(dk_j)
+        dvs.append(dv_j)
+    return dq.to(core), dks, dvs
+
+
+# --------------------------------------------------------------------------- #
+# windowed attention with an additive bias (Swin block)
+# --------------------------------------------------------------------------- #
+class _BiasedAttention(torch.autograd.Function):
+    """``F.scaled_dot_product_attention(q, k, v, attn_mask=bias)`` as the Swin example
+    calls it (examples/swin.py:146-151), differentiable in q, k, v and bias."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, bias):  # noqa: D102
+        scale = q.shape[-1] ** -0.5
+        out, lse = core_forward(q, k, v, scale, bias=bias)
+        ctx.save_for_backward(q, k, v, bias, out, lse)
+        ctx.scale = scale
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):  # noqa: D102
+        q, k, v, bias, out, lse = ctx.saved_tensors
+        need_bias = bias is not None and ctx.needs_input_grad[3]
+        res = core_backward(grad_out, q, k, v, out, lse, ctx.scale, bias=bias, want_dbias=need_bias)
+        dq, dk, dv = res[:3]
+        dbias = None
+        if need_bias:
+            # sum the per-batch-entry gradient over the entries that share a bias matrix
+            sq, sk = q.shape[-2], k.shape[-2]
+            period = bias.numel() // (sq * sk)
+            dbias = res[3].reshape(-1, period, sq, sk).sum(0).reshape(bias.shape).to(bias.dtype)
+        return dq, dk, dv, dbias
+
+
+def window_attention(q, k, v, bias=None):
+    """softmax(q k^T / sqrt(d) + bias) v over the last two axes."""
+    return _BiasedAttention.apply(q, k, v, bias)
+
+
+__all__ = [
+    "attend_step_",
+    "backward",
+    "core_backward",
+    "core_forward",
+    "forward",
+    "fused_online_softmax_merge_",
+    "ring_backward",
+    "ring_forward",
+    "window_attention",
+]

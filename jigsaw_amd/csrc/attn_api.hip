@@ -1,0 +1,99 @@
+// C entry points of the attention core: validate and route to the MFMA flash
+// kernels when they cover the problem, to the generic kernels otherwise.
+#include "jg_common.h"
+
+namespace jg {
+bool attn_generic_supported(int d);
+int attn_generic_fwd(void* out, float* lse, const void* q, const void* k, const void* v,
+                     long long batch, int sq, int sk, int d, float scale, const float* bias,
+                     long long bias_period, int dtype, hipStream_t s);
+int attn_generic_bwd(void* dq, void* dk, void* dv, float* delta, float* dbias, const void* dout,
+                     const void* q, const void* k, const void* v, const void* out,
+                     const float* lse, long long batch, int sq, int sk, int d, float scale,
+                     const float* bias, long long bias_period, int dtype, hipStream_t s);
+bool attn_mfma_fwd_supported(long long batch, int sq, int sk, int d, int dtype, bool has_bias);
+int attn_mfma_fwd(void* out, float* lse, const void* q, const void* k, const void* v,
+                  long long batch, int sq, int sk, float scale, float* out_acc, float* lse_acc,
+                  hipStream_t s);
+bool attn_mfma_bwd_supported(long long batch, int sq, int sk, int d, int dtype, bool has_bias);
+size_t attn_mfma_bwd_workspace(long long batch, int sq, int sk);
+int attn_mfma_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q, const void* k,
+                  const void* v, const void* out, const float* lse, long long batch, int sq,
+                  int sk, float scale, void* ws, hipStream_t s);
+}  // namespace jg
+
+namespace {
+bool known(int dt) { return dt == JG_F32 || dt == JG_BF16 || dt == JG_F16; }
+
+int check_shape(const char* who, int64_t batch, int64_t sq, int64_t sk, int64_t d, float scale,
+                int dtype) {
+  JG_REQUIRE(known(dtype), "%s: unknown dtype %d", who, dtype);
+  JG_REQUIRE(batch >= 0 && sq >= 0 && sk >= 1 && d >= 1, "%s: bad shape", who);
+  JG_REQUIRE(sq < (1ll << 30) && sk < (1ll << 30), "%s: sequence too long", who);
+  JG_REQUIRE(scale > 0.0f, "%s: scale must be positive", who);
+  return JG_OK;
+}
+}  // namespace
+
+extern "C" int jg_attn_fwd(void* out, float* lse, const void* q, const void* k, const void* v,
+                           int64_t batch, int64_t sq, int64_t sk, int64_t d, float scale,
+                           const float* bias, int64_t bias_period, float* out_acc,
+                           float* lse_acc, int dtype, void* stream) {
+  const char* who = "jg_attn_fwd";
+  int rc = check_shape(who, batch, sq, sk, d, scale, dtype);
+  if (rc) return rc;
+  JG_REQUIRE(q && k && v, "%s: NULL input", who);
+  JG_REQUIRE((out_acc == nullptr) == (lse_acc == nullptr),
+             "%s: out_acc and lse_acc go together", who);
+  JG_REQUIRE(out_acc != nullptr || (out != nullptr && lse != nullptr),
+             "%s: nowhere to write the result", who);
+  JG_REQUIRE(bias == nullptr || bias_period >= 1, "%s: bias_period must be >= 1", who);
+  if (batch == 0 || sq == 0) return JG_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (jg::attn_mfma_fwd_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr))
+    return jg::attn_mfma_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, scale, out_acc, lse_acc, s);
+  if (!jg::attn_generic_supported((int)d))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: head size %lld not in {8, 16, 32, 64, 128}", who, (long long)d);
+  if (out_acc != nullptr)
+    JG_FAIL(JG_ERR_UNSUPPORTED,
+            "%s: the fused merge needs the MFMA path (bf16, d = 64, sq %% 128 == 0, sk %% 128 == 0);"
+            " call jg_lse_merge after the core instead", who);
+  rc = jg::attn_generic_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, (int)d, scale, bias,
+                            bias_period, dtype, s);
+  if (rc) return rc;
+  return JG_OK;
+}
+
+extern "C" size_t jg_attn_bwd_workspace_bytes(int64_t batch, int64_t sq, int64_t sk, int64_t d) {
+  if (batch <= 0 || sq <= 0) return 0;
+  (void)sk;
+  (void)d;
+  // delta (batch, sq) fp32; the MFMA path needs nothing beyond it
+  return (size_t)batch * (size_t)sq * sizeof(float);
+}
+
+extern "C" int jg_attn_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q,
+                           const void* k, const void* v, const void* out, const float* lse,
+                           int64_t batch, int64_t sq, int64_t sk, int64_t d, float scale,
+                           const float* bias, int64_t bias_period, float* dbias, int dtype,
+                           void* workspace, size_t workspace_bytes, void* stream) {
+  const char* who = "jg_attn_bwd";
+  int rc = check_shape(who, batch, sq, sk, d, scale, dtype);
+  if (rc) return rc;
+  JG_REQUIRE(dq && dk && dv && dout && q && k && v && out && lse, "%s: NULL pointer", who);
+  JG_REQUIRE(bias == nullptr || bias_period >= 1, "%s: bias_period must be >= 1", who);
+  if (batch == 0 || sq == 0) return JG_OK;
+  if (workspace == nullptr || workspace_bytes < jg_attn_bwd_workspace_bytes(batch, sq, sk, d))
+    JG_FAIL(JG_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", who, workspace_bytes,
+            jg_attn_bwd_workspace_bytes(batch, sq, sk, d));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dbias == nullptr &&
+      jg::attn_mfma_bwd_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr))
+    return jg::attn_mfma_bwd(dq, dk, dv, dout, q, k, v, out, lse, batch, (int)sq, (int)sk, scale,
+                             workspace, s);
+  if (!jg::attn_generic_supported((int)d))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: head size %lld not in {8, 16, 32, 64, 128}", who, (long long)d);
+  return jg::attn_generic_bwd(dq, dk, dv, static_cast<float*>(workspace), dbias, dout, q, k, v, out,
+                              lse, batch, (int)sq, (int)sk, (int)d, scale, bias, bias_period, dtype,
+                              s);
+}

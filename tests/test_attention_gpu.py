@@ -1,0 +1,181 @@
+"""HIP attention core, fused ring step and ring loops against the oracle (GPU).
+
+Tolerances: rel-L2 1e-5 for fp32 tensors, 2e-2 for bf16 / fp16 (north-star bar); the
+reference's own ring tests use atol 1e-3 fp32 / 1e-2 bf16
+(tests/modules/attention/test_ring_attention.py:159-368).
+"""
+
+import pytest
+import torch
+
+from helpers import rel_l2
+from jigsaw_amd import attention as ja
+from oracle import attention as oa
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+
+
+def _qkv(b, h, sq, sk, d, dtype, seed=0):
+    torch.manual_seed(seed)
+    q = (torch.randn(b, h, sq, d) / d**0.5).to(dtype)
+    k = torch.randn(b, h, sk, d).to(dtype)
+    v = torch.randn(b, h, sk, d).to(dtype)
+    return q, k, v
+
+
+CORE_SHAPES = [
+    (3, 6, 64, 64, 16),   # the reference's ring test shape per chunk (b=3, h=6, n=16*4, d=16)
+    (2, 2, 50, 70, 32),   # ragged
+    (1, 3, 130, 33, 64),
+    (1, 2, 128, 128, 64),  # MFMA path for bf16
+    (2, 2, 256, 384, 64),  # MFMA path for bf16
+    (1, 1, 40, 40, 128),
+    (1, 2, 17, 9, 8),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", CORE_SHAPES, ids=lambda s: "b{}h{}q{}k{}d{}".format(*s))
+def test_core_forward_backward_match_oracle(shape, dtype, dev):
+    b, h, sq, sk, d = shape
+    q, k, v = _qkv(b, h, sq, sk, d, dtype)
+    scale = d**-0.5
+    want_o, want_l = oa.core_forward(q.double(), k.double(), v.double(), scale)
+    out, lse, rng = ja.forward(q.to(dev), k.to(dev), v.to(dev), scale, 0.0, layout="bhsd")
+    assert rng is None and out.dtype == dtype and lse.dtype == torch.float32
+    assert rel_l2(out, want_o) < TOL[dtype], f"out {rel_l2(out, want_o):.3e}"
+    assert rel_l2(lse, want_l) < max(TOL[dtype] * 0.1, 1e-5), f"lse {rel_l2(lse, want_l):.3e}"
+
+    dout = torch.randn(b, h, sq, d).to(dtype)
+    # backward from the oracle's own (global) out / lse, rounded as the ring would hold them
+    o_in, l_in = want_o.to(dtype), want_l.float()
+    wdq, wdk, wdv = oa.core_backward(dout.double(), q.double(), k.double(), v.double(), o_in.double(), l_in.double(), scale)
+    dq, dk, dv = ja.backward(dout.to(dev), q.to(dev), k.to(dev), v.to(dev), o_in.to(dev), l_in.to(dev), scale, sq, sk)
+    assert dq.dtype == dtype
+    for name, got, want in (("dq", dq, wdq), ("dk", dk, wdk), ("dv", dv, wdv)):
+        assert rel_l2(got, want) < TOL[dtype], f"{name} {rel_l2(got, want):.3e}"
+
+
+@pytest.mark.parametrize(
+    "b,h,n,d,P,dtype",
+    [
+        (3, 6, 16, 16, 4, torch.float32),
+        (3, 6, 16, 16, 4, torch.bfloat16),
+        (1, 2, 256, 64, 4, torch.bfloat16),
+        (1, 2, 128, 64, 3, torch.float32),
+    ],
+)
+@pytest.mark.parametrize("rank", [0, 2])
+def test_ring_forward_backward_match_full_attention(b, h, n, d, P, dtype, rank, dev):
+    """Ring over P local chunks == full softmax attention over the concatenated K/V
+    (the reference's method, test_ring_attention.py:267-275), forward and backward."""
+    torch.manual_seed(1)
+    scale = d**-0.5
+    q = (torch.randn(b, h, n, d) / d**0.5).to(dtype)
+    ks = [torch.randn(b, h, n, d).to(dtype) for _ in range(P)]
+    vs = [torch.randn(b, h, n, d).to(dtype) for _ in range(P)]
+    K = torch.cat(ks, 2).double().requires_grad_()
+    V = torch.cat(vs, 2).double().requires_grad_()
+    Q = q.double().requires_grad_()
+    s = (Q @ K.mT) * scale
+    full = torch.softmax(s, -1) @ V
+    dout = torch.randn(b, h, n, d).to(dtype)
+    full.backward(dout.double())
+
+    out, lse = ja.ring_forward(q.to(dev), [t.to(dev) for t in ks], [t.to(dev) for t in vs], scale, rank=rank % P)
+    assert out.dtype == dtype and lse.dtype == torch.float32
+    assert rel_l2(out, full.detach()) < TOL[dtype], f"out {rel_l2(out, full.detach()):.3e}"
+    assert rel_l2(lse, torch.logsumexp(s.detach(), -1)) < 1e-3 if dtype != torch.float32 else 1e-5
+    # the oracle's ring loop (its chunk order, merge form and roundings) agrees too
+    o_or, l_or = oa.ring_forward(q.float(), [t.float() for t in ks], [t.float() for t in vs], scale, rank=rank % P)
+    assert rel_l2(out, o_or) < TOL[dtype]
+
+    dq, dks, dvs = ja.ring_backward(dout.to(dev), q.to(dev), out, lse, [t.to(dev) for t in ks], [t.to(dev) for t in vs], scale)
+    assert rel_l2(dq, Q.grad) < TOL[dtype], f"dq {rel_l2(dq, Q.grad):.3e}"
+    assert rel_l2(torch.cat(dks, 2), K.grad) < TOL[dtype], f"dk {rel_l2(torch.cat(dks, 2), K.grad):.3e}"
+    assert rel_l2(torch.cat(dvs, 2), V.grad) < TOL[dtype], f"dv {rel_l2(torch.cat(dvs, 2), V.grad):.3e}"
+
+
+def test_fused_step_equals_core_plus_merge(dev):
+    """The fused epilogue merge and the separate merge kernel give the same accumulator."""
+    q, k, v = _qkv(1, 4, 256, 512, 64, torch.bfloat16, seed=2)
+    q, k, v = q.to(dev), k.to(dev), v.to(dev)
+    scale = 0.125
+    acc1 = torch.randn(1, 4, 256, 64, device=dev)
+    l1 = torch.randn(1, 4, 256, device=dev)
+    acc2, l2 = acc1.clone(), l1.clone()
+    ja.core_forward(q, k, v, scale, out_acc=acc1, lse_acc=l1, want_out=False)
+    out_j, l_j = ja.core_forward(q, k, v, scale)
+    acc2, l2 = ja.fused_online_softmax_merge_(acc2, l2, out_j, l_j, "bhsd")
+    torch.testing.assert_close(acc1, acc2, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(l1, l2, atol=1e-6, rtol=1e-6)
+
+
+def test_config4_shape_properties(dev):
+    """Config 4 at full size: 8 heads, 4096 queries, 4 chunks of 4096 keys, d = 64, bf16.
+    Size-independent checks: ring over 4 chunks == one core call over the concatenated
+    K/V; permuting the chunks changes nothing beyond rounding; 128 sampled query rows
+    match the fp64 oracle over all 16384 keys."""
+    torch.manual_seed(3)
+    b, h, n, d, P = 1, 8, 4096, 64, 4
+    scale = d**-0.5
+    q = (torch.randn(b, h, n, d, device=dev) / 8).bfloat16()
+    ks = [torch.randn(b, h, n, d, device=dev).bfloat16() for _ in range(P)]
+    vs = [torch.randn(b, h, n, d, device=dev).bfloat16() for _ in range(P)]
+    out, lse = ja.ring_forward(q, ks, vs, scale, rank=1)
+    full_o, full_l = ja.core_forward(q, torch.cat(ks, 2), torch.cat(vs, 2), scale)
+    assert rel_l2(out, full_o) < 1e-2
+    assert rel_l2(lse, full_l) < 1e-5
+    out2, lse2 = ja.ring_forward(q, ks[::-1], vs[::-1], scale, rank=0)
+    assert rel_l2(out2, out) < 1e-2 and rel_l2(lse2, lse) < 1e-5
+    rows = torch.arange(0, n, 32)
+    qs = q[:, :, rows].double().cpu()
+    K, V = torch.cat(ks, 2).double().cpu(), torch.cat(vs, 2).double().cpu()
+    s = (qs @ K.mT) * scale
+    want = torch.softmax(s, -1) @ V
+    assert rel_l2(out[:, :, rows], want) < 2e-2
+    assert rel_l2(lse[:, :, rows], torch.logsumexp(s, -1)) < 1e-4
+
+
+def test_window_attention_with_bias_and_mask(dev):
+    """Swin-style windows: (B, nW, heads, N, d) with a (nW, heads, N, N) bias that
+    holds -inf entries (shift mask), forward and backward incl. the bias gradient."""
+    torch.manual_seed(4)
+    B, nW, heads, N, d = 2, 6, 4, 64, 32
+    q, k, v = (torch.randn(B, nW, heads, N, d) for _ in range(3))
+    bias = torch.randn(nW, heads, N, N) * 0.5
+    mask = torch.zeros(nW, 1, N, N)
+    mask[1, :, :32, 32:] = float("-inf")
+    mask[1, :, 32:, :32] = float("-inf")
+    bias = bias + mask
+    qd, kd, vd = (t.double().requires_grad_() for t in (q, k, v))
+    bd = bias.double().requires_grad_()
+    want = oa.window_attention(qd, kd, vd, bd)
+    g = torch.randn_like(want)
+    want.backward(g)
+    qg, kg, vg, bg = (t.to(dev).requires_grad_() for t in (q, k, v, bias))
+    out = ja.window_attention(qg, kg, vg, bg)
+    assert rel_l2(out, want.detach()) < 1e-5
+    out.backward(g.float().to(dev))
+    assert rel_l2(qg.grad, qd.grad) < 1e-5 and rel_l2(kg.grad, kd.grad) < 1e-5 and rel_l2(vg.grad, vd.grad) < 1e-5
+    assert rel_l2(bg.grad, torch.nan_to_num(bd.grad)) < 1e-5
+    # broadcast bias (heads, N, N), bf16 inputs
+    out_b = ja.window_attention(qg.detach().bfloat16(), kg.detach().bfloat16(), vg.detach().bfloat16(), bg.detach()[0])
+    want_b = oa.window_attention(q.bfloat16().double(), k.bfloat16().double(), v.bfloat16().double(), bias[0].double())
+    assert rel_l2(out_b, want_b) < 2e-2
+
+
+def test_core_argument_errors(dev):
+    q = torch.zeros(1, 2, 8, 16, device=dev)
+    with pytest.raises(NotImplementedError):
+        ja.forward(q, q, q, 0.25, 0.0, layout="bshd")
+    with pytest.raises(NotImplementedError):
+        ja.forward(q, q, q, 0.25, 0.1)
+    with pytest.raises(RuntimeError):
+        ja.forward(q, q.bfloat16(), q, 0.25)
+    with pytest.raises(ValueError):
+        ja.forward(q, q[:, :1], q, 0.25)
+    with pytest.raises(NotImplementedError):
+        ja.forward(q[..., :5].contiguous(), q[..., :5].contiguous(), q[..., :5].contiguous(), 0.25)
