@@ -98,6 +98,40 @@ def conv_step(wl):
     return y, gx, gw, gb
 
 
+def attention_figures(dev, iters: int) -> dict:
+    """Configuration 4: one rank's ring-attention step. 8 local heads, 4096 local
+    queries, one K/V chunk of 4096 keys per step (4 steps), head size 64, bf16.
+    Forward = flash core with the LSE merge fused in; backward = dQ + dK/dV kernels
+    from the global out / lse. Also the sharded LayerNorm statistics (dim 512, 256 local)."""
+    from jigsaw_amd import attention as ja
+    from jigsaw_amd import layernorm as jl
+
+    b, h, n, d, P = 1, 8, 4096, 64, 4
+    g = torch.Generator(device=dev).manual_seed(0)
+    q = (torch.randn(b, h, n, d, device=dev, generator=g) / 8).bfloat16()
+    ks = [(torch.randn(b, h, n, d, device=dev, generator=g) / 8).bfloat16() for _ in range(P)]
+    vs = [(torch.randn(b, h, n, d, device=dev, generator=g) / 8).bfloat16() for _ in range(P)]
+    dout = torch.randn(b, h, n, d, device=dev, generator=g).bfloat16()
+    scale = d**-0.5
+    acc = torch.zeros(b, h, n, d, device=dev)
+    lse = torch.full((b, h, n), float("-inf"), device=dev)
+    f_fwd = 4 * b * h * n * n * d
+    f_bwd = 10 * b * h * n * n * d
+    ms_f = time_gpu(lambda: ja.core_forward(q, ks[0], vs[0], scale, out_acc=acc, lse_acc=lse, want_out=False), iters)
+    out, l = ja.ring_forward(q, ks, vs, scale)
+    ms_b = time_gpu(lambda: ja.core_backward(dout, q, ks[0], vs[0], out, l, scale), iters)
+    ms_ring = time_gpu(lambda: ja.ring_forward(q, ks, vs, scale), iters)
+    x = torch.randn(b, n, 256, device=dev, generator=g).bfloat16()
+    ms_ln = time_gpu(lambda: jl.partial_stats(x), iters)
+    tf = lambda f, ms: f / (ms * 1e-3) / 1e12  # noqa: E731
+    return {
+        "attn_fwd_step": {"ms": ms_f, "tflops": tf(f_fwd, ms_f), "frac_mfma_peak": tf(f_fwd, ms_f) / PEAK_BF16_TFLOPS},
+        "attn_bwd_step": {"ms": ms_b, "tflops": tf(f_bwd, ms_b), "frac_mfma_peak": tf(f_bwd, ms_b) / PEAK_BF16_TFLOPS},
+        "attn_ring_fwd_4_steps": {"ms": ms_ring, "tflops": tf(4 * f_fwd, ms_ring)},
+        "ln_partial_stats": {"ms": ms_ln, "GBps": x.numel() * 2 / (ms_ln * 1e-3) / 1e9, "bytes": x.numel() * 2},
+    }
+
+
 def cpu_baseline(seconds_budget: float = 30.0) -> dict:
     """The oracle (the reference's torch CPU operators) timed on the host cores on a
     bounded sample of the same workload: batch 1 of a 512x512, 64 -> 64 tile in fp32
@@ -229,12 +263,7 @@ def main() -> int:
         "halo_assemble": {"ms": ms_asm, "GBps": gbps(ms_asm), "frac_hbm_peak": gbps(ms_asm) / PEAK_HBM_GBPS, "bytes": halo_bytes},
         "halo_fold": {"ms": ms_fold, "GBps": gbps(ms_fold), "frac_hbm_peak": gbps(ms_fold) / PEAK_HBM_GBPS, "bytes": halo_bytes},
     }
-    try:
-        from _bench_attention import attention_figures  # optional: ring-attention step figures
-
-        extra.update(attention_figures(dev, it))
-    except ImportError:
-        pass
+    extra.update(attention_figures(dev, max(10, it)))
 
     line = {
         "metric": METRIC,

@@ -359,6 +359,223 @@ __global__ __launch_bounds__(256) void fold_kernel(typename Arith<DT>::T* __rest
   }
 }
 
+
+// ===================================================================== row kernels
+// Bandwidth versions of assemble and fold. A destination ROW (one (plane, d, h)
+// line along W) is owned by a group of LPR lanes (a whole wavefront for long
+// rows), each lane producing 16-byte vectors j, j + LPR, ... of that row. Row
+// coordinates are decomposed once per lane with multiply-high divisions, the
+// three sources of the row (lower-W strip, middle, upper-W strip) are looked up
+// once, and only the vectors that straddle a region boundary take the
+// element-wise path. Rows start on 4-byte boundaries, which is all the 16-byte
+// global accesses of gfx9 need.
+struct Magic {
+  uint32_t m, s, one;  // n / d = one ? n : (t + ((n - t) >> 1)) >> (s - 1), t = mulhi(m, n)
+};
+
+__device__ __forceinline__ uint32_t mdiv(uint32_t n, const Magic& k) {
+  if (k.one) return n;
+  const uint32_t t = __umulhi(k.m, n);
+  return (t + ((n - t) >> 1)) >> (k.s - 1);
+}
+
+struct RowPlan {
+  uint32_t nrows;   // planes * Da * Ha (assemble) or planes * D * H (fold)
+  int lpr_log2;     // lanes per row = 1 << lpr_log2
+  int iters;        // vectors per lane
+  int nvec;         // vectors per row
+  Magic div_h, div_d;
+};
+
+typedef uint32_t u32x4_s4 __attribute__((ext_vector_type(4), aligned(4)));
+
+template <typename T>
+__global__ __launch_bounds__(256) void assemble_rows_kernel(Table tab, T* __restrict__ dst,
+                                                            Geom g, RowPlan pl) {
+  constexpr int V = Bits<T>::V;
+  const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+  const uint32_t row = t >> pl.lpr_log2;
+  if (row >= pl.nrows) return;
+  const int lir = (int)(t & ((1u << pl.lpr_log2) - 1));
+  const int Da = g.lo[0] + g.n[0] + g.hi[0];
+  const int Ha = g.lo[1] + g.n[1] + g.hi[1];
+  const int Wa = g.lo[2] + g.n[2] + g.hi[2];
+  const uint32_t t2 = mdiv(row, pl.div_h);
+  const int ha = (int)(row - t2 * (uint32_t)Ha);
+  const uint32_t pp = mdiv(t2, pl.div_d);
+  const int da = (int)(t2 - pp * (uint32_t)Da);
+  int rd, cd, ed, rh, ch, eh;
+  region(da, g.lo[0], g.n[0], g.hi[0], rd, cd, ed);
+  region(ha, g.lo[1], g.n[1], g.hi[1], rh, ch, eh);
+  const long long line = ((long long)pp * ed + cd) * eh + ch;  // row index inside a source
+  const int base_idx = rd * 9 + rh * 3;
+  const T* s0 = static_cast<const T*>(table_entry(base_idx + 0));
+  const T* s1 = static_cast<const T*>(table_entry(base_idx + 1));
+  const T* s2 = static_cast<const T*>(table_entry(base_idx + 2));
+  if (s0 != nullptr) s0 += line * g.lo[2];
+  if (s1 != nullptr) s1 += line * g.n[2];
+  if (s2 != nullptr) s2 += line * g.hi[2];
+  T* drow = dst + (long long)row * Wa;
+  const int mid_lo = g.lo[2], mid_hi = g.lo[2] + g.n[2];
+  for (int it = 0; it < pl.iters; ++it) {
+    const int j = lir + (it << pl.lpr_log2);
+    if (j >= pl.nvec) break;
+    const int c0 = j * V;
+    if (c0 >= mid_lo && c0 + V <= mid_hi) {
+      u32x4 val = {0u, 0u, 0u, 0u};
+      if (s1 != nullptr) val = load16_unaligned<T>(s1 + (c0 - mid_lo));
+      *reinterpret_cast<u32x4_s4*>(drow + c0) = val;
+    } else {
+      T tmp[V];
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const int c = c0 + e;
+        T v = T(0);
+        if (c < mid_lo) {
+          if (s0 != nullptr) v = s0[c];
+        } else if (c < mid_hi) {
+          if (s1 != nullptr) v = s1[c - mid_lo];
+        } else if (c < Wa) {
+          if (s2 != nullptr) v = s2[c - mid_hi];
+        }
+        tmp[e] = v;
+      }
+      if (c0 + V <= Wa) {
+        u32x4 val;
+        __builtin_memcpy(&val, tmp, 16);
+        *reinterpret_cast<u32x4_s4*>(drow + c0) = val;
+      } else {
+        for (int e = 0; e < V && c0 + e < Wa; ++e) drow[c0 + e] = tmp[e];
+      }
+    }
+  }
+}
+
+// One element of the fold with the loops left rolled: only the offsets that reach
+// the element cost anything (most edge elements see one or two neighbours).
+template <int DT>
+__device__ __forceinline__ typename Arith<DT>::T fold_one_rolled(
+    const typename Arith<DT>::T* __restrict__ own, const Geom& g, long long p, int d, int h, int w) {
+  typedef typename Arith<DT>::T T;
+  const int Ha = g.lo[1] + g.n[1] + g.hi[1];
+  const int Wa = g.lo[2] + g.n[2] + g.hi[2];
+  const int Da = g.lo[0] + g.n[0] + g.hi[0];
+  float acc_d = 0.0f;
+#pragma unroll 1
+  for (int od = -1; od <= 1; ++od) {
+    int cd, ed;
+    if (!reach(od, d, g.lo[0], g.n[0], g.hi[0], cd, ed)) continue;
+    float acc_h = 0.0f;
+#pragma unroll 1
+    for (int oh = -1; oh <= 1; ++oh) {
+      int ch, eh;
+      if (!reach(oh, h, g.lo[1], g.n[1], g.hi[1], ch, eh)) continue;
+      float acc_w = 0.0f;
+#pragma unroll 1
+      for (int ow = -1; ow <= 1; ++ow) {
+        int cw, ew;
+        if (!reach(ow, w, g.lo[2], g.n[2], g.hi[2], cw, ew)) continue;
+        T bits;
+        if (od == 0 && oh == 0 && ow == 0) {
+          long long off = ((p * Da + (d + g.lo[0])) * Ha + (h + g.lo[1])) * (long long)Wa +
+                          (w + g.lo[2]);
+          bits = own[off];
+        } else {
+          const T* s = static_cast<const T*>(table_entry((od + 1) * 9 + (oh + 1) * 3 + (ow + 1)));
+          if (s == nullptr) continue;
+          long long off = ((p * ed + cd) * eh + ch) * (long long)ew + cw;
+          bits = s[off];
+        }
+        acc_w = Arith<DT>::up(Arith<DT>::down(acc_w + Arith<DT>::up(bits)));
+      }
+      acc_h = Arith<DT>::up(Arith<DT>::down(acc_h + acc_w));
+    }
+    acc_d = Arith<DT>::up(Arith<DT>::down(acc_d + acc_h));
+  }
+  return Arith<DT>::down(acc_d);
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
+                                                        typename Arith<DT>::T* __restrict__ dst,
+                                                        const typename Arith<DT>::T* __restrict__ own,
+                                                        Geom g, RowPlan pl) {
+  typedef typename Arith<DT>::T T;
+  constexpr int V = Bits<T>::V;
+  constexpr T ABS = (T)(~(T(1) << (sizeof(T) * 8 - 1)));
+  const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+  const uint32_t row = t >> pl.lpr_log2;
+  if (row >= pl.nrows) return;
+  const int lir = (int)(t & ((1u << pl.lpr_log2) - 1));
+  const int D = g.n[0], H = g.n[1], W = g.n[2];
+  const int Ha = g.lo[1] + H + g.hi[1];
+  const int Wa = g.lo[2] + W + g.hi[2];
+  const int Da = g.lo[0] + D + g.hi[0];
+  const uint32_t t2 = mdiv(row, pl.div_h);
+  const int h = (int)(row - t2 * (uint32_t)H);
+  const uint32_t pp = mdiv(t2, pl.div_d);
+  const int d = (int)(t2 - pp * (uint32_t)D);
+  const long long p = (long long)pp;
+  // rows that a lower / upper neighbour along D or H reaches take the element path
+  const bool row_plain = (d >= g.hi[0]) && (d < D - g.lo[0]) && (h >= g.hi[1]) && (h < H - g.lo[1]);
+  const T* orow = own + ((p * Da + (d + g.lo[0])) * Ha + (h + g.lo[1])) * (long long)Wa + g.lo[2];
+  T* drow = dst + (long long)row * W;
+  for (int it = 0; it < pl.iters; ++it) {
+    const int j = lir + (it << pl.lpr_log2);
+    if (j >= pl.nvec) break;
+    const int c0 = j * V;
+    if (row_plain && c0 + V <= W) {
+      // `0 + own` for every element (clears the sign of a zero) ...
+      u32x4 val = load16_unaligned<T>(orow + c0);
+      T tmp[V];
+      __builtin_memcpy(tmp, &val, 16);
+#pragma unroll
+      for (int e = 0; e < V; ++e)
+        if ((tmp[e] & ABS) == 0) tmp[e] = 0;
+      // ... and the full ordered sum where a W-neighbour reaches
+      if (c0 < g.hi[2] || c0 + V > W - g.lo[2]) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          const int c = c0 + e;
+          if (c < g.hi[2] || c >= W - g.lo[2]) tmp[e] = fold_one_rolled<DT>(own, g, p, d, h, c);
+        }
+      }
+      __builtin_memcpy(&val, tmp, 16);
+      *reinterpret_cast<u32x4_s4*>(drow + c0) = val;
+    } else {
+      for (int e = 0; e < V && c0 + e < W; ++e) drow[c0 + e] = fold_one_rolled<DT>(own, g, p, d, h, c0 + e);
+    }
+  }
+}
+
+Magic make_magic(uint32_t d) {
+  Magic k;
+  k.one = (d == 1);
+  k.m = 0;
+  k.s = 1;
+  if (d <= 1) return k;
+  uint32_t s = 0;
+  while ((1ull << s) < d) ++s;  // ceil(log2 d)
+  k.s = s;
+  k.m = (uint32_t)(((1ull << 32) * ((1ull << s) - d)) / d + 1);
+  return k;
+}
+
+// Lanes per row / vectors per lane for rows of `nvec` 16-byte vectors.
+bool make_plan(unsigned long long nrows, int nvec, uint32_t div_h, uint32_t div_d, RowPlan* pl) {
+  int lg = 0;
+  while ((1 << lg) < nvec && lg < 6) ++lg;
+  const int lpr = 1 << lg;
+  if (nrows == 0 || nrows * (unsigned long long)lpr >= (1ull << 32)) return false;
+  pl->nrows = (uint32_t)nrows;
+  pl->lpr_log2 = lg;
+  pl->nvec = nvec;
+  pl->iters = (nvec + lpr - 1) / lpr;
+  pl->div_h = make_magic(div_h);
+  pl->div_d = make_magic(div_d);
+  return true;
+}
+
 // ---------------------------------------------------------------- host side
 int check_geom(const jg_halo_geom* g, const char* who, bool adjacent_only) {
   JG_REQUIRE(g != nullptr, "%s: geom is NULL", who);
@@ -432,6 +649,20 @@ extern "C" int jg_halo_assemble_3d(void* x_aug, const void* const src[27],
   for (int a = 0; a < 3; ++a) total *= (unsigned long long)(g.lo[a] + g.n[a] + g.hi[a]);
   if (total == 0) return JG_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const int Da = g.lo[0] + g.n[0] + g.hi[0], Ha = g.lo[1] + g.n[1] + g.hi[1];
+  const int Wa = g.lo[2] + g.n[2] + g.hi[2];
+  RowPlan pl;
+  const int V = 16 / elem_size;
+  if ((Wa * elem_size) % 4 == 0 &&
+      make_plan((unsigned long long)g.planes * Da * Ha, (Wa + V - 1) / V, Ha, Da, &pl)) {
+    const unsigned blocks = (unsigned)((((unsigned long long)pl.nrows << pl.lpr_log2) + 255) / 256);
+    if (elem_size == 2)
+      assemble_rows_kernel<uint16_t><<<blocks, 256, 0, s>>>(tab, static_cast<uint16_t*>(x_aug), g, pl);
+    else
+      assemble_rows_kernel<uint32_t><<<blocks, 256, 0, s>>>(tab, static_cast<uint32_t*>(x_aug), g, pl);
+    JG_CHECK_LAUNCH("jg_halo_assemble_3d");
+    return JG_OK;
+  }
   const bool wide = total >= (1ull << 31);
   if (elem_size == 2) {
     int grid = grid_for((total + 7) / 8);
@@ -559,8 +790,21 @@ extern "C" int jg_halo_fold_3d(void* gx, const void* gx_aug, const void* const s
   for (int a = 0; a < 3; ++a) total_aug *= (unsigned long long)(g.lo[a] + g.n[a] + g.hi[a]);
   if (total == 0) return JG_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool wide = total_aug >= (1ull << 31);
   const int V = 16 / es;
+  RowPlan pl;
+  if ((g.n[2] * es) % 4 == 0 &&
+      make_plan((unsigned long long)g.planes * g.n[0] * g.n[1], (g.n[2] + V - 1) / V, g.n[1], g.n[0], &pl)) {
+    const unsigned blocks = (unsigned)((((unsigned long long)pl.nrows << pl.lpr_log2) + 255) / 256);
+    if (dtype == JG_F32)
+      fold_rows_kernel<JG_F32><<<blocks, 256, 0, s>>>(tab, static_cast<uint32_t*>(gx), static_cast<const uint32_t*>(gx_aug), g, pl);
+    else if (dtype == JG_BF16)
+      fold_rows_kernel<JG_BF16><<<blocks, 256, 0, s>>>(tab, static_cast<uint16_t*>(gx), static_cast<const uint16_t*>(gx_aug), g, pl);
+    else
+      fold_rows_kernel<JG_F16><<<blocks, 256, 0, s>>>(tab, static_cast<uint16_t*>(gx), static_cast<const uint16_t*>(gx_aug), g, pl);
+    JG_CHECK_LAUNCH("jg_halo_fold_3d");
+    return JG_OK;
+  }
+  const bool wide = total_aug >= (1ull << 31);
   int grid = grid_for((total + V - 1) / V);
 #define JG_FOLD(DT)                                                                         \
   do {                                                                                      \
