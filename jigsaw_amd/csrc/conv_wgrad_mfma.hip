@@ -1,26 +1,33 @@
-// Weight gradient of the 2-D 3x3 convolution on the bf16 matrix cores, for
-// 64 -> 64 channels, stride 1, dilation 1, channels-first tensors.
+// Weight gradient of the 3x3 (2-D) and 3x3x3 (3-D) convolution on the bf16 matrix
+// cores, stride 1, dilation 1, channels-first tensors, 32 or 64 channels a side.
 //
-//   gw[co][ci][kh][kw] = sum_{n,h,w} g[n][co][h][w] * x[n][ci][h+kh-ph][w+kw-pw]
+//   gw[co][ci][kd][kh][kw] = sum_{n,d,h,w} g[n][co][d][h][w] * x[n][ci][d+kd-pd][h+kh-ph][w+kw-pw]
 //
-//   GEMM view   M = output channels, N = input channels, K = pixels. Both operands
-//               are pixel-contiguous in the channels-first tensors, so the tiles go
-//               to LDS untransposed.
+//   GEMM view   M = output channels, N = input channels (x depth taps), K = pixels.
+//               Both operands are pixel-contiguous in the channels-first tensors, so
+//               the tiles go to LDS untransposed. A 3-D problem is the 2-D one with
+//               the depth taps folded into the x "channels": channel kd*Cin + ci of a
+//               stage at output depth d is the plane x[n][ci][d + kd - pd].
 //   MFMA roles  A = g (32 channels x 16 pixels of a row), B = x (16 pixels x 32
 //               channels) shifted by the tap. The kw shift is not 16-byte aligned in
 //               LDS, so a lane reads 10 consecutive pixels once (b128 + b32) and
 //               builds the three kw fragments with funnel shifts.
-//   Workgroup   512 threads = 8 wavefronts; wavefront = (co block, ci block) pair x
-//               column half. It keeps its 9 taps x 32x32 fp32 accumulators in
-//               registers for the whole kernel (144 VGPRs) and walks the pixels.
-//   Stage       2 output rows x 64 columns: g tile 64 x 2 x 64, x tile 64 x 4 x 66;
+//   Workgroup   one wavefront per (g channel block, x channel block) pair; it keeps
+//               its 9 taps x 32x32 fp32 accumulators in registers for the whole
+//               kernel (144 VGPRs) and walks the pixels. At most 4 wavefronts, one
+//               per SIMD, so each has the full register file: the prefetch path must
+//               not spill (a scratch reload there waits on every outstanding global
+//               load and serialises the pipeline). 64->64 2-D: 2x2 = 4 wavefronts;
+//               32->32 3-D: 1x3 = 3, plus one that only helps with the prefetch.
+//   Stage       2 output rows x 64 columns: g tile C x 2 x 64, x tile C' x 4 x 72;
 //               prefetched to registers during the MFMAs of the previous stage,
 //               double buffered in LDS (one barrier per stage). Channel strides in
 //               LDS are odd multiples of 16 bytes so that the 32 channel-lanes of a
-//               fragment read hit distinct banks.
-//   Reduction   every workgroup writes its partial (2 halves) to the workspace; a
-//               second kernel sums the partials in a fixed order (deterministic) and
-//               writes gw in the weight layout.
+//               fragment read hit distinct banks. Stages that lie wholly inside the
+//               tensors (a wave-uniform test) take a branch-free vector load path.
+//   Reduction   every workgroup writes its partial to the workspace; a second kernel
+//               sums the partials in a fixed order (deterministic) and writes gw in
+//               the weight layout.
 #include "conv_common.h"
 
 namespace {
@@ -32,117 +39,149 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
-constexpr int C = 64;                 // channels on both sides
-constexpr int THREADS = 512;
 constexpr int SR = 2, SW = 64;        // output rows / columns per stage
 constexpr int XR = SR + 2;            // x rows per stage
 constexpr int G_CH = SR * SW * 2 + 16;        // 272 bytes per g channel
 constexpr int X_ROW = 144;                    // 72 pixels
 constexpr int X_CH = XR * X_ROW + 16;         // 592 bytes per x channel
-constexpr int G_BYTES = C * G_CH;             // 17408
-constexpr int X_BYTES = C * X_CH;             // 37888
-constexpr int STAGE_BYTES = G_BYTES + X_BYTES;
-constexpr int G_CHUNKS = C * SR * (SW / 8);   // 1024 chunks of 8 pixels
-constexpr int X_CPR = 9;                      // chunks per x row (72 pixels)
-constexpr int X_CHUNKS = C * XR * X_CPR;      // 2304
-constexpr int CHUNKS = G_CHUNKS + X_CHUNKS;   // 3328
-constexpr int ROUNDS = (CHUNKS + THREADS - 1) / THREADS;  // 7
-constexpr int PART = C * C * 9;               // floats per partial
+constexpr int X_CPR = 9;                      // 8-pixel chunks per x row
 
 struct WgradParams {
-  const uint16_t* x;  // (N, 64, Hin, Win)
-  const uint16_t* g;  // (N, 64, Hout, Wout)
-  float* part;        // [slots][tap][co][ci]
-  int N, Hin, Win, Hout, Wout, pad_h, pad_w;
+  const uint16_t* x;  // (N, Cin, Din, Hin, Win)
+  const uint16_t* g;  // (N, Cout, Dout, Hout, Wout)
+  float* part;        // [workgroup][tap9][co][c']
+  int Cin, Cout;
+  int Din, Hin, Win, Dout, Hout, Wout;
+  int pad_d, pad_h, pad_w;
   int row_pairs, col_tiles;
-  int total_stages;   // N * col_tiles * row_pairs
+  long long total_stages;  // N * Dout * col_tiles * row_pairs
 };
 
-template <bool EVEN>
-__global__ __launch_bounds__(THREADS) void wgrad3x3_mfma_kernel(WgradParams p) {
+constexpr int wgrad_threads(int cgb, int cxb) { return (cgb * cxb >= 3) ? 256 : 64 * cgb * cxb; }
+
+template <int CGB, int CXB, bool EVEN>
+__global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(WgradParams p) {
+  constexpr int THREADS = wgrad_threads(CGB, CXB);
+  constexpr int CWAVES = CGB * CXB;  // wavefronts that own accumulators
+  constexpr int GC = 32 * CGB, XC = 32 * CXB;
+  constexpr int G_BYTES = GC * G_CH, X_BYTES = XC * X_CH;
+  constexpr int STAGE_BYTES = G_BYTES + X_BYTES;
+  constexpr int G_CHUNKS = GC * SR * (SW / 8);
+  constexpr int X_CHUNKS = XC * XR * X_CPR;
+  constexpr int CHUNKS = G_CHUNKS + X_CHUNKS;
+  constexpr int ROUNDS = (CHUNKS + THREADS - 1) / THREADS;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, kgp = lane >> 5;
-  const int pair = wave & 3, half = wave >> 2;
-  const int cb = pair >> 1, ib = pair & 1;
+  const int pair = wave % (CGB * CXB);
+  const int cb = pair / CXB, ib = pair % CXB;
 
-  // contiguous range of stages for this workgroup; stage -> (n, column tile, row pair),
-  // row pair fastest, so consecutive stages walk down one column of one image
-  const long long per = ((long long)p.total_stages + gridDim.x - 1) / gridDim.x;
+  // contiguous range of stages for this workgroup; stage -> (n, d, column tile, row pair),
+  // row pair fastest, so consecutive stages walk down one column of one plane
+  const long long per = (p.total_stages + gridDim.x - 1) / gridDim.x;
   const long long s_begin = per * blockIdx.x;
   long long s_end = s_begin + per;
   if (s_end > p.total_stages) s_end = p.total_stages;
 
   const size_t plane_x = (size_t)p.Hin * p.Win, plane_g = (size_t)p.Hout * p.Wout;
+  const size_t x_cs = plane_x * p.Din, g_cs = plane_g * p.Dout;  // channel strides
 
-  // chunk bookkeeping (fixed per thread): which 8 pixels of which channel / row
+  // ---- per-thread chunk bookkeeping, fixed for the whole kernel
+  uint32_t c_goff[ROUNDS];  // byte offset from the stage origin of its tensor
+  uint32_t c_lds[ROUNDS];   // byte offset inside a stage buffer
+#pragma unroll
+  for (int rd = 0; rd < ROUNDS; ++rd) {
+    const int q = tid + rd * THREADS;
+    if (q < G_CHUNKS) {
+      const int c8 = q & 7, r = (q >> 3) % SR, ch = q / (8 * SR);
+      c_goff[rd] = (uint32_t)((ch * g_cs + (size_t)r * p.Wout + c8 * 8) * 2);
+      c_lds[rd] = (uint32_t)(ch * G_CH + r * (SW * 2) + c8 * 16);
+    } else if (q < CHUNKS) {
+      const int qx = q - G_CHUNKS;
+      const int c9 = qx % X_CPR;
+      const int rr = qx / X_CPR;
+      const int rho = rr % XR, ch = rr / XR;     // ch = kd * Cin + ci
+      const int kd = ch / p.Cin, ci = ch - kd * p.Cin;
+      c_goff[rd] = (uint32_t)((ci * x_cs + kd * plane_x + (size_t)rho * p.Win + c9 * 8) * 2);
+      c_lds[rd] = (uint32_t)(G_BYTES + ch * X_CH + rho * X_ROW + c9 * 16);
+    } else {
+      c_goff[rd] = 0;
+      c_lds[rd] = 0;
+    }
+  }
+
   u32x4 stg[ROUNDS];
   auto issue_loads = [&](long long stage) {
     const int hp = (int)(stage % p.row_pairs);
-    const long long t = stage / p.row_pairs;
+    long long t = stage / p.row_pairs;
     const int ct = (int)(t % p.col_tiles);
-    const int n = (int)(t / p.col_tiles);
+    t /= p.col_tiles;
+    const int od = (int)(t % p.Dout);
+    const int n = (int)(t / p.Dout);
     const int oh0 = hp * SR, ow0 = ct * SW;
-    const int ih0 = oh0 - p.pad_h, iw0 = ow0 - p.pad_w;
+    const int id0 = od - p.pad_d, ih0 = oh0 - p.pad_h, iw0 = ow0 - p.pad_w;
+    const char* g_org = reinterpret_cast<const char*>(p.g) +
+                        2 * (((size_t)n * p.Cout * p.Dout + od) * plane_g + (size_t)oh0 * p.Wout + ow0);
+    const char* x_org = reinterpret_cast<const char*>(p.x) +
+                        2 * ((ptrdiff_t)((size_t)n * p.Cin * p.Din * plane_x) + (ptrdiff_t)id0 * (ptrdiff_t)plane_x +
+                             (ptrdiff_t)ih0 * p.Win + iw0);
+    const bool inside = EVEN && oh0 + SR <= p.Hout && ow0 + SW <= p.Wout && ih0 >= 0 &&
+                        ih0 + XR <= p.Hin && iw0 >= 0 && iw0 + X_CPR * 8 <= p.Win && id0 >= 0 &&
+                        id0 + (XC / p.Cin) <= p.Din;
+    if (inside) {
 #pragma unroll
-    for (int rd = 0; rd < ROUNDS; ++rd) {
-      const int q = tid + rd * THREADS;
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (q < G_CHUNKS) {
-        const int c8 = q & 7, r = (q >> 3) & (SR - 1), ch = q >> 4;
-        const int oh = oh0 + r, ow = ow0 + c8 * 8;
-        const uint16_t* src = p.g + ((size_t)n * C + ch) * plane_g + (size_t)oh * p.Wout + ow;
-        if (oh < p.Hout) {
-          if (ow + 8 <= p.Wout && (reinterpret_cast<uintptr_t>(src) & 3) == 0) {
-            v = *reinterpret_cast<const u32x4_a4*>(src);
-          } else {
-            uint32_t e[8];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) e[k] = (ow + k < p.Wout) ? (uint32_t)src[k] : 0u;
-            v.x = e[0] | (e[1] << 16); v.y = e[2] | (e[3] << 16);
-            v.z = e[4] | (e[5] << 16); v.w = e[6] | (e[7] << 16);
-          }
-        }
-      } else if (q < CHUNKS) {
-        const int qx = q - G_CHUNKS;
-        const int c9 = qx % X_CPR;
-        const int rr = qx / X_CPR;
-        const int rho = rr & (XR - 1), ch = rr >> 2;
-        const int ih = ih0 + rho, iw = iw0 + c9 * 8;
-        const uint16_t* src = p.x + ((size_t)n * C + ch) * plane_x + (ptrdiff_t)ih * p.Win + iw;
-        if (ih >= 0 && ih < p.Hin) {
-          if (EVEN && iw >= 0 && iw + 8 <= p.Win) {
-            v = *reinterpret_cast<const u32x4_a4*>(src);
-          } else {
-            uint32_t e[8];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) e[k] = (iw + k >= 0 && iw + k < p.Win) ? (uint32_t)src[k] : 0u;
-            v.x = e[0] | (e[1] << 16); v.y = e[2] | (e[3] << 16);
-            v.z = e[4] | (e[5] << 16); v.w = e[6] | (e[7] << 16);
-          }
+      for (int rd = 0; rd < ROUNDS; ++rd) {
+        if (tid + rd * THREADS < CHUNKS) {
+          const char* org = (tid + rd * THREADS < G_CHUNKS) ? g_org : x_org;
+          stg[rd] = *reinterpret_cast<const u32x4_a4*>(org + c_goff[rd]);
         }
       }
-      stg[rd] = v;
+    } else {
+#pragma unroll
+      for (int rd = 0; rd < ROUNDS; ++rd) {
+        const int q = tid + rd * THREADS;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (q < CHUNKS) {
+          const bool is_x = q >= G_CHUNKS;
+          const uint16_t* src;
+          int row, col, rows, cols;
+          bool ok = true;
+          if (!is_x) {
+            const int c8 = q & 7, r = (q >> 3) % SR;
+            src = reinterpret_cast<const uint16_t*>(g_org + c_goff[rd]);
+            row = oh0 + r; col = ow0 + c8 * 8; rows = p.Hout; cols = p.Wout;
+          } else {
+            const int qx = q - G_CHUNKS;
+            const int c9 = qx % X_CPR, rr = qx / X_CPR;
+            const int rho = rr % XR, ch = rr / XR;
+            src = reinterpret_cast<const uint16_t*>(x_org + c_goff[rd]);
+            row = ih0 + rho; col = iw0 + c9 * 8; rows = p.Hin; cols = p.Win;
+            const int dd = id0 + ch / p.Cin;
+            ok = dd >= 0 && dd < p.Din;
+          }
+          if (ok && row >= 0 && row < rows) {
+            if (col >= 0 && col + 8 <= cols && (reinterpret_cast<uintptr_t>(src) & 3) == 0) {
+              v = *reinterpret_cast<const u32x4_a4*>(src);
+            } else {
+              uint32_t e[8];
+#pragma unroll
+              for (int k = 0; k < 8; ++k) e[k] = (col + k >= 0 && col + k < cols) ? (uint32_t)src[k] : 0u;
+              v.x = e[0] | (e[1] << 16); v.y = e[2] | (e[3] << 16);
+              v.z = e[4] | (e[5] << 16); v.w = e[6] | (e[7] << 16);
+            }
+          }
+        }
+        stg[rd] = v;
+      }
     }
   };
 
   auto store_stage = [&](int buf) {
     unsigned char* base = smem + buf * STAGE_BYTES;
 #pragma unroll
-    for (int rd = 0; rd < ROUNDS; ++rd) {
-      const int q = tid + rd * THREADS;
-      if (q < G_CHUNKS) {
-        const int c8 = q & 7, r = (q >> 3) & (SR - 1), ch = q >> 4;
-        *reinterpret_cast<u32x4*>(base + ch * G_CH + r * (SW * 2) + c8 * 16) = stg[rd];
-      } else if (q < CHUNKS) {
-        const int qx = q - G_CHUNKS;
-        const int c9 = qx % X_CPR;
-        const int rr = qx / X_CPR;
-        const int rho = rr & (XR - 1), ch = rr >> 2;
-        *reinterpret_cast<u32x4*>(base + G_BYTES + ch * X_CH + rho * X_ROW + c9 * 16) = stg[rd];
-      }
-    }
+    for (int rd = 0; rd < ROUNDS; ++rd)
+      if (tid + rd * THREADS < CHUNKS) *reinterpret_cast<u32x4*>(base + c_lds[rd]) = stg[rd];
   };
 
   f32x16 acc[3][3];
@@ -157,8 +196,7 @@ __global__ __launch_bounds__(THREADS) void wgrad3x3_mfma_kernel(WgradParams p) {
     const unsigned char* gb = smem + buf * STAGE_BYTES + (cb * 32 + ln) * G_CH + kgp * 16;
     const unsigned char* xb = smem + buf * STAGE_BYTES + G_BYTES + (ib * 32 + ln) * X_CH + kgp * 16;
 #pragma unroll
-    for (int cgi = 0; cgi < 2; ++cgi) {
-      const int cg = half * 2 + cgi;  // 16-pixel column group of this wavefront
+    for (int cg = 0; cg < SW / 16; ++cg) {  // 16-pixel column groups of the stage
       bf16x8 a[SR];
 #pragma unroll
       for (int r = 0; r < SR; ++r)
@@ -197,15 +235,16 @@ __global__ __launch_bounds__(THREADS) void wgrad3x3_mfma_kernel(WgradParams p) {
     for (long long st = s_begin; st < s_end; ++st) {
       const bool has_next = st + 1 < s_end;
       if (has_next) issue_loads(st + 1);
-      compute_stage(buf);
+      if (wave < CWAVES) compute_stage(buf);
       if (has_next) store_stage(buf ^ 1);
       __syncthreads();
       buf ^= 1;
     }
   }
 
-  // partial of this wavefront: slot = workgroup * 2 + half, layout [tap][co][ci]
-  float* out = p.part + ((size_t)blockIdx.x * 2 + half) * PART;
+  // partial of this workgroup: layout [tap9][co][c']
+  if (wave >= CWAVES) return;
+  float* out = p.part + (size_t)blockIdx.x * (size_t)(9 * GC * XC);
 #pragma unroll
   for (int kh = 0; kh < 3; ++kh)
 #pragma unroll
@@ -213,29 +252,31 @@ __global__ __launch_bounds__(THREADS) void wgrad3x3_mfma_kernel(WgradParams p) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int co = cb * 32 + 8 * (i >> 2) + 4 * kgp + (i & 3);
-        out[((kh * 3 + kw) * C + co) * C + ib * 32 + ln] = acc[kh][kw][i];
+        out[((kh * 3 + kw) * GC + co) * XC + ib * 32 + ln] = acc[kh][kw][i];
       }
 }
 
-// out[co][ci][tap] (bf16) = sum over slots of part[slot][tap][co][ci], fixed order.
+// gw[co][ci][kd][kh][kw] (bf16) = sum over workgroups of part[wg][tap9][co][kd*Cin+ci].
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(uint16_t* __restrict__ gw,
                                                            const float* __restrict__ part,
-                                                           int slots) {
-  const int i = blockIdx.x * 256 + threadIdx.x;  // index in [tap][co][ci]
-  if (i >= PART) return;
+                                                           int slots, int GC, int XC, int Cin) {
+  const int count = 9 * GC * XC;
+  const int i = blockIdx.x * 256 + threadIdx.x;  // index in [tap9][co][c']
+  if (i >= count) return;
   // four independent chains keep the loads in flight; the order stays fixed
   float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
   int k = 0;
   for (; k + 4 <= slots; k += 4) {
-    s0 += part[(size_t)(k + 0) * PART + i];
-    s1 += part[(size_t)(k + 1) * PART + i];
-    s2 += part[(size_t)(k + 2) * PART + i];
-    s3 += part[(size_t)(k + 3) * PART + i];
+    s0 += part[(size_t)(k + 0) * count + i];
+    s1 += part[(size_t)(k + 1) * count + i];
+    s2 += part[(size_t)(k + 2) * count + i];
+    s3 += part[(size_t)(k + 3) * count + i];
   }
-  for (; k < slots; ++k) s0 += part[(size_t)k * PART + i];
+  for (; k < slots; ++k) s0 += part[(size_t)k * count + i];
   const float s = (s0 + s1) + (s2 + s3);
-  const int ci = i % C, co = (i / C) % C, tap = i / (C * C);
-  gw[(co * C + ci) * 9 + tap] = jg::f32_to_bf16(s);
+  const int cx = i % XC, co = (i / XC) % GC, tap = i / (XC * GC);
+  const int kd = cx / Cin, ci = cx % Cin, KD = XC / Cin;
+  gw[(((size_t)co * Cin + ci) * KD + kd) * 9 + tap] = jg::f32_to_bf16(s);
 }
 
 int cu_count() {
@@ -257,7 +298,37 @@ int wg_count(long long stages) {
 }
 
 long long stage_count(const ConvGeom& g) {
-  return g.batch * ((g.out[1] + SR - 1) / SR) * ((g.out[2] + SW - 1) / SW);
+  return g.batch * g.out[0] * ((g.out[1] + SR - 1) / SR) * ((g.out[2] + SW - 1) / SW);
+}
+
+// (CGB, CXB) of a geometry, or false when the kernel does not cover it
+bool blocks_of(const ConvGeom& g, int* cgb, int* cxb) {
+  if (g.k[1] != 3 || g.k[2] != 3 || (g.k[0] != 1 && g.k[0] != 3)) return false;
+  if (g.k[0] == 1 && g.in[0] != 1) return false;
+  for (int a = 0; a < 3; ++a)
+    if (g.s[a] != 1 || g.d[a] != 1) return false;
+  if (g.cin != 32 && g.cin != 64) return false;
+  if (g.cout != 32 && g.cout != 64) return false;
+  *cgb = g.cout / 32;
+  *cxb = g.k[0] * g.cin / 32;
+  if (*cgb * *cxb > 4) return false;
+  // per-lane byte offsets inside one batch entry are 32-bit
+  const size_t xs = (size_t)g.cin * g.in[0] * g.in[1] * g.in[2] * 2;
+  const size_t gs = (size_t)g.cout * g.out[0] * g.out[1] * g.out[2] * 2;
+  return xs < (1ull << 31) && gs < (1ull << 31);
+}
+
+template <int CGB, int CXB>
+int launch(const WgradParams& p, bool even, int wgs, hipStream_t s, const char* who) {
+  constexpr int THREADS = wgrad_threads(CGB, CXB);
+  const size_t lds = 2 * (size_t)(32 * CGB * G_CH + 32 * CXB * X_CH);
+  void (*kern)(WgradParams) =
+      even ? &wgrad3x3_mfma_kernel<CGB, CXB, true> : &wgrad3x3_mfma_kernel<CGB, CXB, false>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", who, lds);
+  kern<<<wgs, THREADS, lds, s>>>(p);
+  return JG_OK;
 }
 
 }  // namespace
@@ -265,21 +336,22 @@ long long stage_count(const ConvGeom& g) {
 namespace jg {
 
 bool mfma_wgrad_supported(const ConvGeom& g, int dtype) {
+  int cgb, cxb;
   if (dtype != JG_BF16 || g.batch <= 0) return false;
-  if (g.in[0] != 1 || g.k[0] != 1) return false;
-  if (g.k[1] != 3 || g.k[2] != 3) return false;
-  if (g.s[1] != 1 || g.s[2] != 1 || g.d[1] != 1 || g.d[2] != 1) return false;
-  if (g.cin != C || g.cout != C) return false;
-  return stage_count(g) < (1ll << 40);
+  return blocks_of(g, &cgb, &cxb);
 }
 
 size_t mfma_wgrad_workspace(const ConvGeom& g) {
-  return (size_t)wg_count(stage_count(g)) * 2 * PART * sizeof(float);
+  int cgb = 1, cxb = 1;
+  blocks_of(g, &cgb, &cxb);
+  return (size_t)wg_count(stage_count(g)) * 9 * (32 * cgb) * (32 * cxb) * sizeof(float);
 }
 
 int mfma_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, void* ws,
                size_t ws_bytes, hipStream_t s) {
   const char* who = "jg_conv_wgrad(mfma)";
+  int cgb, cxb;
+  if (!blocks_of(g, &cgb, &cxb)) JG_FAIL(JG_ERR_UNSUPPORTED, "%s: geometry not covered", who);
   if (ws == nullptr || ws_bytes < mfma_wgrad_workspace(g))
     JG_FAIL(JG_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes,
             mfma_wgrad_workspace(g));
@@ -289,26 +361,29 @@ int mfma_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, void*
   p.x = static_cast<const uint16_t*>(x);
   p.g = static_cast<const uint16_t*>(go);
   p.part = static_cast<float*>(ws);
-  p.N = (int)g.batch;
-  p.Hin = g.in[1]; p.Win = g.in[2]; p.Hout = g.out[1]; p.Wout = g.out[2];
-  p.pad_h = g.p[1]; p.pad_w = g.p[2];
+  p.Cin = g.cin; p.Cout = g.cout;
+  p.Din = g.in[0]; p.Hin = g.in[1]; p.Win = g.in[2];
+  p.Dout = g.out[0]; p.Hout = g.out[1]; p.Wout = g.out[2];
+  p.pad_d = g.p[0]; p.pad_h = g.p[1]; p.pad_w = g.p[2];
   p.row_pairs = (g.out[1] + SR - 1) / SR;
   p.col_tiles = (g.out[2] + SW - 1) / SW;
-  const long long stages = stage_count(g);
-  JG_REQUIRE(stages < (1ll << 31), "%s: too many stages", who);
-  p.total_stages = (int)stages;
-  const int wgs = wg_count(stages);
-  const bool even = (p.Win % 2 == 0) && (p.pad_w % 2 == 0) &&
-                    ((reinterpret_cast<uintptr_t>(x) & 3) == 0);
-  const size_t lds = 2 * (size_t)STAGE_BYTES;
-  void (*kern)(WgradParams) = even ? &wgrad3x3_mfma_kernel<true> : &wgrad3x3_mfma_kernel<false>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  if (e != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", who, lds);
-  kern<<<wgs, THREADS, lds, s>>>(p);
+  p.total_stages = stage_count(g);
+  const int wgs = wg_count(p.total_stages);
+  const bool even = (p.Win % 2 == 0) && (p.pad_w % 2 == 0) && (p.Wout % 2 == 0) &&
+                    ((reinterpret_cast<uintptr_t>(x) & 3) == 0) &&
+                    ((reinterpret_cast<uintptr_t>(go) & 3) == 0);
+  int rc;
+  if (cgb == 2 && cxb == 2) rc = launch<2, 2>(p, even, wgs, s, who);
+  else if (cgb == 1 && cxb == 3) rc = launch<1, 3>(p, even, wgs, s, who);
+  else if (cgb == 1 && cxb == 1) rc = launch<1, 1>(p, even, wgs, s, who);
+  else if (cgb == 2 && cxb == 1) rc = launch<2, 1>(p, even, wgs, s, who);
+  else if (cgb == 1 && cxb == 2) rc = launch<1, 2>(p, even, wgs, s, who);
+  else JG_FAIL(JG_ERR_UNSUPPORTED, "%s: channel blocking (%d, %d) not built", who, cgb, cxb);
+  if (rc) return rc;
   JG_CHECK_LAUNCH(who);
-  wgrad_reduce_kernel<<<(PART + 255) / 256, 256, 0, s>>>(static_cast<uint16_t*>(gw), p.part,
-                                                         wgs * 2);
+  const int count = 9 * 32 * cgb * 32 * cxb;
+  wgrad_reduce_kernel<<<(count + 255) / 256, 256, 0, s>>>(static_cast<uint16_t*>(gw), p.part, wgs,
+                                                          32 * cgb, 32 * cxb, g.cin);
   JG_CHECK_LAUNCH(who);
   return JG_OK;
 }
