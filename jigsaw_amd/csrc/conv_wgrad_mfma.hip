@@ -12,20 +12,18 @@
 //               channels) shifted by the tap. The kw shift is not 16-byte aligned in
 //               LDS, so a lane reads 10 consecutive pixels once (b128 + b32) and
 //               builds the three kw fragments with funnel shifts.
-//   Workgroup   one wavefront per (g channel block, x channel block) pair; it keeps
-//               its 9 taps x 32x32 fp32 accumulators in registers for the whole
-//               kernel (144 VGPRs) and walks the pixels. At most 4 wavefronts, one
-//               per SIMD, so each has the full register file: the prefetch path must
-//               not spill (a scratch reload there waits on every outstanding global
-//               load and serialises the pipeline). 64->64 2-D: 2x2 = 4 wavefronts;
-//               32->32 3-D: 1x3 = 3, plus one that only helps with the prefetch.
+//   Workgroup   one wavefront per (g channel block, x channel block, column half);
+//               it keeps its 9 taps x 32x32 fp32 accumulators in registers for the
+//               whole kernel (144 VGPRs) and walks the pixels. 64->64 2-D: 2x2x2 = 8
+//               wavefronts (two per SIMD, which is what hides the barrier and LDS
+//               write phases); 32->32 3-D: 1x3x2 = 6, plus two that only prefetch.
 //   Stage       2 output rows x 64 columns: g tile C x 2 x 64, x tile C' x 4 x 72;
 //               prefetched to registers during the MFMAs of the previous stage,
 //               double buffered in LDS (one barrier per stage). Channel strides in
 //               LDS are odd multiples of 16 bytes so that the 32 channel-lanes of a
 //               fragment read hit distinct banks. Stages that lie wholly inside the
 //               tensors (a wave-uniform test) take a branch-free vector load path.
-//   Reduction   every workgroup writes its partial to the workspace; a second kernel
+//   Reduction   every wavefront writes its partial to the workspace; a second kernel
 //               sums the partials in a fixed order (deterministic) and writes gw in
 //               the weight layout.
 #include "conv_common.h"
@@ -57,12 +55,17 @@ struct WgradParams {
   long long total_stages;  // N * Dout * col_tiles * row_pairs
 };
 
-constexpr int wgrad_threads(int cgb, int cxb) { return (cgb * cxb >= 3) ? 256 : 64 * cgb * cxb; }
+// Wavefronts per workgroup: (g block, x block) pairs x 2 column halves; a 6-wavefront
+// shape gets two more wavefronts that only help with the prefetch.
+constexpr int HALVES = 2;
+constexpr int wgrad_threads(int cgb, int cxb) {
+  return (cgb * cxb * HALVES > 4) ? 512 : 64 * cgb * cxb * HALVES;
+}
 
 template <int CGB, int CXB, bool EVEN>
 __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(WgradParams p) {
   constexpr int THREADS = wgrad_threads(CGB, CXB);
-  constexpr int CWAVES = CGB * CXB;  // wavefronts that own accumulators
+  constexpr int CWAVES = CGB * CXB * HALVES;  // wavefronts that own accumulators
   constexpr int GC = 32 * CGB, XC = 32 * CXB;
   constexpr int G_BYTES = GC * G_CH, X_BYTES = XC * X_CH;
   constexpr int STAGE_BYTES = G_BYTES + X_BYTES;
@@ -74,7 +77,7 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, kgp = lane >> 5;
-  const int pair = wave % (CGB * CXB);
+  const int pair = wave % (CGB * CXB), half = (wave / (CGB * CXB)) % HALVES;
   const int cb = pair / CXB, ib = pair % CXB;
 
   // contiguous range of stages for this workgroup; stage -> (n, d, column tile, row pair),
@@ -196,7 +199,8 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
     const unsigned char* gb = smem + buf * STAGE_BYTES + (cb * 32 + ln) * G_CH + kgp * 16;
     const unsigned char* xb = smem + buf * STAGE_BYTES + G_BYTES + (ib * 32 + ln) * X_CH + kgp * 16;
 #pragma unroll
-    for (int cg = 0; cg < SW / 16; ++cg) {  // 16-pixel column groups of the stage
+    for (int cgi = 0; cgi < SW / 16 / HALVES; ++cgi) {
+      const int cg = half * (SW / 16 / HALVES) + cgi;  // 16-pixel column group of this wavefront
       bf16x8 a[SR];
 #pragma unroll
       for (int r = 0; r < SR; ++r)
@@ -242,9 +246,9 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
     }
   }
 
-  // partial of this workgroup: layout [tap9][co][c']
+  // partial of this wavefront: slot = workgroup * HALVES + half, layout [tap9][co][c']
   if (wave >= CWAVES) return;
-  float* out = p.part + (size_t)blockIdx.x * (size_t)(9 * GC * XC);
+  float* out = p.part + ((size_t)blockIdx.x * HALVES + half) * (size_t)(9 * GC * XC);
 #pragma unroll
   for (int kh = 0; kh < 3; ++kh)
 #pragma unroll
@@ -344,7 +348,7 @@ bool mfma_wgrad_supported(const ConvGeom& g, int dtype) {
 size_t mfma_wgrad_workspace(const ConvGeom& g) {
   int cgb = 1, cxb = 1;
   blocks_of(g, &cgb, &cxb);
-  return (size_t)wg_count(stage_count(g)) * 9 * (32 * cgb) * (32 * cxb) * sizeof(float);
+  return (size_t)wg_count(stage_count(g)) * HALVES * 9 * (32 * cgb) * (32 * cxb) * sizeof(float);
 }
 
 int mfma_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, void* ws,
@@ -382,7 +386,7 @@ int mfma_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, void*
   if (rc) return rc;
   JG_CHECK_LAUNCH(who);
   const int count = 9 * 32 * cgb * 32 * cxb;
-  wgrad_reduce_kernel<<<(count + 255) / 256, 256, 0, s>>>(static_cast<uint16_t*>(gw), p.part, wgs,
+  wgrad_reduce_kernel<<<(count + 255) / 256, 256, 0, s>>>(static_cast<uint16_t*>(gw), p.part, wgs * HALVES,
                                                           32 * cgb, 32 * cxb, g.cin);
   JG_CHECK_LAUNCH(who);
   return JG_OK;
