@@ -1,0 +1,144 @@
+"""One rank's share of a Swin block on the GPU kernels of this package.
+
+Mirrors the example model of the reference (examples/swin.py:64-210): tokens are
+channels-last ``(B, h, w, C)`` tiles of a 2-D token grid; a block is
+``x + unshift(attn(shift(norm1(x))))`` followed by ``x + mlp(norm2(x))``. The
+LayerNorms run on the sharded-LayerNorm kernels (with a channel group of one), the
+shift / unshift on the DistributedRoll kernels, the windowed attention with its
+relative-position bias and shift mask on the attention core with an additive
+bias. The linear layers are plain ``nn.Linear`` (as in the reference example).
+"""
+
+from __future__ import annotations
+
+from collections.abc import Callable
+from typing import Any
+
+import torch
+import torch.nn as nn
+
+from .attention import window_attention
+from .conv import TileGroup
+from .layernorm import layer_norm
+from .roll import _Roll
+
+
+def windows(x: torch.Tensor, window: int) -> torch.Tensor:
+    """Cut a tile ``(B, h, w, C)`` into windows ``(B, nW, window*window, C)``
+    (examples/swin.py:85-89)."""
+    b, h, w, c = x.shape
+    x = x.view(b, h // window, window, w // window, window, c)
+    return x.permute(0, 1, 3, 2, 4, 5).reshape(b, -1, window * window, c)
+
+
+def unwindows(x: torch.Tensor, h: int, w: int, window: int) -> torch.Tensor:
+    """Inverse of :func:`windows` (examples/swin.py:92-96)."""
+    b, c = x.shape[0], x.shape[-1]
+    x = x.view(b, h // window, w // window, window, window, c)
+    return x.permute(0, 1, 3, 2, 4, 5).reshape(b, h, w, c)
+
+
+def relative_position_index(window: int) -> torch.Tensor:
+    """Index into the bias table for every pair of positions inside a window
+    (examples/swin.py:99-104)."""
+    ij = torch.stack(torch.meshgrid(*[torch.arange(window)] * 2, indexing="ij")).flatten(1)
+    rel = ij[:, :, None] - ij[:, None, :] + (window - 1)
+    return rel[0] * (2 * window - 1) + rel[1]
+
+
+def shift_mask(h: int, w: int, window: int, shift: int, groups: tuple) -> torch.Tensor:
+    """Mask ``(nW, N, N)`` of this tile's windows after rolling the token grid by
+    ``-shift``: tokens from the two sides of the image border must not attend to
+    each other; the border lies at the GLOBAL position, so the region of a token
+    follows from where the tile sits (examples/swin.py:107-126)."""
+
+    def region(local_size: int, group: Any) -> torch.Tensor:
+        size = local_size * group.size()
+        idx = group.rank() * local_size + torch.arange(local_size)
+        return (idx >= size - window).long() + (idx >= size - shift).long()
+
+    rows, cols = region(h, groups[0]), region(w, groups[1])
+    ids = (rows[:, None] * 3 + cols[None, :])[None, :, :, None]
+    ids = windows(ids, window).squeeze(-1).squeeze(0)
+    same = ids[:, :, None] == ids[:, None, :]
+    return torch.zeros(same.shape).masked_fill(~same, float("-inf"))
+
+
+class WindowAttention(nn.Module):
+    """Multi-head attention inside windows with a learned relative-position bias
+    (examples/swin.py:129-170); the attention core is this package's kernel."""
+
+    def __init__(self, dim: int, heads: int, window: int, tile: tuple, shift: int, groups: tuple, device) -> None:
+        super().__init__()
+        self.heads, self.window = heads, window
+        self.qkv = nn.Linear(dim, 3 * dim, device=device)
+        self.proj = nn.Linear(dim, dim, device=device)
+        self.bias_table = nn.Parameter(torch.zeros((2 * window - 1) ** 2, heads, device=device))
+        nn.init.trunc_normal_(self.bias_table, std=0.02)
+        self.register_buffer("index", relative_position_index(window).to(device), persistent=False)
+        if shift:
+            self.register_buffer("mask", shift_mask(*tile, window, shift, groups).to(device), persistent=False)
+        else:
+            self.mask = None
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        b, h, w, c = x.shape
+        x = windows(x, self.window)
+        n = x.shape[2]
+        qkv = self.qkv(x).view(b, -1, n, 3, self.heads, c // self.heads)
+        q, k, v = qkv.permute(3, 0, 1, 4, 2, 5).unbind(0)  # (B, nW, heads, N, d)
+        bias = self.bias_table[self.index.view(-1)].view(n, n, -1).permute(2, 0, 1).float()
+        if self.mask is not None:
+            bias = bias[None] + self.mask[:, None]  # (nW, heads, N, N)
+        out = window_attention(q.contiguous(), k.contiguous(), v.contiguous(), bias.contiguous())
+        out = out.transpose(2, 3).reshape(b, -1, n, c)
+        return unwindows(self.proj(out), h, w, self.window)
+
+
+class SwinBlock(nn.Module):
+    """``x + attn(norm(x))`` then ``x + mlp(norm(x))``; the windows may be shifted
+    (examples/swin.py:173-210). ``groups`` are the two spatial groups of the tile
+    (objects with ``size()`` / ``rank()``), ``comm_halo_1d_fn`` the 1-D exchange the
+    roll uses (``RollConfig.comm_halo_1d_fn`` in the reference)."""
+
+    def __init__(self, dim: int, heads: int, window: int, tile: tuple, groups: tuple = None,
+                 comm_halo_1d_fn: Callable | None = None, shift: int = 0, device=None, eps: float = 1e-5) -> None:
+        super().__init__()
+        groups = groups or (TileGroup(1, 0), TileGroup(1, 0))
+        self.groups, self.comm, self.shift_by, self.eps = groups, comm_halo_1d_fn, shift, eps
+        self.norm1 = nn.LayerNorm(dim, eps=eps, device=device)
+        self.attn = WindowAttention(dim, heads, window, tile, shift, groups, device)
+        self.norm2 = nn.LayerNorm(dim, eps=eps, device=device)
+        self.mlp = nn.Sequential(nn.Linear(dim, 4 * dim, device=device), nn.GELU(), nn.Linear(4 * dim, dim, device=device))
+
+    def _roll(self, x: torch.Tensor, shift: int) -> torch.Tensor:
+        if not shift:
+            return x
+        dist_dims = tuple(d for d, g in zip((1, 2), self.groups) if g.size() > 1)
+        dist_groups = tuple(g for g in self.groups if g.size() > 1)
+        return _Roll.apply(x.contiguous(), (shift, shift), (1, 2), dist_dims, dist_groups, self.comm)
+
+    def _norm(self, ln: nn.LayerNorm, x: torch.Tensor) -> torch.Tensor:
+        return layer_norm(x, ln.weight, ln.bias, None, self.eps)
+
+    # The block in stages, so that a single-process harness can run several ranks
+    # in lockstep (the two rolls are the only stages that talk to other ranks).
+    def pre_attention(self, x: torch.Tensor) -> torch.Tensor:
+        return self._norm(self.norm1, x)
+
+    def shift(self, y: torch.Tensor) -> torch.Tensor:
+        return self._roll(y, -self.shift_by)
+
+    def unshift(self, y: torch.Tensor) -> torch.Tensor:
+        return self._roll(y, self.shift_by)
+
+    def finish(self, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+        x = x + y.to(x.dtype)
+        return x + self.mlp(self._norm(self.norm2, x).to(x.dtype))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        y = self.unshift(self.attn(self.shift(self.pre_attention(x))))
+        return self.finish(x, y)
+
+
+__all__ = ["SwinBlock", "WindowAttention", "relative_position_index", "shift_mask", "unwindows", "windows"]

@@ -1,0 +1,125 @@
+"""One rank's Swin block on the GPU kernels against the block on the undivided grid
+(the reference's method, tests/test_examples.py:219-271) (GPU).
+
+Forward: every rank of a 2x2 mesh runs in this process, stage by stage; the slabs
+the two rolls exchange are produced by the roll oracle from the other ranks' stage
+outputs (pure copies, so exact). Backward: on a 1x1 mesh against autograd of the
+oracle block (the roll's backward exchange is covered by test_roll_gpu).
+Tolerance: 1e-4 of max|want| in fp32 (the reference's bound,
+tests/test_examples.py:48-67); rel-L2 2e-2 in bf16.
+"""
+
+import pytest
+import torch
+
+from helpers import mesh_coords, rel_l2
+from jigsaw_amd import swin as js
+from jigsaw_amd.conv import TileGroup
+from oracle import roll as orl
+from oracle import swin as osw
+
+pytestmark = pytest.mark.gpu
+
+DIM, HEADS, WINDOW = 32, 2, 4
+
+
+class Answers:
+    """Stand-in for RollConfig.comm_halo_1d_fn: hands over precomputed slabs."""
+
+    def __init__(self):
+        self.queue = []
+
+    def __call__(self, data, buffer, direction, *, group, async_op):
+        buffer.copy_(self.queue.pop(0).to(buffer.device))
+        return buffer, None
+
+
+def _tiles(glob, mesh, n):
+    return {c: glob[:, c[0] * n[0] : (c[0] + 1) * n[0], c[1] * n[1] : (c[1] + 1) * n[1]].contiguous() for c in mesh_coords(mesh)}
+
+
+def _roll_all(blocks, comms, stage_in, mesh, shift, which):
+    """Run the shift / unshift stage of every rank; exchange answers from the roll oracle."""
+    if shift == 0:
+        return {c: getattr(blocks[c], which)(t) for c, t in stage_in.items()}
+    cpu = {c: t.detach().cpu() for c, t in stage_in.items()}
+    local = {c: torch.roll(t, (shift, shift), (1, 2)) for c, t in cpu.items()}
+    after_h = orl.distributed_roll_mesh({c: t.clone() for c, t in cpu.items()}, mesh, (shift, shift), (1, 2), [1])
+    direction = 1 if shift > 0 else -1
+    sl = slice(0, shift) if shift > 0 else slice(shift, None)
+    out = {}
+    for c in mesh_coords(mesh):
+        src_h = ((c[0] - direction) % mesh[0], c[1])
+        src_w = (c[0], (c[1] - direction) % mesh[1])
+        comms[c].queue = [local[src_h][:, sl].contiguous(), after_h[src_w][:, :, sl].contiguous()]
+        out[c] = getattr(blocks[c], which)(stage_in[c])
+        assert not comms[c].queue
+    return out
+
+
+@pytest.mark.parametrize("shift", [0, 2])
+def test_swin_block_forward_tiled_equals_undivided(shift, dev):
+    torch.manual_seed(0)
+    mesh, n = (2, 2), (8, 8)
+    B = 2
+    glob = torch.randn(B, n[0] * 2, n[1] * 2, DIM)
+    ref_block = js.SwinBlock(DIM, HEADS, WINDOW, (n[0] * 2, n[1] * 2), shift=shift, device=dev)
+    with torch.no_grad():
+        ref_block.attn.bias_table.normal_(0, 0.5)
+    params = {k: v.detach().double().cpu() for k, v in ref_block.state_dict().items()}
+    want = osw.block(glob.double(), params, HEADS, WINDOW, shift)
+
+    tiles = _tiles(glob, mesh, n)
+    blocks, comms = {}, {}
+    for c in mesh_coords(mesh):
+        comms[c] = Answers()
+        groups = (TileGroup(mesh[0], c[0]), TileGroup(mesh[1], c[1]))
+        blocks[c] = js.SwinBlock(DIM, HEADS, WINDOW, n, groups, comms[c], shift=shift, device=dev)
+        blocks[c].load_state_dict(ref_block.state_dict())
+    with torch.no_grad():
+        x = {c: t.to(dev) for c, t in tiles.items()}
+        y = {c: blocks[c].pre_attention(x[c]) for c in x}
+        y = _roll_all(blocks, comms, y, mesh, -shift, "shift")
+        y = {c: blocks[c].attn(y[c]) for c in y}
+        y = _roll_all(blocks, comms, y, mesh, shift, "unshift")
+        out = {c: blocks[c].finish(x[c], y[c]) for c in x}
+    want_tiles = _tiles(want, mesh, n)
+    bound = 1e-4 * want.abs().max().item()
+    for c in mesh_coords(mesh):
+        err = (out[c].double().cpu() - want_tiles[c]).abs().max().item()
+        assert err < bound, f"rank {c}: max err {err:.3e} >= {bound:.3e}"
+
+
+@pytest.mark.parametrize("shift", [0, 2])
+def test_swin_block_backward_matches_autograd(shift, dev):
+    torch.manual_seed(1)
+    n = (8, 12)
+    x = torch.randn(2, *n, DIM)
+    block = js.SwinBlock(DIM, HEADS, WINDOW, n, shift=shift, device=dev)
+    with torch.no_grad():
+        block.attn.bias_table.normal_(0, 0.5)
+    params = {k: v.detach().double().cpu().requires_grad_() for k, v in block.state_dict().items()}
+    xd = x.double().requires_grad_()
+    want = osw.block(xd, params, HEADS, WINDOW, shift)
+    g = torch.randn_like(want)
+    want.backward(g)
+    xg = x.to(dev).requires_grad_()
+    out = block(xg)
+    out.backward(g.float().to(dev))
+    assert rel_l2(out, want.detach()) < 1e-5
+    assert rel_l2(xg.grad, xd.grad) < 1e-4, f"dx {rel_l2(xg.grad, xd.grad):.3e}"
+    for name, prm in block.named_parameters():
+        assert rel_l2(prm.grad, params[name].grad) < 1e-4, f"{name}: {rel_l2(prm.grad, params[name].grad):.3e}"
+
+
+def test_swin_block_bf16_config5_shape(dev):
+    """Config 5 shape (reduced tile): dim 128, 4 heads, 8x8 windows, shift 4, bf16 tokens."""
+    torch.manual_seed(2)
+    n, dim, heads, window, shift = (64, 64), 128, 4, 8, 4
+    x = torch.randn(1, *n, dim)
+    block = js.SwinBlock(dim, heads, window, n, shift=shift, device=dev)
+    params = {k: v.detach().double().cpu() for k, v in block.state_dict().items()}
+    want = osw.block(x.double(), params, heads, window, shift)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = block(x.to(dev))
+    assert rel_l2(out, want) < 2e-2
