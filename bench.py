@@ -34,7 +34,7 @@ METRIC = "halo-conv fwd+bwd & ring-attn step TFLOP/s on 1 GPU; % MFMA peak; halo
 
 # HBM bytes per launch of the forward conv kernel (FETCH_SIZE + WRITE_SIZE from
 # rocprofv3 --pmc, scaled by a copy kernel of known size); None until measured.
-CONV_FWD_TRAFFIC_BYTES = None
+CONV_FWD_TRAFFIC_BYTES = 2.41e9  # profiles/conv2d_cfg2_attn_cfg4_hbm_traffic.txt
 
 
 def _events():
@@ -129,6 +129,72 @@ def attention_figures(dev, iters: int) -> dict:
         "attn_bwd_step": {"ms": ms_b, "tflops": tf(f_bwd, ms_b), "frac_mfma_peak": tf(f_bwd, ms_b) / PEAK_BF16_TFLOPS},
         "attn_ring_fwd_4_steps": {"ms": ms_ring, "tflops": tf(4 * f_fwd, ms_ring)},
         "ln_partial_stats": {"ms": ms_ln, "GBps": x.numel() * 2 / (ms_ln * 1e-3) / 1e9, "bytes": x.numel() * 2},
+    }
+
+
+def conv3d_figures(dev, iters: int) -> dict:
+    """Configuration 3: one rank's 128^3 tile of a 256^3 volume, batch 2, 32 -> 32
+    channels, 3x3x3, pad 1, bf16; 26 seeded halo strips of width 1."""
+    from jigsaw_amd import conv as jc
+    from jigsaw_amd.halo import HaloGeometry, halo_assemble, halo_fold
+
+    g = torch.Generator(device=dev).manual_seed(1)
+    n, lead, ch = (128, 128, 128), (2, 32), 32
+    geom = HaloGeometry(n, (1, 1, 1), (1, 1, 1))
+    x = torch.randn(*lead, *n, device=dev, generator=g).bfloat16()
+    bound = 1.0 / (ch * 27) ** 0.5
+    w = ((torch.rand(ch, ch, 3, 3, 3, device=dev, generator=g) * 2 - 1) * bound).bfloat16()
+    gout = torch.randn(*lead, *n, device=dev, generator=g).bfloat16()
+    sf = {o: torch.randn(*lead, *geom.strip_extent(o, "assemble"), device=dev, generator=g).bfloat16() for o in geom.offsets()}
+    sb = {o: torch.randn(*lead, *geom.strip_extent(o, "fold"), device=dev, generator=g).bfloat16() for o in geom.offsets()}
+    x_aug = halo_assemble(x, sf, geom)
+    gx_aug = jc.conv_nd_input(x_aug.shape, w, gout)
+    flop = 2 * lead[0] * ch * ch * 27 * n[0] * n[1] * n[2]
+    nbytes = (x.numel() + x_aug.numel()) * 2
+    ms = {
+        "fwd": time_gpu(lambda: jc.conv_nd(x_aug, w, None), iters),
+        "dgrad": time_gpu(lambda: jc.conv_nd_input(x_aug.shape, w, gout), iters),
+        "wgrad": time_gpu(lambda: jc.conv_nd_weight(x_aug, w.shape, gout), iters),
+    }
+    gx = torch.empty_like(x)
+    ms_asm = time_gpu(lambda: halo_assemble(x, sf, geom, out=x_aug), iters)
+    ms_fold = time_gpu(lambda: halo_fold(gx_aug, sb, geom, out=gx), iters)
+    out = {f"conv3d_{k}": {"ms": v, "tflops": flop / (v * 1e-3) / 1e12, "frac_mfma_peak": flop / (v * 1e-3) / 1e12 / PEAK_BF16_TFLOPS} for k, v in ms.items()}
+    out["halo3d_assemble"] = {"ms": ms_asm, "GBps": nbytes / (ms_asm * 1e-3) / 1e9, "frac_hbm_peak": nbytes / (ms_asm * 1e-3) / 1e9 / PEAK_HBM_GBPS}
+    out["halo3d_fold"] = {"ms": ms_fold, "GBps": nbytes / (ms_fold * 1e-3) / 1e9, "frac_hbm_peak": nbytes / (ms_fold * 1e-3) / 1e9 / PEAK_HBM_GBPS}
+    return out
+
+
+def swin_figures(dev, iters: int) -> dict:
+    """Configuration 5: one rank's Swin block on a 256x256-token tile, dim 128, 4 heads,
+    8x8 windows, shift 4, bf16 autocast; the roll's cross-tile slabs are seeded."""
+    from jigsaw_amd import roll as jr
+    from jigsaw_amd import swin as js
+    from jigsaw_amd.conv import TileGroup
+
+    g = torch.Generator(device=dev).manual_seed(2)
+
+    def comm(data, buffer, direction, *, group, async_op):
+        buffer.normal_(generator=g)  # the neighbour's slab: seeded stand-in
+        return buffer, None
+
+    n, dim = (256, 256), 128
+    groups = (TileGroup(2, 0), TileGroup(2, 1))
+    block = js.SwinBlock(dim, 4, 8, n, groups, comm, shift=4, device=dev)
+    x = torch.randn(1, *n, dim, device=dev, generator=g).bfloat16().requires_grad_()
+    gout = torch.randn(1, *n, dim, device=dev, generator=g).bfloat16()
+
+    def step():
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            y = block(x)
+        y.backward(gout)
+
+    ms = time_gpu(step, max(3, iters // 2))
+    xr = x.detach()
+    ms_roll = time_gpu(lambda: jr.roll(xr, (-4, -4), (1, 2)), iters)
+    return {
+        "swin_block_fwd_bwd": {"ms": ms},
+        "roll": {"ms": ms_roll, "GBps": 2 * xr.numel() * 2 / (ms_roll * 1e-3) / 1e9, "bytes": 2 * xr.numel() * 2},
     }
 
 
@@ -234,8 +300,9 @@ def main() -> int:
     ms_fwd = time_gpu(lambda: jc.conv_nd(x_aug, wl["w"], wl["b"]), it)
     ms_dgrad = time_gpu(lambda: jc.conv_nd_input(x_aug.shape, wl["w"], wl["g"]), it)
     ms_wgrad = time_gpu(lambda: jc.conv_nd_weight(x_aug, wl["w"].shape, wl["g"]), it)
-    ms_asm = time_gpu(lambda: halo_assemble(wl["x"], wl["strips_fwd"], geom), it)
-    ms_fold = time_gpu(lambda: halo_fold(gx_aug, wl["strips_bwd"], geom), it)
+    gx_buf = torch.empty_like(wl["x"])
+    ms_asm = time_gpu(lambda: halo_assemble(wl["x"], wl["strips_fwd"], geom, out=x_aug), it)
+    ms_fold = time_gpu(lambda: halo_fold(gx_aug, wl["strips_bwd"], geom, out=gx_buf), it)
     es = wl["x"].element_size()
     strip_bytes = sum(t.numel() for t in wl["strips_fwd"].values()) * es
     halo_bytes = (wl["x"].numel() + x_aug.numel()) * es + strip_bytes  # read tile + strips, write padded tile
@@ -264,6 +331,8 @@ def main() -> int:
         "halo_fold": {"ms": ms_fold, "GBps": gbps(ms_fold), "frac_hbm_peak": gbps(ms_fold) / PEAK_HBM_GBPS, "bytes": halo_bytes},
     }
     extra.update(attention_figures(dev, max(10, it)))
+    extra.update(conv3d_figures(dev, it))
+    extra.update(swin_figures(dev, it))
 
     line = {
         "metric": METRIC,

@@ -1,0 +1,58 @@
+"""Small driver for rocprofv3 runs: launches each hot kernel of configuration 2
+(and 4) a few times, plus a plain device copy of known size that calibrates the
+FETCH_SIZE / WRITE_SIZE counters.
+
+    rocprofv3 --kernel-trace --stats -d OUT -o kt --output-format csv -- python3 -m jigsaw_amd.profile_kernels
+    rocprofv3 --pmc FETCH_SIZE -d OUT -o fetch --output-format csv -- python3 -m jigsaw_amd.profile_kernels
+    rocprofv3 --pmc WRITE_SIZE -d OUT -o write --output-format csv -- python3 -m jigsaw_amd.profile_kernels
+"""
+
+from __future__ import annotations
+
+import sys
+
+import torch
+
+
+def main(reps: int = 3) -> None:
+    from jigsaw_amd import attention as ja
+    from jigsaw_amd import conv as jc
+    from jigsaw_amd.halo import HaloGeometry, halo_assemble, halo_fold
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(0)
+    batch, ch, tile = 8, 64, 1024
+    geom = HaloGeometry((tile, tile), (1, 1), (1, 1))
+    lead = (batch, ch)
+    x = torch.randn(*lead, tile, tile, device=dev, generator=g).bfloat16()
+    w = ((torch.rand(ch, ch, 3, 3, device=dev, generator=g) * 2 - 1) / 24).bfloat16()
+    b = ((torch.rand(ch, device=dev, generator=g) * 2 - 1) / 24).bfloat16()
+    gout = torch.randn(*lead, tile, tile, device=dev, generator=g).bfloat16()
+    sf = {o: torch.randn(*lead, *geom.strip_extent(o, "assemble"), device=dev, generator=g).bfloat16() for o in geom.offsets()}
+    sb = {o: torch.randn(*lead, *geom.strip_extent(o, "fold"), device=dev, generator=g).bfloat16() for o in geom.offsets()}
+    x_aug = halo_assemble(x, sf, geom)
+    gx_aug = jc.conv_nd_input(x_aug.shape, w, gout)
+    gx = torch.empty_like(x)
+    copy_dst = torch.empty_like(x)  # calibration copy: reads and writes x.numel() * 2 bytes
+    q = (torch.randn(1, 8, 4096, 64, device=dev, generator=g) / 8).bfloat16()
+    k = torch.randn(1, 8, 4096, 64, device=dev, generator=g).bfloat16()
+    v = torch.randn(1, 8, 4096, 64, device=dev, generator=g).bfloat16()
+    acc = torch.zeros(1, 8, 4096, 64, device=dev)
+    lse = torch.full((1, 8, 4096), float("-inf"), device=dev)
+    out, l = ja.core_forward(q, k, v, 0.125)
+    for _ in range(reps):
+        copy_dst.copy_(x)
+        halo_assemble(x, sf, geom, out=x_aug)
+        jc.conv_nd(x_aug, w, b)
+        jc.conv_nd_input(x_aug.shape, w, gout)
+        jc.conv_nd_weight(x_aug, w.shape, gout)
+        jc.sum_grad_bias(gout, 2)
+        halo_fold(gx_aug, sb, geom, out=gx)
+        ja.core_forward(q, k, v, 0.125, out_acc=acc, lse_acc=lse, want_out=False)
+        ja.core_backward(gout[0, :8, :, :64].reshape(1, 8, 1024 * 1, 64).expand(1, 8, 1024, 64).repeat(1, 1, 4, 1), q, k, v, out, l, 0.125)
+    torch.cuda.synchronize()
+    print("profile_kernels: done", file=sys.stderr)
+
+
+if __name__ == "__main__":
+    main()
