@@ -64,3 +64,16 @@ def special_values_(t: torch.Tensor) -> torch.Tensor:
         flat[3::11] = 0.0
         flat[5::13] = 1e-39 if t.dtype == torch.float32 else 1e-39
     return t
+
+
+def kaiming_uniform_bound(c_in, kernel, a=5 ** 0.5):
+    """Half-width of the uniform weight distribution jigsaw's layers initialise with.
+
+    Follows jigsaw/init.py:115-158 as called from convolution/_conv/base.py:236-238 (a = sqrt(5)):
+    gain = sqrt(2 / (1 + a^2)), bound = sqrt(3) * gain / sqrt(fan_in), fan_in = c_in * prod(kernel).
+    """
+    fan_in = c_in
+    for k in kernel:
+        fan_in *= k
+    gain = (2.0 / (1.0 + a * a)) ** 0.5
+    return (3.0 ** 0.5) * gain / fan_in ** 0.5

@@ -134,3 +134,17 @@ def test_scatter_add_clears_negative_zero():
     grads = {(0, 0): torch.full((1, 1, 6, 4), -0.0), (1, 0): torch.full((1, 1, 6, 4), -0.0)}
     folded = oh.scatter_add_mesh(grads, mesh, k, s, p, d, n)
     assert not torch.signbit(folded[(0, 0)]).any()
+
+
+def test_gather_preserves_negative_zero():
+    """The forward halo is a pure copy: a -0.0 in a neighbour's rows arrives as -0.0 (bit pattern kept)."""
+    mesh, k, s, p, d = (2, 2), (3, 3), (1, 1), (1, 1), (1, 1)
+    x = torch.full((1, 1, 8, 8), -0.0)
+    tiles = oh.split_global(x, mesh)
+    aug = oh.gather_mesh(tiles, mesh, k, s, p, d)
+    t = aug[(0, 0)]
+    assert t.shape[-2:] == (6, 6)
+    bits = t.view(torch.int32)
+    sign = torch.tensor(-0.0).view(torch.int32)
+    assert (bits[..., 1:, 1:] == sign).all()       # own tile and the live neighbours' rows
+    assert (bits[..., 0, :] == 0).all() and (bits[..., :, 0] == 0).all()  # out-of-domain border is +0.0

@@ -165,3 +165,16 @@ def test_window_attention_oracle_equals_sdpa():
     bias[0, :, :, 3] = float("-inf")
     want = F.scaled_dot_product_attention(q, k, v, attn_mask=bias)
     torch.testing.assert_close(oa.window_attention(q, k, v, bias), want, atol=1e-12, rtol=1e-10)
+
+
+def test_kaiming_bound_closed_form():
+    """With a = sqrt(5) the bound collapses to 1/sqrt(fan_in); torch's own initialiser stays inside it."""
+    from helpers import kaiming_uniform_bound
+
+    assert abs(kaiming_uniform_bound(64, (3, 3)) - 1.0 / 24.0) < 1e-12
+    assert abs(kaiming_uniform_bound(32, (3, 3, 3)) - 864 ** -0.5) < 1e-12
+    torch.manual_seed(0)
+    w = torch.empty(64, 64, 3, 3)
+    torch.nn.init.kaiming_uniform_(w, a=5 ** 0.5)
+    bound = kaiming_uniform_bound(64, (3, 3))
+    assert w.abs().max() <= bound and w.abs().max() > 0.99 * bound
