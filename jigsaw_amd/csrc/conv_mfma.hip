@@ -57,6 +57,7 @@ __device__ __forceinline__ int in_slot(int col) { return (col & 7) * OCTS + (col
 
 struct FwdParams {
   const uint16_t* x;    // (N, C, Din, Hin, Win) bf16: the tensor that is convolved
+  const char* x_end;    // one past the last byte of x
   const u32x4* wprep;   // prepared weights, [m_tile][tap9][c16][kg][MT][8]
   const uint16_t* bias; // (M,) or NULL
   uint16_t* y;          // (N, M, Dout, Hout, Wout)
@@ -177,8 +178,11 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(FwdParams p) {
     const char* origin = reinterpret_cast<const char*>(p.x) +
                          2 * ((ptrdiff_t)(((size_t)tc.n * p.C + c0) * chan_stride) +
                               (ptrdiff_t)id * (ptrdiff_t)plane + (ptrdiff_t)ih0 * p.Win + iw0);
+    // The last octet of a row holds 2 pixels that are used and 6 that no fragment
+    // reads, so it may run past the row end as long as it stays inside the tensor.
+    const char* last = origin + 2 * ((size_t)(CK - 1) * chan_stride + (size_t)(IN_ROWS - 1) * p.Win + OCTS * 8);
     const bool interior = depth_ok && ih0 >= 0 && ih0 + IN_ROWS <= p.Hin && iw0 >= 0 &&
-                          iw0 + OCTS * 8 <= p.Win;
+                          iw0 + TW + KW - 1 <= p.Win && last <= p.x_end;
     if (!has_task) return;
     const char* a = origin + t_off;
     if (EVEN && interior) {
@@ -393,6 +397,7 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   JG_CHECK_LAUNCH(who);
 
   FwdParams p;
+  p.x_end = reinterpret_cast<const char*>(L.x) + 2 * (size_t)L.N * L.C * L.Din * L.Hin * L.Win;
   p.x = L.x; p.wprep = reinterpret_cast<const u32x4*>(wprep); p.bias = L.bias; p.y = L.y;
   p.N = L.N; p.C = L.C; p.M = L.M; p.KD = L.KD;
   p.Din = L.Din; p.Hin = L.Hin; p.Win = L.Win;

@@ -47,7 +47,8 @@ constexpr int X_CPR = 9;                      // 8-pixel chunks per x row
 struct WgradParams {
   const uint16_t* x;  // (N, Cin, Din, Hin, Win)
   const uint16_t* g;  // (N, Cout, Dout, Hout, Wout)
-  float* part;        // [workgroup][tap9][co][c']
+  const char* x_end;  // one past the last byte of x
+  float* part;        // [wavefront slot][tap9][co][c']
   int Cin, Cout;
   int Din, Hin, Win, Dout, Hout, Wout;
   int pad_d, pad_h, pad_w;
@@ -129,9 +130,13 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
     const char* x_org = reinterpret_cast<const char*>(p.x) +
                         2 * ((ptrdiff_t)((size_t)n * p.Cin * p.Din * plane_x) + (ptrdiff_t)id0 * (ptrdiff_t)plane_x +
                              (ptrdiff_t)ih0 * p.Win + iw0);
+    // The last 8-pixel chunk of an x row holds 2 pixels that are used and 6 that no
+    // fragment reads, so it may run past the row end as long as it stays inside the tensor.
+    const char* x_last = x_org + 2 * ((size_t)(p.Cin - 1) * x_cs + (size_t)(XC / p.Cin - 1) * plane_x +
+                                      (size_t)(XR - 1) * p.Win + X_CPR * 8);
     const bool inside = EVEN && oh0 + SR <= p.Hout && ow0 + SW <= p.Wout && ih0 >= 0 &&
-                        ih0 + XR <= p.Hin && iw0 >= 0 && iw0 + X_CPR * 8 <= p.Win && id0 >= 0 &&
-                        id0 + (XC / p.Cin) <= p.Din;
+                        ih0 + XR <= p.Hin && iw0 >= 0 && iw0 + SW + 2 <= p.Win && id0 >= 0 &&
+                        id0 + (XC / p.Cin) <= p.Din && x_last <= p.x_end;
     if (inside) {
 #pragma unroll
       for (int rd = 0; rd < ROUNDS; ++rd) {
@@ -365,6 +370,7 @@ int mfma_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, void*
   p.x = static_cast<const uint16_t*>(x);
   p.g = static_cast<const uint16_t*>(go);
   p.part = static_cast<float*>(ws);
+  p.x_end = static_cast<const char*>(x) + 2 * (size_t)g.batch * g.cin * g.in[0] * g.in[1] * g.in[2];
   p.Cin = g.cin; p.Cout = g.cout;
   p.Din = g.in[0]; p.Hin = g.in[1]; p.Win = g.in[2];
   p.Dout = g.out[0]; p.Hout = g.out[1]; p.Wout = g.out[2];
