@@ -122,7 +122,10 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(FwdParams p) {
   const int wrow0 = (wave >> 1) * WROWS, wcol0 = (wave & 1) * 32;
   const int mt = blockIdx.y;
 
-  // ---- tile schedule: XCD x (= blockIdx.x % 8) owns a contiguous range
+  // ---- tile schedule: XCD x (= blockIdx.x % 8) owns a contiguous range of tiles and
+  // walks it cyclically from a start that differs per XCD. Without the stagger, ranges
+  // that coincide with whole images make the 8 XCDs stream addresses that differ by a
+  // multiple of the image size in lockstep, which piles them onto the same memory channels.
   const int G = gridDim.x;
   const int xcd = blockIdx.x & 7, slot_in_xcd = blockIdx.x >> 3;
   const int wg_per_xcd = (G + 7) >> 3;
@@ -130,8 +133,15 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(FwdParams p) {
   const int t_begin = xcd * per_xcd;
   int t_end = t_begin + per_xcd;
   if (t_end > p.total_tiles) t_end = p.total_tiles;
-  const int t_first = t_begin + slot_in_xcd;
-  if (t_first >= t_end) return;
+  const int t_len = t_end - t_begin;
+  if (slot_in_xcd >= t_len) return;
+  const int t_rot = (int)(((long long)xcd * t_len) >> 3);
+  const int my_tiles = (t_len - slot_in_xcd + wg_per_xcd - 1) / wg_per_xcd;
+  auto tile_of = [&](int ti) {  // ti-th tile of this workgroup
+    int i = slot_in_xcd + ti * wg_per_xcd + t_rot;
+    if (i >= t_len) i -= t_len;
+    return t_begin + i;
+  };
 
   // ---- resident weights and bias
   {
@@ -314,29 +324,32 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(FwdParams p) {
     }
   };
 
-  // ---- main loop
+  // ---- main loop over the stages (tile, 16-channel step) of this workgroup. The
+  // global loads of a stage are issued a whole stage ahead: right after the previous
+  // stage's registers were written to LDS, in the middle of the stage before.
+  const int stages = my_tiles * p.nc16;
+  auto issue_stage = [&](int q) {
+    const int ti = q / p.nc16;
+    issue_loads(tile_of(ti), q - ti * p.nc16);
+  };
   int buf = 0;
-  issue_loads(t_first, 0);
+  issue_stage(0);
   store_stage(0);
+  if (stages > 1) issue_stage(1);
   __syncthreads();
-  for (int tile = t_first; tile < t_end; tile += wg_per_xcd) {
+  int q = 0;
+  for (int ti = 0; ti < my_tiles; ++ti) {
     init_acc();
-    for (int c16 = 0; c16 < p.nc16; ++c16) {
-      int nt = tile, nc = c16 + 1;
-      if (nc == p.nc16) {
-        nc = 0;
-        nt = tile + wg_per_xcd;
-      }
-      const bool has_next = nt < t_end;
-      if (has_next) issue_loads(nt, nc);
+    for (int c16 = 0; c16 < p.nc16; ++c16, ++q) {
       compute_kw(buf, c16, 0);
       compute_kw(buf, c16, 1);
-      if (has_next) store_stage(buf ^ 1);  // other buffer: no hazard with this stage's reads
+      if (q + 1 < stages) store_stage(buf ^ 1);  // other buffer: no hazard with this stage's reads
+      if (q + 2 < stages) issue_stage(q + 2);
       compute_kw(buf, c16, 2);
       __syncthreads();
       buf ^= 1;
     }
-    epilogue(tile);
+    epilogue(tile_of(ti));
   }
 }
 

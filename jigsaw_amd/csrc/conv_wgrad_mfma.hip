@@ -200,11 +200,11 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.0f;
 
-  auto compute_stage = [&](int buf) {
+  // one 16-pixel column group (cgi = 0 or 1 of this wavefront's half) of a stage
+  auto compute_group = [&](int buf, int cgi) {
     const unsigned char* gb = smem + buf * STAGE_BYTES + (cb * 32 + ln) * G_CH + kgp * 16;
     const unsigned char* xb = smem + buf * STAGE_BYTES + G_BYTES + (ib * 32 + ln) * X_CH + kgp * 16;
-#pragma unroll
-    for (int cgi = 0; cgi < SW / 16 / HALVES; ++cgi) {
+    {
       const int cg = half * (SW / 16 / HALVES) + cgi;  // 16-pixel column group of this wavefront
       bf16x8 a[SR];
 #pragma unroll
@@ -236,16 +236,20 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
     }
   };
 
+  // The global loads of a stage are issued a whole stage ahead: right after the previous
+  // stage's registers went to LDS, between the two column groups of the stage before.
+  static_assert(SW / 16 / HALVES == 2, "the stage loop is written for two column groups per wavefront");
   if (s_begin < s_end) {
     int buf = 0;
     issue_loads(s_begin);
     store_stage(0);
+    if (s_begin + 1 < s_end) issue_loads(s_begin + 1);
     __syncthreads();
     for (long long st = s_begin; st < s_end; ++st) {
-      const bool has_next = st + 1 < s_end;
-      if (has_next) issue_loads(st + 1);
-      if (wave < CWAVES) compute_stage(buf);
-      if (has_next) store_stage(buf ^ 1);
+      if (wave < CWAVES) compute_group(buf, 0);
+      if (st + 1 < s_end) store_stage(buf ^ 1);
+      if (st + 2 < s_end) issue_loads(st + 2);
+      if (wave < CWAVES) compute_group(buf, 1);
       __syncthreads();
       buf ^= 1;
     }
