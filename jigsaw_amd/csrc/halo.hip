@@ -388,6 +388,7 @@ struct RowPlan {
 };
 
 typedef uint32_t u32x4_s4 __attribute__((ext_vector_type(4), aligned(4)));
+constexpr int ROW_BATCH = 4;  // vectors a lane keeps in flight
 
 template <typename T>
 __global__ __launch_bounds__(256) void assemble_rows_kernel(Table tab, T* __restrict__ dst,
@@ -417,37 +418,40 @@ __global__ __launch_bounds__(256) void assemble_rows_kernel(Table tab, T* __rest
   if (s2 != nullptr) s2 += line * g.hi[2];
   T* drow = dst + (long long)row * Wa;
   const int mid_lo = g.lo[2], mid_hi = g.lo[2] + g.n[2];
-  for (int it = 0; it < pl.iters; ++it) {
-    const int j = lir + (it << pl.lpr_log2);
-    if (j >= pl.nvec) break;
-    const int c0 = j * V;
-    if (c0 >= mid_lo && c0 + V <= mid_hi) {
-      u32x4 val = {0u, 0u, 0u, 0u};
-      if (s1 != nullptr) val = load16_unaligned<T>(s1 + (c0 - mid_lo));
-      *reinterpret_cast<u32x4_s4*>(drow + c0) = val;
-    } else {
-      T tmp[V];
+  // Destination vectors [v_first, v_end) lie wholly inside the middle source: plain
+  // 16-byte moves, all the loads of a batch issued before its first store.
+  const int v_first = (mid_lo + V - 1) / V, v_end = mid_hi / V;
+  const int n_full = v_end > v_first ? v_end - v_first : 0;
+  for (int it0 = 0; (it0 << pl.lpr_log2) < n_full; it0 += ROW_BATCH) {
+    u32x4 val[ROW_BATCH];
 #pragma unroll
-      for (int e = 0; e < V; ++e) {
-        const int c = c0 + e;
-        T v = T(0);
-        if (c < mid_lo) {
-          if (s0 != nullptr) v = s0[c];
-        } else if (c < mid_hi) {
-          if (s1 != nullptr) v = s1[c - mid_lo];
-        } else if (c < Wa) {
-          if (s2 != nullptr) v = s2[c - mid_hi];
-        }
-        tmp[e] = v;
-      }
-      if (c0 + V <= Wa) {
-        u32x4 val;
-        __builtin_memcpy(&val, tmp, 16);
-        *reinterpret_cast<u32x4_s4*>(drow + c0) = val;
-      } else {
-        for (int e = 0; e < V && c0 + e < Wa; ++e) drow[c0 + e] = tmp[e];
-      }
+    for (int u = 0; u < ROW_BATCH; ++u) {
+      const int j = lir + ((it0 + u) << pl.lpr_log2);
+      val[u] = u32x4{0u, 0u, 0u, 0u};
+      if (j < n_full && s1 != nullptr) val[u] = load16_unaligned<T>(s1 + ((v_first + j) * V - mid_lo));
     }
+#pragma unroll
+    for (int u = 0; u < ROW_BATCH; ++u) {
+      const int j = lir + ((it0 + u) << pl.lpr_log2);
+      if (j < n_full) *reinterpret_cast<u32x4_s4*>(drow + (v_first + j) * V) = val[u];
+    }
+  }
+  // The columns before and after those vectors (the W halos and what shares a vector
+  // with them), one element per lane.
+  const int head = n_full > 0 ? v_first * V : Wa;        // columns [0, head)
+  const int tail0 = n_full > 0 ? v_end * V : Wa;         // columns [tail0, Wa)
+  const int n_edge = head + (Wa - tail0);
+  for (int q = lir; q < n_edge; q += (1 << pl.lpr_log2)) {
+    const int c = q < head ? q : tail0 + (q - head);
+    const T* src = nullptr;
+    if (c < mid_lo) {
+      if (s0 != nullptr) src = s0 + c;
+    } else if (c < mid_hi) {
+      if (s1 != nullptr) src = s1 + (c - mid_lo);
+    } else {
+      if (s2 != nullptr) src = s2 + (c - mid_hi);
+    }
+    drow[c] = src != nullptr ? *src : T(0);
   }
 }
 
@@ -520,31 +524,126 @@ __global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
   const bool row_plain = (d >= g.hi[0]) && (d < D - g.lo[0]) && (h >= g.hi[1]) && (h < H - g.lo[1]);
   const T* orow = own + ((p * Da + (d + g.lo[0])) * Ha + (h + g.lo[1])) * (long long)Wa + g.lo[2];
   T* drow = dst + (long long)row * W;
-  for (int it = 0; it < pl.iters; ++it) {
-    const int j = lir + (it << pl.lpr_log2);
-    if (j >= pl.nvec) break;
-    const int c0 = j * V;
-    if (row_plain && c0 + V <= W) {
-      // `0 + own` for every element (clears the sign of a zero) ...
-      u32x4 val = load16_unaligned<T>(orow + c0);
-      T tmp[V];
-      __builtin_memcpy(tmp, &val, 16);
+  if (!row_plain) {
+    // A row that a D or H neighbour reaches: the full ordered sum, a vector of columns
+    // at a time. Per (od, oh) the middle term is one 16-byte load from the own padded
+    // row or from the strip of that neighbour; the W-neighbour terms touch only the
+    // first and last columns.
+    const int up0 = W - g.lo[2];
+    const int n_vec = W / V;
+    for (int j = lir; j < n_vec; j += (1 << pl.lpr_log2)) {
+      const int c0 = j * V;
+      const bool edge = c0 < g.hi[2] || c0 + V > up0;
+      float acc_d[V];
 #pragma unroll
-      for (int e = 0; e < V; ++e)
-        if ((tmp[e] & ABS) == 0) tmp[e] = 0;
-      // ... and the full ordered sum where a W-neighbour reaches
-      if (c0 < g.hi[2] || c0 + V > W - g.lo[2]) {
+      for (int e = 0; e < V; ++e) acc_d[e] = 0.0f;
+#pragma unroll 1
+      for (int od = -1; od <= 1; ++od) {
+        int cd, ed;
+        if (!reach(od, d, g.lo[0], D, g.hi[0], cd, ed)) continue;
+        float acc_h[V];
 #pragma unroll
-        for (int e = 0; e < V; ++e) {
-          const int c = c0 + e;
-          if (c < g.hi[2] || c >= W - g.lo[2]) tmp[e] = fold_one_rolled<DT>(own, g, p, d, h, c);
+        for (int e = 0; e < V; ++e) acc_h[e] = 0.0f;
+#pragma unroll 1
+        for (int oh = -1; oh <= 1; ++oh) {
+          int ch, eh;
+          if (!reach(oh, h, g.lo[1], H, g.hi[1], ch, eh)) continue;
+          const long long line = (p * ed + cd) * eh + ch;  // row index inside a strip of (od, oh)
+          const int slot = (od + 1) * 9 + (oh + 1) * 3;
+          const bool self = od == 0 && oh == 0;
+          const T* mid = self ? orow : static_cast<const T*>(table_entry(slot + 1));
+          if (!self && mid != nullptr) mid += line * W;
+          T mb[V];
+#pragma unroll
+          for (int e = 0; e < V; ++e) mb[e] = T(0);
+          if (mid != nullptr) {
+            const u32x4 mv = load16_unaligned<T>(mid + c0);
+            __builtin_memcpy(mb, &mv, 16);
+          }
+          float acc_w[V];
+          if (!edge) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) acc_w[e] = Arith<DT>::up(Arith<DT>::down(0.0f + Arith<DT>::up(mb[e])));
+          } else {
+            const T* s_lo = static_cast<const T*>(table_entry(slot + 0));
+            const T* s_hi = static_cast<const T*>(table_entry(slot + 2));
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+              const int c = c0 + e;
+              float a = 0.0f;
+              if (c < g.hi[2] && s_lo != nullptr)
+                a = Arith<DT>::up(Arith<DT>::down(a + Arith<DT>::up(s_lo[line * g.hi[2] + c])));
+              a = Arith<DT>::up(Arith<DT>::down(a + Arith<DT>::up(mb[e])));
+              if (c >= up0 && s_hi != nullptr)
+                a = Arith<DT>::up(Arith<DT>::down(a + Arith<DT>::up(s_hi[line * g.lo[2] + (c - up0)])));
+              acc_w[e] = a;
+            }
+          }
+#pragma unroll
+          for (int e = 0; e < V; ++e) acc_h[e] = Arith<DT>::up(Arith<DT>::down(acc_h[e] + acc_w[e]));
         }
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc_d[e] = Arith<DT>::up(Arith<DT>::down(acc_d[e] + acc_h[e]));
       }
-      __builtin_memcpy(&val, tmp, 16);
-      *reinterpret_cast<u32x4_s4*>(drow + c0) = val;
-    } else {
-      for (int e = 0; e < V && c0 + e < W; ++e) drow[c0 + e] = fold_one_rolled<DT>(own, g, p, d, h, c0 + e);
+      T ob[V];
+#pragma unroll
+      for (int e = 0; e < V; ++e) ob[e] = Arith<DT>::down(acc_d[e]);
+      u32x4 out;
+      __builtin_memcpy(&out, ob, 16);
+      *reinterpret_cast<u32x4_s4*>(drow + c0) = out;
     }
+    for (int c = n_vec * V + lir; c < W; c += (1 << pl.lpr_log2)) drow[c] = fold_one_rolled<DT>(own, g, p, d, h, c);
+    return;
+  }
+  // Only W neighbours reach this row. The sums over D and H then add a single term to
+  // zero, which changes nothing after the first rounding, so an element is
+  // ((0 + lower) + own) + upper with the terms that exist.
+  const T* s_lo = static_cast<const T*>(table_entry(9 + 3 + 0));
+  const T* s_hi = static_cast<const T*>(table_entry(9 + 3 + 2));
+  if (s_lo != nullptr) s_lo += (long long)row * g.hi[2];
+  if (s_hi != nullptr) s_hi += (long long)row * g.lo[2];
+  const int up0 = W - g.lo[2];  // first column the upper neighbour reaches
+  auto element = [&](int c, T own_bits) {
+    float acc = 0.0f;
+    if (c < g.hi[2] && s_lo != nullptr) acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(s_lo[c])));
+    acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(own_bits)));
+    if (c >= up0 && s_hi != nullptr) acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(s_hi[c - up0])));
+    return Arith<DT>::down(acc);
+  };
+  // Vectors [v_first, v_end) hold no column that a W neighbour reaches: `0 + own`, which
+  // only clears the sign of a zero. All the loads of a batch precede its first store.
+  const int v_first = (g.hi[2] + V - 1) / V, v_end = up0 / V;
+  const int n_full = v_end > v_first ? v_end - v_first : 0;
+  for (int it0 = 0; (it0 << pl.lpr_log2) < n_full; it0 += ROW_BATCH) {
+    u32x4 val[ROW_BATCH];
+#pragma unroll
+    for (int u = 0; u < ROW_BATCH; ++u) {
+      const int j = lir + ((it0 + u) << pl.lpr_log2);
+      val[u] = u32x4{0u, 0u, 0u, 0u};
+      if (j < n_full) val[u] = load16_unaligned<T>(orow + (v_first + j) * V);
+    }
+#pragma unroll
+    for (int u = 0; u < ROW_BATCH; ++u) {
+      const int j = lir + ((it0 + u) << pl.lpr_log2);
+      if (j < n_full) {
+        T tmp[V];
+        __builtin_memcpy(tmp, &val[u], 16);
+#pragma unroll
+        for (int e = 0; e < V; ++e)
+          if ((tmp[e] & ABS) == 0) tmp[e] = 0;
+        u32x4 out;
+        __builtin_memcpy(&out, tmp, 16);
+        *reinterpret_cast<u32x4_s4*>(drow + (v_first + j) * V) = out;
+      }
+    }
+  }
+  // The columns before and after those vectors, one element per lane.
+  const int head = n_full > 0 ? v_first * V : W;
+  const int tail0 = n_full > 0 ? v_end * V : W;
+  const int n_edge = head + (W - tail0);
+  for (int q = lir; q < n_edge; q += (1 << pl.lpr_log2)) {
+    const int c = q < head ? q : tail0 + (q - head);
+    drow[c] = element(c, orow[c]);
   }
 }
 
@@ -563,8 +662,8 @@ Magic make_magic(uint32_t d) {
 
 // Lanes per row / vectors per lane for rows of `nvec` 16-byte vectors.
 bool make_plan(unsigned long long nrows, int nvec, uint32_t div_h, uint32_t div_d, RowPlan* pl) {
-  int lg = 0;
-  while ((1 << lg) < nvec && lg < 6) ++lg;
+  int lg = 0;  // fewest lanes that cover the row with one batch each, at most a wavefront
+  while ((1 << lg) * 2 < nvec && lg < 6) ++lg;
   const int lpr = 1 << lg;
   if (nrows == 0 || nrows * (unsigned long long)lpr >= (1ull << 32)) return false;
   pl->nrows = (uint32_t)nrows;
