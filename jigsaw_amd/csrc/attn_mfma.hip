@@ -47,8 +47,8 @@ constexpr int ROWB = 144;         // LDS row pitch in bytes (128 + 16: odd multi
 constexpr int KT_BYTES = BN * ROWB;        // K tile   [key][d]
 constexpr int VT_BYTES = D * ROWB;         // V^T tile [dv][key position]
 constexpr int TILE_BYTES = KT_BYTES + VT_BYTES;
-constexpr int HALF_BYTES = 2 * TILE_BYTES; // double buffer of one key half
-constexpr int LDS_BYTES = 2 * HALF_BYTES;  // 73728
+constexpr int HALF_BYTES = 3 * TILE_BYTES; // three buffers of one key half
+constexpr int LDS_BYTES = 2 * HALF_BYTES;  // 110592
 
 struct FwdArgs {
   const uint16_t* q;   // (batch, sq, 64)
@@ -120,9 +120,12 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_mfma_kernel(FwdArgs p) {
       lo.y = __builtin_amdgcn_perm(vst[3], vst[2], sel);
       hi.x = __builtin_amdgcn_perm(vst[5], vst[4], sel);
       hi.y = __builtin_amdgcn_perm(vst[7], vst[6], sel);
+      // 16-byte chunks of a V^T row are XOR-swizzled with (row / 8) % 8: the 32 lanes
+      // of a store, 288 bytes apart, would otherwise share 4 bank groups
       unsigned char* row = vt + (2 * v_dvp + e) * ROWB;
-      *reinterpret_cast<u32x2*>(row + pos_lo * 2) = lo;
-      *reinterpret_cast<u32x2*>(row + pos_hi * 2) = hi;
+      const int sw = (v_dvp >> 2) & 7;
+      *reinterpret_cast<u32x2*>(row + ((((pos_lo * 2) >> 4) ^ sw) << 4) + ((pos_lo * 2) & 15)) = lo;
+      *reinterpret_cast<u32x2*>(row + ((((pos_hi * 2) >> 4) ^ sw) << 4) + ((pos_hi * 2) & 15)) = hi;
     }
   };
 
@@ -132,12 +135,16 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_mfma_kernel(FwdArgs p) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[nb][i] = 0.0f;
   float m = -INFINITY;  // running max of the raw scores of this query
-  float l = 0.0f;       // running sum over the keys THIS lane has seen
+  f32x16 lsum;          // running sum of the probabilities of this query (every register the same)
+#pragma unroll
+  for (int i = 0; i < 16; ++i) lsum[i] = 0.0f;
+  bf16x8 ones;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ones[i] = (__bf16)1.0f;
 
-  auto compute_tile = [&](int buf) {
+  // S^T of one 64-key tile: 2 blocks of 32 keys x 32 queries (prologue only)
+  auto scores = [&](int buf, f32x16 (&s)[2]) {
     const unsigned char* kt = lds + buf * TILE_BYTES;
-    const unsigned char* vt = kt + KT_BYTES;
-    f32x16 s[2];
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
 #pragma unroll
@@ -149,72 +156,154 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_mfma_kernel(FwdArgs p) {
         s[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[c], s[sb], 0, 0, 0);
       }
     }
-    // online softmax, base 2
-    float mx = s[0][0];
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[sb][i]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float mn = fmaxf(m, mx);
-    const float alpha = __builtin_amdgcn_exp2f((m - mn) * c2);
-    const float mc = mn * c2;
-    m = mn;
-    float rs = 0.0f;
-    bf16x8 pf[2][2];
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb)
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        float e[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          e[i] = __builtin_amdgcn_exp2f(s[sb][8 * t + i] * c2 - mc);
-          rs += e[i];
-        }
-        bf16x8 pk;
-#pragma unroll
-        for (int i = 0; i < 8; i += 2) {
-          f32x2 v2 = {e[i], e[i + 1]};
-          const bf16x2 h2 = __builtin_convertvector(v2, bf16x2);
-          pk[i] = h2.x;
-          pk[i + 1] = h2.y;
-        }
-        pf[sb][t] = pk;
-      }
-    l = l * alpha + rs;
-#pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[nb][i] *= alpha;
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb)
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-          const bf16x8 a = __builtin_bit_cast(
-              bf16x8,
-              *reinterpret_cast<const u32x4*>(vt + (nb * 32 + ln) * ROWB + (sb * 32 + 16 * t + 8 * kg) * 2));
-          o[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[sb][t], o[nb], 0, 0, 0);
-        }
   };
 
-  int buf = 0;
+  // Running max of a tile's scores; rescales the state when some lane of the wavefront
+  // saw a larger score (the max settles after a few tiles, so this is a rarely taken,
+  // wave-uniform branch). Returns the exponent offset of the tile.
+  auto new_max = [&](const f32x16 (&s)[2]) {
+    // tree over the 32 scores of the lane (short dependency chains), then the lane that
+    // shares the query (lane ^ 32) through a register swap instead of an LDS round trip
+    float t8[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      t8[i] = fmaxf(fmaxf(s[0][i], s[0][i + 8]), fmaxf(s[1][i], s[1][i + 8]));
+    float mx = fmaxf(fmaxf(fmaxf(t8[0], t8[1]), fmaxf(t8[2], t8[3])), fmaxf(fmaxf(t8[4], t8[5]), fmaxf(t8[6], t8[7])));
+    {
+      const uint32_t bits = __float_as_uint(mx);
+      const auto sw = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+      mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+    }
+    const float mn = fmaxf(m, mx);
+    if (__builtin_amdgcn_ballot_w64(mn > m) != 0) {
+      const float alpha = __builtin_amdgcn_exp2f((m - mn) * c2);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) lsum[i] *= alpha;
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[nb][i] *= alpha;
+      m = mn;
+    }
+    return m * c2;
+  };
+
+  // ---- software pipeline over the tiles, three LDS buffers per key half. In iteration t
+  // the scores of tile t+1 and the P V products of tile t go to the matrix core one
+  // instruction at a time, each followed by about its run time of vector work (the
+  // exponentials of tile t); tile t+2 moves from registers to LDS and the global loads
+  // of tile t+3 are issued. Past the last tile the same instructions run on clamped tile
+  // indices and their results are dropped, which keeps the loop body free of branches
+  // apart from the rare rescale. The fences pin the hand-made instruction order.
+  const int last = ntiles - 1;
   issue_loads(0);
   store_tile(0);
+  issue_loads(last < 1 ? last : 1);
+  store_tile(1);
+  issue_loads(last < 2 ? last : 2);
   __syncthreads();
-  for (int t = 0; t < ntiles; ++t) {
-    const bool has_next = t + 1 < ntiles;
-    if (has_next) issue_loads(t + 1);
-    compute_tile(buf);
-    if (has_next) store_tile(buf ^ 1);
+  f32x16 s_a[2], s_b[2];
+  scores(0, s_a);
+  int b0 = 0, b1 = 1, b2 = 2;  // buffers of tiles t, t+1, t+2
+#define JG_FENCE() __builtin_amdgcn_sched_barrier(0)
+  auto iteration = [&](int t, const f32x16 (&s_in)[2], f32x16 (&s_out)[2]) {
+    const unsigned char* kt = lds + b1 * TILE_BYTES;              // K of tile t+1
+    const unsigned char* vt = lds + b0 * TILE_BYTES + KT_BYTES;   // V^T of tile t
+    // K fragments of the next tile: requested first, they land under the max
+    u32x4 kf[2][4];
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        kf[sb][c] = *reinterpret_cast<const u32x4*>(kt + (sb * 32 + ln) * ROWB + (16 * c + 8 * kg) * 2);
+    JG_FENCE();
+    const float mc = new_max(s_in);
+    JG_FENCE();
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s_out[sb][i] = 0.0f;
+    bf16x8 pk_prev;
+    u32x4 vf_prev[2];
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+      const int sb = f >> 1, tt = f & 1;
+      // V^T fragments of this P fragment (used one stage later)
+      u32x4 vf[2];
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)
+        vf[nb] = *reinterpret_cast<const u32x4*>(vt + (nb * 32 + ln) * ROWB +
+                                                 (((sb * 4 + 2 * tt + kg) ^ ((nb * 4 + (ln >> 3)) & 7)) << 4));
+      float x[8], e[8];
+      // two score instructions of the next tile, vector work behind each
+      s_out[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[sb][2 * tt]), qf[2 * tt],
+                                                          s_out[sb], 0, 0, 0);
+      JG_FENCE();
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = s_in[sb][8 * tt + i] * c2 - mc;
+      JG_FENCE();
+      s_out[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[sb][2 * tt + 1]),
+                                                          qf[2 * tt + 1], s_out[sb], 0, 0, 0);
+      JG_FENCE();
+      e[0] = __builtin_amdgcn_exp2f(x[0]);
+      e[1] = __builtin_amdgcn_exp2f(x[1]);
+      JG_FENCE();
+      // the three P V instructions of the previous fragment
+      if (f > 0) lsum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pk_prev, lsum, 0, 0, 0);
+      JG_FENCE();
+      e[2] = __builtin_amdgcn_exp2f(x[2]);
+      e[3] = __builtin_amdgcn_exp2f(x[3]);
+      JG_FENCE();
+      if (f > 0)
+        o[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf_prev[0]), pk_prev, o[0], 0, 0, 0);
+      JG_FENCE();
+      e[4] = __builtin_amdgcn_exp2f(x[4]);
+      e[5] = __builtin_amdgcn_exp2f(x[5]);
+      JG_FENCE();
+      if (f > 0)
+        o[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf_prev[1]), pk_prev, o[1], 0, 0, 0);
+      JG_FENCE();
+      e[6] = __builtin_amdgcn_exp2f(x[6]);
+      e[7] = __builtin_amdgcn_exp2f(x[7]);
+      bf16x8 pk;
+#pragma unroll
+      for (int i = 0; i < 8; i += 2) {
+        f32x2 v2 = {e[i], e[i + 1]};
+        const bf16x2 h2 = __builtin_convertvector(v2, bf16x2);
+        pk[i] = h2.x;
+        pk[i + 1] = h2.y;
+      }
+      JG_FENCE();
+      pk_prev = pk;
+      vf_prev[0] = vf[0];
+      vf_prev[1] = vf[1];
+    }
+    // last fragment's P V under the tile hand-over
+    lsum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pk_prev, lsum, 0, 0, 0);
+    JG_FENCE();
+    store_tile(b2);
+    JG_FENCE();
+    o[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf_prev[0]), pk_prev, o[0], 0, 0, 0);
+    JG_FENCE();
+    issue_loads(t + 3 < last ? t + 3 : last);
+    JG_FENCE();
+    o[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf_prev[1]), pk_prev, o[1], 0, 0, 0);
     __syncthreads();
-    buf ^= 1;
+    const int tmp = b0;
+    b0 = b1;
+    b1 = b2;
+    b2 = tmp;
+  };
+#undef JG_FENCE
+  int t = 0;
+  for (; t + 1 < ntiles; t += 2) {
+    iteration(t, s_a, s_b);
+    iteration(t + 1, s_b, s_a);
   }
+  if (t < ntiles) iteration(t, s_a, s_b);
 
-  // ---- the two lanes of a query add their sums; the two key halves combine via LDS
-  l += __shfl_xor(l, 32, 64);
+  // ---- the two key halves combine via LDS
+  float l = lsum[0];
   float* xo = reinterpret_cast<float*>(smem) + qb * (32 * 64 + 128);  // [32 regs][64 lanes] + m,l
   if (ks == 1) {
 #pragma unroll
