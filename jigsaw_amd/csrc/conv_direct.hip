@@ -194,16 +194,20 @@ __global__ __launch_bounds__(256) void direct_wgrad_kernel(float* __restrict__ p
       }
 }
 
-// Stage 2: fixed-order sum over the chunk partials (deterministic).
+// Stage 2: fixed-order sum over the chunk partials (deterministic). One wavefront per
+// output: lane j adds partials j, j + 64, ... and a butterfly adds the lanes.
 template <int DT>
 __global__ __launch_bounds__(256) void reduce_parts_kernel(typename Elem<DT>::T* __restrict__ out,
                                                            const float* __restrict__ part,
                                                            long long count, int nparts) {
-  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  const long long i = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
   if (i >= count) return;
   float s = 0.0f;
-  for (int k = 0; k < nparts; ++k) s += part[(long long)k * count + i];
-  out[i] = Elem<DT>::down(s);
+  for (int k = lane; k < nparts; k += 64) s += part[(long long)k * count + i];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+  if (lane == 0) out[i] = Elem<DT>::down(s);
 }
 
 // ----------------------------------------------------------------- bias grad
@@ -333,7 +337,7 @@ int direct_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, int
     if (!empty)                                                                            \
       direct_wgrad_kernel<DT><<<grid, 256, 0, s>>>(part, static_cast<const Elem<DT>::T*>(x), \
                                                    static_cast<const Elem<DT>::T*>(go), g, len); \
-    reduce_parts_kernel<DT><<<(unsigned)((count + 255) / 256), 256, 0, s>>>(               \
+    reduce_parts_kernel<DT><<<(unsigned)((count + 3) / 4), 256, 0, s>>>(               \
         static_cast<Elem<DT>::T*>(gw), part, count, empty ? 0 : chunks);                   \
   } while (0)
   if (dtype == JG_F32) JG_GO(JG_F32);
@@ -374,7 +378,7 @@ extern "C" int jg_bias_grad(void* gb, const void* g, int64_t batch, int64_t chan
     if (!empty)                                                                               \
       bias_grad_kernel<DT><<<grid, 256, 0, s>>>(part, static_cast<const Elem<DT>::T*>(g), batch, \
                                                 (int)channels, spatial, len);                 \
-    reduce_parts_kernel<DT><<<(unsigned)((channels + 255) / 256), 256, 0, s>>>(               \
+    reduce_parts_kernel<DT><<<(unsigned)((channels + 3) / 4), 256, 0, s>>>(               \
         static_cast<Elem<DT>::T*>(gb), part, channels, empty ? 0 : chunks);                   \
   } while (0)
   if (dtype == JG_F32) JG_GO(JG_F32);

@@ -269,24 +269,32 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
       }
 }
 
-// gw[co][ci][kd][kh][kw] (bf16) = sum over workgroups of part[wg][tap9][co][kd*Cin+ci].
+// gw[co][ci][kd][kh][kw] (bf16) = sum over the slots of part[slot][tap9][co][kd*Cin+ci].
+// A block owns 64 consecutive outputs (one per lane, so a slot row is read coalesced);
+// its 4 wavefronts take the slots s = w, w + 4, ... in 4 independent chains each, and the
+// 16 chain sums are added in a fixed order (deterministic).
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(uint16_t* __restrict__ gw,
                                                            const float* __restrict__ part,
                                                            int slots, int GC, int XC, int Cin) {
+  __shared__ float red[4][64];
   const int count = 9 * GC * XC;
-  const int i = blockIdx.x * 256 + threadIdx.x;  // index in [tap9][co][c']
-  if (i >= count) return;
-  // four independent chains keep the loads in flight; the order stays fixed
-  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-  int k = 0;
-  for (; k + 4 <= slots; k += 4) {
-    s0 += part[(size_t)(k + 0) * count + i];
-    s1 += part[(size_t)(k + 1) * count + i];
-    s2 += part[(size_t)(k + 2) * count + i];
-    s3 += part[(size_t)(k + 3) * count + i];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int i = blockIdx.x * 64 + lane;  // index in [tap9][co][c']
+  float c0 = 0.f, c1 = 0.f, c2 = 0.f, c3 = 0.f;
+  if (i < count) {
+    int k = w;
+    for (; k + 12 < slots; k += 16) {
+      c0 += part[(size_t)(k + 0) * count + i];
+      c1 += part[(size_t)(k + 4) * count + i];
+      c2 += part[(size_t)(k + 8) * count + i];
+      c3 += part[(size_t)(k + 12) * count + i];
+    }
+    for (; k < slots; k += 4) c0 += part[(size_t)k * count + i];
   }
-  for (; k < slots; ++k) s0 += part[(size_t)k * count + i];
-  const float s = (s0 + s1) + (s2 + s3);
+  red[w][lane] = (c0 + c1) + (c2 + c3);
+  __syncthreads();
+  if (w != 0 || i >= count) return;
+  const float s = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
   const int cx = i % XC, co = (i / XC) % GC, tap = i / (XC * GC);
   const int kd = cx / Cin, ci = cx % Cin, KD = XC / Cin;
   gw[(((size_t)co * Cin + ci) * KD + kd) * 9 + tap] = jg::f32_to_bf16(s);
@@ -396,7 +404,7 @@ int mfma_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, void*
   if (rc) return rc;
   JG_CHECK_LAUNCH(who);
   const int count = 9 * 32 * cgb * 32 * cxb;
-  wgrad_reduce_kernel<<<(count + 255) / 256, 256, 0, s>>>(static_cast<uint16_t*>(gw), p.part, wgs * HALVES,
+  wgrad_reduce_kernel<<<(count + 63) / 64, 256, 0, s>>>(static_cast<uint16_t*>(gw), p.part, wgs * HALVES,
                                                           32 * cgb, 32 * cxb, g.cin);
   JG_CHECK_LAUNCH(who);
   return JG_OK;

@@ -54,18 +54,9 @@ __device__ __forceinline__ u32x4 load16_unaligned<uint32_t>(const uint32_t* s) {
 
 template <>
 __device__ __forceinline__ u32x4 load16_unaligned<uint16_t>(const uint16_t* s) {
-  uintptr_t a = reinterpret_cast<uintptr_t>(s);
-  if ((a & 3) == 0) return *reinterpret_cast<const u32x4_a4*>(s);
-  // 2-byte phase: read the five dwords that cover the 16 bytes and funnel-shift.
-  const uint32_t* q = reinterpret_cast<const uint32_t*>(a - 2);
-  u32x4_a4 lo4 = *reinterpret_cast<const u32x4_a4*>(q);
-  uint32_t d4 = q[4];
-  u32x4 r;
-  r.x = (lo4.x >> 16) | (lo4.y << 16);
-  r.y = (lo4.y >> 16) | (lo4.z << 16);
-  r.z = (lo4.z >> 16) | (lo4.w << 16);
-  r.w = (lo4.w >> 16) | (d4 << 16);
-  return r;
+  // the memory pipeline of gfx9 takes vector accesses at any alignment
+  typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+  return *reinterpret_cast<const u32x4_a2*>(s);
 }
 
 // Region of a padded coordinate: 0 = lower halo, 1 = interior, 2 = upper halo.
@@ -418,28 +409,28 @@ __global__ __launch_bounds__(256) void assemble_rows_kernel(Table tab, T* __rest
   if (s2 != nullptr) s2 += line * g.hi[2];
   T* drow = dst + (long long)row * Wa;
   const int mid_lo = g.lo[2], mid_hi = g.lo[2] + g.n[2];
-  // Destination vectors [v_first, v_end) lie wholly inside the middle source: plain
-  // 16-byte moves, all the loads of a batch issued before its first store.
-  const int v_first = (mid_lo + V - 1) / V, v_end = mid_hi / V;
-  const int n_full = v_end > v_first ? v_end - v_first : 0;
+  // The middle source in 16-byte vectors of ITS row (aligned loads when the tile rows
+  // are), stored at whatever alignment the padded row gives them; all the loads of a
+  // batch are issued before its first store.
+  typedef uint32_t u32x4_any __attribute__((ext_vector_type(4), aligned(2)));
+  const int n_full = g.n[2] / V;
   for (int it0 = 0; (it0 << pl.lpr_log2) < n_full; it0 += ROW_BATCH) {
     u32x4 val[ROW_BATCH];
 #pragma unroll
     for (int u = 0; u < ROW_BATCH; ++u) {
       const int j = lir + ((it0 + u) << pl.lpr_log2);
       val[u] = u32x4{0u, 0u, 0u, 0u};
-      if (j < n_full && s1 != nullptr) val[u] = load16_unaligned<T>(s1 + ((v_first + j) * V - mid_lo));
+      if (j < n_full && s1 != nullptr) val[u] = *reinterpret_cast<const u32x4_any*>(s1 + j * V);
     }
 #pragma unroll
     for (int u = 0; u < ROW_BATCH; ++u) {
       const int j = lir + ((it0 + u) << pl.lpr_log2);
-      if (j < n_full) *reinterpret_cast<u32x4_s4*>(drow + (v_first + j) * V) = val[u];
+      if (j < n_full) *reinterpret_cast<u32x4_any*>(drow + mid_lo + j * V) = val[u];
     }
   }
-  // The columns before and after those vectors (the W halos and what shares a vector
-  // with them), one element per lane.
-  const int head = n_full > 0 ? v_first * V : Wa;        // columns [0, head)
-  const int tail0 = n_full > 0 ? v_end * V : Wa;         // columns [tail0, Wa)
+  // The W halos and the tail of the middle, one element per lane.
+  const int head = mid_lo;                    // columns [0, head)
+  const int tail0 = mid_lo + n_full * V;      // columns [tail0, Wa)
   const int n_edge = head + (Wa - tail0);
   for (int q = lir; q < n_edge; q += (1 << pl.lpr_log2)) {
     const int c = q < head ? q : tail0 + (q - head);
