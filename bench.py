@@ -3,9 +3,10 @@
 
 One "step" is one pass of the halo-exchange convolution of BASELINE.json's
 configuration 2 for one rank: pack the 8 strips, assemble the padded tile from
-the (seeded, locally held) neighbour strips, convolution forward, then bias
-gradient, dgrad on the padded shape, wgrad, pack of the halo gradients and fold
-of the neighbours' halo gradients. All inputs are resident in HBM before the
+the (seeded, locally held) neighbour strips, convolution forward, then dgrad
+(writing the owned cells and the halo gradients to send in one pass), wgrad with
+the bias gradient from the same pass, and the fold of the neighbours' halo
+gradients into the border. All inputs are resident in HBM before the
 timed region. ``value`` is the convolution's algorithmic FLOPs (fwd + dgrad +
 wgrad) divided by the whole step time, halo movement included.
 
@@ -16,6 +17,7 @@ build runs one rank's share on one GPU and has no collectives.
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -47,12 +49,19 @@ def time_gpu(fn, iters: int, warmup: int = 2) -> float:
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    e0, e1 = _events()
-    e0.record()
-    for _ in range(iters):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
+    # a full collection of the interpreter's garbage collector takes tens of milliseconds
+    # in a process this size and would land inside one of these short loops
+    gc.collect()
+    gc.disable()
+    try:
+        e0, e1 = _events()
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+    finally:
+        gc.enable()
     return e0.elapsed_time(e1) / iters
 
 
@@ -82,19 +91,20 @@ def build_conv2_workload(dev, batch=8, ch=64, tile=1024):
 
 
 def conv_step(wl):
-    """The hot path of one rank for one batch (see the module docstring)."""
+    """The hot path of one rank for one batch (see the module docstring). The backward
+    uses the fused form: dgrad writes the owned cells and the strips it sends in one
+    pass, and the received strips are added to the border afterwards (same bits as
+    dgrad + pack + fold on the padded gradient)."""
     from jigsaw_amd import conv as jc
-    from jigsaw_amd.halo import halo_assemble, halo_fold, halo_pack
+    from jigsaw_amd.halo import halo_assemble, halo_fold_border_, halo_pack
 
     geom, x, w, b, g = wl["geom"], wl["x"], wl["w"], wl["b"], wl["g"]
     halo_pack(x, geom, from_padded=False)  # strips this rank sends
     x_aug = halo_assemble(x, wl["strips_fwd"], geom)
     y = jc.conv_nd(x_aug, w, b)
-    gb = jc.sum_grad_bias(g, 2)
-    gx_aug = jc.conv_nd_input(x_aug.shape, w, g)
-    gw = jc.conv_nd_weight(x_aug, w.shape, g)
-    halo_pack(gx_aug, geom, from_padded=True)  # halo gradients this rank sends
-    gx = halo_fold(gx_aug, wl["strips_bwd"], geom)
+    gx, _send = jc.conv_nd_input_fold(geom, w, g)  # owned cells + halo gradients this rank sends
+    gw, gb = jc.conv_nd_weight(x_aug, w.shape, g, with_bias_grad=True)  # one pass over g for both
+    halo_fold_border_(gx, wl["strips_bwd"], geom)
     return y, gx, gw, gb
 
 
@@ -303,6 +313,10 @@ def main() -> int:
     gx_buf = torch.empty_like(wl["x"])
     ms_asm = time_gpu(lambda: halo_assemble(wl["x"], wl["strips_fwd"], geom, out=x_aug), it)
     ms_fold = time_gpu(lambda: halo_fold(gx_aug, wl["strips_bwd"], geom, out=gx_buf), it)
+    ms_dgrad_fold = time_gpu(lambda: jc.conv_nd_input_fold(geom, wl["w"], wl["g"]), it)
+    from jigsaw_amd.halo import halo_fold_border_
+
+    ms_border = time_gpu(lambda: halo_fold_border_(gx_buf, wl["strips_bwd"], geom), it)
     es = wl["x"].element_size()
     strip_bytes = sum(t.numel() for t in wl["strips_fwd"].values()) * es
     halo_bytes = (wl["x"].numel() + x_aug.numel()) * es + strip_bytes  # read tile + strips, write padded tile
@@ -329,6 +343,8 @@ def main() -> int:
         },
         "halo_assemble": {"ms": ms_asm, "GBps": gbps(ms_asm), "frac_hbm_peak": gbps(ms_asm) / PEAK_HBM_GBPS, "bytes": halo_bytes},
         "halo_fold": {"ms": ms_fold, "GBps": gbps(ms_fold), "frac_hbm_peak": gbps(ms_fold) / PEAK_HBM_GBPS, "bytes": halo_bytes},
+        "conv_dgrad_fused_with_pack_and_fold": {"ms": ms_dgrad_fold, "tflops": tf(ms_dgrad_fold)},
+        "halo_fold_border": {"ms": ms_border},
     }
     extra.update(attention_figures(dev, max(10, it)))
     extra.update(conv3d_figures(dev, it))
@@ -349,7 +365,7 @@ def main() -> int:
         "data": "synthetic",
         "config": {
             "workload": "config 2: one rank's 1024x1024 tile of a 2048x2048 domain, batch 8, 64->64 ch, 3x3, pad 1; "
-            "halo pack + assemble + conv fwd + bias-grad + dgrad + wgrad + halo pack + fold",
+            "halo pack + assemble + conv fwd + dgrad (fused with the halo pack and the own part of the fold) + wgrad (fused with bias-grad) + border fold",
             "flop_per_step": flop_step,
             "frac_mfma_peak": value / PEAK_BF16_TFLOPS,
         },

@@ -113,6 +113,16 @@ int jg_halo_fold_2d(void* gx, const void* gx_aug, const void* const strips[9],
                     int64_t planes, int H, int W, int lo_h, int hi_h, int lo_w,
                     int hi_w, int dtype, void* stream);
 
+/* Second half of a fold whose own contributions are already in place: gx
+ * (planes, D, H, W) holds `0 + own` in every cell (what jg_conv_dgrad_fold
+ * writes) and the cells a neighbour reaches get the neighbours' strips added, in
+ * place, in the order of jg_halo_fold_3d (halo.py:207-249,
+ * distributed.py:378-389). Together with jg_conv_dgrad_fold this gives the same
+ * bits as jg_conv_dgrad + jg_halo_pack_3d(from_padded) + jg_halo_fold_3d without
+ * the padded gradient ever reaching memory. */
+int jg_halo_fold_border_3d(void* gx, const void* const strips[27],
+                           const jg_halo_geom* geom, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------- *
  * DistributedRoll (pure copies; HBM-bound)
  * ------------------------------------------------------------------------- */
@@ -233,11 +243,33 @@ int jg_conv_fwd(void* y, const void* x, const void* w, const void* bias,
 int jg_conv_dgrad(void* gx, const void* w, const void* g, const jg_conv_desc* desc,
                   int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* jg_conv_dgrad with the first half of the fold fused into its epilogue
+ * (distributed.py:346-355 followed by the sends of halo.py:222-226): `desc`
+ * describes the convolution on the padded tile as for jg_conv_dgrad and `geom`
+ * says where the own tile sits inside it (size + lo + hi = desc->in_size,
+ * planes = batch * c_in). Cells of the padded gradient inside the tile go to gx
+ * (planes, *size) as `0 + v`; halo cells go to send[slot of the neighbour that
+ * owns them] in the layout of jg_halo_pack_3d(from_padded = 1); a NULL slot
+ * drops them. Returns JG_ERR_UNSUPPORTED where only the unfused path exists
+ * (workspace as for JG_CONV_DGRAD). Finish with jg_halo_fold_border_3d. */
+int jg_conv_dgrad_fold(void* gx, void* const send[27], const void* w, const void* g,
+                       const jg_conv_desc* desc, const jg_halo_geom* geom, int dtype,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
 /* gw (Cout, Cin, *kernel) — torch.nn.grad.conv*_weight as called at
  * jigsaw/modules/convolution/_conv/distributed.py:359-368. Deterministic
  * (fixed-order two-stage reduction, no atomics). */
 int jg_conv_wgrad(void* gw, const void* x, const void* g, const jg_conv_desc* desc,
                   int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* jg_conv_wgrad that also produces gb (Cout,) = sum of g over batch and pixels
+ * (_sum_grad_bias, jigsaw/modules/convolution/_conv/config.py:117-120) from the
+ * same pass over g, saving the separate read of g by jg_bias_grad. Workspace as
+ * for JG_CONV_WGRAD. Returns JG_ERR_UNSUPPORTED where only the separate kernels
+ * cover the problem. */
+int jg_conv_wgrad_bias(void* gw, void* gb, const void* x, const void* g,
+                       const jg_conv_desc* desc, int dtype, void* workspace,
+                       size_t workspace_bytes, void* stream);
 
 /* gb (C,) = sum of g (N, C, spatial...) over batch and spatial axes —
  * _sum_grad_bias, jigsaw/modules/convolution/_conv/config.py:117-120.

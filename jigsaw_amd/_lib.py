@@ -76,6 +76,7 @@ SIGNATURES: dict[str, tuple] = {
         [POINTER(c_void_p), c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     ),
     "jg_halo_fold_3d": (c_int, [c_void_p, c_void_p, POINTER(c_void_p), POINTER(HaloGeom), c_int, c_void_p]),
+    "jg_halo_fold_border_3d": (c_int, [c_void_p, POINTER(c_void_p), POINTER(HaloGeom), c_int, c_void_p]),
     "jg_halo_fold_2d": (
         c_int,
         [c_void_p, c_void_p, POINTER(c_void_p), c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
@@ -106,7 +107,16 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_void_p, c_void_p, c_void_p, POINTER(ConvDesc), c_int, c_void_p, c_size_t, c_void_p],
     ),
     "jg_conv_dgrad": (c_int, [c_void_p, c_void_p, c_void_p, POINTER(ConvDesc), c_int, c_void_p, c_size_t, c_void_p]),
+    "jg_conv_dgrad_fold": (
+        c_int,
+        [c_void_p, POINTER(c_void_p), c_void_p, c_void_p, POINTER(ConvDesc), POINTER(HaloGeom), c_int, c_void_p, c_size_t,
+         c_void_p],
+    ),
     "jg_conv_wgrad": (c_int, [c_void_p, c_void_p, c_void_p, POINTER(ConvDesc), c_int, c_void_p, c_size_t, c_void_p]),
+    "jg_conv_wgrad_bias": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, POINTER(ConvDesc), c_int, c_void_p, c_size_t, c_void_p],
+    ),
     "jg_bias_grad_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "jg_bias_grad": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p]),
     "jg_attn_fwd": (

@@ -24,7 +24,8 @@ from typing import Any, Protocol
 import torch
 
 from . import _lib
-from .halo import HaloGeometry, halo_assemble, halo_fold, halo_pack
+from .halo import HaloGeometry, halo_assemble, halo_fold, halo_fold_border_, halo_pack
+from .halo import slot as halo_slot
 
 # --------------------------------------------------------------------------- #
 # local primitives
@@ -141,8 +142,61 @@ def conv_nd_input(input_shape, w, g, *, stride=1, padding=0, dilation=1, groups=
     return gx
 
 
-def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, groups=1) -> torch.Tensor:
-    """``torch.nn.grad.conv{1,2,3}d_weight(x, weight_shape, g, ...)`` on the HIP kernels."""
+def conv_nd_input_fold(geom: HaloGeometry, w, g, *, stride=1, padding=0, dilation=1, groups=1, present=None):
+    """Input gradient of the convolution on the halo-padded tile, written to its owners.
+
+    Equivalent to ``conv_nd_input`` on the padded shape followed by
+    ``halo_pack(from_padded=True)``, without the padded gradient reaching memory:
+    returns ``(gx, send)`` where ``gx`` (N, Cin, *geom.size) holds ``0 + own`` in every
+    cell and ``send[offset]`` is the halo block owned by that neighbour (only the
+    offsets in ``present``, all by default). ``halo_fold_border_`` finishes the fold
+    once the neighbours' blocks have arrived. Returns ``None`` where only the
+    unfused kernels cover the problem.
+    """
+    _lib.require_gpu(w, g)
+    n = _check_args(g, w, groups, padding)
+    if g.dtype != w.dtype:
+        raise RuntimeError(f"grad_output type ({g.dtype}) and weight type ({w.dtype}) should be the same")
+    if geom.n_spatial != n:
+        raise ValueError(f"geometry has {geom.n_spatial} spatial axes, the convolution {n}")
+    stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
+    g, w = g.contiguous(), w.contiguous()
+    batch, c_in = int(g.shape[0]), int(w.shape[1])
+    padded = geom.padded
+    out_sp = _out_spatial(padded, w.shape[2:], stride, padding, dilation)
+    if tuple(g.shape) != (batch, w.shape[0], *out_sp):
+        raise ValueError(
+            f"grad_output shape {tuple(g.shape)} does not match the convolution of a padded tile {padded} "
+            f"(expected {(batch, w.shape[0], *out_sp)})"
+        )
+    desc = _desc(batch, c_in, w.shape[0], padded, w.shape[2:], stride, padding, dilation, groups)
+    ws, nbytes = _workspace(desc, 1, g.dtype, g.device)
+    lead = (batch, c_in)
+    offs = geom.offsets() if present is None else [tuple(o) for o in present]
+    send: dict = {}
+    tab = _lib.VoidP27()
+    for o in offs:
+        t = torch.empty(lead + geom.strip_extent(o, "pack_bwd"), dtype=g.dtype, device=g.device)
+        send[o] = t
+        if t.numel():
+            tab[halo_slot(o)] = t.data_ptr()
+    gx = torch.empty(lead + geom.size, dtype=g.dtype, device=g.device)
+    rc = _lib.load().jg_conv_dgrad_fold(
+        _lib.ptr(gx), tab, _lib.ptr(w), _lib.ptr(g), desc, geom.c_geom(batch * c_in), _lib.dtype_code(g.dtype),
+        _lib.ptr(ws), nbytes, _lib.stream_ptr(g.device),
+    )
+    if rc == -2:  # only the unfused kernels cover this geometry / dtype
+        return None
+    _lib.check(rc, "jg_conv_dgrad_fold")
+    return gx, send
+
+
+def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, groups=1, with_bias_grad=False):
+    """``torch.nn.grad.conv{1,2,3}d_weight(x, weight_shape, g, ...)`` on the HIP kernels.
+
+    ``with_bias_grad=True`` returns ``(gw, gb)`` with ``gb = g.sum`` over batch and pixels
+    (config.py:117-120), from the same pass over ``g`` where the MFMA kernel covers the shape.
+    """
     _lib.require_gpu(x, g)
     weight_shape = tuple(int(v) for v in weight_shape)
     n = len(weight_shape) - 2
@@ -160,11 +214,23 @@ def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, group
     gw = torch.empty(weight_shape, dtype=x.dtype, device=x.device)
     desc = _desc(x.shape[0], x.shape[1], weight_shape[0], x.shape[2:], weight_shape[2:], stride, padding, dilation, groups)
     ws, nbytes = _workspace(desc, 2, x.dtype, x.device)
+    if with_bias_grad:
+        # one pass over g for both gradients where the MFMA kernel covers the shape
+        gb = torch.empty(weight_shape[0], dtype=x.dtype, device=x.device)
+        rc = _lib.load().jg_conv_wgrad_bias(
+            _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(x), _lib.ptr(g), desc, _lib.dtype_code(x.dtype), _lib.ptr(ws), nbytes,
+            _lib.stream_ptr(x.device),
+        )
+        if rc != -2:
+            _lib.check(rc, "jg_conv_wgrad_bias")
+            return gw, gb
     rc = _lib.load().jg_conv_wgrad(
         _lib.ptr(gw), _lib.ptr(x), _lib.ptr(g), desc, _lib.dtype_code(x.dtype), _lib.ptr(ws), nbytes,
         _lib.stream_ptr(x.device),
     )
     _lib.check(rc, "jg_conv_wgrad")
+    if with_bias_grad:
+        return gw, sum_grad_bias(g, n)
     return gw
 
 
@@ -290,19 +356,36 @@ def conv_halo_nway_backward(
     n = config.n_spatial
     ranks, sizes = _mesh_position(spatial_groups)
     local_padding = _local_padding(padding, sizes)
-    need_x, need_w = need
+    need_x, need_w = need[0], need[1]
+    # a third entry asks for the bias gradient too; the result then has three entries
+    want_b = len(need) > 2
+    need_b = want_b and need[2]
     g = grad_output.to(weight.dtype)
     kwargs = {"stride": stride, "padding": local_padding, "dilation": dilation, "groups": 1}
-    g_x_need = config.conv_input_fn(x_aug.shape, weight, g, **kwargs) if need_x else None
-    g_w = config.conv_weight_fn(x_aug, weight.shape, g, **kwargs) if need_w else None
+    g_w = g_b = None
+    if need_w and need_b and config.conv_weight_fn is conv_nd_weight:
+        g_w, g_b = conv_nd_weight(x_aug, weight.shape, g, with_bias_grad=True, **kwargs)
+    else:
+        g_w = config.conv_weight_fn(x_aug, weight.shape, g, **kwargs) if need_w else None
+        g_b = config.grad_bias(g.contiguous()) if need_b else None
+    done = (lambda gx: (gx, g_w, g_b)) if want_b else (lambda gx: (gx, g_w))
     if not need_x:
-        return None, g_w
+        return done(None)
     geom = HaloGeometry.for_conv(local_in_spatial, weight.shape[-n:], stride, padding, dilation, ranks, sizes)
     present = _present_offsets(geom, ranks, sizes)
+    if getattr(config, "fused_fold", False) and config.conv_input_fn is conv_nd_input:
+        # dgrad writes the owned cells and the send strips itself; same bits as the
+        # three separate steps below
+        fused = conv_nd_input_fold(geom, weight, g, present=present, **kwargs)
+        if fused is not None:
+            g_x, send = fused
+            recv = config.halo_exchange.backward(send) if present else {}
+            return done(halo_fold_border_(g_x, recv, geom))
+    g_x_need = config.conv_input_fn(x_aug.shape, weight, g, **kwargs)
     send = halo_pack(g_x_need, geom, from_padded=True, present=present) if present else {}
     recv = config.halo_exchange.backward(send) if present else {}
     g_x = halo_fold(g_x_need, recv, geom)
-    return g_x, g_w
+    return done(g_x)
 
 
 class HipConvNdConfig:
@@ -316,6 +399,8 @@ class HipConvNdConfig:
 
     vmapped = False
     channel_local = True
+    fused_fold = True  # dgrad + pack + fold in one pass where the MFMA kernel covers the shape
+    fused_bias_grad = True  # bias gradient from the weight-gradient kernel's pass over g
     groups = 1
     groups_local = 1
 
@@ -375,11 +460,19 @@ class _ConvNd(torch.autograd.Function):
         config = ctx.config
         x_aug = x_aug.to(weight.dtype)
         need_x, need_w, need_b = ctx.needs_input_grad[:3]
-        g_b = config.grad_bias(grad_output.contiguous()) if (need_b and ctx.has_bias) else None
-        g_x, g_w = config.dist_conv_backward_fn(
-            grad_output, x_aug, weight, ctx.stride, ctx.padding, ctx.dilation, ctx.local_in_spatial,
-            ctx.spatial_groups, ctx.channel_group, config, need=(need_x, need_w),
-        )
+        need_b = need_b and ctx.has_bias
+        if getattr(config, "fused_bias_grad", False):
+            # the weight-gradient kernel adds up g on the way
+            g_x, g_w, g_b = config.dist_conv_backward_fn(
+                grad_output, x_aug, weight, ctx.stride, ctx.padding, ctx.dilation, ctx.local_in_spatial,
+                ctx.spatial_groups, ctx.channel_group, config, need=(need_x, need_w, need_b),
+            )
+        else:
+            g_b = config.grad_bias(grad_output.contiguous()) if need_b else None
+            g_x, g_w = config.dist_conv_backward_fn(
+                grad_output, x_aug, weight, ctx.stride, ctx.padding, ctx.dilation, ctx.local_in_spatial,
+                ctx.spatial_groups, ctx.channel_group, config, need=(need_x, need_w),
+            )
         return g_x, g_w, g_b, None, None, None, None, None, None
 
 

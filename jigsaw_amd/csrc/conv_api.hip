@@ -81,6 +81,30 @@ extern "C" int jg_conv_dgrad(void* gx, const void* w, const void* go, const jg_c
   return jg::direct_dgrad(gx, w, go, g, dtype, s);
 }
 
+extern "C" int jg_conv_dgrad_fold(void* gx, void* const send[27], const void* w, const void* go,
+                                  const jg_conv_desc* desc, const jg_halo_geom* geom, int dtype,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+  jg::ConvGeom g;
+  int rc = jg::resolve_conv(desc, "jg_conv_dgrad_fold", &g);
+  if (rc) return rc;
+  JG_REQUIRE(gx && send && w && go && geom, "jg_conv_dgrad_fold: NULL pointer");
+  JG_REQUIRE(known(dtype), "jg_conv_dgrad_fold: unknown dtype %d", dtype);
+  JG_REQUIRE(geom->planes == g.batch * g.cin, "jg_conv_dgrad_fold: geom->planes %lld != batch * c_in %lld",
+             (long long)geom->planes, (long long)(g.batch * g.cin));
+  int lo[3], n[3];
+  for (int a = 0; a < 3; ++a) {
+    lo[a] = geom->lo[a];
+    n[a] = geom->size[a];
+    JG_REQUIRE(lo[a] >= 0 && geom->hi[a] >= 0 && n[a] >= 1 && lo[a] + n[a] + geom->hi[a] == g.in[a],
+               "jg_conv_dgrad_fold: axis %d: lo %d + size %d + hi %d != padded extent %d", a, lo[a], n[a],
+               geom->hi[a], g.in[a]);
+  }
+  if (!jg::mfma_dgrad_supported(g, dtype))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_dgrad_fold: geometry / dtype only has the unfused path");
+  return jg::mfma_dgrad_fold(gx, send, lo, n, w, go, g, workspace, workspace_bytes,
+                             static_cast<hipStream_t>(stream));
+}
+
 extern "C" int jg_conv_wgrad(void* gw, const void* x, const void* go, const jg_conv_desc* desc,
                              int dtype, void* workspace, size_t workspace_bytes, void* stream) {
   jg::ConvGeom g;
@@ -89,6 +113,20 @@ extern "C" int jg_conv_wgrad(void* gw, const void* x, const void* go, const jg_c
   JG_REQUIRE(gw && x && go, "jg_conv_wgrad: NULL pointer");
   JG_REQUIRE(known(dtype), "jg_conv_wgrad: unknown dtype %d", dtype);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (jg::mfma_wgrad_supported(g, dtype)) return jg::mfma_wgrad(gw, x, go, g, workspace, workspace_bytes, s);
+  if (jg::mfma_wgrad_supported(g, dtype))
+    return jg::mfma_wgrad(gw, nullptr, x, go, g, workspace, workspace_bytes, s);
   return jg::direct_wgrad(gw, x, go, g, dtype, workspace, workspace_bytes, s);
+}
+
+extern "C" int jg_conv_wgrad_bias(void* gw, void* gb, const void* x, const void* go,
+                                  const jg_conv_desc* desc, int dtype, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+  jg::ConvGeom g;
+  int rc = jg::resolve_conv(desc, "jg_conv_wgrad_bias", &g);
+  if (rc) return rc;
+  JG_REQUIRE(gw && gb && x && go, "jg_conv_wgrad_bias: NULL pointer");
+  JG_REQUIRE(known(dtype), "jg_conv_wgrad_bias: unknown dtype %d", dtype);
+  if (!jg::mfma_wgrad_supported(g, dtype))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_wgrad_bias: geometry / dtype only has the separate kernels");
+  return jg::mfma_wgrad(gw, gb, x, go, g, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }

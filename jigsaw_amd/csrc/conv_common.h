@@ -37,7 +37,12 @@ int mfma_fwd(void* y, const void* x, const void* w, const void* bias, const Conv
              void* ws, size_t ws_bytes, hipStream_t s);
 int mfma_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, void* ws,
                size_t ws_bytes, hipStream_t s);
-int mfma_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, void* ws,
+// Input gradient split between the unpadded tile and the neighbours' strips: the produced
+// (padded) tensor has extent g.in; [lo, lo + n) of it is the tile.
+int mfma_dgrad_fold(void* gx, void* const strips[27], const int lo[3], const int n[3], const void* w,
+                    const void* go, const ConvGeom& g, void* ws, size_t ws_bytes, hipStream_t s);
+// gb (Cout,) or NULL: the bias gradient from the same pass over go
+int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom& g, void* ws,
                size_t ws_bytes, hipStream_t s);
 
 }  // namespace jg

@@ -68,7 +68,28 @@ struct FwdParams {
   int tiles_h, tiles_w;
   int total_tiles;      // N * Dout * tiles_h * tiles_w
   int nc16;             // KD * C / 16
+  // Fold mode (input gradient written to its owners): y is the unpadded tile
+  // (N, M, nD, nH, nW); produced cells outside [lo, lo + n) go to the strip of the
+  // neighbour that owns them. fold = 0: y is the whole produced tensor.
+  int fold;
+  int lo_d, lo_h, lo_w, nD, nH, nW;
 };
+
+// Strips of the 26 neighbours, slot (dd+1)*9 + (dh+1)*3 + (dw+1); first kernel
+// parameter, so that a lane can index it in the kernel-argument segment.
+struct StripTable {
+  void* p[27];
+};
+
+__device__ __forceinline__ void* strip_entry(int idx) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  void* const* kt = (void* const*)__builtin_amdgcn_kernarg_segment_ptr();
+  return kt[idx];
+#else
+  (void)idx;
+  return nullptr;
+#endif
+}
 
 // ---------------------------------------------------------------- weight prep
 // dst[((mt*9 + tap9)*nc16 + c16)*2 + kg][m_local][8 k] (bf16), contraction channel
@@ -108,7 +129,7 @@ __global__ __launch_bounds__(256) void prep_weights_kernel(uint16_t* __restrict_
 // pixel pair of a task is one aligned dword that is either wholly inside or wholly
 // outside the tensor. Otherwise the prefetch falls back to 2-byte loads.
 template <int MT, bool EVEN>  // MT = produced channels per workgroup: 32 or 64
-__global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(FwdParams p) {
+__global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips, FwdParams p) {
   constexpr int CB = MT / 32;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int w_slots = TAPS * p.nc16 * 2 * MT;  // 16-byte slots of the weight block
@@ -324,6 +345,76 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(FwdParams p) {
     }
   };
 
+  // Fold-mode epilogue: a produced cell goes to the unpadded tile when it lies inside
+  // [lo, lo + n) on every axis, else to the strip of the neighbour that owns it (dropped
+  // when that neighbour does not exist). Values pass through `0 + v`: the sign of a
+  // zero is cleared, as the reference's scatter-add does for every cell.
+  auto epilogue_fold = [&](int tile) {
+    const TileCoord tc = coord(tile);
+    const int ow = tc.tw * TW + wcol0 + ln;
+    const int hi_d = p.Dout - p.lo_d - p.nD, hi_h = p.Hout - p.lo_h - p.nH, hi_w = p.Wout - p.lo_w - p.nW;
+    const int od = tc.od;
+    const int rd = od < p.lo_d ? 0 : (od < p.lo_d + p.nD ? 1 : 2);
+    const int cd = od - (rd == 0 ? 0 : (rd == 1 ? p.lo_d : p.lo_d + p.nD));
+    const int ed = rd == 0 ? p.lo_d : (rd == 1 ? p.nD : hi_d);
+    const int rw = ow < p.lo_w ? 0 : (ow < p.lo_w + p.nW ? 1 : 2);
+    const int cw = ow - (rw == 0 ? 0 : (rw == 1 ? p.lo_w : p.lo_w + p.nW));
+    const int ew = rw == 0 ? p.lo_w : (rw == 1 ? p.nW : hi_w);
+    const size_t plane0 = (size_t)tc.n * p.M + (size_t)mt * MT;
+    // A tile that lies wholly inside the own extent (wave-uniform test): plain rows of
+    // the unpadded tile, no per-cell routing.
+    const int th0 = tc.th * TH, tw0 = tc.tw * TW;
+    if (rd == 1 && th0 >= p.lo_h && th0 + TH <= p.lo_h + p.nH && tw0 >= p.lo_w && tw0 + TW <= p.lo_w + p.nW) {
+      const size_t ps = (size_t)p.nD * p.nH * p.nW;
+      char* ybase = reinterpret_cast<char*>(p.y) + 2 * (plane0 * ps + (size_t)cd * p.nH * p.nW);
+#pragma unroll
+      for (int r = 0; r < WROWS; ++r) {
+        const int oh = th0 + wrow0 + r - p.lo_h;
+        const uint32_t voff = (uint32_t)(2 * ((size_t)(4 * kg) * ps + (size_t)oh * p.nW + (ow - p.lo_w)));
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+          for (int i = 0; i < 16; i += 2) {
+            f32x2 v2 = {acc[cb][r][i] + 0.0f, acc[cb][r][i + 1] + 0.0f};
+            const bf16x2 h2 = __builtin_convertvector(v2, bf16x2);
+            uint32_t bits = __builtin_bit_cast(uint32_t, h2);
+            if ((bits & 0x00007fffu) == 0) bits &= 0xffff0000u;
+            if ((bits & 0x7fff0000u) == 0) bits &= 0x0000ffffu;
+            const int m0 = cb * 32 + 8 * (i >> 2) + (i & 3);
+            *reinterpret_cast<uint16_t*>(ybase + (size_t)m0 * ps * 2 + voff) = (uint16_t)(bits & 0xffffu);
+            *reinterpret_cast<uint16_t*>(ybase + (size_t)(m0 + 1) * ps * 2 + voff) = (uint16_t)(bits >> 16);
+          }
+      }
+      return;
+    }
+#pragma unroll
+    for (int r = 0; r < WROWS; ++r) {
+      const int oh = tc.th * TH + wrow0 + r;
+      if (oh >= p.Hout || ow >= p.Wout) continue;
+      const int rh = oh < p.lo_h ? 0 : (oh < p.lo_h + p.nH ? 1 : 2);
+      const int ch = oh - (rh == 0 ? 0 : (rh == 1 ? p.lo_h : p.lo_h + p.nH));
+      const int eh = rh == 0 ? p.lo_h : (rh == 1 ? p.nH : hi_h);
+      const int slot = rd * 9 + rh * 3 + rw;
+      char* base = slot == 13 ? reinterpret_cast<char*>(p.y) : static_cast<char*>(strip_entry(slot));
+      if (base == nullptr) continue;
+      const size_t ps = (size_t)ed * eh * ew;  // elements per plane of that destination
+      char* dst = base + 2 * ((plane0 + 4 * kg) * ps + ((size_t)cd * eh + ch) * ew + cw);
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          f32x2 v2 = {acc[cb][r][i] + 0.0f, acc[cb][r][i + 1] + 0.0f};
+          const bf16x2 h2 = __builtin_convertvector(v2, bf16x2);
+          uint32_t bits = __builtin_bit_cast(uint32_t, h2);
+          if ((bits & 0x00007fffu) == 0) bits &= 0xffff0000u;
+          if ((bits & 0x7fff0000u) == 0) bits &= 0x0000ffffu;
+          const int m0 = cb * 32 + 8 * (i >> 2) + (i & 3);
+          *reinterpret_cast<uint16_t*>(dst + (size_t)m0 * ps * 2) = (uint16_t)(bits & 0xffffu);
+          *reinterpret_cast<uint16_t*>(dst + (size_t)(m0 + 1) * ps * 2) = (uint16_t)(bits >> 16);
+        }
+    }
+  };
+
   // ---- main loop over the stages (tile, 16-channel step) of this workgroup. The
   // global loads of a stage are issued a whole stage ahead: right after the previous
   // stage's registers were written to LDS, in the middle of the stage before.
@@ -349,7 +440,8 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(FwdParams p) {
       __syncthreads();
       buf ^= 1;
     }
-    epilogue(tile_of(ti));
+    if (p.fold) epilogue_fold(tile_of(ti));
+    else epilogue(tile_of(ti));
   }
 }
 
@@ -394,6 +486,9 @@ struct Launch {
   int Din, Hin, Win, Dout, Hout, Wout;
   int pad_d, pad_h, pad_w;
   int transposed;
+  int fold;                 // fold mode: y is the unpadded tile, strips receive the halo cells
+  int lo[3], n[3];          // own extent inside the produced tensor (fold mode)
+  void* const* strips;      // 27 slots (fold mode)
 };
 
 int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const char* who) {
@@ -422,6 +517,11 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   JG_REQUIRE(tiles < (1ll << 30), "%s: too many tiles", who);
   p.total_tiles = (int)tiles;
   p.nc16 = K / CK;
+  p.fold = L.fold;
+  p.lo_d = L.lo[0]; p.lo_h = L.lo[1]; p.lo_w = L.lo[2];
+  p.nD = L.n[0]; p.nH = L.n[1]; p.nW = L.n[2];
+  StripTable tab;
+  for (int i = 0; i < 27; ++i) tab.p[i] = (L.fold && L.strips != nullptr) ? L.strips[i] : nullptr;
   if (tiles == 0) return JG_OK;
   const size_t lds = (size_t)TAPS * p.nc16 * 2 * MT * 16 + 2 * (size_t)STAGE_BYTES + MT * 4;
   int wgs = cu_count();
@@ -430,13 +530,13 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   dim3 grid((unsigned)wgs, (unsigned)(L.M / MT), 1);
   const bool even = (L.Win % 2 == 0) && (L.pad_w % 2 == 0) &&
                     ((reinterpret_cast<uintptr_t>(L.x) & 3) == 0);
-  void (*kern)(FwdParams) = nullptr;
+  void (*kern)(StripTable, FwdParams) = nullptr;
   if (MT == 64) kern = even ? &conv3x3_mfma_kernel<64, true> : &conv3x3_mfma_kernel<64, false>;
   else kern = even ? &conv3x3_mfma_kernel<32, true> : &conv3x3_mfma_kernel<32, false>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", who, lds);
-  kern<<<grid, THREADS, lds, s>>>(p);
+  kern<<<grid, THREADS, lds, s>>>(tab, p);
   JG_CHECK_LAUNCH(who);
   return JG_OK;
 }
@@ -470,12 +570,17 @@ int mfma_fwd(void* y, const void* x, const void* w, const void* bias, const Conv
   L.Dout = g.out[0]; L.Hout = g.out[1]; L.Wout = g.out[2];
   L.pad_d = g.p[0]; L.pad_h = g.p[1]; L.pad_w = g.p[2];
   L.transposed = 0;
+  L.fold = 0;
+  L.strips = nullptr;
+  for (int a = 0; a < 3; ++a) L.lo[a] = L.n[a] = 0;
   return launch_conv(L, ws, ws_bytes, s, "jg_conv_fwd(mfma)");
 }
 
-int mfma_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, void* ws,
-               size_t ws_bytes, hipStream_t s) {
-  // gx = conv(go zero-padded by k-1-p, flipped / transposed weights)
+// gx = conv(go zero-padded by k-1-p, flipped / transposed weights). With `own` given,
+// the produced tensor is split between the unpadded tile gx and the neighbours' strips.
+static int dgrad_launch(void* gx, void* const* strips, const int* lo, const int* n, const void* w,
+                        const void* go, const ConvGeom& g, void* ws, size_t ws_bytes, hipStream_t s,
+                        const char* who) {
   Launch L;
   L.x = static_cast<const uint16_t*>(go);
   L.w = static_cast<const uint16_t*>(w);
@@ -486,7 +591,23 @@ int mfma_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, void*
   L.Dout = g.in[0]; L.Hout = g.in[1]; L.Wout = g.in[2];
   L.pad_d = g.k[0] - 1 - g.p[0]; L.pad_h = KH - 1 - g.p[1]; L.pad_w = KW - 1 - g.p[2];
   L.transposed = 1;
-  return launch_conv(L, ws, ws_bytes, s, "jg_conv_dgrad(mfma)");
+  L.fold = lo != nullptr;
+  L.strips = strips;
+  for (int a = 0; a < 3; ++a) {
+    L.lo[a] = lo ? lo[a] : 0;
+    L.n[a] = n ? n[a] : 0;
+  }
+  return launch_conv(L, ws, ws_bytes, s, who);
+}
+
+int mfma_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, void* ws,
+               size_t ws_bytes, hipStream_t s) {
+  return dgrad_launch(gx, nullptr, nullptr, nullptr, w, go, g, ws, ws_bytes, s, "jg_conv_dgrad(mfma)");
+}
+
+int mfma_dgrad_fold(void* gx, void* const strips[27], const int lo[3], const int n[3], const void* w,
+                    const void* go, const ConvGeom& g, void* ws, size_t ws_bytes, hipStream_t s) {
+  return dgrad_launch(gx, strips, lo, n, w, go, g, ws, ws_bytes, s, "jg_conv_dgrad_fold(mfma)");
 }
 
 }  // namespace jg

@@ -1,7 +1,9 @@
 // Weight gradient of the 3x3 (2-D) and 3x3x3 (3-D) convolution on the bf16 matrix
-// cores, stride 1, dilation 1, channels-first tensors, 32 or 64 channels a side.
+// cores, stride 1, dilation 1, channels-first tensors, 32 or 64 channels a side;
+// optionally the bias gradient from the same pass over g.
 //
 //   gw[co][ci][kd][kh][kw] = sum_{n,d,h,w} g[n][co][d][h][w] * x[n][ci][d+kd-pd][h+kh-ph][w+kw-pw]
+//   gb[co]                 = sum_{n,d,h,w} g[n][co][d][h][w]
 //
 //   GEMM view   M = output channels, N = input channels (x depth taps), K = pixels.
 //               Both operands are pixel-contiguous in the channels-first tensors, so
@@ -17,12 +19,18 @@
 //               whole kernel (144 VGPRs) and walks the pixels. 64->64 2-D: 2x2x2 = 8
 //               wavefronts (two per SIMD, which is what hides the barrier and LDS
 //               write phases); 32->32 3-D: 1x3x2 = 6, plus two that only prefetch.
-//   Stage       2 output rows x 64 columns: g tile C x 2 x 64, x tile C' x 4 x 72;
-//               prefetched to registers during the MFMAs of the previous stage,
-//               double buffered in LDS (one barrier per stage). Channel strides in
-//               LDS are odd multiples of 16 bytes so that the 32 channel-lanes of a
-//               fragment read hit distinct banks. Stages that lie wholly inside the
-//               tensors (a wave-uniform test) take a branch-free vector load path.
+//   Stage       2 output rows x 64 columns; consecutive stages of a workgroup walk
+//               down one column strip, so two of the four x rows a stage reads are
+//               the previous stage's last two. The x rows therefore live in a ring of
+//               6 rows per channel in LDS and a stage fetches only its two new rows
+//               (each x element is read from memory once per strip, apart from the
+//               8 halo columns), plus its two g rows (double buffered). Loads go
+//               through registers and are issued a whole stage ahead. The first stage
+//               of a strip or of a workgroup fetches its other two rows on the spot.
+//               Channel strides in LDS are odd multiples of 16 bytes so that the 32
+//               channel-lanes of a fragment read hit distinct banks.
+//   Bias grad   the lanes that carry the g chunks to LDS add them up on the way
+//               (fp32), one partial per workgroup and channel.
 //   Reduction   every wavefront writes its partial to the workspace; a second kernel
 //               sums the partials in a fixed order (deterministic) and writes gw in
 //               the weight layout.
@@ -38,17 +46,19 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
 constexpr int SR = 2, SW = 64;        // output rows / columns per stage
-constexpr int XR = SR + 2;            // x rows per stage
+constexpr int XR = SR + 2;            // x rows a stage reads
+constexpr int RING = 6;               // x rows resident per channel
 constexpr int G_CH = SR * SW * 2 + 16;        // 272 bytes per g channel
 constexpr int X_ROW = 144;                    // 72 pixels
-constexpr int X_CH = XR * X_ROW + 16;         // 592 bytes per x channel
-constexpr int X_CPR = 9;                      // 8-pixel chunks per x row
+constexpr int X_CH = RING * X_ROW + 16;       // 880 bytes per x channel
+constexpr int X_CPR = 8;                      // 8-pixel chunks per x row; 2 more pixels follow as one dword
 
 struct WgradParams {
   const uint16_t* x;  // (N, Cin, Din, Hin, Win)
   const uint16_t* g;  // (N, Cout, Dout, Hout, Wout)
   const char* x_end;  // one past the last byte of x
   float* part;        // [wavefront slot][tap9][co][c']
+  float* bias_part;   // [workgroup][co] or NULL
   int Cin, Cout;
   int Din, Hin, Win, Dout, Hout, Wout;
   int pad_d, pad_h, pad_w;
@@ -63,18 +73,27 @@ constexpr int wgrad_threads(int cgb, int cxb) {
   return (cgb * cxb * HALVES > 4) ? 512 : 64 * cgb * cxb * HALVES;
 }
 
+// sum of the 8 bf16 values of a chunk
+__device__ __forceinline__ float sum_bf16x8(const u32x4& v) {
+  float s = __uint_as_float(v.x << 16) + __uint_as_float(v.x & 0xffff0000u);
+  s += __uint_as_float(v.y << 16) + __uint_as_float(v.y & 0xffff0000u);
+  s += __uint_as_float(v.z << 16) + __uint_as_float(v.z & 0xffff0000u);
+  s += __uint_as_float(v.w << 16) + __uint_as_float(v.w & 0xffff0000u);
+  return s;
+}
+
 template <int CGB, int CXB, bool EVEN>
 __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(WgradParams p) {
   constexpr int THREADS = wgrad_threads(CGB, CXB);
   constexpr int CWAVES = CGB * CXB * HALVES;  // wavefronts that own accumulators
   constexpr int GC = 32 * CGB, XC = 32 * CXB;
-  constexpr int G_BYTES = GC * G_CH, X_BYTES = XC * X_CH;
-  constexpr int STAGE_BYTES = G_BYTES + X_BYTES;
+  constexpr int G_BYTES = GC * G_CH;          // one g buffer
   constexpr int G_CHUNKS = GC * SR * (SW / 8);
-  constexpr int X_CHUNKS = XC * XR * X_CPR;
-  constexpr int CHUNKS = G_CHUNKS + X_CHUNKS;
+  constexpr int XP_CHUNKS = XC * 2 * X_CPR;   // one pair of x rows
+  constexpr int CHUNKS = G_CHUNKS + XP_CHUNKS;
   constexpr int ROUNDS = (CHUNKS + THREADS - 1) / THREADS;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  unsigned char* const lds_x = smem + 2 * G_BYTES;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, kgp = lane >> 5;
@@ -82,7 +101,7 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
   const int cb = pair / CXB, ib = pair % CXB;
 
   // contiguous range of stages for this workgroup; stage -> (n, d, column tile, row pair),
-  // row pair fastest, so consecutive stages walk down one column of one plane
+  // row pair fastest, so consecutive stages walk down one column strip of one plane
   const long long per = (p.total_stages + gridDim.x - 1) / gridDim.x;
   const long long s_begin = per * blockIdx.x;
   long long s_end = s_begin + per;
@@ -91,9 +110,11 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
   const size_t plane_x = (size_t)p.Hin * p.Win, plane_g = (size_t)p.Hout * p.Wout;
   const size_t x_cs = plane_x * p.Din, g_cs = plane_g * p.Dout;  // channel strides
 
-  // ---- per-thread chunk bookkeeping, fixed for the whole kernel
-  uint32_t c_goff[ROUNDS];  // byte offset from the stage origin of its tensor
-  uint32_t c_lds[ROUNDS];   // byte offset inside a stage buffer
+  // ---- per-thread chunk bookkeeping, fixed for the whole kernel. Chunk q < G_CHUNKS
+  // is 8 pixels of a g row, the others 8 pixels of one of the two x rows of a pair.
+  uint32_t c_goff[ROUNDS];  // byte offset from the origin of its tensor window
+  uint32_t c_lds[ROUNDS];   // byte offset inside the g buffer / inside the x ring, row slot 0
+  uint32_t x_second = 0;    // bit rd: the chunk belongs to the second row of the pair
 #pragma unroll
   for (int rd = 0; rd < ROUNDS; ++rd) {
     const int q = tid + rd * THREADS;
@@ -103,54 +124,92 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
       c_lds[rd] = (uint32_t)(ch * G_CH + r * (SW * 2) + c8 * 16);
     } else if (q < CHUNKS) {
       const int qx = q - G_CHUNKS;
-      const int c9 = qx % X_CPR;
+      const int c8 = qx % X_CPR;
       const int rr = qx / X_CPR;
-      const int rho = rr % XR, ch = rr / XR;     // ch = kd * Cin + ci
+      const int r2 = rr & 1, ch = rr >> 1;      // ch = kd * Cin + ci
       const int kd = ch / p.Cin, ci = ch - kd * p.Cin;
-      c_goff[rd] = (uint32_t)((ci * x_cs + kd * plane_x + (size_t)rho * p.Win + c9 * 8) * 2);
-      c_lds[rd] = (uint32_t)(G_BYTES + ch * X_CH + rho * X_ROW + c9 * 16);
+      c_goff[rd] = (uint32_t)((ci * x_cs + kd * plane_x + (size_t)r2 * p.Win + c8 * 8) * 2);
+      c_lds[rd] = (uint32_t)(ch * X_CH + c8 * 16);
+      x_second |= (uint32_t)r2 << rd;
     } else {
       c_goff[rd] = 0;
       c_lds[rd] = 0;
     }
   }
+  // pixels 64, 65 of an x row: one dword, carried by the first 2 * XC threads
+  const bool has_tail = tid < 2 * XC;
+  uint32_t t_goff = 0, t_lds = 0;
+  if (has_tail) {
+    const int r2 = tid & 1, ch = tid >> 1;
+    const int kd = ch / p.Cin, ci = ch - kd * p.Cin;
+    t_goff = (uint32_t)((ci * x_cs + kd * plane_x + (size_t)r2 * p.Win + SW) * 2);
+    t_lds = (uint32_t)(ch * X_CH + SW * 2);
+  }
 
-  u32x4 stg[ROUNDS];
-  auto issue_loads = [&](long long stage) {
-    const int hp = (int)(stage % p.row_pairs);
+  struct Staged {
+    u32x4 v[ROUNDS];
+    uint32_t tail;
+  };
+
+  // Loads of one stage into `v`: its two g rows (want_g) and one pair of its x rows
+  // (pair 0: the rows shared with the stage above, pair 1: the two new rows).
+  // Position of a stage: row pair (fastest), column tile, output depth, batch entry.
+  // Decoded once with divisions, then stepped, so the stage loop has none.
+  struct Cursor {
+    int hp, ct, od, n;
+  };
+  auto decode = [&](long long stage) {
+    Cursor c;
+    c.hp = (int)(stage % p.row_pairs);
     long long t = stage / p.row_pairs;
-    const int ct = (int)(t % p.col_tiles);
+    c.ct = (int)(t % p.col_tiles);
     t /= p.col_tiles;
-    const int od = (int)(t % p.Dout);
-    const int n = (int)(t / p.Dout);
+    c.od = (int)(t % p.Dout);
+    c.n = (int)(t / p.Dout);
+    return c;
+  };
+  auto advance = [&](Cursor& c) {
+    if (++c.hp == p.row_pairs) {
+      c.hp = 0;
+      if (++c.ct == p.col_tiles) {
+        c.ct = 0;
+        if (++c.od == p.Dout) {
+          c.od = 0;
+          ++c.n;
+        }
+      }
+    }
+  };
+
+  auto issue_loads = [&](Staged& sg, const Cursor& cur, bool want_g, int xpair) {
+    u32x4 (&v)[ROUNDS] = sg.v;
+    const int hp = cur.hp, ct = cur.ct, od = cur.od, n = cur.n;
     const int oh0 = hp * SR, ow0 = ct * SW;
-    const int id0 = od - p.pad_d, ih0 = oh0 - p.pad_h, iw0 = ow0 - p.pad_w;
+    const int id0 = od - p.pad_d, ih0 = oh0 - p.pad_h + 2 * xpair, iw0 = ow0 - p.pad_w;
     const char* g_org = reinterpret_cast<const char*>(p.g) +
                         2 * (((size_t)n * p.Cout * p.Dout + od) * plane_g + (size_t)oh0 * p.Wout + ow0);
     const char* x_org = reinterpret_cast<const char*>(p.x) +
                         2 * ((ptrdiff_t)((size_t)n * p.Cin * p.Din * plane_x) + (ptrdiff_t)id0 * (ptrdiff_t)plane_x +
                              (ptrdiff_t)ih0 * p.Win + iw0);
-    // The last 8-pixel chunk of an x row holds 2 pixels that are used and 6 that no
-    // fragment reads, so it may run past the row end as long as it stays inside the tensor.
-    const char* x_last = x_org + 2 * ((size_t)(p.Cin - 1) * x_cs + (size_t)(XC / p.Cin - 1) * plane_x +
-                                      (size_t)(XR - 1) * p.Win + X_CPR * 8);
     const bool inside = EVEN && oh0 + SR <= p.Hout && ow0 + SW <= p.Wout && ih0 >= 0 &&
-                        ih0 + XR <= p.Hin && iw0 >= 0 && iw0 + SW + 2 <= p.Win && id0 >= 0 &&
-                        id0 + (XC / p.Cin) <= p.Din && x_last <= p.x_end;
+                        ih0 + 2 <= p.Hin && iw0 >= 0 && iw0 + SW + 2 <= p.Win && id0 >= 0 &&
+                        id0 + (XC / p.Cin) <= p.Din;
     if (inside) {
 #pragma unroll
       for (int rd = 0; rd < ROUNDS; ++rd) {
-        if (tid + rd * THREADS < CHUNKS) {
-          const char* org = (tid + rd * THREADS < G_CHUNKS) ? g_org : x_org;
-          stg[rd] = *reinterpret_cast<const u32x4_a4*>(org + c_goff[rd]);
+        const int q = tid + rd * THREADS;
+        if (q < CHUNKS && (want_g || q >= G_CHUNKS)) {
+          const char* org = (q < G_CHUNKS) ? g_org : x_org;
+          v[rd] = *reinterpret_cast<const u32x4_a4*>(org + c_goff[rd]);
         }
       }
+      if (has_tail) sg.tail = *reinterpret_cast<const uint32_t*>(x_org + t_goff);
     } else {
 #pragma unroll
       for (int rd = 0; rd < ROUNDS; ++rd) {
         const int q = tid + rd * THREADS;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (q < CHUNKS) {
+        u32x4 val = {0u, 0u, 0u, 0u};
+        if (q < CHUNKS && (want_g || q >= G_CHUNKS)) {
           const bool is_x = q >= G_CHUNKS;
           const uint16_t* src;
           int row, col, rows, cols;
@@ -161,35 +220,62 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
             row = oh0 + r; col = ow0 + c8 * 8; rows = p.Hout; cols = p.Wout;
           } else {
             const int qx = q - G_CHUNKS;
-            const int c9 = qx % X_CPR, rr = qx / X_CPR;
-            const int rho = rr % XR, ch = rr / XR;
+            const int c8 = qx % X_CPR, rr = qx / X_CPR;
+            const int r2 = rr & 1, ch = rr >> 1;
             src = reinterpret_cast<const uint16_t*>(x_org + c_goff[rd]);
-            row = ih0 + rho; col = iw0 + c9 * 8; rows = p.Hin; cols = p.Win;
+            row = ih0 + r2; col = iw0 + c8 * 8; rows = p.Hin; cols = p.Win;
             const int dd = id0 + ch / p.Cin;
             ok = dd >= 0 && dd < p.Din;
           }
           if (ok && row >= 0 && row < rows) {
             if (col >= 0 && col + 8 <= cols && (reinterpret_cast<uintptr_t>(src) & 3) == 0) {
-              v = *reinterpret_cast<const u32x4_a4*>(src);
+              val = *reinterpret_cast<const u32x4_a4*>(src);
             } else {
               uint32_t e[8];
 #pragma unroll
               for (int k = 0; k < 8; ++k) e[k] = (col + k >= 0 && col + k < cols) ? (uint32_t)src[k] : 0u;
-              v.x = e[0] | (e[1] << 16); v.y = e[2] | (e[3] << 16);
-              v.z = e[4] | (e[5] << 16); v.w = e[6] | (e[7] << 16);
+              val.x = e[0] | (e[1] << 16); val.y = e[2] | (e[3] << 16);
+              val.z = e[4] | (e[5] << 16); val.w = e[6] | (e[7] << 16);
             }
           }
         }
-        stg[rd] = v;
+        v[rd] = val;
+      }
+      if (has_tail) {
+        const int r2 = tid & 1, ch = tid >> 1;
+        const int row = ih0 + r2, col = iw0 + SW, dd = id0 + ch / p.Cin;
+        const uint16_t* src = reinterpret_cast<const uint16_t*>(x_org + t_goff);
+        uint32_t lo = 0u, hi = 0u;
+        if (dd >= 0 && dd < p.Din && row >= 0 && row < p.Hin) {
+          if (col >= 0 && col < p.Win) lo = src[0];
+          if (col + 1 >= 0 && col + 1 < p.Win) hi = src[1];
+        }
+        sg.tail = lo | (hi << 16);
       }
     }
   };
 
-  auto store_stage = [&](int buf) {
-    unsigned char* base = smem + buf * STAGE_BYTES;
+  // Registers of a stage to LDS: g rows into g buffer `gbuf`, the x pair into ring rows
+  // `slot_a`, `slot_b`; the g chunks are added into the bias partials on the way.
+  float bsum[ROUNDS];
 #pragma unroll
-    for (int rd = 0; rd < ROUNDS; ++rd)
-      if (tid + rd * THREADS < CHUNKS) *reinterpret_cast<u32x4*>(base + c_lds[rd]) = stg[rd];
+  for (int rd = 0; rd < ROUNDS; ++rd) bsum[rd] = 0.0f;
+  auto store_loads = [&](const Staged& sg, bool have_g, int gbuf, int slot_a, int slot_b) {
+    const u32x4 (&v)[ROUNDS] = sg.v;
+#pragma unroll
+    for (int rd = 0; rd < ROUNDS; ++rd) {
+      const int q = tid + rd * THREADS;
+      if (q < G_CHUNKS) {
+        if (have_g) {
+          *reinterpret_cast<u32x4*>(smem + gbuf * G_BYTES + c_lds[rd]) = v[rd];
+          if (p.bias_part != nullptr) bsum[rd] += sum_bf16x8(v[rd]);
+        }
+      } else if (q < CHUNKS) {
+        const int slot = ((x_second >> rd) & 1u) ? slot_b : slot_a;
+        *reinterpret_cast<u32x4*>(lds_x + c_lds[rd] + slot * X_ROW) = v[rd];
+      }
+    }
+    if (has_tail) *reinterpret_cast<uint32_t*>(lds_x + t_lds + ((tid & 1) ? slot_b : slot_a) * X_ROW) = sg.tail;
   };
 
   f32x16 acc[3][3];
@@ -200,58 +286,99 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.0f;
 
-  // one 16-pixel column group (cgi = 0 or 1 of this wavefront's half) of a stage
-  auto compute_group = [&](int buf, int cgi) {
-    const unsigned char* gb = smem + buf * STAGE_BYTES + (cb * 32 + ln) * G_CH + kgp * 16;
-    const unsigned char* xb = smem + buf * STAGE_BYTES + G_BYTES + (ib * 32 + ln) * X_CH + kgp * 16;
-    {
-      const int cg = half * (SW / 16 / HALVES) + cgi;  // 16-pixel column group of this wavefront
-      bf16x8 a[SR];
+  // one 16-pixel column group (cgi = 0 or 1 of this wavefront's half) of a stage whose
+  // four x rows sit in ring rows base .. base + 3 (mod RING)
+  auto compute_group = [&](int gbuf, int base, int cgi) {
+    const unsigned char* gb = smem + gbuf * G_BYTES + (cb * 32 + ln) * G_CH + kgp * 16;
+    const unsigned char* xb = lds_x + (ib * 32 + ln) * X_CH + kgp * 16;
+    const int cg = half * (SW / 16 / HALVES) + cgi;  // 16-pixel column group of this wavefront
+    bf16x8 a[SR];
 #pragma unroll
-      for (int r = 0; r < SR; ++r)
-        a[r] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(gb + r * (SW * 2) + cg * 32));
+    for (int r = 0; r < SR; ++r)
+      a[r] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(gb + r * (SW * 2) + cg * 32));
 #pragma unroll
-      for (int rho = 0; rho < XR; ++rho) {
-        const u32x4 d = *reinterpret_cast<const u32x4*>(xb + rho * X_ROW + cg * 32);
-        const uint32_t d4 = *reinterpret_cast<const uint32_t*>(xb + rho * X_ROW + cg * 32 + 16);
-        u32x4 s1, s2;
-        s1.x = __builtin_amdgcn_alignbit(d.y, d.x, 16);
-        s1.y = __builtin_amdgcn_alignbit(d.z, d.y, 16);
-        s1.z = __builtin_amdgcn_alignbit(d.w, d.z, 16);
-        s1.w = __builtin_amdgcn_alignbit(d4, d.w, 16);
-        s2.x = d.y; s2.y = d.z; s2.z = d.w; s2.w = d4;
-        const bf16x8 b0 = __builtin_bit_cast(bf16x8, d);
-        const bf16x8 b1 = __builtin_bit_cast(bf16x8, s1);
-        const bf16x8 b2 = __builtin_bit_cast(bf16x8, s2);
+    for (int rho = 0; rho < XR; ++rho) {
+      int slot = base + rho;
+      if (slot >= RING) slot -= RING;
+      const u32x4 d = *reinterpret_cast<const u32x4*>(xb + slot * X_ROW + cg * 32);
+      const uint32_t d4 = *reinterpret_cast<const uint32_t*>(xb + slot * X_ROW + cg * 32 + 16);
+      u32x4 s1, s2;
+      s1.x = __builtin_amdgcn_alignbit(d.y, d.x, 16);
+      s1.y = __builtin_amdgcn_alignbit(d.z, d.y, 16);
+      s1.z = __builtin_amdgcn_alignbit(d.w, d.z, 16);
+      s1.w = __builtin_amdgcn_alignbit(d4, d.w, 16);
+      s2.x = d.y; s2.y = d.z; s2.z = d.w; s2.w = d4;
+      const bf16x8 b0 = __builtin_bit_cast(bf16x8, d);
+      const bf16x8 b1 = __builtin_bit_cast(bf16x8, s1);
+      const bf16x8 b2 = __builtin_bit_cast(bf16x8, s2);
 #pragma unroll
-        for (int r = 0; r < SR; ++r) {
-          const int kh = rho - r;
-          if (kh >= 0 && kh < 3) {
-            acc[kh][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r], b0, acc[kh][0], 0, 0, 0);
-            acc[kh][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r], b1, acc[kh][1], 0, 0, 0);
-            acc[kh][2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r], b2, acc[kh][2], 0, 0, 0);
-          }
+      for (int r = 0; r < SR; ++r) {
+        const int kh = rho - r;
+        if (kh >= 0 && kh < 3) {
+          acc[kh][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r], b0, acc[kh][0], 0, 0, 0);
+          acc[kh][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r], b1, acc[kh][1], 0, 0, 0);
+          acc[kh][2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r], b2, acc[kh][2], 0, 0, 0);
         }
       }
     }
   };
 
-  // The global loads of a stage are issued a whole stage ahead: right after the previous
-  // stage's registers went to LDS, between the two column groups of the stage before.
+  // Stage k of this workgroup reads ring rows base_k .. base_k + 3 with base_k = 2k mod 6:
+  // its first two rows are where the stage before put its new rows (base_k-1 + 2, + 3), its
+  // new rows go to base_k + 2, + 3. A stage that does not continue the strip of the stage
+  // before fetches its first two rows itself, into those same ring rows.
   static_assert(SW / 16 / HALVES == 2, "the stage loop is written for two column groups per wavefront");
+  auto wrap = [](int v) { return v >= RING ? v - RING : v; };
   if (s_begin < s_end) {
-    int buf = 0;
-    issue_loads(s_begin);
-    store_stage(0);
-    if (s_begin + 1 < s_end) issue_loads(s_begin + 1);
+    Staged stg;
+    int gbuf = 0, base = 0;
+    Cursor c_next = decode(s_begin);  // stage whose loads are issued next
+    issue_loads(stg, c_next, true, 1);
+    store_loads(stg, true, 0, 2, 3);
+    issue_loads(stg, c_next, false, 0);
+    store_loads(stg, false, 0, 0, 1);
+    advance(c_next);
+    Cursor c_store = c_next;          // stage whose registers are stored next (st + 1)
+    if (s_begin + 1 < s_end) {
+      issue_loads(stg, c_next, true, 1);
+      advance(c_next);
+    }
     __syncthreads();
     for (long long st = s_begin; st < s_end; ++st) {
-      if (wave < CWAVES) compute_group(buf, 0);
-      if (st + 1 < s_end) store_stage(buf ^ 1);
-      if (st + 2 < s_end) issue_loads(st + 2);
-      if (wave < CWAVES) compute_group(buf, 1);
+      if (wave < CWAVES) compute_group(gbuf, base, 0);
+      if (st + 1 < s_end) store_loads(stg, true, gbuf ^ 1, wrap(base + 4), wrap(base + 5));
+      if (st + 2 < s_end) {
+        issue_loads(stg, c_next, true, 1);
+        advance(c_next);
+      }
+      if (wave < CWAVES) compute_group(gbuf, base, 1);
       __syncthreads();
-      buf ^= 1;
+      if (st + 1 < s_end && c_store.hp == 0) {
+        // the next stage starts a new strip: its first two x rows, on the spot
+        Staged top;
+        issue_loads(top, c_store, false, 0);
+        store_loads(top, false, 0, wrap(base + 2), wrap(base + 3));
+        __syncthreads();
+      }
+      advance(c_store);
+      base = wrap(base + 2);
+      gbuf ^= 1;
+    }
+  }
+
+  // bias partial of this workgroup: the 16 lanes that carried a channel's chunks add up
+  if (p.bias_part != nullptr) {
+#pragma unroll
+    for (int rd = 0; rd < ROUNDS; ++rd) {
+      const int q = tid + rd * THREADS;
+      if (rd * THREADS < G_CHUNKS) {  // rounds that hold g chunks (whole rounds: THREADS divides G_CHUNKS)
+        float s = bsum[rd];
+        s += __shfl_xor(s, 8, 64);
+        s += __shfl_xor(s, 4, 64);
+        s += __shfl_xor(s, 2, 64);
+        s += __shfl_xor(s, 1, 64);
+        if (q < G_CHUNKS && (tid & 15) == 0) p.bias_part[(size_t)blockIdx.x * GC + q / (8 * SR)] = s;
+      }
     }
   }
 
@@ -267,6 +394,21 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
         const int co = cb * 32 + 8 * (i >> 2) + 4 * kgp + (i & 3);
         out[((kh * 3 + kw) * GC + co) * XC + ib * 32 + ln] = acc[kh][kw][i];
       }
+}
+
+// gb[co] (bf16) = sum over the workgroups of bias_part[wg][co]; one wavefront per channel,
+// fixed order.
+__global__ __launch_bounds__(256) void wgrad_bias_reduce_kernel(uint16_t* __restrict__ gb,
+                                                                const float* __restrict__ part,
+                                                                int wgs, int GC) {
+  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (c >= GC) return;
+  float s = 0.0f;
+  for (int k = lane; k < wgs; k += 64) s += part[(size_t)k * GC + c];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+  if (lane == 0) gb[c] = jg::f32_to_bf16(s);
 }
 
 // gw[co][ci][kd][kh][kw] (bf16) = sum over the slots of part[slot][tap9][co][kd*Cin+ci].
@@ -342,7 +484,7 @@ bool blocks_of(const ConvGeom& g, int* cgb, int* cxb) {
 template <int CGB, int CXB>
 int launch(const WgradParams& p, bool even, int wgs, hipStream_t s, const char* who) {
   constexpr int THREADS = wgrad_threads(CGB, CXB);
-  const size_t lds = 2 * (size_t)(32 * CGB * G_CH + 32 * CXB * X_CH);
+  const size_t lds = 2 * (size_t)(32 * CGB * G_CH) + (size_t)(32 * CXB * X_CH);
   void (*kern)(WgradParams) =
       even ? &wgrad3x3_mfma_kernel<CGB, CXB, true> : &wgrad3x3_mfma_kernel<CGB, CXB, false>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -365,10 +507,11 @@ bool mfma_wgrad_supported(const ConvGeom& g, int dtype) {
 size_t mfma_wgrad_workspace(const ConvGeom& g) {
   int cgb = 1, cxb = 1;
   blocks_of(g, &cgb, &cxb);
-  return (size_t)wg_count(stage_count(g)) * HALVES * 9 * (32 * cgb) * (32 * cxb) * sizeof(float);
+  const size_t wgs = (size_t)wg_count(stage_count(g));
+  return wgs * HALVES * 9 * (32 * cgb) * (32 * cxb) * sizeof(float) + wgs * (32 * cgb) * sizeof(float);
 }
 
-int mfma_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, void* ws,
+int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom& g, void* ws,
                size_t ws_bytes, hipStream_t s) {
   const char* who = "jg_conv_wgrad(mfma)";
   int cgb, cxb;
@@ -391,6 +534,7 @@ int mfma_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, void*
   p.col_tiles = (g.out[2] + SW - 1) / SW;
   p.total_stages = stage_count(g);
   const int wgs = wg_count(p.total_stages);
+  p.bias_part = gb != nullptr ? p.part + (size_t)wgs * HALVES * 9 * (32 * cgb) * (32 * cxb) : nullptr;
   const bool even = (p.Win % 2 == 0) && (p.pad_w % 2 == 0) && (p.Wout % 2 == 0) &&
                     ((reinterpret_cast<uintptr_t>(x) & 3) == 0) &&
                     ((reinterpret_cast<uintptr_t>(go) & 3) == 0);
@@ -407,6 +551,11 @@ int mfma_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, void*
   wgrad_reduce_kernel<<<(count + 63) / 64, 256, 0, s>>>(static_cast<uint16_t*>(gw), p.part, wgs * HALVES,
                                                           32 * cgb, 32 * cxb, g.cin);
   JG_CHECK_LAUNCH(who);
+  if (gb != nullptr) {
+    wgrad_bias_reduce_kernel<<<(32 * cgb + 3) / 4, 256, 0, s>>>(static_cast<uint16_t*>(gb), p.bias_part, wgs,
+                                                                32 * cgb);
+    JG_CHECK_LAUNCH(who);
+  }
   return JG_OK;
 }
 

@@ -490,6 +490,92 @@ __device__ __forceinline__ typename Arith<DT>::T fold_one_rolled(
   return Arith<DT>::down(acc_d);
 }
 
+// Columns [c0, c0 + cnt), cnt <= V, of a row that D or H neighbours may reach: the full
+// ordered sum. Per (od, oh) the middle term is one 16-byte load (cnt == V) from the own
+// row or from that neighbour's strip; the W-neighbour terms touch only the first and
+// last columns. `self_row` points at column 0 of the own contribution of this row (the
+// padded gradient, or the destination itself for an in-place fold).
+template <int DT>
+__device__ __forceinline__ void fold_span(typename Arith<DT>::T* drow,
+                                          const typename Arith<DT>::T* self_row, const Geom& g,
+                                          long long p, int d, int h, int c0, int cnt) {
+  typedef typename Arith<DT>::T T;
+  constexpr int V = Bits<T>::V;
+  typedef uint32_t u32x4_e __attribute__((ext_vector_type(4), aligned(2)));
+  const int D = g.n[0], H = g.n[1], W = g.n[2];
+  const int up0 = W - g.lo[2];
+  const bool edge = c0 < g.hi[2] || c0 + cnt > up0;
+  float acc_d[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) acc_d[e] = 0.0f;
+#pragma unroll 1
+  for (int od = -1; od <= 1; ++od) {
+    int cd, ed;
+    if (!reach(od, d, g.lo[0], D, g.hi[0], cd, ed)) continue;
+    float acc_h[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc_h[e] = 0.0f;
+#pragma unroll 1
+    for (int oh = -1; oh <= 1; ++oh) {
+      int ch, eh;
+      if (!reach(oh, h, g.lo[1], H, g.hi[1], ch, eh)) continue;
+      const long long line = (p * ed + cd) * eh + ch;  // row index inside a strip of (od, oh)
+      const int slot = (od + 1) * 9 + (oh + 1) * 3;
+      const bool self = od == 0 && oh == 0;
+      const T* mid = self ? self_row : static_cast<const T*>(table_entry(slot + 1));
+      if (!self && mid != nullptr) mid += line * W;
+      T mb[V];
+#pragma unroll
+      for (int e = 0; e < V; ++e) mb[e] = T(0);
+      if (mid != nullptr) {
+        if (cnt == V) {
+          const u32x4 mv = *reinterpret_cast<const u32x4_e*>(mid + c0);
+          __builtin_memcpy(mb, &mv, 16);
+        } else {
+#pragma unroll
+          for (int e = 0; e < V; ++e)
+            if (e < cnt) mb[e] = mid[c0 + e];
+        }
+      }
+      float acc_w[V];
+      if (!edge) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc_w[e] = Arith<DT>::up(Arith<DT>::down(0.0f + Arith<DT>::up(mb[e])));
+      } else {
+        const T* s_lo = static_cast<const T*>(table_entry(slot + 0));
+        const T* s_hi = static_cast<const T*>(table_entry(slot + 2));
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          const int c = c0 + e;
+          float a = 0.0f;
+          if (e < cnt && c < g.hi[2] && s_lo != nullptr)
+            a = Arith<DT>::up(Arith<DT>::down(a + Arith<DT>::up(s_lo[line * g.hi[2] + c])));
+          a = Arith<DT>::up(Arith<DT>::down(a + Arith<DT>::up(mb[e])));
+          if (e < cnt && c >= up0 && s_hi != nullptr)
+            a = Arith<DT>::up(Arith<DT>::down(a + Arith<DT>::up(s_hi[line * g.lo[2] + (c - up0)])));
+          acc_w[e] = a;
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc_h[e] = Arith<DT>::up(Arith<DT>::down(acc_h[e] + acc_w[e]));
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc_d[e] = Arith<DT>::up(Arith<DT>::down(acc_d[e] + acc_h[e]));
+  }
+  T ob[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) ob[e] = Arith<DT>::down(acc_d[e]);
+  if (cnt == V) {
+    u32x4 out;
+    __builtin_memcpy(&out, ob, 16);
+    *reinterpret_cast<u32x4_e*>(drow + c0) = out;
+  } else {
+#pragma unroll
+    for (int e = 0; e < V; ++e)
+      if (e < cnt) drow[c0 + e] = ob[e];
+  }
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
                                                         typename Arith<DT>::T* __restrict__ dst,
@@ -516,74 +602,9 @@ __global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
   const T* orow = own + ((p * Da + (d + g.lo[0])) * Ha + (h + g.lo[1])) * (long long)Wa + g.lo[2];
   T* drow = dst + (long long)row * W;
   if (!row_plain) {
-    // A row that a D or H neighbour reaches: the full ordered sum, a vector of columns
-    // at a time. Per (od, oh) the middle term is one 16-byte load from the own padded
-    // row or from the strip of that neighbour; the W-neighbour terms touch only the
-    // first and last columns.
-    const int up0 = W - g.lo[2];
     const int n_vec = W / V;
-    for (int j = lir; j < n_vec; j += (1 << pl.lpr_log2)) {
-      const int c0 = j * V;
-      const bool edge = c0 < g.hi[2] || c0 + V > up0;
-      float acc_d[V];
-#pragma unroll
-      for (int e = 0; e < V; ++e) acc_d[e] = 0.0f;
-#pragma unroll 1
-      for (int od = -1; od <= 1; ++od) {
-        int cd, ed;
-        if (!reach(od, d, g.lo[0], D, g.hi[0], cd, ed)) continue;
-        float acc_h[V];
-#pragma unroll
-        for (int e = 0; e < V; ++e) acc_h[e] = 0.0f;
-#pragma unroll 1
-        for (int oh = -1; oh <= 1; ++oh) {
-          int ch, eh;
-          if (!reach(oh, h, g.lo[1], H, g.hi[1], ch, eh)) continue;
-          const long long line = (p * ed + cd) * eh + ch;  // row index inside a strip of (od, oh)
-          const int slot = (od + 1) * 9 + (oh + 1) * 3;
-          const bool self = od == 0 && oh == 0;
-          const T* mid = self ? orow : static_cast<const T*>(table_entry(slot + 1));
-          if (!self && mid != nullptr) mid += line * W;
-          T mb[V];
-#pragma unroll
-          for (int e = 0; e < V; ++e) mb[e] = T(0);
-          if (mid != nullptr) {
-            const u32x4 mv = load16_unaligned<T>(mid + c0);
-            __builtin_memcpy(mb, &mv, 16);
-          }
-          float acc_w[V];
-          if (!edge) {
-#pragma unroll
-            for (int e = 0; e < V; ++e) acc_w[e] = Arith<DT>::up(Arith<DT>::down(0.0f + Arith<DT>::up(mb[e])));
-          } else {
-            const T* s_lo = static_cast<const T*>(table_entry(slot + 0));
-            const T* s_hi = static_cast<const T*>(table_entry(slot + 2));
-#pragma unroll
-            for (int e = 0; e < V; ++e) {
-              const int c = c0 + e;
-              float a = 0.0f;
-              if (c < g.hi[2] && s_lo != nullptr)
-                a = Arith<DT>::up(Arith<DT>::down(a + Arith<DT>::up(s_lo[line * g.hi[2] + c])));
-              a = Arith<DT>::up(Arith<DT>::down(a + Arith<DT>::up(mb[e])));
-              if (c >= up0 && s_hi != nullptr)
-                a = Arith<DT>::up(Arith<DT>::down(a + Arith<DT>::up(s_hi[line * g.lo[2] + (c - up0)])));
-              acc_w[e] = a;
-            }
-          }
-#pragma unroll
-          for (int e = 0; e < V; ++e) acc_h[e] = Arith<DT>::up(Arith<DT>::down(acc_h[e] + acc_w[e]));
-        }
-#pragma unroll
-        for (int e = 0; e < V; ++e) acc_d[e] = Arith<DT>::up(Arith<DT>::down(acc_d[e] + acc_h[e]));
-      }
-      T ob[V];
-#pragma unroll
-      for (int e = 0; e < V; ++e) ob[e] = Arith<DT>::down(acc_d[e]);
-      u32x4 out;
-      __builtin_memcpy(&out, ob, 16);
-      *reinterpret_cast<u32x4_s4*>(drow + c0) = out;
-    }
-    for (int c = n_vec * V + lir; c < W; c += (1 << pl.lpr_log2)) drow[c] = fold_one_rolled<DT>(own, g, p, d, h, c);
+    for (int j = lir; j < n_vec; j += (1 << pl.lpr_log2)) fold_span<DT>(drow, orow, g, p, d, h, j * V, V);
+    if (lir == 0 && n_vec * V < W) fold_span<DT>(drow, orow, g, p, d, h, n_vec * V, W - n_vec * V);
     return;
   }
   // Only W neighbours reach this row. The sums over D and H then add a single term to
@@ -635,6 +656,51 @@ __global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
   for (int q = lir; q < n_edge; q += (1 << pl.lpr_log2)) {
     const int c = q < head ? q : tail0 + (q - head);
     drow[c] = element(c, orow[c]);
+  }
+}
+
+// In-place second half of a fold: gx already holds `0 + own`; only the cells that a
+// neighbour reaches change. Eight lanes per row: a row that only W neighbours reach
+// updates its first and last columns, a row that a D or H neighbour reaches is summed
+// in full.
+template <int DT>
+__global__ __launch_bounds__(256) void fold_border_kernel(Table tab, typename Arith<DT>::T* __restrict__ gx,
+                                                          Geom g, RowPlan pl) {
+  typedef typename Arith<DT>::T T;
+  constexpr int V = Bits<T>::V;
+  constexpr int LPR = 8;
+  const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+  const uint32_t row = t / LPR;
+  if (row >= pl.nrows) return;
+  const int lir = (int)(t % LPR);
+  const int D = g.n[0], H = g.n[1], W = g.n[2];
+  const uint32_t t2 = mdiv(row, pl.div_h);
+  const int h = (int)(row - t2 * (uint32_t)H);
+  const uint32_t pp = mdiv(t2, pl.div_d);
+  const int d = (int)(t2 - pp * (uint32_t)D);
+  const long long p = (long long)pp;
+  T* drow = gx + (long long)row * W;
+  const bool row_plain = (d >= g.hi[0]) && (d < D - g.lo[0]) && (h >= g.hi[1]) && (h < H - g.lo[1]);
+  if (!row_plain) {
+    const int n_vec = W / V;
+    for (int j = lir; j < n_vec; j += LPR) fold_span<DT>(drow, drow, g, p, d, h, j * V, V);
+    if (lir == 0 && n_vec * V < W) fold_span<DT>(drow, drow, g, p, d, h, n_vec * V, W - n_vec * V);
+    return;
+  }
+  const T* s_lo = static_cast<const T*>(table_entry(9 + 3 + 0));
+  const T* s_hi = static_cast<const T*>(table_entry(9 + 3 + 2));
+  if (s_lo != nullptr) s_lo += (long long)row * g.hi[2];
+  if (s_hi != nullptr) s_hi += (long long)row * g.lo[2];
+  const int up0 = W - g.lo[2];
+  const int head = g.hi[2] < up0 ? g.hi[2] : up0;  // columns [0, head) and [up0, W), each once
+  const int n_edge = head + (W - up0);
+  for (int q = lir; q < n_edge; q += LPR) {
+    const int c = q < head ? q : up0 + (q - head);
+    float acc = 0.0f;
+    if (c < g.hi[2] && s_lo != nullptr) acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(s_lo[c])));
+    acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(drow[c])));
+    if (c >= up0 && s_hi != nullptr) acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(s_hi[c - up0])));
+    drow[c] = Arith<DT>::down(acc);
   }
 }
 
@@ -911,6 +977,45 @@ extern "C" int jg_halo_fold_3d(void* gx, const void* gx_aug, const void* const s
   else JG_FOLD(JG_F16);
 #undef JG_FOLD
   JG_CHECK_LAUNCH("jg_halo_fold_3d");
+  return JG_OK;
+}
+
+extern "C" int jg_halo_fold_border_3d(void* gx, const void* const strips[27],
+                                      const jg_halo_geom* geom, int dtype, void* stream) {
+  int rc = check_geom(geom, "jg_halo_fold_border_3d", true);
+  if (rc) return rc;
+  JG_REQUIRE(gx != nullptr && strips != nullptr, "jg_halo_fold_border_3d: NULL pointer");
+  JG_REQUIRE(dtype == JG_F32 || dtype == JG_BF16 || dtype == JG_F16,
+             "jg_halo_fold_border_3d: unknown dtype %d", dtype);
+  const int es = (int)jg::dtype_size(dtype);
+  JG_REQUIRE((reinterpret_cast<uintptr_t>(gx) & (es - 1)) == 0,
+             "jg_halo_fold_border_3d: gx is not element aligned");
+  Table tab;
+  for (int i = 0; i < 27; ++i) {
+    tab.p[i] = (i == 13) ? nullptr : strips[i];
+    JG_REQUIRE((reinterpret_cast<uintptr_t>(tab.p[i]) & (es - 1)) == 0,
+               "jg_halo_fold_border_3d: slot %d is not element aligned", i);
+  }
+  Geom g = to_geom(geom);
+  const unsigned long long nrows = (unsigned long long)g.planes * g.n[0] * g.n[1];
+  if (nrows == 0 || g.n[2] == 0) return JG_OK;
+  JG_REQUIRE(nrows * 8 < (1ull << 32), "jg_halo_fold_border_3d: too many rows (%llu)", nrows);
+  RowPlan pl;
+  pl.nrows = (uint32_t)nrows;
+  pl.lpr_log2 = 3;
+  pl.nvec = 0;
+  pl.iters = 0;
+  pl.div_h = make_magic((uint32_t)g.n[1]);
+  pl.div_d = make_magic((uint32_t)g.n[0]);
+  const unsigned blocks = (unsigned)((nrows * 8 + 255) / 256);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == JG_F32)
+    fold_border_kernel<JG_F32><<<blocks, 256, 0, s>>>(tab, static_cast<uint32_t*>(gx), g, pl);
+  else if (dtype == JG_BF16)
+    fold_border_kernel<JG_BF16><<<blocks, 256, 0, s>>>(tab, static_cast<uint16_t*>(gx), g, pl);
+  else
+    fold_border_kernel<JG_F16><<<blocks, 256, 0, s>>>(tab, static_cast<uint16_t*>(gx), g, pl);
+  JG_CHECK_LAUNCH("jg_halo_fold_border_3d");
   return JG_OK;
 }
 

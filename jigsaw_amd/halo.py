@@ -294,10 +294,35 @@ def halo_fold(
     return out
 
 
+def halo_fold_border_(
+    gx: torch.Tensor,
+    strips: Mapping[Offset, torch.Tensor | None],
+    geom: HaloGeometry,
+) -> torch.Tensor:
+    """Second half of a fold whose own contributions are already in ``gx``.
+
+    ``gx`` holds ``0 + own`` in every cell (what ``conv.conv_nd_input_fold``
+    writes); the cells a neighbour reaches get the neighbours' halo blocks added in
+    place, in the order of ``halo_scatter_add`` (halo.py:207-249,
+    distributed.py:378-389), so the result has the bits of ``halo_fold``.
+    """
+    _lib.require_gpu(gx)
+    planes = _check_tile(gx, geom.size, "halo_fold_border_")
+    lead = tuple(gx.shape[: -geom.n_spatial])
+    tab = _table(strips, geom, "fold", lead, gx, None)
+    cg = geom.c_geom(planes)
+    rc = _lib.load().jg_halo_fold_border_3d(
+        _lib.ptr(gx), tab, cg, _lib.dtype_code(gx.dtype), _lib.stream_ptr(gx.device)
+    )
+    _lib.check(rc, "jg_halo_fold_border_3d")
+    return gx
+
+
 __all__ = [
     "HaloGeometry",
     "halo_assemble",
     "halo_fold",
+    "halo_fold_border_",
     "halo_pack",
     "halo_widths",
     "needed_input_span",

@@ -34,6 +34,10 @@ PRIM_CASES = [
     (1, 32, 32, (10, 10, 18), (3, 3, 3), (1, 1, 1), (0, 0, 0), (1, 1, 1)),
     (1, 64, 64, (20, 70), (3, 3), (1, 1), (1, 1), (1, 1)),
     (3, 64, 64, (37, 53), (3, 3), (1, 1), (0, 0), (1, 1)),
+    # several stages per workgroup, strips that start in the middle of a workgroup's range
+    (2, 64, 64, (260, 131), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (2, 32, 32, (6, 70, 130), (3, 3, 3), (1, 1, 1), (0, 0, 0), (1, 1, 1)),
+    (1, 32, 64, (131, 200), (3, 3), (1, 1), (1, 1), (1, 1)),
 ]
 
 
@@ -71,6 +75,10 @@ def test_conv_primitives_match_oracle(case, dtype, dev):
     assert rel_l2(gw, gw_want) < TOL[dtype], f"wgrad rel-L2 {rel_l2(gw, gw_want):.3e}"
     gb = jc.sum_grad_bias(gg, len(k))
     assert rel_l2(gb, gb_want) < TOL[dtype], f"bias grad rel-L2 {rel_l2(gb, gb_want):.3e}"
+    # both gradients from one pass over g (falls back to the two kernels where not covered)
+    gw2, gb2 = jc.conv_nd_weight(xg, w.shape, gg, stride=s, padding=p, dilation=d, with_bias_grad=True)
+    assert torch.equal(gw2, gw)
+    assert gb2.dtype == dtype and rel_l2(gb2, gb_want) < TOL[dtype], f"fused bias grad rel-L2 {rel_l2(gb2, gb_want):.3e}"
 
 
 def test_conv_argument_errors(dev):
@@ -210,3 +218,57 @@ def test_string_padding_is_rejected(dev):
     w = torch.randn(4, 3, 3, 3, device=dev)
     with pytest.raises(NotImplementedError):
         jc.conv_halo_nway(x, w, None, (1, 1), "same", (1, 1), (None, None), None, cfg)
+
+
+FUSED_CASES = [
+    # size, lo, hi, conv padding on the padded tile, N, channels, strips that exist
+    ((32, 64), (1, 1), (1, 1), (0, 0), 2, 64, "all"),
+    ((40, 72), (1, 1), (1, 1), (0, 0), 1, 64, "some"),
+    ((24, 40), (0, 2), (2, 0), (0, 0), 1, 32, "all"),
+    ((16, 96), (1, 0), (1, 0), (0, 1), 1, 64, "all"),     # W axis not split: the conv pads it itself
+    ((8, 8, 16), (1, 1, 1), (1, 1, 1), (0, 0, 0), 1, 32, "all"),
+    ((6, 10, 24), (1, 0, 1), (1, 0, 1), (0, 1, 0), 1, 32, "some"),
+]
+
+
+@pytest.mark.parametrize("case", FUSED_CASES, ids=lambda c: f"{'x'.join(map(str, c[0]))}_lo{''.join(map(str, c[1]))}_hi{''.join(map(str, c[2]))}")
+def test_fused_dgrad_fold_has_the_bits_of_the_three_steps(case, dev):
+    """conv_nd_input_fold + halo_fold_border_ == conv_nd_input + halo_pack + halo_fold, bit for bit."""
+    from jigsaw_amd.halo import HaloGeometry, halo_fold, halo_fold_border_
+
+    size, lo, hi, pad, N, ch, which = case
+    ns = len(size)
+    geom = HaloGeometry(size, lo, hi)
+    torch.manual_seed(3)
+    k = (3,) * ns
+    out_sp = tuple(geom.padded[a] + 2 * pad[a] - 2 for a in range(ns))
+    w = ((torch.rand(ch, ch, *k, device=dev) * 2 - 1) / (ch * 3**ns) ** 0.5).bfloat16()
+    g = torch.randn(N, ch, *out_sp, device=dev).bfloat16()
+    g[0, 0].zero_()          # exact zeros: the fold clears the sign of -0.0
+    g[0, 1] = -g[0, 1].abs() * 1e-30
+    offs = [o for o in geom.offsets() if all(geom.strip_extent(o, "fold")[a] > 0 for a in range(ns))]
+    if which == "some":
+        offs = offs[::2]
+    recv = {o: torch.randn(N, ch, *geom.strip_extent(o, "fold"), device=dev).bfloat16() for o in offs}
+
+    gx_aug = jc.conv_nd_input((N, ch, *geom.padded), w, g, padding=pad)
+    send_u = halo_pack(gx_aug, geom, from_padded=True)
+    gx_u = halo_fold(gx_aug, recv, geom)
+
+    fused = jc.conv_nd_input_fold(geom, w, g, padding=pad)
+    assert fused is not None, "the MFMA path should cover this case"
+    gx_f, send_f = fused
+    halo_fold_border_(gx_f, recv, geom)
+    assert torch.equal(gx_f.view(torch.int16), gx_u.view(torch.int16))
+    assert set(send_f) == set(send_u)
+    for o in send_u:
+        assert torch.equal(send_f[o].view(torch.int16), send_u[o].view(torch.int16)), f"strip {o}"
+
+
+def test_fused_dgrad_fold_declines_what_the_mfma_kernel_does_not_cover(dev):
+    from jigsaw_amd.halo import HaloGeometry
+
+    geom = HaloGeometry((8, 8), (1, 1), (1, 1))
+    w = torch.randn(4, 3, 3, 3, device=dev)
+    g = torch.randn(1, 4, 8, 8, device=dev)
+    assert jc.conv_nd_input_fold(geom, w, g, padding=(0, 0)) is None
