@@ -660,48 +660,82 @@ __global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
 }
 
 // In-place second half of a fold: gx already holds `0 + own`; only the cells that a
-// neighbour reaches change. Eight lanes per row: a row that only W neighbours reach
-// updates its first and last columns, a row that a D or H neighbour reaches is summed
-// in full.
+// neighbour reaches change. Two kernels: the rows that a D or H neighbour reaches are
+// summed in full, one wavefront per row; of the other rows only the first and last
+// columns change, one lane per cell.
+struct BorderPlan {
+  uint32_t rows_per_plane;  // rows of a plane that a D or H neighbour reaches
+  uint32_t total;           // work items of the launch
+  int nbd, nbh;             // border depths / border rows of a non-border depth
+  int n_edge, head;         // W-edge cells of a row: columns [0, head) and [W - lo, W)
+  Magic div_rows, div_h, div_nbh, div_edge, div_hh, div_d;
+};
+
+// k-th border coordinate of an axis of extent n reached over [0, hi) and [n - lo, n)
+__device__ __forceinline__ int border_coord(int k, int n, int lo, int hi) {
+  if (hi + lo >= n) return k;
+  return k < hi ? k : n - lo + (k - hi);
+}
+
 template <int DT>
-__global__ __launch_bounds__(256) void fold_border_kernel(Table tab, typename Arith<DT>::T* __restrict__ gx,
-                                                          Geom g, RowPlan pl) {
+__global__ __launch_bounds__(256) void fold_border_rows_kernel(Table tab, typename Arith<DT>::T* __restrict__ gx,
+                                                               Geom g, BorderPlan bp) {
   typedef typename Arith<DT>::T T;
   constexpr int V = Bits<T>::V;
-  constexpr int LPR = 8;
-  const uint32_t t = blockIdx.x * 256u + threadIdx.x;
-  const uint32_t row = t / LPR;
-  if (row >= pl.nrows) return;
-  const int lir = (int)(t % LPR);
+  const uint32_t item = blockIdx.x * 4u + (threadIdx.x >> 6);  // one wavefront per row
+  if (item >= bp.total) return;
+  const int lane = threadIdx.x & 63;
   const int D = g.n[0], H = g.n[1], W = g.n[2];
-  const uint32_t t2 = mdiv(row, pl.div_h);
-  const int h = (int)(row - t2 * (uint32_t)H);
-  const uint32_t pp = mdiv(t2, pl.div_d);
-  const int d = (int)(t2 - pp * (uint32_t)D);
+  const uint32_t pp = mdiv(item, bp.div_rows);
+  const uint32_t idx = item - pp * bp.rows_per_plane;
+  int d, h;
+  if (idx < (uint32_t)bp.nbd * (uint32_t)H) {
+    const uint32_t k = mdiv(idx, bp.div_h);
+    d = border_coord((int)k, D, g.lo[0], g.hi[0]);
+    h = (int)(idx - k * (uint32_t)H);
+  } else {
+    const uint32_t idx2 = idx - (uint32_t)bp.nbd * (uint32_t)H;
+    const uint32_t di = mdiv(idx2, bp.div_nbh);
+    d = g.hi[0] + (int)di;
+    h = border_coord((int)(idx2 - di * (uint32_t)bp.nbh), H, g.lo[1], g.hi[1]);
+  }
   const long long p = (long long)pp;
-  T* drow = gx + (long long)row * W;
-  const bool row_plain = (d >= g.hi[0]) && (d < D - g.lo[0]) && (h >= g.hi[1]) && (h < H - g.lo[1]);
-  if (!row_plain) {
-    const int n_vec = W / V;
-    for (int j = lir; j < n_vec; j += LPR) fold_span<DT>(drow, drow, g, p, d, h, j * V, V);
-    if (lir == 0 && n_vec * V < W) fold_span<DT>(drow, drow, g, p, d, h, n_vec * V, W - n_vec * V);
-    return;
-  }
-  const T* s_lo = static_cast<const T*>(table_entry(9 + 3 + 0));
-  const T* s_hi = static_cast<const T*>(table_entry(9 + 3 + 2));
-  if (s_lo != nullptr) s_lo += (long long)row * g.hi[2];
-  if (s_hi != nullptr) s_hi += (long long)row * g.lo[2];
+  T* drow = gx + ((p * D + d) * H + h) * (long long)W;
+  const int n_vec = W / V;
+  for (int j = lane; j < n_vec; j += 64) fold_span<DT>(drow, drow, g, p, d, h, j * V, V);
+  if (lane == 0 && n_vec * V < W) fold_span<DT>(drow, drow, g, p, d, h, n_vec * V, W - n_vec * V);
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void fold_border_cols_kernel(Table tab, typename Arith<DT>::T* __restrict__ gx,
+                                                               Geom g, BorderPlan bp) {
+  typedef typename Arith<DT>::T T;
+  const uint32_t item = blockIdx.x * 256u + threadIdx.x;  // (row, edge cell), cell fastest
+  if (item >= bp.total) return;
+  const int D = g.n[0], H = g.n[1], W = g.n[2];
+  const uint32_t row = mdiv(item, bp.div_edge);
+  const int q = (int)(item - row * (uint32_t)bp.n_edge);
+  const uint32_t t2 = mdiv(row, bp.div_hh);
+  const int h = (int)(row - t2 * (uint32_t)H);
+  const uint32_t pp = mdiv(t2, bp.div_d);
+  const int d = (int)(t2 - pp * (uint32_t)D);
+  // rows that a D or H neighbour reaches belong to the other kernel
+  if (!((d >= g.hi[0]) && (d < D - g.lo[0]) && (h >= g.hi[1]) && (h < H - g.lo[1]))) return;
   const int up0 = W - g.lo[2];
-  const int head = g.hi[2] < up0 ? g.hi[2] : up0;  // columns [0, head) and [up0, W), each once
-  const int n_edge = head + (W - up0);
-  for (int q = lir; q < n_edge; q += LPR) {
-    const int c = q < head ? q : up0 + (q - head);
-    float acc = 0.0f;
-    if (c < g.hi[2] && s_lo != nullptr) acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(s_lo[c])));
-    acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(drow[c])));
-    if (c >= up0 && s_hi != nullptr) acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(s_hi[c - up0])));
-    drow[c] = Arith<DT>::down(acc);
+  const int c = q < bp.head ? q : up0 + (q - bp.head);
+  T* cell = gx + (long long)row * W + c;
+  float acc = 0.0f;
+  if (c < g.hi[2]) {
+    const T* s_lo = static_cast<const T*>(table_entry(9 + 3 + 0));
+    if (s_lo != nullptr) acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(s_lo[(long long)row * g.hi[2] + c])));
   }
+  acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(*cell)));
+  if (c >= up0) {
+    const T* s_hi = static_cast<const T*>(table_entry(9 + 3 + 2));
+    if (s_hi != nullptr)
+      acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(s_hi[(long long)row * g.lo[2] + (c - up0)])));
+  }
+  *cell = Arith<DT>::down(acc);
 }
 
 Magic make_magic(uint32_t d) {
@@ -997,24 +1031,43 @@ extern "C" int jg_halo_fold_border_3d(void* gx, const void* const strips[27],
                "jg_halo_fold_border_3d: slot %d is not element aligned", i);
   }
   Geom g = to_geom(geom);
-  const unsigned long long nrows = (unsigned long long)g.planes * g.n[0] * g.n[1];
-  if (nrows == 0 || g.n[2] == 0) return JG_OK;
-  JG_REQUIRE(nrows * 8 < (1ull << 32), "jg_halo_fold_border_3d: too many rows (%llu)", nrows);
-  RowPlan pl;
-  pl.nrows = (uint32_t)nrows;
-  pl.lpr_log2 = 3;
-  pl.nvec = 0;
-  pl.iters = 0;
-  pl.div_h = make_magic((uint32_t)g.n[1]);
-  pl.div_d = make_magic((uint32_t)g.n[0]);
-  const unsigned blocks = (unsigned)((nrows * 8 + 255) / 256);
+  const int D = g.n[0], H = g.n[1], W = g.n[2];
+  const unsigned long long nrows = (unsigned long long)g.planes * D * H;
+  if (nrows == 0 || W == 0) return JG_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == JG_F32)
-    fold_border_kernel<JG_F32><<<blocks, 256, 0, s>>>(tab, static_cast<uint32_t*>(gx), g, pl);
-  else if (dtype == JG_BF16)
-    fold_border_kernel<JG_BF16><<<blocks, 256, 0, s>>>(tab, static_cast<uint16_t*>(gx), g, pl);
-  else
-    fold_border_kernel<JG_F16><<<blocks, 256, 0, s>>>(tab, static_cast<uint16_t*>(gx), g, pl);
+  BorderPlan bp;
+  bp.nbd = (g.hi[0] + g.lo[0] >= D) ? D : g.hi[0] + g.lo[0];
+  bp.nbh = (g.hi[1] + g.lo[1] >= H) ? H : g.hi[1] + g.lo[1];
+  bp.rows_per_plane = (uint32_t)bp.nbd * (uint32_t)H + (uint32_t)(D - bp.nbd) * (uint32_t)bp.nbh;
+  const int up0 = W - g.lo[2];
+  bp.head = g.hi[2] < up0 ? g.hi[2] : up0;
+  bp.n_edge = bp.head + (W - up0);
+  bp.div_rows = make_magic(bp.rows_per_plane);
+  bp.div_h = make_magic((uint32_t)H);
+  bp.div_nbh = make_magic((uint32_t)(bp.nbh > 0 ? bp.nbh : 1));
+  bp.div_edge = make_magic((uint32_t)(bp.n_edge > 0 ? bp.n_edge : 1));
+  bp.div_hh = make_magic((uint32_t)H);
+  bp.div_d = make_magic((uint32_t)D);
+  const unsigned long long row_items = (unsigned long long)g.planes * bp.rows_per_plane;
+  const unsigned long long col_items = nrows * (unsigned long long)bp.n_edge;
+  JG_REQUIRE(row_items < (1ull << 31) && col_items < (1ull << 31) && nrows < (1ull << 31),
+             "jg_halo_fold_border_3d: too many rows (%llu)", nrows);
+#define JG_BORDER(DT)                                                                                   \
+  do {                                                                                                  \
+    typedef Arith<DT>::T T;                                                                             \
+    if (row_items > 0) {                                                                                \
+      bp.total = (uint32_t)row_items;                                                                   \
+      fold_border_rows_kernel<DT><<<(unsigned)((row_items + 3) / 4), 256, 0, s>>>(tab, static_cast<T*>(gx), g, bp); \
+    }                                                                                                   \
+    if (col_items > 0) {                                                                                \
+      bp.total = (uint32_t)col_items;                                                                   \
+      fold_border_cols_kernel<DT><<<(unsigned)((col_items + 255) / 256), 256, 0, s>>>(tab, static_cast<T*>(gx), g, bp); \
+    }                                                                                                   \
+  } while (0)
+  if (dtype == JG_F32) JG_BORDER(JG_F32);
+  else if (dtype == JG_BF16) JG_BORDER(JG_BF16);
+  else JG_BORDER(JG_F16);
+#undef JG_BORDER
   JG_CHECK_LAUNCH("jg_halo_fold_border_3d");
   return JG_OK;
 }
