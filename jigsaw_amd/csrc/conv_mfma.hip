@@ -27,6 +27,8 @@
 //               barrier per stage).
 //   dgrad       the same kernel on the output gradient with virtual zero padding
 //               k-1-p and the weights flipped and transposed by the preparation.
+#include <type_traits>
+
 #include "conv_common.h"
 
 namespace {
@@ -128,7 +130,7 @@ __global__ __launch_bounds__(256) void prep_weights_kernel(uint16_t* __restrict_
 // EVEN: Win, pad_w and the plane size are even and x is 4-byte aligned, so every
 // pixel pair of a task is one aligned dword that is either wholly inside or wholly
 // outside the tensor. Otherwise the prefetch falls back to 2-byte loads.
-template <int MT, bool EVEN>  // MT = produced channels per workgroup: 32 or 64
+template <int MT, bool EVEN, bool FOLD>  // MT = produced channels per workgroup: 32 or 64
 __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips, FwdParams p) {
   constexpr int CB = MT / 32;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -351,19 +353,44 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
   // zero is cleared, as the reference's scatter-add does for every cell.
   auto epilogue_fold = [&](int tile) {
     const TileCoord tc = coord(tile);
+    // bf16 pairs of the whole accumulator first (the fp32 registers are dead after this).
+    // The sign of a zero only matters where a value is zero or rounds to zero, which is
+    // rare: one min3 per two values finds out, and only then the bits are patched.
+    uint32_t pk[CB][WROWS][8];
+    float small = 3.0e38f;
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+      for (int r = 0; r < WROWS; ++r)
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          small = __builtin_fminf(small, __builtin_fminf(__builtin_fabsf(acc[cb][r][i]), __builtin_fabsf(acc[cb][r][i + 1])));
+          f32x2 v2 = {acc[cb][r][i], acc[cb][r][i + 1]};
+          pk[cb][r][i >> 1] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
+        }
+    if (__builtin_amdgcn_ballot_w64(!(small >= 1.0e-39f)) != 0) {  // bf16 rounds |v| <= 2^-134 to zero
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int r = 0; r < WROWS; ++r)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            uint32_t bits = pk[cb][r][j];
+            if ((bits & 0x00007fffu) == 0) bits &= 0xffff0000u;
+            if ((bits & 0x7fff0000u) == 0) bits &= 0x0000ffffu;
+            pk[cb][r][j] = bits;
+          }
+    }
     const int ow = tc.tw * TW + wcol0 + ln;
     const int hi_d = p.Dout - p.lo_d - p.nD, hi_h = p.Hout - p.lo_h - p.nH, hi_w = p.Wout - p.lo_w - p.nW;
     const int od = tc.od;
     const int rd = od < p.lo_d ? 0 : (od < p.lo_d + p.nD ? 1 : 2);
     const int cd = od - (rd == 0 ? 0 : (rd == 1 ? p.lo_d : p.lo_d + p.nD));
     const int ed = rd == 0 ? p.lo_d : (rd == 1 ? p.nD : hi_d);
-    const int rw = ow < p.lo_w ? 0 : (ow < p.lo_w + p.nW ? 1 : 2);
-    const int cw = ow - (rw == 0 ? 0 : (rw == 1 ? p.lo_w : p.lo_w + p.nW));
-    const int ew = rw == 0 ? p.lo_w : (rw == 1 ? p.nW : hi_w);
     const size_t plane0 = (size_t)tc.n * p.M + (size_t)mt * MT;
+    const int th0 = tc.th * TH, tw0 = tc.tw * TW;
     // A tile that lies wholly inside the own extent (wave-uniform test): plain rows of
     // the unpadded tile, no per-cell routing.
-    const int th0 = tc.th * TH, tw0 = tc.tw * TW;
     if (rd == 1 && th0 >= p.lo_h && th0 + TH <= p.lo_h + p.nH && tw0 >= p.lo_w && tw0 + TW <= p.lo_w + p.nW) {
       const size_t ps = (size_t)p.nD * p.nH * p.nW;
       char* ybase = reinterpret_cast<char*>(p.y) + 2 * (plane0 * ps + (size_t)cd * p.nH * p.nW);
@@ -374,22 +401,24 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-          for (int i = 0; i < 16; i += 2) {
-            f32x2 v2 = {acc[cb][r][i] + 0.0f, acc[cb][r][i + 1] + 0.0f};
-            const bf16x2 h2 = __builtin_convertvector(v2, bf16x2);
-            uint32_t bits = __builtin_bit_cast(uint32_t, h2);
-            if ((bits & 0x00007fffu) == 0) bits &= 0xffff0000u;
-            if ((bits & 0x7fff0000u) == 0) bits &= 0x0000ffffu;
-            const int m0 = cb * 32 + 8 * (i >> 2) + (i & 3);
+          for (int j = 0; j < 8; ++j) {
+            const int m0 = cb * 32 + 8 * (j >> 1) + 2 * (j & 1);
+            const uint32_t bits = pk[cb][r][j];
             *reinterpret_cast<uint16_t*>(ybase + (size_t)m0 * ps * 2 + voff) = (uint16_t)(bits & 0xffffu);
             *reinterpret_cast<uint16_t*>(ybase + (size_t)(m0 + 1) * ps * 2 + voff) = (uint16_t)(bits >> 16);
           }
       }
       return;
     }
+    // Otherwise a cell goes to the unpadded tile when it lies inside [lo, lo + n) on every
+    // axis, else to the strip of the neighbour that owns it (dropped when that neighbour
+    // does not exist).
+    const int rw = ow < p.lo_w ? 0 : (ow < p.lo_w + p.nW ? 1 : 2);
+    const int cw = ow - (rw == 0 ? 0 : (rw == 1 ? p.lo_w : p.lo_w + p.nW));
+    const int ew = rw == 0 ? p.lo_w : (rw == 1 ? p.nW : hi_w);
 #pragma unroll
     for (int r = 0; r < WROWS; ++r) {
-      const int oh = tc.th * TH + wrow0 + r;
+      const int oh = th0 + wrow0 + r;
       if (oh >= p.Hout || ow >= p.Wout) continue;
       const int rh = oh < p.lo_h ? 0 : (oh < p.lo_h + p.nH ? 1 : 2);
       const int ch = oh - (rh == 0 ? 0 : (rh == 1 ? p.lo_h : p.lo_h + p.nH));
@@ -397,20 +426,17 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
       const int slot = rd * 9 + rh * 3 + rw;
       char* base = slot == 13 ? reinterpret_cast<char*>(p.y) : static_cast<char*>(strip_entry(slot));
       if (base == nullptr) continue;
-      const size_t ps = (size_t)ed * eh * ew;  // elements per plane of that destination
-      char* dst = base + 2 * ((plane0 + 4 * kg) * ps + ((size_t)cd * eh + ch) * ew + cw);
+      const uint32_t ps = (uint32_t)ed * (uint32_t)eh * (uint32_t)ew;  // elements per plane of that destination
+      char* dst = base + 2 * ((plane0 + 4 * kg) * (size_t)ps + ((size_t)cd * eh + ch) * ew + cw);
+      const uint32_t step = 2u * ps;  // bytes between produced channels (checked on the host to fit)
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-        for (int i = 0; i < 16; i += 2) {
-          f32x2 v2 = {acc[cb][r][i] + 0.0f, acc[cb][r][i + 1] + 0.0f};
-          const bf16x2 h2 = __builtin_convertvector(v2, bf16x2);
-          uint32_t bits = __builtin_bit_cast(uint32_t, h2);
-          if ((bits & 0x00007fffu) == 0) bits &= 0xffff0000u;
-          if ((bits & 0x7fff0000u) == 0) bits &= 0x0000ffffu;
-          const int m0 = cb * 32 + 8 * (i >> 2) + (i & 3);
-          *reinterpret_cast<uint16_t*>(dst + (size_t)m0 * ps * 2) = (uint16_t)(bits & 0xffffu);
-          *reinterpret_cast<uint16_t*>(dst + (size_t)(m0 + 1) * ps * 2) = (uint16_t)(bits >> 16);
+        for (int j = 0; j < 8; ++j) {
+          const uint32_t m0 = (uint32_t)(cb * 32 + 8 * (j >> 1) + 2 * (j & 1));
+          const uint32_t bits = pk[cb][r][j];
+          *reinterpret_cast<uint16_t*>(dst + m0 * step) = (uint16_t)(bits & 0xffffu);
+          *reinterpret_cast<uint16_t*>(dst + (m0 + 1) * step) = (uint16_t)(bits >> 16);
         }
     }
   };
@@ -440,7 +466,7 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
       __syncthreads();
       buf ^= 1;
     }
-    if (p.fold) epilogue_fold(tile_of(ti));
+    if (FOLD) epilogue_fold(tile_of(ti));
     else epilogue(tile_of(ti));
   }
 }
@@ -531,8 +557,13 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   const bool even = (L.Win % 2 == 0) && (L.pad_w % 2 == 0) &&
                     ((reinterpret_cast<uintptr_t>(L.x) & 3) == 0);
   void (*kern)(StripTable, FwdParams) = nullptr;
-  if (MT == 64) kern = even ? &conv3x3_mfma_kernel<64, true> : &conv3x3_mfma_kernel<64, false>;
-  else kern = even ? &conv3x3_mfma_kernel<32, true> : &conv3x3_mfma_kernel<32, false>;
+  if (L.fold) {
+    if (MT == 64) kern = even ? &conv3x3_mfma_kernel<64, true, true> : &conv3x3_mfma_kernel<64, false, true>;
+    else kern = even ? &conv3x3_mfma_kernel<32, true, true> : &conv3x3_mfma_kernel<32, false, true>;
+  } else {
+    if (MT == 64) kern = even ? &conv3x3_mfma_kernel<64, true, false> : &conv3x3_mfma_kernel<64, false, false>;
+    else kern = even ? &conv3x3_mfma_kernel<32, true, false> : &conv3x3_mfma_kernel<32, false, false>;
+  }
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", who, lds);

@@ -172,7 +172,8 @@ struct PackArgs {
   Box box[27];
 };
 
-template <typename T>
+// I: index type (32-bit when the source tensor has fewer than 2^31 elements)
+template <typename T, typename I>
 __global__ __launch_bounds__(256) void pack_kernel(PackArgs a, const T* __restrict__ src,
                                                    long long planes, int Sd, int Sh,
                                                    int Sw) {
@@ -180,18 +181,16 @@ __global__ __launch_bounds__(256) void pack_kernel(PackArgs a, const T* __restri
   T* d = static_cast<T*>(a.dst[slot]);
   if (d == nullptr) return;
   const Box b = a.box[slot];
-  const long long per_plane = (long long)b.ext[0] * b.ext[1] * b.ext[2];
-  const long long total = planes * per_plane;
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total;
-       i += (long long)gridDim.x * 256) {
-    long long r = i / b.ext[2];
-    int cw = (int)(i - r * b.ext[2]);
-    long long r2 = r / b.ext[1];
-    int ch = (int)(r - r2 * b.ext[1]);
-    long long p = r2 / b.ext[0];
-    int cd = (int)(r2 - p * b.ext[0]);
-    long long so = ((p * Sd + (b.org[0] + cd)) * Sh + (b.org[1] + ch)) * (long long)Sw +
-                   (b.org[2] + cw);
+  const I e0 = (I)b.ext[0], e1 = (I)b.ext[1], e2 = (I)b.ext[2];
+  const I total = (I)planes * e0 * e1 * e2;
+  for (I i = (I)blockIdx.x * 256 + threadIdx.x; i < total; i += (I)gridDim.x * 256) {
+    const I r = i / e2;
+    const I cw = i - r * e2;
+    const I r2 = r / e1;
+    const I ch = r - r2 * e1;
+    const I p = r2 / e0;
+    const I cd = r2 - p * e0;
+    const I so = ((p * (I)Sd + ((I)b.org[0] + cd)) * (I)Sh + ((I)b.org[1] + ch)) * (I)Sw + ((I)b.org[2] + cw);
     d[i] = src[so];
   }
 }
@@ -934,12 +933,20 @@ extern "C" int jg_halo_pack_3d(void* const strips[27], const void* src,
   if (bx > 4096) bx = 4096;
   dim3 grid((unsigned)bx, 27, 1);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (elem_size == 2)
-    pack_kernel<uint16_t><<<grid, 256, 0, s>>>(a, static_cast<const uint16_t*>(src), g.planes,
-                                               Sd, Sh, Sw);
-  else
-    pack_kernel<uint32_t><<<grid, 256, 0, s>>>(a, static_cast<const uint32_t*>(src), g.planes,
-                                               Sd, Sh, Sw);
+  const bool narrow = (unsigned long long)g.planes * Sd * Sh * Sw < (1ull << 31);
+  if (elem_size == 2) {
+    if (narrow)
+      pack_kernel<uint16_t, uint32_t><<<grid, 256, 0, s>>>(a, static_cast<const uint16_t*>(src), g.planes, Sd, Sh, Sw);
+    else
+      pack_kernel<uint16_t, unsigned long long><<<grid, 256, 0, s>>>(a, static_cast<const uint16_t*>(src), g.planes, Sd,
+                                                                     Sh, Sw);
+  } else {
+    if (narrow)
+      pack_kernel<uint32_t, uint32_t><<<grid, 256, 0, s>>>(a, static_cast<const uint32_t*>(src), g.planes, Sd, Sh, Sw);
+    else
+      pack_kernel<uint32_t, unsigned long long><<<grid, 256, 0, s>>>(a, static_cast<const uint32_t*>(src), g.planes, Sd,
+                                                                     Sh, Sw);
+  }
   JG_CHECK_LAUNCH("jg_halo_pack_3d");
   return JG_OK;
 }
