@@ -87,14 +87,20 @@ def build_conv2_workload(dev, batch=8, ch=64, tile=1024):
         o: torch.randn(*lead, *geom.strip_extent(o, "fold"), device=dev, generator=g).bfloat16()
         for o in geom.offsets()
     }
-    return {"geom": geom, "x": x, "w": w, "b": b, "g": gout, "strips_fwd": strips_fwd, "strips_bwd": strips_bwd}
+    from jigsaw_amd import conv as jc
+
+    bands = jc.frame_bands(x, geom, w.shape)
+    if bands is None:
+        raise RuntimeError("the framed kernels should cover configuration 2")
+    return {"geom": geom, "x": x, "w": w, "b": b, "g": gout, "strips_fwd": strips_fwd, "strips_bwd": strips_bwd,
+            "bands": bands}
 
 
 def conv_step(wl):
     """The hot path of one rank for one batch (see the module docstring). The backward
-    uses the fused form: dgrad writes the owned cells and the strips it sends in one
-    pass, and the received strips are added to the border afterwards (same bits as
-    dgrad + pack + fold on the padded gradient)."""
+    uses the fused forms, each with the bits of the separate steps it replaces: dgrad
+    writes the owned cells and the strips it sends in one pass, wgrad adds up the bias
+    gradient on the way, and the received strips are added to the border afterwards."""
     from jigsaw_amd import conv as jc
     from jigsaw_amd.halo import halo_assemble, halo_fold_border_, halo_pack
 
@@ -317,6 +323,12 @@ def main() -> int:
     from jigsaw_amd.halo import halo_fold_border_
 
     ms_border = time_gpu(lambda: halo_fold_border_(gx_buf, wl["strips_bwd"], geom), it)
+    x_frame = halo_assemble(wl["x"], wl["strips_fwd"], geom, bands=wl["bands"])
+    ms_frame = time_gpu(lambda: halo_assemble(wl["x"], wl["strips_fwd"], geom, out=x_frame, bands=wl["bands"]), it)
+    ms_fwd_framed = time_gpu(lambda: jc.conv_nd_framed(x_frame, wl["x"], geom, wl["w"], wl["b"]), it)
+    ms_wgrad_framed = time_gpu(
+        lambda: jc.conv_nd_weight_framed(x_frame, wl["x"], geom, wl["w"].shape, wl["g"], with_bias_grad=True), it
+    )
     es = wl["x"].element_size()
     strip_bytes = sum(t.numel() for t in wl["strips_fwd"].values()) * es
     halo_bytes = (wl["x"].numel() + x_aug.numel()) * es + strip_bytes  # read tile + strips, write padded tile
@@ -345,6 +357,9 @@ def main() -> int:
         "halo_fold": {"ms": ms_fold, "GBps": gbps(ms_fold), "frac_hbm_peak": gbps(ms_fold) / PEAK_HBM_GBPS, "bytes": halo_bytes},
         "conv_dgrad_fused_with_pack_and_fold": {"ms": ms_dgrad_fold, "tflops": tf(ms_dgrad_fold)},
         "halo_fold_border": {"ms": ms_border},
+        "halo_assemble_frame": {"ms": ms_frame},
+        "conv_fwd_framed": {"ms": ms_fwd_framed, "tflops": tf(ms_fwd_framed)},
+        "conv_wgrad_framed_with_bias_grad": {"ms": ms_wgrad_framed, "tflops": tf(ms_wgrad_framed)},
     }
     extra.update(attention_figures(dev, max(10, it)))
     extra.update(conv3d_figures(dev, it))

@@ -88,6 +88,16 @@ int jg_halo_assemble_2d(void* x_aug, const void* const src[9], int64_t planes,
                         int H, int W, int lo_h, int hi_h, int lo_w, int hi_w,
                         int elem_size, void* stream);
 
+/* jg_halo_assemble_3d restricted to a frame: only the cells whose padded
+ * coordinate on some axis lies in the first band_lo[axis] or the last
+ * band_hi[axis] positions are written, the rest of x_aug is left untouched. For
+ * the framed convolution entry points, which read the tile itself wherever their
+ * window stays inside it and x_aug only near the edges (bands from
+ * jg_conv_frame_bands). */
+int jg_halo_assemble_frame_3d(void* x_aug, const void* const src[27],
+                              const jg_halo_geom* geom, const int32_t band_lo[3],
+                              const int32_t band_hi[3], int elem_size, void* stream);
+
 /* Cut the strips this rank sends. from_padded = 0: `src` is the own tile
  * (planes, D, H, W) and strip (dd,dh,dw) is the edge block that neighbour needs
  * for its halo (forward; the x.narrow(axis, col, sn) sends of halo.py:134-147).
@@ -242,6 +252,24 @@ int jg_conv_fwd(void* y, const void* x, const void* w, const void* bias,
  * called at jigsaw/modules/convolution/_conv/distributed.py:346-355. */
 int jg_conv_dgrad(void* gx, const void* w, const void* g, const jg_conv_desc* desc,
                   int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Framed input. The halo-padded tile is mostly a shifted copy of the own tile, so the
+ * framed entry points read the own tile x_tile (N, Cin, *geom->size) wherever a
+ * kernel's window lies inside it, and the padded tensor x_frame (N, Cin, *desc->in_size,
+ * geom->size + lo + hi = desc->in_size, planes = batch * c_in) only near the edges.
+ * x_frame therefore only needs the frame that jg_halo_assemble_frame_3d writes with
+ * the bands of jg_conv_frame_bands; results are bit-identical to jg_conv_fwd /
+ * jg_conv_wgrad(_bias) on the fully assembled x_aug (the reference's halo_gather +
+ * F.conv path, distributed.py:264-293, and conv*_weight, :359-368). gb may be NULL.
+ * All three return JG_ERR_UNSUPPORTED where only the unframed kernels exist. */
+int jg_conv_frame_bands(const jg_conv_desc* desc, const jg_halo_geom* geom, int dtype,
+                        int32_t band_lo[3], int32_t band_hi[3]);
+int jg_conv_fwd_framed(void* y, const void* x_frame, const void* x_tile, const void* w,
+                       const void* bias, const jg_conv_desc* desc, const jg_halo_geom* geom,
+                       int dtype, void* workspace, size_t workspace_bytes, void* stream);
+int jg_conv_wgrad_framed(void* gw, void* gb, const void* x_frame, const void* x_tile,
+                         const void* g, const jg_conv_desc* desc, const jg_halo_geom* geom,
+                         int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* jg_conv_dgrad with the first half of the fold fused into its epilogue
  * (distributed.py:346-355 followed by the sends of halo.py:222-226): `desc`

@@ -66,6 +66,10 @@ SIGNATURES: dict[str, tuple] = {
     "jg_last_error": (c_char_p, []),
     "jg_abi_version": (c_int, []),
     "jg_halo_assemble_3d": (c_int, [c_void_p, POINTER(c_void_p), POINTER(HaloGeom), c_int, c_void_p]),
+    "jg_halo_assemble_frame_3d": (
+        c_int,
+        [c_void_p, POINTER(c_void_p), POINTER(HaloGeom), POINTER(c_int32), POINTER(c_int32), c_int, c_void_p],
+    ),
     "jg_halo_assemble_2d": (
         c_int,
         [c_void_p, POINTER(c_void_p), c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
@@ -113,6 +117,17 @@ SIGNATURES: dict[str, tuple] = {
          c_void_p],
     ),
     "jg_conv_wgrad": (c_int, [c_void_p, c_void_p, c_void_p, POINTER(ConvDesc), c_int, c_void_p, c_size_t, c_void_p]),
+    "jg_conv_frame_bands": (c_int, [POINTER(ConvDesc), POINTER(HaloGeom), c_int, POINTER(c_int32), POINTER(c_int32)]),
+    "jg_conv_fwd_framed": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(ConvDesc), POINTER(HaloGeom), c_int, c_void_p,
+         c_size_t, c_void_p],
+    ),
+    "jg_conv_wgrad_framed": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(ConvDesc), POINTER(HaloGeom), c_int, c_void_p,
+         c_size_t, c_void_p],
+    ),
     "jg_conv_wgrad_bias": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, POINTER(ConvDesc), c_int, c_void_p, c_size_t, c_void_p],

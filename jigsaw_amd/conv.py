@@ -18,6 +18,7 @@ that talks to other ranks), and assembles the padded tile in one pass.
 
 from __future__ import annotations
 
+import ctypes
 from collections.abc import Sequence
 from typing import Any, Protocol
 
@@ -140,6 +141,86 @@ def conv_nd_input(input_shape, w, g, *, stride=1, padding=0, dilation=1, groups=
     )
     _lib.check(rc, "jg_conv_dgrad")
     return gx
+
+
+def _framed_desc(x_tile, geom: HaloGeometry, w, stride, padding, dilation, groups):
+    n = geom.n_spatial
+    stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
+    if tuple(x_tile.shape[2:]) != tuple(geom.size):
+        raise ValueError(f"own tile {tuple(x_tile.shape[2:])} does not match the geometry {geom.size}")
+    desc = _desc(x_tile.shape[0], x_tile.shape[1], w.shape[0] if hasattr(w, "shape") else w[0], geom.padded,
+                 (w.shape if hasattr(w, "shape") else w)[2:], stride, padding, dilation, groups)
+    return desc, stride, padding, dilation
+
+
+def frame_bands(x_tile, geom: HaloGeometry, weight_shape, *, stride=1, padding=0, dilation=1, groups=1):
+    """``(band_lo, band_hi)`` per spatial axis: the frame of the padded tile that the framed
+    convolution kernels read (everything else comes from the own tile), or ``None`` where
+    only the unframed kernels cover the problem."""
+    _lib.require_gpu(x_tile)
+    weight_shape = tuple(int(v) for v in weight_shape)
+    desc, *_ = _framed_desc(x_tile, geom, weight_shape, stride, padding, dilation, groups)
+    lo, hi = (ctypes.c_int32 * 3)(), (ctypes.c_int32 * 3)()
+    cg = geom.c_geom(int(x_tile.shape[0]) * int(x_tile.shape[1]))
+    rc = _lib.load().jg_conv_frame_bands(desc, cg, _lib.dtype_code(x_tile.dtype), lo, hi)
+    if rc == -2:
+        return None
+    _lib.check(rc, "jg_conv_frame_bands")
+    pad = 3 - geom.n_spatial
+    return tuple(lo[pad:]), tuple(hi[pad:])
+
+
+def conv_nd_framed(x_frame, x_tile, geom: HaloGeometry, w, b=None, *, stride=1, padding=0, dilation=1, groups=1):
+    """``conv_nd`` on the padded tile of which only the frame (``frame_bands``) holds data:
+    windows inside the own tile are read from ``x_tile``. Same bits as ``conv_nd`` on the
+    fully assembled tile. Returns ``None`` where only the unframed kernel exists."""
+    _lib.require_gpu(x_frame, x_tile, w)
+    n = _check_args(x_frame, w, groups, padding)
+    x_tile, w = x_tile.contiguous(), w.contiguous()
+    desc, stride, padding, dilation = _framed_desc(x_tile, geom, w, stride, padding, dilation, groups)
+    if tuple(x_frame.shape) != (x_tile.shape[0], x_tile.shape[1], *geom.padded) or not x_frame.is_contiguous():
+        raise ValueError("conv_nd_framed: x_frame must be the contiguous padded tensor of the geometry")
+    if b is not None:
+        b = b.contiguous()
+    out_sp = _out_spatial(geom.padded, w.shape[2:], stride, padding, dilation)
+    y = torch.empty((x_tile.shape[0], w.shape[0], *out_sp), dtype=x_tile.dtype, device=x_tile.device)
+    ws, nbytes = _workspace(desc, 0, x_tile.dtype, x_tile.device)
+    rc = _lib.load().jg_conv_fwd_framed(
+        _lib.ptr(y), _lib.ptr(x_frame), _lib.ptr(x_tile), _lib.ptr(w), _lib.ptr(b), desc,
+        geom.c_geom(int(x_tile.shape[0]) * int(x_tile.shape[1])), _lib.dtype_code(x_tile.dtype), _lib.ptr(ws), nbytes,
+        _lib.stream_ptr(x_tile.device),
+    )
+    if rc == -2:
+        return None
+    _lib.check(rc, "jg_conv_fwd_framed")
+    return y
+
+
+def conv_nd_weight_framed(x_frame, x_tile, geom: HaloGeometry, weight_shape, g, *, stride=1, padding=0, dilation=1,
+                          groups=1, with_bias_grad=False):
+    """``conv_nd_weight`` (optionally with the bias gradient) on a framed input, see
+    ``conv_nd_framed``. Returns ``None`` where only the unframed kernel exists."""
+    _lib.require_gpu(x_frame, x_tile, g)
+    weight_shape = tuple(int(v) for v in weight_shape)
+    if x_tile.dtype != g.dtype:
+        raise RuntimeError(f"input type ({x_tile.dtype}) and grad_output type ({g.dtype}) should be the same")
+    x_tile, g = x_tile.contiguous(), g.contiguous()
+    desc, stride, padding, dilation = _framed_desc(x_tile, geom, weight_shape, stride, padding, dilation, groups)
+    out_sp = _out_spatial(geom.padded, weight_shape[2:], stride, padding, dilation)
+    if tuple(g.shape) != (x_tile.shape[0], weight_shape[0], *out_sp) or x_tile.shape[1] != weight_shape[1]:
+        raise ValueError(f"grad_output {tuple(g.shape)} / tile {tuple(x_tile.shape)} do not match weight {weight_shape}")
+    gw = torch.empty(weight_shape, dtype=g.dtype, device=g.device)
+    gb = torch.empty(weight_shape[0], dtype=g.dtype, device=g.device) if with_bias_grad else None
+    ws, nbytes = _workspace(desc, 2, g.dtype, g.device)
+    rc = _lib.load().jg_conv_wgrad_framed(
+        _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(x_frame), _lib.ptr(x_tile), _lib.ptr(g), desc,
+        geom.c_geom(int(x_tile.shape[0]) * int(x_tile.shape[1])), _lib.dtype_code(g.dtype), _lib.ptr(ws), nbytes,
+        _lib.stream_ptr(g.device),
+    )
+    if rc == -2:
+        return None
+    _lib.check(rc, "jg_conv_wgrad_framed")
+    return (gw, gb) if with_bias_grad else gw
 
 
 def conv_nd_input_fold(geom: HaloGeometry, w, g, *, stride=1, padding=0, dilation=1, groups=1, present=None):
@@ -316,6 +397,15 @@ def _needs_halo(sizes, padding, dilation) -> bool:
     return any(s > 1 and (p != 0 or d != 1) for s, p, d in zip(sizes, padding, dilation))
 
 
+def _frame_decision(config, x, geom: HaloGeometry, weight_shape, kwargs):
+    """Bands of the frame when the framed kernels are asked for and cover the problem, else ``None``."""
+    if not getattr(config, "framed", False) or config.conv_fn is not conv_nd or config.conv_weight_fn is not conv_nd_weight:
+        return None
+    if x.dtype != torch.bfloat16:
+        return None
+    return frame_bands(x, geom, weight_shape, **kwargs)
+
+
 def conv_halo_nway(x, w, b, stride, padding, dilation, spatial_groups, channel_group, config):
     """Convolve with a halo exchange on every split axis; returns ``(y, x_aug)``.
 
@@ -337,15 +427,25 @@ def conv_halo_nway(x, w, b, stride, padding, dilation, spatial_groups, channel_g
     present = _present_offsets(geom, ranks, sizes)
     send = halo_pack(x, geom, from_padded=False, present=present) if present else {}
     recv = config.halo_exchange.forward(send) if present else {}
-    x_aug = halo_assemble(x, recv, geom)
     kwargs = {"stride": stride, "padding": _local_padding(padding, sizes), "dilation": dilation, "groups": 1}
+    bands = _frame_decision(config, x, geom, w.shape, kwargs)
+    if bands is not None:
+        # only the frame of the padded tile is built; the kernels read the tile itself elsewhere.
+        # The padded tensor that is returned is then NOT a full copy: its consumer is
+        # conv_halo_nway_backward with x_tile given (what _ConvNd of this module does).
+        x_frame = halo_assemble(x, recv, geom, bands=bands)
+        y = conv_nd_framed(x_frame, x, geom, w, b, **kwargs)
+        if y is None:
+            raise RuntimeError("framed forward: " + _lib.load().jg_last_error().decode())
+        return y, x_frame
+    x_aug = halo_assemble(x, recv, geom)
     y = config.conv_fn(x_aug, w, b, **kwargs) if b is not None else config.conv_fn(x_aug, w, **kwargs)
     return y, x_aug
 
 
 def conv_halo_nway_backward(
     grad_output, x_aug, weight, stride, padding, dilation, local_in_spatial, spatial_groups, channel_group, config,
-    need=(True, True),
+    need=(True, True), x_tile=None,
 ):
     """Gradients of the halo-exchange convolution; returns ``(g_x or None, g_w or None)``.
 
@@ -363,7 +463,20 @@ def conv_halo_nway_backward(
     g = grad_output.to(weight.dtype)
     kwargs = {"stride": stride, "padding": local_padding, "dilation": dilation, "groups": 1}
     g_w = g_b = None
-    if need_w and need_b and config.conv_weight_fn is conv_nd_weight:
+    if x_tile is not None:
+        # x_aug is the frame that the framed forward built (conv_halo_nway with config.framed)
+        if need_w:
+            geom_w = HaloGeometry.for_conv(local_in_spatial, weight.shape[-n:], stride, padding, dilation, ranks, sizes)
+            res = conv_nd_weight_framed(x_aug, x_tile, geom_w, weight.shape, g, with_bias_grad=need_b, **kwargs)
+            if res is None:
+                raise RuntimeError(
+                    "the framed forward was used but the framed weight gradient does not cover this case: "
+                    + _lib.load().jg_last_error().decode()
+                )
+            g_w, g_b = res if need_b else (res, None)
+        elif need_b:
+            g_b = config.grad_bias(g.contiguous())
+    elif need_w and need_b and config.conv_weight_fn is conv_nd_weight:
         g_w, g_b = conv_nd_weight(x_aug, weight.shape, g, with_bias_grad=True, **kwargs)
     else:
         g_w = config.conv_weight_fn(x_aug, weight.shape, g, **kwargs) if need_w else None
@@ -404,8 +517,10 @@ class HipConvNdConfig:
     groups = 1
     groups_local = 1
 
-    def __init__(self, n_spatial: int, bias: Any, halo_exchange: HaloExchange | None = None) -> None:
+    def __init__(self, n_spatial: int, bias: Any, halo_exchange: HaloExchange | None = None, framed: bool = False) -> None:
         self.n_spatial = int(n_spatial)
+        # framed: build only the frame of the padded tile (needs _ConvNd of this module, which keeps the tile)
+        self.framed = bool(framed)
         self.halo_exchange = halo_exchange
         self.conv_fn = conv_nd
         self.native_conv_fn = conv_nd
@@ -448,7 +563,19 @@ class _ConvNd(torch.autograd.Function):
         x, weight, bias, stride, padding, dilation, spatial_groups, channel_group, config = inputs
         _, x_aug = output
         ctx.mark_non_differentiable(x_aug)
-        ctx.save_for_backward(x_aug, weight)
+        # the same decision conv_halo_nway took: x_aug is a frame only, so the tile is kept
+        ctx.framed = False
+        if getattr(config, "framed", False) and isinstance(padding, tuple):
+            n = config.n_spatial
+            ranks, sizes = _mesh_position(spatial_groups)
+            geom = HaloGeometry.for_conv(x.shape[-n:], weight.shape[-n:], stride, padding, dilation, ranks, sizes)
+            kwargs = {"stride": stride, "padding": _local_padding(padding, sizes), "dilation": dilation, "groups": 1}
+            x_c = x if x.dtype == x_aug.dtype else torch.empty(0, dtype=x_aug.dtype, device=x.device).new_empty(x.shape)
+            ctx.framed = _frame_decision(config, x_c, geom, weight.shape, kwargs) is not None
+        if ctx.framed:
+            ctx.save_for_backward(x_aug, weight, x)  # x_aug may be a frame only: keep the tile
+        else:
+            ctx.save_for_backward(x_aug, weight)
         ctx.spatial_groups, ctx.channel_group = spatial_groups, channel_group
         ctx.local_in_spatial = tuple(x.shape[-config.n_spatial :])
         ctx.stride, ctx.padding, ctx.dilation, ctx.config = stride, padding, dilation, config
@@ -456,7 +583,11 @@ class _ConvNd(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output, grad_x_aug):  # noqa: D102
-        x_aug, weight = ctx.saved_tensors
+        if ctx.framed:
+            x_aug, weight, x_tile = ctx.saved_tensors
+            x_tile = x_tile.to(x_aug.dtype)
+        else:
+            (x_aug, weight), x_tile = ctx.saved_tensors, None
         config = ctx.config
         x_aug = x_aug.to(weight.dtype)
         need_x, need_w, need_b = ctx.needs_input_grad[:3]
@@ -466,12 +597,14 @@ class _ConvNd(torch.autograd.Function):
             g_x, g_w, g_b = config.dist_conv_backward_fn(
                 grad_output, x_aug, weight, ctx.stride, ctx.padding, ctx.dilation, ctx.local_in_spatial,
                 ctx.spatial_groups, ctx.channel_group, config, need=(need_x, need_w, need_b),
+                **({"x_tile": x_tile} if x_tile is not None else {}),
             )
         else:
             g_b = config.grad_bias(grad_output.contiguous()) if need_b else None
             g_x, g_w = config.dist_conv_backward_fn(
                 grad_output, x_aug, weight, ctx.stride, ctx.padding, ctx.dilation, ctx.local_in_spatial,
                 ctx.spatial_groups, ctx.channel_group, config, need=(need_x, need_w),
+                **({"x_tile": x_tile} if x_tile is not None else {}),
             )
         return g_x, g_w, g_b, None, None, None, None, None, None
 

@@ -118,6 +118,80 @@ extern "C" int jg_conv_wgrad(void* gw, const void* x, const void* go, const jg_c
   return jg::direct_wgrad(gw, x, go, g, dtype, workspace, workspace_bytes, s);
 }
 
+namespace {
+// Own extent of a framed input inside the padded tensor of `g`; checks the pairing.
+int framed_extent(const jg::ConvGeom& g, const jg_halo_geom* geom, const char* who, int tlo[3], int tn[3]) {
+  JG_REQUIRE(geom != nullptr, "%s: geom is NULL", who);
+  JG_REQUIRE(geom->planes == g.batch * g.cin, "%s: geom->planes %lld != batch * c_in %lld", who,
+             (long long)geom->planes, (long long)(g.batch * g.cin));
+  for (int a = 0; a < 3; ++a) {
+    tlo[a] = geom->lo[a];
+    tn[a] = geom->size[a];
+    JG_REQUIRE(tlo[a] >= 0 && geom->hi[a] >= 0 && tn[a] >= 1 && tlo[a] + tn[a] + geom->hi[a] == g.in[a],
+               "%s: axis %d: lo %d + size %d + hi %d != padded extent %d", who, a, tlo[a], tn[a], geom->hi[a],
+               g.in[a]);
+  }
+  return JG_OK;
+}
+}  // namespace
+
+extern "C" int jg_conv_frame_bands(const jg_conv_desc* desc, const jg_halo_geom* geom, int dtype,
+                                   int32_t band_lo[3], int32_t band_hi[3]) {
+  jg::ConvGeom g;
+  int rc = jg::resolve_conv(desc, "jg_conv_frame_bands", &g);
+  if (rc) return rc;
+  JG_REQUIRE(band_lo && band_hi, "jg_conv_frame_bands: NULL pointer");
+  int tlo[3], tn[3];
+  rc = framed_extent(g, geom, "jg_conv_frame_bands", tlo, tn);
+  if (rc) return rc;
+  if (!jg::mfma_fwd_supported(g, dtype) || !jg::mfma_wgrad_supported(g, dtype) ||
+      !jg::mfma_wgrad_frame_ok(g, tlo, tn))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_frame_bands: geometry / dtype has no framed kernels");
+  int blo[3], bhi[3];
+  jg::mfma_frame_bands(g, tlo, tn, blo, bhi);
+  for (int a = 0; a < 3; ++a) {
+    band_lo[a] = blo[a];
+    band_hi[a] = bhi[a];
+  }
+  return JG_OK;
+}
+
+extern "C" int jg_conv_fwd_framed(void* y, const void* x_frame, const void* x_tile, const void* w,
+                                  const void* bias, const jg_conv_desc* desc, const jg_halo_geom* geom,
+                                  int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  jg::ConvGeom g;
+  int rc = jg::resolve_conv(desc, "jg_conv_fwd_framed", &g);
+  if (rc) return rc;
+  JG_REQUIRE(y && x_frame && x_tile && w, "jg_conv_fwd_framed: NULL pointer");
+  JG_REQUIRE((reinterpret_cast<uintptr_t>(x_tile) & 3) == 0, "jg_conv_fwd_framed: x_tile must be 4-byte aligned");
+  JG_REQUIRE(known(dtype), "jg_conv_fwd_framed: unknown dtype %d", dtype);
+  int tlo[3], tn[3];
+  rc = framed_extent(g, geom, "jg_conv_fwd_framed", tlo, tn);
+  if (rc) return rc;
+  if (!jg::mfma_fwd_supported(g, dtype) || tn[2] % 2 != 0)
+    JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_fwd_framed: geometry / dtype has no framed kernel");
+  return jg::mfma_fwd_framed(y, x_frame, x_tile, tlo, tn, w, bias, g, workspace, workspace_bytes,
+                             static_cast<hipStream_t>(stream));
+}
+
+extern "C" int jg_conv_wgrad_framed(void* gw, void* gb, const void* x_frame, const void* x_tile,
+                                    const void* go, const jg_conv_desc* desc, const jg_halo_geom* geom,
+                                    int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  jg::ConvGeom g;
+  int rc = jg::resolve_conv(desc, "jg_conv_wgrad_framed", &g);
+  if (rc) return rc;
+  JG_REQUIRE(gw && x_frame && x_tile && go, "jg_conv_wgrad_framed: NULL pointer");
+  JG_REQUIRE((reinterpret_cast<uintptr_t>(x_tile) & 3) == 0, "jg_conv_wgrad_framed: x_tile must be 4-byte aligned");
+  JG_REQUIRE(known(dtype), "jg_conv_wgrad_framed: unknown dtype %d", dtype);
+  int tlo[3], tn[3];
+  rc = framed_extent(g, geom, "jg_conv_wgrad_framed", tlo, tn);
+  if (rc) return rc;
+  if (!jg::mfma_wgrad_supported(g, dtype))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_wgrad_framed: geometry / dtype has no framed kernel");
+  return jg::mfma_wgrad(gw, gb, x_frame, go, g, workspace, workspace_bytes, static_cast<hipStream_t>(stream),
+                        x_tile, tlo, tn);
+}
+
 extern "C" int jg_conv_wgrad_bias(void* gw, void* gb, const void* x, const void* go,
                                   const jg_conv_desc* desc, int dtype, void* workspace,
                                   size_t workspace_bytes, void* stream) {

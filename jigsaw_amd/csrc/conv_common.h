@@ -35,6 +35,13 @@ size_t mfma_dgrad_workspace(const ConvGeom& g);
 size_t mfma_wgrad_workspace(const ConvGeom& g);
 int mfma_fwd(void* y, const void* x, const void* w, const void* bias, const ConvGeom& g,
              void* ws, size_t ws_bytes, hipStream_t s);
+// Framed input: x_frame has the padded geometry g.in but only a frame near its edges holds
+// data (mfma_frame_bands); the own tile xt sits at [tlo, tlo + tn) inside it.
+int mfma_fwd_framed(void* y, const void* x_frame, const void* xt, const int tlo[3], const int tn[3],
+                    const void* w, const void* bias, const ConvGeom& g, void* ws, size_t ws_bytes,
+                    hipStream_t s);
+bool mfma_wgrad_frame_ok(const ConvGeom& g, const int tlo[3], const int tn[3]);
+void mfma_frame_bands(const ConvGeom& g, const int tlo[3], const int tn[3], int band_lo[3], int band_hi[3]);
 int mfma_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, void* ws,
                size_t ws_bytes, hipStream_t s);
 // Input gradient split between the unpadded tile and the neighbours' strips: the produced
@@ -42,7 +49,9 @@ int mfma_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, void*
 int mfma_dgrad_fold(void* gx, void* const strips[27], const int lo[3], const int n[3], const void* w,
                     const void* go, const ConvGeom& g, void* ws, size_t ws_bytes, hipStream_t s);
 // gb (Cout,) or NULL: the bias gradient from the same pass over go
+// xt / tlo / tn: framed input as for mfma_fwd_framed, or NULL
 int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom& g, void* ws,
-               size_t ws_bytes, hipStream_t s);
+               size_t ws_bytes, hipStream_t s, const void* xt = nullptr, const int* tlo = nullptr,
+               const int* tn = nullptr);
 
 }  // namespace jg

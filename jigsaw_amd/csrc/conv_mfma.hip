@@ -75,6 +75,11 @@ struct FwdParams {
   // neighbour that owns them. fold = 0: y is the whole produced tensor.
   int fold;
   int lo_d, lo_h, lo_w, nD, nH, nW;
+  // Framed input: xt (N, C, tn_d, tn_h, tn_w) is the own tile, which sits at [tlo, tlo + tn)
+  // inside x. A stage whose window lies inside the tile reads xt, so that only a frame of
+  // x near the edges has to hold data. NULL: everything comes from x.
+  const uint16_t* xt;
+  int tlo_d, tlo_h, tlo_w, tn_d, tn_h, tn_w;
 };
 
 // Strips of the 26 neighbours, slot (dd+1)*9 + (dh+1)*3 + (dw+1); first kernel
@@ -130,7 +135,7 @@ __global__ __launch_bounds__(256) void prep_weights_kernel(uint16_t* __restrict_
 // EVEN: Win, pad_w and the plane size are even and x is 4-byte aligned, so every
 // pixel pair of a task is one aligned dword that is either wholly inside or wholly
 // outside the tensor. Otherwise the prefetch falls back to 2-byte loads.
-template <int MT, bool EVEN, bool FOLD>  // MT = produced channels per workgroup: 32 or 64
+template <int MT, bool EVEN, bool FOLD, bool FRAMED>  // MT = produced channels per workgroup: 32 or 64
 __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips, FwdParams p) {
   constexpr int CB = MT / 32;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -185,6 +190,10 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
   const int g8 = rr / IN_ROWS;
   const uint32_t t_off = (uint32_t)(((size_t)g8 * 8 * chan_stride + (size_t)t_row * p.Win + t_col) * 2);
   const int t_lds = rr * ROW_SLOTS + oct;
+  const size_t plane_t = (size_t)p.tn_h * p.tn_w;
+  const size_t chan_stride_t = plane_t * p.tn_d;
+  const uint32_t chan_bt = (uint32_t)(chan_stride_t * 2);
+  const uint32_t t_off_t = (uint32_t)(((size_t)g8 * 8 * chan_stride_t + (size_t)t_row * p.tn_w + t_col) * 2);
   uint32_t stg[8][4];
 
   struct TileCoord {
@@ -216,6 +225,60 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     const char* last = origin + 2 * ((size_t)(CK - 1) * chan_stride + (size_t)(IN_ROWS - 1) * p.Win + OCTS * 8);
     const bool interior = depth_ok && ih0 >= 0 && ih0 + IN_ROWS <= p.Hin && iw0 >= 0 &&
                           iw0 + TW + KW - 1 <= p.Win && last <= p.x_end;
+    if (FRAMED) {
+      // window inside the own tile (wave-uniform): read the tile itself, at whatever
+      // alignment its rows give the window
+      const int dt = id - p.tlo_d, ht = ih0 - p.tlo_h, wt = iw0 - p.tlo_w;
+      const char* origin_t = reinterpret_cast<const char*>(p.xt) +
+                             2 * ((ptrdiff_t)(((size_t)tc.n * p.C + c0) * chan_stride_t) +
+                                  (ptrdiff_t)dt * (ptrdiff_t)plane_t + (ptrdiff_t)ht * p.tn_w + wt);
+      if (dt >= 0 && dt < p.tn_d && ht >= 0 && ht + IN_ROWS <= p.tn_h && wt >= 0 && wt + TW + KW - 1 <= p.tn_w) {
+        if (!has_task) return;
+        // 4-byte aligned accesses only (2-byte aligned vector loads run at a fraction of the
+        // rate): a window that starts on an odd column is read one pixel early and shifted.
+        const bool odd = ((reinterpret_cast<uintptr_t>(origin_t) + t_off_t) & 2) != 0;  // wave-uniform
+        const char* at = origin_t + t_off_t;
+        if (!odd) {
+          if (oct == OCTS - 1) {
+            // the last octet holds the window's last 2 pixels; the other 6 may lie past the row
+            // (and the tensor), so only one dword is read
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+              stg[c][0] = *reinterpret_cast<const uint32_t*>(at + (size_t)c * chan_bt);
+              stg[c][1] = 0u; stg[c][2] = 0u; stg[c][3] = 0u;
+            }
+          } else {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+              const u32x4_a4 v = *reinterpret_cast<const u32x4_a4*>(at + (size_t)c * chan_bt);
+              stg[c][0] = v.x; stg[c][1] = v.y; stg[c][2] = v.z; stg[c][3] = v.w;
+            }
+          }
+        } else {
+          uint32_t d0[8];
+#pragma unroll
+          for (int c = 0; c < 8; ++c) d0[c] = *reinterpret_cast<const uint32_t*>(at - 2 + (size_t)c * chan_bt);
+          if (oct == OCTS - 1) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+              const uint32_t d1 = *reinterpret_cast<const uint32_t*>(at + 2 + (size_t)c * chan_bt);
+              stg[c][0] = __builtin_amdgcn_alignbit(d1, d0[c], 16);
+              stg[c][1] = 0u; stg[c][2] = 0u; stg[c][3] = 0u;
+            }
+          } else {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+              const u32x4_a4 v = *reinterpret_cast<const u32x4_a4*>(at + 2 + (size_t)c * chan_bt);
+              stg[c][0] = __builtin_amdgcn_alignbit(v.x, d0[c], 16);
+              stg[c][1] = __builtin_amdgcn_alignbit(v.y, v.x, 16);
+              stg[c][2] = __builtin_amdgcn_alignbit(v.z, v.y, 16);
+              stg[c][3] = __builtin_amdgcn_alignbit(v.w, v.z, 16);
+            }
+          }
+        }
+        return;
+      }
+    }
     if (!has_task) return;
     const char* a = origin + t_off;
     if (EVEN && interior) {
@@ -515,6 +578,8 @@ struct Launch {
   int fold;                 // fold mode: y is the unpadded tile, strips receive the halo cells
   int lo[3], n[3];          // own extent inside the produced tensor (fold mode)
   void* const* strips;      // 27 slots (fold mode)
+  const uint16_t* xt;       // own tile for the framed input, or NULL
+  int tlo[3], tn[3];
 };
 
 int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const char* who) {
@@ -546,6 +611,9 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   p.fold = L.fold;
   p.lo_d = L.lo[0]; p.lo_h = L.lo[1]; p.lo_w = L.lo[2];
   p.nD = L.n[0]; p.nH = L.n[1]; p.nW = L.n[2];
+  p.xt = L.xt;
+  p.tlo_d = L.tlo[0]; p.tlo_h = L.tlo[1]; p.tlo_w = L.tlo[2];
+  p.tn_d = L.tn[0]; p.tn_h = L.tn[1]; p.tn_w = L.tn[2];
   StripTable tab;
   for (int i = 0; i < 27; ++i) tab.p[i] = (L.fold && L.strips != nullptr) ? L.strips[i] : nullptr;
   if (tiles == 0) return JG_OK;
@@ -558,11 +626,14 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
                     ((reinterpret_cast<uintptr_t>(L.x) & 3) == 0);
   void (*kern)(StripTable, FwdParams) = nullptr;
   if (L.fold) {
-    if (MT == 64) kern = even ? &conv3x3_mfma_kernel<64, true, true> : &conv3x3_mfma_kernel<64, false, true>;
-    else kern = even ? &conv3x3_mfma_kernel<32, true, true> : &conv3x3_mfma_kernel<32, false, true>;
+    if (MT == 64) kern = even ? &conv3x3_mfma_kernel<64, true, true, false> : &conv3x3_mfma_kernel<64, false, true, false>;
+    else kern = even ? &conv3x3_mfma_kernel<32, true, true, false> : &conv3x3_mfma_kernel<32, false, true, false>;
+  } else if (L.xt != nullptr) {
+    if (MT == 64) kern = even ? &conv3x3_mfma_kernel<64, true, false, true> : &conv3x3_mfma_kernel<64, false, false, true>;
+    else kern = even ? &conv3x3_mfma_kernel<32, true, false, true> : &conv3x3_mfma_kernel<32, false, false, true>;
   } else {
-    if (MT == 64) kern = even ? &conv3x3_mfma_kernel<64, true, false> : &conv3x3_mfma_kernel<64, false, false>;
-    else kern = even ? &conv3x3_mfma_kernel<32, true, false> : &conv3x3_mfma_kernel<32, false, false>;
+    if (MT == 64) kern = even ? &conv3x3_mfma_kernel<64, true, false, false> : &conv3x3_mfma_kernel<64, false, false, false>;
+    else kern = even ? &conv3x3_mfma_kernel<32, true, false, false> : &conv3x3_mfma_kernel<32, false, false, false>;
   }
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -589,8 +660,9 @@ bool mfma_dgrad_supported(const ConvGeom& g, int dtype) {
 size_t mfma_fwd_workspace(const ConvGeom& g) { return prep_bytes(g.k[0] * g.cin, g.cout); }
 size_t mfma_dgrad_workspace(const ConvGeom& g) { return prep_bytes(g.k[0] * g.cout, g.cin); }
 
-int mfma_fwd(void* y, const void* x, const void* w, const void* bias, const ConvGeom& g, void* ws,
-             size_t ws_bytes, hipStream_t s) {
+static int fwd_launch(void* y, const void* x, const void* xt, const int* tlo, const int* tn, const void* w,
+                      const void* bias, const ConvGeom& g, void* ws, size_t ws_bytes, hipStream_t s,
+                      const char* who) {
   Launch L;
   L.x = static_cast<const uint16_t*>(x);
   L.w = static_cast<const uint16_t*>(w);
@@ -603,8 +675,59 @@ int mfma_fwd(void* y, const void* x, const void* w, const void* bias, const Conv
   L.transposed = 0;
   L.fold = 0;
   L.strips = nullptr;
-  for (int a = 0; a < 3; ++a) L.lo[a] = L.n[a] = 0;
-  return launch_conv(L, ws, ws_bytes, s, "jg_conv_fwd(mfma)");
+  L.xt = static_cast<const uint16_t*>(xt);
+  for (int a = 0; a < 3; ++a) {
+    L.lo[a] = L.n[a] = 0;
+    L.tlo[a] = tlo ? tlo[a] : 0;
+    L.tn[a] = tn ? tn[a] : 0;
+  }
+  return launch_conv(L, ws, ws_bytes, s, who);
+}
+
+int mfma_fwd(void* y, const void* x, const void* w, const void* bias, const ConvGeom& g, void* ws,
+             size_t ws_bytes, hipStream_t s) {
+  return fwd_launch(y, x, nullptr, nullptr, nullptr, w, bias, g, ws, ws_bytes, s, "jg_conv_fwd(mfma)");
+}
+
+int mfma_fwd_framed(void* y, const void* x_frame, const void* xt, const int tlo[3], const int tn[3],
+                    const void* w, const void* bias, const ConvGeom& g, void* ws, size_t ws_bytes,
+                    hipStream_t s) {
+  return fwd_launch(y, x_frame, xt, tlo, tn, w, bias, g, ws, ws_bytes, s, "jg_conv_fwd_framed(mfma)");
+}
+
+// Bands of the padded tile that the framed kernels read from x_frame: everything a
+// 16 x 64 output tile window (18 x 72 cells) touches when it does not lie inside the tile.
+void mfma_frame_bands(const ConvGeom& g, const int tlo[3], const int tn[3], int band_lo[3], int band_hi[3]) {
+  // depth: a stage reads one plane; planes outside the tile are read whole
+  band_lo[0] = tlo[0];
+  band_hi[0] = g.in[0] - tlo[0] - tn[0];
+  const int tile[3] = {1, TH, TW};
+  const int reach[3] = {1, IN_ROWS, OCTS * 8};  // cells a window may touch (the last octet in full)
+  const int need[3] = {1, IN_ROWS, TW + KW - 1};
+  for (int a = 1; a < 3; ++a) {
+    const int ntiles = (g.out[a] + tile[a] - 1) / tile[a];
+    int first_in = -1, last_in = -1;  // tiles whose window lies inside [tlo, tlo + tn)
+    for (int t = 0; t < ntiles; ++t) {
+      const int w0 = t * tile[a] - g.p[a];
+      if (w0 >= tlo[a] && w0 + need[a] <= tlo[a] + tn[a]) {
+        if (first_in < 0) first_in = t;
+        last_in = t;
+      }
+    }
+    if (first_in < 0) {  // no tile reads the own tile along this axis: everything from the frame
+      band_lo[a] = g.in[a];
+      band_hi[a] = 0;
+      continue;
+    }
+    int lo_end = (first_in - 1) * tile[a] - g.p[a] + reach[a];  // end of the last window before
+    if (first_in == 0 || lo_end < 0) lo_end = 0;
+    if (lo_end > g.in[a]) lo_end = g.in[a];
+    int hi_begin = (last_in + 1) * tile[a] - g.p[a];             // start of the first window after
+    if (last_in == ntiles - 1 || hi_begin > g.in[a]) hi_begin = g.in[a];
+    if (hi_begin < 0) hi_begin = 0;
+    band_lo[a] = lo_end;
+    band_hi[a] = g.in[a] - hi_begin;
+  }
 }
 
 // gx = conv(go zero-padded by k-1-p, flipped / transposed weights). With `own` given,
@@ -624,9 +747,11 @@ static int dgrad_launch(void* gx, void* const* strips, const int* lo, const int*
   L.transposed = 1;
   L.fold = lo != nullptr;
   L.strips = strips;
+  L.xt = nullptr;
   for (int a = 0; a < 3; ++a) {
     L.lo[a] = lo ? lo[a] : 0;
     L.n[a] = n ? n[a] : 0;
+    L.tlo[a] = L.tn[a] = 0;
   }
   return launch_conv(L, ws, ws_bytes, s, who);
 }

@@ -39,6 +39,7 @@
 namespace {
 
 using jg::ConvGeom;
+using jg::mfma_frame_bands;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -59,6 +60,10 @@ struct WgradParams {
   const char* x_end;  // one past the last byte of x
   float* part;        // [wavefront slot][tap9][co][c']
   float* bias_part;   // [workgroup][co] or NULL
+  // Framed input: xt (N, Cin, tn_d, tn_h, tn_w) is the own tile, at [tlo, tlo + tn) inside x.
+  // A row pair whose window lies inside the tile is read from xt. NULL: all from x.
+  const uint16_t* xt;
+  int tlo_d, tlo_h, tlo_w, tn_d, tn_h, tn_w;
   int Cin, Cout;
   int Din, Hin, Win, Dout, Hout, Wout;
   int pad_d, pad_h, pad_w;
@@ -82,7 +87,7 @@ __device__ __forceinline__ float sum_bf16x8(const u32x4& v) {
   return s;
 }
 
-template <int CGB, int CXB, bool EVEN>
+template <int CGB, int CXB, bool EVEN, bool FRAMED>
 __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(WgradParams p) {
   constexpr int THREADS = wgrad_threads(CGB, CXB);
   constexpr int CWAVES = CGB * CXB * HALVES;  // wavefronts that own accumulators
@@ -145,6 +150,32 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
     t_goff = (uint32_t)((ci * x_cs + kd * plane_x + (size_t)r2 * p.Win + SW) * 2);
     t_lds = (uint32_t)(ch * X_CH + SW * 2);
   }
+  // the same x offsets inside the own tile (framed input)
+  const size_t plane_t = (size_t)p.tn_h * p.tn_w, t_cs = plane_t * p.tn_d;
+  uint32_t c_toff[ROUNDS];
+  uint32_t t_toff = 0;
+  uint32_t x_kd = 0;  // 2 bits per round: depth tap of the chunk; bits 30-31: of the tail
+  if (FRAMED) {
+#pragma unroll
+    for (int rd = 0; rd < ROUNDS; ++rd) {
+      const int q = tid + rd * THREADS;
+      c_toff[rd] = 0;
+      if (q >= G_CHUNKS && q < CHUNKS) {
+        const int qx = q - G_CHUNKS;
+        const int c8 = qx % X_CPR, rr = qx / X_CPR;
+        const int r2 = rr & 1, ch = rr >> 1;
+        const int kd = ch / p.Cin, ci = ch - kd * p.Cin;
+        c_toff[rd] = (uint32_t)((ci * t_cs + kd * plane_t + (size_t)r2 * p.tn_w + c8 * 8) * 2);
+        x_kd |= (uint32_t)kd << (2 * rd);
+      }
+    }
+    if (has_tail) {
+      const int r2 = tid & 1, ch = tid >> 1;
+      const int kd = ch / p.Cin, ci = ch - kd * p.Cin;
+      t_toff = (uint32_t)((ci * t_cs + kd * plane_t + (size_t)r2 * p.tn_w + SW) * 2);
+      x_kd |= (uint32_t)kd << 30;
+    }
+  }
 
   struct Staged {
     u32x4 v[ROUNDS];
@@ -194,6 +225,77 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
     const bool inside = EVEN && oh0 + SR <= p.Hout && ow0 + SW <= p.Wout && ih0 >= 0 &&
                         ih0 + 2 <= p.Hin && iw0 >= 0 && iw0 + SW + 2 <= p.Win && id0 >= 0 &&
                         id0 + (XC / p.Cin) <= p.Din;
+    if (FRAMED && inside) {
+      // Rows and columns of the pair's window inside the own tile (wave-uniform): a chunk
+      // whose depth plane is a plane of the tile comes from the tile itself, at whatever
+      // alignment its rows give the window; the planes outside the tile are halo planes,
+      // which the frame holds whole.
+      const int dt = id0 - p.tlo_d, ht = ih0 - p.tlo_h, wt = iw0 - p.tlo_w;
+      if (ht >= 0 && ht + 2 <= p.tn_h && wt >= 0 && wt + SW + 2 <= p.tn_w) {
+        const char* t_org = reinterpret_cast<const char*>(p.xt) +
+                            2 * ((ptrdiff_t)((size_t)n * p.Cin * t_cs) + (ptrdiff_t)dt * (ptrdiff_t)plane_t +
+                                 (ptrdiff_t)ht * p.tn_w + wt);
+        // 4-byte aligned accesses only (2-byte aligned vector loads run at a fraction of the
+        // rate): a window that starts on an odd column is read one pixel early and shifted.
+        // tn_w is even (checked on the host), so the parity is the same for every chunk.
+        const bool odd = (reinterpret_cast<uintptr_t>(t_org) & 2) != 0;  // wave-uniform
+        uint32_t lead[ROUNDS];
+#pragma unroll
+        for (int rd = 0; rd < ROUNDS; ++rd) {
+          const int q = tid + rd * THREADS;
+          lead[rd] = 0u;
+          if (q < G_CHUNKS) {
+            if (want_g) v[rd] = *reinterpret_cast<const u32x4_a4*>(g_org + c_goff[rd]);
+          } else if (q < CHUNKS) {
+            const int dd = dt + (int)((x_kd >> (2 * rd)) & 3u);
+            if (dd >= 0 && dd < p.tn_d) {
+              if (odd) {
+                lead[rd] = *reinterpret_cast<const uint32_t*>(t_org + c_toff[rd] - 2);
+                v[rd] = *reinterpret_cast<const u32x4_a4*>(t_org + c_toff[rd] + 2);
+              } else {
+                v[rd] = *reinterpret_cast<const u32x4_a4*>(t_org + c_toff[rd]);
+              }
+            } else {
+              v[rd] = *reinterpret_cast<const u32x4_a4*>(x_org + c_goff[rd]);
+            }
+          }
+        }
+        uint32_t tail_lead = 0u;
+        bool tail_shift = false;
+        if (has_tail) {
+          const int dd = dt + (int)(x_kd >> 30);
+          if (dd >= 0 && dd < p.tn_d) {
+            if (odd) {
+              tail_lead = *reinterpret_cast<const uint32_t*>(t_org + t_toff - 2);
+              sg.tail = *reinterpret_cast<const uint32_t*>(t_org + t_toff + 2);
+              tail_shift = true;
+            } else {
+              sg.tail = *reinterpret_cast<const uint32_t*>(t_org + t_toff);
+            }
+          } else {
+            sg.tail = *reinterpret_cast<const uint32_t*>(x_org + t_goff);
+          }
+        }
+        if (odd) {
+#pragma unroll
+          for (int rd = 0; rd < ROUNDS; ++rd) {
+            const int q = tid + rd * THREADS;
+            if (q >= G_CHUNKS && q < CHUNKS) {
+              const int dd = dt + (int)((x_kd >> (2 * rd)) & 3u);
+              if (dd >= 0 && dd < p.tn_d) {
+                const u32x4 t = v[rd];
+                v[rd].x = __builtin_amdgcn_alignbit(t.x, lead[rd], 16);
+                v[rd].y = __builtin_amdgcn_alignbit(t.y, t.x, 16);
+                v[rd].z = __builtin_amdgcn_alignbit(t.z, t.y, 16);
+                v[rd].w = __builtin_amdgcn_alignbit(t.w, t.z, 16);
+              }
+            }
+          }
+          if (tail_shift) sg.tail = __builtin_amdgcn_alignbit(sg.tail, tail_lead, 16);
+        }
+        return;
+      }
+    }
     if (inside) {
 #pragma unroll
       for (int rd = 0; rd < ROUNDS; ++rd) {
@@ -485,8 +587,11 @@ template <int CGB, int CXB>
 int launch(const WgradParams& p, bool even, int wgs, hipStream_t s, const char* who) {
   constexpr int THREADS = wgrad_threads(CGB, CXB);
   const size_t lds = 2 * (size_t)(32 * CGB * G_CH) + (size_t)(32 * CXB * X_CH);
-  void (*kern)(WgradParams) =
-      even ? &wgrad3x3_mfma_kernel<CGB, CXB, true> : &wgrad3x3_mfma_kernel<CGB, CXB, false>;
+  void (*kern)(WgradParams);
+  if (p.xt != nullptr)
+    kern = &wgrad3x3_mfma_kernel<CGB, CXB, true, true>;  // the framed input needs the even layout (checked by the caller)
+  else
+    kern = even ? &wgrad3x3_mfma_kernel<CGB, CXB, true, false> : &wgrad3x3_mfma_kernel<CGB, CXB, false, false>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", who, lds);
@@ -511,8 +616,33 @@ size_t mfma_wgrad_workspace(const ConvGeom& g) {
   return wgs * HALVES * 9 * (32 * cgb) * (32 * cxb) * sizeof(float) + wgs * (32 * cgb) * sizeof(float);
 }
 
+// Whether the framed weight-gradient kernel covers a geometry: even row lengths (its
+// vector loads), and every row pair / column tile whose window leaves the own tile lies
+// inside the bands that the frame holds.
+bool mfma_wgrad_frame_ok(const ConvGeom& g, const int tlo[3], const int tn[3]) {
+  if (g.in[2] % 2 != 0 || g.p[2] % 2 != 0 || g.out[2] % 2 != 0 || tn[2] % 2 != 0) return false;
+  int blo[3], bhi[3];
+  mfma_frame_bands(g, tlo, tn, blo, bhi);
+  const int row_pairs = (g.out[1] + SR - 1) / SR, col_tiles = (g.out[2] + SW - 1) / SW;
+  for (int j = 0; j < row_pairs + 1; ++j) {  // x row pairs of all stages: [2j - pad, 2j - pad + 2)
+    const int r = 2 * j - g.p[1];
+    const bool in_tile = r >= tlo[1] && r + 2 <= tlo[1] + tn[1];
+    const int r_end = r + 2 < g.in[1] ? r + 2 : g.in[1];  // what lies past the tensor is not read
+    const bool in_band = r_end <= blo[1] || r >= g.in[1] - bhi[1];
+    if (!in_tile && !in_band) return false;
+  }
+  for (int ct = 0; ct < col_tiles; ++ct) {
+    const int c = ct * SW - g.p[2];
+    const bool in_tile = c >= tlo[2] && c + SW + 2 <= tlo[2] + tn[2];
+    const int c_end = c + SW + 2 < g.in[2] ? c + SW + 2 : g.in[2];
+    const bool in_band = c_end <= blo[2] || c >= g.in[2] - bhi[2];
+    if (!in_tile && !in_band) return false;
+  }
+  return true;
+}
+
 int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom& g, void* ws,
-               size_t ws_bytes, hipStream_t s) {
+               size_t ws_bytes, hipStream_t s, const void* xt, const int* tlo, const int* tn) {
   const char* who = "jg_conv_wgrad(mfma)";
   int cgb, cxb;
   if (!blocks_of(g, &cgb, &cxb)) JG_FAIL(JG_ERR_UNSUPPORTED, "%s: geometry not covered", who);
@@ -534,10 +664,15 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
   p.col_tiles = (g.out[2] + SW - 1) / SW;
   p.total_stages = stage_count(g);
   const int wgs = wg_count(p.total_stages);
+  p.xt = static_cast<const uint16_t*>(xt);
+  p.tlo_d = tlo ? tlo[0] : 0; p.tlo_h = tlo ? tlo[1] : 0; p.tlo_w = tlo ? tlo[2] : 0;
+  p.tn_d = tn ? tn[0] : 0; p.tn_h = tn ? tn[1] : 0; p.tn_w = tn ? tn[2] : 0;
   p.bias_part = gb != nullptr ? p.part + (size_t)wgs * HALVES * 9 * (32 * cgb) * (32 * cxb) : nullptr;
   const bool even = (p.Win % 2 == 0) && (p.pad_w % 2 == 0) && (p.Wout % 2 == 0) &&
                     ((reinterpret_cast<uintptr_t>(x) & 3) == 0) &&
                     ((reinterpret_cast<uintptr_t>(go) & 3) == 0);
+  if (xt != nullptr && (!even || !mfma_wgrad_frame_ok(g, tlo, tn)))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: the framed input does not cover this geometry / alignment", who);
   int rc;
   if (cgb == 2 && cxb == 2) rc = launch<2, 2>(p, even, wgs, s, who);
   else if (cgb == 1 && cxb == 3) rc = launch<1, 3>(p, even, wgs, s, who);

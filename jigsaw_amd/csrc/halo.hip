@@ -445,6 +445,109 @@ __global__ __launch_bounds__(256) void assemble_rows_kernel(Table tab, T* __rest
   }
 }
 
+// k-th border coordinate of an axis of extent n reached over [0, hi) and [n - lo, n)
+__device__ __forceinline__ int border_coord(int k, int n, int lo, int hi) {
+  if (hi + lo >= n) return k;
+  return k < hi ? k : n - lo + (k - hi);
+}
+
+// Assemble restricted to a frame of the padded tile: only the cells whose padded
+// coordinate lies in the first band_lo or the last band_hi positions of some axis are
+// written. Two kinds of launches of one kernel: `full_rows` = the rows inside a D or H
+// band, written whole; otherwise the remaining rows, of which only columns
+// [c_begin, c_end) (a W band) are written.
+struct FramePlan {
+  uint32_t rows_per_plane, total_rows;
+  int full_rows;
+  int nbd, nbh;                 // band rows along D / H (first + last), clipped to the extent
+  int bd_lo, bd_hi, bh_lo, bh_hi;
+  int c_begin, c_end;
+  int lpr_log2;
+  Magic div_rows, div_a, div_b;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void assemble_frame_kernel(Table tab, T* __restrict__ dst, Geom g,
+                                                             FramePlan fp) {
+  constexpr int V = Bits<T>::V;
+  typedef uint32_t u32x4_any __attribute__((ext_vector_type(4), aligned(2)));
+  const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+  const uint32_t item = t >> fp.lpr_log2;
+  if (item >= fp.total_rows) return;
+  const int lir = (int)(t & ((1u << fp.lpr_log2) - 1));
+  const int Da = g.lo[0] + g.n[0] + g.hi[0];
+  const int Ha = g.lo[1] + g.n[1] + g.hi[1];
+  const int Wa = g.lo[2] + g.n[2] + g.hi[2];
+  const uint32_t pp = mdiv(item, fp.div_rows);
+  const uint32_t idx = item - pp * fp.rows_per_plane;
+  int da, ha;
+  if (fp.full_rows) {
+    if (idx < (uint32_t)fp.nbd * (uint32_t)Ha) {
+      const uint32_t k = mdiv(idx, fp.div_a);  // / Ha
+      da = border_coord((int)k, Da, fp.bd_hi, fp.bd_lo);
+      ha = (int)(idx - k * (uint32_t)Ha);
+    } else {
+      const uint32_t idx2 = idx - (uint32_t)fp.nbd * (uint32_t)Ha;
+      const uint32_t di = mdiv(idx2, fp.div_b);  // / nbh
+      da = fp.bd_lo + (int)di;
+      ha = border_coord((int)(idx2 - di * (uint32_t)fp.nbh), Ha, fp.bh_hi, fp.bh_lo);
+    }
+  } else {
+    const uint32_t di = mdiv(idx, fp.div_a);  // / (Ha - nbh)
+    da = fp.bd_lo + (int)di;
+    ha = fp.bh_lo + (int)(idx - di * (uint32_t)(Ha - fp.nbh));
+  }
+  int rd, cd, ed, rh, ch, eh;
+  region(da, g.lo[0], g.n[0], g.hi[0], rd, cd, ed);
+  region(ha, g.lo[1], g.n[1], g.hi[1], rh, ch, eh);
+  const long long line = ((long long)pp * ed + cd) * eh + ch;
+  const int base_idx = rd * 9 + rh * 3;
+  const T* s0 = static_cast<const T*>(table_entry(base_idx + 0));
+  const T* s1 = static_cast<const T*>(table_entry(base_idx + 1));
+  const T* s2 = static_cast<const T*>(table_entry(base_idx + 2));
+  if (s0 != nullptr) s0 += line * g.lo[2];
+  if (s1 != nullptr) s1 += line * g.n[2];
+  if (s2 != nullptr) s2 += line * g.hi[2];
+  T* drow = dst + (((long long)pp * Da + da) * Ha + ha) * (long long)Wa;
+  const int mid_lo = g.lo[2], mid_hi = g.lo[2] + g.n[2];
+  // middle source in 16-byte vectors of its own row, clipped to the column window
+  const int m_begin = fp.c_begin > mid_lo ? fp.c_begin : mid_lo;
+  const int m_end = fp.c_end < mid_hi ? fp.c_end : mid_hi;
+  const int j0 = (m_begin - mid_lo + V - 1) / V, j1 = (m_end - mid_lo) / V;  // whole vectors [j0, j1)
+  const int n_full = j1 > j0 ? j1 - j0 : 0;
+  for (int it0 = 0; (it0 << fp.lpr_log2) < n_full; it0 += ROW_BATCH) {
+    u32x4 val[ROW_BATCH];
+#pragma unroll
+    for (int u = 0; u < ROW_BATCH; ++u) {
+      const int j = lir + ((it0 + u) << fp.lpr_log2);
+      val[u] = u32x4{0u, 0u, 0u, 0u};
+      if (j < n_full && s1 != nullptr) val[u] = *reinterpret_cast<const u32x4_any*>(s1 + (j0 + j) * V);
+    }
+#pragma unroll
+    for (int u = 0; u < ROW_BATCH; ++u) {
+      const int j = lir + ((it0 + u) << fp.lpr_log2);
+      if (j < n_full) *reinterpret_cast<u32x4_any*>(drow + mid_lo + (j0 + j) * V) = val[u];
+    }
+  }
+  // what the vectors left of the window: [c_begin, head_end) and [tail0, c_end)
+  const int head_end = n_full > 0 ? mid_lo + j0 * V : fp.c_end;
+  const int tail0 = n_full > 0 ? mid_lo + j1 * V : fp.c_end;
+  const int n_head = head_end - fp.c_begin;
+  const int n_edge = n_head + (fp.c_end - tail0);
+  for (int q = lir; q < n_edge; q += (1 << fp.lpr_log2)) {
+    const int c = q < n_head ? fp.c_begin + q : tail0 + (q - n_head);
+    const T* src = nullptr;
+    if (c < mid_lo) {
+      if (s0 != nullptr) src = s0 + c;
+    } else if (c < mid_hi) {
+      if (s1 != nullptr) src = s1 + (c - mid_lo);
+    } else {
+      if (s2 != nullptr) src = s2 + (c - mid_hi);
+    }
+    drow[c] = src != nullptr ? *src : T(0);
+  }
+}
+
 // One element of the fold with the loops left rolled: only the offsets that reach
 // the element cost anything (most edge elements see one or two neighbours).
 template <int DT>
@@ -670,11 +773,6 @@ struct BorderPlan {
   Magic div_rows, div_h, div_nbh, div_edge, div_hh, div_d;
 };
 
-// k-th border coordinate of an axis of extent n reached over [0, hi) and [n - lo, n)
-__device__ __forceinline__ int border_coord(int k, int n, int lo, int hi) {
-  if (hi + lo >= n) return k;
-  return k < hi ? k : n - lo + (k - hi);
-}
 
 template <int DT>
 __global__ __launch_bounds__(256) void fold_border_rows_kernel(Table tab, typename Arith<DT>::T* __restrict__ gx,
@@ -872,6 +970,80 @@ extern "C" int jg_halo_assemble_3d(void* x_aug, const void* const src[27],
   }
   JG_CHECK_LAUNCH("jg_halo_assemble_3d");
   return JG_OK;
+}
+
+extern "C" int jg_halo_assemble_frame_3d(void* x_aug, const void* const src[27],
+                                         const jg_halo_geom* geom, const int32_t band_lo[3],
+                                         const int32_t band_hi[3], int elem_size, void* stream) {
+  const char* who = "jg_halo_assemble_frame_3d";
+  int rc = check_geom(geom, who, true);
+  if (rc) return rc;
+  JG_REQUIRE(x_aug != nullptr && src != nullptr && band_lo != nullptr && band_hi != nullptr, "%s: NULL pointer", who);
+  JG_REQUIRE(src[13] != nullptr, "%s: slot 13 (own tile) is NULL", who);
+  JG_REQUIRE(elem_size == 2 || elem_size == 4, "%s: elem_size %d not in {2, 4}", who, elem_size);
+  Table tab;
+  for (int i = 0; i < 27; ++i) {
+    tab.p[i] = src[i];
+    JG_REQUIRE((reinterpret_cast<uintptr_t>(src[i]) & (elem_size - 1)) == 0, "%s: slot %d is not element aligned", who, i);
+  }
+  JG_REQUIRE((reinterpret_cast<uintptr_t>(x_aug) & (elem_size - 1)) == 0, "%s: x_aug is not element aligned", who);
+  Geom g = to_geom(geom);
+  int ext[3], blo[3], bhi[3];
+  for (int a = 0; a < 3; ++a) {
+    ext[a] = g.lo[a] + g.n[a] + g.hi[a];
+    JG_REQUIRE(band_lo[a] >= 0 && band_hi[a] >= 0, "%s: negative band on axis %d", who, a);
+    blo[a] = band_lo[a];
+    bhi[a] = band_hi[a];
+    if (blo[a] + bhi[a] >= ext[a]) {  // the bands meet: the whole axis
+      blo[a] = ext[a];
+      bhi[a] = 0;
+    }
+  }
+  if (g.planes == 0 || ext[0] == 0 || ext[1] == 0 || ext[2] == 0) return JG_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int V = 16 / elem_size;
+  FramePlan fp;
+  fp.bd_lo = blo[0]; fp.bd_hi = bhi[0]; fp.bh_lo = blo[1]; fp.bh_hi = bhi[1];
+  fp.nbd = blo[0] + bhi[0];
+  fp.nbh = blo[1] + bhi[1];
+  auto launch = [&](int full_rows, int c_begin, int c_end) -> int {
+    if (c_end <= c_begin) return JG_OK;
+    fp.full_rows = full_rows;
+    fp.c_begin = c_begin;
+    fp.c_end = c_end;
+    unsigned long long rpp;
+    if (full_rows) {
+      rpp = (unsigned long long)fp.nbd * ext[1] + (unsigned long long)(ext[0] - fp.nbd) * fp.nbh;
+      fp.div_a = make_magic((uint32_t)ext[1]);
+      fp.div_b = make_magic((uint32_t)(fp.nbh > 0 ? fp.nbh : 1));
+    } else {
+      rpp = (unsigned long long)(ext[0] - fp.nbd) * (ext[1] - fp.nbh);
+      fp.div_a = make_magic((uint32_t)(ext[1] - fp.nbh > 0 ? ext[1] - fp.nbh : 1));
+      fp.div_b = fp.div_a;
+    }
+    if (rpp == 0) return JG_OK;
+    const int nvec = (c_end - c_begin + V - 1) / V + 1;
+    int lg = 0;
+    while ((1 << lg) * 2 < nvec && lg < 6) ++lg;
+    fp.lpr_log2 = lg;
+    const unsigned long long rows = (unsigned long long)g.planes * rpp;
+    JG_REQUIRE((rows << lg) < (1ull << 32), "%s: too many rows (%llu)", who, rows);
+    fp.rows_per_plane = (uint32_t)rpp;
+    fp.total_rows = (uint32_t)rows;
+    fp.div_rows = make_magic((uint32_t)rpp);
+    const unsigned blocks = (unsigned)(((rows << lg) + 255) / 256);
+    if (elem_size == 2)
+      assemble_frame_kernel<uint16_t><<<blocks, 256, 0, s>>>(tab, static_cast<uint16_t*>(x_aug), g, fp);
+    else
+      assemble_frame_kernel<uint32_t><<<blocks, 256, 0, s>>>(tab, static_cast<uint32_t*>(x_aug), g, fp);
+    JG_CHECK_LAUNCH(who);
+    return JG_OK;
+  };
+  rc = launch(1, 0, ext[2]);                        // rows inside a D or H band, whole
+  if (rc) return rc;
+  rc = launch(0, 0, blo[2]);                        // other rows: first W band
+  if (rc) return rc;
+  return launch(0, ext[2] - bhi[2], ext[2]);        // other rows: last W band
 }
 
 extern "C" int jg_halo_assemble_2d(void* x_aug, const void* const src[9], int64_t planes,

@@ -13,6 +13,7 @@ gradient and folds the received ones in the reference's association order
 
 from __future__ import annotations
 
+import ctypes
 import itertools
 from dataclasses import dataclass
 from typing import Mapping, Sequence
@@ -211,11 +212,18 @@ def halo_assemble(
     strips: Mapping[Offset, torch.Tensor | None],
     geom: HaloGeometry,
     out: torch.Tensor | None = None,
+    bands: tuple | None = None,
 ) -> torch.Tensor:
     """Padded tile from the own tile and the strips received from the neighbours.
 
     A missing / ``None`` strip is a neighbour outside the domain and reads as
     zero (halo.py:77). Bit-exact copy, one pass over the destination.
+
+    ``bands = (band_lo, band_hi)`` (one entry per spatial axis) writes only the
+    frame of the padded tile: the cells within ``band_lo[a]`` of the start or
+    ``band_hi[a]`` of the end of some axis. The rest of the result is left
+    uninitialised; it is meant for the framed convolution functions, which read
+    the own tile everywhere else (``conv.frame_bands``).
     """
     _lib.require_gpu(x)
     planes = _check_tile(x, geom.size, "halo_assemble")
@@ -226,8 +234,20 @@ def halo_assemble(
         raise ValueError("halo_assemble: `out` has the wrong shape / dtype / layout")
     tab = _table(strips, geom, "assemble", lead, x, x)
     cg = geom.c_geom(planes)
-    rc = _lib.load().jg_halo_assemble_3d(_lib.ptr(out), tab, cg, x.element_size(), _lib.stream_ptr(x.device))
-    _lib.check(rc, "jg_halo_assemble_3d")
+    if bands is None:
+        rc = _lib.load().jg_halo_assemble_3d(_lib.ptr(out), tab, cg, x.element_size(), _lib.stream_ptr(x.device))
+        _lib.check(rc, "jg_halo_assemble_3d")
+        return out
+    band_lo, band_hi = bands
+    if len(band_lo) != geom.n_spatial or len(band_hi) != geom.n_spatial:
+        raise ValueError("halo_assemble: `bands` needs one (lo, hi) entry per spatial axis")
+    pad = 3 - geom.n_spatial
+    c_lo = (ctypes.c_int32 * 3)(*([0] * pad + [int(v) for v in band_lo]))
+    c_hi = (ctypes.c_int32 * 3)(*([0] * pad + [int(v) for v in band_hi]))
+    rc = _lib.load().jg_halo_assemble_frame_3d(
+        _lib.ptr(out), tab, cg, c_lo, c_hi, x.element_size(), _lib.stream_ptr(x.device)
+    )
+    _lib.check(rc, "jg_halo_assemble_frame_3d")
     return out
 
 

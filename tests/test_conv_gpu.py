@@ -172,7 +172,8 @@ def test_distributed_conv_matches_global_conv(case, dev):
     # pass 1: forward of every rank, and the padded dgrad every rank will send from
     cfgs, outs, leaves, gx_need = {}, {}, {}, {}
     for c in mesh_coords(mesh):
-        cfgs[c] = jc.HipConvNdConfig(ns, Bg, TableExchange(fwd_tabs[c], None))
+        # bf16 cases also take the framed forward (only the frame of the padded tile is built)
+        cfgs[c] = jc.HipConvNdConfig(ns, Bg, TableExchange(fwd_tabs[c], None), framed=dtype == torch.bfloat16)
         groups = tuple(jc.TileGroup(mesh[a], c[a]) for a in range(ns))
         xl = tiles[c].clone().requires_grad_()
         wl, bl = Wg.clone().requires_grad_(), Bg.clone().requires_grad_()
@@ -272,3 +273,59 @@ def test_fused_dgrad_fold_declines_what_the_mfma_kernel_does_not_cover(dev):
     w = torch.randn(4, 3, 3, 3, device=dev)
     g = torch.randn(1, 4, 8, 8, device=dev)
     assert jc.conv_nd_input_fold(geom, w, g, padding=(0, 0)) is None
+
+
+FRAMED_CASES = [
+    # size, lo, hi, conv padding on the padded tile, N, channels
+    ((96, 256), (1, 1), (1, 1), (0, 0), 2, 64),
+    ((70, 200), (1, 1), (1, 1), (0, 0), 1, 64),
+    ((40, 330), (1, 0), (1, 0), (0, 1), 1, 32),       # W axis not split: the conv pads it itself
+    ((66, 130), (0, 2), (2, 0), (0, 0), 1, 64),
+    ((4, 40, 140), (1, 1, 1), (1, 1, 1), (0, 0, 0), 1, 32),
+]
+
+
+@pytest.mark.parametrize("case", FRAMED_CASES, ids=lambda c: f"{'x'.join(map(str, c[0]))}_lo{''.join(map(str, c[1]))}_hi{''.join(map(str, c[2]))}")
+def test_framed_conv_has_the_bits_of_the_assembled_tile(case, dev):
+    """Forward and weight gradient that read the own tile directly, plus a frame of the padded
+    tile near the edges, equal the kernels on the fully assembled tile bit for bit; what lies
+    outside the frame is never read (it holds NaN here)."""
+    from jigsaw_amd.halo import HaloGeometry, halo_assemble
+
+    size, lo, hi, pad, N, ch = case
+    ns = len(size)
+    geom = HaloGeometry(size, lo, hi)
+    torch.manual_seed(5)
+    k = (3,) * ns
+    x = torch.randn(N, ch, *size, device=dev).bfloat16()
+    strips = {o: torch.randn(N, ch, *geom.strip_extent(o, "assemble"), device=dev).bfloat16() for o in geom.offsets()}
+    w = ((torch.rand(ch, ch, *k, device=dev) * 2 - 1) / (ch * 3**ns) ** 0.5).bfloat16()
+    b = (torch.randn(ch, device=dev) * 0.1).bfloat16()
+    x_aug = halo_assemble(x, strips, geom)
+    y_ref = jc.conv_nd(x_aug, w, b, padding=pad)
+    g = torch.randn_like(y_ref)
+    gw_ref, gb_ref = jc.conv_nd_weight(x_aug, w.shape, g, padding=pad, with_bias_grad=True)
+
+    bands = jc.frame_bands(x, geom, w.shape, padding=pad)
+    if bands is None:
+        # the framed weight-gradient kernel needs an even padding along W; callers assemble the whole tile then
+        assert pad[-1] % 2 == 1
+        return
+    frame = torch.full_like(x_aug, float("nan"))
+    halo_assemble(x, strips, geom, out=frame, bands=bands)
+    # the frame holds exactly the band cells of the assembled tile
+    inside = torch.ones(geom.padded, dtype=torch.bool, device=dev)
+    for a in range(ns):
+        idx = torch.arange(geom.padded[a], device=dev)
+        in_band = (idx < bands[0][a]) | (idx >= geom.padded[a] - bands[1][a])
+        shape = [1] * ns
+        shape[a] = -1
+        inside &= ~in_band.view(shape)
+    assert torch.equal(frame[..., ~inside].view(torch.int16), x_aug[..., ~inside].view(torch.int16))
+    assert torch.isnan(frame[..., inside]).all()
+
+    y = jc.conv_nd_framed(frame, x, geom, w, b, padding=pad)
+    assert y is not None and torch.equal(y.view(torch.int16), y_ref.view(torch.int16))
+    gw, gb = jc.conv_nd_weight_framed(frame, x, geom, w.shape, g, padding=pad, with_bias_grad=True)
+    assert torch.equal(gw.view(torch.int16), gw_ref.view(torch.int16))
+    assert torch.equal(gb.view(torch.int16), gb_ref.view(torch.int16))
