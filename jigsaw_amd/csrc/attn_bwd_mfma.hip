@@ -90,6 +90,27 @@ __device__ __forceinline__ bf16x8 lds_frag(const unsigned char* p) {
   return __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(p));
 }
 
+// Natural (untransposed) 64 x 64 tiles travel from memory straight into LDS (no registers,
+// no ds_write): a wavefront instruction lands 64 x 16 bytes contiguously, lane order. Rows
+// are 128 bytes, and the 16-byte chunks of a row are XOR-swizzled with (row / 2) % 8 so that
+// the 16 lanes a fragment read serves per cycle hit 16 distinct chunks of the banks.
+constexpr int NAT = BT * D * 2;  // 8192 bytes
+
+// Four of the 8 instructions of a tile: the 256 threads of a half fetch 4 KB per call.
+__device__ __forceinline__ void nat_dma(const uint16_t* tile, unsigned char* lds_tile, int th, int part) {
+  const int w = (th >> 6) + 4 * part;          // instruction 0..7 -> rows 8w .. 8w+7
+  const int i = th & 63;
+  const int row = 8 * w + (i >> 3);
+  const int chunk = (i & 7) ^ ((row >> 1) & 7);
+  __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(tile) + row * (D * 2) + chunk * 16,
+                                   (__attribute__((address_space(3))) void*)(lds_tile + w * 1024), 16, 0, 0);
+}
+
+// fragment of a natural tile: row r (0..63), 16-byte chunk c (0..7)
+__device__ __forceinline__ bf16x8 nat_frag(const unsigned char* nat, int r, int c) {
+  return __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(nat + r * (D * 2) + ((c ^ ((r >> 1) & 7)) << 4)));
+}
+
 __device__ __forceinline__ bf16x8 pack8(const float* e) {
   bf16x8 pk;
 #pragma unroll
@@ -118,9 +139,9 @@ struct BwdArgs {
 };
 
 // ------------------------------------------------------------------ dQ kernel
-constexpr int DQ_BUF = 3 * TILE;            // K natural, K transposed, V natural
+constexpr int DQ_BUF = 2 * NAT + TILE;       // K natural, V natural, K transposed
 constexpr int DQ_HALF = 2 * DQ_BUF;         // double buffered
-constexpr int DQ_LDS = 2 * DQ_HALF;         // 110592
+constexpr int DQ_LDS = 2 * DQ_HALF;         // 102400
 
 __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -161,16 +182,22 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
   }
   const float lse2 = p.lse[qi] * LOG2E;
 
-  Task tk, tv;
-  auto issue_loads = [&](int t) {
-    task_load(tk, kbase + (long long)t * BT * D, g8, cp);
-    task_load(tv, vbase + (long long)t * BT * D, g8, cp);
+  Task tk;
+  // K and V of tile t straight into buffer `buf` (it must be free: the barrier that ended
+  // the iteration before), K once more through registers for the transposed copy
+  auto issue_loads = [&](int t, int buf) {
+    unsigned char* base = lds + buf * DQ_BUF;
+    const uint16_t* kt_g = kbase + (long long)t * BT * D;
+    const uint16_t* vt_g = vbase + (long long)t * BT * D;
+    nat_dma(kt_g, base, th, 0);
+    nat_dma(kt_g, base, th, 1);
+    nat_dma(vt_g, base + NAT, th, 0);
+    nat_dma(vt_g, base + NAT, th, 1);
+    task_load(tk, kt_g, g8, cp);
   };
   auto store_tile = [&](int buf) {
-    unsigned char* base = lds + buf * DQ_BUF;
-    task_store_nat(tk, base, g8, cp);
-    task_store_tr(tk, base + TILE, g8, cp);
-    task_store_nat(tv, base + 2 * TILE, g8, cp);
+    task_store_tr(tk, lds + buf * DQ_BUF + 2 * NAT, g8, cp);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the direct-to-LDS loads of this buffer have landed
   };
 
   f32x16 dq[2];
@@ -179,54 +206,80 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) dq[nb][i] = 0.0f;
 
+  // One 64-key tile. The two 32-key blocks are software pipelined: the score / dP
+  // products of block 1 go to the matrix core one instruction at a time with the
+  // exponentials of block 0 behind them, and the dQ products of a fragment run under
+  // the vector work of the next one. The fences pin that order. dS is kept without the
+  // softmax scale, which multiplies dQ once at the end.
+#define JG_FENCE() __builtin_amdgcn_sched_barrier(0)
   auto compute_tile = [&](int buf) {
     const unsigned char* kn = lds + buf * DQ_BUF;
-    const unsigned char* kt = kn + TILE;
-    const unsigned char* vn = kn + 2 * TILE;
-    bf16x8 dsf[2][2];
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb) {
-      f32x16 s, dp;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        s[i] = 0.0f;
-        dp[i] = 0.0f;
-      }
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const int off = (sb * 32 + ln) * ROWB + (16 * c + 8 * kg) * 2;
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(kn + off), qf[c], s, 0, 0, 0);
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(vn + off), dof[c], dp, 0, 0, 0);
-      }
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        float e[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const float pr = __builtin_amdgcn_exp2f(s[8 * t + i] * c2 - lse2);
-          e[i] = pr * (dp[8 * t + i] - delta) * p.scale;
-        }
-        dsf[sb][t] = pack8(e);
-      }
-    }
+    const unsigned char* vn = kn + NAT;
+    const unsigned char* kt = kn + 2 * NAT;
+    f32x16 s[2], dp[2];
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+      for (int i = 0; i < 16; ++i) {
+        s[sb][i] = 0.0f;
+        dp[sb][i] = 0.0f;
+      }
+    // fragment (sb, t): 8 probabilities -> dS, packed for the dQ product
+    auto ds_frag = [&](int sb, int t) {
+      float e[8];
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb)
-          dq[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              lds_frag(kt + (nb * 32 + ln) * ROWB + (sb * 32 + 16 * t + 8 * kg) * 2), dsf[sb][t],
-              dq[nb], 0, 0, 0);
+      for (int i = 0; i < 8; ++i) {
+        const float pr = __builtin_amdgcn_exp2f(s[sb][8 * t + i] * c2 - lse2);
+        e[i] = pr * (dp[sb][8 * t + i] - delta);
+      }
+      return pack8(e);
+    };
+    auto dq_mfma = [&](int sb, int t, int nb, const bf16x8& f) {
+      dq[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+          lds_frag(kt + (nb * 32 + ln) * ROWB + (sb * 32 + 16 * t + 8 * kg) * 2), f, dq[nb], 0, 0, 0);
+    };
+    // block 0: scores and dP
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nat_frag(kn, ln, 2 * c + kg), qf[c], s[0], 0, 0, 0);
+      dp[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nat_frag(vn, ln, 2 * c + kg), dof[c], dp[0], 0, 0, 0);
+    }
+    JG_FENCE();
+    // block 1 products with the vector work of block 0 behind them
+    bf16x8 f00, f01;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nat_frag(kn, 32 + ln, 2 * c + kg), qf[c], s[1], 0, 0, 0);
+      dp[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nat_frag(vn, 32 + ln, 2 * c + kg), dof[c], dp[1], 0, 0, 0);
+      if (c == 1) f00 = ds_frag(0, 0);
+      if (c == 3) f01 = ds_frag(0, 1);
+      JG_FENCE();
+    }
+    // dQ products of block 0 under the vector work of block 1
+    dq_mfma(0, 0, 0, f00);
+    dq_mfma(0, 0, 1, f00);
+    JG_FENCE();
+    const bf16x8 f10 = ds_frag(1, 0);
+    JG_FENCE();
+    dq_mfma(0, 1, 0, f01);
+    dq_mfma(0, 1, 1, f01);
+    JG_FENCE();
+    const bf16x8 f11 = ds_frag(1, 1);
+    JG_FENCE();
+    dq_mfma(1, 0, 0, f10);
+    dq_mfma(1, 0, 1, f10);
+    dq_mfma(1, 1, 0, f11);
+    dq_mfma(1, 1, 1, f11);
   };
+#undef JG_FENCE
 
   int buf = 0;
-  issue_loads(0);
+  issue_loads(0, 0);
   store_tile(0);
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
     const bool has_next = t + 1 < ntiles;
-    if (has_next) issue_loads(t + 1);
+    if (has_next) issue_loads(t + 1, buf ^ 1);
     compute_tile(buf);
     if (has_next) store_tile(buf ^ 1);
     __syncthreads();
@@ -248,10 +301,10 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       f32x4 val;
-      val.x = dq[nb][4 * j + 0] + xo[(nb * 16 + 4 * j + 0) * 64 + lane];
-      val.y = dq[nb][4 * j + 1] + xo[(nb * 16 + 4 * j + 1) * 64 + lane];
-      val.z = dq[nb][4 * j + 2] + xo[(nb * 16 + 4 * j + 2) * 64 + lane];
-      val.w = dq[nb][4 * j + 3] + xo[(nb * 16 + 4 * j + 3) * 64 + lane];
+      val.x = (dq[nb][4 * j + 0] + xo[(nb * 16 + 4 * j + 0) * 64 + lane]) * p.scale;
+      val.y = (dq[nb][4 * j + 1] + xo[(nb * 16 + 4 * j + 1) * 64 + lane]) * p.scale;
+      val.z = (dq[nb][4 * j + 2] + xo[(nb * 16 + 4 * j + 2) * 64 + lane]) * p.scale;
+      val.w = (dq[nb][4 * j + 3] + xo[(nb * 16 + 4 * j + 3) * 64 + lane]) * p.scale;
       *reinterpret_cast<bf16x4*>(p.dq + qi * D + nb * 32 + 8 * j + 4 * kg) =
           __builtin_convertvector(val, bf16x4);
     }
@@ -260,7 +313,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
 // -------------------------------------------------------------- dK/dV kernel
 constexpr int DKV_STATS = 2 * BT * 4;                 // lse2[64], delta[64] as floats
 constexpr int DKV_HALF = 4 * TILE + DKV_STATS;        // Q nat, Q tr, dO nat, dO tr + stats
-constexpr int DKV_LDS = 2 * DKV_HALF;                 // 74752 (single buffered per half)
+constexpr int DKV_LDS = 4 * DKV_HALF;                 // 149504: two query halves, double buffered
 
 __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -277,12 +330,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
   const float c2 = p.scale * LOG2E;
   const long long ki = b * p.sk + k0 + ln;
 
-  unsigned char* lds = smem + qs * DKV_HALF;
-  unsigned char* qn = lds;
-  unsigned char* qt = lds + TILE;
-  unsigned char* dn = lds + 2 * TILE;
-  unsigned char* dt = lds + 3 * TILE;
-  float* st = reinterpret_cast<float*>(lds + 4 * TILE);  // lse2[64] then delta[64]
+  unsigned char* lds = smem + qs * (2 * DKV_HALF);  // two buffers: Q nat, Q tr, dO nat, dO tr, stats
   const long long qrow0 = b * p.sq + (long long)qs * qhalf;
   const uint16_t* qbase = p.q + qrow0 * D;
   const uint16_t* dbase = p.dout + qrow0 * D;
@@ -306,12 +354,13 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
     if (th < BT) st_reg = p.lse[qrow0 + (long long)t * BT + th] * LOG2E;
     else if (th < 2 * BT) st_reg = p.delta[qrow0 + (long long)t * BT + th - BT];
   };
-  auto store_tile = [&]() {
-    task_store_nat(tq, qn, g8, cp);
-    task_store_tr(tq, qt, g8, cp);
-    task_store_nat(tdo, dn, g8, cp);
-    task_store_tr(tdo, dt, g8, cp);
-    if (th < 2 * BT) st[th] = st_reg;
+  auto store_tile = [&](int buf) {
+    unsigned char* base = lds + buf * DKV_HALF;
+    task_store_nat(tq, base, g8, cp);
+    task_store_tr(tq, base + TILE, g8, cp);
+    task_store_nat(tdo, base + 2 * TILE, g8, cp);
+    task_store_tr(tdo, base + 3 * TILE, g8, cp);
+    if (th < 2 * BT) reinterpret_cast<float*>(base + 4 * TILE)[th] = st_reg;
   };
 
   f32x16 dk[2], dv[2];
@@ -323,7 +372,13 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
       dv[nb][i] = 0.0f;
     }
 
-  auto compute_tile = [&]() {
+  // dS is kept without the softmax scale, which multiplies dK once at the end
+  auto compute_tile = [&](int buf) {
+    const unsigned char* qn = lds + buf * DKV_HALF;
+    const unsigned char* qt = qn + TILE;
+    const unsigned char* dn = qn + 2 * TILE;
+    const unsigned char* dt = qn + 3 * TILE;
+    const float* st = reinterpret_cast<const float*>(qn + 4 * TILE);  // lse2[64] then delta[64]
     bf16x8 pf[2][2], dsf[2][2];
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
@@ -352,7 +407,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
           for (int e = 0; e < 4; ++e) {
             const float pr = __builtin_amdgcn_exp2f(s[4 * j + e] * c2 - l4[e]);
             pe[4 * jj + e] = pr;
-            de[4 * jj + e] = pr * (dp[4 * j + e] - d4[e]) * p.scale;
+            de[4 * jj + e] = pr * (dp[4 * j + e] - d4[e]);
           }
         }
         pf[sb][t] = pack8(pe);
@@ -371,13 +426,17 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
         }
   };
 
+  int buf = 0;
   issue_loads(0);
+  store_tile(0);
+  __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
-    store_tile();
+    const bool has_next = t + 1 < ntiles;
+    if (has_next) issue_loads(t + 1);
+    compute_tile(buf);
+    if (has_next) store_tile(buf ^ 1);
     __syncthreads();
-    if (t + 1 < ntiles) issue_loads(t + 1);
-    compute_tile();
-    __syncthreads();
+    buf ^= 1;
   }
 
   // combine the two query halves, then write dK / dV (lane = key)
@@ -400,7 +459,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
       f32x4 a, c;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        a[e] = dk[nb][4 * j + e] + xo[(nb * 16 + 4 * j + e) * 64 + lane];
+        a[e] = (dk[nb][4 * j + e] + xo[(nb * 16 + 4 * j + e) * 64 + lane]) * p.scale;
         c[e] = dv[nb][4 * j + e] + xo[(32 + nb * 16 + 4 * j + e) * 64 + lane];
       }
       const int col = nb * 32 + 8 * j + 4 * kg;
