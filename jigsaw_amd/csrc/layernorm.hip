@@ -223,20 +223,37 @@ __global__ __launch_bounds__(kThreads) void ln_partial_bwd_kernel(
   }
 }
 
-// Stage 2: one thread per column sums the block partials in block order.
+// Stage 2: a block owns 64 consecutive columns (one per lane, so a partial row is read
+// coalesced); its 4 wavefronts take the block partials k = w, w + 4, ... in 4 independent
+// chains each, and the 16 chain sums are added in a fixed order (deterministic).
 __global__ __launch_bounds__(256) void ln_colreduce_kernel(float* __restrict__ gw,
                                                            float* __restrict__ gb,
                                                            const float* __restrict__ part,
                                                            int nblocks, long long cols) {
-  long long c = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (c >= cols) return;
-  float a = 0.0f, b = 0.0f;
-  for (int k = 0; k < nblocks; ++k) {
-    a += part[((long long)k * 2 + 0) * cols + c];
-    b += part[((long long)k * 2 + 1) * cols + c];
+  __shared__ float red[4][2][64];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const long long c = (long long)blockIdx.x * 64 + lane;
+  float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
+  if (c < cols) {
+    int k = w;
+    for (; k + 12 < nblocks; k += 16) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        a[u] += part[((long long)(k + 4 * u) * 2 + 0) * cols + c];
+        b[u] += part[((long long)(k + 4 * u) * 2 + 1) * cols + c];
+      }
+    }
+    for (; k < nblocks; k += 4) {
+      a[0] += part[((long long)k * 2 + 0) * cols + c];
+      b[0] += part[((long long)k * 2 + 1) * cols + c];
+    }
   }
-  if (gw != nullptr) gw[c] = a;
-  if (gb != nullptr) gb[c] = b;
+  red[w][0][lane] = (a[0] + a[1]) + (a[2] + a[3]);
+  red[w][1][lane] = (b[0] + b[1]) + (b[2] + b[3]);
+  __syncthreads();
+  if (w != 0 || c >= cols) return;
+  if (gw != nullptr) gw[c] = (red[0][0][lane] + red[1][0][lane]) + (red[2][0][lane] + red[3][0][lane]);
+  if (gb != nullptr) gb[c] = (red[0][1][lane] + red[1][1][lane]) + (red[2][1][lane] + red[3][1][lane]);
 }
 
 template <int DT>
@@ -409,7 +426,7 @@ extern "C" int jg_ln_partial_bwd(float* mean_gxn, float* dot_gxn_xhat, float* gw
   if (rc) return rc;
   JG_CHECK_LAUNCH("jg_ln_partial_bwd");
   if (want_cols) {
-    ln_colreduce_kernel<<<jg::cdiv(cols, 256), 256, 0, s>>>(gw, gb, part, bwd_blocks(rows), cols);
+    ln_colreduce_kernel<<<jg::cdiv(cols, 64), 256, 0, s>>>(gw, gb, part, bwd_blocks(rows), cols);
     JG_CHECK_LAUNCH("jg_ln_partial_bwd(colreduce)");
   }
   return JG_OK;
