@@ -107,8 +107,11 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
 
   // contiguous range of stages for this workgroup; stage -> (n, d, column tile, row pair),
   // row pair fastest, so consecutive stages walk down one column strip of one plane
+  // Workgroups are dealt to the 8 XCDs round robin; the ranges are numbered so that one
+  // XCD holds neighbouring column strips, whose x rows share cache lines in that XCD's L2.
+  const unsigned wg_rank = gridDim.x % 8 == 0 ? (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8 : blockIdx.x;
   const long long per = (p.total_stages + gridDim.x - 1) / gridDim.x;
-  const long long s_begin = per * blockIdx.x;
+  const long long s_begin = per * wg_rank;
   long long s_end = s_begin + per;
   if (s_end > p.total_stages) s_end = p.total_stages;
 
