@@ -97,6 +97,7 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
   constexpr int XP_CHUNKS = XC * 2 * X_CPR;   // one pair of x rows
   constexpr int CHUNKS = G_CHUNKS + XP_CHUNKS;
   constexpr int ROUNDS = (CHUNKS + THREADS - 1) / THREADS;
+  static_assert(G_CHUNKS % THREADS == 0, "a load round holds g chunks or x chunks, never both");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   unsigned char* const lds_x = smem + 2 * G_BYTES;
   const int tid = threadIdx.x;
@@ -217,6 +218,9 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
 
   auto issue_loads = [&](Staged& sg, const Cursor& cur, bool want_g, int xpair) {
     u32x4 (&v)[ROUNDS] = sg.v;
+#ifdef JG_EXP_NOLOAD
+    return;
+#endif
     const int hp = cur.hp, ct = cur.ct, od = cur.od, n = cur.n;
     const int oh0 = hp * SR, ow0 = ct * SW;
     const int id0 = od - p.pad_d, ih0 = oh0 - p.pad_h + 2 * xpair, iw0 = ow0 - p.pad_w;
@@ -300,15 +304,17 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
       }
     }
     if (inside) {
+      // Every lane loads in every round it is asked for (the lanes past the last chunk and
+      // those without a tail read offset 0 of the window, which is there): a load under a
+      // per-lane condition merges the register with its old value, and the wait the
+      // compiler puts before such a merge stands behind this stage's loads, which are
+      // still in flight then.
 #pragma unroll
       for (int rd = 0; rd < ROUNDS; ++rd) {
-        const int q = tid + rd * THREADS;
-        if (q < CHUNKS && (want_g || q >= G_CHUNKS)) {
-          const char* org = (q < G_CHUNKS) ? g_org : x_org;
-          v[rd] = *reinterpret_cast<const u32x4_a4*>(org + c_goff[rd]);
-        }
+        const bool g_round = (rd + 1) * THREADS <= G_CHUNKS;  // THREADS divides G_CHUNKS
+        if (want_g || !g_round) v[rd] = *reinterpret_cast<const u32x4_a4*>((g_round ? g_org : x_org) + c_goff[rd]);
       }
-      if (has_tail) sg.tail = *reinterpret_cast<const uint32_t*>(x_org + t_goff);
+      sg.tail = *reinterpret_cast<const uint32_t*>(x_org + t_goff);
     } else {
 #pragma unroll
       for (int rd = 0; rd < ROUNDS; ++rd) {
@@ -397,6 +403,9 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
     const unsigned char* gb = smem + gbuf * G_BYTES + (cb * 32 + ln) * G_CH + kgp * 16;
     const unsigned char* xb = lds_x + (ib * 32 + ln) * X_CH + kgp * 16;
     const int cg = half * (SW / 16 / HALVES) + cgi;  // 16-pixel column group of this wavefront
+#ifdef JG_EXP_NOCOMP
+    return;
+#endif
     bf16x8 a[SR];
 #pragma unroll
     for (int r = 0; r < SR; ++r)
@@ -405,8 +414,12 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
     for (int rho = 0; rho < XR; ++rho) {
       int slot = base + rho;
       if (slot >= RING) slot -= RING;
-      const u32x4 d = *reinterpret_cast<const u32x4*>(xb + slot * X_ROW + cg * 32);
-      const uint32_t d4 = *reinterpret_cast<const uint32_t*>(xb + slot * X_ROW + cg * 32 + 16);
+      u32x4 d = *reinterpret_cast<const u32x4*>(xb + slot * X_ROW + cg * 32);
+      uint32_t d4 = *reinterpret_cast<const uint32_t*>(xb + slot * X_ROW + cg * 32 + 16);
+      // The values are made opaque so that the kw = 2 fragment below is built with register
+      // moves: left alone, the compiler reads it again from LDS at a 4-byte offset, as dword
+      // pairs whose 880-byte lane stride runs into 4-way bank conflicts.
+      asm("" : "+v"(d), "+v"(d4));
       u32x4 s1, s2;
       s1.x = __builtin_amdgcn_alignbit(d.y, d.x, 16);
       s1.y = __builtin_amdgcn_alignbit(d.z, d.y, 16);
