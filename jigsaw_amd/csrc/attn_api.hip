@@ -1,5 +1,7 @@
 // C entry points of the attention core: validate and route to the MFMA flash
 // kernels when they cover the problem, to the generic kernels otherwise.
+#include <initializer_list>
+
 #include "jg_common.h"
 
 namespace jg {
@@ -20,6 +22,14 @@ size_t attn_mfma_bwd_workspace(long long batch, int sq, int sk);
 int attn_mfma_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q, const void* k,
                   const void* v, const void* out, const float* lse, long long batch, int sq,
                   int sk, float scale, void* ws, hipStream_t s);
+bool attn_window_supported(long long batch, int sq, int sk, int d, int dtype);
+int attn_window_fwd(void* out, float* lse, const void* q, const void* k, const void* v,
+                    long long batch, float scale, const float* bias, long long bias_period,
+                    hipStream_t s);
+int attn_window_bwd(void* dq, void* dk, void* dv, float* dbias, const void* dout, const void* q,
+                    const void* k, const void* v, const void* out, const float* lse,
+                    long long batch, float scale, const float* bias, long long bias_period,
+                    hipStream_t s);
 }  // namespace jg
 
 namespace {
@@ -32,6 +42,13 @@ int check_shape(const char* who, int64_t batch, int64_t sq, int64_t sk, int64_t 
   JG_REQUIRE(sq < (1ll << 30) && sk < (1ll << 30), "%s: sequence too long", who);
   JG_REQUIRE(scale > 0.0f, "%s: scale must be positive", who);
   return JG_OK;
+}
+
+// The window kernels move 16 bytes per lane.
+bool aligned16(std::initializer_list<const void*> ptrs) {
+  for (const void* q : ptrs)
+    if ((reinterpret_cast<uintptr_t>(q) & 15) != 0) return false;
+  return true;
 }
 }  // namespace
 
@@ -52,6 +69,9 @@ extern "C" int jg_attn_fwd(void* out, float* lse, const void* q, const void* k, 
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (jg::attn_mfma_fwd_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr))
     return jg::attn_mfma_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, scale, out_acc, lse_acc, s);
+  if (out_acc == nullptr && jg::attn_window_supported(batch, (int)sq, (int)sk, (int)d, dtype) &&
+      aligned16({out, q, k, v, bias}))
+    return jg::attn_window_fwd(out, lse, q, k, v, batch, scale, bias, bias_period, s);
   if (!jg::attn_generic_supported((int)d))
     JG_FAIL(JG_ERR_UNSUPPORTED, "%s: head size %lld not in {8, 16, 32, 64, 128}", who, (long long)d);
   if (out_acc != nullptr)
@@ -91,6 +111,10 @@ extern "C" int jg_attn_bwd(void* dq, void* dk, void* dv, const void* dout, const
       jg::attn_mfma_bwd_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr))
     return jg::attn_mfma_bwd(dq, dk, dv, dout, q, k, v, out, lse, batch, (int)sq, (int)sk, scale,
                              workspace, s);
+  if (jg::attn_window_supported(batch, (int)sq, (int)sk, (int)d, dtype) &&
+      aligned16({dq, dk, dv, dout, q, k, v, out, bias, dbias}))
+    return jg::attn_window_bwd(dq, dk, dv, dbias, dout, q, k, v, out, lse, batch, scale, bias,
+                               bias_period, s);
   if (!jg::attn_generic_supported((int)d))
     JG_FAIL(JG_ERR_UNSUPPORTED, "%s: head size %lld not in {8, 16, 32, 64, 128}", who, (long long)d);
   return jg::attn_generic_bwd(dq, dk, dv, static_cast<float*>(workspace), dbias, dout, q, k, v, out,

@@ -6,7 +6,9 @@ channels-last ``(B, h, w, C)`` tiles of a 2-D token grid; a block is
 LayerNorms run on the sharded-LayerNorm kernels (with a channel group of one), the
 shift / unshift on the DistributedRoll kernels, the windowed attention with its
 relative-position bias and shift mask on the attention core with an additive
-bias. The linear layers are plain ``nn.Linear`` (as in the reference example).
+bias. The linear layers are ``nn.Linear`` parameters (as in the reference example)
+applied through the library GEMMs; only the weight gradient is arranged differently
+(split over the tokens), because its output is a few tiles and its contraction 65536 long.
 """
 
 from __future__ import annotations
@@ -21,6 +23,53 @@ from .attention import window_attention
 from .conv import TileGroup
 from .layernorm import layer_norm
 from .roll import _Roll
+
+
+class _TokenLinear(torch.autograd.Function):
+    """``F.linear`` over ``(tokens, features)`` whose weight gradient is a batched GEMM
+    over chunks of the tokens, summed in fp32. ``dW = dy^T x`` has an output of only
+    ``out x in`` (a handful of GEMM tiles) and a contraction as long as the token count,
+    so a single library GEMM runs on a few compute units; the chunks spread it over the
+    chip. Same arithmetic as ``nn.Linear`` otherwise (examples/swin.py:136-170, 183-190)."""
+
+    CHUNK = 1024  # tokens per partial product
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):  # noqa: D102
+        ctx.dtypes = (x.dtype, weight.dtype, bias.dtype if bias is not None else None)
+        if torch.is_autocast_enabled():
+            dt = torch.get_autocast_dtype("cuda")
+            x, weight = x.to(dt), weight.to(dt)
+            bias = bias.to(dt) if bias is not None else None
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
+        return torch.nn.functional.linear(x, weight, bias)
+
+    @staticmethod
+    def backward(ctx, gy):  # noqa: D102
+        x, weight = ctx.saved_tensors
+        need_x, need_w, need_b = ctx.needs_input_grad
+        gy2 = gy.reshape(-1, gy.shape[-1])
+        x2 = x.reshape(-1, x.shape[-1])
+        dt_x, dt_w, dt_b = ctx.dtypes
+        gy2 = gy2.to(weight.dtype)
+        gx = (gy2 @ weight).view(x.shape).to(dt_x) if need_x else None
+        gw = None
+        if need_w:
+            t = x2.shape[0]
+            chunk = _TokenLinear.CHUNK
+            if t % chunk == 0 and t // chunk > 1:
+                parts = torch.bmm(gy2.view(t // chunk, chunk, -1).transpose(1, 2), x2.view(t // chunk, chunk, -1))
+                gw = parts.sum(0, dtype=torch.float32).to(dt_w)
+            else:
+                gw = (gy2.t() @ x2).to(dt_w)
+        gb = gy2.sum(0, dtype=torch.float32).to(dt_b) if need_b and ctx.has_bias else None
+        return gx, gw, gb
+
+
+def token_linear(x: torch.Tensor, layer: nn.Linear) -> torch.Tensor:
+    """``layer(x)`` with the token-split weight gradient."""
+    return _TokenLinear.apply(x, layer.weight, layer.bias)
 
 
 def windows(x: torch.Tensor, window: int) -> torch.Tensor:
@@ -85,14 +134,14 @@ class WindowAttention(nn.Module):
         b, h, w, c = x.shape
         x = windows(x, self.window)
         n = x.shape[2]
-        qkv = self.qkv(x).view(b, -1, n, 3, self.heads, c // self.heads)
+        qkv = token_linear(x, self.qkv).view(b, -1, n, 3, self.heads, c // self.heads)
         q, k, v = qkv.permute(3, 0, 1, 4, 2, 5).unbind(0)  # (B, nW, heads, N, d)
         bias = self.bias_table[self.index.view(-1)].view(n, n, -1).permute(2, 0, 1).float()
         if self.mask is not None:
             bias = bias[None] + self.mask[:, None]  # (nW, heads, N, N)
         out = window_attention(q.contiguous(), k.contiguous(), v.contiguous(), bias.contiguous())
         out = out.transpose(2, 3).reshape(b, -1, n, c)
-        return unwindows(self.proj(out), h, w, self.window)
+        return unwindows(token_linear(out, self.proj), h, w, self.window)
 
 
 class SwinBlock(nn.Module):
@@ -134,7 +183,8 @@ class SwinBlock(nn.Module):
 
     def finish(self, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
         x = x + y.to(x.dtype)
-        return x + self.mlp(self._norm(self.norm2, x).to(x.dtype))
+        y = token_linear(self._norm(self.norm2, x).to(x.dtype), self.mlp[0])
+        return x + token_linear(self.mlp[1](y), self.mlp[2])
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         y = self.unshift(self.attn(self.shift(self.pre_attention(x))))

@@ -167,6 +167,43 @@ def test_window_attention_with_bias_and_mask(dev):
     assert rel_l2(out_b, want_b) < 2e-2
 
 
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_window_kernels_bf16(with_bias, dev):
+    """64-token windows, head size 32, bf16: the dedicated window kernels (one wavefront
+    per window and head), forward and backward with the bias gradient, against the
+    oracle in fp64 on the same bf16 inputs. 15 entries: the last workgroup is ragged."""
+    torch.manual_seed(11)
+    B, nW, heads, N, d = 1, 5, 3, 64, 32
+    q, k, v = (torch.randn(B, nW, heads, N, d).bfloat16() for _ in range(3))
+    bias = None
+    if with_bias:
+        bias = torch.randn(nW, heads, N, N) * 0.5
+        bias[2, :, :24, 24:] = float("-inf")
+        bias[2, :, 24:, :24] = float("-inf")
+    qd, kd, vd = (t.double().requires_grad_() for t in (q, k, v))
+    bd = bias.double().requires_grad_() if with_bias else None
+    want = oa.window_attention(qd, kd, vd, bd if with_bias else torch.zeros(N, N, dtype=torch.float64))
+    g = torch.randn_like(want).bfloat16()
+    want.backward(g.double())
+    qg, kg, vg = (t.to(dev).requires_grad_() for t in (q, k, v))
+    bg = bias.to(dev).requires_grad_() if with_bias else None
+    out = ja.window_attention(qg, kg, vg, bg)
+    assert out.dtype == torch.bfloat16
+    assert rel_l2(out, want.detach()) < 2e-2
+    out.backward(g.to(dev))
+    assert rel_l2(qg.grad, qd.grad) < 2e-2 and rel_l2(kg.grad, kd.grad) < 2e-2 and rel_l2(vg.grad, vd.grad) < 2e-2
+    if with_bias:
+        assert rel_l2(bg.grad, torch.nan_to_num(bd.grad)) < 2e-2
+        assert (bg.grad[2, :, :24, 24:] == 0).all()
+    # lse of the same call through the core interface
+    out2, lse = ja.core_forward(qg.detach(), kg.detach(), vg.detach(), d ** -0.5, bias=bg.detach() if with_bias else None)
+    s = torch.einsum("bwhqd,bwhkd->bwhqk", q.double(), k.double()) * d ** -0.5
+    if with_bias:
+        s = s + bias.double()
+    assert rel_l2(lse, torch.logsumexp(s, -1)) < 1e-4
+    assert torch.equal(out2, out.detach())
+
+
 def test_core_argument_errors(dev):
     q = torch.zeros(1, 2, 8, 16, device=dev)
     with pytest.raises(NotImplementedError):
