@@ -36,7 +36,7 @@ METRIC = "halo-conv fwd+bwd & ring-attn step TFLOP/s on 1 GPU; % MFMA peak; halo
 
 # HBM bytes per launch of the forward conv kernel (FETCH_SIZE + WRITE_SIZE from
 # rocprofv3 --pmc, scaled by a copy kernel of known size); None until measured.
-CONV_FWD_TRAFFIC_BYTES = 2.41e9  # profiles/conv2d_cfg2_attn_cfg4_hbm_traffic.txt
+CONV_FWD_TRAFFIC_BYTES = 2.32e9
 
 
 def _events():
@@ -96,7 +96,7 @@ def build_conv2_workload(dev, batch=8, ch=64, tile=1024):
             "bands": bands}
 
 
-def conv_step(wl):
+def conv_step(wl, fwd_events=None):
     """The hot path of one rank for one batch (see the module docstring). The backward
     uses the fused forms, each with the bits of the separate steps it replaces: dgrad
     writes the owned cells and the strips it sends in one pass, wgrad adds up the bias
@@ -107,7 +107,13 @@ def conv_step(wl):
     geom, x, w, b, g = wl["geom"], wl["x"], wl["w"], wl["b"], wl["g"]
     halo_pack(x, geom, from_padded=False)  # strips this rank sends
     x_aug = halo_assemble(x, wl["strips_fwd"], geom)
+    if fwd_events is not None:  # HIP events around the forward launch, on its stream
+        e0, e1 = _events()
+        e0.record()
     y = jc.conv_nd(x_aug, w, b)
+    if fwd_events is not None:
+        e1.record()
+        fwd_events.append((e0, e1))
     gx, _send = jc.conv_nd_input_fold(geom, w, g)  # owned cells + halo gradients this rank sends
     gw, gb = jc.conv_nd_weight(x_aug, w.shape, g, with_bias_grad=True)  # one pass over g for both
     halo_fold_border_(gx, wl["strips_bwd"], geom)
@@ -263,12 +269,64 @@ def cpu_baseline(seconds_budget: float = 30.0) -> dict:
     }
 
 
+def conv2_extras(wl, x_aug, it: int, flop_one: int, flop_step: int, ms_fwd: float) -> dict:
+    """Per-operator figures of configuration 2 beside the forward kernel: the separate
+    dgrad / wgrad / fold, the fused forms the step uses, and the framed-input variants."""
+    from jigsaw_amd import conv as jc
+    from jigsaw_amd.halo import halo_assemble, halo_fold
+
+    geom = wl["geom"]
+    tf = lambda ms: flop_one / (ms * 1e-3) / 1e12  # noqa: E731
+    gx_aug = jc.conv_nd_input(x_aug.shape, wl["w"], wl["g"])
+    ms_fwd_loop = time_gpu(lambda: jc.conv_nd(x_aug, wl["w"], wl["b"]), it)  # launched back to back
+    ms_dgrad = time_gpu(lambda: jc.conv_nd_input(x_aug.shape, wl["w"], wl["g"]), it)
+    ms_wgrad = time_gpu(lambda: jc.conv_nd_weight(x_aug, wl["w"].shape, wl["g"]), it)
+    gx_buf = torch.empty_like(wl["x"])
+    ms_asm = time_gpu(lambda: halo_assemble(wl["x"], wl["strips_fwd"], geom, out=x_aug), it)
+    ms_fold = time_gpu(lambda: halo_fold(gx_aug, wl["strips_bwd"], geom, out=gx_buf), it)
+    ms_dgrad_fold = time_gpu(lambda: jc.conv_nd_input_fold(geom, wl["w"], wl["g"]), it)
+    from jigsaw_amd.halo import halo_fold_border_
+
+    ms_border = time_gpu(lambda: halo_fold_border_(gx_buf, wl["strips_bwd"], geom), it)
+    x_frame = halo_assemble(wl["x"], wl["strips_fwd"], geom, bands=wl["bands"])
+    ms_frame = time_gpu(lambda: halo_assemble(wl["x"], wl["strips_fwd"], geom, out=x_frame, bands=wl["bands"]), it)
+    ms_fwd_framed = time_gpu(lambda: jc.conv_nd_framed(x_frame, wl["x"], geom, wl["w"], wl["b"]), it)
+    ms_wgrad_framed = time_gpu(
+        lambda: jc.conv_nd_weight_framed(x_frame, wl["x"], geom, wl["w"].shape, wl["g"], with_bias_grad=True), it
+    )
+    es = wl["x"].element_size()
+    strip_bytes = sum(t.numel() for t in wl["strips_fwd"].values()) * es
+    halo_bytes = (wl["x"].numel() + x_aug.numel()) * es + strip_bytes  # read tile + strips, write padded tile
+    gbps = lambda ms: halo_bytes / (ms * 1e-3) / 1e9  # noqa: E731
+
+    return {
+        "conv_fwd_back_to_back": {"ms": ms_fwd_loop, "tflops": tf(ms_fwd_loop)},
+        "conv_dgrad": {"ms": ms_dgrad, "tflops": tf(ms_dgrad), "frac_mfma_peak": tf(ms_dgrad) / PEAK_BF16_TFLOPS},
+        "conv_wgrad": {"ms": ms_wgrad, "tflops": tf(ms_wgrad), "frac_mfma_peak": tf(ms_wgrad) / PEAK_BF16_TFLOPS},
+        "conv_fwd_bwd_kernels_only": {
+            "ms": ms_fwd + ms_dgrad + ms_wgrad,
+            "tflops": flop_step / ((ms_fwd + ms_dgrad + ms_wgrad) * 1e-3) / 1e12,
+            "frac_mfma_peak": flop_step / ((ms_fwd + ms_dgrad + ms_wgrad) * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+        },
+        "halo_assemble": {"ms": ms_asm, "GBps": gbps(ms_asm), "frac_hbm_peak": gbps(ms_asm) / PEAK_HBM_GBPS, "bytes": halo_bytes},
+        "halo_fold": {"ms": ms_fold, "GBps": gbps(ms_fold), "frac_hbm_peak": gbps(ms_fold) / PEAK_HBM_GBPS, "bytes": halo_bytes},
+        "conv_dgrad_fused_with_pack_and_fold": {"ms": ms_dgrad_fold, "tflops": tf(ms_dgrad_fold)},
+        "halo_fold_border": {"ms": ms_border},
+        "halo_assemble_frame": {"ms": ms_frame},
+        "conv_fwd_framed": {"ms": ms_fwd_framed, "tflops": tf(ms_fwd_framed)},
+        "conv_wgrad_framed_with_bias_grad": {"ms": ms_wgrad_framed, "tflops": tf(ms_wgrad_framed)},
+    }
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="only the timed steps and the roofline kernel (a kernel trace of this run then "
+                    "holds the forward kernel's launches under a name of their own)")
     ns = ap.parse_args()
     if ns.gpus != 1:
         print(
@@ -299,8 +357,9 @@ def main() -> int:
     t0 = time.perf_counter()
     e0, e1 = _events()
     e0.record()
+    fwd_events: list = []
     for _ in range(ns.steps):
-        conv_step(wl)
+        conv_step(wl, fwd_events)
     e1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / ns.steps
@@ -311,30 +370,11 @@ def main() -> int:
     # ---- per-kernel figures (HIP events around repeated launches of one operator)
     geom = wl["geom"]
     x_aug = halo_assemble(wl["x"], wl["strips_fwd"], geom)
-    gx_aug = jc.conv_nd_input(x_aug.shape, wl["w"], wl["g"])
     it = max(5, ns.steps)
-    ms_fwd = time_gpu(lambda: jc.conv_nd(x_aug, wl["w"], wl["b"]), it)
-    ms_dgrad = time_gpu(lambda: jc.conv_nd_input(x_aug.shape, wl["w"], wl["g"]), it)
-    ms_wgrad = time_gpu(lambda: jc.conv_nd_weight(x_aug, wl["w"].shape, wl["g"]), it)
-    gx_buf = torch.empty_like(wl["x"])
-    ms_asm = time_gpu(lambda: halo_assemble(wl["x"], wl["strips_fwd"], geom, out=x_aug), it)
-    ms_fold = time_gpu(lambda: halo_fold(gx_aug, wl["strips_bwd"], geom, out=gx_buf), it)
-    ms_dgrad_fold = time_gpu(lambda: jc.conv_nd_input_fold(geom, wl["w"], wl["g"]), it)
-    from jigsaw_amd.halo import halo_fold_border_
-
-    ms_border = time_gpu(lambda: halo_fold_border_(gx_buf, wl["strips_bwd"], geom), it)
-    x_frame = halo_assemble(wl["x"], wl["strips_fwd"], geom, bands=wl["bands"])
-    ms_frame = time_gpu(lambda: halo_assemble(wl["x"], wl["strips_fwd"], geom, out=x_frame, bands=wl["bands"]), it)
-    ms_fwd_framed = time_gpu(lambda: jc.conv_nd_framed(x_frame, wl["x"], geom, wl["w"], wl["b"]), it)
-    ms_wgrad_framed = time_gpu(
-        lambda: jc.conv_nd_weight_framed(x_frame, wl["x"], geom, wl["w"].shape, wl["g"], with_bias_grad=True), it
-    )
-    es = wl["x"].element_size()
-    strip_bytes = sum(t.numel() for t in wl["strips_fwd"].values()) * es
-    halo_bytes = (wl["x"].numel() + x_aug.numel()) * es + strip_bytes  # read tile + strips, write padded tile
+    # the dominant kernel: average duration of the forward launches of the timed steps
+    # (the 5 us weight re-layout launch that precedes each one is inside the bracket)
+    ms_fwd = sum(a.elapsed_time(b) for a, b in fwd_events) / len(fwd_events)
     tf = lambda ms: flop_one / (ms * 1e-3) / 1e12  # noqa: E731
-    gbps = lambda ms: halo_bytes / (ms * 1e-3) / 1e9  # noqa: E731
-
     roofline = {
         "kernel": "conv3x3_mfma_kernel (forward, config 2)",
         "bound": "mfma",
@@ -344,26 +384,12 @@ def main() -> int:
         "frac": tf(ms_fwd) / PEAK_BF16_TFLOPS,
         "traffic": CONV_FWD_TRAFFIC_BYTES,
     }
-    extra = {
-        "conv_fwd": {"ms": ms_fwd, "tflops": tf(ms_fwd), "frac_mfma_peak": tf(ms_fwd) / PEAK_BF16_TFLOPS},
-        "conv_dgrad": {"ms": ms_dgrad, "tflops": tf(ms_dgrad), "frac_mfma_peak": tf(ms_dgrad) / PEAK_BF16_TFLOPS},
-        "conv_wgrad": {"ms": ms_wgrad, "tflops": tf(ms_wgrad), "frac_mfma_peak": tf(ms_wgrad) / PEAK_BF16_TFLOPS},
-        "conv_fwd_bwd_kernels_only": {
-            "ms": ms_fwd + ms_dgrad + ms_wgrad,
-            "tflops": flop_step / ((ms_fwd + ms_dgrad + ms_wgrad) * 1e-3) / 1e12,
-            "frac_mfma_peak": flop_step / ((ms_fwd + ms_dgrad + ms_wgrad) * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
-        },
-        "halo_assemble": {"ms": ms_asm, "GBps": gbps(ms_asm), "frac_hbm_peak": gbps(ms_asm) / PEAK_HBM_GBPS, "bytes": halo_bytes},
-        "halo_fold": {"ms": ms_fold, "GBps": gbps(ms_fold), "frac_hbm_peak": gbps(ms_fold) / PEAK_HBM_GBPS, "bytes": halo_bytes},
-        "conv_dgrad_fused_with_pack_and_fold": {"ms": ms_dgrad_fold, "tflops": tf(ms_dgrad_fold)},
-        "halo_fold_border": {"ms": ms_border},
-        "halo_assemble_frame": {"ms": ms_frame},
-        "conv_fwd_framed": {"ms": ms_fwd_framed, "tflops": tf(ms_fwd_framed)},
-        "conv_wgrad_framed_with_bias_grad": {"ms": ms_wgrad_framed, "tflops": tf(ms_wgrad_framed)},
-    }
-    extra.update(attention_figures(dev, max(10, it)))
-    extra.update(conv3d_figures(dev, it))
-    extra.update(swin_figures(dev, it))
+    extra = {"conv_fwd": {"ms": ms_fwd, "tflops": tf(ms_fwd), "frac_mfma_peak": tf(ms_fwd) / PEAK_BF16_TFLOPS}}
+    if not ns.no_extras:
+        extra.update(conv2_extras(wl, x_aug, it, flop_one, flop_step, ms_fwd))
+        extra.update(attention_figures(dev, max(10, it)))
+        extra.update(conv3d_figures(dev, it))
+        extra.update(swin_figures(dev, it))
 
     line = {
         "metric": METRIC,
