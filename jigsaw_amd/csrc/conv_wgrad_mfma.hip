@@ -218,9 +218,6 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
 
   auto issue_loads = [&](Staged& sg, const Cursor& cur, bool want_g, int xpair) {
     u32x4 (&v)[ROUNDS] = sg.v;
-#ifdef JG_EXP_NOLOAD
-    return;
-#endif
     const int hp = cur.hp, ct = cur.ct, od = cur.od, n = cur.n;
     const int oh0 = hp * SR, ow0 = ct * SW;
     const int id0 = od - p.pad_d, ih0 = oh0 - p.pad_h + 2 * xpair, iw0 = ow0 - p.pad_w;
@@ -403,9 +400,6 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
     const unsigned char* gb = smem + gbuf * G_BYTES + (cb * 32 + ln) * G_CH + kgp * 16;
     const unsigned char* xb = lds_x + (ib * 32 + ln) * X_CH + kgp * 16;
     const int cg = half * (SW / 16 / HALVES) + cgi;  // 16-pixel column group of this wavefront
-#ifdef JG_EXP_NOCOMP
-    return;
-#endif
     bf16x8 a[SR];
 #pragma unroll
     for (int r = 0; r < SR; ++r)
