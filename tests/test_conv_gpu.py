@@ -329,3 +329,109 @@ def test_framed_conv_has_the_bits_of_the_assembled_tile(case, dev):
     gw, gb = jc.conv_nd_weight_framed(frame, x, geom, w.shape, g, padding=pad, with_bias_grad=True)
     assert torch.equal(gw.view(torch.int16), gw_ref.view(torch.int16))
     assert torch.equal(gb.view(torch.int16), gb_ref.view(torch.int16))
+
+
+def _crop_check(y, x_aug, w, b, windows, what):
+    """Output windows of the full-size result against the oracle on the matching input
+    crops (a k=3, pad-0 conv: output rows h0..h0+H come from input rows h0..h0+H+2)."""
+    ns = y.dim() - 2
+    for n, *org in windows:
+        ext = (32,) * (ns - 1) + (64,)
+        ext = tuple(min(e, y.shape[2 + a] - org[a]) for a, e in enumerate(ext))
+        osl = (n, slice(None)) + tuple(slice(o, o + e) for o, e in zip(org, ext))
+        isl = (slice(n, n + 1), slice(None)) + tuple(slice(o, o + e + 2) for o, e in zip(org, ext))
+        want = oc.forward(x_aug[isl].float().cpu(), w.float().cpu(), None if b is None else b.float().cpu(),
+                          (1,) * ns, (0,) * ns, (1,) * ns)[0]
+        assert rel_l2(y[osl], want) < 2e-2, f"{what}: window {n, *org}"
+
+
+def test_config2_full_size_properties(dev):
+    """Configuration 2 at full size (8 x 64 x 1024^2 bf16, all 8 neighbours live): output
+    windows from the corners, edges and interior of several batch entries against the oracle
+    on the matching crops; the fused backward against the separate steps bit for bit; the
+    weight gradient as the sum of per-entry weight gradients, one of them against the oracle;
+    the bias gradient against the plain sum."""
+    from jigsaw_amd.halo import HaloGeometry, halo_assemble, halo_fold, halo_fold_border_
+
+    torch.manual_seed(0)
+    N, C, T = 8, 64, 1024
+    geom = HaloGeometry((T, T), (1, 1), (1, 1))
+    x = torch.randn(N, C, T, T, device=dev).bfloat16()
+    w = ((torch.rand(C, C, 3, 3, device=dev) * 2 - 1) / 24).bfloat16()
+    b = ((torch.rand(C, device=dev) * 2 - 1) / 24).bfloat16()
+    g = torch.randn(N, C, T, T, device=dev).bfloat16()
+    sf = {o: torch.randn(N, C, *geom.strip_extent(o, "assemble"), device=dev).bfloat16() for o in geom.offsets()}
+    sb = {o: torch.randn(N, C, *geom.strip_extent(o, "fold"), device=dev).bfloat16() for o in geom.offsets()}
+
+    x_aug = halo_assemble(x, sf, geom)
+    y = jc.conv_nd(x_aug, w, b)
+    wins = [(0, 0, 0), (0, 0, T - 64), (3, T - 32, 0), (7, T - 32, T - 64), (5, 496, 480), (2, 16, 960), (6, 1000, 64)]
+    _crop_check(y, x_aug, w, b, wins, "forward")
+
+    # backward: fused == separate, and the padded gradient against the oracle (dgrad of a
+    # k=3 conv is the conv of the zero-padded g with the flipped, transposed weight)
+    gx_aug = jc.conv_nd_input(x_aug.shape, w, g)
+    wt = w.flip(-1, -2).transpose(0, 1).contiguous()
+    g_pad = torch.nn.functional.pad(g, (2, 2, 2, 2))
+    wins_aug = [(0, 0, 0), (1, 0, T + 2 - 64), (4, T + 2 - 32, 0), (7, T + 2 - 32, T + 2 - 64), (3, 500, 500)]
+    _crop_check(gx_aug, g_pad, wt, None, wins_aug, "dgrad")
+    gx_u = halo_fold(gx_aug, sb, geom)
+    send_u = halo_pack(gx_aug, geom, from_padded=True)
+    del gx_aug, g_pad
+    gx_f, send_f = jc.conv_nd_input_fold(geom, w, g)
+    halo_fold_border_(gx_f, sb, geom)
+    assert torch.equal(gx_f.view(torch.int16), gx_u.view(torch.int16))
+    for o in send_u:
+        assert torch.equal(send_f[o].view(torch.int16), send_u[o].view(torch.int16)), f"strip {o}"
+    del gx_u, gx_f
+
+    gw, gb = jc.conv_nd_weight(x_aug, w.shape, g, with_bias_grad=True)
+    parts = [jc.conv_nd_weight(x_aug[n:n + 1], w.shape, g[n:n + 1]).float() for n in range(N)]
+    assert rel_l2(gw, sum(parts)) < 1e-2
+    want1 = oc.wgrad(x_aug[5:6].float().cpu(), w.shape, g[5:6].float().cpu(), (1, 1), (0, 0), (1, 1))
+    assert rel_l2(parts[5], want1) < 2e-2
+    assert rel_l2(gb, g.float().sum((0, 2, 3))) < 1e-2
+
+
+def test_config3_full_size_properties(dev):
+    """Configuration 3 at full size (2 x 32 x 128^3 bf16, 26 neighbours): forward and padded
+    gradient windows against the oracle on crops, the fused backward against the separate
+    steps bit for bit, the weight gradient of one entry against the oracle."""
+    from jigsaw_amd.halo import HaloGeometry, halo_assemble, halo_fold, halo_fold_border_
+
+    torch.manual_seed(1)
+    N, C, T = 2, 32, 128
+    geom = HaloGeometry((T, T, T), (1, 1, 1), (1, 1, 1))
+    x = torch.randn(N, C, T, T, T, device=dev).bfloat16()
+    w = ((torch.rand(C, C, 3, 3, 3, device=dev) * 2 - 1) / 864 ** 0.5).bfloat16()
+    b = ((torch.rand(C, device=dev) * 2 - 1) / 864 ** 0.5).bfloat16()
+    g = torch.randn(N, C, T, T, T, device=dev).bfloat16()
+    sf = {o: torch.randn(N, C, *geom.strip_extent(o, "assemble"), device=dev).bfloat16() for o in geom.offsets()}
+    sb = {o: torch.randn(N, C, *geom.strip_extent(o, "fold"), device=dev).bfloat16() for o in geom.offsets()}
+
+    x_aug = halo_assemble(x, sf, geom)
+    y = jc.conv_nd(x_aug, w, b)
+    wins = [(0, 0, 0, 0), (1, T - 32, T - 32, T - 64), (0, 0, T - 32, 64), (1, 96, 0, 0), (0, 50, 50, 30)]
+    _crop_check(y, x_aug, w, b, wins, "forward")
+
+    gx_aug = jc.conv_nd_input(x_aug.shape, w, g)
+    wt = w.flip(-1, -2, -3).transpose(0, 1).contiguous()
+    g_pad = torch.nn.functional.pad(g, (2,) * 6)
+    wins_aug = [(0, 0, 0, 0), (1, T + 2 - 32, T + 2 - 32, T + 2 - 64), (0, 40, 98, 66), (1, 0, 98, 0)]
+    _crop_check(gx_aug, g_pad, wt, None, wins_aug, "dgrad")
+    gx_u = halo_fold(gx_aug, sb, geom)
+    send_u = halo_pack(gx_aug, geom, from_padded=True)
+    fused = jc.conv_nd_input_fold(geom, w, g)
+    assert fused is not None
+    gx_f, send_f = fused
+    halo_fold_border_(gx_f, sb, geom)
+    assert torch.equal(gx_f.view(torch.int16), gx_u.view(torch.int16))
+    for o in send_u:
+        assert torch.equal(send_f[o].view(torch.int16), send_u[o].view(torch.int16)), f"strip {o}"
+
+    gw, gb = jc.conv_nd_weight(x_aug, w.shape, g, with_bias_grad=True)
+    parts = [jc.conv_nd_weight(x_aug[n:n + 1], w.shape, g[n:n + 1]).float() for n in range(N)]
+    assert rel_l2(gw, sum(parts)) < 1e-2
+    want0 = oc.wgrad(x_aug[0:1].float().cpu(), w.shape, g[0:1].float().cpu(), (1, 1, 1), (0, 0, 0), (1, 1, 1))
+    assert rel_l2(parts[0], want0) < 2e-2
+    assert rel_l2(gb, g.float().sum((0, 2, 3, 4))) < 1e-2
