@@ -135,6 +135,17 @@ __global__ __launch_bounds__(256) void prep_weights_kernel(uint16_t* __restrict_
 // EVEN: Win, pad_w and the plane size are even and x is 4-byte aligned, so every
 // pixel pair of a task is one aligned dword that is either wholly inside or wholly
 // outside the tensor. Otherwise the prefetch falls back to 2-byte loads.
+// 2-byte stores with a scalar base and a 32-bit lane offset. The epilogue issues 128 of
+// them per lane and tile; with the 64-bit lane addresses the compiler builds for plain
+// pointer code each one moves 512 bytes of addresses to the memory pipeline, which is what
+// the epilogue then waits on. `base` must be wave-uniform.
+__device__ inline void store_bf16_lo(const void* base, uint32_t lane_off, uint32_t pair) {
+  asm volatile("global_store_short %0, %1, %2" : : "v"(lane_off), "v"(pair), "s"(base) : "memory");
+}
+__device__ inline void store_bf16_hi(const void* base, uint32_t lane_off, uint32_t pair) {
+  asm volatile("global_store_short_d16_hi %0, %1, %2" : : "v"(lane_off), "v"(pair), "s"(base) : "memory");
+}
+
 template <int MT, bool EVEN, bool FOLD, bool FRAMED>  // MT = produced channels per workgroup: 32 or 64
 __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips, FwdParams p) {
   constexpr int CB = MT / 32;
@@ -401,10 +412,10 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
 #pragma unroll
           for (int i = 0; i < 16; i += 2) {
             f32x2 v2 = {acc[cb][r][i], acc[cb][r][i + 1]};
-            const bf16x2 h2 = __builtin_convertvector(v2, bf16x2);
+            const uint32_t h2 = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
             const int m0 = cb * 32 + 8 * (i >> 2) + (i & 3);
-            *reinterpret_cast<__bf16*>(ybase + (size_t)m0 * ochan * 2 + voff) = h2.x;
-            *reinterpret_cast<__bf16*>(ybase + (size_t)(m0 + 1) * ochan * 2 + voff) = h2.y;
+            store_bf16_lo(ybase + (size_t)m0 * ochan * 2, voff, h2);
+            store_bf16_hi(ybase + (size_t)(m0 + 1) * ochan * 2, voff, h2);
           }
       }
     }
@@ -467,8 +478,8 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
           for (int j = 0; j < 8; ++j) {
             const int m0 = cb * 32 + 8 * (j >> 1) + 2 * (j & 1);
             const uint32_t bits = pk[cb][r][j];
-            *reinterpret_cast<uint16_t*>(ybase + (size_t)m0 * ps * 2 + voff) = (uint16_t)(bits & 0xffffu);
-            *reinterpret_cast<uint16_t*>(ybase + (size_t)(m0 + 1) * ps * 2 + voff) = (uint16_t)(bits >> 16);
+            store_bf16_lo(ybase + (size_t)m0 * ps * 2, voff, bits);
+            store_bf16_hi(ybase + (size_t)(m0 + 1) * ps * 2, voff, bits);
           }
       }
       return;
