@@ -140,16 +140,21 @@ DIST_CASES = [
     ((2, 2), (32, 64), 1, 64, 64, (3, 3), (1, 1), torch.bfloat16),
     ((2, 2, 2), (8, 8, 16), 1, 32, 32, (3, 3, 3), (1, 1, 1), torch.bfloat16),
     ((2, 2, 2), (6, 6, 6), 1, 3, 4, (3, 3, 3), (1, 1, 1), torch.float32),
+    # strided / dilated halos (needed_input_span with s > 1, d > 1): one-sided and 2-wide halos
+    ((2, 2), (8, 12), 2, 4, 6, (3, 3), (1, 1), torch.float32, (2, 2), (1, 1)),
+    ((3, 2), (8, 10), 1, 3, 5, (3, 3), (2, 2), torch.float32, (1, 1), (2, 2)),
+    ((2, 2), (16, 32), 1, 32, 32, (3, 3), (1, 2), torch.bfloat16, (2, 1), (1, 2)),
+    ((2, 1, 2), (4, 6, 8), 1, 2, 3, (3, 3, 3), (1, 1, 2), torch.float32, (2, 1, 1), (1, 1, 2)),
 ]
 
 
-@pytest.mark.parametrize("case", DIST_CASES, ids=lambda c: f"mesh{'x'.join(map(str, c[0]))}_{c[3]}to{c[4]}_{str(c[7]).split('.')[-1]}")
+@pytest.mark.parametrize("case", DIST_CASES, ids=lambda c: f"mesh{'x'.join(map(str, c[0]))}_{c[3]}to{c[4]}_{str(c[7]).split('.')[-1]}" + (f"_s{''.join(map(str, c[8]))}_d{''.join(map(str, c[9]))}" if len(c) > 8 else ""))
 def test_distributed_conv_matches_global_conv(case, dev):
     """The reference's parity method: every rank's y / dx and the summed dw / db equal
     the serial conv on the gathered tensor (test_conv2d_multi_spatial.py:73-233)."""
-    mesh, n, N, cin, cout, k, p, dtype = case
+    mesh, n, N, cin, cout, k, p, dtype = case[:8]
     ns = len(mesh)
-    s, d = (1,) * ns, (1,) * ns
+    s, d = (case[8], case[9]) if len(case) > 8 else ((1,) * ns, (1,) * ns)
     torch.manual_seed(0)
     gshape = tuple(a * b for a, b in zip(n, mesh))
     X = torch.randn(N, cin, *gshape).to(dtype)
@@ -193,7 +198,9 @@ def test_distributed_conv_matches_global_conv(case, dev):
         outs[c].backward(gtiles[c])
         xl, wl, bl = leaves[c]
         sl = (slice(None), slice(None)) + tuple(slice(c[a] * n[a], (c[a] + 1) * n[a]) for a in range(ns))
-        assert rel_l2(outs[c], Y.detach()[sl]) < tol, f"y of rank {c}: {rel_l2(outs[c], Y.detach()[sl]):.3e}"
+        no = tuple(Y.shape[2 + a] // mesh[a] for a in range(ns))  # output rows per rank
+        so = (slice(None), slice(None)) + tuple(slice(c[a] * no[a], (c[a] + 1) * no[a]) for a in range(ns))
+        assert rel_l2(outs[c], Y.detach()[so]) < tol, f"y of rank {c}: {rel_l2(outs[c], Y.detach()[so]):.3e}"
         assert rel_l2(xl.grad, Xd.grad[sl]) < tol, f"dx of rank {c}: {rel_l2(xl.grad, Xd.grad[sl]):.3e}"
         gw_sum += wl.grad.double().cpu()
         gb_sum += bl.grad.double().cpu()
