@@ -187,6 +187,33 @@ def conv3d_figures(dev, iters: int) -> dict:
     return out
 
 
+def groupnorm_figures(dev, iters: int) -> dict:
+    """GroupNorm over a spatially sharded activation of configuration 2's shape
+    (8 x 64 x 1024^2 bf16, 8 groups), one rank's passes: forward = sum, centred squares,
+    normalise + affine (reads x three times, writes y and x_norm); backward = partial
+    sums over g and x_norm, then the input gradient."""
+    from jigsaw_amd import groupnorm as jgn
+
+    g = torch.Generator(device=dev).manual_seed(3)
+    x = torch.randn(8, 64, 1024, 1024, device=dev, generator=g).bfloat16().requires_grad_()
+    w = (1 + 0.1 * torch.randn(64, device=dev, generator=g)).bfloat16().requires_grad_()
+    b = (0.1 * torch.randn(64, device=dev, generator=g)).bfloat16().requires_grad_()
+    gy = torch.randn(8, 64, 1024, 1024, device=dev, generator=g).bfloat16()
+    nbytes = x.numel() * 2
+    ms_fwd = time_gpu(lambda: jgn.group_norm(x.detach(), 8, w.detach(), b.detach(), (), 1e-5), iters)
+
+    def fwd_bwd():
+        x.grad = None
+        jgn.group_norm(x, 8, w, b, (), 1e-5).backward(gy)
+
+    ms_both = time_gpu(fwd_bwd, max(3, iters // 2))
+    ms_bwd = ms_both - ms_fwd
+    return {
+        "groupnorm_fwd": {"ms": ms_fwd, "GBps": 5 * nbytes / (ms_fwd * 1e-3) / 1e9, "bytes": 5 * nbytes},
+        "groupnorm_bwd": {"ms": ms_bwd, "GBps": 5 * nbytes / (ms_bwd * 1e-3) / 1e9, "bytes": 5 * nbytes},
+    }
+
+
 def swin_figures(dev, iters: int) -> dict:
     """Configuration 5: one rank's Swin block on a 256x256-token tile, dim 128, 4 heads,
     8x8 windows, shift 4, bf16 autocast; the roll's cross-tile slabs are seeded."""
@@ -390,6 +417,7 @@ def main() -> int:
         extra.update(attention_figures(dev, max(10, it)))
         extra.update(conv3d_figures(dev, it))
         extra.update(swin_figures(dev, it))
+        extra.update(groupnorm_figures(dev, it))
 
     line = {
         "metric": METRIC,

@@ -195,6 +195,57 @@ int jg_ln_bwd_apply(void* gx, const void* g, const void* x_hat, const void* w,
                     int dtype, void* stream);
 
 /* ------------------------------------------------------------------------- *
+ * GroupNorm over a spatially sharded input (HBM-bound)
+ *
+ * x (batch, channels, spatial) dense, `spatial` = product of the LOCAL spatial
+ * extents; `groups` channel groups of channels / groups consecutive channels,
+ * none of which straddles a channel shard. The sums are the rank's partials:
+ * the caller adds them up over the spatial process groups (one all-reduce of
+ * (count, sum), one of the centred squares; backward one of the two sums),
+ * as _GroupNorm does (jigsaw/modules/normalization/_functional.py:317-468).
+ * workspace: jg_gn_workspace_bytes(batch, channels, spatial) bytes of device
+ * scratch (block partials, added up in a fixed order: deterministic).
+ * ------------------------------------------------------------------------- */
+size_t jg_gn_workspace_bytes(int64_t batch, int64_t channels, int64_t spatial);
+
+/* sum[n][grp] = sum of x over the group's channels and the local positions
+ * (_functional.py:356-359; the count is channels / groups * spatial). */
+int jg_gn_partial_sum(float* sum, const void* x, int64_t batch, int64_t channels,
+                      int64_t spatial, int64_t groups, int dtype, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
+/* sq[n][grp] = sum of (x - mean[n][grp])^2 with the GLOBAL mean: the two-pass
+ * variance of _functional.py:364-366. */
+int jg_gn_partial_sqdev(float* sq, const void* x, const float* mean, int64_t batch,
+                        int64_t channels, int64_t spatial, int64_t groups, int dtype,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* x_norm = (x - mean) * rstd, y = x_norm * weight[c] + bias[c]
+ * (_functional.py:370-381). weight / bias (channels,) in `dtype`, either may be
+ * NULL. mean / rstd fp32 (batch, groups). */
+int jg_gn_apply(void* y, void* x_norm, const void* x, const float* mean, const float* rstd,
+                const void* weight, const void* bias, int64_t batch, int64_t channels,
+                int64_t spatial, int64_t groups, int dtype, void* stream);
+
+/* Backward partials (_functional.py:438-462), one pass over g and x_norm:
+ *   gsum[n][grp]  = sum of g * weight[c]            over the group, local positions
+ *   gxsum[n][grp] = sum of g * weight[c] * x_norm   "
+ *   gw[c] = sum over batch and positions of g * x_norm,  gb[c] = sum of g
+ * gw / gb fp32 (channels,), either may be NULL; weight may be NULL (= 1). */
+int jg_gn_partial_bwd(float* gsum, float* gxsum, float* gw, float* gb, const void* g,
+                      const void* x_norm, const void* weight, int64_t batch,
+                      int64_t channels, int64_t spatial, int64_t groups, int dtype,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
+/* gx = rstd * (g * weight[c] - gsum / count - x_norm * gxsum / count) with the
+ * COMBINED sums and the global element count per (sample, group), fp32
+ * (batch, groups) each (_functional.py:465). */
+int jg_gn_bwd_apply(void* gx, const void* g, const void* x_norm, const void* weight,
+                    const float* rstd, const float* gsum, const float* gxsum,
+                    const float* count, int64_t batch, int64_t channels, int64_t spatial,
+                    int64_t groups, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------- *
  * Online-softmax / log-sum-exp merge of ring attention (HBM-bound)
  * ------------------------------------------------------------------------- */
 

@@ -105,6 +105,30 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int,
          c_void_p],
     ),
+    "jg_gn_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
+    "jg_gn_partial_sum": (
+        c_int,
+        [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p],
+    ),
+    "jg_gn_partial_sqdev": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p],
+    ),
+    "jg_gn_apply": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
+         c_int, c_void_p],
+    ),
+    "jg_gn_partial_bwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
+         c_int, c_void_p, c_size_t, c_void_p],
+    ),
+    "jg_gn_bwd_apply": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+         c_int64, c_int, c_void_p],
+    ),
     "jg_conv_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int, c_int]),
     "jg_conv_fwd": (
         c_int,

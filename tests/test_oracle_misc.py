@@ -178,3 +178,27 @@ def test_kaiming_bound_closed_form():
     torch.nn.init.kaiming_uniform_(w, a=5 ** 0.5)
     bound = kaiming_uniform_bound(64, (3, 3))
     assert w.abs().max() <= bound and w.abs().max() > 0.99 * bound
+
+
+def test_groupnorm_oracle_equals_torch_on_the_undivided_tensor():
+    """The sharded restatement (sums over the shards in place of the all-reduces) against
+    F.group_norm and autograd on the gathered tensor; weight / bias gradients of the
+    shards add up to the global ones."""
+    from oracle import groupnorm as ogn
+
+    torch.manual_seed(12)
+    for shape, G, P, dim in [((2, 8, 6, 10), 4, 2, 2), ((1, 6, 4, 9, 5), 3, 3, 3), ((3, 4, 8), 1, 4, 2)]:
+        X = (torch.randn(*shape, dtype=torch.float64) * 2 + 0.5).requires_grad_()
+        W = (1 + 0.3 * torch.randn(shape[1], dtype=torch.float64)).requires_grad_()
+        B = (0.3 * torch.randn(shape[1], dtype=torch.float64)).requires_grad_()
+        GR = torch.randn(*shape, dtype=torch.float64)
+        Y = torch.nn.functional.group_norm(X, G, W, B, 1e-5)
+        Y.backward(GR)
+        xs, gs = list(X.detach().chunk(P, dim=dim)), list(GR.chunk(P, dim=dim))
+        outs, rstd, n = ogn.forward(xs, G, W.detach(), B.detach(), 1e-5)
+        assert torch.allclose(torch.cat([o[0] for o in outs], dim=dim), Y.detach(), rtol=1e-10, atol=1e-12)
+        assert float(n.flatten()[0]) == X[0].numel() / G
+        back = ogn.backward(gs, [o[1] for o in outs], rstd, n, G, W.detach())
+        assert torch.allclose(torch.cat([b[0] for b in back], dim=dim), X.grad, rtol=1e-9, atol=1e-11)
+        assert torch.allclose(sum(b[1] for b in back), W.grad, rtol=1e-9, atol=1e-11)
+        assert torch.allclose(sum(b[2] for b in back), B.grad, rtol=1e-9, atol=1e-11)
