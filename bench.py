@@ -321,6 +321,20 @@ def conv2_extras(wl, x_aug, it: int, flop_one: int, flop_step: int, ms_fwd: floa
     ms_wgrad_framed = time_gpu(
         lambda: jc.conv_nd_weight_framed(x_frame, wl["x"], geom, wl["w"].shape, wl["g"], with_bias_grad=True), it
     )
+    # transposed convolution of the same shape (k3 s1 p1, 64 -> 64): the mirror image of the
+    # step, on the same kernels (forward = dgrad with the fold epilogue + border fold,
+    # backward = assemble + plain conv + weight gradient with the operands exchanged)
+    def convt_fwd():
+        y_t, _ = jc.conv_nd_input_fold(geom, wl["w"], wl["x"])
+        halo_fold_border_(y_t, wl["strips_bwd"], geom)
+
+    def convt_bwd():
+        g_raw = halo_assemble(wl["g"], wl["strips_fwd"], geom, out=x_aug)
+        jc.conv_nd(g_raw, wl["w"], None)
+        jc.conv_nd_weight(g_raw, wl["w"].shape, wl["x"])
+
+    ms_convt_fwd = time_gpu(convt_fwd, it)
+    ms_convt_bwd = time_gpu(convt_bwd, it)
     es = wl["x"].element_size()
     strip_bytes = sum(t.numel() for t in wl["strips_fwd"].values()) * es
     halo_bytes = (wl["x"].numel() + x_aug.numel()) * es + strip_bytes  # read tile + strips, write padded tile
@@ -342,6 +356,8 @@ def conv2_extras(wl, x_aug, it: int, flop_one: int, flop_step: int, ms_fwd: floa
         "halo_assemble_frame": {"ms": ms_frame},
         "conv_fwd_framed": {"ms": ms_fwd_framed, "tflops": tf(ms_fwd_framed)},
         "conv_wgrad_framed_with_bias_grad": {"ms": ms_wgrad_framed, "tflops": tf(ms_wgrad_framed)},
+        "conv_transpose_fwd": {"ms": ms_convt_fwd, "tflops": tf(ms_convt_fwd)},
+        "conv_transpose_bwd": {"ms": ms_convt_bwd, "tflops": 2 * tf(ms_convt_bwd)},
     }
 
 
