@@ -158,7 +158,7 @@ def conv3d_figures(dev, iters: int) -> dict:
     """Configuration 3: one rank's 128^3 tile of a 256^3 volume, batch 2, 32 -> 32
     channels, 3x3x3, pad 1, bf16; 26 seeded halo strips of width 1."""
     from jigsaw_amd import conv as jc
-    from jigsaw_amd.halo import HaloGeometry, halo_assemble, halo_fold
+    from jigsaw_amd.halo import HaloGeometry, halo_assemble, halo_fold, halo_fold_border_, halo_pack
 
     g = torch.Generator(device=dev).manual_seed(1)
     n, lead, ch = (128, 128, 128), (2, 32), 32
@@ -184,6 +184,13 @@ def conv3d_figures(dev, iters: int) -> dict:
     out = {f"conv3d_{k}": {"ms": v, "tflops": flop / (v * 1e-3) / 1e12, "frac_mfma_peak": flop / (v * 1e-3) / 1e12 / PEAK_BF16_TFLOPS} for k, v in ms.items()}
     out["halo3d_assemble"] = {"ms": ms_asm, "GBps": nbytes / (ms_asm * 1e-3) / 1e9, "frac_hbm_peak": nbytes / (ms_asm * 1e-3) / 1e9 / PEAK_HBM_GBPS}
     out["halo3d_fold"] = {"ms": ms_fold, "GBps": nbytes / (ms_fold * 1e-3) / 1e9, "frac_hbm_peak": nbytes / (ms_fold * 1e-3) / 1e9 / PEAK_HBM_GBPS}
+    # the fused backward the layer runs by default, and its small companions
+    ms_fused = time_gpu(lambda: jc.conv_nd_input_fold(geom, w, gout), iters)
+    ms_border = time_gpu(lambda: halo_fold_border_(gx, sb, geom), iters)
+    ms_pack = time_gpu(lambda: halo_pack(x, geom, from_padded=False), iters)
+    out["conv3d_dgrad_fused_with_pack_and_fold"] = {"ms": ms_fused, "tflops": flop / (ms_fused * 1e-3) / 1e12}
+    out["halo3d_fold_border"] = {"ms": ms_border}
+    out["halo3d_pack"] = {"ms": ms_pack}
     return out
 
 

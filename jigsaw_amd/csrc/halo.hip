@@ -724,42 +724,44 @@ __global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
     if (c >= up0 && s_hi != nullptr) acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(s_hi[c - up0])));
     return Arith<DT>::down(acc);
   };
-  // Vectors [v_first, v_end) hold no column that a W neighbour reaches: `0 + own`, which
-  // only clears the sign of a zero. All the loads of a batch precede its first store.
-  const int v_first = (g.hi[2] + V - 1) / V, v_end = up0 / V;
-  const int n_full = v_end > v_first ? v_end - v_first : 0;
-  for (int it0 = 0; (it0 << pl.lpr_log2) < n_full; it0 += ROW_BATCH) {
+  // Whole 16-byte vectors: `0 + own` for the columns no W neighbour reaches, which only
+  // clears the sign of a zero; the few columns at either end of the row that a neighbour
+  // does reach are patched inside their vector. All the loads of a batch precede its
+  // first store.
+  const int n_vec = W / V;
+  for (int it0 = 0; (it0 << pl.lpr_log2) < n_vec; it0 += ROW_BATCH) {
     u32x4 val[ROW_BATCH];
 #pragma unroll
     for (int u = 0; u < ROW_BATCH; ++u) {
       const int j = lir + ((it0 + u) << pl.lpr_log2);
       val[u] = u32x4{0u, 0u, 0u, 0u};
-      if (j < n_full) val[u] = load16_unaligned<T>(orow + (v_first + j) * V);
+      if (j < n_vec) val[u] = load16_unaligned<T>(orow + j * V);
     }
 #pragma unroll
     for (int u = 0; u < ROW_BATCH; ++u) {
       const int j = lir + ((it0 + u) << pl.lpr_log2);
-      if (j < n_full) {
+      if (j < n_vec) {
         T tmp[V];
         __builtin_memcpy(tmp, &val[u], 16);
+        const int c0 = j * V;
+        if (c0 < g.hi[2] || c0 + V > up0) {
 #pragma unroll
-        for (int e = 0; e < V; ++e)
-          if ((tmp[e] & ABS) == 0) tmp[e] = 0;
+          for (int e = 0; e < V; ++e) tmp[e] = element(c0 + e, tmp[e]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < V; ++e)
+            if ((tmp[e] & ABS) == 0) tmp[e] = 0;
+        }
         u32x4 out;
         __builtin_memcpy(&out, tmp, 16);
-        *reinterpret_cast<u32x4_s4*>(drow + (v_first + j) * V) = out;
+        *reinterpret_cast<u32x4_s4*>(drow + c0) = out;
       }
     }
   }
-  // The columns before and after those vectors, one element per lane.
-  const int head = n_full > 0 ? v_first * V : W;
-  const int tail0 = n_full > 0 ? v_end * V : W;
-  const int n_edge = head + (W - tail0);
-  for (int q = lir; q < n_edge; q += (1 << pl.lpr_log2)) {
-    const int c = q < head ? q : tail0 + (q - head);
-    drow[c] = element(c, orow[c]);
-  }
+  // what is left of a row that is not a whole number of vectors, one element per lane
+  for (int c = n_vec * V + lir; c < W; c += (1 << pl.lpr_log2)) drow[c] = element(c, orow[c]);
 }
+
 
 // In-place second half of a fold: gx already holds `0 + own`; only the cells that a
 // neighbour reaches change. Two kernels: the rows that a D or H neighbour reaches are
