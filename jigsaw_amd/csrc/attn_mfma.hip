@@ -164,17 +164,25 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_mfma_kernel(FwdArgs p) {
   auto new_max = [&](const f32x16 (&s)[2]) {
     // tree over the 32 scores of the lane (short dependency chains), then the lane that
     // shares the query (lane ^ 32) through a register swap instead of an LDS round trip
-    float t8[8];
+    // (three-input maxima: v_max3_f32 halves the instruction count of the tree)
+    auto max3 = [](float a, float b, float c) { return fmaxf(fmaxf(a, b), c); };
+    float t[12];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-      t8[i] = fmaxf(fmaxf(s[0][i], s[0][i + 8]), fmaxf(s[1][i], s[1][i + 8]));
-    float mx = fmaxf(fmaxf(fmaxf(t8[0], t8[1]), fmaxf(t8[2], t8[3])), fmaxf(fmaxf(t8[4], t8[5]), fmaxf(t8[6], t8[7])));
+    for (int i = 0; i < 5; ++i) {
+      t[i] = max3(s[0][3 * i], s[0][3 * i + 1], s[0][3 * i + 2]);
+      t[5 + i] = max3(s[1][3 * i], s[1][3 * i + 1], s[1][3 * i + 2]);
+    }
+    t[10] = s[0][15];
+    t[11] = s[1][15];
+    const float u0 = max3(t[0], t[1], t[2]), u1 = max3(t[3], t[4], t[5]);
+    const float u2 = max3(t[6], t[7], t[8]), u3 = max3(t[9], t[10], t[11]);
+    float mx = fmaxf(max3(u0, u1, u2), u3);
+    float mn;
     {
       const uint32_t bits = __float_as_uint(mx);
       const auto sw = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
-      mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+      mn = max3(__uint_as_float(sw[0]), __uint_as_float(sw[1]), m);
     }
-    const float mn = fmaxf(m, mx);
     if (__builtin_amdgcn_ballot_w64(mn > m) != 0) {
       const float alpha = __builtin_amdgcn_exp2f((m - mn) * c2);
 #pragma unroll
