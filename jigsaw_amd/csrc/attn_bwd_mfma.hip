@@ -351,8 +351,11 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
   auto issue_loads = [&](int t) {
     task_load(tq, qbase + (long long)t * BT * D, g8, cp);
     task_load(tdo, dbase + (long long)t * BT * D, g8, cp);
-    if (th < BT) st_reg = p.lse[qrow0 + (long long)t * BT + th] * LOG2E;
-    else if (th < 2 * BT) st_reg = p.delta[qrow0 + (long long)t * BT + th - BT];
+    // One plain load for every lane, used only when the tile goes to LDS: a load under a
+    // per-lane condition, or arithmetic on its result here, would make the wavefront wait
+    // for it (and for the tile loads issued before it) on the spot.
+    const float* src = th < BT ? p.lse : p.delta;
+    st_reg = src[qrow0 + (long long)t * BT + (th & (BT - 1))];
   };
   auto store_tile = [&](int buf) {
     unsigned char* base = lds + buf * DKV_HALF;
@@ -360,7 +363,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
     task_store_tr(tq, base + TILE, g8, cp);
     task_store_nat(tdo, base + 2 * TILE, g8, cp);
     task_store_tr(tdo, base + 3 * TILE, g8, cp);
-    if (th < 2 * BT) reinterpret_cast<float*>(base + 4 * TILE)[th] = st_reg;
+    if (th < 2 * BT) reinterpret_cast<float*>(base + 4 * TILE)[th] = th < BT ? st_reg * LOG2E : st_reg;
   };
 
   f32x16 dk[2], dv[2];
@@ -429,6 +432,11 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
   int buf = 0;
   issue_loads(0);
   store_tile(0);
+  // The K / V fragments came straight from memory: they are waited for here, once. Left
+  // to the first MFMA that reads them, the wait would sit inside the loop, behind the
+  // tile loads that every iteration has just issued.
+#pragma unroll
+  for (int c = 0; c < 4; ++c) asm volatile("" : "+v"(kf[c]), "+v"(vf[c]));
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
     const bool has_next = t + 1 < ntiles;
