@@ -36,7 +36,7 @@ CORE_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape", CORE_SHAPES, ids=lambda s: "b{}h{}q{}k{}d{}".format(*s))
 def test_core_forward_backward_match_oracle(shape, dtype, dev):
     b, h, sq, sk, d = shape

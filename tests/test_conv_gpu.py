@@ -45,7 +45,7 @@ def _pid(c):
     return "n{}_ci{}_co{}_in{}_k{}_s{}_p{}_d{}".format(c[0], c[1], c[2], *["x".join(map(str, v)) for v in c[3:]])
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("case", PRIM_CASES, ids=_pid)
 def test_conv_primitives_match_oracle(case, dtype, dev):
     N, cin, cout, insp, k, s, p, d = case

@@ -16,7 +16,7 @@ from oracle import groupnorm as ogn
 
 pytestmark = pytest.mark.gpu
 
-TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 4e-3}
 
 
 @pytest.fixture(scope="module")
@@ -47,6 +47,7 @@ CASES = [
     ((1, 4, 256, 300), 2, torch.float32, True, True, 2),       # long spans: several chunks per group and row
     ((3, 16, 8, 8), 16, torch.float32, False, False, 2),       # one channel per group, no affine
     ((2, 32, 32, 48), 4, torch.bfloat16, False, True, 4),
+    ((2, 12, 10, 16), 3, torch.float16, True, True, 2),
 ]
 
 

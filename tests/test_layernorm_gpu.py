@@ -39,7 +39,7 @@ class ShardGroup:
 @pytest.mark.parametrize("rows,cols", [((4, 33), 256), ((2, 5, 7), 96), ((1, 4096), 256), ((3,), 1000), ((9,), 130)])
 def test_partial_stats(rows, cols, dev):
     torch.manual_seed(0)
-    for dtype in (torch.float32, torch.bfloat16):
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
         x = (torch.randn(*rows, cols) * 3 + 1.5).to(dtype)
         m, v = jl.partial_stats(x.to(dev))
         wm, wv = ol.partial_stats(x.double())
