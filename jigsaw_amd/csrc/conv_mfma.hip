@@ -60,7 +60,7 @@ __device__ __forceinline__ int in_slot(int col) { return (col & 7) * OCTS + (col
 struct FwdParams {
   const uint16_t* x;    // (N, C, Din, Hin, Win) bf16: the tensor that is convolved
   const char* x_end;    // one past the last byte of x
-  const u32x4* wprep;   // prepared weights, [m_tile][tap9][c16][kg][MT][8]
+  const u32x4* wprep;   // prepared weights, [m_tile][group][tap9][wc16][kg][MT][8]
   const uint16_t* bias; // (M,) or NULL
   uint16_t* y;          // (N, M, Dout, Hout, Wout)
   int N, C, M;          // batch, channels of x, produced channels
@@ -70,6 +70,8 @@ struct FwdParams {
   int tiles_h, tiles_w;
   int total_tiles;      // N * Dout * tiles_h * tiles_w
   int nc16;             // KD * C / 16
+  int wc16;             // 16-channel steps whose weights sit in LDS at a time (a group)
+  int ngroups;          // ceil(nc16 / wc16); > 1: the weights are reloaded group by group
   // Fold mode (input gradient written to its owners): y is the unpadded tile
   // (N, M, nD, nH, nW); produced cells outside [lo, lo + n) go to the strip of the
   // neighbour that owns them. fold = 0: y is the whole produced tensor.
@@ -99,34 +101,36 @@ __device__ __forceinline__ void* strip_entry(int idx) {
 }
 
 // ---------------------------------------------------------------- weight prep
-// dst[((mt*9 + tap9)*nc16 + c16)*2 + kg][m_local][8 k] (bf16), contraction channel
+// dst[(((mt*ngroups + group)*9 + tap9)*wc16 + c16 in group)*2 + kg][m_local][8 k] (bf16), contraction channel
 // k = kd*C + c. transposed = 0: A[m][k] = w[m][c][kd][kh][kw] (forward, w is
 // (M, C, KD, 3, 3)); transposed = 1: A[m][k] = w[c][m][KD-1-kd][2-kh][2-kw] (input
 // gradient, w is (C, M, KD, 3, 3)).
 __global__ __launch_bounds__(256) void prep_weights_kernel(uint16_t* __restrict__ dst,
                                                            const uint16_t* __restrict__ w,
-                                                           int M, int C, int KD, int MT,
-                                                           int transposed) {
+                                                           int M, int C, int KD, int MT, int mtiles,
+                                                           int wc16, int ngroups, int transposed) {
   const int K = KD * C;
-  const int total = M * K * TAPS;
+  const int total = mtiles * ngroups * TAPS * wc16 * 2 * MT * 8;
   for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
     int e = i & 7;
     int r = i >> 3;
     int ml = r % MT; r /= MT;
     int kg = r & 1; r >>= 1;
-    const int nc16 = K / CK;
-    int c16 = r % nc16; r /= nc16;
-    int tap = r % TAPS;
-    int mt = r / TAPS;
+    int c16l = r % wc16; r /= wc16;
+    int tap = r % TAPS; r /= TAPS;
+    int grp = r % ngroups;
+    int mt = r / ngroups;
     const int m = mt * MT + ml;
-    const int k = c16 * CK + kg * 8 + e;
-    const int kd = k / C, c = k - kd * C;
-    const int kh = tap / KW, kw = tap % KW;
-    uint16_t v;
-    if (!transposed)
-      v = w[((((size_t)m * C + c) * KD + kd) * KH + kh) * KW + kw];
-    else
-      v = w[((((size_t)c * M + m) * KD + (KD - 1 - kd)) * KH + (KH - 1 - kh)) * KW + (KW - 1 - kw)];
+    const int k = (grp * wc16 + c16l) * CK + kg * 8 + e;
+    uint16_t v = 0;  // rows past M and steps past K are padding
+    if (m < M && k < K) {
+      const int kd = k / C, c = k - kd * C;
+      const int kh = tap / KW, kw = tap % KW;
+      if (!transposed)
+        v = w[((((size_t)m * C + c) * KD + kd) * KH + kh) * KW + kw];
+      else
+        v = w[((((size_t)c * M + m) * KD + (KD - 1 - kd)) * KH + (KH - 1 - kh)) * KW + (KW - 1 - kw)];
+    }
     dst[i] = v;
   }
 }
@@ -150,7 +154,7 @@ template <int MT, bool EVEN, bool FOLD, bool FRAMED>  // MT = produced channels 
 __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips, FwdParams p) {
   constexpr int CB = MT / 32;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int w_slots = TAPS * p.nc16 * 2 * MT;  // 16-byte slots of the weight block
+  const int w_slots = TAPS * p.wc16 * 2 * MT;  // 16-byte slots of one group of weights
   u32x4* lds_w = reinterpret_cast<u32x4*>(smem);
   u32x4* lds_in = lds_w + w_slots;  // two stages
   float* lds_bias = reinterpret_cast<float*>(lds_in + 2 * STAGE_SLOTS);
@@ -182,12 +186,16 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     return t_begin + i;
   };
 
-  // ---- resident weights and bias
-  {
-    const u32x4* src = p.wprep + (size_t)mt * w_slots;
+  // ---- weights and bias. With one group the weights stay in LDS for the life of the
+  // workgroup; with more (many input channels) group g is loaded before the stages that
+  // contract its channels.
+  auto load_weights = [&](int grp) {
+    const u32x4* src = p.wprep + ((size_t)mt * p.ngroups + grp) * w_slots;
     for (int i = tid; i < w_slots; i += THREADS) lds_w[i] = src[i];
-    if (tid < MT) lds_bias[tid] = p.bias != nullptr ? jg::bf16_to_f32(p.bias[mt * MT + tid]) : 0.0f;
-  }
+  };
+  if (p.ngroups == 1) load_weights(0);
+  if (tid < MT)
+    lds_bias[tid] = (p.bias != nullptr && mt * MT + tid < p.M) ? jg::bf16_to_f32(p.bias[mt * MT + tid]) : 0.0f;
 
   // ---- prefetch bookkeeping. A task = 8 channels x 8 pixels of one input row.
   const size_t plane = (size_t)p.Hin * p.Win;
@@ -346,13 +354,13 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
   // One third (one kw) of a stage's MFMAs.
   auto compute_kw = [&](int buf, int c16, int kw) {
     const u32x4* in = lds_in + buf * STAGE_SLOTS + kg * (IN_ROWS * ROW_SLOTS);
-    const u32x4* wt = lds_w + ((size_t)c16 * 2 + kg) * MT + ln;
+    const u32x4* wt = lds_w + ((size_t)(c16 % p.wc16) * 2 + kg) * MT + ln;
     bf16x8 a[KH][CB];
 #pragma unroll
     for (int kh = 0; kh < KH; ++kh)
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb) {
-        u32x4 t = wt[(size_t)(kh * KW + kw) * p.nc16 * 2 * MT + cb * 32];
+        u32x4 t = wt[(size_t)(kh * KW + kw) * p.wc16 * 2 * MT + cb * 32];
         a[kh][cb] = __builtin_bit_cast(bf16x8, t);
       }
     const u32x4* inb = in + wrow0 * ROW_SLOTS + in_slot(wcol0 + ln + kw);
@@ -397,11 +405,15 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
 
   const size_t plane_o = (size_t)p.Hout * p.Wout;
   const size_t ochan = plane_o * p.Dout;  // elements between produced channels
-  auto epilogue = [&](int tile) {
+  // RAGGED: the last tile of produced channels when M is not a multiple of MT (its weight
+  // rows past M are zero padding); a lane then stores only the channels that exist.
+  auto epilogue_rows = [&](int tile, auto ragged) {
+    constexpr bool RAGGED = decltype(ragged)::value;
     const TileCoord tc = coord(tile);
     const int ow = tc.tw * TW + wcol0 + ln;
     char* ybase = reinterpret_cast<char*>(p.y) +
                   2 * (((size_t)tc.n * p.M + (size_t)mt * MT) * ochan + (size_t)tc.od * plane_o);
+    const int m_left = p.M - mt * MT - 4 * kg;  // channels from this lane's first one to the end
 #pragma unroll
     for (int r = 0; r < WROWS; ++r) {
       const int oh = tc.th * TH + wrow0 + r;
@@ -414,11 +426,15 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
             f32x2 v2 = {acc[cb][r][i], acc[cb][r][i + 1]};
             const uint32_t h2 = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
             const int m0 = cb * 32 + 8 * (i >> 2) + (i & 3);
-            store_bf16_lo(ybase + (size_t)m0 * ochan * 2, voff, h2);
-            store_bf16_hi(ybase + (size_t)(m0 + 1) * ochan * 2, voff, h2);
+            if (!RAGGED || m0 < m_left) store_bf16_lo(ybase + (size_t)m0 * ochan * 2, voff, h2);
+            if (!RAGGED || m0 + 1 < m_left) store_bf16_hi(ybase + (size_t)(m0 + 1) * ochan * 2, voff, h2);
           }
       }
     }
+  };
+  auto epilogue = [&](int tile) {
+    if ((mt + 1) * MT <= p.M) epilogue_rows(tile, std::false_type{});
+    else epilogue_rows(tile, std::true_type{});
   };
 
   // Fold-mode epilogue: a produced cell goes to the unpadded tile when it lies inside
@@ -532,6 +548,11 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
   for (int ti = 0; ti < my_tiles; ++ti) {
     init_acc();
     for (int c16 = 0; c16 < p.nc16; ++c16, ++q) {
+      if (p.ngroups > 1 && c16 % p.wc16 == 0) {
+        // every wavefront is past the barrier that closed the last stage of the group before
+        load_weights(c16 / p.wc16);
+        __syncthreads();
+      }
       compute_kw(buf, c16, 0);
       compute_kw(buf, c16, 1);
       if (q + 1 < stages) store_stage(buf ^ 1);  // other buffer: no hazard with this stage's reads
@@ -557,6 +578,32 @@ int cu_count() {
   return n;
 }
 
+// How a problem maps onto the kernel: produced channels in tiles of MT (M padded up to a
+// multiple of 32 with zero weight rows), contraction steps of 16 channels in groups of wc16
+// steps whose weights fit LDS beside the two input stages.
+struct Layout {
+  int MT, mtiles, nc16, wc16, ngroups;
+  size_t prep_bytes, lds_bytes;
+};
+
+Layout layout_of(int K, int M) {
+  Layout L;
+  const int mpad = (M + 31) / 32 * 32;
+  L.MT = (mpad % 64 == 0) ? 64 : 32;
+  L.mtiles = mpad / L.MT;
+  L.nc16 = K / CK;
+  const size_t budget = 160 * 1024 - 2 * (size_t)STAGE_BYTES - L.MT * 4;
+  int cap = (int)(budget / ((size_t)TAPS * 2 * L.MT * 16));
+  if (cap < 1) cap = 1;
+  L.wc16 = L.nc16 < cap ? L.nc16 : cap;
+  if (L.wc16 < 1) L.wc16 = 1;
+  L.ngroups = (L.nc16 + L.wc16 - 1) / L.wc16;
+  const size_t slots = (size_t)TAPS * L.wc16 * 2 * L.MT;
+  L.prep_bytes = (size_t)L.mtiles * L.ngroups * slots * 16;
+  L.lds_bytes = slots * 16 + 2 * (size_t)STAGE_BYTES + L.MT * 4;
+  return L;
+}
+
 // C = channels of the convolved tensor, M = produced channels
 bool shape_ok(int C, int M, const ConvGeom& g) {
   if (g.k[1] != KH || g.k[2] != KW) return false;
@@ -564,18 +611,14 @@ bool shape_ok(int C, int M, const ConvGeom& g) {
   if (g.k[0] == 1 && (g.in[0] != 1 || g.p[0] != 0)) return false;
   for (int a = 0; a < 3; ++a)
     if (g.s[a] != 1 || g.d[a] != 1) return false;
-  if (C % CK != 0 || M % 32 != 0) return false;
-  const int MT = (M % 64 == 0) ? 64 : 32;
-  const int K = g.k[0] * C;
-  const size_t lds = (size_t)TAPS * (K / CK) * 2 * MT * 16 + 2 * (size_t)STAGE_BYTES + MT * 4;
-  if (lds > 160 * 1024) return false;
+  if (C % CK != 0 || C <= 0 || M <= 0) return false;
   // per-lane byte offsets inside one batch entry are 32-bit
   const size_t in_sz = (size_t)g.in[0] * g.in[1] * g.in[2], out_sz = (size_t)g.out[0] * g.out[1] * g.out[2];
   const size_t big = in_sz > out_sz ? in_sz : out_sz;
   return big * 2 * 72 < (1ull << 31);
 }
 
-size_t prep_bytes(int K, int M) { return (size_t)K * M * TAPS * sizeof(uint16_t); }
+size_t prep_bytes(int K, int M) { return layout_of(K, M).prep_bytes; }
 
 struct Launch {
   const uint16_t* x;
@@ -599,11 +642,13 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
     JG_FAIL(JG_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, prep_bytes(K, L.M));
   JG_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 15) == 0, "%s: workspace must be 16-byte aligned",
              who);
-  const int MT = (L.M % 64 == 0) ? 64 : 32;
+  const Layout lay = layout_of(K, L.M);
+  const int MT = lay.MT;
   uint16_t* wprep = static_cast<uint16_t*>(ws);
-  const int total_w = L.M * K * TAPS;
-  prep_weights_kernel<<<(total_w + 255) / 256, 256, 0, s>>>(wprep, L.w, L.M, L.C, L.KD, MT,
-                                                            L.transposed);
+  const size_t total_w = lay.prep_bytes / 2;
+  JG_REQUIRE(total_w < (1ull << 31), "%s: weight tensor too large", who);
+  prep_weights_kernel<<<(unsigned)((total_w + 255) / 256), 256, 0, s>>>(wprep, L.w, L.M, L.C, L.KD, MT, lay.mtiles,
+                                                                         lay.wc16, lay.ngroups, L.transposed);
   JG_CHECK_LAUNCH(who);
 
   FwdParams p;
@@ -618,7 +663,9 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   const long long tiles = (long long)L.N * L.Dout * p.tiles_h * p.tiles_w;
   JG_REQUIRE(tiles < (1ll << 30), "%s: too many tiles", who);
   p.total_tiles = (int)tiles;
-  p.nc16 = K / CK;
+  p.nc16 = lay.nc16;
+  p.wc16 = lay.wc16;
+  p.ngroups = lay.ngroups;
   p.fold = L.fold;
   p.lo_d = L.lo[0]; p.lo_h = L.lo[1]; p.lo_w = L.lo[2];
   p.nD = L.n[0]; p.nH = L.n[1]; p.nW = L.n[2];
@@ -628,11 +675,11 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   StripTable tab;
   for (int i = 0; i < 27; ++i) tab.p[i] = (L.fold && L.strips != nullptr) ? L.strips[i] : nullptr;
   if (tiles == 0) return JG_OK;
-  const size_t lds = (size_t)TAPS * p.nc16 * 2 * MT * 16 + 2 * (size_t)STAGE_BYTES + MT * 4;
+  const size_t lds = lay.lds_bytes;
   int wgs = cu_count();
   if (wgs > tiles) wgs = (int)tiles;
   wgs = (wgs + 7) & ~7;  // whole XCD rounds
-  dim3 grid((unsigned)wgs, (unsigned)(L.M / MT), 1);
+  dim3 grid((unsigned)wgs, (unsigned)lay.mtiles, 1);
   const bool even = (L.Win % 2 == 0) && (L.pad_w % 2 == 0) &&
                     ((reinterpret_cast<uintptr_t>(L.x) & 3) == 0);
   void (*kern)(StripTable, FwdParams) = nullptr;
@@ -774,6 +821,10 @@ int mfma_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, void*
 
 int mfma_dgrad_fold(void* gx, void* const strips[27], const int lo[3], const int n[3], const void* w,
                     const void* go, const ConvGeom& g, void* ws, size_t ws_bytes, hipStream_t s) {
+  // the fold epilogue has no path for a ragged last tile of produced channels
+  const Layout lay = layout_of(g.k[0] * g.cout, g.cin);
+  if (lay.mtiles * lay.MT != g.cin)
+    JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_dgrad_fold(mfma): %d input channels are not a multiple of %d", g.cin, lay.MT);
   return dgrad_launch(gx, strips, lo, n, w, go, g, ws, ws_bytes, s, "jg_conv_dgrad_fold(mfma)");
 }
 

@@ -64,7 +64,9 @@ struct WgradParams {
   // A row pair whose window lies inside the tile is read from xt. NULL: all from x.
   const uint16_t* xt;
   int tlo_d, tlo_h, tlo_w, tn_d, tn_h, tn_w;
-  int Cin, Cout;
+  int Cin, Cout;            // channels of the block this launch works on (32 or 64 a side)
+  int cin_valid, cout_valid;  // how many of them exist; the others repeat the last one and are dropped
+  int cin_total, cout_total;  // channels of the tensors (batch strides); x and g point at the block's first
   int Din, Hin, Win, Dout, Hout, Wout;
   int pad_d, pad_h, pad_w;
   int row_pairs, col_tiles;
@@ -129,14 +131,16 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
     const int q = tid + rd * THREADS;
     if (q < G_CHUNKS) {
       const int c8 = q & 7, r = (q >> 3) % SR, ch = q / (8 * SR);
-      c_goff[rd] = (uint32_t)((ch * g_cs + (size_t)r * p.Wout + c8 * 8) * 2);
+      const int che = ch < p.cout_valid ? ch : p.cout_valid - 1;  // a channel past the last one reads the last
+      c_goff[rd] = (uint32_t)((che * g_cs + (size_t)r * p.Wout + c8 * 8) * 2);
       c_lds[rd] = (uint32_t)(ch * G_CH + r * (SW * 2) + c8 * 16);
     } else if (q < CHUNKS) {
       const int qx = q - G_CHUNKS;
       const int c8 = qx % X_CPR;
       const int rr = qx / X_CPR;
       const int r2 = rr & 1, ch = rr >> 1;      // ch = kd * Cin + ci
-      const int kd = ch / p.Cin, ci = ch - kd * p.Cin;
+      const int kd = ch / p.Cin, cib = ch - kd * p.Cin;
+      const int ci = cib < p.cin_valid ? cib : p.cin_valid - 1;
       c_goff[rd] = (uint32_t)((ci * x_cs + kd * plane_x + (size_t)r2 * p.Win + c8 * 8) * 2);
       c_lds[rd] = (uint32_t)(ch * X_CH + c8 * 16);
       x_second |= (uint32_t)r2 << rd;
@@ -150,7 +154,8 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
   uint32_t t_goff = 0, t_lds = 0;
   if (has_tail) {
     const int r2 = tid & 1, ch = tid >> 1;
-    const int kd = ch / p.Cin, ci = ch - kd * p.Cin;
+    const int kd = ch / p.Cin, cib = ch - kd * p.Cin;
+    const int ci = cib < p.cin_valid ? cib : p.cin_valid - 1;
     t_goff = (uint32_t)((ci * x_cs + kd * plane_x + (size_t)r2 * p.Win + SW) * 2);
     t_lds = (uint32_t)(ch * X_CH + SW * 2);
   }
@@ -222,9 +227,9 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
     const int oh0 = hp * SR, ow0 = ct * SW;
     const int id0 = od - p.pad_d, ih0 = oh0 - p.pad_h + 2 * xpair, iw0 = ow0 - p.pad_w;
     const char* g_org = reinterpret_cast<const char*>(p.g) +
-                        2 * (((size_t)n * p.Cout * p.Dout + od) * plane_g + (size_t)oh0 * p.Wout + ow0);
+                        2 * (((size_t)n * p.cout_total * p.Dout + od) * plane_g + (size_t)oh0 * p.Wout + ow0);
     const char* x_org = reinterpret_cast<const char*>(p.x) +
-                        2 * ((ptrdiff_t)((size_t)n * p.Cin * p.Din * plane_x) + (ptrdiff_t)id0 * (ptrdiff_t)plane_x +
+                        2 * ((ptrdiff_t)((size_t)n * p.cin_total * p.Din * plane_x) + (ptrdiff_t)id0 * (ptrdiff_t)plane_x +
                              (ptrdiff_t)ih0 * p.Win + iw0);
     const bool inside = EVEN && oh0 + SR <= p.Hout && ow0 + SW <= p.Wout && ih0 >= 0 &&
                         ih0 + 2 <= p.Hin && iw0 >= 0 && iw0 + SW + 2 <= p.Win && id0 >= 0 &&
@@ -237,7 +242,7 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
       const int dt = id0 - p.tlo_d, ht = ih0 - p.tlo_h, wt = iw0 - p.tlo_w;
       if (ht >= 0 && ht + 2 <= p.tn_h && wt >= 0 && wt + SW + 2 <= p.tn_w) {
         const char* t_org = reinterpret_cast<const char*>(p.xt) +
-                            2 * ((ptrdiff_t)((size_t)n * p.Cin * t_cs) + (ptrdiff_t)dt * (ptrdiff_t)plane_t +
+                            2 * ((ptrdiff_t)((size_t)n * p.cin_total * t_cs) + (ptrdiff_t)dt * (ptrdiff_t)plane_t +
                                  (ptrdiff_t)ht * p.tn_w + wt);
         // 4-byte aligned accesses only (2-byte aligned vector loads run at a fraction of the
         // rate): a window that starts on an odd column is read one pixel early and shifted.
@@ -509,13 +514,13 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
 }
 
 // gb[co] (bf16) = sum over the workgroups of bias_part[wg][co]; one wavefront per channel,
-// fixed order.
+// fixed order. GC = channels per partial row, `valid` of them exist.
 __global__ __launch_bounds__(256) void wgrad_bias_reduce_kernel(uint16_t* __restrict__ gb,
                                                                 const float* __restrict__ part,
-                                                                int wgs, int GC) {
+                                                                int wgs, int GC, int valid) {
   const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
-  if (c >= GC) return;
+  if (c >= valid) return;
   float s = 0.0f;
   for (int k = lane; k < wgs; k += 64) s += part[(size_t)k * GC + c];
 #pragma unroll
@@ -523,13 +528,16 @@ __global__ __launch_bounds__(256) void wgrad_bias_reduce_kernel(uint16_t* __rest
   if (lane == 0) gb[c] = jg::f32_to_bf16(s);
 }
 
-// gw[co][ci][kd][kh][kw] (bf16) = sum over the slots of part[slot][tap9][co][kd*Cin+ci].
+// gw[co0 + co][ci0 + ci][kd][kh][kw] (bf16) = sum over the slots of
+// part[slot][tap9][co][kd*CinB+ci] for the channels of the block that exist (gw points at
+// the block's first element, cin_total is the channel count of the whole weight tensor).
 // A block owns 64 consecutive outputs (one per lane, so a slot row is read coalesced);
 // its 4 wavefronts take the slots s = w, w + 4, ... in 4 independent chains each, and the
 // 16 chain sums are added in a fixed order (deterministic).
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(uint16_t* __restrict__ gw,
                                                            const float* __restrict__ part,
-                                                           int slots, int GC, int XC, int Cin) {
+                                                           int slots, int GC, int XC, int CinB,
+                                                           int cout_valid, int cin_valid, int cin_total) {
   __shared__ float red[4][64];
   const int count = 9 * GC * XC;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -550,8 +558,9 @@ __global__ __launch_bounds__(256) void wgrad_reduce_kernel(uint16_t* __restrict_
   if (w != 0 || i >= count) return;
   const float s = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
   const int cx = i % XC, co = (i / XC) % GC, tap = i / (XC * GC);
-  const int kd = cx / Cin, ci = cx % Cin, KD = XC / Cin;
-  gw[(((size_t)co * Cin + ci) * KD + kd) * 9 + tap] = jg::f32_to_bf16(s);
+  const int kd = cx / CinB, ci = cx % CinB, KD = XC / CinB;
+  if (co >= cout_valid || ci >= cin_valid) return;
+  gw[(((size_t)co * cin_total + ci) * KD + kd) * 9 + tap] = jg::f32_to_bf16(s);
 }
 
 int cu_count() {
@@ -577,21 +586,34 @@ long long stage_count(const ConvGeom& g) {
 }
 
 // (CGB, CXB) of a geometry, or false when the kernel does not cover it
-bool blocks_of(const ConvGeom& g, int* cgb, int* cxb) {
+// Channel blocking. One launch accumulates a block of `cob` output x `cib` input channels
+// (32 or 64 each; with a depth kernel of 3 always 32 x 32, so that the x side spans 96);
+// more channels are covered block by block, a last block with fewer channels than its
+// width re-reads its last channel and its extra rows and columns are dropped.
+struct Blocking {
+  int cob, cib;  // width of the first (largest) block
+  int KD;
+};
+bool blocks_of(const ConvGeom& g, Blocking* b) {
   if (g.k[1] != 3 || g.k[2] != 3 || (g.k[0] != 1 && g.k[0] != 3)) return false;
   if (g.k[0] == 1 && g.in[0] != 1) return false;
   for (int a = 0; a < 3; ++a)
     if (g.s[a] != 1 || g.d[a] != 1) return false;
-  if (g.cin != 32 && g.cin != 64) return false;
-  if (g.cout != 32 && g.cout != 64) return false;
-  *cgb = g.cout / 32;
-  *cxb = g.k[0] * g.cin / 32;
-  if (*cgb * *cxb > 4) return false;
+  if (g.cin <= 0 || g.cout <= 0) return false;
+  b->KD = g.k[0];
+  if (b->KD == 3) {
+    b->cob = 32; b->cib = 32;
+  } else {
+    b->cob = g.cout > 32 ? 64 : 32;
+    b->cib = g.cin > 32 ? 64 : 32;
+  }
   // per-lane byte offsets inside one batch entry are 32-bit
   const size_t xs = (size_t)g.cin * g.in[0] * g.in[1] * g.in[2] * 2;
   const size_t gs = (size_t)g.cout * g.out[0] * g.out[1] * g.out[2] * 2;
   return xs < (1ull << 31) && gs < (1ull << 31);
 }
+// width of the block that starts at channel c0 of `total`
+int block_width(int total, int c0, int first) { return (first == 64 && total - c0 > 32) ? 64 : 32; }
 
 template <int CGB, int CXB>
 int launch(const WgradParams& p, bool even, int wgs, hipStream_t s, const char* who) {
@@ -614,16 +636,16 @@ int launch(const WgradParams& p, bool even, int wgs, hipStream_t s, const char* 
 namespace jg {
 
 bool mfma_wgrad_supported(const ConvGeom& g, int dtype) {
-  int cgb, cxb;
+  Blocking b;
   if (dtype != JG_BF16 || g.batch <= 0) return false;
-  return blocks_of(g, &cgb, &cxb);
+  return blocks_of(g, &b);
 }
 
 size_t mfma_wgrad_workspace(const ConvGeom& g) {
-  int cgb = 1, cxb = 1;
-  blocks_of(g, &cgb, &cxb);
+  Blocking b{32, 32, 1};
+  blocks_of(g, &b);
   const size_t wgs = (size_t)wg_count(stage_count(g));
-  return wgs * HALVES * 9 * (32 * cgb) * (32 * cxb) * sizeof(float) + wgs * (32 * cgb) * sizeof(float);
+  return wgs * HALVES * 9 * b.cob * (b.KD * b.cib) * sizeof(float) + wgs * b.cob * sizeof(float);
 }
 
 // Whether the framed weight-gradient kernel covers a geometry: even row lengths (its
@@ -631,6 +653,8 @@ size_t mfma_wgrad_workspace(const ConvGeom& g) {
 // inside the bands that the frame holds.
 bool mfma_wgrad_frame_ok(const ConvGeom& g, const int tlo[3], const int tn[3]) {
   if (g.in[2] % 2 != 0 || g.p[2] % 2 != 0 || g.out[2] % 2 != 0 || tn[2] % 2 != 0) return false;
+  Blocking b;  // the framed input is read by a single block of exactly its width
+  if (!blocks_of(g, &b) || g.cin != b.cib || g.cout != b.cob) return false;
   int blo[3], bhi[3];
   mfma_frame_bands(g, tlo, tn, blo, bhi);
   const int row_pairs = (g.out[1] + SR - 1) / SR, col_tiles = (g.out[2] + SW - 1) / SW;
@@ -654,19 +678,23 @@ bool mfma_wgrad_frame_ok(const ConvGeom& g, const int tlo[3], const int tn[3]) {
 int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom& g, void* ws,
                size_t ws_bytes, hipStream_t s, const void* xt, const int* tlo, const int* tn) {
   const char* who = "jg_conv_wgrad(mfma)";
-  int cgb, cxb;
-  if (!blocks_of(g, &cgb, &cxb)) JG_FAIL(JG_ERR_UNSUPPORTED, "%s: geometry not covered", who);
+  Blocking bl;
+  if (!blocks_of(g, &bl)) JG_FAIL(JG_ERR_UNSUPPORTED, "%s: geometry not covered", who);
   if (ws == nullptr || ws_bytes < mfma_wgrad_workspace(g))
     JG_FAIL(JG_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes,
             mfma_wgrad_workspace(g));
   JG_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 15) == 0, "%s: workspace must be 16-byte aligned",
              who);
+  const bool even = (g.in[2] % 2 == 0) && (g.p[2] % 2 == 0) && (g.out[2] % 2 == 0) &&
+                    ((reinterpret_cast<uintptr_t>(x) & 3) == 0) &&
+                    ((reinterpret_cast<uintptr_t>(go) & 3) == 0);
+  if (xt != nullptr && (!even || !mfma_wgrad_frame_ok(g, tlo, tn)))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: the framed input does not cover this geometry / alignment", who);
+  const size_t x_cs = (size_t)g.in[0] * g.in[1] * g.in[2], g_cs = (size_t)g.out[0] * g.out[1] * g.out[2];
   WgradParams p;
-  p.x = static_cast<const uint16_t*>(x);
-  p.g = static_cast<const uint16_t*>(go);
   p.part = static_cast<float*>(ws);
-  p.x_end = static_cast<const char*>(x) + 2 * (size_t)g.batch * g.cin * g.in[0] * g.in[1] * g.in[2];
-  p.Cin = g.cin; p.Cout = g.cout;
+  p.x_end = static_cast<const char*>(x) + 2 * (size_t)g.batch * g.cin * x_cs;
+  p.cin_total = g.cin; p.cout_total = g.cout;
   p.Din = g.in[0]; p.Hin = g.in[1]; p.Win = g.in[2];
   p.Dout = g.out[0]; p.Hout = g.out[1]; p.Wout = g.out[2];
   p.pad_d = g.p[0]; p.pad_h = g.p[1]; p.pad_w = g.p[2];
@@ -677,29 +705,40 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
   p.xt = static_cast<const uint16_t*>(xt);
   p.tlo_d = tlo ? tlo[0] : 0; p.tlo_h = tlo ? tlo[1] : 0; p.tlo_w = tlo ? tlo[2] : 0;
   p.tn_d = tn ? tn[0] : 0; p.tn_h = tn ? tn[1] : 0; p.tn_w = tn ? tn[2] : 0;
-  p.bias_part = gb != nullptr ? p.part + (size_t)wgs * HALVES * 9 * (32 * cgb) * (32 * cxb) : nullptr;
-  const bool even = (p.Win % 2 == 0) && (p.pad_w % 2 == 0) && (p.Wout % 2 == 0) &&
-                    ((reinterpret_cast<uintptr_t>(x) & 3) == 0) &&
-                    ((reinterpret_cast<uintptr_t>(go) & 3) == 0);
-  if (xt != nullptr && (!even || !mfma_wgrad_frame_ok(g, tlo, tn)))
-    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: the framed input does not cover this geometry / alignment", who);
-  int rc;
-  if (cgb == 2 && cxb == 2) rc = launch<2, 2>(p, even, wgs, s, who);
-  else if (cgb == 1 && cxb == 3) rc = launch<1, 3>(p, even, wgs, s, who);
-  else if (cgb == 1 && cxb == 1) rc = launch<1, 1>(p, even, wgs, s, who);
-  else if (cgb == 2 && cxb == 1) rc = launch<2, 1>(p, even, wgs, s, who);
-  else if (cgb == 1 && cxb == 2) rc = launch<1, 2>(p, even, wgs, s, who);
-  else JG_FAIL(JG_ERR_UNSUPPORTED, "%s: channel blocking (%d, %d) not built", who, cgb, cxb);
-  if (rc) return rc;
-  JG_CHECK_LAUNCH(who);
-  const int count = 9 * 32 * cgb * 32 * cxb;
-  wgrad_reduce_kernel<<<(count + 63) / 64, 256, 0, s>>>(static_cast<uint16_t*>(gw), p.part, wgs * HALVES,
-                                                          32 * cgb, 32 * cxb, g.cin);
-  JG_CHECK_LAUNCH(who);
-  if (gb != nullptr) {
-    wgrad_bias_reduce_kernel<<<(32 * cgb + 3) / 4, 256, 0, s>>>(static_cast<uint16_t*>(gb), p.bias_part, wgs,
-                                                                32 * cgb);
-    JG_CHECK_LAUNCH(who);
+  for (int co0 = 0; co0 < g.cout;) {
+    const int cob = block_width(g.cout, co0, bl.cob);
+    for (int ci0 = 0; ci0 < g.cin;) {
+      const int cib = block_width(g.cin, ci0, bl.cib);
+      const int cgb = cob / 32, cxb = bl.KD * cib / 32;
+      p.Cin = cib; p.Cout = cob;
+      p.cin_valid = g.cin - ci0 < cib ? g.cin - ci0 : cib;
+      p.cout_valid = g.cout - co0 < cob ? g.cout - co0 : cob;
+      p.x = static_cast<const uint16_t*>(x) + ci0 * x_cs;
+      p.g = static_cast<const uint16_t*>(go) + co0 * g_cs;
+      // the bias gradient comes from the g rows: once per block of output channels
+      p.bias_part = (gb != nullptr && ci0 == 0) ? p.part + (size_t)wgs * HALVES * 9 * cob * (bl.KD * cib) : nullptr;
+      int rc;
+      if (cgb == 2 && cxb == 2) rc = launch<2, 2>(p, even, wgs, s, who);
+      else if (cgb == 1 && cxb == 3) rc = launch<1, 3>(p, even, wgs, s, who);
+      else if (cgb == 1 && cxb == 1) rc = launch<1, 1>(p, even, wgs, s, who);
+      else if (cgb == 2 && cxb == 1) rc = launch<2, 1>(p, even, wgs, s, who);
+      else if (cgb == 1 && cxb == 2) rc = launch<1, 2>(p, even, wgs, s, who);
+      else JG_FAIL(JG_ERR_UNSUPPORTED, "%s: channel blocking (%d, %d) not built", who, cgb, cxb);
+      if (rc) return rc;
+      JG_CHECK_LAUNCH(who);
+      const int count = 9 * cob * bl.KD * cib;
+      uint16_t* gw_blk = static_cast<uint16_t*>(gw) + ((size_t)co0 * g.cin + ci0) * bl.KD * 9;
+      wgrad_reduce_kernel<<<(count + 63) / 64, 256, 0, s>>>(gw_blk, p.part, wgs * HALVES, cob, bl.KD * cib, cib,
+                                                              p.cout_valid, p.cin_valid, g.cin);
+      JG_CHECK_LAUNCH(who);
+      if (p.bias_part != nullptr) {
+        wgrad_bias_reduce_kernel<<<(cob + 3) / 4, 256, 0, s>>>(static_cast<uint16_t*>(gb) + co0, p.bias_part,
+                                                               wgs, cob, p.cout_valid);
+        JG_CHECK_LAUNCH(who);
+      }
+      ci0 += cib;
+    }
+    co0 += cob;
   }
   return JG_OK;
 }

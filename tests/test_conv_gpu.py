@@ -38,6 +38,14 @@ PRIM_CASES = [
     (2, 64, 64, (260, 131), (3, 3), (1, 1), (0, 0), (1, 1)),
     (2, 32, 32, (6, 70, 130), (3, 3, 3), (1, 1, 1), (0, 0, 0), (1, 1, 1)),
     (1, 32, 64, (131, 200), (3, 3), (1, 1), (1, 1), (1, 1)),
+    # channel counts beyond one group of LDS-resident weights, and produced channels that are
+    # not a multiple of the 32-row MFMA tile (padded with zero weight rows, not stored)
+    (1, 128, 128, (20, 70), (3, 3), (1, 1), (1, 1), (1, 1)),
+    (2, 16, 3, (37, 66), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (1, 48, 80, (33, 40), (3, 3), (1, 1), (1, 1), (1, 1)),
+    (1, 256, 64, (18, 34), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (1, 96, 32, (5, 18, 34), (3, 3, 3), (1, 1, 1), (1, 0, 1), (1, 1, 1)),
+    (1, 80, 16, (4, 20, 36), (3, 3, 3), (1, 1, 1), (0, 0, 0), (1, 1, 1)),
 ]
 
 
