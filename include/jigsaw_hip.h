@@ -246,6 +246,38 @@ int jg_gn_bwd_apply(void* gx, const void* g, const void* x_norm, const void* wei
                     int64_t groups, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------- *
+ * Token projections around the attention core, head split / merge fused into
+ * the GEMM addressing (MFMA-bound for bf16)
+ *
+ * Stand in for `self.qkv(x)` + rearrange "... n s (three h d) -> three ... n h s d"
+ * and for rearrange "... n h s d -> ... n s (h d)" + `.contiguous()` +
+ * `self.head_concat(out)` of DistributedAttention.forward
+ * (jigsaw/modules/attention/_attention.py:881-918), and for their backward.
+ *
+ * A token x feature matrix is either row-major (tokens, features) or, with its
+ * *_heads flag set, the dense tensor (t, B, H, S, D): token = b * S + s,
+ * feature = (t * H + h) * D + d, B * S = rows, features = t * H * D.
+ * fp32 accumulation; all operands share `dtype`.
+ * ------------------------------------------------------------------------- */
+
+/* out(r, n) = sum_k a(r, k) * w[n][k] + bias[n];  w (n_out, k_in) row-major,
+ * bias (n_out,) or NULL. Forward of both projections; with the transposed
+ * weight also the gradient of a projection's input. */
+int jg_proj_nt(void* out, const void* a, const void* w, const void* bias, int dtype,
+               int64_t rows, int n_out, int k_in, int a_heads, int out_heads,
+               int B, int H, int S, int D, void* stream);
+
+/* gw[n][c] = sum_r g(r, n) * x(r, c)  (n, c) row-major, and gb[n] = sum_r g(r, n)
+ * (gb may be NULL): weight and bias gradient of a projection (torch's
+ * Linear backward; g = grad of the projection's output, x = its input).
+ * workspace: jg_proj_tn_workspace(rows, n, c) bytes of device scratch (partial
+ * sums per token range, added up in a fixed order: deterministic). */
+size_t jg_proj_tn_workspace(int64_t rows, int n, int c);
+int jg_proj_tn(void* gw, void* gb, const void* g, const void* x, int dtype, int64_t rows,
+               int n, int c, int g_heads, int x_heads, int B, int H, int S, int D,
+               void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------- *
  * Online-softmax / log-sum-exp merge of ring attention (HBM-bound)
  * ------------------------------------------------------------------------- */
 

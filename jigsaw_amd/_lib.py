@@ -129,6 +129,17 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
          c_int64, c_int, c_void_p],
     ),
+    "jg_proj_nt": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+         c_int, c_void_p],
+    ),
+    "jg_proj_tn_workspace": (c_size_t, [c_int64, c_int, c_int]),
+    "jg_proj_tn": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+         c_int, c_void_p, c_size_t, c_void_p],
+    ),
     "jg_conv_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int, c_int]),
     "jg_conv_fwd": (
         c_int,

@@ -1,0 +1,161 @@
+"""Token projections around the attention core with the head split / merge fused in.
+
+Host-side mirror of the pre- and post-processing of ``DistributedAttention.forward``
+(jigsaw/modules/attention/_attention.py:881-918):
+
+* :func:`qkv_projection` stands for ``self.qkv(x)`` followed by
+  ``rearrange(qkv, "... n s (three h d) -> three ... n h s d")``: the GEMM writes q, k
+  and v straight into their ``(..., h, s, d)`` places, no rearrange copy;
+* :func:`heads_projection` stands for
+  ``rearrange(out, "... n h s d -> ... n s (h d)").contiguous()`` followed by
+  ``self.head_concat(out)``: the GEMM reads the attention output where it lies.
+
+Both are ``autograd`` functions; their backward reads and writes the head layouts the
+same way (input gradient: the same GEMM with the transposed weight; weight and bias
+gradient: one GEMM contracted over the tokens). The weights are the rank's local
+``nn.Linear`` parameters ``(out_features, in_features)``.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+
+
+def _nt(out, a, w, bias, rows, n_out, k_in, a_heads, out_heads, dims) -> None:
+    lib = _lib.load()
+    b, h, s, d = dims
+    rc = lib.jg_proj_nt(_lib.ptr(out), _lib.ptr(a), _lib.ptr(w), _lib.ptr(bias), _lib.dtype_code(a.dtype), rows, n_out,
+                        k_in, int(a_heads), int(out_heads), b, h, s, d, _lib.stream_ptr(a.device))
+    _lib.check(rc, "jg_proj_nt")
+
+
+def _tn(g, x, rows, n, c, g_heads, x_heads, dims, want_bias):
+    lib = _lib.load()
+    b, h, s, d = dims
+    gw = torch.empty(n, c, dtype=g.dtype, device=g.device)
+    gb = torch.empty(n, dtype=g.dtype, device=g.device) if want_bias else None
+    nbytes = int(lib.jg_proj_tn_workspace(rows, n, c))
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=g.device)
+    rc = lib.jg_proj_tn(_lib.ptr(gw), _lib.ptr(gb), _lib.ptr(g), _lib.ptr(x), _lib.dtype_code(g.dtype), rows, n, c,
+                        int(g_heads), int(x_heads), b, h, s, d, _lib.ptr(ws), nbytes, _lib.stream_ptr(g.device))
+    _lib.check(rc, "jg_proj_tn")
+    return gw, gb
+
+
+class _QkvProjection(torch.autograd.Function):
+    """``(*lead, s, C) -> (3, *lead, h, s, d)`` with ``weight (3 h d, C)``."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, heads):  # noqa: D102
+        _lib.require_gpu(x, weight, bias)
+        if x.dim() < 2:
+            raise ValueError("x must be (..., seq, channels)")
+        n_out, c = weight.shape
+        if x.shape[-1] != c:
+            raise ValueError(f"x has {x.shape[-1]} channels, the weight takes {c}")
+        if n_out % (3 * heads) != 0:
+            raise ValueError(f"{n_out} output features do not split into 3 x {heads} heads")
+        d = n_out // (3 * heads)
+        lead, s = tuple(x.shape[:-2]), x.shape[-2]
+        b = math.prod(lead)
+        xc = x.contiguous()
+        w = weight.to(x.dtype).contiguous()
+        bs = None if bias is None else bias.to(x.dtype).contiguous()
+        out = torch.empty((3, *lead, heads, s, d), dtype=x.dtype, device=x.device)
+        if b * s:
+            _nt(out, xc, w, bs, b * s, n_out, c, False, True, (b, heads, s, d))
+        ctx.save_for_backward(xc, w)
+        ctx.dims = (b, heads, s, d)
+        ctx.has_bias = bias is not None
+        ctx.dtypes = (weight.dtype, None if bias is None else bias.dtype)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):  # noqa: D102
+        xc, w = ctx.saved_tensors
+        b, h, s, d = ctx.dims
+        n_out, c = w.shape
+        g = grad.to(xc.dtype).contiguous()
+        gx = gw = gb = None
+        if b * s == 0:
+            gx = torch.zeros_like(xc) if ctx.needs_input_grad[0] else None
+            gw = torch.zeros_like(w) if ctx.needs_input_grad[1] else None
+            gb = torch.zeros(n_out, dtype=w.dtype, device=w.device) if ctx.has_bias and ctx.needs_input_grad[2] else None
+        else:
+            if ctx.needs_input_grad[0]:
+                gx = torch.empty_like(xc)
+                _nt(gx, g, w.t().contiguous(), None, b * s, c, n_out, True, False, ctx.dims)
+            need_b = ctx.has_bias and ctx.needs_input_grad[2]
+            if ctx.needs_input_grad[1] or need_b:
+                gw, gb = _tn(g, xc, b * s, n_out, c, True, False, ctx.dims, need_b)
+        dt_w, dt_b = ctx.dtypes
+        return (gx, None if gw is None or not ctx.needs_input_grad[1] else gw.to(dt_w),
+                None if gb is None else gb.to(dt_b), None)
+
+
+class _HeadsProjection(torch.autograd.Function):
+    """``(*lead, h, s, d) -> (*lead, s, n_out)`` with ``weight (n_out, h d)``."""
+
+    @staticmethod
+    def forward(ctx, out, weight, bias):  # noqa: D102
+        _lib.require_gpu(out, weight, bias)
+        if out.dim() < 3:
+            raise ValueError("out must be (..., heads, seq, head_dim)")
+        n_out, k = weight.shape
+        h, s, d = out.shape[-3:]
+        if h * d != k:
+            raise ValueError(f"heads x head_dim = {h * d}, the weight takes {k}")
+        lead = tuple(out.shape[:-3])
+        b = math.prod(lead)
+        oc = out.contiguous()
+        w = weight.to(out.dtype).contiguous()
+        bs = None if bias is None else bias.to(out.dtype).contiguous()
+        y = torch.empty((*lead, s, n_out), dtype=out.dtype, device=out.device)
+        if b * s:
+            _nt(y, oc, w, bs, b * s, n_out, k, True, False, (b, h, s, d))
+        ctx.save_for_backward(oc, w)
+        ctx.dims = (b, h, s, d)
+        ctx.has_bias = bias is not None
+        ctx.dtypes = (weight.dtype, None if bias is None else bias.dtype)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad):  # noqa: D102
+        oc, w = ctx.saved_tensors
+        b, h, s, d = ctx.dims
+        n_out, k = w.shape
+        g = grad.to(oc.dtype).contiguous()
+        go = gw = gb = None
+        if b * s == 0:
+            go = torch.zeros_like(oc) if ctx.needs_input_grad[0] else None
+            gw = torch.zeros_like(w) if ctx.needs_input_grad[1] else None
+            gb = torch.zeros(n_out, dtype=w.dtype, device=w.device) if ctx.has_bias and ctx.needs_input_grad[2] else None
+        else:
+            if ctx.needs_input_grad[0]:
+                go = torch.empty_like(oc)
+                _nt(go, g, w.t().contiguous(), None, b * s, k, n_out, False, True, ctx.dims)
+            need_b = ctx.has_bias and ctx.needs_input_grad[2]
+            if ctx.needs_input_grad[1] or need_b:
+                gw, gb = _tn(g, oc, b * s, n_out, k, False, True, ctx.dims, need_b)
+        dt_w, dt_b = ctx.dtypes
+        return (go, None if gw is None or not ctx.needs_input_grad[1] else gw.to(dt_w),
+                None if gb is None else gb.to(dt_b))
+
+
+def qkv_projection(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, heads: int) -> torch.Tensor:
+    """``rearrange(F.linear(x, weight, bias), "... s (three h d) -> three ... h s d", three=3, h=heads)``
+    without the intermediate ``(..., s, 3 h d)`` tensor (_attention.py:881-890)."""
+    return _QkvProjection.apply(x, weight, bias, heads)
+
+
+def heads_projection(out: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """``F.linear(rearrange(out, "... h s d -> ... s (h d)"), weight, bias)`` without the
+    contiguous copy of the rearranged tensor (_attention.py:909-916)."""
+    return _HeadsProjection.apply(out, weight, bias)
+
+
+__all__ = ["heads_projection", "qkv_projection"]

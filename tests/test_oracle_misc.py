@@ -202,3 +202,39 @@ def test_groupnorm_oracle_equals_torch_on_the_undivided_tensor():
         assert torch.allclose(torch.cat([b[0] for b in back], dim=dim), X.grad, rtol=1e-9, atol=1e-11)
         assert torch.allclose(sum(b[1] for b in back), W.grad, rtol=1e-9, atol=1e-11)
         assert torch.allclose(sum(b[2] for b in back), B.grad, rtol=1e-9, atol=1e-11)
+
+
+def test_projection_oracle_equals_linear_and_rearrange():
+    """The restated projections against F.linear + einops' rearrange with the reference's
+    patterns (_attention.py:885-890, 909-916) and autograd through them."""
+    from einops import rearrange
+
+    from oracle import projection as op
+
+    torch.manual_seed(13)
+    for lead, s, c, heads, d in [((2,), 5, 6, 2, 3), ((2, 3), 4, 8, 3, 2), ((), 7, 4, 1, 4)]:
+        x = torch.randn(*lead, s, c, dtype=torch.float64, requires_grad=True)
+        w = torch.randn(3 * heads * d, c, dtype=torch.float64, requires_grad=True)
+        b = torch.randn(3 * heads * d, dtype=torch.float64, requires_grad=True)
+        want = rearrange(torch.nn.functional.linear(x, w, b), "... s (three h d) -> three ... h s d", three=3, h=heads)
+        got = op.qkv_forward(x.detach(), w.detach(), b.detach(), heads)
+        assert got.shape == want.shape and torch.allclose(got, want.detach(), rtol=1e-12, atol=1e-12)
+        g = torch.randn_like(want)
+        want.backward(g)
+        gx, gw, gb = op.qkv_backward(g, x.detach(), w.detach(), heads)
+        assert torch.allclose(gx, x.grad, rtol=1e-11, atol=1e-11)
+        assert torch.allclose(gw, w.grad, rtol=1e-11, atol=1e-11)
+        assert torch.allclose(gb, b.grad, rtol=1e-11, atol=1e-11)
+
+        o = torch.randn(*lead, heads, s, d, dtype=torch.float64, requires_grad=True)
+        wo = torch.randn(5, heads * d, dtype=torch.float64, requires_grad=True)
+        bo = torch.randn(5, dtype=torch.float64, requires_grad=True)
+        want = torch.nn.functional.linear(rearrange(o, "... h s d -> ... s (h d)").contiguous(), wo, bo)
+        got = op.heads_forward(o.detach(), wo.detach(), bo.detach())
+        assert got.shape == want.shape and torch.allclose(got, want.detach(), rtol=1e-12, atol=1e-12)
+        g = torch.randn_like(want)
+        want.backward(g)
+        go, gw, gb = op.heads_backward(g, o.detach(), wo.detach())
+        assert torch.allclose(go, o.grad, rtol=1e-11, atol=1e-11)
+        assert torch.allclose(gw, wo.grad, rtol=1e-11, atol=1e-11)
+        assert torch.allclose(gb, bo.grad, rtol=1e-11, atol=1e-11)

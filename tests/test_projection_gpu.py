@@ -1,0 +1,125 @@
+"""Projections around the attention core (head split / merge fused into the GEMM):
+HIP kernels through the C ABI against the oracle (fp64 on the same rounded inputs).
+
+Tolerances: rel-L2 <= 1e-5 in fp32, 2e-2 in bf16, 4e-3 in fp16. The layout itself is
+checked exactly: with a one-hot weight the projection is a pure copy.
+"""
+
+import pytest
+import torch
+
+from helpers import rel_l2
+from jigsaw_amd import projection as jp
+from oracle import projection as op
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 4e-3}
+
+
+@pytest.fixture(scope="module")
+def dev():
+    return torch.device("cuda:0")
+
+
+CASES = [
+    # lead, seq, channels, heads, head_dim, out features of the second projection, dtype, bias
+    ((1,), 4096, 512, 8, 64, 512, torch.bfloat16, True),     # the ring-attention configuration
+    ((4, 16), 64, 128, 4, 32, 128, torch.bfloat16, True),    # Swin windows: two leading axes
+    ((2,), 200, 96, 3, 32, 80, torch.bfloat16, False),       # ragged tiles: 400 tokens, 288 / 96 / 80 features
+    ((3,), 50, 72, 3, 24, 40, torch.bfloat16, True),         # head_dim 24, contraction not a multiple of 64
+    ((1,), 130, 64, 2, 20, 24, torch.bfloat16, True),        # head_dim 20: not a multiple of 8, FMA path
+    ((2,), 33, 24, 2, 8, 10, torch.float32, True),
+    ((2, 2), 17, 16, 1, 16, 16, torch.float16, True),
+    ((0,), 16, 32, 2, 16, 32, torch.bfloat16, True),         # empty batch
+]
+
+
+def _id(c):
+    return f"{'x'.join(map(str, c[0]))}_{c[1]}x{c[2]}_h{c[3]}d{c[4]}_{c[5]}_{str(c[6]).split('.')[-1]}"
+
+
+@pytest.mark.parametrize("case", CASES, ids=_id)
+def test_projections_match_oracle(case, dev):
+    lead, s, c, heads, d, n2, dtype, has_b = case
+    tol = TOL[dtype]
+    torch.manual_seed(21)
+    x = torch.randn(*lead, s, c).to(dtype)
+    w = (torch.randn(3 * heads * d, c) / c ** 0.5).to(dtype)
+    b = (0.1 * torch.randn(3 * heads * d)).to(dtype) if has_b else None
+    g = torch.randn(3, *lead, heads, s, d).to(dtype)
+    print(f"qkv_projection {case}", flush=True)
+    xd, wd = x.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+    bd = b.to(dev).requires_grad_() if has_b else None
+    y = jp.qkv_projection(xd, wd, bd, heads)
+    assert y.shape == (3, *lead, heads, s, d) and y.dtype == dtype and y.is_contiguous()
+    y.backward(g.to(dev))
+    want = op.qkv_forward(x.double(), w.double(), b.double() if has_b else None, heads)
+    gx, gw, gb = op.qkv_backward(g.double(), x.double(), w.double(), heads)
+    if x.numel():
+        assert rel_l2(y.detach().cpu(), want) <= tol
+        assert rel_l2(xd.grad.cpu(), gx) <= tol
+        assert rel_l2(wd.grad.cpu(), gw) <= tol
+        if has_b:
+            assert rel_l2(bd.grad.cpu(), gb) <= tol
+    else:
+        assert float(wd.grad.abs().sum()) == 0.0 and xd.grad.shape == x.shape
+
+    o = torch.randn(*lead, heads, s, d).to(dtype)
+    wo = (torch.randn(n2, heads * d) / (heads * d) ** 0.5).to(dtype)
+    bo = (0.1 * torch.randn(n2)).to(dtype) if has_b else None
+    g2 = torch.randn(*lead, s, n2).to(dtype)
+    print(f"heads_projection {case}", flush=True)
+    od, wod = o.to(dev).requires_grad_(), wo.to(dev).requires_grad_()
+    bod = bo.to(dev).requires_grad_() if has_b else None
+    z = jp.heads_projection(od, wod, bod)
+    assert z.shape == (*lead, s, n2) and z.dtype == dtype
+    z.backward(g2.to(dev))
+    want = op.heads_forward(o.double(), wo.double(), bo.double() if has_b else None)
+    go, gw, gb = op.heads_backward(g2.double(), o.double(), wo.double())
+    if o.numel():
+        assert rel_l2(z.detach().cpu(), want) <= tol
+        assert rel_l2(od.grad.cpu(), go) <= tol
+        assert rel_l2(wod.grad.cpu(), gw) <= tol
+        if has_b:
+            assert rel_l2(bod.grad.cpu(), gb) <= tol
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_identity_weight_is_the_rearrange_exactly(dtype, dev):
+    """With the identity as weight and no bias the projection only moves data: the
+    result must equal torch's reshape / permute of the input bit for bit."""
+    torch.manual_seed(22)
+    lead, s, heads, d = (2, 3), 40, 3, 16
+    c = 3 * heads * d
+    x = torch.randn(*lead, s, c, device=dev).to(dtype)
+    eye = torch.eye(c, device=dev, dtype=dtype)
+    y = jp.qkv_projection(x, eye, None, heads)
+    want = x.reshape(*lead, s, 3, heads, d).permute(3, 0, 1, 4, 2, 5).contiguous()
+    assert torch.equal(y, want)
+    o = torch.randn(*lead, heads, s, d, device=dev).to(dtype)
+    eye = torch.eye(heads * d, device=dev, dtype=dtype)
+    z = jp.heads_projection(o, eye, None)
+    want = o.permute(0, 1, 3, 2, 4).reshape(*lead, s, heads * d)
+    assert torch.equal(z, want)
+
+
+def test_full_size_against_torch_gemm(dev):
+    """Eight sequences of the ring-attention configuration: the fused projections against
+    torch's own bf16 GEMM + rearrange on the GPU (both accumulate in fp32 and round once,
+    so they agree to a few bf16 roundings), and forward -> backward runs at full size."""
+    torch.manual_seed(23)
+    bsz, s, c, heads, d = 8, 4096, 512, 8, 64
+    x = torch.randn(bsz, s, c, device=dev).bfloat16().requires_grad_()
+    w = (torch.randn(3 * c, c, device=dev) / c ** 0.5).bfloat16().requires_grad_()
+    b = (0.1 * torch.randn(3 * c, device=dev)).bfloat16().requires_grad_()
+    y = jp.qkv_projection(x, w, b, heads)
+    want = torch.nn.functional.linear(x.detach(), w.detach(), b.detach())
+    want = want.reshape(bsz, s, 3, heads, d).permute(2, 0, 3, 1, 4)
+    assert rel_l2(y.detach().float(), want.float()) <= 4e-3
+    g = torch.randn_like(y)
+    y.backward(g)
+    gflat = g.permute(1, 3, 0, 2, 4).reshape(bsz * s, 3 * c)
+    assert rel_l2(x.grad.float(), (gflat.float() @ w.detach().float()).reshape(bsz, s, c)) <= 4e-3
+    assert rel_l2(w.grad.float(), gflat.float().t() @ x.detach().reshape(-1, c).float()) <= 4e-3
+    assert rel_l2(b.grad.float(), gflat.float().sum(0)) <= 4e-3
