@@ -29,6 +29,8 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
@@ -75,14 +77,9 @@ struct RowWalk {
   }
 };
 
-constexpr int THREADS = 256;
-constexpr int TILE = 128;  // rows and columns of a workgroup tile
 
 // ------------------------------------------------------------------------ NT
-constexpr int BK = 64;                 // contraction elements per stage
-constexpr int NT_OP = 8 * TILE;        // slots of one operand per stage: [chunk of 8 k][row ^ 2 chunk]
-constexpr int NT_STAGE = 2 * NT_OP;
-constexpr int NT_LDS = 2 * NT_STAGE * 16;
+constexpr int BK = 64;  // contraction elements per stage
 
 struct NtParams {
   const uint16_t* a;
@@ -95,79 +92,110 @@ struct NtParams {
   int tiles_n;
 };
 
-__device__ __forceinline__ int nt_slot(int chunk, int row) { return chunk * TILE + (row ^ (2 * chunk)); }
+// Shape of a workgroup: WM x WN wavefronts, each with IM x JN blocks of 32 tokens x 32 features.
+template <int IM, int JN, int WM, int WN>
+struct NtShape {
+  static constexpr int TM = 32 * IM * WM, TNF = 32 * JN * WN;  // tokens, features of a tile
+  static constexpr int THREADS = 64 * WM * WN;
+  static constexpr int OP_A = 8 * TM, OP_W = 8 * TNF;          // 16-byte slots per stage: [chunk of 8 k][row ^ 2 chunk]
+  static constexpr int STAGE = OP_A + OP_W;
+  static constexpr int OUT_PITCH = TNF + 8;                    // elements per token row of the result tile in LDS
+  static constexpr int MAIN = 2 * STAGE * 16 > TM * OUT_PITCH * 2 ? 2 * STAGE * 16 : TM * OUT_PITCH * 2;
+  static constexpr int LDS = MAIN + TNF * 4;                   // then the bias of the tile as floats
+  static constexpr int PASS_A = TM * 8 / THREADS, PASS_W = TNF * 8 / THREADS;
+  static_assert(TM * 8 % THREADS == 0 && TNF * 8 % THREADS == 0, "whole load passes");
+};
 
-__global__ __launch_bounds__(THREADS) void proj_nt_kernel(NtParams p) {
+template <int IM, int JN, int WM, int WN>
+__global__ __launch_bounds__(64 * WM * WN) void proj_nt_kernel(NtParams p) {
+  typedef NtShape<IM, JN, WM, WN> SH;
+  constexpr int TM = SH::TM, TNF = SH::TNF, THREADS = SH::THREADS;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   u32x4* lds = reinterpret_cast<u32x4*>(smem);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, kg = lane >> 5;
-  const int wm = wave & 1, wn = wave >> 1;
-  const long long m0 = (long long)(blockIdx.x / p.tiles_n) * TILE;
-  const int n0 = (blockIdx.x % p.tiles_n) * TILE;
+  const int wm = wave % WM, wn = wave / WM;
+  const long long m0 = (long long)(blockIdx.x / p.tiles_n) * TM;
+  const int n0 = (blockIdx.x % p.tiles_n) * TNF;
+  if (tid < TNF)  // read after the barriers of the stage loop
+    reinterpret_cast<float*>(smem + SH::MAIN)[tid] =
+        (p.bias != nullptr && n0 + tid < p.N) ? jg::bf16_to_f32(p.bias[n0 + tid]) : 0.0f;
 
-  // loads of a stage: chunk column c, rows tid / 8 + 32 i of both operands
+  // loads of a stage: chunk column c, rows tid / 8 + (THREADS / 8) i of both operands
+  constexpr int RSTEP = THREADS / 8;
   const int c = tid & 7, lrow = tid >> 3;
-  long long a_row[4], w_row[4];
+  // byte offsets from the start of a / w: 32 bits (the host checks the tensor sizes), so that a
+  // load takes the uniform base from scalar registers and one vector register per address
+  uint32_t a_row[SH::PASS_A], w_row[SH::PASS_W];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    long long r = m0 + lrow + 32 * i;
+  for (int i = 0; i < SH::PASS_A; ++i) {
+    long long r = m0 + lrow + RSTEP * i;
     if (r > p.rows - 1) r = p.rows - 1;  // a row past the end repeats the last one and is dropped
-    a_row[i] = row_part(p.am, r);
-    int n = n0 + lrow + 32 * i;
-    if (n > p.N - 1) n = p.N - 1;
-    w_row[i] = (long long)n * p.K;
+    a_row[i] = (uint32_t)(row_part(p.am, r) * 2);
   }
-  u32x4 ra[4], rw[4];
+#pragma unroll
+  for (int i = 0; i < SH::PASS_W; ++i) {
+    int n = n0 + lrow + RSTEP * i;
+    if (n > p.N - 1) n = p.N - 1;
+    w_row[i] = (uint32_t)((long long)n * p.K * 2);
+  }
+  const char* a_bytes = reinterpret_cast<const char*>(p.a);
+  const char* w_bytes = reinterpret_cast<const char*>(p.w);
+  u32x4 ra[SH::PASS_A], rw[SH::PASS_W];
   bool ld_ok = true;
   auto load = [&](int ks) {
     const int k = ks * BK + c * 8;
     ld_ok = k < p.K;  // a chunk past the contraction length is read at k = 0 and zeroed on the way to LDS
     const int kk = ld_ok ? k : 0;
-    const long long fa = feat_part(p.am, kk);
+    const uint32_t fa = (uint32_t)(feat_part(p.am, kk) * 2), fw = (uint32_t)kk * 2;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      ra[i] = *reinterpret_cast<const u32x4*>(p.a + a_row[i] + fa);
-      rw[i] = *reinterpret_cast<const u32x4*>(p.w + w_row[i] + kk);
-    }
+    for (int i = 0; i < SH::PASS_A; ++i) ra[i] = *reinterpret_cast<const u32x4*>(a_bytes + (size_t)(a_row[i] + fa));
+#pragma unroll
+    for (int i = 0; i < SH::PASS_W; ++i) rw[i] = *reinterpret_cast<const u32x4*>(w_bytes + (size_t)(w_row[i] + fw));
   };
   auto store = [&](int buf) {
-    u32x4* sa = lds + buf * NT_STAGE;
-    u32x4* sw = sa + NT_OP;
+    u32x4* sa = lds + buf * SH::STAGE;
+    u32x4* sw = sa + SH::OP_A;
     const u32x4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int slot = nt_slot(c, lrow + 32 * i);
-      sa[slot] = ld_ok ? ra[i] : zero;
-      sw[slot] = ld_ok ? rw[i] : zero;
-    }
+    for (int i = 0; i < SH::PASS_A; ++i) sa[c * TM + ((lrow + RSTEP * i) ^ (2 * c))] = ld_ok ? ra[i] : zero;
+#pragma unroll
+    for (int i = 0; i < SH::PASS_W; ++i) sw[c * TNF + ((lrow + RSTEP * i) ^ (2 * c))] = ld_ok ? rw[i] : zero;
   };
 
-  f32x16 acc[2][2];
+  f32x16 acc[IM][JN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < IM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < JN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
+  // acc[i][j] = w fragment (rows: features) x a fragment (columns: tokens). The fragments of
+  // the next 16-wide step are requested before the MFMAs of this one are issued.
   auto compute = [&](int buf) {
-    const u32x4* sa = lds + buf * NT_STAGE;
-    const u32x4* sw = sa + NT_OP;
+    const u32x4* sa = lds + buf * SH::STAGE;
+    const u32x4* sw = sa + SH::OP_A;
+    u32x4 fr[2][IM + JN];
+    auto fetch = [&](int kk, u32x4 (&f)[IM + JN]) {
+      const int cc = kk * 2 + kg;
+#pragma unroll
+      for (int t = 0; t < IM; ++t) f[t] = sa[cc * TM + ((wm * 32 * IM + t * 32 + ln) ^ (2 * cc))];
+#pragma unroll
+      for (int t = 0; t < JN; ++t) f[IM + t] = sw[cc * TNF + ((wn * 32 * JN + t * 32 + ln) ^ (2 * cc))];
+    };
+    fetch(0, fr[0]);
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
-      const int cc = kk * 2 + kg;
-      bf16x8 af[2], wf[2];
+      if (kk + 1 < BK / 16) fetch(kk + 1, fr[(kk + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        af[t] = __builtin_bit_cast(bf16x8, sa[nt_slot(cc, wm * 64 + t * 32 + ln)]);
-        wf[t] = __builtin_bit_cast(bf16x8, sw[nt_slot(cc, wn * 64 + t * 32 + ln)]);
-      }
+      for (int i = 0; i < IM; ++i)
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < JN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fr[kk & 1][IM + j]),
+                                                              __builtin_bit_cast(bf16x8, fr[kk & 1][i]), acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
@@ -182,46 +210,63 @@ __global__ __launch_bounds__(THREADS) void proj_nt_kernel(NtParams p) {
     __syncthreads();
   }
 
-  // accumulator lane (ln, kg), register e of block (i, j): token m0 + wm*64 + i*32 +
-  // 8*(e/4) + 4*kg + e%4, feature n0 + wn*64 + j*32 + ln
-  long long fo[2];
-  float bv[2];
-  bool n_ok[2];
+  // Accumulator lane (ln, kg), register e of block (i, j): feature (wn*JN + j)*32 + 8*(e/4) +
+  // 4*kg + e%4, token (wm*IM + i)*32 + ln. The tile goes to LDS as bf16 [token][feature]
+  // (the stages are done with), and leaves it in 16-byte pieces of 8 features.
+  uint16_t* tile = reinterpret_cast<uint16_t*>(smem);
+  const float* lds_bias = reinterpret_cast<const float*>(smem + SH::MAIN);
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int n = n0 + wn * 64 + j * 32 + ln;
-    n_ok[j] = n < p.N;
-    fo[j] = feat_part(p.om, n_ok[j] ? n : 0);
-    bv[j] = (p.bias != nullptr && n_ok[j]) ? jg::bf16_to_f32(p.bias[n]) : 0.0f;
-  }
+  for (int i = 0; i < IM; ++i)
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const long long rbase = m0 + wm * 64 + i * 32 + kg * 4;
-    RowWalk rwk;
-    rwk.start(p.om, rbase);
+    for (int j = 0; j < JN; ++j)
 #pragma unroll
-    for (int e4 = 0; e4 < 4; ++e4) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const long long r = rbase + e4 * 8 + e;
-        const long long ro = rwk.part(p.om);
-        if (r < p.rows) {
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-            if (n_ok[j]) p.out[ro + fo[j]] = jg::f32_to_bf16(acc[i][j][e4 * 4 + e] + bv[j]);
-        }
-        rwk.advance(p.om, e == 3 ? 5 : 1);
+      for (int e4 = 0; e4 < 4; ++e4) {
+        const int f = (wn * JN + j) * 32 + e4 * 8 + kg * 4;
+        const int tok = (wm * IM + i) * 32 + ln;
+        const f32x4 bq = *reinterpret_cast<const f32x4*>(lds_bias + f);
+        const f32x2 lo = {acc[i][j][e4 * 4 + 0] + bq.x, acc[i][j][e4 * 4 + 1] + bq.y};
+        const f32x2 hi = {acc[i][j][e4 * 4 + 2] + bq.z, acc[i][j][e4 * 4 + 3] + bq.w};
+        u32x2 pk;
+        pk.x = __builtin_bit_cast(uint32_t, __builtin_convertvector(lo, bf16x2));
+        pk.y = __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, bf16x2));
+        *reinterpret_cast<u32x2*>(tile + tok * SH::OUT_PITCH + f) = pk;
       }
+  __syncthreads();
+  {
+    constexpr int CPR = TNF / 8, RPP = THREADS / CPR;  // 16-byte pieces per token row, rows per pass
+    const int fc = tid % CPR, trow = tid / CPR;
+    const int n = n0 + fc * 8;
+    const long long fo = feat_part(p.om, n < p.N ? n : 0);
+    RowWalk rwk;
+    rwk.start(p.om, m0 + trow);
+#pragma unroll 4
+    for (int q = 0; q < TM / RPP; ++q) {
+      const long long r = m0 + trow + RPP * q;
+      if (r < p.rows && n < p.N)
+        *reinterpret_cast<u32x4*>(p.out + rwk.part(p.om) + fo) =
+            *reinterpret_cast<const u32x4*>(tile + (trow + RPP * q) * SH::OUT_PITCH + fc * 8);
+      rwk.advance(p.om, RPP);
     }
   }
 }
 
+template <int IM, int JN, int WM, int WN>
+int launch_nt(NtParams& p, hipStream_t s, const char* who) {
+  typedef NtShape<IM, JN, WM, WN> SH;
+  p.tiles_n = jg::cdiv(p.N, SH::TNF);
+  const long long tiles = (long long)jg::cdiv(p.rows, SH::TM) * p.tiles_n;
+  JG_REQUIRE(tiles < (1ll << 31), "%s: too many tiles", who);
+  void (*kern)(NtParams) = &proj_nt_kernel<IM, JN, WM, WN>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     SH::LDS);
+  if (e != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS", who, SH::LDS);
+  kern<<<(unsigned)tiles, SH::THREADS, SH::LDS, s>>>(p);
+  JG_CHECK_LAUNCH(who);
+  return JG_OK;
+}
+
 // ------------------------------------------------------------------------ TN
-constexpr int BR = 64;             // tokens per stage
-constexpr int TN_PITCH = TILE + TILE / 8;  // slots per chunk of 8 tokens: feature f at f + f / 8
-constexpr int TN_OP = 8 * TN_PITCH;
-constexpr int TN_STAGE = 2 * TN_OP;
-constexpr int TN_LDS = 2 * TN_STAGE * 16;
+constexpr int BR = 64;  // tokens per stage
 
 struct TnParams {
   const uint16_t* g;  // tokens x N
@@ -235,6 +280,20 @@ struct TnParams {
   int stages_per_split;
 };
 
+// WM x WN wavefronts, each with IM x JN blocks of 32 features of g x 32 features of x; the tile is
+// square (T x T) and the workgroup has 2 T threads: one 8 token x 8 feature block per thread and stage.
+template <int IM, int JN, int WM, int WN>
+struct TnShape {
+  static constexpr int T = 32 * IM * WM;
+  static_assert(T == 32 * JN * WN, "square tile");
+  static constexpr int THREADS = 64 * WM * WN;
+  static_assert(THREADS == 2 * T, "one block per thread");
+  static constexpr int PITCH = T + T / 8;  // slots per chunk of 8 tokens: feature f at f + f / 8
+  static constexpr int OP = 8 * PITCH;
+  static constexpr int STAGE = 2 * OP;
+  static constexpr int LDS = 2 * STAGE * 16;
+};
+
 __device__ __forceinline__ float sum_bf16x8(const u32x4& v) {
   float s = 0.0f;
 #pragma unroll
@@ -245,23 +304,26 @@ __device__ __forceinline__ float sum_bf16x8(const u32x4& v) {
   return s;
 }
 
-__global__ __launch_bounds__(THREADS) void proj_tn_kernel(TnParams p) {
+template <int IM, int JN, int WM, int WN>
+__global__ __launch_bounds__(64 * WM * WN) void proj_tn_kernel(TnParams p) {
+  typedef TnShape<IM, JN, WM, WN> SH;
+  constexpr int T = SH::T;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   u32x4* lds = reinterpret_cast<u32x4*>(smem);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, kg = lane >> 5;
-  const int wn = wave & 1, wc = wave >> 1;
+  const int wn = wave % WM, wc = wave / WM;
   const int tile_c = blockIdx.x % p.tiles_c, tile_n = blockIdx.x / p.tiles_c;
-  const int n0 = tile_n * TILE, c0 = tile_c * TILE;
+  const int n0 = tile_n * T, c0 = tile_c * T;
   const int split = blockIdx.y;
   const long long r_first = (long long)split * p.stages_per_split * BR;
   long long r_last = r_first + (long long)p.stages_per_split * BR;
   if (r_last > p.rows) r_last = p.rows;
   const int nst = r_last > r_first ? (int)((r_last - r_first + BR - 1) / BR) : 0;
 
-  // loads: waves 0-1 fetch g, waves 2-3 fetch x; a thread owns an 8 token x 8 feature block
-  const int half = tid >> 7, tt = tid & 127;
-  const int jc = tt & 15, ro = tt >> 4;
+  // loads: the first half of the threads fetches g, the second x; a thread owns an 8 token x 8 feature block
+  const int half = tid / T, tt = tid % T;
+  const int jc = tt % (T / 8), ro = tt / (T / 8);
   const Map& mp = half ? p.xm : p.gm;
   const uint16_t* src = half ? p.x : p.g;
   const int f_count = half ? p.C : p.N;
@@ -277,24 +339,25 @@ __global__ __launch_bounds__(THREADS) void proj_tn_kernel(TnParams p) {
 
   u32x4 v[8];
   long long r_loaded = 0;
+  const long long tok_stride = mp.heads ? mp.D : mp.ld;  // between consecutive tokens of one batch entry
   auto load = [&](int st) {
-    // tokens r_first + st*BR + ro*8 + i; `walk` stands at i = 0
+    // tokens r_first + st*BR + ro*8 + i, all of one batch entry (S % 8 == 0); `walk` stands at i = 0.
+    // A token past the end repeats the last one (or token 0) and is zeroed on the way to LDS.
     r_loaded = r_first + (long long)st * BR + ro * 8;
-    RowWalk w = walk;
+    const long long left = p.rows - r_loaded;
+    const int last = left >= 8 ? 7 : (left > 0 ? (int)left - 1 : 0);
+    const uint16_t* b0 = src + (left > 0 ? walk.part(mp) : 0) + fpart;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      // a token past the end is read from token 0 (always there) and zeroed on the way to LDS
-      const long long off = (r_loaded + i < p.rows) ? w.part(mp) : 0;
-      v[i] = *reinterpret_cast<const u32x4*>(src + off + fpart);
-      w.advance(mp, 1);
-    }
+    for (int i = 0; i < 8; ++i) v[i] = *reinterpret_cast<const u32x4*>(b0 + (i < last ? i : last) * tok_stride);
     walk.advance(mp, BR);
   };
   auto store = [&](int buf) {
-    u32x4* dst = lds + buf * TN_STAGE + half * TN_OP + ro * TN_PITCH + jc * 9;
+    u32x4* dst = lds + buf * SH::STAGE + half * SH::OP + ro * SH::PITCH + jc * 9;
+    if (r_loaded + 8 > p.rows) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-      if (r_loaded + i >= p.rows) v[i] = u32x4{0u, 0u, 0u, 0u};
+      for (int i = 0; i < 8; ++i)
+        if (r_loaded + i >= p.rows) v[i] = u32x4{0u, 0u, 0u, 0u};
+    }
 #pragma unroll
     for (int px = 0; px < 8; ++px) {
       const uint32_t sel = (px & 1) ? 0x07060302u : 0x05040100u;
@@ -308,32 +371,43 @@ __global__ __launch_bounds__(THREADS) void proj_tn_kernel(TnParams p) {
     }
   };
 
-  f32x16 acc[2][2];
+  f32x16 acc[IM][JN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < IM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < JN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   auto compute = [&](int buf) {
-    const u32x4* sg = lds + buf * TN_STAGE;
-    const u32x4* sx = sg + TN_OP;
-#pragma unroll
-    for (int kk = 0; kk < BR / 16; ++kk) {
+    const u32x4* sg = lds + buf * SH::STAGE;
+    const u32x4* sx = sg + SH::OP;
+    u32x4 fr[2][IM + JN];
+    auto fetch = [&](int kk, u32x4 (&fq)[IM + JN]) {
       const int cc = kk * 2 + kg;
-      bf16x8 gf[2], xf[2];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const int fg = wn * 64 + t * 32 + ln, fx = wc * 64 + t * 32 + ln;
-        gf[t] = __builtin_bit_cast(bf16x8, sg[cc * TN_PITCH + fg + (fg >> 3)]);
-        xf[t] = __builtin_bit_cast(bf16x8, sx[cc * TN_PITCH + fx + (fx >> 3)]);
+      for (int t = 0; t < IM; ++t) {
+        const int fg = (wn * IM + t) * 32 + ln;
+        fq[t] = sg[cc * SH::PITCH + fg + (fg >> 3)];
       }
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int t = 0; t < JN; ++t) {
+        const int fx = (wc * JN + t) * 32 + ln;
+        fq[IM + t] = sx[cc * SH::PITCH + fx + (fx >> 3)];
+      }
+    };
+    fetch(0, fr[0]);
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gf[i], xf[j], acc[i][j], 0, 0, 0);
+    for (int kk = 0; kk < BR / 16; ++kk) {
+      if (kk + 1 < BR / 16) fetch(kk + 1, fr[(kk + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < IM; ++i)
+#pragma unroll
+        for (int j = 0; j < JN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fr[kk & 1][i]),
+                                                              __builtin_bit_cast(bf16x8, fr[kk & 1][IM + j]), acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
@@ -349,35 +423,35 @@ __global__ __launch_bounds__(THREADS) void proj_tn_kernel(TnParams p) {
     __syncthreads();
   }
 
-  // register e of block (i, j): row n0 + wn*64 + i*32 + 8*(e/4) + 4*kg + e%4, column c0 + wc*64 + j*32 + ln
+  // register e of block (i, j): row n0 + (wn*IM + i)*32 + 8*(e/4) + 4*kg + e%4, column c0 + (wc*JN + j)*32 + ln
   float* part = p.part + (size_t)split * p.N * p.C;
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < IM; ++i)
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      const int n = n0 + wn * 64 + i * 32 + (e >> 2) * 8 + kg * 4 + (e & 3);
+      const int n = n0 + (wn * IM + i) * 32 + (e >> 2) * 8 + kg * 4 + (e & 3);
       if (n < p.N) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int cidx = c0 + wc * 64 + j * 32 + ln;
+        for (int j = 0; j < JN; ++j) {
+          const int cidx = c0 + (wc * JN + j) * 32 + ln;
           if (cidx < p.C) part[(size_t)n * p.C + cidx] = acc[i][j][e];
         }
       }
     }
 
   if (p.bias_part != nullptr && tile_c == 0) {  // uniform over the workgroup
-    float* red = reinterpret_cast<float*>(smem);  // [8 token octets][128 features]; the stages are done with
+    float* red = reinterpret_cast<float*>(smem);  // [8 token octets][T features]; the stages are done with
     if (half == 0) {
 #pragma unroll
-      for (int px = 0; px < 8; ++px) red[ro * TILE + jc * 8 + px] = bsum[px];
+      for (int px = 0; px < 8; ++px) red[ro * T + jc * 8 + px] = bsum[px];
     }
     __syncthreads();
-    if (tid < TILE) {
-      float s = 0.0f;
+    if (tid < T) {
+      float sum = 0.0f;
 #pragma unroll
-      for (int o = 0; o < 8; ++o) s += red[o * TILE + tid];
+      for (int o = 0; o < 8; ++o) sum += red[o * T + tid];
       // a clamped block would count the last features twice: only features of this tile are written
-      if (n0 + tid < p.N && (n0 + (tid & ~7) <= p.N - 8)) p.bias_part[(size_t)split * p.N + n0 + tid] = s;
+      if (n0 + tid < p.N && (n0 + (tid & ~7) <= p.N - 8)) p.bias_part[(size_t)split * p.N + n0 + tid] = sum;
     }
   }
 }
@@ -508,14 +582,43 @@ bool map_vec_ok(const Map& m, long long features) {
   if (features % 8 != 0) return false;
   return m.heads ? (m.D % 8 == 0) : (m.ld % 8 == 0);
 }
+// eight consecutive tokens starting at a multiple of 8 belong to one batch entry
+bool map_octets_ok(const Map& m) { return !m.heads || m.S % 8 == 0; }
 
-int tn_splits(long long rows, int tiles) {
+// Token ranges (splits) the contraction is cut into so that `tiles` tiles fill the chip; a
+// split is worth its partial tile from about 8 stages on.
+int splits_for(long long rows, int tiles, int target) {
   const long long stages = (rows + BR - 1) / BR;
-  long long want = (1024 + tiles - 1) / tiles;  // about four workgroups per compute unit
-  if (want > stages) want = stages;
+  long long want = (target + tiles - 1) / tiles;
+  if (want > stages / 8) want = stages / 8;
   if (want < 1) want = 1;
   if (want > 64) want = 64;
   return (int)want;
+}
+// Tile edge of the weight-gradient kernel: 256 (half the operand traffic per MFMA, one workgroup
+// per compute unit) when such tiles and their splits still fill most of the chip, else 128.
+int tn_tile(long long rows, int n, int c) {
+  if (n < 256 || c < 256) return 128;
+  const int tiles = jg::cdiv(n, 256) * jg::cdiv(c, 256);
+  return tiles * splits_for(rows, tiles, 256) >= 192 ? 256 : 128;
+}
+int tn_splits(long long rows, int n, int c) {
+  const int t = tn_tile(rows, n, c);
+  return splits_for(rows, jg::cdiv(n, t) * jg::cdiv(c, t), t == 256 ? 256 : 1024);
+}
+
+template <int IM, int JN, int WM, int WN>
+int launch_tn(TnParams& p, int splits, hipStream_t s, const char* who) {
+  typedef TnShape<IM, JN, WM, WN> SH;
+  p.tiles_c = jg::cdiv(p.C, SH::T);
+  const int tiles = jg::cdiv(p.N, SH::T) * p.tiles_c;
+  void (*kern)(TnParams) = &proj_tn_kernel<IM, JN, WM, WN>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     SH::LDS);
+  if (e != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS", who, SH::LDS);
+  kern<<<dim3((unsigned)tiles, (unsigned)splits), SH::THREADS, SH::LDS, s>>>(p);
+  JG_CHECK_LAUNCH(who);
+  return JG_OK;
 }
 
 template <bool TRANS>
@@ -550,8 +653,9 @@ int jg_proj_nt(void* out, const void* a, const void* w, const void* bias, int dt
   rc = make_map(&om, out_heads, n_out, rows, B, H, S, D, who, "output");
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool fast = dtype == JG_BF16 && map_vec_ok(am, k_in) && aligned16(a) && aligned16(w) &&
-                    rows < (1ll << 31) - TILE;
+  const bool fast = dtype == JG_BF16 && map_vec_ok(am, k_in) && map_vec_ok(om, n_out) && aligned16(a) &&
+                    aligned16(w) && aligned16(out) && rows < (1ll << 31) - 256 &&
+                    (unsigned long long)rows * k_in < (1ull << 31) && (unsigned long long)n_out * k_in < (1ull << 31);
   if (!fast) {
     GenParams gp;
     gp.p = a; gp.q = w; gp.bias = bias; gp.out = out;
@@ -566,21 +670,15 @@ int jg_proj_nt(void* out, const void* a, const void* w, const void* bias, int dt
   p.out = static_cast<uint16_t*>(out);
   p.am = am; p.om = om;
   p.rows = rows; p.N = n_out; p.K = k_in;
-  p.tiles_n = jg::cdiv(n_out, TILE);
-  const long long tiles = (long long)jg::cdiv(rows, TILE) * p.tiles_n;
-  JG_REQUIRE(tiles < (1ll << 31), "%s: too many tiles", who);
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&proj_nt_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, NT_LDS);
-  if (e != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS", who, NT_LDS);
-  proj_nt_kernel<<<(unsigned)tiles, THREADS, NT_LDS, s>>>(p);
-  JG_CHECK_LAUNCH(who);
-  return JG_OK;
+  // 256 x 256 tiles (half the operand traffic per MFMA) once they fill the chip, else 128 x 128
+  const long long big_tiles = (long long)jg::cdiv(rows, 256) * jg::cdiv(n_out, 256);
+  if (big_tiles >= 256) return launch_nt<4, 2, 2, 4>(p, s, who);
+  return launch_nt<2, 2, 2, 2>(p, s, who);
 }
 
 size_t jg_proj_tn_workspace(int64_t rows, int n, int c) {
   if (rows <= 0 || n <= 0 || c <= 0) return 0;
-  const int tiles = jg::cdiv(n, TILE) * jg::cdiv(c, TILE);
-  const size_t splits = (size_t)tn_splits(rows, tiles);
+  const size_t splits = (size_t)tn_splits(rows, n, c);
   return splits * ((size_t)n * c + n) * sizeof(float);
 }
 
@@ -596,7 +694,8 @@ int jg_proj_tn(void* gw, void* gb, const void* g, const void* x, int dtype, int6
   rc = make_map(&xm, x_heads, c, rows, B, H, S, D, who, "input");
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool fast = dtype == JG_BF16 && map_vec_ok(gm, n) && map_vec_ok(xm, c) && aligned16(g) && aligned16(x);
+  const bool fast = dtype == JG_BF16 && map_vec_ok(gm, n) && map_vec_ok(xm, c) && map_octets_ok(gm) &&
+                    map_octets_ok(xm) && aligned16(g) && aligned16(x);
   if (!fast) {
     GenParams gp;
     gp.p = g; gp.q = x; gp.bias = nullptr; gp.out = gw;
@@ -623,18 +722,13 @@ int jg_proj_tn(void* gw, void* gb, const void* g, const void* x, int dtype, int6
   p.x = static_cast<const uint16_t*>(x);
   p.gm = gm; p.xm = xm;
   p.rows = rows; p.N = n; p.C = c;
-  p.tiles_c = jg::cdiv(c, TILE);
-  const int tiles = jg::cdiv(n, TILE) * p.tiles_c;
-  const int splits = tn_splits(rows, tiles);
+  const int splits = tn_splits(rows, n, c);
   const long long stages = (rows + BR - 1) / BR;
   p.stages_per_split = (int)((stages + splits - 1) / splits);
   p.part = static_cast<float*>(workspace);
   p.bias_part = gb != nullptr ? p.part + (size_t)splits * n * c : nullptr;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&proj_tn_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, TN_LDS);
-  if (e != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS", who, TN_LDS);
-  proj_tn_kernel<<<dim3((unsigned)tiles, (unsigned)splits), THREADS, TN_LDS, s>>>(p);
-  JG_CHECK_LAUNCH(who);
+  rc = tn_tile(rows, n, c) == 256 ? launch_tn<4, 2, 2, 4>(p, splits, s, who) : launch_tn<2, 2, 2, 2>(p, splits, s, who);
+  if (rc) return rc;
   const size_t count = (size_t)n * c;
   proj_reduce_kernel<<<(unsigned)((count + 255) / 256), 256, 0, s>>>(static_cast<uint16_t*>(gw), p.part, splits, count);
   JG_CHECK_LAUNCH(who);

@@ -22,6 +22,7 @@ import torch.nn as nn
 from .attention import window_attention
 from .conv import TileGroup
 from .layernorm import layer_norm
+from .projection import heads_projection, qkv_projection
 from .roll import _Roll
 
 
@@ -134,12 +135,18 @@ class WindowAttention(nn.Module):
         b, h, w, c = x.shape
         x = windows(x, self.window)
         n = x.shape[2]
-        qkv = token_linear(x, self.qkv).view(b, -1, n, 3, self.heads, c // self.heads)
-        q, k, v = qkv.permute(3, 0, 1, 4, 2, 5).unbind(0)  # (B, nW, heads, N, d)
+        fused = x.dtype == torch.bfloat16  # the projections write / read the head layout themselves
+        if fused:
+            q, k, v = qkv_projection(x, self.qkv.weight, self.qkv.bias, self.heads).unbind(0)
+        else:
+            qkv = token_linear(x, self.qkv).view(b, -1, n, 3, self.heads, c // self.heads)
+            q, k, v = (t.contiguous() for t in qkv.permute(3, 0, 1, 4, 2, 5).unbind(0))  # (B, nW, heads, N, d)
         bias = self.bias_table[self.index.view(-1)].view(n, n, -1).permute(2, 0, 1).float()
         if self.mask is not None:
             bias = bias[None] + self.mask[:, None]  # (nW, heads, N, N)
-        out = window_attention(q.contiguous(), k.contiguous(), v.contiguous(), bias.contiguous())
+        out = window_attention(q, k, v, bias.contiguous())
+        if fused:
+            return unwindows(heads_projection(out, self.proj.weight, self.proj.bias), h, w, self.window)
         out = out.transpose(2, 3).reshape(b, -1, n, c)
         return unwindows(token_linear(out, self.proj), h, w, self.window)
 
