@@ -221,6 +221,34 @@ def groupnorm_figures(dev, iters: int) -> dict:
     }
 
 
+def projection_figures(dev, iters: int) -> dict:
+    """The projections around the attention core with the head split / merge fused into the
+    GEMM addressing, on 8 sequences of configuration 4 (32768 tokens, 512 channels, 8 heads
+    of 64, bf16): qkv projection writing (3, b, h, s, d), output projection reading
+    (b, h, s, d); the qkv backward is the input gradient (one GEMM) plus the weight and
+    bias gradient (one GEMM contracted over the tokens and its reduction)."""
+    from jigsaw_amd import projection as jp
+
+    g = torch.Generator(device=dev).manual_seed(4)
+    bsz, s, c, heads = 8, 4096, 512, 8
+    x = torch.randn(bsz, s, c, device=dev, generator=g).bfloat16().requires_grad_()
+    w = (torch.randn(3 * c, c, device=dev, generator=g) / c ** 0.5).bfloat16().requires_grad_()
+    b = (0.1 * torch.randn(3 * c, device=dev, generator=g)).bfloat16().requires_grad_()
+    wo = (torch.randn(c, c, device=dev, generator=g) / c ** 0.5).bfloat16()
+    o = torch.randn(bsz, heads, s, c // heads, device=dev, generator=g).bfloat16()
+    gy = torch.randn(3, bsz, heads, s, c // heads, device=dev, generator=g).bfloat16()
+    flops = 2.0 * bsz * s * c * 3 * c
+    ms_qkv = time_gpu(lambda: jp.qkv_projection(x.detach(), w.detach(), b.detach(), heads), iters)
+    ms_out = time_gpu(lambda: jp.heads_projection(o, wo, None), iters)
+    y = jp.qkv_projection(x, w, b, heads)
+    ms_bwd = time_gpu(lambda: torch.autograd.grad(y, (x, w, b), gy, retain_graph=True), iters)
+    return {
+        "qkv_projection_fwd": {"ms": ms_qkv, "TFLOPs": flops / (ms_qkv * 1e-3) / 1e12},
+        "heads_projection_fwd": {"ms": ms_out, "TFLOPs": flops / 3 / (ms_out * 1e-3) / 1e12},
+        "qkv_projection_bwd": {"ms": ms_bwd, "TFLOPs": 2 * flops / (ms_bwd * 1e-3) / 1e12},
+    }
+
+
 def swin_figures(dev, iters: int) -> dict:
     """Configuration 5: one rank's Swin block on a 256x256-token tile, dim 128, 4 heads,
     8x8 windows, shift 4, bf16 autocast; the roll's cross-tile slabs are seeded."""
@@ -441,6 +469,7 @@ def main() -> int:
         extra.update(conv3d_figures(dev, it))
         extra.update(swin_figures(dev, it))
         extra.update(groupnorm_figures(dev, it))
+        extra.update(projection_figures(dev, it))
 
     line = {
         "metric": METRIC,
