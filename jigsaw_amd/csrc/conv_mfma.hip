@@ -64,12 +64,13 @@ struct FwdParams {
   const uint16_t* bias; // (M,) or NULL
   uint16_t* y;          // (N, M, Dout, Hout, Wout)
   int N, C, M;          // batch, channels of x, produced channels
+  int Cp;               // C rounded up to a multiple of 16: contraction channels per depth tap
   int KD;               // depth taps (1 for 2-D); contraction channels K = KD * C
   int Din, Hin, Win, Dout, Hout, Wout;
   int pad_d, pad_h, pad_w;  // virtual zero padding of x
   int tiles_h, tiles_w;
   int total_tiles;      // N * Dout * tiles_h * tiles_w
-  int nc16;             // KD * C / 16
+  int nc16;             // KD * Cp / 16
   int wc16;             // 16-channel steps whose weights sit in LDS at a time (a group)
   int ngroups;          // ceil(nc16 / wc16); > 1: the weights are reloaded group by group
   // Fold mode (input gradient written to its owners): y is the unpadded tile
@@ -102,14 +103,14 @@ __device__ __forceinline__ void* strip_entry(int idx) {
 
 // ---------------------------------------------------------------- weight prep
 // dst[(((mt*ngroups + group)*9 + tap9)*wc16 + c16 in group)*2 + kg][m_local][8 k] (bf16), contraction channel
-// k = kd*C + c. transposed = 0: A[m][k] = w[m][c][kd][kh][kw] (forward, w is
+// k = kd*Cp + c (channels C..Cp-1 are zero padding). transposed = 0: A[m][k] = w[m][c][kd][kh][kw] (forward, w is
 // (M, C, KD, 3, 3)); transposed = 1: A[m][k] = w[c][m][KD-1-kd][2-kh][2-kw] (input
 // gradient, w is (C, M, KD, 3, 3)).
 __global__ __launch_bounds__(256) void prep_weights_kernel(uint16_t* __restrict__ dst,
                                                            const uint16_t* __restrict__ w,
-                                                           int M, int C, int KD, int MT, int mtiles,
+                                                           int M, int C, int Cp, int KD, int MT, int mtiles,
                                                            int wc16, int ngroups, int transposed) {
-  const int K = KD * C;
+  const int K = KD * Cp;
   const int total = mtiles * ngroups * TAPS * wc16 * 2 * MT * 8;
   for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
     int e = i & 7;
@@ -123,8 +124,8 @@ __global__ __launch_bounds__(256) void prep_weights_kernel(uint16_t* __restrict_
     const int m = mt * MT + ml;
     const int k = (grp * wc16 + c16l) * CK + kg * 8 + e;
     uint16_t v = 0;  // rows past M and steps past K are padding
-    if (m < M && k < K) {
-      const int kd = k / C, c = k - kd * C;
+    const int kd = k / Cp, c = k - kd * Cp;
+    if (m < M && k < K && c < C) {
       const int kh = tap / KW, kw = tap % KW;
       if (!transposed)
         v = w[((((size_t)m * C + c) * KD + kd) * KH + kh) * KW + kw];
@@ -231,7 +232,11 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
 
   auto issue_loads = [&](int tile, int c16) {
     const TileCoord tc = coord(tile);
-    const int kd = (c16 * CK) / p.C, c0 = c16 * CK - kd * p.C;
+    const int kd = (c16 * CK) / p.Cp, c0 = c16 * CK - kd * p.Cp;
+    // Channels of this task that exist (all 8 unless C is not a multiple of 16). The vector
+    // path below reads the others anyway (they lie inside the tensor: the interior test covers
+    // all 16 channel planes) and store_stage zeroes them; the guarded paths skip them.
+    const int cvalid = p.C - c0 - g8 * 8;
     const int id = tc.od + kd - p.pad_d;
     const int ih0 = tc.th * TH - p.pad_h, iw0 = tc.tw * TW - p.pad_w;
     const bool depth_ok = id >= 0 && id < p.Din;
@@ -316,12 +321,13 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
       for (int c = 0; c < 8; ++c)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          stg[c][j] = ok[j] ? *reinterpret_cast<const uint32_t*>(a + (size_t)c * chan_b + 4 * j) : 0u;
+          stg[c][j] = (ok[j] && c < cvalid) ? *reinterpret_cast<const uint32_t*>(a + (size_t)c * chan_b + 4 * j) : 0u;
     } else {
       const int ih = ih0 + t_row, iw = iw0 + t_col;
-      const bool row_ok = depth_ok && (ih >= 0) && (ih < p.Hin);
+      const bool rows_ok = depth_ok && (ih >= 0) && (ih < p.Hin);
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
+        const bool row_ok = rows_ok && c < cvalid;
         const uint16_t* e = reinterpret_cast<const uint16_t*>(a + (size_t)c * chan_b);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -333,8 +339,16 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     }
   };
 
-  auto store_stage = [&](int buf) {
+  auto store_stage = [&](int buf, int c16) {
     if (!has_task) return;
+    if (p.Cp != p.C) {  // uniform: zero the channels of this step that do not exist
+      const int cvalid = p.C - (c16 * CK) % p.Cp - g8 * 8;
+#pragma unroll
+      for (int c = 0; c < 8; ++c)
+        if (c >= cvalid) {
+          stg[c][0] = 0u; stg[c][1] = 0u; stg[c][2] = 0u; stg[c][3] = 0u;
+        }
+    }
     u32x4* row_base = lds_in + buf * STAGE_SLOTS + t_lds;
 #pragma unroll
     for (int px = 0; px < 8; ++px) {
@@ -541,7 +555,7 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
   };
   int buf = 0;
   issue_stage(0);
-  store_stage(0);
+  store_stage(0, 0);
   if (stages > 1) issue_stage(1);
   __syncthreads();
   int q = 0;
@@ -555,7 +569,7 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
       }
       compute_kw(buf, c16, 0);
       compute_kw(buf, c16, 1);
-      if (q + 1 < stages) store_stage(buf ^ 1);  // other buffer: no hazard with this stage's reads
+      if (q + 1 < stages) store_stage(buf ^ 1, c16 + 1 < p.nc16 ? c16 + 1 : 0);  // other buffer: no hazard with this stage's reads
       if (q + 2 < stages) issue_stage(q + 2);
       compute_kw(buf, c16, 2);
       __syncthreads();
@@ -586,6 +600,9 @@ struct Layout {
   size_t prep_bytes, lds_bytes;
 };
 
+int pad16(int c) { return (c + CK - 1) / CK * CK; }
+
+// K: contraction length with the channels padded to a multiple of 16 per depth tap
 Layout layout_of(int K, int M) {
   Layout L;
   const int mpad = (M + 31) / 32 * 32;
@@ -611,7 +628,7 @@ bool shape_ok(int C, int M, const ConvGeom& g) {
   if (g.k[0] == 1 && (g.in[0] != 1 || g.p[0] != 0)) return false;
   for (int a = 0; a < 3; ++a)
     if (g.s[a] != 1 || g.d[a] != 1) return false;
-  if (C % CK != 0 || C <= 0 || M <= 0) return false;
+  if (C <= 0 || M <= 0) return false;
   // per-lane byte offsets inside one batch entry are 32-bit
   const size_t in_sz = (size_t)g.in[0] * g.in[1] * g.in[2], out_sz = (size_t)g.out[0] * g.out[1] * g.out[2];
   const size_t big = in_sz > out_sz ? in_sz : out_sz;
@@ -637,7 +654,7 @@ struct Launch {
 };
 
 int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const char* who) {
-  const int K = L.KD * L.C;
+  const int K = L.KD * pad16(L.C);
   if (ws == nullptr || ws_bytes < prep_bytes(K, L.M))
     JG_FAIL(JG_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, prep_bytes(K, L.M));
   JG_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 15) == 0, "%s: workspace must be 16-byte aligned",
@@ -647,7 +664,7 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   uint16_t* wprep = static_cast<uint16_t*>(ws);
   const size_t total_w = lay.prep_bytes / 2;
   JG_REQUIRE(total_w < (1ull << 31), "%s: weight tensor too large", who);
-  prep_weights_kernel<<<(unsigned)((total_w + 255) / 256), 256, 0, s>>>(wprep, L.w, L.M, L.C, L.KD, MT, lay.mtiles,
+  prep_weights_kernel<<<(unsigned)((total_w + 255) / 256), 256, 0, s>>>(wprep, L.w, L.M, L.C, pad16(L.C), L.KD, MT, lay.mtiles,
                                                                          lay.wc16, lay.ngroups, L.transposed);
   JG_CHECK_LAUNCH(who);
 
@@ -655,6 +672,7 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   p.x_end = reinterpret_cast<const char*>(L.x) + 2 * (size_t)L.N * L.C * L.Din * L.Hin * L.Win;
   p.x = L.x; p.wprep = reinterpret_cast<const u32x4*>(wprep); p.bias = L.bias; p.y = L.y;
   p.N = L.N; p.C = L.C; p.M = L.M; p.KD = L.KD;
+  p.Cp = pad16(L.C);
   p.Din = L.Din; p.Hin = L.Hin; p.Win = L.Win;
   p.Dout = L.Dout; p.Hout = L.Hout; p.Wout = L.Wout;
   p.pad_d = L.pad_d; p.pad_h = L.pad_h; p.pad_w = L.pad_w;
@@ -715,8 +733,8 @@ bool mfma_dgrad_supported(const ConvGeom& g, int dtype) {
   return shape_ok(g.cout, g.cin, g);
 }
 
-size_t mfma_fwd_workspace(const ConvGeom& g) { return prep_bytes(g.k[0] * g.cin, g.cout); }
-size_t mfma_dgrad_workspace(const ConvGeom& g) { return prep_bytes(g.k[0] * g.cout, g.cin); }
+size_t mfma_fwd_workspace(const ConvGeom& g) { return prep_bytes(g.k[0] * pad16(g.cin), g.cout); }
+size_t mfma_dgrad_workspace(const ConvGeom& g) { return prep_bytes(g.k[0] * pad16(g.cout), g.cin); }
 
 static int fwd_launch(void* y, const void* x, const void* xt, const int* tlo, const int* tn, const void* w,
                       const void* bias, const ConvGeom& g, void* ws, size_t ws_bytes, hipStream_t s,
@@ -822,7 +840,7 @@ int mfma_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, void*
 int mfma_dgrad_fold(void* gx, void* const strips[27], const int lo[3], const int n[3], const void* w,
                     const void* go, const ConvGeom& g, void* ws, size_t ws_bytes, hipStream_t s) {
   // the fold epilogue has no path for a ragged last tile of produced channels
-  const Layout lay = layout_of(g.k[0] * g.cout, g.cin);
+  const Layout lay = layout_of(g.k[0] * pad16(g.cout), g.cin);
   if (lay.mtiles * lay.MT != g.cin)
     JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_dgrad_fold(mfma): %d input channels are not a multiple of %d", g.cin, lay.MT);
   return dgrad_launch(gx, strips, lo, n, w, go, g, ws, ws_bytes, s, "jg_conv_dgrad_fold(mfma)");

@@ -46,6 +46,10 @@ PRIM_CASES = [
     (1, 256, 64, (18, 34), (3, 3), (1, 1), (0, 0), (1, 1)),
     (1, 96, 32, (5, 18, 34), (3, 3, 3), (1, 1, 1), (1, 0, 1), (1, 1, 1)),
     (1, 80, 16, (4, 20, 36), (3, 3, 3), (1, 1, 1), (0, 0, 0), (1, 1, 1)),
+    # contraction channels that are not a multiple of the 16-channel MFMA step (first / last layers)
+    (2, 69, 64, (37, 66), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (1, 64, 69, (20, 70), (3, 3), (1, 1), (1, 1), (1, 1)),
+    (2, 20, 24, (5, 18, 34), (3, 3, 3), (1, 1, 1), (1, 0, 1), (1, 1, 1)),
 ]
 
 
@@ -87,6 +91,25 @@ def test_conv_primitives_match_oracle(case, dtype, dev):
     gw2, gb2 = jc.conv_nd_weight(xg, w.shape, gg, stride=s, padding=p, dilation=d, with_bias_grad=True)
     assert torch.equal(gw2, gw)
     assert gb2.dtype == dtype and rel_l2(gb2, gb_want) < TOL[dtype], f"fused bias grad rel-L2 {rel_l2(gb2, gb_want):.3e}"
+
+
+def test_partial_channel_step_ignores_what_lies_behind_the_last_channel(dev):
+    """3 input channels fill 3 of the 16 slots of an MFMA step; the slots behind them are read
+    from whatever follows in memory (the next batch entry) and must not reach the result:
+    batch entry 1 is all NaN, batch entry 0 must still match the oracle (and stay finite)."""
+    torch.manual_seed(3)
+    x = torch.randn(2, 3, 40, 70).bfloat16()
+    x[1] = float("nan")
+    w = ((torch.rand(16, 3, 3, 3) * 2 - 1) / 27**0.5).bfloat16()
+    y = jc.conv_nd(x.to(dev), w.to(dev), None)
+    assert torch.isfinite(y[0]).all() and torch.isnan(y[1]).all()
+    assert rel_l2(y[0:1], oc.forward(x[0:1].double(), w.double(), None, (1, 1), (0, 0), (1, 1))) < TOL[torch.bfloat16]
+    g = torch.randn(2, 3, 38, 68).bfloat16()  # gradient of a 16 -> 3 layer: dgrad contracts over 3 channels
+    g[1] = float("nan")
+    wt = ((torch.rand(3, 16, 3, 3) * 2 - 1) / 12).bfloat16()
+    gx = jc.conv_nd_input((2, 16, 40, 70), wt.to(dev), g.to(dev))
+    assert torch.isfinite(gx[0]).all()
+    assert rel_l2(gx[0:1], oc.dgrad((1, 16, 40, 70), wt.double(), g[0:1].double(), (1, 1), (0, 0), (1, 1))) < TOL[torch.bfloat16]
 
 
 def test_conv_argument_errors(dev):
