@@ -45,11 +45,11 @@ extern "C" size_t jg_conv_workspace_bytes(const jg_conv_desc* desc, int op, int 
   if (jg::resolve_conv(desc, "jg_conv_workspace_bytes", &g) != JG_OK) return 0;
   switch (op) {
     case JG_CONV_FWD:
-      return jg::mfma_fwd_supported(g, dtype) ? jg::mfma_fwd_workspace(g) : 0;
+      return jg::mfma_fwd_supported(g, dtype) ? jg::mfma_fwd_workspace(g, dtype) : 0;
     case JG_CONV_DGRAD:
-      return jg::mfma_dgrad_supported(g, dtype) ? jg::mfma_dgrad_workspace(g) : 0;
+      return jg::mfma_dgrad_supported(g, dtype) ? jg::mfma_dgrad_workspace(g, dtype) : 0;
     case JG_CONV_WGRAD:
-      return jg::mfma_wgrad_supported(g, dtype) ? jg::mfma_wgrad_workspace(g)
+      return jg::mfma_wgrad_supported(g, dtype) ? jg::mfma_wgrad_workspace(g, dtype)
                                                 : jg::direct_wgrad_workspace(g);
     default:
       return 0;
@@ -65,7 +65,7 @@ extern "C" int jg_conv_fwd(void* y, const void* x, const void* w, const void* bi
   JG_REQUIRE(y && x && w, "jg_conv_fwd: NULL pointer");
   JG_REQUIRE(known(dtype), "jg_conv_fwd: unknown dtype %d", dtype);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (jg::mfma_fwd_supported(g, dtype)) return jg::mfma_fwd(y, x, w, bias, g, workspace, workspace_bytes, s);
+  if (jg::mfma_fwd_supported(g, dtype)) return jg::mfma_fwd(y, x, w, bias, g, workspace, workspace_bytes, s, dtype);
   return jg::direct_fwd(y, x, w, bias, g, dtype, s);
 }
 
@@ -77,7 +77,7 @@ extern "C" int jg_conv_dgrad(void* gx, const void* w, const void* go, const jg_c
   JG_REQUIRE(gx && w && go, "jg_conv_dgrad: NULL pointer");
   JG_REQUIRE(known(dtype), "jg_conv_dgrad: unknown dtype %d", dtype);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (jg::mfma_dgrad_supported(g, dtype)) return jg::mfma_dgrad(gx, w, go, g, workspace, workspace_bytes, s);
+  if (jg::mfma_dgrad_supported(g, dtype)) return jg::mfma_dgrad(gx, w, go, g, workspace, workspace_bytes, s, dtype);
   return jg::direct_dgrad(gx, w, go, g, dtype, s);
 }
 
@@ -99,7 +99,7 @@ extern "C" int jg_conv_dgrad_fold(void* gx, void* const send[27], const void* w,
                "jg_conv_dgrad_fold: axis %d: lo %d + size %d + hi %d != padded extent %d", a, lo[a], n[a],
                geom->hi[a], g.in[a]);
   }
-  if (!jg::mfma_dgrad_supported(g, dtype))
+  if (dtype != JG_BF16 || !jg::mfma_dgrad_supported(g, dtype))
     JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_dgrad_fold: geometry / dtype only has the unfused path");
   return jg::mfma_dgrad_fold(gx, send, lo, n, w, go, g, workspace, workspace_bytes,
                              static_cast<hipStream_t>(stream));
@@ -114,7 +114,7 @@ extern "C" int jg_conv_wgrad(void* gw, const void* x, const void* go, const jg_c
   JG_REQUIRE(known(dtype), "jg_conv_wgrad: unknown dtype %d", dtype);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (jg::mfma_wgrad_supported(g, dtype))
-    return jg::mfma_wgrad(gw, nullptr, x, go, g, workspace, workspace_bytes, s);
+    return jg::mfma_wgrad(gw, nullptr, x, go, g, workspace, workspace_bytes, s, nullptr, nullptr, nullptr, dtype);
   return jg::direct_wgrad(gw, x, go, g, dtype, workspace, workspace_bytes, s);
 }
 
@@ -144,7 +144,7 @@ extern "C" int jg_conv_frame_bands(const jg_conv_desc* desc, const jg_halo_geom*
   int tlo[3], tn[3];
   rc = framed_extent(g, geom, "jg_conv_frame_bands", tlo, tn);
   if (rc) return rc;
-  if (!jg::mfma_fwd_supported(g, dtype) || !jg::mfma_wgrad_supported(g, dtype) ||
+  if (dtype != JG_BF16 || !jg::mfma_fwd_supported(g, dtype) || !jg::mfma_wgrad_supported(g, dtype) ||
       !jg::mfma_wgrad_frame_ok(g, tlo, tn))
     JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_frame_bands: geometry / dtype has no framed kernels");
   int blo[3], bhi[3];
@@ -168,7 +168,7 @@ extern "C" int jg_conv_fwd_framed(void* y, const void* x_frame, const void* x_ti
   int tlo[3], tn[3];
   rc = framed_extent(g, geom, "jg_conv_fwd_framed", tlo, tn);
   if (rc) return rc;
-  if (!jg::mfma_fwd_supported(g, dtype) || tn[2] % 2 != 0)
+  if (dtype != JG_BF16 || !jg::mfma_fwd_supported(g, dtype) || tn[2] % 2 != 0)
     JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_fwd_framed: geometry / dtype has no framed kernel");
   return jg::mfma_fwd_framed(y, x_frame, x_tile, tlo, tn, w, bias, g, workspace, workspace_bytes,
                              static_cast<hipStream_t>(stream));
@@ -186,7 +186,7 @@ extern "C" int jg_conv_wgrad_framed(void* gw, void* gb, const void* x_frame, con
   int tlo[3], tn[3];
   rc = framed_extent(g, geom, "jg_conv_wgrad_framed", tlo, tn);
   if (rc) return rc;
-  if (!jg::mfma_wgrad_supported(g, dtype))
+  if (dtype != JG_BF16 || !jg::mfma_wgrad_supported(g, dtype))
     JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_wgrad_framed: geometry / dtype has no framed kernel");
   return jg::mfma_wgrad(gw, gb, x_frame, go, g, workspace, workspace_bytes, static_cast<hipStream_t>(stream),
                         x_tile, tlo, tn);
@@ -200,7 +200,7 @@ extern "C" int jg_conv_wgrad_bias(void* gw, void* gb, const void* x, const void*
   if (rc) return rc;
   JG_REQUIRE(gw && gb && x && go, "jg_conv_wgrad_bias: NULL pointer");
   JG_REQUIRE(known(dtype), "jg_conv_wgrad_bias: unknown dtype %d", dtype);
-  if (!jg::mfma_wgrad_supported(g, dtype))
+  if (dtype != JG_BF16 || !jg::mfma_wgrad_supported(g, dtype))
     JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_wgrad_bias: geometry / dtype only has the separate kernels");
   return jg::mfma_wgrad(gw, gb, x, go, g, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }

@@ -30,11 +30,11 @@ int direct_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, int
 bool mfma_fwd_supported(const ConvGeom& g, int dtype);
 bool mfma_dgrad_supported(const ConvGeom& g, int dtype);
 bool mfma_wgrad_supported(const ConvGeom& g, int dtype);
-size_t mfma_fwd_workspace(const ConvGeom& g);
-size_t mfma_dgrad_workspace(const ConvGeom& g);
-size_t mfma_wgrad_workspace(const ConvGeom& g);
+size_t mfma_fwd_workspace(const ConvGeom& g, int dtype = JG_BF16);
+size_t mfma_dgrad_workspace(const ConvGeom& g, int dtype = JG_BF16);
+size_t mfma_wgrad_workspace(const ConvGeom& g, int dtype = JG_BF16);
 int mfma_fwd(void* y, const void* x, const void* w, const void* bias, const ConvGeom& g,
-             void* ws, size_t ws_bytes, hipStream_t s);
+             void* ws, size_t ws_bytes, hipStream_t s, int dtype = JG_BF16);
 // Framed input: x_frame has the padded geometry g.in but only a frame near its edges holds
 // data (mfma_frame_bands); the own tile xt sits at [tlo, tlo + tn) inside it.
 int mfma_fwd_framed(void* y, const void* x_frame, const void* xt, const int tlo[3], const int tn[3],
@@ -43,7 +43,7 @@ int mfma_fwd_framed(void* y, const void* x_frame, const void* xt, const int tlo[
 bool mfma_wgrad_frame_ok(const ConvGeom& g, const int tlo[3], const int tn[3]);
 void mfma_frame_bands(const ConvGeom& g, const int tlo[3], const int tn[3], int band_lo[3], int band_hi[3]);
 int mfma_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, void* ws,
-               size_t ws_bytes, hipStream_t s);
+               size_t ws_bytes, hipStream_t s, int dtype = JG_BF16);
 // Input gradient split between the unpadded tile and the neighbours' strips: the produced
 // (padded) tensor has extent g.in; [lo, lo + n) of it is the tile.
 int mfma_dgrad_fold(void* gx, void* const strips[27], const int lo[3], const int n[3], const void* w,
@@ -52,6 +52,9 @@ int mfma_dgrad_fold(void* gx, void* const strips[27], const int lo[3], const int
 // xt / tlo / tn: framed input as for mfma_fwd_framed, or NULL
 int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom& g, void* ws,
                size_t ws_bytes, hipStream_t s, const void* xt = nullptr, const int* tlo = nullptr,
-               const int* tn = nullptr);
+               const int* tn = nullptr, int dtype = JG_BF16);
+// dst (batch, 3, per_batch) bf16 = high / middle / low bf16 parts of src (batch, per_batch) fp32,
+// whose sum is src: the operand layout of the fp32 ("split") mode of the MFMA kernels.
+int split3_bf16(uint16_t* dst, const float* src, size_t batch, size_t per_batch, hipStream_t s);
 
 }  // namespace jg

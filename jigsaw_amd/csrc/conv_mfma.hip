@@ -65,6 +65,13 @@ struct FwdParams {
   uint16_t* y;          // (N, M, Dout, Hout, Wout)
   int N, C, M;          // batch, channels of x, produced channels
   int Cp;               // C rounded up to a multiple of 16: contraction channels per depth tap
+  // Split mode (fp32 operands as sums of three bf16 parts): x holds Cx = 3 C channels per batch
+  // entry ([high | middle | low] parts), the contraction runs over nblk = 6 blocks of KD * Cp
+  // channels, block b reads part (xmap >> 2 b) & 3 of x against the weight part the
+  // preparation put there. Plain mode: nblk = 1, xmap = 0, Cx = C.
+  int nblk, Cx;
+  uint32_t xmap;
+  int out32;            // y (and bias) are fp32
   int KD;               // depth taps (1 for 2-D); contraction channels K = KD * C
   int Din, Hin, Win, Dout, Hout, Wout;
   int pad_d, pad_h, pad_w;  // virtual zero padding of x
@@ -136,6 +143,74 @@ __global__ __launch_bounds__(256) void prep_weights_kernel(uint16_t* __restrict_
   }
 }
 
+// ---------------------------------------------------------------- split mode
+// An fp32 value is the sum of three bf16 parts (8 + 8 + 8 significand bits): high = bf16(v),
+// middle = bf16(v - high), low = bf16(v - high - middle); the subtractions are exact. A
+// product of two fp32 values is then, to 2^-24 relative, the sum of the six part products
+// whose indices add up to at most 2, each of which the bf16 matrix cores form exactly and
+// add in fp32.
+__device__ __forceinline__ uint16_t split_part(float v, int part) {
+  const uint16_t hi = jg::f32_to_bf16(v);
+  if (part == 0) return hi;
+  const float hf = jg::bf16_to_f32(hi);
+  const float r1 = (hf - hf == 0.0f) ? v - hf : 0.0f;  // an infinite (or NaN) high part carries everything
+  const uint16_t mid = jg::f32_to_bf16(r1);
+  if (part == 1) return mid;
+  return jg::f32_to_bf16(r1 - jg::bf16_to_f32(mid));
+}
+__constant__ const int kWeightPart[6] = {0, 1, 0, 2, 1, 0};  // weight part of contraction block b
+constexpr uint32_t kInputParts = 0u | (0u << 2) | (1u << 4) | (0u << 6) | (1u << 8) | (2u << 10);  // input part of block b
+
+// dst (batch, 3, per_batch) bf16 = the three parts of src (batch, per_batch) fp32
+__global__ __launch_bounds__(256) void split3_kernel(uint16_t* __restrict__ dst, const float* __restrict__ src,
+                                                     size_t per_batch, size_t total) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+    const size_t n = i / per_batch, r = i - n * per_batch;
+    const float v = src[i];
+    const uint16_t hi = jg::f32_to_bf16(v);
+    const float hf = jg::bf16_to_f32(hi);
+    const float r1 = (hf - hf == 0.0f) ? v - hf : 0.0f;
+    const uint16_t mid = jg::f32_to_bf16(r1);
+    const uint16_t lo = jg::f32_to_bf16(r1 - jg::bf16_to_f32(mid));
+    uint16_t* d = dst + n * 3 * per_batch + r;
+    d[0] = hi;
+    d[per_batch] = mid;
+    d[2 * per_batch] = lo;
+  }
+}
+
+// prep_weights_kernel for split mode: w is fp32, the contraction has 6 blocks of KD * Cp
+// channels, block b holds part kWeightPart[b] of the weights.
+__global__ __launch_bounds__(256) void prep_weights_split_kernel(uint16_t* __restrict__ dst,
+                                                                 const float* __restrict__ w, int M, int C, int Cp,
+                                                                 int KD, int MT, int mtiles, int wc16, int ngroups,
+                                                                 int transposed) {
+  const int KB = KD * Cp, K = 6 * KB;
+  const int total = mtiles * ngroups * TAPS * wc16 * 2 * MT * 8;
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
+    int e = i & 7;
+    int r = i >> 3;
+    int ml = r % MT; r /= MT;
+    int kg = r & 1; r >>= 1;
+    int c16l = r % wc16; r /= wc16;
+    int tap = r % TAPS; r /= TAPS;
+    int grp = r % ngroups;
+    int mt = r / ngroups;
+    const int m = mt * MT + ml;
+    const int k = (grp * wc16 + c16l) * CK + kg * 8 + e;
+    const int blk = k / KB, kin = k - blk * KB;
+    const int kd = kin / Cp, c = kin - kd * Cp;
+    uint16_t v = 0;
+    if (m < M && k < K && c < C) {
+      const int kh = tap / KW, kw = tap % KW;
+      const float f = !transposed ? w[((((size_t)m * C + c) * KD + kd) * KH + kh) * KW + kw]
+                                  : w[((((size_t)c * M + m) * KD + (KD - 1 - kd)) * KH + (KH - 1 - kh)) * KW + (KW - 1 - kw)];
+      v = split_part(f, kWeightPart[blk]);
+    }
+    dst[i] = v;
+  }
+}
+
 // ------------------------------------------------------------ forward kernel
 // EVEN: Win, pad_w and the plane size are even and x is 4-byte aligned, so every
 // pixel pair of a task is one aligned dword that is either wholly inside or wholly
@@ -149,6 +224,9 @@ __device__ inline void store_bf16_lo(const void* base, uint32_t lane_off, uint32
 }
 __device__ inline void store_bf16_hi(const void* base, uint32_t lane_off, uint32_t pair) {
   asm volatile("global_store_short_d16_hi %0, %1, %2" : : "v"(lane_off), "v"(pair), "s"(base) : "memory");
+}
+__device__ inline void store_f32(const void* base, uint32_t lane_off, float v) {
+  asm volatile("global_store_dword %0, %1, %2" : : "v"(lane_off), "v"(v), "s"(base) : "memory");
 }
 
 template <int MT, bool EVEN, bool FOLD, bool FRAMED>  // MT = produced channels per workgroup: 32 or 64
@@ -196,7 +274,9 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
   };
   if (p.ngroups == 1) load_weights(0);
   if (tid < MT)
-    lds_bias[tid] = (p.bias != nullptr && mt * MT + tid < p.M) ? jg::bf16_to_f32(p.bias[mt * MT + tid]) : 0.0f;
+    lds_bias[tid] = (p.bias == nullptr || mt * MT + tid >= p.M) ? 0.0f
+                    : p.out32 ? reinterpret_cast<const float*>(p.bias)[mt * MT + tid]
+                              : jg::bf16_to_f32(p.bias[mt * MT + tid]);
 
   // ---- prefetch bookkeeping. A task = 8 channels x 8 pixels of one input row.
   const size_t plane = (size_t)p.Hin * p.Win;
@@ -232,7 +312,10 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
 
   auto issue_loads = [&](int tile, int c16) {
     const TileCoord tc = coord(tile);
-    const int kd = (c16 * CK) / p.Cp, c0 = c16 * CK - kd * p.Cp;
+    const int per_blk = p.nc16 / p.nblk;  // 16-channel steps of one contraction block
+    const int blk = c16 / per_blk, inner = (c16 - blk * per_blk) * CK;
+    const int kd = inner / p.Cp, c0 = inner - kd * p.Cp;
+    const int cx0 = (int)((p.xmap >> (2 * blk)) & 3u) * p.C + c0;  // first channel of the step in x
     // Channels of this task that exist (all 8 unless C is not a multiple of 16). The vector
     // path below reads the others anyway (they lie inside the tensor: the interior test covers
     // all 16 channel planes) and store_stage zeroes them; the guarded paths skip them.
@@ -242,7 +325,7 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     const bool depth_ok = id >= 0 && id < p.Din;
     // wave-uniform origin of the stage window (lies before the tensor where padded)
     const char* origin = reinterpret_cast<const char*>(p.x) +
-                         2 * ((ptrdiff_t)(((size_t)tc.n * p.C + c0) * chan_stride) +
+                         2 * ((ptrdiff_t)(((size_t)tc.n * p.Cx + cx0) * chan_stride) +
                               (ptrdiff_t)id * (ptrdiff_t)plane + (ptrdiff_t)ih0 * p.Win + iw0);
     // The last octet of a row holds 2 pixels that are used and 6 that no fragment
     // reads, so it may run past the row end as long as it stays inside the tensor.
@@ -254,7 +337,7 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
       // alignment its rows give the window
       const int dt = id - p.tlo_d, ht = ih0 - p.tlo_h, wt = iw0 - p.tlo_w;
       const char* origin_t = reinterpret_cast<const char*>(p.xt) +
-                             2 * ((ptrdiff_t)(((size_t)tc.n * p.C + c0) * chan_stride_t) +
+                             2 * ((ptrdiff_t)(((size_t)tc.n * p.Cx + cx0) * chan_stride_t) +
                                   (ptrdiff_t)dt * (ptrdiff_t)plane_t + (ptrdiff_t)ht * p.tn_w + wt);
       if (dt >= 0 && dt < p.tn_d && ht >= 0 && ht + IN_ROWS <= p.tn_h && wt >= 0 && wt + TW + KW - 1 <= p.tn_w) {
         if (!has_task) return;
@@ -428,6 +511,25 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     char* ybase = reinterpret_cast<char*>(p.y) +
                   2 * (((size_t)tc.n * p.M + (size_t)mt * MT) * ochan + (size_t)tc.od * plane_o);
     const int m_left = p.M - mt * MT - 4 * kg;  // channels from this lane's first one to the end
+    if (p.out32) {  // uniform: the same walk with 4-byte stores
+      char* ybase32 = reinterpret_cast<char*>(p.y) +
+                      4 * (((size_t)tc.n * p.M + (size_t)mt * MT) * ochan + (size_t)tc.od * plane_o);
+#pragma unroll
+      for (int r = 0; r < WROWS; ++r) {
+        const int oh = tc.th * TH + wrow0 + r;
+        if (oh < p.Hout && ow < p.Wout) {
+          const uint32_t voff = (uint32_t)(4 * ((size_t)(4 * kg) * ochan + (size_t)oh * p.Wout + ow));
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const int m0 = cb * 32 + 8 * (i >> 2) + (i & 3);
+              if (!RAGGED || m0 < m_left) store_f32(ybase32 + (size_t)m0 * ochan * 4, voff, acc[cb][r][i]);
+            }
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int r = 0; r < WROWS; ++r) {
       const int oh = tc.th * TH + wrow0 + r;
@@ -638,10 +740,11 @@ bool shape_ok(int C, int M, const ConvGeom& g) {
 size_t prep_bytes(int K, int M) { return layout_of(K, M).prep_bytes; }
 
 struct Launch {
-  const uint16_t* x;
-  const uint16_t* w;
-  const uint16_t* bias;
-  uint16_t* y;
+  const void* x;
+  const void* w;
+  const void* bias;
+  void* y;
+  int split;                // fp32 tensors, computed as six bf16 products (split mode)
   int N, C, M, KD;
   int Din, Hin, Win, Dout, Hout, Wout;
   int pad_d, pad_h, pad_w;
@@ -649,14 +752,24 @@ struct Launch {
   int fold;                 // fold mode: y is the unpadded tile, strips receive the halo cells
   int lo[3], n[3];          // own extent inside the produced tensor (fold mode)
   void* const* strips;      // 27 slots (fold mode)
-  const uint16_t* xt;       // own tile for the framed input, or NULL
+  const uint16_t* xt;       // own tile for the framed input, or NULL (bf16 only)
   int tlo[3], tn[3];
 };
 
+// Bytes of the split copy of an fp32 input (three bf16 parts), rounded to 256
+size_t split_bytes(size_t elements) { return (elements * 3 * 2 + 255) / 256 * 256; }
+size_t conv_ws_bytes(int split, int KD, int C, int M, size_t x_elements) {
+  const size_t prep = prep_bytes((split ? 6 : 1) * KD * pad16(C), M);
+  return split ? (prep + 255) / 256 * 256 + split_bytes(x_elements) : prep;
+}
+
 int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const char* who) {
-  const int K = L.KD * pad16(L.C);
-  if (ws == nullptr || ws_bytes < prep_bytes(K, L.M))
-    JG_FAIL(JG_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, prep_bytes(K, L.M));
+  const int nblk = L.split ? 6 : 1;
+  const int K = nblk * L.KD * pad16(L.C);
+  const size_t x_elements = (size_t)L.N * L.C * L.Din * L.Hin * L.Win;
+  const size_t need = conv_ws_bytes(L.split, L.KD, L.C, L.M, x_elements);
+  if (ws == nullptr || ws_bytes < need)
+    JG_FAIL(JG_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, need);
   JG_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 15) == 0, "%s: workspace must be 16-byte aligned",
              who);
   const Layout lay = layout_of(K, L.M);
@@ -664,15 +777,34 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   uint16_t* wprep = static_cast<uint16_t*>(ws);
   const size_t total_w = lay.prep_bytes / 2;
   JG_REQUIRE(total_w < (1ull << 31), "%s: weight tensor too large", who);
-  prep_weights_kernel<<<(unsigned)((total_w + 255) / 256), 256, 0, s>>>(wprep, L.w, L.M, L.C, pad16(L.C), L.KD, MT, lay.mtiles,
-                                                                         lay.wc16, lay.ngroups, L.transposed);
-  JG_CHECK_LAUNCH(who);
+  const uint16_t* x16 = static_cast<const uint16_t*>(L.x);
+  if (L.split) {
+    prep_weights_split_kernel<<<(unsigned)((total_w + 255) / 256), 256, 0, s>>>(
+        wprep, static_cast<const float*>(L.w), L.M, L.C, pad16(L.C), L.KD, MT, lay.mtiles, lay.wc16, lay.ngroups,
+        L.transposed);
+    JG_CHECK_LAUNCH(who);
+    uint16_t* x3 = reinterpret_cast<uint16_t*>(static_cast<char*>(ws) + (lay.prep_bytes + 255) / 256 * 256);
+    if (x_elements > 0) {
+      size_t blocks = (x_elements + 255) / 256;
+      if (blocks > 65536) blocks = 65536;
+      split3_kernel<<<(unsigned)blocks, 256, 0, s>>>(x3, static_cast<const float*>(L.x), x_elements / L.N, x_elements);
+      JG_CHECK_LAUNCH(who);
+    }
+    x16 = x3;
+  } else {
+    prep_weights_kernel<<<(unsigned)((total_w + 255) / 256), 256, 0, s>>>(wprep, static_cast<const uint16_t*>(L.w), L.M,
+                                                                           L.C, pad16(L.C), L.KD, MT, lay.mtiles,
+                                                                           lay.wc16, lay.ngroups, L.transposed);
+    JG_CHECK_LAUNCH(who);
+  }
 
   FwdParams p;
-  p.x_end = reinterpret_cast<const char*>(L.x) + 2 * (size_t)L.N * L.C * L.Din * L.Hin * L.Win;
-  p.x = L.x; p.wprep = reinterpret_cast<const u32x4*>(wprep); p.bias = L.bias; p.y = L.y;
+  p.x_end = reinterpret_cast<const char*>(x16) + 2 * x_elements * (L.split ? 3 : 1);
+  p.x = x16; p.wprep = reinterpret_cast<const u32x4*>(wprep);
+  p.bias = static_cast<const uint16_t*>(L.bias); p.y = static_cast<uint16_t*>(L.y);
   p.N = L.N; p.C = L.C; p.M = L.M; p.KD = L.KD;
   p.Cp = pad16(L.C);
+  p.nblk = nblk; p.Cx = nblk == 6 ? 3 * L.C : L.C; p.xmap = nblk == 6 ? kInputParts : 0u; p.out32 = L.split;
   p.Din = L.Din; p.Hin = L.Hin; p.Win = L.Win;
   p.Dout = L.Dout; p.Hout = L.Hout; p.Wout = L.Wout;
   p.pad_d = L.pad_d; p.pad_h = L.pad_h; p.pad_w = L.pad_w;
@@ -699,7 +831,7 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   wgs = (wgs + 7) & ~7;  // whole XCD rounds
   dim3 grid((unsigned)wgs, (unsigned)lay.mtiles, 1);
   const bool even = (L.Win % 2 == 0) && (L.pad_w % 2 == 0) &&
-                    ((reinterpret_cast<uintptr_t>(L.x) & 3) == 0);
+                    ((reinterpret_cast<uintptr_t>(x16) & 3) == 0);
   void (*kern)(StripTable, FwdParams) = nullptr;
   if (L.fold) {
     if (MT == 64) kern = even ? &conv3x3_mfma_kernel<64, true, true, false> : &conv3x3_mfma_kernel<64, false, true, false>;
@@ -723,27 +855,48 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
 
 namespace jg {
 
+// fp32 runs in split mode (three bf16 parts per operand, fp32 result); its 4-byte stores halve
+// the extent the 32-bit lane offsets reach.
+static bool dtype_ok(const ConvGeom& g, int dtype) {
+  if (dtype == JG_BF16) return true;
+  if (dtype != JG_F32) return false;
+  const size_t in_sz = (size_t)g.in[0] * g.in[1] * g.in[2], out_sz = (size_t)g.out[0] * g.out[1] * g.out[2];
+  const size_t big = in_sz > out_sz ? in_sz : out_sz;
+  return big * 4 * 72 < (1ull << 31);
+}
+int split3_bf16(uint16_t* dst, const float* src, size_t batch, size_t per_batch, hipStream_t s) {
+  const size_t total = batch * per_batch;
+  if (total == 0) return JG_OK;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  split3_kernel<<<(unsigned)blocks, 256, 0, s>>>(dst, src, per_batch, total);
+  JG_CHECK_LAUNCH("split3_bf16");
+  return JG_OK;
+}
+
 bool mfma_fwd_supported(const ConvGeom& g, int dtype) {
-  return dtype == JG_BF16 && shape_ok(g.cin, g.cout, g) && g.batch > 0;
+  return dtype_ok(g, dtype) && shape_ok(g.cin, g.cout, g) && g.batch > 0;
 }
 bool mfma_dgrad_supported(const ConvGeom& g, int dtype) {
-  if (dtype != JG_BF16 || g.batch <= 0) return false;
+  if (!dtype_ok(g, dtype) || g.batch <= 0) return false;
   for (int a = 0; a < 3; ++a)
     if (g.p[a] > g.k[a] - 1) return false;
   return shape_ok(g.cout, g.cin, g);
 }
 
-size_t mfma_fwd_workspace(const ConvGeom& g) { return prep_bytes(g.k[0] * pad16(g.cin), g.cout); }
-size_t mfma_dgrad_workspace(const ConvGeom& g) { return prep_bytes(g.k[0] * pad16(g.cout), g.cin); }
+size_t mfma_fwd_workspace(const ConvGeom& g, int dtype) {
+  return conv_ws_bytes(dtype == JG_F32, g.k[0], g.cin, g.cout, (size_t)g.batch * g.cin * g.in[0] * g.in[1] * g.in[2]);
+}
+size_t mfma_dgrad_workspace(const ConvGeom& g, int dtype) {
+  return conv_ws_bytes(dtype == JG_F32, g.k[0], g.cout, g.cin, (size_t)g.batch * g.cout * g.out[0] * g.out[1] * g.out[2]);
+}
 
 static int fwd_launch(void* y, const void* x, const void* xt, const int* tlo, const int* tn, const void* w,
                       const void* bias, const ConvGeom& g, void* ws, size_t ws_bytes, hipStream_t s,
-                      const char* who) {
+                      const char* who, int dtype = JG_BF16) {
   Launch L;
-  L.x = static_cast<const uint16_t*>(x);
-  L.w = static_cast<const uint16_t*>(w);
-  L.bias = static_cast<const uint16_t*>(bias);
-  L.y = static_cast<uint16_t*>(y);
+  L.x = x; L.w = w; L.bias = bias; L.y = y;
+  L.split = dtype == JG_F32;
   L.N = (int)g.batch; L.C = g.cin; L.M = g.cout; L.KD = g.k[0];
   L.Din = g.in[0]; L.Hin = g.in[1]; L.Win = g.in[2];
   L.Dout = g.out[0]; L.Hout = g.out[1]; L.Wout = g.out[2];
@@ -761,8 +914,8 @@ static int fwd_launch(void* y, const void* x, const void* xt, const int* tlo, co
 }
 
 int mfma_fwd(void* y, const void* x, const void* w, const void* bias, const ConvGeom& g, void* ws,
-             size_t ws_bytes, hipStream_t s) {
-  return fwd_launch(y, x, nullptr, nullptr, nullptr, w, bias, g, ws, ws_bytes, s, "jg_conv_fwd(mfma)");
+             size_t ws_bytes, hipStream_t s, int dtype) {
+  return fwd_launch(y, x, nullptr, nullptr, nullptr, w, bias, g, ws, ws_bytes, s, "jg_conv_fwd(mfma)", dtype);
 }
 
 int mfma_fwd_framed(void* y, const void* x_frame, const void* xt, const int tlo[3], const int tn[3],
@@ -810,12 +963,10 @@ void mfma_frame_bands(const ConvGeom& g, const int tlo[3], const int tn[3], int 
 // the produced tensor is split between the unpadded tile gx and the neighbours' strips.
 static int dgrad_launch(void* gx, void* const* strips, const int* lo, const int* n, const void* w,
                         const void* go, const ConvGeom& g, void* ws, size_t ws_bytes, hipStream_t s,
-                        const char* who) {
+                        const char* who, int dtype = JG_BF16) {
   Launch L;
-  L.x = static_cast<const uint16_t*>(go);
-  L.w = static_cast<const uint16_t*>(w);
-  L.bias = nullptr;
-  L.y = static_cast<uint16_t*>(gx);
+  L.x = go; L.w = w; L.bias = nullptr; L.y = gx;
+  L.split = dtype == JG_F32;
   L.N = (int)g.batch; L.C = g.cout; L.M = g.cin; L.KD = g.k[0];
   L.Din = g.out[0]; L.Hin = g.out[1]; L.Win = g.out[2];
   L.Dout = g.in[0]; L.Hout = g.in[1]; L.Wout = g.in[2];
@@ -833,8 +984,8 @@ static int dgrad_launch(void* gx, void* const* strips, const int* lo, const int*
 }
 
 int mfma_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, void* ws,
-               size_t ws_bytes, hipStream_t s) {
-  return dgrad_launch(gx, nullptr, nullptr, nullptr, w, go, g, ws, ws_bytes, s, "jg_conv_dgrad(mfma)");
+               size_t ws_bytes, hipStream_t s, int dtype) {
+  return dgrad_launch(gx, nullptr, nullptr, nullptr, w, go, g, ws, ws_bytes, s, "jg_conv_dgrad(mfma)", dtype);
 }
 
 int mfma_dgrad_fold(void* gx, void* const strips[27], const int lo[3], const int n[3], const void* w,

@@ -534,10 +534,11 @@ __global__ __launch_bounds__(256) void wgrad_bias_reduce_kernel(uint16_t* __rest
 // A block owns 64 consecutive outputs (one per lane, so a slot row is read coalesced);
 // its 4 wavefronts take the slots s = w, w + 4, ... in 4 independent chains each, and the
 // 16 chain sums are added in a fixed order (deterministic).
-__global__ __launch_bounds__(256) void wgrad_reduce_kernel(uint16_t* __restrict__ gw,
+template <bool OUT32>
+__global__ __launch_bounds__(256) void wgrad_reduce_kernel(void* __restrict__ gw_out,
                                                            const float* __restrict__ part,
                                                            int slots, int GC, int XC, int CinB,
-                                                           int cout_valid, int cin_valid, int cin_total) {
+                                                           int cout_valid, int cin_valid, int cin_total, int accumulate) {
   __shared__ float red[4][64];
   const int count = 9 * GC * XC;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -560,7 +561,31 @@ __global__ __launch_bounds__(256) void wgrad_reduce_kernel(uint16_t* __restrict_
   const int cx = i % XC, co = (i / XC) % GC, tap = i / (XC * GC);
   const int kd = cx / CinB, ci = cx % CinB, KD = XC / CinB;
   if (co >= cout_valid || ci >= cin_valid) return;
-  gw[(((size_t)co * cin_total + ci) * KD + kd) * 9 + tap] = jg::f32_to_bf16(s);
+  const size_t at = (((size_t)co * cin_total + ci) * KD + kd) * 9 + tap;
+  if (OUT32) {
+    // split mode: the six part products of a block are added up here, one launch after the other
+    float* gw = static_cast<float*>(gw_out);
+    gw[at] = accumulate ? gw[at] + s : s;
+  } else {
+    static_cast<uint16_t*>(gw_out)[at] = jg::f32_to_bf16(s);
+  }
+}
+
+// gw[co][ci][t] (fp32) = sum over the part pairs (i, j), i + j <= 2, smallest first, of
+// tmp[i * cout + co][j * cin + ci][t]: the part products of the split mode from one launch.
+__global__ __launch_bounds__(256) void wgrad_combine_parts_kernel(float* __restrict__ gw, const float* __restrict__ tmp,
+                                                                  int cout, int cin, int taps) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= cout * cin * taps) return;
+  const int t = idx % taps, ci = (idx / taps) % cin, co = idx / (taps * cin);
+  auto at = [&](int i, int j) { return tmp[((size_t)(i * cout + co) * (3 * cin) + (j * cin + ci)) * taps + t]; };
+  float sum = at(0, 2);
+  sum += at(1, 1);
+  sum += at(2, 0);
+  sum += at(0, 1);
+  sum += at(1, 0);
+  sum += at(0, 0);
+  gw[idx] = sum;
 }
 
 int cu_count() {
@@ -593,6 +618,8 @@ long long stage_count(const ConvGeom& g) {
 struct Blocking {
   int cob, cib;  // width of the first (largest) block
   int KD;
+  int cob_max() const { return KD == 3 ? 32 : 64; }
+  int cib_max() const { return KD == 3 ? 32 : 64; }
 };
 bool blocks_of(const ConvGeom& g, Blocking* b) {
   if (g.k[1] != 3 || g.k[2] != 3 || (g.k[0] != 1 && g.k[0] != 3)) return false;
@@ -635,17 +662,42 @@ int launch(const WgradParams& p, bool even, int wgs, hipStream_t s, const char* 
 
 namespace jg {
 
+// Split mode with few channels: the three parts of both operands fit one block.
+static bool parts_fit_one_block(const ConvGeom& g, const Blocking& bl) {
+  return 3 * g.cout <= bl.cob_max() && 3 * g.cin <= bl.cib_max();
+}
+static size_t parts_tmp_bytes(const ConvGeom& g, const Blocking& bl) {
+  if (!parts_fit_one_block(g, bl)) return 0;
+  return ((size_t)9 * g.cout * g.cin * bl.KD * 9 * sizeof(float) + 255) / 256 * 256;
+}
+
+// fp32 runs in split mode: both operands are copied as three bf16 parts each (as extra channels)
+// and the six part products whose indices add up to at most 2 are accumulated in fp32.
 bool mfma_wgrad_supported(const ConvGeom& g, int dtype) {
   Blocking b;
-  if (dtype != JG_BF16 || g.batch <= 0) return false;
+  if ((dtype != JG_BF16 && dtype != JG_F32) || g.batch <= 0) return false;
   return blocks_of(g, &b);
 }
 
-size_t mfma_wgrad_workspace(const ConvGeom& g) {
+static size_t partial_bytes(const ConvGeom& g) {
   Blocking b{32, 32, 1};
   blocks_of(g, &b);
   const size_t wgs = (size_t)wg_count(stage_count(g));
-  return wgs * HALVES * 9 * b.cob * (b.KD * b.cib) * sizeof(float) + wgs * b.cob * sizeof(float);
+  // sized for the widest block any mode launches
+  const size_t n = wgs * HALVES * 9 * b.cob_max() * (b.KD * b.cib_max()) * sizeof(float) + wgs * b.cob_max() * sizeof(float);
+  return (n + 255) / 256 * 256;
+}
+static size_t split_copy_bytes(size_t elements) { return (elements * 3 * 2 + 255) / 256 * 256; }
+size_t mfma_wgrad_workspace(const ConvGeom& g, int dtype) {
+  size_t n = partial_bytes(g);
+  if (dtype == JG_F32) {
+    n += split_copy_bytes((size_t)g.batch * g.cin * g.in[0] * g.in[1] * g.in[2]);
+    n += split_copy_bytes((size_t)g.batch * g.cout * g.out[0] * g.out[1] * g.out[2]);
+    Blocking b{32, 32, 1};
+    blocks_of(g, &b);
+    n += parts_tmp_bytes(g, b);  // last in the workspace
+  }
+  return n;
 }
 
 // Whether the framed weight-gradient kernel covers a geometry: even row lengths (its
@@ -676,25 +728,43 @@ bool mfma_wgrad_frame_ok(const ConvGeom& g, const int tlo[3], const int tn[3]) {
 }
 
 int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom& g, void* ws,
-               size_t ws_bytes, hipStream_t s, const void* xt, const int* tlo, const int* tn) {
+               size_t ws_bytes, hipStream_t s, const void* xt, const int* tlo, const int* tn, int dtype) {
   const char* who = "jg_conv_wgrad(mfma)";
   Blocking bl;
   if (!blocks_of(g, &bl)) JG_FAIL(JG_ERR_UNSUPPORTED, "%s: geometry not covered", who);
-  if (ws == nullptr || ws_bytes < mfma_wgrad_workspace(g))
+  if (ws == nullptr || ws_bytes < mfma_wgrad_workspace(g, dtype))
     JG_FAIL(JG_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes,
-            mfma_wgrad_workspace(g));
+            mfma_wgrad_workspace(g, dtype));
   JG_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 15) == 0, "%s: workspace must be 16-byte aligned",
              who);
+  const size_t x_cs = (size_t)g.in[0] * g.in[1] * g.in[2], g_cs = (size_t)g.out[0] * g.out[1] * g.out[2];
+  const bool split = dtype == JG_F32;
+  if (split) {
+    if (gb != nullptr || xt != nullptr)
+      JG_FAIL(JG_ERR_UNSUPPORTED, "%s: fp32 has neither the fused bias gradient nor the framed input", who);
+    char* base = static_cast<char*>(ws) + partial_bytes(g);
+    uint16_t* x3 = reinterpret_cast<uint16_t*>(base);
+    uint16_t* g3 = reinterpret_cast<uint16_t*>(base + split_copy_bytes((size_t)g.batch * g.cin * x_cs));
+    int rc = split3_bf16(x3, static_cast<const float*>(x), (size_t)g.batch, (size_t)g.cin * x_cs, s);
+    if (rc) return rc;
+    rc = split3_bf16(g3, static_cast<const float*>(go), (size_t)g.batch, (size_t)g.cout * g_cs, s);
+    if (rc) return rc;
+    x = x3;
+    go = g3;
+  }
   const bool even = (g.in[2] % 2 == 0) && (g.p[2] % 2 == 0) && (g.out[2] % 2 == 0) &&
                     ((reinterpret_cast<uintptr_t>(x) & 3) == 0) &&
                     ((reinterpret_cast<uintptr_t>(go) & 3) == 0);
   if (xt != nullptr && (!even || !mfma_wgrad_frame_ok(g, tlo, tn)))
     JG_FAIL(JG_ERR_UNSUPPORTED, "%s: the framed input does not cover this geometry / alignment", who);
-  const size_t x_cs = (size_t)g.in[0] * g.in[1] * g.in[2], g_cs = (size_t)g.out[0] * g.out[1] * g.out[2];
+  // part products (g part, x part), smallest first; plain mode: the one product
+  static const int kPairs[6][2] = {{0, 2}, {1, 1}, {2, 0}, {0, 1}, {1, 0}, {0, 0}};
+  const int npairs = split ? 6 : 1, first_pair = split ? 0 : 5;
+  const int parts = split ? 3 : 1;
   WgradParams p;
   p.part = static_cast<float*>(ws);
-  p.x_end = static_cast<const char*>(x) + 2 * (size_t)g.batch * g.cin * x_cs;
-  p.cin_total = g.cin; p.cout_total = g.cout;
+  p.x_end = static_cast<const char*>(x) + 2 * (size_t)g.batch * parts * g.cin * x_cs;
+  p.cin_total = parts * g.cin; p.cout_total = parts * g.cout;
   p.Din = g.in[0]; p.Hin = g.in[1]; p.Win = g.in[2];
   p.Dout = g.out[0]; p.Hout = g.out[1]; p.Wout = g.out[2];
   p.pad_d = g.p[0]; p.pad_h = g.p[1]; p.pad_w = g.p[2];
@@ -705,36 +775,70 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
   p.xt = static_cast<const uint16_t*>(xt);
   p.tlo_d = tlo ? tlo[0] : 0; p.tlo_h = tlo ? tlo[1] : 0; p.tlo_w = tlo ? tlo[2] : 0;
   p.tn_d = tn ? tn[0] : 0; p.tn_h = tn ? tn[1] : 0; p.tn_w = tn ? tn[2] : 0;
+  // One block of channels: g channels [gch, gch + cout_valid), x channels [xch, xch + cin_valid) of the
+  // tensors as they lie in memory (split mode: parts are channel groups), into out (+ gb_out).
+  auto run_block = [&](size_t gch, size_t xch, int cob, int cib, int cout_valid, int cin_valid, void* out,
+                       int out_cin_total, bool out32, bool accumulate, uint16_t* gb_out) -> int {
+    const int cgb = cob / 32, cxb = bl.KD * cib / 32;
+    p.Cin = cib; p.Cout = cob;
+    p.cin_valid = cin_valid; p.cout_valid = cout_valid;
+    p.x = static_cast<const uint16_t*>(x) + xch * x_cs;
+    p.g = static_cast<const uint16_t*>(go) + gch * g_cs;
+    p.bias_part = gb_out != nullptr ? p.part + (size_t)wgs * HALVES * 9 * cob * (bl.KD * cib) : nullptr;
+    int rc;
+    if (cgb == 2 && cxb == 2) rc = launch<2, 2>(p, even, wgs, s, who);
+    else if (cgb == 1 && cxb == 3) rc = launch<1, 3>(p, even, wgs, s, who);
+    else if (cgb == 1 && cxb == 1) rc = launch<1, 1>(p, even, wgs, s, who);
+    else if (cgb == 2 && cxb == 1) rc = launch<2, 1>(p, even, wgs, s, who);
+    else if (cgb == 1 && cxb == 2) rc = launch<1, 2>(p, even, wgs, s, who);
+    else JG_FAIL(JG_ERR_UNSUPPORTED, "%s: channel blocking (%d, %d) not built", who, cgb, cxb);
+    if (rc) return rc;
+    JG_CHECK_LAUNCH(who);
+    const int count = 9 * cob * bl.KD * cib;
+    if (out32)
+      wgrad_reduce_kernel<true><<<(count + 63) / 64, 256, 0, s>>>(out, p.part, wgs * HALVES, cob, bl.KD * cib, cib,
+                                                                    cout_valid, cin_valid, out_cin_total, accumulate);
+    else
+      wgrad_reduce_kernel<false><<<(count + 63) / 64, 256, 0, s>>>(out, p.part, wgs * HALVES, cob, bl.KD * cib, cib,
+                                                                     cout_valid, cin_valid, out_cin_total, 0);
+    JG_CHECK_LAUNCH(who);
+    if (gb_out != nullptr) {
+      wgrad_bias_reduce_kernel<<<(cob + 3) / 4, 256, 0, s>>>(gb_out, p.bias_part, wgs, cob, cout_valid);
+      JG_CHECK_LAUNCH(who);
+    }
+    return JG_OK;
+  };
+
+  if (split && parts_fit_one_block(g, bl)) {
+    // few channels: all nine part products in one launch (the parts are 3 x cout and 3 x cin channels
+    // of one block), then the six that count are added up
+    float* tmp = reinterpret_cast<float*>(static_cast<char*>(ws) + mfma_wgrad_workspace(g, dtype) -
+                                          parts_tmp_bytes(g, bl));
+    const int cob = 3 * g.cout > 32 ? 64 : 32, cib = 3 * g.cin > 32 ? 64 : 32;  // within the block limits (checked)
+    int rc = run_block(0, 0, cob, cib, 3 * g.cout, 3 * g.cin, tmp, 3 * g.cin, true, false, nullptr);
+    if (rc) return rc;
+    const int total = g.cout * g.cin * bl.KD * 9;
+    wgrad_combine_parts_kernel<<<(total + 255) / 256, 256, 0, s>>>(static_cast<float*>(gw), tmp, g.cout, g.cin,
+                                                                   bl.KD * 9);
+    JG_CHECK_LAUNCH(who);
+    return JG_OK;
+  }
   for (int co0 = 0; co0 < g.cout;) {
     const int cob = block_width(g.cout, co0, bl.cob);
     for (int ci0 = 0; ci0 < g.cin;) {
       const int cib = block_width(g.cin, ci0, bl.cib);
-      const int cgb = cob / 32, cxb = bl.KD * cib / 32;
-      p.Cin = cib; p.Cout = cob;
-      p.cin_valid = g.cin - ci0 < cib ? g.cin - ci0 : cib;
-      p.cout_valid = g.cout - co0 < cob ? g.cout - co0 : cob;
-      p.x = static_cast<const uint16_t*>(x) + ci0 * x_cs;
-      p.g = static_cast<const uint16_t*>(go) + co0 * g_cs;
-      // the bias gradient comes from the g rows: once per block of output channels
-      p.bias_part = (gb != nullptr && ci0 == 0) ? p.part + (size_t)wgs * HALVES * 9 * cob * (bl.KD * cib) : nullptr;
-      int rc;
-      if (cgb == 2 && cxb == 2) rc = launch<2, 2>(p, even, wgs, s, who);
-      else if (cgb == 1 && cxb == 3) rc = launch<1, 3>(p, even, wgs, s, who);
-      else if (cgb == 1 && cxb == 1) rc = launch<1, 1>(p, even, wgs, s, who);
-      else if (cgb == 2 && cxb == 1) rc = launch<2, 1>(p, even, wgs, s, who);
-      else if (cgb == 1 && cxb == 2) rc = launch<1, 2>(p, even, wgs, s, who);
-      else JG_FAIL(JG_ERR_UNSUPPORTED, "%s: channel blocking (%d, %d) not built", who, cgb, cxb);
-      if (rc) return rc;
-      JG_CHECK_LAUNCH(who);
-      const int count = 9 * cob * bl.KD * cib;
-      uint16_t* gw_blk = static_cast<uint16_t*>(gw) + ((size_t)co0 * g.cin + ci0) * bl.KD * 9;
-      wgrad_reduce_kernel<<<(count + 63) / 64, 256, 0, s>>>(gw_blk, p.part, wgs * HALVES, cob, bl.KD * cib, cib,
-                                                              p.cout_valid, p.cin_valid, g.cin);
-      JG_CHECK_LAUNCH(who);
-      if (p.bias_part != nullptr) {
-        wgrad_bias_reduce_kernel<<<(cob + 3) / 4, 256, 0, s>>>(static_cast<uint16_t*>(gb) + co0, p.bias_part,
-                                                               wgs, cob, p.cout_valid);
-        JG_CHECK_LAUNCH(who);
+      const int cin_valid = g.cin - ci0 < cib ? g.cin - ci0 : cib;
+      const int cout_valid = g.cout - co0 < cob ? g.cout - co0 : cob;
+      const size_t blk_at = ((size_t)co0 * g.cin + ci0) * bl.KD * 9;
+      for (int pr = 0; pr < npairs; ++pr) {
+        const int gpart = kPairs[first_pair + pr][0], xpart = kPairs[first_pair + pr][1];
+        void* out = split ? static_cast<void*>(static_cast<float*>(gw) + blk_at)
+                          : static_cast<void*>(static_cast<uint16_t*>(gw) + blk_at);
+        // the bias gradient comes from the g rows: once per block of output channels
+        uint16_t* gb_out = (gb != nullptr && ci0 == 0) ? static_cast<uint16_t*>(gb) + co0 : nullptr;
+        int rc = run_block((size_t)gpart * g.cout + co0, (size_t)xpart * g.cin + ci0, cob, cib, cout_valid, cin_valid,
+                           out, g.cin, split, pr > 0, gb_out);
+        if (rc) return rc;
       }
       ci0 += cib;
     }
