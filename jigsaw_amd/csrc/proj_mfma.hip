@@ -115,8 +115,12 @@ __global__ __launch_bounds__(64 * WM * WN) void proj_nt_kernel(NtParams p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, kg = lane >> 5;
   const int wm = wave % WM, wn = wave / WM;
-  const long long m0 = (long long)(blockIdx.x / p.tiles_n) * TM;
-  const int n0 = (blockIdx.x % p.tiles_n) * TNF;
+  // Workgroups go to the 8 XCDs round-robin; give each XCD a contiguous range of tiles, so that the
+  // tiles that share a panel of `a` (consecutive ids) meet in one L2.
+  const unsigned per_xcd = gridDim.x / 8;
+  const unsigned tile_id = blockIdx.x < per_xcd * 8 ? (blockIdx.x % 8) * per_xcd + blockIdx.x / 8 : blockIdx.x;
+  const long long m0 = (long long)(tile_id / p.tiles_n) * TM;
+  const int n0 = (tile_id % p.tiles_n) * TNF;
   if (tid < TNF)  // read after the barriers of the stage loop
     reinterpret_cast<float*>(smem + SH::MAIN)[tid] =
         (p.bias != nullptr && n0 + tid < p.N) ? jg::bf16_to_f32(p.bias[n0 + tid]) : 0.0f;

@@ -166,6 +166,9 @@ DIST_CASES = [
     # mesh, local spatial, N, Cin, Cout, kernel, padding, dtype
     ((2, 2), (32, 32), 2, 3, 16, (3, 3), (1, 1), torch.float32),
     ((2, 2), (32, 32), 2, 16, 3, (3, 3), (1, 1), torch.float32),
+    # the reference's CPU-runnable configuration at its real size: 2 x 2 mesh of 256 x 256 tiles, batch 4, fp32
+    ((2, 2), (256, 256), 4, 3, 16, (3, 3), (1, 1), torch.float32),
+    ((2, 2), (256, 256), 4, 16, 3, (3, 3), (1, 1), torch.float32),
     ((3, 3), (8, 12), 1, 4, 5, (5, 3), (2, 1), torch.float32),
     ((2, 1), (16, 20), 2, 4, 4, (3, 3), (1, 1), torch.float32),
     ((2, 2), (32, 64), 1, 64, 64, (3, 3), (1, 1), torch.bfloat16),
