@@ -11,7 +11,7 @@
 //               row), so an accumulator lane owns one pixel and 16 produced channels
 //               and the stores run along W of the channels-first output.
 //   Workgroup   512 threads = 8 wavefronts; output tile 16 rows x 64 columns x MT
-//               produced channels; wavefront w owns rows 4*(w/2).., columns 32*(w%2)..
+//               produced channels; wavefront w owns rows 4*((w + 2*(w/4))%4).., columns 32*(w/4)..
 //   LDS         the whole prepared weight block of the workgroup's produced-channel
 //               tile stays resident; the input tile is streamed in stages of 16
 //               contraction channels, double buffered (2 x 40.5 KiB). Input pixels
@@ -241,7 +241,10 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, kg = lane >> 5;
-  const int wrow0 = (wave >> 1) * WROWS, wcol0 = (wave & 1) * 32;
+  // Wavefronts w and w + 4 share a SIMD. They hold different column halves, so when a tile's second
+  // half lies past the row end every SIMD drops half of that tile's MFMAs, and row groups two apart,
+  // so a tile with few valid rows keeps two SIMDs busy instead of one.
+  const int wrow0 = ((wave + 2 * (wave >> 2)) & 3) * WROWS, wcol0 = (wave >> 2) * 32;
   const int mt = blockIdx.y;
 
   // ---- tile schedule: XCD x (= blockIdx.x % 8) owns a contiguous range of tiles and
@@ -663,17 +666,23 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
   int q = 0;
   for (int ti = 0; ti < my_tiles; ++ti) {
     init_acc();
+    // a wavefront whose 4 x 32 pixels all lie outside the produced tensor (ragged last tiles) only
+    // takes part in the staging and the barriers
+    const TileCoord tcur = coord(tile_of(ti));
+    const bool live = tcur.tw * TW + wcol0 < p.Wout && tcur.th * TH + wrow0 < p.Hout;
     for (int c16 = 0; c16 < p.nc16; ++c16, ++q) {
       if (p.ngroups > 1 && c16 % p.wc16 == 0) {
         // every wavefront is past the barrier that closed the last stage of the group before
         load_weights(c16 / p.wc16);
         __syncthreads();
       }
-      compute_kw(buf, c16, 0);
-      compute_kw(buf, c16, 1);
+      if (live) {
+        compute_kw(buf, c16, 0);
+        compute_kw(buf, c16, 1);
+      }
       if (q + 1 < stages) store_stage(buf ^ 1, c16 + 1 < p.nc16 ? c16 + 1 : 0);  // other buffer: no hazard with this stage's reads
       if (q + 2 < stages) issue_stage(q + 2);
-      compute_kw(buf, c16, 2);
+      if (live) compute_kw(buf, c16, 2);
       __syncthreads();
       buf ^= 1;
     }
