@@ -772,6 +772,7 @@ struct BorderPlan {
   uint32_t total;           // work items of the launch
   int nbd, nbh;             // border depths / border rows of a non-border depth
   int n_edge, head;         // W-edge cells of a row: columns [0, head) and [W - lo, W)
+  int lpr;                  // lanes per row of the rows kernel
   Magic div_rows, div_h, div_nbh, div_edge, div_hh, div_d;
 };
 
@@ -781,9 +782,10 @@ __global__ __launch_bounds__(256) void fold_border_rows_kernel(Table tab, typena
                                                                Geom g, BorderPlan bp) {
   typedef typename Arith<DT>::T T;
   constexpr int V = Bits<T>::V;
-  const uint32_t item = blockIdx.x * 4u + (threadIdx.x >> 6);  // one wavefront per row
+  // a row is owned by bp.lpr lanes (a power of two up to 64: a whole wavefront for long rows)
+  const uint32_t item = (blockIdx.x * 256u + threadIdx.x) / (uint32_t)bp.lpr;
   if (item >= bp.total) return;
-  const int lane = threadIdx.x & 63;
+  const int lane = threadIdx.x & (bp.lpr - 1);
   const int D = g.n[0], H = g.n[1], W = g.n[2];
   const uint32_t pp = mdiv(item, bp.div_rows);
   const uint32_t idx = item - pp * bp.rows_per_plane;
@@ -801,7 +803,7 @@ __global__ __launch_bounds__(256) void fold_border_rows_kernel(Table tab, typena
   const long long p = (long long)pp;
   T* drow = gx + ((p * D + d) * H + h) * (long long)W;
   const int n_vec = W / V;
-  for (int j = lane; j < n_vec; j += 64) fold_span<DT>(drow, drow, g, p, d, h, j * V, V);
+  for (int j = lane; j < n_vec; j += bp.lpr) fold_span<DT>(drow, drow, g, p, d, h, j * V, V);
   if (lane == 0 && n_vec * V < W) fold_span<DT>(drow, drow, g, p, d, h, n_vec * V, W - n_vec * V);
 }
 
@@ -1238,7 +1240,12 @@ extern "C" int jg_halo_fold_border_3d(void* gx, const void* const strips[27],
     typedef Arith<DT>::T T;                                                                             \
     if (row_items > 0) {                                                                                \
       bp.total = (uint32_t)row_items;                                                                   \
-      fold_border_rows_kernel<DT><<<(unsigned)((row_items + 3) / 4), 256, 0, s>>>(tab, static_cast<T*>(gx), g, bp); \
+      const int vecs = W / (16 / (int)sizeof(T));                                                       \
+      bp.lpr = 1;                                                                                       \
+      while (bp.lpr < 64 && bp.lpr < vecs) bp.lpr *= 2;                                                 \
+      const unsigned long long threads = row_items * (unsigned long long)bp.lpr;                        \
+      JG_REQUIRE(threads < (1ull << 32), "jg_halo_fold_border_3d: too many border rows (%llu)", row_items); \
+      fold_border_rows_kernel<DT><<<(unsigned)((threads + 255) / 256), 256, 0, s>>>(tab, static_cast<T*>(gx), g, bp); \
     }                                                                                                   \
     if (col_items > 0) {                                                                                \
       bp.total = (uint32_t)col_items;                                                                   \
