@@ -59,6 +59,13 @@ __device__ __forceinline__ u32x4 load16_unaligned<uint16_t>(const uint16_t* s) {
   return *reinterpret_cast<const u32x4_a2*>(s);
 }
 
+// Store 16 bytes to an address that is only sizeof(T)-aligned.
+__device__ __forceinline__ void store16_unaligned(uint32_t* d, u32x4 v) { *reinterpret_cast<u32x4_a4*>(d) = v; }
+__device__ __forceinline__ void store16_unaligned(uint16_t* d, u32x4 v) {
+  typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+  *reinterpret_cast<u32x4_a2*>(d) = v;
+}
+
 // Region of a padded coordinate: 0 = lower halo, 1 = interior, 2 = upper halo.
 __device__ __forceinline__ void region(int x, int lo, int n, int hi, int& r, int& c,
                                        int& ext) {
@@ -172,26 +179,35 @@ struct PackArgs {
   Box box[27];
 };
 
-// I: index type (32-bit when the source tensor has fewer than 2^31 elements)
+// I: index type (32-bit when the source tensor has fewer than 2^31 elements). A thread moves one
+// chunk of up to V = 16 / sizeof(T) consecutive elements of a strip row: one 16-byte access each
+// way for the faces whose rows run along W, single elements for the faces that are one column wide.
 template <typename T, typename I>
 __global__ __launch_bounds__(256) void pack_kernel(PackArgs a, const T* __restrict__ src,
                                                    long long planes, int Sd, int Sh,
                                                    int Sw) {
+  constexpr int V = Bits<T>::V;
   const int slot = blockIdx.y;
   T* d = static_cast<T*>(a.dst[slot]);
   if (d == nullptr) return;
   const Box b = a.box[slot];
   const I e0 = (I)b.ext[0], e1 = (I)b.ext[1], e2 = (I)b.ext[2];
-  const I total = (I)planes * e0 * e1 * e2;
+  const I cpr = (e2 + V - 1) / V;  // chunks per row
+  const I total = (I)planes * e0 * e1 * cpr;
   for (I i = (I)blockIdx.x * 256 + threadIdx.x; i < total; i += (I)gridDim.x * 256) {
-    const I r = i / e2;
-    const I cw = i - r * e2;
+    const I r = i / cpr;
+    const I cw = (i - r * cpr) * V;
     const I r2 = r / e1;
     const I ch = r - r2 * e1;
     const I p = r2 / e0;
     const I cd = r2 - p * e0;
     const I so = ((p * (I)Sd + ((I)b.org[0] + cd)) * (I)Sh + ((I)b.org[1] + ch)) * (I)Sw + ((I)b.org[2] + cw);
-    d[i] = src[so];
+    const I to = r * e2 + cw;
+    if (cw + V <= e2) {
+      store16_unaligned(d + to, load16_unaligned<T>(src + so));
+    } else {
+      for (I k = 0; cw + k < e2; ++k) d[to + k] = src[so + k];
+    }
   }
 }
 
