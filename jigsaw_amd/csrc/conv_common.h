@@ -53,8 +53,8 @@ int mfma_dgrad_fold(void* gx, void* const strips[27], const int lo[3], const int
 int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom& g, void* ws,
                size_t ws_bytes, hipStream_t s, const void* xt = nullptr, const int* tlo = nullptr,
                const int* tn = nullptr, int dtype = JG_BF16);
-// dst (batch, 3, per_batch) bf16 = high / middle / low bf16 parts of src (batch, per_batch) fp32,
-// whose sum is src: the operand layout of the fp32 ("split") mode of the MFMA kernels.
-int split3_bf16(uint16_t* dst, const float* src, size_t batch, size_t per_batch, hipStream_t s);
+// dst (batch, parts, per_batch) bf16 = the bf16 parts of src (batch, per_batch), whose sum is src:
+// three for fp32, two for fp16. The operand layout of the split mode of the MFMA kernels.
+int split_parts_bf16(uint16_t* dst, const void* src, int src_dtype, size_t batch, size_t per_batch, hipStream_t s);
 
 }  // namespace jg

@@ -37,6 +37,7 @@ using jg::ConvGeom;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -65,13 +66,13 @@ struct FwdParams {
   uint16_t* y;          // (N, M, Dout, Hout, Wout)
   int N, C, M;          // batch, channels of x, produced channels
   int Cp;               // C rounded up to a multiple of 16: contraction channels per depth tap
-  // Split mode (fp32 operands as sums of three bf16 parts): x holds Cx = 3 C channels per batch
-  // entry ([high | middle | low] parts), the contraction runs over nblk = 6 blocks of KD * Cp
+  // Split mode (fp32 / fp16 operands as sums of 3 / 2 bf16 parts): x holds Cx = parts * C channels per
+  // batch entry (one channel group per part), the contraction runs over nblk = 6 / 3 blocks of KD * Cp
   // channels, block b reads part (xmap >> 2 b) & 3 of x against the weight part the
   // preparation put there. Plain mode: nblk = 1, xmap = 0, Cx = C.
   int nblk, Cx;
   uint32_t xmap;
-  int out32;            // y (and bias) are fp32
+  int out_kind;         // dtype of y and bias: 0 bf16, 1 fp32, 2 fp16
   int KD;               // depth taps (1 for 2-D); contraction channels K = KD * C
   int Din, Hin, Win, Dout, Hout, Wout;
   int pad_d, pad_h, pad_w;  // virtual zero padding of x
@@ -148,7 +149,8 @@ __global__ __launch_bounds__(256) void prep_weights_kernel(uint16_t* __restrict_
 // middle = bf16(v - high), low = bf16(v - high - middle); the subtractions are exact. A
 // product of two fp32 values is then, to 2^-24 relative, the sum of the six part products
 // whose indices add up to at most 2, each of which the bf16 matrix cores form exactly and
-// add in fp32.
+// add in fp32. An fp16 value (11 significand bits) is the sum of two parts, and the three
+// products (0,0), (0,1), (1,0) carry it to 2^-16 relative, far below fp16's own rounding.
 __device__ __forceinline__ uint16_t split_part(float v, int part) {
   const uint16_t hi = jg::f32_to_bf16(v);
   if (part == 0) return hi;
@@ -158,34 +160,49 @@ __device__ __forceinline__ uint16_t split_part(float v, int part) {
   if (part == 1) return mid;
   return jg::f32_to_bf16(r1 - jg::bf16_to_f32(mid));
 }
-__constant__ const int kWeightPart[6] = {0, 1, 0, 2, 1, 0};  // weight part of contraction block b
-constexpr uint32_t kInputParts = 0u | (0u << 2) | (1u << 4) | (0u << 6) | (1u << 8) | (2u << 10);  // input part of block b
+// Contraction blocks of a split mode: block b multiplies input part x[b] with weight part w[b]
+// (two bits each, block 0 in the lowest bits).
+struct SplitSpec {
+  int parts, nblk;
+  uint32_t xparts, wparts;
+};
+constexpr uint32_t pack_parts(int a, int b, int c, int d, int e, int f) {
+  return (uint32_t)a | ((uint32_t)b << 2) | ((uint32_t)c << 4) | ((uint32_t)d << 6) | ((uint32_t)e << 8) | ((uint32_t)f << 10);
+}
+inline SplitSpec split_spec(int mode) {
+  if (mode == 1) return SplitSpec{3, 6, pack_parts(0, 0, 1, 0, 1, 2), pack_parts(0, 1, 0, 2, 1, 0)};  // fp32
+  if (mode == 2) return SplitSpec{2, 3, pack_parts(0, 0, 1, 0, 0, 0), pack_parts(0, 1, 0, 0, 0, 0)};  // fp16
+  return SplitSpec{1, 1, 0u, 0u};
+}
+template <typename SRC>
+__device__ __forceinline__ float to_float(SRC v) { return (float)v; }
 
-// dst (batch, 3, per_batch) bf16 = the three parts of src (batch, per_batch) fp32
-__global__ __launch_bounds__(256) void split3_kernel(uint16_t* __restrict__ dst, const float* __restrict__ src,
-                                                     size_t per_batch, size_t total) {
+// dst (batch, parts, per_batch) bf16 = the parts of src (batch, per_batch), fp32 or fp16
+template <typename SRC>
+__global__ __launch_bounds__(256) void split_kernel(uint16_t* __restrict__ dst, const SRC* __restrict__ src,
+                                                    size_t per_batch, size_t total, int parts) {
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
     const size_t n = i / per_batch, r = i - n * per_batch;
-    const float v = src[i];
+    const float v = to_float(src[i]);
     const uint16_t hi = jg::f32_to_bf16(v);
     const float hf = jg::bf16_to_f32(hi);
     const float r1 = (hf - hf == 0.0f) ? v - hf : 0.0f;
     const uint16_t mid = jg::f32_to_bf16(r1);
-    const uint16_t lo = jg::f32_to_bf16(r1 - jg::bf16_to_f32(mid));
-    uint16_t* d = dst + n * 3 * per_batch + r;
+    uint16_t* d = dst + n * parts * per_batch + r;
     d[0] = hi;
     d[per_batch] = mid;
-    d[2 * per_batch] = lo;
+    if (parts == 3) d[2 * per_batch] = jg::f32_to_bf16(r1 - jg::bf16_to_f32(mid));
   }
 }
 
-// prep_weights_kernel for split mode: w is fp32, the contraction has 6 blocks of KD * Cp
-// channels, block b holds part kWeightPart[b] of the weights.
+// prep_weights_kernel for a split mode: w is fp32 or fp16, the contraction has nblk blocks of
+// KD * Cp channels, block b holds part (wparts >> 2 b) & 3 of the weights.
+template <typename SRC>
 __global__ __launch_bounds__(256) void prep_weights_split_kernel(uint16_t* __restrict__ dst,
-                                                                 const float* __restrict__ w, int M, int C, int Cp,
+                                                                 const SRC* __restrict__ w, int M, int C, int Cp,
                                                                  int KD, int MT, int mtiles, int wc16, int ngroups,
-                                                                 int transposed) {
-  const int KB = KD * Cp, K = 6 * KB;
+                                                                 int transposed, int nblk, uint32_t wparts) {
+  const int KB = KD * Cp, K = nblk * KB;
   const int total = mtiles * ngroups * TAPS * wc16 * 2 * MT * 8;
   for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
     int e = i & 7;
@@ -203,9 +220,9 @@ __global__ __launch_bounds__(256) void prep_weights_split_kernel(uint16_t* __res
     uint16_t v = 0;
     if (m < M && k < K && c < C) {
       const int kh = tap / KW, kw = tap % KW;
-      const float f = !transposed ? w[((((size_t)m * C + c) * KD + kd) * KH + kh) * KW + kw]
-                                  : w[((((size_t)c * M + m) * KD + (KD - 1 - kd)) * KH + (KH - 1 - kh)) * KW + (KW - 1 - kw)];
-      v = split_part(f, kWeightPart[blk]);
+      const float f = to_float(!transposed ? w[((((size_t)m * C + c) * KD + kd) * KH + kh) * KW + kw]
+                                           : w[((((size_t)c * M + m) * KD + (KD - 1 - kd)) * KH + (KH - 1 - kh)) * KW + (KW - 1 - kw)]);
+      v = split_part(f, (int)((wparts >> (2 * blk)) & 3u));
     }
     dst[i] = v;
   }
@@ -278,8 +295,9 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
   if (p.ngroups == 1) load_weights(0);
   if (tid < MT)
     lds_bias[tid] = (p.bias == nullptr || mt * MT + tid >= p.M) ? 0.0f
-                    : p.out32 ? reinterpret_cast<const float*>(p.bias)[mt * MT + tid]
-                              : jg::bf16_to_f32(p.bias[mt * MT + tid]);
+                    : p.out_kind == 1 ? reinterpret_cast<const float*>(p.bias)[mt * MT + tid]
+                    : p.out_kind == 2 ? (float)reinterpret_cast<const _Float16*>(p.bias)[mt * MT + tid]
+                                      : jg::bf16_to_f32(p.bias[mt * MT + tid]);
 
   // ---- prefetch bookkeeping. A task = 8 channels x 8 pixels of one input row.
   const size_t plane = (size_t)p.Hin * p.Win;
@@ -514,7 +532,7 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     char* ybase = reinterpret_cast<char*>(p.y) +
                   2 * (((size_t)tc.n * p.M + (size_t)mt * MT) * ochan + (size_t)tc.od * plane_o);
     const int m_left = p.M - mt * MT - 4 * kg;  // channels from this lane's first one to the end
-    if (p.out32) {  // uniform: the same walk with 4-byte stores
+    if (p.out_kind == 1) {  // uniform: the same walk with 4-byte stores
       char* ybase32 = reinterpret_cast<char*>(p.y) +
                       4 * (((size_t)tc.n * p.M + (size_t)mt * MT) * ochan + (size_t)tc.od * plane_o);
 #pragma unroll
@@ -543,7 +561,8 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
 #pragma unroll
           for (int i = 0; i < 16; i += 2) {
             f32x2 v2 = {acc[cb][r][i], acc[cb][r][i + 1]};
-            const uint32_t h2 = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
+            const uint32_t h2 = p.out_kind == 2 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, f16x2))
+                                                : __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
             const int m0 = cb * 32 + 8 * (i >> 2) + (i & 3);
             if (!RAGGED || m0 < m_left) store_bf16_lo(ybase + (size_t)m0 * ochan * 2, voff, h2);
             if (!RAGGED || m0 + 1 < m_left) store_bf16_hi(ybase + (size_t)(m0 + 1) * ochan * 2, voff, h2);
@@ -753,7 +772,7 @@ struct Launch {
   const void* w;
   const void* bias;
   void* y;
-  int split;                // fp32 tensors, computed as six bf16 products (split mode)
+  int split;                // split mode: 0 bf16 tensors, 1 fp32 (six bf16 products), 2 fp16 (three)
   int N, C, M, KD;
   int Din, Hin, Win, Dout, Hout, Wout;
   int pad_d, pad_h, pad_w;
@@ -765,15 +784,28 @@ struct Launch {
   int tlo[3], tn[3];
 };
 
-// Bytes of the split copy of an fp32 input (three bf16 parts), rounded to 256
-size_t split_bytes(size_t elements) { return (elements * 3 * 2 + 255) / 256 * 256; }
+// Bytes of the split copy of an input (its bf16 parts), rounded to 256
+size_t split_bytes(size_t elements, int parts) { return (elements * parts * 2 + 255) / 256 * 256; }
 size_t conv_ws_bytes(int split, int KD, int C, int M, size_t x_elements) {
-  const size_t prep = prep_bytes((split ? 6 : 1) * KD * pad16(C), M);
-  return split ? (prep + 255) / 256 * 256 + split_bytes(x_elements) : prep;
+  const SplitSpec sp = split_spec(split);
+  const size_t prep = prep_bytes(sp.nblk * KD * pad16(C), M);
+  return split ? (prep + 255) / 256 * 256 + split_bytes(x_elements, sp.parts) : prep;
+}
+
+template <typename SRC>
+int split_launch(uint16_t* dst, const SRC* src, size_t batch, size_t per_batch, int parts, hipStream_t s) {
+  const size_t total = batch * per_batch;
+  if (total == 0) return JG_OK;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  split_kernel<SRC><<<(unsigned)blocks, 256, 0, s>>>(dst, src, per_batch, total, parts);
+  JG_CHECK_LAUNCH("split_parts_bf16");
+  return JG_OK;
 }
 
 int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const char* who) {
-  const int nblk = L.split ? 6 : 1;
+  const SplitSpec sp = split_spec(L.split);
+  const int nblk = sp.nblk;
   const int K = nblk * L.KD * pad16(L.C);
   const size_t x_elements = (size_t)L.N * L.C * L.Din * L.Hin * L.Win;
   const size_t need = conv_ws_bytes(L.split, L.KD, L.C, L.M, x_elements);
@@ -788,18 +820,23 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   JG_REQUIRE(total_w < (1ull << 31), "%s: weight tensor too large", who);
   const uint16_t* x16 = static_cast<const uint16_t*>(L.x);
   if (L.split) {
-    prep_weights_split_kernel<<<(unsigned)((total_w + 255) / 256), 256, 0, s>>>(
-        wprep, static_cast<const float*>(L.w), L.M, L.C, pad16(L.C), L.KD, MT, lay.mtiles, lay.wc16, lay.ngroups,
-        L.transposed);
-    JG_CHECK_LAUNCH(who);
-    uint16_t* x3 = reinterpret_cast<uint16_t*>(static_cast<char*>(ws) + (lay.prep_bytes + 255) / 256 * 256);
-    if (x_elements > 0) {
-      size_t blocks = (x_elements + 255) / 256;
-      if (blocks > 65536) blocks = 65536;
-      split3_kernel<<<(unsigned)blocks, 256, 0, s>>>(x3, static_cast<const float*>(L.x), x_elements / L.N, x_elements);
-      JG_CHECK_LAUNCH(who);
+    const unsigned wblocks = (unsigned)((total_w + 255) / 256);
+    uint16_t* xs = reinterpret_cast<uint16_t*>(static_cast<char*>(ws) + (lay.prep_bytes + 255) / 256 * 256);
+    int rc;
+    if (L.split == 1) {
+      prep_weights_split_kernel<float><<<wblocks, 256, 0, s>>>(wprep, static_cast<const float*>(L.w), L.M, L.C,
+                                                                pad16(L.C), L.KD, MT, lay.mtiles, lay.wc16, lay.ngroups,
+                                                                L.transposed, nblk, sp.wparts);
+      rc = split_launch(xs, static_cast<const float*>(L.x), (size_t)L.N, x_elements / L.N, sp.parts, s);
+    } else {
+      prep_weights_split_kernel<_Float16><<<wblocks, 256, 0, s>>>(wprep, static_cast<const _Float16*>(L.w), L.M, L.C,
+                                                                   pad16(L.C), L.KD, MT, lay.mtiles, lay.wc16,
+                                                                   lay.ngroups, L.transposed, nblk, sp.wparts);
+      rc = split_launch(xs, static_cast<const _Float16*>(L.x), (size_t)L.N, x_elements / L.N, sp.parts, s);
     }
-    x16 = x3;
+    JG_CHECK_LAUNCH(who);
+    if (rc) return rc;
+    x16 = xs;
   } else {
     prep_weights_kernel<<<(unsigned)((total_w + 255) / 256), 256, 0, s>>>(wprep, static_cast<const uint16_t*>(L.w), L.M,
                                                                            L.C, pad16(L.C), L.KD, MT, lay.mtiles,
@@ -808,12 +845,12 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   }
 
   FwdParams p;
-  p.x_end = reinterpret_cast<const char*>(x16) + 2 * x_elements * (L.split ? 3 : 1);
+  p.x_end = reinterpret_cast<const char*>(x16) + 2 * x_elements * sp.parts;
   p.x = x16; p.wprep = reinterpret_cast<const u32x4*>(wprep);
   p.bias = static_cast<const uint16_t*>(L.bias); p.y = static_cast<uint16_t*>(L.y);
   p.N = L.N; p.C = L.C; p.M = L.M; p.KD = L.KD;
   p.Cp = pad16(L.C);
-  p.nblk = nblk; p.Cx = nblk == 6 ? 3 * L.C : L.C; p.xmap = nblk == 6 ? kInputParts : 0u; p.out32 = L.split;
+  p.nblk = nblk; p.Cx = sp.parts * L.C; p.xmap = sp.xparts; p.out_kind = L.split;
   p.Din = L.Din; p.Hin = L.Hin; p.Win = L.Win;
   p.Dout = L.Dout; p.Hout = L.Hout; p.Wout = L.Wout;
   p.pad_d = L.pad_d; p.pad_h = L.pad_h; p.pad_w = L.pad_w;
@@ -866,21 +903,17 @@ namespace jg {
 
 // fp32 runs in split mode (three bf16 parts per operand, fp32 result); its 4-byte stores halve
 // the extent the 32-bit lane offsets reach.
+static int split_mode(int dtype) { return dtype == JG_F32 ? 1 : (dtype == JG_F16 ? 2 : 0); }
 static bool dtype_ok(const ConvGeom& g, int dtype) {
-  if (dtype == JG_BF16) return true;
+  if (dtype == JG_BF16 || dtype == JG_F16) return true;
   if (dtype != JG_F32) return false;
   const size_t in_sz = (size_t)g.in[0] * g.in[1] * g.in[2], out_sz = (size_t)g.out[0] * g.out[1] * g.out[2];
   const size_t big = in_sz > out_sz ? in_sz : out_sz;
   return big * 4 * 72 < (1ull << 31);
 }
-int split3_bf16(uint16_t* dst, const float* src, size_t batch, size_t per_batch, hipStream_t s) {
-  const size_t total = batch * per_batch;
-  if (total == 0) return JG_OK;
-  size_t blocks = (total + 255) / 256;
-  if (blocks > 65536) blocks = 65536;
-  split3_kernel<<<(unsigned)blocks, 256, 0, s>>>(dst, src, per_batch, total);
-  JG_CHECK_LAUNCH("split3_bf16");
-  return JG_OK;
+int split_parts_bf16(uint16_t* dst, const void* src, int src_dtype, size_t batch, size_t per_batch, hipStream_t s) {
+  if (src_dtype == JG_F32) return split_launch(dst, static_cast<const float*>(src), batch, per_batch, 3, s);
+  return split_launch(dst, static_cast<const _Float16*>(src), batch, per_batch, 2, s);
 }
 
 bool mfma_fwd_supported(const ConvGeom& g, int dtype) {
@@ -894,10 +927,10 @@ bool mfma_dgrad_supported(const ConvGeom& g, int dtype) {
 }
 
 size_t mfma_fwd_workspace(const ConvGeom& g, int dtype) {
-  return conv_ws_bytes(dtype == JG_F32, g.k[0], g.cin, g.cout, (size_t)g.batch * g.cin * g.in[0] * g.in[1] * g.in[2]);
+  return conv_ws_bytes(split_mode(dtype), g.k[0], g.cin, g.cout, (size_t)g.batch * g.cin * g.in[0] * g.in[1] * g.in[2]);
 }
 size_t mfma_dgrad_workspace(const ConvGeom& g, int dtype) {
-  return conv_ws_bytes(dtype == JG_F32, g.k[0], g.cout, g.cin, (size_t)g.batch * g.cout * g.out[0] * g.out[1] * g.out[2]);
+  return conv_ws_bytes(split_mode(dtype), g.k[0], g.cout, g.cin, (size_t)g.batch * g.cout * g.out[0] * g.out[1] * g.out[2]);
 }
 
 static int fwd_launch(void* y, const void* x, const void* xt, const int* tlo, const int* tn, const void* w,
@@ -905,7 +938,7 @@ static int fwd_launch(void* y, const void* x, const void* xt, const int* tlo, co
                       const char* who, int dtype = JG_BF16) {
   Launch L;
   L.x = x; L.w = w; L.bias = bias; L.y = y;
-  L.split = dtype == JG_F32;
+  L.split = split_mode(dtype);
   L.N = (int)g.batch; L.C = g.cin; L.M = g.cout; L.KD = g.k[0];
   L.Din = g.in[0]; L.Hin = g.in[1]; L.Win = g.in[2];
   L.Dout = g.out[0]; L.Hout = g.out[1]; L.Wout = g.out[2];
@@ -975,7 +1008,7 @@ static int dgrad_launch(void* gx, void* const* strips, const int* lo, const int*
                         const char* who, int dtype = JG_BF16) {
   Launch L;
   L.x = go; L.w = w; L.bias = nullptr; L.y = gx;
-  L.split = dtype == JG_F32;
+  L.split = split_mode(dtype);
   L.N = (int)g.batch; L.C = g.cout; L.M = g.cin; L.KD = g.k[0];
   L.Din = g.out[0]; L.Hin = g.out[1]; L.Win = g.out[2];
   L.Dout = g.in[0]; L.Hout = g.in[1]; L.Wout = g.in[2];

@@ -571,21 +571,25 @@ __global__ __launch_bounds__(256) void wgrad_reduce_kernel(void* __restrict__ gw
   }
 }
 
-// gw[co][ci][t] (fp32) = sum over the part pairs (i, j), i + j <= 2, smallest first, of
+// gw[co][ci][t] (fp32) = sum over the part pairs (i, j), i + j <= parts - 1, smallest first, of
 // tmp[i * cout + co][j * cin + ci][t]: the part products of the split mode from one launch.
 __global__ __launch_bounds__(256) void wgrad_combine_parts_kernel(float* __restrict__ gw, const float* __restrict__ tmp,
-                                                                  int cout, int cin, int taps) {
+                                                                  int cout, int cin, int taps, int parts) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= cout * cin * taps) return;
   const int t = idx % taps, ci = (idx / taps) % cin, co = idx / (taps * cin);
-  auto at = [&](int i, int j) { return tmp[((size_t)(i * cout + co) * (3 * cin) + (j * cin + ci)) * taps + t]; };
-  float sum = at(0, 2);
-  sum += at(1, 1);
-  sum += at(2, 0);
-  sum += at(0, 1);
-  sum += at(1, 0);
-  sum += at(0, 0);
+  float sum = 0.0f;
+  for (int order = parts - 1; order >= 0; --order)
+    for (int i = 0; i <= order; ++i) {
+      const int j = order - i;
+      sum += tmp[((size_t)(i * cout + co) * (parts * cin) + (j * cin + ci)) * taps + t];
+    }
   gw[idx] = sum;
+}
+
+__global__ __launch_bounds__(256) void f32_to_f16_kernel(_Float16* __restrict__ dst, const float* __restrict__ src, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = (_Float16)src[i];
 }
 
 int cu_count() {
@@ -662,20 +666,25 @@ int launch(const WgradParams& p, bool even, int wgs, hipStream_t s, const char* 
 
 namespace jg {
 
-// Split mode with few channels: the three parts of both operands fit one block.
-static bool parts_fit_one_block(const ConvGeom& g, const Blocking& bl) {
-  return 3 * g.cout <= bl.cob_max() && 3 * g.cin <= bl.cib_max();
+static int parts_of(int dtype) { return dtype == JG_F32 ? 3 : (dtype == JG_F16 ? 2 : 1); }
+// Split mode with few channels: the parts of both operands fit one block.
+static bool parts_fit_one_block(const ConvGeom& g, const Blocking& bl, int parts) {
+  return parts > 1 && parts * g.cout <= bl.cob_max() && parts * g.cin <= bl.cib_max();
 }
-static size_t parts_tmp_bytes(const ConvGeom& g, const Blocking& bl) {
-  if (!parts_fit_one_block(g, bl)) return 0;
-  return ((size_t)9 * g.cout * g.cin * bl.KD * 9 * sizeof(float) + 255) / 256 * 256;
+static size_t parts_tmp_bytes(const ConvGeom& g, const Blocking& bl, int parts) {
+  if (!parts_fit_one_block(g, bl, parts)) return 0;
+  return ((size_t)parts * parts * g.cout * g.cin * bl.KD * 9 * sizeof(float) + 255) / 256 * 256;
+}
+// fp16: the part products are added up in fp32 here before the one rounding to fp16
+static size_t acc32_bytes(const ConvGeom& g, int dtype) {
+  return dtype == JG_F16 ? ((size_t)g.cout * g.cin * g.k[0] * 9 * sizeof(float) + 255) / 256 * 256 : 0;
 }
 
-// fp32 runs in split mode: both operands are copied as three bf16 parts each (as extra channels)
-// and the six part products whose indices add up to at most 2 are accumulated in fp32.
+// fp32 / fp16 run in split mode: both operands are copied as three / two bf16 parts each (as extra
+// channels) and the six / three part products whose indices add up to at most 2 / 1 are accumulated in fp32.
 bool mfma_wgrad_supported(const ConvGeom& g, int dtype) {
   Blocking b;
-  if ((dtype != JG_BF16 && dtype != JG_F32) || g.batch <= 0) return false;
+  if ((dtype != JG_BF16 && dtype != JG_F32 && dtype != JG_F16) || g.batch <= 0) return false;
   return blocks_of(g, &b);
 }
 
@@ -687,15 +696,18 @@ static size_t partial_bytes(const ConvGeom& g) {
   const size_t n = wgs * HALVES * 9 * b.cob_max() * (b.KD * b.cib_max()) * sizeof(float) + wgs * b.cob_max() * sizeof(float);
   return (n + 255) / 256 * 256;
 }
-static size_t split_copy_bytes(size_t elements) { return (elements * 3 * 2 + 255) / 256 * 256; }
+static size_t split_copy_bytes(size_t elements, int parts) { return (elements * parts * 2 + 255) / 256 * 256; }
+// workspace: [partials | x parts | g parts | fp32 sum (fp16 only) | part products of the one-block launch]
 size_t mfma_wgrad_workspace(const ConvGeom& g, int dtype) {
   size_t n = partial_bytes(g);
-  if (dtype == JG_F32) {
-    n += split_copy_bytes((size_t)g.batch * g.cin * g.in[0] * g.in[1] * g.in[2]);
-    n += split_copy_bytes((size_t)g.batch * g.cout * g.out[0] * g.out[1] * g.out[2]);
+  const int parts = parts_of(dtype);
+  if (parts > 1) {
+    n += split_copy_bytes((size_t)g.batch * g.cin * g.in[0] * g.in[1] * g.in[2], parts);
+    n += split_copy_bytes((size_t)g.batch * g.cout * g.out[0] * g.out[1] * g.out[2], parts);
+    n += acc32_bytes(g, dtype);
     Blocking b{32, 32, 1};
     blocks_of(g, &b);
-    n += parts_tmp_bytes(g, b);  // last in the workspace
+    n += parts_tmp_bytes(g, b, parts);
   }
   return n;
 }
@@ -738,19 +750,27 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
   JG_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 15) == 0, "%s: workspace must be 16-byte aligned",
              who);
   const size_t x_cs = (size_t)g.in[0] * g.in[1] * g.in[2], g_cs = (size_t)g.out[0] * g.out[1] * g.out[2];
-  const bool split = dtype == JG_F32;
+  const int parts = parts_of(dtype);
+  const bool split = parts > 1;
+  float* sum32 = static_cast<float*>(gw);  // where the part products are added up (split mode)
+  float* one_block_tmp = nullptr;
   if (split) {
     if (gb != nullptr || xt != nullptr)
-      JG_FAIL(JG_ERR_UNSUPPORTED, "%s: fp32 has neither the fused bias gradient nor the framed input", who);
+      JG_FAIL(JG_ERR_UNSUPPORTED, "%s: fp32 / fp16 have neither the fused bias gradient nor the framed input", who);
     char* base = static_cast<char*>(ws) + partial_bytes(g);
-    uint16_t* x3 = reinterpret_cast<uint16_t*>(base);
-    uint16_t* g3 = reinterpret_cast<uint16_t*>(base + split_copy_bytes((size_t)g.batch * g.cin * x_cs));
-    int rc = split3_bf16(x3, static_cast<const float*>(x), (size_t)g.batch, (size_t)g.cin * x_cs, s);
+    uint16_t* xs = reinterpret_cast<uint16_t*>(base);
+    base += split_copy_bytes((size_t)g.batch * g.cin * x_cs, parts);
+    uint16_t* gs = reinterpret_cast<uint16_t*>(base);
+    base += split_copy_bytes((size_t)g.batch * g.cout * g_cs, parts);
+    if (dtype == JG_F16) sum32 = reinterpret_cast<float*>(base);
+    base += acc32_bytes(g, dtype);
+    one_block_tmp = reinterpret_cast<float*>(base);
+    int rc = split_parts_bf16(xs, x, dtype, (size_t)g.batch, (size_t)g.cin * x_cs, s);
     if (rc) return rc;
-    rc = split3_bf16(g3, static_cast<const float*>(go), (size_t)g.batch, (size_t)g.cout * g_cs, s);
+    rc = split_parts_bf16(gs, go, dtype, (size_t)g.batch, (size_t)g.cout * g_cs, s);
     if (rc) return rc;
-    x = x3;
-    go = g3;
+    x = xs;
+    go = gs;
   }
   const bool even = (g.in[2] % 2 == 0) && (g.p[2] % 2 == 0) && (g.out[2] % 2 == 0) &&
                     ((reinterpret_cast<uintptr_t>(x) & 3) == 0) &&
@@ -759,8 +779,15 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
     JG_FAIL(JG_ERR_UNSUPPORTED, "%s: the framed input does not cover this geometry / alignment", who);
   // part products (g part, x part), smallest first; plain mode: the one product
   static const int kPairs[6][2] = {{0, 2}, {1, 1}, {2, 0}, {0, 1}, {1, 0}, {0, 0}};
-  const int npairs = split ? 6 : 1, first_pair = split ? 0 : 5;
-  const int parts = split ? 3 : 1;
+  const int npairs = parts == 3 ? 6 : (parts == 2 ? 3 : 1), first_pair = 6 - npairs;
+  const int gw_count = g.cout * g.cin * g.k[0] * 9;
+  auto finish = [&]() -> int {  // fp16: the one rounding of the fp32 sum
+    if (dtype == JG_F16) {
+      f32_to_f16_kernel<<<(gw_count + 255) / 256, 256, 0, s>>>(static_cast<_Float16*>(gw), sum32, gw_count);
+      JG_CHECK_LAUNCH(who);
+    }
+    return JG_OK;
+  };
   WgradParams p;
   p.part = static_cast<float*>(ws);
   p.x_end = static_cast<const char*>(x) + 2 * (size_t)g.batch * parts * g.cin * x_cs;
@@ -809,19 +836,16 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
     return JG_OK;
   };
 
-  if (split && parts_fit_one_block(g, bl)) {
-    // few channels: all nine part products in one launch (the parts are 3 x cout and 3 x cin channels
-    // of one block), then the six that count are added up
-    float* tmp = reinterpret_cast<float*>(static_cast<char*>(ws) + mfma_wgrad_workspace(g, dtype) -
-                                          parts_tmp_bytes(g, bl));
-    const int cob = 3 * g.cout > 32 ? 64 : 32, cib = 3 * g.cin > 32 ? 64 : 32;  // within the block limits (checked)
-    int rc = run_block(0, 0, cob, cib, 3 * g.cout, 3 * g.cin, tmp, 3 * g.cin, true, false, nullptr);
+  if (parts_fit_one_block(g, bl, parts)) {
+    // few channels: all part products in one launch (the parts are parts x cout and parts x cin
+    // channels of one block), then the ones that count are added up
+    const int cob = parts * g.cout > 32 ? 64 : 32, cib = parts * g.cin > 32 ? 64 : 32;  // within the block limits (checked)
+    int rc = run_block(0, 0, cob, cib, parts * g.cout, parts * g.cin, one_block_tmp, parts * g.cin, true, false, nullptr);
     if (rc) return rc;
-    const int total = g.cout * g.cin * bl.KD * 9;
-    wgrad_combine_parts_kernel<<<(total + 255) / 256, 256, 0, s>>>(static_cast<float*>(gw), tmp, g.cout, g.cin,
-                                                                   bl.KD * 9);
+    wgrad_combine_parts_kernel<<<(gw_count + 255) / 256, 256, 0, s>>>(sum32, one_block_tmp, g.cout, g.cin, bl.KD * 9,
+                                                                      parts);
     JG_CHECK_LAUNCH(who);
-    return JG_OK;
+    return finish();
   }
   for (int co0 = 0; co0 < g.cout;) {
     const int cob = block_width(g.cout, co0, bl.cob);
@@ -832,7 +856,7 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
       const size_t blk_at = ((size_t)co0 * g.cin + ci0) * bl.KD * 9;
       for (int pr = 0; pr < npairs; ++pr) {
         const int gpart = kPairs[first_pair + pr][0], xpart = kPairs[first_pair + pr][1];
-        void* out = split ? static_cast<void*>(static_cast<float*>(gw) + blk_at)
+        void* out = split ? static_cast<void*>(sum32 + blk_at)
                           : static_cast<void*>(static_cast<uint16_t*>(gw) + blk_at);
         // the bias gradient comes from the g rows: once per block of output channels
         uint16_t* gb_out = (gb != nullptr && ci0 == 0) ? static_cast<uint16_t*>(gb) + co0 : nullptr;
@@ -844,7 +868,7 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
     }
     co0 += cob;
   }
-  return JG_OK;
+  return finish();
 }
 
 }  // namespace jg
