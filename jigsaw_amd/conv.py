@@ -90,6 +90,95 @@ def _check_args(x_like, w, groups, padding):
     return n
 
 
+# --------------------------------------------------------------------------- #
+# Non-overlapping kernels (kernel == stride, no padding, no dilation: patch embeddings,
+# 1 x 1 convolutions) are a GEMM over the patches: the patch matrix is laid out once and the
+# MFMA projection kernels (jg_proj_nt / jg_proj_tn) do the arithmetic.
+# --------------------------------------------------------------------------- #
+def _patch_gemm_ok(dtype, c_in, c_out, kernel, stride, padding, dilation) -> bool:
+    if dtype != torch.bfloat16:
+        return False
+    if any(k != s for k, s in zip(kernel, stride)) or any(padding) or any(d != 1 for d in dilation):
+        return False
+    k_elems = c_in
+    for k in kernel:
+        k_elems *= int(k)
+    return k_elems % 8 == 0 and c_out % 8 == 0
+
+
+def _patchify(x: torch.Tensor, kernel, out_sp) -> torch.Tensor:
+    """``(N, C, *spatial) -> (N * prod(out), C * prod(kernel))``, features ordered as the weight's ``(C, *kernel)``."""
+    n = len(kernel)
+    x = x[(slice(None), slice(None)) + tuple(slice(0, o * k) for o, k in zip(out_sp, kernel))]
+    shape = [x.shape[0], x.shape[1]]
+    for o, k in zip(out_sp, kernel):
+        shape += [o, k]
+    x = x.reshape(shape)
+    o_dims = [2 + 2 * i for i in range(n)]
+    k_dims = [3 + 2 * i for i in range(n)]
+    rows = x.shape[0]
+    for o in out_sp:
+        rows *= o
+    return x.permute(0, *o_dims, 1, *k_dims).reshape(rows, -1)
+
+
+def _unpatchify(p: torch.Tensor, input_shape, kernel, out_sp) -> torch.Tensor:
+    """Inverse of :func:`_patchify`; cells no patch covers (a remainder of the extent) are zero."""
+    n = len(kernel)
+    batch, c = input_shape[0], input_shape[1]
+    p = p.reshape(batch, *out_sp, c, *kernel)
+    perm = [0, n + 1]
+    for i in range(n):
+        perm += [1 + i, n + 2 + i]
+    covered = tuple(o * k for o, k in zip(out_sp, kernel))
+    body = p.permute(perm).reshape(batch, c, *covered)
+    if covered == tuple(input_shape[2:]):
+        return body.contiguous()
+    gx = torch.zeros(input_shape, dtype=p.dtype, device=p.device)
+    gx[(slice(None), slice(None)) + tuple(slice(0, v) for v in covered)] = body
+    return gx
+
+
+def _proj_nt(a: torch.Tensor, w2: torch.Tensor, bias) -> torch.Tensor:
+    rows, k = a.shape
+    out = torch.empty(rows, w2.shape[0], dtype=a.dtype, device=a.device)
+    if rows:
+        rc = _lib.load().jg_proj_nt(_lib.ptr(out), _lib.ptr(a), _lib.ptr(w2), _lib.ptr(bias), _lib.dtype_code(a.dtype),
+                                    rows, w2.shape[0], k, 0, 0, 1, 1, 1, 1, _lib.stream_ptr(a.device))
+        _lib.check(rc, "jg_proj_nt")
+    return out
+
+
+def _tokens_of(g: torch.Tensor) -> torch.Tensor:
+    """``(N, M, *out) -> (N * prod(out), M)``."""
+    n = g.dim() - 2
+    return g.permute(0, *range(2, 2 + n), 1).reshape(-1, g.shape[1])
+
+
+# --------------------------------------------------------------------------- #
+# Kernels with extents 1 or 3 per axis (1 x 1, 1 x 3, 3 x 1, ...) at stride 1 run on the 3 x 3 (x 3)
+# MFMA kernels: the weights sit in the centre of a zero 3 x 3 (x 3) kernel and the padding grows
+# by one on the axes that were 1. Same result (the added taps multiply zeros), and although most of
+# the matrix-core work is on zeros it is far faster than the FMA kernels.
+# --------------------------------------------------------------------------- #
+def _embed3(kernel, stride, dilation):
+    """Per-axis tap offset ((3 - k) / 2) when the kernel embeds into 3 x 3 (x 3), else ``None``."""
+    n = len(kernel)
+    if n not in (2, 3) or all(k == 3 for k in kernel):
+        return None
+    if any(k not in (1, 3) for k in kernel) or any(s != 1 for s in stride):
+        return None
+    if any(d != 1 and k != 1 for d, k in zip(dilation, kernel)):
+        return None
+    return tuple((3 - k) // 2 for k in kernel)
+
+
+def _embed_weight(w: torch.Tensor, off) -> torch.Tensor:
+    w3 = torch.zeros((w.shape[0], w.shape[1]) + (3,) * len(off), dtype=w.dtype, device=w.device)
+    w3[(slice(None), slice(None)) + tuple(slice(o, 3 - o) for o in off)] = w
+    return w3
+
+
 def conv_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1) -> torch.Tensor:
     """``F.conv{1,2,3}d(x, w, b, stride, padding, dilation, groups)`` on the HIP kernels."""
     _lib.require_gpu(x, w, b)
@@ -101,9 +190,15 @@ def conv_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1) -> torch
     if x.shape[1] != w.shape[1]:
         raise RuntimeError(f"expected input to have {w.shape[1]} channels, but got {x.shape[1]} channels instead")
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
+    off = _embed3(tuple(w.shape[2:]), stride, dilation)
+    if off is not None:
+        return conv_nd(x, _embed_weight(w, off), b, stride=1, padding=tuple(p + o for p, o in zip(padding, off)))
     x, w = x.contiguous(), w.contiguous()
     b = None if b is None else b.contiguous()
     out_sp = _out_spatial(x.shape[2:], w.shape[2:], stride, padding, dilation)
+    if _patch_gemm_ok(x.dtype, x.shape[1], w.shape[0], w.shape[2:], stride, padding, dilation):
+        y_tok = _proj_nt(_patchify(x, w.shape[2:], out_sp), w.reshape(w.shape[0], -1), b)
+        return y_tok.reshape(x.shape[0], *out_sp, w.shape[0]).permute(0, n + 1, *range(1, n + 1)).contiguous()
     y = torch.empty((x.shape[0], w.shape[0], *out_sp), dtype=x.dtype, device=x.device)
     desc = _desc(x.shape[0], x.shape[1], w.shape[0], x.shape[2:], w.shape[2:], stride, padding, dilation, groups)
     ws, nbytes = _workspace(desc, 0, x.dtype, x.device)
@@ -125,6 +220,10 @@ def conv_nd_input(input_shape, w, g, *, stride=1, padding=0, dilation=1, groups=
     if g.dtype != w.dtype:
         raise RuntimeError(f"grad_output type ({g.dtype}) and weight type ({w.dtype}) should be the same")
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
+    off = _embed3(tuple(w.shape[2:]), stride, dilation)
+    if off is not None:
+        return conv_nd_input(input_shape, _embed_weight(w, off), g, stride=1,
+                             padding=tuple(p + o for p, o in zip(padding, off)))
     g, w = g.contiguous(), w.contiguous()
     out_sp = _out_spatial(input_shape[2:], w.shape[2:], stride, padding, dilation)
     if tuple(g.shape) != (input_shape[0], w.shape[0], *out_sp):
@@ -132,6 +231,10 @@ def conv_nd_input(input_shape, w, g, *, stride=1, padding=0, dilation=1, groups=
             f"grad_output shape {tuple(g.shape)} does not match the convolution of an input of shape {input_shape} "
             f"(expected {(input_shape[0], w.shape[0], *out_sp)})"
         )
+    if _patch_gemm_ok(g.dtype, w.shape[1], w.shape[0], w.shape[2:], stride, padding, dilation):
+        # gradient of every patch = g_tokens x W, then back to the image layout
+        w2t = w.reshape(w.shape[0], -1).t().contiguous()
+        return _unpatchify(_proj_nt(_tokens_of(g).contiguous(), w2t, None), input_shape, w.shape[2:], out_sp)
     gx = torch.empty(input_shape, dtype=g.dtype, device=g.device)
     desc = _desc(input_shape[0], input_shape[1], w.shape[0], input_shape[2:], w.shape[2:], stride, padding, dilation, groups)
     ws, nbytes = _workspace(desc, 1, g.dtype, g.device)
@@ -288,10 +391,37 @@ def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, group
     if x.dtype != g.dtype:
         raise RuntimeError(f"input type ({x.dtype}) and grad_output type ({g.dtype}) should be the same")
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
+    off = _embed3(weight_shape[2:], stride, dilation)
+    if off is not None:
+        # gradient of the 3 x 3 (x 3) kernel the weights sit in; its centre taps are the answer
+        res = conv_nd_weight(x, weight_shape[:2] + (3,) * n, g, stride=1,
+                             padding=tuple(p + o for p, o in zip(padding, off)), with_bias_grad=with_bias_grad)
+        gw3 = res[0] if with_bias_grad else res
+        gw = gw3[(slice(None), slice(None)) + tuple(slice(o, 3 - o) for o in off)].contiguous()
+        return (gw, res[1]) if with_bias_grad else gw
     x, g = x.contiguous(), g.contiguous()
     out_sp = _out_spatial(x.shape[2:], weight_shape[2:], stride, padding, dilation)
     if tuple(g.shape) != (x.shape[0], weight_shape[0], *out_sp) or x.shape[1] != weight_shape[1]:
         raise ValueError(f"grad_output {tuple(g.shape)} / input {tuple(x.shape)} do not match weight {weight_shape}")
+    if _patch_gemm_ok(x.dtype, weight_shape[1], weight_shape[0], weight_shape[2:], stride, padding, dilation):
+        # gw = g_tokens^T x patches (contraction over the patches), the bias gradient from the same pass
+        patches, g_tok = _patchify(x, weight_shape[2:], out_sp), _tokens_of(g).contiguous()
+        rows, k = patches.shape
+        lib = _lib.load()
+        gw2 = torch.empty(weight_shape[0], k, dtype=x.dtype, device=x.device)
+        gb = torch.empty(weight_shape[0], dtype=x.dtype, device=x.device) if with_bias_grad else None
+        if rows:
+            nb = int(lib.jg_proj_tn_workspace(rows, weight_shape[0], k))
+            pws = torch.empty(max(nb, 16), dtype=torch.uint8, device=x.device)
+            rc = lib.jg_proj_tn(_lib.ptr(gw2), _lib.ptr(gb), _lib.ptr(g_tok), _lib.ptr(patches), _lib.dtype_code(x.dtype),
+                                rows, weight_shape[0], k, 0, 0, 1, 1, 1, 1, _lib.ptr(pws), nb, _lib.stream_ptr(x.device))
+            _lib.check(rc, "jg_proj_tn")
+        else:
+            gw2.zero_()
+            if gb is not None:
+                gb.zero_()
+        gw = gw2.reshape(weight_shape)
+        return (gw, gb) if with_bias_grad else gw
     gw = torch.empty(weight_shape, dtype=x.dtype, device=x.device)
     desc = _desc(x.shape[0], x.shape[1], weight_shape[0], x.shape[2:], weight_shape[2:], stride, padding, dilation, groups)
     ws, nbytes = _workspace(desc, 2, x.dtype, x.device)

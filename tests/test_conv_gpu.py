@@ -50,6 +50,19 @@ PRIM_CASES = [
     (2, 69, 64, (37, 66), (3, 3), (1, 1), (0, 0), (1, 1)),
     (1, 64, 69, (20, 70), (3, 3), (1, 1), (1, 1), (1, 1)),
     (2, 20, 24, (5, 18, 34), (3, 3, 3), (1, 1, 1), (1, 0, 1), (1, 1, 1)),
+    # non-overlapping kernels (patch embeddings, 1 x 1): a GEMM over the patches in bf16
+    (2, 8, 16, (16, 24), (4, 4), (4, 4), (0, 0), (1, 1)),
+    (2, 16, 32, (9, 11), (1, 1), (1, 1), (0, 0), (1, 1)),
+    (2, 8, 8, (17, 19), (4, 4), (4, 4), (0, 0), (1, 1)),
+    (1, 4, 8, (4, 8, 10), (2, 2, 2), (2, 2, 2), (0, 0, 0), (1, 1, 1)),
+    (3, 72, 264, (64, 48), (8, 8), (8, 8), (0, 0), (1, 1)),
+    (2, 16, 32, (20, 36), (2, 2), (2, 2), (0, 0), (1, 1)),
+    # extents 1 or 3 at stride 1: embedded in the 3 x 3 (x 3) MFMA kernels
+    (2, 64, 64, (20, 70), (1, 1), (1, 1), (0, 0), (1, 1)),
+    (1, 16, 24, (19, 33), (1, 3), (1, 1), (0, 1), (1, 1)),
+    (2, 8, 5, (12, 40), (3, 1), (1, 1), (1, 0), (1, 1)),
+    (1, 16, 16, (5, 10, 34), (1, 1, 1), (1, 1, 1), (0, 0, 0), (1, 1, 1)),
+    (1, 8, 8, (6, 9, 20), (3, 1, 3), (1, 1, 1), (1, 0, 0), (1, 1, 1)),
 ]
 
 
