@@ -179,6 +179,27 @@ def _embed_weight(w: torch.Tensor, off) -> torch.Tensor:
     return w3
 
 
+# --------------------------------------------------------------------------- #
+# Strided kernels with extents 1 or 3 (3 x 3 stride 2 down-sampling, ...): the stride-1 result
+# sampled at the stride (forward), and the stride-1 gradients of the output gradient with zeros
+# between its cells (backward). Costs prod(stride) times the matrix-core work of the strided
+# layer and a copy, and still beats the FMA kernels by an order of magnitude.
+# --------------------------------------------------------------------------- #
+def _dense_stride_ok(kernel, stride, dilation) -> bool:
+    if len(kernel) not in (2, 3) or all(s == 1 for s in stride):
+        return False
+    if any(k not in (1, 3) for k in kernel) or any(d != 1 for d in dilation):
+        return False
+    return not all(k == s for k, s in zip(kernel, stride))  # kernel = stride has its own route
+
+
+def _stuffed(g: torch.Tensor, dense_sp, stride) -> torch.Tensor:
+    """``g`` with ``stride - 1`` zeros between its cells: the output gradient of the stride-1 layer."""
+    up = torch.zeros((g.shape[0], g.shape[1], *dense_sp), dtype=g.dtype, device=g.device)
+    up[(slice(None), slice(None)) + tuple(slice(0, (o - 1) * s + 1, s) for o, s in zip(g.shape[2:], stride))] = g
+    return up
+
+
 def conv_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1) -> torch.Tensor:
     """``F.conv{1,2,3}d(x, w, b, stride, padding, dilation, groups)`` on the HIP kernels."""
     _lib.require_gpu(x, w, b)
@@ -190,6 +211,10 @@ def conv_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1) -> torch
     if x.shape[1] != w.shape[1]:
         raise RuntimeError(f"expected input to have {w.shape[1]} channels, but got {x.shape[1]} channels instead")
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
+    if _dense_stride_ok(tuple(w.shape[2:]), stride, dilation):
+        out_sp = _out_spatial(x.shape[2:], w.shape[2:], stride, padding, dilation)
+        dense = conv_nd(x, w, b, stride=1, padding=padding)
+        return dense[(slice(None), slice(None)) + tuple(slice(0, (o - 1) * s + 1, s) for o, s in zip(out_sp, stride))].contiguous()
     off = _embed3(tuple(w.shape[2:]), stride, dilation)
     if off is not None:
         return conv_nd(x, _embed_weight(w, off), b, stride=1, padding=tuple(p + o for p, o in zip(padding, off)))
@@ -220,6 +245,9 @@ def conv_nd_input(input_shape, w, g, *, stride=1, padding=0, dilation=1, groups=
     if g.dtype != w.dtype:
         raise RuntimeError(f"grad_output type ({g.dtype}) and weight type ({w.dtype}) should be the same")
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
+    if _dense_stride_ok(tuple(w.shape[2:]), stride, dilation):
+        dense_sp = _out_spatial(input_shape[2:], w.shape[2:], (1,) * n, padding, dilation)
+        return conv_nd_input(input_shape, w, _stuffed(g, dense_sp, stride), stride=1, padding=padding)
     off = _embed3(tuple(w.shape[2:]), stride, dilation)
     if off is not None:
         return conv_nd_input(input_shape, _embed_weight(w, off), g, stride=1,
@@ -391,6 +419,10 @@ def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, group
     if x.dtype != g.dtype:
         raise RuntimeError(f"input type ({x.dtype}) and grad_output type ({g.dtype}) should be the same")
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
+    if _dense_stride_ok(weight_shape[2:], stride, dilation):
+        dense_sp = _out_spatial(x.shape[2:], weight_shape[2:], (1,) * n, padding, dilation)
+        return conv_nd_weight(x, weight_shape, _stuffed(g, dense_sp, stride), stride=1, padding=padding,
+                              with_bias_grad=with_bias_grad)
     off = _embed3(weight_shape[2:], stride, dilation)
     if off is not None:
         # gradient of the 3 x 3 (x 3) kernel the weights sit in; its centre taps are the answer

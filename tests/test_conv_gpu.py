@@ -63,6 +63,11 @@ PRIM_CASES = [
     (2, 8, 5, (12, 40), (3, 1), (1, 1), (1, 0), (1, 1)),
     (1, 16, 16, (5, 10, 34), (1, 1, 1), (1, 1, 1), (0, 0, 0), (1, 1, 1)),
     (1, 8, 8, (6, 9, 20), (3, 1, 3), (1, 1, 1), (1, 0, 0), (1, 1, 1)),
+    # strided 3 x 3 (down-sampling): the stride-1 kernels, sampled / zero-stuffed
+    (2, 16, 32, (33, 40), (3, 3), (2, 2), (1, 1), (1, 1)),
+    (1, 8, 8, (20, 31), (3, 3), (2, 3), (0, 1), (1, 1)),
+    (1, 8, 16, (7, 12, 18), (3, 3, 3), (2, 2, 2), (1, 1, 1), (1, 1, 1)),
+    (2, 8, 8, (16, 16), (1, 1), (2, 2), (0, 0), (1, 1)),
 ]
 
 
