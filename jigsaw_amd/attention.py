@@ -97,12 +97,30 @@ def _bias_args(bias, batch, sq, sk):
     return bias, period
 
 
+def _pads_to_64(q, k, bias) -> bool:
+    """Head sizes below 64 take the head-size-64 MFMA kernels on zero-padded q, k, v: the padded
+    columns add nothing to the scores and give zero output columns, and half of the matrix-core
+    work on zeros is still tens of times faster than the one-thread-per-row kernel."""
+    return (
+        bias is None and q.dtype == torch.bfloat16 and q.shape[-1] < 64 and q.shape[-2] % 128 == 0
+        and k.shape[-2] % 128 == 0 and q.shape[-2] > 0 and k.shape[-2] > 0
+    )
+
+
+def _pad64(t: torch.Tensor) -> torch.Tensor:
+    return torch.nn.functional.pad(t, (0, 64 - t.shape[-1]))
+
+
 def core_forward(q, k, v, scale, bias=None, out_acc=None, lse_acc=None, want_out=True):
     """One attention core call; optionally merges into ``(out_acc, lse_acc)`` in place.
 
     Returns ``(out, lse)`` (``None`` each when ``want_out`` is false).
     """
     _check_qkv(q, k, v)
+    if out_acc is None and lse_acc is None and want_out and _pads_to_64(q, k, bias):
+        d = q.shape[-1]
+        out, lse = core_forward(_pad64(q), _pad64(k), _pad64(v), scale)
+        return out[..., :d].contiguous(), lse
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     batch, sq, d = _flat(q)
     sk = int(k.shape[-2])
@@ -134,6 +152,11 @@ def core_backward(grad_out, q, k, v, out, logsumexp, scale, bias=None, want_dbia
     """``(dq, dk, dv[, dbias])`` of one chunk from the global ``out`` / ``logsumexp``."""
     _check_qkv(q, k, v)
     _lib.require_gpu(grad_out, out, logsumexp)
+    if not want_dbias and _pads_to_64(q, k, bias):
+        d = q.shape[-1]
+        grads = core_backward(_pad64(grad_out.to(q.dtype)), _pad64(q), _pad64(k), _pad64(v), _pad64(out.to(q.dtype)),
+                              logsumexp, scale)
+        return tuple(g[..., :d].contiguous() for g in grads)
     dt = q.dtype
     grad_out, out = grad_out.to(dt).contiguous(), out.to(dt).contiguous()
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()

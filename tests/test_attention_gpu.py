@@ -33,6 +33,8 @@ CORE_SHAPES = [
     (2, 2, 256, 384, 64),  # MFMA path for bf16
     (1, 1, 40, 40, 128),
     (1, 2, 17, 9, 8),
+    (1, 3, 256, 128, 32),  # head size below 64: bf16 runs the head-size-64 MFMA kernels on zero-padded q, k, v
+    (2, 2, 128, 256, 16),
 ]
 
 
