@@ -97,18 +97,91 @@ def _bias_args(bias, batch, sq, sk):
     return bias, period
 
 
-def _pads_to_64(q, k, bias) -> bool:
-    """Head sizes below 64 take the head-size-64 MFMA kernels on zero-padded q, k, v: the padded
-    columns add nothing to the scores and give zero output columns, and half of the matrix-core
-    work on zeros is still tens of times faster than the one-thread-per-row kernel."""
-    return (
-        bias is None and q.dtype == torch.bfloat16 and q.shape[-1] < 64 and q.shape[-2] % 128 == 0
-        and k.shape[-2] % 128 == 0 and q.shape[-2] > 0 and k.shape[-2] > 0
-    )
+# --------------------------------------------------------------------------- #
+# Shapes the MFMA kernels do not take as they are (head size below 64, sequence lengths that are
+# not multiples of 128) are brought to them on the host, in bf16 and without a bias:
+#   * head size: zero columns are appended to q, k, v (they add nothing to the scores and give
+#     zero output columns);
+#   * queries: zero rows are appended and their results dropped;
+#   * keys, head size below 64: rows are appended whose first spare column holds a large negative
+#     number, against a column of ones in q: their scores are about -30000, their probabilities 0;
+#   * keys, head size 64 (no spare column): the multiple of 128 goes through the MFMA kernels, the
+#     remaining keys through the one-thread-per-row kernel, and the two (out, lse) pairs are merged
+#     like two ring steps; the backward treats the two key ranges like two ring chunks, the short
+#     one filled up with zero keys (which the backward's arithmetic ignores by itself).
+# Half of the matrix-core work on zeros is still tens of times faster than the FMA kernel.
+# --------------------------------------------------------------------------- #
+_MASKED_SCORE = -30000.0
 
 
-def _pad64(t: torch.Tensor) -> torch.Tensor:
-    return torch.nn.functional.pad(t, (0, 64 - t.shape[-1]))
+def _shapeable(q, k, bias) -> bool:
+    d, sq, sk = q.shape[-1], q.shape[-2], k.shape[-2]
+    if bias is not None or q.dtype != torch.bfloat16 or d > 64 or sq == 0 or sk < 128:
+        return False
+    return d < 64 or sq % 128 != 0 or sk % 128 != 0
+
+
+def _pad_last(t: torch.Tensor, to: int) -> torch.Tensor:
+    return t if t.shape[-1] == to else torch.nn.functional.pad(t, (0, to - t.shape[-1]))
+
+
+def _pad_rows(t: torch.Tensor, to: int) -> torch.Tensor:
+    return t if t.shape[-2] == to else torch.nn.functional.pad(t, (0, 0, 0, to - t.shape[-2]))
+
+
+def _up128(n: int) -> int:
+    return (n + 127) // 128 * 128
+
+
+def _shape_qkv(q, k, v, scale):
+    """q, k, v as the MFMA kernels take them: ``(q, k, v, key ranges)``; a key range is
+    ``(start, stop)`` in the (possibly padded) k / v, the first one a multiple of 128 long."""
+    d, sq, sk = q.shape[-1], q.shape[-2], k.shape[-2]
+    qp = _pad_rows(_pad_last(q, 64), _up128(sq))
+    kp, vp = _pad_last(k, 64), _pad_last(v, 64)
+    if sk % 128 == 0:
+        return qp, kp, vp, [(0, sk)]
+    if d < 64:
+        qp[..., d] = 1.0
+        kp, vp = _pad_rows(kp, _up128(sk)), _pad_rows(vp, _up128(sk))
+        kp[..., sk:, d] = _MASKED_SCORE / float(scale)
+        return qp, kp, vp, [(0, _up128(sk))]
+    main = sk // 128 * 128
+    return qp, kp, vp, [(0, main), (main, sk)]
+
+
+def _shaped_forward(q, k, v, scale):
+    d, sq = q.shape[-1], q.shape[-2]
+    qp, kp, vp, ranges = _shape_qkv(q, k, v, scale)
+    out, lse = _core_forward(qp, kp[..., ranges[0][0]:ranges[0][1], :], vp[..., ranges[0][0]:ranges[0][1], :], scale)
+    if len(ranges) == 2:
+        o2, l2 = _core_forward(qp, kp[..., ranges[1][0]:ranges[1][1], :], vp[..., ranges[1][0]:ranges[1][1], :], scale)
+        rows = qp.shape[-2]
+        merged = fused_online_softmax_merge_(out.float().reshape(1, -1, rows, 64), lse.reshape(1, -1, rows),
+                                             o2.reshape(1, -1, rows, 64), l2.reshape(1, -1, rows), "bhsd")
+        out, lse = merged[0].to(q.dtype).reshape(out.shape), merged[1].reshape(lse.shape)
+    return out[..., :sq, :d].contiguous(), lse[..., :sq].contiguous()
+
+
+def _shaped_backward(grad_out, q, k, v, out, lse, scale):
+    d, sq, sk = q.shape[-1], q.shape[-2], k.shape[-2]
+    qp, kp, vp, ranges = _shape_qkv(q, k, v, scale)
+    rows = qp.shape[-2]
+    gp, op = _pad_rows(_pad_last(grad_out, 64), rows), _pad_rows(_pad_last(out, 64), rows)
+    lp = lse if lse.shape[-1] == rows else torch.nn.functional.pad(lse, (0, rows - lse.shape[-1]))
+    dq, dks, dvs = None, [], []
+    for lo, hi in ranges:
+        # A key range shorter than a tile is filled up with zero keys: with the global out / lse a
+        # zero key adds nothing to dq (its k is zero) and its own dk / dv rows are dropped, so the
+        # backward needs no mask.
+        kj, vj = _pad_rows(kp[..., lo:hi, :], _up128(hi - lo)), _pad_rows(vp[..., lo:hi, :], _up128(hi - lo))
+        dq_j, dk_j, dv_j = _core_backward(gp, qp, kj, vj, op, lp, scale)
+        dq = dq_j.float() if dq is None else dq + dq_j.float()
+        dks.append(dk_j[..., : hi - lo, :])
+        dvs.append(dv_j[..., : hi - lo, :])
+    dk = dks[0] if len(dks) == 1 else torch.cat(dks, dim=-2)
+    dv = dvs[0] if len(dvs) == 1 else torch.cat(dvs, dim=-2)
+    return (dq[..., :sq, :d].to(q.dtype).contiguous(), dk[..., :sk, :d].contiguous(), dv[..., :sk, :d].contiguous())
 
 
 def core_forward(q, k, v, scale, bias=None, out_acc=None, lse_acc=None, want_out=True):
@@ -117,10 +190,12 @@ def core_forward(q, k, v, scale, bias=None, out_acc=None, lse_acc=None, want_out
     Returns ``(out, lse)`` (``None`` each when ``want_out`` is false).
     """
     _check_qkv(q, k, v)
-    if out_acc is None and lse_acc is None and want_out and _pads_to_64(q, k, bias):
-        d = q.shape[-1]
-        out, lse = core_forward(_pad64(q), _pad64(k), _pad64(v), scale)
-        return out[..., :d].contiguous(), lse
+    if out_acc is None and lse_acc is None and want_out and _shapeable(q, k, bias):
+        return _shaped_forward(q, k, v, scale)
+    return _core_forward(q, k, v, scale, bias, out_acc, lse_acc, want_out)
+
+
+def _core_forward(q, k, v, scale, bias=None, out_acc=None, lse_acc=None, want_out=True):
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     batch, sq, d = _flat(q)
     sk = int(k.shape[-2])
@@ -152,11 +227,12 @@ def core_backward(grad_out, q, k, v, out, logsumexp, scale, bias=None, want_dbia
     """``(dq, dk, dv[, dbias])`` of one chunk from the global ``out`` / ``logsumexp``."""
     _check_qkv(q, k, v)
     _lib.require_gpu(grad_out, out, logsumexp)
-    if not want_dbias and _pads_to_64(q, k, bias):
-        d = q.shape[-1]
-        grads = core_backward(_pad64(grad_out.to(q.dtype)), _pad64(q), _pad64(k), _pad64(v), _pad64(out.to(q.dtype)),
-                              logsumexp, scale)
-        return tuple(g[..., :d].contiguous() for g in grads)
+    if not want_dbias and _shapeable(q, k, bias):
+        return _shaped_backward(grad_out.to(q.dtype), q, k, v, out.to(q.dtype), logsumexp.to(torch.float32), scale)
+    return _core_backward(grad_out, q, k, v, out, logsumexp, scale, bias, want_dbias)
+
+
+def _core_backward(grad_out, q, k, v, out, logsumexp, scale, bias=None, want_dbias=False):
     dt = q.dtype
     grad_out, out = grad_out.to(dt).contiguous(), out.to(dt).contiguous()
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()

@@ -35,6 +35,10 @@ CORE_SHAPES = [
     (1, 2, 17, 9, 8),
     (1, 3, 256, 128, 32),  # head size below 64: bf16 runs the head-size-64 MFMA kernels on zero-padded q, k, v
     (2, 2, 128, 256, 16),
+    (1, 2, 200, 300, 32),  # ragged queries and keys below head size 64: padded, spare-column key mask
+    (1, 2, 130, 260, 64),  # ragged at head size 64: MFMA on 256 keys + FMA kernel on 4, merged
+    (2, 1, 128, 130, 16),
+    (1, 1, 70, 1000, 64),
 ]
 
 
