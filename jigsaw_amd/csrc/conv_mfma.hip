@@ -27,6 +27,14 @@
 //               barrier per stage).
 //   dgrad       the same kernel on the output gradient with virtual zero padding
 //               k-1-p and the weights flipped and transposed by the preparation.
+//   Channels    any counts: the contraction is padded to 16-channel steps per depth tap
+//               (zero weights; the registers of channels that do not exist are zeroed on
+//               their way to LDS), the weights stay in LDS in groups of steps when they
+//               do not fit at once, produced channels are padded to 32 and a ragged last
+//               tile predicates its stores.
+//   fp32, fp16  "split mode": an operand is the exact sum of three (two) bf16 parts, kept
+//               as extra channel groups; the contraction runs over the six (three) part
+//               products that matter and the result is stored as fp32 (fp16).
 #include <type_traits>
 
 #include "conv_common.h"

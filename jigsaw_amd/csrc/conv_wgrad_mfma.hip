@@ -1,6 +1,9 @@
 // Weight gradient of the 3x3 (2-D) and 3x3x3 (3-D) convolution on the bf16 matrix
-// cores, stride 1, dilation 1, channels-first tensors, 32 or 64 channels a side;
-// optionally the bias gradient from the same pass over g.
+// cores, stride 1, dilation 1, channels-first tensors; a launch covers a block of 32 or
+// 64 channels a side, any other channel counts are walked block by block. Optionally the
+// bias gradient from the same pass over g. fp32 / fp16 tensors run as sums of three / two
+// bf16 parts per operand ("split mode": the parts are extra channels, their products are
+// added up in fp32).
 //
 //   gw[co][ci][kd][kh][kw] = sum_{n,d,h,w} g[n][co][d][h][w] * x[n][ci][d+kd-pd][h+kh-ph][w+kw-pw]
 //   gb[co]                 = sum_{n,d,h,w} g[n][co][d][h][w]
