@@ -1,5 +1,6 @@
 // C entry points of the attention core: validate and route to the MFMA flash
-// kernels when they cover the problem, to the generic kernels otherwise.
+// kernels (head size 64; head sizes 96 and 128) when they cover the problem, to the
+// window or generic kernels otherwise.
 #include <initializer_list>
 
 #include "jg_common.h"
@@ -22,6 +23,12 @@ size_t attn_mfma_bwd_workspace(long long batch, int sq, int sk);
 int attn_mfma_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q, const void* k,
                   const void* v, const void* out, const float* lse, long long batch, int sq,
                   int sk, float scale, void* ws, hipStream_t s);
+bool attn_wide_supported(long long batch, int sq, int sk, int d, int dtype, bool has_bias);
+int attn_wide_fwd(void* out, float* lse, const void* q, const void* k, const void* v, long long batch,
+                  int sq, int sk, int d, float scale, hipStream_t s);
+int attn_wide_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q, const void* k,
+                  const void* v, const void* out, const float* lse, long long batch, int sq, int sk,
+                  int d, float scale, void* ws, hipStream_t s);
 bool attn_window_supported(long long batch, int sq, int sk, int d, int dtype);
 int attn_window_fwd(void* out, float* lse, const void* q, const void* k, const void* v,
                     long long batch, float scale, const float* bias, long long bias_period,
@@ -69,11 +76,15 @@ extern "C" int jg_attn_fwd(void* out, float* lse, const void* q, const void* k, 
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (jg::attn_mfma_fwd_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr))
     return jg::attn_mfma_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, scale, out_acc, lse_acc, s);
+  if (out_acc == nullptr &&
+      jg::attn_wide_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr) &&
+      aligned16({out, q, k, v}))
+    return jg::attn_wide_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, (int)d, scale, s);
   if (out_acc == nullptr && jg::attn_window_supported(batch, (int)sq, (int)sk, (int)d, dtype) &&
       aligned16({out, q, k, v, bias}))
     return jg::attn_window_fwd(out, lse, q, k, v, batch, scale, bias, bias_period, s);
   if (!jg::attn_generic_supported((int)d))
-    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: head size %lld not in {8, 16, 32, 64, 128}", who, (long long)d);
+    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: head size %lld not in {8, 16, 32, 64, 96, 128}", who, (long long)d);
   if (out_acc != nullptr)
     JG_FAIL(JG_ERR_UNSUPPORTED,
             "%s: the fused merge needs the MFMA path (bf16, d = 64, sq %% 128 == 0, sk %% 128 == 0);"
@@ -111,12 +122,17 @@ extern "C" int jg_attn_bwd(void* dq, void* dk, void* dv, const void* dout, const
       jg::attn_mfma_bwd_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr))
     return jg::attn_mfma_bwd(dq, dk, dv, dout, q, k, v, out, lse, batch, (int)sq, (int)sk, scale,
                              workspace, s);
+  if (dbias == nullptr &&
+      jg::attn_wide_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr) &&
+      aligned16({dq, dk, dv, dout, q, k, v, out}))
+    return jg::attn_wide_bwd(dq, dk, dv, dout, q, k, v, out, lse, batch, (int)sq, (int)sk, (int)d,
+                             scale, workspace, s);
   if (jg::attn_window_supported(batch, (int)sq, (int)sk, (int)d, dtype) &&
       aligned16({dq, dk, dv, dout, q, k, v, out, bias, dbias}))
     return jg::attn_window_bwd(dq, dk, dv, dbias, dout, q, k, v, out, lse, batch, scale, bias,
                                bias_period, s);
   if (!jg::attn_generic_supported((int)d))
-    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: head size %lld not in {8, 16, 32, 64, 128}", who, (long long)d);
+    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: head size %lld not in {8, 16, 32, 64, 96, 128}", who, (long long)d);
   return jg::attn_generic_bwd(dq, dk, dv, static_cast<float*>(workspace), dbias, dout, q, k, v, out,
                               lse, batch, (int)sq, (int)sk, (int)d, scale, bias, bias_period, dtype,
                               s);

@@ -230,7 +230,7 @@ __global__ __launch_bounds__(kRows) void attn_bwd_dkv_generic(
 
 namespace jg {
 
-bool attn_generic_supported(int d) { return d == 8 || d == 16 || d == 32 || d == 64 || d == 128; }
+bool attn_generic_supported(int d) { return d == 8 || d == 16 || d == 32 || d == 64 || d == 96 || d == 128; }
 
 #define JG_ATTN_DISPATCH(CALL)                                   \
   do {                                                           \
@@ -239,6 +239,7 @@ bool attn_generic_supported(int d) { return d == 8 || d == 16 || d == 32 || d ==
       case 16: CALL(16); break;                                  \
       case 32: CALL(32); break;                                  \
       case 64: CALL(64); break;                                  \
+      case 96: CALL(96); break;                                  \
       default: CALL(128); break;                                 \
     }                                                            \
   } while (0)

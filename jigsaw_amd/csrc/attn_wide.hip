@@ -1,0 +1,493 @@
+// Blockwise (flash-style) attention of one K/V chunk on the bf16 matrix cores for head
+// sizes 96 and 128, non-causal, no bias: forward (output + natural-log LSE) and backward
+// from a given (global) output and LSE. Same arithmetic as the head-size-64 kernels,
+// written for clarity rather than hand-scheduled: tiles of 32 keys (forward, dQ) or 32
+// queries (dK/dV) pass through a double-buffered LDS stage, fetched to registers one tile
+// ahead.
+//
+//   forward / dQ   lane = query. S^T = K Q^T (A = K rows from LDS, B = Q rows kept in
+//                  registers), so the running max / sum, lse and delta of a query are
+//                  scalars of the two lanes that share it. P^T (or dS^T) leaves the
+//                  accumulator already in B-fragment position for O^T += V^T P^T
+//                  (dQ^T += K^T dS^T): the A operand is a transposed copy of the tile in
+//                  LDS whose 32 columns are stored in the order the accumulator holds its
+//                  rows (key_pos).
+//   dK / dV        lane = key. S = Q K^T and dP = dO V^T with K, V rows in registers;
+//                  lse and delta of the tile's queries are read from LDS per accumulator
+//                  row; dV^T += dO^T P and dK^T += Q^T dS use transposed copies of the dO
+//                  and Q tiles.
+//
+// Reference behaviour restated here:
+//   jigsaw/modules/attention/_functional/cores/math.py:69-78   (forward)
+//   jigsaw/modules/attention/_functional/cores/math.py:125-149 (backward)
+#include "jg_common.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int WAVES = 4, THREADS = WAVES * 64;
+constexpr int BQ = 32 * WAVES;  // rows (queries or keys) of a workgroup, 32 per wavefront
+constexpr int BT = 32;          // rows of a streamed tile
+constexpr float LOG2E = 1.4426950408889634f;
+
+template <int D>
+struct Geo {
+  static constexpr int C16 = D / 16, NB = D / 32;
+  static constexpr int RP = D * 2 + 16;   // bytes per row of a row-major tile (32 rows of D): an odd number of 16-byte units
+  static constexpr int TP = BT * 2 + 16;  // bytes per row of a transposed tile (D rows of 32)
+  static constexpr int ROWMAJ = BT * RP, TRANS = D * TP;
+  static constexpr int CHUNKS = BT * D / 8;  // 16-byte pieces of a tile
+  static constexpr int PER = (CHUNKS + THREADS - 1) / THREADS;
+};
+
+// Column of a transposed tile that holds tile row x: inside a group of 16 rows the order is the
+// one in which an MFMA accumulator lane holds its rows, so that probabilities need no shuffle
+// on their way from accumulator to B operand.
+__device__ __forceinline__ int key_pos(int x) {
+  const int y = x & 15;
+  return (x & 16) + ((y & 7) >> 2) * 8 + (y >> 3) * 4 + (y & 3);
+}
+
+template <int D>
+struct TileRegs {
+  u32x4 v[Geo<D>::PER];
+};
+
+// 32 rows x D of a row-major (row stride D) bf16 matrix to registers
+template <int D>
+__device__ __forceinline__ void tile_fetch(TileRegs<D>& r, const uint16_t* src) {
+#pragma unroll
+  for (int i = 0; i < Geo<D>::PER; ++i) {
+    const int c = threadIdx.x + i * THREADS;
+    if (c < Geo<D>::CHUNKS) r.v[i] = *reinterpret_cast<const u32x4*>(src + c * 8);  // rows are contiguous: chunk c = 8 elements at c*8
+  }
+}
+template <int D>
+__device__ __forceinline__ void tile_store_rows(const TileRegs<D>& r, unsigned char* dst) {
+#pragma unroll
+  for (int i = 0; i < Geo<D>::PER; ++i) {
+    const int c = threadIdx.x + i * THREADS;
+    if (c < Geo<D>::CHUNKS) {
+      const int row = c / (D / 8), col8 = c % (D / 8);
+      *reinterpret_cast<u32x4*>(dst + row * Geo<D>::RP + col8 * 16) = r.v[i];
+    }
+  }
+}
+template <int D>
+__device__ __forceinline__ void tile_store_transposed(const TileRegs<D>& r, unsigned char* dst) {
+#pragma unroll
+  for (int i = 0; i < Geo<D>::PER; ++i) {
+    const int c = threadIdx.x + i * THREADS;
+    if (c < Geo<D>::CHUNKS) {
+      const int row = c / (D / 8), col8 = c % (D / 8);
+      unsigned char* at = dst + (col8 * 8) * Geo<D>::TP + key_pos(row) * 2;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t w = r.v[i][e >> 1];
+        *reinterpret_cast<uint16_t*>(at + e * Geo<D>::TP) = (uint16_t)((e & 1) ? (w >> 16) : (w & 0xffffu));
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ bf16x8 pack8(const float* v) {
+  bf16x8 r;
+#pragma unroll
+  for (int j = 0; j < 8; j += 2) {
+    const f32x2 v2 = {v[j], v[j + 1]};
+    const bf16x2 h2 = __builtin_convertvector(v2, bf16x2);
+    r[j] = h2.x;
+    r[j + 1] = h2.y;
+  }
+  return r;
+}
+__device__ __forceinline__ u32x2 pack4(float a, float b, float c, float d) {
+  const f32x2 lo = {a, b}, hi = {c, d};
+  u32x2 r;
+  r.x = __builtin_bit_cast(uint32_t, __builtin_convertvector(lo, bf16x2));
+  r.y = __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, bf16x2));
+  return r;
+}
+__device__ __forceinline__ f32x16 zero16() {
+  f32x16 z;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) z[i] = 0.0f;
+  return z;
+}
+__device__ __forceinline__ bf16x8 frag(const unsigned char* at) {
+  return __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(at));
+}
+
+struct Args {
+  const uint16_t* q;
+  const uint16_t* k;
+  const uint16_t* v;
+  const uint16_t* out;   // backward: the global output
+  const uint16_t* dout;  // backward
+  const float* lse_in;   // backward: the global lse
+  float* delta;          // backward workspace (batch, sq): written by the dQ kernel, read by the dK/dV kernel
+  uint16_t* o;           // forward output
+  float* lse;            // forward output
+  uint16_t* dq;
+  uint16_t* dk;
+  uint16_t* dv;
+  int sq, sk;
+  float scale;
+};
+
+// ------------------------------------------------------------------- forward
+template <int D>
+__global__ __launch_bounds__(THREADS) void attn_wide_fwd_kernel(Args p) {
+  typedef Geo<D> G;
+  constexpr int BUF = G::ROWMAJ + G::TRANS;  // K rows, then V^T
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ln = lane & 31, kg = lane >> 5;
+  const long long bh = blockIdx.y;
+  const int qi = blockIdx.x * BQ + wave * 32 + ln;
+  const uint16_t* qrow = p.q + (bh * p.sq + qi) * D;
+  const uint16_t* kb = p.k + bh * p.sk * D;
+  const uint16_t* vb = p.v + bh * p.sk * D;
+  const float c2 = p.scale * LOG2E;
+
+  bf16x8 qf[G::C16];
+#pragma unroll
+  for (int c = 0; c < G::C16; ++c) qf[c] = frag(reinterpret_cast<const unsigned char*>(qrow + 16 * c + 8 * kg));
+
+  f32x16 o[G::NB];
+#pragma unroll
+  for (int nb = 0; nb < G::NB; ++nb) o[nb] = zero16();
+  float m = -INFINITY, l = 0.0f;
+
+  TileRegs<D> rk, rv;
+  const int ntiles = p.sk / BT;
+  tile_fetch<D>(rk, kb);
+  tile_fetch<D>(rv, vb);
+  tile_store_rows<D>(rk, smem);
+  tile_store_transposed<D>(rv, smem + G::ROWMAJ);
+  __syncthreads();
+  for (int t = 0; t < ntiles; ++t) {
+    const unsigned char* kt = smem + (t & 1) * BUF;
+    const unsigned char* vt = kt + G::ROWMAJ;
+    if (t + 1 < ntiles) {
+      tile_fetch<D>(rk, kb + (long long)(t + 1) * BT * D);
+      tile_fetch<D>(rv, vb + (long long)(t + 1) * BT * D);
+    }
+    // S^T: lane = query ln, register i = key 8*(i/4) + 4*kg + i%4 of the tile
+    f32x16 s = zero16();
+#pragma unroll
+    for (int c = 0; c < G::C16; ++c)
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(kt + ln * G::RP + (16 * c + 8 * kg) * 2), qf[c], s, 0, 0, 0);
+    float mx = s[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mn = fmaxf(m, mx);
+    const float alpha = __builtin_amdgcn_exp2f((m - mn) * c2);  // first tile: exp2(-inf) = 0
+    m = mn;
+    float pr[16], sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      pr[i] = __builtin_amdgcn_exp2f((s[i] - mn) * c2);
+      sum += pr[i];
+    }
+    l = l * alpha + sum;
+#pragma unroll
+    for (int nb = 0; nb < G::NB; ++nb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[nb][i] *= alpha;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const bf16x8 pf = pack8(pr + 8 * ks);
+#pragma unroll
+      for (int nb = 0; nb < G::NB; ++nb)
+        o[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(vt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2), pf,
+                                                        o[nb], 0, 0, 0);
+    }
+    if (t + 1 < ntiles) {
+      unsigned char* nk = smem + ((t + 1) & 1) * BUF;
+      tile_store_rows<D>(rk, nk);
+      tile_store_transposed<D>(rv, nk + G::ROWMAJ);
+    }
+    __syncthreads();
+  }
+  // the two lanes of a query saw the same maxima; their sums cover disjoint keys
+  l += __shfl_xor(l, 32, 64);
+  const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+  uint16_t* orow = p.o + (bh * p.sq + qi) * D;
+  // register i of block nb: output column nb*32 + 8*(i/4) + 4*kg + i%4
+#pragma unroll
+  for (int nb = 0; nb < G::NB; ++nb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      *reinterpret_cast<u32x2*>(orow + nb * 32 + 8 * j + 4 * kg) =
+          pack4(o[nb][4 * j] * inv, o[nb][4 * j + 1] * inv, o[nb][4 * j + 2] * inv, o[nb][4 * j + 3] * inv);
+  if (kg == 0) p.lse[bh * p.sq + qi] = l > 0.0f ? m * p.scale + __logf(l) : -INFINITY;
+}
+
+// ------------------------------------------------------------------- dQ (and delta)
+template <int D>
+__global__ __launch_bounds__(THREADS) void attn_wide_dq_kernel(Args p) {
+  typedef Geo<D> G;
+  constexpr int BUF = 2 * G::ROWMAJ + G::TRANS;  // K rows, V rows, K^T
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ln = lane & 31, kg = lane >> 5;
+  const long long bh = blockIdx.y;
+  const int qi = blockIdx.x * BQ + wave * 32 + ln;
+  const long long qoff = (bh * p.sq + qi) * D;
+  const uint16_t* kb = p.k + bh * p.sk * D;
+  const uint16_t* vb = p.v + bh * p.sk * D;
+  const float c2 = p.scale * LOG2E;
+
+  bf16x8 qf[G::C16], dof[G::C16];
+  float dl = 0.0f;
+#pragma unroll
+  for (int c = 0; c < G::C16; ++c) {
+    qf[c] = frag(reinterpret_cast<const unsigned char*>(p.q + qoff + 16 * c + 8 * kg));
+    dof[c] = frag(reinterpret_cast<const unsigned char*>(p.dout + qoff + 16 * c + 8 * kg));
+    const bf16x8 of = frag(reinterpret_cast<const unsigned char*>(p.out + qoff + 16 * c + 8 * kg));
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dl += (float)dof[c][j] * (float)of[j];
+  }
+  // delta = rowsum(dO o O): the two lanes of a query hold disjoint halves of the row
+  const float delta = dl + __shfl_xor(dl, 32, 64);
+  if (kg == 0) p.delta[bh * p.sq + qi] = delta;
+  const float lse2 = p.lse_in[bh * p.sq + qi] * LOG2E;
+
+  f32x16 dq[G::NB];
+#pragma unroll
+  for (int nb = 0; nb < G::NB; ++nb) dq[nb] = zero16();
+
+  TileRegs<D> rk, rv;
+  const int ntiles = p.sk / BT;
+  tile_fetch<D>(rk, kb);
+  tile_fetch<D>(rv, vb);
+  tile_store_rows<D>(rk, smem);
+  tile_store_rows<D>(rv, smem + G::ROWMAJ);
+  tile_store_transposed<D>(rk, smem + 2 * G::ROWMAJ);
+  __syncthreads();
+  for (int t = 0; t < ntiles; ++t) {
+    const unsigned char* kt = smem + (t & 1) * BUF;
+    const unsigned char* vt = kt + G::ROWMAJ;
+    const unsigned char* ktt = kt + 2 * G::ROWMAJ;
+    if (t + 1 < ntiles) {
+      tile_fetch<D>(rk, kb + (long long)(t + 1) * BT * D);
+      tile_fetch<D>(rv, vb + (long long)(t + 1) * BT * D);
+    }
+    f32x16 s = zero16(), dp = zero16();
+#pragma unroll
+    for (int c = 0; c < G::C16; ++c) {
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(kt + ln * G::RP + (16 * c + 8 * kg) * 2), qf[c], s, 0, 0, 0);
+      dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(vt + ln * G::RP + (16 * c + 8 * kg) * 2), dof[c], dp, 0, 0, 0);
+    }
+    float ds[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) ds[i] = __builtin_amdgcn_exp2f(s[i] * c2 - lse2) * (dp[i] - delta);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const bf16x8 dsf = pack8(ds + 8 * ks);
+#pragma unroll
+      for (int nb = 0; nb < G::NB; ++nb)
+        dq[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(ktt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2),
+                                                         dsf, dq[nb], 0, 0, 0);
+    }
+    if (t + 1 < ntiles) {
+      unsigned char* nk = smem + ((t + 1) & 1) * BUF;
+      tile_store_rows<D>(rk, nk);
+      tile_store_rows<D>(rv, nk + G::ROWMAJ);
+      tile_store_transposed<D>(rk, nk + 2 * G::ROWMAJ);
+    }
+    __syncthreads();
+  }
+  uint16_t* row = p.dq + qoff;
+#pragma unroll
+  for (int nb = 0; nb < G::NB; ++nb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      *reinterpret_cast<u32x2*>(row + nb * 32 + 8 * j + 4 * kg) =
+          pack4(dq[nb][4 * j] * p.scale, dq[nb][4 * j + 1] * p.scale, dq[nb][4 * j + 2] * p.scale,
+                dq[nb][4 * j + 3] * p.scale);
+}
+
+// ------------------------------------------------------------------- dK, dV
+template <int D>
+__global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
+  typedef Geo<D> G;
+  constexpr int STATS = 2 * BT * 4;                           // lse * log2(e) and delta of the tile's queries
+  constexpr int BUF = 2 * G::ROWMAJ + 2 * G::TRANS + STATS;   // Q rows, dO rows, Q^T, dO^T, stats
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ln = lane & 31, kg = lane >> 5;
+  const long long bh = blockIdx.y;
+  const int ki = blockIdx.x * BQ + wave * 32 + ln;
+  const long long koff = (bh * p.sk + ki) * D;
+  const uint16_t* qb = p.q + bh * p.sq * D;
+  const uint16_t* gb = p.dout + bh * p.sq * D;
+  const float* lb = p.lse_in + bh * p.sq;
+  const float* db = p.delta + bh * p.sq;
+  const float c2 = p.scale * LOG2E;
+
+  bf16x8 kf[G::C16], vf[G::C16];
+#pragma unroll
+  for (int c = 0; c < G::C16; ++c) {
+    kf[c] = frag(reinterpret_cast<const unsigned char*>(p.k + koff + 16 * c + 8 * kg));
+    vf[c] = frag(reinterpret_cast<const unsigned char*>(p.v + koff + 16 * c + 8 * kg));
+  }
+  f32x16 dk[G::NB], dv[G::NB];
+#pragma unroll
+  for (int nb = 0; nb < G::NB; ++nb) {
+    dk[nb] = zero16();
+    dv[nb] = zero16();
+  }
+
+  TileRegs<D> rq, rg;
+  float st = 0.0f;  // one statistic per thread of the first wavefront: lse2 (lanes 0-31) or delta (32-63)
+  const int ntiles = p.sq / BT;
+  auto fetch = [&](int t) {
+    tile_fetch<D>(rq, qb + (long long)t * BT * D);
+    tile_fetch<D>(rg, gb + (long long)t * BT * D);
+    if (threadIdx.x < 2 * BT) {
+      const float* src = threadIdx.x < BT ? lb : db;  // every lane loads; the factor is applied when stored
+      st = src[t * BT + (threadIdx.x & (BT - 1))];
+    }
+  };
+  auto store = [&](int buf) {
+    unsigned char* base = smem + buf * BUF;
+    tile_store_rows<D>(rq, base);
+    tile_store_rows<D>(rg, base + G::ROWMAJ);
+    tile_store_transposed<D>(rq, base + 2 * G::ROWMAJ);
+    tile_store_transposed<D>(rg, base + 2 * G::ROWMAJ + G::TRANS);
+    if (threadIdx.x < 2 * BT)
+      reinterpret_cast<float*>(base + 2 * G::ROWMAJ + 2 * G::TRANS)[threadIdx.x] = threadIdx.x < BT ? st * LOG2E : st;
+  };
+  fetch(0);
+  store(0);
+  __syncthreads();
+  for (int t = 0; t < ntiles; ++t) {
+    const unsigned char* qt = smem + (t & 1) * BUF;
+    const unsigned char* gt = qt + G::ROWMAJ;
+    const unsigned char* qtt = qt + 2 * G::ROWMAJ;
+    const unsigned char* gtt = qtt + G::TRANS;
+    const float* stats = reinterpret_cast<const float*>(gtt + G::TRANS);
+    if (t + 1 < ntiles) fetch(t + 1);
+    // S and dP: lane = key ln, register i = query 8*(i/4) + 4*kg + i%4 of the tile
+    f32x16 s = zero16(), dp = zero16();
+#pragma unroll
+    for (int c = 0; c < G::C16; ++c) {
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(qt + ln * G::RP + (16 * c + 8 * kg) * 2), kf[c], s, 0, 0, 0);
+      dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(gt + ln * G::RP + (16 * c + 8 * kg) * 2), vf[c], dp, 0, 0, 0);
+    }
+    float pr[16], ds[16];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const f32x4 l4 = *reinterpret_cast<const f32x4*>(stats + 8 * j + 4 * kg);
+      const f32x4 d4 = *reinterpret_cast<const f32x4*>(stats + BT + 8 * j + 4 * kg);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int i = 4 * j + e;
+        pr[i] = __builtin_amdgcn_exp2f(s[i] * c2 - l4[e]);
+        ds[i] = pr[i] * (dp[i] - d4[e]);
+      }
+    }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const bf16x8 pf = pack8(pr + 8 * ks), dsf = pack8(ds + 8 * ks);
+#pragma unroll
+      for (int nb = 0; nb < G::NB; ++nb) {
+        dv[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(gtt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2), pf,
+                                                         dv[nb], 0, 0, 0);
+        dk[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(qtt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2), dsf,
+                                                         dk[nb], 0, 0, 0);
+      }
+    }
+    if (t + 1 < ntiles) store((t + 1) & 1);
+    __syncthreads();
+  }
+  uint16_t* krow = p.dk + koff;
+  uint16_t* vrow = p.dv + koff;
+#pragma unroll
+  for (int nb = 0; nb < G::NB; ++nb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      *reinterpret_cast<u32x2*>(krow + nb * 32 + 8 * j + 4 * kg) =
+          pack4(dk[nb][4 * j] * p.scale, dk[nb][4 * j + 1] * p.scale, dk[nb][4 * j + 2] * p.scale,
+                dk[nb][4 * j + 3] * p.scale);
+      *reinterpret_cast<u32x2*>(vrow + nb * 32 + 8 * j + 4 * kg) =
+          pack4(dv[nb][4 * j], dv[nb][4 * j + 1], dv[nb][4 * j + 2], dv[nb][4 * j + 3]);
+    }
+}
+
+template <int D>
+int launch_fwd(const Args& a, long long batch, hipStream_t s) {
+  attn_wide_fwd_kernel<D><<<dim3((unsigned)(a.sq / BQ), (unsigned)batch, 1), THREADS, 0, s>>>(a);
+  JG_CHECK_LAUNCH("jg_attn_fwd(wide)");
+  return JG_OK;
+}
+
+template <int D>
+int launch_bwd(const Args& a, long long batch, hipStream_t s) {
+  typedef Geo<D> G;
+  constexpr int DQ_LDS = 2 * (2 * G::ROWMAJ + G::TRANS);
+  constexpr int DKV_LDS = 2 * (2 * G::ROWMAJ + 2 * G::TRANS + 2 * BT * 4);
+  void (*dqk)(Args) = &attn_wide_dq_kernel<D>;
+  void (*dkvk)(Args) = &attn_wide_dkv_kernel<D>;
+  hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(dqk), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      DQ_LDS);
+  hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(dkvk), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      DKV_LDS);
+  if (e1 != hipSuccess || e2 != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "jg_attn_bwd(wide): cannot reserve LDS");
+  dqk<<<dim3((unsigned)(a.sq / BQ), (unsigned)batch, 1), THREADS, DQ_LDS, s>>>(a);
+  JG_CHECK_LAUNCH("jg_attn_bwd(wide, dq)");
+  dkvk<<<dim3((unsigned)(a.sk / BQ), (unsigned)batch, 1), THREADS, DKV_LDS, s>>>(a);
+  JG_CHECK_LAUNCH("jg_attn_bwd(wide, dkv)");
+  return JG_OK;
+}
+
+}  // namespace
+
+namespace jg {
+
+bool attn_wide_supported(long long batch, int sq, int sk, int d, int dtype, bool has_bias) {
+  return dtype == JG_BF16 && !has_bias && (d == 96 || d == 128) && sq > 0 && sk > 0 && sq % BQ == 0 &&
+         sk % BQ == 0 && batch > 0 && batch <= 65535;
+}
+
+int attn_wide_fwd(void* out, float* lse, const void* q, const void* k, const void* v, long long batch, int sq,
+                  int sk, int d, float scale, hipStream_t s) {
+  Args a{};
+  a.q = static_cast<const uint16_t*>(q);
+  a.k = static_cast<const uint16_t*>(k);
+  a.v = static_cast<const uint16_t*>(v);
+  a.o = static_cast<uint16_t*>(out);
+  a.lse = lse;
+  a.sq = sq; a.sk = sk; a.scale = scale;
+  return d == 128 ? launch_fwd<128>(a, batch, s) : launch_fwd<96>(a, batch, s);
+}
+
+int attn_wide_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q, const void* k, const void* v,
+                  const void* out, const float* lse, long long batch, int sq, int sk, int d, float scale,
+                  void* ws, hipStream_t s) {
+  Args a{};
+  a.q = static_cast<const uint16_t*>(q);
+  a.k = static_cast<const uint16_t*>(k);
+  a.v = static_cast<const uint16_t*>(v);
+  a.out = static_cast<const uint16_t*>(out);
+  a.dout = static_cast<const uint16_t*>(dout);
+  a.lse_in = lse;
+  a.delta = static_cast<float*>(ws);
+  a.dq = static_cast<uint16_t*>(dq);
+  a.dk = static_cast<uint16_t*>(dk);
+  a.dv = static_cast<uint16_t*>(dv);
+  a.sq = sq; a.sk = sk; a.scale = scale;
+  return d == 128 ? launch_bwd<128>(a, batch, s) : launch_bwd<96>(a, batch, s);
+}
+
+}  // namespace jg

@@ -39,6 +39,9 @@ CORE_SHAPES = [
     (1, 2, 130, 260, 64),  # ragged at head size 64: MFMA on 256 keys + FMA kernel on 4, merged
     (2, 1, 128, 130, 16),
     (1, 1, 70, 1000, 64),
+    (1, 2, 128, 256, 128),  # head sizes 96 and 128: their own MFMA kernels for bf16
+    (2, 2, 256, 128, 96),
+    (1, 1, 384, 640, 128),
 ]
 
 
