@@ -11,7 +11,7 @@
 //                  accumulator already in B-fragment position for O^T += V^T P^T
 //                  (dQ^T += K^T dS^T): the A operand is a transposed copy of the tile in
 //                  LDS whose 32 columns are stored in the order the accumulator holds its
-//                  rows (key_pos).
+//                  rows.
 //   dK / dV        lane = key. S = Q K^T and dP = dO V^T with K, V rows in registers;
 //                  lse and delta of the tile's queries are read from LDS per accumulator
 //                  row; dV^T += dO^T P and dK^T += Q^T dS use transposed copies of the dO
@@ -48,12 +48,8 @@ struct Geo {
 };
 
 // Column of a transposed tile that holds tile row x: inside a group of 16 rows the order is the
-// one in which an MFMA accumulator lane holds its rows, so that probabilities need no shuffle
-// on their way from accumulator to B operand.
-__device__ __forceinline__ int key_pos(int x) {
-  const int y = x & 15;
-  return (x & 16) + ((y & 7) >> 2) * 8 + (y >> 3) * 4 + (y & 3);
-}
+// one in which an MFMA accumulator lane holds its rows, so that probabilities need no shuffle on
+// their way from accumulator to B operand: 16*(x/16) + ((x%8)/4)*8 + ((x%16)/8)*4 + x%4.
 
 template <int D>
 struct TileRegs {
@@ -80,19 +76,37 @@ __device__ __forceinline__ void tile_store_rows(const TileRegs<D>& r, unsigned c
     }
   }
 }
+// Transposed staging: a thread takes 8 rows x 2 columns of the tile (8 dwords) and writes, for each
+// of its two columns, the 8 values as two 8-byte pieces of the transposed tile's row.
 template <int D>
-__device__ __forceinline__ void tile_store_transposed(const TileRegs<D>& r, unsigned char* dst) {
+struct TransRegs {
+  uint32_t w[8];
+};
+template <int D>
+__device__ __forceinline__ void trans_fetch(TransRegs<D>& r, const uint16_t* src) {
+  if (threadIdx.x < 4 * (D / 2)) {
+    const int g8 = threadIdx.x / (D / 2), cp = threadIdx.x % (D / 2);
 #pragma unroll
-  for (int i = 0; i < Geo<D>::PER; ++i) {
-    const int c = threadIdx.x + i * THREADS;
-    if (c < Geo<D>::CHUNKS) {
-      const int row = c / (D / 8), col8 = c % (D / 8);
-      unsigned char* at = dst + (col8 * 8) * Geo<D>::TP + key_pos(row) * 2;
+    for (int i = 0; i < 8; ++i) r.w[i] = *reinterpret_cast<const uint32_t*>(src + (g8 * 8 + i) * D + 2 * cp);
+  }
+}
+template <int D>
+__device__ __forceinline__ void trans_store(const TransRegs<D>& r, unsigned char* dst) {
+  if (threadIdx.x < 4 * (D / 2)) {
+    const int g8 = threadIdx.x / (D / 2), cp = threadIdx.x % (D / 2);
+    // rows 8*g8 .. 8*g8+7 of the tile: the first four land at the place of row 8*g8, the last four 8 places on
+    const int pos_lo = (g8 >> 1) * 16 + (g8 & 1) * 4, pos_hi = pos_lo + 8;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const uint32_t w = r.v[i][e >> 1];
-        *reinterpret_cast<uint16_t*>(at + e * Geo<D>::TP) = (uint16_t)((e & 1) ? (w >> 16) : (w & 0xffffu));
-      }
+    for (int e = 0; e < 2; ++e) {
+      const uint32_t sel = e ? 0x07060302u : 0x05040100u;
+      u32x2 lo, hi;
+      lo.x = __builtin_amdgcn_perm(r.w[1], r.w[0], sel);
+      lo.y = __builtin_amdgcn_perm(r.w[3], r.w[2], sel);
+      hi.x = __builtin_amdgcn_perm(r.w[5], r.w[4], sel);
+      hi.y = __builtin_amdgcn_perm(r.w[7], r.w[6], sel);
+      unsigned char* row = dst + (2 * cp + e) * Geo<D>::TP;
+      *reinterpret_cast<u32x2*>(row + pos_lo * 2) = lo;
+      *reinterpret_cast<u32x2*>(row + pos_hi * 2) = hi;
     }
   }
 }
@@ -166,19 +180,20 @@ __global__ __launch_bounds__(THREADS) void attn_wide_fwd_kernel(Args p) {
   for (int nb = 0; nb < G::NB; ++nb) o[nb] = zero16();
   float m = -INFINITY, l = 0.0f;
 
-  TileRegs<D> rk, rv;
+  TileRegs<D> rk;
+  TransRegs<D> rv;
   const int ntiles = p.sk / BT;
   tile_fetch<D>(rk, kb);
-  tile_fetch<D>(rv, vb);
+  trans_fetch<D>(rv, vb);
   tile_store_rows<D>(rk, smem);
-  tile_store_transposed<D>(rv, smem + G::ROWMAJ);
+  trans_store<D>(rv, smem + G::ROWMAJ);
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
     const unsigned char* kt = smem + (t & 1) * BUF;
     const unsigned char* vt = kt + G::ROWMAJ;
     if (t + 1 < ntiles) {
       tile_fetch<D>(rk, kb + (long long)(t + 1) * BT * D);
-      tile_fetch<D>(rv, vb + (long long)(t + 1) * BT * D);
+      trans_fetch<D>(rv, vb + (long long)(t + 1) * BT * D);
     }
     // S^T: lane = query ln, register i = key 8*(i/4) + 4*kg + i%4 of the tile
     f32x16 s = zero16();
@@ -190,19 +205,24 @@ __global__ __launch_bounds__(THREADS) void attn_wide_fwd_kernel(Args p) {
     for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float mn = fmaxf(m, mx);
-    const float alpha = __builtin_amdgcn_exp2f((m - mn) * c2);  // first tile: exp2(-inf) = 0
-    m = mn;
+    // the maximum settles after a few tiles: rescale only when some query of the wavefront saw a larger score
+    if (__builtin_amdgcn_ballot_w64(mn > m) != 0) {
+      const float alpha = __builtin_amdgcn_exp2f((m - mn) * c2);  // first tile: exp2(-inf) = 0
+      l *= alpha;
+#pragma unroll
+      for (int nb = 0; nb < G::NB; ++nb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[nb][i] *= alpha;
+      m = mn;
+    }
+    const float off = m * c2;
     float pr[16], sum = 0.0f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      pr[i] = __builtin_amdgcn_exp2f((s[i] - mn) * c2);
+      pr[i] = __builtin_amdgcn_exp2f(s[i] * c2 - off);
       sum += pr[i];
     }
-    l = l * alpha + sum;
-#pragma unroll
-    for (int nb = 0; nb < G::NB; ++nb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[nb][i] *= alpha;
+    l += sum;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       const bf16x8 pf = pack8(pr + 8 * ks);
@@ -214,7 +234,7 @@ __global__ __launch_bounds__(THREADS) void attn_wide_fwd_kernel(Args p) {
     if (t + 1 < ntiles) {
       unsigned char* nk = smem + ((t + 1) & 1) * BUF;
       tile_store_rows<D>(rk, nk);
-      tile_store_transposed<D>(rv, nk + G::ROWMAJ);
+      trans_store<D>(rv, nk + G::ROWMAJ);
     }
     __syncthreads();
   }
@@ -267,12 +287,14 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dq_kernel(Args p) {
   for (int nb = 0; nb < G::NB; ++nb) dq[nb] = zero16();
 
   TileRegs<D> rk, rv;
+  TransRegs<D> rkt;
   const int ntiles = p.sk / BT;
   tile_fetch<D>(rk, kb);
   tile_fetch<D>(rv, vb);
+  trans_fetch<D>(rkt, kb);
   tile_store_rows<D>(rk, smem);
   tile_store_rows<D>(rv, smem + G::ROWMAJ);
-  tile_store_transposed<D>(rk, smem + 2 * G::ROWMAJ);
+  trans_store<D>(rkt, smem + 2 * G::ROWMAJ);
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
     const unsigned char* kt = smem + (t & 1) * BUF;
@@ -281,6 +303,7 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dq_kernel(Args p) {
     if (t + 1 < ntiles) {
       tile_fetch<D>(rk, kb + (long long)(t + 1) * BT * D);
       tile_fetch<D>(rv, vb + (long long)(t + 1) * BT * D);
+      trans_fetch<D>(rkt, kb + (long long)(t + 1) * BT * D);
     }
     f32x16 s = zero16(), dp = zero16();
 #pragma unroll
@@ -303,7 +326,7 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dq_kernel(Args p) {
       unsigned char* nk = smem + ((t + 1) & 1) * BUF;
       tile_store_rows<D>(rk, nk);
       tile_store_rows<D>(rv, nk + G::ROWMAJ);
-      tile_store_transposed<D>(rk, nk + 2 * G::ROWMAJ);
+      trans_store<D>(rkt, nk + 2 * G::ROWMAJ);
     }
     __syncthreads();
   }
@@ -349,11 +372,14 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
   }
 
   TileRegs<D> rq, rg;
+  TransRegs<D> rqt, rgt;
   float st = 0.0f;  // one statistic per thread of the first wavefront: lse2 (lanes 0-31) or delta (32-63)
   const int ntiles = p.sq / BT;
   auto fetch = [&](int t) {
     tile_fetch<D>(rq, qb + (long long)t * BT * D);
     tile_fetch<D>(rg, gb + (long long)t * BT * D);
+    trans_fetch<D>(rqt, qb + (long long)t * BT * D);
+    trans_fetch<D>(rgt, gb + (long long)t * BT * D);
     if (threadIdx.x < 2 * BT) {
       const float* src = threadIdx.x < BT ? lb : db;  // every lane loads; the factor is applied when stored
       st = src[t * BT + (threadIdx.x & (BT - 1))];
@@ -363,8 +389,8 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
     unsigned char* base = smem + buf * BUF;
     tile_store_rows<D>(rq, base);
     tile_store_rows<D>(rg, base + G::ROWMAJ);
-    tile_store_transposed<D>(rq, base + 2 * G::ROWMAJ);
-    tile_store_transposed<D>(rg, base + 2 * G::ROWMAJ + G::TRANS);
+    trans_store<D>(rqt, base + 2 * G::ROWMAJ);
+    trans_store<D>(rgt, base + 2 * G::ROWMAJ + G::TRANS);
     if (threadIdx.x < 2 * BT)
       reinterpret_cast<float*>(base + 2 * G::ROWMAJ + 2 * G::TRANS)[threadIdx.x] = threadIdx.x < BT ? st * LOG2E : st;
   };
