@@ -98,14 +98,16 @@ def _bias_args(bias, batch, sq, sk):
 
 
 # --------------------------------------------------------------------------- #
-# Shapes the MFMA kernels do not take as they are (head size below 64, sequence lengths that are
-# not multiples of 128) are brought to them on the host, in bf16 and without a bias:
+# Shapes the MFMA kernels do not take as they are (head sizes other than 64, 96 and 128 -- the
+# "widths" below --, sequence lengths that are not multiples of 128) are brought to them on the
+# host, in bf16 and without a bias:
 #   * head size: zero columns are appended to q, k, v (they add nothing to the scores and give
 #     zero output columns);
 #   * queries: zero rows are appended and their results dropped;
-#   * keys, head size below 64: rows are appended whose first spare column holds a large negative
-#     number, against a column of ones in q: their scores are about -30000, their probabilities 0;
-#   * keys, head size 64 (no spare column): the multiple of 128 goes through the MFMA kernels, the
+#   * keys, head size below its width: rows are appended whose first spare column holds a large
+#     negative number, against a column of ones in q: their scores are about -30000, their
+#     probabilities 0;
+#   * keys, head size equal to its width (no spare column): the multiple of 128 goes through the MFMA kernels, the
 #     remaining keys through the one-thread-per-row kernel, and the two (out, lse) pairs are merged
 #     like two ring steps; the backward treats the two key ranges like two ring chunks, the short
 #     one filled up with zero keys (which the backward's arithmetic ignores by itself).
@@ -114,11 +116,25 @@ def _bias_args(bias, batch, sq, sk):
 _MASKED_SCORE = -30000.0
 
 
+def _width(d: int) -> int:
+    """Head size of the MFMA kernels that take a head of ``d`` columns."""
+    return 64 if d <= 64 else 96 if d <= 96 else 128
+
+
+_KERNEL_HEAD_SIZES = (8, 16, 32, 64, 96, 128)
+
+
+def _kernel_head_size(d: int) -> int:
+    """Smallest head size the one-thread-per-row kernels are built for that holds ``d`` columns (zero
+    columns change neither scores nor the other outputs); ``d`` itself beyond the largest."""
+    return next((n for n in _KERNEL_HEAD_SIZES if n >= d), d)
+
+
 def _shapeable(q, k, bias) -> bool:
     d, sq, sk = q.shape[-1], q.shape[-2], k.shape[-2]
-    if bias is not None or q.dtype != torch.bfloat16 or d > 64 or sq == 0 or sk < 128:
+    if bias is not None or q.dtype != torch.bfloat16 or d > 128 or sq == 0 or sk < 128:
         return False
-    return d < 64 or sq % 128 != 0 or sk % 128 != 0
+    return d != _width(d) or sq % 128 != 0 or sk % 128 != 0
 
 
 def _pad_last(t: torch.Tensor, to: int) -> torch.Tensor:
@@ -137,11 +153,12 @@ def _shape_qkv(q, k, v, scale):
     """q, k, v as the MFMA kernels take them: ``(q, k, v, key ranges)``; a key range is
     ``(start, stop)`` in the (possibly padded) k / v, the first one a multiple of 128 long."""
     d, sq, sk = q.shape[-1], q.shape[-2], k.shape[-2]
-    qp = _pad_rows(_pad_last(q, 64), _up128(sq))
-    kp, vp = _pad_last(k, 64), _pad_last(v, 64)
+    w = _width(d)
+    qp = _pad_rows(_pad_last(q, w), _up128(sq))
+    kp, vp = _pad_last(k, w), _pad_last(v, w)
     if sk % 128 == 0:
         return qp, kp, vp, [(0, sk)]
-    if d < 64:
+    if d < w:
         qp[..., d] = 1.0
         kp, vp = _pad_rows(kp, _up128(sk)), _pad_rows(vp, _up128(sk))
         kp[..., sk:, d] = _MASKED_SCORE / float(scale)
@@ -156,9 +173,9 @@ def _shaped_forward(q, k, v, scale):
     out, lse = _core_forward(qp, kp[..., ranges[0][0]:ranges[0][1], :], vp[..., ranges[0][0]:ranges[0][1], :], scale)
     if len(ranges) == 2:
         o2, l2 = _core_forward(qp, kp[..., ranges[1][0]:ranges[1][1], :], vp[..., ranges[1][0]:ranges[1][1], :], scale)
-        rows = qp.shape[-2]
-        merged = fused_online_softmax_merge_(out.float().reshape(1, -1, rows, 64), lse.reshape(1, -1, rows),
-                                             o2.reshape(1, -1, rows, 64), l2.reshape(1, -1, rows), "bhsd")
+        rows, w = qp.shape[-2], qp.shape[-1]
+        merged = fused_online_softmax_merge_(out.float().reshape(1, -1, rows, w), lse.reshape(1, -1, rows),
+                                             o2.reshape(1, -1, rows, w), l2.reshape(1, -1, rows), "bhsd")
         out, lse = merged[0].to(q.dtype).reshape(out.shape), merged[1].reshape(lse.shape)
     return out[..., :sq, :d].contiguous(), lse[..., :sq].contiguous()
 
@@ -166,8 +183,8 @@ def _shaped_forward(q, k, v, scale):
 def _shaped_backward(grad_out, q, k, v, out, lse, scale):
     d, sq, sk = q.shape[-1], q.shape[-2], k.shape[-2]
     qp, kp, vp, ranges = _shape_qkv(q, k, v, scale)
-    rows = qp.shape[-2]
-    gp, op = _pad_rows(_pad_last(grad_out, 64), rows), _pad_rows(_pad_last(out, 64), rows)
+    rows, w = qp.shape[-2], qp.shape[-1]
+    gp, op = _pad_rows(_pad_last(grad_out, w), rows), _pad_rows(_pad_last(out, w), rows)
     lp = lse if lse.shape[-1] == rows else torch.nn.functional.pad(lse, (0, rows - lse.shape[-1]))
     dq, dks, dvs = None, [], []
     for lo, hi in ranges:
@@ -192,6 +209,10 @@ def core_forward(q, k, v, scale, bias=None, out_acc=None, lse_acc=None, want_out
     _check_qkv(q, k, v)
     if out_acc is None and lse_acc is None and want_out and _shapeable(q, k, bias):
         return _shaped_forward(q, k, v, scale)
+    d, dp = q.shape[-1], _kernel_head_size(q.shape[-1])
+    if dp != d and out_acc is None and lse_acc is None:
+        out, lse = _core_forward(_pad_last(q, dp), _pad_last(k, dp), _pad_last(v, dp), scale, bias, None, None, want_out)
+        return (out[..., :d].contiguous() if want_out else None), lse
     return _core_forward(q, k, v, scale, bias, out_acc, lse_acc, want_out)
 
 
@@ -229,6 +250,11 @@ def core_backward(grad_out, q, k, v, out, logsumexp, scale, bias=None, want_dbia
     _lib.require_gpu(grad_out, out, logsumexp)
     if not want_dbias and _shapeable(q, k, bias):
         return _shaped_backward(grad_out.to(q.dtype), q, k, v, out.to(q.dtype), logsumexp.to(torch.float32), scale)
+    d, dp = q.shape[-1], _kernel_head_size(q.shape[-1])
+    if dp != d:
+        res = _core_backward(_pad_last(grad_out, dp), _pad_last(q, dp), _pad_last(k, dp), _pad_last(v, dp),
+                             _pad_last(out, dp), logsumexp, scale, bias, want_dbias)
+        return tuple(t[..., :d].contiguous() for t in res[:3]) + tuple(res[3:])
     return _core_backward(grad_out, q, k, v, out, logsumexp, scale, bias, want_dbias)
 
 

@@ -42,6 +42,10 @@ CORE_SHAPES = [
     (1, 2, 128, 256, 128),  # head sizes 96 and 128: their own MFMA kernels for bf16
     (2, 2, 256, 128, 96),
     (1, 1, 384, 640, 128),
+    (1, 2, 200, 300, 80),   # padded to head size 96, spare-column key mask
+    (1, 1, 130, 260, 128),  # ragged at head size 128: MFMA on 256 keys + FMA kernel on 4, merged
+    (1, 1, 70, 200, 96),
+    (1, 2, 256, 128, 72),
 ]
 
 
@@ -223,5 +227,20 @@ def test_core_argument_errors(dev):
         ja.forward(q, q.bfloat16(), q, 0.25)
     with pytest.raises(ValueError):
         ja.forward(q, q[:, :1], q, 0.25)
+    wide = torch.zeros(1, 2, 8, 136, device=dev)  # beyond the largest head size the kernels are built for
     with pytest.raises(NotImplementedError):
-        ja.forward(q[..., :5].contiguous(), q[..., :5].contiguous(), q[..., :5].contiguous(), 0.25)
+        ja.forward(wide, wide, wide, 0.25)
+
+
+@pytest.mark.parametrize("d", [5, 40, 72])
+def test_head_sizes_between_the_kernel_sizes_are_zero_padded(d, dev):
+    q, k, v = _qkv(1, 2, 33, 47, d, torch.float32)
+    scale = d**-0.5
+    want_o, want_l = oa.core_forward(q.double(), k.double(), v.double(), scale)
+    out, lse, _ = ja.forward(q.to(dev), k.to(dev), v.to(dev), scale)
+    assert out.shape == q.shape and rel_l2(out, want_o) < 1e-5 and rel_l2(lse, want_l) < 1e-5
+    dout = torch.randn(1, 2, 33, d)
+    want = oa.core_backward(dout.double(), q.double(), k.double(), v.double(), want_o, want_l, scale)
+    got = ja.backward(dout.to(dev), q.to(dev), k.to(dev), v.to(dev), want_o.float().to(dev), want_l.float().to(dev), scale, 33, 47)
+    for g, w in zip(got, want):
+        assert g.shape == w.shape and rel_l2(g, w) < 1e-5
