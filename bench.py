@@ -221,6 +221,28 @@ def groupnorm_figures(dev, iters: int) -> dict:
     }
 
 
+def attention_wide_figures(dev, iters: int) -> dict:
+    """The attention core at head size 128 (its own MFMA kernels): 32 heads, 4096 queries x 4096
+    keys, bf16; forward, and backward (dQ + dK/dV) from the global out / lse."""
+    from jigsaw_amd import attention as ja
+
+    h, n, d = 32, 4096, 128
+    g = torch.Generator(device=dev).manual_seed(5)
+    q = (torch.randn(1, h, n, d, device=dev, generator=g) / d**0.5).bfloat16()
+    k = torch.randn(1, h, n, d, device=dev, generator=g).bfloat16()
+    v = torch.randn(1, h, n, d, device=dev, generator=g).bfloat16()
+    dout = torch.randn(1, h, n, d, device=dev, generator=g).bfloat16()
+    out, lse = ja.core_forward(q, k, v, d**-0.5)
+    ms_f = time_gpu(lambda: ja.core_forward(q, k, v, d**-0.5), iters)
+    ms_b = time_gpu(lambda: ja.core_backward(dout, q, k, v, out, lse, d**-0.5), iters)
+    f_fwd = 4.0 * h * n * n * d
+    tf = lambda f, ms: f / (ms * 1e-3) / 1e12  # noqa: E731
+    return {
+        "attn_d128_fwd": {"ms": ms_f, "tflops": tf(f_fwd, ms_f), "frac_mfma_peak": tf(f_fwd, ms_f) / PEAK_BF16_TFLOPS},
+        "attn_d128_bwd": {"ms": ms_b, "tflops": tf(2.5 * f_fwd, ms_b), "frac_mfma_peak": tf(2.5 * f_fwd, ms_b) / PEAK_BF16_TFLOPS},
+    }
+
+
 def projection_figures(dev, iters: int) -> dict:
     """The projections around the attention core with the head split / merge fused into the
     GEMM addressing, on 8 sequences of configuration 4 (32768 tokens, 512 channels, 8 heads
@@ -470,6 +492,7 @@ def main() -> int:
         extra.update(swin_figures(dev, it))
         extra.update(groupnorm_figures(dev, it))
         extra.update(projection_figures(dev, it))
+        extra.update(attention_wide_figures(dev, it))
 
     line = {
         "metric": METRIC,

@@ -5,6 +5,10 @@ FETCH_SIZE / WRITE_SIZE counters.
     rocprofv3 --kernel-trace --stats -d OUT -o kt --output-format csv -- python3 -m jigsaw_amd.profile_kernels
     rocprofv3 --pmc FETCH_SIZE -d OUT -o fetch --output-format csv -- python3 -m jigsaw_amd.profile_kernels
     rocprofv3 --pmc WRITE_SIZE -d OUT -o write --output-format csv -- python3 -m jigsaw_amd.profile_kernels
+
+With the argument ``around-attention`` it launches instead the kernels either side of the ring
+step: the attention core at head size 128 (32 heads, 4096 x 4096 tokens) and the qkv / output
+projections with the head split fused in (8 x 4096 tokens, 512 channels, 8 heads).
 """
 
 from __future__ import annotations
@@ -59,5 +63,39 @@ def main(reps: int = 3) -> None:
     print("profile_kernels: done", file=sys.stderr)
 
 
+def around_attention(reps: int = 3) -> None:
+    from jigsaw_amd import attention as ja
+    from jigsaw_amd import projection as jp
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(1)
+    h, n, d = 32, 4096, 128
+    q = (torch.randn(1, h, n, d, device=dev, generator=g) / d**0.5).bfloat16()
+    k = torch.randn(1, h, n, d, device=dev, generator=g).bfloat16()
+    v = torch.randn(1, h, n, d, device=dev, generator=g).bfloat16()
+    dout = torch.randn(1, h, n, d, device=dev, generator=g).bfloat16()
+    out, lse = ja.core_forward(q, k, v, d**-0.5)
+    bsz, c, heads = 8, 512, 8
+    x = torch.randn(bsz, n, c, device=dev, generator=g).bfloat16().requires_grad_()
+    w = (torch.randn(3 * c, c, device=dev, generator=g) / c**0.5).bfloat16().requires_grad_()
+    b = (0.1 * torch.randn(3 * c, device=dev, generator=g)).bfloat16().requires_grad_()
+    wo = (torch.randn(c, c, device=dev, generator=g) / c**0.5).bfloat16()
+    o = torch.randn(bsz, heads, n, c // heads, device=dev, generator=g).bfloat16()
+    gy = torch.randn(3, bsz, heads, n, c // heads, device=dev, generator=g).bfloat16()
+    for _ in range(reps):
+        ja.core_forward(q, k, v, d**-0.5)
+        ja.core_backward(dout, q, k, v, out, lse, d**-0.5)
+        y = jp.qkv_projection(x, w, b, heads)
+        torch.autograd.grad(y, (x, w, b), gy)
+        jp.heads_projection(o, wo, None)
+    torch.cuda.synchronize()
+    print("profile_kernels: done", file=sys.stderr)
+
+
 if __name__ == "__main__":
-    main()
+    if sys.argv[1:] == ["around-attention"]:
+        around_attention()
+    elif sys.argv[1:]:
+        raise SystemExit(f"unknown argument {sys.argv[1:]}; the only one is 'around-attention'")
+    else:
+        main()
