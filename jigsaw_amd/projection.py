@@ -146,6 +146,58 @@ class _HeadsProjection(torch.autograd.Function):
                 None if gb is None else gb.to(dt_b))
 
 
+class _Linear(torch.autograd.Function):
+    """``(*lead, k) -> (*lead, n)`` with ``weight (n, k)``: ``F.linear`` on the same GEMM kernels,
+    the bias gradient summed inside the weight-gradient GEMM."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):  # noqa: D102
+        _lib.require_gpu(x, weight, bias)
+        n_out, k = weight.shape
+        if x.dim() < 1 or x.shape[-1] != k:
+            raise ValueError(f"x has {x.shape[-1] if x.dim() else 0} features, the weight takes {k}")
+        xc = x.contiguous()
+        rows = xc.numel() // k
+        w = weight.to(x.dtype).contiguous()
+        bs = None if bias is None else bias.to(x.dtype).contiguous()
+        y = torch.empty((*x.shape[:-1], n_out), dtype=x.dtype, device=x.device)
+        if rows:
+            _nt(y, xc, w, bs, rows, n_out, k, False, False, (1, 1, 1, 1))
+        ctx.save_for_backward(xc, w)
+        ctx.has_bias = bias is not None
+        ctx.dtypes = (weight.dtype, None if bias is None else bias.dtype)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad):  # noqa: D102
+        xc, w = ctx.saved_tensors
+        n_out, k = w.shape
+        rows = xc.numel() // k
+        g = grad.to(xc.dtype).contiguous()
+        gx = gw = gb = None
+        need_b = ctx.has_bias and ctx.needs_input_grad[2]
+        if rows == 0:
+            gx = torch.zeros_like(xc) if ctx.needs_input_grad[0] else None
+            gw = torch.zeros_like(w) if ctx.needs_input_grad[1] else None
+            gb = torch.zeros(n_out, dtype=w.dtype, device=w.device) if need_b else None
+        else:
+            if ctx.needs_input_grad[0]:
+                gx = torch.empty_like(xc)
+                _nt(gx, g, w.t().contiguous(), None, rows, k, n_out, False, False, (1, 1, 1, 1))
+            if ctx.needs_input_grad[1] or need_b:
+                gw, gb = _tn(g, xc, rows, n_out, k, False, False, (1, 1, 1, 1), need_b)
+        dt_w, dt_b = ctx.dtypes
+        return (gx, None if gw is None or not ctx.needs_input_grad[1] else gw.to(dt_w),
+                None if gb is None else gb.to(dt_b))
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """``F.linear(x, weight, bias)`` in ``x.dtype`` on this package's GEMM kernels (the MLP and any
+    other token-wise layer around the attention core); its backward forms the weight and the bias
+    gradient in one pass over the output gradient."""
+    return _Linear.apply(x, weight, bias)
+
+
 def qkv_projection(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, heads: int) -> torch.Tensor:
     """``rearrange(F.linear(x, weight, bias), "... s (three h d) -> three ... h s d", three=3, h=heads)``
     without the intermediate ``(..., s, 3 h d)`` tensor (_attention.py:881-890)."""
@@ -158,4 +210,4 @@ def heads_projection(out: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor
     return _HeadsProjection.apply(out, weight, bias)
 
 
-__all__ = ["heads_projection", "qkv_projection"]
+__all__ = ["heads_projection", "linear", "qkv_projection"]

@@ -22,7 +22,7 @@ import torch.nn as nn
 from .attention import window_attention
 from .conv import TileGroup
 from .layernorm import layer_norm
-from .projection import heads_projection, qkv_projection
+from .projection import heads_projection, linear, qkv_projection
 from .roll import _Roll
 
 
@@ -68,8 +68,16 @@ class _TokenLinear(torch.autograd.Function):
         return gx, gw, gb
 
 
+def _compute_dtype(x: torch.Tensor) -> torch.dtype:
+    """The dtype a linear layer computes in: the autocast dtype when autocast is on."""
+    return torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else x.dtype
+
+
 def token_linear(x: torch.Tensor, layer: nn.Linear) -> torch.Tensor:
-    """``layer(x)`` with the token-split weight gradient."""
+    """``layer(x)``: in bf16 on this package's GEMM kernels (bias gradient fused into the weight
+    gradient), otherwise through the library GEMM with the token-split weight gradient."""
+    if x.is_cuda and _compute_dtype(x) == torch.bfloat16 and x.shape[-1] % 8 == 0 and layer.weight.shape[0] % 8 == 0:
+        return linear(x.to(torch.bfloat16), layer.weight, layer.bias)
     return _TokenLinear.apply(x, layer.weight, layer.bias)
 
 
@@ -180,7 +188,10 @@ class SwinBlock(nn.Module):
     # The block in stages, so that a single-process harness can run several ranks
     # in lockstep (the two rolls are the only stages that talk to other ranks).
     def pre_attention(self, x: torch.Tensor) -> torch.Tensor:
-        return self._norm(self.norm1, x)
+        # Under autocast the LayerNorm yields fp32 and the qkv layer would round it to the autocast
+        # dtype; rounding before the roll and the window partition (pure copies) gives the same
+        # numbers and halves the bytes those copies move.
+        return self._norm(self.norm1, x).to(_compute_dtype(x))
 
     def shift(self, y: torch.Tensor) -> torch.Tensor:
         return self._roll(y, -self.shift_by)

@@ -123,3 +123,39 @@ def test_full_size_against_torch_gemm(dev):
     assert rel_l2(x.grad.float(), (gflat.float() @ w.detach().float()).reshape(bsz, s, c)) <= 4e-3
     assert rel_l2(w.grad.float(), gflat.float().t() @ x.detach().reshape(-1, c).float()) <= 4e-3
     assert rel_l2(b.grad.float(), gflat.float().sum(0)) <= 4e-3
+
+
+@pytest.mark.parametrize("shape,n_out,dtype,has_b", [
+    ((1, 256, 256, 128), 512, torch.bfloat16, True),   # the MLP of a Swin block on a 256 x 256 token tile
+    ((3, 50, 72), 40, torch.bfloat16, True),
+    ((130, 64), 24, torch.bfloat16, False),
+    ((2, 33, 24), 10, torch.float32, True),
+    ((0, 32), 16, torch.bfloat16, True),
+], ids=lambda v: str(v).replace(" ", ""))
+def test_linear_matches_oracle(shape, n_out, dtype, has_b, dev):
+    """``projection.linear`` is the output projection with one head: the oracle's heads_forward /
+    heads_backward on ``x`` viewed as ``(..., 1, tokens, features)``."""
+    tol = TOL[dtype]
+    torch.manual_seed(5)
+    k = shape[-1]
+    x = torch.randn(*shape).to(dtype)
+    w = (torch.randn(n_out, k) / k ** 0.5).to(dtype)
+    b = (0.1 * torch.randn(n_out)).to(dtype) if has_b else None
+    g = torch.randn(*shape[:-1], n_out).to(dtype)
+    print(f"linear {shape} -> {n_out} {dtype}", flush=True)
+    xd, wd = x.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+    bd = b.to(dev).requires_grad_() if has_b else None
+    y = jp.linear(xd, wd, bd)
+    assert y.shape == g.shape and y.dtype == dtype
+    y.backward(g.to(dev))
+    if x.numel():
+        x3 = x.reshape(1, 1, -1, k).double()
+        want = op.heads_forward(x3, w.double(), b.double() if has_b else None).reshape(g.shape)
+        gx, gw, gb = op.heads_backward(g.reshape(1, -1, n_out).double(), x3, w.double())
+        assert rel_l2(y.detach().cpu(), want) <= tol
+        assert rel_l2(xd.grad.cpu(), gx.reshape(shape)) <= tol
+        assert rel_l2(wd.grad.cpu(), gw) <= tol
+        if has_b:
+            assert rel_l2(bd.grad.cpu(), gb) <= tol
+    else:
+        assert float(wd.grad.abs().sum()) == 0.0 and xd.grad.shape == x.shape
