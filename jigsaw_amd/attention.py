@@ -377,7 +377,8 @@ class _BiasedAttention(torch.autograd.Function):
             # sum the per-batch-entry gradient over the entries that share a bias matrix
             sq, sk = q.shape[-2], k.shape[-2]
             period = bias.numel() // (sq * sk)
-            dbias = res[3].reshape(-1, period, sq, sk).sum(0).reshape(bias.shape).to(bias.dtype)
+            per_entry = res[3].reshape(-1, period, sq, sk)
+            dbias = (per_entry[0] if per_entry.shape[0] == 1 else per_entry.sum(0)).reshape(bias.shape).to(bias.dtype)
         return dq, dk, dv, dbias
 
 

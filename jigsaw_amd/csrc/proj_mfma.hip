@@ -460,14 +460,57 @@ __global__ __launch_bounds__(64 * WM * WN) void proj_tn_kernel(TnParams p) {
   }
 }
 
-// out[i] (bf16) = sum over the splits of part[split][i], fixed order
-__global__ __launch_bounds__(256) void proj_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ part,
-                                                          int splits, size_t count) {
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= count) return;
-  float s = 0.0f;
-  for (int k = 0; k < splits; ++k) s += part[(size_t)k * count + i];
-  out[i] = jg::f32_to_bf16(s);
+// out[i] (bf16) = sum over the splits of part[split][i], for the weight gradient and (blocks behind
+// it) the bias gradient in one launch. A block takes 256 consecutive outputs: 64 lanes x 4 values,
+// and its four wavefronts each add every fourth split; the four sums are then added in a fixed
+// order, so the result does not depend on scheduling.
+struct ReduceArgs {
+  uint16_t* out_w;
+  const float* part_w;
+  size_t count_w;
+  uint16_t* out_b;  // NULL: no bias gradient
+  const float* part_b;
+  size_t count_b;
+  int splits;
+};
+
+__global__ __launch_bounds__(256) void proj_reduce_kernel(ReduceArgs a) {
+  __shared__ f32x4 sm[4][64];
+  const size_t blocks_w = (a.count_w + 255) / 256;
+  const bool second = blockIdx.x >= blocks_w;
+  uint16_t* out = second ? a.out_b : a.out_w;
+  const float* part = second ? a.part_b : a.part_w;
+  const size_t count = second ? a.count_b : a.count_w;
+  const int q = threadIdx.x & 63, grp = threadIdx.x >> 6;
+  const size_t i0 = (blockIdx.x - (second ? blocks_w : 0)) * 256 + (size_t)q * 4;
+  // every split's slice starts 16-byte aligned when the count is a multiple of 4 and the base is aligned
+  const bool vec = (count & 3) == 0 && (reinterpret_cast<uintptr_t>(part) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(out) & 7) == 0;
+  f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (i0 < count) {
+    if (vec) {
+      for (int k = grp; k < a.splits; k += 4) acc += *reinterpret_cast<const f32x4*>(part + (size_t)k * count + i0);
+    } else {
+      for (int k = grp; k < a.splits; k += 4)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (i0 + e < count) acc[e] += part[(size_t)k * count + i0 + e];
+    }
+  }
+  sm[grp][q] = acc;
+  __syncthreads();
+  if (grp != 0 || i0 >= count) return;
+  const f32x4 t = ((sm[0][q] + sm[1][q]) + sm[2][q]) + sm[3][q];
+  if (vec) {
+    u32x2 o;
+    o.x = (uint32_t)jg::f32_to_bf16(t[0]) | ((uint32_t)jg::f32_to_bf16(t[1]) << 16);
+    o.y = (uint32_t)jg::f32_to_bf16(t[2]) | ((uint32_t)jg::f32_to_bf16(t[3]) << 16);
+    *reinterpret_cast<u32x2*>(out + i0) = o;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (i0 + e < count) out[i0 + e] = jg::f32_to_bf16(t[e]);
+  }
 }
 
 // ------------------------------------------------------------------- generic
@@ -733,14 +776,17 @@ int jg_proj_tn(void* gw, void* gb, const void* g, const void* x, int dtype, int6
   p.bias_part = gb != nullptr ? p.part + (size_t)splits * n * c : nullptr;
   rc = tn_tile(rows, n, c) == 256 ? launch_tn<4, 2, 2, 4>(p, splits, s, who) : launch_tn<2, 2, 2, 2>(p, splits, s, who);
   if (rc) return rc;
-  const size_t count = (size_t)n * c;
-  proj_reduce_kernel<<<(unsigned)((count + 255) / 256), 256, 0, s>>>(static_cast<uint16_t*>(gw), p.part, splits, count);
+  ReduceArgs ra{};
+  ra.out_w = static_cast<uint16_t*>(gw);
+  ra.part_w = p.part;
+  ra.count_w = (size_t)n * c;
+  ra.out_b = static_cast<uint16_t*>(gb);
+  ra.part_b = p.bias_part;
+  ra.count_b = gb != nullptr ? (size_t)n : 0;
+  ra.splits = splits;
+  const size_t blocks = (ra.count_w + 255) / 256 + (ra.count_b + 255) / 256;
+  proj_reduce_kernel<<<(unsigned)blocks, 256, 0, s>>>(ra);
   JG_CHECK_LAUNCH(who);
-  if (gb != nullptr) {
-    proj_reduce_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(static_cast<uint16_t*>(gb), p.bias_part, splits,
-                                                                    (size_t)n);
-    JG_CHECK_LAUNCH(who);
-  }
   return JG_OK;
 }
 
