@@ -194,6 +194,29 @@ int jg_ln_bwd_apply(void* gx, const void* g, const void* x_hat, const void* w,
                     const float* std, int64_t rows, int64_t cols, int64_t n_global,
                     int dtype, void* stream);
 
+/* LayerNorm over rows that are NOT split over a channel group (nn.LayerNorm as the
+ * example Swin block applies it, examples/swin.py:186-188, 209-210): statistics and
+ * apply in one pass, y = w * (x - mean) * rstd + b with rstd = 1/sqrt(var + eps)
+ * (biased variance), fp32 arithmetic. w, b (may be NULL) are fp32; x and y may
+ * differ in dtype when one of them is fp32 (autocast: bf16 in, fp32 or bf16 out).
+ * mean, rstd (rows) fp32 are what the backward needs besides x. cols must be a
+ * multiple of 8 and at most 2048 (jg_ln_plain_supported), x / y 16-byte aligned;
+ * JG_ERR_UNSUPPORTED otherwise: use the partial-statistics entry points above. */
+int jg_ln_plain_supported(int64_t cols);
+int jg_ln_plain_fwd(void* y, float* mean, float* rstd, const void* x, const float* w,
+                    const float* b, int64_t rows, int64_t cols, float eps, int x_dtype,
+                    int y_dtype, void* stream);
+
+/* Backward of jg_ln_plain_fwd from (x, mean, rstd): x_hat = (x - mean) * rstd,
+ * gx = rstd * (g w - mean_c(g w) - x_hat * mean_c(g w x_hat)) in x's dtype (gx may
+ * be NULL), gw[c] = sum_r g x_hat, gb[c] = sum_r g (fp32, either may be NULL;
+ * two-stage deterministic column sums through the workspace). */
+size_t jg_ln_plain_bwd_workspace_bytes(int64_t rows, int64_t cols);
+int jg_ln_plain_bwd(void* gx, float* gw, float* gb, const void* g, const void* x,
+                    const float* mean, const float* rstd, const float* w, int64_t rows,
+                    int64_t cols, int g_dtype, int x_dtype, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------- *
  * GroupNorm over a spatially sharded input (HBM-bound)
  *

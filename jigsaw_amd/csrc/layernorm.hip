@@ -306,6 +306,272 @@ bool vec_aligned(const void* p, long long cols, int dtype) {
 
 bool known(int dt) { return dt == JG_F32 || dt == JG_BF16 || dt == JG_F16; }
 
+// ------------------------------------------------------------------ unsharded
+// LayerNorm over rows that one rank holds whole (nn.LayerNorm as the Swin block uses it,
+// examples/swin.py:186-188, 209-210): statistics and apply in one pass over x, and a backward
+// that recomputes x_hat from (x, mean, rstd). A row is held in registers: G lanes share a row
+// (8 columns per lane and chunk, at most kPlainChunks chunks), 64 / G rows per wavefront, so
+// narrow rows still use every lane. x, y, g and gx may each have their own dtype; w, b fp32.
+constexpr int kPlainVec = 8;
+constexpr int kPlainChunks = 4;
+
+template <int DT>
+__device__ __forceinline__ void load8(const typename Elem<DT>::T* p, float out[kPlainVec]) {
+  typedef typename Elem<DT>::T T;
+  struct alignas(16) Pack { T v[16 / sizeof(T)]; };
+  constexpr int PER = 16 / sizeof(T);
+#pragma unroll
+  for (int h = 0; h < kPlainVec / PER; ++h) {
+    const Pack q = *reinterpret_cast<const Pack*>(p + h * PER);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) out[h * PER + i] = Elem<DT>::up(q.v[i]);
+  }
+}
+template <int DT>
+__device__ __forceinline__ void store8(typename Elem<DT>::T* p, const float in[kPlainVec]) {
+  typedef typename Elem<DT>::T T;
+  struct alignas(16) Pack { T v[16 / sizeof(T)]; };
+  constexpr int PER = 16 / sizeof(T);
+#pragma unroll
+  for (int h = 0; h < kPlainVec / PER; ++h) {
+    Pack q;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) q.v[i] = Elem<DT>::down(in[h * PER + i]);
+    *reinterpret_cast<Pack*>(p + h * PER) = q;
+  }
+}
+
+// sum over the G lanes (a power of two) that share a row
+__device__ __forceinline__ float group_sum(float v, int G) {
+  for (int o = G >> 1; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+
+template <int XDT, int YDT, int CH>
+__global__ __launch_bounds__(kThreads) void ln_plain_fwd_kernel(
+    typename Elem<YDT>::T* __restrict__ y, float* __restrict__ mean, float* __restrict__ rstd,
+    const typename Elem<XDT>::T* __restrict__ x, const float* __restrict__ w,
+    const float* __restrict__ b, long long rows, int cols, float eps, int G) {
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
+  const float inv = 1.0f / (float)cols;
+  float wv[CH][kPlainVec], bv[CH][kPlainVec];
+#pragma unroll
+  for (int k = 0; k < CH; ++k) {
+    const int c = (k * G + sl) * kPlainVec;
+#pragma unroll
+    for (int i = 0; i < kPlainVec; ++i) {
+      wv[k][i] = c < cols ? w[c + i] : 0.0f;
+      bv[k][i] = (c < cols && b != nullptr) ? b[c + i] : 0.0f;
+    }
+  }
+  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows;
+       r0 += (long long)gridDim.x * kWavesPerBlock * rpw) {
+    const long long r = r0 + sub;
+    const bool live = r < rows;
+    float v[CH][kPlainVec];
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+      const int c = (k * G + sl) * kPlainVec;
+      if (live && c < cols) {
+        load8<XDT>(x + r * cols + c, v[k]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < kPlainVec; ++i) v[k][i] = 0.0f;
+      }
+#pragma unroll
+      for (int i = 0; i < kPlainVec; ++i) s += v[k][i];
+    }
+    const float m = group_sum(s, G) * inv;
+    float q = 0.0f;
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+      const int c = (k * G + sl) * kPlainVec;
+      if (c < cols) {
+#pragma unroll
+        for (int i = 0; i < kPlainVec; ++i) {
+          const float d = v[k][i] - m;
+          q += d * d;
+        }
+      }
+    }
+    const float rs = rsqrtf(group_sum(q, G) * inv + eps);
+    if (!live) continue;  // after the shuffles: every lane of the wavefront takes part in them
+    if (sl == 0) {
+      mean[r] = m;
+      rstd[r] = rs;
+    }
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+      const int c = (k * G + sl) * kPlainVec;
+      if (c < cols) {
+        float out[kPlainVec];
+#pragma unroll
+        for (int i = 0; i < kPlainVec; ++i) out[i] = (v[k][i] - m) * rs * wv[k][i] + bv[k][i];
+        store8<YDT>(y + r * cols + c, out);
+      }
+    }
+  }
+}
+
+// gx = rstd * (g w - mean_c(g w) - x_hat * mean_c(g w x_hat)); column partials of g x_hat and g
+// per block in part[blk][which][col] (ln_colreduce_kernel finishes them).
+template <int GDT, int XDT, int CH>
+__global__ __launch_bounds__(kThreads) void ln_plain_bwd_kernel(
+    typename Elem<XDT>::T* __restrict__ gx, float* __restrict__ part,
+    const typename Elem<GDT>::T* __restrict__ g, const typename Elem<XDT>::T* __restrict__ x,
+    const float* __restrict__ mean, const float* __restrict__ rstd, const float* __restrict__ w,
+    long long rows, int cols, int G, bool want_cols) {
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
+  const float inv = 1.0f / (float)cols;
+  float wv[CH][kPlainVec], agw[CH][kPlainVec], agb[CH][kPlainVec];
+#pragma unroll
+  for (int k = 0; k < CH; ++k) {
+    const int c = (k * G + sl) * kPlainVec;
+#pragma unroll
+    for (int i = 0; i < kPlainVec; ++i) {
+      wv[k][i] = c < cols ? w[c + i] : 0.0f;
+      agw[k][i] = 0.0f;
+      agb[k][i] = 0.0f;
+    }
+  }
+  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows;
+       r0 += (long long)gridDim.x * kWavesPerBlock * rpw) {
+    const long long r = r0 + sub;
+    const bool live = r < rows;
+    const float m = live ? mean[r] : 0.0f, rs = live ? rstd[r] : 0.0f;
+    float gv[CH][kPlainVec], xh[CH][kPlainVec];
+    float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+      const int c = (k * G + sl) * kPlainVec;
+      if (live && c < cols) {
+        load8<GDT>(g + r * cols + c, gv[k]);
+        load8<XDT>(x + r * cols + c, xh[k]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < kPlainVec; ++i) {
+          gv[k][i] = 0.0f;
+          xh[k][i] = m;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < kPlainVec; ++i) {
+        xh[k][i] = (xh[k][i] - m) * rs;
+        const float gxn = gv[k][i] * wv[k][i];
+        s1 += gxn;
+        s2 += gxn * xh[k][i];
+        agw[k][i] += gv[k][i] * xh[k][i];
+        agb[k][i] += gv[k][i];
+      }
+    }
+    s1 = group_sum(s1, G) * inv;
+    s2 = group_sum(s2, G) * inv;
+    if (!live || gx == nullptr) continue;
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+      const int c = (k * G + sl) * kPlainVec;
+      if (c < cols) {
+        float out[kPlainVec];
+#pragma unroll
+        for (int i = 0; i < kPlainVec; ++i) out[i] = rs * (gv[k][i] * wv[k][i] - s1 - xh[k][i] * s2);
+        store8<XDT>(gx + r * cols + c, out);
+      }
+    }
+  }
+  if (!want_cols) return;
+  // the rows of a wavefront that share a column set: lanes sl, sl + G, ...
+#pragma unroll
+  for (int k = 0; k < CH; ++k)
+#pragma unroll
+    for (int i = 0; i < kPlainVec; ++i)
+      for (int o = G; o < kWave; o <<= 1) {
+        agw[k][i] += __shfl_xor(agw[k][i], o, kWave);
+        agb[k][i] += __shfl_xor(agb[k][i], o, kWave);
+      }
+  __shared__ float red[kWavesPerBlock][2][kPlainChunks * kWave * kPlainVec];
+  if (sub == 0) {
+#pragma unroll
+    for (int k = 0; k < CH; ++k)
+#pragma unroll
+      for (int i = 0; i < kPlainVec; ++i) {
+        red[wave][0][(k * G + sl) * kPlainVec + i] = agw[k][i];
+        red[wave][1][(k * G + sl) * kPlainVec + i] = agb[k][i];
+      }
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < cols; c += kThreads) {
+    float a = 0.0f, b2 = 0.0f;
+#pragma unroll
+    for (int wv2 = 0; wv2 < kWavesPerBlock; ++wv2) {
+      a += red[wv2][0][c];
+      b2 += red[wv2][1][c];
+    }
+    part[((long long)blockIdx.x * 2 + 0) * cols + c] = a;
+    part[((long long)blockIdx.x * 2 + 1) * cols + c] = b2;
+  }
+}
+
+// lanes per row: the power of two that covers cols / 8 columns-octets in the fewest chunks
+int plain_group(long long cols) {
+  int G = 1;
+  while (G < kWave && (long long)G * kPlainVec < cols) G <<= 1;
+  return G;
+}
+int plain_chunks(long long cols) {
+  const int G = plain_group(cols);
+  return (int)((cols + (long long)G * kPlainVec - 1) / ((long long)G * kPlainVec));
+}
+bool plain_ok(long long cols) { return cols >= kPlainVec && cols % kPlainVec == 0 && plain_chunks(cols) <= kPlainChunks; }
+int plain_blocks(long long rows, long long cols) {
+  const int rpw = kWave / plain_group(cols);
+  long long b = (rows + (long long)kWavesPerBlock * rpw - 1) / ((long long)kWavesPerBlock * rpw);
+  if (b > 1024) b = 1024;
+  if (b < 1) b = 1;
+  return (int)b;
+}
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+template <int XDT, int YDT>
+void launch_plain_fwd(void* y, float* mean, float* rstd, const void* x, const float* w, const float* b,
+                      long long rows, int cols, float eps, hipStream_t s) {
+  typedef typename Elem<XDT>::T XT;
+  typedef typename Elem<YDT>::T YT;
+  const int G = plain_group(cols), blocks = plain_blocks(rows, cols) * 4 > 65536 ? 65536 : plain_blocks(rows, cols) * 4;
+#define JG_GO(CH)                                                                                   \
+  ln_plain_fwd_kernel<XDT, YDT, CH><<<blocks, kThreads, 0, s>>>(static_cast<YT*>(y), mean, rstd,     \
+                                                                static_cast<const XT*>(x), w, b, rows, cols, eps, G)
+  switch (plain_chunks(cols)) {
+    case 1: JG_GO(1); break;
+    case 2: JG_GO(2); break;
+    case 3: JG_GO(3); break;
+    default: JG_GO(4); break;
+  }
+#undef JG_GO
+}
+
+template <int GDT, int XDT>
+void launch_plain_bwd(void* gx, float* part, const void* g, const void* x, const float* mean, const float* rstd,
+                      const float* w, long long rows, int cols, bool want_cols, hipStream_t s) {
+  typedef typename Elem<GDT>::T GT;
+  typedef typename Elem<XDT>::T XT;
+  const int G = plain_group(cols), blocks = plain_blocks(rows, cols);
+#define JG_GO(CH)                                                                                     \
+  ln_plain_bwd_kernel<GDT, XDT, CH><<<blocks, kThreads, 0, s>>>(static_cast<XT*>(gx), part,            \
+                                                                static_cast<const GT*>(g),             \
+                                                                static_cast<const XT*>(x), mean, rstd, \
+                                                                w, rows, cols, G, want_cols)
+  switch (plain_chunks(cols)) {
+    case 1: JG_GO(1); break;
+    case 2: JG_GO(2); break;
+    case 3: JG_GO(3); break;
+    default: JG_GO(4); break;
+  }
+#undef JG_GO
+}
+
 }  // namespace
 
 extern "C" int jg_ln_partial_fwd(float* mean, float* var, const void* x, int64_t rows,
@@ -458,5 +724,97 @@ extern "C" int jg_ln_bwd_apply(void* gx, const void* g, const void* x_hat, const
   else JG_GO(JG_F16);
 #undef JG_GO
   JG_CHECK_LAUNCH("jg_ln_bwd_apply");
+  return JG_OK;
+}
+
+
+extern "C" int jg_ln_plain_supported(int64_t cols) { return plain_ok(cols) ? 1 : 0; }
+
+extern "C" int jg_ln_plain_fwd(void* y, float* mean, float* rstd, const void* x, const float* w,
+                               const float* b, int64_t rows, int64_t cols, float eps, int x_dtype,
+                               int y_dtype, void* stream) {
+  const char* who = "jg_ln_plain_fwd";
+  JG_REQUIRE(y && mean && rstd && x && w, "%s: NULL pointer", who);
+  JG_REQUIRE(rows >= 0 && cols >= 1, "%s: bad shape (%lld, %lld)", who, (long long)rows, (long long)cols);
+  JG_REQUIRE(known(x_dtype) && known(y_dtype), "%s: unknown dtype", who);
+  if (!plain_ok(cols))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: %lld columns (needs a multiple of 8, at most %d)", who, (long long)cols,
+            kPlainChunks * kWave * kPlainVec);
+  JG_REQUIRE(aligned16(y) && aligned16(x), "%s: x and y must be 16-byte aligned", who);
+  JG_REQUIRE(y_dtype == x_dtype || y_dtype == JG_F32 || x_dtype == JG_F32, "%s: x dtype %d with y dtype %d", who,
+             x_dtype, y_dtype);
+  if (rows == 0) return JG_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define JG_GO(X, Y) launch_plain_fwd<X, Y>(y, mean, rstd, x, w, b, rows, (int)cols, eps, s)
+  if (x_dtype == JG_F32) {
+    if (y_dtype == JG_F32) JG_GO(JG_F32, JG_F32);
+    else if (y_dtype == JG_BF16) JG_GO(JG_F32, JG_BF16);
+    else JG_GO(JG_F32, JG_F16);
+  } else if (x_dtype == JG_BF16) {
+    if (y_dtype == JG_F32) JG_GO(JG_BF16, JG_F32);
+    else JG_GO(JG_BF16, JG_BF16);
+  } else {
+    if (y_dtype == JG_F32) JG_GO(JG_F16, JG_F32);
+    else JG_GO(JG_F16, JG_F16);
+  }
+#undef JG_GO
+  JG_CHECK_LAUNCH(who);
+  return JG_OK;
+}
+
+extern "C" size_t jg_ln_plain_bwd_workspace_bytes(int64_t rows, int64_t cols) {
+  if (rows <= 0 || cols <= 0 || !plain_ok(cols)) return 0;
+  return (size_t)plain_blocks(rows, cols) * 2 * (size_t)cols * sizeof(float);
+}
+
+extern "C" int jg_ln_plain_bwd(void* gx, float* gw, float* gb, const void* g, const void* x,
+                               const float* mean, const float* rstd, const float* w, int64_t rows,
+                               int64_t cols, int g_dtype, int x_dtype, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+  const char* who = "jg_ln_plain_bwd";
+  JG_REQUIRE(g && x && mean && rstd && w, "%s: NULL pointer", who);
+  JG_REQUIRE(rows >= 0 && cols >= 1, "%s: bad shape (%lld, %lld)", who, (long long)rows, (long long)cols);
+  JG_REQUIRE(known(x_dtype) && known(g_dtype), "%s: unknown dtype", who);
+  if (!plain_ok(cols))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: %lld columns (needs a multiple of 8, at most %d)", who, (long long)cols,
+            kPlainChunks * kWave * kPlainVec);
+  JG_REQUIRE(aligned16(g) && aligned16(x) && (gx == nullptr || aligned16(gx)), "%s: g, x and gx must be 16-byte aligned",
+             who);
+  JG_REQUIRE(g_dtype == x_dtype || g_dtype == JG_F32 || x_dtype == JG_F32, "%s: g dtype %d with x dtype %d", who,
+             g_dtype, x_dtype);
+  const bool want_cols = gw != nullptr || gb != nullptr;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (rows == 0) {
+    // no rows: the column sums are zero (a fill kernel, so that the call can be captured in a graph)
+    if (want_cols) {
+      ln_colreduce_kernel<<<(unsigned)((cols + 63) / 64), 256, 0, s>>>(gw, gb, nullptr, 0, cols);
+      JG_CHECK_LAUNCH(who);
+    }
+    return JG_OK;
+  }
+  float* part = static_cast<float*>(workspace);
+  if (want_cols) {
+    const size_t need = jg_ln_plain_bwd_workspace_bytes(rows, cols);
+    if (workspace == nullptr || workspace_bytes < need)
+      JG_FAIL(JG_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", who, workspace_bytes, need);
+  }
+#define JG_GO(G_, X) launch_plain_bwd<G_, X>(gx, part, g, x, mean, rstd, w, rows, (int)cols, want_cols, s)
+  if (x_dtype == JG_F32) {
+    if (g_dtype == JG_F32) JG_GO(JG_F32, JG_F32);
+    else if (g_dtype == JG_BF16) JG_GO(JG_BF16, JG_F32);
+    else JG_GO(JG_F16, JG_F32);
+  } else if (x_dtype == JG_BF16) {
+    if (g_dtype == JG_F32) JG_GO(JG_F32, JG_BF16);
+    else JG_GO(JG_BF16, JG_BF16);
+  } else {
+    if (g_dtype == JG_F32) JG_GO(JG_F32, JG_F16);
+    else JG_GO(JG_F16, JG_F16);
+  }
+#undef JG_GO
+  JG_CHECK_LAUNCH(who);
+  if (want_cols) {
+    ln_colreduce_kernel<<<(unsigned)((cols + 63) / 64), 256, 0, s>>>(gw, gb, part, plain_blocks(rows, cols), cols);
+    JG_CHECK_LAUNCH(who);
+  }
   return JG_OK;
 }

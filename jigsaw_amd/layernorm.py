@@ -153,4 +153,68 @@ def layer_norm(x, weight, bias, channel_group=None, eps: float = 1e-5) -> torch.
     return _LayerNorm.apply(x, weight, bias, channel_group, eps)[0]
 
 
-__all__ = ["_LayerNorm", "layer_norm", "partial_stats"]
+class _PlainLayerNorm(torch.autograd.Function):
+    """``nn.LayerNorm`` over rows one rank holds whole: one fused kernel forward, one backward
+    (plus the column reduction) that recomputes ``x_hat`` from ``(x, mean, rstd)``."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, eps, out_dtype):  # noqa: D102
+        _lib.require_gpu(x, weight, bias)
+        xc = x.contiguous()
+        cols = xc.shape[-1]
+        rows = xc.numel() // cols
+        w = weight.to(torch.float32).contiguous()
+        b = None if bias is None else bias.to(torch.float32).contiguous()
+        y = torch.empty(xc.shape, dtype=out_dtype, device=x.device)
+        mean = torch.empty(rows, dtype=torch.float32, device=x.device)
+        rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
+        rc = _lib.load().jg_ln_plain_fwd(_lib.ptr(y), _lib.ptr(mean), _lib.ptr(rstd), _lib.ptr(xc), _lib.ptr(w), _lib.ptr(b),
+                                         rows, cols, float(eps), _lib.dtype_code(xc.dtype), _lib.dtype_code(out_dtype),
+                                         _lib.stream_ptr(x.device))
+        _lib.check(rc, "jg_ln_plain_fwd")
+        ctx.save_for_backward(xc, mean, rstd, w)
+        ctx.has_bias = bias is not None
+        ctx.param_dtypes = (weight.dtype, None if bias is None else bias.dtype)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad):  # noqa: D102
+        xc, mean, rstd, w = ctx.saved_tensors
+        cols = xc.shape[-1]
+        rows = xc.numel() // cols
+        g = grad.contiguous()
+        if g.dtype != xc.dtype and torch.float32 not in (g.dtype, xc.dtype):
+            g = g.to(xc.dtype)
+        dev = g.device
+        need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        need_b = ctx.has_bias and ctx.needs_input_grad[2]
+        gx = torch.empty_like(xc) if need_x else None
+        gw = torch.empty(cols, dtype=torch.float32, device=dev) if need_w else None
+        gb = torch.empty(cols, dtype=torch.float32, device=dev) if need_b else None
+        lib = _lib.load()
+        nbytes = int(lib.jg_ln_plain_bwd_workspace_bytes(rows, cols)) if (need_w or need_b) else 0
+        ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=dev)
+        rc = lib.jg_ln_plain_bwd(_lib.ptr(gx), _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(g), _lib.ptr(xc), _lib.ptr(mean),
+                                 _lib.ptr(rstd), _lib.ptr(w), rows, cols, _lib.dtype_code(g.dtype), _lib.dtype_code(xc.dtype),
+                                 _lib.ptr(ws), nbytes, _lib.stream_ptr(dev))
+        _lib.check(rc, "jg_ln_plain_bwd")
+        wdt, bdt = ctx.param_dtypes
+        return gx, (gw.to(wdt) if need_w else None), (gb.to(bdt) if need_b else None), None, None
+
+
+def plain_layer_norm(x, weight, bias, eps: float = 1e-5, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """``F.layer_norm(x, (x.shape[-1],), weight, bias, eps)`` for rows that are not split over a
+    channel group (the ``nn.LayerNorm`` of examples/swin.py:186-188). ``out_dtype`` defaults to
+    what torch yields: fp32 under autocast, else ``x.dtype``; a caller whose next layer rounds to the
+    autocast dtype anyway may ask for that dtype here and save the fp32 round trip. Widths the fused
+    kernels do not take (not a multiple of 8, above 2048) go through :func:`layer_norm`."""
+    odt = out_dtype or _compute_dtype(x)
+    if x.numel() == 0:  # nothing to launch; torch keeps the (empty) graph connected
+        return torch.nn.functional.layer_norm(x.to(odt), x.shape[-1:], weight.to(odt),
+                                              None if bias is None else bias.to(odt), eps)
+    if not _lib.load().jg_ln_plain_supported(x.shape[-1]):
+        return layer_norm(x, weight, bias, None, eps).to(odt)
+    return _PlainLayerNorm.apply(x, weight, bias, eps, odt)
+
+
+__all__ = ["_LayerNorm", "layer_norm", "partial_stats", "plain_layer_norm"]

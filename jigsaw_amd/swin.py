@@ -21,7 +21,7 @@ import torch.nn as nn
 
 from .attention import window_attention
 from .conv import TileGroup
-from .layernorm import layer_norm
+from .layernorm import plain_layer_norm
 from .projection import heads_projection, linear, qkv_projection
 from .roll import _Roll
 
@@ -183,15 +183,15 @@ class SwinBlock(nn.Module):
         return _Roll.apply(x.contiguous(), (shift, shift), (1, 2), dist_dims, dist_groups, self.comm)
 
     def _norm(self, ln: nn.LayerNorm, x: torch.Tensor) -> torch.Tensor:
-        return layer_norm(x, ln.weight, ln.bias, None, self.eps)
+        # Both LayerNorms feed a linear layer (through pure copies), which under autocast rounds
+        # its input to the autocast dtype: asking for that dtype here gives the same numbers
+        # without the fp32 tensor in between.
+        return plain_layer_norm(x, ln.weight, ln.bias, self.eps, out_dtype=_compute_dtype(x))
 
     # The block in stages, so that a single-process harness can run several ranks
     # in lockstep (the two rolls are the only stages that talk to other ranks).
     def pre_attention(self, x: torch.Tensor) -> torch.Tensor:
-        # Under autocast the LayerNorm yields fp32 and the qkv layer would round it to the autocast
-        # dtype; rounding before the roll and the window partition (pure copies) gives the same
-        # numbers and halves the bytes those copies move.
-        return self._norm(self.norm1, x).to(_compute_dtype(x))
+        return self._norm(self.norm1, x)
 
     def shift(self, y: torch.Tensor) -> torch.Tensor:
         return self._roll(y, -self.shift_by)
@@ -201,7 +201,7 @@ class SwinBlock(nn.Module):
 
     def finish(self, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
         x = x + y.to(x.dtype)
-        y = token_linear(self._norm(self.norm2, x).to(x.dtype), self.mlp[0])
+        y = token_linear(self._norm(self.norm2, x), self.mlp[0])
         return x + token_linear(self.mlp[1](y), self.mlp[2])
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:

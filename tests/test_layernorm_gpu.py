@@ -125,3 +125,60 @@ def test_layernorm_bf16_config4_shape(dev):
         y = jl.layer_norm(xs[r].bfloat16().to(dev), ws[r].bfloat16().to(dev), bs[r].bfloat16().to(dev), grp, eps)
         assert y.dtype == torch.bfloat16
         assert rel_l2(y, want.chunk(G, -1)[r]) < 2e-2
+
+
+# --------------------------------------------------------------------------- #
+# nn.LayerNorm over rows one rank holds whole (fused kernels): the oracle with a single shard
+# --------------------------------------------------------------------------- #
+PLAIN_CASES = [
+    # shape, x dtype, out dtype, grad dtype, bias
+    ((1, 256, 256, 128), torch.bfloat16, torch.bfloat16, torch.bfloat16, True),   # Swin block tile, autocast
+    ((3, 70, 128), torch.bfloat16, torch.float32, torch.float32, True),           # torch's autocast dtypes
+    ((5, 33, 8), torch.float32, torch.float32, torch.float32, True),              # one lane per row
+    ((2, 9, 200), torch.float32, torch.float32, torch.float32, False),            # 32 lanes, the last ones idle
+    ((7, 1000), torch.float32, torch.bfloat16, torch.bfloat16, True),             # two chunks per lane
+    ((3, 2048), torch.float16, torch.float16, torch.float16, True),               # widest row the kernels hold
+    ((4, 16, 64), torch.float32, torch.float32, torch.bfloat16, True),            # low-precision gradient
+]
+
+
+@pytest.mark.parametrize("case", PLAIN_CASES, ids=lambda c: f"{'x'.join(map(str, c[0]))}_{str(c[1])[6:]}_{str(c[2])[6:]}")
+def test_plain_layer_norm_matches_oracle(case, dev):
+    shape, xdt, odt, gdt, has_b = case
+    torch.manual_seed(11)
+    C, eps = shape[-1], 1e-5
+    x = (2.0 * torch.randn(*shape) + 0.5).to(xdt)
+    w, b = 1 + 0.2 * torch.randn(C), (0.2 * torch.randn(C) if has_b else None)
+    g = torch.randn(*shape).to(gdt)
+    print(f"plain_layer_norm {case}", flush=True)
+    xr = x.to(dev).requires_grad_()
+    wr = w.to(dev).requires_grad_()
+    br = b.to(dev).requires_grad_() if has_b else None
+    y = jl.plain_layer_norm(xr, wr, br, eps, out_dtype=odt)
+    assert y.dtype == odt and y.shape == x.shape
+    y.backward(g.to(dev))
+    ys, xns, std = ol.forward([x.double()], [w.double()], [b.double() if has_b else None], eps)
+    gxs, gws, gbs = ol.backward([g.double()], xns, [w.double()], std, has_bias=has_b)
+    lo = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 4e-3}
+    assert rel_l2(y.detach().cpu(), ys[0]) < lo[odt]
+    tol_g = max(lo[gdt], lo[xdt])
+    assert xr.grad.dtype == xdt and rel_l2(xr.grad.cpu(), gxs[0]) < tol_g
+    assert wr.grad.dtype == torch.float32 and rel_l2(wr.grad.cpu(), gws[0]) < max(lo[gdt], 1e-5)
+    if has_b:
+        assert rel_l2(br.grad.cpu(), gbs[0]) < max(lo[gdt], 1e-5)
+
+
+def test_plain_layer_norm_defaults_and_fallback(dev):
+    """Default output dtype is torch's (fp32 under autocast); a width the fused kernels do not take
+    (not a multiple of 8) goes through the partial-statistics kernels; no rows is fine."""
+    torch.manual_seed(12)
+    x = torch.randn(4, 50, 128).bfloat16().to(dev)
+    w, b = torch.ones(128, device=dev), torch.zeros(128, device=dev)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        assert jl.plain_layer_norm(x, w, b).dtype == torch.float32
+    assert jl.plain_layer_norm(x, w, b).dtype == torch.bfloat16
+    x2 = torch.randn(6, 130, device=dev)
+    w2, b2 = torch.randn(130, device=dev), torch.randn(130, device=dev)
+    torch.testing.assert_close(jl.plain_layer_norm(x2, w2, b2).cpu(), F.layer_norm(x2.cpu(), (130,), w2.cpu(), b2.cpu()),
+                               atol=1e-5, rtol=1e-5)
+    assert jl.plain_layer_norm(x[:0], w, b).shape == (0, 50, 128)
