@@ -224,26 +224,27 @@ __global__ __launch_bounds__(kThreads) void ln_partial_bwd_kernel(
 }
 
 // Stage 2: a block owns 64 consecutive columns (one per lane, so a partial row is read
-// coalesced); its 4 wavefronts take the block partials k = w, w + 4, ... in 4 independent
-// chains each, and the 16 chain sums are added in a fixed order (deterministic).
-__global__ __launch_bounds__(256) void ln_colreduce_kernel(float* __restrict__ gw,
-                                                           float* __restrict__ gb,
-                                                           const float* __restrict__ part,
-                                                           int nblocks, long long cols) {
-  __shared__ float red[4][2][64];
+// coalesced); its 16 wavefronts take the block partials k = w, w + 16, ... in 4 independent
+// chains each, and the 64 chain sums are added in a fixed order (deterministic).
+constexpr int kReduceWaves = 16;
+__global__ __launch_bounds__(kReduceWaves * 64) void ln_colreduce_kernel(float* __restrict__ gw,
+                                                                         float* __restrict__ gb,
+                                                                         const float* __restrict__ part,
+                                                                         int nblocks, long long cols) {
+  __shared__ float red[kReduceWaves][2][64];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const long long c = (long long)blockIdx.x * 64 + lane;
   float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
   if (c < cols) {
     int k = w;
-    for (; k + 12 < nblocks; k += 16) {
+    for (; k + 3 * kReduceWaves < nblocks; k += 4 * kReduceWaves) {
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        a[u] += part[((long long)(k + 4 * u) * 2 + 0) * cols + c];
-        b[u] += part[((long long)(k + 4 * u) * 2 + 1) * cols + c];
+        a[u] += part[((long long)(k + kReduceWaves * u) * 2 + 0) * cols + c];
+        b[u] += part[((long long)(k + kReduceWaves * u) * 2 + 1) * cols + c];
       }
     }
-    for (; k < nblocks; k += 4) {
+    for (; k < nblocks; k += kReduceWaves) {
       a[0] += part[((long long)k * 2 + 0) * cols + c];
       b[0] += part[((long long)k * 2 + 1) * cols + c];
     }
@@ -252,8 +253,14 @@ __global__ __launch_bounds__(256) void ln_colreduce_kernel(float* __restrict__ g
   red[w][1][lane] = (b[0] + b[1]) + (b[2] + b[3]);
   __syncthreads();
   if (w != 0 || c >= cols) return;
-  if (gw != nullptr) gw[c] = (red[0][0][lane] + red[1][0][lane]) + (red[2][0][lane] + red[3][0][lane]);
-  if (gb != nullptr) gb[c] = (red[0][1][lane] + red[1][1][lane]) + (red[2][1][lane] + red[3][1][lane]);
+  float sw = 0.0f, sb = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kReduceWaves; ++i) {
+    sw += red[i][0][lane];
+    sb += red[i][1][lane];
+  }
+  if (gw != nullptr) gw[c] = sw;
+  if (gb != nullptr) gb[c] = sb;
 }
 
 template <int DT>
@@ -347,7 +354,23 @@ __device__ __forceinline__ float group_sum(float v, int G) {
   return v;
 }
 
-template <int XDT, int YDT, int CH>
+// w (and b) of the columns a lane owns, as 16-byte loads
+template <int CH>
+__device__ __forceinline__ void load_params(float (&dst)[CH][kPlainVec], const float* src, int G, int sl, int cols) {
+#pragma unroll
+  for (int k = 0; k < CH; ++k) {
+    const int c = (k * G + sl) * kPlainVec;
+    if (c < cols && src != nullptr) {
+      load8<JG_F32>(src + c, dst[k]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < kPlainVec; ++i) dst[k][i] = 0.0f;
+    }
+  }
+}
+
+// U rows per lane group are in flight at once (their loads and shuffles interleave).
+template <int XDT, int YDT, int CH, int U>
 __global__ __launch_bounds__(kThreads) void ln_plain_fwd_kernel(
     typename Elem<YDT>::T* __restrict__ y, float* __restrict__ mean, float* __restrict__ rstd,
     const typename Elem<XDT>::T* __restrict__ x, const float* __restrict__ w,
@@ -355,61 +378,70 @@ __global__ __launch_bounds__(kThreads) void ln_plain_fwd_kernel(
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
   const float inv = 1.0f / (float)cols;
+  const long long stride = (long long)gridDim.x * kWavesPerBlock * rpw;
   float wv[CH][kPlainVec], bv[CH][kPlainVec];
+  load_params<CH>(wv, w, G, sl, cols);
+  load_params<CH>(bv, b, G, sl, cols);
+  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows; r0 += stride * U) {
+    float v[U][CH][kPlainVec], m[U], rs[U];
+    bool live[U];
 #pragma unroll
-  for (int k = 0; k < CH; ++k) {
-    const int c = (k * G + sl) * kPlainVec;
+    for (int u = 0; u < U; ++u) {
+      const long long r = r0 + u * stride + sub;
+      live[u] = r < rows;
 #pragma unroll
-    for (int i = 0; i < kPlainVec; ++i) {
-      wv[k][i] = c < cols ? w[c + i] : 0.0f;
-      bv[k][i] = (c < cols && b != nullptr) ? b[c + i] : 0.0f;
-    }
-  }
-  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows;
-       r0 += (long long)gridDim.x * kWavesPerBlock * rpw) {
-    const long long r = r0 + sub;
-    const bool live = r < rows;
-    float v[CH][kPlainVec];
-    float s = 0.0f;
+      for (int k = 0; k < CH; ++k) {
+        const int c = (k * G + sl) * kPlainVec;
+        if (live[u] && c < cols) {
+          load8<XDT>(x + r * cols + c, v[u][k]);
+        } else {
 #pragma unroll
-    for (int k = 0; k < CH; ++k) {
-      const int c = (k * G + sl) * kPlainVec;
-      if (live && c < cols) {
-        load8<XDT>(x + r * cols + c, v[k]);
-      } else {
-#pragma unroll
-        for (int i = 0; i < kPlainVec; ++i) v[k][i] = 0.0f;
-      }
-#pragma unroll
-      for (int i = 0; i < kPlainVec; ++i) s += v[k][i];
-    }
-    const float m = group_sum(s, G) * inv;
-    float q = 0.0f;
-#pragma unroll
-    for (int k = 0; k < CH; ++k) {
-      const int c = (k * G + sl) * kPlainVec;
-      if (c < cols) {
-#pragma unroll
-        for (int i = 0; i < kPlainVec; ++i) {
-          const float d = v[k][i] - m;
-          q += d * d;
+          for (int i = 0; i < kPlainVec; ++i) v[u][k][i] = 0.0f;
         }
       }
     }
-    const float rs = rsqrtf(group_sum(q, G) * inv + eps);
-    if (!live) continue;  // after the shuffles: every lane of the wavefront takes part in them
-    if (sl == 0) {
-      mean[r] = m;
-      rstd[r] = rs;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float s = 0.0f;
+#pragma unroll
+      for (int k = 0; k < CH; ++k)
+#pragma unroll
+        for (int i = 0; i < kPlainVec; ++i) s += v[u][k][i];
+      m[u] = group_sum(s, G) * inv;
     }
 #pragma unroll
-    for (int k = 0; k < CH; ++k) {
-      const int c = (k * G + sl) * kPlainVec;
-      if (c < cols) {
-        float out[kPlainVec];
+    for (int u = 0; u < U; ++u) {
+      float q = 0.0f;
 #pragma unroll
-        for (int i = 0; i < kPlainVec; ++i) out[i] = (v[k][i] - m) * rs * wv[k][i] + bv[k][i];
-        store8<YDT>(y + r * cols + c, out);
+      for (int k = 0; k < CH; ++k) {
+        if ((k * G + sl) * kPlainVec < cols) {
+#pragma unroll
+          for (int i = 0; i < kPlainVec; ++i) {
+            const float d = v[u][k][i] - m[u];
+            q += d * d;
+          }
+        }
+      }
+      rs[u] = rsqrtf(group_sum(q, G) * inv + eps);
+    }
+    // every lane of the wavefront took part in the shuffles above; only now do dead rows drop out
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (!live[u]) continue;
+      const long long r = r0 + u * stride + sub;
+      if (sl == 0) {
+        mean[r] = m[u];
+        rstd[r] = rs[u];
+      }
+#pragma unroll
+      for (int k = 0; k < CH; ++k) {
+        const int c = (k * G + sl) * kPlainVec;
+        if (c < cols) {
+          float out[kPlainVec];
+#pragma unroll
+          for (int i = 0; i < kPlainVec; ++i) out[i] = (v[u][k][i] - m[u]) * rs[u] * wv[k][i] + bv[k][i];
+          store8<YDT>(y + r * cols + c, out);
+        }
       }
     }
   }
@@ -417,7 +449,7 @@ __global__ __launch_bounds__(kThreads) void ln_plain_fwd_kernel(
 
 // gx = rstd * (g w - mean_c(g w) - x_hat * mean_c(g w x_hat)); column partials of g x_hat and g
 // per block in part[blk][which][col] (ln_colreduce_kernel finishes them).
-template <int GDT, int XDT, int CH>
+template <int GDT, int XDT, int CH, int U>
 __global__ __launch_bounds__(kThreads) void ln_plain_bwd_kernel(
     typename Elem<XDT>::T* __restrict__ gx, float* __restrict__ part,
     const typename Elem<GDT>::T* __restrict__ g, const typename Elem<XDT>::T* __restrict__ x,
@@ -426,58 +458,72 @@ __global__ __launch_bounds__(kThreads) void ln_plain_bwd_kernel(
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
   const float inv = 1.0f / (float)cols;
+  const long long stride = (long long)gridDim.x * kWavesPerBlock * rpw;
   float wv[CH][kPlainVec], agw[CH][kPlainVec], agb[CH][kPlainVec];
+  load_params<CH>(wv, w, G, sl, cols);
 #pragma unroll
-  for (int k = 0; k < CH; ++k) {
-    const int c = (k * G + sl) * kPlainVec;
+  for (int k = 0; k < CH; ++k)
 #pragma unroll
     for (int i = 0; i < kPlainVec; ++i) {
-      wv[k][i] = c < cols ? w[c + i] : 0.0f;
       agw[k][i] = 0.0f;
       agb[k][i] = 0.0f;
     }
-  }
-  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows;
-       r0 += (long long)gridDim.x * kWavesPerBlock * rpw) {
-    const long long r = r0 + sub;
-    const bool live = r < rows;
-    const float m = live ? mean[r] : 0.0f, rs = live ? rstd[r] : 0.0f;
-    float gv[CH][kPlainVec], xh[CH][kPlainVec];
-    float s1 = 0.0f, s2 = 0.0f;
+  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows; r0 += stride * U) {
+    float gv[U][CH][kPlainVec], xh[U][CH][kPlainVec], m[U], rs[U], s1[U], s2[U];
+    bool live[U];
 #pragma unroll
-    for (int k = 0; k < CH; ++k) {
-      const int c = (k * G + sl) * kPlainVec;
-      if (live && c < cols) {
-        load8<GDT>(g + r * cols + c, gv[k]);
-        load8<XDT>(x + r * cols + c, xh[k]);
-      } else {
+    for (int u = 0; u < U; ++u) {
+      const long long r = r0 + u * stride + sub;
+      live[u] = r < rows;
+      m[u] = live[u] ? mean[r] : 0.0f;
+      rs[u] = live[u] ? rstd[r] : 0.0f;
 #pragma unroll
-        for (int i = 0; i < kPlainVec; ++i) {
-          gv[k][i] = 0.0f;
-          xh[k][i] = m;
+      for (int k = 0; k < CH; ++k) {
+        const int c = (k * G + sl) * kPlainVec;
+        if (live[u] && c < cols) {
+          load8<GDT>(g + r * cols + c, gv[u][k]);
+          load8<XDT>(x + r * cols + c, xh[u][k]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < kPlainVec; ++i) {
+            gv[u][k][i] = 0.0f;
+            xh[u][k][i] = m[u];
+          }
         }
       }
-#pragma unroll
-      for (int i = 0; i < kPlainVec; ++i) {
-        xh[k][i] = (xh[k][i] - m) * rs;
-        const float gxn = gv[k][i] * wv[k][i];
-        s1 += gxn;
-        s2 += gxn * xh[k][i];
-        agw[k][i] += gv[k][i] * xh[k][i];
-        agb[k][i] += gv[k][i];
-      }
     }
-    s1 = group_sum(s1, G) * inv;
-    s2 = group_sum(s2, G) * inv;
-    if (!live || gx == nullptr) continue;
 #pragma unroll
-    for (int k = 0; k < CH; ++k) {
-      const int c = (k * G + sl) * kPlainVec;
-      if (c < cols) {
-        float out[kPlainVec];
+    for (int u = 0; u < U; ++u) {
+      float a1 = 0.0f, a2 = 0.0f;
 #pragma unroll
-        for (int i = 0; i < kPlainVec; ++i) out[i] = rs * (gv[k][i] * wv[k][i] - s1 - xh[k][i] * s2);
-        store8<XDT>(gx + r * cols + c, out);
+      for (int k = 0; k < CH; ++k)
+#pragma unroll
+        for (int i = 0; i < kPlainVec; ++i) {
+          xh[u][k][i] = (xh[u][k][i] - m[u]) * rs[u];
+          const float gxn = gv[u][k][i] * wv[k][i];
+          a1 += gxn;
+          a2 += gxn * xh[u][k][i];
+          agw[k][i] += gv[u][k][i] * xh[u][k][i];
+          agb[k][i] += gv[u][k][i];
+        }
+      s1[u] = group_sum(a1, G) * inv;
+      s2[u] = group_sum(a2, G) * inv;
+    }
+    if (gx == nullptr) continue;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (!live[u]) continue;
+      const long long r = r0 + u * stride + sub;
+#pragma unroll
+      for (int k = 0; k < CH; ++k) {
+        const int c = (k * G + sl) * kPlainVec;
+        if (c < cols) {
+          float out[kPlainVec];
+#pragma unroll
+          for (int i = 0; i < kPlainVec; ++i)
+            out[i] = rs[u] * (gv[u][k][i] * wv[k][i] - s1[u] - xh[u][k][i] * s2[u]);
+          store8<XDT>(gx + r * cols + c, out);
+        }
       }
     }
   }
@@ -539,15 +585,15 @@ void launch_plain_fwd(void* y, float* mean, float* rstd, const void* x, const fl
                       long long rows, int cols, float eps, hipStream_t s) {
   typedef typename Elem<XDT>::T XT;
   typedef typename Elem<YDT>::T YT;
-  const int G = plain_group(cols), blocks = plain_blocks(rows, cols) * 4 > 65536 ? 65536 : plain_blocks(rows, cols) * 4;
-#define JG_GO(CH)                                                                                   \
-  ln_plain_fwd_kernel<XDT, YDT, CH><<<blocks, kThreads, 0, s>>>(static_cast<YT*>(y), mean, rstd,     \
-                                                                static_cast<const XT*>(x), w, b, rows, cols, eps, G)
+  const int G = plain_group(cols), blocks = plain_blocks(rows, cols);
+#define JG_GO(CH, U)                                                                                   \
+  ln_plain_fwd_kernel<XDT, YDT, CH, U><<<blocks, kThreads, 0, s>>>(static_cast<YT*>(y), mean, rstd,     \
+                                                                   static_cast<const XT*>(x), w, b, rows, cols, eps, G)
   switch (plain_chunks(cols)) {
-    case 1: JG_GO(1); break;
-    case 2: JG_GO(2); break;
-    case 3: JG_GO(3); break;
-    default: JG_GO(4); break;
+    case 1: JG_GO(1, 2); break;
+    case 2: JG_GO(2, 2); break;
+    case 3: JG_GO(3, 1); break;
+    default: JG_GO(4, 1); break;
   }
 #undef JG_GO
 }
@@ -558,16 +604,16 @@ void launch_plain_bwd(void* gx, float* part, const void* g, const void* x, const
   typedef typename Elem<GDT>::T GT;
   typedef typename Elem<XDT>::T XT;
   const int G = plain_group(cols), blocks = plain_blocks(rows, cols);
-#define JG_GO(CH)                                                                                     \
-  ln_plain_bwd_kernel<GDT, XDT, CH><<<blocks, kThreads, 0, s>>>(static_cast<XT*>(gx), part,            \
-                                                                static_cast<const GT*>(g),             \
-                                                                static_cast<const XT*>(x), mean, rstd, \
-                                                                w, rows, cols, G, want_cols)
+#define JG_GO(CH, U)                                                                                     \
+  ln_plain_bwd_kernel<GDT, XDT, CH, U><<<blocks, kThreads, 0, s>>>(static_cast<XT*>(gx), part,            \
+                                                                   static_cast<const GT*>(g),             \
+                                                                   static_cast<const XT*>(x), mean, rstd, \
+                                                                   w, rows, cols, G, want_cols)
   switch (plain_chunks(cols)) {
-    case 1: JG_GO(1); break;
-    case 2: JG_GO(2); break;
-    case 3: JG_GO(3); break;
-    default: JG_GO(4); break;
+    case 1: JG_GO(1, 2); break;
+    case 2: JG_GO(2, 2); break;
+    case 3: JG_GO(3, 1); break;
+    default: JG_GO(4, 1); break;
   }
 #undef JG_GO
 }
@@ -692,7 +738,7 @@ extern "C" int jg_ln_partial_bwd(float* mean_gxn, float* dot_gxn_xhat, float* gw
   if (rc) return rc;
   JG_CHECK_LAUNCH("jg_ln_partial_bwd");
   if (want_cols) {
-    ln_colreduce_kernel<<<jg::cdiv(cols, 64), 256, 0, s>>>(gw, gb, part, bwd_blocks(rows), cols);
+    ln_colreduce_kernel<<<jg::cdiv(cols, 64), kReduceWaves * 64, 0, s>>>(gw, gb, part, bwd_blocks(rows), cols);
     JG_CHECK_LAUNCH("jg_ln_partial_bwd(colreduce)");
   }
   return JG_OK;
@@ -740,7 +786,7 @@ extern "C" int jg_ln_plain_fwd(void* y, float* mean, float* rstd, const void* x,
   if (!plain_ok(cols))
     JG_FAIL(JG_ERR_UNSUPPORTED, "%s: %lld columns (needs a multiple of 8, at most %d)", who, (long long)cols,
             kPlainChunks * kWave * kPlainVec);
-  JG_REQUIRE(aligned16(y) && aligned16(x), "%s: x and y must be 16-byte aligned", who);
+  JG_REQUIRE(aligned16(y) && aligned16(x) && aligned16(w) && aligned16(b), "%s: x, y, w and b must be 16-byte aligned", who);
   JG_REQUIRE(y_dtype == x_dtype || y_dtype == JG_F32 || x_dtype == JG_F32, "%s: x dtype %d with y dtype %d", who,
              x_dtype, y_dtype);
   if (rows == 0) return JG_OK;
@@ -778,8 +824,8 @@ extern "C" int jg_ln_plain_bwd(void* gx, float* gw, float* gb, const void* g, co
   if (!plain_ok(cols))
     JG_FAIL(JG_ERR_UNSUPPORTED, "%s: %lld columns (needs a multiple of 8, at most %d)", who, (long long)cols,
             kPlainChunks * kWave * kPlainVec);
-  JG_REQUIRE(aligned16(g) && aligned16(x) && (gx == nullptr || aligned16(gx)), "%s: g, x and gx must be 16-byte aligned",
-             who);
+  JG_REQUIRE(aligned16(g) && aligned16(x) && aligned16(w) && (gx == nullptr || aligned16(gx)),
+             "%s: g, x, w and gx must be 16-byte aligned", who);
   JG_REQUIRE(g_dtype == x_dtype || g_dtype == JG_F32 || x_dtype == JG_F32, "%s: g dtype %d with x dtype %d", who,
              g_dtype, x_dtype);
   const bool want_cols = gw != nullptr || gb != nullptr;
@@ -787,7 +833,7 @@ extern "C" int jg_ln_plain_bwd(void* gx, float* gw, float* gb, const void* g, co
   if (rows == 0) {
     // no rows: the column sums are zero (a fill kernel, so that the call can be captured in a graph)
     if (want_cols) {
-      ln_colreduce_kernel<<<(unsigned)((cols + 63) / 64), 256, 0, s>>>(gw, gb, nullptr, 0, cols);
+      ln_colreduce_kernel<<<(unsigned)((cols + 63) / 64), kReduceWaves * 64, 0, s>>>(gw, gb, nullptr, 0, cols);
       JG_CHECK_LAUNCH(who);
     }
     return JG_OK;
@@ -813,7 +859,7 @@ extern "C" int jg_ln_plain_bwd(void* gx, float* gw, float* gb, const void* g, co
 #undef JG_GO
   JG_CHECK_LAUNCH(who);
   if (want_cols) {
-    ln_colreduce_kernel<<<(unsigned)((cols + 63) / 64), 256, 0, s>>>(gw, gb, part, plain_blocks(rows, cols), cols);
+    ln_colreduce_kernel<<<(unsigned)((cols + 63) / 64), kReduceWaves * 64, 0, s>>>(gw, gb, part, plain_blocks(rows, cols), cols);
     JG_CHECK_LAUNCH(who);
   }
   return JG_OK;
