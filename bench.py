@@ -290,7 +290,11 @@ def swin_figures(dev, iters: int) -> dict:
     x = torch.randn(1, *n, dim, device=dev, generator=g).bfloat16().requires_grad_()
     gout = torch.randn(1, *n, dim, device=dev, generator=g).bfloat16()
 
+    leaves = [x, *block.parameters()]
+
     def step():
+        for t in leaves:  # what optimizer.zero_grad() does: the backward then assigns instead of adding
+            t.grad = None
         with torch.autocast("cuda", dtype=torch.bfloat16):
             y = block(x)
         y.backward(gout)

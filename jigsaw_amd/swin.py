@@ -134,6 +134,10 @@ class WindowAttention(nn.Module):
         self.bias_table = nn.Parameter(torch.zeros((2 * window - 1) ** 2, heads, device=device))
         nn.init.trunc_normal_(self.bias_table, std=0.02)
         self.register_buffer("index", relative_position_index(window).to(device), persistent=False)
+        # The gather bias_table[index] as a product with a one-hot matrix (N*N, table rows): the same
+        # numbers (1 * v plus zeros), and its backward is a small GEMM instead of a sorted scatter-add.
+        onehot = torch.nn.functional.one_hot(self.index.view(-1), (2 * window - 1) ** 2).to(torch.float32)
+        self.register_buffer("onehot", onehot, persistent=False)
         if shift:
             self.register_buffer("mask", shift_mask(*tile, window, shift, groups).to(device), persistent=False)
         else:
@@ -149,7 +153,8 @@ class WindowAttention(nn.Module):
         else:
             qkv = token_linear(x, self.qkv).view(b, -1, n, 3, self.heads, c // self.heads)
             q, k, v = (t.contiguous() for t in qkv.permute(3, 0, 1, 4, 2, 5).unbind(0))  # (B, nW, heads, N, d)
-        bias = self.bias_table[self.index.view(-1)].view(n, n, -1).permute(2, 0, 1).float()
+        with torch.autocast("cuda", enabled=False):
+            bias = (self.onehot @ self.bias_table.float()).view(n, n, -1).permute(2, 0, 1)
         if self.mask is not None:
             bias = bias[None] + self.mask[:, None]  # (nW, heads, N, N)
         out = window_attention(q, k, v, bias.contiguous())
