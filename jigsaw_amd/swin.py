@@ -3,12 +3,13 @@
 Mirrors the example model of the reference (examples/swin.py:64-210): tokens are
 channels-last ``(B, h, w, C)`` tiles of a 2-D token grid; a block is
 ``x + unshift(attn(shift(norm1(x))))`` followed by ``x + mlp(norm2(x))``. The
-LayerNorms run on the sharded-LayerNorm kernels (with a channel group of one), the
-shift / unshift on the DistributedRoll kernels, the windowed attention with its
+LayerNorms (not sharded in the example) run on the fused unsharded-LayerNorm kernels,
+the shift / unshift on the DistributedRoll kernels, the windowed attention with its
 relative-position bias and shift mask on the attention core with an additive
-bias. The linear layers are ``nn.Linear`` parameters (as in the reference example)
-applied through the library GEMMs; only the weight gradient is arranged differently
-(split over the tokens), because its output is a few tiles and its contraction 65536 long.
+bias. The linear layers are ``nn.Linear`` parameters (as in the reference example);
+in bf16 they run on this package's projection GEMMs (head split / merge and bias
+gradient fused in), otherwise through the library GEMMs with the weight gradient split
+over the tokens, because its output is a few tiles and its contraction 65536 long.
 """
 
 from __future__ import annotations
