@@ -293,11 +293,13 @@ int jg_proj_nt(void* out, const void* a, const void* w, const void* bias, int dt
 /* gw[n][c] = sum_r g(r, n) * x(r, c)  (n, c) row-major, and gb[n] = sum_r g(r, n)
  * (gb may be NULL): weight and bias gradient of a projection (torch's
  * Linear backward; g = grad of the projection's output, x = its input).
+ * gw and gb have dtype grad_dtype: `dtype`, or JG_F32 (fp32 parameters under
+ * autocast: the fp32 sums are stored without a rounding to the operands' dtype).
  * workspace: jg_proj_tn_workspace(rows, n, c) bytes of device scratch (partial
  * sums per token range, added up in a fixed order: deterministic). */
 size_t jg_proj_tn_workspace(int64_t rows, int n, int c);
-int jg_proj_tn(void* gw, void* gb, const void* g, const void* x, int dtype, int64_t rows,
-               int n, int c, int g_heads, int x_heads, int B, int H, int S, int D,
+int jg_proj_tn(void* gw, void* gb, const void* g, const void* x, int dtype, int grad_dtype,
+               int64_t rows, int n, int c, int g_heads, int x_heads, int B, int H, int S, int D,
                void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------- *

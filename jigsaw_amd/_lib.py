@@ -148,7 +148,7 @@ SIGNATURES: dict[str, tuple] = {
     "jg_proj_tn_workspace": (c_size_t, [c_int64, c_int, c_int]),
     "jg_proj_tn": (
         c_int,
-        [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
          c_int, c_void_p, c_size_t, c_void_p],
     ),
     "jg_conv_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int, c_int]),

@@ -448,7 +448,7 @@ def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, group
             nb = int(lib.jg_proj_tn_workspace(rows, weight_shape[0], k))
             pws = torch.empty(max(nb, 16), dtype=torch.uint8, device=x.device)
             rc = lib.jg_proj_tn(_lib.ptr(gw2), _lib.ptr(gb), _lib.ptr(g_tok), _lib.ptr(patches), _lib.dtype_code(x.dtype),
-                                rows, weight_shape[0], k, 0, 0, 1, 1, 1, 1, _lib.ptr(pws), nb, _lib.stream_ptr(x.device))
+                                _lib.dtype_code(x.dtype), rows, weight_shape[0], k, 0, 0, 1, 1, 1, 1, _lib.ptr(pws), nb, _lib.stream_ptr(x.device))
             _lib.check(rc, "jg_proj_tn")
         else:
             gw2.zero_()

@@ -465,27 +465,28 @@ __global__ __launch_bounds__(64 * WM * WN) void proj_tn_kernel(TnParams p) {
 // and its four wavefronts each add every fourth split; the four sums are then added in a fixed
 // order, so the result does not depend on scheduling.
 struct ReduceArgs {
-  uint16_t* out_w;
+  void* out_w;
   const float* part_w;
   size_t count_w;
-  uint16_t* out_b;  // NULL: no bias gradient
+  void* out_b;  // NULL: no bias gradient
   const float* part_b;
   size_t count_b;
   int splits;
+  int out32;  // write fp32 instead of bf16
 };
 
 __global__ __launch_bounds__(256) void proj_reduce_kernel(ReduceArgs a) {
   __shared__ f32x4 sm[4][64];
   const size_t blocks_w = (a.count_w + 255) / 256;
   const bool second = blockIdx.x >= blocks_w;
-  uint16_t* out = second ? a.out_b : a.out_w;
+  void* out_any = second ? a.out_b : a.out_w;
   const float* part = second ? a.part_b : a.part_w;
   const size_t count = second ? a.count_b : a.count_w;
   const int q = threadIdx.x & 63, grp = threadIdx.x >> 6;
   const size_t i0 = (blockIdx.x - (second ? blocks_w : 0)) * 256 + (size_t)q * 4;
   // every split's slice starts 16-byte aligned when the count is a multiple of 4 and the base is aligned
   const bool vec = (count & 3) == 0 && (reinterpret_cast<uintptr_t>(part) & 15) == 0 &&
-                   (reinterpret_cast<uintptr_t>(out) & 7) == 0;
+                   (reinterpret_cast<uintptr_t>(out_any) & 15) == 0;
   f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
   if (i0 < count) {
     if (vec) {
@@ -501,6 +502,18 @@ __global__ __launch_bounds__(256) void proj_reduce_kernel(ReduceArgs a) {
   __syncthreads();
   if (grp != 0 || i0 >= count) return;
   const f32x4 t = ((sm[0][q] + sm[1][q]) + sm[2][q]) + sm[3][q];
+  if (a.out32) {
+    float* o32 = static_cast<float*>(out_any);
+    if (vec) {
+      *reinterpret_cast<f32x4*>(o32 + i0) = t;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (i0 + e < count) o32[i0 + e] = t[e];
+    }
+    return;
+  }
+  uint16_t* out = static_cast<uint16_t*>(out_any);
   if (vec) {
     u32x2 o;
     o.x = (uint32_t)jg::f32_to_bf16(t[0]) | ((uint32_t)jg::f32_to_bf16(t[1]) << 16);
@@ -544,6 +557,7 @@ struct GenParams {
   long long I;     // NT: tokens; TN: features of g
   int J;
   long long L;     // contraction length: NT: K; TN: tokens
+  int out32;       // TN: write fp32 whatever the operands' dtype
 };
 
 // out(i, j) = sum_l P(i, l) * Q(j, l): 16 x 16 outputs per workgroup, the operands pass
@@ -583,7 +597,8 @@ __global__ __launch_bounds__(256) void proj_generic_kernel(GenParams p) {
   if (i >= p.I || j >= p.J) return;
   T* out = static_cast<T*>(p.out);
   if (TRANS) {
-    out[i * p.J + j] = Elem<DT>::down(acc);
+    if (p.out32) static_cast<float*>(p.out)[i * p.J + j] = acc;
+    else out[i * p.J + j] = Elem<DT>::down(acc);
   } else {
     if (p.bias != nullptr) acc += Elem<DT>::up(static_cast<const T*>(p.bias)[j]);
     out[row_part(p.om, i) + feat_part(p.om, j)] = Elem<DT>::down(acc);
@@ -592,7 +607,7 @@ __global__ __launch_bounds__(256) void proj_generic_kernel(GenParams p) {
 
 // gb[n] = sum over the tokens of g(r, n): one workgroup per feature, fixed order
 template <int DT>
-__global__ __launch_bounds__(256) void proj_colsum_kernel(void* gb, const void* g, Map gm, long long rows) {
+__global__ __launch_bounds__(256) void proj_colsum_kernel(void* gb, const void* g, Map gm, long long rows, bool out32) {
   typedef typename Elem<DT>::T T;
   __shared__ float red[256];
   const int n = blockIdx.x;
@@ -605,7 +620,10 @@ __global__ __launch_bounds__(256) void proj_colsum_kernel(void* gb, const void* 
     if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
     __syncthreads();
   }
-  if (threadIdx.x == 0) static_cast<T*>(gb)[n] = Elem<DT>::down(red[0]);
+  if (threadIdx.x == 0) {
+    if (out32) static_cast<float*>(gb)[n] = red[0];
+    else static_cast<T*>(gb)[n] = Elem<DT>::down(red[0]);
+  }
 }
 
 // --------------------------------------------------------------------- host
@@ -708,6 +726,7 @@ int jg_proj_nt(void* out, const void* a, const void* w, const void* bias, int dt
     gp.p = a; gp.q = w; gp.bias = bias; gp.out = out;
     gp.pm = am; gp.qm = am; gp.om = om;
     gp.I = rows; gp.J = n_out; gp.L = k_in;
+    gp.out32 = 0;
     return launch_generic<false>(gp, dtype, s, who);
   }
   NtParams p;
@@ -729,11 +748,15 @@ size_t jg_proj_tn_workspace(int64_t rows, int n, int c) {
   return splits * ((size_t)n * c + n) * sizeof(float);
 }
 
-int jg_proj_tn(void* gw, void* gb, const void* g, const void* x, int dtype, int64_t rows, int n, int c, int g_heads,
-               int x_heads, int B, int H, int S, int D, void* workspace, size_t workspace_bytes, void* stream) {
+int jg_proj_tn(void* gw, void* gb, const void* g, const void* x, int dtype, int grad_dtype, int64_t rows, int n, int c,
+               int g_heads, int x_heads, int B, int H, int S, int D, void* workspace, size_t workspace_bytes,
+               void* stream) {
   const char* who = "jg_proj_tn";
   JG_REQUIRE(gw && g && x, "%s: null pointer", who);
   JG_REQUIRE(jg::dtype_size(dtype) != 0, "%s: unknown dtype %d", who, dtype);
+  JG_REQUIRE(grad_dtype == dtype || grad_dtype == JG_F32, "%s: gradient dtype %d with operand dtype %d", who, grad_dtype,
+             dtype);
+  const bool out32 = grad_dtype == JG_F32 && dtype != JG_F32;
   JG_REQUIRE(rows > 0 && n > 0 && c > 0, "%s: bad sizes rows=%lld n=%d c=%d", who, (long long)rows, n, c);
   Map gm, xm;
   int rc = make_map(&gm, g_heads, n, rows, B, H, S, D, who, "gradient");
@@ -748,13 +771,14 @@ int jg_proj_tn(void* gw, void* gb, const void* g, const void* x, int dtype, int6
     gp.p = g; gp.q = x; gp.bias = nullptr; gp.out = gw;
     gp.pm = gm; gp.qm = xm; gp.om = gm;
     gp.I = n; gp.J = c; gp.L = rows;
+    gp.out32 = out32 ? 1 : 0;
     rc = launch_generic<true>(gp, dtype, s, who);
     if (rc) return rc;
     if (gb != nullptr) {
       switch (dtype) {
-        case JG_F32: proj_colsum_kernel<JG_F32><<<n, 256, 0, s>>>(gb, g, gm, rows); break;
-        case JG_BF16: proj_colsum_kernel<JG_BF16><<<n, 256, 0, s>>>(gb, g, gm, rows); break;
-        default: proj_colsum_kernel<JG_F16><<<n, 256, 0, s>>>(gb, g, gm, rows); break;
+        case JG_F32: proj_colsum_kernel<JG_F32><<<n, 256, 0, s>>>(gb, g, gm, rows, out32); break;
+        case JG_BF16: proj_colsum_kernel<JG_BF16><<<n, 256, 0, s>>>(gb, g, gm, rows, out32); break;
+        default: proj_colsum_kernel<JG_F16><<<n, 256, 0, s>>>(gb, g, gm, rows, out32); break;
       }
       JG_CHECK_LAUNCH(who);
     }
@@ -777,13 +801,14 @@ int jg_proj_tn(void* gw, void* gb, const void* g, const void* x, int dtype, int6
   rc = tn_tile(rows, n, c) == 256 ? launch_tn<4, 2, 2, 4>(p, splits, s, who) : launch_tn<2, 2, 2, 2>(p, splits, s, who);
   if (rc) return rc;
   ReduceArgs ra{};
-  ra.out_w = static_cast<uint16_t*>(gw);
+  ra.out_w = gw;
   ra.part_w = p.part;
   ra.count_w = (size_t)n * c;
-  ra.out_b = static_cast<uint16_t*>(gb);
+  ra.out_b = gb;
   ra.part_b = p.bias_part;
   ra.count_b = gb != nullptr ? (size_t)n : 0;
   ra.splits = splits;
+  ra.out32 = out32 ? 1 : 0;
   const size_t blocks = (ra.count_w + 255) / 256 + (ra.count_b + 255) / 256;
   proj_reduce_kernel<<<(unsigned)blocks, 256, 0, s>>>(ra);
   JG_CHECK_LAUNCH(who);

@@ -33,14 +33,21 @@ def _nt(out, a, w, bias, rows, n_out, k_in, a_heads, out_heads, dims) -> None:
     _lib.check(rc, "jg_proj_nt")
 
 
-def _tn(g, x, rows, n, c, g_heads, x_heads, dims, want_bias):
+def _grad_dtype(compute: torch.dtype, dtypes) -> torch.dtype:
+    """fp32 when every parameter that gets a gradient is fp32 (autocast), else the compute dtype."""
+    return torch.float32 if all(dt in (None, torch.float32) for dt in dtypes) else compute
+
+
+def _tn(g, x, rows, n, c, g_heads, x_heads, dims, want_bias, grad_dtype=None):
     lib = _lib.load()
     b, h, s, d = dims
-    gw = torch.empty(n, c, dtype=g.dtype, device=g.device)
-    gb = torch.empty(n, dtype=g.dtype, device=g.device) if want_bias else None
+    gdt = grad_dtype or g.dtype
+    gw = torch.empty(n, c, dtype=gdt, device=g.device)
+    gb = torch.empty(n, dtype=gdt, device=g.device) if want_bias else None
     nbytes = int(lib.jg_proj_tn_workspace(rows, n, c))
     ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=g.device)
-    rc = lib.jg_proj_tn(_lib.ptr(gw), _lib.ptr(gb), _lib.ptr(g), _lib.ptr(x), _lib.dtype_code(g.dtype), rows, n, c,
+    rc = lib.jg_proj_tn(_lib.ptr(gw), _lib.ptr(gb), _lib.ptr(g), _lib.ptr(x), _lib.dtype_code(g.dtype),
+                        _lib.dtype_code(gdt), rows, n, c,
                         int(g_heads), int(x_heads), b, h, s, d, _lib.ptr(ws), nbytes, _lib.stream_ptr(g.device))
     _lib.check(rc, "jg_proj_tn")
     return gw, gb
@@ -91,7 +98,7 @@ class _QkvProjection(torch.autograd.Function):
                 _nt(gx, g, w.t().contiguous(), None, b * s, c, n_out, True, False, ctx.dims)
             need_b = ctx.has_bias and ctx.needs_input_grad[2]
             if ctx.needs_input_grad[1] or need_b:
-                gw, gb = _tn(g, xc, b * s, n_out, c, True, False, ctx.dims, need_b)
+                gw, gb = _tn(g, xc, b * s, n_out, c, True, False, ctx.dims, need_b, _grad_dtype(g.dtype, ctx.dtypes))
         dt_w, dt_b = ctx.dtypes
         return (gx, None if gw is None or not ctx.needs_input_grad[1] else gw.to(dt_w),
                 None if gb is None else gb.to(dt_b), None)
@@ -140,7 +147,7 @@ class _HeadsProjection(torch.autograd.Function):
                 _nt(go, g, w.t().contiguous(), None, b * s, k, n_out, False, True, ctx.dims)
             need_b = ctx.has_bias and ctx.needs_input_grad[2]
             if ctx.needs_input_grad[1] or need_b:
-                gw, gb = _tn(g, oc, b * s, n_out, k, False, True, ctx.dims, need_b)
+                gw, gb = _tn(g, oc, b * s, n_out, k, False, True, ctx.dims, need_b, _grad_dtype(g.dtype, ctx.dtypes))
         dt_w, dt_b = ctx.dtypes
         return (go, None if gw is None or not ctx.needs_input_grad[1] else gw.to(dt_w),
                 None if gb is None else gb.to(dt_b))
@@ -185,7 +192,7 @@ class _Linear(torch.autograd.Function):
                 gx = torch.empty_like(xc)
                 _nt(gx, g, w.t().contiguous(), None, rows, k, n_out, False, False, (1, 1, 1, 1))
             if ctx.needs_input_grad[1] or need_b:
-                gw, gb = _tn(g, xc, rows, n_out, k, False, False, (1, 1, 1, 1), need_b)
+                gw, gb = _tn(g, xc, rows, n_out, k, False, False, (1, 1, 1, 1), need_b, _grad_dtype(g.dtype, ctx.dtypes))
         dt_w, dt_b = ctx.dtypes
         return (gx, None if gw is None or not ctx.needs_input_grad[1] else gw.to(dt_w),
                 None if gb is None else gb.to(dt_b))

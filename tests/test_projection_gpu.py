@@ -159,3 +159,21 @@ def test_linear_matches_oracle(shape, n_out, dtype, has_b, dev):
             assert rel_l2(bd.grad.cpu(), gb) <= tol
     else:
         assert float(wd.grad.abs().sum()) == 0.0 and xd.grad.shape == x.shape
+
+
+@pytest.mark.parametrize("shape,n_out", [((4, 64, 128), 256), ((3, 50, 20), 12)], ids=["mfma", "fma"])
+def test_fp32_parameters_get_unrounded_fp32_gradients(shape, n_out, dev):
+    """fp32 parameters with bf16 activations (autocast): the weight and bias gradients come back in
+    fp32 straight from the fp32 sums, closer to the oracle than one bf16 rounding allows."""
+    torch.manual_seed(6)
+    k = shape[-1]
+    x = torch.randn(*shape).bfloat16()
+    w, b = torch.randn(n_out, k) / k ** 0.5, 0.1 * torch.randn(n_out)
+    g = torch.randn(*shape[:-1], n_out).bfloat16()
+    xd = x.to(dev).requires_grad_()
+    wd, bd = w.to(dev).requires_grad_(), b.to(dev).requires_grad_()
+    jp.linear(xd, wd, bd).backward(g.to(dev))
+    assert wd.grad.dtype == torch.float32 and bd.grad.dtype == torch.float32
+    x3 = x.reshape(1, 1, -1, k).double()
+    _, gw, gb = op.heads_backward(g.reshape(1, -1, n_out).double(), x3, w.bfloat16().double())
+    assert rel_l2(wd.grad.cpu(), gw) < 1e-5 and rel_l2(bd.grad.cpu(), gb) < 1e-5
