@@ -91,7 +91,7 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_mfma_kernel(FwdArgs p) {
   // ---- tile prefetch: K rows copied, V rows transposed to [dv][key position]
   u32x4 kst[2];
   uint32_t vst[8];
-  const int k_row0 = th >> 3, k_c16 = th & 7;          // K chunk of round 0 (round 1: +32 rows)
+  const int k_row0 = th >> 3, k_c16 = th & 7;          // K chunk of the first pass (second pass: +32 rows)
   const int v_g8 = th >> 5, v_dvp = th & 31;           // V task: 8 keys x 2 dv
   auto issue_loads = [&](int t) {
     const uint16_t* kt = kbase + (long long)t * BN * D;
