@@ -300,7 +300,7 @@ def backward(grad_out, q, k, v, out, logsumexp, scale, *args, dropout_p=0.0, see
 # --------------------------------------------------------------------------- #
 def _fused_ok(q, k) -> bool:
     return (
-        q.dtype == torch.bfloat16 and q.shape[-1] == 64 and q.shape[-2] % 128 == 0 and k.shape[-2] % 128 == 0
+        q.dtype == torch.bfloat16 and q.shape[-1] in (64, 96, 128) and q.shape[-2] % 128 == 0 and k.shape[-2] % 128 == 0
     )
 
 

@@ -25,7 +25,7 @@ int attn_mfma_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q,
                   int sk, float scale, void* ws, hipStream_t s);
 bool attn_wide_supported(long long batch, int sq, int sk, int d, int dtype, bool has_bias);
 int attn_wide_fwd(void* out, float* lse, const void* q, const void* k, const void* v, long long batch,
-                  int sq, int sk, int d, float scale, hipStream_t s);
+                  int sq, int sk, int d, float scale, float* out_acc, float* lse_acc, hipStream_t s);
 int attn_wide_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q, const void* k,
                   const void* v, const void* out, const float* lse, long long batch, int sq, int sk,
                   int d, float scale, void* ws, hipStream_t s);
@@ -76,10 +76,9 @@ extern "C" int jg_attn_fwd(void* out, float* lse, const void* q, const void* k, 
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (jg::attn_mfma_fwd_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr))
     return jg::attn_mfma_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, scale, out_acc, lse_acc, s);
-  if (out_acc == nullptr &&
-      jg::attn_wide_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr) &&
-      aligned16({out, q, k, v}))
-    return jg::attn_wide_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, (int)d, scale, s);
+  if (jg::attn_wide_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr) &&
+      aligned16({out, q, k, v, out_acc}))
+    return jg::attn_wide_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, (int)d, scale, out_acc, lse_acc, s);
   if (out_acc == nullptr && jg::attn_window_supported(batch, (int)sq, (int)sk, (int)d, dtype) &&
       aligned16({out, q, k, v, bias}))
     return jg::attn_window_fwd(out, lse, q, k, v, batch, scale, bias, bias_period, s);
@@ -87,7 +86,7 @@ extern "C" int jg_attn_fwd(void* out, float* lse, const void* q, const void* k, 
     JG_FAIL(JG_ERR_UNSUPPORTED, "%s: head size %lld not in {8, 16, 32, 64, 96, 128}", who, (long long)d);
   if (out_acc != nullptr)
     JG_FAIL(JG_ERR_UNSUPPORTED,
-            "%s: the fused merge needs the MFMA path (bf16, d = 64, sq %% 128 == 0, sk %% 128 == 0);"
+            "%s: the fused merge needs an MFMA path (bf16, d in {64, 96, 128}, sq %% 128 == 0, sk %% 128 == 0);"
             " call jg_lse_merge after the core instead", who);
   rc = jg::attn_generic_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, (int)d, scale, bias,
                             bias_period, dtype, s);

@@ -147,8 +147,10 @@ struct Args {
   const uint16_t* dout;  // backward
   const float* lse_in;   // backward: the global lse
   float* delta;          // backward workspace (batch, sq): written by the dQ kernel, read by the dK/dV kernel
-  uint16_t* o;           // forward output
-  float* lse;            // forward output
+  uint16_t* o;           // forward output, or NULL when only the merge is wanted
+  float* lse;            // forward output, or NULL
+  float* out_acc;        // forward: fp32 (batch, sq, d) accumulator of the ring, merged in place, or NULL
+  float* lse_acc;        // forward: fp32 (batch, sq), merged in place, or NULL
   uint16_t* dq;
   uint16_t* dk;
   uint16_t* dv;
@@ -241,15 +243,37 @@ __global__ __launch_bounds__(THREADS) void attn_wide_fwd_kernel(Args p) {
   // the two lanes of a query saw the same maxima; their sums cover disjoint keys
   l += __shfl_xor(l, 32, 64);
   const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-  uint16_t* orow = p.o + (bh * p.sq + qi) * D;
+  const float lse_j = l > 0.0f ? m * p.scale + __logf(l) : -INFINITY;
+  const long long row = bh * p.sq + qi;
+  // Ring merge (the reference's _online_softmax_merge_): w = sigmoid(lse_j - lse), out += w (out_j - out),
+  // lse = logaddexp(lse, lse_j), with out_j rounded to the core's output dtype first as the unfused path has it.
+  float w = 0.0f;
+  if (p.out_acc != nullptr) {
+    const float l_old = p.lse_acc[row];  // both lanes of the query read it before lane kg = 0 writes
+    w = 1.0f / (1.0f + __expf(l_old - lse_j));  // l_old = -inf -> 1
+    if (kg == 0) p.lse_acc[row] = fmaxf(l_old, lse_j) + log1pf(__expf(-fabsf(l_old - lse_j)));
+  }
+  if (p.lse != nullptr && kg == 0) p.lse[row] = lse_j;
   // register i of block nb: output column nb*32 + 8*(i/4) + 4*kg + i%4
 #pragma unroll
   for (int nb = 0; nb < G::NB; ++nb)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      *reinterpret_cast<u32x2*>(orow + nb * 32 + 8 * j + 4 * kg) =
-          pack4(o[nb][4 * j] * inv, o[nb][4 * j + 1] * inv, o[nb][4 * j + 2] * inv, o[nb][4 * j + 3] * inv);
-  if (kg == 0) p.lse[bh * p.sq + qi] = l > 0.0f ? m * p.scale + __logf(l) : -INFINITY;
+    for (int j = 0; j < 4; ++j) {
+      const int dv = nb * 32 + 8 * j + 4 * kg;
+      const u32x2 h = pack4(o[nb][4 * j] * inv, o[nb][4 * j + 1] * inv, o[nb][4 * j + 2] * inv, o[nb][4 * j + 3] * inv);
+      if (p.o != nullptr) *reinterpret_cast<u32x2*>(p.o + row * D + dv) = h;
+      if (p.out_acc != nullptr) {
+        f32x4* dst = reinterpret_cast<f32x4*>(p.out_acc + row * D + dv);
+        f32x4 a = *dst;
+        const float h0 = __uint_as_float(h.x << 16), h1 = __uint_as_float(h.x & 0xffff0000u);
+        const float h2 = __uint_as_float(h.y << 16), h3 = __uint_as_float(h.y & 0xffff0000u);
+        a.x += w * (h0 - a.x);
+        a.y += w * (h1 - a.y);
+        a.z += w * (h2 - a.z);
+        a.w += w * (h3 - a.w);
+        *dst = a;
+      }
+    }
 }
 
 // ------------------------------------------------------------------- dQ (and delta)
@@ -487,13 +511,15 @@ bool attn_wide_supported(long long batch, int sq, int sk, int d, int dtype, bool
 }
 
 int attn_wide_fwd(void* out, float* lse, const void* q, const void* k, const void* v, long long batch, int sq,
-                  int sk, int d, float scale, hipStream_t s) {
+                  int sk, int d, float scale, float* out_acc, float* lse_acc, hipStream_t s) {
   Args a{};
   a.q = static_cast<const uint16_t*>(q);
   a.k = static_cast<const uint16_t*>(k);
   a.v = static_cast<const uint16_t*>(v);
   a.o = static_cast<uint16_t*>(out);
   a.lse = lse;
+  a.out_acc = out_acc;
+  a.lse_acc = lse_acc;
   a.sq = sq; a.sk = sk; a.scale = scale;
   return d == 128 ? launch_fwd<128>(a, batch, s) : launch_fwd<96>(a, batch, s);
 }

@@ -78,6 +78,8 @@ def test_core_forward_backward_match_oracle(shape, dtype, dev):
         (3, 6, 16, 16, 4, torch.bfloat16),
         (1, 2, 256, 64, 4, torch.bfloat16),
         (1, 2, 128, 64, 3, torch.float32),
+        (1, 2, 128, 128, 3, torch.bfloat16),  # head sizes 128 and 96: their own kernels, merge fused as well
+        (1, 1, 256, 96, 2, torch.bfloat16),
     ],
 )
 @pytest.mark.parametrize("rank", [0, 2])
@@ -111,12 +113,13 @@ def test_ring_forward_backward_match_full_attention(b, h, n, d, P, dtype, rank, 
     assert rel_l2(torch.cat(dvs, 2), V.grad) < TOL[dtype], f"dv {rel_l2(torch.cat(dvs, 2), V.grad):.3e}"
 
 
-def test_fused_step_equals_core_plus_merge(dev):
+@pytest.mark.parametrize("d", [64, 96, 128])
+def test_fused_step_equals_core_plus_merge(d, dev):
     """The fused epilogue merge and the separate merge kernel give the same accumulator."""
-    q, k, v = _qkv(1, 4, 256, 512, 64, torch.bfloat16, seed=2)
+    q, k, v = _qkv(1, 4, 256, 512, d, torch.bfloat16, seed=2)
     q, k, v = q.to(dev), k.to(dev), v.to(dev)
-    scale = 0.125
-    acc1 = torch.randn(1, 4, 256, 64, device=dev)
+    scale = d**-0.5
+    acc1 = torch.randn(1, 4, 256, d, device=dev)
     l1 = torch.randn(1, 4, 256, device=dev)
     acc2, l2 = acc1.clone(), l1.clone()
     ja.core_forward(q, k, v, scale, out_acc=acc1, lse_acc=l1, want_out=False)
