@@ -8,7 +8,9 @@ FETCH_SIZE / WRITE_SIZE counters.
 
 With the argument ``around-attention`` it launches instead the kernels either side of the ring
 step: the attention core at head size 128 (32 heads, 4096 x 4096 tokens) and the qkv / output
-projections with the head split fused in (8 x 4096 tokens, 512 channels, 8 heads).
+projections with the head split fused in (8 x 4096 tokens, 512 channels, 8 heads). With
+``swin-block`` it runs forward + backward of one Swin block on a 256 x 256 token tile (dim 128,
+4 heads, 8 x 8 windows, shift 4, bf16 autocast; the neighbours' roll slabs are random stand-ins).
 """
 
 from __future__ import annotations
@@ -92,10 +94,38 @@ def around_attention(reps: int = 3) -> None:
     print("profile_kernels: done", file=sys.stderr)
 
 
+def swin_block(reps: int = 5) -> None:
+    from jigsaw_amd import swin as js
+    from jigsaw_amd.conv import TileGroup
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(2)
+
+    def comm(data, buffer, direction, *, group, async_op):
+        buffer.normal_(generator=g)
+        return buffer, None
+
+    n, dim = (256, 256), 128
+    block = js.SwinBlock(dim, 4, 8, n, (TileGroup(2, 0), TileGroup(2, 1)), comm, shift=4, device=dev)
+    x = torch.randn(1, *n, dim, device=dev, generator=g).bfloat16().requires_grad_()
+    gout = torch.randn(1, *n, dim, device=dev, generator=g).bfloat16()
+    leaves = [x, *block.parameters()]
+    for _ in range(reps):
+        for t in leaves:
+            t.grad = None
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            y = block(x)
+        y.backward(gout)
+    torch.cuda.synchronize()
+    print("profile_kernels: done", file=sys.stderr)
+
+
 if __name__ == "__main__":
     if sys.argv[1:] == ["around-attention"]:
         around_attention()
+    elif sys.argv[1:] == ["swin-block"]:
+        swin_block()
     elif sys.argv[1:]:
-        raise SystemExit(f"unknown argument {sys.argv[1:]}; the only one is 'around-attention'")
+        raise SystemExit(f"unknown argument {sys.argv[1:]}; known: 'around-attention', 'swin-block'")
     else:
         main()
