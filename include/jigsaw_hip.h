@@ -416,7 +416,7 @@ int jg_bias_grad(void* gb, const void* g, int64_t batch, int64_t channels,
                  void* stream);
 
 /* ------------------------------------------------------------------------- *
- * Attention core of the ring step (MFMA kernels for bf16 at head sizes 64, 96, 128)
+ * Attention core of the ring step (MFMA kernels: bf16 at head sizes 64, 96, 128; fp16 at 96, 128)
  *
  * q (batch, sq, d), k / v (batch, sk, d), dense, `batch` = all leading axes
  * flattened (b*h for the "bhsd" layout of jigsaw's sdpa / math cores). One dtype
@@ -434,8 +434,8 @@ int jg_bias_grad(void* gb, const void* g, int64_t batch, int64_t channels,
  * (batch, sq)) are given, this chunk's result is merged into them in place,
  *   w = sigmoid(lse - lse_acc); out_acc += w*(out - out_acc); lse_acc = logaddexp,
  * which is _online_softmax_merge_ (forward.py:23-61) without the round trip of
- * out_j through HBM; `out` / `lse` may then be NULL (bf16, d = 64, 96 or 128, sq
- * and sk multiples of 128 only; JG_ERR_UNSUPPORTED otherwise).
+ * out_j through HBM; `out` / `lse` may then be NULL (bf16 with d = 64, 96 or 128, fp16
+ * with d = 96 or 128, sq and sk multiples of 128 only; JG_ERR_UNSUPPORTED otherwise).
  * d must be one of 8, 16, 32, 64, 96, 128 (JG_ERR_UNSUPPORTED otherwise; zero
  * columns appended to q, k, v leave out's other columns and lse unchanged). */
 int jg_attn_fwd(void* out, float* lse, const void* q, const void* k, const void* v,

@@ -18,6 +18,7 @@ Host-side mirror of
 
 from __future__ import annotations
 
+import math
 from collections.abc import Sequence
 
 import torch
@@ -99,14 +100,14 @@ def _bias_args(bias, batch, sq, sk):
 
 # --------------------------------------------------------------------------- #
 # Shapes the MFMA kernels do not take as they are (head sizes other than 64, 96 and 128 -- the
-# "widths" below --, sequence lengths that are not multiples of 128) are brought to them on the
-# host, in bf16 and without a bias:
+# "widths" below; fp16 has kernels for 96 and 128 only --, sequence lengths that are not multiples
+# of 128) are brought to them on the host, in bf16 / fp16 and without a bias:
 #   * head size: zero columns are appended to q, k, v (they add nothing to the scores and give
 #     zero output columns);
 #   * queries: zero rows are appended and their results dropped;
-#   * keys, head size below its width: rows are appended whose first spare column holds a large
-#     negative number, against a column of ones in q: their scores are about -30000, their
-#     probabilities 0;
+#   * keys, head size below its width: rows are appended whose first spare column holds -c, against
+#     a column of c in q, c = sqrt(30000 / scale) (a value fp16 can hold): their scores are
+#     -30000, their probabilities 0;
 #   * keys, head size equal to its width (no spare column): the multiple of 128 goes through the MFMA kernels, the
 #     remaining keys through the one-thread-per-row kernel, and the two (out, lse) pairs are merged
 #     like two ring steps; the backward treats the two key ranges like two ring chunks, the short
@@ -116,9 +117,9 @@ def _bias_args(bias, batch, sq, sk):
 _MASKED_SCORE = -30000.0
 
 
-def _width(d: int) -> int:
-    """Head size of the MFMA kernels that take a head of ``d`` columns."""
-    return 64 if d <= 64 else 96 if d <= 96 else 128
+def _width(d: int, dtype: torch.dtype) -> int:
+    """Head size of the MFMA kernels that take a head of ``d`` columns (fp16: 96 and 128 only)."""
+    return 64 if d <= 64 and dtype == torch.bfloat16 else 96 if d <= 96 else 128
 
 
 _KERNEL_HEAD_SIZES = (8, 16, 32, 64, 96, 128)
@@ -132,9 +133,9 @@ def _kernel_head_size(d: int) -> int:
 
 def _shapeable(q, k, bias) -> bool:
     d, sq, sk = q.shape[-1], q.shape[-2], k.shape[-2]
-    if bias is not None or q.dtype != torch.bfloat16 or d > 128 or sq == 0 or sk < 128:
+    if bias is not None or q.dtype not in (torch.bfloat16, torch.float16) or d > 128 or sq == 0 or sk < 128:
         return False
-    return d != _width(d) or sq % 128 != 0 or sk % 128 != 0
+    return d != _width(d, q.dtype) or sq % 128 != 0 or sk % 128 != 0
 
 
 def _pad_last(t: torch.Tensor, to: int) -> torch.Tensor:
@@ -153,15 +154,16 @@ def _shape_qkv(q, k, v, scale):
     """q, k, v as the MFMA kernels take them: ``(q, k, v, key ranges)``; a key range is
     ``(start, stop)`` in the (possibly padded) k / v, the first one a multiple of 128 long."""
     d, sq, sk = q.shape[-1], q.shape[-2], k.shape[-2]
-    w = _width(d)
+    w = _width(d, q.dtype)
     qp = _pad_rows(_pad_last(q, w), _up128(sq))
     kp, vp = _pad_last(k, w), _pad_last(v, w)
     if sk % 128 == 0:
         return qp, kp, vp, [(0, sk)]
     if d < w:
-        qp[..., d] = 1.0
+        c = math.sqrt(-_MASKED_SCORE / float(scale))
+        qp[..., d] = c
         kp, vp = _pad_rows(kp, _up128(sk)), _pad_rows(vp, _up128(sk))
-        kp[..., sk:, d] = _MASKED_SCORE / float(scale)
+        kp[..., sk:, d] = -c
         return qp, kp, vp, [(0, _up128(sk))]
     main = sk // 128 * 128
     return qp, kp, vp, [(0, main), (main, sk)]
@@ -299,8 +301,10 @@ def backward(grad_out, q, k, v, out, logsumexp, scale, *args, dropout_p=0.0, see
 # per-rank ring loops over local chunks
 # --------------------------------------------------------------------------- #
 def _fused_ok(q, k) -> bool:
+    d = q.shape[-1]
     return (
-        q.dtype == torch.bfloat16 and q.shape[-1] in (64, 96, 128) and q.shape[-2] % 128 == 0 and k.shape[-2] % 128 == 0
+        q.dtype in (torch.bfloat16, torch.float16) and d in (64, 96, 128) and d == _width(d, q.dtype)
+        and q.shape[-2] % 128 == 0 and k.shape[-2] % 128 == 0
     )
 
 

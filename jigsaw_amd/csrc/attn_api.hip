@@ -25,10 +25,11 @@ int attn_mfma_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q,
                   int sk, float scale, void* ws, hipStream_t s);
 bool attn_wide_supported(long long batch, int sq, int sk, int d, int dtype, bool has_bias);
 int attn_wide_fwd(void* out, float* lse, const void* q, const void* k, const void* v, long long batch,
-                  int sq, int sk, int d, float scale, float* out_acc, float* lse_acc, hipStream_t s);
+                  int sq, int sk, int d, int dtype, float scale, float* out_acc, float* lse_acc,
+                  hipStream_t s);
 int attn_wide_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q, const void* k,
                   const void* v, const void* out, const float* lse, long long batch, int sq, int sk,
-                  int d, float scale, void* ws, hipStream_t s);
+                  int d, int dtype, float scale, void* ws, hipStream_t s);
 bool attn_window_supported(long long batch, int sq, int sk, int d, int dtype);
 int attn_window_fwd(void* out, float* lse, const void* q, const void* k, const void* v,
                     long long batch, float scale, const float* bias, long long bias_period,
@@ -78,7 +79,8 @@ extern "C" int jg_attn_fwd(void* out, float* lse, const void* q, const void* k, 
     return jg::attn_mfma_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, scale, out_acc, lse_acc, s);
   if (jg::attn_wide_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr) &&
       aligned16({out, q, k, v, out_acc}))
-    return jg::attn_wide_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, (int)d, scale, out_acc, lse_acc, s);
+    return jg::attn_wide_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, (int)d, dtype, scale, out_acc,
+                             lse_acc, s);
   if (out_acc == nullptr && jg::attn_window_supported(batch, (int)sq, (int)sk, (int)d, dtype) &&
       aligned16({out, q, k, v, bias}))
     return jg::attn_window_fwd(out, lse, q, k, v, batch, scale, bias, bias_period, s);
@@ -125,7 +127,7 @@ extern "C" int jg_attn_bwd(void* dq, void* dk, void* dv, const void* dout, const
       jg::attn_wide_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr) &&
       aligned16({dq, dk, dv, dout, q, k, v, out}))
     return jg::attn_wide_bwd(dq, dk, dv, dout, q, k, v, out, lse, batch, (int)sq, (int)sk, (int)d,
-                             scale, workspace, s);
+                             dtype, scale, workspace, s);
   if (jg::attn_window_supported(batch, (int)sq, (int)sk, (int)d, dtype) &&
       aligned16({dq, dk, dv, dout, q, k, v, out, bias, dbias}))
     return jg::attn_window_bwd(dq, dk, dv, dbias, dout, q, k, v, out, lse, batch, scale, bias,

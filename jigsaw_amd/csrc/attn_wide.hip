@@ -1,4 +1,4 @@
-// Blockwise (flash-style) attention of one K/V chunk on the bf16 matrix cores for head
+// Blockwise (flash-style) attention of one K/V chunk on the bf16 / fp16 matrix cores for head
 // sizes 96 and 128, non-causal, no bias: forward (output + natural-log LSE) and backward
 // from a given (global) output and LSE. Same arithmetic as the head-size-64 kernels,
 // written for clarity rather than hand-scheduled: tiles of 32 keys (forward, dQ) or 32
@@ -26,6 +26,8 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -111,32 +113,66 @@ __device__ __forceinline__ void trans_store(const TransRegs<D>& r, unsigned char
   }
 }
 
-__device__ __forceinline__ bf16x8 pack8(const float* v) {
-  bf16x8 r;
-#pragma unroll
-  for (int j = 0; j < 8; j += 2) {
-    const f32x2 v2 = {v[j], v[j + 1]};
-    const bf16x2 h2 = __builtin_convertvector(v2, bf16x2);
-    r[j] = h2.x;
-    r[j + 1] = h2.y;
-  }
-  return r;
-}
-__device__ __forceinline__ u32x2 pack4(float a, float b, float c, float d) {
-  const f32x2 lo = {a, b}, hi = {c, d};
-  u32x2 r;
-  r.x = __builtin_bit_cast(uint32_t, __builtin_convertvector(lo, bf16x2));
-  r.y = __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, bf16x2));
-  return r;
-}
 __device__ __forceinline__ f32x16 zero16() {
   f32x16 z;
 #pragma unroll
   for (int i = 0; i < 16; ++i) z[i] = 0.0f;
   return z;
 }
-__device__ __forceinline__ bf16x8 frag(const unsigned char* at) {
-  return __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(at));
+// The 16-bit element type of q, k, v: bf16 or fp16. Both have a 32x32x16 MFMA with the same operand
+// layout; they differ in the conversions from and to fp32.
+template <bool F16>
+struct Half;
+template <>
+struct Half<false> {
+  typedef bf16x8 x8;
+  __device__ static __forceinline__ f32x16 mma(x8 a, x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ uint32_t pair(float a, float b) {
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+  }
+  __device__ static __forceinline__ void unpair(uint32_t w, float& a, float& b) {
+    a = __uint_as_float(w << 16);
+    b = __uint_as_float(w & 0xffff0000u);
+  }
+};
+template <>
+struct Half<true> {
+  typedef f16x8 x8;
+  __device__ static __forceinline__ f32x16 mma(x8 a, x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ uint32_t pair(float a, float b) {
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+  }
+  __device__ static __forceinline__ void unpair(uint32_t w, float& a, float& b) {
+    const f32x2 v = __builtin_convertvector(__builtin_bit_cast(f16x2, w), f32x2);
+    a = v.x;
+    b = v.y;
+  }
+};
+template <bool F16>
+__device__ __forceinline__ typename Half<F16>::x8 frag(const unsigned char* at) {
+  return __builtin_bit_cast(typename Half<F16>::x8, *reinterpret_cast<const u32x4*>(at));
+}
+template <bool F16>
+__device__ __forceinline__ typename Half<F16>::x8 pack8(const float* v) {
+  u32x4 r;
+  r.x = Half<F16>::pair(v[0], v[1]);
+  r.y = Half<F16>::pair(v[2], v[3]);
+  r.z = Half<F16>::pair(v[4], v[5]);
+  r.w = Half<F16>::pair(v[6], v[7]);
+  return __builtin_bit_cast(typename Half<F16>::x8, r);
+}
+template <bool F16>
+__device__ __forceinline__ u32x2 pack4(float a, float b, float c, float d) {
+  u32x2 r;
+  r.x = Half<F16>::pair(a, b);
+  r.y = Half<F16>::pair(c, d);
+  return r;
 }
 
 struct Args {
@@ -159,9 +195,10 @@ struct Args {
 };
 
 // ------------------------------------------------------------------- forward
-template <int D>
+template <int D, bool F16>
 __global__ __launch_bounds__(THREADS) void attn_wide_fwd_kernel(Args p) {
   typedef Geo<D> G;
+  typedef typename Half<F16>::x8 X8;
   constexpr int BUF = G::ROWMAJ + G::TRANS;  // K rows, then V^T
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -173,9 +210,9 @@ __global__ __launch_bounds__(THREADS) void attn_wide_fwd_kernel(Args p) {
   const uint16_t* vb = p.v + bh * p.sk * D;
   const float c2 = p.scale * LOG2E;
 
-  bf16x8 qf[G::C16];
+  X8 qf[G::C16];
 #pragma unroll
-  for (int c = 0; c < G::C16; ++c) qf[c] = frag(reinterpret_cast<const unsigned char*>(qrow + 16 * c + 8 * kg));
+  for (int c = 0; c < G::C16; ++c) qf[c] = frag<F16>(reinterpret_cast<const unsigned char*>(qrow + 16 * c + 8 * kg));
 
   f32x16 o[G::NB];
 #pragma unroll
@@ -201,7 +238,7 @@ __global__ __launch_bounds__(THREADS) void attn_wide_fwd_kernel(Args p) {
     f32x16 s = zero16();
 #pragma unroll
     for (int c = 0; c < G::C16; ++c)
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(kt + ln * G::RP + (16 * c + 8 * kg) * 2), qf[c], s, 0, 0, 0);
+      s = Half<F16>::mma(frag<F16>(kt + ln * G::RP + (16 * c + 8 * kg) * 2), qf[c], s);
     float mx = s[0];
 #pragma unroll
     for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
@@ -227,11 +264,11 @@ __global__ __launch_bounds__(THREADS) void attn_wide_fwd_kernel(Args p) {
     l += sum;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      const bf16x8 pf = pack8(pr + 8 * ks);
+      const X8 pf = pack8<F16>(pr + 8 * ks);
 #pragma unroll
       for (int nb = 0; nb < G::NB; ++nb)
-        o[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(vt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2), pf,
-                                                        o[nb], 0, 0, 0);
+        o[nb] = Half<F16>::mma(frag<F16>(vt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2), pf,
+                                                        o[nb]);
     }
     if (t + 1 < ntiles) {
       unsigned char* nk = smem + ((t + 1) & 1) * BUF;
@@ -260,13 +297,14 @@ __global__ __launch_bounds__(THREADS) void attn_wide_fwd_kernel(Args p) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int dv = nb * 32 + 8 * j + 4 * kg;
-      const u32x2 h = pack4(o[nb][4 * j] * inv, o[nb][4 * j + 1] * inv, o[nb][4 * j + 2] * inv, o[nb][4 * j + 3] * inv);
+      const u32x2 h = pack4<F16>(o[nb][4 * j] * inv, o[nb][4 * j + 1] * inv, o[nb][4 * j + 2] * inv, o[nb][4 * j + 3] * inv);
       if (p.o != nullptr) *reinterpret_cast<u32x2*>(p.o + row * D + dv) = h;
       if (p.out_acc != nullptr) {
         f32x4* dst = reinterpret_cast<f32x4*>(p.out_acc + row * D + dv);
         f32x4 a = *dst;
-        const float h0 = __uint_as_float(h.x << 16), h1 = __uint_as_float(h.x & 0xffff0000u);
-        const float h2 = __uint_as_float(h.y << 16), h3 = __uint_as_float(h.y & 0xffff0000u);
+        float h0, h1, h2, h3;
+        Half<F16>::unpair(h.x, h0, h1);
+        Half<F16>::unpair(h.y, h2, h3);
         a.x += w * (h0 - a.x);
         a.y += w * (h1 - a.y);
         a.z += w * (h2 - a.z);
@@ -277,9 +315,10 @@ __global__ __launch_bounds__(THREADS) void attn_wide_fwd_kernel(Args p) {
 }
 
 // ------------------------------------------------------------------- dQ (and delta)
-template <int D>
+template <int D, bool F16>
 __global__ __launch_bounds__(THREADS) void attn_wide_dq_kernel(Args p) {
   typedef Geo<D> G;
+  typedef typename Half<F16>::x8 X8;
   constexpr int BUF = 2 * G::ROWMAJ + G::TRANS;  // K rows, V rows, K^T
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -291,13 +330,13 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dq_kernel(Args p) {
   const uint16_t* vb = p.v + bh * p.sk * D;
   const float c2 = p.scale * LOG2E;
 
-  bf16x8 qf[G::C16], dof[G::C16];
+  X8 qf[G::C16], dof[G::C16];
   float dl = 0.0f;
 #pragma unroll
   for (int c = 0; c < G::C16; ++c) {
-    qf[c] = frag(reinterpret_cast<const unsigned char*>(p.q + qoff + 16 * c + 8 * kg));
-    dof[c] = frag(reinterpret_cast<const unsigned char*>(p.dout + qoff + 16 * c + 8 * kg));
-    const bf16x8 of = frag(reinterpret_cast<const unsigned char*>(p.out + qoff + 16 * c + 8 * kg));
+    qf[c] = frag<F16>(reinterpret_cast<const unsigned char*>(p.q + qoff + 16 * c + 8 * kg));
+    dof[c] = frag<F16>(reinterpret_cast<const unsigned char*>(p.dout + qoff + 16 * c + 8 * kg));
+    const X8 of = frag<F16>(reinterpret_cast<const unsigned char*>(p.out + qoff + 16 * c + 8 * kg));
 #pragma unroll
     for (int j = 0; j < 8; ++j) dl += (float)dof[c][j] * (float)of[j];
   }
@@ -332,19 +371,19 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dq_kernel(Args p) {
     f32x16 s = zero16(), dp = zero16();
 #pragma unroll
     for (int c = 0; c < G::C16; ++c) {
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(kt + ln * G::RP + (16 * c + 8 * kg) * 2), qf[c], s, 0, 0, 0);
-      dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(vt + ln * G::RP + (16 * c + 8 * kg) * 2), dof[c], dp, 0, 0, 0);
+      s = Half<F16>::mma(frag<F16>(kt + ln * G::RP + (16 * c + 8 * kg) * 2), qf[c], s);
+      dp = Half<F16>::mma(frag<F16>(vt + ln * G::RP + (16 * c + 8 * kg) * 2), dof[c], dp);
     }
     float ds[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) ds[i] = __builtin_amdgcn_exp2f(s[i] * c2 - lse2) * (dp[i] - delta);
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      const bf16x8 dsf = pack8(ds + 8 * ks);
+      const X8 dsf = pack8<F16>(ds + 8 * ks);
 #pragma unroll
       for (int nb = 0; nb < G::NB; ++nb)
-        dq[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(ktt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2),
-                                                         dsf, dq[nb], 0, 0, 0);
+        dq[nb] = Half<F16>::mma(frag<F16>(ktt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2),
+                                                         dsf, dq[nb]);
     }
     if (t + 1 < ntiles) {
       unsigned char* nk = smem + ((t + 1) & 1) * BUF;
@@ -360,14 +399,15 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dq_kernel(Args p) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       *reinterpret_cast<u32x2*>(row + nb * 32 + 8 * j + 4 * kg) =
-          pack4(dq[nb][4 * j] * p.scale, dq[nb][4 * j + 1] * p.scale, dq[nb][4 * j + 2] * p.scale,
+          pack4<F16>(dq[nb][4 * j] * p.scale, dq[nb][4 * j + 1] * p.scale, dq[nb][4 * j + 2] * p.scale,
                 dq[nb][4 * j + 3] * p.scale);
 }
 
 // ------------------------------------------------------------------- dK, dV
-template <int D>
+template <int D, bool F16>
 __global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
   typedef Geo<D> G;
+  typedef typename Half<F16>::x8 X8;
   constexpr int STATS = 2 * BT * 4;                           // lse * log2(e) and delta of the tile's queries
   constexpr int BUF = 2 * G::ROWMAJ + 2 * G::TRANS + STATS;   // Q rows, dO rows, Q^T, dO^T, stats
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -382,11 +422,11 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
   const float* db = p.delta + bh * p.sq;
   const float c2 = p.scale * LOG2E;
 
-  bf16x8 kf[G::C16], vf[G::C16];
+  X8 kf[G::C16], vf[G::C16];
 #pragma unroll
   for (int c = 0; c < G::C16; ++c) {
-    kf[c] = frag(reinterpret_cast<const unsigned char*>(p.k + koff + 16 * c + 8 * kg));
-    vf[c] = frag(reinterpret_cast<const unsigned char*>(p.v + koff + 16 * c + 8 * kg));
+    kf[c] = frag<F16>(reinterpret_cast<const unsigned char*>(p.k + koff + 16 * c + 8 * kg));
+    vf[c] = frag<F16>(reinterpret_cast<const unsigned char*>(p.v + koff + 16 * c + 8 * kg));
   }
   f32x16 dk[G::NB], dv[G::NB];
 #pragma unroll
@@ -432,8 +472,8 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
     f32x16 s = zero16(), dp = zero16();
 #pragma unroll
     for (int c = 0; c < G::C16; ++c) {
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(qt + ln * G::RP + (16 * c + 8 * kg) * 2), kf[c], s, 0, 0, 0);
-      dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(gt + ln * G::RP + (16 * c + 8 * kg) * 2), vf[c], dp, 0, 0, 0);
+      s = Half<F16>::mma(frag<F16>(qt + ln * G::RP + (16 * c + 8 * kg) * 2), kf[c], s);
+      dp = Half<F16>::mma(frag<F16>(gt + ln * G::RP + (16 * c + 8 * kg) * 2), vf[c], dp);
     }
     float pr[16], ds[16];
 #pragma unroll
@@ -449,13 +489,13 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
     }
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      const bf16x8 pf = pack8(pr + 8 * ks), dsf = pack8(ds + 8 * ks);
+      const X8 pf = pack8<F16>(pr + 8 * ks), dsf = pack8<F16>(ds + 8 * ks);
 #pragma unroll
       for (int nb = 0; nb < G::NB; ++nb) {
-        dv[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(gtt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2), pf,
-                                                         dv[nb], 0, 0, 0);
-        dk[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(qtt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2), dsf,
-                                                         dk[nb], 0, 0, 0);
+        dv[nb] = Half<F16>::mma(frag<F16>(gtt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2), pf,
+                                                         dv[nb]);
+        dk[nb] = Half<F16>::mma(frag<F16>(qtt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2), dsf,
+                                                         dk[nb]);
       }
     }
     if (t + 1 < ntiles) store((t + 1) & 1);
@@ -468,27 +508,27 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       *reinterpret_cast<u32x2*>(krow + nb * 32 + 8 * j + 4 * kg) =
-          pack4(dk[nb][4 * j] * p.scale, dk[nb][4 * j + 1] * p.scale, dk[nb][4 * j + 2] * p.scale,
+          pack4<F16>(dk[nb][4 * j] * p.scale, dk[nb][4 * j + 1] * p.scale, dk[nb][4 * j + 2] * p.scale,
                 dk[nb][4 * j + 3] * p.scale);
       *reinterpret_cast<u32x2*>(vrow + nb * 32 + 8 * j + 4 * kg) =
-          pack4(dv[nb][4 * j], dv[nb][4 * j + 1], dv[nb][4 * j + 2], dv[nb][4 * j + 3]);
+          pack4<F16>(dv[nb][4 * j], dv[nb][4 * j + 1], dv[nb][4 * j + 2], dv[nb][4 * j + 3]);
     }
 }
 
-template <int D>
+template <int D, bool F16>
 int launch_fwd(const Args& a, long long batch, hipStream_t s) {
-  attn_wide_fwd_kernel<D><<<dim3((unsigned)(a.sq / BQ), (unsigned)batch, 1), THREADS, 0, s>>>(a);
+  attn_wide_fwd_kernel<D, F16><<<dim3((unsigned)(a.sq / BQ), (unsigned)batch, 1), THREADS, 0, s>>>(a);
   JG_CHECK_LAUNCH("jg_attn_fwd(wide)");
   return JG_OK;
 }
 
-template <int D>
+template <int D, bool F16>
 int launch_bwd(const Args& a, long long batch, hipStream_t s) {
   typedef Geo<D> G;
   constexpr int DQ_LDS = 2 * (2 * G::ROWMAJ + G::TRANS);
   constexpr int DKV_LDS = 2 * (2 * G::ROWMAJ + 2 * G::TRANS + 2 * BT * 4);
-  void (*dqk)(Args) = &attn_wide_dq_kernel<D>;
-  void (*dkvk)(Args) = &attn_wide_dkv_kernel<D>;
+  void (*dqk)(Args) = &attn_wide_dq_kernel<D, F16>;
+  void (*dkvk)(Args) = &attn_wide_dkv_kernel<D, F16>;
   hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(dqk), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       DQ_LDS);
   hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(dkvk), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -506,12 +546,12 @@ int launch_bwd(const Args& a, long long batch, hipStream_t s) {
 namespace jg {
 
 bool attn_wide_supported(long long batch, int sq, int sk, int d, int dtype, bool has_bias) {
-  return dtype == JG_BF16 && !has_bias && (d == 96 || d == 128) && sq > 0 && sk > 0 && sq % BQ == 0 &&
+  return (dtype == JG_BF16 || dtype == JG_F16) && !has_bias && (d == 96 || d == 128) && sq > 0 && sk > 0 && sq % BQ == 0 &&
          sk % BQ == 0 && batch > 0 && batch <= 65535;
 }
 
 int attn_wide_fwd(void* out, float* lse, const void* q, const void* k, const void* v, long long batch, int sq,
-                  int sk, int d, float scale, float* out_acc, float* lse_acc, hipStream_t s) {
+                  int sk, int d, int dtype, float scale, float* out_acc, float* lse_acc, hipStream_t s) {
   Args a{};
   a.q = static_cast<const uint16_t*>(q);
   a.k = static_cast<const uint16_t*>(k);
@@ -521,12 +561,13 @@ int attn_wide_fwd(void* out, float* lse, const void* q, const void* k, const voi
   a.out_acc = out_acc;
   a.lse_acc = lse_acc;
   a.sq = sq; a.sk = sk; a.scale = scale;
-  return d == 128 ? launch_fwd<128>(a, batch, s) : launch_fwd<96>(a, batch, s);
+  if (dtype == JG_F16) return d == 128 ? launch_fwd<128, true>(a, batch, s) : launch_fwd<96, true>(a, batch, s);
+  return d == 128 ? launch_fwd<128, false>(a, batch, s) : launch_fwd<96, false>(a, batch, s);
 }
 
 int attn_wide_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q, const void* k, const void* v,
-                  const void* out, const float* lse, long long batch, int sq, int sk, int d, float scale,
-                  void* ws, hipStream_t s) {
+                  const void* out, const float* lse, long long batch, int sq, int sk, int d, int dtype,
+                  float scale, void* ws, hipStream_t s) {
   Args a{};
   a.q = static_cast<const uint16_t*>(q);
   a.k = static_cast<const uint16_t*>(k);
@@ -539,7 +580,8 @@ int attn_wide_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q,
   a.dk = static_cast<uint16_t*>(dk);
   a.dv = static_cast<uint16_t*>(dv);
   a.sq = sq; a.sk = sk; a.scale = scale;
-  return d == 128 ? launch_bwd<128>(a, batch, s) : launch_bwd<96>(a, batch, s);
+  if (dtype == JG_F16) return d == 128 ? launch_bwd<128, true>(a, batch, s) : launch_bwd<96, true>(a, batch, s);
+  return d == 128 ? launch_bwd<128, false>(a, batch, s) : launch_bwd<96, false>(a, batch, s);
 }
 
 }  // namespace jg

@@ -80,6 +80,8 @@ def test_core_forward_backward_match_oracle(shape, dtype, dev):
         (1, 2, 128, 64, 3, torch.float32),
         (1, 2, 128, 128, 3, torch.bfloat16),  # head sizes 128 and 96: their own kernels, merge fused as well
         (1, 1, 256, 96, 2, torch.bfloat16),
+        (1, 2, 128, 128, 2, torch.float16),   # fp16 on the matrix cores, merge fused
+        (1, 2, 256, 64, 2, torch.float16),    # fp16, head size 64: padded to the 96-wide kernels per step
     ],
 )
 @pytest.mark.parametrize("rank", [0, 2])
