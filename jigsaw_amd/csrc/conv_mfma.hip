@@ -32,9 +32,12 @@
 //               their way to LDS), the weights stay in LDS in groups of steps when they
 //               do not fit at once, produced channels are padded to 32 and a ragged last
 //               tile predicates its stores.
-//   fp32, fp16  "split mode": an operand is the exact sum of three (two) bf16 parts, kept
-//               as extra channel groups; the contraction runs over the six (three) part
-//               products that matter and the result is stored as fp32 (fp16).
+//   fp16        the same kernel on v_mfma_f32_32x32x16_f16 (a template flag; the staging moves
+//               16-bit values without looking at them).
+//   fp32        "split mode": an operand is the exact sum of three bf16 parts, kept as extra
+//               channel groups; the contraction runs over the six part products that matter
+//               and the result is stored as fp32. (A two-part form of it for fp16 operands
+//               remains in the split kernels and is not dispatched.)
 #include <type_traits>
 
 #include "conv_common.h"
@@ -46,6 +49,7 @@ using jg::ConvGeom;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -254,7 +258,9 @@ __device__ inline void store_f32(const void* base, uint32_t lane_off, float v) {
   asm volatile("global_store_dword %0, %1, %2" : : "v"(lane_off), "v"(v), "s"(base) : "memory");
 }
 
-template <int MT, bool EVEN, bool FOLD, bool FRAMED>  // MT = produced channels per workgroup: 32 or 64
+// F16: the 16-bit tensors hold fp16 instead of bf16 (v_mfma_f32_32x32x16_f16; everything else moves
+// 16-bit values without looking at them, the epilogue converts by out_kind).
+template <int MT, bool EVEN, bool FOLD, bool FRAMED, bool F16 = false>  // MT = produced channels per workgroup: 32 or 64
 __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips, FwdParams p) {
   constexpr int CB = MT / 32;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -504,7 +510,11 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
         if (r >= 0 && r < WROWS) {
 #pragma unroll
           for (int cb = 0; cb < CB; ++cb)
-            acc[cb][r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kh][cb], b, acc[cb][r], 0, 0, 0);
+            if (F16)
+              acc[cb][r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[kh][cb]),
+                                                                  __builtin_bit_cast(f16x8, b), acc[cb][r], 0, 0, 0);
+            else
+              acc[cb][r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kh][cb], b, acc[cb][r], 0, 0, 0);
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -780,7 +790,8 @@ struct Launch {
   const void* w;
   const void* bias;
   void* y;
-  int split;                // split mode: 0 bf16 tensors, 1 fp32 (six bf16 products), 2 fp16 (three)
+  int split;                // split mode: 0 16-bit tensors as they are, 1 fp32 (six bf16 products), 2 fp16 (three)
+  int f16;                  // the 16-bit tensors are fp16 (split 0 only)
   int N, C, M, KD;
   int Din, Hin, Win, Dout, Hout, Wout;
   int pad_d, pad_h, pad_w;
@@ -858,7 +869,7 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   p.bias = static_cast<const uint16_t*>(L.bias); p.y = static_cast<uint16_t*>(L.y);
   p.N = L.N; p.C = L.C; p.M = L.M; p.KD = L.KD;
   p.Cp = pad16(L.C);
-  p.nblk = nblk; p.Cx = sp.parts * L.C; p.xmap = sp.xparts; p.out_kind = L.split;
+  p.nblk = nblk; p.Cx = sp.parts * L.C; p.xmap = sp.xparts; p.out_kind = L.f16 ? 2 : L.split;
   p.Din = L.Din; p.Hin = L.Hin; p.Win = L.Win;
   p.Dout = L.Dout; p.Hout = L.Hout; p.Wout = L.Wout;
   p.pad_d = L.pad_d; p.pad_h = L.pad_h; p.pad_w = L.pad_w;
@@ -887,12 +898,19 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   const bool even = (L.Win % 2 == 0) && (L.pad_w % 2 == 0) &&
                     ((reinterpret_cast<uintptr_t>(x16) & 3) == 0);
   void (*kern)(StripTable, FwdParams) = nullptr;
+  if (L.f16 && (L.fold || L.xt != nullptr))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: the fold epilogue and the framed input are built for bf16 only", who);
   if (L.fold) {
     if (MT == 64) kern = even ? &conv3x3_mfma_kernel<64, true, true, false> : &conv3x3_mfma_kernel<64, false, true, false>;
     else kern = even ? &conv3x3_mfma_kernel<32, true, true, false> : &conv3x3_mfma_kernel<32, false, true, false>;
   } else if (L.xt != nullptr) {
     if (MT == 64) kern = even ? &conv3x3_mfma_kernel<64, true, false, true> : &conv3x3_mfma_kernel<64, false, false, true>;
     else kern = even ? &conv3x3_mfma_kernel<32, true, false, true> : &conv3x3_mfma_kernel<32, false, false, true>;
+  } else if (L.f16) {
+    if (MT == 64)
+      kern = even ? &conv3x3_mfma_kernel<64, true, false, false, true> : &conv3x3_mfma_kernel<64, false, false, false, true>;
+    else
+      kern = even ? &conv3x3_mfma_kernel<32, true, false, false, true> : &conv3x3_mfma_kernel<32, false, false, false, true>;
   } else {
     if (MT == 64) kern = even ? &conv3x3_mfma_kernel<64, true, false, false> : &conv3x3_mfma_kernel<64, false, false, false>;
     else kern = even ? &conv3x3_mfma_kernel<32, true, false, false> : &conv3x3_mfma_kernel<32, false, false, false>;
@@ -911,7 +929,8 @@ namespace jg {
 
 // fp32 runs in split mode (three bf16 parts per operand, fp32 result); its 4-byte stores halve
 // the extent the 32-bit lane offsets reach.
-static int split_mode(int dtype) { return dtype == JG_F32 ? 1 : (dtype == JG_F16 ? 2 : 0); }
+// fp32 runs in split mode; fp16 has its own MFMA instruction and runs like bf16
+static int split_mode(int dtype) { return dtype == JG_F32 ? 1 : 0; }
 static bool dtype_ok(const ConvGeom& g, int dtype) {
   if (dtype == JG_BF16 || dtype == JG_F16) return true;
   if (dtype != JG_F32) return false;
@@ -947,6 +966,7 @@ static int fwd_launch(void* y, const void* x, const void* xt, const int* tlo, co
   Launch L;
   L.x = x; L.w = w; L.bias = bias; L.y = y;
   L.split = split_mode(dtype);
+  L.f16 = dtype == JG_F16 ? 1 : 0;
   L.N = (int)g.batch; L.C = g.cin; L.M = g.cout; L.KD = g.k[0];
   L.Din = g.in[0]; L.Hin = g.in[1]; L.Win = g.in[2];
   L.Dout = g.out[0]; L.Hout = g.out[1]; L.Wout = g.out[2];
@@ -1017,6 +1037,7 @@ static int dgrad_launch(void* gx, void* const* strips, const int* lo, const int*
   Launch L;
   L.x = go; L.w = w; L.bias = nullptr; L.y = gx;
   L.split = split_mode(dtype);
+  L.f16 = dtype == JG_F16 ? 1 : 0;
   L.N = (int)g.batch; L.C = g.cout; L.M = g.cin; L.KD = g.k[0];
   L.Din = g.out[0]; L.Hin = g.out[1]; L.Win = g.out[2];
   L.Dout = g.in[0]; L.Hout = g.in[1]; L.Wout = g.in[2];

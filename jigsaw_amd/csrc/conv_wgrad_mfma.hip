@@ -1,9 +1,10 @@
 // Weight gradient of the 3x3 (2-D) and 3x3x3 (3-D) convolution on the bf16 matrix
 // cores, stride 1, dilation 1, channels-first tensors; a launch covers a block of 32 or
 // 64 channels a side, any other channel counts are walked block by block. Optionally the
-// bias gradient from the same pass over g. fp32 / fp16 tensors run as sums of three / two
-// bf16 parts per operand ("split mode": the parts are extra channels, their products are
-// added up in fp32).
+// bias gradient from the same pass over g. fp16 tensors run the same kernel on the fp16
+// MFMA instruction (the gradient is reduced in fp32 and rounded to fp16 once); fp32 tensors
+// run as sums of three bf16 parts per operand ("split mode": the parts are extra channels,
+// their products are added up in fp32).
 //
 //   gw[co][ci][kd][kh][kw] = sum_{n,d,h,w} g[n][co][d][h][w] * x[n][ci][d+kd-pd][h+kh-ph][w+kw-pw]
 //   gb[co]                 = sum_{n,d,h,w} g[n][co][d][h][w]
@@ -45,6 +46,7 @@ using jg::ConvGeom;
 using jg::mfma_frame_bands;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
@@ -92,7 +94,8 @@ __device__ __forceinline__ float sum_bf16x8(const u32x4& v) {
   return s;
 }
 
-template <int CGB, int CXB, bool EVEN, bool FRAMED>
+// F16: x and g hold fp16 instead of bf16 (v_mfma_f32_32x32x16_f16); the partial sums are fp32 either way.
+template <int CGB, int CXB, bool EVEN, bool FRAMED, bool F16 = false>
 __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(WgradParams p) {
   constexpr int THREADS = wgrad_threads(CGB, CXB);
   constexpr int CWAVES = CGB * CXB * HALVES;  // wavefronts that own accumulators
@@ -435,9 +438,16 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
       for (int r = 0; r < SR; ++r) {
         const int kh = rho - r;
         if (kh >= 0 && kh < 3) {
-          acc[kh][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r], b0, acc[kh][0], 0, 0, 0);
-          acc[kh][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r], b1, acc[kh][1], 0, 0, 0);
-          acc[kh][2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r], b2, acc[kh][2], 0, 0, 0);
+          if (F16) {
+            const f16x8 ah = __builtin_bit_cast(f16x8, a[r]);
+            acc[kh][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, __builtin_bit_cast(f16x8, b0), acc[kh][0], 0, 0, 0);
+            acc[kh][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, __builtin_bit_cast(f16x8, b1), acc[kh][1], 0, 0, 0);
+            acc[kh][2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, __builtin_bit_cast(f16x8, b2), acc[kh][2], 0, 0, 0);
+          } else {
+            acc[kh][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r], b0, acc[kh][0], 0, 0, 0);
+            acc[kh][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r], b1, acc[kh][1], 0, 0, 0);
+            acc[kh][2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r], b2, acc[kh][2], 0, 0, 0);
+          }
         }
       }
     }
@@ -650,11 +660,13 @@ bool blocks_of(const ConvGeom& g, Blocking* b) {
 int block_width(int total, int c0, int first) { return (first == 64 && total - c0 > 32) ? 64 : 32; }
 
 template <int CGB, int CXB>
-int launch(const WgradParams& p, bool even, int wgs, hipStream_t s, const char* who) {
+int launch(const WgradParams& p, bool even, bool f16, int wgs, hipStream_t s, const char* who) {
   constexpr int THREADS = wgrad_threads(CGB, CXB);
   const size_t lds = 2 * (size_t)(32 * CGB * G_CH) + (size_t)(32 * CXB * X_CH);
   void (*kern)(WgradParams);
-  if (p.xt != nullptr)
+  if (f16)  // never framed (checked by the caller)
+    kern = even ? &wgrad3x3_mfma_kernel<CGB, CXB, true, false, true> : &wgrad3x3_mfma_kernel<CGB, CXB, false, false, true>;
+  else if (p.xt != nullptr)
     kern = &wgrad3x3_mfma_kernel<CGB, CXB, true, true>;  // the framed input needs the even layout (checked by the caller)
   else
     kern = even ? &wgrad3x3_mfma_kernel<CGB, CXB, true, false> : &wgrad3x3_mfma_kernel<CGB, CXB, false, false>;
@@ -669,7 +681,8 @@ int launch(const WgradParams& p, bool even, int wgs, hipStream_t s, const char* 
 
 namespace jg {
 
-static int parts_of(int dtype) { return dtype == JG_F32 ? 3 : (dtype == JG_F16 ? 2 : 1); }
+// fp32 is split into three bf16 parts per operand; fp16 has its own MFMA instruction and runs like bf16
+static int parts_of(int dtype) { return dtype == JG_F32 ? 3 : 1; }
 // Split mode with few channels: the parts of both operands fit one block.
 static bool parts_fit_one_block(const ConvGeom& g, const Blocking& bl, int parts) {
   return parts > 1 && parts * g.cout <= bl.cob_max() && parts * g.cin <= bl.cib_max();
@@ -678,13 +691,13 @@ static size_t parts_tmp_bytes(const ConvGeom& g, const Blocking& bl, int parts) 
   if (!parts_fit_one_block(g, bl, parts)) return 0;
   return ((size_t)parts * parts * g.cout * g.cin * bl.KD * 9 * sizeof(float) + 255) / 256 * 256;
 }
-// fp16: the part products are added up in fp32 here before the one rounding to fp16
+// fp16: the gradient is reduced into fp32 here before the one rounding to fp16
 static size_t acc32_bytes(const ConvGeom& g, int dtype) {
   return dtype == JG_F16 ? ((size_t)g.cout * g.cin * g.k[0] * 9 * sizeof(float) + 255) / 256 * 256 : 0;
 }
 
-// fp32 / fp16 run in split mode: both operands are copied as three / two bf16 parts each (as extra
-// channels) and the six / three part products whose indices add up to at most 2 / 1 are accumulated in fp32.
+// fp32 runs in split mode: both operands are copied as three bf16 parts each (as extra channels) and
+// the six part products whose indices add up to at most 2 are accumulated in fp32.
 bool mfma_wgrad_supported(const ConvGeom& g, int dtype) {
   Blocking b;
   if ((dtype != JG_BF16 && dtype != JG_F32 && dtype != JG_F16) || g.batch <= 0) return false;
@@ -700,14 +713,14 @@ static size_t partial_bytes(const ConvGeom& g) {
   return (n + 255) / 256 * 256;
 }
 static size_t split_copy_bytes(size_t elements, int parts) { return (elements * parts * 2 + 255) / 256 * 256; }
-// workspace: [partials | x parts | g parts | fp32 sum (fp16 only) | part products of the one-block launch]
+// workspace: [partials | fp32 sum (fp16 only) | x parts | g parts (fp32 only) | part products of the one-block launch]
 size_t mfma_wgrad_workspace(const ConvGeom& g, int dtype) {
   size_t n = partial_bytes(g);
   const int parts = parts_of(dtype);
+  n += acc32_bytes(g, dtype);  // fp16 only, directly behind the partial sums
   if (parts > 1) {
     n += split_copy_bytes((size_t)g.batch * g.cin * g.in[0] * g.in[1] * g.in[2], parts);
     n += split_copy_bytes((size_t)g.batch * g.cout * g.out[0] * g.out[1] * g.out[2], parts);
-    n += acc32_bytes(g, dtype);
     Blocking b{32, 32, 1};
     blocks_of(g, &b);
     n += parts_tmp_bytes(g, b, parts);
@@ -755,18 +768,18 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
   const size_t x_cs = (size_t)g.in[0] * g.in[1] * g.in[2], g_cs = (size_t)g.out[0] * g.out[1] * g.out[2];
   const int parts = parts_of(dtype);
   const bool split = parts > 1;
+  const bool f16 = dtype == JG_F16;
   float* sum32 = static_cast<float*>(gw);  // where the part products are added up (split mode)
   float* one_block_tmp = nullptr;
+  if ((split || f16) && (gb != nullptr || xt != nullptr))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: fp32 / fp16 have neither the fused bias gradient nor the framed input", who);
+  if (f16) sum32 = reinterpret_cast<float*>(static_cast<char*>(ws) + partial_bytes(g));
   if (split) {
-    if (gb != nullptr || xt != nullptr)
-      JG_FAIL(JG_ERR_UNSUPPORTED, "%s: fp32 / fp16 have neither the fused bias gradient nor the framed input", who);
     char* base = static_cast<char*>(ws) + partial_bytes(g);
     uint16_t* xs = reinterpret_cast<uint16_t*>(base);
     base += split_copy_bytes((size_t)g.batch * g.cin * x_cs, parts);
     uint16_t* gs = reinterpret_cast<uint16_t*>(base);
     base += split_copy_bytes((size_t)g.batch * g.cout * g_cs, parts);
-    if (dtype == JG_F16) sum32 = reinterpret_cast<float*>(base);
-    base += acc32_bytes(g, dtype);
     one_block_tmp = reinterpret_cast<float*>(base);
     int rc = split_parts_bf16(xs, x, dtype, (size_t)g.batch, (size_t)g.cin * x_cs, s);
     if (rc) return rc;
@@ -816,11 +829,11 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
     p.g = static_cast<const uint16_t*>(go) + gch * g_cs;
     p.bias_part = gb_out != nullptr ? p.part + (size_t)wgs * HALVES * 9 * cob * (bl.KD * cib) : nullptr;
     int rc;
-    if (cgb == 2 && cxb == 2) rc = launch<2, 2>(p, even, wgs, s, who);
-    else if (cgb == 1 && cxb == 3) rc = launch<1, 3>(p, even, wgs, s, who);
-    else if (cgb == 1 && cxb == 1) rc = launch<1, 1>(p, even, wgs, s, who);
-    else if (cgb == 2 && cxb == 1) rc = launch<2, 1>(p, even, wgs, s, who);
-    else if (cgb == 1 && cxb == 2) rc = launch<1, 2>(p, even, wgs, s, who);
+    if (cgb == 2 && cxb == 2) rc = launch<2, 2>(p, even, f16, wgs, s, who);
+    else if (cgb == 1 && cxb == 3) rc = launch<1, 3>(p, even, f16, wgs, s, who);
+    else if (cgb == 1 && cxb == 1) rc = launch<1, 1>(p, even, f16, wgs, s, who);
+    else if (cgb == 2 && cxb == 1) rc = launch<2, 1>(p, even, f16, wgs, s, who);
+    else if (cgb == 1 && cxb == 2) rc = launch<1, 2>(p, even, f16, wgs, s, who);
     else JG_FAIL(JG_ERR_UNSUPPORTED, "%s: channel blocking (%d, %d) not built", who, cgb, cxb);
     if (rc) return rc;
     JG_CHECK_LAUNCH(who);
@@ -859,12 +872,12 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
       const size_t blk_at = ((size_t)co0 * g.cin + ci0) * bl.KD * 9;
       for (int pr = 0; pr < npairs; ++pr) {
         const int gpart = kPairs[first_pair + pr][0], xpart = kPairs[first_pair + pr][1];
-        void* out = split ? static_cast<void*>(sum32 + blk_at)
-                          : static_cast<void*>(static_cast<uint16_t*>(gw) + blk_at);
+        void* out = (split || f16) ? static_cast<void*>(sum32 + blk_at)
+                                   : static_cast<void*>(static_cast<uint16_t*>(gw) + blk_at);
         // the bias gradient comes from the g rows: once per block of output channels
         uint16_t* gb_out = (gb != nullptr && ci0 == 0) ? static_cast<uint16_t*>(gb) + co0 : nullptr;
         int rc = run_block((size_t)gpart * g.cout + co0, (size_t)xpart * g.cin + ci0, cob, cib, cout_valid, cin_valid,
-                           out, g.cin, split, pr > 0, gb_out);
+                           out, g.cin, split || f16, pr > 0, gb_out);
         if (rc) return rc;
       }
       ci0 += cib;
