@@ -1,6 +1,6 @@
 // C entry points of the attention core: validate and route to the MFMA flash
-// kernels (head size 64; head sizes 96 and 128) when they cover the problem, to the
-// window or generic kernels otherwise.
+// kernels (bf16 at head size 64; bf16 / fp16 at head sizes 96 and 128) when they cover
+// the problem, to the window or generic kernels otherwise.
 #include <initializer_list>
 
 #include "jg_common.h"
@@ -88,7 +88,8 @@ extern "C" int jg_attn_fwd(void* out, float* lse, const void* q, const void* k, 
     JG_FAIL(JG_ERR_UNSUPPORTED, "%s: head size %lld not in {8, 16, 32, 64, 96, 128}", who, (long long)d);
   if (out_acc != nullptr)
     JG_FAIL(JG_ERR_UNSUPPORTED,
-            "%s: the fused merge needs an MFMA path (bf16, d in {64, 96, 128}, sq %% 128 == 0, sk %% 128 == 0);"
+            "%s: the fused merge needs an MFMA path (bf16 with d in {64, 96, 128} or fp16 with d in {96, 128},"
+            " sq %% 128 == 0, sk %% 128 == 0);"
             " call jg_lse_merge after the core instead", who);
   rc = jg::attn_generic_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, (int)d, scale, bias,
                             bias_period, dtype, s);
