@@ -143,6 +143,29 @@ def attention_figures(dev, iters: int) -> dict:
     out, l = ja.ring_forward(q, ks, vs, scale)
     ms_b = time_gpu(lambda: ja.core_backward(dout, q, ks[0], vs[0], out, l, scale), iters)
     ms_ring = time_gpu(lambda: ja.ring_forward(q, ks, vs, scale), iters)
+    # The same ring with the K/V hop in the loop: every step receives the next chunk, on the compute
+    # thread or on a side stream. A device copy of the 8 MiB stands in for the neighbour's transfer;
+    # "link" adds one copy of 128 MiB, about the 55 us the 8 MiB take over one 153 GB/s xGMI link.
+    from jigsaw_amd import ring as jr
+
+    kvs = [torch.stack((k, v)) for k, v in zip(ks, vs)]
+    side = torch.cuda.Stream()
+
+    pad_src = torch.empty(128 << 20, dtype=torch.uint8, device=dev)
+    pad_dst = torch.empty_like(pad_src)
+
+    def ring_with_hop(link, stream):
+        def send(src, buf, *, direction, group, async_op, tag):
+            if link:
+                pad_dst.copy_(pad_src)
+            buf.copy_(kvs[(tag + 1) % P])
+            return buf, None
+
+        return time_gpu(lambda: jr.ring_forward_from_provider(
+            q, jr.RingKVProvider(ks[0], vs[0], 0, P, send, comm_stream=stream), scale), iters)
+
+    hop = {"ms_copy_inline": ring_with_hop(False, None), "ms_copy_side_stream": ring_with_hop(False, side),
+           "ms_link_inline": ring_with_hop(True, None), "ms_link_side_stream": ring_with_hop(True, side)}
     x = torch.randn(b, n, 256, device=dev, generator=g).bfloat16()
     ms_ln = time_gpu(lambda: jl.partial_stats(x), iters)
     tf = lambda f, ms: f / (ms * 1e-3) / 1e12  # noqa: E731
@@ -150,6 +173,7 @@ def attention_figures(dev, iters: int) -> dict:
         "attn_fwd_step": {"ms": ms_f, "tflops": tf(f_fwd, ms_f), "frac_mfma_peak": tf(f_fwd, ms_f) / PEAK_BF16_TFLOPS},
         "attn_bwd_step": {"ms": ms_b, "tflops": tf(f_bwd, ms_b), "frac_mfma_peak": tf(f_bwd, ms_b) / PEAK_BF16_TFLOPS},
         "attn_ring_fwd_4_steps": {"ms": ms_ring, "tflops": tf(4 * f_fwd, ms_ring)},
+        "attn_ring_fwd_4_steps_with_hop": hop,
         "ln_partial_stats": {"ms": ms_ln, "GBps": x.numel() * 2 / (ms_ln * 1e-3) / 1e9, "bytes": x.numel() * 2},
     }
 
