@@ -738,7 +738,9 @@ int jg_proj_nt(void* out, const void* a, const void* w, const void* bias, int dt
   p.rows = rows; p.N = n_out; p.K = k_in;
   // 256 x 256 tiles (half the operand traffic per MFMA) once they fill the chip, else 128 x 128
   const long long big_tiles = (long long)jg::cdiv(rows, 256) * jg::cdiv(n_out, 256);
-  if (big_tiles >= 256) return launch_nt<4, 2, 2, 4>(p, s, who);
+  // the 256-wide tile only where its last column of tiles is more than half full
+  const int waste = jg::cdiv(n_out, 256) * 256 - n_out;
+  if (big_tiles >= 256 && waste < 128) return launch_nt<4, 2, 2, 4>(p, s, who);
   return launch_nt<2, 2, 2, 2>(p, s, who);
 }
 
