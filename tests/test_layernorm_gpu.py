@@ -182,3 +182,36 @@ def test_plain_layer_norm_defaults_and_fallback(dev):
     torch.testing.assert_close(jl.plain_layer_norm(x2, w2, b2).cpu(), F.layer_norm(x2.cpu(), (130,), w2.cpu(), b2.cpu()),
                                atol=1e-5, rtol=1e-5)
     assert jl.plain_layer_norm(x[:0], w, b).shape == (0, 50, 128)
+
+
+def test_plain_layer_norm_entry_point_refuses_what_it_cannot_do(dev):
+    """Through the C ABI: widths that are not a multiple of 8 or beyond 2048 columns are 'unsupported'
+    (status -2, NotImplementedError), a bf16 input with an fp16 output is a bad argument (status -1)."""
+    from jigsaw_amd import _lib
+
+    lib = _lib.load()
+    assert lib.jg_ln_plain_supported(128) == 1 and lib.jg_ln_plain_supported(2048) == 1
+    assert lib.jg_ln_plain_supported(12) == 0 and lib.jg_ln_plain_supported(2056) == 0 and lib.jg_ln_plain_supported(4) == 0
+    x = torch.randn(4, 16, device=dev)
+    y, mean, rstd, w = torch.empty_like(x), torch.empty(4, device=dev), torch.empty(4, device=dev), torch.ones(16, device=dev)
+
+    def call(cols, x_dt, y_dt):
+        return lib.jg_ln_plain_fwd(_lib.ptr(y), _lib.ptr(mean), _lib.ptr(rstd), _lib.ptr(x), _lib.ptr(w), None, 4, cols, 1e-5,
+                                   x_dt, y_dt, _lib.stream_ptr(dev))
+
+    f32, bf16, f16 = (_lib.dtype_code(t) for t in (torch.float32, torch.bfloat16, torch.float16))
+    assert call(16, f32, f32) == 0
+    assert call(12, f32, f32) == -2
+    assert call(16, bf16, f16) == -1
+    with pytest.raises(NotImplementedError):
+        _lib.check(call(12, f32, f32), "jg_ln_plain_fwd")
+    torch.cuda.synchronize()
+
+
+def test_plain_layer_norm_takes_non_contiguous_input(dev):
+    torch.manual_seed(13)
+    x = torch.randn(6, 64, 10, device=dev).transpose(1, 2)  # (6, 10, 64) view with strides
+    w, b = torch.randn(64, device=dev), torch.randn(64, device=dev)
+    got = jl.plain_layer_norm(x, w, b)
+    want = F.layer_norm(x.cpu().double(), (64,), w.cpu().double(), b.cpu().double())
+    assert rel_l2(got.cpu(), want) < 1e-5

@@ -77,3 +77,18 @@ def test_provider_argument_errors(dev):
     prov = jr.RingKVProvider(k, k, 0, 2, send)
     with pytest.raises(ValueError):
         prov.get(1)  # step 0 first
+
+
+def test_provider_ring_in_fp16_with_the_fused_step(dev):
+    """fp16 at head size 128 runs the fused step kernel; the provider loop still equals the list loop."""
+    torch.manual_seed(8)
+    P, shape = 3, (1, 2, 128, 128)
+    q = (torch.randn(*shape) / 128 ** 0.5).half().to(dev)
+    ks = [torch.randn(*shape).half().to(dev) for _ in range(P)]
+    vs = [torch.randn(*shape).half().to(dev) for _ in range(P)]
+    side = torch.cuda.Stream()
+    prov = jr.RingKVProvider(ks[1], vs[1], 1, P, _neighbour(ks, vs, 1, [], with_work=False), comm_stream=side)
+    out, lse = jr.ring_forward_from_provider(q, prov, 128 ** -0.5)
+    want_o, want_l = ja.ring_forward(q, ks, vs, 128 ** -0.5, rank=1)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float16 and torch.equal(out, want_o) and torch.equal(lse, want_l)
