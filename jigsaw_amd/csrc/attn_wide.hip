@@ -175,6 +175,23 @@ __device__ __forceinline__ u32x2 pack4(float a, float b, float c, float d) {
   return r;
 }
 
+// Workgroup -> (batch entry, row block). Consecutive workgroup ids go to the 8 XCDs in turn; each
+// XCD is given a contiguous range of (batch entry, block) pairs, so the workgroups that stream the
+// same K / V (or Q / dO) share one L2. Falls back to the plain order when the count does not divide.
+struct BlockOf {
+  long long bh;
+  int blk;
+};
+__device__ __forceinline__ BlockOf block_of() {
+  const unsigned nblk = gridDim.x, total = gridDim.x * gridDim.y;
+  unsigned id = blockIdx.y * gridDim.x + blockIdx.x;
+  if ((total & 7u) == 0) id = (id & 7u) * (total >> 3) + (id >> 3);
+  BlockOf b;
+  b.bh = id / nblk;
+  b.blk = (int)(id % nblk);
+  return b;
+}
+
 struct Args {
   const uint16_t* q;
   const uint16_t* k;
@@ -203,8 +220,9 @@ __global__ __launch_bounds__(THREADS) void attn_wide_fwd_kernel(Args p) {
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int ln = lane & 31, kg = lane >> 5;
-  const long long bh = blockIdx.y;
-  const int qi = blockIdx.x * BQ + wave * 32 + ln;
+  const BlockOf wg = block_of();
+  const long long bh = wg.bh;
+  const int qi = wg.blk * BQ + wave * 32 + ln;
   const uint16_t* qrow = p.q + (bh * p.sq + qi) * D;
   const uint16_t* kb = p.k + bh * p.sk * D;
   const uint16_t* vb = p.v + bh * p.sk * D;
@@ -323,8 +341,9 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dq_kernel(Args p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int ln = lane & 31, kg = lane >> 5;
-  const long long bh = blockIdx.y;
-  const int qi = blockIdx.x * BQ + wave * 32 + ln;
+  const BlockOf wg = block_of();
+  const long long bh = wg.bh;
+  const int qi = wg.blk * BQ + wave * 32 + ln;
   const long long qoff = (bh * p.sq + qi) * D;
   const uint16_t* kb = p.k + bh * p.sk * D;
   const uint16_t* vb = p.v + bh * p.sk * D;
@@ -413,8 +432,9 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int ln = lane & 31, kg = lane >> 5;
-  const long long bh = blockIdx.y;
-  const int ki = blockIdx.x * BQ + wave * 32 + ln;
+  const BlockOf wg = block_of();
+  const long long bh = wg.bh;
+  const int ki = wg.blk * BQ + wave * 32 + ln;
   const long long koff = (bh * p.sk + ki) * D;
   const uint16_t* qb = p.q + bh * p.sq * D;
   const uint16_t* gb = p.dout + bh * p.sq * D;
