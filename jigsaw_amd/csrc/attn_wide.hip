@@ -423,10 +423,16 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dq_kernel(Args p) {
 }
 
 // ------------------------------------------------------------------- dK, dV
-template <int D, bool F16>
-__global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
+// MODE 0 forms dK and dV in one pass (two d x 32 accumulators a wavefront). That fits two workgroups
+// per CU in 256 registers a lane at head size 96 but not at 128 (it would spill, and ran 1.3x slower
+// that way), so head size 128 runs the kernel twice: MODE 1 forms dV only (from P), MODE 2 dK only
+// (from dS), each with one accumulator and two workgroups per CU; the scores are computed in both.
+// A launch with no more workgroups than CUs gains nothing from that and keeps the single pass.
+template <int D, bool F16, int MODE>
+__global__ __launch_bounds__(THREADS, (D <= 96 || MODE != 0) ? 2 : 1) void attn_wide_dkv_kernel(Args p) {
   typedef Geo<D> G;
   typedef typename Half<F16>::x8 X8;
+  constexpr bool DV = MODE != 2, DK = MODE != 1;
   constexpr int STATS = 2 * BT * 4;                           // lse * log2(e) and delta of the tile's queries
   constexpr int BUF = 2 * G::ROWMAJ + 2 * G::TRANS + STATS;   // Q rows, dO rows, Q^T, dO^T, stats
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -442,28 +448,28 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
   const float* db = p.delta + bh * p.sq;
   const float c2 = p.scale * LOG2E;
 
-  X8 kf[G::C16], vf[G::C16];
+  X8 kf[G::C16], vf[DK ? G::C16 : 1];
 #pragma unroll
   for (int c = 0; c < G::C16; ++c) {
     kf[c] = frag<F16>(reinterpret_cast<const unsigned char*>(p.k + koff + 16 * c + 8 * kg));
-    vf[c] = frag<F16>(reinterpret_cast<const unsigned char*>(p.v + koff + 16 * c + 8 * kg));
+    if (DK) vf[c] = frag<F16>(reinterpret_cast<const unsigned char*>(p.v + koff + 16 * c + 8 * kg));
   }
-  f32x16 dk[G::NB], dv[G::NB];
+  f32x16 dk[DK ? G::NB : 1], dv[DV ? G::NB : 1];
 #pragma unroll
   for (int nb = 0; nb < G::NB; ++nb) {
-    dk[nb] = zero16();
-    dv[nb] = zero16();
+    if (DK) dk[nb] = zero16();
+    if (DV) dv[nb] = zero16();
   }
 
-  TileRegs<D> rq, rg;
-  TransRegs<D> rqt, rgt;
+  TileRegs<D> rq, rg;        // Q rows (scores); dO rows (dP: dK only)
+  TransRegs<D> rqt, rgt;     // Q^T (dK only); dO^T (dV only)
   float st = 0.0f;  // one statistic per thread of the first wavefront: lse2 (lanes 0-31) or delta (32-63)
   const int ntiles = p.sq / BT;
   auto fetch = [&](int t) {
     tile_fetch<D>(rq, qb + (long long)t * BT * D);
-    tile_fetch<D>(rg, gb + (long long)t * BT * D);
-    trans_fetch<D>(rqt, qb + (long long)t * BT * D);
-    trans_fetch<D>(rgt, gb + (long long)t * BT * D);
+    if (DK) tile_fetch<D>(rg, gb + (long long)t * BT * D);
+    if (DK) trans_fetch<D>(rqt, qb + (long long)t * BT * D);
+    if (DV) trans_fetch<D>(rgt, gb + (long long)t * BT * D);
     if (threadIdx.x < 2 * BT) {
       const float* src = threadIdx.x < BT ? lb : db;  // every lane loads; the factor is applied when stored
       st = src[t * BT + (threadIdx.x & (BT - 1))];
@@ -472,9 +478,9 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
   auto store = [&](int buf) {
     unsigned char* base = smem + buf * BUF;
     tile_store_rows<D>(rq, base);
-    tile_store_rows<D>(rg, base + G::ROWMAJ);
-    trans_store<D>(rqt, base + 2 * G::ROWMAJ);
-    trans_store<D>(rgt, base + 2 * G::ROWMAJ + G::TRANS);
+    if (DK) tile_store_rows<D>(rg, base + G::ROWMAJ);
+    if (DK) trans_store<D>(rqt, base + 2 * G::ROWMAJ);
+    if (DV) trans_store<D>(rgt, base + 2 * G::ROWMAJ + G::TRANS);
     if (threadIdx.x < 2 * BT)
       reinterpret_cast<float*>(base + 2 * G::ROWMAJ + 2 * G::TRANS)[threadIdx.x] = threadIdx.x < BT ? st * LOG2E : st;
   };
@@ -493,13 +499,14 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
 #pragma unroll
     for (int c = 0; c < G::C16; ++c) {
       s = Half<F16>::mma(frag<F16>(qt + ln * G::RP + (16 * c + 8 * kg) * 2), kf[c], s);
-      dp = Half<F16>::mma(frag<F16>(gt + ln * G::RP + (16 * c + 8 * kg) * 2), vf[c], dp);
+      if (DK) dp = Half<F16>::mma(frag<F16>(gt + ln * G::RP + (16 * c + 8 * kg) * 2), vf[c], dp);
     }
     float pr[16], ds[16];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const f32x4 l4 = *reinterpret_cast<const f32x4*>(stats + 8 * j + 4 * kg);
-      const f32x4 d4 = *reinterpret_cast<const f32x4*>(stats + BT + 8 * j + 4 * kg);
+      f32x4 d4 = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (DK) d4 = *reinterpret_cast<const f32x4*>(stats + BT + 8 * j + 4 * kg);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int i = 4 * j + e;
@@ -509,13 +516,17 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
     }
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      const X8 pf = pack8<F16>(pr + 8 * ks), dsf = pack8<F16>(ds + 8 * ks);
+      if (DV) {
+        const X8 pf = pack8<F16>(pr + 8 * ks);
 #pragma unroll
-      for (int nb = 0; nb < G::NB; ++nb) {
-        dv[nb] = Half<F16>::mma(frag<F16>(gtt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2), pf,
-                                                         dv[nb]);
-        dk[nb] = Half<F16>::mma(frag<F16>(qtt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2), dsf,
-                                                         dk[nb]);
+        for (int nb = 0; nb < G::NB; ++nb)
+          dv[nb] = Half<F16>::mma(frag<F16>(gtt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2), pf, dv[nb]);
+      }
+      if (DK) {
+        const X8 dsf = pack8<F16>(ds + 8 * ks);
+#pragma unroll
+        for (int nb = 0; nb < G::NB; ++nb)
+          dk[nb] = Half<F16>::mma(frag<F16>(qtt + (nb * 32 + ln) * G::TP + (16 * ks + 8 * kg) * 2), dsf, dk[nb]);
       }
     }
     if (t + 1 < ntiles) store((t + 1) & 1);
@@ -527,12 +538,27 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dkv_kernel(Args p) {
   for (int nb = 0; nb < G::NB; ++nb)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      *reinterpret_cast<u32x2*>(krow + nb * 32 + 8 * j + 4 * kg) =
-          pack4<F16>(dk[nb][4 * j] * p.scale, dk[nb][4 * j + 1] * p.scale, dk[nb][4 * j + 2] * p.scale,
-                dk[nb][4 * j + 3] * p.scale);
-      *reinterpret_cast<u32x2*>(vrow + nb * 32 + 8 * j + 4 * kg) =
-          pack4<F16>(dv[nb][4 * j], dv[nb][4 * j + 1], dv[nb][4 * j + 2], dv[nb][4 * j + 3]);
+      if (DK)
+        *reinterpret_cast<u32x2*>(krow + nb * 32 + 8 * j + 4 * kg) =
+            pack4<F16>(dk[nb][4 * j] * p.scale, dk[nb][4 * j + 1] * p.scale, dk[nb][4 * j + 2] * p.scale,
+                       dk[nb][4 * j + 3] * p.scale);
+      if (DV)
+        *reinterpret_cast<u32x2*>(vrow + nb * 32 + 8 * j + 4 * kg) =
+            pack4<F16>(dv[nb][4 * j], dv[nb][4 * j + 1], dv[nb][4 * j + 2], dv[nb][4 * j + 3]);
     }
+}
+
+int cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cus = n;
+    else
+      cus = 256;
+  }
+  return cus;
 }
 
 template <int D, bool F16>
@@ -548,16 +574,27 @@ int launch_bwd(const Args& a, long long batch, hipStream_t s) {
   constexpr int DQ_LDS = 2 * (2 * G::ROWMAJ + G::TRANS);
   constexpr int DKV_LDS = 2 * (2 * G::ROWMAJ + 2 * G::TRANS + 2 * BT * 4);
   void (*dqk)(Args) = &attn_wide_dq_kernel<D, F16>;
-  void (*dkvk)(Args) = &attn_wide_dkv_kernel<D, F16>;
   hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(dqk), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       DQ_LDS);
-  hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(dkvk), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      DKV_LDS);
-  if (e1 != hipSuccess || e2 != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "jg_attn_bwd(wide): cannot reserve LDS");
+  if (e1 != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "jg_attn_bwd(wide): cannot reserve LDS");
   dqk<<<dim3((unsigned)(a.sq / BQ), (unsigned)batch, 1), THREADS, DQ_LDS, s>>>(a);
   JG_CHECK_LAUNCH("jg_attn_bwd(wide, dq)");
-  dkvk<<<dim3((unsigned)(a.sk / BQ), (unsigned)batch, 1), THREADS, DKV_LDS, s>>>(a);
-  JG_CHECK_LAUNCH("jg_attn_bwd(wide, dkv)");
+  // head size 96: dK and dV in one pass; head size 128: one pass each when the launch has more
+  // workgroups than the chip has CUs (register budget, see the kernel)
+  void (*passes[2])(Args) = {&attn_wide_dkv_kernel<D, F16, 0>, nullptr};
+  if constexpr (D > 96) {
+    if ((long long)(a.sk / BQ) * batch > cu_count()) {
+      passes[0] = &attn_wide_dkv_kernel<D, F16, 1>;
+      passes[1] = &attn_wide_dkv_kernel<D, F16, 2>;
+    }
+  }
+  for (int i = 0; i < 2 && passes[i] != nullptr; ++i) {
+    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(passes[i]),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, DKV_LDS);
+    if (e2 != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "jg_attn_bwd(wide): cannot reserve LDS");
+    passes[i]<<<dim3((unsigned)(a.sk / BQ), (unsigned)batch, 1), THREADS, DKV_LDS, s>>>(a);
+    JG_CHECK_LAUNCH("jg_attn_bwd(wide, dkv)");
+  }
   return JG_OK;
 }
 
