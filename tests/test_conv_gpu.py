@@ -1,6 +1,6 @@
 """HIP convolution kernels against the oracle (torch CPU operators in fp64) (GPU).
 
-Tolerances (rel-L2 of the whole tensor): fp32 tensors 1e-5, bf16 / fp16 tensors 2e-2,
+Tolerances (rel-L2 of the whole tensor): fp32 tensors 1e-5, bf16 tensors 2e-2, fp16 tensors 2e-3,
 as the north-star states; the reference's own conv tests use atol/rtol 1e-4 for
 y / dx / db and a looser bound for dw (tests/modules/convolution/conv/test_conv2d_multi_spatial.py:207-233).
 """
@@ -18,7 +18,7 @@ from oracle import halo as oh
 
 pytestmark = pytest.mark.gpu
 
-TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 2e-3}
 
 PRIM_CASES = [
     # (N, Cin, Cout, in spatial, kernel, stride, padding, dilation)
