@@ -1,7 +1,7 @@
 """HIP convolution kernels against the oracle (torch CPU operators in fp64) (GPU).
 
-Tolerances (rel-L2 of the whole tensor): fp32 tensors 1e-5, bf16 tensors 2e-2, fp16 tensors 2e-3,
-as the north-star states; the reference's own conv tests use atol/rtol 1e-4 for
+Tolerances (rel-L2 of the whole tensor): fp32 tensors 1e-5 and bf16 tensors 2e-2, as the north-star
+states, fp16 tensors 2e-3; the reference's own conv tests use atol/rtol 1e-4 for
 y / dx / db and a looser bound for dw (tests/modules/convolution/conv/test_conv2d_multi_spatial.py:207-233).
 """
 
