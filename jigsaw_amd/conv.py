@@ -598,6 +598,7 @@ def conv_halo_nway(x, w, b, stride, padding, dilation, spatial_groups, channel_g
         # The padded tensor that is returned is then NOT a full copy: its consumer is
         # conv_halo_nway_backward with x_tile given (what _ConvNd of this module does).
         x_frame = halo_assemble(x, recv, geom, bands=bands)
+        x_frame._jg_frame_only = True  # read by conv_halo_nway_backward: no weight gradient without the tile
         y = conv_nd_framed(x_frame, x, geom, w, b, **kwargs)
         if y is None:
             raise RuntimeError("framed forward: " + _lib.load().jg_last_error().decode())
@@ -627,6 +628,12 @@ def conv_halo_nway_backward(
     g = grad_output.to(weight.dtype)
     kwargs = {"stride": stride, "padding": local_padding, "dilation": dilation, "groups": 1}
     g_w = g_b = None
+    if x_tile is None and need_w and getattr(config, "framed", False) and getattr(x_aug, "_jg_frame_only", False):
+        raise RuntimeError(
+            "x_aug is the frame of a framed forward (config.framed) and its interior is undefined: the weight "
+            "gradient needs the rank's tile as x_tile=. Use _ConvNd of this package, which keeps the tile, or "
+            "build the config without framed=True."
+        )
     if x_tile is not None:
         # x_aug is the frame that the framed forward built (conv_halo_nway with config.framed)
         if need_w:
@@ -665,40 +672,124 @@ def conv_halo_nway_backward(
     return done(g_x)
 
 
-class HipConvNdConfig:
-    """Kernel table of one distributed convolution layer, HIP edition.
+_CHANNEL_COMMS = ("auto", "all_to_all", "isend", "batch_isend_irecv")
 
-    Carries the attributes ``_ConvNd`` and the two ``dist_conv_*`` functions read
-    from the reference's ``ConvNdConfig`` (config.py:62-95): ``n_spatial``,
-    ``conv_fn``, ``conv_input_fn``, ``conv_weight_fn``, ``grad_bias``,
-    ``dist_conv_fn``, ``dist_conv_backward_fn``, plus ``halo_exchange``.
-    """
+
+def _resolve_channel_comm(channel_comm: Any, device: Any) -> str:
+    """The string a layer finds in ``config.channel_comm`` (and hands back when it rebuilds
+    the config for a new channel group): ``"all_gather"`` is kept, ``"auto"`` becomes the
+    transport of the device, unknown names raise ``ValueError``
+    (jigsaw/modules/convolution/_common/channel_comm.py:25-58, jigsaw/_core/comm.py:101-137)."""
+    if channel_comm == "all_gather":
+        return "all_gather"
+    name = str(getattr(channel_comm, "value", channel_comm)).lower()
+    if name not in _CHANNEL_COMMS:
+        raise ValueError(f"channel_comm must be 'all_gather' or one of {list(_CHANNEL_COMMS)}, got {channel_comm!r}")
+    kind = getattr(device, "type", str(device).split(":")[0]) if device is not None else "cuda"
+    if kind not in ("cuda", "cpu"):
+        raise ValueError(f"Unsupported device {kind}")
+    if name == "auto":
+        return "all_to_all" if kind == "cuda" else "batch_isend_irecv"
+    if name == "all_to_all" and kind != "cuda":
+        raise ValueError(f"comm='all_to_all' needs a GPU, got device {kind!r}; use 'isend' or 'batch_isend_irecv'")
+    return name
+
+
+def layer_key(channel_group: Any, bias: Any, kernel_size, stride, groups: int) -> dict:
+    """The properties of a layer a kernel table is built for; the reference's layers compare
+    them entry by entry with their own and refuse a table built for another layer
+    (jigsaw/modules/convolution/_common/config.py:9-43, jigsaw/_core/config.py:6-34)."""
+    return {
+        "n_spatial": len(kernel_size),
+        "bias": bias is not None,
+        "kernel_size == stride": tuple(kernel_size) == tuple(stride),
+        "groups": groups,
+        "channel group size": channel_group.size(),
+    }
+
+
+class _HipLayerConfig:
+    """What the two kernel tables share: the constructor arguments of the reference's
+    configs in their order (a layer rebuilds its config as
+    ``type(config)(channel_group, bias, kernel_size, stride, device, channel_comm, groups)``,
+    jigsaw/modules/convolution/_conv/base.py:572-580), the ``_layer_key`` the layer
+    validates, and the options of this package, which live on the CLASS so that such a
+    rebuild keeps them (see :meth:`bound`)."""
 
     vmapped = False
-    channel_local = True
-    fused_fold = True  # dgrad + pack + fold in one pass where the MFMA kernel covers the shape
-    fused_bias_grad = True  # bias gradient from the weight-gradient kernel's pass over g
-    groups = 1
-    groups_local = 1
+    halo_exchange: HaloExchange | None = None  # transport of the strips; None on a 1 x ... x 1 mesh
 
-    def __init__(self, n_spatial: int, bias: Any, halo_exchange: HaloExchange | None = None, framed: bool = False) -> None:
-        self.n_spatial = int(n_spatial)
-        # framed: build only the frame of the padded tile (needs _ConvNd of this module, which keeps the tile)
-        self.framed = bool(framed)
-        self.halo_exchange = halo_exchange
-        self.conv_fn = conv_nd
-        self.native_conv_fn = conv_nd
-        self.conv_input_fn = conv_nd_input
-        self.conv_weight_fn = conv_nd_weight
+    def __init__(self, channel_group: Any, bias: Any, kernel_size, stride, device: Any = None,
+                 channel_comm: Any = "auto", groups: int = 1, **options: Any) -> None:
+        unknown = set(options) - set(self._OPTIONS)
+        if unknown:
+            raise TypeError(f"unknown option(s) {sorted(unknown)}; this config takes {list(self._OPTIONS)}")
+        for name, value in options.items():
+            setattr(self, name, value)
+        kernel_size, stride = tuple(kernel_size), tuple(stride)
+        if len(kernel_size) != len(stride):
+            raise ValueError(f"kernel_size {kernel_size} and stride {stride} differ in length")
+        self.n_spatial = len(kernel_size)
+        self.channel_comm = _resolve_channel_comm(channel_comm, device)
+        self.groups = int(groups)
+        self._layer_key = layer_key(channel_group, bias, kernel_size, stride, groups)
+        size = channel_group.size()
+        self.channel_local = groups % size == 0
+        self.groups_local = groups // size if self.channel_local else 1
+        if size != 1 or groups != 1:
+            raise NotImplementedError(
+                "the HIP kernel table covers channel-local layers with groups = 1 "
+                f"(channel group size {size}, groups {groups})"
+            )
         self.grad_bias = self._no_bias if bias is None else self._sum_grad_bias
-        self.dist_conv_fn = conv_halo_nway
-        self.dist_conv_backward_fn = conv_halo_nway_backward
+
+    @classmethod
+    def bound(cls, **options: Any):
+        """A subclass with ``options`` (``halo_exchange=...``, ...) as class attributes, for
+        layers that rebuild their config from its type."""
+        unknown = set(options) - set(cls._OPTIONS)
+        if unknown:
+            raise TypeError(f"unknown option(s) {sorted(unknown)}; this config takes {list(cls._OPTIONS)}")
+        return type(cls.__name__, (cls,), dict(options))
+
+    @classmethod
+    def for_rank(cls, n_spatial: int, bias: Any, halo_exchange: HaloExchange | None = None, **options: Any):
+        """Short form for a channel-local layer whose kernel is not its stride (the layers
+        that exchange halos): only the number of spatial axes and the bias matter."""
+        return cls(TileGroup(1, 0), bias, (3,) * int(n_spatial), (1,) * int(n_spatial), None,
+                   halo_exchange=halo_exchange, **options)
 
     def _no_bias(self, *args: Any, **kwargs: Any) -> None:
         return None
 
     def _sum_grad_bias(self, grad_output: torch.Tensor) -> torch.Tensor:
         return sum_grad_bias(grad_output, self.n_spatial)
+
+
+class HipConvNdConfig(_HipLayerConfig):
+    """Kernel table of one distributed convolution layer, HIP edition: built like the
+    reference's ``ConvNdConfig`` (config.py:32-95) and carrying the attributes the layer,
+    ``_ConvNd`` and the two ``dist_conv_*`` functions read from it — ``_layer_key``,
+    ``n_spatial``, ``channel_comm``, ``groups``, ``channel_local``, ``groups_local``,
+    ``conv_fn``, ``native_conv_fn``, ``conv_input_fn``, ``conv_weight_fn``, ``grad_bias``,
+    ``dist_conv_fn``, ``dist_conv_backward_fn`` — plus this package's options."""
+
+    _OPTIONS = ("halo_exchange", "framed", "fused_fold", "fused_bias_grad")
+    framed = False  # build only the frame of the padded tile (needs _ConvNd of this module, which keeps the tile)
+    fused_fold = True  # dgrad + pack + fold in one pass where the MFMA kernel covers the shape
+    fused_bias_grad = True  # bias gradient from the weight-gradient kernel's pass over g
+
+    def __init__(self, channel_group: Any, bias: Any, kernel_size, stride, device: Any = None,
+                 channel_comm: Any = "auto", groups: int = 1, **options: Any) -> None:
+        super().__init__(channel_group, bias, kernel_size, stride, device, channel_comm, groups, **options)
+        self.conv_fn = conv_nd
+        self.native_conv_fn = conv_nd
+        self.conv_input_fn = conv_nd_input
+        self.conv_weight_fn = conv_nd_weight
+        # kernel == stride tiles the domain without overlap; conv_halo_nway finds no strips
+        # to exchange there and runs the local kernels only
+        self.dist_conv_fn = conv_halo_nway
+        self.dist_conv_backward_fn = conv_halo_nway_backward
 
 
 def _cast_to_autocast_dtype(*tensors):
@@ -747,12 +838,24 @@ class _ConvNd(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output, grad_x_aug):  # noqa: D102
+        config = ctx.config
         if ctx.framed:
             x_aug, weight, x_tile = ctx.saved_tensors
             x_tile = x_tile.to(x_aug.dtype)
+            if weight.dtype != x_aug.dtype:
+                # the forward ran in the autocast dtype, the backward runs in the weight's
+                # (functional.py:126-129): the framed kernels do not cover that, so the tile
+                # goes back into its frame and the padded tile takes the unframed route
+                n = config.n_spatial
+                ranks, sizes = _mesh_position(ctx.spatial_groups)
+                geom = HaloGeometry.for_conv(ctx.local_in_spatial, weight.shape[-n:], ctx.stride, ctx.padding,
+                                             ctx.dilation, ranks, sizes)
+                x_aug = x_aug.clone()
+                inner = tuple(slice(lo, lo + sz) for lo, sz in zip(geom.lo, geom.size))
+                x_aug[(Ellipsis, *inner)] = x_tile
+                x_tile = None
         else:
             (x_aug, weight), x_tile = ctx.saved_tensors, None
-        config = ctx.config
         x_aug = x_aug.to(weight.dtype)
         need_x, need_w, need_b = ctx.needs_input_grad[:3]
         need_b = need_b and ctx.has_bias
@@ -777,6 +880,7 @@ __all__ = [
     "HaloExchange",
     "HipConvNdConfig",
     "TileGroup",
+    "layer_key",
     "_ConvNd",
     "conv_halo_nway",
     "conv_halo_nway_backward",

@@ -21,8 +21,8 @@ from typing import Any
 import torch
 
 from .conv import (
-    HaloExchange,
     _cast_to_autocast_dtype,
+    _HipLayerConfig,
     _local_padding,
     _mesh_position,
     _present_offsets,
@@ -30,7 +30,6 @@ from .conv import (
     conv_nd_input,
     conv_nd_input_fold,
     conv_nd_weight,
-    sum_grad_bias,
 )
 from .halo import HaloGeometry, halo_assemble, halo_fold, halo_fold_border_, halo_pack
 
@@ -150,31 +149,22 @@ def conv_transpose_halo_nway_backward(
     return g_x, g_w
 
 
-class HipConvTransposeNdConfig:
-    """Kernel table of one distributed transposed convolution layer: the attributes
-    ``_ConvTransposeNd`` and the two ``dist_conv_transpose_*`` functions read from the
-    reference's ``ConvTransposeNdConfig`` (config.py:47-84), plus ``halo_exchange``."""
+class HipConvTransposeNdConfig(_HipLayerConfig):
+    """Kernel table of one distributed transposed convolution layer: built like the
+    reference's ``ConvTransposeNdConfig`` (_conv_transpose/config.py:47-84) and carrying
+    the attributes the layer, ``_ConvTransposeNd`` and the two ``dist_conv_transpose_*``
+    functions read from it, ``_layer_key`` included, plus ``halo_exchange``."""
 
-    vmapped = False
-    channel_local = True
+    _OPTIONS = ("halo_exchange", "fused_fold")
     fused_fold = True
-    groups = 1
-    groups_local = 1
 
-    def __init__(self, n_spatial: int, bias: Any, halo_exchange: HaloExchange | None = None) -> None:
-        self.n_spatial = int(n_spatial)
-        self.halo_exchange = halo_exchange
+    def __init__(self, channel_group: Any, bias: Any, kernel_size, stride, device: Any = None,
+                 channel_comm: Any = "auto", groups: int = 1, **options: Any) -> None:
+        super().__init__(channel_group, bias, kernel_size, stride, device, channel_comm, groups, **options)
         self.conv_transpose_fn = conv_transpose_nd
         self.native_conv_transpose_fn = conv_transpose_nd
-        self.grad_bias = self._no_bias if bias is None else self._sum_grad_bias
         self.dist_conv_transpose_fn = conv_transpose_halo_nway
         self.dist_conv_transpose_backward_fn = conv_transpose_halo_nway_backward
-
-    def _no_bias(self, *args: Any, **kwargs: Any) -> None:
-        return None
-
-    def _sum_grad_bias(self, grad_output: torch.Tensor) -> torch.Tensor:
-        return sum_grad_bias(grad_output, self.n_spatial)
 
 
 class _ConvTransposeNd(torch.autograd.Function):

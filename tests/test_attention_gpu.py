@@ -104,7 +104,9 @@ def test_ring_forward_backward_match_full_attention(b, h, n, d, P, dtype, rank, 
     out, lse = ja.ring_forward(q.to(dev), [t.to(dev) for t in ks], [t.to(dev) for t in vs], scale, rank=rank % P)
     assert out.dtype == dtype and lse.dtype == torch.float32
     assert rel_l2(out, full.detach()) < TOL[dtype], f"out {rel_l2(out, full.detach()):.3e}"
-    assert rel_l2(lse, torch.logsumexp(s.detach(), -1)) < 1e-3 if dtype != torch.float32 else 1e-5
+    lse_tol = 1e-5 if dtype == torch.float32 else 1e-3
+    lse_err = rel_l2(lse, torch.logsumexp(s.detach(), -1))
+    assert lse_err < lse_tol, f"lse {lse_err:.3e}"
     # the oracle's ring loop (its chunk order, merge form and roundings) agrees too
     o_or, l_or = oa.ring_forward(q.float(), [t.float() for t in ks], [t.float() for t in vs], scale, rank=rank % P)
     assert rel_l2(out, o_or) < TOL[dtype]
@@ -155,6 +157,51 @@ def test_config4_shape_properties(dev):
     want = torch.softmax(s, -1) @ V
     assert rel_l2(out[:, :, rows], want) < 2e-2
     assert rel_l2(lse[:, :, rows], torch.logsumexp(s, -1)) < 1e-4
+
+
+def test_config4_backward_shape_properties(dev):
+    """Config 4 backward at full size (8 heads, 4096 queries, 4 chunks of 4096 keys, d = 64,
+    bf16), from the GLOBAL out / lse as the ring holds them (backward.py:176-270).
+    Size-independent checks against fp64 on samples: the rows of ``sum_j dq_j`` for 128
+    sampled queries (each needs all 16384 keys), and the rows of ``dk_j`` / ``dv_j`` for 128
+    sampled keys of every chunk (each needs all 4096 queries); plus ``sum_j dq_j`` == dq of
+    one core call over the concatenated K/V."""
+    torch.manual_seed(5)
+    b, h, n, d, P = 1, 8, 4096, 64, 4
+    scale = d**-0.5
+    q = (torch.randn(b, h, n, d, device=dev) / 8).bfloat16()
+    ks = [torch.randn(b, h, n, d, device=dev).bfloat16() for _ in range(P)]
+    vs = [torch.randn(b, h, n, d, device=dev).bfloat16() for _ in range(P)]
+    dout = torch.randn(b, h, n, d, device=dev).bfloat16()
+    out, lse = ja.ring_forward(q, ks, vs, scale, rank=0)
+    dq, dks, dvs = ja.ring_backward(dout, q, out, lse, ks, vs, scale)
+    assert dq.dtype == torch.bfloat16 and len(dks) == P and len(dvs) == P
+
+    Kc, Vc = torch.cat(ks, 2), torch.cat(vs, 2)
+    dq_full, dk_full, dv_full = ja.backward(dout, q, Kc, Vc, out, lse, scale, n, P * n)
+    assert rel_l2(dq, dq_full) < 1e-2
+    assert rel_l2(torch.cat(dks, 2), dk_full) < 1e-2 and rel_l2(torch.cat(dvs, 2), dv_full) < 1e-2
+
+    # fp64 on the host from the same bf16 inputs and the same (rounded) global out / lse
+    Q, K, V = q.double().cpu(), Kc.double().cpu(), Vc.double().cpu()
+    dO, O, L = dout.double().cpu(), out.double().cpu(), lse.double().cpu()
+    D = (dO * O).sum(-1)  # (b, h, n)
+    rows = torch.arange(5, n, 32)
+    s = (Q[:, :, rows] @ K.mT) * scale
+    p = torch.exp(s - L[:, :, rows, None])
+    dp = dO[:, :, rows] @ V.mT
+    ds = p * (dp - D[:, :, rows, None]) * scale
+    assert rel_l2(dq[:, :, rows], ds @ K) < 2e-2, f"dq rows {rel_l2(dq[:, :, rows], ds @ K):.3e}"
+    keys = torch.arange(3, n, 32)
+    for j in range(P):
+        kj, vj = K[:, :, j * n + keys], V[:, :, j * n + keys]
+        s = (Q @ kj.mT) * scale  # (b, h, n, 128)
+        p = torch.exp(s - L[..., None])
+        want_dv = p.mT @ dO
+        ds = p * (dO @ vj.mT - D[..., None]) * scale
+        want_dk = ds.mT @ Q
+        assert rel_l2(dvs[j][:, :, keys], want_dv) < 2e-2, f"dv chunk {j}: {rel_l2(dvs[j][:, :, keys], want_dv):.3e}"
+        assert rel_l2(dks[j][:, :, keys], want_dk) < 2e-2, f"dk chunk {j}: {rel_l2(dks[j][:, :, keys], want_dk):.3e}"
 
 
 def test_window_attention_with_bias_and_mask(dev):

@@ -204,6 +204,24 @@ DIST_CASES = [
 def test_distributed_conv_matches_global_conv(case, dev):
     """The reference's parity method: every rank's y / dx and the summed dw / db equal
     the serial conv on the gathered tensor (test_conv2d_multi_spatial.py:73-233)."""
+    # bf16 cases also take the framed forward (only the frame of the padded tile is built)
+    _run_mesh_case(case, dev, framed=case[7] == torch.bfloat16, autocast=None)
+
+
+@pytest.mark.parametrize("framed", [False, True], ids=["assembled", "framed"])
+@pytest.mark.parametrize("case", [
+    ((2, 2), (32, 64), 1, 64, 64, (3, 3), (1, 1), torch.float32),
+    ((2, 2, 2), (8, 8, 16), 1, 32, 32, (3, 3, 3), (1, 1, 1), torch.float32),
+], ids=["2d", "3d"])
+def test_distributed_conv_under_autocast(case, framed, dev):
+    """fp32 leaves under bf16 autocast: the forward casts x / w / b down
+    (_core/autocast.py:44-66, functional.py:53), the backward runs outside autocast in the
+    weight's dtype on the saved bf16 padded tile (functional.py:126-129). Gradients come
+    back in the leaves' dtype. Bar: bf16 (the forward's operands are rounded to it)."""
+    _run_mesh_case(case, dev, framed=framed, autocast=torch.bfloat16)
+
+
+def _run_mesh_case(case, dev, framed, autocast):
     mesh, n, N, cin, cout, k, p, dtype = case[:8]
     ns = len(mesh)
     s, d = (case[8], case[9]) if len(case) > 8 else ((1,) * ns, (1,) * ns)
@@ -229,14 +247,15 @@ def test_distributed_conv_matches_global_conv(case, dev):
     # pass 1: forward of every rank, and the padded dgrad every rank will send from
     cfgs, outs, leaves, gx_need = {}, {}, {}, {}
     for c in mesh_coords(mesh):
-        # bf16 cases also take the framed forward (only the frame of the padded tile is built)
-        cfgs[c] = jc.HipConvNdConfig(ns, Bg, TableExchange(fwd_tabs[c], None), framed=dtype == torch.bfloat16)
+        cfgs[c] = jc.HipConvNdConfig.for_rank(ns, Bg, TableExchange(fwd_tabs[c], None), framed=framed)
         groups = tuple(jc.TileGroup(mesh[a], c[a]) for a in range(ns))
         xl = tiles[c].clone().requires_grad_()
         wl, bl = Wg.clone().requires_grad_(), Bg.clone().requires_grad_()
-        y, x_aug = jc._ConvNd.apply(xl, wl, bl, s, p, d, groups, None, cfgs[c])
+        with torch.autocast("cuda", dtype=autocast or torch.bfloat16, enabled=autocast is not None):
+            y, x_aug = jc._ConvNd.apply(xl, wl, bl, s, p, d, groups, None, cfgs[c])
         outs[c], leaves[c] = y, (xl, wl, bl)
         assert not x_aug.requires_grad
+        assert y.dtype == (autocast or dtype) and x_aug.dtype == (autocast or dtype)
         lp = oh.local_padding(p, mesh)
         gx_need[c] = jc.conv_nd_input(x_aug.shape, Wg, gtiles[c], stride=s, padding=lp, dilation=d)
     bwd_tabs = _recv_tables(gx_need, geoms, mesh, from_padded=True)
@@ -244,11 +263,12 @@ def test_distributed_conv_matches_global_conv(case, dev):
     # pass 2: backward of every rank
     gw_sum = torch.zeros_like(W, dtype=torch.float64)
     gb_sum = torch.zeros_like(B, dtype=torch.float64)
-    tol = TOL[dtype]
+    tol = TOL[autocast or dtype]
     for c in mesh_coords(mesh):
         cfgs[c].halo_exchange.bwd = bwd_tabs[c]
-        outs[c].backward(gtiles[c])
+        outs[c].backward(gtiles[c].to(outs[c].dtype))
         xl, wl, bl = leaves[c]
+        assert xl.grad.dtype == dtype and wl.grad.dtype == dtype and bl.grad.dtype == dtype
         sl = (slice(None), slice(None)) + tuple(slice(c[a] * n[a], (c[a] + 1) * n[a]) for a in range(ns))
         no = tuple(Y.shape[2 + a] // mesh[a] for a in range(ns))  # output rows per rank
         so = (slice(None), slice(None)) + tuple(slice(c[a] * no[a], (c[a] + 1) * no[a]) for a in range(ns))
@@ -261,9 +281,28 @@ def test_distributed_conv_matches_global_conv(case, dev):
     assert rel_l2(gb_sum, Bd.grad) < tol, f"db: {rel_l2(gb_sum, Bd.grad):.3e}"
 
 
+def test_frame_without_its_tile_is_refused(dev):
+    """A caller that keeps only ``x_aug`` (as the reference's own autograd function does)
+    cannot take the weight gradient from a frame: the backward says so instead of
+    reading the undefined interior."""
+    torch.manual_seed(0)
+    mesh, n = (2, 2), (32, 64)
+    X = torch.randn(1, 64, 64, 128).bfloat16()
+    tiles = {c: t.to(dev) for c, t in oh.split_global(X, mesh).items()}
+    geoms = {c: conv_geometry(n, mesh, c, (3, 3), (1, 1), (1, 1), (1, 1)) for c in tiles}
+    tabs = _recv_tables(tiles, geoms, mesh, from_padded=False)
+    c = (0, 1)
+    cfg = jc.HipConvNdConfig.for_rank(2, None, TableExchange(tabs[c], {}), framed=True)
+    groups = tuple(jc.TileGroup(mesh[a], c[a]) for a in range(2))
+    w = (torch.randn(64, 64, 3, 3) / 24).bfloat16().to(dev)
+    y, x_aug = jc.conv_halo_nway(tiles[c], w, None, (1, 1), (1, 1), (1, 1), groups, None, cfg)
+    with pytest.raises(RuntimeError, match="x_tile"):
+        jc.conv_halo_nway_backward(torch.ones_like(y), x_aug, w, (1, 1), (1, 1), (1, 1), n, groups, None, cfg)
+
+
 def test_first_layer_skips_dgrad(dev):
     """needs_input_grad gating (functional.py:131-148): no input grad -> no dgrad, no fold."""
-    cfg = jc.HipConvNdConfig(2, None, TableExchange({}, {}))
+    cfg = jc.HipConvNdConfig.for_rank(2, None, TableExchange({}, {}))
     x = torch.randn(1, 3, 8, 8, device=dev)
     w = torch.randn(4, 3, 3, 3, device=dev, requires_grad=True)
     groups = (jc.TileGroup(1, 0), jc.TileGroup(1, 0))
@@ -273,7 +312,7 @@ def test_first_layer_skips_dgrad(dev):
 
 
 def test_string_padding_is_rejected(dev):
-    cfg = jc.HipConvNdConfig(2, None, TableExchange({}, {}))
+    cfg = jc.HipConvNdConfig.for_rank(2, None, TableExchange({}, {}))
     x = torch.randn(1, 3, 8, 8, device=dev)
     w = torch.randn(4, 3, 3, 3, device=dev)
     with pytest.raises(NotImplementedError):

@@ -111,7 +111,7 @@ def test_distributed_transposed_conv_matches_global(case, dev):
     gb_sum = torch.zeros_like(B, dtype=torch.float64)
     no = tuple(Y.shape[2 + a] // mesh[a] for a in range(ns))
     for c in mesh_coords(mesh):
-        cfg = jct.HipConvTransposeNdConfig(ns, Bg, TableExchange(fwd_tabs[c], bwd_tabs[c]))
+        cfg = jct.HipConvTransposeNdConfig.for_rank(ns, Bg, TableExchange(fwd_tabs[c], bwd_tabs[c]))
         groups = tuple(jc.TileGroup(mesh[a], c[a]) for a in range(ns))
         xl = tiles[c].clone().requires_grad_()
         wl, bl = Wg.clone().requires_grad_(), Bg.clone().requires_grad_()

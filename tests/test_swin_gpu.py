@@ -123,3 +123,31 @@ def test_swin_block_bf16_config5_shape(dev):
     with torch.autocast("cuda", dtype=torch.bfloat16):
         out = block(x.to(dev))
     assert rel_l2(out, want) < 2e-2
+
+
+@pytest.mark.parametrize("shift,n", [(4, (256, 256)), (0, (64, 128)), (4, (64, 64))])
+def test_swin_block_bf16_backward_config5(shift, n, dev):
+    """Config 5's block (dim 128, 4 heads, 8x8 windows, shift 4, bf16 autocast, at its real
+    256 x 256 tile) forward AND backward on the bf16 kernels the benchmark times, against
+    autograd of the fp64 oracle block: rel-L2 2e-2 on the output, dx and every parameter
+    gradient."""
+    torch.manual_seed(3)
+    dim, heads, window = 128, 4, 8
+    x = torch.randn(1, *n, dim)
+    block = js.SwinBlock(dim, heads, window, n, shift=shift, device=dev)
+    with torch.no_grad():
+        block.attn.bias_table.normal_(0, 0.5)
+    params = {k: v.detach().double().cpu().requires_grad_() for k, v in block.state_dict().items()}
+    xd = x.double().requires_grad_()
+    want = osw.block(xd, params, heads, window, shift)
+    g = torch.randn_like(want)
+    want.backward(g)
+    xg = x.to(dev).requires_grad_()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = block(xg)
+    out.backward(g.to(out.dtype).to(dev))
+    assert rel_l2(out, want.detach()) < 2e-2, f"out {rel_l2(out, want.detach()):.3e}"
+    assert rel_l2(xg.grad, xd.grad) < 2e-2, f"dx {rel_l2(xg.grad, xd.grad):.3e}"
+    for name, prm in block.named_parameters():
+        err = rel_l2(prm.grad, params[name].grad)
+        assert err < 2e-2, f"{name}: {err:.3e}"
