@@ -797,7 +797,7 @@ def _cast_to_autocast_dtype(*tensors):
     (jigsaw/_core/autocast.py:44-66)."""
     if not torch.is_autocast_enabled():
         return tensors
-    dt = torch.get_autocast_gpu_dtype()
+    dt = torch.get_autocast_dtype("cuda")
     return tuple(t if t is None or not t.is_floating_point() else t.to(dt) for t in tensors)
 
 

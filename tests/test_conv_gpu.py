@@ -241,7 +241,12 @@ def _run_mesh_case(case, dev, framed, autocast):
     tiles = {c: t.to(dev) for c, t in oh.split_global(X, mesh).items()}
     gtiles = {c: t.to(dev) for c, t in oh.split_global(G, mesh).items()}
     geoms = {c: conv_geometry(n, mesh, c, k, s, p, d) for c in tiles}
-    fwd_tabs = _recv_tables(tiles, geoms, mesh, from_padded=False)
+    if autocast is not None:
+        # the strips travel in the autocast dtype; the upstream gradient arrives rounded to it
+        fwd_tabs = _recv_tables({c: t.to(autocast) for c, t in tiles.items()}, geoms, mesh, from_padded=False)
+        gtiles = {c: t.to(autocast).to(dtype) for c, t in gtiles.items()}
+    else:
+        fwd_tabs = _recv_tables(tiles, geoms, mesh, from_padded=False)
     Wg, Bg = W.to(dev), B.to(dev)
 
     # pass 1: forward of every rank, and the padded dgrad every rank will send from
