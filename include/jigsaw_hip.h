@@ -187,6 +187,22 @@ int jg_ln_partial_bwd(float* mean_gxn, float* dot_gxn_xhat, float* gw, float* gb
                       int64_t cols, int dtype, void* workspace, size_t workspace_bytes,
                       void* stream);
 
+/* jg_ln_partial_bwd without a workspace argument, for callers that cannot allocate
+ * device memory (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc). No counterpart in the reference. Same kernels, same results, same
+ * arguments otherwise; the column partials go to a device array built into the library
+ * (JG_LN_BWD_STATIC_SCRATCH_BYTES per GPU, held until the process ends). The call
+ * allocates and frees nothing. Limits: jg_ln_bwd_workspace_bytes(rows, cols) must fit
+ * that array when gw or gb is asked for (min(ceil(rows / 4), 1024) * 2 * cols * 4 bytes:
+ * any row count up to 1024 local columns) - JG_ERR_WORKSPACE otherwise; calls on one GPU
+ * share the array, so two calls that overlap in time on one GPU (different streams or
+ * host threads) race: serialise them. The first call on a device resolves the array's
+ * address and must happen outside a stream capture. */
+#define JG_LN_BWD_STATIC_SCRATCH_BYTES (8u << 20)
+int jg_ln_partial_bwd_static(float* mean_gxn, float* dot_gxn_xhat, float* gw, float* gb,
+                             const void* g, const void* x_hat, const void* w, int64_t rows,
+                             int64_t cols, int dtype, void* stream);
+
 /* gx = (1/std) * (g*w - mean_gxn - x_hat * dot_gxn_xhat / n_global) with the
  * COMBINED row terms (_functional.py:173-175). */
 int jg_ln_bwd_apply(void* gx, const void* g, const void* x_hat, const void* w,

@@ -9,6 +9,8 @@
 //   jigsaw/modules/normalization/_functional.py:141-175 (backward)
 #include "jg_common.h"
 
+#include <mutex>
+
 namespace {
 
 constexpr int kWave = 64;
@@ -742,6 +744,62 @@ extern "C" int jg_ln_partial_bwd(float* mean_gxn, float* dot_gxn_xhat, float* gw
     JG_CHECK_LAUNCH("jg_ln_partial_bwd(colreduce)");
   }
   return JG_OK;
+}
+
+// ---- jg_ln_partial_bwd for callers that cannot allocate ---------------------------------
+// The column partials of stage 1 live in a device array that is part of the library's image
+// (every GPU the library runs on holds its own copy until the process ends) instead of a
+// caller-supplied workspace. In host code the array's NAME is only a handle: the address a
+// kernel can use comes from hipGetSymbolAddress, once per device, with that device current.
+constexpr size_t kStaticScratchBytes = JG_LN_BWD_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mu;
+void* scratch_ptr[kMaxDevices];  // per device: address of that device's copy of `scratch`
+
+// Address of the current device's scratch array. The first call on a device resolves it
+// (under the mutex); later calls read the table only.
+int scratch_of_current_device(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "jg_ln_partial_bwd_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    JG_FAIL(JG_ERR_UNSUPPORTED, "jg_ln_partial_bwd_static: device index %d outside 0..%d", dev, kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(scratch_mu);
+  if (scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      JG_FAIL(JG_ERR_LAUNCH, "jg_ln_partial_bwd_static: hipGetSymbolAddress on device %d: %s", dev,
+              hipGetErrorString(e));
+    scratch_ptr[dev] = p;
+  }
+  *out = static_cast<float*>(scratch_ptr[dev]);
+  return JG_OK;
+}
+}  // namespace
+
+extern "C" int jg_ln_partial_bwd_static(float* mean_gxn, float* dot_gxn_xhat, float* gw, float* gb,
+                                        const void* g, const void* x_hat, const void* w,
+                                        int64_t rows, int64_t cols, int dtype, void* stream) {
+  JG_REQUIRE(rows >= 0 && cols >= 1, "jg_ln_partial_bwd_static: bad shape");
+  const size_t need = (gw != nullptr || gb != nullptr) ? jg_ln_bwd_workspace_bytes(rows, cols) : 0;
+  if (need > kStaticScratchBytes)
+    JG_FAIL(JG_ERR_WORKSPACE,
+            "jg_ln_partial_bwd_static: %lld rows x %lld columns need %zu bytes of column partials, the "
+            "built-in scratch holds %zu; use jg_ln_partial_bwd with a workspace",
+            (long long)rows, (long long)cols, need, kStaticScratchBytes);
+  float* part = nullptr;
+  if (need != 0) {
+    int rc = scratch_of_current_device(&part);
+    if (rc) return rc;
+  }
+  // Every partial that stage 2 reads is written by stage 1 of the same call, so nothing has
+  // to start at zero; the shared kernels take the address as they take a workspace.
+  return jg_ln_partial_bwd(mean_gxn, dot_gxn_xhat, gw, gb, g, x_hat, w, rows, cols, dtype, part,
+                           kStaticScratchBytes, stream);
 }
 
 extern "C" int jg_ln_bwd_apply(void* gx, const void* g, const void* x_hat, const void* w,
