@@ -143,29 +143,45 @@ def attention_figures(dev, iters: int) -> dict:
     out, l = ja.ring_forward(q, ks, vs, scale)
     ms_b = time_gpu(lambda: ja.core_backward(dout, q, ks[0], vs[0], out, l, scale), iters)
     ms_ring = time_gpu(lambda: ja.ring_forward(q, ks, vs, scale), iters)
-    # The same ring with the K/V hop in the loop: every step receives the next chunk, on the compute
-    # thread or on a side stream. A device copy of the 8 MiB stands in for the neighbour's transfer;
-    # "link" adds one copy of 128 MiB, about the 55 us the 8 MiB take over one 153 GB/s xGMI link.
+    # The same ring with the hops in the loop (jigsaw_amd.ring.RingSeat): every step forwards the chunk
+    # it holds and receives the next one, on the compute stream or on the seat's transfer stream. The
+    # neighbour's transfer is a device copy of the 2 x 4 MiB; "link" puts a spinning one-thread kernel of
+    # about the time the message takes over one 153 GB/s xGMI link in front of it (a transfer over the
+    # link, unlike a big device copy, occupies neither the compute units nor HBM).
     from jigsaw_amd import ring as jr
 
-    kvs = [torch.stack((k, v)) for k, v in zip(ks, vs)]
-    side = torch.cuda.Stream()
+    cal = 2_000_000
+    ms_cal = time_gpu(lambda: torch.cuda._sleep(cal), 5)
+    link_cycles = int(cal * (ks[0].numel() * 2 / 153e9 * 1e3) / ms_cal)  # one K or V message
 
-    pad_src = torch.empty(128 << 20, dtype=torch.uint8, device=dev)
-    pad_dst = torch.empty_like(pad_src)
+    def seat_for(link, overlap, scope):
+        seen = {}
 
-    def ring_with_hop(link, stream):
-        def send(src, buf, *, direction, group, async_op, tag):
+        def hop(src, buf, direction, *, group, async_op, tag):
+            which = seen.get(tag, 0) % 2  # K first, then V
+            seen[tag] = which + 1
             if link:
-                pad_dst.copy_(pad_src)
-            buf.copy_(kvs[(tag + 1) % P])
+                torch.cuda._sleep(link_cycles)
+            buf.copy_((ks, vs)[which][(tag + 1) % P])
             return buf, None
 
-        return time_gpu(lambda: jr.ring_forward_from_provider(
-            q, jr.RingKVProvider(ks[0], vs[0], 0, P, send, comm_stream=stream), scale), iters)
+        def relay(src, buf, offset, *, group, async_op, step):
+            if link:
+                torch.cuda._sleep(link_cycles)
+            buf.copy_(src)  # the partial the peer would have sent: same size
+            return buf, None
 
-    hop = {"ms_copy_inline": ring_with_hop(False, None), "ms_copy_side_stream": ring_with_hop(False, side),
-           "ms_link_inline": ring_with_hop(True, None), "ms_link_side_stream": ring_with_hop(True, side)}
+        return jr.RingSeat(0, P, ks[0], hop, relay_fn=relay, save_scope=scope, overlap=overlap)
+
+    hop, hop_bwd = {}, {}
+    for name, link, overlap in (("ms_copy_inline", False, False), ("ms_copy_overlapped", False, True),
+                                ("ms_link_inline", True, False), ("ms_link_overlapped", True, True)):
+        seat = seat_for(link, overlap, "local")
+        hop[name] = time_gpu(lambda: seat.forward(q, ks[0], vs[0], scale), iters)
+        _, _, saved = seat.forward(q, ks[0], vs[0], scale)
+        hop_bwd[name] = time_gpu(lambda: seat.backward(dout, q, out, l, scale, saved), iters)
+    hop["ms_no_hop"] = ms_ring
+    hop_bwd["ms_no_hop"] = time_gpu(lambda: ja.ring_backward(dout, q, out, l, ks, vs, scale), iters)
     x = torch.randn(b, n, 256, device=dev, generator=g).bfloat16()
     ms_ln = time_gpu(lambda: jl.partial_stats(x), iters)
     tf = lambda f, ms: f / (ms * 1e-3) / 1e12  # noqa: E731
@@ -174,6 +190,7 @@ def attention_figures(dev, iters: int) -> dict:
         "attn_bwd_step": {"ms": ms_b, "tflops": tf(f_bwd, ms_b), "frac_mfma_peak": tf(f_bwd, ms_b) / PEAK_BF16_TFLOPS},
         "attn_ring_fwd_4_steps": {"ms": ms_ring, "tflops": tf(4 * f_fwd, ms_ring)},
         "attn_ring_fwd_4_steps_with_hop": hop,
+        "attn_ring_bwd_4_steps_with_hop_and_dkv_relay": hop_bwd,
         "ln_partial_stats": {"ms": ms_ln, "GBps": x.numel() * 2 / (ms_ln * 1e-3) / 1e9, "bytes": x.numel() * 2},
     }
 

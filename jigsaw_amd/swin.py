@@ -7,9 +7,8 @@ LayerNorms (not sharded in the example) run on the fused unsharded-LayerNorm ker
 the shift / unshift on the DistributedRoll kernels, the windowed attention with its
 relative-position bias and shift mask on the attention core with an additive
 bias. The linear layers are ``nn.Linear`` parameters (as in the reference example);
-in bf16 they run on this package's projection GEMMs (head split / merge and bias
-gradient fused in), otherwise through the library GEMMs with the weight gradient split
-over the tokens, because its output is a few tiles and its contraction 65536 long.
+they run on this package's projection GEMMs (head split / merge and bias gradient fused
+in): bf16 on the matrix cores, other dtypes on the FMA kernel with the same addressing.
 """
 
 from __future__ import annotations
@@ -27,64 +26,21 @@ from .projection import heads_projection, linear, qkv_projection
 from .roll import _Roll
 
 
-class _TokenLinear(torch.autograd.Function):
-    """``F.linear`` over ``(tokens, features)`` whose weight gradient is a batched GEMM
-    over chunks of the tokens, summed in fp32. ``dW = dy^T x`` has an output of only
-    ``out x in`` (a handful of GEMM tiles) and a contraction as long as the token count,
-    so a single library GEMM runs on a few compute units; the chunks spread it over the
-    chip. Same arithmetic as ``nn.Linear`` otherwise (examples/swin.py:136-170, 183-190)."""
-
-    CHUNK = 1024  # tokens per partial product
-
-    @staticmethod
-    def forward(ctx, x, weight, bias):  # noqa: D102
-        ctx.dtypes = (x.dtype, weight.dtype, bias.dtype if bias is not None else None)
-        if torch.is_autocast_enabled():
-            dt = torch.get_autocast_dtype("cuda")
-            x, weight = x.to(dt), weight.to(dt)
-            bias = bias.to(dt) if bias is not None else None
-        ctx.save_for_backward(x, weight)
-        ctx.has_bias = bias is not None
-        return torch.nn.functional.linear(x, weight, bias)
-
-    @staticmethod
-    def backward(ctx, gy):  # noqa: D102
-        x, weight = ctx.saved_tensors
-        need_x, need_w, need_b = ctx.needs_input_grad
-        gy2 = gy.reshape(-1, gy.shape[-1])
-        x2 = x.reshape(-1, x.shape[-1])
-        dt_x, dt_w, dt_b = ctx.dtypes
-        gy2 = gy2.to(weight.dtype)
-        gx = (gy2 @ weight).view(x.shape).to(dt_x) if need_x else None
-        gw = None
-        if need_w:
-            t = x2.shape[0]
-            chunk = _TokenLinear.CHUNK
-            if t % chunk == 0 and t // chunk > 1:
-                parts = torch.bmm(gy2.view(t // chunk, chunk, -1).transpose(1, 2), x2.view(t // chunk, chunk, -1))
-                gw = parts.sum(0, dtype=torch.float32).to(dt_w)
-            else:
-                gw = (gy2.t() @ x2).to(dt_w)
-        gb = gy2.sum(0, dtype=torch.float32).to(dt_b) if need_b and ctx.has_bias else None
-        return gx, gw, gb
-
-
 def _compute_dtype(x: torch.Tensor) -> torch.dtype:
     """The dtype a linear layer computes in: the autocast dtype when autocast is on."""
     return torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else x.dtype
 
 
 def token_linear(x: torch.Tensor, layer: nn.Linear) -> torch.Tensor:
-    """``layer(x)``: in bf16 on this package's GEMM kernels (bias gradient fused into the weight
-    gradient), otherwise through the library GEMM with the token-split weight gradient."""
-    if x.is_cuda and _compute_dtype(x) == torch.bfloat16 and x.shape[-1] % 8 == 0 and layer.weight.shape[0] % 8 == 0:
-        return linear(x.to(torch.bfloat16), layer.weight, layer.bias)
-    return _TokenLinear.apply(x, layer.weight, layer.bias)
+    """``layer(x)`` on this package's GEMM kernels in the compute dtype (bf16 on the matrix
+    cores, other dtypes on the FMA kernel with the same addressing); the bias gradient is
+    summed inside the weight-gradient GEMM."""
+    return linear(x.to(_compute_dtype(x)), layer.weight, layer.bias)
 
 
 def windows(x: torch.Tensor, window: int) -> torch.Tensor:
-    """Cut a tile ``(B, h, w, C)`` into windows ``(B, nW, window*window, C)``
-    (examples/swin.py:85-89)."""
+    """Cut a tile ``(B, h, w, C)`` into windows ``(B, nW, window*window, C)``, windows and the
+    tokens inside a window both in row-major order (examples/swin.py:85-89)."""
     b, h, w, c = x.shape
     x = x.view(b, h // window, window, w // window, window, c)
     return x.permute(0, 1, 3, 2, 4, 5).reshape(b, -1, window * window, c)
@@ -98,29 +54,40 @@ def unwindows(x: torch.Tensor, h: int, w: int, window: int) -> torch.Tensor:
 
 
 def relative_position_index(window: int) -> torch.Tensor:
-    """Index into the bias table for every pair of positions inside a window
-    (examples/swin.py:99-104)."""
-    ij = torch.stack(torch.meshgrid(*[torch.arange(window)] * 2, indexing="ij")).flatten(1)
-    rel = ij[:, :, None] - ij[:, None, :] + (window - 1)
-    return rel[0] * (2 * window - 1) + rel[1]
+    """``(N, N)`` row of the bias table for a (query, key) pair of one window: the table is
+    a ``(2W-1) x (2W-1)`` grid of displacements, row-major, displacement = query - key
+    shifted to start at 0 (what examples/swin.py:99-104 computes)."""
+    token = torch.arange(window * window)
+    ty, tx = token // window, token % window
+    dy = ty[:, None] - ty[None, :] + (window - 1)
+    dx = tx[:, None] - tx[None, :] + (window - 1)
+    return dy * (2 * window - 1) + dx
+
+
+def border_sides(h: int, w: int, window: int, shift: int, groups: tuple) -> torch.Tensor:
+    """``(nW, N)`` integer code per token of the rolled tile: bit 1 set when the roll by
+    ``-shift`` carried the token across the lower image border, bit 0 when across the right
+    one. A token at rolled GLOBAL position ``g`` came from ``g + shift``; it crossed iff that
+    lies beyond the grid. The grid size and the tile's place in it come from the two spatial
+    groups (objects with ``size()`` and ``rank()``)."""
+
+    def crossed(local: int, group: Any) -> torch.Tensor:
+        g = group.rank() * local + torch.arange(local)
+        return g + shift >= local * group.size()
+
+    code = crossed(h, groups[0])[:, None].long() * 2 + crossed(w, groups[1])[None, :].long()
+    return windows(code[None, :, :, None], window)[0, :, :, 0]
 
 
 def shift_mask(h: int, w: int, window: int, shift: int, groups: tuple) -> torch.Tensor:
-    """Mask ``(nW, N, N)`` of this tile's windows after rolling the token grid by
-    ``-shift``: tokens from the two sides of the image border must not attend to
-    each other; the border lies at the GLOBAL position, so the region of a token
-    follows from where the tile sits (examples/swin.py:107-126)."""
-
-    def region(local_size: int, group: Any) -> torch.Tensor:
-        size = local_size * group.size()
-        idx = group.rank() * local_size + torch.arange(local_size)
-        return (idx >= size - window).long() + (idx >= size - shift).long()
-
-    rows, cols = region(h, groups[0]), region(w, groups[1])
-    ids = (rows[:, None] * 3 + cols[None, :])[None, :, :, None]
-    ids = windows(ids, window).squeeze(-1).squeeze(0)
-    same = ids[:, :, None] == ids[:, None, :]
-    return torch.zeros(same.shape).masked_fill(~same, float("-inf"))
+    """Additive mask ``(nW, N, N)`` of this tile's windows after rolling the token grid by
+    ``-shift``: 0 where query and key lie on the same side of the image borders, ``-inf``
+    where the roll brought them together across one (the pairs examples/swin.py:107-126
+    masks; a window holds tokens from both sides only if it touches the border of the
+    GLOBAL grid, so the mask depends on where the tile sits)."""
+    side = border_sides(h, w, window, shift, groups)
+    apart = side[:, :, None] != side[:, None, :]
+    return torch.zeros(apart.shape).masked_fill(apart, float("-inf"))
 
 
 class WindowAttention(nn.Module):
@@ -146,23 +113,16 @@ class WindowAttention(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         b, h, w, c = x.shape
-        x = windows(x, self.window)
+        x = windows(x, self.window).to(_compute_dtype(x))
         n = x.shape[2]
-        fused = x.dtype == torch.bfloat16  # the projections write / read the head layout themselves
-        if fused:
-            q, k, v = qkv_projection(x, self.qkv.weight, self.qkv.bias, self.heads).unbind(0)
-        else:
-            qkv = token_linear(x, self.qkv).view(b, -1, n, 3, self.heads, c // self.heads)
-            q, k, v = (t.contiguous() for t in qkv.permute(3, 0, 1, 4, 2, 5).unbind(0))  # (B, nW, heads, N, d)
+        # the projections write / read the (B, nW, heads, N, d) head layout themselves
+        q, k, v = qkv_projection(x, self.qkv.weight, self.qkv.bias, self.heads).unbind(0)
         with torch.autocast("cuda", enabled=False):
             bias = (self.onehot @ self.bias_table.float()).view(n, n, -1).permute(2, 0, 1)
         if self.mask is not None:
             bias = bias[None] + self.mask[:, None]  # (nW, heads, N, N)
         out = window_attention(q, k, v, bias.contiguous())
-        if fused:
-            return unwindows(heads_projection(out, self.proj.weight, self.proj.bias), h, w, self.window)
-        out = out.transpose(2, 3).reshape(b, -1, n, c)
-        return unwindows(token_linear(out, self.proj), h, w, self.window)
+        return unwindows(heads_projection(out, self.proj.weight, self.proj.bias), h, w, self.window)
 
 
 class SwinBlock(nn.Module):
@@ -215,4 +175,4 @@ class SwinBlock(nn.Module):
         return self.finish(x, y)
 
 
-__all__ = ["SwinBlock", "WindowAttention", "relative_position_index", "shift_mask", "unwindows", "windows"]
+__all__ = ["SwinBlock", "WindowAttention", "border_sides", "relative_position_index", "shift_mask", "unwindows", "windows"]

@@ -100,6 +100,43 @@ def ring_backward(dout, q, out, lse, k_chunks, v_chunks, scale):
     return dq, dks, dvs
 
 
+def ring_all_ranks(qs, ks, vs, douts, scale, save_scope="global"):
+    """Every rank of a ring of ``P = len(qs)`` ranks, forward and backward, with the
+    cross-rank dK/dV sums: ``([out_r], [lse_r], [dq_r], [dk_r], [dv_r])``.
+
+    Rank ``r`` holds ``qs[r], ks[r], vs[r]``. Forward as :func:`ring_forward`. Backward
+    per rank as :func:`ring_backward`; the owner of chunk ``r`` then sums what the ranks
+    computed for it:
+
+    * ``"global"`` (saved chunks, SEND_DKV; backward.py:272-277): a SUM all-reduce of
+      each step's partial, i.e. the contributions of ranks 0 .. P-1 added in the core dtype;
+    * ``"local"`` (re-circulated chunks, SEND_DKV; backward.py:484-538): the own step-0
+      partial first, then at step ``s`` the partial received from rank ``r - s``
+      (which holds chunk ``r`` at its step ``s``), added in arrival order.
+    """
+    P = len(qs)
+    outs, lses, dqs, parts = [], [], [], []
+    for r in range(P):
+        o, l = ring_forward(qs[r], ks, vs, scale, rank=r)
+        dq, dkj, dvj = ring_backward(douts[r], qs[r], o, l, ks, vs, scale)
+        outs.append(o), lses.append(l), dqs.append(dq), parts.append((dkj, dvj))
+    dks, dvs = [], []
+    for r in range(P):
+        if save_scope == "global":
+            order = list(range(P))
+        elif save_scope == "local":
+            order = [(r - s) % P for s in range(P)]
+        else:
+            raise ValueError(save_scope)
+        dk = parts[order[0]][0][r].clone()
+        dv = parts[order[0]][1][r].clone()
+        for src in order[1:]:
+            dk += parts[src][0][r]
+            dv += parts[src][1][r]
+        dks.append(dk), dvs.append(dv)
+    return outs, lses, dqs, dks, dvs
+
+
 def window_attention(q, k, v, bias):
     """Windowed attention with an additive bias / mask, as the Swin example calls
     ``F.scaled_dot_product_attention(q, k, v, attn_mask=bias)`` (examples/swin.py:148-151):

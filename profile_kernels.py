@@ -2,9 +2,9 @@
 (and 4) a few times, plus a plain device copy of known size that calibrates the
 FETCH_SIZE / WRITE_SIZE counters.
 
-    rocprofv3 --kernel-trace --stats -d OUT -o kt --output-format csv -- python3 -m jigsaw_amd.profile_kernels
-    rocprofv3 --pmc FETCH_SIZE -d OUT -o fetch --output-format csv -- python3 -m jigsaw_amd.profile_kernels
-    rocprofv3 --pmc WRITE_SIZE -d OUT -o write --output-format csv -- python3 -m jigsaw_amd.profile_kernels
+    rocprofv3 --kernel-trace --stats -d OUT -o kt --output-format csv -- python3 profile_kernels.py
+    rocprofv3 --pmc FETCH_SIZE -d OUT -o fetch --output-format csv -- python3 profile_kernels.py
+    rocprofv3 --pmc WRITE_SIZE -d OUT -o write --output-format csv -- python3 profile_kernels.py
 
 With the argument ``around-attention`` it launches instead the kernels either side of the ring
 step: the attention core at head size 128 (32 heads, 4096 x 4096 tokens) and the qkv / output

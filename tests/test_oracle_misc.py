@@ -50,6 +50,28 @@ def test_ring_backward_equals_autograd_of_full_attention():
     torch.testing.assert_close(torch.cat(dvs, 2), V.grad, atol=1e-11, rtol=1e-9)
 
 
+@pytest.mark.parametrize("scope", ["global", "local"])
+def test_ring_all_ranks_equals_autograd_of_full_attention(scope):
+    """All P ranks of the ring with the owners' dK/dV sums == autograd through full
+    softmax attention of the concatenated queries over the concatenated K/V."""
+    torch.manual_seed(11)
+    P, b, h, n, d = 3, 2, 2, 8, 4
+    scale = d**-0.5
+    qs = [torch.randn(b, h, n, d, dtype=torch.float64) for _ in range(P)]
+    ks = [torch.randn(b, h, n, d, dtype=torch.float64) for _ in range(P)]
+    vs = [torch.randn(b, h, n, d, dtype=torch.float64) for _ in range(P)]
+    douts = [torch.randn(b, h, n, d, dtype=torch.float64) for _ in range(P)]
+    Q, K, V = (torch.cat(t, 2).requires_grad_() for t in (qs, ks, vs))
+    full = torch.softmax((Q @ K.mT) * scale, -1) @ V
+    full.backward(torch.cat(douts, 2))
+    outs, lses, dqs, dks, dvs = oa.ring_all_ranks(qs, ks, vs, douts, scale, save_scope=scope)
+    torch.testing.assert_close(torch.cat(outs, 2), full.detach(), atol=1e-12, rtol=1e-10)
+    torch.testing.assert_close(torch.cat(lses, 2), torch.logsumexp((Q @ K.mT).detach() * scale, -1), atol=1e-12, rtol=1e-10)
+    torch.testing.assert_close(torch.cat(dqs, 2), Q.grad, atol=1e-11, rtol=1e-9)
+    torch.testing.assert_close(torch.cat(dks, 2), K.grad, atol=1e-11, rtol=1e-9)
+    torch.testing.assert_close(torch.cat(dvs, 2), V.grad, atol=1e-11, rtol=1e-9)
+
+
 @pytest.mark.parametrize("form", ["eager", "fused"])
 def test_merge_special_cases(form):
     torch.manual_seed(2)

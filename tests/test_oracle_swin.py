@@ -162,3 +162,26 @@ def test_block_against_per_token_restatement(h, w, win, shift):
     got = osw.block(x, p, heads, win, shift)
     want = _block_per_token(x, p, heads, win, shift, 1e-5)
     torch.testing.assert_close(got, want, atol=1e-11, rtol=1e-9)
+
+
+@pytest.mark.parametrize("H,W,win,shift", [(16, 16, 4, 2), (16, 24, 4, 1), (32, 32, 8, 4), (8, 8, 2, 1)])
+def test_package_index_and_mask_on_1x1_and_2x2_tilings(H, W, win, shift):
+    """The package's own index and mask builders (built from rolled global positions) agree
+    with the pinned oracle: on the undivided grid, and tile by tile on a 2 x 2 tiling, where
+    the mask depends on where the tile sits."""
+    from jigsaw_amd import swin as js
+    from jigsaw_amd.conv import TileGroup
+
+    assert torch.equal(js.relative_position_index(win), osw.relative_position_index(win))
+    full = osw.shift_mask_global(H, W, win, shift)
+    one = js.shift_mask(H, W, win, shift, (TileGroup(1, 0), TileGroup(1, 0)))
+    assert torch.equal(one.double(), full)
+    h, w = H // 2, W // 2
+    by_window = full.view(H // win, W // win, win * win, win * win)
+    for r, c in itertools.product(range(2), repeat=2):
+        got = js.shift_mask(h, w, win, shift, (TileGroup(2, r), TileGroup(2, c)))
+        want = by_window[r * (h // win) : (r + 1) * (h // win), c * (w // win) : (c + 1) * (w // win)]
+        assert torch.equal(got.double().view(want.shape), want), f"tile ({r}, {c})"
+    # the side code the mask is built from: 0 everywhere except in the last window row / column of the grid
+    side = js.border_sides(H, W, win, shift, (TileGroup(1, 0), TileGroup(1, 0))).view(H // win, W // win, -1)
+    assert int(side[:-1, :-1].abs().sum()) == 0 and int(side[-1, -1].max()) == 3

@@ -1,16 +1,25 @@
-"""Chunk providers of the ring (the K/V hop beside the attention core) on one GPU: the
-neighbour's transfer is a device copy of the chunk it would have sent. The provider loop
-must visit the chunks in ring order and give exactly what the loop over the chunk list gives
-(same kernels, same order: bit-identical), with the hop on the compute thread or on a side
-stream."""
+"""One rank's seat in the K/V ring (jigsaw_amd.ring.RingSeat) on one GPU, forward and
+backward, against the all-ranks ring oracle (oracle.attention.ring_all_ranks, pinned on
+the CPU against autograd of full attention).
+
+Every rank of the ring runs in this process, one after the other. The transports are
+stand-ins that copy in what the peer would have sent: the K/V hop knows the global chunk
+list; the dK/dV partials of the other ranks come from a first, recording pass (the core is
+deterministic, so the second pass sends the same partials again). Tolerances: rel-L2 2e-2
+for bf16, 1e-5 for fp32 tensors (the reference's ring tests: atol 1e-2 / 1e-3,
+tests/modules/attention/test_ring_attention.py:159-368).
+"""
 
 import pytest
 import torch
 
-from jigsaw_amd import attention as ja
+from helpers import rel_l2
 from jigsaw_amd import ring as jr
+from oracle import attention as oa
 
 pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
 
 
 class _Work:
@@ -18,77 +27,147 @@ class _Work:
         self.log = log
 
     def wait(self):
-        self.log.append("wait")
+        self.log.append(("wait", torch.cuda.current_stream().cuda_stream))
 
 
-def _neighbour(ks, vs, rank, log, with_work):
-    """send_op_fn of rank ``rank``: what arrives at step tag + 1 is global chunk rank + tag + 1."""
-    P = len(ks)
+class Peers:
+    """Transport stand-ins of one rank. ``partials[src_rank][step]`` = (dk, dv) that rank sent."""
 
-    def send(src, buf, *, direction, group, async_op, tag):
-        assert direction == -1 and async_op and buf.shape == src.shape
-        j = (rank + tag + 1) % P
-        buf.copy_(torch.stack((ks[j], vs[j])))
-        log.append(("send", tag, torch.cuda.current_stream().cuda_stream))
-        return buf, (_Work(log) if with_work else None)
+    def __init__(self, rank, ks, vs, with_work, partials=None, sums=None):
+        self.rank, self.ks, self.vs, self.P = rank, ks, vs, len(ks)
+        self.with_work, self.partials, self.sums = with_work, partials, sums
+        self.log, self.sent, self._seen = [], {}, {}
 
-    return send
+    def hop(self, src, buf, direction, *, group, async_op, tag):
+        assert direction == -1 and async_op and buf.shape == src.shape and buf.data_ptr() != src.data_ptr()
+        which = self._seen.get(tag, 0)  # first message of a step is K, second V
+        self._seen[tag] = which + 1
+        j = (self.rank + tag + 1) % self.P
+        held = (self.ks, self.vs)[which][(self.rank + tag) % self.P]
+        assert torch.equal(src, held), "the hop must forward the chunk of the current step"
+        buf.copy_((self.ks, self.vs)[which][j])
+        self.log.append(("hop", tag, torch.cuda.current_stream().cuda_stream))
+        return buf, (_Work(self.log) if self.with_work else None)
+
+    def relay(self, src, buf, offset, *, group, async_op, step):
+        assert offset == step and 1 <= step < self.P
+        self.sent.setdefault(step, []).append(src.clone())
+        which = len(self.sent[step]) - 1  # dk first, then dv
+        if self.partials is None:
+            buf.zero_()
+        else:
+            buf.copy_(self.partials[(self.rank - step) % self.P][step][which])
+        self.log.append(("relay", step, torch.cuda.current_stream().cuda_stream))
+        return buf, (_Work(self.log) if self.with_work else None)
+
+    def reduce(self, dk_j, dv_j, step):
+        self.sent[step] = (dk_j.clone(), dv_j.clone())
+        if self.sums is None:
+            return dk_j, dv_j
+        return self.sums[step]
 
 
-@pytest.mark.parametrize("overlap", [False, True], ids=["plain", "side-stream"])
-@pytest.mark.parametrize("shape,P,dtype", [
-    ((1, 2, 256, 64), 4, torch.bfloat16),    # fused step kernel
+def _inputs(shape, P, dtype, dev):
+    b, h, n, d = shape
+    mk = lambda scale=1.0: [(torch.randn(b, h, n, d) * scale).to(dtype) for _ in range(P)]  # noqa: E731
+    qs, ks, vs, douts = mk(d ** -0.5), mk(), mk(), mk()
+    gpu = lambda ts: [t.to(dev) for t in ts]  # noqa: E731
+    return (qs, ks, vs, douts), tuple(gpu(t) for t in (qs, ks, vs, douts))
+
+
+CASES = [
+    ((1, 2, 256, 64), 4, torch.bfloat16),    # fused step kernel (head size 64)
     ((1, 2, 128, 128), 3, torch.bfloat16),   # head size 128
     ((2, 3, 40, 16), 4, torch.float32),      # generic kernels + merge kernel
     ((1, 1, 128, 64), 1, torch.bfloat16),    # a ring of one: no transfer at all
-])
-def test_provider_ring_equals_chunk_list_ring(shape, P, dtype, overlap, dev):
+]
+
+
+@pytest.mark.parametrize("overlap", [False, True], ids=["plain", "overlapped"])
+@pytest.mark.parametrize("scope", ["global", "local"])
+@pytest.mark.parametrize("shape,P,dtype", CASES, ids=["d64", "d128", "fp32", "ring-of-one"])
+def test_ring_seat_matches_all_ranks_oracle(shape, P, dtype, scope, overlap, dev):
     torch.manual_seed(7)
-    b, h, n, d = shape
-    scale = d ** -0.5
-    q = (torch.randn(b, h, n, d) / d ** 0.5).to(dtype).to(dev)
-    ks = [torch.randn(b, h, n, d).to(dtype).to(dev) for _ in range(P)]
-    vs = [torch.randn(b, h, n, d).to(dtype).to(dev) for _ in range(P)]
-    side = torch.cuda.Stream() if overlap else None
-    for rank in range(P):
-        log = []
-        prov = jr.RingKVProvider(ks[rank], vs[rank], rank, P, _neighbour(ks, vs, rank, log, with_work=not overlap),
-                                 comm_stream=side)
-        out, lse = jr.ring_forward_from_provider(q, prov, scale)
-        want_o, want_l = ja.ring_forward(q, ks, vs, scale, rank=rank)
-        torch.cuda.synchronize()
-        assert torch.equal(out, want_o) and torch.equal(lse, want_l)
-        sends = [e for e in log if e != "wait"]
-        assert [e[1] for e in sends] == list(range(P - 1))          # one hop per step but the last
-        assert [prov.global_chunk_idx(s) for s in range(P)] == [(rank + s) % P for s in range(P)]
-        if overlap:
-            assert all(e[2] == side.cuda_stream for e in sends)     # every hop was issued on the side stream
+    (qs, ks, vs, douts), (gq, gk, gv, gd) = _inputs(shape, P, dtype, dev)
+    scale = shape[-1] ** -0.5
+    dbl = lambda ts: [t.double() for t in ts]  # noqa: E731
+    want = oa.ring_all_ranks(dbl(qs), dbl(ks), dbl(vs), dbl(douts), scale, save_scope=scope)
+    tol = TOL[dtype]
+
+    def run(partials=None, sums=None):
+        res, peers = [], []
+        for r in range(P):
+            pr = Peers(r, gk, gv, with_work=not overlap, partials=partials, sums=sums)
+            seat = jr.RingSeat(r, P, gk[r], pr.hop if P > 1 else None, relay_fn=pr.relay, reduce_fn=pr.reduce,
+                               save_scope=scope, overlap=overlap)
+            out, lse, saved = seat.forward(gq[r], gk[r], gv[r], scale)
+            # a second forward on the same seat: the slots and events are reused
+            pr._seen.clear(); pr.log.clear()
+            out2, lse2, saved = seat.forward(gq[r], gk[r], gv[r], scale)
+            torch.cuda.synchronize()
+            assert torch.equal(out, out2) and torch.equal(lse, lse2)
+            fwd_log = list(pr.log)
+            pr._seen.clear(); pr.log.clear()
+            dq, dk, dv = seat.backward(gd[r], gq[r], out, lse, scale, saved)
+            torch.cuda.synchronize()
+            res.append((out, lse, dq, dk, dv))
+            peers.append((pr, fwd_log, seat))
+        return res, peers
+
+    res, peers = run()
+    if scope == "local":
+        partials = [{s: tuple(pr.sent[s]) for s in pr.sent} for pr, _, _ in peers]
+        res, peers = run(partials=partials)
+    else:
+        sums = {}
+        for s in range(P):
+            dk = peers[0][0].sent[s][0].clone()
+            dv = peers[0][0].sent[s][1].clone()
+            for pr, _, _ in peers[1:]:
+                dk += pr.sent[s][0]
+                dv += pr.sent[s][1]
+            sums[s] = (dk, dv)
+        res, peers = run(sums=sums)
+
+    for r in range(P):
+        out, lse, dq, dk, dv = res[r]
+        assert out.dtype == dtype and lse.dtype == torch.float32 and dq.dtype == dtype and dk.dtype == dtype
+        for name, got, w in zip(("out", "lse", "dq", "dk", "dv"), (out, lse, dq, dk, dv), (want[i][r] for i in range(5))):
+            bound = tol if name != "lse" else max(tol * 0.05, 1e-5)
+            assert rel_l2(got, w) < bound, f"rank {r} {name}: {rel_l2(got, w):.3e}"
+        pr, fwd_log, seat = peers[r]
+        hops = [e for e in fwd_log if e[0] == "hop"]
+        assert [e[1] for e in hops] == [s for s in range(P - 1) for _ in (0, 1)]  # K and V, one hop per step but the last
+        assert [seat.chunk_at(s) for s in range(P)] == [(r + s) % P for s in range(P)]
+        main = torch.cuda.current_stream().cuda_stream
+        if overlap and P > 1:
+            assert all(e[2] != main for e in hops), "the hops belong on the transfer stream"
+            assert not any(e[0] == "wait" for e in fwd_log)
+        elif P > 1:
+            assert all(e[-1] == main for e in fwd_log)
+            assert sum(e[0] == "wait" for e in fwd_log) == 2 * (P - 1)  # the host waited for every handle
+        if scope == "local":
+            relays = [e for e in pr.log if e[0] == "relay"]
+            assert [e[1] for e in relays] == [s for s in range(1, P) for _ in (0, 1)]
+            assert len([e for e in pr.log if e[0] == "hop"]) == 2 * (P - 1)  # K/V circulate again in the backward
+            if overlap and P > 1:
+                assert all(e[2] != main for e in relays)
         else:
-            assert log.count("wait") == P - 1                       # the host waited for every handle
+            assert not [e for e in pr.log if e[0] in ("hop", "relay")]  # saved chunks: nothing travels but the sums
 
 
-def test_provider_argument_errors(dev):
+def test_ring_seat_argument_errors(dev):
     k = torch.zeros(1, 1, 128, 64, device=dev, dtype=torch.bfloat16)
-    send = lambda *a, **kw: (a[1], None)  # noqa: E731
+    hop = lambda src, buf, direction, **kw: (buf, None)  # noqa: E731
     with pytest.raises(ValueError):
-        jr.RingKVProvider(k, k[..., :32], 0, 2, send)
+        jr.RingSeat(2, 2, k, hop)
     with pytest.raises(ValueError):
-        jr.RingKVProvider(k, k, 2, 2, send)
-    prov = jr.RingKVProvider(k, k, 0, 2, send)
+        jr.RingSeat(0, 2, k, None)
     with pytest.raises(ValueError):
-        prov.get(1)  # step 0 first
-
-
-def test_provider_ring_in_fp16_with_the_fused_step(dev):
-    """fp16 at head size 128 runs the fused step kernel; the provider loop still equals the list loop."""
-    torch.manual_seed(8)
-    P, shape = 3, (1, 2, 128, 128)
-    q = (torch.randn(*shape) / 128 ** 0.5).half().to(dev)
-    ks = [torch.randn(*shape).half().to(dev) for _ in range(P)]
-    vs = [torch.randn(*shape).half().to(dev) for _ in range(P)]
-    side = torch.cuda.Stream()
-    prov = jr.RingKVProvider(ks[1], vs[1], 1, P, _neighbour(ks, vs, 1, [], with_work=False), comm_stream=side)
-    out, lse = jr.ring_forward_from_provider(q, prov, 128 ** -0.5)
-    want_o, want_l = ja.ring_forward(q, ks, vs, 128 ** -0.5, rank=1)
-    torch.cuda.synchronize()
-    assert out.dtype == torch.float16 and torch.equal(out, want_o) and torch.equal(lse, want_l)
+        jr.RingSeat(0, 2, k, hop, save_scope="elsewhere")
+    seat = jr.RingSeat(0, 2, k, hop, save_scope="local")
+    with pytest.raises(ValueError):
+        seat.forward(k, k, k[..., :32], 0.125)
+    out, lse, saved = seat.forward(k, k, k, 0.125)
+    with pytest.raises(ValueError, match="relay_fn"):
+        seat.backward(k, k, out, lse, 0.125, saved)
