@@ -133,6 +133,44 @@ def test_fused_step_equals_core_plus_merge(d, dev):
     torch.testing.assert_close(l1, l2, atol=1e-6, rtol=1e-6)
 
 
+@pytest.mark.parametrize("pattern", ["late_spike", "rising", "first_tile_low", "huge_logits", "one_hot_rows"])
+def test_mfma_forward_when_the_running_max_moves(pattern, dev):
+    """The head-size-64 kernel keeps a per-query reference exponent that follows the running
+    max lazily (it moves only when a tile exceeds it by 2^8) and folds it into the score
+    product. Score patterns that move the max late, often, by hundreds of powers of two, or
+    start far below zero must give the fp64 softmax all the same (bf16 bar), and so must
+    the merge into a ring accumulator that already holds a chunk."""
+    torch.manual_seed(11)
+    b, h, sq, sk, d = 1, 2, 256, 1024, 64
+    q = torch.randn(b, h, sq, d)
+    k = torch.randn(b, h, sk, d)
+    v = torch.randn(b, h, sk, d)
+    if pattern == "late_spike":        # a few keys near the end dominate everything before them
+        k[:, :, 900:905] *= 12.0
+    elif pattern == "rising":          # the max moves in almost every tile
+        k *= torch.linspace(0.2, 6.0, sk)[None, None, :, None]
+    elif pattern == "first_tile_low":  # the first tiles hold only very negative scores
+        k[:, :, :128] = -3.0 * q[:, :, :1].mean(2, keepdim=True).expand(b, h, 128, d) - 4.0
+        q = q.abs()
+    elif pattern == "huge_logits":     # logits in the thousands: softmax is one-hot, nothing may overflow
+        q, k = q * 30.0, k * 30.0
+    elif pattern == "one_hot_rows":    # every query has exactly one matching key, somewhere in the chunk
+        k = torch.nn.functional.normalize(k, dim=-1) * 40.0
+        q = k[:, :, torch.randperm(sk)[:sq]].clone()
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    scale = d**-0.5
+    want_o, want_l = oa.core_forward(q.double(), k.double(), v.double(), scale)
+    out, lse = ja.core_forward(q.to(dev), k.to(dev), v.to(dev), scale)
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    assert rel_l2(out, want_o) < 2e-2, f"out {rel_l2(out, want_o):.3e}"
+    assert rel_l2(lse, want_l) < 2e-3, f"lse {rel_l2(lse, want_l):.3e}"  # the core test's bar for bf16
+    # the same chunk as the second step of a ring whose first chunk is ordinary
+    k0, v0 = torch.randn(b, h, 256, d).bfloat16(), torch.randn(b, h, 256, d).bfloat16()
+    ring_o, ring_l = ja.ring_forward(q.to(dev), [k0.to(dev), k.to(dev)], [v0.to(dev), v.to(dev)], scale)
+    full_o, full_l = oa.core_forward(q.double(), torch.cat([k0, k], 2).double(), torch.cat([v0, v], 2).double(), scale)
+    assert rel_l2(ring_o, full_o) < 2e-2 and rel_l2(ring_l, full_l) < 2e-3
+
+
 def test_config4_shape_properties(dev):
     """Config 4 at full size: 8 heads, 4096 queries, 4 chunks of 4096 keys, d = 64, bf16.
     Size-independent checks: ring over 4 chunks == one core call over the concatenated
