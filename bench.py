@@ -34,9 +34,14 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 
 METRIC = "halo-conv fwd+bwd & ring-attn step TFLOP/s on 1 GPU; % MFMA peak; halo GB/s"
 
-# HBM bytes per launch of the forward conv kernel (FETCH_SIZE + WRITE_SIZE from
-# rocprofv3 --pmc, scaled by a copy kernel of known size); None until measured.
-CONV_FWD_TRAFFIC_BYTES = 2.32e9
+# HBM bytes per launch of the three convolution kernels of the step (FETCH_SIZE + WRITE_SIZE
+# from rocprofv3 --pmc, scaled by a copy kernel of known size).
+CONV_TRAFFIC_BYTES = {"fwd": 2.32e9, "dgrad_fold": 2.38e9, "wgrad_bias": 2.27e9}
+CONV_KERNEL_NAMES = {
+    "fwd": "conv3x3_mfma_kernel (forward, config 2)",
+    "dgrad_fold": "conv3x3_mfma_kernel (dgrad with the fold epilogue, config 2)",
+    "wgrad_bias": "wgrad3x3_mfma_kernel + reduction (weight and bias gradient, config 2)",
+}
 
 
 def _events():
@@ -96,26 +101,35 @@ def build_conv2_workload(dev, batch=8, ch=64, tile=1024):
             "bands": bands}
 
 
-def conv_step(wl, fwd_events=None):
+def conv_step(wl, kernel_events=None):
     """The hot path of one rank for one batch (see the module docstring). The backward
     uses the fused forms, each with the bits of the separate steps it replaces: dgrad
     writes the owned cells and the strips it sends in one pass, wgrad adds up the bias
-    gradient on the way, and the received strips are added to the border afterwards."""
+    gradient on the way, and the received strips are added to the border afterwards.
+    ``kernel_events`` collects HIP-event brackets (on the launch stream) around the three
+    convolution launches of the step."""
     from jigsaw_amd import conv as jc
     from jigsaw_amd.halo import halo_assemble, halo_fold_border_, halo_pack
 
     geom, x, w, b, g = wl["geom"], wl["x"], wl["w"], wl["b"], wl["g"]
-    halo_pack(x, geom, from_padded=False)  # strips this rank sends
-    x_aug = halo_assemble(x, wl["strips_fwd"], geom)
-    if fwd_events is not None:  # HIP events around the forward launch, on its stream
+
+    def bracket(name, fn):
+        if kernel_events is None:
+            return fn()
         e0, e1 = _events()
         e0.record()
-    y = jc.conv_nd(x_aug, w, b)
-    if fwd_events is not None:
+        out = fn()
         e1.record()
-        fwd_events.append((e0, e1))
-    gx, _send = jc.conv_nd_input_fold(geom, w, g)  # owned cells + halo gradients this rank sends
-    gw, gb = jc.conv_nd_weight(x_aug, w.shape, g, with_bias_grad=True)  # one pass over g for both
+        kernel_events.setdefault(name, []).append((e0, e1))
+        return out
+
+    halo_pack(x, geom, from_padded=False)  # strips this rank sends
+    x_aug = halo_assemble(x, wl["strips_fwd"], geom)
+    y = bracket("fwd", lambda: jc.conv_nd(x_aug, w, b))
+    # owned cells + halo gradients this rank sends
+    gx, _send = bracket("dgrad_fold", lambda: jc.conv_nd_input_fold(geom, w, g))
+    # one pass over g for the weight and the bias gradient
+    gw, gb = bracket("wgrad_bias", lambda: jc.conv_nd_weight(x_aug, w.shape, g, with_bias_grad=True))
     halo_fold_border_(gx, wl["strips_bwd"], geom)
     return y, gx, gw, gb
 
@@ -349,52 +363,77 @@ def swin_figures(dev, iters: int) -> dict:
     }
 
 
-def cpu_baseline(seconds_budget: float = 30.0) -> dict:
-    """The oracle (the reference's torch CPU operators) timed on the host cores on a
-    bounded sample of the same workload: batch 1 of a 512x512, 64 -> 64 tile in fp32
-    (1/32 of the step's FLOPs), rank (0, 0) of a 2x2 mesh."""
+def _cpu_conv2_step(batch: int, tile: int, dtype: torch.dtype):
+    """One step of configuration 2 for rank (0, 0) of a 2 x 2 mesh on the oracle (the torch CPU
+    operators the reference calls): halo gather of the whole mesh, conv forward, bias gradient,
+    dgrad on the padded tile, wgrad, scatter-add. Returns seconds."""
     from oracle import conv as oc
     from oracle import halo as oh
 
-    cores = torch.get_num_threads()
-    batch, ch, tile = 1, 64, 512
+    ch = 64
     torch.manual_seed(0)
-    # a 2x2 mesh so that the oracle's exchange-by-axis code runs; rank (0, 0) is timed
     mesh, k, s, p, d = (2, 2), (3, 3), (1, 1), (1, 1), (1, 1)
-    glob = torch.randn(batch, ch, 2 * tile, 2 * tile)
-    w = (torch.rand(ch, ch, 3, 3) * 2 - 1) / 24
-    b = (torch.rand(ch) * 2 - 1) / 24
-    gout = torch.randn(batch, ch, tile, tile)
+    glob = torch.randn(batch, ch, 2 * tile, 2 * tile).to(dtype)
+    w = ((torch.rand(ch, ch, 3, 3) * 2 - 1) / 24).to(dtype)
+    b = ((torch.rand(ch) * 2 - 1) / 24).to(dtype)
+    gout = torch.randn(batch, ch, tile, tile).to(dtype)
     tiles = oh.split_global(glob, mesh)
-
-    def step():
-        aug = oh.gather_mesh(tiles, mesh, k, s, p, d)
-        lp = oh.local_padding(p, mesh)
-        y = oc.forward(aug[(0, 0)], w, b, s, lp, d)
-        gb = oc.grad_bias(gout, 2)
-        gx_aug = {c: oc.dgrad(aug[c].shape, w, gout, s, lp, d) if c == (0, 0) else torch.zeros_like(aug[c]) for c in aug}
-        gw = oc.wgrad(aug[(0, 0)], w.shape, gout, s, lp, d)
-        gx = oh.scatter_add_mesh(gx_aug, mesh, k, s, p, d, (tile, tile))
-        return y, gx, gw, gb
-
-    step()  # warm-up (thread pools, oneDNN primitive cache)
+    del glob
     t0 = time.perf_counter()
-    reps = 0
-    while True:
-        step()
-        reps += 1
-        if time.perf_counter() - t0 > seconds_budget / 3:  # about 10 s of CPU work
-            break
-    sec = (time.perf_counter() - t0) / reps
-    flop = 3 * 2 * batch * ch * ch * 9 * tile * tile
+    aug = oh.gather_mesh(tiles, mesh, k, s, p, d)
+    lp = oh.local_padding(p, mesh)
+    y = oc.forward(aug[(0, 0)], w, b, s, lp, d)
+    gb = oc.grad_bias(gout, 2)
+    gx_aug = {c: oc.dgrad(aug[c].shape, w, gout, s, lp, d) if c == (0, 0) else torch.zeros_like(aug[c]) for c in aug}
+    gw = oc.wgrad(aug[(0, 0)], w.shape, gout, s, lp, d)
+    gx = oh.scatter_add_mesh(gx_aug, mesh, k, s, p, d, (tile, tile))
+    sec = time.perf_counter() - t0
+    del y, gb, gx_aug, gw, gx, aug
+    return sec
+
+
+def cpu_baseline(seconds_budget: float = 25.0) -> dict:
+    """The oracle (the reference's torch CPU operators) timed on the host cores. Runs BEFORE this
+    process touches the GPU (its second leg starts child processes).
+
+    Leg 1, the ``value``: configuration 2 at its real tile (1024 x 1024 of 2048 x 2048, 64 -> 64,
+    bf16, rank (0, 0) of the 2 x 2 mesh; the gather and the scatter-add move the whole mesh). A
+    small probe step estimates the rate; the batch (8 in the configuration) is cut to what fits
+    the time budget and reported, the tile is not cut.
+    Leg 2: configuration 1 as the reference runs it: four gloo ranks (fresh processes), one
+    training step of the 3 -> 16 -> 3 model on 512 x 512 images, batch 4, fp32, with the halo
+    all-to-alls, the loss and gradient all-reduces and Adam."""
+    from oracle import train_step as ots
+
+    cores = torch.get_num_threads()
+    dtype = torch.bfloat16
+    flop = lambda batch, tile: 3 * 2 * batch * 64 * 64 * 9 * tile * tile  # noqa: E731
+    _cpu_conv2_step(1, 128, dtype)  # warm-up (thread pools, oneDNN primitive cache)
+    probe = _cpu_conv2_step(1, 256, dtype)
+    per_batch_entry = probe * 16.0  # a 1024^2 tile is 16 times the probe
+    batch = int(max(1, min(8, seconds_budget / 2 / max(per_batch_entry, 1e-3))))
+    secs = [_cpu_conv2_step(batch, 1024, dtype)]
+    while sum(secs) + secs[-1] < seconds_budget / 2 and len(secs) < 5:
+        secs.append(_cpu_conv2_step(batch, 1024, dtype))
+    sec = sorted(secs)[len(secs) // 2]
+    c1 = {}
+    try:
+        ranks = ots.run_four_ranks(steps=3, warmup=1, batch=4, size=512, threads=max(1, cores // 4), timeout=240.0)
+        c1 = {"config1_ms_per_step": max(r[1] for r in ranks.values()) * 1e3, "config1_ranks": 4,
+              "config1_threads_per_rank": max(1, cores // 4), "config1_loss": ranks[0][0][-1]}
+    except Exception as exc:  # the CPU leg must not take the GPU figures down with it
+        c1 = {"config1_error": repr(exc)}
     return {
-        "value": flop / sec / 1e12,
+        "value": flop(batch, 1024) / sec / 1e12,
         "unit": "TFLOP/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"oracle halo gather + conv fwd/dgrad/wgrad/bias-grad + scatter-add, fp32, batch {batch} of a "
-        f"{tile}x{tile} 64->64 tile ({flop / 1e9:.1f} GFLOP of the step's 1855 GFLOP), {reps} reps, "
-        f"torch {torch.__version__} CPU, {cores} threads of {os.cpu_count()} logical cores",
+        "sample": f"configuration 2 on the oracle (torch CPU operators): halo gather + conv fwd/dgrad/wgrad/bias-grad + "
+        f"scatter-add, bf16, real 1024x1024 tile of a 2x2 mesh, 64->64, batch {batch} of 8 "
+        f"({flop(batch, 1024) / 1e9:.1f} of the step's {flop(8, 1024) / 1e9:.1f} GFLOP), {len(secs)} timed step(s) of "
+        f"{sec:.2f} s, torch {torch.__version__}, {cores} threads of {os.cpu_count()} logical cores; "
+        "configuration 1: one training step of 4 gloo ranks (see config1_* keys)",
+        **c1,
     }
 
 
@@ -469,6 +508,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
+    ap.add_argument("--cpu-baseline-only", action="store_true", help="run only the CPU leg and print its JSON object")
     ap.add_argument("--no-extras", action="store_true",
                     help="only the timed steps and the roofline kernel (a kernel trace of this run then "
                     "holds the forward kernel's launches under a name of their own)")
@@ -480,6 +520,22 @@ def main() -> int:
             file=sys.stderr,
         )
         return 2
+    if ns.cpu_baseline_only:
+        print(json.dumps(cpu_baseline()))
+        return 0
+    # The CPU leg runs first, in a child process of its own, before this process has touched
+    # the GPU: it starts further processes (the gloo ranks), and its thread pools and buffers
+    # would otherwise stay behind in the process that issues the GPU work.
+    cpu = None
+    if not ns.no_cpu_baseline:
+        import subprocess
+
+        try:
+            done = subprocess.run([sys.executable, os.path.abspath(__file__), "--cpu-baseline-only"],
+                                  capture_output=True, text=True, timeout=900)
+            cpu = json.loads(done.stdout.strip().splitlines()[-1])
+        except Exception as exc:
+            cpu = {"value": None, "unit": "TFLOP/s", "cores": None, "kind": "port", "sample": f"CPU leg failed: {exc!r}"}
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the HIP kernels have no CPU fallback.", file=sys.stderr)
         return 2
@@ -502,9 +558,9 @@ def main() -> int:
     t0 = time.perf_counter()
     e0, e1 = _events()
     e0.record()
-    fwd_events: list = []
+    kernel_events: dict = {}
     for _ in range(ns.steps):
-        conv_step(wl, fwd_events)
+        conv_step(wl, kernel_events)
     e1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / ns.steps
@@ -516,20 +572,24 @@ def main() -> int:
     geom = wl["geom"]
     x_aug = halo_assemble(wl["x"], wl["strips_fwd"], geom)
     it = max(5, ns.steps)
-    # the dominant kernel: average duration of the forward launches of the timed steps
-    # (the 5 us weight re-layout launch that precedes each one is inside the bracket)
-    ms_fwd = sum(a.elapsed_time(b) for a, b in fwd_events) / len(fwd_events)
+    # the three convolution launches of the timed steps (the small weight re-layout and
+    # reduction launches that belong to each are inside its bracket); the roofline entry is
+    # the DOMINANT one: the longest
+    ms_kernel = {k: sum(a.elapsed_time(b) for a, b in v) / len(v) for k, v in kernel_events.items()}
+    ms_fwd = ms_kernel["fwd"]
+    dominant = max(ms_kernel, key=ms_kernel.get)
     tf = lambda ms: flop_one / (ms * 1e-3) / 1e12  # noqa: E731
     roofline = {
-        "kernel": "conv3x3_mfma_kernel (forward, config 2)",
+        "kernel": CONV_KERNEL_NAMES[dominant],
         "bound": "mfma",
-        "achieved": tf(ms_fwd),
+        "achieved": tf(ms_kernel[dominant]),
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
-        "frac": tf(ms_fwd) / PEAK_BF16_TFLOPS,
-        "traffic": CONV_FWD_TRAFFIC_BYTES,
+        "frac": tf(ms_kernel[dominant]) / PEAK_BF16_TFLOPS,
+        "traffic": CONV_TRAFFIC_BYTES[dominant],
     }
-    extra = {"conv_fwd": {"ms": ms_fwd, "tflops": tf(ms_fwd), "frac_mfma_peak": tf(ms_fwd) / PEAK_BF16_TFLOPS}}
+    extra = {f"conv_{k}_in_step": {"ms": v, "tflops": tf(v), "frac_mfma_peak": tf(v) / PEAK_BF16_TFLOPS}
+             for k, v in ms_kernel.items()}
     if not ns.no_extras:
         extra.update(conv2_extras(wl, x_aug, it, flop_one, flop_step, ms_fwd))
         extra.update(attention_figures(dev, max(10, it)))
@@ -559,7 +619,7 @@ def main() -> int:
             "frac_mfma_peak": value / PEAK_BF16_TFLOPS,
         },
         "roofline": roofline,
-        "cpu_baseline": None if ns.no_cpu_baseline else cpu_baseline(),
+        "cpu_baseline": cpu,
         "extra": extra,
     }
     print(json.dumps(line))

@@ -143,8 +143,9 @@ class RingSeat:
                     for w in self._issue_hop(held, into, s):
                         w.wait()  # a torch.distributed handle makes the CURRENT stream wait, not the host
                     self._landed[(s + 1) % 2].record(wire)
-                for t in (*held, *into):
-                    t.record_stream(wire)
+                # No record_stream() on the tensors the transfer touched: the compute stream waits for
+                # `landed` before the pass ends, so whatever it frees or reuses afterwards is ordered
+                # behind every access of the transfer stream (and record_stream is slow on the host).
             held = into
 
     # ------------------------------------------------------------------ forward
@@ -203,6 +204,7 @@ class RingSeat:
             raise ValueError("save_scope='local' relays the dK/dV partials: pass relay_fn")
         dk_own = dv_own = None
         inbox: tuple | None = None  # (recv_dk, recv_dv, works or event) of the previous step's relay
+        keep_alive: list = []       # partials a transfer may still be reading; dropped after the last `arrived` wait
         wire = self._wire_back if self._wire is not None else None
         if wire is not None:
             compute = torch.cuda.current_stream(q.device)
@@ -242,8 +244,7 @@ class RingSeat:
                         if w is not None:
                             w.wait()
                     arrived.record(wire)
-                for t in (dk_j, dv_j, r_dk, r_dv):
-                    t.record_stream(wire)
+                keep_alive.append((dk_j, dv_j))  # read by the transfer stream until `arrived`
                 inbox = (r_dk, r_dv, arrived)
         if inbox is not None:
             take(inbox)
