@@ -6,7 +6,7 @@
 //                    S^T  = K Q^T                 A = K rows,    B = Q (registers)
 //                    dP^T = V dO^T                A = V rows,    B = dO (registers)
 //                    dS^T = P^T o (dP^T - delta) * scale      (lane-local)
-//                    dQ^T += K^T dS^T             A = K^T (transposed LDS copy),
+//                    dQ^T += K^T dS^T             A = K^T (LDS transpose reads),
 //                                                 B = dS^T straight from registers
 //                  It also computes delta = rowsum(dO o O) and leaves it in the
 //                  workspace for the second kernel.
@@ -14,16 +14,19 @@
 //                    S  = Q K^T                   A = Q rows,    B = K (registers)
 //                    dP = dO V^T                  A = dO rows,   B = V (registers)
 //                    P, dS from lse / delta of the tile (broadcast LDS reads)
-//                    dV^T += dO^T P               A = dO^T (transposed LDS copy)
-//                    dK^T += Q^T dS               A = Q^T  (transposed LDS copy)
+//                    dV^T += dO^T P               A = dO^T (LDS transpose reads)
+//                    dK^T += Q^T dS               A = Q^T  (LDS transpose reads)
 //   The score tile is recomputed in each kernel (7 matrix products instead of the
 //   5 of a one-kernel formulation) so that P / dS are always produced in the
 //   register layout the next MFMA consumes and never travel through LDS.
 //
 //   Workgroup: 512 threads = 8 wavefronts = 4 blocks of 32 rows (queries for dQ,
 //   keys for dK/dV) x 2 halves of the streamed side, combined through LDS.
-//   Streamed tiles are fetched as 8-row x 2-column dword tasks, which one thread
-//   can write both untransposed and transposed (8 channels-per-slot trick).
+//   Streamed tiles (64 rows x 128 bytes) travel from memory straight into LDS, row-major
+//   with the 16-byte chunks of a row XOR-swizzled by row % 8 (no registers, no vector
+//   instructions, no second, transposed copy): the transposed fragments come from
+//   ds_read_b64_tr_b16 (within 16 lanes, lane i receives element i % 4 of the 8 bytes
+//   that lanes i / 4 + 4 j point at, j = 0..3), two reads of 4 consecutive rows each.
 //
 // Reference behaviour restated here:
 //   jigsaw/modules/attention/_functional/cores/math.py:125-149
@@ -39,76 +42,64 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
 
 constexpr int D = 64;
 constexpr int BR = 128;           // resident rows per workgroup (4 blocks of 32)
 constexpr int BT = 64;            // streamed rows per tile
 constexpr int THREADS = 512;
-constexpr int ROWB = 144;         // LDS row pitch in bytes
-constexpr int TILE = BT * ROWB;   // 9216: one 64 x 64 bf16 tile, natural or transposed
+constexpr int ROWB = D * 2;       // bytes per row of a tile in LDS (no padding)
+constexpr int NAT = BT * ROWB;    // 8192: one 64 x 64 bf16 tile
 constexpr float LOG2E = 1.4426950408889634f;
-
-// Transposed tiles hold streamed row x (0..63) at position
-//   (x & ~15) | ((x % 8) / 4) * 8 | ((x % 16) / 8) * 4 | (x % 4):
-// inside each group of 16 the order is the one an accumulator lane holds its rows in.
-
-// A task = 8 consecutive streamed rows x 2 consecutive columns, held as 8 dwords.
-struct Task {
-  uint32_t w[8];
-};
-
-__device__ __forceinline__ void task_load(Task& t, const uint16_t* tile, int g8, int cp) {
-#pragma unroll
-  for (int i = 0; i < 8; ++i)
-    t.w[i] = *reinterpret_cast<const uint32_t*>(tile + (g8 * 8 + i) * D + 2 * cp);
-}
-
-__device__ __forceinline__ void task_store_nat(const Task& t, unsigned char* nat, int g8, int cp) {
-#pragma unroll
-  for (int i = 0; i < 8; ++i)
-    *reinterpret_cast<uint32_t*>(nat + (g8 * 8 + i) * ROWB + 4 * cp) = t.w[i];
-}
-
-__device__ __forceinline__ void task_store_tr(const Task& t, unsigned char* tr, int g8, int cp) {
-  const int pos_lo = (g8 >> 1) * 16 + (g8 & 1) * 4;  // rows 8*g8 .. +3
-  const int pos_hi = pos_lo + 8;                     // rows 8*g8+4 .. +7
-#pragma unroll
-  for (int e = 0; e < 2; ++e) {
-    const uint32_t sel = e ? 0x07060302u : 0x05040100u;
-    u32x2 lo, hi;
-    lo.x = __builtin_amdgcn_perm(t.w[1], t.w[0], sel);
-    lo.y = __builtin_amdgcn_perm(t.w[3], t.w[2], sel);
-    hi.x = __builtin_amdgcn_perm(t.w[5], t.w[4], sel);
-    hi.y = __builtin_amdgcn_perm(t.w[7], t.w[6], sel);
-    unsigned char* row = tr + (2 * cp + e) * ROWB;
-    *reinterpret_cast<u32x2*>(row + pos_lo * 2) = lo;
-    *reinterpret_cast<u32x2*>(row + pos_hi * 2) = hi;
-  }
-}
 
 __device__ __forceinline__ bf16x8 lds_frag(const unsigned char* p) {
   return __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(p));
 }
 
-// Natural (untransposed) 64 x 64 tiles travel from memory straight into LDS (no registers,
-// no ds_write): a wavefront instruction lands 64 x 16 bytes contiguously, lane order. Rows
-// are 128 bytes, and the 16-byte chunks of a row are XOR-swizzled with (row / 2) % 8 so that
-// the 16 lanes a fragment read serves per cycle hit 16 distinct chunks of the banks.
-constexpr int NAT = BT * D * 2;  // 8192 bytes
-
-// Four of the 8 instructions of a tile: the 256 threads of a half fetch 4 KB per call.
-__device__ __forceinline__ void nat_dma(const uint16_t* tile, unsigned char* lds_tile, int th, int part) {
-  const int w = (th >> 6) + 4 * part;          // instruction 0..7 -> rows 8w .. 8w+7
-  const int i = th & 63;
-  const int row = 8 * w + (i >> 3);
-  const int chunk = (i & 7) ^ ((row >> 1) & 7);
-  __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(tile) + row * (D * 2) + chunk * 16,
-                                   (__attribute__((address_space(3))) void*)(lds_tile + w * 1024), 16, 0, 0);
+// One wavefront instruction lands 64 x 16 bytes contiguously in LDS, lane order = 8 rows: lane L
+// sits at row L / 8, chunk position L % 8 and fetches chunk (L % 8) ^ (row % 8) of its row.
+// Written in assembly: wave-uniform 64-bit source in scalar registers, the lane's constant
+// offset, the LDS address of the 1 KB block in M0. (With the compiler's own form of this load
+// it orders every later LDS read behind ALL outstanding transfers, also those of the tile
+// after next; the kernels order reads and transfers themselves, by their waits and barriers.)
+__device__ __forceinline__ uint32_t dma_lane_offset(int lane) {
+  return (uint32_t)((lane >> 3) * ROWB + (((lane & 7) ^ (lane >> 3)) << 4));
+}
+__device__ __forceinline__ void dma_1k(const char* src, uint32_t lane_off, uint32_t lds_dst) {
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_off), "s"(src), "s"(lds_dst) : "m0");
+}
+__device__ __forceinline__ uint32_t lds_address(const unsigned char* p) {
+  typedef __attribute__((address_space(3))) unsigned char* lds_bytes;
+  return (uint32_t)(uintptr_t)((lds_bytes)p);
 }
 
-// fragment of a natural tile: row r (0..63), 16-byte chunk c (0..7)
+// fragment of a row-major tile: row r (0..63), 16-byte chunk c (0..7)
 __device__ __forceinline__ bf16x8 nat_frag(const unsigned char* nat, int r, int c) {
-  return __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(nat + r * (D * 2) + ((c ^ ((r >> 1) & 7)) << 4)));
+  return lds_frag(nat + r * ROWB + ((c ^ (r & 7)) << 4));
+}
+
+// Per-lane constant part of the address of a TRANSPOSED fragment (A operand: 32 columns of the
+// tile x 16 of its rows): lane p of a group of 16 points at row +4 kg + p / 4, columns 32 nb +
+// 16 (group % 2) + 4 (p % 4); the row's swizzle is 4 kg + p / 4 whatever multiple of 8 the
+// fragment starts at.
+__device__ __forceinline__ int tr_lane_offset(int lane, int nb) {
+  const int pp = lane & 15, g1 = (lane >> 4) & 1, kg = lane >> 5;
+  const int rsw = 4 * kg + (pp >> 2);
+  return rsw * ROWB + (((4 * nb + 2 * g1 + ((pp & 3) >> 1)) ^ rsw) << 4) + 8 * (pp & 1);
+}
+// Transposed fragment whose 16 rows start at `row0` (a multiple of 16): slots 0..3 = rows
+// row0 + 4 kg + 0..3, slots 4..7 = rows row0 + 8 + 4 kg + 0..3: the order an accumulator lane
+// holds its rows in.
+__device__ __forceinline__ bf16x8 tr_frag(const unsigned char* nat, int lane_off, int row0) {
+  typedef __attribute__((address_space(3))) i16x4* tr_ptr;
+  const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr)(nat + lane_off + row0 * ROWB));
+  const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr)(nat + lane_off + (row0 + 8) * ROWB));
+  u32x4 w;
+  w.x = __builtin_bit_cast(u32x2, lo).x;
+  w.y = __builtin_bit_cast(u32x2, lo).y;
+  w.z = __builtin_bit_cast(u32x2, hi).x;
+  w.w = __builtin_bit_cast(u32x2, hi).y;
+  return __builtin_bit_cast(bf16x8, w);
 }
 
 __device__ __forceinline__ bf16x8 pack8(const float* e) {
@@ -139,9 +130,9 @@ struct BwdArgs {
 };
 
 // ------------------------------------------------------------------ dQ kernel
-constexpr int DQ_BUF = 2 * NAT + TILE;       // K natural, V natural, K transposed
+constexpr int DQ_BUF = 2 * NAT;             // K tile, V tile
 constexpr int DQ_HALF = 2 * DQ_BUF;         // double buffered
-constexpr int DQ_LDS = 2 * DQ_HALF;         // 102400
+constexpr int DQ_LDS = 2 * DQ_HALF;         // 65536 (and at least 4 x 32 x 64 floats for the hand-over)
 
 __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -149,8 +140,6 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
   const int lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, kg = lane >> 5;
   const int qb = wave & 3, ks = wave >> 2;
-  const int th = tid & 255;
-  const int g8 = th >> 5, cp = th & 31;
   const long long b = blockIdx.y;
   const int q0 = blockIdx.x * BR + qb * 32;
   const int khalf = p.sk >> 1;
@@ -159,8 +148,13 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
   const long long qi = b * p.sq + q0 + ln;
 
   unsigned char* lds = smem + ks * DQ_HALF;
-  const uint16_t* kbase = p.k + (b * p.sk + (long long)ks * khalf) * D;
-  const uint16_t* vbase = p.v + (b * p.sk + (long long)ks * khalf) * D;
+  // this wavefront moves rows 16 qb .. 16 qb + 15 of the K tile and of the V tile of its half
+  const int ks_u = __builtin_amdgcn_readfirstlane(ks), qb_u = __builtin_amdgcn_readfirstlane(qb);
+  const char* kdma = reinterpret_cast<const char*>(p.k + (b * p.sk + (long long)ks_u * khalf) * D) + 16 * qb_u * ROWB;
+  const char* vdma = reinterpret_cast<const char*>(p.v + (b * p.sk + (long long)ks_u * khalf) * D) + 16 * qb_u * ROWB;
+  const uint32_t dma_off = dma_lane_offset(lane);
+  const uint32_t lds_dma = lds_address(smem) + (uint32_t)(ks_u * DQ_HALF + 16 * qb_u * ROWB);
+  const int tr_off[2] = {tr_lane_offset(lane, 0), tr_lane_offset(lane, 1)};
 
   bf16x8 qf[4], dof[4];
   float delta;
@@ -182,22 +176,18 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
   }
   const float lse2 = p.lse[qi] * LOG2E;
 
-  Task tk;
   // K and V of tile t straight into buffer `buf` (it must be free: the barrier that ended
-  // the iteration before), K once more through registers for the transposed copy
+  // the iteration before)
   auto issue_loads = [&](int t, int buf) {
-    unsigned char* base = lds + buf * DQ_BUF;
-    const uint16_t* kt_g = kbase + (long long)t * BT * D;
-    const uint16_t* vt_g = vbase + (long long)t * BT * D;
-    nat_dma(kt_g, base, th, 0);
-    nat_dma(kt_g, base, th, 1);
-    nat_dma(vt_g, base + NAT, th, 0);
-    nat_dma(vt_g, base + NAT, th, 1);
-    task_load(tk, kt_g, g8, cp);
+    const long long off = (long long)t * NAT;
+    const uint32_t dst = lds_dma + (uint32_t)(buf * DQ_BUF);
+    dma_1k(kdma + off, dma_off, dst);
+    dma_1k(kdma + off + 8 * ROWB, dma_off, dst + 8 * ROWB);
+    dma_1k(vdma + off, dma_off, dst + NAT);
+    dma_1k(vdma + off + 8 * ROWB, dma_off, dst + NAT + 8 * ROWB);
   };
-  auto store_tile = [&](int buf) {
-    task_store_tr(tk, lds + buf * DQ_BUF + 2 * NAT, g8, cp);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the direct-to-LDS loads of this buffer have landed
+  auto tiles_landed = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the transfers into the other buffer have landed
   };
 
   f32x16 dq[2];
@@ -215,7 +205,6 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
   auto compute_tile = [&](int buf) {
     const unsigned char* kn = lds + buf * DQ_BUF;
     const unsigned char* vn = kn + NAT;
-    const unsigned char* kt = kn + 2 * NAT;
     f32x16 s[2], dp[2];
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb)
@@ -235,8 +224,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
       return pack8(e);
     };
     auto dq_mfma = [&](int sb, int t, int nb, const bf16x8& f) {
-      dq[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-          lds_frag(kt + (nb * 32 + ln) * ROWB + (sb * 32 + 16 * t + 8 * kg) * 2), f, dq[nb], 0, 0, 0);
+      dq[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(kn, tr_off[nb], sb * 32 + 16 * t), f, dq[nb], 0, 0, 0);
     };
     // block 0: scores and dP
 #pragma unroll
@@ -275,13 +263,13 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
 
   int buf = 0;
   issue_loads(0, 0);
-  store_tile(0);
+  tiles_landed();
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
     const bool has_next = t + 1 < ntiles;
     if (has_next) issue_loads(t + 1, buf ^ 1);
     compute_tile(buf);
-    if (has_next) store_tile(buf ^ 1);
+    tiles_landed();
     __syncthreads();
     buf ^= 1;
   }
@@ -312,8 +300,9 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
 
 // -------------------------------------------------------------- dK/dV kernel
 constexpr int DKV_STATS = 2 * BT * 4;                 // lse2[64], delta[64] as floats
-constexpr int DKV_HALF = 4 * TILE + DKV_STATS;        // Q nat, Q tr, dO nat, dO tr + stats
-constexpr int DKV_LDS = 4 * DKV_HALF;                 // 149504: two query halves, double buffered
+constexpr int DKV_HALF = 2 * NAT + DKV_STATS;         // Q tile, dO tile + stats
+constexpr int DKV_LDS = 4 * DKV_HALF;                 // 67584: two query halves, double buffered
+static_assert(DKV_LDS >= 4 * 64 * 64 * 4, "the hand-over of the partial dK / dV reuses the tile buffers");
 
 __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -322,7 +311,6 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
   const int ln = lane & 31, kg = lane >> 5;
   const int kb = wave & 3, qs = wave >> 2;
   const int th = tid & 255;
-  const int g8 = th >> 5, cp = th & 31;
   const long long b = blockIdx.y;
   const int k0 = blockIdx.x * BR + kb * 32;
   const int qhalf = p.sq >> 1;
@@ -330,10 +318,16 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
   const float c2 = p.scale * LOG2E;
   const long long ki = b * p.sk + k0 + ln;
 
-  unsigned char* lds = smem + qs * (2 * DKV_HALF);  // two buffers: Q nat, Q tr, dO nat, dO tr, stats
+  unsigned char* lds = smem + qs * (2 * DKV_HALF);  // two buffers: Q tile, dO tile, stats
   const long long qrow0 = b * p.sq + (long long)qs * qhalf;
-  const uint16_t* qbase = p.q + qrow0 * D;
-  const uint16_t* dbase = p.dout + qrow0 * D;
+  // this wavefront moves rows 16 kb .. 16 kb + 15 of the Q tile and of the dO tile of its half
+  const int qs_u = __builtin_amdgcn_readfirstlane(qs), kb_u = __builtin_amdgcn_readfirstlane(kb);
+  const long long qrow0_u = b * p.sq + (long long)qs_u * qhalf;
+  const char* qdma = reinterpret_cast<const char*>(p.q + qrow0_u * D) + 16 * kb_u * ROWB;
+  const char* ddma = reinterpret_cast<const char*>(p.dout + qrow0_u * D) + 16 * kb_u * ROWB;
+  const uint32_t dma_off = dma_lane_offset(lane);
+  const uint32_t lds_dma = lds_address(smem) + (uint32_t)(qs_u * (2 * DKV_HALF) + 16 * kb_u * ROWB);
+  const int tr_off[2] = {tr_lane_offset(lane, 0), tr_lane_offset(lane, 1)};
 
   bf16x8 kf[4], vf[4];
   {
@@ -346,24 +340,24 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
     }
   }
 
-  Task tq, tdo;
   float st_reg = 0.0f;
-  auto issue_loads = [&](int t) {
-    task_load(tq, qbase + (long long)t * BT * D, g8, cp);
-    task_load(tdo, dbase + (long long)t * BT * D, g8, cp);
-    // One plain load for every lane, used only when the tile goes to LDS: a load under a
+  auto issue_loads = [&](int t, int buf) {
+    const long long off = (long long)t * NAT;
+    const uint32_t dst = lds_dma + (uint32_t)(buf * DKV_HALF);
+    dma_1k(qdma + off, dma_off, dst);
+    dma_1k(qdma + off + 8 * ROWB, dma_off, dst + 8 * ROWB);
+    dma_1k(ddma + off, dma_off, dst + NAT);
+    dma_1k(ddma + off + 8 * ROWB, dma_off, dst + NAT + 8 * ROWB);
+    // One plain load for every lane, used only when the statistics go to LDS: a load under a
     // per-lane condition, or arithmetic on its result here, would make the wavefront wait
-    // for it (and for the tile loads issued before it) on the spot.
+    // for it (and for the transfers issued before it) on the spot.
     const float* src = th < BT ? p.lse : p.delta;
     st_reg = src[qrow0 + (long long)t * BT + (th & (BT - 1))];
   };
-  auto store_tile = [&](int buf) {
+  auto store_stats = [&](int buf) {
     unsigned char* base = lds + buf * DKV_HALF;
-    task_store_nat(tq, base, g8, cp);
-    task_store_tr(tq, base + TILE, g8, cp);
-    task_store_nat(tdo, base + 2 * TILE, g8, cp);
-    task_store_tr(tdo, base + 3 * TILE, g8, cp);
-    if (th < 2 * BT) reinterpret_cast<float*>(base + 4 * TILE)[th] = th < BT ? st_reg * LOG2E : st_reg;
+    if (th < 2 * BT) reinterpret_cast<float*>(base + 2 * NAT)[th] = th < BT ? st_reg * LOG2E : st_reg;
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the transfers into this buffer have landed
   };
 
   f32x16 dk[2], dv[2];
@@ -378,10 +372,8 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
   // dS is kept without the softmax scale, which multiplies dK once at the end
   auto compute_tile = [&](int buf) {
     const unsigned char* qn = lds + buf * DKV_HALF;
-    const unsigned char* qt = qn + TILE;
-    const unsigned char* dn = qn + 2 * TILE;
-    const unsigned char* dt = qn + 3 * TILE;
-    const float* st = reinterpret_cast<const float*>(qn + 4 * TILE);  // lse2[64] then delta[64]
+    const unsigned char* dn = qn + NAT;
+    const float* st = reinterpret_cast<const float*>(qn + 2 * NAT);  // lse2[64] then delta[64]
     bf16x8 pf[2][2], dsf[2][2];
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
@@ -393,9 +385,8 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
       }
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        const int off = (sb * 32 + ln) * ROWB + (16 * c + 8 * kg) * 2;
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(qn + off), kf[c], s, 0, 0, 0);
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(dn + off), vf[c], dp, 0, 0, 0);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nat_frag(qn, sb * 32 + ln, 2 * c + kg), kf[c], s, 0, 0, 0);
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nat_frag(dn, sb * 32 + ln, 2 * c + kg), vf[c], dp, 0, 0, 0);
       }
       // register i of this lane: query sb*32 + 8*(i/4) + 4*kg + i%4, key ln
 #pragma unroll
@@ -423,15 +414,14 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) {
-          const int off = (nb * 32 + ln) * ROWB + (sb * 32 + 16 * t + 8 * kg) * 2;
-          dv[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(dt + off), pf[sb][t], dv[nb], 0, 0, 0);
-          dk[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(qt + off), dsf[sb][t], dk[nb], 0, 0, 0);
+          dv[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(dn, tr_off[nb], sb * 32 + 16 * t), pf[sb][t], dv[nb], 0, 0, 0);
+          dk[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(qn, tr_off[nb], sb * 32 + 16 * t), dsf[sb][t], dk[nb], 0, 0, 0);
         }
   };
 
   int buf = 0;
-  issue_loads(0);
-  store_tile(0);
+  issue_loads(0, 0);
+  store_stats(0);
   // The K / V fragments came straight from memory: they are waited for here, once. Left
   // to the first MFMA that reads them, the wait would sit inside the loop, behind the
   // tile loads that every iteration has just issued.
@@ -440,9 +430,9 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
     const bool has_next = t + 1 < ntiles;
-    if (has_next) issue_loads(t + 1);
+    if (has_next) issue_loads(t + 1, buf ^ 1);
     compute_tile(buf);
-    if (has_next) store_tile(buf ^ 1);
+    if (has_next) store_stats(buf ^ 1);
     __syncthreads();
     buf ^= 1;
   }

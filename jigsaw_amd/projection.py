@@ -33,6 +33,41 @@ def _nt(out, a, w, bias, rows, n_out, k_in, a_heads, out_heads, dims) -> None:
     _lib.check(rc, "jg_proj_nt")
 
 
+def _cast_cached(t: torch.Tensor | None, dtype: torch.dtype, transposed: bool = False) -> torch.Tensor | None:
+    """``t`` in ``dtype``, contiguous (optionally its transpose), remembered on the tensor until
+    its next in-place update: under autocast the parameters are fp32 and every forward and
+    backward would otherwise launch a cast (and the input gradient a transpose copy) per layer.
+    The tensor's version counter, which every in-place update (an optimizer step) bumps,
+    invalidates the copies."""
+    if t is None:
+        return None
+    if not transposed and t.dtype == dtype and t.is_contiguous():
+        return t
+    key = (dtype, transposed)
+    cache = getattr(t, "_jg_casts", None)
+    if cache is None or cache[0] != t._version:
+        cache = (t._version, {})
+        try:
+            t._jg_casts = cache
+        except AttributeError:  # a tensor subclass without a __dict__: no cache
+            pass
+    got = cache[1].get(key)
+    if got is None:
+        src = t.detach()
+        got = (src.t() if transposed else src).to(dtype).contiguous()
+        cache[1][key] = got
+    return got
+
+
+def _transposed(ctx, w: torch.Tensor) -> torch.Tensor:
+    """The transposed weight of the input-gradient GEMM: the cached copy of the parameter when
+    the parameter is still the one the forward saw, else a transpose of the saved cast."""
+    ref = getattr(ctx, "weight_ref", None)
+    if ref is not None and ref._version == ctx.weight_version:
+        return _cast_cached(ref, w.dtype, transposed=True)
+    return w.t().contiguous()
+
+
 def _grad_dtype(compute: torch.dtype, dtypes) -> torch.dtype:
     """fp32 when every parameter that gets a gradient is fp32 (autocast), else the compute dtype."""
     return torch.float32 if all(dt in (None, torch.float32) for dt in dtypes) else compute
@@ -70,12 +105,13 @@ class _QkvProjection(torch.autograd.Function):
         lead, s = tuple(x.shape[:-2]), x.shape[-2]
         b = math.prod(lead)
         xc = x.contiguous()
-        w = weight.to(x.dtype).contiguous()
-        bs = None if bias is None else bias.to(x.dtype).contiguous()
+        w = _cast_cached(weight, x.dtype)
+        bs = _cast_cached(bias, x.dtype)
         out = torch.empty((3, *lead, heads, s, d), dtype=x.dtype, device=x.device)
         if b * s:
             _nt(out, xc, w, bs, b * s, n_out, c, False, True, (b, heads, s, d))
         ctx.save_for_backward(xc, w)
+        ctx.weight_ref, ctx.weight_version = weight, weight._version
         ctx.dims = (b, heads, s, d)
         ctx.has_bias = bias is not None
         ctx.dtypes = (weight.dtype, None if bias is None else bias.dtype)
@@ -95,7 +131,7 @@ class _QkvProjection(torch.autograd.Function):
         else:
             if ctx.needs_input_grad[0]:
                 gx = torch.empty_like(xc)
-                _nt(gx, g, w.t().contiguous(), None, b * s, c, n_out, True, False, ctx.dims)
+                _nt(gx, g, _transposed(ctx, w), None, b * s, c, n_out, True, False, ctx.dims)
             need_b = ctx.has_bias and ctx.needs_input_grad[2]
             if ctx.needs_input_grad[1] or need_b:
                 gw, gb = _tn(g, xc, b * s, n_out, c, True, False, ctx.dims, need_b, _grad_dtype(g.dtype, ctx.dtypes))
@@ -119,12 +155,13 @@ class _HeadsProjection(torch.autograd.Function):
         lead = tuple(out.shape[:-3])
         b = math.prod(lead)
         oc = out.contiguous()
-        w = weight.to(out.dtype).contiguous()
-        bs = None if bias is None else bias.to(out.dtype).contiguous()
+        w = _cast_cached(weight, out.dtype)
+        bs = _cast_cached(bias, out.dtype)
         y = torch.empty((*lead, s, n_out), dtype=out.dtype, device=out.device)
         if b * s:
             _nt(y, oc, w, bs, b * s, n_out, k, True, False, (b, h, s, d))
         ctx.save_for_backward(oc, w)
+        ctx.weight_ref, ctx.weight_version = weight, weight._version
         ctx.dims = (b, h, s, d)
         ctx.has_bias = bias is not None
         ctx.dtypes = (weight.dtype, None if bias is None else bias.dtype)
@@ -144,7 +181,7 @@ class _HeadsProjection(torch.autograd.Function):
         else:
             if ctx.needs_input_grad[0]:
                 go = torch.empty_like(oc)
-                _nt(go, g, w.t().contiguous(), None, b * s, k, n_out, False, True, ctx.dims)
+                _nt(go, g, _transposed(ctx, w), None, b * s, k, n_out, False, True, ctx.dims)
             need_b = ctx.has_bias and ctx.needs_input_grad[2]
             if ctx.needs_input_grad[1] or need_b:
                 gw, gb = _tn(g, oc, b * s, n_out, k, False, True, ctx.dims, need_b, _grad_dtype(g.dtype, ctx.dtypes))
@@ -165,12 +202,13 @@ class _Linear(torch.autograd.Function):
             raise ValueError(f"x has {x.shape[-1] if x.dim() else 0} features, the weight takes {k}")
         xc = x.contiguous()
         rows = xc.numel() // k
-        w = weight.to(x.dtype).contiguous()
-        bs = None if bias is None else bias.to(x.dtype).contiguous()
+        w = _cast_cached(weight, x.dtype)
+        bs = _cast_cached(bias, x.dtype)
         y = torch.empty((*x.shape[:-1], n_out), dtype=x.dtype, device=x.device)
         if rows:
             _nt(y, xc, w, bs, rows, n_out, k, False, False, (1, 1, 1, 1))
         ctx.save_for_backward(xc, w)
+        ctx.weight_ref, ctx.weight_version = weight, weight._version
         ctx.has_bias = bias is not None
         ctx.dtypes = (weight.dtype, None if bias is None else bias.dtype)
         return y
@@ -190,7 +228,7 @@ class _Linear(torch.autograd.Function):
         else:
             if ctx.needs_input_grad[0]:
                 gx = torch.empty_like(xc)
-                _nt(gx, g, w.t().contiguous(), None, rows, k, n_out, False, False, (1, 1, 1, 1))
+                _nt(gx, g, _transposed(ctx, w), None, rows, k, n_out, False, False, (1, 1, 1, 1))
             if ctx.needs_input_grad[1] or need_b:
                 gw, gb = _tn(g, xc, rows, n_out, k, False, False, (1, 1, 1, 1), need_b, _grad_dtype(g.dtype, ctx.dtypes))
         dt_w, dt_b = ctx.dtypes
