@@ -130,9 +130,15 @@ struct BwdArgs {
 };
 
 // ------------------------------------------------------------------ dQ kernel
+constexpr int NBUF = 4;                     // tiles in flight per half: read back, current, read ahead, landing
 constexpr int DQ_BUF = 2 * NAT;             // K tile, V tile
-constexpr int DQ_HALF = 2 * DQ_BUF;         // double buffered
-constexpr int DQ_LDS = 2 * DQ_HALF;         // 65536 (and at least 4 x 32 x 64 floats for the hand-over)
+constexpr int DQ_HALF = NBUF * DQ_BUF;
+constexpr int DQ_LDS = 2 * DQ_HALF;         // 131072 (and at least 4 x 32 x 64 floats for the hand-over)
+
+// Scheduling classes of __builtin_amdgcn_sched_group_barrier
+#define JG_GROUP_VALU 0x002
+#define JG_GROUP_MFMA 0x008
+#define JG_GROUP_DS_READ 0x100
 
 __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -155,6 +161,27 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
   const uint32_t dma_off = dma_lane_offset(lane);
   const uint32_t lds_dma = lds_address(smem) + (uint32_t)(ks_u * DQ_HALF + 16 * qb_u * ROWB);
   const int tr_off[2] = {tr_lane_offset(lane, 0), tr_lane_offset(lane, 1)};
+  // row fragments: row ln of a 32-row block, chunk 2 c + kg
+  int row_off[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) row_off[c] = ln * ROWB + (((2 * c + kg) ^ (ln & 7)) << 4);
+
+  // K and V of tile t straight into its buffer (free since the barrier that ended the tile before)
+  auto issue_loads = [&](int t) {
+    const long long off = (long long)t * NAT;
+    const uint32_t dst = lds_dma + (uint32_t)((t & (NBUF - 1)) * DQ_BUF);
+    dma_1k(kdma + off, dma_off, dst);
+    dma_1k(kdma + off + 8 * ROWB, dma_off, dst + 8 * ROWB);
+    dma_1k(vdma + off, dma_off, dst + NAT);
+    dma_1k(vdma + off + 8 * ROWB, dma_off, dst + NAT + 8 * ROWB);
+  };
+  auto tiles_landed = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's transfers have landed
+  };
+
+  // the first tiles are on their way while the wavefront fetches its own rows
+  issue_loads(0);
+  if (ntiles > 1) issue_loads(1);
 
   bf16x8 qf[4], dof[4];
   float delta;
@@ -175,20 +202,9 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
     if (ks == 0 && kg == 0) p.delta[qi] = delta;
   }
   const float lse2 = p.lse[qi] * LOG2E;
-
-  // K and V of tile t straight into buffer `buf` (it must be free: the barrier that ended
-  // the iteration before)
-  auto issue_loads = [&](int t, int buf) {
-    const long long off = (long long)t * NAT;
-    const uint32_t dst = lds_dma + (uint32_t)(buf * DQ_BUF);
-    dma_1k(kdma + off, dma_off, dst);
-    dma_1k(kdma + off + 8 * ROWB, dma_off, dst + 8 * ROWB);
-    dma_1k(vdma + off, dma_off, dst + NAT);
-    dma_1k(vdma + off + 8 * ROWB, dma_off, dst + NAT + 8 * ROWB);
-  };
-  auto tiles_landed = [&]() {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the transfers into the other buffer have landed
-  };
+  f32x16 minus_delta;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) minus_delta[i] = -delta;
 
   f32x16 dq[2];
 #pragma unroll
@@ -196,83 +212,91 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) dq[nb][i] = 0.0f;
 
-  // One 64-key tile. The two 32-key blocks are software pipelined: the score / dP
-  // products of block 1 go to the matrix core one instruction at a time with the
-  // exponentials of block 0 behind them, and the dQ products of a fragment run under
-  // the vector work of the next one. The fences pin that order. dS is kept without the
-  // softmax scale, which multiplies dQ once at the end.
-#define JG_FENCE() __builtin_amdgcn_sched_barrier(0)
-  auto compute_tile = [&](int buf) {
-    const unsigned char* kn = lds + buf * DQ_BUF;
-    const unsigned char* vn = kn + NAT;
-    f32x16 s[2], dp[2];
+  // The stream of 32-key blocks is software pipelined three deep. While the vector unit turns the
+  // scores and dP of block j into dS (B), the matrix core computes the scores and dP of block
+  // j + 1 (A, 8 instructions) and adds block j - 1 to dQ (C, 4 instructions): the three are
+  // independent, so every matrix instruction has about seven vector instructions to run
+  // under it. dS is kept without the softmax scale, which multiplies dQ once at the end.
+  f32x16 s_cur, dp_cur;
+  bf16x8 ds_prev[2];
+  auto scores = [&](const unsigned char* kn, int sb, f32x16& s, f32x16& dp) {
 #pragma unroll
-    for (int sb = 0; sb < 2; ++sb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        s[sb][i] = 0.0f;
-        dp[sb][i] = 0.0f;
-      }
-    // fragment (sb, t): 8 probabilities -> dS, packed for the dQ product
-    auto ds_frag = [&](int sb, int t) {
-      float e[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float pr = __builtin_amdgcn_exp2f(s[sb][8 * t + i] * c2 - lse2);
-        e[i] = pr * (dp[sb][8 * t + i] - delta);
-      }
-      return pack8(e);
-    };
-    auto dq_mfma = [&](int sb, int t, int nb, const bf16x8& f) {
-      dq[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(kn, tr_off[nb], sb * 32 + 16 * t), f, dq[nb], 0, 0, 0);
-    };
-    // block 0: scores and dP
+    for (int i = 0; i < 16; ++i) s[i] = 0.0f;
+    // dP starts from -delta (a lane is one query): the product then leaves dP - delta behind
+    dp = minus_delta;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nat_frag(kn, ln, 2 * c + kg), qf[c], s[0], 0, 0, 0);
-      dp[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nat_frag(vn, ln, 2 * c + kg), dof[c], dp[0], 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(kn + sb * 32 * ROWB + row_off[c]), qf[c], s, 0, 0, 0);
+      dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(kn + NAT + sb * 32 * ROWB + row_off[c]), dof[c], dp, 0, 0, 0);
     }
-    JG_FENCE();
-    // block 1 products with the vector work of block 0 behind them
-    bf16x8 f00, f01;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nat_frag(kn, 32 + ln, 2 * c + kg), qf[c], s[1], 0, 0, 0);
-      dp[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nat_frag(vn, 32 + ln, 2 * c + kg), dof[c], dp[1], 0, 0, 0);
-      if (c == 1) f00 = ds_frag(0, 0);
-      if (c == 3) f01 = ds_frag(0, 1);
-      JG_FENCE();
-    }
-    // dQ products of block 0 under the vector work of block 1
-    dq_mfma(0, 0, 0, f00);
-    dq_mfma(0, 0, 1, f00);
-    JG_FENCE();
-    const bf16x8 f10 = ds_frag(1, 0);
-    JG_FENCE();
-    dq_mfma(0, 1, 0, f01);
-    dq_mfma(0, 1, 1, f01);
-    JG_FENCE();
-    const bf16x8 f11 = ds_frag(1, 1);
-    JG_FENCE();
-    dq_mfma(1, 0, 0, f10);
-    dq_mfma(1, 0, 1, f10);
-    dq_mfma(1, 1, 0, f11);
-    dq_mfma(1, 1, 1, f11);
   };
-#undef JG_FENCE
+  auto ds_frag = [&](int t) {
+    float e[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float pr = __builtin_amdgcn_exp2f(s_cur[8 * t + i] * c2 - lse2);
+      e[i] = pr * dp_cur[8 * t + i];
+    }
+    return pack8(e);
+  };
+  auto add_to_dq = [&](const unsigned char* kn, int sb) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)
+        dq[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(kn, tr_off[nb], sb * 32 + 16 * t), ds_prev[t], dq[nb], 0, 0, 0);
+  };
+  // one step of the pipeline: A of (k_next, sb_next), B of the current block, C of (k_prev, sb_prev)
+  auto step = [&](const unsigned char* k_next, int sb_next, const unsigned char* k_prev, int sb_prev, bool ahead) {
+    f32x16 s_n, dp_n;
+    if (ahead) scores(k_next, sb_next, s_n, dp_n);
+    bf16x8 ds_now[2];
+    ds_now[0] = ds_frag(0);
+    ds_now[1] = ds_frag(1);
+    add_to_dq(k_prev, sb_prev);
+    if (ahead) {
+#define JG_SLOT(reads)                                               \
+  __builtin_amdgcn_sched_group_barrier(JG_GROUP_MFMA, 1, 0);          \
+  __builtin_amdgcn_sched_group_barrier(JG_GROUP_DS_READ, reads, 0);   \
+  __builtin_amdgcn_sched_group_barrier(JG_GROUP_VALU, 7, 0);
+      JG_SLOT(2) JG_SLOT(2) JG_SLOT(2) JG_SLOT(2) JG_SLOT(2) JG_SLOT(2) JG_SLOT(2) JG_SLOT(2)
+      JG_SLOT(0) JG_SLOT(0) JG_SLOT(0) JG_SLOT(0)
+#undef JG_SLOT
+      s_cur = s_n;
+      dp_cur = dp_n;
+    }
+    ds_prev[0] = ds_now[0];
+    ds_prev[1] = ds_now[1];
+  };
 
-  int buf = 0;
-  issue_loads(0, 0);
   tiles_landed();
   __syncthreads();
-  for (int t = 0; t < ntiles; ++t) {
-    const bool has_next = t + 1 < ntiles;
-    if (has_next) issue_loads(t + 1, buf ^ 1);
-    compute_tile(buf);
+  scores(lds, 0, s_cur, dp_cur);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    ds_prev[0][i] = (__bf16)0.0f;  // block -1 adds nothing (times the finite K of block 0)
+    ds_prev[1][i] = (__bf16)0.0f;
+  }
+  const unsigned char* k_back = lds;  // tile of the block before the current one
+  int sb_back = 0;
+  for (int t = 0; t + 1 < ntiles; ++t) {
+    if (t + 2 < ntiles) issue_loads(t + 2);
+    const unsigned char* kn = lds + (t & (NBUF - 1)) * DQ_BUF;
+    const unsigned char* kn1 = lds + ((t + 1) & (NBUF - 1)) * DQ_BUF;
+    step(kn, 1, k_back, sb_back, true);
+    step(kn1, 0, kn, 0, true);
+    k_back = kn;
+    sb_back = 1;
     tiles_landed();
     __syncthreads();
-    buf ^= 1;
   }
+  {
+    const unsigned char* kn = lds + ((ntiles - 1) & (NBUF - 1)) * DQ_BUF;
+    step(kn, 1, k_back, sb_back, true);
+    step(kn, 0, kn, 0, false);
+    add_to_dq(kn, 1);
+  }
+  __syncthreads();  // the hand-over below reuses the tile buffers
 
   // combine the two key halves, then write dQ (lane = query, 4 consecutive d per store)
   float* xo = reinterpret_cast<float*>(smem) + qb * (32 * 64);
@@ -329,17 +353,6 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
   const uint32_t lds_dma = lds_address(smem) + (uint32_t)(qs_u * (2 * DKV_HALF) + 16 * kb_u * ROWB);
   const int tr_off[2] = {tr_lane_offset(lane, 0), tr_lane_offset(lane, 1)};
 
-  bf16x8 kf[4], vf[4];
-  {
-    const uint16_t* krow = p.k + ki * D + 8 * kg;
-    const uint16_t* vrow = p.v + ki * D + 8 * kg;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      kf[c] = lds_frag(reinterpret_cast<const unsigned char*>(krow + 16 * c));
-      vf[c] = lds_frag(reinterpret_cast<const unsigned char*>(vrow + 16 * c));
-    }
-  }
-
   float st_reg = 0.0f;
   auto issue_loads = [&](int t, int buf) {
     const long long off = (long long)t * NAT;
@@ -356,9 +369,23 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
   };
   auto store_stats = [&](int buf) {
     unsigned char* base = lds + buf * DKV_HALF;
-    if (th < 2 * BT) reinterpret_cast<float*>(base + 2 * NAT)[th] = th < BT ? st_reg * LOG2E : st_reg;
+    if (th < 2 * BT) reinterpret_cast<float*>(base + 2 * NAT)[th] = th < BT ? st_reg * LOG2E : -st_reg;
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the transfers into this buffer have landed
   };
+
+  // the first tile is on its way while the wavefront fetches its own rows
+  issue_loads(0, 0);
+
+  bf16x8 kf[4], vf[4];
+  {
+    const uint16_t* krow = p.k + ki * D + 8 * kg;
+    const uint16_t* vrow = p.v + ki * D + 8 * kg;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      kf[c] = lds_frag(reinterpret_cast<const unsigned char*>(krow + 16 * c));
+      vf[c] = lds_frag(reinterpret_cast<const unsigned char*>(vrow + 16 * c));
+    }
+  }
 
   f32x16 dk[2], dv[2];
 #pragma unroll
@@ -373,15 +400,19 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
   auto compute_tile = [&](int buf) {
     const unsigned char* qn = lds + buf * DKV_HALF;
     const unsigned char* dn = qn + NAT;
-    const float* st = reinterpret_cast<const float*>(qn + 2 * NAT);  // lse2[64] then delta[64]
+    const float* st = reinterpret_cast<const float*>(qn + 2 * NAT);  // lse2[64] then -delta[64]
     bf16x8 pf[2][2], dsf[2][2];
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
       f32x16 s, dp;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        s[i] = 0.0f;
-        dp[i] = 0.0f;
+      for (int i = 0; i < 16; ++i) s[i] = 0.0f;
+      // dP starts from -delta of its queries (register i: query sb*32 + 8*(i/4) + 4*kg + i%4)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(st + BT + sb * 32 + 8 * j + 4 * kg);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dp[4 * j + e] = d4[e];
       }
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
@@ -396,12 +427,11 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
         for (int jj = 0; jj < 2; ++jj) {
           const int j = 2 * t + jj;
           const f32x4 l4 = *reinterpret_cast<const f32x4*>(st + sb * 32 + 8 * j + 4 * kg);
-          const f32x4 d4 = *reinterpret_cast<const f32x4*>(st + BT + sb * 32 + 8 * j + 4 * kg);
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const float pr = __builtin_amdgcn_exp2f(s[4 * j + e] * c2 - l4[e]);
             pe[4 * jj + e] = pr;
-            de[4 * jj + e] = pr * (dp[4 * j + e] - d4[e]);
+            de[4 * jj + e] = pr * dp[4 * j + e];
           }
         }
         pf[sb][t] = pack8(pe);
@@ -420,7 +450,6 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
   };
 
   int buf = 0;
-  issue_loads(0, 0);
   store_stats(0);
   // The K / V fragments came straight from memory: they are waited for here, once. Left
   // to the first MFMA that reads them, the wait would sit inside the loop, behind the
