@@ -89,6 +89,7 @@ struct FwdParams {
   int Din, Hin, Win, Dout, Hout, Wout;
   int pad_d, pad_h, pad_w;  // virtual zero padding of x
   int tiles_h, tiles_w;
+  int sw;               // tile order inside a plane: row-major inside bands of sw tile columns, band after band
   int total_tiles;      // N * Dout * tiles_h * tiles_w
   int nc16;             // KD * Cp / 16
   int wc16;             // 16-channel steps whose weights sit in LDS at a time (a group)
@@ -254,6 +255,9 @@ __device__ inline void store_bf16_lo(const void* base, uint32_t lane_off, uint32
 __device__ inline void store_bf16_hi(const void* base, uint32_t lane_off, uint32_t pair) {
   asm volatile("global_store_short_d16_hi %0, %1, %2" : : "v"(lane_off), "v"(pair), "s"(base) : "memory");
 }
+__device__ inline void store_16_bytes(const void* base, uint32_t lane_off, u32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, %2" : : "v"(lane_off), "v"(v), "s"(base) : "memory");
+}
 __device__ inline void store_f32(const void* base, uint32_t lane_off, float v) {
   asm volatile("global_store_dword %0, %1, %2" : : "v"(lane_off), "v"(v), "s"(base) : "memory");
 }
@@ -336,10 +340,15 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
   };
   auto coord = [&](int tile) {
     TileCoord c;
-    c.tw = tile % p.tiles_w;
-    int tq = tile / p.tiles_w;
-    c.th = tq % p.tiles_h;
-    tq /= p.tiles_h;
+    const int per_plane = p.tiles_h * p.tiles_w;
+    int tq = tile / per_plane;
+    int j = tile - tq * per_plane;
+    const int band = p.tiles_h * p.sw;          // tiles in a full band
+    const int b = j / band;                     // band number; the last one may be narrower
+    j -= b * band;
+    const int width = min(p.sw, p.tiles_w - b * p.sw);
+    c.th = j / width;
+    c.tw = b * p.sw + (j - c.th * width);
     c.od = tq % p.Dout;
     c.n = tq / p.Dout;
     return c;
@@ -430,16 +439,33 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
         stg[c][0] = v.x; stg[c][1] = v.y; stg[c][2] = v.z; stg[c][3] = v.w;
       }
     } else if (EVEN) {
+      // A window that sticks out of the tensor (the border tiles of a padded problem: one tile in
+      // seven of configuration 2's input gradient). Most of its tasks still lie wholly inside and
+      // keep their 16-byte loads, the ones wholly outside load nothing; only the tasks that
+      // straddle an edge go dword by dword.
       const int ih = ih0 + t_row, iw = iw0 + t_col;
       const bool row_ok = depth_ok && (ih >= 0) && (ih < p.Hin);
-      bool ok[4];
+      if (row_ok && iw >= 0 && iw + 8 <= p.Win && cvalid >= 8) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) ok[j] = row_ok && iw + 2 * j >= 0 && iw + 2 * j + 2 <= p.Win;
+        for (int c = 0; c < 8; ++c) {
+          const u32x4_a4 v = *reinterpret_cast<const u32x4_a4*>(a + (size_t)c * chan_b);
+          stg[c][0] = v.x; stg[c][1] = v.y; stg[c][2] = v.z; stg[c][3] = v.w;
+        }
+      } else if (!row_ok || iw + 8 <= 0 || iw >= p.Win) {
 #pragma unroll
-      for (int c = 0; c < 8; ++c)
+        for (int c = 0; c < 8; ++c) {
+          stg[c][0] = 0u; stg[c][1] = 0u; stg[c][2] = 0u; stg[c][3] = 0u;
+        }
+      } else {
+        bool ok[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          stg[c][j] = (ok[j] && c < cvalid) ? *reinterpret_cast<const uint32_t*>(a + (size_t)c * chan_b + 4 * j) : 0u;
+        for (int j = 0; j < 4; ++j) ok[j] = iw + 2 * j >= 0 && iw + 2 * j + 2 <= p.Win;
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            stg[c][j] = (ok[j] && c < cvalid) ? *reinterpret_cast<const uint32_t*>(a + (size_t)c * chan_b + 4 * j) : 0u;
+      }
     } else {
       const int ih = ih0 + t_row, iw = iw0 + t_col;
       const bool rows_ok = depth_ok && (ih >= 0) && (ih < p.Hin);
@@ -543,10 +569,63 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
   const size_t ochan = plane_o * p.Dout;  // elements between produced channels
   // RAGGED: the last tile of produced channels when M is not a multiple of MT (its weight
   // rows past M are zero padding); a lane then stores only the channels that exist.
-  auto epilogue_rows = [&](int tile, auto ragged) {
+  // Rows of a wavefront through LDS: the accumulator holds one pixel and 32 channels per lane,
+  // memory wants runs of pixels. A row of the wavefront (32 pixels x MT channels) is written to
+  // LDS as 16-bit values, 64 bytes per channel, and read back as 16-byte pieces that go out as
+  // 16-byte stores: 4 store instructions per row instead of 32 (MT = 64). The two channels a
+  // lane pair (kg = 0, 1) writes at once, m and m + 4, sit in neighbouring 64-byte rows of the
+  // scratch, so that the halves of the wavefront use different banks. `scratch`: 64 * MT bytes of
+  // LDS of this wavefront. Needs 16-byte aligned row segments in y (checked by the caller).
+  // `ytile` is wave-uniform (a scalar base), `row_off` the byte offset of the wavefront's row segment from it.
+  // `pair(cb, i)`: the 16-bit values of accumulator registers i (low half) and i + 1 of block cb.
+  auto row_through_lds = [&](unsigned char* scratch, auto pair, char* ytile, uint32_t row_off, size_t chan_bytes) {
+    // lane's part of the write address: pixel ln of LDS row kg
+    unsigned char* wr = scratch + kg * 64 + ln * 2;
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) {
+        const uint32_t h2 = pair(cb, i);
+        // channel cb*32 + 8*(i/4) + i%4 (+ 4 kg): LDS row (that & ~7) + 2*(i%4) (+ kg); i + 1: two rows on
+        const int row = cb * 32 + 8 * (i >> 2) + 2 * (i & 3);
+        *reinterpret_cast<uint16_t*>(wr + row * 64) = (uint16_t)(h2 & 0xffffu);
+        *reinterpret_cast<uint16_t*>(wr + (row + 2) * 64) = (uint16_t)(h2 >> 16);
+      }
+    // piece g = 64 q + lane: LDS row g / 4 = 16 q + lane / 4, pixels 8 (lane % 4) ..; its channel is
+    // 16 q + (lane/4 & 8) + (lane/4 >> 1 & 3) + 4 (lane/4 & 1)
+    const int l4 = lane >> 2;
+    const int m_lane = (l4 & 8) + ((l4 >> 1) & 3) + ((l4 & 1) << 2);
+    const uint32_t voff = (uint32_t)(m_lane * chan_bytes) + 16u * (lane & 3) + row_off;
+#pragma unroll
+    for (int q = 0; q < MT / 16; ++q) {
+      const u32x4 piece = *reinterpret_cast<const u32x4*>(scratch + (q * 64 + lane) * 16);
+      store_16_bytes(ytile + (size_t)q * 16 * chan_bytes, voff, piece);
+    }
+  };
+
+  auto epilogue_rows = [&](int tile, auto ragged, int free_buf) {
     constexpr bool RAGGED = decltype(ragged)::value;
     const TileCoord tc = coord(tile);
     const int ow = tc.tw * TW + wcol0 + ln;
+    if (!RAGGED && p.out_kind != 1 && (p.Wout & 7) == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 &&
+        tc.tw * TW + wcol0 + 32 <= p.Wout) {  // wave-uniform
+      unsigned char* scratch = reinterpret_cast<unsigned char*>(lds_in + free_buf * STAGE_SLOTS) + wave * (STAGE_BYTES / WAVES);
+      char* ytile = reinterpret_cast<char*>(p.y) +
+                    2 * (((size_t)tc.n * p.M + (size_t)mt * MT) * (plane_o * p.Dout) + (size_t)tc.od * plane_o +
+                         (size_t)(tc.tw * TW));
+#pragma unroll
+      for (int r = 0; r < WROWS; ++r) {
+        const int oh = tc.th * TH + wrow0 + r;
+        auto pair = [&](int cb, int i) {
+          f32x2 v2 = {acc[cb][r][i], acc[cb][r][i + 1]};
+          return p.out_kind == 2 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, f16x2))
+                                 : __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
+        };
+        if (oh < p.Hout)
+          row_through_lds(scratch, pair, ytile, (uint32_t)(2 * ((size_t)oh * p.Wout + wcol0)), 2 * plane_o * p.Dout);
+      }
+      return;
+    }
     char* ybase = reinterpret_cast<char*>(p.y) +
                   2 * (((size_t)tc.n * p.M + (size_t)mt * MT) * ochan + (size_t)tc.od * plane_o);
     const int m_left = p.M - mt * MT - 4 * kg;  // channels from this lane's first one to the end
@@ -588,9 +667,9 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
       }
     }
   };
-  auto epilogue = [&](int tile) {
-    if ((mt + 1) * MT <= p.M) epilogue_rows(tile, std::false_type{});
-    else epilogue_rows(tile, std::true_type{});
+  auto epilogue = [&](int tile, int free_buf) {
+    if ((mt + 1) * MT <= p.M) epilogue_rows(tile, std::false_type{}, free_buf);
+    else epilogue_rows(tile, std::true_type{}, free_buf);
   };
 
   // Fold-mode epilogue: a produced cell goes to the unpadded tile when it lies inside
@@ -723,8 +802,15 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
       __syncthreads();
       buf ^= 1;
     }
-    if (FOLD) epilogue_fold(tile_of(ti));
-    else epilogue(tile_of(ti));
+    if (FOLD) {
+      epilogue_fold(tile_of(ti));
+    } else {
+      // the stage buffer the last stage was computed from is free until the next stage is
+      // stored into it: the epilogue stages its rows there, and the barrier keeps a wavefront
+      // that is already in the next tile from storing over them
+      epilogue(tile_of(ti), buf ^ 1);
+      __syncthreads();
+    }
   }
 }
 
@@ -875,6 +961,7 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   p.pad_d = L.pad_d; p.pad_h = L.pad_h; p.pad_w = L.pad_w;
   p.tiles_h = (L.Hout + TH - 1) / TH;
   p.tiles_w = (L.Wout + TW - 1) / TW;
+  p.sw = p.tiles_w;
   const long long tiles = (long long)L.N * L.Dout * p.tiles_h * p.tiles_w;
   JG_REQUIRE(tiles < (1ll << 30), "%s: too many tiles", who);
   p.total_tiles = (int)tiles;
