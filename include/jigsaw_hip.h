@@ -473,6 +473,26 @@ int jg_attn_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q,
                 const float* bias, int64_t bias_period, float* dbias, int dtype,
                 void* workspace, size_t workspace_bytes, void* stream);
 
+/* Windowed attention of a Swin block on the token grid itself (examples/swin.py:129-170:
+ * F.scaled_dot_product_attention over (B, nW, heads, 64, 32) windows with attn_mask = the
+ * relative-position bias, index of examples/swin.py:99-104, plus the shift mask of 107-126).
+ * q, k, v, out: (images, heads, gh * gw, 32) bf16, tokens in row-major grid order; the kernel
+ * addresses the 8 x 8 windows in place, so no window partition is materialised. table: (225, heads)
+ * fp32, the learned bias by relative position. side: (windows of one image, 64) bytes or NULL, a
+ * code per token; tokens of one window with different codes do not attend each other.
+ * lse: (images * windows * heads, 64) fp32, for the backward. */
+int jg_attn_swin_fwd(void* out, float* lse, const void* q, const void* k, const void* v, const float* table,
+                     const uint8_t* side, int64_t images, int64_t heads, int64_t gh, int64_t gw, int64_t d,
+                     float scale, int dtype, void* stream);
+
+/* Gradients of jg_attn_swin_fwd (autograd of the same call in the reference). dtable: (225, heads)
+ * fp32 or NULL; when wanted, workspace must hold jg_attn_swin_bwd_workspace_bytes bytes. */
+size_t jg_attn_swin_bwd_workspace_bytes(int64_t images, int64_t heads, int64_t gh, int64_t gw);
+int jg_attn_swin_bwd(void* dq, void* dk, void* dv, float* dtable, const void* dout, const void* q, const void* k,
+                     const void* v, const void* out, const float* lse, const float* table, const uint8_t* side,
+                     int64_t images, int64_t heads, int64_t gh, int64_t gw, int64_t d, float scale, int dtype,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -195,6 +195,17 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
          c_int64, c_int64, c_float, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_size_t, c_void_p],
     ),
+    "jg_attn_swin_fwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
+         c_int64, c_float, c_int, c_void_p],
+    ),
+    "jg_attn_swin_bwd_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
+    "jg_attn_swin_bwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_void_p, c_size_t, c_void_p],
+    ),
     "jg_lse_merge": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int,

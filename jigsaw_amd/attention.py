@@ -391,6 +391,77 @@ def window_attention(q, k, v, bias=None):
     return _BiasedAttention.apply(q, k, v, bias)
 
 
+SWIN_WINDOW, SWIN_HEAD_SIZE = 8, 32
+
+
+def swin_grid_supported(q: torch.Tensor, grid: tuple, window: int) -> bool:
+    """Whether :func:`swin_grid_attention` has a kernel for these tensors: bf16, head size 32,
+    8 x 8 windows tiling the token grid."""
+    return (
+        q.dtype == torch.bfloat16 and q.shape[-1] == SWIN_HEAD_SIZE and window == SWIN_WINDOW
+        and grid[0] % window == 0 and grid[1] % window == 0 and grid[0] * grid[1] == q.shape[-2]
+    )
+
+
+class _SwinGridAttention(torch.autograd.Function):
+    """Attention inside the 8 x 8 windows of a token grid, ``q, k, v`` of shape (B, heads, gh * gw, 32)
+    with the tokens in grid order; relative-position bias from ``table`` (225, heads) and the shift
+    mask from the per-token codes ``side`` (windows, 64) are formed inside the kernel
+    (examples/swin.py:99-170). Differentiable in q, k, v and table."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, table, side, grid):  # noqa: D102
+        lib = _lib.load()
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        table = table.detach().float().contiguous()
+        images, heads, tokens, d = q.shape
+        gh, gw = grid
+        scale = d ** -0.5
+        out = torch.empty_like(q)
+        lse = torch.empty(images * heads * tokens, dtype=torch.float32, device=q.device)
+        rc = lib.jg_attn_swin_fwd(
+            _lib.ptr(out), _lib.ptr(lse), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(table), _lib.ptr(side),
+            images, heads, gh, gw, d, float(scale), _lib.dtype_code(q.dtype), _lib.stream_ptr(q.device),
+        )
+        _lib.check(rc, "jg_attn_swin_fwd")
+        ctx.save_for_backward(q, k, v, table, side, out, lse)
+        ctx.grid, ctx.scale = (gh, gw), scale
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):  # noqa: D102
+        lib = _lib.load()
+        q, k, v, table, side, out, lse = ctx.saved_tensors
+        images, heads, tokens, d = q.shape
+        gh, gw = ctx.grid
+        grad_out = grad_out.contiguous()
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dtable = ws = None
+        ws_bytes = 0
+        if ctx.needs_input_grad[3]:
+            dtable = torch.empty_like(table)
+            ws_bytes = lib.jg_attn_swin_bwd_workspace_bytes(images, heads, gh, gw)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+        rc = lib.jg_attn_swin_bwd(
+            _lib.ptr(dq), _lib.ptr(dk), _lib.ptr(dv), _lib.ptr(dtable), _lib.ptr(grad_out), _lib.ptr(q), _lib.ptr(k),
+            _lib.ptr(v), _lib.ptr(out), _lib.ptr(lse), _lib.ptr(table), _lib.ptr(side), images, heads, gh, gw, d,
+            float(ctx.scale), _lib.dtype_code(q.dtype), _lib.ptr(ws), ws_bytes, _lib.stream_ptr(q.device),
+        )
+        _lib.check(rc, "jg_attn_swin_bwd")
+        return dq, dk, dv, dtable, None, None
+
+
+def swin_grid_attention(q, k, v, table, side, grid):
+    """See :class:`_SwinGridAttention`. ``side`` is a uint8 tensor (windows, 64) or ``None``."""
+    if not swin_grid_supported(q, grid, SWIN_WINDOW):
+        raise NotImplementedError("swin_grid_attention: bf16, head size 32 and 8 x 8 windows only")
+    if side is not None and (side.dtype != torch.uint8 or side.numel() != q.shape[-2]):
+        raise ValueError("side must be a uint8 code per token, (windows, 64)")
+    if table.shape != (225, q.shape[1]):
+        raise ValueError(f"table must be (225, heads = {q.shape[1]}), got {tuple(table.shape)}")
+    return _SwinGridAttention.apply(q, k, v, table, side, grid)
+
+
 __all__ = [
     "attend_step_",
     "backward",
@@ -400,5 +471,7 @@ __all__ = [
     "fused_online_softmax_merge_",
     "ring_backward",
     "ring_forward",
+    "swin_grid_attention",
+    "swin_grid_supported",
     "window_attention",
 ]

@@ -19,7 +19,7 @@ from typing import Any
 import torch
 import torch.nn as nn
 
-from .attention import window_attention
+from .attention import swin_grid_attention, swin_grid_supported, window_attention
 from .conv import TileGroup
 from .layernorm import plain_layer_norm
 from .projection import heads_projection, linear, qkv_projection
@@ -108,12 +108,22 @@ class WindowAttention(nn.Module):
         self.register_buffer("onehot", onehot, persistent=False)
         if shift:
             self.register_buffer("mask", shift_mask(*tile, window, shift, groups).to(device), persistent=False)
+            side = border_sides(*tile, window, shift, groups).to(torch.uint8)
+            self.register_buffer("side", side.contiguous().to(device), persistent=False)
         else:
-            self.mask = None
+            self.mask = self.side = None
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         b, h, w, c = x.shape
-        x = windows(x, self.window).to(_compute_dtype(x))
+        dt = _compute_dtype(x)
+        if dt == torch.bfloat16 and c // self.heads == 32 and self.window == 8 and h % 8 == 0 and w % 8 == 0:
+            # the kernel addresses the windows on the token grid and forms bias and mask itself:
+            # no window partition, no (nW, heads, N, N) bias tensor
+            q, k, v = qkv_projection(x.to(dt).view(b, h * w, c), self.qkv.weight, self.qkv.bias, self.heads).unbind(0)
+            assert swin_grid_supported(q, (h, w), self.window)
+            out = swin_grid_attention(q, k, v, self.bias_table, self.side, (h, w))
+            return heads_projection(out, self.proj.weight, self.proj.bias).view(b, h, w, c)
+        x = windows(x, self.window).to(dt)
         n = x.shape[2]
         # the projections write / read the (B, nW, heads, N, d) head layout themselves
         q, k, v = qkv_projection(x, self.qkv.weight, self.qkv.bias, self.heads).unbind(0)
