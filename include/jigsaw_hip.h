@@ -306,6 +306,19 @@ int jg_proj_nt(void* out, const void* a, const void* w, const void* bias, int dt
                int64_t rows, int n_out, int k_in, int a_heads, int out_heads,
                int B, int H, int S, int D, void* stream);
 
+/* jg_proj_nt on row-major bf16 operands with an elementwise step of the two-layer MLP of a
+ * transformer block folded into the way out (examples/swin.py:190-194: Linear, GELU, Linear and
+ * the residual sum around them; the values are the bf16-rounded results a separate pass over
+ * the stored tensor would see, arithmetic in fp32). aux has the shape of out.
+ *   JG_EPI_GELU  (1): out = y, aux = gelu(y) (erf form); aux is written
+ *   JG_EPI_DGELU (2): out = y * gelu'(aux); aux is read (the saved pre-activation)
+ *   JG_EPI_ADD   (3): out = y + aux; aux is read (the residual) */
+#define JG_EPI_GELU 1
+#define JG_EPI_DGELU 2
+#define JG_EPI_ADD 3
+int jg_proj_nt_fused(void* out, void* aux, int epilogue, const void* a, const void* w, const void* bias, int dtype,
+                     int64_t rows, int n_out, int k_in, void* stream);
+
 /* gw[n][c] = sum_r g(r, n) * x(r, c)  (n, c) row-major, and gb[n] = sum_r g(r, n)
  * (gb may be NULL): weight and bias gradient of a projection (torch's
  * Linear backward; g = grad of the projection's output, x = its input).

@@ -404,62 +404,74 @@ def swin_grid_supported(q: torch.Tensor, grid: tuple, window: int) -> bool:
 
 
 class _SwinGridAttention(torch.autograd.Function):
-    """Attention inside the 8 x 8 windows of a token grid, ``q, k, v`` of shape (B, heads, gh * gw, 32)
-    with the tokens in grid order; relative-position bias from ``table`` (225, heads) and the shift
-    mask from the per-token codes ``side`` (windows, 64) are formed inside the kernel
-    (examples/swin.py:99-170). Differentiable in q, k, v and table."""
+    """Attention inside the 8 x 8 windows of a token grid. ``qkv`` is (3, B, heads, gh * gw, 32), the
+    tokens in grid order, as the qkv projection writes it; relative-position bias from ``table``
+    (225, heads) and the shift mask from the per-token codes ``side`` (windows, 64) are formed inside
+    the kernel (examples/swin.py:99-170). Differentiable in qkv and table; the gradient comes back
+    as one (3, ...) tensor, so that nothing is stacked or split on the way to the projection."""
 
     @staticmethod
-    def forward(ctx, q, k, v, table, side, grid):  # noqa: D102
+    def forward(ctx, qkv, table, side, grid):  # noqa: D102
         lib = _lib.load()
-        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        qkv = qkv.contiguous()
         table = table.detach().float().contiguous()
-        images, heads, tokens, d = q.shape
+        _, images, heads, tokens, d = qkv.shape
         gh, gw = grid
         scale = d ** -0.5
-        out = torch.empty_like(q)
-        lse = torch.empty(images * heads * tokens, dtype=torch.float32, device=q.device)
+        out = torch.empty_like(qkv[0])
+        lse = torch.empty(images * heads * tokens, dtype=torch.float32, device=qkv.device)
         rc = lib.jg_attn_swin_fwd(
-            _lib.ptr(out), _lib.ptr(lse), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(table), _lib.ptr(side),
-            images, heads, gh, gw, d, float(scale), _lib.dtype_code(q.dtype), _lib.stream_ptr(q.device),
+            _lib.ptr(out), _lib.ptr(lse), _lib.ptr(qkv[0]), _lib.ptr(qkv[1]), _lib.ptr(qkv[2]), _lib.ptr(table),
+            _lib.ptr(side), images, heads, gh, gw, d, float(scale), _lib.dtype_code(qkv.dtype),
+            _lib.stream_ptr(qkv.device),
         )
         _lib.check(rc, "jg_attn_swin_fwd")
-        ctx.save_for_backward(q, k, v, table, side, out, lse)
+        ctx.save_for_backward(qkv, table, side, out, lse)
         ctx.grid, ctx.scale = (gh, gw), scale
         return out
 
     @staticmethod
     def backward(ctx, grad_out):  # noqa: D102
         lib = _lib.load()
-        q, k, v, table, side, out, lse = ctx.saved_tensors
-        images, heads, tokens, d = q.shape
+        qkv, table, side, out, lse = ctx.saved_tensors
+        _, images, heads, tokens, d = qkv.shape
         gh, gw = ctx.grid
         grad_out = grad_out.contiguous()
-        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dqkv = torch.empty_like(qkv)
         dtable = ws = None
         ws_bytes = 0
-        if ctx.needs_input_grad[3]:
+        if ctx.needs_input_grad[1]:
             dtable = torch.empty_like(table)
             ws_bytes = lib.jg_attn_swin_bwd_workspace_bytes(images, heads, gh, gw)
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=qkv.device)
         rc = lib.jg_attn_swin_bwd(
-            _lib.ptr(dq), _lib.ptr(dk), _lib.ptr(dv), _lib.ptr(dtable), _lib.ptr(grad_out), _lib.ptr(q), _lib.ptr(k),
-            _lib.ptr(v), _lib.ptr(out), _lib.ptr(lse), _lib.ptr(table), _lib.ptr(side), images, heads, gh, gw, d,
-            float(ctx.scale), _lib.dtype_code(q.dtype), _lib.ptr(ws), ws_bytes, _lib.stream_ptr(q.device),
+            _lib.ptr(dqkv[0]), _lib.ptr(dqkv[1]), _lib.ptr(dqkv[2]), _lib.ptr(dtable), _lib.ptr(grad_out),
+            _lib.ptr(qkv[0]), _lib.ptr(qkv[1]), _lib.ptr(qkv[2]), _lib.ptr(out), _lib.ptr(lse), _lib.ptr(table),
+            _lib.ptr(side), images, heads, gh, gw, d, float(ctx.scale), _lib.dtype_code(qkv.dtype), _lib.ptr(ws),
+            ws_bytes, _lib.stream_ptr(qkv.device),
         )
         _lib.check(rc, "jg_attn_swin_bwd")
-        return dq, dk, dv, dtable, None, None
+        return dqkv, dtable, None, None
+
+
+def swin_grid_attention_packed(qkv, table, side, grid):
+    """:func:`swin_grid_attention` on the (3, B, heads, tokens, 32) tensor of the qkv projection."""
+    if qkv.dim() != 5 or qkv.shape[0] != 3 or not swin_grid_supported(qkv[0], grid, SWIN_WINDOW):
+        raise NotImplementedError("swin_grid_attention: (3, B, heads, tokens, 32) bf16 and 8 x 8 windows only")
+    if side is not None and (side.dtype != torch.uint8 or side.numel() != qkv.shape[-2]):
+        raise ValueError("side must be a uint8 code per token, (windows, 64)")
+    if table.shape != (225, qkv.shape[2]):
+        raise ValueError(f"table must be (225, heads = {qkv.shape[2]}), got {tuple(table.shape)}")
+    return _SwinGridAttention.apply(qkv, table, side, grid)
 
 
 def swin_grid_attention(q, k, v, table, side, grid):
-    """See :class:`_SwinGridAttention`. ``side`` is a uint8 tensor (windows, 64) or ``None``."""
+    """Attention inside the 8 x 8 windows of a token grid for separate ``q, k, v`` of shape
+    (B, heads, gh * gw, 32) (stacked here; see :func:`swin_grid_attention_packed`). ``side`` is a uint8
+    tensor (windows, 64) or ``None``."""
     if not swin_grid_supported(q, grid, SWIN_WINDOW):
         raise NotImplementedError("swin_grid_attention: bf16, head size 32 and 8 x 8 windows only")
-    if side is not None and (side.dtype != torch.uint8 or side.numel() != q.shape[-2]):
-        raise ValueError("side must be a uint8 code per token, (windows, 64)")
-    if table.shape != (225, q.shape[1]):
-        raise ValueError(f"table must be (225, heads = {q.shape[1]}), got {tuple(table.shape)}")
-    return _SwinGridAttention.apply(q, k, v, table, side, grid)
+    return swin_grid_attention_packed(torch.stack((q, k, v)), table, side, grid)
 
 
 __all__ = [
@@ -472,6 +484,7 @@ __all__ = [
     "ring_backward",
     "ring_forward",
     "swin_grid_attention",
+    "swin_grid_attention_packed",
     "swin_grid_supported",
     "window_attention",
 ]

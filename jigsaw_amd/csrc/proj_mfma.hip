@@ -90,7 +90,35 @@ struct NtParams {
   long long rows;
   int N, K;
   int tiles_n;
+  // What happens to a result on its way out (the values are the bf16-rounded acc + bias, as a
+  // separate elementwise pass over the stored tensor would see them; arithmetic in fp32):
+  //   EPI_NONE  out = y
+  //   EPI_GELU  out = y, aux = gelu(y)                (aux is written)
+  //   EPI_DGELU out = y * gelu'(aux)                  (aux is read: the saved pre-activation)
+  //   EPI_ADD   out = y + aux                         (aux is read: the residual)
+  // aux has the layout of out.
+  int epi;
+  uint16_t* aux;
 };
+constexpr int EPI_NONE = 0, EPI_GELU = 1, EPI_DGELU = 2, EPI_ADD = 3;
+
+// exact GELU (erf form, torch.nn.GELU's default) and its derivative
+__device__ __forceinline__ float gelu_f(float h) { return 0.5f * h * (1.0f + erff(h * 0.70710678118654752f)); }
+__device__ __forceinline__ float dgelu_f(float h) {
+  return 0.5f * (1.0f + erff(h * 0.70710678118654752f)) + h * 0.3989422804014327f * __expf(-0.5f * h * h);
+}
+// op on 8 bf16 values packed in 16 bytes (second operand optional)
+template <typename F>
+__device__ __forceinline__ u32x4 map8(u32x4 y, u32x4 r, F f) {
+  uint32_t yy[4] = {y.x, y.y, y.z, y.w}, rr[4] = {r.x, r.y, r.z, r.w}, oo[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const f32x2 v = {f(__uint_as_float(yy[i] << 16), __uint_as_float(rr[i] << 16)),
+                     f(__uint_as_float(yy[i] & 0xffff0000u), __uint_as_float(rr[i] & 0xffff0000u))};
+    oo[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+  }
+  return u32x4{oo[0], oo[1], oo[2], oo[3]};
+}
 
 // Shape of a workgroup: WM x WN wavefronts, each with IM x JN blocks of 32 tokens x 32 features.
 template <int IM, int JN, int WM, int WN>
@@ -246,9 +274,18 @@ __global__ __launch_bounds__(64 * WM * WN) void proj_nt_kernel(NtParams p) {
 #pragma unroll 4
     for (int q = 0; q < TM / RPP; ++q) {
       const long long r = m0 + trow + RPP * q;
-      if (r < p.rows && n < p.N)
-        *reinterpret_cast<u32x4*>(p.out + rwk.part(p.om) + fo) =
-            *reinterpret_cast<const u32x4*>(tile + (trow + RPP * q) * SH::OUT_PITCH + fc * 8);
+      if (r < p.rows && n < p.N) {
+        const long long at = rwk.part(p.om) + fo;
+        u32x4 y = *reinterpret_cast<const u32x4*>(tile + (trow + RPP * q) * SH::OUT_PITCH + fc * 8);
+        if (p.epi == EPI_GELU) {
+          *reinterpret_cast<u32x4*>(p.aux + at) = map8(y, y, [](float h, float) { return gelu_f(h); });
+        } else if (p.epi == EPI_DGELU) {
+          y = map8(y, *reinterpret_cast<const u32x4*>(p.aux + at), [](float g, float h) { return g * dgelu_f(h); });
+        } else if (p.epi == EPI_ADD) {
+          y = map8(y, *reinterpret_cast<const u32x4*>(p.aux + at), [](float a, float b) { return a + b; });
+        }
+        *reinterpret_cast<u32x4*>(p.out + at) = y;
+      }
       rwk.advance(p.om, RPP);
     }
   }
@@ -704,9 +741,9 @@ int launch_generic(const GenParams& gp, int dtype, hipStream_t s, const char* wh
 
 extern "C" {
 
-int jg_proj_nt(void* out, const void* a, const void* w, const void* bias, int dtype, int64_t rows, int n_out,
-               int k_in, int a_heads, int out_heads, int B, int H, int S, int D, void* stream) {
-  const char* who = "jg_proj_nt";
+static int proj_nt_common(const char* who, void* out, void* aux, int epi, const void* a, const void* w, const void* bias,
+                          int dtype, int64_t rows, int n_out, int k_in, int a_heads, int out_heads, int B, int H, int S,
+                          int D, void* stream) {
   JG_REQUIRE(out && a && w, "%s: null pointer", who);
   JG_REQUIRE(jg::dtype_size(dtype) != 0, "%s: unknown dtype %d", who, dtype);
   JG_REQUIRE(rows >= 0 && n_out > 0 && k_in > 0, "%s: bad sizes rows=%lld n_out=%d k_in=%d", who, (long long)rows, n_out,
@@ -722,6 +759,8 @@ int jg_proj_nt(void* out, const void* a, const void* w, const void* bias, int dt
                     aligned16(w) && aligned16(out) && rows < (1ll << 31) - 256 &&
                     (unsigned long long)rows * k_in < (1ull << 31) && (unsigned long long)n_out * k_in < (1ull << 31);
   if (!fast) {
+    if (epi != EPI_NONE)
+      JG_FAIL(JG_ERR_UNSUPPORTED, "%s: the fused epilogues are built for bf16 operands on 16-byte aligned rows", who);
     GenParams gp;
     gp.p = a; gp.q = w; gp.bias = bias; gp.out = out;
     gp.pm = am; gp.qm = am; gp.om = om;
@@ -730,6 +769,8 @@ int jg_proj_nt(void* out, const void* a, const void* w, const void* bias, int dt
     return launch_generic<false>(gp, dtype, s, who);
   }
   NtParams p;
+  p.epi = epi;
+  p.aux = static_cast<uint16_t*>(aux);
   p.a = static_cast<const uint16_t*>(a);
   p.w = static_cast<const uint16_t*>(w);
   p.bias = static_cast<const uint16_t*>(bias);
@@ -742,6 +783,21 @@ int jg_proj_nt(void* out, const void* a, const void* w, const void* bias, int dt
   const int waste = jg::cdiv(n_out, 256) * 256 - n_out;
   if (big_tiles >= 256 && waste < 128) return launch_nt<4, 2, 2, 4>(p, s, who);
   return launch_nt<2, 2, 2, 2>(p, s, who);
+}
+
+int jg_proj_nt(void* out, const void* a, const void* w, const void* bias, int dtype, int64_t rows, int n_out,
+               int k_in, int a_heads, int out_heads, int B, int H, int S, int D, void* stream) {
+  return proj_nt_common("jg_proj_nt", out, nullptr, EPI_NONE, a, w, bias, dtype, rows, n_out, k_in, a_heads, out_heads,
+                        B, H, S, D, stream);
+}
+
+int jg_proj_nt_fused(void* out, void* aux, int epilogue, const void* a, const void* w, const void* bias, int dtype,
+                     int64_t rows, int n_out, int k_in, void* stream) {
+  const char* who = "jg_proj_nt_fused";
+  JG_REQUIRE(epilogue == EPI_GELU || epilogue == EPI_DGELU || epilogue == EPI_ADD, "%s: unknown epilogue %d", who,
+             epilogue);
+  JG_REQUIRE(aux != nullptr && aligned16(aux), "%s: aux must be a 16-byte aligned tensor of the shape of out", who);
+  return proj_nt_common(who, out, aux, epilogue, a, w, bias, dtype, rows, n_out, k_in, 0, 0, 1, 1, 1, 1, stream);
 }
 
 size_t jg_proj_tn_workspace(int64_t rows, int n, int c) {

@@ -243,6 +243,88 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
     return _Linear.apply(x, weight, bias)
 
 
+EPI_GELU, EPI_DGELU, EPI_ADD = 1, 2, 3
+
+
+def _nt_fused(out, aux, epilogue, a, w, bias, rows, n_out, k_in) -> None:
+    rc = _lib.load().jg_proj_nt_fused(_lib.ptr(out), _lib.ptr(aux), epilogue, _lib.ptr(a), _lib.ptr(w), _lib.ptr(bias),
+                                      _lib.dtype_code(a.dtype), rows, n_out, k_in, _lib.stream_ptr(a.device))
+    _lib.check(rc, "jg_proj_nt_fused")
+
+
+def mlp_fusable(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, residual: torch.Tensor | None) -> bool:
+    """Whether :func:`gelu_mlp` runs on the fused epilogues: bf16 tokens, feature counts that are
+    multiples of 8 (16-byte rows), a bf16 residual of the output's shape."""
+    ok = x.dtype == torch.bfloat16 and x.numel() > 0 and all(n % 8 == 0 for n in (*w1.shape, *w2.shape))
+    return ok and (residual is None or (residual.dtype == torch.bfloat16 and residual.shape[:-1] == x.shape[:-1]))
+
+
+class _GeluMlp(torch.autograd.Function):
+    """``residual + F.linear(F.gelu(F.linear(x, w1, b1)), w2, b2)`` (examples/swin.py:190-194 with the
+    residual sum of 206-209) as four GEMM launches forward and backward apart from the weight
+    gradients: GELU leaves the first GEMM beside the pre-activation, the residual is added on the way
+    out of the second, and in the backward the GELU derivative multiplies the input gradient of the
+    second layer on its way out."""
+
+    @staticmethod
+    def forward(ctx, x, w1, b1, w2, b2, residual):  # noqa: D102
+        _lib.require_gpu(x, w1, b1, w2, b2, residual)
+        hid, k = w1.shape
+        n_out = w2.shape[0]
+        xc = x.contiguous()
+        rows = xc.numel() // k
+        dt = x.dtype
+        w1c, b1c, w2c, b2c = (_cast_cached(t, dt) for t in (w1, b1, w2, b2))
+        pre = torch.empty((*x.shape[:-1], hid), dtype=dt, device=x.device)
+        act = torch.empty_like(pre)
+        _nt_fused(pre, act, EPI_GELU, xc, w1c, b1c, rows, hid, k)
+        out = torch.empty((*x.shape[:-1], n_out), dtype=dt, device=x.device)
+        if residual is None:
+            _nt(out, act, w2c, b2c, rows, n_out, hid, False, False, (1, 1, 1, 1))
+        else:
+            _nt_fused(out, residual.contiguous(), EPI_ADD, act, w2c, b2c, rows, n_out, hid)
+        ctx.save_for_backward(xc, pre, act, w1c, w2c)
+        ctx.refs = ((w1, w1._version), (w2, w2._version))
+        ctx.dtypes = tuple(None if t is None else t.dtype for t in (w1, b1, w2, b2))
+        ctx.has_residual = residual is not None
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):  # noqa: D102
+        xc, pre, act, w1c, w2c = ctx.saved_tensors
+        hid, k = w1c.shape
+        n_out = w2c.shape[0]
+        rows = xc.numel() // k
+        g = grad.to(xc.dtype).contiguous()
+        dt_w1, dt_b1, dt_w2, dt_b2 = ctx.dtypes
+
+        def transposed(i, wc):
+            ref, version = ctx.refs[i]
+            return _cast_cached(ref, wc.dtype, transposed=True) if ref._version == version else wc.t().contiguous()
+
+        gw2, gb2 = _tn(g, act, rows, n_out, hid, False, False, (1, 1, 1, 1), dt_b2 is not None,
+                       _grad_dtype(g.dtype, (dt_w2, dt_b2)))
+        dpre = torch.empty_like(pre)  # dL/d(pre-activation) = (g W2) * gelu'(pre)
+        _nt_fused(dpre, pre, EPI_DGELU, g, transposed(1, w2c), None, rows, hid, n_out)
+        gw1, gb1 = _tn(dpre, xc, rows, hid, k, False, False, (1, 1, 1, 1), dt_b1 is not None,
+                       _grad_dtype(g.dtype, (dt_w1, dt_b1)))
+        gx = None
+        if ctx.needs_input_grad[0]:
+            gx = torch.empty_like(xc)
+            _nt(gx, dpre, transposed(0, w1c), None, rows, k, hid, False, False, (1, 1, 1, 1))
+        return (gx, gw1.to(dt_w1), None if gb1 is None else gb1.to(dt_b1), gw2.to(dt_w2),
+                None if gb2 is None else gb2.to(dt_b2), g if ctx.has_residual else None)
+
+
+def gelu_mlp(x, w1, b1, w2, b2, residual=None):
+    """``(residual +) linear(gelu(linear(x, w1, b1)), w2, b2)``; GELU, its derivative and the residual
+    sum ride on the GEMMs when :func:`mlp_fusable`, else the same from separate steps."""
+    if mlp_fusable(x, w1, w2, residual):
+        return _GeluMlp.apply(x, w1, b1, w2, b2, residual)
+    y = linear(torch.nn.functional.gelu(linear(x, w1, b1)), w2, b2)
+    return y if residual is None else residual + y.to(residual.dtype)
+
+
 def qkv_projection(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, heads: int) -> torch.Tensor:
     """``rearrange(F.linear(x, weight, bias), "... s (three h d) -> three ... h s d", three=3, h=heads)``
     without the intermediate ``(..., s, 3 h d)`` tensor (_attention.py:881-890)."""
@@ -255,4 +337,4 @@ def heads_projection(out: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor
     return _HeadsProjection.apply(out, weight, bias)
 
 
-__all__ = ["heads_projection", "linear", "qkv_projection"]
+__all__ = ["gelu_mlp", "heads_projection", "linear", "mlp_fusable", "qkv_projection"]

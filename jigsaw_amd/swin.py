@@ -19,10 +19,10 @@ from typing import Any
 import torch
 import torch.nn as nn
 
-from .attention import swin_grid_attention, swin_grid_supported, window_attention
+from .attention import swin_grid_attention_packed, window_attention
 from .conv import TileGroup
 from .layernorm import plain_layer_norm
-from .projection import heads_projection, linear, qkv_projection
+from .projection import gelu_mlp, heads_projection, linear, qkv_projection
 from .roll import _Roll
 
 
@@ -119,9 +119,8 @@ class WindowAttention(nn.Module):
         if dt == torch.bfloat16 and c // self.heads == 32 and self.window == 8 and h % 8 == 0 and w % 8 == 0:
             # the kernel addresses the windows on the token grid and forms bias and mask itself:
             # no window partition, no (nW, heads, N, N) bias tensor
-            q, k, v = qkv_projection(x.to(dt).view(b, h * w, c), self.qkv.weight, self.qkv.bias, self.heads).unbind(0)
-            assert swin_grid_supported(q, (h, w), self.window)
-            out = swin_grid_attention(q, k, v, self.bias_table, self.side, (h, w))
+            qkv = qkv_projection(x.to(dt).view(b, h * w, c), self.qkv.weight, self.qkv.bias, self.heads)
+            out = swin_grid_attention_packed(qkv, self.bias_table, self.side, (h, w))
             return heads_projection(out, self.proj.weight, self.proj.bias).view(b, h, w, c)
         x = windows(x, self.window).to(dt)
         n = x.shape[2]
@@ -177,8 +176,8 @@ class SwinBlock(nn.Module):
 
     def finish(self, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
         x = x + y.to(x.dtype)
-        y = token_linear(self._norm(self.norm2, x), self.mlp[0])
-        return x + token_linear(self.mlp[1](y), self.mlp[2])
+        fc1, fc2 = self.mlp[0], self.mlp[2]
+        return gelu_mlp(self._norm(self.norm2, x), fc1.weight, fc1.bias, fc2.weight, fc2.bias, residual=x)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         y = self.unshift(self.attn(self.shift(self.pre_attention(x))))

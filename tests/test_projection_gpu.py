@@ -177,3 +177,45 @@ def test_fp32_parameters_get_unrounded_fp32_gradients(shape, n_out, dev):
     x3 = x.reshape(1, 1, -1, k).double()
     _, gw, gb = op.heads_backward(g.reshape(1, -1, n_out).double(), x3, w.bfloat16().double())
     assert rel_l2(wd.grad.cpu(), gw) < 1e-5 and rel_l2(bd.grad.cpu(), gb) < 1e-5
+
+
+@pytest.mark.parametrize("rows,dim,hid,with_res", [((3, 50), 64, 256, True), ((200,), 128, 512, True), ((2, 33), 40, 96, False)])
+def test_gelu_mlp_fused_epilogues(rows, dim, hid, with_res, dev):
+    """residual + Linear(GELU(Linear(x))) on the fused epilogues (GELU beside the pre-activation, the
+    GELU derivative and the residual sum on the way out of a GEMM) against fp64 autograd of the same
+    expression with torch's erf GELU (examples/swin.py:190-209). rel-L2 2e-2: bf16 operands, the bar
+    of the other bf16 projection tests; fp32 parameters get fp32 gradients."""
+    torch.manual_seed(11)
+    x = torch.randn(*rows, dim).bfloat16()
+    res = torch.randn(*rows, dim).bfloat16() if with_res else None
+    w1, b1 = torch.randn(hid, dim) * dim**-0.5, torch.randn(hid) * 0.1
+    w2, b2 = torch.randn(dim, hid) * hid**-0.5, torch.randn(dim) * 0.1
+    g = torch.randn(*rows, dim).bfloat16()
+
+    leaves = [t.double().requires_grad_() for t in (x, w1.bfloat16(), b1.bfloat16(), w2.bfloat16(), b2.bfloat16())]
+    xd, w1d, b1d, w2d, b2d = leaves
+    want = torch.nn.functional.linear(torch.nn.functional.gelu(torch.nn.functional.linear(xd, w1d, b1d)), w2d, b2d)
+    if with_res:
+        rd = res.double().requires_grad_()
+        want = rd + want
+    want.backward(g.double())
+
+    gx = x.to(dev).requires_grad_()
+    params = [t.to(dev).requires_grad_() for t in (w1, b1, w2, b2)]  # fp32 parameters, as under autocast
+    gres = res.to(dev).requires_grad_() if with_res else None
+    assert jp.mlp_fusable(gx, params[0], params[2], gres)
+    out = jp.gelu_mlp(gx, *params, residual=gres)
+    out.backward(g.to(dev))
+    torch.cuda.synchronize()
+    assert out.dtype == torch.bfloat16 and rel_l2(out, want) < 2e-2
+    assert rel_l2(gx.grad, xd.grad) < 2e-2
+    for name, got, w in zip(("w1", "b1", "w2", "b2"), params, (w1d, b1d, w2d, b2d)):
+        assert got.grad.dtype == torch.float32
+        assert rel_l2(got.grad, w.grad) < 2e-2, f"{name}: {rel_l2(got.grad, w.grad):.3e}"
+    if with_res:
+        assert torch.equal(gres.grad, g.to(dev))
+    # the separate-steps form of the same function (what runs when the fused form does not apply)
+    y2 = jp.linear(torch.nn.functional.gelu(jp.linear(gx.detach(), *[p.detach() for p in params[:2]])), *[p.detach() for p in params[2:]])
+    if with_res:
+        y2 = gres.detach() + y2
+    assert rel_l2(out, y2) < 1e-2
