@@ -153,6 +153,18 @@ int jg_roll_pack(void* strip, const void* x, int ndim, const int64_t* sizes,
 int jg_roll_unpack(void* x, const void* strip, int ndim, const int64_t* sizes,
                    int axis, int64_t window, int elem_size, void* stream);
 
+/* The steps of distributed_roll (_distributed_roll.py:63-113) folded into one pass each.
+ * jg_roll_pack_fused: jg_roll, then jg_roll_pack of the rolled tensor along `axis`, then the
+ * clearing of `clear` (the buffer the neighbour's slab is received in; may be NULL): lines 99 and
+ * 44-49. jg_roll_unpack_pack: jg_roll_unpack of the slab received along axis1, then
+ * jg_roll_pack along axis2 of the tensor so updated, then the clearing of clear2: line 59 of one
+ * exchange and 44-49 of the next. Both need 16-byte aligned tensors whose trailing axes (behind
+ * the slab axes, not rolled) span a multiple of 16 bytes; JG_ERR_UNSUPPORTED otherwise. */
+int jg_roll_pack_fused(void* dst, void* strip, void* clear, const void* src, int ndim, const int64_t* sizes,
+                       const int64_t* shifts, int axis, int64_t window, int elem_size, void* stream);
+int jg_roll_unpack_pack(void* x, const void* recv1, int axis1, int64_t window1, void* strip2, void* clear2,
+                        int axis2, int64_t window2, int ndim, const int64_t* sizes, int elem_size, void* stream);
+
 /* ------------------------------------------------------------------------- *
  * Sharded LayerNorm (last axis split over the channel group; HBM-bound)
  *

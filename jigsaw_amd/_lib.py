@@ -87,6 +87,16 @@ SIGNATURES: dict[str, tuple] = {
     ),
     "jg_roll": (c_int, [c_void_p, c_void_p, c_int, POINTER(c_int64), POINTER(c_int64), c_int, c_void_p]),
     "jg_roll_pack": (c_int, [c_void_p, c_void_p, c_int, POINTER(c_int64), c_int, c_int64, c_int, c_void_p]),
+    "jg_roll_pack_fused": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int, POINTER(c_int64), POINTER(c_int64), c_int, c_int64, c_int,
+         c_void_p],
+    ),
+    "jg_roll_unpack_pack": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_int64, c_void_p, c_void_p, c_int, c_int64, c_int, POINTER(c_int64), c_int,
+         c_void_p],
+    ),
     "jg_roll_unpack": (c_int, [c_void_p, c_void_p, c_int, POINTER(c_int64), c_int, c_int64, c_int, c_void_p]),
     "jg_ln_partial_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
     "jg_ln_apply": (

@@ -63,6 +63,74 @@ __global__ __launch_bounds__(256) void slab_kernel(T* __restrict__ x_or_strip_ds
   }
 }
 
+// x viewed as (outer, len, inner) along one axis; the slab is rows [start, start + win) of it.
+struct SlabView {
+  long long len, inner, start, win;
+  __device__ __forceinline__ bool holds(long long idx, long long* strip_idx) const {
+    const long long r = idx / inner, ci = idx - r * inner;
+    const long long o = r / len, l = r - o * len;
+    *strip_idx = (o * win + (l - start)) * inner + ci;
+    return l >= start && l < start + win;
+  }
+  __device__ __forceinline__ long long place(long long strip_idx) const {
+    const long long r = strip_idx / inner, ci = strip_idx - r * inner;
+    const long long o = r / win, a = r - o * win;
+    return (o * len + start + a) * inner + ci;
+  }
+};
+
+// The local roll, and on the way the wrapped slab of the ROLLED tensor along one axis cut into
+// `strip`, with the buffer the neighbour's slab will be received in cleared (what the reference
+// does in three passes: torch.roll, x[sl].contiguous(), torch.zeros_like).
+template <typename T>
+__global__ __launch_bounds__(256) void roll_pack_kernel(T* __restrict__ dst, const T* __restrict__ src, RollArgs a,
+                                                        long long total, T* __restrict__ strip, T* __restrict__ clear,
+                                                        SlabView v) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long long)gridDim.x * 256) {
+    long long rem = i, so = 0, stride = 1;
+#pragma unroll
+    for (int k = kMaxDims - 1; k >= 0; --k) {
+      if (k < a.nd) {
+        long long q = rem / a.size[k];
+        long long c = rem - q * a.size[k];
+        rem = q;
+        long long sc = c - a.shift[k];
+        if (sc < 0) sc += a.size[k];
+        so += sc * stride;
+        stride *= a.size[k];
+      }
+    }
+    const T val = src[so];
+    dst[i] = val;
+    long long j;
+    if (v.holds(i, &j)) {
+      strip[j] = val;
+      if (clear != nullptr) clear[j] = T{};
+    }
+  }
+}
+
+// Between two exchanges: the slab received along the first axis goes into x, and the slab to
+// send along the second axis is cut from x as it will be AFTER that write: where the two slabs
+// cross, the cut takes the received values directly, so the two steps do not wait for each other.
+// The buffer for the second exchange is cleared on the way.
+template <typename T>
+__global__ __launch_bounds__(256) void unpack_pack_kernel(T* __restrict__ x, const T* __restrict__ recv1, SlabView v1,
+                                                          long long n1, T* __restrict__ strip2, T* __restrict__ clear2,
+                                                          SlabView v2, long long n2) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n1 + n2; i += (long long)gridDim.x * 256) {
+    if (i < n1) {
+      x[v1.place(i)] = recv1[i];
+    } else {
+      const long long j = i - n1;
+      const long long idx = v2.place(j);
+      long long j1;
+      strip2[j] = v1.holds(idx, &j1) ? recv1[j1] : x[idx];
+      if (clear2 != nullptr) clear2[j] = T{};
+    }
+  }
+}
+
 int grid_for(long long n) {
   long long b = (n + 255) / 256;
   if (b > (1 << 20)) b = 1 << 20;
@@ -199,4 +267,110 @@ extern "C" int jg_roll_unpack(void* x, const void* strip, int ndim, const int64_
                               int axis, int64_t window, int elem_size, void* stream) {
   return slab_common(x, strip, x, ndim, sizes, axis, window, elem_size, stream, false,
                      "jg_roll_unpack");
+}
+
+
+namespace {
+struct Axis {
+  long long outer, len, inner, start, win;
+};
+int axis_view(Axis* v, int ndim, const int64_t* sizes, int axis, int64_t window, const char* who) {
+  JG_REQUIRE(axis >= 0 && axis < ndim, "%s: axis %d out of range", who, axis);
+  v->outer = v->inner = 1;
+  for (int i = 0; i < ndim; ++i) {
+    JG_REQUIRE(sizes[i] >= 0, "%s: negative size", who);
+    if (i < axis) v->outer *= sizes[i];
+    if (i > axis) v->inner *= sizes[i];
+  }
+  v->len = sizes[axis];
+  v->win = window < 0 ? -window : window;
+  JG_REQUIRE(v->win <= v->len, "%s: |window| = %lld exceeds the local size %lld", who, v->win, v->len);
+  v->start = window > 0 ? 0 : v->len - v->win;
+  return JG_OK;
+}
+}  // namespace
+
+// jg_roll, jg_roll_pack of the rolled tensor along `axis` and the clearing of the receive buffer in
+// one pass (_distributed_roll.py:99 followed by 44-49 of the first exchange). 16-byte runs only:
+// the trailing axes that are not rolled (and lie behind `axis`) must make up a multiple of 16 bytes.
+extern "C" int jg_roll_pack_fused(void* dst, void* strip, void* clear, const void* src, int ndim, const int64_t* sizes,
+                                  const int64_t* shifts, int axis, int64_t window, int elem_size, void* stream) {
+  const char* who = "jg_roll_pack_fused";
+  JG_REQUIRE(dst && strip && src && sizes && shifts, "%s: NULL pointer", who);
+  JG_REQUIRE(dst != src, "%s: dst must not alias src", who);
+  JG_REQUIRE(ndim >= 1 && ndim <= kMaxDims, "%s: ndim %d not in [1, %d]", who, ndim, kMaxDims);
+  JG_REQUIRE(elem_size == 2 || elem_size == 4, "%s: elem_size %d not in {2, 4}", who, elem_size);
+  Axis ax;
+  int rc = axis_view(&ax, ndim, sizes, axis, window, who);
+  if (rc) return rc;
+  long long total = 1;
+  for (int i = 0; i < ndim; ++i) total *= sizes[i];
+  if (total == 0) return JG_OK;
+  int last = ndim;  // axes [last, ndim) are not rolled
+  while (last > 0 && (shifts[last - 1] % sizes[last - 1]) == 0) --last;
+  if (last <= axis) last = axis + 1;  // the slab axis keeps an index of its own
+  long long run = 1;
+  for (int i = last; i < ndim; ++i) run *= sizes[i];
+  const long long run_bytes = run * elem_size;
+  if (run_bytes % 16 != 0 || !aligned16(dst) || !aligned16(src) || !aligned16(strip) || (clear && !aligned16(clear)))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: needs 16-byte aligned tensors whose unrolled trailing axes span a multiple of 16 bytes", who);
+  JG_REQUIRE(last + 1 <= kMaxDims, "%s: too many rolled axes", who);
+  RollArgs a;
+  a.nd = 0;
+  for (int i = 0; i < last; ++i) {
+    long long m = shifts[i] % sizes[i];
+    if (m < 0) m += sizes[i];
+    a.size[a.nd] = sizes[i];
+    a.shift[a.nd] = m;
+    ++a.nd;
+  }
+  const long long words = run_bytes / 16;
+  a.size[a.nd] = words;
+  a.shift[a.nd] = 0;
+  ++a.nd;
+  // the slab view in 16-byte words: inner = (axes between `axis` and `last`) * words
+  SlabView v;
+  v.len = ax.len; v.start = ax.start; v.win = ax.win;
+  v.inner = ax.inner / run * words;
+  const long long n = total / run * words;
+  roll_pack_kernel<u32x4><<<grid_for(n), 256, 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), a, n, static_cast<u32x4*>(strip),
+      static_cast<u32x4*>(clear), v);
+  JG_CHECK_LAUNCH(who);
+  return JG_OK;
+}
+
+// jg_roll_unpack of the slab received along axis1 and jg_roll_pack of the slab to send along axis2
+// (with its receive buffer cleared) in one pass (_distributed_roll.py:59 of one exchange, 44-49 of
+// the next). The innermost axis must span a multiple of 16 bytes and lie behind both axes.
+extern "C" int jg_roll_unpack_pack(void* x, const void* recv1, int axis1, int64_t window1, void* strip2, void* clear2,
+                                   int axis2, int64_t window2, int ndim, const int64_t* sizes, int elem_size,
+                                   void* stream) {
+  const char* who = "jg_roll_unpack_pack";
+  JG_REQUIRE(x && recv1 && strip2 && sizes, "%s: NULL pointer", who);
+  JG_REQUIRE(ndim >= 1 && ndim <= 8, "%s: ndim %d out of range", who, ndim);
+  JG_REQUIRE(elem_size == 2 || elem_size == 4, "%s: elem_size %d not in {2, 4}", who, elem_size);
+  JG_REQUIRE(axis1 != axis2, "%s: the two axes must differ", who);
+  Axis a1, a2;
+  int rc = axis_view(&a1, ndim, sizes, axis1, window1, who);
+  if (rc) return rc;
+  rc = axis_view(&a2, ndim, sizes, axis2, window2, who);
+  if (rc) return rc;
+  const int deeper = axis1 > axis2 ? axis1 : axis2;
+  long long run = 1;
+  for (int i = deeper + 1; i < ndim; ++i) run *= sizes[i];
+  const long long run_bytes = run * elem_size;
+  if (run_bytes % 16 != 0 || !aligned16(x) || !aligned16(recv1) || !aligned16(strip2) || (clear2 && !aligned16(clear2)))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: needs 16-byte aligned tensors whose axes behind both slab axes span a multiple of 16 bytes", who);
+  const long long words = run_bytes / 16;
+  SlabView v1, v2;
+  v1.len = a1.len; v1.start = a1.start; v1.win = a1.win; v1.inner = a1.inner / run * words;
+  v2.len = a2.len; v2.start = a2.start; v2.win = a2.win; v2.inner = a2.inner / run * words;
+  const long long n1 = a1.outer * a1.win * v1.inner, n2 = a2.outer * a2.win * v2.inner;
+  if (n1 + n2 == 0) return JG_OK;
+  unpack_pack_kernel<u32x4><<<grid_for(n1 + n2), 256, 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<u32x4*>(x), static_cast<const u32x4*>(recv1), v1, n1, static_cast<u32x4*>(strip2),
+      static_cast<u32x4*>(clear2), v2, n2);
+  JG_CHECK_LAUNCH(who);
+  return JG_OK;
 }

@@ -103,6 +103,19 @@ def exchange_halo_1d(
     return slab_unpack_(x, recv, dim, window_size)
 
 
+def _fused_steps_ok(x: torch.Tensor, per_axis: list, axes: list) -> bool:
+    """Whether the one-pass kernels take this roll: distinct slab axes, and behind the last rolled
+    axis and the last slab axis a run of whole 16-byte words."""
+    if x.numel() == 0 or x.dim() > 5 or x.element_size() not in (2, 4) or len(set(axes)) != len(axes):
+        return False
+    rolled = [a for a, s in enumerate(per_axis) if s % x.shape[a] != 0]
+    tail_from = max([*rolled, *axes]) + 1
+    run = 1
+    for n in x.shape[tail_from:]:
+        run *= n
+    return (run * x.element_size()) % 16 == 0 and x.data_ptr() % 16 == 0
+
+
 def distributed_roll(
     x: torch.Tensor,
     shifts: tuple,
@@ -115,19 +128,61 @@ def distributed_roll(
 
     Same contract and error behaviour as ``distributed_roll`` of
     jigsaw/modules/roll/_distributed_roll.py:63-113 (``exchange_halo_1d_fn`` is,
-    as there, the 1-D communication function).
+    as there, the 1-D communication function). Where the layout allows, the passes between
+    two exchanges are one launch each: roll + cut of the first slab + clearing of its receive
+    buffer; write-back of a received slab + cut of the next one; the last write-back.
     """
-    x = roll(x, shifts, dims)
-    dim_to_shift = {d % x.ndim: s for d, s in zip(dims, shifts)}
+    if len(shifts) != len(dims):
+        raise RuntimeError(f"shifts and dimensions must align. shifts: {len(shifts)}, dims:{len(dims)}")
+    nd = x.dim()
+    dim_to_shift = {d % nd: s for d, s in zip(dims, shifts)}
     if len(distributed_dims) != len(spatial_process_groups):
         raise ValueError("distributed_dims and spatial_process_groups differ in length")
+    steps = []
     for d, pg in zip(distributed_dims, spatial_process_groups):
-        if d % x.ndim not in dim_to_shift:
+        if d % nd not in dim_to_shift:
             raise ValueError(f"distributed dim {d} not in dims {dims}")
-        x = exchange_halo_1d(
-            x, dim=d, window_size=dim_to_shift[d % x.ndim], group=pg, comm_halo_1d_fn=exchange_halo_1d_fn
-        )
-    return x
+        if dim_to_shift[d % nd] != 0:
+            steps.append((d % nd, int(dim_to_shift[d % nd]), pg))
+    per_axis = [0] * nd
+    for s, d in zip(shifts, dims):
+        per_axis[d % nd] += int(s)
+    x = x.contiguous()
+    if not steps or not _fused_steps_ok(x, per_axis, [a for a, _, _ in steps]):
+        x = roll(x, shifts, dims)
+        for axis, window, pg in steps:
+            x = exchange_halo_1d(x, dim=axis, window_size=window, group=pg, comm_halo_1d_fn=exchange_halo_1d_fn)
+        return x
+
+    _lib.require_gpu(x)
+    lib = _lib.load()
+    shape, esize, stream = _lib.i64_array(x.shape), x.element_size(), _lib.stream_ptr(x.device)
+
+    def buffers(axis, window):
+        slab = list(x.shape)
+        slab[axis] = abs(window)
+        return torch.empty(slab, dtype=x.dtype, device=x.device), torch.empty(slab, dtype=x.dtype, device=x.device)
+
+    out = torch.empty_like(x)
+    axis, window, pg = steps[0]
+    if abs(window) > x.shape[axis]:
+        raise ValueError(f"|window| = {abs(window)} exceeds the local size {x.shape[axis]} along dim {axis}")
+    strip, recv = buffers(axis, window)
+    rc = lib.jg_roll_pack_fused(_lib.ptr(out), _lib.ptr(strip), _lib.ptr(recv), _lib.ptr(x), nd, shape,
+                                _lib.i64_array(per_axis), axis, window, esize, stream)
+    _lib.check(rc, "jg_roll_pack_fused")
+    recv, _ = exchange_halo_1d_fn(strip, recv, 1 if window > 0 else -1, group=pg, async_op=False)
+    for axis2, window2, pg2 in steps[1:]:
+        if abs(window2) > x.shape[axis2]:
+            raise ValueError(f"|window| = {abs(window2)} exceeds the local size {x.shape[axis2]} along dim {axis2}")
+        strip2, recv2 = buffers(axis2, window2)
+        recv = recv.to(dtype=x.dtype).contiguous()
+        rc = lib.jg_roll_unpack_pack(_lib.ptr(out), _lib.ptr(recv), axis, window, _lib.ptr(strip2), _lib.ptr(recv2),
+                                     axis2, window2, nd, shape, esize, stream)
+        _lib.check(rc, "jg_roll_unpack_pack")
+        recv, _ = exchange_halo_1d_fn(strip2, recv2, 1 if window2 > 0 else -1, group=pg2, async_op=False)
+        axis, window = axis2, window2
+    return slab_unpack_(out, recv, axis, window)
 
 
 class _Roll(torch.autograd.Function):
