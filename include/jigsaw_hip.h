@@ -244,6 +244,14 @@ int jg_ln_plain_bwd(void* gx, float* gw, float* gb, const void* g, const void* x
                     const float* mean, const float* rstd, const float* w, int64_t rows,
                     int64_t cols, int g_dtype, int x_dtype, void* workspace,
                     size_t workspace_bytes, void* stream);
+/* jg_ln_plain_bwd with the gradient that reaches x past the normalisation added in:
+ * gx = round(gx of jg_ln_plain_bwd) + add, add (rows, cols) in x's dtype. For the pre-norm
+ * residual blocks x + f(norm(x)) (examples/swin.py:206-209), where autograd would add the two
+ * gradient tensors in a pass of its own. */
+int jg_ln_plain_bwd_add(void* gx, float* gw, float* gb, const void* g, const void* x,
+                        const float* mean, const float* rstd, const float* w, int64_t rows,
+                        int64_t cols, int g_dtype, int x_dtype, void* workspace,
+                        size_t workspace_bytes, const void* add, void* stream);
 
 /* ------------------------------------------------------------------------- *
  * GroupNorm over a spatially sharded input (HBM-bound)

@@ -130,6 +130,11 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int,
          c_void_p, c_size_t, c_void_p],
     ),
+    "jg_ln_plain_bwd_add": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int,
+         c_void_p, c_size_t, c_void_p, c_void_p],
+    ),
     "jg_gn_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "jg_gn_partial_sum": (
         c_int,

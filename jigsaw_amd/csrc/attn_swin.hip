@@ -19,9 +19,9 @@
 //   Backward   the two passes of the plain window kernel (lane = query for dQ, lane = key for
 //              dK / dV). The gradient of the table is what pass A's dS^T scatters by the same row
 //              arithmetic: each wavefront adds it into 2 x 225 bins of its own in LDS (one set per
-//              lane half, inside which the rows of an instruction's lanes are all different, so no
-//              two lanes of an add meet and the order of additions is fixed), writes the bins out,
-//              and two small kernels add the entries' bins per head in a fixed order.
+//              lane half, inside which the rows of an instruction's lanes are all different, so a
+//              plain read, add, write per register is exact and its order fixed), writes the bins
+//              out, and two small kernels add the entries' bins per head in a fixed order.
 #include "attn_window_common.h"
 
 namespace {
@@ -259,10 +259,10 @@ __global__ __launch_bounds__(WAVES * 64) void attn_swin_bwd_kernel(SwinArgs p) {
     float* bl = bins + kg * ROWS + row0;
     const uint64_t ap = sd.mixed ? apart_from(sd, qi) >> (4 * kg) : 0ull;
     f32x16 dqa = zero16();
+    float ds[2][16];
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) {
       const uint32_t word = (uint32_t)(ap >> (32 * mb));
-      float ds[16];
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4)
 #pragma unroll
@@ -271,12 +271,31 @@ __global__ __launch_bounds__(WAVES * 64) void attn_swin_bwd_kernel(SwinArgs p) {
           const int c = TOP - (60 * mb + 15 * i4 + r);
           float pr = __builtin_amdgcn_exp2f(s[mb][i] * c2 + tl[c] - lse_q[nb]);
           if (sd.mixed && ((word >> (8 * i4 + r)) & 1u)) pr = 0.0f;
-          ds[i] = pr * (dp[mb][i] - delta_q[nb]);
-          if (DTABLE && valid) __hip_atomic_fetch_add(bl + c, ds[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+          ds[mb][i] = pr * (dp[mb][i] - delta_q[nb]);
         }
 #pragma unroll
       for (int h = 0; h < 2; ++h)
-        dqa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(kt, mb * 2 + h, ln, kg), pack_half(ds, h), dqa, 0, 0, 0);
+        dqa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(kt, mb * 2 + h, ln, kg), pack_half(ds[mb], h), dqa, 0, 0, 0);
+    }
+    if (DTABLE && valid) {
+      // dS^T into the bins, register by register: the 32 lanes of a half hit 32 different rows, and
+      // so do a register of key block 0 and its twin of block 1 (their rows differ by 60, more
+      // than the queries of a 32-lane block are apart), so the pair is read, added to and
+      // written back as plain LDS accesses; the LDS keeps a wavefront's accesses in order.
+      // (LDS float atomics do the same job at about 800 cycles an instruction.)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int i = i4 * 4 + r;
+          const int c0 = TOP - (15 * i4 + r), c1 = c0 - 60;
+          const float b0 = bl[c0], b1 = bl[c1];
+          bl[c0] = b0 + ds[0][i];
+          bl[c1] = b1 + ds[1][i];
+          // for one lane the rows of different registers never coincide, so the compiler would be
+          // free to read ahead; other lanes' rows do coincide with them: one step after the other
+          asm volatile("" ::: "memory");
+        }
     }
     if (valid) {
       uint16_t* row = p.dq + en.base + en.rowoff[nb];

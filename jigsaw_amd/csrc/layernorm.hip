@@ -456,7 +456,7 @@ __global__ __launch_bounds__(kThreads) void ln_plain_bwd_kernel(
     typename Elem<XDT>::T* __restrict__ gx, float* __restrict__ part,
     const typename Elem<GDT>::T* __restrict__ g, const typename Elem<XDT>::T* __restrict__ x,
     const float* __restrict__ mean, const float* __restrict__ rstd, const float* __restrict__ w,
-    long long rows, int cols, int G, bool want_cols) {
+    long long rows, int cols, int G, bool want_cols, const typename Elem<XDT>::T* __restrict__ add) {
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
   const float inv = 1.0f / (float)cols;
@@ -524,6 +524,14 @@ __global__ __launch_bounds__(kThreads) void ln_plain_bwd_kernel(
 #pragma unroll
           for (int i = 0; i < kPlainVec; ++i)
             out[i] = rs[u] * (gv[u][k][i] * wv[k][i] - s1[u] - xh[u][k][i] * s2[u]);
+          if (add != nullptr) {
+            // the gradient that reaches x past the normalisation (a residual connection): added
+            // to the rounded result, as the separate sum of the two gradient tensors would
+            float past[kPlainVec];
+            load8<XDT>(add + r * cols + c, past);
+#pragma unroll
+            for (int i = 0; i < kPlainVec; ++i) out[i] = Elem<XDT>::up(Elem<XDT>::down(out[i])) + past[i];
+          }
           store8<XDT>(gx + r * cols + c, out);
         }
       }
@@ -602,7 +610,7 @@ void launch_plain_fwd(void* y, float* mean, float* rstd, const void* x, const fl
 
 template <int GDT, int XDT>
 void launch_plain_bwd(void* gx, float* part, const void* g, const void* x, const float* mean, const float* rstd,
-                      const float* w, long long rows, int cols, bool want_cols, hipStream_t s) {
+                      const float* w, long long rows, int cols, bool want_cols, const void* add, hipStream_t s) {
   typedef typename Elem<GDT>::T GT;
   typedef typename Elem<XDT>::T XT;
   const int G = plain_group(cols), blocks = plain_blocks(rows, cols);
@@ -610,7 +618,7 @@ void launch_plain_bwd(void* gx, float* part, const void* g, const void* x, const
   ln_plain_bwd_kernel<GDT, XDT, CH, U><<<blocks, kThreads, 0, s>>>(static_cast<XT*>(gx), part,            \
                                                                    static_cast<const GT*>(g),             \
                                                                    static_cast<const XT*>(x), mean, rstd, \
-                                                                   w, rows, cols, G, want_cols)
+                                                                   w, rows, cols, G, want_cols, static_cast<const XT*>(add))
   switch (plain_chunks(cols)) {
     case 1: JG_GO(1, 2); break;
     case 2: JG_GO(2, 2); break;
@@ -871,12 +879,12 @@ extern "C" size_t jg_ln_plain_bwd_workspace_bytes(int64_t rows, int64_t cols) {
   return (size_t)plain_blocks(rows, cols) * 2 * (size_t)cols * sizeof(float);
 }
 
-extern "C" int jg_ln_plain_bwd(void* gx, float* gw, float* gb, const void* g, const void* x,
-                               const float* mean, const float* rstd, const float* w, int64_t rows,
-                               int64_t cols, int g_dtype, int x_dtype, void* workspace,
-                               size_t workspace_bytes, void* stream) {
-  const char* who = "jg_ln_plain_bwd";
+static int plain_bwd_common(const char* who, void* gx, float* gw, float* gb, const void* g, const void* x,
+                            const float* mean, const float* rstd, const float* w, int64_t rows, int64_t cols,
+                            int g_dtype, int x_dtype, void* workspace, size_t workspace_bytes, const void* add,
+                            void* stream) {
   JG_REQUIRE(g && x && mean && rstd && w, "%s: NULL pointer", who);
+  JG_REQUIRE(add == nullptr || (gx != nullptr && aligned16(add)), "%s: add needs gx and 16-byte alignment", who);
   JG_REQUIRE(rows >= 0 && cols >= 1, "%s: bad shape (%lld, %lld)", who, (long long)rows, (long long)cols);
   JG_REQUIRE(known(x_dtype) && known(g_dtype), "%s: unknown dtype", who);
   if (!plain_ok(cols))
@@ -902,7 +910,7 @@ extern "C" int jg_ln_plain_bwd(void* gx, float* gw, float* gb, const void* g, co
     if (workspace == nullptr || workspace_bytes < need)
       JG_FAIL(JG_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", who, workspace_bytes, need);
   }
-#define JG_GO(G_, X) launch_plain_bwd<G_, X>(gx, part, g, x, mean, rstd, w, rows, (int)cols, want_cols, s)
+#define JG_GO(G_, X) launch_plain_bwd<G_, X>(gx, part, g, x, mean, rstd, w, rows, (int)cols, want_cols, add, s)
   if (x_dtype == JG_F32) {
     if (g_dtype == JG_F32) JG_GO(JG_F32, JG_F32);
     else if (g_dtype == JG_BF16) JG_GO(JG_BF16, JG_F32);
@@ -921,4 +929,22 @@ extern "C" int jg_ln_plain_bwd(void* gx, float* gw, float* gb, const void* g, co
     JG_CHECK_LAUNCH(who);
   }
   return JG_OK;
+}
+
+extern "C" int jg_ln_plain_bwd(void* gx, float* gw, float* gb, const void* g, const void* x,
+                               const float* mean, const float* rstd, const float* w, int64_t rows,
+                               int64_t cols, int g_dtype, int x_dtype, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+  return plain_bwd_common("jg_ln_plain_bwd", gx, gw, gb, g, x, mean, rstd, w, rows, cols, g_dtype, x_dtype, workspace,
+                          workspace_bytes, nullptr, stream);
+}
+
+extern "C" int jg_ln_plain_bwd_add(void* gx, float* gw, float* gb, const void* g, const void* x,
+                                   const float* mean, const float* rstd, const float* w, int64_t rows,
+                                   int64_t cols, int g_dtype, int x_dtype, void* workspace,
+                                   size_t workspace_bytes, const void* add, void* stream) {
+  const char* who = "jg_ln_plain_bwd_add";
+  JG_REQUIRE(add != nullptr && gx != nullptr, "%s: NULL pointer", who);
+  return plain_bwd_common(who, gx, gw, gb, g, x, mean, rstd, w, rows, cols, g_dtype, x_dtype, workspace,
+                          workspace_bytes, add, stream);
 }

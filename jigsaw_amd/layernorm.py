@@ -178,7 +178,7 @@ class _PlainLayerNorm(torch.autograd.Function):
         return y
 
     @staticmethod
-    def backward(ctx, grad):  # noqa: D102
+    def backward(ctx, grad, past=None):  # noqa: D102
         xc, mean, rstd, w = ctx.saved_tensors
         cols = xc.shape[-1]
         rows = xc.numel() // cols
@@ -194,12 +194,48 @@ class _PlainLayerNorm(torch.autograd.Function):
         lib = _lib.load()
         nbytes = int(lib.jg_ln_plain_bwd_workspace_bytes(rows, cols)) if (need_w or need_b) else 0
         ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=dev)
-        rc = lib.jg_ln_plain_bwd(_lib.ptr(gx), _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(g), _lib.ptr(xc), _lib.ptr(mean),
-                                 _lib.ptr(rstd), _lib.ptr(w), rows, cols, _lib.dtype_code(g.dtype), _lib.dtype_code(xc.dtype),
-                                 _lib.ptr(ws), nbytes, _lib.stream_ptr(dev))
-        _lib.check(rc, "jg_ln_plain_bwd")
+        if past is not None and need_x:
+            past = past.to(xc.dtype).contiguous()
+            rc = lib.jg_ln_plain_bwd_add(_lib.ptr(gx), _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(g), _lib.ptr(xc), _lib.ptr(mean),
+                                         _lib.ptr(rstd), _lib.ptr(w), rows, cols, _lib.dtype_code(g.dtype),
+                                         _lib.dtype_code(xc.dtype), _lib.ptr(ws), nbytes, _lib.ptr(past), _lib.stream_ptr(dev))
+            _lib.check(rc, "jg_ln_plain_bwd_add")
+        else:
+            rc = lib.jg_ln_plain_bwd(_lib.ptr(gx), _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(g), _lib.ptr(xc), _lib.ptr(mean),
+                                     _lib.ptr(rstd), _lib.ptr(w), rows, cols, _lib.dtype_code(g.dtype), _lib.dtype_code(xc.dtype),
+                                     _lib.ptr(ws), nbytes, _lib.stream_ptr(dev))
+            _lib.check(rc, "jg_ln_plain_bwd")
         wdt, bdt = ctx.param_dtypes
         return gx, (gw.to(wdt) if need_w else None), (gb.to(bdt) if need_b else None), None, None
+
+
+class _PlainLayerNormFork(torch.autograd.Function):
+    """``(LayerNorm(x), x)``: the normalised rows for a branch and the rows themselves for the
+    residual connection around it (``x + f(norm(x))``, examples/swin.py:206-209). The backward adds
+    the gradient that arrives over the connection inside the LayerNorm backward kernel, where
+    autograd would otherwise add the two gradient tensors of ``x`` in a pass of its own."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, eps, out_dtype):  # noqa: D102
+        y = _PlainLayerNorm.forward(ctx, x, weight, bias, eps, out_dtype)
+        return y, x.view_as(x)
+
+    @staticmethod
+    def backward(ctx, grad, past):  # noqa: D102
+        if grad is None:  # the branch was not used
+            return past, None, None, None, None
+        return _PlainLayerNorm.backward(ctx, grad, past)
+
+
+def plain_layer_norm_fork(x, weight, bias, eps: float = 1e-5, out_dtype: torch.dtype | None = None):
+    """``(plain_layer_norm(x, ...), x)`` for a pre-norm residual block: use the second result where
+    the block adds ``x`` back, and the sum of the two gradients of ``x`` is formed inside the
+    LayerNorm backward (see :class:`_PlainLayerNormFork`). Falls back to the two separate results
+    where :func:`plain_layer_norm` itself does."""
+    odt = out_dtype or _compute_dtype(x)
+    if x.numel() == 0 or not _lib.load().jg_ln_plain_supported(x.shape[-1]):
+        return plain_layer_norm(x, weight, bias, eps, out_dtype), x
+    return _PlainLayerNormFork.apply(x, weight, bias, eps, odt)
 
 
 def plain_layer_norm(x, weight, bias, eps: float = 1e-5, out_dtype: torch.dtype | None = None) -> torch.Tensor:
@@ -217,4 +253,4 @@ def plain_layer_norm(x, weight, bias, eps: float = 1e-5, out_dtype: torch.dtype 
     return _PlainLayerNorm.apply(x, weight, bias, eps, odt)
 
 
-__all__ = ["_LayerNorm", "layer_norm", "partial_stats", "plain_layer_norm"]
+__all__ = ["_LayerNorm", "layer_norm", "partial_stats", "plain_layer_norm", "plain_layer_norm_fork"]

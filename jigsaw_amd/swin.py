@@ -21,7 +21,7 @@ import torch.nn as nn
 
 from .attention import swin_grid_attention_packed, window_attention
 from .conv import TileGroup
-from .layernorm import plain_layer_norm
+from .layernorm import plain_layer_norm, plain_layer_norm_fork
 from .projection import gelu_mlp, heads_projection, linear, qkv_projection
 from .roll import _Roll
 
@@ -180,8 +180,14 @@ class SwinBlock(nn.Module):
         return gelu_mlp(self._norm(self.norm2, x), fc1.weight, fc1.bias, fc2.weight, fc2.bias, residual=x)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        y = self.unshift(self.attn(self.shift(self.pre_attention(x))))
-        return self.finish(x, y)
+        # x + f(norm(x)) twice; the rows that go round a branch come out of the LayerNorm call beside
+        # the normalised ones, so that the backward adds the two gradients of x inside its kernel
+        dt = _compute_dtype(x)
+        y, x = plain_layer_norm_fork(x, self.norm1.weight, self.norm1.bias, self.eps, out_dtype=dt)
+        x = x + self.unshift(self.attn(self.shift(y))).to(x.dtype)
+        y, x = plain_layer_norm_fork(x, self.norm2.weight, self.norm2.bias, self.eps, out_dtype=dt)
+        fc1, fc2 = self.mlp[0], self.mlp[2]
+        return gelu_mlp(y, fc1.weight, fc1.bias, fc2.weight, fc2.bias, residual=x)
 
 
 __all__ = ["SwinBlock", "WindowAttention", "border_sides", "relative_position_index", "shift_mask", "unwindows", "windows"]

@@ -215,3 +215,38 @@ def test_plain_layer_norm_takes_non_contiguous_input(dev):
     got = jl.plain_layer_norm(x, w, b)
     want = F.layer_norm(x.cpu().double(), (64,), w.cpu().double(), b.cpu().double())
     assert rel_l2(got.cpu(), want) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_plain_layer_norm_fork_adds_the_residual_gradient_in_the_kernel(dtype, dev):
+    """x + f(norm(x)) through plain_layer_norm_fork against the same expression with the plain call
+    and autograd's own sum of the two gradients of x: same numbers (the kernel adds the gradient
+    that comes over the residual connection to the rounded LayerNorm gradient, as the separate sum
+    does)."""
+    from jigsaw_amd import layernorm as jl
+
+    torch.manual_seed(5)
+    x = torch.randn(3, 37, 128, device=dev).to(dtype)
+    w, b = torch.randn(128, device=dev), torch.randn(128, device=dev)
+    g = torch.randn(3, 37, 128, device=dev).to(dtype)
+
+    def run(fork):
+        xs = x.clone().requires_grad_()
+        ws, bs = w.clone().requires_grad_(), b.clone().requires_grad_()
+        if fork:
+            y, keep = jl.plain_layer_norm_fork(xs, ws, bs, 1e-5, out_dtype=dtype)
+        else:
+            y, keep = jl.plain_layer_norm(xs, ws, bs, 1e-5, out_dtype=dtype), xs
+        out = keep + torch.tanh(y)
+        out.backward(g)
+        return out, xs.grad, ws.grad, bs.grad
+
+    a, b_ = run(True), run(False)
+    torch.cuda.synchronize()
+    for got, want in zip(a, b_):
+        assert torch.equal(got, want)
+    # only the branch, and only the connection
+    xs = x.clone().requires_grad_()
+    y, keep = jl.plain_layer_norm_fork(xs, w, b, 1e-5, out_dtype=dtype)
+    keep.backward(g)
+    assert torch.equal(xs.grad, g)
