@@ -745,6 +745,23 @@ __global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
   // does reach are patched inside their vector. All the loads of a batch precede its
   // first store.
   const int n_vec = W / V;
+  // Halos one column wide (3-wide kernels): column 0 and column W - 1 are the only ones a W
+  // neighbour reaches. Their strip values are asked for here, with the row's own loads, and their
+  // own values are taken from the vectors as they pass, so that finishing them below costs no
+  // further trip to memory.
+  const int lpr_mask = (1 << pl.lpr_log2) - 1;
+  const bool thin = g.hi[2] == 1 && g.lo[2] == 1 && n_vec >= 2;
+  const bool owns_first = thin && lir == 0, owns_last = thin && lir == ((n_vec - 1) & lpr_mask);
+  T strip_first = T(0), strip_last = T(0);
+  if (owns_first && s_lo != nullptr) strip_first = s_lo[0];
+  if (owns_last && s_hi != nullptr) strip_last = s_hi[W - 1 - up0];
+  auto ends = [&](T lower, T own_bits, T upper, bool has_lower, bool has_upper) {
+    float acc = 0.0f;
+    if (has_lower) acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(lower)));
+    acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(own_bits)));
+    if (has_upper) acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(upper)));
+    return Arith<DT>::down(acc);
+  };
   for (int it0 = 0; (it0 << pl.lpr_log2) < n_vec; it0 += ROW_BATCH) {
     u32x4 val[ROW_BATCH];
 #pragma unroll
@@ -760,19 +777,31 @@ __global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
         T tmp[V];
         __builtin_memcpy(tmp, &val[u], 16);
         const int c0 = j * V;
-        if (c0 < g.hi[2] || c0 + V > up0) {
+        const T first_bits = tmp[0], last_bits = tmp[V - 1];
+        // `0 + own` for every column; then the two columns of a thin halo get their ordered sum
+        // (wider halos: below). Running the ordered sum for all 8 elements of the first and of the
+        // last vector, one lane active, was three quarters of the kernel's instructions.
 #pragma unroll
-          for (int e = 0; e < V; ++e) tmp[e] = element(c0 + e, tmp[e]);
-        } else {
-#pragma unroll
-          for (int e = 0; e < V; ++e)
-            if ((tmp[e] & ABS) == 0) tmp[e] = 0;
-        }
+        for (int e = 0; e < V; ++e)
+          if ((tmp[e] & ABS) == 0) tmp[e] = 0;
+        if (owns_first && j == 0) tmp[0] = ends(strip_first, first_bits, T(0), s_lo != nullptr, false);
+        if (owns_last && j == n_vec - 1 && n_vec * V == W) tmp[V - 1] = ends(T(0), last_bits, strip_last, false, s_hi != nullptr);
         u32x4 out;
         __builtin_memcpy(&out, tmp, 16);
         *reinterpret_cast<u32x4_s4*>(drow + c0) = out;
       }
     }
+  }
+  // Wider halos: the columns a W neighbour reaches, one at a time, by the lane whose vector store
+  // covered them (a lane's own stores to one address keep their order): vector j belongs to lane
+  // j % lanes-per-row.
+  if (!thin) {
+    const int head = g.hi[2] < n_vec * V ? g.hi[2] : n_vec * V;
+    for (int c = 0; c < head; ++c)
+      if (((c / V) & lpr_mask) == lir) drow[c] = element(c, orow[c]);
+    const int tail0 = up0 > head ? up0 : head;
+    for (int c = tail0; c < n_vec * V; ++c)
+      if (((c / V) & lpr_mask) == lir) drow[c] = element(c, orow[c]);
   }
   // what is left of a row that is not a whole number of vectors, one element per lane
   for (int c = n_vec * V + lir; c < W; c += (1 << pl.lpr_log2)) drow[c] = element(c, orow[c]);
