@@ -698,7 +698,7 @@ template <int DT>
 __global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
                                                         typename Arith<DT>::T* __restrict__ dst,
                                                         const typename Arith<DT>::T* __restrict__ own,
-                                                        Geom g, RowPlan pl) {
+                                                        Geom g, RowPlan pl, bool defer_border) {
   typedef typename Arith<DT>::T T;
   constexpr int V = Bits<T>::V;
   constexpr T ABS = (T)(~(T(1) << (sizeof(T) * 8 - 1)));
@@ -719,7 +719,11 @@ __global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
   const bool row_plain = (d >= g.hi[0]) && (d < D - g.lo[0]) && (h >= g.hi[1]) && (h < H - g.lo[1]);
   const T* orow = own + ((p * Da + (d + g.lo[0])) * Ha + (h + g.lo[1])) * (long long)Wa + g.lo[2];
   T* drow = dst + (long long)row * W;
-  if (!row_plain) {
+  // defer_border: such a row only gets `0 + own` here, like the columns of a plain row that no
+  // neighbour reaches, and fold_border_rows_kernel sums it in full afterwards, a whole wavefront
+  // per row (in a volume every eighth wavefront of this kernel holds such a row and would walk
+  // the long path with a few lanes active).
+  if (!row_plain && !defer_border) {
     const int n_vec = W / V;
     for (int j = lir; j < n_vec; j += (1 << pl.lpr_log2)) fold_span<DT>(drow, orow, g, p, d, h, j * V, V);
     if (lir == 0 && n_vec * V < W) fold_span<DT>(drow, orow, g, p, d, h, n_vec * V, W - n_vec * V);
@@ -732,6 +736,7 @@ __global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
   const T* s_hi = static_cast<const T*>(table_entry(9 + 3 + 2));
   if (s_lo != nullptr) s_lo += (long long)row * g.hi[2];
   if (s_hi != nullptr) s_hi += (long long)row * g.lo[2];
+  if (!row_plain) s_lo = s_hi = nullptr;  // deferred: no neighbour's term here
   const int up0 = W - g.lo[2];  // first column the upper neighbour reaches
   auto element = [&](int c, T own_bits) {
     float acc = 0.0f;
@@ -1183,6 +1188,43 @@ extern "C" int jg_halo_pack_2d(void* const strips[9], const void* src, int64_t p
   return jg_halo_pack_3d(t, src, &g, from_padded, elem_size, stream);
 }
 
+namespace {
+// Plan of the two in-place border kernels; false when the counts do not fit their 32-bit indices.
+bool border_plan(const Geom& g, BorderPlan* bp, unsigned long long* row_items, unsigned long long* col_items) {
+  const int D = g.n[0], H = g.n[1], W = g.n[2];
+  const unsigned long long nrows = (unsigned long long)g.planes * D * H;
+  bp->nbd = (g.hi[0] + g.lo[0] >= D) ? D : g.hi[0] + g.lo[0];
+  bp->nbh = (g.hi[1] + g.lo[1] >= H) ? H : g.hi[1] + g.lo[1];
+  bp->rows_per_plane = (uint32_t)bp->nbd * (uint32_t)H + (uint32_t)(D - bp->nbd) * (uint32_t)bp->nbh;
+  const int up0 = W - g.lo[2];
+  bp->head = g.hi[2] < up0 ? g.hi[2] : up0;
+  bp->n_edge = bp->head + (W - up0);
+  bp->div_rows = make_magic(bp->rows_per_plane > 0 ? bp->rows_per_plane : 1);
+  bp->div_h = make_magic((uint32_t)H);
+  bp->div_nbh = make_magic((uint32_t)(bp->nbh > 0 ? bp->nbh : 1));
+  bp->div_edge = make_magic((uint32_t)(bp->n_edge > 0 ? bp->n_edge : 1));
+  bp->div_hh = make_magic((uint32_t)H);
+  bp->div_d = make_magic((uint32_t)D);
+  *row_items = (unsigned long long)g.planes * bp->rows_per_plane;
+  *col_items = nrows * (unsigned long long)bp->n_edge;
+  return *row_items < (1ull << 31) && *col_items < (1ull << 31) && nrows < (1ull << 31);
+}
+// The rows a D or H neighbour reaches, summed in full in place; false if there are too many.
+template <int DT>
+bool launch_border_rows(const Table& tab, void* gx, const Geom& g, BorderPlan bp, unsigned long long row_items, hipStream_t s) {
+  typedef typename Arith<DT>::T T;
+  if (row_items == 0) return true;
+  bp.total = (uint32_t)row_items;
+  const int vecs = g.n[2] / (16 / (int)sizeof(T));
+  bp.lpr = 1;
+  while (bp.lpr < 64 && bp.lpr < vecs) bp.lpr *= 2;
+  const unsigned long long threads = row_items * (unsigned long long)bp.lpr;
+  if (threads >= (1ull << 32)) return false;
+  fold_border_rows_kernel<DT><<<(unsigned)((threads + 255) / 256), 256, 0, s>>>(tab, static_cast<T*>(gx), g, bp);
+  return true;
+}
+}  // namespace
+
 extern "C" int jg_halo_fold_3d(void* gx, const void* gx_aug, const void* const strips[27],
                                const jg_halo_geom* geom, int dtype, void* stream) {
   int rc = check_geom(geom, "jg_halo_fold_3d", true);
@@ -1213,12 +1255,30 @@ extern "C" int jg_halo_fold_3d(void* gx, const void* gx_aug, const void* const s
   if ((g.n[2] * es) % 4 == 0 &&
       make_plan((unsigned long long)g.planes * g.n[0] * g.n[1], (g.n[2] + V - 1) / V, g.n[1], g.n[0], &pl)) {
     const unsigned blocks = (unsigned)((((unsigned long long)pl.nrows << pl.lpr_log2) + 255) / 256);
-    if (dtype == JG_F32)
-      fold_rows_kernel<JG_F32><<<blocks, 256, 0, s>>>(tab, static_cast<uint32_t*>(gx), static_cast<const uint32_t*>(gx_aug), g, pl);
-    else if (dtype == JG_BF16)
-      fold_rows_kernel<JG_BF16><<<blocks, 256, 0, s>>>(tab, static_cast<uint16_t*>(gx), static_cast<const uint16_t*>(gx_aug), g, pl);
-    else
-      fold_rows_kernel<JG_F16><<<blocks, 256, 0, s>>>(tab, static_cast<uint16_t*>(gx), static_cast<const uint16_t*>(gx_aug), g, pl);
+    // Two launches when the rows a D or H neighbour reaches are many enough to matter (more than one
+    // row in 64) and fit the border kernel's indices: the row pass defers them, the border kernel
+    // sums them in place from the `0 + own` the row pass left (the same bits: the ordered sum starts
+    // from zero, so the sign of a zero in the own term cannot reach the result).
+    BorderPlan bp;
+    unsigned long long row_items = 0, col_items = 0;
+    const bool planned = border_plan(g, &bp, &row_items, &col_items);
+    const int vecs = g.n[2] / V;
+    int border_lpr = 1;
+    while (border_lpr < 64 && border_lpr < vecs) border_lpr *= 2;
+    const bool defer = planned && row_items * 64 > (unsigned long long)pl.nrows &&
+                       row_items * (unsigned long long)border_lpr < (1ull << 32);
+    bool ok = true;
+    if (dtype == JG_F32) {
+      fold_rows_kernel<JG_F32><<<blocks, 256, 0, s>>>(tab, static_cast<uint32_t*>(gx), static_cast<const uint32_t*>(gx_aug), g, pl, defer);
+      if (defer) ok = launch_border_rows<JG_F32>(tab, gx, g, bp, row_items, s);
+    } else if (dtype == JG_BF16) {
+      fold_rows_kernel<JG_BF16><<<blocks, 256, 0, s>>>(tab, static_cast<uint16_t*>(gx), static_cast<const uint16_t*>(gx_aug), g, pl, defer);
+      if (defer) ok = launch_border_rows<JG_BF16>(tab, gx, g, bp, row_items, s);
+    } else {
+      fold_rows_kernel<JG_F16><<<blocks, 256, 0, s>>>(tab, static_cast<uint16_t*>(gx), static_cast<const uint16_t*>(gx_aug), g, pl, defer);
+      if (defer) ok = launch_border_rows<JG_F16>(tab, gx, g, bp, row_items, s);
+    }
+    JG_REQUIRE(ok, "jg_halo_fold_3d: too many border rows");
     JG_CHECK_LAUNCH("jg_halo_fold_3d");
     return JG_OK;
   }
@@ -1264,34 +1324,13 @@ extern "C" int jg_halo_fold_border_3d(void* gx, const void* const strips[27],
   if (nrows == 0 || W == 0) return JG_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   BorderPlan bp;
-  bp.nbd = (g.hi[0] + g.lo[0] >= D) ? D : g.hi[0] + g.lo[0];
-  bp.nbh = (g.hi[1] + g.lo[1] >= H) ? H : g.hi[1] + g.lo[1];
-  bp.rows_per_plane = (uint32_t)bp.nbd * (uint32_t)H + (uint32_t)(D - bp.nbd) * (uint32_t)bp.nbh;
-  const int up0 = W - g.lo[2];
-  bp.head = g.hi[2] < up0 ? g.hi[2] : up0;
-  bp.n_edge = bp.head + (W - up0);
-  bp.div_rows = make_magic(bp.rows_per_plane);
-  bp.div_h = make_magic((uint32_t)H);
-  bp.div_nbh = make_magic((uint32_t)(bp.nbh > 0 ? bp.nbh : 1));
-  bp.div_edge = make_magic((uint32_t)(bp.n_edge > 0 ? bp.n_edge : 1));
-  bp.div_hh = make_magic((uint32_t)H);
-  bp.div_d = make_magic((uint32_t)D);
-  const unsigned long long row_items = (unsigned long long)g.planes * bp.rows_per_plane;
-  const unsigned long long col_items = nrows * (unsigned long long)bp.n_edge;
-  JG_REQUIRE(row_items < (1ull << 31) && col_items < (1ull << 31) && nrows < (1ull << 31),
-             "jg_halo_fold_border_3d: too many rows (%llu)", nrows);
+  unsigned long long row_items = 0, col_items = 0;
+  JG_REQUIRE(border_plan(g, &bp, &row_items, &col_items), "jg_halo_fold_border_3d: too many rows (%llu)", nrows);
 #define JG_BORDER(DT)                                                                                   \
   do {                                                                                                  \
     typedef Arith<DT>::T T;                                                                             \
-    if (row_items > 0) {                                                                                \
-      bp.total = (uint32_t)row_items;                                                                   \
-      const int vecs = W / (16 / (int)sizeof(T));                                                       \
-      bp.lpr = 1;                                                                                       \
-      while (bp.lpr < 64 && bp.lpr < vecs) bp.lpr *= 2;                                                 \
-      const unsigned long long threads = row_items * (unsigned long long)bp.lpr;                        \
-      JG_REQUIRE(threads < (1ull << 32), "jg_halo_fold_border_3d: too many border rows (%llu)", row_items); \
-      fold_border_rows_kernel<DT><<<(unsigned)((threads + 255) / 256), 256, 0, s>>>(tab, static_cast<T*>(gx), g, bp); \
-    }                                                                                                   \
+    JG_REQUIRE(launch_border_rows<DT>(tab, gx, g, bp, row_items, s),                                    \
+               "jg_halo_fold_border_3d: too many border rows (%llu)", row_items);                      \
     if (col_items > 0) {                                                                                \
       bp.total = (uint32_t)col_items;                                                                   \
       fold_border_cols_kernel<DT><<<(unsigned)((col_items + 255) / 256), 256, 0, s>>>(tab, static_cast<T*>(gx), g, bp); \
