@@ -219,3 +219,37 @@ def test_gelu_mlp_fused_epilogues(rows, dim, hid, with_res, dev):
     if with_res:
         y2 = gres.detach() + y2
     assert rel_l2(out, y2) < 1e-2
+
+
+def test_fused_projection_entry_refuses_what_it_has_no_kernel_for(dev):
+    """jg_proj_nt_fused: an unknown epilogue code and a missing aux tensor are bad arguments
+    (ValueError), operands other than bf16 are not supported (NotImplementedError); the host
+    function gelu_mlp then takes the separate-steps route by itself."""
+    from jigsaw_amd import _lib
+
+    x = torch.randn(16, 64, device=dev).bfloat16()
+    w = torch.randn(32, 64, device=dev).bfloat16()
+    out, aux = torch.empty(16, 32, device=dev).bfloat16(), torch.empty(16, 32, device=dev).bfloat16()
+    lib = _lib.load()
+
+    def call(epi, a=x, wt=w, o=out, au=aux):
+        return lib.jg_proj_nt_fused(_lib.ptr(o), _lib.ptr(au), epi, _lib.ptr(a), _lib.ptr(wt), None,
+                                    _lib.dtype_code(a.dtype), 16, 32, 64, _lib.stream_ptr(dev))
+
+    with pytest.raises(ValueError):
+        _lib.check(call(9), "jg_proj_nt_fused")
+    with pytest.raises(ValueError):
+        _lib.check(call(jp.EPI_ADD, au=None), "jg_proj_nt_fused")
+    with pytest.raises(NotImplementedError):
+        _lib.check(call(jp.EPI_GELU, a=x.float(), wt=w.float(), o=out.float(), au=aux.float()), "jg_proj_nt_fused")
+    assert _lib.check(call(jp.EPI_GELU), "jg_proj_nt_fused") is None
+    torch.cuda.synchronize()
+    want = torch.nn.functional.gelu((x.float() @ w.float().T).bfloat16().float())
+    assert rel_l2(aux, want) < 1e-2
+    # fp32 tokens: not fusable, same function through separate steps
+    xf = torch.randn(4, 64, device=dev)
+    w2 = torch.randn(64, 32, device=dev)
+    assert not jp.mlp_fusable(xf, w.float(), w2, None)
+    y = jp.gelu_mlp(xf, w.float(), None, w2, None)
+    ref = torch.nn.functional.linear(torch.nn.functional.gelu(torch.nn.functional.linear(xf, w.float())), w2)
+    assert rel_l2(y, ref) < 1e-5
