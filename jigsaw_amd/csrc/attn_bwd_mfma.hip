@@ -114,6 +114,24 @@ __device__ __forceinline__ bf16x8 pack8(const float* e) {
   return pk;
 }
 
+// Workgroup -> (batch entry, row block). Consecutive workgroup ids go to the 8 XCDs in turn; each
+// XCD is given a contiguous range of (batch entry, block) pairs, so the workgroups that stream the
+// same K / V (or Q / dO) share one L2 instead of every L2 holding every head. Falls back to the
+// plain order when the count does not divide.
+struct BlockOf {
+  long long bh;
+  int blk;
+};
+__device__ __forceinline__ BlockOf block_of() {
+  const unsigned nblk = gridDim.x, total = gridDim.x * gridDim.y;
+  unsigned id = blockIdx.y * gridDim.x + blockIdx.x;
+  if ((total & 7u) == 0) id = (id & 7u) * (total >> 3) + (id >> 3);
+  BlockOf b;
+  b.bh = id / nblk;
+  b.blk = (int)(id % nblk);
+  return b;
+}
+
 struct BwdArgs {
   const uint16_t* dout;
   const uint16_t* q;
@@ -146,8 +164,9 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
   const int lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, kg = lane >> 5;
   const int qb = wave & 3, ks = wave >> 2;
-  const long long b = blockIdx.y;
-  const int q0 = blockIdx.x * BR + qb * 32;
+  const BlockOf where = block_of();
+  const long long b = where.bh;
+  const int q0 = where.blk * BR + qb * 32;
   const int khalf = p.sk >> 1;
   const int ntiles = khalf / BT;
   const float c2 = p.scale * LOG2E;
@@ -326,17 +345,30 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
 constexpr int DKV_STATS = 2 * BT * 4;                 // lse2[64], delta[64] as floats
 constexpr int DKV_HALF = 2 * NAT + DKV_STATS;         // Q tile, dO tile + stats
 constexpr int DKV_LDS = 4 * DKV_HALF;                 // 67584: two query halves, double buffered
-static_assert(DKV_LDS >= 4 * 64 * 64 * 4, "the hand-over of the partial dK / dV reuses the tile buffers");
+// Key blocks per workgroup. With 2 (4 wavefronts, 64 keys) a launch has twice the workgroups, two of
+// which share a CU: the two wavefronts of a SIMD then belong to different workgroups and do not
+// march in step (the barrier per tile keeps the wavefronts of ONE workgroup in the same phase:
+// all in their matrix instructions, then all in their exponentials).
+#ifndef JG_DKV_KB
+#define JG_DKV_KB 4
+#endif
+constexpr int DKV_KB = JG_DKV_KB;
+constexpr int DKV_THREADS = 64 * 2 * DKV_KB;
+constexpr int DKV_ROWS = 32 * DKV_KB;                 // keys per workgroup
+constexpr int DKV_SHARE = BT / DKV_KB;                // rows of a streamed tile each wavefront of a half moves
+static_assert(DKV_LDS >= DKV_KB * 64 * 64 * 4, "the hand-over of the partial dK / dV reuses the tile buffers");
+static_assert(64 * DKV_KB >= 2 * BT, "one thread of a half per statistic");
 
-__global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
+__global__ __launch_bounds__(DKV_THREADS, 8 / (2 * DKV_KB) >= 2 ? 2 : 1) void attn_bwd_dkv_kernel(BwdArgs p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, kg = lane >> 5;
-  const int kb = wave & 3, qs = wave >> 2;
-  const int th = tid & 255;
-  const long long b = blockIdx.y;
-  const int k0 = blockIdx.x * BR + kb * 32;
+  const int kb = wave % DKV_KB, qs = wave / DKV_KB;
+  const int th = tid % (64 * DKV_KB);
+  const BlockOf where = block_of();
+  const long long b = where.bh;
+  const int k0 = where.blk * DKV_ROWS + kb * 32;
   const int qhalf = p.sq >> 1;
   const int ntiles = qhalf / BT;
   const float c2 = p.scale * LOG2E;
@@ -344,23 +376,24 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkv_kernel(BwdArgs p) {
 
   unsigned char* lds = smem + qs * (2 * DKV_HALF);  // two buffers: Q tile, dO tile, stats
   const long long qrow0 = b * p.sq + (long long)qs * qhalf;
-  // this wavefront moves rows 16 kb .. 16 kb + 15 of the Q tile and of the dO tile of its half
+  // this wavefront moves its share of the rows of the Q tile and of the dO tile of its half
   const int qs_u = __builtin_amdgcn_readfirstlane(qs), kb_u = __builtin_amdgcn_readfirstlane(kb);
   const long long qrow0_u = b * p.sq + (long long)qs_u * qhalf;
-  const char* qdma = reinterpret_cast<const char*>(p.q + qrow0_u * D) + 16 * kb_u * ROWB;
-  const char* ddma = reinterpret_cast<const char*>(p.dout + qrow0_u * D) + 16 * kb_u * ROWB;
+  const char* qdma = reinterpret_cast<const char*>(p.q + qrow0_u * D) + DKV_SHARE * kb_u * ROWB;
+  const char* ddma = reinterpret_cast<const char*>(p.dout + qrow0_u * D) + DKV_SHARE * kb_u * ROWB;
   const uint32_t dma_off = dma_lane_offset(lane);
-  const uint32_t lds_dma = lds_address(smem) + (uint32_t)(qs_u * (2 * DKV_HALF) + 16 * kb_u * ROWB);
+  const uint32_t lds_dma = lds_address(smem) + (uint32_t)(qs_u * (2 * DKV_HALF) + DKV_SHARE * kb_u * ROWB);
   const int tr_off[2] = {tr_lane_offset(lane, 0), tr_lane_offset(lane, 1)};
 
   float st_reg = 0.0f;
   auto issue_loads = [&](int t, int buf) {
     const long long off = (long long)t * NAT;
     const uint32_t dst = lds_dma + (uint32_t)(buf * DKV_HALF);
-    dma_1k(qdma + off, dma_off, dst);
-    dma_1k(qdma + off + 8 * ROWB, dma_off, dst + 8 * ROWB);
-    dma_1k(ddma + off, dma_off, dst + NAT);
-    dma_1k(ddma + off + 8 * ROWB, dma_off, dst + NAT + 8 * ROWB);
+#pragma unroll
+    for (int r = 0; r < DKV_SHARE; r += 8) {
+      dma_1k(qdma + off + r * ROWB, dma_off, dst + r * ROWB);
+      dma_1k(ddma + off + r * ROWB, dma_off, dst + NAT + r * ROWB);
+    }
     // One plain load for every lane, used only when the statistics go to LDS: a load under a
     // per-lane condition, or arithmetic on its result here, would make the wavefront wait
     // for it (and for the transfers issued before it) on the spot.
@@ -501,7 +534,7 @@ namespace jg {
 
 bool attn_mfma_bwd_supported(long long batch, int sq, int sk, int d, int dtype, bool has_bias) {
   return dtype == JG_BF16 && !has_bias && d == D && sq > 0 && sk > 0 && sq % BR == 0 &&
-         sk % BR == 0 && batch > 0 && batch <= 65535;
+         sk % BR == 0 && sk % DKV_ROWS == 0 && batch > 0 && batch <= 65535;
 }
 
 size_t attn_mfma_bwd_workspace(long long batch, int sq, int) {
@@ -537,7 +570,7 @@ int attn_mfma_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q,
   }
   attn_bwd_dq_kernel<<<dim3((unsigned)(sq / BR), (unsigned)batch, 1), THREADS, DQ_LDS, s>>>(a);
   JG_CHECK_LAUNCH("jg_attn_bwd(dq)");
-  attn_bwd_dkv_kernel<<<dim3((unsigned)(sk / BR), (unsigned)batch, 1), THREADS, DKV_LDS, s>>>(a);
+  attn_bwd_dkv_kernel<<<dim3((unsigned)(sk / DKV_ROWS), (unsigned)batch, 1), DKV_THREADS, DKV_LDS, s>>>(a);
   JG_CHECK_LAUNCH("jg_attn_bwd(dkv)");
   return JG_OK;
 }

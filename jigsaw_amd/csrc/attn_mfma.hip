@@ -99,6 +99,24 @@ __device__ __forceinline__ void pair32(float v, float& a, float& b) {
   b = __uint_as_float(sw[1]);
 }
 
+// Workgroup -> (batch entry, row block). Consecutive workgroup ids go to the 8 XCDs in turn; each
+// XCD is given a contiguous range of (batch entry, block) pairs, so the workgroups that stream the
+// same K / V (or Q / dO) share one L2 instead of every L2 holding every head. Falls back to the
+// plain order when the count does not divide.
+struct BlockOf {
+  long long bh;
+  int blk;
+};
+__device__ __forceinline__ BlockOf block_of() {
+  const unsigned nblk = gridDim.x, total = gridDim.x * gridDim.y;
+  unsigned id = blockIdx.y * gridDim.x + blockIdx.x;
+  if ((total & 7u) == 0) id = (id & 7u) * (total >> 3) + (id >> 3);
+  BlockOf b;
+  b.bh = id / nblk;
+  b.blk = (int)(id % nblk);
+  return b;
+}
+
 __global__ __launch_bounds__(THREADS) void attn_fwd_mfma_kernel(FwdArgs p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x;
@@ -106,8 +124,9 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_mfma_kernel(FwdArgs p) {
   const int ln = lane & 31, kg = lane >> 5;
   const int qg = wave & 1, kq = wave >> 1;
   const int th = tid & 127;  // thread index inside the key quarter
-  const long long b = blockIdx.y;
-  const int q0 = blockIdx.x * BM + qg * 64;
+  const BlockOf where = block_of();
+  const long long b = where.bh;
+  const int q0 = where.blk * BM + qg * 64;
   const int kquarter = p.sk >> 2;
   const int ntiles = kquarter / BN;
   const float c2 = p.scale * 1.4426950408889634f;  // scores are handled in base 2
@@ -408,7 +427,7 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_mfma_kernel(FwdArgs p) {
       const float inv = 1.0f / lt[qb];
       const float lse_j = (m[qb] * c2 + log2f(lt[qb])) * 0.6931471805599453f;  // natural log
       const int ql = qg * 64 + qb * 32 + ln;  // query inside the workgroup
-      const long long qi = b * p.sq + blockIdx.x * BM + ql;
+      const long long qi = b * p.sq + where.blk * BM + ql;
       if (kg == 0) {
         float w = 0.0f;
         if (p.out_acc != nullptr) {
@@ -434,7 +453,7 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_mfma_kernel(FwdArgs p) {
   }
   __syncthreads();
   {
-    const long long row0 = b * p.sq + (long long)blockIdx.x * BM;
+    const long long row0 = b * p.sq + (long long)where.blk * BM;
     f32x4 hv[4], acc[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {  // piece e = tid + 512 i of the 128 x 16 pieces of 4 floats
