@@ -89,6 +89,11 @@ struct FwdParams {
   int Din, Hin, Win, Dout, Hout, Wout;
   int pad_d, pad_h, pad_w;  // virtual zero padding of x
   int tiles_h, tiles_w;
+  // Tile column tw covers produced columns [org_w + tw * TW, + TW), org_w <= 0: the host shifts the
+  // grid to put the staged row segments on cache-line boundaries where that is free.
+  // The staged window starts `lead` (0 / 1) pixels before the first one a tile needs, so that its
+  // rows stay 4-byte aligned whatever the parity of pad_w - org_w.
+  int org_w, lead;
   int sw;               // tile order inside a plane: row-major inside bands of sw tile columns, band after band
   int total_tiles;      // N * Dout * tiles_h * tiles_w
   int nc16;             // KD * Cp / 16
@@ -256,7 +261,10 @@ __device__ inline void store_bf16_hi(const void* base, uint32_t lane_off, uint32
   asm volatile("global_store_short_d16_hi %0, %1, %2" : : "v"(lane_off), "v"(pair), "s"(base) : "memory");
 }
 __device__ inline void store_16_bytes(const void* base, uint32_t lane_off, u32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, %2" : : "v"(lane_off), "v"(v), "s"(base) : "memory");
+  // The store reads its 16 bytes of data from the registers a little after it issues; a vector
+  // instruction that overwrites them within two wait states would be stored instead. The
+  // compiler pads that for its own stores but does not look inside an asm statement.
+  asm volatile("global_store_dwordx4 %0, %1, %2\n\ts_nop 1" : : "v"(lane_off), "v"(v), "s"(base) : "memory");
 }
 __device__ inline void store_f32(const void* base, uint32_t lane_off, float v) {
   asm volatile("global_store_dword %0, %1, %2" : : "v"(lane_off), "v"(v), "s"(base) : "memory");
@@ -354,36 +362,75 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     return c;
   };
 
-  auto issue_loads = [&](int tile, int c16) {
-    const TileCoord tc = coord(tile);
-    const int per_blk = p.nc16 / p.nblk;  // 16-channel steps of one contraction block
-    const int blk = c16 / per_blk, inner = (c16 - blk * per_blk) * CK;
-    const int kd = inner / p.Cp, c0 = inner - kd * p.Cp;
-    const int cx0 = (int)((p.xmap >> (2 * blk)) & 3u) * p.C + c0;  // first channel of the step in x
+  // ---- load cursor: the (tile, 16-channel step) whose loads are issued next; it runs two stages
+  // ahead of the MFMAs. Everything that takes a division (the tile's coordinates) is done when
+  // the cursor enters a tile; inside a tile the step moves by additions.
+  struct Cursor {
+    int ti;          // index into this workgroup's tiles
+    int blk, inner;  // contraction block, channel offset inside it (= kd * Cp + c0)
+    int kd, c0;      // depth tap and first channel of the step
+    int od;          // produced depth plane of the tile
+    int ih0, iw0;    // window origin in the input plane
+    bool window_in;  // rows and columns of the window lie inside the plane
+    bool window_in_t;  // ... inside the rank's own tile (framed input)
+    const char* base;    // window origin in channel 0 of the batch entry, depth plane 0
+    const char* base_t;  // the same in the rank's own tile (framed input)
+  } cur;
+  const int per_blk_ch = (p.nc16 / p.nblk) * CK;  // contraction channels (x depth taps) of one block
+  auto cursor_enter = [&](int ti) __attribute__((always_inline)) {
+    cur.ti = ti;
+    cur.blk = 0; cur.inner = 0; cur.kd = 0; cur.c0 = 0;
+    if (ti >= my_tiles) return;
+    const TileCoord tc = coord(tile_of(ti));
+    cur.od = tc.od;
+    cur.ih0 = tc.th * TH - p.pad_h;
+    cur.iw0 = tc.tw * TW + p.org_w - p.pad_w - p.lead;
+    cur.window_in = cur.ih0 >= 0 && cur.ih0 + IN_ROWS <= p.Hin && cur.iw0 >= 0 && cur.iw0 + p.lead + TW + KW - 1 <= p.Win;
+    cur.base = reinterpret_cast<const char*>(p.x) +
+               2 * ((ptrdiff_t)((size_t)tc.n * p.Cx * chan_stride) + (ptrdiff_t)cur.ih0 * p.Win + cur.iw0);
+    if (FRAMED) {
+      const int ht = cur.ih0 - p.tlo_h, wt = cur.iw0 - p.tlo_w;
+      cur.window_in_t = ht >= 0 && ht + IN_ROWS <= p.tn_h && wt >= 0 && wt + p.lead + TW + KW - 1 <= p.tn_w;
+      cur.base_t = reinterpret_cast<const char*>(p.xt) +
+                   2 * ((ptrdiff_t)((size_t)tc.n * p.Cx * chan_stride_t) + (ptrdiff_t)ht * p.tn_w + wt);
+    }
+  };
+  auto cursor_advance = [&]() __attribute__((always_inline)) {
+    cur.inner += CK;
+    cur.c0 += CK;
+    if (cur.c0 >= p.Cp) {
+      cur.c0 = 0;
+      ++cur.kd;
+    }
+    if (cur.inner == per_blk_ch) {
+      cur.inner = 0; cur.kd = 0; cur.c0 = 0;
+      if (++cur.blk == p.nblk) cursor_enter(cur.ti + 1);
+    }
+  };
+
+  // Loads of the stage under the cursor.
+  auto issue_loads = [&]() __attribute__((always_inline)) {
+    const int kd = cur.kd, c0 = cur.c0;
+    const int cx0 = (int)((p.xmap >> (2 * cur.blk)) & 3u) * p.C + c0;  // first channel of the step in x
     // Channels of this task that exist (all 8 unless C is not a multiple of 16). The vector
     // path below reads the others anyway (they lie inside the tensor: the interior test covers
     // all 16 channel planes) and store_stage zeroes them; the guarded paths skip them.
     const int cvalid = p.C - c0 - g8 * 8;
-    const int id = tc.od + kd - p.pad_d;
-    const int ih0 = tc.th * TH - p.pad_h, iw0 = tc.tw * TW - p.pad_w;
+    const int id = cur.od + kd - p.pad_d;
+    const int ih0 = cur.ih0, iw0 = cur.iw0;
     const bool depth_ok = id >= 0 && id < p.Din;
     // wave-uniform origin of the stage window (lies before the tensor where padded)
-    const char* origin = reinterpret_cast<const char*>(p.x) +
-                         2 * ((ptrdiff_t)(((size_t)tc.n * p.Cx + cx0) * chan_stride) +
-                              (ptrdiff_t)id * (ptrdiff_t)plane + (ptrdiff_t)ih0 * p.Win + iw0);
+    const char* origin = cur.base + 2 * ((ptrdiff_t)((size_t)cx0 * chan_stride) + (ptrdiff_t)id * (ptrdiff_t)plane);
     // The last octet of a row holds 2 pixels that are used and 6 that no fragment
     // reads, so it may run past the row end as long as it stays inside the tensor.
     const char* last = origin + 2 * ((size_t)(CK - 1) * chan_stride + (size_t)(IN_ROWS - 1) * p.Win + OCTS * 8);
-    const bool interior = depth_ok && ih0 >= 0 && ih0 + IN_ROWS <= p.Hin && iw0 >= 0 &&
-                          iw0 + TW + KW - 1 <= p.Win && last <= p.x_end;
+    const bool interior = depth_ok && cur.window_in && last <= p.x_end;
     if (FRAMED) {
       // window inside the own tile (wave-uniform): read the tile itself, at whatever
       // alignment its rows give the window
-      const int dt = id - p.tlo_d, ht = ih0 - p.tlo_h, wt = iw0 - p.tlo_w;
-      const char* origin_t = reinterpret_cast<const char*>(p.xt) +
-                             2 * ((ptrdiff_t)(((size_t)tc.n * p.Cx + cx0) * chan_stride_t) +
-                                  (ptrdiff_t)dt * (ptrdiff_t)plane_t + (ptrdiff_t)ht * p.tn_w + wt);
-      if (dt >= 0 && dt < p.tn_d && ht >= 0 && ht + IN_ROWS <= p.tn_h && wt >= 0 && wt + TW + KW - 1 <= p.tn_w) {
+      const int dt = id - p.tlo_d;
+      const char* origin_t = cur.base_t + 2 * ((ptrdiff_t)((size_t)cx0 * chan_stride_t) + (ptrdiff_t)dt * (ptrdiff_t)plane_t);
+      if (dt >= 0 && dt < p.tn_d && cur.window_in_t) {
         if (!has_task) return;
         // 4-byte aligned accesses only (2-byte aligned vector loads run at a fraction of the
         // rate): a window that starts on an odd column is read one pixel early and shifted.
@@ -483,10 +530,10 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     }
   };
 
-  auto store_stage = [&](int buf, int c16) {
+  auto store_stage = [&](int buf, int stage) {  // stage: counted over this workgroup's tiles
     if (!has_task) return;
     if (p.Cp != p.C) {  // uniform: zero the channels of this step that do not exist
-      const int cvalid = p.C - (c16 * CK) % p.Cp - g8 * 8;
+      const int cvalid = p.C - ((stage % p.nc16) * CK) % p.Cp - g8 * 8;
 #pragma unroll
       for (int c = 0; c < 8; ++c)
         if (c >= cvalid) {
@@ -509,26 +556,39 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
 
   f32x16 acc[CB][WROWS];
 
-  // One third (one kw) of a stage's MFMAs.
-  auto compute_kw = [&](int buf, int c16, int kw) {
-    const u32x4* in = lds_in + buf * STAGE_SLOTS + kg * (IN_ROWS * ROW_SLOTS);
-    const u32x4* wt = lds_w + ((size_t)(c16 % p.wc16) * 2 + kg) * MT + ln;
-    bf16x8 a[KH][CB];
+  // One third (one kw) of a stage's MFMAs. The fragments roll through the stage: the weight
+  // fragments of tap row kh are last used by input row kh + WROWS - 1 of the group, and the
+  // same registers are refilled right there with the next group's fragments (the next kw, or
+  // after the last kw the first group of the next stage: the weights do not change at the
+  // barrier), and the group's last step requests the first input fragment of the next kw. So
+  // only the first input fragment of a stage is waited for with nothing else to issue.
+  bf16x8 a[KH][CB];
+  u32x4 bnext;
+  int a_step = -1;  // the step inside the weight group whose kw = 0 fragments `a` holds
+  auto weight_frag = [&](int wstep, int kh, int kw, int cb) {
+    const u32x4* wt = lds_w + ((size_t)wstep * 2 + kg) * MT + ln;
+    return __builtin_bit_cast(bf16x8, wt[(size_t)(kh * KW + kw) * p.wc16 * 2 * MT + cb * 32]);
+  };
+  auto compute_kw = [&](int buf, int wstep, int kw, int wstep_next) {  // wstep: the stage's step inside its weight group
+    const u32x4* in = lds_in + buf * STAGE_SLOTS + kg * (IN_ROWS * ROW_SLOTS) + wrow0 * ROW_SLOTS;
+    const int col0 = wcol0 + ln + p.lead;  // the tile's pixel 0 sits `lead` slots into the staged row
+    const u32x4* inb = in + in_slot(col0 + kw);
+    if (kw == 0) {
+      if (a_step != wstep) {  // wave-uniform: the first stage, after a tile without work, after a weight reload
 #pragma unroll
-    for (int kh = 0; kh < KH; ++kh)
+        for (int kh = 0; kh < KH; ++kh)
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) {
-        u32x4 t = wt[(size_t)(kh * KW + kw) * p.wc16 * 2 * MT + cb * 32];
-        a[kh][cb] = __builtin_bit_cast(bf16x8, t);
+          for (int cb = 0; cb < CB; ++cb) a[kh][cb] = weight_frag(wstep, kh, 0, cb);
       }
-    const u32x4* inb = in + wrow0 * ROW_SLOTS + in_slot(wcol0 + ln + kw);
+      bnext = inb[0];
+    }
     // software pipeline over the input rows: the fragment of row rho+1 is requested
     // before the MFMAs of row rho are issued, so its LDS latency hides behind them
-    u32x4 bnext = inb[0];
 #pragma unroll
     for (int rho = 0; rho < WROWS + KH - 1; ++rho) {
       const bf16x8 b = __builtin_bit_cast(bf16x8, bnext);
       if (rho + 1 < WROWS + KH - 1) bnext = inb[(rho + 1) * ROW_SLOTS];
+      else if (kw + 1 < KW) bnext = in[in_slot(col0 + kw + 1)];
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int kh = 0; kh < KH; ++kh) {
@@ -544,7 +604,19 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
         }
       }
       __builtin_amdgcn_sched_barrier(0);
+      const int kh_done = rho - (WROWS - 1);  // this tap row's weights are not read again in this group
+      if (kh_done >= 0) {
+        if (kw + 1 < KW) {
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb) a[kh_done][cb] = weight_frag(wstep, kh_done, kw + 1, cb);
+        } else if (p.ngroups == 1) {
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb) a[kh_done][cb] = weight_frag(wstep_next, kh_done, 0, cb);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
+    if (kw == KW - 1) a_step = p.ngroups == 1 ? wstep_next : -1;
   };
 
   // Accumulator lane (ln, kg), register i of block cb: produced channel
@@ -596,29 +668,30 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     const int l4 = lane >> 2;
     const int m_lane = (l4 & 8) + ((l4 >> 1) & 3) + ((l4 & 1) << 2);
     const uint32_t voff = (uint32_t)(m_lane * chan_bytes) + 16u * (lane & 3) + row_off;
+    // all the row's pieces are requested before the first is stored: one LDS latency per row
+    u32x4 piece[MT / 16];
 #pragma unroll
-    for (int q = 0; q < MT / 16; ++q) {
-      const u32x4 piece = *reinterpret_cast<const u32x4*>(scratch + (q * 64 + lane) * 16);
-      store_16_bytes(ytile + (size_t)q * 16 * chan_bytes, voff, piece);
-    }
+    for (int q = 0; q < MT / 16; ++q) piece[q] = *reinterpret_cast<const u32x4*>(scratch + (q * 64 + lane) * 16);
+#pragma unroll
+    for (int q = 0; q < MT / 16; ++q) store_16_bytes(ytile + (size_t)q * 16 * chan_bytes, voff, piece[q]);
   };
 
-  auto epilogue_rows = [&](int tile, auto ragged, int free_buf) {
+  auto epilogue_rows = [&](const TileCoord& tc, auto ragged, int free_buf) {
     constexpr bool RAGGED = decltype(ragged)::value;
-    const TileCoord tc = coord(tile);
-    const int ow = tc.tw * TW + wcol0 + ln;
-    if (!RAGGED && p.out_kind != 1 && (p.Wout & 7) == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 &&
-        tc.tw * TW + wcol0 + 32 <= p.Wout) {  // wave-uniform
+    const int tw0 = tc.tw * TW + p.org_w;  // first produced column of the tile
+    const int ow = tw0 + wcol0 + ln;
+    if (!RAGGED && p.out_kind != 1 && (p.Wout & 7) == 0 && (tw0 & 7) == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 &&
+        tw0 + wcol0 >= 0 && tw0 + wcol0 + 32 <= p.Wout) {  // wave-uniform
       unsigned char* scratch = reinterpret_cast<unsigned char*>(lds_in + free_buf * STAGE_SLOTS) + wave * (STAGE_BYTES / WAVES);
       char* ytile = reinterpret_cast<char*>(p.y) +
                     2 * (((size_t)tc.n * p.M + (size_t)mt * MT) * (plane_o * p.Dout) + (size_t)tc.od * plane_o +
-                         (size_t)(tc.tw * TW));
+                         (size_t)tw0);
 #pragma unroll
       for (int r = 0; r < WROWS; ++r) {
         const int oh = tc.th * TH + wrow0 + r;
         auto pair = [&](int cb, int i) {
           f32x2 v2 = {acc[cb][r][i], acc[cb][r][i + 1]};
-          return p.out_kind == 2 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, f16x2))
+          return F16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, f16x2))
                                  : __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
         };
         if (oh < p.Hout)
@@ -635,7 +708,7 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
 #pragma unroll
       for (int r = 0; r < WROWS; ++r) {
         const int oh = tc.th * TH + wrow0 + r;
-        if (oh < p.Hout && ow < p.Wout) {
+        if (oh < p.Hout && ow >= 0 && ow < p.Wout) {
           const uint32_t voff = (uint32_t)(4 * ((size_t)(4 * kg) * ochan + (size_t)oh * p.Wout + ow));
 #pragma unroll
           for (int cb = 0; cb < CB; ++cb)
@@ -651,14 +724,14 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
 #pragma unroll
     for (int r = 0; r < WROWS; ++r) {
       const int oh = tc.th * TH + wrow0 + r;
-      if (oh < p.Hout && ow < p.Wout) {
+      if (oh < p.Hout && ow >= 0 && ow < p.Wout) {
         const uint32_t voff = (uint32_t)(2 * ((size_t)(4 * kg) * ochan + (size_t)oh * p.Wout + ow));
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
           for (int i = 0; i < 16; i += 2) {
             f32x2 v2 = {acc[cb][r][i], acc[cb][r][i + 1]};
-            const uint32_t h2 = p.out_kind == 2 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, f16x2))
+            const uint32_t h2 = F16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, f16x2))
                                                 : __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
             const int m0 = cb * 32 + 8 * (i >> 2) + (i & 3);
             if (!RAGGED || m0 < m_left) store_bf16_lo(ybase + (size_t)m0 * ochan * 2, voff, h2);
@@ -667,17 +740,16 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
       }
     }
   };
-  auto epilogue = [&](int tile, int free_buf) {
-    if ((mt + 1) * MT <= p.M) epilogue_rows(tile, std::false_type{}, free_buf);
-    else epilogue_rows(tile, std::true_type{}, free_buf);
+  auto epilogue = [&](const TileCoord& tc, int free_buf) {
+    if ((mt + 1) * MT <= p.M) epilogue_rows(tc, std::false_type{}, free_buf);
+    else epilogue_rows(tc, std::true_type{}, free_buf);
   };
 
   // Fold-mode epilogue: a produced cell goes to the unpadded tile when it lies inside
   // [lo, lo + n) on every axis, else to the strip of the neighbour that owns it (dropped
   // when that neighbour does not exist). Values pass through `0 + v`: the sign of a
   // zero is cleared, as the reference's scatter-add does for every cell.
-  auto epilogue_fold = [&](int tile) {
-    const TileCoord tc = coord(tile);
+  auto epilogue_fold = [&](const TileCoord& tc, int free_buf) {
     // bf16 pairs of the whole accumulator first (the fp32 registers are dead after this).
     // The sign of a zero only matters where a value is zero or rounds to zero, which is
     // rare: one min3 per two values finds out, and only then the bits are patched.
@@ -706,19 +778,33 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
             pk[cb][r][j] = bits;
           }
     }
-    const int ow = tc.tw * TW + wcol0 + ln;
+    const int ow = tc.tw * TW + p.org_w + wcol0 + ln;
     const int hi_d = p.Dout - p.lo_d - p.nD, hi_h = p.Hout - p.lo_h - p.nH, hi_w = p.Wout - p.lo_w - p.nW;
     const int od = tc.od;
     const int rd = od < p.lo_d ? 0 : (od < p.lo_d + p.nD ? 1 : 2);
     const int cd = od - (rd == 0 ? 0 : (rd == 1 ? p.lo_d : p.lo_d + p.nD));
     const int ed = rd == 0 ? p.lo_d : (rd == 1 ? p.nD : hi_d);
     const size_t plane0 = (size_t)tc.n * p.M + (size_t)mt * MT;
-    const int th0 = tc.th * TH, tw0 = tc.tw * TW;
+    const int th0 = tc.th * TH, tw0 = tc.tw * TW + p.org_w;
     // A tile that lies wholly inside the own extent (wave-uniform test): plain rows of
     // the unpadded tile, no per-cell routing.
     if (rd == 1 && th0 >= p.lo_h && th0 + TH <= p.lo_h + p.nH && tw0 >= p.lo_w && tw0 + TW <= p.lo_w + p.nW) {
       const size_t ps = (size_t)p.nD * p.nH * p.nW;
       char* ybase = reinterpret_cast<char*>(p.y) + 2 * (plane0 * ps + (size_t)cd * p.nH * p.nW);
+      if (((tw0 - p.lo_w) & 7) == 0 && (p.nW & 7) == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0) {  // uniform
+        // the tile's rows start on the 16-byte grid of the unpadded tile (the host shifts the tile
+        // grid to make it so): 16-byte stores through this wavefront's slice of the free stage buffer
+        unsigned char* scratch =
+            reinterpret_cast<unsigned char*>(lds_in + free_buf * STAGE_SLOTS) + wave * (STAGE_BYTES / WAVES);
+        char* ytile = ybase + 2 * (ptrdiff_t)(tw0 - p.lo_w);
+#pragma unroll
+        for (int r = 0; r < WROWS; ++r) {
+          const int oh = th0 + wrow0 + r - p.lo_h;
+          auto pair = [&](int cb, int i) { return pk[cb][r][i >> 1]; };
+          row_through_lds(scratch, pair, ytile, (uint32_t)(2 * ((size_t)oh * p.nW + wcol0)), 2 * ps);
+        }
+        return;
+      }
 #pragma unroll
       for (int r = 0; r < WROWS; ++r) {
         const int oh = th0 + wrow0 + r - p.lo_h;
@@ -744,7 +830,7 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
 #pragma unroll
     for (int r = 0; r < WROWS; ++r) {
       const int oh = th0 + wrow0 + r;
-      if (oh >= p.Hout || ow >= p.Wout) continue;
+      if (oh >= p.Hout || ow >= p.Wout || ow < 0) continue;
       const int rh = oh < p.lo_h ? 0 : (oh < p.lo_h + p.nH ? 1 : 2);
       const int ch = oh - (rh == 0 ? 0 : (rh == 1 ? p.lo_h : p.lo_h + p.nH));
       const int eh = rh == 0 ? p.lo_h : (rh == 1 ? p.nH : hi_h);
@@ -770,14 +856,15 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
   // global loads of a stage are issued a whole stage ahead: right after the previous
   // stage's registers were written to LDS, in the middle of the stage before.
   const int stages = my_tiles * p.nc16;
-  auto issue_stage = [&](int q) {
-    const int ti = q / p.nc16;
-    issue_loads(tile_of(ti), q - ti * p.nc16);
+  auto issue_stage = [&]() __attribute__((always_inline)) {
+    issue_loads();
+    cursor_advance();
   };
   int buf = 0;
-  issue_stage(0);
+  cursor_enter(0);
+  issue_stage();
   store_stage(0, 0);
-  if (stages > 1) issue_stage(1);
+  if (stages > 1) issue_stage();
   __syncthreads();
   int q = 0;
   for (int ti = 0; ti < my_tiles; ++ti) {
@@ -785,32 +872,37 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     // a wavefront whose 4 x 32 pixels all lie outside the produced tensor (ragged last tiles) only
     // takes part in the staging and the barriers
     const TileCoord tcur = coord(tile_of(ti));
-    const bool live = tcur.tw * TW + wcol0 < p.Wout && tcur.th * TH + wrow0 < p.Hout;
+    const int wave_col = tcur.tw * TW + p.org_w + wcol0;
+    const bool live = wave_col < p.Wout && wave_col + 32 > 0 && tcur.th * TH + wrow0 < p.Hout;
+    int wstep = 0, wgroup = 0;
     for (int c16 = 0; c16 < p.nc16; ++c16, ++q) {
-      if (p.ngroups > 1 && c16 % p.wc16 == 0) {
+      if (p.ngroups > 1 && wstep == 0) {
         // every wavefront is past the barrier that closed the last stage of the group before
-        load_weights(c16 / p.wc16);
+        load_weights(wgroup);
         __syncthreads();
       }
+      const int wstep_next = wstep + 1 == p.wc16 ? 0 : wstep + 1;
       if (live) {
-        compute_kw(buf, c16, 0);
-        compute_kw(buf, c16, 1);
+        compute_kw(buf, wstep, 0, wstep_next);
+        compute_kw(buf, wstep, 1, wstep_next);
       }
-      if (q + 1 < stages) store_stage(buf ^ 1, c16 + 1 < p.nc16 ? c16 + 1 : 0);  // other buffer: no hazard with this stage's reads
-      if (q + 2 < stages) issue_stage(q + 2);
-      if (live) compute_kw(buf, c16, 2);
+      if (c16 == 0 && ti > 0) __syncthreads();  // the buffer written next was the last epilogue's scratch
+      if (q + 1 < stages) store_stage(buf ^ 1, q + 1);  // other buffer: no hazard with this stage's reads
+      if (q + 2 < stages) issue_stage();
+      if (live) compute_kw(buf, wstep, 2, wstep_next);
       __syncthreads();
       buf ^= 1;
+      if (++wstep == p.wc16) {
+        wstep = 0;
+        ++wgroup;
+      }
     }
-    if (FOLD) {
-      epilogue_fold(tile_of(ti));
-    } else {
-      // the stage buffer the last stage was computed from is free until the next stage is
-      // stored into it: the epilogue stages its rows there, and the barrier keeps a wavefront
-      // that is already in the next tile from storing over them
-      epilogue(tile_of(ti), buf ^ 1);
-      __syncthreads();
-    }
+    // The epilogue stages its rows in the stage buffer the last stage was computed from, which is
+    // free until the next stage is stored into it. That store waits (barrier above, in the first
+    // stage of the next tile) until every wavefront has left this epilogue; until then a
+    // wavefront that is done early already runs the next tile's MFMAs.
+    if (FOLD) epilogue_fold(tcur, buf ^ 1);
+    else epilogue(tcur, buf ^ 1);
   }
 }
 
@@ -960,7 +1052,19 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   p.Dout = L.Dout; p.Hout = L.Hout; p.Wout = L.Wout;
   p.pad_d = L.pad_d; p.pad_h = L.pad_h; p.pad_w = L.pad_w;
   p.tiles_h = (L.Hout + TH - 1) / TH;
-  p.tiles_w = (L.Wout + TW - 1) / TW;
+  // Where to put the tile grid. A tile's staged rows start at input column org_w + TW * tw - pad_w.
+  // When the rows of x are a multiple of 128 bytes apart, an origin that makes this a multiple of
+  // TW puts every staged row segment on a cache-line boundary (144 bytes: two lines instead of
+  // three); it is taken when it costs no extra tile column.
+  p.org_w = 0;
+  // (not where it would take the 16-byte store path away: a plain 16-bit result with rows of whole pieces)
+  const bool wide_rows = !L.fold && L.split != 1 && L.Wout % 8 == 0;
+  if (!wide_rows && L.pad_w % TW != 0 && L.Win % 64 == 0 && (reinterpret_cast<uintptr_t>(x16) & 127) == 0) {
+    const int org = L.pad_w % TW - TW;
+    if ((L.Wout - org + TW - 1) / TW <= (L.Wout + TW - 1) / TW) p.org_w = org;
+  }
+  p.lead = (L.pad_w - p.org_w) & 1;
+  p.tiles_w = (L.Wout - p.org_w + TW - 1) / TW;
   p.sw = p.tiles_w;
   const long long tiles = (long long)L.N * L.Dout * p.tiles_h * p.tiles_w;
   JG_REQUIRE(tiles < (1ll << 30), "%s: too many tiles", who);
@@ -982,8 +1086,8 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   if (wgs > tiles) wgs = (int)tiles;
   wgs = (wgs + 7) & ~7;  // whole XCD rounds
   dim3 grid((unsigned)wgs, (unsigned)lay.mtiles, 1);
-  const bool even = (L.Win % 2 == 0) && (L.pad_w % 2 == 0) &&
-                    ((reinterpret_cast<uintptr_t>(x16) & 3) == 0);
+  // rows of the staged windows start at even columns (`lead` sees to that): 4-byte aligned loads
+  const bool even = (L.Win % 2 == 0) && ((reinterpret_cast<uintptr_t>(x16) & 3) == 0);
   void (*kern)(StripTable, FwdParams) = nullptr;
   if (L.f16 && (L.fold || L.xt != nullptr))
     JG_FAIL(JG_ERR_UNSUPPORTED, "%s: the fold epilogue and the framed input are built for bf16 only", who);
