@@ -25,8 +25,7 @@ from typing import Any, Protocol
 import torch
 
 from . import _lib
-from .halo import HaloGeometry, halo_assemble, halo_fold, halo_fold_border_, halo_pack
-from .halo import slot as halo_slot
+from .halo import HaloGeometry, halo_assemble, halo_fold, halo_fold_border_, halo_pack, new_strips
 
 # --------------------------------------------------------------------------- #
 # local primitives
@@ -387,13 +386,7 @@ def conv_nd_input_fold(geom: HaloGeometry, w, g, *, stride=1, padding=0, dilatio
     ws, nbytes = _workspace(desc, 1, g.dtype, g.device)
     lead = (batch, c_in)
     offs = geom.offsets() if present is None else [tuple(o) for o in present]
-    send: dict = {}
-    tab = _lib.VoidP27()
-    for o in offs:
-        t = torch.empty(lead + geom.strip_extent(o, "pack_bwd"), dtype=g.dtype, device=g.device)
-        send[o] = t
-        if t.numel():
-            tab[halo_slot(o)] = t.data_ptr()
+    send, tab = new_strips(geom, "pack_bwd", lead, offs, g.dtype, g.device)
     gx = torch.empty(lead + geom.size, dtype=g.dtype, device=g.device)
     rc = _lib.load().jg_conv_dgrad_fold(
         _lib.ptr(gx), tab, _lib.ptr(w), _lib.ptr(g), desc, geom.c_geom(batch * c_in), _lib.dtype_code(g.dtype),

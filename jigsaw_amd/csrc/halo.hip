@@ -211,6 +211,48 @@ __global__ __launch_bounds__(256) void pack_kernel(PackArgs a, const T* __restri
   }
 }
 
+// The two faces across W (slots 12 and 14) of a tile whose rows are longer than a cache line:
+// every row gives a few cells from each end, so each face alone touches one line of every row.
+// One thread takes both ends of ROWS rows, 256 rows apart, all loads before the first store: the
+// two lines of a row are asked for together (neighbouring lanes: neighbouring rows, so whole
+// DRAM pages are read in one go instead of half now and half when the other face is packed),
+// and a lane has up to 2 * ROWS * ext loads in flight.
+template <typename T>
+__global__ __launch_bounds__(256) void pack_w_faces_kernel(T* __restrict__ dlo, T* __restrict__ dhi,
+                                                           const T* __restrict__ src, Box blo, Box bhi,
+                                                           unsigned rows, int Sd, int Sh, int Sw) {
+  constexpr int ROWS = 4;
+  const unsigned e0 = (unsigned)blo.ext[0], e1 = (unsigned)blo.ext[1];
+  const int nlo = blo.ext[2], nhi = bhi.ext[2];
+  const unsigned first = blockIdx.x * (256u * ROWS) + threadIdx.x;
+  T vlo[ROWS][2], vhi[ROWS][2];
+#pragma unroll
+  for (int k = 0; k < ROWS; ++k) {
+    const unsigned r = first + 256u * k;
+    if (r < rows) {
+      const unsigned r2 = r / e1, ch = r - r2 * e1;
+      const unsigned pl = r2 / e0, cd = r2 - pl * e0;
+      const T* row = src + (((size_t)pl * Sd + (blo.org[0] + cd)) * Sh + (blo.org[1] + ch)) * (size_t)Sw;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (j < nlo) vlo[k][j] = row[blo.org[2] + j];
+        if (j < nhi) vhi[k][j] = row[bhi.org[2] + j];
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < ROWS; ++k) {
+    const unsigned r = first + 256u * k;
+    if (r < rows) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (j < nlo) dlo[(size_t)r * nlo + j] = vlo[k][j];
+        if (j < nhi) dhi[(size_t)r * nhi + j] = vhi[k][j];
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------------- fold
 // Arithmetic of one `acc += v` in the tensor dtype (what Tensor.add_ does).
 template <int DT>
@@ -1143,8 +1185,10 @@ extern "C" int jg_halo_pack_3d(void* const strips[27], const void* src,
           a.box[slot].org[ax] = org;
           a.box[slot].ext[ax] = ext;
         }
+        // work items of the slot: 16-byte chunks, whole rows of the strip each
+        const int per_vec = 16 / elem_size;
         long long cnt = g.planes * (long long)a.box[slot].ext[0] * a.box[slot].ext[1] *
-                        a.box[slot].ext[2];
+                        ((a.box[slot].ext[2] + per_vec - 1) / per_vec);
         if (cnt == 0) a.dst[slot] = nullptr;
         if (a.dst[slot] != nullptr && cnt > biggest) biggest = cnt;
       }
@@ -1155,10 +1199,35 @@ extern "C" int jg_halo_pack_3d(void* const strips[27], const void* src,
     Sh += g.lo[1] + g.hi[1];
     Sw += g.lo[2] + g.hi[2];
   }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // Both faces across W wanted, at most two cells thick, from rows of more than one cache line,
+  // and many of them: one pass that takes both ends of a row (the kernel above says why).
+  {
+    const Box &lo = a.box[12], &hi = a.box[14];
+    const unsigned long long rows = (unsigned long long)g.planes * lo.ext[0] * lo.ext[1];
+    if (a.dst[12] != nullptr && a.dst[14] != nullptr && lo.ext[2] <= 2 && hi.ext[2] <= 2 &&
+        (long long)Sw * elem_size > 128 && rows >= (1u << 16) && rows < (1ull << 32)) {
+      const unsigned blocks = (unsigned)((rows + 1023) / 1024);
+      if (elem_size == 2)
+        pack_w_faces_kernel<uint16_t><<<blocks, 256, 0, s>>>(static_cast<uint16_t*>(a.dst[12]), static_cast<uint16_t*>(a.dst[14]),
+                                                             static_cast<const uint16_t*>(src), lo, hi, (unsigned)rows, Sd, Sh, Sw);
+      else
+        pack_w_faces_kernel<uint32_t><<<blocks, 256, 0, s>>>(static_cast<uint32_t*>(a.dst[12]), static_cast<uint32_t*>(a.dst[14]),
+                                                             static_cast<const uint32_t*>(src), lo, hi, (unsigned)rows, Sd, Sh, Sw);
+      JG_CHECK_LAUNCH("jg_halo_pack_3d");
+      a.dst[12] = a.dst[14] = nullptr;
+      biggest = 0;
+      for (int slot = 0; slot < 27; ++slot) {
+        const long long cnt = g.planes * (long long)a.box[slot].ext[0] * a.box[slot].ext[1] *
+                              ((a.box[slot].ext[2] + 16 / elem_size - 1) / (16 / elem_size));
+        if (a.dst[slot] != nullptr && cnt > biggest) biggest = cnt;
+      }
+      if (biggest == 0) return JG_OK;
+    }
+  }
   long long bx = (biggest + 255) / 256;
   if (bx > 4096) bx = 4096;
   dim3 grid((unsigned)bx, 27, 1);
-  hipStream_t s = static_cast<hipStream_t>(stream);
   const bool narrow = (unsigned long long)g.planes * Sd * Sh * Sw < (1ull << 31);
   if (elem_size == 2) {
     if (narrow)

@@ -251,6 +251,50 @@ def halo_assemble(
     return out
 
 
+_LAYOUTS: dict = {}
+
+
+def _strip_layout(geom: "HaloGeometry", verb: str, lead: tuple, offs: tuple, elem_size: int) -> tuple:
+    """Where each strip of a pack sits in one flat buffer: ``(offset, shape, strides, start, count)`` per
+    strip in elements, starts rounded up to 256 bytes, and the buffer's length. Cached per geometry."""
+    key = (tuple(geom.size), tuple(geom.lo), tuple(geom.hi), verb, lead, offs, elem_size)
+    hit = _LAYOUTS.get(key)
+    if hit is not None:
+        return hit
+    per = 256 // elem_size
+    rows, start = [], 0
+    for o in offs:
+        shape = lead + geom.strip_extent(o, verb)
+        strides, count = [], 1
+        for n in reversed(shape):
+            strides.append(count)
+            count *= n
+        rows.append((o, shape, tuple(reversed(strides)), start, count))
+        start += (count + per - 1) // per * per
+    if len(_LAYOUTS) > 256:
+        _LAYOUTS.clear()
+    _LAYOUTS[key] = (tuple(rows), start)
+    return _LAYOUTS[key]
+
+
+def new_strips(geom: "HaloGeometry", verb: str, lead: tuple, offs: Sequence, dtype: torch.dtype, device) -> tuple:
+    """Uninitialised strips for the offsets ``offs`` (``{offset: tensor}``) and the pointer table
+    the C entry points take. One allocation holds them all, each strip a contiguous view that
+    starts on a 256-byte boundary: 26 separate allocations cost more host time than the kernels
+    that fill the strips take on the GPU."""
+    elem = torch.empty((), dtype=dtype).element_size()
+    layout, total = _strip_layout(geom, verb, tuple(lead), tuple(offs), elem)
+    flat = torch.empty(total, dtype=dtype, device=device)
+    base = flat.data_ptr()
+    out: dict = {}
+    tab = VoidP27()
+    for o, shape, strides, start, count in layout:
+        out[o] = flat.as_strided(shape, strides, start)
+        if count:
+            tab[slot(o)] = base + start * elem
+    return out, tab
+
+
 def halo_pack(
     src: torch.Tensor,
     geom: HaloGeometry,
@@ -272,13 +316,7 @@ def halo_pack(
     lead = tuple(src.shape[: -geom.n_spatial])
     verb = "pack_bwd" if from_padded else "pack_fwd"
     offs = geom.offsets() if present is None else [tuple(o) for o in present]
-    out: dict = {}
-    tab = VoidP27()
-    for o in offs:
-        t = torch.empty(lead + geom.strip_extent(o, verb), dtype=src.dtype, device=src.device)
-        out[o] = t
-        if t.numel():
-            tab[slot(o)] = t.data_ptr()
+    out, tab = new_strips(geom, verb, lead, offs, src.dtype, src.device)
     cg = geom.c_geom(planes)
     rc = _lib.load().jg_halo_pack_3d(
         tab, _lib.ptr(src), cg, int(from_padded), src.element_size(), _lib.stream_ptr(src.device)
@@ -345,6 +383,7 @@ __all__ = [
     "halo_fold_border_",
     "halo_pack",
     "halo_widths",
+    "new_strips",
     "needed_input_span",
     "slot",
 ]
