@@ -159,7 +159,7 @@ def attention_figures(dev, iters: int) -> dict:
     ms_ring = time_gpu(lambda: ja.ring_forward(q, ks, vs, scale), iters)
     # The same ring with the hops in the loop (jigsaw_amd.ring.RingSeat): every step forwards the chunk
     # it holds and receives the next one, on the compute stream or on the seat's transfer stream. The
-    # neighbour's transfer is a device copy of the 2 x 4 MiB; "link" puts a spinning one-thread kernel of
+    # neighbour's transfer is a device copy of the 8 MiB (K and V of a chunk in one message); "link" puts a spinning one-thread kernel of
     # about the time the message takes over one 153 GB/s xGMI link in front of it (a transfer over the
     # link, unlike a big device copy, occupies neither the compute units nor HBM).
     from jigsaw_amd import ring as jr
@@ -168,15 +168,13 @@ def attention_figures(dev, iters: int) -> dict:
     ms_cal = time_gpu(lambda: torch.cuda._sleep(cal), 5)
     link_cycles = int(cal * (ks[0].numel() * 2 / 153e9 * 1e3) / ms_cal)  # one K or V message
 
-    def seat_for(link, overlap, scope):
-        seen = {}
+    kvs = [torch.stack((k, v)) for k, v in zip(ks, vs)]  # a chunk travels as one message: K and V together
 
+    def seat_for(link, overlap, scope):
         def hop(src, buf, direction, *, group, async_op, tag):
-            which = seen.get(tag, 0) % 2  # K first, then V
-            seen[tag] = which + 1
             if link:
-                torch.cuda._sleep(link_cycles)
-            buf.copy_((ks, vs)[which][(tag + 1) % P])
+                torch.cuda._sleep(2 * link_cycles)
+            buf.copy_(kvs[(tag + 1) % P])
             return buf, None
 
         def relay(src, buf, offset, *, group, async_op, step):
@@ -191,8 +189,9 @@ def attention_figures(dev, iters: int) -> dict:
     for name, link, overlap in (("ms_copy_inline", False, False), ("ms_copy_overlapped", False, True),
                                 ("ms_link_inline", True, False), ("ms_link_overlapped", True, True)):
         seat = seat_for(link, overlap, "local")
-        hop[name] = time_gpu(lambda: seat.forward(q, ks[0], vs[0], scale), iters)
-        _, _, saved = seat.forward(q, ks[0], vs[0], scale)
+        k0, v0 = kvs[0][0], kvs[0][1]  # V behind K in memory, as the packed projection leaves them: sent from where they lie
+        hop[name] = time_gpu(lambda: seat.forward(q, k0, v0, scale), iters)
+        _, _, saved = seat.forward(q, k0, v0, scale)
         hop_bwd[name] = time_gpu(lambda: seat.backward(dout, q, out, l, scale, saved), iters)
     hop["ms_no_hop"] = ms_ring
     hop_bwd["ms_no_hop"] = time_gpu(lambda: ja.ring_backward(dout, q, out, l, ks, vs, scale), iters)

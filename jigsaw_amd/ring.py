@@ -8,24 +8,28 @@ tensors of the caller: the receive slots, the transfer streams and a fixed set o
 pass allocates no stream or event and (with ``save_scope="local"``) no receive buffer.
 
 Schedule of a pass over ``P`` chunks. At step ``s`` the rank holds global chunk
-``(rank + s) % P`` (forward_chunk_provider.py:190-192) in slot ``s % 2``; step 0 reads the
-caller's own tensors. Per step, in this order on the host:
+``(rank + s) % P`` (forward_chunk_provider.py:190-192); step 0 reads the caller's own
+tensors, step ``s > 0`` receive slot ``s - 1``. A chunk travels as ONE message: K and V of a
+slot are the two halves of one ``(2, ...)`` buffer, and the caller's own pair is sent from
+where it lies when V follows K in memory (the packed projection output), else from one
+packed copy. There are ``P - 1`` slots (memory is not what a 288 GB device is short of), so
+within a pass no transfer has to wait for a core to leave a slot. On the host:
 
-1. the compute stream waits for ``landed[s % 2]`` (the hop that filled the slot);
-2. the attention core of step ``s`` is enqueued (fused with the merge into the fp32
-   accumulator where the kernel covers the shape);
-3. ``idle[s % 2]`` is recorded behind it on the compute stream;
-4. the hop for step ``s + 1`` is issued on the transfer stream: it sends the slot the core
-   is reading (two readers, no hazard) and receives into slot ``(s + 1) % 2``, which the core
-   of step ``s - 1`` may still be reading, so the transfer stream first waits for
-   ``idle[(s + 1) % 2]`` -- that one event, not for the compute stream as a whole -- and then
-   records ``landed[(s + 1) % 2]`` behind the transfer.
+1. ``start`` is recorded on the compute stream (behind whatever produced K and V and behind
+   every earlier pass), the transfer stream waits for it once, hop 0 is issued and the
+   attention core of step 0 is enqueued;
+2. the other ``P - 2`` hops are issued on the transfer stream: hop ``s`` sends the chunk of
+   step ``s`` (the caller's pair, then slot ``s - 1``: stream order makes it wait for the hop
+   that filled it) and receives into slot ``s``, then records ``landed[s]``. The host is done
+   with the transfers while step 0 still computes;
+3. per later step the compute stream waits for ``landed[s - 1]`` and the core is enqueued
+   (fused with the merge into the fp32 accumulator where the kernel covers the shape).
 
-The core is enqueued before the hop is issued, so the host cost of issuing the hop sits
-behind a running kernel instead of in front of it, and the transfer of step ``s + 1`` runs
-while step ``s`` computes. K and V travel as two messages from the tensors they live in
-(no packed copy). Without a transfer stream (``overlap=False``) the same steps run on the
-compute stream and the host waits on the handle the transport returns.
+Every cross-stream wait and every change of the current stream costs the host 7-10 us here,
+about a fifth of what one core of configuration 4 takes on the GPU: the schedule above needs
+one wait per step and one change of stream per pass. Without a transfer stream
+(``overlap=False``) the same steps run on the compute stream, the hop for step ``s + 1``
+behind the core of step ``s``, and the host waits on the handle the transport returns.
 
 The transport is the caller's, with the reference's signatures:
 
@@ -78,11 +82,10 @@ class RingSeat:
         self._like = like
         on_gpu = like.is_cuda
         self._wire = torch.cuda.Stream(device=like.device) if (overlap and on_gpu and world > 1) else None
-        # slot i holds (k, v) of the steps with s % 2 == i; allocated on first use, then kept
-        self._slots: list[tuple[torch.Tensor, torch.Tensor] | None] = [None, None]
+        # slot i holds the chunk of step i + 1, K and V as the halves of one buffer; allocated on first use, then kept
+        self._slots: list = [None] * max(self.world - 1, 0)
         if self._wire is not None:
-            self._landed = [torch.cuda.Event(), torch.cuda.Event()]
-            self._idle = [torch.cuda.Event(), torch.cuda.Event()]
+            self._landed = [torch.cuda.Event() for _ in range(self.world - 1)]
             self._start = torch.cuda.Event()
             # the dK/dV partials go to other peers than the K/V hops (other links), on a stream of their own
             self._wire_back = torch.cuda.Stream(device=like.device) if save_scope == "local" else None
@@ -94,59 +97,70 @@ class RingSeat:
         """Global index of the chunk the rank holds at ``step`` while chunks circulate."""
         return (self.rank + step) % self.world
 
-    def _slot(self, i: int, fresh: bool) -> tuple[torch.Tensor, torch.Tensor]:
+    def _slot(self, i: int, fresh: bool) -> torch.Tensor:
+        shape = (2, *self._like.shape)
         if fresh:
-            return torch.empty_like(self._like), torch.empty_like(self._like)
+            return self._like.new_empty(shape)
         if self._slots[i] is None:
-            self._slots[i] = (torch.empty_like(self._like), torch.empty_like(self._like))
+            self._slots[i] = self._like.new_empty(shape)
         return self._slots[i]
 
-    # ------------------------------------------------------------------ the hop
-    def _issue_hop(self, held: tuple, into: tuple, step: int) -> Any:
-        """Send ``held`` towards ``rank - 1`` and receive the chunk of ``step + 1`` into ``into``."""
-        works = []
-        for src, buf in zip(held, into):
-            _, work = self._hop(src, buf, -1, group=self.group, async_op=True, tag=step)
-            if work is not None:
-                works.append(work)
-        return works
+    @staticmethod
+    def _packed(k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+        """``(2, ...)`` tensor with ``k`` then ``v``: a view when ``v`` follows ``k`` in memory, else a copy."""
+        if (k.is_contiguous() and v.is_contiguous() and v.storage_offset() == k.storage_offset() + k.numel()
+                and k.untyped_storage().data_ptr() == v.untyped_storage().data_ptr()):
+            return torch.as_strided(k, (2, *k.shape), (k.numel(), *k.stride()))
+        return torch.stack((k, v))
 
+    # ------------------------------------------------------------------ the hops
     def _circulate(self, k: torch.Tensor, v: torch.Tensor, keep: bool):
         """Generator over ``(step, k_s, v_s)``; the consumer enqueues its kernels for a step
-        and then resumes the generator, which issues the hop for the next step behind them."""
+        and then resumes the generator."""
         P, wire = self.world, self._wire
-        held = (k, v)
-        if wire is not None:
-            compute = torch.cuda.current_stream(self._like.device)
-            # the transfers come behind whatever produced k and v and behind every earlier pass
-            self._start.record(compute)
-            wire.wait_event(self._start)
-        pending: list = []
-        for s in range(P):
-            if s > 0:
-                if wire is not None:
-                    compute.wait_event(self._landed[s % 2])
-                else:
-                    for w in pending:
-                        w.wait()
-            yield s, held[0], held[1]
-            if s + 1 == P:
-                break
-            into = self._slot((s + 1) % 2, fresh=keep)
-            if wire is None:
-                pending = self._issue_hop(held, into, s)
-            else:
-                self._idle[s % 2].record(compute)
-                if s >= 1 and not keep:
-                    wire.wait_event(self._idle[(s + 1) % 2])  # the core of step s - 1 has left that slot
-                with torch.cuda.stream(wire):
-                    for w in self._issue_hop(held, into, s):
-                        w.wait()  # a torch.distributed handle makes the CURRENT stream wait, not the host
-                    self._landed[(s + 1) % 2].record(wire)
-                # No record_stream() on the tensors the transfer touched: the compute stream waits for
-                # `landed` before the pass ends, so whatever it frees or reuses afterwards is ordered
-                # behind every access of the transfer stream (and record_stream is slow on the host).
-            held = into
+        if P == 1:
+            yield 0, k, v
+            return
+        held = self._packed(k, v)
+        if wire is None:
+            ks, vs = k, v
+            for s in range(P):
+                yield s, ks, vs
+                if s + 1 == P:
+                    break
+                into = self._slot(s, fresh=keep)
+                _, work = self._hop(held, into, -1, group=self.group, async_op=True, tag=s)
+                if work is not None:
+                    work.wait()
+                held, ks, vs = into, into[0], into[1]
+            return
+        compute = torch.cuda.current_stream(self._like.device)
+        slots = [self._slot(s, fresh=keep) for s in range(P - 1)]  # allocated while the compute stream is current
+        self._start.record(compute)
+        wire.wait_event(self._start)
+
+        def issue(first: int, last: int, held: torch.Tensor) -> torch.Tensor:
+            torch.cuda.set_stream(wire)  # (a `with torch.cuda.stream` block costs several times as much host time)
+            try:
+                for s in range(first, last):
+                    _, work = self._hop(held, slots[s], -1, group=self.group, async_op=True, tag=s)
+                    if work is not None:
+                        work.wait()  # a torch.distributed handle makes the CURRENT stream wait, not the host
+                    self._landed[s].record(wire)
+                    held = slots[s]
+            finally:
+                torch.cuda.set_stream(compute)
+            return held
+
+        held = issue(0, 1, held)  # the first transfer starts before the host turns to the core of step 0
+        yield 0, k, v
+        issue(1, P - 1, held)
+        # No record_stream() on the tensors the transfers touch: the compute stream waits for every
+        # `landed` before the pass ends, so whatever it frees or reuses afterwards is ordered behind
+        # every access of the transfer stream (and record_stream is slow on the host).
+        for s in range(1, P):
+            compute.wait_event(self._landed[s - 1])
+            yield s, slots[s - 1][0], slots[s - 1][1]
 
     # ------------------------------------------------------------------ forward
     def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float):
@@ -237,13 +251,16 @@ class RingSeat:
             else:
                 ready, arrived = self._ready[s % 2], self._arrived[s % 2]
                 ready.record(compute)
-                with torch.cuda.stream(wire):
-                    wire.wait_event(ready)
+                wire.wait_event(ready)
+                torch.cuda.set_stream(wire)
+                try:
                     for src, buf in ((dk_j, r_dk), (dv_j, r_dv)):
                         _, w = self._relay(src, buf, s, group=self.group, async_op=True, step=s)
                         if w is not None:
                             w.wait()
                     arrived.record(wire)
+                finally:
+                    torch.cuda.set_stream(compute)
                 keep_alive.append((dk_j, dv_j))  # read by the transfer stream until `arrived`
                 inbox = (r_dk, r_dv, arrived)
         if inbox is not None:

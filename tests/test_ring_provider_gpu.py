@@ -36,16 +36,17 @@ class Peers:
     def __init__(self, rank, ks, vs, with_work, partials=None, sums=None):
         self.rank, self.ks, self.vs, self.P = rank, ks, vs, len(ks)
         self.with_work, self.partials, self.sums = with_work, partials, sums
-        self.log, self.sent, self._seen = [], {}, {}
+        self.log, self.sent = [], {}
 
     def hop(self, src, buf, direction, *, group, async_op, tag):
+        # one message per hop: K and V of a chunk as the two halves of a (2, ...) tensor
         assert direction == -1 and async_op and buf.shape == src.shape and buf.data_ptr() != src.data_ptr()
-        which = self._seen.get(tag, 0)  # first message of a step is K, second V
-        self._seen[tag] = which + 1
-        j = (self.rank + tag + 1) % self.P
-        held = (self.ks, self.vs)[which][(self.rank + tag) % self.P]
-        assert torch.equal(src, held), "the hop must forward the chunk of the current step"
-        buf.copy_((self.ks, self.vs)[which][j])
+        assert src.shape[0] == 2 and src.is_contiguous() and buf.is_contiguous()
+        here, j = (self.rank + tag) % self.P, (self.rank + tag + 1) % self.P
+        assert torch.equal(src[0], self.ks[here]) and torch.equal(src[1], self.vs[here]), \
+            "the hop must forward the chunk of the current step"
+        buf[0].copy_(self.ks[j])
+        buf[1].copy_(self.vs[j])
         self.log.append(("hop", tag, torch.cuda.current_stream().cuda_stream))
         return buf, (_Work(self.log) if self.with_work else None)
 
@@ -102,12 +103,12 @@ def test_ring_seat_matches_all_ranks_oracle(shape, P, dtype, scope, overlap, dev
                                save_scope=scope, overlap=overlap)
             out, lse, saved = seat.forward(gq[r], gk[r], gv[r], scale)
             # a second forward on the same seat: the slots and events are reused
-            pr._seen.clear(); pr.log.clear()
+            pr.log.clear()
             out2, lse2, saved = seat.forward(gq[r], gk[r], gv[r], scale)
             torch.cuda.synchronize()
             assert torch.equal(out, out2) and torch.equal(lse, lse2)
             fwd_log = list(pr.log)
-            pr._seen.clear(); pr.log.clear()
+            pr.log.clear()
             dq, dk, dv = seat.backward(gd[r], gq[r], out, lse, scale, saved)
             torch.cuda.synchronize()
             res.append((out, lse, dq, dk, dv))
@@ -137,7 +138,7 @@ def test_ring_seat_matches_all_ranks_oracle(shape, P, dtype, scope, overlap, dev
             assert rel_l2(got, w) < bound, f"rank {r} {name}: {rel_l2(got, w):.3e}"
         pr, fwd_log, seat = peers[r]
         hops = [e for e in fwd_log if e[0] == "hop"]
-        assert [e[1] for e in hops] == [s for s in range(P - 1) for _ in (0, 1)]  # K and V, one hop per step but the last
+        assert [e[1] for e in hops] == list(range(P - 1))  # one message (K and V together) per step but the last
         assert [seat.chunk_at(s) for s in range(P)] == [(r + s) % P for s in range(P)]
         main = torch.cuda.current_stream().cuda_stream
         if overlap and P > 1:
@@ -145,11 +146,11 @@ def test_ring_seat_matches_all_ranks_oracle(shape, P, dtype, scope, overlap, dev
             assert not any(e[0] == "wait" for e in fwd_log)
         elif P > 1:
             assert all(e[-1] == main for e in fwd_log)
-            assert sum(e[0] == "wait" for e in fwd_log) == 2 * (P - 1)  # the host waited for every handle
+            assert sum(e[0] == "wait" for e in fwd_log) == P - 1  # the host waited for every handle
         if scope == "local":
             relays = [e for e in pr.log if e[0] == "relay"]
             assert [e[1] for e in relays] == [s for s in range(1, P) for _ in (0, 1)]
-            assert len([e for e in pr.log if e[0] == "hop"]) == 2 * (P - 1)  # K/V circulate again in the backward
+            assert len([e for e in pr.log if e[0] == "hop"]) == P - 1  # K/V circulate again in the backward
             if overlap and P > 1:
                 assert all(e[2] != main for e in relays)
         else:
