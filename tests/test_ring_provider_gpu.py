@@ -172,3 +172,34 @@ def test_ring_seat_argument_errors(dev):
     out, lse, saved = seat.forward(k, k, k, 0.125)
     with pytest.raises(ValueError, match="relay_fn"):
         seat.backward(k, k, out, lse, 0.125, saved)
+
+
+@pytest.mark.parametrize("overlap", [False, True], ids=["plain", "overlapped"])
+def test_own_chunk_is_sent_from_where_it_lies_when_v_follows_k(overlap, dev):
+    """K and V that are adjacent in memory (the packed projection output) leave as one message
+    without a packed copy; separate tensors are packed once. Results are the same either way,
+    and the saved chunks of a pass do not alias the slots the next pass writes."""
+    torch.manual_seed(3)
+    P, shape = 3, (1, 2, 128, 64)
+    q = (torch.randn(shape, device=dev) * 0.125).bfloat16()
+    kvs = [torch.randn(2, *shape, device=dev).bfloat16() for _ in range(P)]
+    first_src = []
+
+    def hop(src, buf, direction, *, group, async_op, tag):
+        if tag == 0:
+            first_src.append(src.data_ptr())
+        buf.copy_(kvs[tag + 1])
+        return buf, None
+
+    seat = jr.RingSeat(0, P, kvs[0][0], hop, save_scope="global", overlap=overlap)
+    out_a, lse_a, saved_a = seat.forward(q, kvs[0][0], kvs[0][1], 0.125)  # views of one (2, ...) tensor
+    k_sep, v_sep = kvs[0][0].clone(), kvs[0][1].clone()
+    out_b, lse_b, saved_b = seat.forward(q, k_sep, v_sep, 0.125)          # two tensors of their own
+    torch.cuda.synchronize()
+    assert first_src[0] == kvs[0].data_ptr(), "adjacent K / V must be sent in place"
+    assert first_src[1] not in (k_sep.data_ptr(), kvs[0].data_ptr()), "separate K / V are packed into one message"
+    assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)
+    for j in range(P):
+        for a, b in zip(saved_a[j], saved_b[j]):
+            assert torch.equal(a, b) and (j == 0 or a.data_ptr() != b.data_ptr())
+        assert torch.equal(saved_a[j][0], kvs[j][0]) and torch.equal(saved_a[j][1], kvs[j][1])
