@@ -24,7 +24,16 @@
 //   Schedule    persistent workgroups (one per CU) walk a contiguous, XCD-local
 //               range of tiles; the global loads of stage s+1 are issued before the
 //               MFMAs of stage s and written to LDS between its MFMA groups (one
-//               barrier per stage).
+//               barrier per stage). A cursor decodes a tile's coordinates once and steps
+//               through its stages by additions; the weight fragments of a group of 24
+//               MFMAs are fetched under the group before, into the registers it frees.
+//   Tile grid   tile column tw covers produced columns [org_w + 64 tw, + 64). The host picks
+//               org_w <= 0 so that the staged row segments (144 bytes from input column
+//               org_w + 64 tw - pad_w) start on cache lines where that costs no extra
+//               tile column, and stages a window from one pixel earlier (lead) when it
+//               would otherwise start on an odd column (4-byte aligned loads throughout).
+//   Epilogue    16-bit results with rows of whole 16-byte pieces pass through LDS and leave as
+//               16-byte stores; everything else as 2- or 4-byte stores along W.
 //   dgrad       the same kernel on the output gradient with virtual zero padding
 //               k-1-p and the weights flipped and transposed by the preparation.
 //   Channels    any counts: the contraction is padded to 16-channel steps per depth tap
