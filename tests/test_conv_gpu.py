@@ -38,6 +38,11 @@ PRIM_CASES = [
     (2, 64, 64, (260, 131), (3, 3), (1, 1), (0, 0), (1, 1)),
     (2, 32, 32, (6, 70, 130), (3, 3, 3), (1, 1, 1), (0, 0, 0), (1, 1, 1)),
     (1, 32, 64, (131, 200), (3, 3), (1, 1), (1, 1), (1, 1)),
+    # row lengths of whole cache lines: the input gradient's tile grid moves so that its staged rows start on
+    # a line (an odd distance: staged from one pixel earlier), the first tile column mostly hangs out of the tensor
+    (2, 32, 32, (20, 128), (3, 3), (1, 1), (1, 1), (1, 1)),
+    (1, 64, 64, (35, 192), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (1, 32, 16, (4, 18, 64), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
     # channel counts beyond one group of LDS-resident weights, and produced channels that are
     # not a multiple of the 32-row MFMA tile (padded with zero weight rows, not stored)
     (1, 128, 128, (20, 70), (3, 3), (1, 1), (1, 1), (1, 1)),
@@ -330,6 +335,8 @@ FUSED_CASES = [
     ((40, 72), (1, 1), (1, 1), (0, 0), 1, 64, "some"),
     ((24, 40), (0, 2), (2, 0), (0, 0), 1, 32, "all"),
     ((16, 96), (1, 0), (1, 0), (0, 1), 1, 64, "all"),     # W axis not split: the conv pads it itself
+    ((48, 128), (1, 1), (1, 1), (0, 0), 2, 64, "all"),    # rows of g are whole cache lines: the tile grid is shifted
+    ((20, 192), (1, 1), (1, 1), (0, 0), 1, 32, "some"),
     ((8, 8, 16), (1, 1, 1), (1, 1, 1), (0, 0, 0), 1, 32, "all"),
     ((6, 10, 24), (1, 0, 1), (1, 0, 1), (0, 1, 0), 1, 32, "some"),
 ]
