@@ -359,7 +359,8 @@ def swin_figures(dev, iters: int) -> dict:
             y = block(x)
         y.backward(gout)
 
-    ms = time_gpu(step, max(3, iters // 2))
+    # a host-bound step of ~40 launches: a handful of cold iterations says little, so more of them
+    ms = time_gpu(step, max(20, iters), warmup=5)
     xr = x.detach()
     ms_roll = time_gpu(lambda: jr.roll(xr, (-4, -4), (1, 2)), iters)
     return {
