@@ -124,3 +124,42 @@ def test_assemble_fold_full_size_properties(dtype, dev):
     cut = halo_pack(aug, geom, from_padded=True)
     for o, t in strips.items():
         assert torch.equal(cut[o], t), o
+
+
+def _slices(geom, offset, from_padded):
+    """The block of the source a pack takes for neighbour ``offset``, per spatial axis."""
+    out = []
+    for o, n, lo, hi in zip(offset, geom.size, geom.lo, geom.hi):
+        if not from_padded:  # forward: the part of my tile that lies in that neighbour's halo
+            out.append(slice(0, hi) if o < 0 else slice(0, n) if o == 0 else slice(n - lo, n))
+        else:                # backward: the part of my padded gradient that neighbour owns
+            out.append(slice(0, lo) if o < 0 else slice(lo, lo + n) if o == 0 else slice(lo + n, lo + n + hi))
+    return tuple(out)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("from_padded", [False, True], ids=["own-tile", "padded"])
+@pytest.mark.parametrize("size,lo,hi", [
+    ((1024, 80), (1, 2), (1, 2)),      # 65536 rows of more than a cache line: the two W faces leave in one pass
+    ((1024, 80), (1, 2), (0, 1)),      # faces of different thickness
+    ((1024, 80), (0, 0), (1, 2)),      # one of the two faces is empty: the general kernel takes the other
+    ((8, 96, 96), (1, 1, 1), (1, 1, 1)),
+], ids=["w2", "w2-1", "one-face", "3d"])
+def test_pack_takes_the_blocks_the_neighbours_need(size, lo, hi, from_padded, dtype, dev):
+    """Every strip of ``halo_pack`` equals the slice of the source it stands for (bit for bit), whichever kernel
+    cut it; the strips of one call do not overlap in memory."""
+    torch.manual_seed(11)
+    geom = HaloGeometry(size, lo, hi)
+    lead = (64, 1) if len(size) == 2 else (9, 2)
+    spatial = geom.padded if from_padded else geom.size
+    src = torch.randn(*lead, *spatial, device=dev).to(dtype)
+    strips = halo_pack(src, geom, from_padded=from_padded)
+    spans = []
+    for o, t in strips.items():
+        want = src[(..., *_slices(geom, o, from_padded))]
+        assert t.shape == want.shape and t.is_contiguous(), o
+        assert torch.equal(t, want), o
+        if t.numel():
+            spans.append((t.data_ptr(), t.data_ptr() + t.numel() * t.element_size()))
+    spans.sort()
+    assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))
