@@ -67,6 +67,15 @@ int jg_abi_version(void);
  *   pack_fwd (send)      hi           size          lo     <- their halo of me
  *   pack_bwd (send)      lo           size          hi     <- my halo's grads
  *   fold     (recv)      hi           size          lo     <- their halo of me
+ *
+ * Where the need spans drift against the tiles (out_local * stride != n,
+ * halo.py:49-63) the widths differ from rank to rank. The two verbs marked
+ * "their halo of me" then take a geometry with hi = the hi width of the lower
+ * neighbour and lo = the lo width of the upper neighbour: jg_halo_pack_3d with
+ * from_padded = 0 and jg_halo_fold_border_3d, which read no padded tensor.
+ * jg_halo_fold_3d indexes the padded gradient and the strips with one set of
+ * widths; for a drifting span call it with an empty strip table (gx = 0 + own)
+ * and finish with jg_halo_fold_border_3d.
  * ------------------------------------------------------------------------- */
 typedef struct {
   int64_t planes;

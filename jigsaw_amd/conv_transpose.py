@@ -31,7 +31,7 @@ from .conv import (
     conv_nd_input_fold,
     conv_nd_weight,
 )
-from .halo import HaloGeometry, halo_assemble, halo_fold, halo_fold_border_, halo_pack
+from .halo import HaloGeometry, halo_assemble, halo_fold, halo_fold_border_, halo_pack, neighbour_widths
 
 
 def produced_output_span(rank, group_size, local_in_size, kernel, stride, padding, dilation):
@@ -53,33 +53,49 @@ def produced_output_span(rank, group_size, local_in_size, kernel, stride, paddin
     return base, wloc, out_local, global_out
 
 
+def raw_span_widths(rank, group_size, local_in_size, kernel, stride, padding, dilation):
+    """``(left, right, out_local)``: how many raw output columns of a rank lie before and
+    behind the block it keeps. They change from rank to rank when ``extent != stride +
+    2 * padding`` (the raw spans drift against the blocks). Accepted: the raw span covers
+    the kept block and reaches at most one block to either side, so that every overlap
+    is with an adjacent rank; anything else raises ``NotImplementedError``."""
+    base, wloc, out_local, _ = produced_output_span(rank, group_size, local_in_size, kernel, stride, padding, dilation)
+    left = rank * out_local - base
+    right = wloc - left - out_local
+    if left < 0 or right < 0:
+        raise NotImplementedError(
+            f"transposed conv on a split axis: the raw span [{base}, {base + wloc}) of rank {rank} does not cover "
+            f"the block it keeps [{rank * out_local}, {(rank + 1) * out_local})"
+        )
+    if left > out_local or right > out_local:
+        raise NotImplementedError(
+            f"transposed conv on a split axis: the raw span of rank {rank} reaches {left} / {right} columns past its "
+            f"block of {out_local}: overlaps with non-adjacent ranks"
+        )
+    return left, right, out_local
+
+
 def transpose_geometry(local_in_spatial, kernel, stride, padding, dilation, ranks, group_sizes) -> HaloGeometry:
     """The raw span of a rank as a halo geometry: the owned output block with ``lo`` raw
-    columns before it and ``hi`` after. Axes with a group of one carry no halo (the local
-    transposed conv applies their padding itself). Only spans that sit the same way around
-    every rank's block are covered (``extent == stride + 2 * padding``, e.g. k4 s2 p1,
-    k3 s1 p1, k2 s2 p0); others would need rows from non-adjacent peers."""
-    size, lo, hi = [], [], []
+    columns before it and ``hi`` after, and the neighbours' widths where the spans drift
+    (_conv_transpose/halo.py:14-71 and the per-peer overlaps of :134-152). Axes with a
+    group of one carry no halo (the local transposed conv applies their padding itself)."""
+    size, lo, hi, tlo, thi = [], [], [], [], []
     for a, n in enumerate(local_in_spatial):
         k, s, p, d = kernel[a], stride[a], padding[a], dilation[a]
-        extent = d * (k - 1) + 1
         if group_sizes[a] <= 1:
-            size.append((n - 1) * s - 2 * p + extent)
-            lo.append(0)
-            hi.append(0)
+            size.append((n - 1) * s - 2 * p + d * (k - 1) + 1)
+            for w in (lo, hi, tlo, thi):
+                w.append(0)
             continue
-        base, wloc, out_local, _ = produced_output_span(ranks[a], group_sizes[a], n, k, s, p, d)
-        left = ranks[a] * out_local - base
-        right = wloc - left - out_local
-        if out_local != n * s or left < 0 or right < 0 or left > out_local or right > out_local:
-            raise NotImplementedError(
-                f"transposed conv on a split axis: kernel {k}, stride {s}, padding {p}, dilation {d} make the raw "
-                "spans drift against the output blocks; only extent == stride + 2 * padding is covered"
-            )
-        size.append(out_local)
-        lo.append(left)
-        hi.append(right)
-    return HaloGeometry(tuple(size), tuple(lo), tuple(hi))
+        args = (group_sizes[a], n, k, s, p, d)
+        l, h, tl, th = neighbour_widths(lambda r: raw_span_widths(r, *args), ranks[a], group_sizes[a])  # noqa: B023
+        size.append(raw_span_widths(ranks[a], *args)[2])
+        lo.append(l)
+        hi.append(h)
+        tlo.append(tl)
+        thi.append(th)
+    return HaloGeometry(tuple(size), tuple(lo), tuple(hi), tuple(tlo), tuple(thi))
 
 
 def conv_transpose_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1) -> torch.Tensor:
@@ -206,5 +222,6 @@ __all__ = [
     "conv_transpose_halo_nway_backward",
     "conv_transpose_nd",
     "produced_output_span",
+    "raw_span_widths",
     "transpose_geometry",
 ]

@@ -61,28 +61,36 @@ def halo_widths(
 ) -> tuple[int, int, int]:
     """``(lo_width, hi_width, out_local)`` of the need span around the owned rows.
 
-    Only the regime all fused kernels handle is accepted: the span starts at most
-    one tile before and ends at most one tile after the owned rows, it covers the
-    owned rows completely, and its offset is the same on every rank (so every
-    strip comes from an adjacent rank). Anything else raises
-    ``NotImplementedError``.
+    The widths may differ from rank to rank (a span that drifts against the tiles,
+    ``out_local * stride != local size``, e.g. a convolution without padding). Accepted is
+    what the fused kernels handle: the span covers the owned rows completely and starts
+    at most one tile before / ends at most one tile after them, so that every strip
+    comes from an adjacent rank. Anything else raises ``NotImplementedError``.
     """
     n = local_in_size
     lo, hi, _, out_local = needed_input_span(rank, group_size, n, kernel, stride, padding, dilation)
     lo_w = rank * n - lo
     hi_w = hi - (rank + 1) * n
-    if out_local * stride != n:
-        raise NotImplementedError(
-            f"need span drifts across ranks (out_local*stride = {out_local * stride} != local size {n}); "
-            "strips would come from non-adjacent ranks"
-        )
     if lo_w < 0 or hi_w < 0:
         raise NotImplementedError(
-            f"need span ({lo}, {hi}) does not cover the owned rows [{rank * n}, {(rank + 1) * n})"
+            f"need span ({lo}, {hi}) of rank {rank} does not cover its owned rows [{rank * n}, {(rank + 1) * n})"
         )
     if lo_w > n or hi_w > n:
-        raise NotImplementedError(f"halo ({lo_w}, {hi_w}) wider than the tile ({n})")
+        raise NotImplementedError(
+            f"halo ({lo_w}, {hi_w}) of rank {rank} wider than the tile ({n}): strips would come from non-adjacent ranks"
+        )
     return lo_w, hi_w, out_local
+
+
+def neighbour_widths(widths, rank: int, group_size: int) -> tuple[int, int, int, int]:
+    """``(lo, hi, their_lo, their_hi)`` of a rank: its own halo widths, the lo width of
+    the rank above and the hi width of the rank below (what those need of this rank's
+    tile). ``widths(r)`` returns ``(lo, hi, ...)`` of rank ``r``; a side without a
+    neighbour repeats the own width (nothing is sent there)."""
+    lo, hi = widths(rank)[:2]
+    their_lo = widths(rank + 1)[0] if rank + 1 < group_size else lo
+    their_hi = widths(rank - 1)[1] if rank >= 1 else hi
+    return lo, hi, their_lo, their_hi
 
 
 def slot(offset: Sequence[int]) -> int:
@@ -95,16 +103,33 @@ def slot(offset: Sequence[int]) -> int:
 
 @dataclass(frozen=True)
 class HaloGeometry:
-    """Tile size and halo widths of one rank (1 to 3 spatial axes)."""
+    """Tile size and halo widths of one rank (1 to 3 spatial axes).
+
+    ``their_lo`` / ``their_hi`` are the halos the neighbours have of this rank's tile:
+    the lo width of the rank above and the hi width of the rank below, per axis. They
+    size what this rank sends forward and what it receives in the fold. ``None``: the
+    same as ``lo`` / ``hi`` (every rank's span sits the same way around its tile)."""
 
     size: tuple  # interior extent per spatial axis
     lo: tuple  # halo in front of the interior
     hi: tuple  # halo behind the interior
+    their_lo: tuple | None = None
+    their_hi: tuple | None = None
 
     def __post_init__(self) -> None:
         ns = len(self.size)
         if not 1 <= ns <= 3 or len(self.lo) != ns or len(self.hi) != ns:
             raise ValueError("HaloGeometry needs 1 to 3 spatial axes with matching lo / hi")
+        for name in ("their_lo", "their_hi"):
+            v = getattr(self, name)
+            if v is None:
+                continue
+            if len(v) != ns:
+                raise ValueError(f"HaloGeometry: {name} needs one entry per spatial axis")
+            if tuple(v) == tuple(self.lo if name == "their_lo" else self.hi):
+                object.__setattr__(self, name, None)  # one spelling per geometry (cache keys, equality)
+            else:
+                object.__setattr__(self, name, tuple(int(x) for x in v))
 
     @property
     def n_spatial(self) -> int:
@@ -114,6 +139,17 @@ class HaloGeometry:
     def padded(self) -> tuple:
         return tuple(l + n + h for l, n, h in zip(self.lo, self.size, self.hi))
 
+    @property
+    def same_on_every_rank(self) -> bool:
+        return self.their_lo is None and self.their_hi is None
+
+    def theirs(self) -> "HaloGeometry":
+        """The geometry whose halos are the neighbours' halos of this tile."""
+        if self.same_on_every_rank:
+            return self
+        return HaloGeometry(self.size, self.lo if self.their_lo is None else self.their_lo,
+                            self.hi if self.their_hi is None else self.their_hi)
+
     def offsets(self) -> list:
         """All neighbour offsets except the rank itself."""
         return [o for o in itertools.product((-1, 0, 1), repeat=self.n_spatial) if any(o)]
@@ -122,12 +158,13 @@ class HaloGeometry:
         """Spatial extent of the strip of ``offset`` for ``verb``.
 
         ``assemble`` / ``pack_bwd``: (lo, size, hi) for offset (-1, 0, +1);
-        ``fold`` / ``pack_fwd``: (hi, size, lo).
+        ``fold`` / ``pack_fwd``: (their hi, size, their lo).
         """
         if verb in ("assemble", "pack_bwd"):
             pick = lambda a, o: (self.lo[a], self.size[a], self.hi[a])[o + 1]  # noqa: E731
         elif verb in ("fold", "pack_fwd"):
-            pick = lambda a, o: (self.hi[a], self.size[a], self.lo[a])[o + 1]  # noqa: E731
+            t = self.theirs()
+            pick = lambda a, o: (t.hi[a], t.size[a], t.lo[a])[o + 1]  # noqa: E731
         else:
             raise ValueError(f"unknown verb {verb!r}")
         return tuple(pick(a, o) for a, o in enumerate(offset))
@@ -156,16 +193,19 @@ class HaloGeometry:
     ) -> "HaloGeometry":
         """Geometry of a rank's need span; axes with a group of one are not padded
         (the local conv pads them itself, spatial_split.py:75-82)."""
-        lo, hi = [], []
+        lo, hi, tlo, thi = [], [], [], []
         for a, n in enumerate(local_in_spatial):
             if group_sizes[a] <= 1:
-                lo.append(0)
-                hi.append(0)
+                for w in (lo, hi, tlo, thi):
+                    w.append(0)
                 continue
-            l, h, _ = halo_widths(ranks[a], group_sizes[a], n, kernel[a], stride[a], padding[a], dilation[a])
+            args = (group_sizes[a], n, kernel[a], stride[a], padding[a], dilation[a])
+            l, h, tl, th = neighbour_widths(lambda r: halo_widths(r, *args), ranks[a], group_sizes[a])  # noqa: B023
             lo.append(l)
             hi.append(h)
-        return cls(tuple(int(n) for n in local_in_spatial), tuple(lo), tuple(hi))
+            tlo.append(tl)
+            thi.append(th)
+        return cls(tuple(int(n) for n in local_in_spatial), tuple(lo), tuple(hi), tuple(tlo), tuple(thi))
 
 
 def _check_tile(x: torch.Tensor, spatial: tuple, what: str) -> int:
@@ -257,7 +297,7 @@ _LAYOUTS: dict = {}
 def _strip_layout(geom: "HaloGeometry", verb: str, lead: tuple, offs: tuple, elem_size: int) -> tuple:
     """Where each strip of a pack sits in one flat buffer: ``(offset, shape, strides, start, count)`` per
     strip in elements, starts rounded up to 256 bytes, and the buffer's length. Cached per geometry."""
-    key = (tuple(geom.size), tuple(geom.lo), tuple(geom.hi), verb, lead, offs, elem_size)
+    key = (tuple(geom.size), tuple(geom.lo), tuple(geom.hi), geom.their_lo, geom.their_hi, verb, lead, offs, elem_size)
     hit = _LAYOUTS.get(key)
     if hit is not None:
         return hit
@@ -317,7 +357,8 @@ def halo_pack(
     verb = "pack_bwd" if from_padded else "pack_fwd"
     offs = geom.offsets() if present is None else [tuple(o) for o in present]
     out, tab = new_strips(geom, verb, lead, offs, src.dtype, src.device)
-    cg = geom.c_geom(planes)
+    # forward: the blocks are sized by the neighbours' halos of this tile
+    cg = (geom if from_padded else geom.theirs()).c_geom(planes)
     rc = _lib.load().jg_halo_pack_3d(
         tab, _lib.ptr(src), cg, int(from_padded), src.element_size(), _lib.stream_ptr(src.device)
     )
@@ -345,6 +386,19 @@ def halo_fold(
         raise ValueError("halo_fold: `out` has the wrong shape / dtype / layout")
     tab = _table(strips, geom, "fold", lead, gx_aug, None)
     cg = geom.c_geom(planes)
+    if not geom.same_on_every_rank:
+        # The neighbours' blocks are not as wide as the own halos: the own part first
+        # (0 + own in every cell, the fold without neighbours), then the neighbours' blocks
+        # by their widths. Same additions in the same order as the one-pass fold.
+        rc = _lib.load().jg_halo_fold_3d(
+            _lib.ptr(out), _lib.ptr(gx_aug), VoidP27(), cg, _lib.dtype_code(gx_aug.dtype), _lib.stream_ptr(gx_aug.device)
+        )
+        _lib.check(rc, "jg_halo_fold_3d")
+        rc = _lib.load().jg_halo_fold_border_3d(
+            _lib.ptr(out), tab, geom.theirs().c_geom(planes), _lib.dtype_code(out.dtype), _lib.stream_ptr(out.device)
+        )
+        _lib.check(rc, "jg_halo_fold_border_3d")
+        return out
     rc = _lib.load().jg_halo_fold_3d(
         _lib.ptr(out), _lib.ptr(gx_aug), tab, cg, _lib.dtype_code(gx_aug.dtype), _lib.stream_ptr(gx_aug.device)
     )
@@ -368,7 +422,7 @@ def halo_fold_border_(
     planes = _check_tile(gx, geom.size, "halo_fold_border_")
     lead = tuple(gx.shape[: -geom.n_spatial])
     tab = _table(strips, geom, "fold", lead, gx, None)
-    cg = geom.c_geom(planes)
+    cg = geom.theirs().c_geom(planes)
     rc = _lib.load().jg_halo_fold_border_3d(
         _lib.ptr(gx), tab, cg, _lib.dtype_code(gx.dtype), _lib.stream_ptr(gx.device)
     )
@@ -383,6 +437,7 @@ __all__ = [
     "halo_fold_border_",
     "halo_pack",
     "halo_widths",
+    "neighbour_widths",
     "new_strips",
     "needed_input_span",
     "slot",

@@ -202,6 +202,12 @@ DIST_CASES = [
     ((3, 2), (8, 10), 1, 3, 5, (3, 3), (2, 2), torch.float32, (1, 1), (2, 2)),
     ((2, 2), (16, 32), 1, 32, 32, (3, 3), (1, 2), torch.bfloat16, (2, 1), (1, 2)),
     ((2, 1, 2), (4, 6, 8), 1, 2, 3, (3, 3, 3), (1, 1, 2), torch.float32, (2, 1, 1), (1, 1, 2)),
+    # need spans that drift against the tiles (halo.py:49-63 with out_local * stride != n): the widths change from rank to rank
+    ((2, 2), (16, 20), 2, 4, 6, (3, 3), (0, 0), torch.float32),                    # no padding: (0, 1) and (1, 0)
+    ((4, 2), (6, 12), 1, 3, 5, (5, 3), (0, 1), torch.float32),                     # four ranks: (r, 3 - r)
+    ((2, 2), (8, 8), 1, 3, 4, (6, 6), (0, 0), torch.float32, (2, 2), (1, 1)),      # strided and drifting
+    ((2, 2), (16, 32), 1, 32, 32, (3, 3), (0, 0), torch.bfloat16),                 # MFMA path, fused fold, framed forward
+    ((2, 1, 2), (4, 6, 8), 1, 2, 3, (3, 3, 5), (0, 1, 1), torch.float32),
 ]
 
 

@@ -59,8 +59,13 @@ def test_transpose_geometry_and_spans():
     assert g.size == (16, 16) and g.lo == (1, 1) and g.hi == (1, 1)
     g = jct.transpose_geometry((8, 5), (2, 3), (2, 1), (0, 1), (1, 1), (0, 0), (2, 1))
     assert g.size == (16, 5) and g.lo == (0, 0) and g.hi == (0, 0)
-    with pytest.raises(NotImplementedError):  # k5 s1 p1 on a split axis: the raw spans drift
-        jct.transpose_geometry((6,), (5,), (1,), (1,), (1,), (0,), (2,))
+    # k5 s1 p1 on a split axis: 14 columns come out of 12, 7 per rank, the raw spans (10 wide) drift
+    g0 = jct.transpose_geometry((6,), (5,), (1,), (1,), (1,), (0,), (2,))
+    g1 = jct.transpose_geometry((6,), (5,), (1,), (1,), (1,), (1,), (2,))
+    assert (g0.size, g0.lo, g0.hi) == ((7,), (1,), (2,)) and (g1.size, g1.lo, g1.hi) == ((7,), (2,), (1,))
+    assert g0.strip_extent((1,), "fold") == (2,) and g1.strip_extent((-1,), "fold") == (2,)
+    with pytest.raises(NotImplementedError):  # a raw span that starts behind the block its rank keeps
+        jct.transpose_geometry((4,), (2,), (2,), (2,), (1,), (2,), (4,))
     for args in [(1, 3, 4, 4, 2, 1, 1), (0, 2, 5, 3, 1, 1, 2)]:
         assert jct.produced_output_span(*args) == oct_.produced_output_span(*args)
     with pytest.raises(NotImplementedError):
@@ -77,6 +82,11 @@ CASES = [
     ((2, 2), (16, 32), 1, 32, 32, (3, 3), (1, 1), (1, 1), (1, 1), torch.bfloat16),  # MFMA path, fused fold
     ((2, 2), (16, 32), 1, 64, 64, (3, 3), (1, 1), (1, 1), (1, 1), torch.bfloat16),
     ((2, 2, 2), (3, 4, 4), 1, 2, 3, (4, 3, 4), (2, 1, 2), (1, 1, 1), (1, 1, 1), torch.float32),
+    # raw spans that drift against the kept blocks (extent != stride + 2 * padding)
+    ((2, 2), (6, 6), 2, 2, 2, (5, 3), (1, 3), (1, 0), (1, 1), torch.float32),
+    ((2, 2), (5, 7), 1, 3, 2, (4, 4), (2, 2), (0, 0), (1, 1), torch.float32),      # k4 s2 p0: one column more per rank
+    ((4, 1), (4, 5), 1, 2, 3, (5, 3), (1, 1), (0, 1), (1, 1), torch.float32),      # four ranks: (lo r, hi 3 - r)
+    ((2, 2), (16, 32), 1, 32, 32, (3, 3), (1, 1), (0, 0), (1, 1), torch.bfloat16),  # MFMA path, drifting
 ]
 
 

@@ -25,6 +25,11 @@ CASES = [
     ((2, 2, 2), (6, 5, 8), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
     ((3, 3, 3), (4, 5, 6), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
     ((3, 1, 3), (4, 5, 6), (5, 3, 3), (1, 1, 1), (2, 1, 1), (1, 1, 1)),
+    # spans that drift against the tiles: the halo widths change from rank to rank
+    ((2, 2), (8, 10), (3, 3), (1, 1), (0, 0), (1, 1)),  # no padding: (lo 0, hi 1) on rank 0, (lo 1, hi 0) on rank 1
+    ((4, 2), (6, 8), (5, 3), (1, 1), (0, 0), (1, 1)),   # four ranks: (lo r, hi 3 - r)
+    ((2, 2), (8, 8), (6, 6), (2, 2), (0, 0), (1, 1)),   # strided and drifting
+    ((2, 1, 2), (4, 5, 6), (3, 3, 5), (1, 1, 1), (0, 1, 1), (1, 1, 1)),
 ]
 
 
@@ -94,11 +99,27 @@ def test_assemble_rejects_wrong_shapes(dev):
         halo_assemble(torch.zeros(1, 2, 8, 8), {}, g)
 
 
-def test_geometry_rejects_drifting_spans():
-    # kernel 3, stride 2, padding 1 on 8 rows per rank is fine; padding 0 drifts
-    HaloGeometry.for_conv((8,), (3,), (2,), (1,), (1,), (1,), (2,))
+def test_geometry_of_drifting_spans():
+    # kernel 3, stride 2, padding 1 on 8 rows per rank: every rank's span sits the same way
+    g = HaloGeometry.for_conv((8,), (3,), (2,), (1,), (1,), (1,), (2,))
+    assert g.same_on_every_rank and (g.lo, g.hi) == ((1,), (0,))
+    # no padding: 16 of 18 rows come out, 8 per rank; rank 0 needs a row of rank 1 and the other way round
+    g0 = HaloGeometry.for_conv((9,), (3,), (1,), (0,), (1,), (0,), (2,))
+    g1 = HaloGeometry.for_conv((9,), (3,), (1,), (0,), (1,), (1,), (2,))
+    assert (g0.lo, g0.hi, g1.lo, g1.hi) == ((0,), (1,), (1,), (0,))
+    assert g0.strip_extent((1,), "pack_fwd") == (1,) and g0.strip_extent((1,), "assemble") == (1,)
+    assert g1.strip_extent((-1,), "pack_fwd") == (1,) and g1.strip_extent((-1,), "fold") == (1,)
+    assert g0.theirs().lo == (1,) and g1.theirs().hi == (1,)
+    # four ranks, kernel 5: (lo r, hi 3 - r); rank 1 sends 1 row down (rank 0's hi is 3 ... of which rank 1 owns 3)
+    gs = [HaloGeometry.for_conv((6,), (5,), (1,), (0,), (1,), (r,), (4,)) for r in range(4)]
+    assert [(g.lo[0], g.hi[0]) for g in gs] == [(0, 3), (1, 2), (2, 1), (3, 0)]
+    assert gs[1].strip_extent((-1,), "pack_fwd") == (3,) and gs[1].strip_extent((1,), "pack_fwd") == (2,)
+    # a span that leaves out owned rows (stride 2 without padding on 9 rows per rank) is not covered
     with pytest.raises(NotImplementedError):
-        HaloGeometry.for_conv((9,), (3,), (1,), (0,), (1,), (1,), (2,))
+        HaloGeometry.for_conv((9,), (3,), (2,), (0,), (1,), (1,), (2,))
+    # nor is a halo wider than the tile
+    with pytest.raises(NotImplementedError):
+        HaloGeometry.for_conv((2,), (7,), (1,), (3,), (1,), (1,), (3,))
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
