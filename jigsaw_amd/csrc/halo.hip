@@ -43,6 +43,41 @@ struct Bits<uint32_t> {
   static constexpr int V = 4;
 };
 
+// `0 + v` for every element of a dword: the only value the addition changes is -0.0, which
+// becomes +0.0. On the packed 16-bit halves without unpacking them: bit 15 of (t + 0x7fff) | t
+// is set exactly where the 15 magnitude bits t of a half are not all zero, and only there the
+// sign is kept.
+template <typename T>
+__device__ __forceinline__ uint32_t zero_plus(uint32_t v);
+template <>
+__device__ __forceinline__ uint32_t zero_plus<uint32_t>(uint32_t v) {
+  return v == 0x80000000u ? 0u : v;
+}
+template <>
+__device__ __forceinline__ uint32_t zero_plus<uint16_t>(uint32_t v) {
+  const uint32_t t = v & 0x7fff7fffu;
+  const uint32_t keep = ((t + 0x7fff7fffu) | t) & 0x80008000u;
+  return t | (v & keep);
+}
+
+// One element from an address that is the same in every lane, through the scalar cache: the
+// aligned dword that holds it (which lies in the same page) and, for a 16-bit element, a shift.
+__device__ __forceinline__ uint32_t uniform_dword(const uint32_t* q) {
+  // the address in scalar registers, whatever the compiler worked out about it
+  const uint64_t a = reinterpret_cast<uint64_t>(q);
+  const uint64_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+  const uint64_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32));
+  q = reinterpret_cast<const uint32_t*>((hi << 32) | lo);
+  uint32_t w;
+  asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(w) : "s"(q) : "memory");
+  return w;
+}
+__device__ __forceinline__ uint32_t uniform_element(const uint32_t* s) { return uniform_dword(s); }
+__device__ __forceinline__ uint16_t uniform_element(const uint16_t* s) {
+  const uint32_t odd = (uint32_t)(reinterpret_cast<uintptr_t>(s) >> 1) & 1u;
+  return (uint16_t)(uniform_dword(reinterpret_cast<const uint32_t*>(s - odd)) >> (odd * 16));
+}
+
 // Load 16 bytes from an address that is only sizeof(T)-aligned.
 template <typename T>
 __device__ __forceinline__ u32x4 load16_unaligned(const T* s);
@@ -54,9 +89,21 @@ __device__ __forceinline__ u32x4 load16_unaligned<uint32_t>(const uint32_t* s) {
 
 template <>
 __device__ __forceinline__ u32x4 load16_unaligned<uint16_t>(const uint16_t* s) {
-  // the memory pipeline of gfx9 takes vector accesses at any alignment
-  typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
-  return *reinterpret_cast<const u32x4_a2*>(s);
+  // The memory pipeline takes vector accesses at any alignment, but one that starts on an odd
+  // halfword runs at a fraction of the rate of a dword-aligned one. Such a piece is read from one
+  // element earlier, with the dword that follows, and shifted; no branch, and the extra dword of a
+  // piece that needs none is its own last one, so nothing past the piece is touched.
+  const uint32_t odd = (uint32_t)(reinterpret_cast<uintptr_t>(s) >> 1) & 1u;
+  const uint32_t* q = reinterpret_cast<const uint32_t*>(s - odd);
+  const u32x4 v = *reinterpret_cast<const u32x4_a4*>(q);
+  const uint32_t x = q[3 + odd];
+  const uint32_t sh = odd << 4;
+  u32x4 r;
+  r.x = __builtin_amdgcn_alignbit(v.y, v.x, sh);
+  r.y = __builtin_amdgcn_alignbit(v.z, v.y, sh);
+  r.z = __builtin_amdgcn_alignbit(v.w, v.z, sh);
+  r.w = __builtin_amdgcn_alignbit(x, v.w, sh);
+  return r;
 }
 
 // Store 16 bytes to an address that is only sizeof(T)-aligned.
@@ -348,7 +395,6 @@ __global__ __launch_bounds__(256) void fold_kernel(typename Arith<DT>::T* __rest
                                                    Table tab, Geom g, I total) {
   typedef typename Arith<DT>::T T;
   constexpr int V = Bits<T>::V;
-  constexpr T ABS = (T)(~(T(1) << (sizeof(T) * 8 - 1)));
   const I nvec = (total + V - 1) / V;
   const int D = g.n[0], H = g.n[1], W = g.n[2];
   const int Ha = g.lo[1] + H + g.hi[1];
@@ -372,12 +418,10 @@ __global__ __launch_bounds__(256) void fold_kernel(typename Arith<DT>::T* __rest
       long long off = ((p * Da + (d + g.lo[0])) * Ha + (h + g.lo[1])) * (long long)Wa +
                       (w + g.lo[2]);
       u32x4 val = load16_unaligned<T>(own + off);
-      T tmp[V];
-      __builtin_memcpy(tmp, &val, 16);
-#pragma unroll
-      for (int i = 0; i < V; ++i)
-        if ((tmp[i] & ABS) == 0) tmp[i] = 0;
-      __builtin_memcpy(&val, tmp, 16);
+      val.x = zero_plus<T>(val.x);
+      val.y = zero_plus<T>(val.y);
+      val.z = zero_plus<T>(val.z);
+      val.w = zero_plus<T>(val.w);
       *reinterpret_cast<u32x4*>(dst + e0) = val;
     } else {
       T tmp[V];
@@ -458,9 +502,18 @@ __global__ __launch_bounds__(256) void assemble_rows_kernel(Table tab, T* __rest
   region(ha, g.lo[1], g.n[1], g.hi[1], rh, ch, eh);
   const long long line = ((long long)pp * ed + cd) * eh + ch;  // row index inside a source
   const int base_idx = rd * 9 + rh * 3;
-  const T* s0 = static_cast<const T*>(table_entry(base_idx + 0));
-  const T* s1 = static_cast<const T*>(table_entry(base_idx + 1));
-  const T* s2 = static_cast<const T*>(table_entry(base_idx + 2));
+  // Rows of the tile itself (all but the halo rows): their three sources are table entries
+  // with constant indices, which are scalar loads done once at the head of the kernel. Only
+  // the halo rows look the table up with a per-lane index, a trip to memory that the row's
+  // own loads would have to wait for.
+  const T* s0 = static_cast<const T*>(tab.p[12]);
+  const T* s1 = static_cast<const T*>(tab.p[13]);
+  const T* s2 = static_cast<const T*>(tab.p[14]);
+  if (base_idx != 12) {
+    s0 = static_cast<const T*>(table_entry(base_idx + 0));
+    s1 = static_cast<const T*>(table_entry(base_idx + 1));
+    s2 = static_cast<const T*>(table_entry(base_idx + 2));
+  }
   if (s0 != nullptr) s0 += line * g.lo[2];
   if (s1 != nullptr) s1 += line * g.n[2];
   if (s2 != nullptr) s2 += line * g.hi[2];
@@ -560,9 +613,18 @@ __global__ __launch_bounds__(256) void assemble_frame_kernel(Table tab, T* __res
   region(ha, g.lo[1], g.n[1], g.hi[1], rh, ch, eh);
   const long long line = ((long long)pp * ed + cd) * eh + ch;
   const int base_idx = rd * 9 + rh * 3;
-  const T* s0 = static_cast<const T*>(table_entry(base_idx + 0));
-  const T* s1 = static_cast<const T*>(table_entry(base_idx + 1));
-  const T* s2 = static_cast<const T*>(table_entry(base_idx + 2));
+  // Rows of the tile itself (all but the halo rows): their three sources are table entries
+  // with constant indices, which are scalar loads done once at the head of the kernel. Only
+  // the halo rows look the table up with a per-lane index, a trip to memory that the row's
+  // own loads would have to wait for.
+  const T* s0 = static_cast<const T*>(tab.p[12]);
+  const T* s1 = static_cast<const T*>(tab.p[13]);
+  const T* s2 = static_cast<const T*>(tab.p[14]);
+  if (base_idx != 12) {
+    s0 = static_cast<const T*>(table_entry(base_idx + 0));
+    s1 = static_cast<const T*>(table_entry(base_idx + 1));
+    s2 = static_cast<const T*>(table_entry(base_idx + 2));
+  }
   if (s0 != nullptr) s0 += line * g.lo[2];
   if (s1 != nullptr) s1 += line * g.n[2];
   if (s2 != nullptr) s2 += line * g.hi[2];
@@ -743,7 +805,6 @@ __global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
                                                         Geom g, RowPlan pl, bool defer_border) {
   typedef typename Arith<DT>::T T;
   constexpr int V = Bits<T>::V;
-  constexpr T ABS = (T)(~(T(1) << (sizeof(T) * 8 - 1)));
   const uint32_t t = blockIdx.x * 256u + threadIdx.x;
   const uint32_t row = t >> pl.lpr_log2;
   if (row >= pl.nrows) return;
@@ -799,9 +860,28 @@ __global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
   const int lpr_mask = (1 << pl.lpr_log2) - 1;
   const bool thin = g.hi[2] == 1 && g.lo[2] == 1 && n_vec >= 2;
   const bool owns_first = thin && lir == 0, owns_last = thin && lir == ((n_vec - 1) & lpr_mask);
+  // One load instruction for both: the lane that owns the first vector reads the lower strip,
+  // the lane that owns the last one the upper strip (a row with a single vector per lane
+  // group has one lane that owns both; it takes the second value with a load of its own).
   T strip_first = T(0), strip_last = T(0);
-  if (owns_first && s_lo != nullptr) strip_first = s_lo[0];
-  if (owns_last && s_hi != nullptr) strip_last = s_hi[W - 1 - up0];
+  // A whole wavefront per row: the row and with it the two addresses are the same in every
+  // lane, so the two values come through the scalar cache (the aligned dword that holds the
+  // element) and cost the vector memory pipeline nothing. They are fetched below, behind the
+  // first batch of vector loads, whose latency covers the wait.
+  const bool by_scalar = thin && pl.lpr_log2 == 6;
+  const long long row_u = (long long)__builtin_amdgcn_readfirstlane((int)row);
+  const T* const base_lo = by_scalar && row_plain ? static_cast<const T*>(table_entry(9 + 3 + 0)) : nullptr;
+  const T* const base_hi = by_scalar && row_plain ? static_cast<const T*>(table_entry(9 + 3 + 2)) : nullptr;
+  if (!by_scalar) {
+    const T* sp = nullptr;
+    if (owns_first && s_lo != nullptr) sp = s_lo;
+    else if (owns_last && s_hi != nullptr) sp = s_hi + (W - 1 - up0);
+    T got = T(0);
+    if (sp != nullptr) got = *sp;
+    if (owns_first) strip_first = got;
+    else strip_last = got;
+    if (owns_first && owns_last && s_hi != nullptr) strip_last = s_hi[W - 1 - up0];
+  }
   auto ends = [&](T lower, T own_bits, T upper, bool has_lower, bool has_upper) {
     float acc = 0.0f;
     if (has_lower) acc = Arith<DT>::up(Arith<DT>::down(acc + Arith<DT>::up(lower)));
@@ -817,24 +897,33 @@ __global__ __launch_bounds__(256) void fold_rows_kernel(Table tab,
       val[u] = u32x4{0u, 0u, 0u, 0u};
       if (j < n_vec) val[u] = load16_unaligned<T>(orow + j * V);
     }
+    if (by_scalar && it0 == 0) {
+      if (base_lo != nullptr) strip_first = uniform_element(base_lo + row_u * g.hi[2]);
+      if (base_hi != nullptr) strip_last = uniform_element(base_hi + row_u * g.lo[2] + (W - 1 - up0));
+    }
 #pragma unroll
     for (int u = 0; u < ROW_BATCH; ++u) {
       const int j = lir + ((it0 + u) << pl.lpr_log2);
       if (j < n_vec) {
-        T tmp[V];
-        __builtin_memcpy(tmp, &val[u], 16);
         const int c0 = j * V;
-        const T first_bits = tmp[0], last_bits = tmp[V - 1];
+        constexpr int EB = (int)sizeof(T) * 8;
+        const T first_bits = (T)val[u].x, last_bits = (T)(val[u].w >> (32 - EB));
         // `0 + own` for every column; then the two columns of a thin halo get their ordered sum
         // (wider halos: below). Running the ordered sum for all 8 elements of the first and of the
         // last vector, one lane active, was three quarters of the kernel's instructions.
-#pragma unroll
-        for (int e = 0; e < V; ++e)
-          if ((tmp[e] & ABS) == 0) tmp[e] = 0;
-        if (owns_first && j == 0) tmp[0] = ends(strip_first, first_bits, T(0), s_lo != nullptr, false);
-        if (owns_last && j == n_vec - 1 && n_vec * V == W) tmp[V - 1] = ends(T(0), last_bits, strip_last, false, s_hi != nullptr);
         u32x4 out;
-        __builtin_memcpy(&out, tmp, 16);
+        out.x = zero_plus<T>(val[u].x);
+        out.y = zero_plus<T>(val[u].y);
+        out.z = zero_plus<T>(val[u].z);
+        out.w = zero_plus<T>(val[u].w);
+        if (owns_first && j == 0) {
+          const uint32_t e = (uint32_t)ends(strip_first, first_bits, T(0), s_lo != nullptr, false);
+          out.x = EB == 32 ? e : ((out.x & 0xffff0000u) | e);
+        }
+        if (owns_last && j == n_vec - 1 && n_vec * V == W) {
+          const uint32_t e = (uint32_t)ends(T(0), last_bits, strip_last, false, s_hi != nullptr);
+          out.w = EB == 32 ? e : ((out.w & 0x0000ffffu) | (e << 16));
+        }
         *reinterpret_cast<u32x4_s4*>(drow + c0) = out;
       }
     }
