@@ -19,6 +19,7 @@ that talks to other ranks), and assembles the padded tile in one pass.
 from __future__ import annotations
 
 import ctypes
+import math
 from collections.abc import Sequence
 from typing import Any, Protocol
 
@@ -184,12 +185,67 @@ def _embed_weight(w: torch.Tensor, off) -> torch.Tensor:
 # between its cells (backward). Costs prod(stride) times the matrix-core work of the strided
 # layer and a copy, and still beats the FMA kernels by an order of magnitude.
 # --------------------------------------------------------------------------- #
-def _dense_stride_ok(kernel, stride, dilation) -> bool:
+def _dense_stride_ok(kernel, stride, dilation, padding=None) -> bool:
     if len(kernel) not in (2, 3) or all(s == 1 for s in stride):
         return False
-    if any(k not in (1, 3) for k in kernel) or any(d != 1 for d in dilation):
+    if any(k not in (1, 3) for k in kernel):
+        return False
+    if any(d != 1 for d in dilation) and (padding is None or not _dilated_ok(kernel, (1,) * len(kernel), padding, dilation)):
         return False
     return not all(k == s for k, s in zip(kernel, stride))  # kernel = stride has its own route
+
+
+# --------------------------------------------------------------------------- #
+# Dilated 3-tap kernels at stride 1 whose padding is a multiple of the dilation ("same" padding
+# p = d, and the halo-padded tile with p = 0): output cell d * o + r reads input cells
+# d * (o + t - p / d) + r, so the cells of one residue r form a plain 3-tap convolution of
+# their own. The prod(dilation) residue images go into the batch, the undilated MFMA kernels
+# run once over all of them, and the result is interleaved back: the same arithmetic, two
+# permutation copies per tensor.
+# --------------------------------------------------------------------------- #
+def _dilated_ok(kernel, stride, padding, dilation) -> bool:
+    if len(kernel) not in (2, 3) or any(s != 1 for s in stride):
+        return False
+    if any(k not in (1, 3) for k in kernel):
+        return False
+    if not any(d > 1 and k == 3 for k, d in zip(kernel, dilation)):
+        return False
+    return all(p % d == 0 for k, p, d in zip(kernel, padding, dilation) if d > 1 and k == 3)
+
+
+def _phase_counts(kernel, dilation) -> tuple:
+    return tuple(int(d) if k == 3 else 1 for k, d in zip(kernel, dilation))
+
+
+def _to_phases(t: torch.Tensor, phases, ext) -> torch.Tensor:
+    """``(N, C, *spatial) -> (prod(phases) * N, C, *ext)``: image ``r`` of an axis holds the cells
+    ``r, r + P, r + 2 P, ...`` of that axis, zero beyond the tensor's end."""
+    n = len(phases)
+    full = tuple(e * p for e, p in zip(ext, phases))
+    if tuple(t.shape[2:]) != full:
+        grown = torch.zeros((t.shape[0], t.shape[1], *full), dtype=t.dtype, device=t.device)
+        keep = tuple(slice(0, min(a, b)) for a, b in zip(t.shape[2:], full))
+        grown[(slice(None), slice(None)) + keep] = t[(slice(None), slice(None)) + keep]
+        t = grown
+    shape = [t.shape[0], t.shape[1]]
+    for e, p in zip(ext, phases):
+        shape += [e, p]
+    t = t.reshape(shape)
+    p_dims = [3 + 2 * i for i in range(n)]
+    e_dims = [2 + 2 * i for i in range(n)]
+    return t.permute(*p_dims, 0, 1, *e_dims).reshape(-1, shape[1], *ext)
+
+
+def _from_phases(tb: torch.Tensor, phases, batch, sizes) -> torch.Tensor:
+    """Inverse of :func:`_to_phases`, cut to ``sizes``."""
+    n = len(phases)
+    ext = tuple(tb.shape[2:])
+    t = tb.reshape(*phases, batch, tb.shape[1], *ext)
+    perm = [n, n + 1]
+    for i in range(n):
+        perm += [n + 2 + i, i]
+    t = t.permute(perm).reshape(batch, tb.shape[1], *(e * p for e, p in zip(ext, phases)))
+    return t[(slice(None), slice(None)) + tuple(slice(0, v) for v in sizes)].contiguous()
 
 
 def _stuffed(g: torch.Tensor, dense_sp, stride) -> torch.Tensor:
@@ -210,10 +266,16 @@ def conv_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1) -> torch
     if x.shape[1] != w.shape[1]:
         raise RuntimeError(f"expected input to have {w.shape[1]} channels, but got {x.shape[1]} channels instead")
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
-    if _dense_stride_ok(tuple(w.shape[2:]), stride, dilation):
+    if _dense_stride_ok(tuple(w.shape[2:]), stride, dilation, padding):
         out_sp = _out_spatial(x.shape[2:], w.shape[2:], stride, padding, dilation)
-        dense = conv_nd(x, w, b, stride=1, padding=padding)
+        dense = conv_nd(x, w, b, stride=1, padding=padding, dilation=dilation)
         return dense[(slice(None), slice(None)) + tuple(slice(0, (o - 1) * s + 1, s) for o, s in zip(out_sp, stride))].contiguous()
+    if _dilated_ok(tuple(w.shape[2:]), stride, padding, dilation):
+        phases = _phase_counts(w.shape[2:], dilation)
+        out_sp = _out_spatial(x.shape[2:], w.shape[2:], stride, padding, dilation)
+        ext_in = tuple(-(-int(i) // p) for i, p in zip(x.shape[2:], phases))
+        yb = conv_nd(_to_phases(x, phases, ext_in), w, b, stride=1, padding=tuple(pp // p for pp, p in zip(padding, phases)))
+        return _from_phases(yb, phases, x.shape[0], out_sp)
     off = _embed3(tuple(w.shape[2:]), stride, dilation)
     if off is not None:
         return conv_nd(x, _embed_weight(w, off), b, stride=1, padding=tuple(p + o for p, o in zip(padding, off)))
@@ -244,9 +306,20 @@ def conv_nd_input(input_shape, w, g, *, stride=1, padding=0, dilation=1, groups=
     if g.dtype != w.dtype:
         raise RuntimeError(f"grad_output type ({g.dtype}) and weight type ({w.dtype}) should be the same")
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
-    if _dense_stride_ok(tuple(w.shape[2:]), stride, dilation):
+    if _dense_stride_ok(tuple(w.shape[2:]), stride, dilation, padding):
         dense_sp = _out_spatial(input_shape[2:], w.shape[2:], (1,) * n, padding, dilation)
-        return conv_nd_input(input_shape, w, _stuffed(g, dense_sp, stride), stride=1, padding=padding)
+        return conv_nd_input(input_shape, w, _stuffed(g, dense_sp, stride), stride=1, padding=padding, dilation=dilation)
+    if _dilated_ok(tuple(w.shape[2:]), stride, padding, dilation):
+        phases = _phase_counts(w.shape[2:], dilation)
+        out_sp = _out_spatial(input_shape[2:], w.shape[2:], stride, padding, dilation)
+        if tuple(g.shape) != (input_shape[0], w.shape[0], *out_sp):
+            raise ValueError(f"grad_output shape {tuple(g.shape)} does not match the convolution of an input of shape {input_shape}")
+        ext_in = tuple(-(-i // p) for i, p in zip(input_shape[2:], phases))
+        pad0 = tuple(pp // p for pp, p in zip(padding, phases))
+        ext_out = _out_spatial(ext_in, w.shape[2:], (1,) * n, pad0, (1,) * n)
+        gxb = conv_nd_input((g.shape[0] * math.prod(phases), input_shape[1], *ext_in), w, _to_phases(g, phases, ext_out),
+                            stride=1, padding=pad0)
+        return _from_phases(gxb, phases, input_shape[0], input_shape[2:])
     off = _embed3(tuple(w.shape[2:]), stride, dilation)
     if off is not None:
         return conv_nd_input(input_shape, _embed_weight(w, off), g, stride=1,
@@ -414,10 +487,21 @@ def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, group
     if x.dtype != g.dtype:
         raise RuntimeError(f"input type ({x.dtype}) and grad_output type ({g.dtype}) should be the same")
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
-    if _dense_stride_ok(weight_shape[2:], stride, dilation):
+    if _dense_stride_ok(weight_shape[2:], stride, dilation, padding):
         dense_sp = _out_spatial(x.shape[2:], weight_shape[2:], (1,) * n, padding, dilation)
-        return conv_nd_weight(x, weight_shape, _stuffed(g, dense_sp, stride), stride=1, padding=padding,
+        return conv_nd_weight(x, weight_shape, _stuffed(g, dense_sp, stride), stride=1, padding=padding, dilation=dilation,
                               with_bias_grad=with_bias_grad)
+    if _dilated_ok(weight_shape[2:], stride, padding, dilation):
+        phases = _phase_counts(weight_shape[2:], dilation)
+        out_sp = _out_spatial(x.shape[2:], weight_shape[2:], stride, padding, dilation)
+        if tuple(g.shape) != (x.shape[0], weight_shape[0], *out_sp) or x.shape[1] != weight_shape[1]:
+            raise ValueError(f"grad_output {tuple(g.shape)} / input {tuple(x.shape)} do not match weight {weight_shape}")
+        ext_in = tuple(-(-int(i) // p) for i, p in zip(x.shape[2:], phases))
+        pad0 = tuple(pp // p for pp, p in zip(padding, phases))
+        ext_out = _out_spatial(ext_in, weight_shape[2:], (1,) * n, pad0, (1,) * n)
+        # every residue image is one more batch entry of the undilated layer: the sum over the batch is the answer
+        return conv_nd_weight(_to_phases(x, phases, ext_in), weight_shape, _to_phases(g, phases, ext_out), stride=1,
+                              padding=pad0, with_bias_grad=with_bias_grad)
     off = _embed3(weight_shape[2:], stride, dilation)
     if off is not None:
         # gradient of the 3 x 3 (x 3) kernel the weights sit in; its centre taps are the answer

@@ -76,6 +76,7 @@ struct WgradParams {
   int pad_d, pad_h, pad_w;
   int row_pairs, col_tiles;
   long long total_stages;  // N * Dout * col_tiles * row_pairs
+  int w_first, w_last;     // what a stage of the first / last column strip costs, in stages of the other strips
 };
 
 // Wavefronts per workgroup: (g block, x block) pairs x 2 column halves; a 6-wavefront
@@ -95,9 +96,15 @@ __device__ __forceinline__ float sum_bf16x8(const u32x4& v) {
 }
 
 // F16: x and g hold fp16 instead of bf16 (v_mfma_f32_32x32x16_f16); the partial sums are fp32 either way.
-template <int CGB, int CXB, bool EVEN, bool FRAMED, bool F16 = false>
+// EVEN: 0 = no assumption about the rows (every load checks its bounds), 1 = even row lengths,
+// 4-byte aligned tensors and an even padding across W, so that a stage's windows start on dwords and
+// the 16-byte vector loads apply, 2 = the same with an odd padding: the x window is staged from one
+// pixel earlier, where it is dword aligned again, and the fragments are built one pixel further in.
+template <int CGB, int CXB, int EVEN, bool FRAMED, bool F16 = false>
 __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(WgradParams p) {
   constexpr int THREADS = wgrad_threads(CGB, CXB);
+  constexpr int LEAD = EVEN == 2 ? 1 : 0;
+  static_assert(!(FRAMED && EVEN != 1), "the framed input is read with even windows only");
   constexpr int CWAVES = CGB * CXB * HALVES;  // wavefronts that own accumulators
   constexpr int GC = 32 * CGB, XC = 32 * CXB;
   constexpr int G_BYTES = GC * G_CH;          // one g buffer
@@ -119,10 +126,29 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
   // Workgroups are dealt to the 8 XCDs round robin; the ranges are numbered so that one
   // XCD holds neighbouring column strips, whose x rows share cache lines in that XCD's L2.
   const unsigned wg_rank = gridDim.x % 8 == 0 ? (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8 : blockIdx.x;
-  const long long per = (p.total_stages + gridDim.x - 1) / gridDim.x;
-  const long long s_begin = per * wg_rank;
-  long long s_end = s_begin + per;
-  if (s_end > p.total_stages) s_end = p.total_stages;
+  // The ranges hold equal cost, not equal counts: the stages of a column strip whose windows
+  // stick out of the tensor (or whose last columns do not exist) load with bounds checks and
+  // take about twice as long, and a workgroup whose whole range lay in such a strip would set
+  // the kernel's time. Cost runs like the stages: per plane the first strip at w_first a
+  // stage, the middle strips at 1, the last at w_last; with both at 1 the ranges are counts.
+  const long long strip_first = (long long)p.row_pairs * p.w_first;
+  const long long strip_mid = (long long)p.row_pairs * (p.col_tiles > 2 ? p.col_tiles - 2 : 0);
+  const long long strip_last = p.col_tiles > 1 ? (long long)p.row_pairs * p.w_last : 0;
+  const long long plane_cost = strip_first + strip_mid + strip_last;
+  const long long plane_stages = (long long)p.row_pairs * p.col_tiles;
+  const long long total_cost = (p.total_stages / plane_stages) * plane_cost;
+  auto stage_at = [&](long long cost) -> long long {
+    if (cost >= total_cost) return p.total_stages;
+    const long long pl = cost / plane_cost, rem = cost - pl * plane_cost;
+    long long st;
+    if (rem < strip_first) st = rem / p.w_first;
+    else if (rem < strip_first + strip_mid) st = p.row_pairs + (rem - strip_first);
+    else st = (long long)p.row_pairs * (p.col_tiles - 1) + (rem - strip_first - strip_mid) / p.w_last;
+    return pl * plane_stages + st;
+  };
+  const long long per = (total_cost + gridDim.x - 1) / gridDim.x;
+  const long long s_begin = stage_at(per * wg_rank);
+  const long long s_end = stage_at(per * (wg_rank + 1));
 
   const size_t plane_x = (size_t)p.Hin * p.Win, plane_g = (size_t)p.Hout * p.Wout;
   const size_t x_cs = plane_x * p.Din, g_cs = plane_g * p.Dout;  // channel strides
@@ -155,7 +181,8 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
       c_lds[rd] = 0;
     }
   }
-  // pixels 64, 65 of an x row: one dword, carried by the first 2 * XC threads
+  // pixels 64, 65 of an x row (and 66, 67 of a window staged one pixel early): one or two dwords,
+  // carried by the first 2 * XC threads
   const bool has_tail = tid < 2 * XC;
   uint32_t t_goff = 0, t_lds = 0;
   if (has_tail) {
@@ -195,6 +222,7 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
   struct Staged {
     u32x4 v[ROUNDS];
     uint32_t tail;
+    uint32_t tail_b;  // LEAD only
   };
 
   // Loads of one stage into `v`: its two g rows (want_g) and one pair of its x rows
@@ -231,14 +259,15 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
     u32x4 (&v)[ROUNDS] = sg.v;
     const int hp = cur.hp, ct = cur.ct, od = cur.od, n = cur.n;
     const int oh0 = hp * SR, ow0 = ct * SW;
-    const int id0 = od - p.pad_d, ih0 = oh0 - p.pad_h + 2 * xpair, iw0 = ow0 - p.pad_w;
+    const int id0 = od - p.pad_d, ih0 = oh0 - p.pad_h + 2 * xpair, iw0 = ow0 - p.pad_w - LEAD;
     const char* g_org = reinterpret_cast<const char*>(p.g) +
                         2 * (((size_t)n * p.cout_total * p.Dout + od) * plane_g + (size_t)oh0 * p.Wout + ow0);
     const char* x_org = reinterpret_cast<const char*>(p.x) +
                         2 * ((ptrdiff_t)((size_t)n * p.cin_total * p.Din * plane_x) + (ptrdiff_t)id0 * (ptrdiff_t)plane_x +
                              (ptrdiff_t)ih0 * p.Win + iw0);
-    const bool inside = EVEN && oh0 + SR <= p.Hout && ow0 + SW <= p.Wout && ih0 >= 0 &&
-                        ih0 + 2 <= p.Hin && iw0 >= 0 && iw0 + SW + 2 <= p.Win && id0 >= 0 &&
+    // (with LEAD the window's last dword holds one pixel more than is used; it shares its dword with one that is)
+    const bool inside = EVEN != 0 && oh0 + SR <= p.Hout && ow0 + SW <= p.Wout && ih0 >= 0 &&
+                        ih0 + 2 <= p.Hin && iw0 >= 0 && iw0 + SW + 2 + LEAD <= p.Win && id0 >= 0 &&
                         id0 + (XC / p.Cin) <= p.Din;
     if (FRAMED && inside) {
       // Rows and columns of the pair's window inside the own tile (wave-uniform): a chunk
@@ -323,6 +352,7 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
         if (want_g || !g_round) v[rd] = *reinterpret_cast<const u32x4_a4*>((g_round ? g_org : x_org) + c_goff[rd]);
       }
       sg.tail = *reinterpret_cast<const uint32_t*>(x_org + t_goff);
+      if (LEAD) sg.tail_b = *reinterpret_cast<const uint32_t*>(x_org + t_goff + 4);
     } else {
 #pragma unroll
       for (int rd = 0; rd < ROUNDS; ++rd) {
@@ -364,12 +394,14 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
         const int r2 = tid & 1, ch = tid >> 1;
         const int row = ih0 + r2, col = iw0 + SW, dd = id0 + ch / p.Cin;
         const uint16_t* src = reinterpret_cast<const uint16_t*>(x_org + t_goff);
-        uint32_t lo = 0u, hi = 0u;
+        uint32_t e[4] = {0u, 0u, 0u, 0u};
         if (dd >= 0 && dd < p.Din && row >= 0 && row < p.Hin) {
-          if (col >= 0 && col < p.Win) lo = src[0];
-          if (col + 1 >= 0 && col + 1 < p.Win) hi = src[1];
+#pragma unroll
+          for (int k = 0; k < 2 + 2 * LEAD; ++k)
+            if (col + k >= 0 && col + k < p.Win) e[k] = src[k];
         }
-        sg.tail = lo | (hi << 16);
+        sg.tail = e[0] | (e[1] << 16);
+        sg.tail_b = e[2] | (e[3] << 16);
       }
     }
   };
@@ -394,7 +426,11 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
         *reinterpret_cast<u32x4*>(lds_x + c_lds[rd] + slot * X_ROW) = v[rd];
       }
     }
-    if (has_tail) *reinterpret_cast<uint32_t*>(lds_x + t_lds + ((tid & 1) ? slot_b : slot_a) * X_ROW) = sg.tail;
+    if (has_tail) {
+      unsigned char* at = lds_x + t_lds + ((tid & 1) ? slot_b : slot_a) * X_ROW;
+      *reinterpret_cast<uint32_t*>(at) = sg.tail;
+      if (LEAD) *reinterpret_cast<uint32_t*>(at + 4) = sg.tail_b;
+    }
   };
 
   f32x16 acc[3][3];
@@ -421,19 +457,26 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
       if (slot >= RING) slot -= RING;
       u32x4 d = *reinterpret_cast<const u32x4*>(xb + slot * X_ROW + cg * 32);
       uint32_t d4 = *reinterpret_cast<const uint32_t*>(xb + slot * X_ROW + cg * 32 + 16);
+      uint32_t d5 = 0u;
+      if (LEAD) d5 = *reinterpret_cast<const uint32_t*>(xb + slot * X_ROW + cg * 32 + 20);
       // The values are made opaque so that the kw = 2 fragment below is built with register
       // moves: left alone, the compiler reads it again from LDS at a 4-byte offset, as dword
       // pairs whose 880-byte lane stride runs into 4-way bank conflicts.
-      asm("" : "+v"(d), "+v"(d4));
+      asm("" : "+v"(d), "+v"(d4), "+v"(d5));
       u32x4 s1, s2;
       s1.x = __builtin_amdgcn_alignbit(d.y, d.x, 16);
       s1.y = __builtin_amdgcn_alignbit(d.z, d.y, 16);
       s1.z = __builtin_amdgcn_alignbit(d.w, d.z, 16);
       s1.w = __builtin_amdgcn_alignbit(d4, d.w, 16);
       s2.x = d.y; s2.y = d.z; s2.z = d.w; s2.w = d4;
-      const bf16x8 b0 = __builtin_bit_cast(bf16x8, d);
-      const bf16x8 b1 = __builtin_bit_cast(bf16x8, s1);
-      const bf16x8 b2 = __builtin_bit_cast(bf16x8, s2);
+      u32x4 s3;  // LEAD: the window was staged one pixel early, the taps sit one pixel further in
+      s3.x = __builtin_amdgcn_alignbit(d.z, d.y, 16);
+      s3.y = __builtin_amdgcn_alignbit(d.w, d.z, 16);
+      s3.z = __builtin_amdgcn_alignbit(d4, d.w, 16);
+      s3.w = __builtin_amdgcn_alignbit(d5, d4, 16);
+      const bf16x8 b0 = __builtin_bit_cast(bf16x8, LEAD ? s1 : d);
+      const bf16x8 b1 = __builtin_bit_cast(bf16x8, LEAD ? s2 : s1);
+      const bf16x8 b2 = __builtin_bit_cast(bf16x8, LEAD ? s3 : s2);
 #pragma unroll
       for (int r = 0; r < SR; ++r) {
         const int kh = rho - r;
@@ -660,16 +703,18 @@ bool blocks_of(const ConvGeom& g, Blocking* b) {
 int block_width(int total, int c0, int first) { return (first == 64 && total - c0 > 32) ? 64 : 32; }
 
 template <int CGB, int CXB>
-int launch(const WgradParams& p, bool even, bool f16, int wgs, hipStream_t s, const char* who) {
+int launch(const WgradParams& p, int even, bool f16, int wgs, hipStream_t s, const char* who) {
   constexpr int THREADS = wgrad_threads(CGB, CXB);
   const size_t lds = 2 * (size_t)(32 * CGB * G_CH) + (size_t)(32 * CXB * X_CH);
   void (*kern)(WgradParams);
   if (f16)  // never framed (checked by the caller)
-    kern = even ? &wgrad3x3_mfma_kernel<CGB, CXB, true, false, true> : &wgrad3x3_mfma_kernel<CGB, CXB, false, false, true>;
+    kern = even == 1 ? &wgrad3x3_mfma_kernel<CGB, CXB, 1, false, true>
+                     : (even == 2 ? &wgrad3x3_mfma_kernel<CGB, CXB, 2, false, true> : &wgrad3x3_mfma_kernel<CGB, CXB, 0, false, true>);
   else if (p.xt != nullptr)
-    kern = &wgrad3x3_mfma_kernel<CGB, CXB, true, true>;  // the framed input needs the even layout (checked by the caller)
+    kern = &wgrad3x3_mfma_kernel<CGB, CXB, 1, true>;  // the framed input needs the even layout (checked by the caller)
   else
-    kern = even ? &wgrad3x3_mfma_kernel<CGB, CXB, true, false> : &wgrad3x3_mfma_kernel<CGB, CXB, false, false>;
+    kern = even == 1 ? &wgrad3x3_mfma_kernel<CGB, CXB, 1, false>
+                     : (even == 2 ? &wgrad3x3_mfma_kernel<CGB, CXB, 2, false> : &wgrad3x3_mfma_kernel<CGB, CXB, 0, false>);
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", who, lds);
@@ -788,10 +833,11 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
     x = xs;
     go = gs;
   }
-  const bool even = (g.in[2] % 2 == 0) && (g.p[2] % 2 == 0) && (g.out[2] % 2 == 0) &&
-                    ((reinterpret_cast<uintptr_t>(x) & 3) == 0) &&
-                    ((reinterpret_cast<uintptr_t>(go) & 3) == 0);
-  if (xt != nullptr && (!even || !mfma_wgrad_frame_ok(g, tlo, tn)))
+  // 0, 1 or 2: the EVEN mode of the kernel (2: odd padding across W, windows staged one pixel early)
+  const bool even_rows = (g.in[2] % 2 == 0) && (g.out[2] % 2 == 0) && ((reinterpret_cast<uintptr_t>(x) & 3) == 0) &&
+                         ((reinterpret_cast<uintptr_t>(go) & 3) == 0);
+  const int even = !even_rows ? 0 : (g.p[2] % 2 == 0 ? 1 : 2);
+  if (xt != nullptr && (even != 1 || !mfma_wgrad_frame_ok(g, tlo, tn)))
     JG_FAIL(JG_ERR_UNSUPPORTED, "%s: the framed input does not cover this geometry / alignment", who);
   // part products (g part, x part), smallest first; plain mode: the one product
   static const int kPairs[6][2] = {{0, 2}, {1, 1}, {2, 0}, {0, 1}, {1, 0}, {0, 0}};
@@ -814,6 +860,20 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
   p.row_pairs = (g.out[1] + SR - 1) / SR;
   p.col_tiles = (g.out[2] + SW - 1) / SW;
   p.total_stages = stage_count(g);
+  {
+    // column strips outside the kernel's vector-load path (see the kernel's `inside`)
+    const int last_ow0 = (p.col_tiles - 1) * SW;
+    const bool first_slow = g.p[2] > 0;
+    const int lead = even == 2 ? 1 : 0;
+    const bool last_slow = last_ow0 + SW > g.out[2] || last_ow0 - g.p[2] - lead + SW + 2 + lead > g.in[2];
+    p.w_first = p.w_last = 1;
+    // measured: such a stage costs about four plain ones; 3 gave the shortest kernels over the shapes tried
+    constexpr int SLOW = 3;
+    if (even) {  // without the even layout every stage takes that path
+      if (p.col_tiles == 1) p.w_first = (first_slow || last_slow) ? SLOW : 1;
+      else { p.w_first = first_slow ? SLOW : 1; p.w_last = last_slow ? SLOW : 1; }
+    }
+  }
   const int wgs = wg_count(p.total_stages);
   p.xt = static_cast<const uint16_t*>(xt);
   p.tlo_d = tlo ? tlo[0] : 0; p.tlo_h = tlo ? tlo[1] : 0; p.tlo_w = tlo ? tlo[2] : 0;

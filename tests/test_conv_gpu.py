@@ -43,6 +43,11 @@ PRIM_CASES = [
     (2, 32, 32, (20, 128), (3, 3), (1, 1), (1, 1), (1, 1)),
     (1, 64, 64, (35, 192), (3, 3), (1, 1), (0, 0), (1, 1)),
     (1, 32, 16, (4, 18, 64), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+    # weight gradient: several stages per workgroup with column strips of unequal cost (windows that stick out
+    # across W, a last strip with fewer columns), odd padding across even rows (staged one pixel early)
+    (2, 64, 64, (150, 330), (3, 3), (1, 1), (1, 1), (1, 1)),
+    (2, 32, 32, (140, 200), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (1, 32, 32, (5, 40, 136), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
     # channel counts beyond one group of LDS-resident weights, and produced channels that are
     # not a multiple of the 32-row MFMA tile (padded with zero weight rows, not stored)
     (1, 128, 128, (20, 70), (3, 3), (1, 1), (1, 1), (1, 1)),
@@ -73,6 +78,15 @@ PRIM_CASES = [
     (1, 8, 8, (20, 31), (3, 3), (2, 3), (0, 1), (1, 1)),
     (1, 8, 16, (7, 12, 18), (3, 3, 3), (2, 2, 2), (1, 1, 1), (1, 1, 1)),
     (2, 8, 8, (16, 16), (1, 1), (2, 2), (0, 0), (1, 1)),
+    # dilated 3-tap kernels whose padding is a multiple of the dilation: the residue images as batch
+    # entries of the undilated MFMA kernels (extents that the dilation does and does not divide)
+    (2, 32, 64, (33, 47), (3, 3), (1, 1), (2, 3), (2, 3)),
+    (1, 64, 64, (40, 64), (3, 3), (1, 1), (0, 0), (2, 2)),
+    (2, 16, 8, (21, 30), (3, 3), (1, 1), (4, 0), (2, 1)),
+    (1, 8, 16, (9, 3), (3, 1), (1, 1), (4, 0), (4, 5)),
+    (1, 32, 32, (6, 19, 34), (3, 3, 3), (1, 1, 1), (1, 2, 2), (1, 2, 2)),
+    (2, 16, 32, (33, 40), (3, 3), (2, 2), (2, 2), (2, 2)),   # strided and dilated
+    (1, 4, 6, (17, 23), (3, 3), (1, 1), (1, 1), (2, 2)),     # padding not a multiple: the direct kernels
 ]
 
 
