@@ -19,43 +19,52 @@ struct RollArgs {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-template <typename T>
+// I: the index arithmetic's type, int where the word count allows it: a 64-bit division is some
+// hundred instructions, and with one per axis and word they, not the memory, set the kernel's time.
+template <typename I>
+__device__ __forceinline__ I rolled_source(const RollArgs& a, I i) {
+  I rem = i, so = 0, stride = 1;
+#pragma unroll
+  for (int k = kMaxDims - 1; k >= 0; --k) {
+    if (k < a.nd) {
+      const I size = (I)a.size[k];
+      const I q = rem / size;
+      const I c = rem - q * size;
+      rem = q;
+      I sc = c - (I)a.shift[k];
+      if (sc < 0) sc += size;
+      so += sc * stride;
+      stride *= size;
+    }
+  }
+  return so;
+}
+
+template <typename T, typename I>
 __global__ __launch_bounds__(256) void roll_kernel(T* __restrict__ dst,
                                                    const T* __restrict__ src, RollArgs a,
                                                    long long total) {
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total;
-       i += (long long)gridDim.x * 256) {
-    long long rem = i, so = 0, stride = 1;
-#pragma unroll
-    for (int k = kMaxDims - 1; k >= 0; --k) {
-      if (k < a.nd) {
-        long long q = rem / a.size[k];
-        long long c = rem - q * a.size[k];
-        rem = q;
-        long long sc = c - a.shift[k];
-        if (sc < 0) sc += a.size[k];
-        so += sc * stride;
-        stride *= a.size[k];
-      }
-    }
-    dst[i] = src[so];
-  }
+       i += (long long)gridDim.x * 256)
+    dst[i] = src[rolled_source<I>(a, (I)i)];
 }
 
 // Slab copy between x viewed as (outer, len, inner) and a dense (outer, win, inner).
-template <typename T, bool PACK>
+template <typename T, bool PACK, typename I>
 __global__ __launch_bounds__(256) void slab_kernel(T* __restrict__ x_or_strip_dst,
                                                    const T* __restrict__ src, long long outer,
-                                                   long long len, long long inner,
-                                                   long long start, long long win) {
-  const long long total = outer * win * inner;
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total;
-       i += (long long)gridDim.x * 256) {
-    long long r = i / inner;
-    long long ci = i - r * inner;
-    long long o = r / win;
-    long long a = r - o * win;
-    long long xo = (o * len + start + a) * inner + ci;
+                                                   long long len_, long long inner_,
+                                                   long long start_, long long win_) {
+  const long long total = outer * win_ * inner_;
+  const I len = (I)len_, inner = (I)inner_, start = (I)start_, win = (I)win_;
+  for (long long i_ = (long long)blockIdx.x * 256 + threadIdx.x; i_ < total;
+       i_ += (long long)gridDim.x * 256) {
+    const I i = (I)i_;
+    I r = i / inner;
+    I ci = i - r * inner;
+    I o = r / win;
+    I a = r - o * win;
+    I xo = (o * len + start + a) * inner + ci;
     if (PACK)
       x_or_strip_dst[i] = src[xo];
     else
@@ -66,44 +75,35 @@ __global__ __launch_bounds__(256) void slab_kernel(T* __restrict__ x_or_strip_ds
 // x viewed as (outer, len, inner) along one axis; the slab is rows [start, start + win) of it.
 struct SlabView {
   long long len, inner, start, win;
-  __device__ __forceinline__ bool holds(long long idx, long long* strip_idx) const {
-    const long long r = idx / inner, ci = idx - r * inner;
-    const long long o = r / len, l = r - o * len;
-    *strip_idx = (o * win + (l - start)) * inner + ci;
-    return l >= start && l < start + win;
+  template <typename I>
+  __device__ __forceinline__ bool holds(I idx, I* strip_idx) const {
+    const I inner_ = (I)inner, len_ = (I)len, start_ = (I)start, win_ = (I)win;
+    const I r = idx / inner_, ci = idx - r * inner_;
+    const I o = r / len_, l = r - o * len_;
+    *strip_idx = (o * win_ + (l - start_)) * inner_ + ci;
+    return l >= start_ && l < start_ + win_;
   }
-  __device__ __forceinline__ long long place(long long strip_idx) const {
-    const long long r = strip_idx / inner, ci = strip_idx - r * inner;
-    const long long o = r / win, a = r - o * win;
-    return (o * len + start + a) * inner + ci;
+  template <typename I>
+  __device__ __forceinline__ I place(I strip_idx) const {
+    const I inner_ = (I)inner, len_ = (I)len, start_ = (I)start, win_ = (I)win;
+    const I r = strip_idx / inner_, ci = strip_idx - r * inner_;
+    const I o = r / win_, a = r - o * win_;
+    return (o * len_ + start_ + a) * inner_ + ci;
   }
 };
 
 // The local roll, and on the way the wrapped slab of the ROLLED tensor along one axis cut into
 // `strip`, with the buffer the neighbour's slab will be received in cleared (what the reference
 // does in three passes: torch.roll, x[sl].contiguous(), torch.zeros_like).
-template <typename T>
+template <typename T, typename I>
 __global__ __launch_bounds__(256) void roll_pack_kernel(T* __restrict__ dst, const T* __restrict__ src, RollArgs a,
                                                         long long total, T* __restrict__ strip, T* __restrict__ clear,
                                                         SlabView v) {
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long long)gridDim.x * 256) {
-    long long rem = i, so = 0, stride = 1;
-#pragma unroll
-    for (int k = kMaxDims - 1; k >= 0; --k) {
-      if (k < a.nd) {
-        long long q = rem / a.size[k];
-        long long c = rem - q * a.size[k];
-        rem = q;
-        long long sc = c - a.shift[k];
-        if (sc < 0) sc += a.size[k];
-        so += sc * stride;
-        stride *= a.size[k];
-      }
-    }
-    const T val = src[so];
+    const T val = src[rolled_source<I>(a, (I)i)];
     dst[i] = val;
-    long long j;
-    if (v.holds(i, &j)) {
+    I j;
+    if (v.holds<I>((I)i, &j)) {
       strip[j] = val;
       if (clear != nullptr) clear[j] = T{};
     }
@@ -114,18 +114,18 @@ __global__ __launch_bounds__(256) void roll_pack_kernel(T* __restrict__ dst, con
 // send along the second axis is cut from x as it will be AFTER that write: where the two slabs
 // cross, the cut takes the received values directly, so the two steps do not wait for each other.
 // The buffer for the second exchange is cleared on the way.
-template <typename T>
+template <typename T, typename I>
 __global__ __launch_bounds__(256) void unpack_pack_kernel(T* __restrict__ x, const T* __restrict__ recv1, SlabView v1,
                                                           long long n1, T* __restrict__ strip2, T* __restrict__ clear2,
                                                           SlabView v2, long long n2) {
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n1 + n2; i += (long long)gridDim.x * 256) {
     if (i < n1) {
-      x[v1.place(i)] = recv1[i];
+      x[v1.place<I>((I)i)] = recv1[i];
     } else {
-      const long long j = i - n1;
-      const long long idx = v2.place(j);
-      long long j1;
-      strip2[j] = v1.holds(idx, &j1) ? recv1[j1] : x[idx];
+      const I j = (I)(i - n1);
+      const I idx = v2.place<I>(j);
+      I j1;
+      strip2[j] = v1.holds<I>(idx, &j1) ? recv1[j1] : x[idx];
       if (clear2 != nullptr) clear2[j] = T{};
     }
   }
@@ -139,6 +139,8 @@ int grid_for(long long n) {
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+// whether every index of a tensor of `words` copy words fits the 32-bit arithmetic
+bool small(long long words) { return words < (1ll << 30); }
 
 int slab_common(void* dst, const void* src, const void* x, int ndim, const int64_t* sizes,
                 int axis, int64_t window, int elem_size, void* stream, bool pack,
@@ -165,21 +167,28 @@ int slab_common(void* dst, const void* src, const void* x, int ndim, const int64
   if (inner_bytes % 16 == 0 && aligned16(x) && aligned16(strip)) {
     const long long iv = inner_bytes / 16;
     const long long total = outer * win * iv;
-    if (pack)
-      slab_kernel<u32x4, true><<<grid_for(total), 256, 0, s>>>(
+    const bool i32 = small(outer * len * iv);
+    if (pack && i32)
+      slab_kernel<u32x4, true, int><<<grid_for(total), 256, 0, s>>>(
+          static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), outer, len, iv, start, win);
+    else if (pack)
+      slab_kernel<u32x4, true, long long><<<grid_for(total), 256, 0, s>>>(
+          static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), outer, len, iv, start, win);
+    else if (i32)
+      slab_kernel<u32x4, false, int><<<grid_for(total), 256, 0, s>>>(
           static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), outer, len, iv, start, win);
     else
-      slab_kernel<u32x4, false><<<grid_for(total), 256, 0, s>>>(
+      slab_kernel<u32x4, false, long long><<<grid_for(total), 256, 0, s>>>(
           static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), outer, len, iv, start, win);
   } else {
     const long long total = outer * win * inner;
 #define JG_SLAB(T)                                                                         \
   do {                                                                                     \
     if (pack)                                                                              \
-      slab_kernel<T, true><<<grid_for(total), 256, 0, s>>>(                                \
+      slab_kernel<T, true, long long><<<grid_for(total), 256, 0, s>>>(                     \
           static_cast<T*>(dst), static_cast<const T*>(src), outer, len, inner, start, win); \
     else                                                                                   \
-      slab_kernel<T, false><<<grid_for(total), 256, 0, s>>>(                               \
+      slab_kernel<T, false, long long><<<grid_for(total), 256, 0, s>>>(                    \
           static_cast<T*>(dst), static_cast<const T*>(src), outer, len, inner, start, win); \
   } while (0)
     if (elem_size == 2) JG_SLAB(uint16_t);
@@ -238,8 +247,10 @@ extern "C" int jg_roll(void* dst, const void* src, int ndim, const int64_t* size
     a.shift[a.nd] = 0;
     ++a.nd;
     const long long n = total * elem_size / 16;
-    roll_kernel<u32x4><<<grid_for(n), 256, 0, s>>>(static_cast<u32x4*>(dst),
-                                                   static_cast<const u32x4*>(src), a, n);
+    if (small(n))
+      roll_kernel<u32x4, int><<<grid_for(n), 256, 0, s>>>(static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), a, n);
+    else
+      roll_kernel<u32x4, long long><<<grid_for(n), 256, 0, s>>>(static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), a, n);
   } else {
     if (run > 1 || a.nd == 0) {
       a.size[a.nd] = run;
@@ -247,10 +258,10 @@ extern "C" int jg_roll(void* dst, const void* src, int ndim, const int64_t* size
       ++a.nd;
     }
     if (elem_size == 2)
-      roll_kernel<uint16_t><<<grid_for(total), 256, 0, s>>>(
+      roll_kernel<uint16_t, long long><<<grid_for(total), 256, 0, s>>>(
           static_cast<uint16_t*>(dst), static_cast<const uint16_t*>(src), a, total);
     else
-      roll_kernel<uint32_t><<<grid_for(total), 256, 0, s>>>(
+      roll_kernel<uint32_t, long long><<<grid_for(total), 256, 0, s>>>(
           static_cast<uint32_t*>(dst), static_cast<const uint32_t*>(src), a, total);
   }
   JG_CHECK_LAUNCH("jg_roll");
@@ -333,9 +344,14 @@ extern "C" int jg_roll_pack_fused(void* dst, void* strip, void* clear, const voi
   v.len = ax.len; v.start = ax.start; v.win = ax.win;
   v.inner = ax.inner / run * words;
   const long long n = total / run * words;
-  roll_pack_kernel<u32x4><<<grid_for(n), 256, 0, static_cast<hipStream_t>(stream)>>>(
-      static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), a, n, static_cast<u32x4*>(strip),
-      static_cast<u32x4*>(clear), v);
+  if (small(n))
+    roll_pack_kernel<u32x4, int><<<grid_for(n), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), a, n, static_cast<u32x4*>(strip),
+        static_cast<u32x4*>(clear), v);
+  else
+    roll_pack_kernel<u32x4, long long><<<grid_for(n), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), a, n, static_cast<u32x4*>(strip),
+        static_cast<u32x4*>(clear), v);
   JG_CHECK_LAUNCH(who);
   return JG_OK;
 }
@@ -368,9 +384,15 @@ extern "C" int jg_roll_unpack_pack(void* x, const void* recv1, int axis1, int64_
   v2.len = a2.len; v2.start = a2.start; v2.win = a2.win; v2.inner = a2.inner / run * words;
   const long long n1 = a1.outer * a1.win * v1.inner, n2 = a2.outer * a2.win * v2.inner;
   if (n1 + n2 == 0) return JG_OK;
-  unpack_pack_kernel<u32x4><<<grid_for(n1 + n2), 256, 0, static_cast<hipStream_t>(stream)>>>(
-      static_cast<u32x4*>(x), static_cast<const u32x4*>(recv1), v1, n1, static_cast<u32x4*>(strip2),
-      static_cast<u32x4*>(clear2), v2, n2);
+  // indices run over x (in words), the largest of the three tensors
+  if (small(a1.outer * a1.len * v1.inner))
+    unpack_pack_kernel<u32x4, int><<<grid_for(n1 + n2), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<u32x4*>(x), static_cast<const u32x4*>(recv1), v1, n1, static_cast<u32x4*>(strip2),
+        static_cast<u32x4*>(clear2), v2, n2);
+  else
+    unpack_pack_kernel<u32x4, long long><<<grid_for(n1 + n2), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<u32x4*>(x), static_cast<const u32x4*>(recv1), v1, n1, static_cast<u32x4*>(strip2),
+        static_cast<u32x4*>(clear2), v2, n2);
   JG_CHECK_LAUNCH(who);
   return JG_OK;
 }
