@@ -294,7 +294,16 @@ def ptr(t: torch.Tensor | None) -> c_void_p:
     return c_void_p(0 if t is None else t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(device: torch.device | None = None) -> c_void_p:
+    """The current stream of ``device`` as the raw handle the C entry points take. Asked of torch's
+    C layer directly where it offers that (a tenth of the time of building a ``torch.cuda.Stream``
+    object for every launch, which adds up in steps of 40 launches)."""
+    if _raw_stream is not None:
+        index = device.index if device is not None and device.index is not None else torch.cuda.current_device()
+        return c_void_p(_raw_stream(index))
     return c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
