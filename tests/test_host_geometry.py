@@ -1,0 +1,170 @@
+"""Host-side geometry of the halo exchange and of the dilation route, on the CPU.
+
+Pins, without a GPU and without the kernels: the halo widths of every rank against a brute-force
+enumeration of the cells a rank's outputs touch (also where the need spans drift against the
+tiles and the widths change from rank to rank), that the two ends of every exchange agree on
+the strip shapes, the raw spans of the transposed convolution, and the identity behind the
+dilated route (the residues of the pixel index are undilated problems of their own).
+"""
+
+import itertools
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from jigsaw_amd import conv as jc
+from jigsaw_amd import conv_transpose as jct
+from jigsaw_amd.halo import HaloGeometry, halo_widths
+
+from helpers import mesh_coords, neighbour
+
+
+def touched_span(rank, G, n, k, s, p, d):
+    """First and one-past-last input row touched by the outputs of `rank`, by enumeration."""
+    extent = d * (k - 1) + 1
+    gout = (G * n + 2 * p - extent) // s + 1
+    if gout % G:
+        return None
+    ol = gout // G
+    rows = [o * s - p + t * d for o in range(rank * ol, (rank + 1) * ol) for t in range(k)]
+    return min(rows), max(rows) + 1, ol
+
+
+def test_halo_widths_against_enumeration():
+    accepted = rejected = drifting = 0
+    for G, n, k, s, p, d in itertools.product([2, 3, 4], [4, 6, 8, 9], [1, 2, 3, 5], [1, 2, 3], [0, 1, 2], [1, 2]):
+        if G * n + 2 * p < d * (k - 1) + 1:
+            continue
+        for rank in range(G):
+            span = touched_span(rank, G, n, k, s, p, d)
+            if span is None:
+                with pytest.raises(NotImplementedError):
+                    halo_widths(rank, G, n, k, s, p, d)
+                continue
+            lo, hi, ol = span
+            lo_w, hi_w = rank * n - lo, hi - (rank + 1) * n
+            if 0 <= lo_w <= n and 0 <= hi_w <= n:
+                assert halo_widths(rank, G, n, k, s, p, d) == (lo_w, hi_w, ol)
+                accepted += 1
+                drifting += ol * s != n
+            else:
+                with pytest.raises(NotImplementedError):
+                    halo_widths(rank, G, n, k, s, p, d)
+                rejected += 1
+    assert accepted > 500 and rejected > 50 and drifting > 100
+
+
+MESH_CASES = [
+    # mesh, local size, kernel, stride, padding, dilation
+    ((2, 2), (8, 10), (3, 3), (1, 1), (0, 0), (1, 1)),
+    ((4, 2), (6, 8), (5, 3), (1, 1), (0, 1), (1, 1)),
+    ((2, 2), (8, 8), (6, 6), (2, 2), (0, 0), (1, 1)),
+    ((3, 3), (4, 6), (3, 5), (2, 2), (1, 2), (1, 1)),
+    ((2, 1, 2), (4, 5, 6), (3, 3, 5), (1, 1, 1), (0, 1, 1), (1, 1, 1)),
+    ((2, 2, 2), (6, 5, 8), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", MESH_CASES)
+def test_both_ends_of_an_exchange_agree_on_the_strip(case):
+    """What a rank cuts for a neighbour (forward: by the neighbour's halo, backward: its own halo's
+    gradient) has the shape the neighbour expects from that side."""
+    mesh, n, k, s, p, d = case
+    geoms = {c: HaloGeometry.for_conv(n, k, s, p, d, c, mesh) for c in mesh_coords(mesh)}
+    pairs = 0
+    for c, g in geoms.items():
+        assert g.padded == tuple(
+            (touched_span(c[a], mesh[a], n[a], k[a], s[a], p[a], d[a])[1] - touched_span(c[a], mesh[a], n[a], k[a], s[a], p[a], d[a])[0])
+            if mesh[a] > 1 else n[a] for a in range(len(mesh)))
+        for o in g.offsets():
+            nb = neighbour(c, o, mesh)
+            if nb is None:
+                continue
+            back = tuple(-v for v in o)
+            assert g.strip_extent(o, "pack_fwd") == geoms[nb].strip_extent(back, "assemble"), (c, o)
+            assert g.strip_extent(o, "pack_bwd") == geoms[nb].strip_extent(back, "fold"), (c, o)
+            pairs += 1
+    assert pairs > 0
+
+
+def test_raw_spans_of_the_transposed_convolution_against_enumeration():
+    """Input column i, tap j writes output column i * s - p + d * j."""
+    accepted = drifting = 0
+    for G, n, k, s, p, d in itertools.product([2, 3, 4], [3, 4, 6], [1, 2, 3, 4, 5], [1, 2, 3], [0, 1, 2], [1, 2]):
+        extent = d * (k - 1) + 1
+        gout = (G * n - 1) * s - 2 * p + extent
+        if gout <= 0 or gout % G:
+            continue
+        ol = gout // G
+        for rank in range(G):
+            cols = [i * s - p + d * j for i in range(rank * n, (rank + 1) * n) for j in range(k)]
+            left, right = rank * ol - min(cols), max(cols) + 1 - (rank + 1) * ol
+            if 0 <= left <= ol and 0 <= right <= ol:
+                assert jct.raw_span_widths(rank, G, n, k, s, p, d) == (left, right, ol)
+                accepted += 1
+                drifting += extent != s + 2 * p
+            else:
+                with pytest.raises(NotImplementedError):
+                    jct.raw_span_widths(rank, G, n, k, s, p, d)
+    assert accepted > 100 and drifting > 20
+
+
+def test_transposed_neighbours_agree_on_the_overlap():
+    n, k, s, p, d, mesh = (5, 7), (4, 4), (2, 2), (0, 0), (1, 1), (2, 2)
+    geoms = {c: jct.transpose_geometry(n, k, s, p, d, c, mesh) for c in mesh_coords(mesh)}
+    for c, g in geoms.items():
+        for o in g.offsets():
+            nb = neighbour(c, o, mesh)
+            if nb is not None:
+                back = tuple(-v for v in o)
+                assert g.strip_extent(o, "pack_bwd") == geoms[nb].strip_extent(back, "fold")
+                assert g.strip_extent(o, "pack_fwd") == geoms[nb].strip_extent(back, "assemble")
+
+
+DILATED = [
+    # in spatial, kernel, padding, dilation
+    ((13, 17), (3, 3), (2, 3), (2, 3)),
+    ((12, 16), (3, 3), (0, 0), (2, 2)),
+    ((9, 10), (3, 1), (4, 0), (2, 5)),
+    ((5, 9, 11), (3, 3, 3), (1, 2, 4), (1, 2, 2)),
+]
+
+
+@pytest.mark.parametrize("case", DILATED)
+def test_residue_images_are_undilated_problems(case):
+    """The route of the dilated convolution, with torch's CPU operators in place of the kernels:
+    forward, input gradient and weight gradient of the residue images give those of the dilated layer."""
+    insp, k, p, d = case
+    ns = len(k)
+    assert jc._dilated_ok(k, (1,) * ns, p, d)
+    conv = {2: F.conv2d, 3: F.conv3d}[ns]
+    torch.manual_seed(0)
+    x = torch.randn(2, 3, *insp, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(4, 3, *k, dtype=torch.float64, requires_grad=True)
+    y = conv(x, w, None, 1, p, d)
+    g = torch.randn_like(y)
+    y.backward(g)
+
+    phases = jc._phase_counts(k, d)
+    ext_in = tuple(-(-i // q) for i, q in zip(insp, phases))
+    pad0 = tuple(pp // q for pp, q in zip(p, phases))
+    xb = jc._to_phases(x.detach(), phases, ext_in).requires_grad_()
+    wb = w.detach().clone().requires_grad_()
+    yb = conv(xb, wb, None, 1, pad0, 1)
+    assert torch.allclose(jc._from_phases(yb.detach(), phases, 2, y.shape[2:]), y.detach(), atol=1e-12)
+    gb = jc._to_phases(g, phases, tuple(yb.shape[2:]))
+    yb.backward(gb)
+    assert torch.allclose(jc._from_phases(xb.grad, phases, 2, insp), x.grad, atol=1e-12)
+    assert torch.allclose(wb.grad, w.grad, atol=1e-10)
+    # and the two permutations are inverses of each other on the cells that exist
+    assert torch.equal(jc._from_phases(jc._to_phases(x.detach(), phases, ext_in), phases, 2, insp), x.detach())
+
+
+def test_the_dilated_route_takes_only_what_it_covers():
+    assert not jc._dilated_ok((3, 3), (1, 1), (1, 1), (2, 2))      # padding not a multiple of the dilation
+    assert not jc._dilated_ok((3, 3), (2, 1), (2, 2), (2, 2))      # strided: through the stride-1 route first
+    assert not jc._dilated_ok((5, 3), (1, 1), (4, 2), (2, 2))      # five taps
+    assert not jc._dilated_ok((3, 3), (1, 1), (1, 1), (1, 1))      # nothing dilated
+    assert jc._dilated_ok((1, 3), (1, 1), (0, 4), (7, 2))          # a dilation on a one-tap axis means nothing
+    assert jc._dense_stride_ok((3, 3), (2, 2), (2, 2), (2, 2)) and not jc._dense_stride_ok((3, 3), (2, 2), (2, 2), (1, 1))
