@@ -19,10 +19,20 @@ from typing import Any
 import torch
 import torch.nn as nn
 
-from .attention import swin_grid_attention_packed, window_attention
+from . import _lib
+from .attention import _SwinGridAttention, swin_grid_attention_packed, window_attention
 from .conv import TileGroup
-from .layernorm import plain_layer_norm, plain_layer_norm_fork
-from .projection import gelu_mlp, heads_projection, linear, qkv_projection
+from .layernorm import _PlainLayerNormFork, plain_layer_norm, plain_layer_norm_fork
+from .projection import (
+    _GeluMlp,
+    _HeadsProjection,
+    _QkvProjection,
+    gelu_mlp,
+    heads_projection,
+    linear,
+    mlp_fusable,
+    qkv_projection,
+)
 from .roll import _Roll
 
 
@@ -134,6 +144,63 @@ class WindowAttention(nn.Module):
         return unwindows(heads_projection(out, self.proj.weight, self.proj.bias), h, w, self.window)
 
 
+class _Stage:
+    """What one of the block's autograd functions keeps for its backward when the whole block is a
+    single autograd function: the part of a ``ctx`` those functions use."""
+
+    needs_input_grad = (True,) * 8
+    saved_tensors: tuple = ()
+
+    def save_for_backward(self, *tensors) -> None:
+        self.saved_tensors = tensors
+
+
+class _WholeBlock(torch.autograd.Function):
+    """The block of :class:`SwinBlock` as ONE node of the autograd graph: the same launches in the
+    same order as the functions it is made of (their ``forward`` / ``backward`` are called as they
+    are, each with a :class:`_Stage` for its ``ctx``), so the numbers are theirs bit for bit. What
+    goes is the bookkeeping of eight nodes per step, forward and in the engine's backward walk, which
+    on a slow host is a third of the step's wall clock."""
+
+    @staticmethod
+    def forward(ctx, x, n1w, n1b, qkv_w, qkv_b, table, proj_w, proj_b, n2w, n2b, w1, b1, w2, b2, block):  # noqa: D102
+        b, h, w, c = x.shape
+        dt, eps, heads = _compute_dtype(x), block.eps, block.attn.heads
+        st = [_Stage() for _ in range(8)]
+        roll_args = block._roll_args()
+        y = _PlainLayerNormFork.forward(st[0], x, n1w, n1b, eps, dt)[0]
+        if block.shift_by:
+            y = _Roll.forward(st[1], y.contiguous(), (-block.shift_by,) * 2, (1, 2), *roll_args)
+        qkv = _QkvProjection.forward(st[2], y.view(b, h * w, c), qkv_w, qkv_b, heads)
+        out = _SwinGridAttention.forward(st[3], qkv, table, block.attn.side, (h, w))
+        a = _HeadsProjection.forward(st[4], out, proj_w, proj_b).view(b, h, w, c)
+        if block.shift_by:
+            a = _Roll.forward(st[5], a.contiguous(), (block.shift_by,) * 2, (1, 2), *roll_args)
+        x1 = x + a.to(x.dtype)
+        y2 = _PlainLayerNormFork.forward(st[6], x1, n2w, n2b, eps, dt)[0]
+        result = _GeluMlp.forward(st[7], y2, w1, b1, w2, b2, x1)
+        ctx.stages, ctx.shifted, ctx.branch_dtype, ctx.grid = st, bool(block.shift_by), a.dtype, (b, h, w, c)
+        return result
+
+    @staticmethod
+    def backward(ctx, grad):  # noqa: D102
+        st, (b, h, w, c) = ctx.stages, ctx.grid
+        gy2, gw1, gb1, gw2, gb2, over = _GeluMlp.backward(st[7], grad)
+        gx1, gn2w, gn2b = _PlainLayerNormFork.backward(st[6], gy2, over)[:3]
+        ga = gx1.to(ctx.branch_dtype)
+        if ctx.shifted:
+            ga = _Roll.backward(st[5], ga)[0]
+        gout, gpw, gpb = _HeadsProjection.backward(st[4], ga.view(b, h * w, c))[:3]
+        dqkv, dtable = _SwinGridAttention.backward(st[3], gout)[:2]
+        gy, gqw, gqb = _QkvProjection.backward(st[2], dqkv)[:3]
+        gy = gy.view(b, h, w, c)
+        if ctx.shifted:
+            gy = _Roll.backward(st[1], gy)[0]
+        gx, gn1w, gn1b = _PlainLayerNormFork.backward(st[0], gy, gx1)[:3]
+        ctx.stages = None
+        return gx, gn1w, gn1b, gqw, gqb, dtable, gpw, gpb, gn2w, gn2b, gw1, gb1, gw2, gb2, None
+
+
 class SwinBlock(nn.Module):
     """``x + attn(norm(x))`` then ``x + mlp(norm(x))``; the windows may be shifted
     (examples/swin.py:173-210). ``groups`` are the two spatial groups of the tile
@@ -141,21 +208,40 @@ class SwinBlock(nn.Module):
     roll uses (``RollConfig.comm_halo_1d_fn`` in the reference)."""
 
     def __init__(self, dim: int, heads: int, window: int, tile: tuple, groups: tuple = None,
-                 comm_halo_1d_fn: Callable | None = None, shift: int = 0, device=None, eps: float = 1e-5) -> None:
+                 comm_halo_1d_fn: Callable | None = None, shift: int = 0, device=None, eps: float = 1e-5,
+                 one_node: bool = True) -> None:
         super().__init__()
         groups = groups or (TileGroup(1, 0), TileGroup(1, 0))
         self.groups, self.comm, self.shift_by, self.eps = groups, comm_halo_1d_fn, shift, eps
+        self.one_node = one_node  # the whole block as one autograd function where its fused kernels apply
         self.norm1 = nn.LayerNorm(dim, eps=eps, device=device)
         self.attn = WindowAttention(dim, heads, window, tile, shift, groups, device)
         self.norm2 = nn.LayerNorm(dim, eps=eps, device=device)
         self.mlp = nn.Sequential(nn.Linear(dim, 4 * dim, device=device), nn.GELU(), nn.Linear(4 * dim, dim, device=device))
 
+    def _roll_args(self) -> tuple:
+        dist_dims = tuple(d for d, g in zip((1, 2), self.groups) if g.size() > 1)
+        dist_groups = tuple(g for g in self.groups if g.size() > 1)
+        return dist_dims, dist_groups, self.comm
+
     def _roll(self, x: torch.Tensor, shift: int) -> torch.Tensor:
         if not shift:
             return x
-        dist_dims = tuple(d for d, g in zip((1, 2), self.groups) if g.size() > 1)
-        dist_groups = tuple(g for g in self.groups if g.size() > 1)
-        return _Roll.apply(x.contiguous(), (shift, shift), (1, 2), dist_dims, dist_groups, self.comm)
+        return _Roll.apply(x.contiguous(), (shift, shift), (1, 2), *self._roll_args())
+
+    def _one_node(self, x: torch.Tensor) -> bool:
+        """Whether the block runs as one autograd function: the shapes all of its fused kernels take."""
+        if not self.one_node or x.dim() != 4 or not x.is_cuda or x.numel() == 0:
+            return False
+        if x.dtype != torch.bfloat16 or _compute_dtype(x) != torch.bfloat16:
+            return False
+        b, h, w, c = x.shape
+        attn, fc1, fc2 = self.attn, self.mlp[0], self.mlp[2]
+        if c % attn.heads or c // attn.heads != 32 or attn.window != 8 or h % 8 or w % 8:
+            return False
+        if not _lib.load().jg_ln_plain_supported(c) or any(t is None for t in (attn.qkv.bias, attn.proj.bias, fc1.bias, fc2.bias)):
+            return False
+        return mlp_fusable(x, fc1.weight, fc2.weight, x)
 
     def _norm(self, ln: nn.LayerNorm, x: torch.Tensor) -> torch.Tensor:
         # Both LayerNorms feed a linear layer (through pure copies), which under autocast rounds
@@ -183,6 +269,11 @@ class SwinBlock(nn.Module):
         # x + f(norm(x)) twice; the rows that go round a branch come out of the LayerNorm call beside
         # the normalised ones, so that the backward adds the two gradients of x inside its kernel
         dt = _compute_dtype(x)
+        if self._one_node(x):
+            attn, fc1, fc2 = self.attn, self.mlp[0], self.mlp[2]
+            return _WholeBlock.apply(x, self.norm1.weight, self.norm1.bias, attn.qkv.weight, attn.qkv.bias, attn.bias_table,
+                                     attn.proj.weight, attn.proj.bias, self.norm2.weight, self.norm2.bias, fc1.weight, fc1.bias,
+                                     fc2.weight, fc2.bias, self)
         y, x = plain_layer_norm_fork(x, self.norm1.weight, self.norm1.bias, self.eps, out_dtype=dt)
         x = x + self.unshift(self.attn(self.shift(y))).to(x.dtype)
         y, x = plain_layer_norm_fork(x, self.norm2.weight, self.norm2.bias, self.eps, out_dtype=dt)

@@ -151,3 +151,39 @@ def test_swin_block_bf16_backward_config5(shift, n, dev):
     for name, prm in block.named_parameters():
         err = rel_l2(prm.grad, params[name].grad)
         assert err < 2e-2, f"{name}: {err:.3e}"
+
+
+@pytest.mark.parametrize("shift,n", [(4, (256, 256)), (0, (64, 128)), (4, (64, 64))])
+def test_block_as_one_autograd_node_has_the_bits_of_its_parts(shift, n, dev):
+    """bf16 tokens under bf16 autocast (what the benchmark times): the block runs as a single
+    autograd function that calls the forward / backward of the functions it is made of. Output,
+    dx and every parameter gradient equal those of the block composed of the separate functions
+    bit for bit, and meet the oracle at the bf16 bar."""
+    torch.manual_seed(5)
+    dim, heads, window = 128, 4, 8
+    one = js.SwinBlock(dim, heads, window, n, shift=shift, device=dev)
+    parts = js.SwinBlock(dim, heads, window, n, shift=shift, device=dev, one_node=False)
+    with torch.no_grad():
+        one.attn.bias_table.normal_(0, 0.5)
+    parts.load_state_dict(one.state_dict())
+    x = torch.randn(1, *n, dim).bfloat16()
+    g = torch.randn(1, *n, dim).bfloat16()
+    results = []
+    for block in (one, parts):
+        xg = x.to(dev).requires_grad_()
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = block(xg)
+        results.append((out, xg, block))
+        out.backward(g.to(dev))
+    assert "WholeBlock" in type(results[0][0].grad_fn).__name__ and "WholeBlock" not in type(results[1][0].grad_fn).__name__
+    (o1, x1, b1), (o2, x2, b2) = results
+    assert torch.equal(o1, o2) and torch.equal(x1.grad, x2.grad)
+    for (name, p1), (_, p2) in zip(b1.named_parameters(), b2.named_parameters()):
+        assert p1.grad is not None and torch.equal(p1.grad, p2.grad), name
+    params = {k: v.detach().double().cpu().requires_grad_() for k, v in one.state_dict().items()}
+    xd = x.double().requires_grad_()
+    want = osw.block(xd, params, heads, window, shift)
+    want.backward(g.double())
+    assert rel_l2(o1, want.detach()) < 2e-2 and rel_l2(x1.grad, xd.grad) < 2e-2
+    for name, prm in one.named_parameters():
+        assert rel_l2(prm.grad, params[name].grad) < 2e-2, name
