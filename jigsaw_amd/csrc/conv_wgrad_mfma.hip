@@ -77,6 +77,7 @@ struct WgradParams {
   int row_pairs, col_tiles;
   long long total_stages;  // N * Dout * col_tiles * row_pairs
   int w_first, w_last;     // what a stage of the first / last column strip costs, in stages of the other strips
+  int wd_first, wd_last;   // the same for every stage of the first / last output depth (1: a plane like the others)
 };
 
 // Wavefronts per workgroup: (g block, x block) pairs x 2 column halves; a 6-wavefront
@@ -128,23 +129,44 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
   const unsigned wg_rank = gridDim.x % 8 == 0 ? (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8 : blockIdx.x;
   // The ranges hold equal cost, not equal counts: the stages of a column strip whose windows
   // stick out of the tensor (or whose last columns do not exist) load with bounds checks and
-  // take about twice as long, and a workgroup whose whole range lay in such a strip would set
+  // take several times as long, and a workgroup whose whole range lay in such a strip would set
   // the kernel's time. Cost runs like the stages: per plane the first strip at w_first a
-  // stage, the middle strips at 1, the last at w_last; with both at 1 the ranges are counts.
+  // stage, the middle strips at 1, the last at w_last; a plane at the first / last output depth
+  // whose depth taps stick out is slow as a whole (wd_first / wd_last a stage). With all four at
+  // 1 the ranges are counts.
   const long long strip_first = (long long)p.row_pairs * p.w_first;
   const long long strip_mid = (long long)p.row_pairs * (p.col_tiles > 2 ? p.col_tiles - 2 : 0);
   const long long strip_last = p.col_tiles > 1 ? (long long)p.row_pairs * p.w_last : 0;
   const long long plane_cost = strip_first + strip_mid + strip_last;
   const long long plane_stages = (long long)p.row_pairs * p.col_tiles;
-  const long long total_cost = (p.total_stages / plane_stages) * plane_cost;
+  const long long head_cost = p.wd_first > 1 ? plane_stages * p.wd_first : plane_cost;
+  const long long tail_cost = p.Dout > 1 ? (p.wd_last > 1 ? plane_stages * p.wd_last : plane_cost) : 0;
+  const long long mid_cost = (p.Dout > 2 ? p.Dout - 2 : 0) * plane_cost;
+  const long long entry_cost = head_cost + mid_cost + tail_cost;  // one batch entry
+  const long long total_cost = (p.total_stages / (plane_stages * p.Dout)) * entry_cost;
+  auto in_plane = [&](long long rem) -> long long {  // stage inside a plane of ordinary cost
+    if (rem < strip_first) return rem / p.w_first;
+    if (rem < strip_first + strip_mid) return p.row_pairs + (rem - strip_first);
+    return (long long)p.row_pairs * (p.col_tiles - 1) + (rem - strip_first - strip_mid) / p.w_last;
+  };
   auto stage_at = [&](long long cost) -> long long {
     if (cost >= total_cost) return p.total_stages;
-    const long long pl = cost / plane_cost, rem = cost - pl * plane_cost;
-    long long st;
-    if (rem < strip_first) st = rem / p.w_first;
-    else if (rem < strip_first + strip_mid) st = p.row_pairs + (rem - strip_first);
-    else st = (long long)p.row_pairs * (p.col_tiles - 1) + (rem - strip_first - strip_mid) / p.w_last;
-    return pl * plane_stages + st;
+    const long long n = cost / entry_cost;
+    long long rem = cost - n * entry_cost, od, st;
+    if (rem < head_cost) {
+      od = 0;
+      st = p.wd_first > 1 ? rem / p.wd_first : in_plane(rem);
+    } else if (rem < head_cost + mid_cost) {
+      rem -= head_cost;
+      const long long k = rem / plane_cost;
+      od = 1 + k;
+      st = in_plane(rem - k * plane_cost);
+    } else {
+      rem -= head_cost + mid_cost;
+      od = p.Dout - 1;
+      st = p.wd_last > 1 ? rem / p.wd_last : in_plane(rem);
+    }
+    return (n * p.Dout + od) * plane_stages + st;
   };
   const long long per = (total_cost + gridDim.x - 1) / gridDim.x;
   const long long s_begin = stage_at(per * wg_rank);
@@ -866,12 +888,16 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
     const bool first_slow = g.p[2] > 0;
     const int lead = even == 2 ? 1 : 0;
     const bool last_slow = last_ow0 + SW > g.out[2] || last_ow0 - g.p[2] - lead + SW + 2 + lead > g.in[2];
-    p.w_first = p.w_last = 1;
+    p.w_first = p.w_last = p.wd_first = p.wd_last = 1;
     // measured: such a stage costs about four plain ones; 3 gave the shortest kernels over the shapes tried
     constexpr int SLOW = 3;
     if (even) {  // without the even layout every stage takes that path
       if (p.col_tiles == 1) p.w_first = (first_slow || last_slow) ? SLOW : 1;
       else { p.w_first = first_slow ? SLOW : 1; p.w_last = last_slow ? SLOW : 1; }
+      // output depths whose depth taps reach outside x: all their stages take that path
+      const bool head_slow = g.p[0] > 0, tail_slow = g.out[0] - 1 - g.p[0] + g.k[0] > g.in[0];
+      if (g.out[0] == 1) p.wd_first = (head_slow || tail_slow) ? SLOW : 1;
+      else { p.wd_first = head_slow ? SLOW : 1; p.wd_last = tail_slow ? SLOW : 1; }
     }
   }
   const int wgs = wg_count(p.total_stages);
