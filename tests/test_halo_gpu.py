@@ -25,6 +25,10 @@ CASES = [
     ((2, 2, 2), (6, 5, 8), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
     ((3, 3, 3), (4, 5, 6), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
     ((3, 1, 3), (4, 5, 6), (5, 3, 3), (1, 1, 1), (2, 1, 1), (1, 1, 1)),
+    # rows long enough for a whole wavefront each (the W strips' elements then come through the scalar cache)
+    ((1, 3), (4, 1040), (3, 3), (1, 1), (1, 1), (1, 1)),
+    ((2, 2), (6, 528), (3, 3), (1, 1), (1, 1), (1, 1)),
+    ((2, 3), (5, 600), (3, 5), (1, 1), (1, 2), (1, 1)),  # two columns wide: the per-column path on long rows
     # spans that drift against the tiles: the halo widths change from rank to rank
     ((2, 2), (8, 10), (3, 3), (1, 1), (0, 0), (1, 1)),  # no padding: (lo 0, hi 1) on rank 0, (lo 1, hi 0) on rank 1
     ((4, 2), (6, 8), (5, 3), (1, 1), (0, 0), (1, 1)),   # four ranks: (lo r, hi 3 - r)
