@@ -384,7 +384,8 @@ int jg_lse_merge(void* o1, const float* l1, const void* o2, const float* l2,
  * `padding` is the LOCAL padding of the call: zero on split axes, whose halo is
  * already in x (jigsaw/modules/convolution/_common/spatial_split.py:75-82).
  * out = (in + 2*padding - dilation*(kernel-1) - 1) / stride + 1 per axis.
- * groups must be 1.
+ * groups >= 1 divides c_in and c_out; w is then (Cout, Cin / groups, *kernel), as
+ * torch's. groups > 1 runs the direct kernels (the matrix-core kernels take groups = 1).
  *
  * Workspace: query with jg_conv_workspace_bytes(desc, op, dtype) (op: 0 = fwd,
  * 1 = dgrad, 2 = wgrad); may be 0, then `workspace` may be NULL. Contents are
@@ -392,7 +393,7 @@ int jg_lse_merge(void* o1, const float* l1, const void* o2, const float* l2,
  * ------------------------------------------------------------------------- */
 typedef struct {
   int32_t n_spatial; /* 1, 2 or 3 */
-  int32_t groups;    /* 1 */
+  int32_t groups;    /* >= 1, divides c_in and c_out */
   int64_t batch;
   int32_t c_in;
   int32_t c_out;

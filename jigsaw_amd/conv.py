@@ -82,8 +82,8 @@ def _workspace(desc: _lib.ConvDesc, op: int, dtype: torch.dtype, device) -> tupl
 def _check_args(x_like, w, groups, padding):
     if isinstance(padding, str):
         raise NotImplementedError(f"string padding ({padding!r}) is not supported; pass per-axis integers")
-    if groups != 1:
-        raise NotImplementedError(f"groups = {groups}: only groups = 1 is covered by the HIP kernels")
+    if not isinstance(groups, int) or groups < 1 or w.shape[0] % groups:
+        raise ValueError(f"groups = {groups} must be a positive integer that divides the {w.shape[0]} output channels")
     n = w.dim() - 2
     if n not in (1, 2, 3):
         raise ValueError(f"weight must be (Cout, Cin, *kernel) with 1 to 3 spatial axes, got {tuple(w.shape)}")
@@ -263,26 +263,27 @@ def conv_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1) -> torch
         raise ValueError(f"expected a batched (N, C, *spatial) input with {n} spatial axes, got {tuple(x.shape)}")
     if x.dtype != w.dtype or (b is not None and b.dtype != x.dtype):
         raise RuntimeError(f"Input type ({x.dtype}) and weight / bias type ({w.dtype}) should be the same")
-    if x.shape[1] != w.shape[1]:
-        raise RuntimeError(f"expected input to have {w.shape[1]} channels, but got {x.shape[1]} channels instead")
+    if x.shape[1] != w.shape[1] * groups:
+        raise RuntimeError(f"expected input to have {w.shape[1] * groups} channels, but got {x.shape[1]} channels instead")
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
-    if _dense_stride_ok(tuple(w.shape[2:]), stride, dilation, padding):
+    plain = groups == 1  # the routes below re-shape ungrouped layers; grouped ones run the direct kernels as they are
+    if plain and _dense_stride_ok(tuple(w.shape[2:]), stride, dilation, padding):
         out_sp = _out_spatial(x.shape[2:], w.shape[2:], stride, padding, dilation)
         dense = conv_nd(x, w, b, stride=1, padding=padding, dilation=dilation)
         return dense[(slice(None), slice(None)) + tuple(slice(0, (o - 1) * s + 1, s) for o, s in zip(out_sp, stride))].contiguous()
-    if _dilated_ok(tuple(w.shape[2:]), stride, padding, dilation):
+    if plain and _dilated_ok(tuple(w.shape[2:]), stride, padding, dilation):
         phases = _phase_counts(w.shape[2:], dilation)
         out_sp = _out_spatial(x.shape[2:], w.shape[2:], stride, padding, dilation)
         ext_in = tuple(-(-int(i) // p) for i, p in zip(x.shape[2:], phases))
         yb = conv_nd(_to_phases(x, phases, ext_in), w, b, stride=1, padding=tuple(pp // p for pp, p in zip(padding, phases)))
         return _from_phases(yb, phases, x.shape[0], out_sp)
-    off = _embed3(tuple(w.shape[2:]), stride, dilation)
+    off = _embed3(tuple(w.shape[2:]), stride, dilation) if plain else None
     if off is not None:
         return conv_nd(x, _embed_weight(w, off), b, stride=1, padding=tuple(p + o for p, o in zip(padding, off)))
     x, w = x.contiguous(), w.contiguous()
     b = None if b is None else b.contiguous()
     out_sp = _out_spatial(x.shape[2:], w.shape[2:], stride, padding, dilation)
-    if _patch_gemm_ok(x.dtype, x.shape[1], w.shape[0], w.shape[2:], stride, padding, dilation):
+    if plain and _patch_gemm_ok(x.dtype, x.shape[1], w.shape[0], w.shape[2:], stride, padding, dilation):
         y_tok = _proj_nt(_patchify(x, w.shape[2:], out_sp), w.reshape(w.shape[0], -1), b)
         return y_tok.reshape(x.shape[0], *out_sp, w.shape[0]).permute(0, n + 1, *range(1, n + 1)).contiguous()
     y = torch.empty((x.shape[0], w.shape[0], *out_sp), dtype=x.dtype, device=x.device)
@@ -306,10 +307,13 @@ def conv_nd_input(input_shape, w, g, *, stride=1, padding=0, dilation=1, groups=
     if g.dtype != w.dtype:
         raise RuntimeError(f"grad_output type ({g.dtype}) and weight type ({w.dtype}) should be the same")
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
-    if _dense_stride_ok(tuple(w.shape[2:]), stride, dilation, padding):
+    if input_shape[1] != w.shape[1] * groups:
+        raise ValueError(f"input_shape has {input_shape[1]} channels, the weight takes {w.shape[1] * groups}")
+    plain = groups == 1  # as in conv_nd
+    if plain and _dense_stride_ok(tuple(w.shape[2:]), stride, dilation, padding):
         dense_sp = _out_spatial(input_shape[2:], w.shape[2:], (1,) * n, padding, dilation)
         return conv_nd_input(input_shape, w, _stuffed(g, dense_sp, stride), stride=1, padding=padding, dilation=dilation)
-    if _dilated_ok(tuple(w.shape[2:]), stride, padding, dilation):
+    if plain and _dilated_ok(tuple(w.shape[2:]), stride, padding, dilation):
         phases = _phase_counts(w.shape[2:], dilation)
         out_sp = _out_spatial(input_shape[2:], w.shape[2:], stride, padding, dilation)
         if tuple(g.shape) != (input_shape[0], w.shape[0], *out_sp):
@@ -320,7 +324,7 @@ def conv_nd_input(input_shape, w, g, *, stride=1, padding=0, dilation=1, groups=
         gxb = conv_nd_input((g.shape[0] * math.prod(phases), input_shape[1], *ext_in), w, _to_phases(g, phases, ext_out),
                             stride=1, padding=pad0)
         return _from_phases(gxb, phases, input_shape[0], input_shape[2:])
-    off = _embed3(tuple(w.shape[2:]), stride, dilation)
+    off = _embed3(tuple(w.shape[2:]), stride, dilation) if plain else None
     if off is not None:
         return conv_nd_input(input_shape, _embed_weight(w, off), g, stride=1,
                              padding=tuple(p + o for p, o in zip(padding, off)))
@@ -331,7 +335,7 @@ def conv_nd_input(input_shape, w, g, *, stride=1, padding=0, dilation=1, groups=
             f"grad_output shape {tuple(g.shape)} does not match the convolution of an input of shape {input_shape} "
             f"(expected {(input_shape[0], w.shape[0], *out_sp)})"
         )
-    if _patch_gemm_ok(g.dtype, w.shape[1], w.shape[0], w.shape[2:], stride, padding, dilation):
+    if plain and _patch_gemm_ok(g.dtype, w.shape[1], w.shape[0], w.shape[2:], stride, padding, dilation):
         # gradient of every patch = g_tokens x W, then back to the image layout
         w2t = w.reshape(w.shape[0], -1).t().contiguous()
         return _unpatchify(_proj_nt(_tokens_of(g).contiguous(), w2t, None), input_shape, w.shape[2:], out_sp)
@@ -443,11 +447,11 @@ def conv_nd_input_fold(geom: HaloGeometry, w, g, *, stride=1, padding=0, dilatio
         raise RuntimeError(f"grad_output type ({g.dtype}) and weight type ({w.dtype}) should be the same")
     if geom.n_spatial != n:
         raise ValueError(f"geometry has {geom.n_spatial} spatial axes, the convolution {n}")
-    if g.dtype != torch.bfloat16:  # the fold epilogue exists for bf16 only: say so before sizing a workspace
+    if g.dtype != torch.bfloat16 or groups != 1:  # the fold epilogue exists for ungrouped bf16 layers: say so before sizing a workspace
         return None
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
     g, w = g.contiguous(), w.contiguous()
-    batch, c_in = int(g.shape[0]), int(w.shape[1])
+    batch, c_in = int(g.shape[0]), int(w.shape[1]) * groups
     padded = geom.padded
     out_sp = _out_spatial(padded, w.shape[2:], stride, padding, dilation)
     if tuple(g.shape) != (batch, w.shape[0], *out_sp):
@@ -482,16 +486,17 @@ def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, group
     n = len(weight_shape) - 2
     if isinstance(padding, str):
         raise NotImplementedError(f"string padding ({padding!r}) is not supported; pass per-axis integers")
-    if groups != 1:
-        raise NotImplementedError(f"groups = {groups}: only groups = 1 is covered by the HIP kernels")
+    if not isinstance(groups, int) or groups < 1 or weight_shape[0] % groups:
+        raise ValueError(f"groups = {groups} must be a positive integer that divides the {weight_shape[0]} output channels")
     if x.dtype != g.dtype:
         raise RuntimeError(f"input type ({x.dtype}) and grad_output type ({g.dtype}) should be the same")
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
-    if _dense_stride_ok(weight_shape[2:], stride, dilation, padding):
+    plain = groups == 1  # as in conv_nd
+    if plain and _dense_stride_ok(weight_shape[2:], stride, dilation, padding):
         dense_sp = _out_spatial(x.shape[2:], weight_shape[2:], (1,) * n, padding, dilation)
         return conv_nd_weight(x, weight_shape, _stuffed(g, dense_sp, stride), stride=1, padding=padding, dilation=dilation,
                               with_bias_grad=with_bias_grad)
-    if _dilated_ok(weight_shape[2:], stride, padding, dilation):
+    if plain and _dilated_ok(weight_shape[2:], stride, padding, dilation):
         phases = _phase_counts(weight_shape[2:], dilation)
         out_sp = _out_spatial(x.shape[2:], weight_shape[2:], stride, padding, dilation)
         if tuple(g.shape) != (x.shape[0], weight_shape[0], *out_sp) or x.shape[1] != weight_shape[1]:
@@ -502,7 +507,7 @@ def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, group
         # every residue image is one more batch entry of the undilated layer: the sum over the batch is the answer
         return conv_nd_weight(_to_phases(x, phases, ext_in), weight_shape, _to_phases(g, phases, ext_out), stride=1,
                               padding=pad0, with_bias_grad=with_bias_grad)
-    off = _embed3(weight_shape[2:], stride, dilation)
+    off = _embed3(weight_shape[2:], stride, dilation) if plain else None
     if off is not None:
         # gradient of the 3 x 3 (x 3) kernel the weights sit in; its centre taps are the answer
         res = conv_nd_weight(x, weight_shape[:2] + (3,) * n, g, stride=1,
@@ -512,9 +517,9 @@ def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, group
         return (gw, res[1]) if with_bias_grad else gw
     x, g = x.contiguous(), g.contiguous()
     out_sp = _out_spatial(x.shape[2:], weight_shape[2:], stride, padding, dilation)
-    if tuple(g.shape) != (x.shape[0], weight_shape[0], *out_sp) or x.shape[1] != weight_shape[1]:
+    if tuple(g.shape) != (x.shape[0], weight_shape[0], *out_sp) or x.shape[1] != weight_shape[1] * groups:
         raise ValueError(f"grad_output {tuple(g.shape)} / input {tuple(x.shape)} do not match weight {weight_shape}")
-    if _patch_gemm_ok(x.dtype, weight_shape[1], weight_shape[0], weight_shape[2:], stride, padding, dilation):
+    if plain and _patch_gemm_ok(x.dtype, weight_shape[1], weight_shape[0], weight_shape[2:], stride, padding, dilation):
         # gw = g_tokens^T x patches (contraction over the patches), the bias gradient from the same pass
         patches, g_tok = _patchify(x, weight_shape[2:], out_sp), _tokens_of(g).contiguous()
         rows, k = patches.shape
@@ -668,7 +673,7 @@ def conv_halo_nway(x, w, b, stride, padding, dilation, spatial_groups, channel_g
     present = _present_offsets(geom, ranks, sizes)
     send = halo_pack(x, geom, from_padded=False, present=present) if present else {}
     recv = config.halo_exchange.forward(send) if present else {}
-    kwargs = {"stride": stride, "padding": _local_padding(padding, sizes), "dilation": dilation, "groups": 1}
+    kwargs = {"stride": stride, "padding": _local_padding(padding, sizes), "dilation": dilation, "groups": int(getattr(config, "groups_local", 1))}
     bands = _frame_decision(config, x, geom, w.shape, kwargs)
     if bands is not None:
         # only the frame of the padded tile is built; the kernels read the tile itself elsewhere.
@@ -703,7 +708,7 @@ def conv_halo_nway_backward(
     want_b = len(need) > 2
     need_b = want_b and need[2]
     g = grad_output.to(weight.dtype)
-    kwargs = {"stride": stride, "padding": local_padding, "dilation": dilation, "groups": 1}
+    kwargs = {"stride": stride, "padding": local_padding, "dilation": dilation, "groups": int(getattr(config, "groups_local", 1))}
     g_w = g_b = None
     if x_tile is None and need_w and getattr(config, "framed", False) and getattr(x_aug, "_jg_frame_only", False):
         raise RuntimeError(
@@ -813,10 +818,10 @@ class _HipLayerConfig:
         size = channel_group.size()
         self.channel_local = groups % size == 0
         self.groups_local = groups // size if self.channel_local else 1
-        if size != 1 or groups != 1:
+        if size != 1:
             raise NotImplementedError(
-                "the HIP kernel table covers channel-local layers with groups = 1 "
-                f"(channel group size {size}, groups {groups})"
+                f"the HIP kernel table covers channel-local layers (channel group size {size}); "
+                "channel-sharded convolution is outside this package"
             )
         self.grad_bias = self._no_bias if bias is None else self._sum_grad_bias
 
@@ -901,7 +906,7 @@ class _ConvNd(torch.autograd.Function):
             n = config.n_spatial
             ranks, sizes = _mesh_position(spatial_groups)
             geom = HaloGeometry.for_conv(x.shape[-n:], weight.shape[-n:], stride, padding, dilation, ranks, sizes)
-            kwargs = {"stride": stride, "padding": _local_padding(padding, sizes), "dilation": dilation, "groups": 1}
+            kwargs = {"stride": stride, "padding": _local_padding(padding, sizes), "dilation": dilation, "groups": int(getattr(config, "groups_local", 1))}
             x_c = x if x.dtype == x_aug.dtype else torch.empty(0, dtype=x_aug.dtype, device=x.device).new_empty(x.shape)
             ctx.framed = _frame_decision(config, x_c, geom, weight.shape, kwargs) is not None
         if ctx.framed:

@@ -105,7 +105,7 @@ def conv_transpose_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1
     tup = lambda v: (v,) * n if isinstance(v, int) else tuple(v)  # noqa: E731
     s, p, d = tup(stride), tup(padding), tup(dilation)
     raw = tuple((x.shape[2 + a] - 1) * s[a] - 2 * p[a] + d[a] * (w.shape[2 + a] - 1) + 1 for a in range(n))
-    y = conv_nd_input((x.shape[0], w.shape[1], *raw), w, x, stride=s, padding=p, dilation=d, groups=groups)
+    y = conv_nd_input((x.shape[0], w.shape[1] * groups, *raw), w, x, stride=s, padding=p, dilation=d, groups=groups)
     if b is not None:
         y += b.to(y.dtype).view((1, -1) + (1,) * n)
     return y
@@ -124,14 +124,14 @@ def conv_transpose_halo_nway(x, w, b, stride, padding, dilation, spatial_groups,
     x = x.contiguous()
     geom = transpose_geometry(x.shape[-n:], w.shape[-n:], stride, padding, dilation, ranks, sizes)
     present = _present_offsets(geom, ranks, sizes)
-    kwargs = {"stride": stride, "padding": _local_padding(padding, sizes), "dilation": dilation, "groups": 1}
+    kwargs = {"stride": stride, "padding": _local_padding(padding, sizes), "dilation": dilation, "groups": int(getattr(config, "groups_local", 1))}
     fused = conv_nd_input_fold(geom, w, x, present=present, **kwargs) if getattr(config, "fused_fold", False) else None
     if fused is not None:
         y, send = fused
         recv = config.halo_exchange.forward(send) if present else {}
         halo_fold_border_(y, recv, geom)
     else:
-        y_raw = conv_nd_input((x.shape[0], w.shape[1], *geom.padded), w, x, **kwargs)
+        y_raw = conv_nd_input((x.shape[0], w.shape[1] * kwargs["groups"], *geom.padded), w, x, **kwargs)
         send = halo_pack(y_raw, geom, from_padded=True, present=present) if present else {}
         recv = config.halo_exchange.forward(send) if present else {}
         y = halo_fold(y_raw, recv, geom)
@@ -159,7 +159,7 @@ def conv_transpose_halo_nway_backward(
     send = halo_pack(g, geom, from_padded=False, present=present) if present else {}
     recv = config.halo_exchange.backward(send) if present else {}
     g_raw = halo_assemble(g, recv, geom)
-    kwargs = {"stride": stride, "padding": _local_padding(padding, sizes), "dilation": dilation, "groups": 1}
+    kwargs = {"stride": stride, "padding": _local_padding(padding, sizes), "dilation": dilation, "groups": int(getattr(config, "groups_local", 1))}
     g_x = conv_nd(g_raw, weight, None, **kwargs) if need_x else None
     g_w = conv_nd_weight(g_raw, weight.shape, x_aug.to(weight.dtype), **kwargs) if need_w else None
     return g_x, g_w

@@ -9,9 +9,11 @@ int resolve_conv(const jg_conv_desc* d, const char* who, ConvGeom* out) {
   JG_REQUIRE(d != nullptr, "%s: desc is NULL", who);
   JG_REQUIRE(d->n_spatial >= 1 && d->n_spatial <= 3, "%s: n_spatial %d not in 1..3", who,
              d->n_spatial);
-  if (d->groups != 1) JG_FAIL(JG_ERR_UNSUPPORTED, "%s: groups = %d (only 1)", who, d->groups);
   JG_REQUIRE(d->batch >= 0 && d->c_in >= 1 && d->c_out >= 1, "%s: bad batch / channels", who);
+  JG_REQUIRE(d->groups >= 1 && d->c_in % d->groups == 0 && d->c_out % d->groups == 0,
+             "%s: groups = %d must divide the channels (%d in, %d out)", who, d->groups, d->c_in, d->c_out);
   ConvGeom g;
+  g.groups = d->groups;
   g.batch = d->batch;
   g.cin = d->c_in;
   g.cout = d->c_out;

@@ -7,7 +7,8 @@ namespace jg {
 // Resolved geometry; 1-D and 2-D problems carry leading axes of extent 1.
 struct ConvGeom {
   long long batch;
-  int cin, cout;
+  int cin, cout;  // channels of the whole tensors
+  int groups;     // cin and cout divide into `groups` independent blocks (F.conv's groups)
   int in[3];   // input spatial extent (the padded tile)
   int out[3];  // output spatial extent
   int k[3], s[3], p[3], d[3];

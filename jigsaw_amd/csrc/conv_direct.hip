@@ -48,7 +48,11 @@ __global__ __launch_bounds__(256) void direct_fwd_kernel(typename Elem<DT>::T* _
   const long long si = (long long)g.in[0] * g.in[1] * g.in[2];
   const int taps = g.k[0] * g.k[1] * g.k[2];
   const long long sp = (long long)blockIdx.x * 256 + threadIdx.x;
-  const int co0 = blockIdx.y * kCB;
+  // blockIdx.y = (group, block of kCB of the group's output channels)
+  const int cin_g = g.cin / g.groups, cout_g = g.cout / g.groups;
+  const int blocks_g = (cout_g + kCB - 1) / kCB;
+  const int grp = blockIdx.y / blocks_g;
+  const int co0 = grp * cout_g + (blockIdx.y - grp * blocks_g) * kCB, co_end = (grp + 1) * cout_g;
   const long long n = blockIdx.z;
   if (sp >= so) return;
   const int ow = (int)(sp % g.out[2]);
@@ -58,9 +62,9 @@ __global__ __launch_bounds__(256) void direct_fwd_kernel(typename Elem<DT>::T* _
   float acc[kCB];
 #pragma unroll
   for (int j = 0; j < kCB; ++j)
-    acc[j] = (bias != nullptr && co0 + j < g.cout) ? Elem<DT>::up(bias[co0 + j]) : 0.0f;
-  const typename Elem<DT>::T* xn = x + n * g.cin * si;
-  for (int ci = 0; ci < g.cin; ++ci) {
+    acc[j] = (bias != nullptr && co0 + j < co_end) ? Elem<DT>::up(bias[co0 + j]) : 0.0f;
+  const typename Elem<DT>::T* xn = x + (n * g.cin + (long long)grp * cin_g) * si;
+  for (int ci = 0; ci < cin_g; ++ci) {
     for (int kd = 0; kd < g.k[0]; ++kd) {
       const int id = od * g.s[0] - g.p[0] + kd * g.d[0];
       if (id < 0 || id >= g.in[0]) continue;
@@ -75,8 +79,8 @@ __global__ __launch_bounds__(256) void direct_fwd_kernel(typename Elem<DT>::T* _
           const int tap = (kd * g.k[1] + kh) * g.k[2] + kw;
 #pragma unroll
           for (int j = 0; j < kCB; ++j) {
-            if (co0 + j < g.cout)
-              acc[j] += xv * Elem<DT>::up(w[((long long)(co0 + j) * g.cin + ci) * taps + tap]);
+            if (co0 + j < co_end)
+              acc[j] += xv * Elem<DT>::up(w[((long long)(co0 + j) * cin_g + ci) * taps + tap]);
           }
         }
       }
@@ -84,7 +88,7 @@ __global__ __launch_bounds__(256) void direct_fwd_kernel(typename Elem<DT>::T* _
   }
 #pragma unroll
   for (int j = 0; j < kCB; ++j)
-    if (co0 + j < g.cout) y[(n * g.cout + co0 + j) * so + sp] = Elem<DT>::down(acc[j]);
+    if (co0 + j < co_end) y[(n * g.cout + co0 + j) * so + sp] = Elem<DT>::down(acc[j]);
 }
 
 // --------------------------------------------------------------------- dgrad
@@ -96,7 +100,12 @@ __global__ __launch_bounds__(256) void direct_dgrad_kernel(
   const long long si = (long long)g.in[0] * g.in[1] * g.in[2];
   const int taps = g.k[0] * g.k[1] * g.k[2];
   const long long sp = (long long)blockIdx.x * 256 + threadIdx.x;
-  const int ci0 = blockIdx.y * kCB;
+  // blockIdx.y = (group, block of kCB of the group's input channels)
+  const int cin_g = g.cin / g.groups, cout_g = g.cout / g.groups;
+  const int blocks_g = (cin_g + kCB - 1) / kCB;
+  const int grp = blockIdx.y / blocks_g;
+  const int cl0 = (blockIdx.y - grp * blocks_g) * kCB;  // first channel of the block inside its group
+  const int ci0 = grp * cin_g + cl0;
   const long long n = blockIdx.z;
   if (sp >= si) return;
   const int iw = (int)(sp % g.in[2]);
@@ -106,7 +115,7 @@ __global__ __launch_bounds__(256) void direct_dgrad_kernel(
   float acc[kCB];
 #pragma unroll
   for (int j = 0; j < kCB; ++j) acc[j] = 0.0f;
-  const typename Elem<DT>::T* gn = go + n * g.cout * so;
+  const typename Elem<DT>::T* gn = go + (n * g.cout + (long long)grp * cout_g) * so;
   for (int kd = 0; kd < g.k[0]; ++kd) {
     const int td = id + g.p[0] - kd * g.d[0];
     if (td < 0 || td % g.s[0]) continue;
@@ -124,19 +133,19 @@ __global__ __launch_bounds__(256) void direct_dgrad_kernel(
         if (ow >= g.out[2]) continue;
         const int tap = (kd * g.k[1] + kh) * g.k[2] + kw;
         const long long po = ((long long)od * g.out[1] + oh) * g.out[2] + ow;
-        for (int co = 0; co < g.cout; ++co) {
+        for (int co = 0; co < cout_g; ++co) {
           const float gv = Elem<DT>::up(gn[co * so + po]);
 #pragma unroll
           for (int j = 0; j < kCB; ++j)
-            if (ci0 + j < g.cin)
-              acc[j] += gv * Elem<DT>::up(w[((long long)co * g.cin + ci0 + j) * taps + tap]);
+            if (cl0 + j < cin_g)
+              acc[j] += gv * Elem<DT>::up(w[((long long)(grp * cout_g + co) * cin_g + cl0 + j) * taps + tap]);
         }
       }
     }
   }
 #pragma unroll
   for (int j = 0; j < kCB; ++j)
-    if (ci0 + j < g.cin) gx[(n * g.cin + ci0 + j) * si + sp] = Elem<DT>::down(acc[j]);
+    if (cl0 + j < cin_g) gx[(n * g.cin + ci0 + j) * si + sp] = Elem<DT>::down(acc[j]);
 }
 
 // --------------------------------------------------------------------- wgrad
@@ -150,8 +159,8 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   return red[0] + red[1] + red[2] + red[3];
 }
 
-// Stage 1: block (chunk, ci, co) reduces its share of the N*Do*Ho*Wo domain for
-// every tap; part[chunk][co][ci][tap].
+// Stage 1: block (chunk, ci inside the group of co, co) reduces its share of the N*Do*Ho*Wo
+// domain for every tap; part[chunk][co][ci in group][tap].
 template <int DT>
 __global__ __launch_bounds__(256) void direct_wgrad_kernel(float* __restrict__ part,
                                                            const typename Elem<DT>::T* __restrict__ x,
@@ -162,7 +171,9 @@ __global__ __launch_bounds__(256) void direct_wgrad_kernel(float* __restrict__ p
   const long long si = (long long)g.in[0] * g.in[1] * g.in[2];
   const long long dom = g.batch * so;
   const int taps = g.k[0] * g.k[1] * g.k[2];
-  const int ci = blockIdx.y, co = blockIdx.z;
+  const int cin_g = g.cin / g.groups;
+  const int co = blockIdx.z, cil = blockIdx.y;  // cil: channel inside the group
+  const int ci = (co / (g.cout / g.groups)) * cin_g + cil;
   const long long r0 = (long long)blockIdx.x * chunk_len;
   long long r1 = r0 + chunk_len;
   if (r1 > dom) r1 = dom;
@@ -190,7 +201,7 @@ __global__ __launch_bounds__(256) void direct_wgrad_kernel(float* __restrict__ p
         s = block_sum(s, red);
         const int tap = (kd * g.k[1] + kh) * g.k[2] + kw;
         if (threadIdx.x == 0)
-          part[(((long long)blockIdx.x * g.cout + co) * g.cin + ci) * taps + tap] = s;
+          part[(((long long)blockIdx.x * g.cout + co) * cin_g + cil) * taps + tap] = s;
       }
 }
 
@@ -278,7 +289,7 @@ size_t direct_wgrad_workspace(const ConvGeom& g) {
   long long len;
   const long long so = (long long)g.out[0] * g.out[1] * g.out[2];
   const int chunks = wgrad_chunks(g.batch * so, &len);
-  return (size_t)chunks * g.cout * g.cin * g.k[0] * g.k[1] * g.k[2] * sizeof(float);
+  return (size_t)chunks * g.cout * (g.cin / g.groups) * g.k[0] * g.k[1] * g.k[2] * sizeof(float);
 }
 
 int direct_fwd(void* y, const void* x, const void* w, const void* bias, const ConvGeom& g,
@@ -286,7 +297,7 @@ int direct_fwd(void* y, const void* x, const void* w, const void* bias, const Co
   const long long so = (long long)g.out[0] * g.out[1] * g.out[2];
   if (g.batch == 0 || so == 0) return JG_OK;
   JG_REQUIRE(g.batch <= 65535, "conv fwd (direct): batch %lld exceeds 65535", (long long)g.batch);
-  dim3 grid((unsigned)((so + 255) / 256), (unsigned)((g.cout + kCB - 1) / kCB), (unsigned)g.batch);
+  dim3 grid((unsigned)((so + 255) / 256), (unsigned)(g.groups * ((g.cout / g.groups + kCB - 1) / kCB)), (unsigned)g.batch);
 #define JG_GO(DT)                                                                           \
   direct_fwd_kernel<DT><<<grid, 256, 0, s>>>(                                               \
       static_cast<Elem<DT>::T*>(y), static_cast<const Elem<DT>::T*>(x),                     \
@@ -305,7 +316,7 @@ int direct_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, int
   if (g.batch == 0 || si == 0) return JG_OK;
   JG_REQUIRE(g.batch <= 65535, "conv dgrad (direct): batch %lld exceeds 65535",
              (long long)g.batch);
-  dim3 grid((unsigned)((si + 255) / 256), (unsigned)((g.cin + kCB - 1) / kCB), (unsigned)g.batch);
+  dim3 grid((unsigned)((si + 255) / 256), (unsigned)(g.groups * ((g.cin / g.groups + kCB - 1) / kCB)), (unsigned)g.batch);
 #define JG_GO(DT)                                                                           \
   direct_dgrad_kernel<DT><<<grid, 256, 0, s>>>(                                             \
       static_cast<Elem<DT>::T*>(gx), static_cast<const Elem<DT>::T*>(w),                    \
@@ -321,7 +332,7 @@ int direct_dgrad(void* gx, const void* w, const void* go, const ConvGeom& g, int
 int direct_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, int dtype, void* ws,
                  size_t ws_bytes, hipStream_t s) {
   const long long so = (long long)g.out[0] * g.out[1] * g.out[2];
-  const long long count = (long long)g.cout * g.cin * g.k[0] * g.k[1] * g.k[2];
+  const long long count = (long long)g.cout * (g.cin / g.groups) * g.k[0] * g.k[1] * g.k[2];
   if (count == 0) return JG_OK;
   JG_REQUIRE(g.cin <= 65535 && g.cout <= 65535, "conv wgrad (direct): too many channels");
   long long len;
@@ -331,7 +342,7 @@ int direct_wgrad(void* gw, const void* x, const void* go, const ConvGeom& g, int
             direct_wgrad_workspace(g));
   float* part = static_cast<float*>(ws);
   const bool empty = (g.batch * so == 0);  // nothing to reduce: the gradient is zero
-  dim3 grid((unsigned)chunks, (unsigned)g.cin, (unsigned)g.cout);
+  dim3 grid((unsigned)chunks, (unsigned)(g.cin / g.groups), (unsigned)g.cout);
 #define JG_GO(DT)                                                                          \
   do {                                                                                     \
     if (!empty)                                                                            \

@@ -1132,6 +1132,7 @@ namespace jg {
 // fp32 runs in split mode; fp16 has its own MFMA instruction and runs like bf16
 static int split_mode(int dtype) { return dtype == JG_F32 ? 1 : 0; }
 static bool dtype_ok(const ConvGeom& g, int dtype) {
+  if (g.groups != 1) return false;  // grouped layers run the direct kernels
   if (dtype == JG_BF16 || dtype == JG_F16) return true;
   if (dtype != JG_F32) return false;
   const size_t in_sz = (size_t)g.in[0] * g.in[1] * g.in[2], out_sz = (size_t)g.out[0] * g.out[1] * g.out[2];

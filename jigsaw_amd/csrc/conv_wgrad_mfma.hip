@@ -704,6 +704,7 @@ struct Blocking {
   int cib_max() const { return KD == 3 ? 32 : 64; }
 };
 bool blocks_of(const ConvGeom& g, Blocking* b) {
+  if (g.groups != 1) return false;
   if (g.k[1] != 3 || g.k[2] != 3 || (g.k[0] != 1 && g.k[0] != 3)) return false;
   if (g.k[0] == 1 && g.in[0] != 1) return false;
   for (int a = 0; a < 3; ++a)

@@ -86,8 +86,8 @@ def test_short_form_and_unsupported_layers():
     assert cfg.framed and cfg._layer_key["n_spatial"] == 3 and not cfg._layer_key["kernel_size == stride"]
     with pytest.raises(NotImplementedError):
         jc.HipConvNdConfig(jc.TileGroup(2, 1), None, (3, 3), (1, 1), torch.device("cuda"))
-    with pytest.raises(NotImplementedError):
-        jc.HipConvNdConfig(jc.TileGroup(1, 0), None, (3, 3), (1, 1), torch.device("cuda"), groups=2)
+    grouped = jc.HipConvNdConfig(jc.TileGroup(1, 0), None, (3, 3), (1, 1), torch.device("cuda"), groups=2)
+    assert grouped.groups == 2 and grouped.groups_local == 2 and grouped.channel_local and grouped._layer_key["groups"] == 2
     with pytest.raises(ValueError):
         jc.HipConvNdConfig(jc.TileGroup(1, 0), None, (3, 3), (1, 1), torch.device("cuda"), channel_comm="carrier_pigeon")
     with pytest.raises(ValueError):

@@ -87,45 +87,55 @@ PRIM_CASES = [
     (1, 32, 32, (6, 19, 34), (3, 3, 3), (1, 1, 1), (1, 2, 2), (1, 2, 2)),
     (2, 16, 32, (33, 40), (3, 3), (2, 2), (2, 2), (2, 2)),   # strided and dilated
     (1, 4, 6, (17, 23), (3, 3), (1, 1), (1, 1), (2, 2)),     # padding not a multiple: the direct kernels
+    # grouped layers (ninth entry: groups), depthwise among them: the direct kernels
+    (2, 8, 12, (13, 17), (3, 3), (1, 1), (1, 1), (1, 1), 4),
+    (1, 32, 32, (20, 22), (3, 3), (1, 1), (1, 1), (1, 1), 32),
+    (2, 6, 9, (11, 14), (3, 5), (2, 1), (1, 2), (1, 2), 3),
+    (1, 16, 16, (5, 9, 10), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 2),
+    (2, 64, 64, (18, 34), (3, 3), (1, 1), (0, 0), (1, 1), 2),   # a shape the MFMA kernels would take ungrouped
+    (1, 12, 8, (30,), (5,), (1,), (2,), (1,), 4),
 ]
 
 
 def _pid(c):
-    return "n{}_ci{}_co{}_in{}_k{}_s{}_p{}_d{}".format(c[0], c[1], c[2], *["x".join(map(str, v)) for v in c[3:]])
+    name = "n{}_ci{}_co{}_in{}_k{}_s{}_p{}_d{}".format(c[0], c[1], c[2], *["x".join(map(str, v)) for v in c[3:8]])
+    return name + (f"_g{c[8]}" if len(c) > 8 else "")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("case", PRIM_CASES, ids=_pid)
 def test_conv_primitives_match_oracle(case, dtype, dev):
-    N, cin, cout, insp, k, s, p, d = case
+    N, cin, cout, insp, k, s, p, d = case[:8]
+    groups = case[8] if len(case) > 8 else 1
     torch.manual_seed(0)
     x = torch.randn(N, cin, *insp).to(dtype)
-    fan_in = cin * int(torch.tensor(k).prod())
-    w = ((torch.rand(cout, cin, *k) * 2 - 1) / fan_in**0.5).to(dtype)
+    fan_in = cin // groups * int(torch.tensor(k).prod())
+    w = ((torch.rand(cout, cin // groups, *k) * 2 - 1) / fan_in**0.5).to(dtype)
     b = (torch.randn(cout) * 0.1).to(dtype)
     xd, wd, bd = x.double(), w.double(), b.double()
-    y_want = oc.forward(xd, wd, bd, s, p, d)
+    y_want = oc.forward(xd, wd, bd, s, p, d, groups)
     g = torch.randn_like(y_want).to(dtype)
     gd = g.double()
-    gx_want = oc.dgrad(x.shape, wd, gd, s, p, d)
-    gw_want = oc.wgrad(xd, w.shape, gd, s, p, d)
+    gx_want = oc.dgrad(x.shape, wd, gd, s, p, d, groups)
+    gw_want = oc.wgrad(xd, w.shape, gd, s, p, d, groups)
     gb_want = oc.grad_bias(gd, len(k))
 
     xg, wg, bg, gg = x.to(dev), w.to(dev), b.to(dev), g.to(dev)
-    y = jc.conv_nd(xg, wg, bg, stride=s, padding=p, dilation=d)
+    kw = dict(stride=s, padding=p, dilation=d, groups=groups)
+    y = jc.conv_nd(xg, wg, bg, **kw)
     assert y.dtype == dtype and y.shape == y_want.shape
     assert rel_l2(y, y_want) < TOL[dtype], f"fwd rel-L2 {rel_l2(y, y_want):.3e}"
-    y0 = jc.conv_nd(xg, wg, None, stride=s, padding=p, dilation=d)
-    assert rel_l2(y0, oc.forward(xd, wd, None, s, p, d)) < TOL[dtype]
-    gx = jc.conv_nd_input(x.shape, wg, gg, stride=s, padding=p, dilation=d)
+    y0 = jc.conv_nd(xg, wg, None, **kw)
+    assert rel_l2(y0, oc.forward(xd, wd, None, s, p, d, groups)) < TOL[dtype]
+    gx = jc.conv_nd_input(x.shape, wg, gg, **kw)
     assert rel_l2(gx, gx_want) < TOL[dtype], f"dgrad rel-L2 {rel_l2(gx, gx_want):.3e}"
-    gw = jc.conv_nd_weight(xg, w.shape, gg, stride=s, padding=p, dilation=d)
+    gw = jc.conv_nd_weight(xg, w.shape, gg, **kw)
     assert gw.shape == w.shape
     assert rel_l2(gw, gw_want) < TOL[dtype], f"wgrad rel-L2 {rel_l2(gw, gw_want):.3e}"
     gb = jc.sum_grad_bias(gg, len(k))
     assert rel_l2(gb, gb_want) < TOL[dtype], f"bias grad rel-L2 {rel_l2(gb, gb_want):.3e}"
     # both gradients from one pass over g (falls back to the two kernels where not covered)
-    gw2, gb2 = jc.conv_nd_weight(xg, w.shape, gg, stride=s, padding=p, dilation=d, with_bias_grad=True)
+    gw2, gb2 = jc.conv_nd_weight(xg, w.shape, gg, with_bias_grad=True, **kw)
     assert torch.equal(gw2, gw)
     assert gb2.dtype == dtype and rel_l2(gb2, gb_want) < TOL[dtype], f"fused bias grad rel-L2 {rel_l2(gb2, gb_want):.3e}"
 
@@ -154,8 +164,10 @@ def test_conv_argument_errors(dev):
     w = torch.zeros(4, 4, 3, 3, device=dev)
     with pytest.raises(NotImplementedError):
         jc.conv_nd(x, w, padding="same")
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError):  # 4 input channels against a weight that takes 4 per group, two groups
         jc.conv_nd(x, w, groups=2)
+    with pytest.raises(ValueError):
+        jc.conv_nd(x, w, groups=3)
     with pytest.raises(RuntimeError):
         jc.conv_nd(x, w.bfloat16())
     with pytest.raises(RuntimeError):

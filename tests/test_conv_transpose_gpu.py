@@ -146,3 +146,15 @@ def test_transposed_conv_primitive_equals_torch(dev):
         want = CONVT[len(shape) - 2](x.double(), w.double(), b.double(), stride=s, padding=p, dilation=d)
         got = jct.conv_transpose_nd(x.to(dev), w.to(dev), b.to(dev), stride=s, padding=p, dilation=d)
         assert rel_l2(got, want) < 1e-5
+
+
+@pytest.mark.gpu
+def test_grouped_transposed_conv_primitive_equals_torch(dev):
+    """``groups`` of ``F.conv_transpose2d``: the weight is (C_in, C_out / groups, *k) and the output has
+    ``groups`` times its second extent in channels."""
+    torch.manual_seed(4)
+    for groups, cin, cout_g in [(2, 6, 3), (4, 4, 1)]:
+        x, w, b = torch.randn(2, cin, 7, 9), torch.randn(cin, cout_g, 3, 4) * 0.3, torch.randn(cout_g * groups)
+        want = CONVT[2](x.double(), w.double(), b.double(), stride=(2, 1), padding=(1, 0), dilation=(1, 2), groups=groups)
+        got = jct.conv_transpose_nd(x.to(dev), w.to(dev), b.to(dev), stride=(2, 1), padding=(1, 0), dilation=(1, 2), groups=groups)
+        assert got.shape == want.shape and rel_l2(got, want) < 1e-5
