@@ -835,10 +835,11 @@ class _HipLayerConfig:
         return type(cls.__name__, (cls,), dict(options))
 
     @classmethod
-    def for_rank(cls, n_spatial: int, bias: Any, halo_exchange: HaloExchange | None = None, **options: Any):
+    def for_rank(cls, n_spatial: int, bias: Any, halo_exchange: HaloExchange | None = None, groups: int = 1,
+                 **options: Any):
         """Short form for a channel-local layer whose kernel is not its stride (the layers
-        that exchange halos): only the number of spatial axes and the bias matter."""
-        return cls(TileGroup(1, 0), bias, (3,) * int(n_spatial), (1,) * int(n_spatial), None,
+        that exchange halos): only the number of spatial axes, the bias and ``groups`` matter."""
+        return cls(TileGroup(1, 0), bias, (3,) * int(n_spatial), (1,) * int(n_spatial), None, groups=groups,
                    halo_exchange=halo_exchange, **options)
 
     def _no_bias(self, *args: Any, **kwargs: Any) -> None:

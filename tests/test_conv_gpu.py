@@ -234,10 +234,13 @@ DIST_CASES = [
     ((2, 2), (8, 8), 1, 3, 4, (6, 6), (0, 0), torch.float32, (2, 2), (1, 1)),      # strided and drifting
     ((2, 2), (16, 32), 1, 32, 32, (3, 3), (0, 0), torch.bfloat16),                 # MFMA path, fused fold, framed forward
     ((2, 1, 2), (4, 6, 8), 1, 2, 3, (3, 3, 5), (0, 1, 1), torch.float32),
+    # grouped layers (eleventh entry: groups) through the distributed functions
+    ((2, 2), (8, 12), 2, 6, 9, (3, 3), (1, 1), torch.float32, (1, 1), (1, 1), 3),
+    ((2, 2), (16, 32), 1, 32, 32, (3, 3), (1, 1), torch.bfloat16, (1, 1), (1, 1), 32),
 ]
 
 
-@pytest.mark.parametrize("case", DIST_CASES, ids=lambda c: f"mesh{'x'.join(map(str, c[0]))}_{c[3]}to{c[4]}_{str(c[7]).split('.')[-1]}" + (f"_s{''.join(map(str, c[8]))}_d{''.join(map(str, c[9]))}" if len(c) > 8 else ""))
+@pytest.mark.parametrize("case", DIST_CASES, ids=lambda c: f"mesh{'x'.join(map(str, c[0]))}_{c[3]}to{c[4]}_{str(c[7]).split('.')[-1]}" + (f"_s{''.join(map(str, c[8]))}_d{''.join(map(str, c[9]))}" if len(c) > 8 else "") + (f"_g{c[10]}" if len(c) > 10 else ""))
 def test_distributed_conv_matches_global_conv(case, dev):
     """The reference's parity method: every rank's y / dx and the summed dw / db equal
     the serial conv on the gathered tensor (test_conv2d_multi_spatial.py:73-233)."""
@@ -262,16 +265,17 @@ def _run_mesh_case(case, dev, framed, autocast):
     mesh, n, N, cin, cout, k, p, dtype = case[:8]
     ns = len(mesh)
     s, d = (case[8], case[9]) if len(case) > 8 else ((1,) * ns, (1,) * ns)
+    conv_groups = case[10] if len(case) > 10 else 1
     torch.manual_seed(0)
     gshape = tuple(a * b for a, b in zip(n, mesh))
     X = torch.randn(N, cin, *gshape).to(dtype)
-    fan_in = cin * int(torch.tensor(k).prod())
-    W = ((torch.rand(cout, cin, *k) * 2 - 1) / fan_in**0.5).to(dtype)
+    fan_in = cin // conv_groups * int(torch.tensor(k).prod())
+    W = ((torch.rand(cout, cin // conv_groups, *k) * 2 - 1) / fan_in**0.5).to(dtype)
     B = (torch.randn(cout) * 0.1).to(dtype)
     Xd = X.double().requires_grad_()
     Wd = W.double().requires_grad_()
     Bd = B.double().requires_grad_()
-    Y = oc.forward(Xd, Wd, Bd, s, p, d)
+    Y = oc.forward(Xd, Wd, Bd, s, p, d, conv_groups)
     G = torch.randn_like(Y).to(dtype)
     Y.backward(G.double())
 
@@ -289,7 +293,7 @@ def _run_mesh_case(case, dev, framed, autocast):
     # pass 1: forward of every rank, and the padded dgrad every rank will send from
     cfgs, outs, leaves, gx_need = {}, {}, {}, {}
     for c in mesh_coords(mesh):
-        cfgs[c] = jc.HipConvNdConfig.for_rank(ns, Bg, TableExchange(fwd_tabs[c], None), framed=framed)
+        cfgs[c] = jc.HipConvNdConfig.for_rank(ns, Bg, TableExchange(fwd_tabs[c], None), groups=conv_groups, framed=framed)
         groups = tuple(jc.TileGroup(mesh[a], c[a]) for a in range(ns))
         xl = tiles[c].clone().requires_grad_()
         wl, bl = Wg.clone().requires_grad_(), Bg.clone().requires_grad_()
@@ -299,7 +303,7 @@ def _run_mesh_case(case, dev, framed, autocast):
         assert not x_aug.requires_grad
         assert y.dtype == (autocast or dtype) and x_aug.dtype == (autocast or dtype)
         lp = oh.local_padding(p, mesh)
-        gx_need[c] = jc.conv_nd_input(x_aug.shape, Wg, gtiles[c], stride=s, padding=lp, dilation=d)
+        gx_need[c] = jc.conv_nd_input(x_aug.shape, Wg, gtiles[c], stride=s, padding=lp, dilation=d, groups=conv_groups)
     bwd_tabs = _recv_tables(gx_need, geoms, mesh, from_padded=True)
 
     # pass 2: backward of every rank
