@@ -19,6 +19,7 @@ that talks to other ranks), and assembles the padded tile in one pass.
 from __future__ import annotations
 
 import ctypes
+import itertools
 import math
 from collections.abc import Sequence
 from typing import Any, Protocol
@@ -188,11 +189,13 @@ def _embed_weight(w: torch.Tensor, off) -> torch.Tensor:
 def _dense_stride_ok(kernel, stride, dilation, padding=None) -> bool:
     if len(kernel) not in (2, 3) or all(s == 1 for s in stride):
         return False
-    if any(k not in (1, 3) for k in kernel):
+    if all(k == s for k, s in zip(kernel, stride)):  # kernel = stride has its own route
         return False
+    if any(k not in (1, 3) for k in kernel):
+        return _big_kernel_ok(kernel, (1,) * len(kernel), dilation)
     if any(d != 1 for d in dilation) and (padding is None or not _dilated_ok(kernel, (1,) * len(kernel), padding, dilation)):
         return False
-    return not all(k == s for k, s in zip(kernel, stride))  # kernel = stride has its own route
+    return True
 
 
 # --------------------------------------------------------------------------- #
@@ -248,6 +251,74 @@ def _from_phases(tb: torch.Tensor, phases, batch, sizes) -> torch.Tensor:
     return t[(slice(None), slice(None)) + tuple(slice(0, v) for v in sizes)].contiguous()
 
 
+# --------------------------------------------------------------------------- #
+# Kernels with more than three taps on an axis (5 x 5, 7 x 7, 4 x 4 at stride 1 ...): the taps of an
+# axis, filled up in front with zeros to a multiple of three, are blocks of three, and tap 3 i + u
+# of block i reads what tap u reads of the input moved by 3 i cells. The moved copies of the input
+# (zero padding included) become channel blocks of ONE three-tap layer, which the MFMA kernels run
+# without padding: the same products, summed in the same fp32 accumulators, at prod(blocks) times
+# the input in memory. The input gradient is the forward of the output gradient under the
+# transposed, reversed kernel; the weight gradient is that of the three-tap layer, put back in order.
+# --------------------------------------------------------------------------- #
+_MAX_TAP_BLOCKS = 9
+
+
+def _tap_blocks(kernel) -> tuple:
+    """Per axis ``(blocks of three taps, zero taps in front)``."""
+    return tuple(((k + 2) // 3, (k + 2) // 3 * 3 - k) for k in kernel)
+
+
+def _big_kernel_ok(kernel, stride, dilation) -> bool:
+    if len(kernel) not in (2, 3) or any(s != 1 for s in stride) or any(d != 1 for d in dilation):
+        return False
+    return any(k > 3 for k in kernel) and math.prod(b for b, _ in _tap_blocks(kernel)) <= _MAX_TAP_BLOCKS
+
+
+def _moved_copies(x: torch.Tensor, kernel, padding, out_sp) -> torch.Tensor:
+    """``(N, C, *spatial) -> (N, prod(blocks) * C, *(out + 2))``: block ``(i, j, ..)`` holds the zero-padded
+    input moved by ``(3 i, 3 j, ..)`` cells, cut to what a three-tap layer without padding needs."""
+    blocks = _tap_blocks(kernel)
+    pads = []
+    for (_, lead), p in reversed(list(zip(blocks, padding))):  # F.pad counts from the last axis
+        pads += [p + lead, p]
+    xp = torch.nn.functional.pad(x, pads)
+    parts = []
+    for idx in itertools.product(*(range(b) for b, _ in blocks)):
+        cut = tuple(slice(3 * i, 3 * i + o + 2) for i, o in zip(idx, out_sp))
+        parts.append(xp[(slice(None), slice(None)) + cut])
+    return torch.cat(parts, dim=1)
+
+
+def _tap_block_weight(w: torch.Tensor) -> torch.Tensor:
+    """``(M, C, *k) -> (M, prod(blocks) * C, 3, 3[, 3])``, channel blocks in the order of :func:`_moved_copies`."""
+    n = w.dim() - 2
+    blocks = _tap_blocks(w.shape[2:])
+    pads = []
+    for _, lead in reversed(blocks):
+        pads += [lead, 0]
+    w6 = torch.nn.functional.pad(w, pads)
+    shape = [w.shape[0], w.shape[1]]
+    for b, _ in blocks:
+        shape += [b, 3]
+    w6 = w6.reshape(shape)
+    b_dims = [2 + 2 * i for i in range(n)]
+    t_dims = [3 + 2 * i for i in range(n)]
+    return w6.permute(0, *b_dims, 1, *t_dims).reshape(w.shape[0], -1, *(3,) * n).contiguous()
+
+
+def _from_tap_blocks(gw3: torch.Tensor, weight_shape) -> torch.Tensor:
+    """Inverse of :func:`_tap_block_weight` for a gradient: back to ``weight_shape``, the zero taps dropped."""
+    n = len(weight_shape) - 2
+    blocks = _tap_blocks(weight_shape[2:])
+    m, c = weight_shape[0], weight_shape[1]
+    g6 = gw3.reshape(m, *(b for b, _ in blocks), c, *(3,) * n)
+    perm = [0, n + 1]
+    for i in range(n):
+        perm += [1 + i, n + 2 + i]
+    g6 = g6.permute(perm).reshape(m, c, *(3 * b for b, _ in blocks))
+    return g6[(slice(None), slice(None)) + tuple(slice(lead, None) for _, lead in blocks)].contiguous()
+
+
 def _stuffed(g: torch.Tensor, dense_sp, stride) -> torch.Tensor:
     """``g`` with ``stride - 1`` zeros between its cells: the output gradient of the stride-1 layer."""
     up = torch.zeros((g.shape[0], g.shape[1], *dense_sp), dtype=g.dtype, device=g.device)
@@ -277,6 +348,9 @@ def conv_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1) -> torch
         ext_in = tuple(-(-int(i) // p) for i, p in zip(x.shape[2:], phases))
         yb = conv_nd(_to_phases(x, phases, ext_in), w, b, stride=1, padding=tuple(pp // p for pp, p in zip(padding, phases)))
         return _from_phases(yb, phases, x.shape[0], out_sp)
+    if plain and _big_kernel_ok(tuple(w.shape[2:]), stride, dilation):
+        out_sp = _out_spatial(x.shape[2:], w.shape[2:], stride, padding, dilation)
+        return conv_nd(_moved_copies(x, w.shape[2:], padding, out_sp), _tap_block_weight(w), b, stride=1, padding=0)
     off = _embed3(tuple(w.shape[2:]), stride, dilation) if plain else None
     if off is not None:
         return conv_nd(x, _embed_weight(w, off), b, stride=1, padding=tuple(p + o for p, o in zip(padding, off)))
@@ -324,6 +398,13 @@ def conv_nd_input(input_shape, w, g, *, stride=1, padding=0, dilation=1, groups=
         gxb = conv_nd_input((g.shape[0] * math.prod(phases), input_shape[1], *ext_in), w, _to_phases(g, phases, ext_out),
                             stride=1, padding=pad0)
         return _from_phases(gxb, phases, input_shape[0], input_shape[2:])
+    if plain and _big_kernel_ok(tuple(w.shape[2:]), stride, dilation) and all(p <= k - 1 for p, k in zip(padding, w.shape[2:])):
+        out_sp = _out_spatial(input_shape[2:], w.shape[2:], stride, padding, dilation)
+        if tuple(g.shape) != (input_shape[0], w.shape[0], *out_sp):
+            raise ValueError(f"grad_output shape {tuple(g.shape)} does not match the convolution of an input of shape {input_shape}")
+        # the forward of g under the transposed kernel with its taps reversed, padded by k - 1 - p
+        back = w.transpose(0, 1).flip(*range(2, 2 + n))
+        return conv_nd(g, back, None, stride=1, padding=tuple(k - 1 - p for p, k in zip(padding, w.shape[2:])))
     off = _embed3(tuple(w.shape[2:]), stride, dilation) if plain else None
     if off is not None:
         return conv_nd_input(input_shape, _embed_weight(w, off), g, stride=1,
@@ -507,6 +588,15 @@ def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, group
         # every residue image is one more batch entry of the undilated layer: the sum over the batch is the answer
         return conv_nd_weight(_to_phases(x, phases, ext_in), weight_shape, _to_phases(g, phases, ext_out), stride=1,
                               padding=pad0, with_bias_grad=with_bias_grad)
+    if plain and _big_kernel_ok(weight_shape[2:], stride, dilation):
+        out_sp = _out_spatial(x.shape[2:], weight_shape[2:], stride, padding, dilation)
+        if tuple(g.shape) != (x.shape[0], weight_shape[0], *out_sp) or x.shape[1] != weight_shape[1]:
+            raise ValueError(f"grad_output {tuple(g.shape)} / input {tuple(x.shape)} do not match weight {weight_shape}")
+        moved = _moved_copies(x, weight_shape[2:], padding, out_sp)
+        res = conv_nd_weight(moved, (weight_shape[0], moved.shape[1]) + (3,) * n, g, stride=1, padding=0,
+                             with_bias_grad=with_bias_grad)
+        gw = _from_tap_blocks(res[0] if with_bias_grad else res, weight_shape)
+        return (gw, res[1]) if with_bias_grad else gw
     off = _embed3(weight_shape[2:], stride, dilation) if plain else None
     if off is not None:
         # gradient of the 3 x 3 (x 3) kernel the weights sit in; its centre taps are the answer

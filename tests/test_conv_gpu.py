@@ -87,6 +87,14 @@ PRIM_CASES = [
     (1, 32, 32, (6, 19, 34), (3, 3, 3), (1, 1, 1), (1, 2, 2), (1, 2, 2)),
     (2, 16, 32, (33, 40), (3, 3), (2, 2), (2, 2), (2, 2)),   # strided and dilated
     (1, 4, 6, (17, 23), (3, 3), (1, 1), (1, 1), (2, 2)),     # padding not a multiple: the direct kernels
+    # more than three taps on an axis: tap blocks of three as channel blocks of a three-tap layer
+    (1, 16, 32, (20, 33), (5, 5), (1, 1), (2, 2), (1, 1)),
+    (2, 8, 8, (15, 18), (7, 7), (1, 1), (3, 3), (1, 1)),
+    (1, 8, 16, (12, 14), (4, 4), (2, 2), (1, 1), (1, 1)),
+    (1, 6, 4, (13, 16), (1, 5), (1, 1), (0, 0), (1, 1)),
+    (2, 4, 6, (11, 9), (5, 2), (1, 1), (4, 1), (1, 1)),
+    (1, 4, 6, (6, 9, 10), (5, 3, 3), (1, 1, 1), (2, 1, 1), (1, 1, 1)),
+    (1, 3, 5, (14, 14), (7, 7), (2, 2), (3, 3), (1, 1)),     # a 7 x 7 stem at stride 2
     # grouped layers (ninth entry: groups), depthwise among them: the direct kernels
     (2, 8, 12, (13, 17), (3, 3), (1, 1), (1, 1), (1, 1), 4),
     (1, 32, 32, (20, 22), (3, 3), (1, 1), (1, 1), (1, 1), 32),

@@ -168,3 +168,41 @@ def test_the_dilated_route_takes_only_what_it_covers():
     assert not jc._dilated_ok((3, 3), (1, 1), (1, 1), (1, 1))      # nothing dilated
     assert jc._dilated_ok((1, 3), (1, 1), (0, 4), (7, 2))          # a dilation on a one-tap axis means nothing
     assert jc._dense_stride_ok((3, 3), (2, 2), (2, 2), (2, 2)) and not jc._dense_stride_ok((3, 3), (2, 2), (2, 2), (1, 1))
+
+
+@pytest.mark.parametrize("insp,k,p", [
+    ((12, 13), (5, 5), (2, 2)), ((11, 14), (7, 4), (3, 0)), ((9, 10), (5, 3), (0, 1)), ((6, 9, 10), (5, 3, 4), (2, 1, 0)),
+    ((10, 10), (9, 9), (4, 4)), ((12, 12), (2, 5), (0, 2)),
+])
+def test_tap_blocks_are_channel_blocks_of_a_three_tap_layer(insp, k, p):
+    """The route of kernels with more than three taps, with torch's CPU operators in place of the
+    kernels: forward and weight gradient of the three-tap layer over the moved copies of the input,
+    input gradient as the forward of the output gradient under the transposed, reversed kernel."""
+    ns = len(k)
+    assert jc._big_kernel_ok(k, (1,) * ns, (1,) * ns)
+    conv = {2: F.conv2d, 3: F.conv3d}[ns]
+    torch.manual_seed(0)
+    x = torch.randn(2, 3, *insp, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(4, 3, *k, dtype=torch.float64, requires_grad=True)
+    y = conv(x, w, None, 1, p)
+    g = torch.randn_like(y)
+    y.backward(g)
+    moved = jc._moved_copies(x.detach(), k, p, tuple(y.shape[2:])).requires_grad_()
+    w3 = jc._tap_block_weight(w.detach()).requires_grad_()
+    y3 = conv(moved, w3, None, 1, 0)
+    assert y3.shape == y.shape and torch.allclose(y3, y.detach(), atol=1e-10)
+    y3.backward(g)
+    assert torch.allclose(jc._from_tap_blocks(w3.grad, w.shape), w.grad, atol=1e-9)
+    if all(pp <= kk - 1 for pp, kk in zip(p, k)):
+        back = w.detach().transpose(0, 1).flip(*range(2, 2 + ns))
+        gx = conv(g, back, None, 1, tuple(kk - 1 - pp for pp, kk in zip(p, k)))
+        assert gx.shape == x.shape and torch.allclose(gx, x.grad, atol=1e-9)
+
+
+def test_the_tap_block_route_takes_only_what_it_covers():
+    assert not jc._big_kernel_ok((3, 3), (1, 1), (1, 1))          # three taps: the kernels as they are
+    assert not jc._big_kernel_ok((5, 5), (2, 2), (1, 1))          # strided: through the stride-1 route first
+    assert jc._dense_stride_ok((5, 5), (2, 2), (1, 1), (2, 2)) and not jc._dense_stride_ok((4, 4), (4, 4), (1, 1), (0, 0))
+    assert not jc._big_kernel_ok((5, 5), (1, 1), (2, 1))          # dilated
+    assert not jc._big_kernel_ok((11, 11), (1, 1), (1, 1))        # 16 blocks: too many copies of the input
+    assert not jc._big_kernel_ok((5,), (1,), (1,))                # one axis: the direct kernels
