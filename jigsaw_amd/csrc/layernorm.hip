@@ -10,6 +10,7 @@
 #include "jg_common.h"
 
 #include <mutex>
+#include <type_traits>
 
 namespace {
 
@@ -31,7 +32,8 @@ template <>
 struct Elem<JG_BF16> {
   typedef uint16_t T;
   __device__ static __forceinline__ float up(uint16_t v) { return jg::bf16_to_f32(v); }
-  __device__ static __forceinline__ uint16_t down(float v) { return jg::f32_to_bf16(v); }
+  // the hardware's conversion: round to nearest even, as jg::f32_to_bf16 (any NaN becomes a quiet one)
+  __device__ static __forceinline__ uint16_t down(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }
 };
 template <>
 struct Elem<JG_F16> {
@@ -355,6 +357,17 @@ __device__ __forceinline__ float group_sum(float v, int G) {
   for (int o = G >> 1; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
   return v;
 }
+// N such sums at once: the N shuffles of a step do not wait for each other
+template <int N>
+__device__ __forceinline__ void group_sums(float (&v)[N], int G) {
+  for (int o = G >> 1; o > 0; o >>= 1) {
+    float t[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) t[i] = __shfl_xor(v[i], o, kWave);
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] += t[i];
+  }
+}
 
 // w (and b) of the columns a lane owns, as 16-byte loads
 template <int CH>
@@ -409,8 +422,11 @@ __global__ __launch_bounds__(kThreads) void ln_plain_fwd_kernel(
       for (int k = 0; k < CH; ++k)
 #pragma unroll
         for (int i = 0; i < kPlainVec; ++i) s += v[u][k][i];
-      m[u] = group_sum(s, G) * inv;
+      m[u] = s;
     }
+    group_sums<U>(m, G);
+#pragma unroll
+    for (int u = 0; u < U; ++u) m[u] *= inv;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       float q = 0.0f;
@@ -424,8 +440,11 @@ __global__ __launch_bounds__(kThreads) void ln_plain_fwd_kernel(
           }
         }
       }
-      rs[u] = rsqrtf(group_sum(q, G) * inv + eps);
+      rs[u] = q;
     }
+    group_sums<U>(rs, G);
+#pragma unroll
+    for (int u = 0; u < U; ++u) rs[u] = rsqrtf(rs[u] * inv + eps);
     // every lane of the wavefront took part in the shuffles above; only now do dead rows drop out
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -471,7 +490,7 @@ __global__ __launch_bounds__(kThreads) void ln_plain_bwd_kernel(
       agb[k][i] = 0.0f;
     }
   for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows; r0 += stride * U) {
-    float gv[U][CH][kPlainVec], xh[U][CH][kPlainVec], m[U], rs[U], s1[U], s2[U];
+    float gv[U][CH][kPlainVec], xh[U][CH][kPlainVec], m[U], rs[U], s1[U], s2[U], s12[2 * U];
     bool live[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -508,8 +527,14 @@ __global__ __launch_bounds__(kThreads) void ln_plain_bwd_kernel(
           agw[k][i] += gv[u][k][i] * xh[u][k][i];
           agb[k][i] += gv[u][k][i];
         }
-      s1[u] = group_sum(a1, G) * inv;
-      s2[u] = group_sum(a2, G) * inv;
+      s12[u] = a1;
+      s12[U + u] = a2;
+    }
+    group_sums<2 * U>(s12, G);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      s1[u] = s12[u] * inv;
+      s2[u] = s12[U + u] * inv;
     }
     if (gx == nullptr) continue;
 #pragma unroll
@@ -570,6 +595,296 @@ __global__ __launch_bounds__(kThreads) void ln_plain_bwd_kernel(
   }
 }
 
+// ------------------------------------------------- sharded, rows held in registers
+// The four row kernels of the sharded LayerNorm once more, for local widths that fit the register
+// layout of the unsharded kernels (a multiple of 8 columns, at most G * 8 * kPlainChunks): G lanes
+// share a row, 64 / G rows per wavefront, 16-byte accesses, U rows of a lane group in flight and
+// one pass over the memory. The arithmetic per element is that of the kernels above.
+template <int DT, int CH>
+__device__ __forceinline__ void load_params_of(float (&dst)[CH][kPlainVec], const typename Elem<DT>::T* src, int G,
+                                               int sl, int cols) {
+#pragma unroll
+  for (int k = 0; k < CH; ++k) {
+    const int c = (k * G + sl) * kPlainVec;
+    if (c < cols && src != nullptr) {
+      load8<DT>(src + c, dst[k]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < kPlainVec; ++i) dst[k][i] = 0.0f;
+    }
+  }
+}
+
+// 8 columns of a row from an address that is always inside the tensor (row and column clamped), zero
+// where the lane owns nothing: the loads of a wavefront leave back to back, under no branch.
+template <int DT>
+__device__ __forceinline__ void load8_or_zero(const typename Elem<DT>::T* base, long long r, long long rows, int c,
+                                              int cols, float out[kPlainVec]) {
+  const bool ok = r < rows && c < cols;
+  load8<DT>(base + (r < rows ? r : rows - 1) * cols + (c < cols ? c : 0), out);
+#pragma unroll
+  for (int i = 0; i < kPlainVec; ++i) out[i] = ok ? out[i] : 0.0f;
+}
+
+template <int DT, int CH, int U>
+__global__ __launch_bounds__(kThreads) void ln_partial_fwd_rows_kernel(
+    float* __restrict__ mean, float* __restrict__ var, const typename Elem<DT>::T* __restrict__ x,
+    long long rows, int cols, int G) {
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
+  const float inv = 1.0f / (float)cols;
+  const long long stride = (long long)gridDim.x * kWavesPerBlock * rpw;
+  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows; r0 += stride * U) {
+    float v[U][CH][kPlainVec], m[U], qs[U];
+    bool live[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const long long r = r0 + u * stride + sub;
+      live[u] = r < rows;
+#pragma unroll
+      for (int k = 0; k < CH; ++k) {
+        const int c = (k * G + sl) * kPlainVec;
+        load8_or_zero<DT>(x, r, rows, c, cols, v[u][k]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float s = 0.0f;
+#pragma unroll
+      for (int k = 0; k < CH; ++k)
+#pragma unroll
+        for (int i = 0; i < kPlainVec; ++i) s += v[u][k][i];
+      m[u] = s;
+    }
+    group_sums<U>(m, G);
+#pragma unroll
+    for (int u = 0; u < U; ++u) m[u] *= inv;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float q = 0.0f;
+#pragma unroll
+      for (int k = 0; k < CH; ++k) {
+        if ((k * G + sl) * kPlainVec < cols) {
+#pragma unroll
+          for (int i = 0; i < kPlainVec; ++i) {
+            const float d = v[u][k][i] - m[u];
+            q += d * d;
+          }
+        }
+      }
+      qs[u] = q;
+    }
+    group_sums<U>(qs, G);
+    // every lane of the wavefront took part in the shuffles; dead rows drop out only here
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (live[u] && sl == 0) {
+        const long long r = r0 + u * stride + sub;
+        mean[r] = m[u];
+        var[r] = qs[u] * inv;
+      }
+    }
+  }
+}
+
+template <int XDT, int ODT, int CH, int U>
+__global__ __launch_bounds__(kThreads) void ln_apply_rows_kernel(
+    typename Elem<ODT>::T* __restrict__ y, typename Elem<ODT>::T* __restrict__ x_hat,
+    float* __restrict__ std_out, const typename Elem<XDT>::T* __restrict__ x,
+    const float* __restrict__ mean, const float* __restrict__ var,
+    const typename Elem<ODT>::T* __restrict__ w, const typename Elem<ODT>::T* __restrict__ b,
+    long long rows, int cols, float eps, int G) {
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
+  const long long stride = (long long)gridDim.x * kWavesPerBlock * rpw;
+  float wv[CH][kPlainVec], bv[CH][kPlainVec];
+  load_params_of<ODT, CH>(wv, w, G, sl, cols);
+  load_params_of<ODT, CH>(bv, b, G, sl, cols);
+  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows; r0 += stride * U) {
+    float v[U][CH][kPlainVec], m[U], sd[U];
+    bool live[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const long long r = r0 + u * stride + sub;
+      live[u] = r < rows;
+      const long long rc = live[u] ? r : rows - 1;  // a dead row reads the last one's and stores nothing
+      m[u] = mean[rc];
+      sd[u] = var[rc];
+#pragma unroll
+      for (int k = 0; k < CH; ++k) {
+        const int c = (k * G + sl) * kPlainVec;
+        load8_or_zero<XDT>(x, r, rows, c, cols, v[u][k]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (!live[u]) continue;
+      const long long r = r0 + u * stride + sub;
+      const float s = sqrtf(sd[u] + eps);
+      if (sl == 0 && std_out != nullptr) std_out[r] = s;
+#pragma unroll
+      for (int k = 0; k < CH; ++k) {
+        const int c = (k * G + sl) * kPlainVec;
+        if (c < cols) {
+          float xh[kPlainVec], out[kPlainVec];
+#pragma unroll
+          for (int i = 0; i < kPlainVec; ++i) {
+            // x_hat in the output dtype before the affine map (see ln_apply_kernel)
+            xh[i] = Elem<ODT>::up(Elem<ODT>::down((v[u][k][i] - m[u]) / s));
+            out[i] = wv[k][i] * xh[i] + bv[k][i];
+          }
+          if (x_hat != nullptr) store8<ODT>(x_hat + r * cols + c, xh);
+          store8<ODT>(y + r * cols + c, out);
+        }
+      }
+    }
+  }
+}
+
+// The column partials leave the kernel as those of ln_partial_bwd_kernel do: part[blk][which][col].
+template <int DT, int CH, int U>
+__global__ __launch_bounds__(kThreads) void ln_partial_bwd_rows_kernel(
+    float* __restrict__ mean_gxn, float* __restrict__ dot, float* __restrict__ part,
+    const typename Elem<DT>::T* __restrict__ g, const typename Elem<DT>::T* __restrict__ x_hat,
+    const typename Elem<DT>::T* __restrict__ w, long long rows, int cols, int G, bool want_cols) {
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
+  const float inv = 1.0f / (float)cols;
+  const long long stride = (long long)gridDim.x * kWavesPerBlock * rpw;
+  float wv[CH][kPlainVec], agw[CH][kPlainVec], agb[CH][kPlainVec];
+  load_params_of<DT, CH>(wv, w, G, sl, cols);
+#pragma unroll
+  for (int k = 0; k < CH; ++k)
+#pragma unroll
+    for (int i = 0; i < kPlainVec; ++i) {
+      agw[k][i] = 0.0f;
+      agb[k][i] = 0.0f;
+    }
+  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows; r0 += stride * U) {
+    float gv[U][CH][kPlainVec], xh[U][CH][kPlainVec], s12[2 * U];
+    bool live[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const long long r = r0 + u * stride + sub;
+      live[u] = r < rows;
+#pragma unroll
+      for (int k = 0; k < CH; ++k) {
+        const int c = (k * G + sl) * kPlainVec;
+        load8_or_zero<DT>(g, r, rows, c, cols, gv[u][k]);
+        load8_or_zero<DT>(x_hat, r, rows, c, cols, xh[u][k]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float a1 = 0.0f, a2 = 0.0f;
+#pragma unroll
+      for (int k = 0; k < CH; ++k)
+#pragma unroll
+        for (int i = 0; i < kPlainVec; ++i) {
+          // g * w in the tensor dtype, as the reference materialises grad_x_norm
+          const float gxn = Elem<DT>::up(Elem<DT>::down(gv[u][k][i] * wv[k][i]));
+          a1 += gxn;
+          a2 += gxn * xh[u][k][i];
+          agw[k][i] += gv[u][k][i] * xh[u][k][i];
+          agb[k][i] += gv[u][k][i];
+        }
+      s12[u] = a1;
+      s12[U + u] = a2;
+    }
+    group_sums<2 * U>(s12, G);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (live[u] && sl == 0) {
+        const long long r = r0 + u * stride + sub;
+        mean_gxn[r] = s12[u] * inv;
+        dot[r] = s12[U + u];
+      }
+    }
+  }
+  if (!want_cols) return;
+  // the rows of a wavefront that share a column set: lanes sl, sl + G, ...
+#pragma unroll
+  for (int k = 0; k < CH; ++k)
+#pragma unroll
+    for (int i = 0; i < kPlainVec; ++i)
+      for (int o = G; o < kWave; o <<= 1) {
+        agw[k][i] += __shfl_xor(agw[k][i], o, kWave);
+        agb[k][i] += __shfl_xor(agb[k][i], o, kWave);
+      }
+  __shared__ float red[kWavesPerBlock][2][kPlainChunks * kWave * kPlainVec];
+  if (sub == 0) {
+#pragma unroll
+    for (int k = 0; k < CH; ++k)
+#pragma unroll
+      for (int i = 0; i < kPlainVec; ++i) {
+        red[wave][0][(k * G + sl) * kPlainVec + i] = agw[k][i];
+        red[wave][1][(k * G + sl) * kPlainVec + i] = agb[k][i];
+      }
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < cols; c += kThreads) {
+    float a = 0.0f, b2 = 0.0f;
+#pragma unroll
+    for (int wv2 = 0; wv2 < kWavesPerBlock; ++wv2) {
+      a += red[wv2][0][c];
+      b2 += red[wv2][1][c];
+    }
+    part[((long long)blockIdx.x * 2 + 0) * cols + c] = a;
+    part[((long long)blockIdx.x * 2 + 1) * cols + c] = b2;
+  }
+}
+
+template <int DT, int CH, int U>
+__global__ __launch_bounds__(kThreads) void ln_bwd_apply_rows_kernel(
+    typename Elem<DT>::T* __restrict__ gx, const typename Elem<DT>::T* __restrict__ g,
+    const typename Elem<DT>::T* __restrict__ x_hat, const typename Elem<DT>::T* __restrict__ w,
+    const float* __restrict__ mean_gxn, const float* __restrict__ dot, const float* __restrict__ stdv,
+    long long rows, int cols, float inv_n, int G) {
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
+  const long long stride = (long long)gridDim.x * kWavesPerBlock * rpw;
+  float wv[CH][kPlainVec];
+  load_params_of<DT, CH>(wv, w, G, sl, cols);
+  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows; r0 += stride * U) {
+    float gv[U][CH][kPlainVec], xh[U][CH][kPlainVec], m[U], dn[U], sd[U];
+    bool live[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const long long r = r0 + u * stride + sub;
+      live[u] = r < rows;
+      const long long rc = live[u] ? r : rows - 1;  // a dead row reads the last one's and stores nothing
+      m[u] = mean_gxn[rc];
+      dn[u] = dot[rc];
+      sd[u] = stdv[rc];
+#pragma unroll
+      for (int k = 0; k < CH; ++k) {
+        const int c = (k * G + sl) * kPlainVec;
+        load8_or_zero<DT>(g, r, rows, c, cols, gv[u][k]);
+        load8_or_zero<DT>(x_hat, r, rows, c, cols, xh[u][k]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (!live[u]) continue;
+      const long long r = r0 + u * stride + sub;
+      const float rs = 1.0f / sd[u], d = dn[u] * inv_n;
+#pragma unroll
+      for (int k = 0; k < CH; ++k) {
+        const int c = (k * G + sl) * kPlainVec;
+        if (c < cols) {
+          float out[kPlainVec];
+#pragma unroll
+          for (int i = 0; i < kPlainVec; ++i) {
+            const float gxn = Elem<DT>::up(Elem<DT>::down(gv[u][k][i] * wv[k][i]));
+            out[i] = rs * (gxn - m[u] - xh[u][k][i] * d);
+          }
+          store8<DT>(gx + r * cols + c, out);
+        }
+      }
+    }
+  }
+}
+
 // lanes per row: the power of two that covers cols / 8 columns-octets in the fewest chunks
 int plain_group(long long cols) {
   int G = 1;
@@ -581,14 +896,28 @@ int plain_chunks(long long cols) {
   return (int)((cols + (long long)G * kPlainVec - 1) / ((long long)G * kPlainVec));
 }
 bool plain_ok(long long cols) { return cols >= kPlainVec && cols % kPlainVec == 0 && plain_chunks(cols) <= kPlainChunks; }
-int plain_blocks(long long rows, long long cols) {
+int plain_blocks(long long rows, long long cols, int most = 1024) {
   const int rpw = kWave / plain_group(cols);
   long long b = (rows + (long long)kWavesPerBlock * rpw - 1) / ((long long)kWavesPerBlock * rpw);
-  if (b > 1024) b = 1024;
+  if (b > most) b = most;
   if (b < 1) b = 1;
   return (int)b;
 }
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// Chunks per lane and rows in flight of the rows-in-registers kernels, as compile-time constants:
+// f(chunks, rows_in_flight) with std::integral_constant arguments. U1 = rows in flight where a lane
+// holds one chunk of a row (the kernels that only read keep more loads in the air).
+template <int U1, typename F>
+void with_row_shape(long long cols, F&& f) {
+  using std::integral_constant;
+  switch (plain_chunks(cols)) {
+    case 1: f(integral_constant<int, 1>(), integral_constant<int, U1>()); break;
+    case 2: f(integral_constant<int, 2>(), integral_constant<int, 2>()); break;
+    case 3: f(integral_constant<int, 3>(), integral_constant<int, 1>()); break;
+    default: f(integral_constant<int, 4>(), integral_constant<int, 1>()); break;
+  }
+}
 
 template <int XDT, int YDT>
 void launch_plain_fwd(void* y, float* mean, float* rstd, const void* x, const float* w, const float* b,
@@ -639,9 +968,17 @@ extern "C" int jg_ln_partial_fwd(float* mean, float* var, const void* x, int64_t
   if (rows == 0) return JG_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool v = vec_aligned(x, cols, x_dtype);
-#define JG_GO(DT)                                                          \
-  ln_partial_fwd_kernel<DT><<<row_grid(rows), kThreads, 0, s>>>(           \
-      mean, var, static_cast<const Elem<DT>::T*>(x), rows, cols, v)
+  const bool in_regs = plain_ok(cols) && aligned16(x);
+  const int G = in_regs ? plain_group(cols) : 0, blocks = in_regs ? plain_blocks(rows, cols, 2048) : 0;
+#define JG_GO(DT)                                                                                  \
+  if (in_regs)                                                                                     \
+    with_row_shape<4>(cols, [&](auto ch, auto u) {                                                 \
+      ln_partial_fwd_rows_kernel<DT, decltype(ch)::value, decltype(u)::value>                      \
+          <<<blocks, kThreads, 0, s>>>(mean, var, static_cast<const Elem<DT>::T*>(x), rows, (int)cols, G); \
+    });                                                                                            \
+  else                                                                                             \
+    ln_partial_fwd_kernel<DT><<<row_grid(rows), kThreads, 0, s>>>(                                 \
+        mean, var, static_cast<const Elem<DT>::T*>(x), rows, cols, v)
   if (x_dtype == JG_F32) JG_GO(JG_F32);
   else if (x_dtype == JG_BF16) JG_GO(JG_BF16);
   else JG_GO(JG_F16);
@@ -659,6 +996,15 @@ static void launch_apply(void* y, void* x_hat, float* std_out, const void* x, co
   const bool vx = vec_aligned(x, cols, XDT);
   const bool vo = vec_aligned(y, cols, ODT) && (x_hat == nullptr || vec_aligned(x_hat, cols, ODT));
   const bool vw = vec_aligned(w, cols, ODT) && (b == nullptr || vec_aligned(b, cols, ODT));
+  if (plain_ok(cols) && aligned16(x) && aligned16(y) && aligned16(x_hat) && aligned16(w) && aligned16(b)) {
+    const int G = plain_group(cols), blocks = plain_blocks(rows, cols);
+    with_row_shape<2>(cols, [&](auto ch, auto u) {
+      ln_apply_rows_kernel<XDT, ODT, decltype(ch)::value, decltype(u)::value><<<blocks, kThreads, 0, s>>>(
+          static_cast<OT*>(y), static_cast<OT*>(x_hat), std_out, static_cast<const XT*>(x), mean, var,
+          static_cast<const OT*>(w), static_cast<const OT*>(b), rows, (int)cols, eps, G);
+    });
+    return;
+  }
   ln_apply_kernel<XDT, ODT><<<row_grid(rows), kThreads, 0, s>>>(
       static_cast<OT*>(y), static_cast<OT*>(x_hat), std_out, static_cast<const XT*>(x), mean, var,
       static_cast<const OT*>(w), static_cast<const OT*>(b), rows, cols, eps, vx, vo, vw);
@@ -699,8 +1045,19 @@ extern "C" size_t jg_ln_bwd_workspace_bytes(int64_t rows, int64_t cols) {
 template <int DT>
 static int launch_partial_bwd(float* mean_gxn, float* dot, float* part, const void* g,
                               const void* x_hat, const void* w, int64_t rows, int64_t cols,
-                              bool want_cols, hipStream_t s) {
+                              bool want_cols, hipStream_t s, int* blocks_used) {
   typedef typename Elem<DT>::T T;
+  if (plain_ok(cols) && aligned16(g) && aligned16(x_hat) && aligned16(w)) {
+    const int G = plain_group(cols), blocks = plain_blocks(rows, cols);  // never more than bwd_blocks(rows)
+    *blocks_used = blocks;
+    with_row_shape<2>(cols, [&](auto ch, auto u) {
+      ln_partial_bwd_rows_kernel<DT, decltype(ch)::value, decltype(u)::value><<<blocks, kThreads, 0, s>>>(
+          mean_gxn, dot, part, static_cast<const T*>(g), static_cast<const T*>(x_hat), static_cast<const T*>(w),
+          rows, (int)cols, G, want_cols);
+    });
+    return JG_OK;
+  }
+  *blocks_used = bwd_blocks(rows);
   const bool v = vec_aligned(g, cols, DT) && vec_aligned(x_hat, cols, DT);
   const bool vw = vec_aligned(w, cols, DT);
   const int nb = bwd_blocks(rows);
@@ -738,17 +1095,17 @@ extern "C" int jg_ln_partial_bwd(float* mean_gxn, float* dot_gxn_xhat, float* gw
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   float* part = static_cast<float*>(workspace);
-  int rc;
+  int rc, nparts = 0;
   if (dtype == JG_F32)
-    rc = launch_partial_bwd<JG_F32>(mean_gxn, dot_gxn_xhat, part, g, x_hat, w, rows, cols, want_cols, s);
+    rc = launch_partial_bwd<JG_F32>(mean_gxn, dot_gxn_xhat, part, g, x_hat, w, rows, cols, want_cols, s, &nparts);
   else if (dtype == JG_BF16)
-    rc = launch_partial_bwd<JG_BF16>(mean_gxn, dot_gxn_xhat, part, g, x_hat, w, rows, cols, want_cols, s);
+    rc = launch_partial_bwd<JG_BF16>(mean_gxn, dot_gxn_xhat, part, g, x_hat, w, rows, cols, want_cols, s, &nparts);
   else
-    rc = launch_partial_bwd<JG_F16>(mean_gxn, dot_gxn_xhat, part, g, x_hat, w, rows, cols, want_cols, s);
+    rc = launch_partial_bwd<JG_F16>(mean_gxn, dot_gxn_xhat, part, g, x_hat, w, rows, cols, want_cols, s, &nparts);
   if (rc) return rc;
   JG_CHECK_LAUNCH("jg_ln_partial_bwd");
   if (want_cols) {
-    ln_colreduce_kernel<<<jg::cdiv(cols, 64), kReduceWaves * 64, 0, s>>>(gw, gb, part, bwd_blocks(rows), cols);
+    ln_colreduce_kernel<<<jg::cdiv(cols, 64), kReduceWaves * 64, 0, s>>>(gw, gb, part, nparts, cols);
     JG_CHECK_LAUNCH("jg_ln_partial_bwd(colreduce)");
   }
   return JG_OK;
@@ -827,6 +1184,15 @@ extern "C" int jg_ln_bwd_apply(void* gx, const void* g, const void* x_hat, const
     const bool v = vec_aligned(g, cols, DT) && vec_aligned(x_hat, cols, DT) &&             \
                    vec_aligned(gx, cols, DT);                                              \
     const bool vw = vec_aligned(w, cols, DT);                                              \
+    if (plain_ok(cols) && aligned16(gx) && aligned16(g) && aligned16(x_hat) && aligned16(w)) { \
+      const int G = plain_group(cols), blocks = plain_blocks(rows, cols);                  \
+      with_row_shape<2>(cols, [&](auto ch, auto u) {                                       \
+        ln_bwd_apply_rows_kernel<DT, decltype(ch)::value, decltype(u)::value>              \
+            <<<blocks, kThreads, 0, s>>>(static_cast<T*>(gx), static_cast<const T*>(g),    \
+                                         static_cast<const T*>(x_hat), static_cast<const T*>(w), \
+                                         mean_gxn, dot_gxn_xhat, std, rows, (int)cols, inv_n, G); \
+      });                                                                                  \
+    } else                                                                                 \
     ln_bwd_apply_kernel<DT><<<row_grid(rows), kThreads, 0, s>>>(                           \
         static_cast<T*>(gx), static_cast<const T*>(g), static_cast<const T*>(x_hat),       \
         static_cast<const T*>(w), mean_gxn, dot_gxn_xhat, std, rows, cols, inv_n, v, vw);  \

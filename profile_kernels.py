@@ -11,6 +11,9 @@ step: the attention core at head size 128 (32 heads, 4096 x 4096 tokens) and the
 projections with the head split fused in (8 x 4096 tokens, 512 channels, 8 heads). With
 ``swin-block`` it runs forward + backward of one Swin block on a 256 x 256 token tile (dim 128,
 4 heads, 8 x 8 windows, shift 4, bf16 autocast; the neighbours' roll slabs are random stand-ins made once).
+With ``sharded-layernorm`` it runs forward + backward of the channel-sharded LayerNorm on one shard's
+rows, bf16, at configuration 4's local width and at a row count that fills the chip (2 ** 18 rows of
+256 channels), then at 2 ** 20 rows of 64 channels and, for the kernels that walk a row, of 132.
 """
 
 from __future__ import annotations
@@ -124,12 +127,31 @@ def swin_block(reps: int = 5) -> None:
     print("profile_kernels: done", file=sys.stderr)
 
 
+def sharded_layernorm(reps: int = 3) -> None:
+    from jigsaw_amd import layernorm as jl
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(3)
+    for rows, cols in ((1 << 18, 256), (1 << 20, 64), (1 << 18, 132)):
+        x = torch.randn(rows, cols, device=dev, generator=g).bfloat16().requires_grad_()
+        w = torch.ones(cols, device=dev, dtype=torch.bfloat16, requires_grad=True)
+        b = torch.zeros(cols, device=dev, dtype=torch.bfloat16, requires_grad=True)
+        gout = torch.randn(rows, cols, device=dev, generator=g).bfloat16()
+        for _ in range(reps):
+            x.grad = w.grad = b.grad = None
+            jl.layer_norm(x, w, b, None).backward(gout)
+        torch.cuda.synchronize()
+    print("profile_kernels: done", file=sys.stderr)
+
+
 if __name__ == "__main__":
     if sys.argv[1:] == ["around-attention"]:
         around_attention()
+    elif sys.argv[1:] == ["sharded-layernorm"]:
+        sharded_layernorm()
     elif sys.argv[1:] == ["swin-block"]:
         swin_block()
     elif sys.argv[1:]:
-        raise SystemExit(f"unknown argument {sys.argv[1:]}; known: 'around-attention', 'swin-block'")
+        raise SystemExit(f"unknown argument {sys.argv[1:]}; known: 'around-attention', 'swin-block', 'sharded-layernorm'")
     else:
         main()

@@ -92,6 +92,54 @@ def test_layernorm_forward_backward_fp32(G, bias, dev):
             assert grp.calls == ["avg", "avg", "avg", "sum"]
 
 
+WIDTH_CASES = [
+    # local width, leading shape, dtype: widths that are a multiple of 8 up to 2048 run on the kernels that
+    # hold rows in registers (1 to 4 chunks a lane, several rows a wavefront when narrow), the rest on
+    # the kernels that walk a row
+    (8, (3, 5), torch.float32), (24, (67,), torch.float32), (24, (67,), torch.bfloat16), (128, (1,), torch.float32),
+    (136, (2, 77), torch.float16), (512, (130,), torch.bfloat16), (1000, (41,), torch.float32),
+    (1536, (9,), torch.bfloat16), (2048, (2, 3), torch.float32), (2048, (35,), torch.bfloat16),
+    (130, (19,), torch.float32), (1996, (5,), torch.bfloat16), (4, (33,), torch.float32),
+]
+
+
+@pytest.mark.parametrize("cols,lead,dtype", WIDTH_CASES, ids=lambda v: str(v).replace("torch.", ""))
+def test_layernorm_two_shards_over_widths(cols, lead, dtype, dev):
+    """Forward and backward of one of two channel shards, over the local widths that pick the
+    different row kernels, against the oracle in fp64."""
+    torch.manual_seed(cols)
+    G, eps = 2, 1e-5
+    C = cols * G
+    x = (torch.randn(*lead, C) * 2 + 0.5).to(dtype)
+    w = (1 + 0.2 * torch.randn(C)).to(dtype)
+    b = (0.2 * torch.randn(C)).to(dtype)
+    g = torch.randn(*lead, C).to(dtype)
+    xs, ws, bs, gs = (list(t.chunk(G, -1)) for t in (x, w, b, g))
+    ys, xns, std = ol.forward([t.double() for t in xs], [t.double() for t in ws], [t.double() for t in bs], eps)
+    gxs, gws, gbs = ol.backward([t.double() for t in gs], xns, [t.double() for t in ws], std, has_bias=True)
+    lm = [ol.partial_stats(t.double()) for t in xs]
+    mean = torch.stack([m for m, _ in lm]).mean(0)
+    gxn = [gs[i].double() * ws[i].double() for i in range(G)]
+    r, o = 1, 0
+    grp = ShardGroup(G, [[lm[o][0]], [lm[o][1] + (lm[o][0] - mean) ** 2],
+                         [gxn[o].mean(-1, keepdim=True)], [(gxn[o] * xns[o]).sum(-1, keepdim=True)]])
+    xr, wr, br = (t.to(dev).requires_grad_() for t in (xs[r], ws[r], bs[r]))
+    y, x_norm, _, var_eps = jl._LayerNorm.apply(xr, wr, br, grp, eps)
+    y.backward(gs[r].to(dev))
+    assert grp.calls == ["avg", "avg", "avg", "sum"]
+    # the statistics travel in the tensor dtype
+    tol = 1e-4 if dtype == torch.float32 else 1e-2
+    torch.testing.assert_close(var_eps.cpu().double(), std**2, atol=tol, rtol=tol)
+    if dtype == torch.float32:
+        for got, want, tol in ((y, ys[r], 1e-5), (x_norm, xns[r], 1e-5), (xr.grad, gxs[r], 2e-5)):
+            torch.testing.assert_close(got.cpu().double(), want, atol=tol, rtol=1e-5)
+        torch.testing.assert_close(wr.grad.cpu().double(), gws[r], atol=2e-4, rtol=1e-4)
+        torch.testing.assert_close(br.grad.cpu().double(), gbs[r], atol=2e-4, rtol=1e-4)
+    else:
+        for got, want in ((y, ys[r]), (x_norm, xns[r]), (xr.grad, gxs[r]), (wr.grad, gws[r]), (br.grad, gbs[r])):
+            assert got.dtype == dtype and rel_l2(got, want) < 2e-2
+
+
 def test_layernorm_under_autocast_returns_fp32_and_leaf_dtype_grad(dev):
     """LayerNorm under autocast computes in fp32 (reference: tests/test_autocast.py:265-292)."""
     torch.manual_seed(2)
