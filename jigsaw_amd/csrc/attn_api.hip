@@ -30,6 +30,9 @@ int attn_wide_fwd(void* out, float* lse, const void* q, const void* k, const voi
 int attn_wide_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q, const void* k,
                   const void* v, const void* out, const float* lse, long long batch, int sq, int sk,
                   int d, int dtype, float scale, void* ws, hipStream_t s);
+bool attn_f32_mfma_fwd_supported(long long batch, int sq, int sk, int d, int dtype, bool has_bias);
+int attn_f32_mfma_fwd(void* out, float* lse, const void* q, const void* k, const void* v, long long batch, int sq,
+                      int sk, int d, float scale, float* out_acc, float* lse_acc, hipStream_t s);
 bool attn_window_supported(long long batch, int sq, int sk, int d, int dtype);
 int attn_window_fwd(void* out, float* lse, const void* q, const void* k, const void* v,
                     long long batch, float scale, const float* bias, long long bias_period,
@@ -84,12 +87,15 @@ extern "C" int jg_attn_fwd(void* out, float* lse, const void* q, const void* k, 
   if (out_acc == nullptr && jg::attn_window_supported(batch, (int)sq, (int)sk, (int)d, dtype) &&
       aligned16({out, q, k, v, bias}))
     return jg::attn_window_fwd(out, lse, q, k, v, batch, scale, bias, bias_period, s);
+  if (jg::attn_f32_mfma_fwd_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr) &&
+      aligned16({out, q, k, v, out_acc}))
+    return jg::attn_f32_mfma_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, (int)d, scale, out_acc, lse_acc, s);
   if (!jg::attn_generic_supported((int)d))
     JG_FAIL(JG_ERR_UNSUPPORTED, "%s: head size %lld not in {8, 16, 32, 64, 96, 128}", who, (long long)d);
   if (out_acc != nullptr)
     JG_FAIL(JG_ERR_UNSUPPORTED,
             "%s: the fused merge needs an MFMA path (bf16 with d in {64, 96, 128} or fp16 with d in {96, 128},"
-            " sq %% 128 == 0, sk %% 128 == 0);"
+            " sq %% 128 == 0, sk %% 128 == 0; fp32 with d in {32, 64, 128}, no bias);"
             " call jg_lse_merge after the core instead", who);
   rc = jg::attn_generic_fwd(out, lse, q, k, v, batch, (int)sq, (int)sk, (int)d, scale, bias,
                             bias_period, dtype, s);
