@@ -125,10 +125,16 @@ def _width(d: int, dtype: torch.dtype) -> int:
 _KERNEL_HEAD_SIZES = (8, 16, 32, 64, 96, 128)
 
 
-def _kernel_head_size(d: int) -> int:
-    """Smallest head size the one-thread-per-row kernels are built for that holds ``d`` columns (zero
-    columns change neither scores nor the other outputs); ``d`` itself beyond the largest."""
-    return next((n for n in _KERNEL_HEAD_SIZES if n >= d), d)
+_F32_MFMA_HEAD_SIZES = (32, 64, 128)
+
+
+def _kernel_head_size(d: int, dtype=None, has_bias: bool = False) -> int:
+    """Smallest head size the kernels are built for that holds ``d`` columns (zero columns change
+    neither scores nor the other outputs); ``d`` itself beyond the largest. fp32 without a bias
+    goes to the sizes of its matrix-core kernels, everything else to those of the
+    one-thread-per-row kernels."""
+    sizes = _F32_MFMA_HEAD_SIZES if dtype == torch.float32 and not has_bias else _KERNEL_HEAD_SIZES
+    return next((n for n in sizes if n >= d), d)
 
 
 def _shapeable(q, k, bias) -> bool:
@@ -211,7 +217,7 @@ def core_forward(q, k, v, scale, bias=None, out_acc=None, lse_acc=None, want_out
     _check_qkv(q, k, v)
     if out_acc is None and lse_acc is None and want_out and _shapeable(q, k, bias):
         return _shaped_forward(q, k, v, scale)
-    d, dp = q.shape[-1], _kernel_head_size(q.shape[-1])
+    d, dp = q.shape[-1], _kernel_head_size(q.shape[-1], q.dtype, bias is not None)
     if dp != d and out_acc is None and lse_acc is None:
         out, lse = _core_forward(_pad_last(q, dp), _pad_last(k, dp), _pad_last(v, dp), scale, bias, None, None, want_out)
         return (out[..., :d].contiguous() if want_out else None), lse
@@ -252,7 +258,7 @@ def core_backward(grad_out, q, k, v, out, logsumexp, scale, bias=None, want_dbia
     _lib.require_gpu(grad_out, out, logsumexp)
     if not want_dbias and _shapeable(q, k, bias):
         return _shaped_backward(grad_out.to(q.dtype), q, k, v, out.to(q.dtype), logsumexp.to(torch.float32), scale)
-    d, dp = q.shape[-1], _kernel_head_size(q.shape[-1])
+    d, dp = q.shape[-1], _kernel_head_size(q.shape[-1], q.dtype, bias is not None)
     if dp != d:
         res = _core_backward(_pad_last(grad_out, dp), _pad_last(q, dp), _pad_last(k, dp), _pad_last(v, dp),
                              _pad_last(out, dp), logsumexp, scale, bias, want_dbias)

@@ -33,6 +33,10 @@ int attn_wide_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q,
 bool attn_f32_mfma_fwd_supported(long long batch, int sq, int sk, int d, int dtype, bool has_bias);
 int attn_f32_mfma_fwd(void* out, float* lse, const void* q, const void* k, const void* v, long long batch, int sq,
                       int sk, int d, float scale, float* out_acc, float* lse_acc, hipStream_t s);
+bool attn_f32_mfma_bwd_supported(long long batch, int sq, int sk, int d, int dtype, bool has_bias);
+int attn_f32_mfma_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q, const void* k, const void* v,
+                      const void* out, const float* lse, long long batch, int sq, int sk, int d, float scale,
+                      void* workspace, hipStream_t s);
 bool attn_window_supported(long long batch, int sq, int sk, int d, int dtype);
 int attn_window_fwd(void* out, float* lse, const void* q, const void* k, const void* v,
                     long long batch, float scale, const float* bias, long long bias_period,
@@ -139,6 +143,10 @@ extern "C" int jg_attn_bwd(void* dq, void* dk, void* dv, const void* dout, const
       aligned16({dq, dk, dv, dout, q, k, v, out, bias, dbias}))
     return jg::attn_window_bwd(dq, dk, dv, dbias, dout, q, k, v, out, lse, batch, scale, bias,
                                bias_period, s);
+  if (dbias == nullptr && jg::attn_f32_mfma_bwd_supported(batch, (int)sq, (int)sk, (int)d, dtype, bias != nullptr) &&
+      aligned16({dq, dk, dv, dout, q, k, v, out}))
+    return jg::attn_f32_mfma_bwd(dq, dk, dv, dout, q, k, v, out, lse, batch, (int)sq, (int)sk, (int)d, scale,
+                                 workspace, s);
   if (!jg::attn_generic_supported((int)d))
     JG_FAIL(JG_ERR_UNSUPPORTED, "%s: head size %lld not in {8, 16, 32, 64, 96, 128}", who, (long long)d);
   return jg::attn_generic_bwd(dq, dk, dv, static_cast<float*>(workspace), dbias, dout, q, k, v, out,

@@ -133,6 +133,50 @@ def test_fused_step_equals_core_plus_merge(d, dev):
     torch.testing.assert_close(l1, l2, atol=1e-6, rtol=1e-6)
 
 
+@pytest.mark.parametrize("d,sq,sk", [(32, 200, 300), (64, 130, 33), (128, 257, 96), (64, 128, 4096)])
+def test_fp32_matrix_core_step_with_merge(d, sq, sk, dev):
+    """fp32 on the matrix cores, ragged lengths: the step against the oracle in fp64, the fused merge
+    against the separate merge kernel and against the merge done in fp64, and a second merge on top."""
+    q, k, v = _qkv(2, 3, sq, sk, d, torch.float32, seed=3)
+    scale = d**-0.5
+    want_o, want_l = oa.core_forward(q.double(), k.double(), v.double(), scale)
+    q, k, v = q.to(dev), k.to(dev), v.to(dev)
+    out_j, l_j = ja.core_forward(q, k, v, scale)
+    assert rel_l2(out_j, want_o) < 1e-5 and rel_l2(l_j, want_l) < 1e-5
+    acc1 = torch.randn(2, 3, sq, d, device=dev)
+    l1 = torch.randn(2, 3, sq, device=dev)
+    acc0, l0 = acc1.double().cpu(), l1.double().cpu()
+    acc2, l2 = acc1.clone(), l1.clone()
+    assert ja.core_forward(q, k, v, scale, out_acc=acc1, lse_acc=l1, want_out=False) == (None, None)
+    acc2, l2 = ja.fused_online_softmax_merge_(acc2, l2, out_j, l_j, "bhsd")
+    torch.testing.assert_close(acc1, acc2, atol=2e-6, rtol=2e-6)
+    torch.testing.assert_close(l1, l2, atol=2e-6, rtol=2e-6)
+    l_new = torch.logaddexp(l0, want_l)
+    acc_new = acc0 * (l0 - l_new).exp().unsqueeze(-1) + want_o * (want_l - l_new).exp().unsqueeze(-1)
+    assert rel_l2(acc1, acc_new) < 1e-5 and rel_l2(l1, l_new) < 1e-5
+    # a fresh accumulator (lse -inf) takes the step as it is, and hands it out on request
+    acc3 = torch.zeros_like(acc1)
+    l3 = torch.full_like(l1, float("-inf"))
+    out3, lse3 = ja.core_forward(q, k, v, scale, out_acc=acc3, lse_acc=l3)
+    assert torch.equal(out3, out_j) and torch.equal(lse3, l_j)
+    torch.testing.assert_close(acc3, out_j, atol=1e-7, rtol=1e-6)
+    torch.testing.assert_close(l3, l_j, atol=1e-6, rtol=1e-6)
+
+
+@pytest.mark.parametrize("d", [8, 16, 96])
+def test_fp32_head_sizes_between_the_matrix_core_sizes(d, dev):
+    q, k, v = _qkv(1, 2, 70, 45, d, torch.float32, seed=4)
+    scale = d**-0.5
+    want_o, want_l = oa.core_forward(q.double(), k.double(), v.double(), scale)
+    dout = torch.randn(1, 2, 70, d)
+    wdq, wdk, wdv = oa.core_backward(dout.double(), q.double(), k.double(), v.double(), want_o, want_l, scale)
+    out, lse = ja.core_forward(q.to(dev), k.to(dev), v.to(dev), scale)
+    assert out.shape == q.shape and rel_l2(out, want_o) < 1e-5 and rel_l2(lse, want_l) < 1e-5
+    dq, dk, dv = ja.core_backward(dout.to(dev), q.to(dev), k.to(dev), v.to(dev), want_o.float().to(dev), want_l.float().to(dev), scale)
+    for got, want in ((dq, wdq), (dk, wdk), (dv, wdv)):
+        assert got.shape == want.shape and rel_l2(got, want) < 1e-5
+
+
 @pytest.mark.parametrize("pattern", ["late_spike", "rising", "first_tile_low", "huge_logits", "one_hot_rows"])
 def test_mfma_forward_when_the_running_max_moves(pattern, dev):
     """The head-size-64 kernel keeps a per-query reference exponent that follows the running
