@@ -31,6 +31,7 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
+PEAK_FP32_TFLOPS = 157.3  # MI355X dense fp32 MFMA (and vector FMA)
 
 METRIC = "halo-conv fwd+bwd & ring-attn step TFLOP/s on 1 GPU; % MFMA peak; halo GB/s"
 
@@ -197,6 +198,16 @@ def attention_figures(dev, iters: int) -> dict:
     hop_bwd["ms_no_hop"] = time_gpu(lambda: ja.ring_backward(dout, q, out, l, ks, vs, scale), iters)
     x = torch.randn(b, n, 256, device=dev, generator=g).bfloat16()
     ms_ln = time_gpu(lambda: jl.partial_stats(x), iters)
+    # the same statistics on a shard that fills the chip (2 ** 18 rows of the same local width)
+    xl = torch.randn(1 << 18, 256, device=dev, generator=g).bfloat16()
+    ms_ln_big = time_gpu(lambda: jl.partial_stats(xl), iters)
+    del xl
+    # the ring step on fp32 inputs: the fp32 matrix-core kernels (peak 157.3 TFLOP/s)
+    q32, k32, v32, do32 = q.float(), ks[0].float(), vs[0].float(), dout.float()
+    acc32, lse32 = torch.zeros(b, h, n, d, device=dev), torch.full((b, h, n), float("-inf"), device=dev)
+    ms_f32 = time_gpu(lambda: ja.core_forward(q32, k32, v32, scale, out_acc=acc32, lse_acc=lse32, want_out=False), iters)
+    o32, l32 = ja.core_forward(q32, k32, v32, scale)
+    ms_b32 = time_gpu(lambda: ja.core_backward(do32, q32, k32, v32, o32, l32, scale), iters)
     tf = lambda f, ms: f / (ms * 1e-3) / 1e12  # noqa: E731
     return {
         "attn_fwd_step": {"ms": ms_f, "tflops": tf(f_fwd, ms_f), "frac_mfma_peak": tf(f_fwd, ms_f) / PEAK_BF16_TFLOPS},
@@ -204,7 +215,11 @@ def attention_figures(dev, iters: int) -> dict:
         "attn_ring_fwd_4_steps": {"ms": ms_ring, "tflops": tf(4 * f_fwd, ms_ring)},
         "attn_ring_fwd_4_steps_with_hop": hop,
         "attn_ring_bwd_4_steps_with_hop_and_dkv_relay": hop_bwd,
+        "attn_fp32_fwd_step": {"ms": ms_f32, "tflops": tf(f_fwd, ms_f32), "frac_fp32_mfma_peak": tf(f_fwd, ms_f32) / PEAK_FP32_TFLOPS},
+        "attn_fp32_bwd_step": {"ms": ms_b32, "tflops": tf(f_bwd, ms_b32), "frac_fp32_mfma_peak": tf(f_bwd, ms_b32) / PEAK_FP32_TFLOPS},
         "ln_partial_stats": {"ms": ms_ln, "GBps": x.numel() * 2 / (ms_ln * 1e-3) / 1e9, "bytes": x.numel() * 2},
+        "ln_partial_stats_262144_rows": {"ms": ms_ln_big, "GBps": (1 << 18) * 256 * 2 / (ms_ln_big * 1e-3) / 1e9,
+                                         "bytes": (1 << 18) * 256 * 2, "frac_hbm_peak": (1 << 18) * 256 * 2 / (ms_ln_big * 1e-3) / 1e9 / PEAK_HBM_GBPS},
     }
 
 

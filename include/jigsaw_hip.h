@@ -494,7 +494,10 @@ int jg_bias_grad(void* gb, const void* g, int64_t batch, int64_t channels,
  *   w = sigmoid(lse - lse_acc); out_acc += w*(out - out_acc); lse_acc = logaddexp,
  * which is _online_softmax_merge_ (forward.py:23-61) without the round trip of
  * out_j through HBM; `out` / `lse` may then be NULL (bf16 with d = 64, 96 or 128, fp16
- * with d = 96 or 128, sq and sk multiples of 128 only; JG_ERR_UNSUPPORTED otherwise).
+ * with d = 96 or 128, sq and sk multiples of 128; fp32 with d = 32, 64 or 128, no bias,
+ * 16-byte aligned tensors, any sq and sk; JG_ERR_UNSUPPORTED otherwise).
+ * fp32 without a bias at d = 32, 64 or 128 runs on the fp32 matrix-core instructions
+ * (forward and backward), other fp32 calls on one-thread-per-row kernels.
  * d must be one of 8, 16, 32, 64, 96, 128 (JG_ERR_UNSUPPORTED otherwise; zero
  * columns appended to q, k, v leave out's other columns and lse unchanged). */
 int jg_attn_fwd(void* out, float* lse, const void* q, const void* k, const void* v,

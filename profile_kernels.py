@@ -14,6 +14,8 @@ projections with the head split fused in (8 x 4096 tokens, 512 channels, 8 heads
 With ``sharded-layernorm`` it runs forward + backward of the channel-sharded LayerNorm on one shard's
 rows, bf16, at configuration 4's local width and at a row count that fills the chip (2 ** 18 rows of
 256 channels), then at 2 ** 20 rows of 64 channels and, for the kernels that walk a row, of 132.
+With ``attention-fp32`` it runs the attention core forward + backward on fp32 inputs (8 heads,
+4096 x 4096 tokens) at head sizes 64, 128 and 32.
 """
 
 from __future__ import annotations
@@ -127,6 +129,22 @@ def swin_block(reps: int = 5) -> None:
     print("profile_kernels: done", file=sys.stderr)
 
 
+def attention_fp32(reps: int = 3) -> None:
+    from jigsaw_amd import attention as ja
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(4)
+    for d in (64, 128, 32):
+        b, h, n = 1, 8, 4096
+        q, k, v, dout = (torch.randn(b, h, n, d, device=dev, generator=g) / 8 for _ in range(4))
+        scale = d**-0.5
+        for _ in range(reps):
+            out, lse = ja.core_forward(q, k, v, scale)
+            ja.core_backward(dout, q, k, v, out, lse, scale)
+        torch.cuda.synchronize()
+    print("profile_kernels: done", file=sys.stderr)
+
+
 def sharded_layernorm(reps: int = 3) -> None:
     from jigsaw_amd import layernorm as jl
 
@@ -149,9 +167,11 @@ if __name__ == "__main__":
         around_attention()
     elif sys.argv[1:] == ["sharded-layernorm"]:
         sharded_layernorm()
+    elif sys.argv[1:] == ["attention-fp32"]:
+        attention_fp32()
     elif sys.argv[1:] == ["swin-block"]:
         swin_block()
     elif sys.argv[1:]:
-        raise SystemExit(f"unknown argument {sys.argv[1:]}; known: 'around-attention', 'swin-block', 'sharded-layernorm'")
+        raise SystemExit(f"unknown argument {sys.argv[1:]}; known: 'around-attention', 'swin-block', 'sharded-layernorm', 'attention-fp32'")
     else:
         main()
