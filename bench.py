@@ -202,6 +202,19 @@ def attention_figures(dev, iters: int) -> dict:
     xl = torch.randn(1 << 18, 256, device=dev, generator=g).bfloat16()
     ms_ln_big = time_gpu(lambda: jl.partial_stats(xl), iters)
     del xl
+    # the separate LSE merge (what a step runs when its core cannot fuse it): fp32 accumulator read and
+    # written, the step's bf16 output read; at the step's size and at 16 x the heads
+    merge = {}
+    for name, hh in (("lse_merge_step", h), ("lse_merge_128_heads", 16 * h)):
+        o1 = torch.randn(b, hh, n, d, device=dev, generator=g)
+        l1 = torch.randn(b, hh, n, device=dev, generator=g)
+        o2 = torch.randn(b, hh, n, d, device=dev, generator=g).bfloat16()
+        l2 = torch.randn(b, hh, n, device=dev, generator=g)
+        ms_m = time_gpu(lambda: ja.fused_online_softmax_merge_(o1, l1, o2, l2, "bhsd"), iters)
+        nbytes = o1.numel() * (4 + 4 + 2) + l1.numel() * 12
+        merge[name] = {"ms": ms_m, "GBps": nbytes / (ms_m * 1e-3) / 1e9, "bytes": nbytes,
+                       "frac_hbm_peak": nbytes / (ms_m * 1e-3) / 1e9 / PEAK_HBM_GBPS}
+        del o1, l1, o2, l2
     # the ring step on fp32 inputs: the fp32 matrix-core kernels (peak 157.3 TFLOP/s)
     q32, k32, v32, do32 = q.float(), ks[0].float(), vs[0].float(), dout.float()
     acc32, lse32 = torch.zeros(b, h, n, d, device=dev), torch.full((b, h, n), float("-inf"), device=dev)
@@ -217,6 +230,7 @@ def attention_figures(dev, iters: int) -> dict:
         "attn_ring_bwd_4_steps_with_hop_and_dkv_relay": hop_bwd,
         "attn_fp32_fwd_step": {"ms": ms_f32, "tflops": tf(f_fwd, ms_f32), "frac_fp32_mfma_peak": tf(f_fwd, ms_f32) / PEAK_FP32_TFLOPS},
         "attn_fp32_bwd_step": {"ms": ms_b32, "tflops": tf(f_bwd, ms_b32), "frac_fp32_mfma_peak": tf(f_bwd, ms_b32) / PEAK_FP32_TFLOPS},
+        **merge,
         "ln_partial_stats": {"ms": ms_ln, "GBps": x.numel() * 2 / (ms_ln * 1e-3) / 1e9, "bytes": x.numel() * 2},
         "ln_partial_stats_262144_rows": {"ms": ms_ln_big, "GBps": (1 << 18) * 256 * 2 / (ms_ln_big * 1e-3) / 1e9,
                                          "bytes": (1 << 18) * 256 * 2, "frac_hbm_peak": (1 << 18) * 256 * 2 / (ms_ln_big * 1e-3) / 1e9 / PEAK_HBM_GBPS},
