@@ -206,3 +206,16 @@ def test_the_tap_block_route_takes_only_what_it_covers():
     assert not jc._big_kernel_ok((5, 5), (1, 1), (2, 1))          # dilated
     assert not jc._big_kernel_ok((11, 11), (1, 1), (1, 1))        # 16 blocks: too many copies of the input
     assert not jc._big_kernel_ok((5,), (1,), (1,))                # one axis: the direct kernels
+
+
+def test_head_sizes_the_attention_host_pads_to():
+    """fp32 without a bias goes to the head sizes of its matrix-core kernels, everything else to those
+    of the one-thread-per-row kernels; a head size beyond the largest is passed on for the library to refuse."""
+    from jigsaw_amd import attention as ja
+
+    for d, want in ((1, 32), (8, 32), (32, 32), (33, 64), (64, 64), (72, 128), (96, 128), (128, 128), (129, 129)):
+        assert ja._kernel_head_size(d, torch.float32, False) == want
+    for d, want in ((1, 8), (8, 8), (9, 16), (33, 64), (72, 96), (96, 96), (100, 128), (129, 129)):
+        assert ja._kernel_head_size(d, torch.float32, True) == want
+        assert ja._kernel_head_size(d, torch.bfloat16, False) == want
+        assert ja._kernel_head_size(d) == want
