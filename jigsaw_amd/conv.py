@@ -319,6 +319,17 @@ def _from_tap_blocks(gw3: torch.Tensor, weight_shape) -> torch.Tensor:
     return g6[(slice(None), slice(None)) + tuple(slice(lead, None) for _, lead in blocks)].contiguous()
 
 
+# Grouped layers: a group is an ungrouped layer of its own on a slice of the channels. Where a group has
+# at least _GROUP_MIN channels on either side it runs as that layer (on the matrix cores where they
+# cover it, through the routes above otherwise), at the price of a contiguous copy of each slice;
+# narrower groups (depthwise layers) stay on the direct kernels, which walk a group per block.
+_GROUP_MIN = 8
+
+
+def _per_group_ok(groups: int, c_in_group: int, c_out_group: int, n_spatial: int) -> bool:
+    return groups > 1 and n_spatial >= 2 and c_in_group >= _GROUP_MIN and c_out_group >= _GROUP_MIN
+
+
 def _stuffed(g: torch.Tensor, dense_sp, stride) -> torch.Tensor:
     """``g`` with ``stride - 1`` zeros between its cells: the output gradient of the stride-1 layer."""
     up = torch.zeros((g.shape[0], g.shape[1], *dense_sp), dtype=g.dtype, device=g.device)
@@ -337,7 +348,13 @@ def conv_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1) -> torch
     if x.shape[1] != w.shape[1] * groups:
         raise RuntimeError(f"expected input to have {w.shape[1] * groups} channels, but got {x.shape[1]} channels instead")
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
-    plain = groups == 1  # the routes below re-shape ungrouped layers; grouped ones run the direct kernels as they are
+    if _per_group_ok(groups, w.shape[1], w.shape[0] // groups, n):
+        cg, mg = w.shape[1], w.shape[0] // groups
+        return torch.cat([
+            conv_nd(x[:, i * cg:(i + 1) * cg].contiguous(), w[i * mg:(i + 1) * mg], None if b is None else b[i * mg:(i + 1) * mg],
+                    stride=stride, padding=padding, dilation=dilation)
+            for i in range(groups)], dim=1)
+    plain = groups == 1  # the routes below re-shape ungrouped layers; narrow groups run the direct kernels as they are
     if plain and _dense_stride_ok(tuple(w.shape[2:]), stride, dilation, padding):
         out_sp = _out_spatial(x.shape[2:], w.shape[2:], stride, padding, dilation)
         dense = conv_nd(x, w, b, stride=1, padding=padding, dilation=dilation)
@@ -383,6 +400,14 @@ def conv_nd_input(input_shape, w, g, *, stride=1, padding=0, dilation=1, groups=
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
     if input_shape[1] != w.shape[1] * groups:
         raise ValueError(f"input_shape has {input_shape[1]} channels, the weight takes {w.shape[1] * groups}")
+    if _per_group_ok(groups, w.shape[1], w.shape[0] // groups, n):
+        cg, mg = w.shape[1], w.shape[0] // groups
+        if g.shape[1] != w.shape[0]:
+            raise ValueError(f"grad_output has {g.shape[1]} channels, the weight produces {w.shape[0]}")
+        return torch.cat([
+            conv_nd_input((input_shape[0], cg, *input_shape[2:]), w[i * mg:(i + 1) * mg], g[:, i * mg:(i + 1) * mg].contiguous(),
+                          stride=stride, padding=padding, dilation=dilation)
+            for i in range(groups)], dim=1)
     plain = groups == 1  # as in conv_nd
     if plain and _dense_stride_ok(tuple(w.shape[2:]), stride, dilation, padding):
         dense_sp = _out_spatial(input_shape[2:], w.shape[2:], (1,) * n, padding, dilation)
@@ -572,6 +597,16 @@ def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, group
     if x.dtype != g.dtype:
         raise RuntimeError(f"input type ({x.dtype}) and grad_output type ({g.dtype}) should be the same")
     stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
+    if _per_group_ok(groups, weight_shape[1], weight_shape[0] // groups, n):
+        cg, mg = weight_shape[1], weight_shape[0] // groups
+        if x.shape[1] != cg * groups or g.shape[1] != weight_shape[0]:
+            raise ValueError(f"{x.shape[1]} input and {g.shape[1]} output channels do not fit a weight of shape {weight_shape} in {groups} groups")
+        parts = [conv_nd_weight(x[:, i * cg:(i + 1) * cg].contiguous(), (mg, cg, *weight_shape[2:]), g[:, i * mg:(i + 1) * mg].contiguous(),
+                                stride=stride, padding=padding, dilation=dilation, with_bias_grad=with_bias_grad)
+                 for i in range(groups)]
+        if with_bias_grad:
+            return torch.cat([gw for gw, _ in parts], dim=0), torch.cat([gb for _, gb in parts], dim=0)
+        return torch.cat(parts, dim=0)
     plain = groups == 1  # as in conv_nd
     if plain and _dense_stride_ok(weight_shape[2:], stride, dilation, padding):
         dense_sp = _out_spatial(x.shape[2:], weight_shape[2:], (1,) * n, padding, dilation)

@@ -102,6 +102,10 @@ PRIM_CASES = [
     (1, 16, 16, (5, 9, 10), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 2),
     (2, 64, 64, (18, 34), (3, 3), (1, 1), (0, 0), (1, 1), 2),   # a shape the MFMA kernels would take ungrouped
     (1, 12, 8, (30,), (5,), (1,), (2,), (1,), 4),
+    # groups of at least 8 channels a side: each group as an ungrouped layer of its own (matrix cores, and the routes above)
+    (2, 48, 32, (20, 22), (3, 3), (2, 2), (1, 1), (1, 1), 2),
+    (1, 32, 64, (17, 19), (5, 5), (1, 1), (2, 2), (1, 1), 4),
+    (1, 24, 24, (6, 10, 12), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 2, 2), 3),
 ]
 
 
@@ -245,6 +249,7 @@ DIST_CASES = [
     # grouped layers (eleventh entry: groups) through the distributed functions
     ((2, 2), (8, 12), 2, 6, 9, (3, 3), (1, 1), torch.float32, (1, 1), (1, 1), 3),
     ((2, 2), (16, 32), 1, 32, 32, (3, 3), (1, 1), torch.bfloat16, (1, 1), (1, 1), 32),
+    ((2, 2), (16, 32), 2, 32, 48, (3, 3), (1, 1), torch.bfloat16, (1, 1), (1, 1), 2),   # 16 -> 24 channels a group: each group on the matrix cores
 ]
 
 
