@@ -191,10 +191,11 @@ def _dense_stride_ok(kernel, stride, dilation, padding=None) -> bool:
         return False
     if all(k == s for k, s in zip(kernel, stride)):  # kernel = stride has its own route
         return False
+    ones = (1,) * len(kernel)
+    if any(d != 1 for d in dilation):
+        return padding is not None and (_dilated_ok(kernel, ones, padding, dilation) or _prepad(kernel, ones, padding, dilation) is not None)
     if any(k not in (1, 3) for k in kernel):
-        return _big_kernel_ok(kernel, (1,) * len(kernel), dilation)
-    if any(d != 1 for d in dilation) and (padding is None or not _dilated_ok(kernel, (1,) * len(kernel), padding, dilation)):
-        return False
+        return _big_kernel_ok(kernel, ones, dilation)
     return True
 
 
@@ -209,15 +210,34 @@ def _dense_stride_ok(kernel, stride, dilation, padding=None) -> bool:
 def _dilated_ok(kernel, stride, padding, dilation) -> bool:
     if len(kernel) not in (2, 3) or any(s != 1 for s in stride):
         return False
-    if any(k not in (1, 3) for k in kernel):
+    ones = (1,) * len(kernel)
+    if any(k not in (1, 3) for k in kernel) and not _big_kernel_ok(kernel, ones, ones):
+        return False  # the undilated layer of a residue image must have a route of its own
+    if not any(d > 1 and k > 1 for k, d in zip(kernel, dilation)):
         return False
-    if not any(d > 1 and k == 3 for k, d in zip(kernel, dilation)):
-        return False
-    return all(p % d == 0 for k, p, d in zip(kernel, padding, dilation) if d > 1 and k == 3)
+    return all(p % d == 0 for k, p, d in zip(kernel, padding, dilation) if d > 1 and k > 1)
 
 
 def _phase_counts(kernel, dilation) -> tuple:
-    return tuple(int(d) if k == 3 else 1 for k, d in zip(kernel, dilation))
+    return tuple(int(d) if k > 1 else 1 for k, d in zip(kernel, dilation))
+
+
+def _prepad(kernel, stride, padding, dilation):
+    """A padding that is no multiple of the dilation: the cells to lay around the input as zeros (per
+    axis) so that what remains of the padding is one, or ``None`` where that opens no route."""
+    if len(kernel) not in (2, 3) or any(s != 1 for s in stride):
+        return None
+    extra = tuple(p % d if d > 1 and k > 1 else 0 for k, p, d in zip(kernel, padding, dilation))
+    if not any(extra):
+        return None
+    return extra if _dilated_ok(kernel, stride, tuple(p - e for p, e in zip(padding, extra)), dilation) else None
+
+
+def _zero_rim(x: torch.Tensor, extra) -> torch.Tensor:
+    pads = []
+    for e in reversed(extra):
+        pads += [e, e]
+    return torch.nn.functional.pad(x, pads)
 
 
 def _to_phases(t: torch.Tensor, phases, ext) -> torch.Tensor:
@@ -271,7 +291,8 @@ def _tap_blocks(kernel) -> tuple:
 def _big_kernel_ok(kernel, stride, dilation) -> bool:
     if len(kernel) not in (2, 3) or any(s != 1 for s in stride) or any(d != 1 for d in dilation):
         return False
-    return any(k > 3 for k in kernel) and math.prod(b for b, _ in _tap_blocks(kernel)) <= _MAX_TAP_BLOCKS
+    # two taps are one block with a zero tap in front
+    return any(k not in (1, 3) for k in kernel) and math.prod(b for b, _ in _tap_blocks(kernel)) <= _MAX_TAP_BLOCKS
 
 
 def _moved_copies(x: torch.Tensor, kernel, padding, out_sp) -> torch.Tensor:
@@ -359,6 +380,9 @@ def conv_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1) -> torch
         out_sp = _out_spatial(x.shape[2:], w.shape[2:], stride, padding, dilation)
         dense = conv_nd(x, w, b, stride=1, padding=padding, dilation=dilation)
         return dense[(slice(None), slice(None)) + tuple(slice(0, (o - 1) * s + 1, s) for o, s in zip(out_sp, stride))].contiguous()
+    extra = _prepad(tuple(w.shape[2:]), stride, padding, dilation) if plain else None
+    if extra is not None:
+        return conv_nd(_zero_rim(x, extra), w, b, stride=1, padding=tuple(p - e for p, e in zip(padding, extra)), dilation=dilation)
     if plain and _dilated_ok(tuple(w.shape[2:]), stride, padding, dilation):
         phases = _phase_counts(w.shape[2:], dilation)
         out_sp = _out_spatial(x.shape[2:], w.shape[2:], stride, padding, dilation)
@@ -412,6 +436,11 @@ def conv_nd_input(input_shape, w, g, *, stride=1, padding=0, dilation=1, groups=
     if plain and _dense_stride_ok(tuple(w.shape[2:]), stride, dilation, padding):
         dense_sp = _out_spatial(input_shape[2:], w.shape[2:], (1,) * n, padding, dilation)
         return conv_nd_input(input_shape, w, _stuffed(g, dense_sp, stride), stride=1, padding=padding, dilation=dilation)
+    extra = _prepad(tuple(w.shape[2:]), stride, padding, dilation) if plain else None
+    if extra is not None:
+        rimmed = input_shape[:2] + tuple(v + 2 * e for v, e in zip(input_shape[2:], extra))
+        gxr = conv_nd_input(rimmed, w, g, stride=1, padding=tuple(p - e for p, e in zip(padding, extra)), dilation=dilation)
+        return gxr[(slice(None), slice(None)) + tuple(slice(e, e + v) for v, e in zip(input_shape[2:], extra))].contiguous()
     if plain and _dilated_ok(tuple(w.shape[2:]), stride, padding, dilation):
         phases = _phase_counts(w.shape[2:], dilation)
         out_sp = _out_spatial(input_shape[2:], w.shape[2:], stride, padding, dilation)
@@ -612,6 +641,10 @@ def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, group
         dense_sp = _out_spatial(x.shape[2:], weight_shape[2:], (1,) * n, padding, dilation)
         return conv_nd_weight(x, weight_shape, _stuffed(g, dense_sp, stride), stride=1, padding=padding, dilation=dilation,
                               with_bias_grad=with_bias_grad)
+    extra = _prepad(weight_shape[2:], stride, padding, dilation) if plain else None
+    if extra is not None:
+        return conv_nd_weight(_zero_rim(x, extra), weight_shape, g, stride=1, padding=tuple(p - e for p, e in zip(padding, extra)),
+                              dilation=dilation, with_bias_grad=with_bias_grad)
     if plain and _dilated_ok(weight_shape[2:], stride, padding, dilation):
         phases = _phase_counts(weight_shape[2:], dilation)
         out_sp = _out_spatial(x.shape[2:], weight_shape[2:], stride, padding, dilation)

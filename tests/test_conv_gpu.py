@@ -102,6 +102,14 @@ PRIM_CASES = [
     (1, 16, 16, (5, 9, 10), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 2),
     (2, 64, 64, (18, 34), (3, 3), (1, 1), (0, 0), (1, 1), 2),   # a shape the MFMA kernels would take ungrouped
     (1, 12, 8, (30,), (5,), (1,), (2,), (1,), 4),
+    # dilated kernels of more than three taps (residue images on the tap-block route), a padding that is no multiple of
+    # the dilation (the remainder as a rim of zeros around the input), two taps an axis (a block with a zero tap in front)
+    (2, 3, 5, (15, 18), (5, 3), (1, 1), (4, 2), (2, 2)),
+    (1, 4, 6, (13, 17), (3, 3), (1, 1), (1, 3), (2, 2)),
+    (2, 5, 4, (14, 15), (3, 3), (2, 2), (1, 1), (2, 3)),
+    (1, 6, 7, (9, 11), (2, 2), (1, 1), (1, 0), (1, 1)),
+    (1, 3, 4, (6, 7, 8), (1, 2, 2), (1, 1, 1), (0, 1, 1), (1, 1, 1)),
+    (2, 4, 4, (12, 12), (2, 2), (1, 1), (0, 0), (2, 2)),
     # groups of at least 8 channels a side: each group as an ungrouped layer of its own (matrix cores, and the routes above)
     (2, 48, 32, (20, 22), (3, 3), (2, 2), (1, 1), (1, 1), 2),
     (1, 32, 64, (17, 19), (5, 5), (1, 1), (2, 2), (1, 1), 4),

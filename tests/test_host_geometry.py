@@ -128,6 +128,8 @@ DILATED = [
     ((12, 16), (3, 3), (0, 0), (2, 2)),
     ((9, 10), (3, 1), (4, 0), (2, 5)),
     ((5, 9, 11), (3, 3, 3), (1, 2, 4), (1, 2, 2)),
+    ((15, 18), (5, 3), (4, 2), (2, 2)),     # five taps: the residue images are undilated five-tap problems
+    ((11, 12), (2, 4), (3, 0), (3, 2)),
 ]
 
 
@@ -161,18 +163,46 @@ def test_residue_images_are_undilated_problems(case):
     assert torch.equal(jc._from_phases(jc._to_phases(x.detach(), phases, ext_in), phases, 2, insp), x.detach())
 
 
+@pytest.mark.parametrize("insp,k,p,d", [((13, 17), (3, 3), (1, 3), (2, 2)), ((12, 15), (5, 3), (3, 1), (2, 3)), ((7, 9, 11), (3, 3, 3), (0, 1, 2), (1, 2, 4))])
+def test_a_zero_rim_makes_the_padding_a_multiple_of_the_dilation(insp, k, p, d):
+    """The route for paddings that are no multiple of the dilation, with torch's CPU operators in place of the kernels."""
+    ns = len(k)
+    extra = jc._prepad(k, (1,) * ns, p, d)
+    assert extra is not None and all((pp - e) % dd == 0 for pp, e, dd in zip(p, extra, d))
+    conv = {2: F.conv2d, 3: F.conv3d}[ns]
+    torch.manual_seed(0)
+    x = torch.randn(2, 3, *insp, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(4, 3, *k, dtype=torch.float64, requires_grad=True)
+    y = conv(x, w, None, 1, p, d)
+    g = torch.randn_like(y)
+    y.backward(g)
+    xr = jc._zero_rim(x.detach(), extra).requires_grad_()
+    wr = w.detach().clone().requires_grad_()
+    rest = tuple(pp - e for pp, e in zip(p, extra))
+    yr = conv(xr, wr, None, 1, rest, d)
+    assert yr.shape == y.shape and torch.allclose(yr, y.detach(), atol=1e-12)
+    yr.backward(g)
+    inner = (slice(None), slice(None)) + tuple(slice(e, e + v) for v, e in zip(insp, extra))
+    assert torch.allclose(xr.grad[inner], x.grad, atol=1e-12) and torch.allclose(wr.grad, w.grad, atol=1e-10)
+
+
 def test_the_dilated_route_takes_only_what_it_covers():
     assert not jc._dilated_ok((3, 3), (1, 1), (1, 1), (2, 2))      # padding not a multiple of the dilation
     assert not jc._dilated_ok((3, 3), (2, 1), (2, 2), (2, 2))      # strided: through the stride-1 route first
-    assert not jc._dilated_ok((5, 3), (1, 1), (4, 2), (2, 2))      # five taps
+    assert jc._dilated_ok((5, 3), (1, 1), (4, 2), (2, 2))          # five taps: the residue images take the tap-block route
+    assert not jc._dilated_ok((11, 11), (1, 1), (10, 10), (2, 2))  # ... where that route takes the undilated layer
     assert not jc._dilated_ok((3, 3), (1, 1), (1, 1), (1, 1))      # nothing dilated
     assert jc._dilated_ok((1, 3), (1, 1), (0, 4), (7, 2))          # a dilation on a one-tap axis means nothing
-    assert jc._dense_stride_ok((3, 3), (2, 2), (2, 2), (2, 2)) and not jc._dense_stride_ok((3, 3), (2, 2), (2, 2), (1, 1))
+    assert jc._dense_stride_ok((3, 3), (2, 2), (2, 2), (2, 2)) and jc._dense_stride_ok((3, 3), (2, 2), (2, 2), (1, 1))
+    # a padding that is no multiple of the dilation: the remainder is laid around the input as zeros
+    assert jc._prepad((3, 3), (1, 1), (1, 1), (2, 2)) == (1, 1) and jc._prepad((3, 3), (1, 1), (3, 4), (2, 2)) == (1, 0)
+    assert jc._prepad((3, 3), (1, 1), (2, 4), (2, 2)) is None and jc._prepad((3, 1), (1, 1), (1, 3), (1, 2)) is None
+    assert jc._prepad((3, 3), (2, 1), (1, 1), (2, 2)) is None
 
 
 @pytest.mark.parametrize("insp,k,p", [
     ((12, 13), (5, 5), (2, 2)), ((11, 14), (7, 4), (3, 0)), ((9, 10), (5, 3), (0, 1)), ((6, 9, 10), (5, 3, 4), (2, 1, 0)),
-    ((10, 10), (9, 9), (4, 4)), ((12, 12), (2, 5), (0, 2)),
+    ((10, 10), (9, 9), (4, 4)), ((12, 12), (2, 5), (0, 2)), ((9, 11), (2, 2), (1, 0)), ((8, 9), (2, 3), (0, 1)), ((6, 7, 8), (1, 2, 2), (0, 1, 1)),
 ])
 def test_tap_blocks_are_channel_blocks_of_a_three_tap_layer(insp, k, p):
     """The route of kernels with more than three taps, with torch's CPU operators in place of the
@@ -201,6 +231,7 @@ def test_tap_blocks_are_channel_blocks_of_a_three_tap_layer(insp, k, p):
 
 def test_the_tap_block_route_takes_only_what_it_covers():
     assert not jc._big_kernel_ok((3, 3), (1, 1), (1, 1))          # three taps: the kernels as they are
+    assert not jc._big_kernel_ok((1, 3), (1, 1), (1, 1)) and jc._big_kernel_ok((2, 2), (1, 1), (1, 1))  # two taps: a block with a zero tap in front
     assert not jc._big_kernel_ok((5, 5), (2, 2), (1, 1))          # strided: through the stride-1 route first
     assert jc._dense_stride_ok((5, 5), (2, 2), (1, 1), (2, 2)) and not jc._dense_stride_ok((4, 4), (4, 4), (1, 1), (0, 0))
     assert not jc._big_kernel_ok((5, 5), (1, 1), (2, 1))          # dilated
