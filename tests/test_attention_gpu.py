@@ -241,6 +241,43 @@ def test_config4_shape_properties(dev):
     assert rel_l2(lse[:, :, rows], torch.logsumexp(s, -1)) < 1e-4
 
 
+def test_config4_shape_in_fp32_on_the_matrix_cores(dev):
+    """Config 4's ring at full size with fp32 inputs (8 heads, 4096 queries, 4 chunks of 4096 keys, d = 64):
+    ring of fused steps == one core call over the concatenated K/V, forward and backward; sampled
+    rows against fp64; and the bf16 kernels' result within bf16's tolerance of it."""
+    torch.manual_seed(6)
+    b, h, n, d, P = 1, 8, 4096, 64, 4
+    scale = d**-0.5
+    q = torch.randn(b, h, n, d, device=dev) / 8
+    ks = [torch.randn(b, h, n, d, device=dev) for _ in range(P)]
+    vs = [torch.randn(b, h, n, d, device=dev) for _ in range(P)]
+    dout = torch.randn(b, h, n, d, device=dev)
+    Kc, Vc = torch.cat(ks, 2), torch.cat(vs, 2)
+    out, lse = ja.ring_forward(q, ks, vs, scale, rank=1)
+    full_o, full_l = ja.core_forward(q, Kc, Vc, scale)
+    assert out.dtype == torch.float32 and rel_l2(out, full_o) < 1e-5 and rel_l2(lse, full_l) < 1e-6
+    rows = torch.arange(5, n, 64)
+    qs = q[:, :, rows].double().cpu()
+    s = (qs @ Kc.double().cpu().mT) * scale
+    assert rel_l2(out[:, :, rows], torch.softmax(s, -1) @ Vc.double().cpu()) < 1e-5
+    assert rel_l2(lse[:, :, rows], torch.logsumexp(s, -1)) < 1e-6
+    o16, l16 = ja.ring_forward(q.bfloat16(), [t.bfloat16() for t in ks], [t.bfloat16() for t in vs], scale, rank=1)
+    assert rel_l2(o16, out) < 2e-2 and rel_l2(l16, lse) < 1e-3
+
+    dq, dks, dvs = ja.ring_backward(dout, q, out, lse, ks, vs, scale)
+    fdq, fdk, fdv = ja.core_backward(dout, q, Kc, Vc, out, lse, scale)
+    assert rel_l2(dq, fdq) < 1e-5 and rel_l2(torch.cat(dks, 2), fdk) < 1e-5 and rel_l2(torch.cat(dvs, 2), fdv) < 1e-5
+    # sampled keys of one chunk against fp64 (every query takes part)
+    keys = torch.arange(3, n, 128)
+    Q, O, dO, L = q.double().cpu(), out.double().cpu(), dout.double().cpu(), lse.double().cpu()
+    Kj, Vj = ks[2][:, :, keys].double().cpu(), vs[2][:, :, keys].double().cpu()
+    p = torch.exp((Q @ Kj.mT) * scale - L.unsqueeze(-1))
+    delta = (dO * O).sum(-1, keepdim=True)
+    ds = p * (dO @ Vj.mT - delta) * scale
+    assert rel_l2(dvs[2][:, :, keys], p.mT @ dO) < 1e-5
+    assert rel_l2(dks[2][:, :, keys], ds.mT @ Q) < 1e-5
+
+
 def test_config4_backward_shape_properties(dev):
     """Config 4 backward at full size (8 heads, 4096 queries, 4 chunks of 4096 keys, d = 64,
     bf16), from the GLOBAL out / lse as the ring holds them (backward.py:176-270).
