@@ -392,8 +392,12 @@ def swin_figures(dev, iters: int) -> dict:
     ms = time_gpu(step, max(20, iters), warmup=5)
     xr = x.detach()
     ms_roll = time_gpu(lambda: jr.roll(xr, (-4, -4), (1, 2)), iters)
+    # the same step recorded once in a HIP graph (no host work per launch) and replayed
+    recorded = block.captured_step(xr.clone(), gout.clone())
+    ms_graph = time_gpu(recorded.replay, max(20, iters), warmup=5)
     return {
         "swin_block_fwd_bwd": {"ms": ms},
+        "swin_block_fwd_bwd_hip_graph": {"ms": ms_graph},
         "roll": {"ms": ms_roll, "GBps": 2 * xr.numel() * 2 / (ms_roll * 1e-3) / 1e9, "bytes": 2 * xr.numel() * 2},
     }
 

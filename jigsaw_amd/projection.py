@@ -18,6 +18,7 @@ gradient: one GEMM contracted over the tokens). The weights are the rank's local
 
 from __future__ import annotations
 
+import contextlib
 import math
 
 import torch
@@ -33,6 +34,21 @@ def _nt(out, a, w, bias, rows, n_out, k_in, a_heads, out_heads, dims) -> None:
     _lib.check(rc, "jg_proj_nt")
 
 
+_remember_casts = True
+
+
+@contextlib.contextmanager
+def fresh_casts():
+    """Inside, the casts of the parameters are made anew and not remembered: for work that is recorded
+    in a HIP graph, where a remembered copy would be read at every replay in place of the parameter."""
+    global _remember_casts
+    before, _remember_casts = _remember_casts, False
+    try:
+        yield
+    finally:
+        _remember_casts = before
+
+
 def _cast_cached(t: torch.Tensor | None, dtype: torch.dtype, transposed: bool = False) -> torch.Tensor | None:
     """``t`` in ``dtype``, contiguous (optionally its transpose), remembered on the tensor until
     its next in-place update: under autocast the parameters are fp32 and every forward and
@@ -43,6 +59,9 @@ def _cast_cached(t: torch.Tensor | None, dtype: torch.dtype, transposed: bool = 
         return None
     if not transposed and t.dtype == dtype and t.is_contiguous():
         return t
+    if not _remember_casts:
+        src = t.detach()
+        return (src.t() if transposed else src).to(dtype).contiguous()
     key = (dtype, transposed)
     cache = getattr(t, "_jg_casts", None)
     if cache is None or cache[0] != t._version:

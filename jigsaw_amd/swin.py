@@ -32,6 +32,7 @@ from .projection import (
     linear,
     mlp_fusable,
     qkv_projection,
+    fresh_casts,
 )
 from .roll import _Roll
 
@@ -201,6 +202,47 @@ class _WholeBlock(torch.autograd.Function):
         return gx, gn1w, gn1b, gqw, gqb, dtable, gpw, gpb, gn2w, gn2b, gw1, gb1, gw2, gb2, None
 
 
+class CapturedStep:
+    """One forward + backward of a :class:`SwinBlock` as a HIP graph (see ``SwinBlock.captured_step``).
+
+    ``x`` / ``grad_out``: the input buffers. After :meth:`replay`: ``y`` the block's output, ``grad_x``
+    the gradient of ``x``, ``grads`` the gradients of the parameters by name (fresh values at every
+    replay, not accumulated into ``.grad``). A replay only enqueues work on the current stream."""
+
+    _NAMES = ("norm1.weight", "norm1.bias", "attn.qkv.weight", "attn.qkv.bias", "attn.bias_table", "attn.proj.weight",
+              "attn.proj.bias", "norm2.weight", "norm2.bias", "mlp.0.weight", "mlp.0.bias", "mlp.2.weight", "mlp.2.bias")
+
+    def __init__(self, block: "SwinBlock", x: torch.Tensor, grad_out: torch.Tensor, warmup: int):
+        self.x, self.grad_out = x, grad_out
+        named = dict(block.named_parameters())
+        params = [named[n].detach() for n in self._NAMES]
+
+        def step():
+            ctx = _Stage()
+            ctx.needs_input_grad = (True,) * 15
+            # the bf16 copies of the fp32 parameters are made inside the step, so a replay reads the parameters
+            with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16), fresh_casts():
+                y = _WholeBlock.forward(ctx, self.x, *params, block)
+                return y, _WholeBlock.backward(ctx, self.grad_out)
+
+        # first calls outside the capture: one-time set-up of the kernels (LDS reservations, lookup tables)
+        # and the allocator's pool for the capturing stream
+        side = torch.cuda.Stream(device=x.device)
+        side.wait_stream(torch.cuda.current_stream(x.device))
+        with torch.cuda.stream(side):
+            for _ in range(max(1, warmup)):
+                step()
+        torch.cuda.current_stream(x.device).wait_stream(side)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, stream=side):
+            self.y, grads = step()
+        self.grad_x = grads[0]
+        self.grads = dict(zip(self._NAMES, grads[1:14]))
+
+    def replay(self) -> None:
+        self.graph.replay()
+
+
 class SwinBlock(nn.Module):
     """``x + attn(norm(x))`` then ``x + mlp(norm(x))``; the windows may be shifted
     (examples/swin.py:173-210). ``groups`` are the two spatial groups of the tile
@@ -242,6 +284,27 @@ class SwinBlock(nn.Module):
         if not _lib.load().jg_ln_plain_supported(c) or any(t is None for t in (attn.qkv.bias, attn.proj.bias, fc1.bias, fc2.bias)):
             return False
         return mlp_fusable(x, fc1.weight, fc2.weight, x)
+
+    def captured_step(self, x: torch.Tensor, grad_out: torch.Tensor, warmup: int = 3) -> "CapturedStep":
+        """Forward + backward of the block for these shapes, recorded once in a HIP graph.
+
+        The launches are those of the one-node form (bf16 tokens, 8 x 8 windows, heads of 32), issued
+        by calling its ``forward`` / ``backward`` directly, with no autograd engine in between: no
+        worker thread, no accumulation nodes, nothing a stream capture refuses. ``x`` and
+        ``grad_out`` become the graph's input buffers (copy new values into them before a replay),
+        the block's parameters are read where they lie at every replay, and the results are written to
+        the same tensors every time. The roll's ``comm_fn`` runs while the graph is recorded, on the
+        capturing stream: whatever it launches there is replayed with the rest."""
+        if not self._one_node_ok(x):
+            raise NotImplementedError("captured_step needs the shapes of the one-node block: bf16 tokens, 8 x 8 windows, "
+                                      "heads of 32, biases present")
+        if grad_out.shape != x.shape or grad_out.dtype != x.dtype:
+            raise ValueError(f"grad_out {tuple(grad_out.shape)} {grad_out.dtype} does not match x {tuple(x.shape)} {x.dtype}")
+        return CapturedStep(self, x.detach(), grad_out.detach(), warmup)
+
+    def _one_node_ok(self, x: torch.Tensor) -> bool:
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            return self._one_node(x)
 
     def _norm(self, ln: nn.LayerNorm, x: torch.Tensor) -> torch.Tensor:
         # Both LayerNorms feed a linear layer (through pure copies), which under autocast rounds

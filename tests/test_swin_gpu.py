@@ -187,3 +187,48 @@ def test_block_as_one_autograd_node_has_the_bits_of_its_parts(shift, n, dev):
     assert rel_l2(o1, want.detach()) < 2e-2 and rel_l2(x1.grad, xd.grad) < 2e-2
     for name, prm in one.named_parameters():
         assert rel_l2(prm.grad, params[name].grad) < 2e-2, name
+
+
+@pytest.mark.parametrize("shift", [0, 4])
+def test_block_step_recorded_in_a_hip_graph_replays_the_eager_step(shift, dev):
+    """``SwinBlock.captured_step``: forward + backward recorded once, replayed several times with eager
+    work and synchronisations in between; every replay gives the eager step's output, input gradient
+    and parameter gradients bit for bit, also after new values were copied into the input buffers and
+    after a parameter changed in place."""
+    torch.manual_seed(7)
+    dim, heads, window, n = 128, 4, 8, (32, 48)
+    block = js.SwinBlock(dim, heads, window, n, shift=shift, device=dev)
+    with torch.no_grad():
+        block.attn.bias_table.normal_(0, 0.5)
+
+    def eager(x, g):
+        for p in block.parameters():
+            p.grad = None
+        xg = x.clone().requires_grad_()
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = block(xg)
+        out.backward(g)
+        return out.detach(), xg.grad, {k: p.grad.clone() for k, p in block.named_parameters()}
+
+    x = torch.randn(1, *n, dim, device=dev).bfloat16()
+    g = torch.randn(1, *n, dim, device=dev).bfloat16()
+    step = block.captured_step(x.clone(), g.clone())
+    assert set(step.grads) == {k for k, _ in block.named_parameters()}
+    for rep in range(4):
+        if rep == 2:  # new values in the graph's input buffers
+            x, g = torch.randn_like(x), torch.randn_like(g)
+            step.x.copy_(x)
+            step.grad_out.copy_(g)
+        if rep == 3:  # parameters are read where they lie
+            with torch.no_grad():
+                for prm in block.parameters():
+                    prm.mul_(1.25).add_(0.01)
+        step.replay()
+        torch.cuda.synchronize()
+        y, gx, grads = eager(x, g)  # eager work between the replays, and the values to meet
+        torch.cuda.synchronize()
+        assert torch.equal(step.y, y) and torch.equal(step.grad_x, gx), rep
+        for k, want in grads.items():
+            assert step.grads[k].dtype == want.dtype and torch.equal(step.grads[k], want), (rep, k)
+    with pytest.raises(NotImplementedError):
+        block.captured_step(x.float(), g.float())
