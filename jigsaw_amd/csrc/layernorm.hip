@@ -997,7 +997,7 @@ static void launch_apply(void* y, void* x_hat, float* std_out, const void* x, co
   const bool vo = vec_aligned(y, cols, ODT) && (x_hat == nullptr || vec_aligned(x_hat, cols, ODT));
   const bool vw = vec_aligned(w, cols, ODT) && (b == nullptr || vec_aligned(b, cols, ODT));
   if (plain_ok(cols) && aligned16(x) && aligned16(y) && aligned16(x_hat) && aligned16(w) && aligned16(b)) {
-    const int G = plain_group(cols), blocks = plain_blocks(rows, cols);
+    const int G = plain_group(cols), blocks = plain_blocks(rows, cols, 2048);
     with_row_shape<2>(cols, [&](auto ch, auto u) {
       ln_apply_rows_kernel<XDT, ODT, decltype(ch)::value, decltype(u)::value><<<blocks, kThreads, 0, s>>>(
           static_cast<OT*>(y), static_cast<OT*>(x_hat), std_out, static_cast<const XT*>(x), mean, var,
@@ -1185,7 +1185,7 @@ extern "C" int jg_ln_bwd_apply(void* gx, const void* g, const void* x_hat, const
                    vec_aligned(gx, cols, DT);                                              \
     const bool vw = vec_aligned(w, cols, DT);                                              \
     if (plain_ok(cols) && aligned16(gx) && aligned16(g) && aligned16(x_hat) && aligned16(w)) { \
-      const int G = plain_group(cols), blocks = plain_blocks(rows, cols);                  \
+      const int G = plain_group(cols), blocks = plain_blocks(rows, cols, 2048);                  \
       with_row_shape<2>(cols, [&](auto ch, auto u) {                                       \
         ln_bwd_apply_rows_kernel<DT, decltype(ch)::value, decltype(u)::value>              \
             <<<blocks, kThreads, 0, s>>>(static_cast<T*>(gx), static_cast<const T*>(g),    \
