@@ -924,7 +924,7 @@ void launch_plain_fwd(void* y, float* mean, float* rstd, const void* x, const fl
                       long long rows, int cols, float eps, hipStream_t s) {
   typedef typename Elem<XDT>::T XT;
   typedef typename Elem<YDT>::T YT;
-  const int G = plain_group(cols), blocks = plain_blocks(rows, cols);
+  const int G = plain_group(cols), blocks = plain_blocks(rows, cols, 2048);
 #define JG_GO(CH, U)                                                                                   \
   ln_plain_fwd_kernel<XDT, YDT, CH, U><<<blocks, kThreads, 0, s>>>(static_cast<YT*>(y), mean, rstd,     \
                                                                    static_cast<const XT*>(x), w, b, rows, cols, eps, G)
