@@ -18,6 +18,7 @@ from __future__ import annotations
 
 import argparse
 import gc
+import itertools
 import json
 import os
 import sys
@@ -102,13 +103,31 @@ def build_conv2_workload(dev, batch=8, ch=64, tile=1024):
             "bands": bands}
 
 
-def conv_step(wl, kernel_events=None):
+def conv_step_buffers(wl) -> dict:
+    """Every tensor one step writes, and the three workspaces, allocated once: the timed steps then
+    allocate nothing (``out=`` / ``workspace=`` of the host functions)."""
+    from jigsaw_amd import conv as jc
+    from jigsaw_amd.halo import halo_assemble, halo_pack
+
+    geom, x, w, g = wl["geom"], wl["x"], wl["w"], wl["g"]
+    dev = x.device
+    ws = lambda: torch.empty(256 << 20, dtype=torch.uint8, device=dev)  # noqa: E731  (more than any of the three asks for)
+    buf = {"ws_fwd": ws(), "ws_dgrad": ws(), "ws_wgrad": ws()}
+    buf["pack"] = halo_pack(x, geom, from_padded=False)
+    buf["x_aug"] = halo_assemble(x, wl["strips_fwd"], geom)
+    buf["y"] = jc.conv_nd(buf["x_aug"], w, wl["b"])
+    buf["gx_send"] = jc.conv_nd_input_fold(geom, w, g)
+    buf["gw_gb"] = jc.conv_nd_weight(buf["x_aug"], w.shape, g, with_bias_grad=True)
+    return buf
+
+
+def conv_step(wl, buf, kernel_events=None):
     """The hot path of one rank for one batch (see the module docstring). The backward
     uses the fused forms, each with the bits of the separate steps it replaces: dgrad
     writes the owned cells and the strips it sends in one pass, wgrad adds up the bias
     gradient on the way, and the received strips are added to the border afterwards.
-    ``kernel_events`` collects HIP-event brackets (on the launch stream) around the three
-    convolution launches of the step."""
+    ``kernel_events`` maps a name to (start, end) HIP events, made before the loop, recorded here on the
+    launch stream around the three convolution launches of the step."""
     from jigsaw_amd import conv as jc
     from jigsaw_amd.halo import halo_assemble, halo_fold_border_, halo_pack
 
@@ -117,22 +136,57 @@ def conv_step(wl, kernel_events=None):
     def bracket(name, fn):
         if kernel_events is None:
             return fn()
-        e0, e1 = _events()
+        e0, e1 = kernel_events[name]
         e0.record()
         out = fn()
         e1.record()
-        kernel_events.setdefault(name, []).append((e0, e1))
         return out
 
-    halo_pack(x, geom, from_padded=False)  # strips this rank sends
-    x_aug = halo_assemble(x, wl["strips_fwd"], geom)
-    y = bracket("fwd", lambda: jc.conv_nd(x_aug, w, b))
+    halo_pack(x, geom, from_padded=False, out=buf["pack"])  # strips this rank sends
+    x_aug = halo_assemble(x, wl["strips_fwd"], geom, out=buf["x_aug"])
+    y = bracket("fwd", lambda: jc.conv_nd(x_aug, w, b, out=buf["y"], workspace=buf["ws_fwd"]))
     # owned cells + halo gradients this rank sends
-    gx, _send = bracket("dgrad_fold", lambda: jc.conv_nd_input_fold(geom, w, g))
+    gx, _send = bracket("dgrad_fold", lambda: jc.conv_nd_input_fold(geom, w, g, out=buf["gx_send"], workspace=buf["ws_dgrad"]))
     # one pass over g for the weight and the bias gradient
-    gw, gb = bracket("wgrad_bias", lambda: jc.conv_nd_weight(x_aug, w.shape, g, with_bias_grad=True))
+    gw, gb = bracket("wgrad_bias", lambda: jc.conv_nd_weight(x_aug, w.shape, g, with_bias_grad=True, out=buf["gw_gb"],
+                                                             workspace=buf["ws_wgrad"]))
     halo_fold_border_(gx, wl["strips_bwd"], geom)
     return y, gx, gw, gb
+
+
+def timed_conv_steps(wl, steps: int, warmup: int) -> dict:
+    """W warm-up steps, then exactly K timed steps with the collector off and nothing allocated:
+    HIP events around every step and around its three convolution launches (all events made
+    before the loop), a synchronisation on both sides. Returns per-step and per-kernel times."""
+    buf = conv_step_buffers(wl)
+    names = ("fwd", "dgrad_fold", "wgrad_bias")
+    step_ev = [_events() for _ in range(steps)]
+    kern_ev = [{n: _events() for n in names} for _ in range(steps)]
+    for _ in range(warmup):
+        conv_step(wl, buf)
+    torch.cuda.synchronize()
+    gc.collect()
+    gc.disable()
+    try:
+        t0 = time.perf_counter()
+        for i in range(steps):
+            step_ev[i][0].record()
+            conv_step(wl, buf, kern_ev[i])
+            step_ev[i][1].record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+    finally:
+        gc.enable()
+    per_step = [a.elapsed_time(b) for a, b in step_ev]
+    span_ms = step_ev[0][0].elapsed_time(step_ev[-1][1])  # first step's start to last step's end, gaps included
+    per_kernel = {n: [ev[n][0].elapsed_time(ev[n][1]) for ev in kern_ev] for n in names}
+    return {"per_step": per_step, "span_ms": span_ms, "wall_ms": wall_ms, "per_kernel": per_kernel, "buf": buf}
+
+
+def _median(v):
+    v = sorted(v)
+    n = len(v)
+    return v[n // 2] if n % 2 else 0.5 * (v[n // 2 - 1] + v[n // 2])
 
 
 def attention_figures(dev, iters: int) -> dict:
@@ -198,10 +252,13 @@ def attention_figures(dev, iters: int) -> dict:
     hop_bwd["ms_no_hop"] = time_gpu(lambda: ja.ring_backward(dout, q, out, l, ks, vs, scale), iters)
     x = torch.randn(b, n, 256, device=dev, generator=g).bfloat16()
     ms_ln = time_gpu(lambda: jl.partial_stats(x), iters)
-    # the same statistics on a shard that fills the chip (2 ** 18 rows of the same local width)
-    xl = torch.randn(1 << 18, 256, device=dev, generator=g).bfloat16()
-    ms_ln_big = time_gpu(lambda: jl.partial_stats(xl), iters)
-    del xl
+    # the same statistics on a shard that fills the chip (2 ** 18 rows of the same local width), over six
+    # different 134 MB tensors in turn: one alone would stay in the 256 MB last-level cache and the
+    # figure would not be an HBM rate
+    xls = [torch.randn(1 << 18, 256, device=dev, generator=g).bfloat16() for _ in range(6)]
+    turn = itertools.count()
+    ms_ln_big = time_gpu(lambda: jl.partial_stats(xls[next(turn) % len(xls)]), max(iters, 2 * len(xls)), warmup=len(xls))
+    del xls
     # the separate LSE merge (what a step runs when its core cannot fuse it): fp32 accumulator read and
     # written, the step's bf16 output read; at the step's size and at 16 x the heads
     merge = {}
@@ -354,15 +411,16 @@ def projection_figures(dev, iters: int) -> dict:
     }
 
 
-def swin_figures(dev, iters: int) -> dict:
-    """Configuration 5: one rank's Swin block on a 256x256-token tile, dim 128, 4 heads,
-    8x8 windows, shift 4, bf16 autocast; the roll's cross-tile slabs are seeded."""
-    from jigsaw_amd import roll as jr
+def _swin_step(dev):
+    """Configuration 5's block, its inputs and ``step()`` = one forward + backward under bf16 autocast."""
+    from jigsaw_amd import projection as jp
     from jigsaw_amd import swin as js
     from jigsaw_amd.conv import TileGroup
 
+    # the bf16 copies of the fp32 parameters are kept between steps, as a training loop whose optimizer
+    # updates the parameters in place would ask for (nothing here writes through ``.data``)
+    jp.remember_casts(True)
     g = torch.Generator(device=dev).manual_seed(2)
-
     slabs = {}
 
     def comm(data, buffer, direction, *, group, async_op):
@@ -378,7 +436,6 @@ def swin_figures(dev, iters: int) -> dict:
     block = js.SwinBlock(dim, 4, 8, n, groups, comm, shift=4, device=dev)
     x = torch.randn(1, *n, dim, device=dev, generator=g).bfloat16().requires_grad_()
     gout = torch.randn(1, *n, dim, device=dev, generator=g).bfloat16()
-
     leaves = [x, *block.parameters()]
 
     def step():
@@ -388,16 +445,21 @@ def swin_figures(dev, iters: int) -> dict:
             y = block(x)
         y.backward(gout)
 
+    return step, x
+
+
+def swin_figures(dev, iters: int) -> dict:
+    """Configuration 5: one rank's Swin block on a 256x256-token tile, dim 128, 4 heads,
+    8x8 windows, shift 4, bf16 autocast; the roll's cross-tile slabs are seeded."""
+    from jigsaw_amd import roll as jr
+
+    step, x = _swin_step(dev)
     # a host-bound step of ~40 launches: a handful of cold iterations says little, so more of them
     ms = time_gpu(step, max(20, iters), warmup=5)
     xr = x.detach()
     ms_roll = time_gpu(lambda: jr.roll(xr, (-4, -4), (1, 2)), iters)
-    # the same step recorded once in a HIP graph (no host work per launch) and replayed
-    recorded = block.captured_step(xr.clone(), gout.clone())
-    ms_graph = time_gpu(recorded.replay, max(20, iters), warmup=5)
     return {
         "swin_block_fwd_bwd": {"ms": ms},
-        "swin_block_fwd_bwd_hip_graph": {"ms": ms_graph},
         "roll": {"ms": ms_roll, "GBps": 2 * xr.numel() * 2 / (ms_roll * 1e-3) / 1e9, "bytes": 2 * xr.numel() * 2},
     }
 
@@ -541,6 +603,157 @@ def conv2_extras(wl, x_aug, it: int, flop_one: int, flop_step: int, ms_fwd: floa
     }
 
 
+# --------------------------------------------------------------------------- #
+# Launch-only modes for rocprofv3 (``--profile MODE``): each runs a few repetitions of one group of
+# kernels and prints no figures, so that a kernel trace or a counter run of the command holds those
+# launches and little else.
+# --------------------------------------------------------------------------- #
+def profile_conv2_attention(reps: int = 3) -> None:
+    """Every hot kernel of configuration 2 (the step as the benchmark runs it, then the separate
+    operators the fused ones replace) and the attention core of configuration 4, plus a plain device copy
+    of known size that calibrates the FETCH_SIZE / WRITE_SIZE counters."""
+    from jigsaw_amd import attention as ja
+    from jigsaw_amd import conv as jc
+    from jigsaw_amd.halo import halo_fold, halo_fold_border_
+
+    dev = torch.device("cuda:0")
+    wl = build_conv2_workload(dev)
+    buf = conv_step_buffers(wl)
+    geom, x, w, gout = wl["geom"], wl["x"], wl["w"], wl["g"]
+    x_aug = buf["x_aug"]
+    gx_aug = jc.conv_nd_input(x_aug.shape, w, gout)
+    gx = torch.empty_like(x)
+    copy_dst = torch.empty_like(x)  # calibration copy: reads and writes x.numel() * 2 bytes
+    g = torch.Generator(device=dev).manual_seed(0)
+    q = (torch.randn(1, 8, 4096, 64, device=dev, generator=g) / 8).bfloat16()
+    k = torch.randn(1, 8, 4096, 64, device=dev, generator=g).bfloat16()
+    v = torch.randn(1, 8, 4096, 64, device=dev, generator=g).bfloat16()
+    dout = torch.randn(1, 8, 4096, 64, device=dev, generator=g).bfloat16()
+    acc = torch.zeros(1, 8, 4096, 64, device=dev)
+    lse = torch.full((1, 8, 4096), float("-inf"), device=dev)
+    out, l = ja.core_forward(q, k, v, 0.125)
+    for _ in range(reps):
+        copy_dst.copy_(x)
+        conv_step(wl, buf)
+        # the separate steps the fused ones replace
+        jc.conv_nd_input(x_aug.shape, w, gout)
+        jc.sum_grad_bias(gout, 2)
+        halo_fold(gx_aug, wl["strips_bwd"], geom, out=gx)
+        halo_fold_border_(gx, wl["strips_bwd"], geom)
+        ja.core_forward(q, k, v, 0.125, out_acc=acc, lse_acc=lse, want_out=False)
+        ja.core_backward(dout, q, k, v, out, l, 0.125)
+    torch.cuda.synchronize()
+
+
+def profile_around_attention(reps: int = 3) -> None:
+    """The kernels either side of the ring step: the attention core at head size 128 (32 heads, 4096 x 4096
+    tokens) and the qkv / output projections with the head split fused in (8 x 4096 tokens, 512 channels, 8 heads)."""
+    from jigsaw_amd import attention as ja
+    from jigsaw_amd import projection as jp
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(1)
+    h, n, d = 32, 4096, 128
+    q = (torch.randn(1, h, n, d, device=dev, generator=g) / d**0.5).bfloat16()
+    k = torch.randn(1, h, n, d, device=dev, generator=g).bfloat16()
+    v = torch.randn(1, h, n, d, device=dev, generator=g).bfloat16()
+    dout = torch.randn(1, h, n, d, device=dev, generator=g).bfloat16()
+    out, lse = ja.core_forward(q, k, v, d**-0.5)
+    bsz, c, heads = 8, 512, 8
+    x = torch.randn(bsz, n, c, device=dev, generator=g).bfloat16().requires_grad_()
+    w = (torch.randn(3 * c, c, device=dev, generator=g) / c**0.5).bfloat16().requires_grad_()
+    b = (0.1 * torch.randn(3 * c, device=dev, generator=g)).bfloat16().requires_grad_()
+    wo = (torch.randn(c, c, device=dev, generator=g) / c**0.5).bfloat16()
+    o = torch.randn(bsz, heads, n, c // heads, device=dev, generator=g).bfloat16()
+    gy = torch.randn(3, bsz, heads, n, c // heads, device=dev, generator=g).bfloat16()
+    for _ in range(reps):
+        ja.core_forward(q, k, v, d**-0.5)
+        ja.core_backward(dout, q, k, v, out, lse, d**-0.5)
+        y = jp.qkv_projection(x, w, b, heads)
+        torch.autograd.grad(y, (x, w, b), gy)
+        jp.heads_projection(o, wo, None)
+    torch.cuda.synchronize()
+
+
+def profile_ring(reps: int = 3) -> None:
+    """Configuration 4's ring, forward and backward over the four resident chunks (no hops)."""
+    from jigsaw_amd import attention as ja
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(0)
+    b, h, n, d, P = 1, 8, 4096, 64, 4
+    q = (torch.randn(b, h, n, d, device=dev, generator=g) / 8).bfloat16()
+    ks = [(torch.randn(b, h, n, d, device=dev, generator=g) / 8).bfloat16() for _ in range(P)]
+    vs = [(torch.randn(b, h, n, d, device=dev, generator=g) / 8).bfloat16() for _ in range(P)]
+    dout = torch.randn(b, h, n, d, device=dev, generator=g).bfloat16()
+    for _ in range(reps):
+        out, l = ja.ring_forward(q, ks, vs, d**-0.5)
+        ja.ring_backward(dout, q, out, l, ks, vs, d**-0.5)
+    torch.cuda.synchronize()
+
+
+def profile_swin_block(reps: int = 5) -> None:
+    """Forward + backward of one Swin block of configuration 5 (256 x 256 token tile, dim 128, 4 heads,
+    8 x 8 windows, shift 4, bf16 autocast; the neighbours' roll slabs are random stand-ins made once)."""
+    step = _swin_step(torch.device("cuda:0"))[0]
+    for _ in range(reps):
+        step()
+    torch.cuda.synchronize()
+
+
+def profile_attention_fp32(reps: int = 3) -> None:
+    """The attention core forward + backward on fp32 inputs (8 heads, 4096 x 4096 tokens) at head sizes 64, 128, 32."""
+    from jigsaw_amd import attention as ja
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(4)
+    for d in (64, 128, 32):
+        b, h, n = 1, 8, 4096
+        q, k, v, dout = (torch.randn(b, h, n, d, device=dev, generator=g) / 8 for _ in range(4))
+        scale = d**-0.5
+        for _ in range(reps):
+            out, lse = ja.core_forward(q, k, v, scale)
+            ja.core_backward(dout, q, k, v, out, lse, scale)
+        torch.cuda.synchronize()
+
+
+def profile_sharded_layernorm(reps: int = 3) -> None:
+    """Forward + backward of the channel-sharded LayerNorm on one shard's rows, bf16: 2 ** 18 rows of 256
+    channels (configuration 4's local width at a row count that fills the chip), 2 ** 20 rows of 64, and, for
+    the kernels that walk a row, 2 ** 18 rows of 132."""
+    from jigsaw_amd import layernorm as jl
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(3)
+    for rows, cols in ((1 << 18, 256), (1 << 20, 64), (1 << 18, 132)):
+        x = torch.randn(rows, cols, device=dev, generator=g).bfloat16().requires_grad_()
+        w = torch.ones(cols, device=dev, dtype=torch.bfloat16, requires_grad=True)
+        b = torch.zeros(cols, device=dev, dtype=torch.bfloat16, requires_grad=True)
+        gout = torch.randn(rows, cols, device=dev, generator=g).bfloat16()
+        for _ in range(reps):
+            x.grad = w.grad = b.grad = None
+            jl.layer_norm(x, w, b, None).backward(gout)
+        torch.cuda.synchronize()
+
+
+def profile_conv3d(reps: int = 3) -> None:
+    """Configuration 3: pack, assemble, forward, fused dgrad, wgrad, border fold and the separate fold."""
+    conv3d_figures(torch.device("cuda:0"), reps)
+
+
+PROFILE_MODES = {
+    "conv2-attention": profile_conv2_attention,
+    "around-attention": profile_around_attention,
+    "ring": profile_ring,
+    "swin-block": profile_swin_block,
+    "attention-fp32": profile_attention_fp32,
+    "sharded-layernorm": profile_sharded_layernorm,
+    "conv3d": profile_conv3d,
+}
+
+EXTRA_GROUPS = ("conv2", "attention", "conv3d", "swin", "groupnorm", "projection", "attention-wide")
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -551,6 +764,10 @@ def main() -> int:
     ap.add_argument("--no-extras", action="store_true",
                     help="only the timed steps and the roofline kernel (a kernel trace of this run then "
                     "holds the forward kernel's launches under a name of their own)")
+    ap.add_argument("--only", default=None, metavar="GROUPS",
+                    help="comma-separated groups of the figures under `extra` to run (default: all): " + ", ".join(EXTRA_GROUPS))
+    ap.add_argument("--profile", default=None, choices=sorted(PROFILE_MODES),
+                    help="launch one group of kernels a few times and print no figures (for rocprofv3 runs)")
     ns = ap.parse_args()
     if ns.gpus != 1:
         print(
@@ -561,6 +778,24 @@ def main() -> int:
         return 2
     if ns.cpu_baseline_only:
         print(json.dumps(cpu_baseline()))
+        return 0
+    groups = set(EXTRA_GROUPS)
+    if ns.only is not None:
+        groups = {v.strip() for v in ns.only.split(",") if v.strip()}
+        if groups - set(EXTRA_GROUPS):
+            print(f"bench.py: unknown group(s) {sorted(groups - set(EXTRA_GROUPS))}; known: {', '.join(EXTRA_GROUPS)}", file=sys.stderr)
+            return 2
+    if ns.no_extras:
+        groups = set()
+    if ns.profile is not None:
+        if not torch.cuda.is_available():
+            print("bench.py: no GPU visible; the HIP kernels have no CPU fallback.", file=sys.stderr)
+            return 2
+        import jigsaw_amd
+
+        jigsaw_amd.load()
+        PROFILE_MODES[ns.profile]()
+        print(f"bench.py --profile {ns.profile}: done", file=sys.stderr)
         return 0
     # The CPU leg runs first, in a child process of its own, before this process has touched
     # the GPU: it starts further processes (the gloo ranks), and its thread pools and buffers
@@ -580,8 +815,6 @@ def main() -> int:
         return 2
 
     import jigsaw_amd
-    from jigsaw_amd import conv as jc
-    from jigsaw_amd.halo import halo_assemble, halo_fold
 
     jigsaw_amd.load()  # fail loudly if the library is not built
     dev = torch.device("cuda:0")
@@ -591,30 +824,23 @@ def main() -> int:
     flop_step = 3 * flop_one
 
     # ---- the timed region: W warm-up steps, then exactly K steps
-    for _ in range(ns.warmup):
-        conv_step(wl)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    e0, e1 = _events()
-    e0.record()
-    kernel_events: dict = {}
-    for _ in range(ns.steps):
-        conv_step(wl, kernel_events)
-    e1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / ns.steps
-    ms_per_step = e0.elapsed_time(e1) / ns.steps
-    ms_per_step = max(ms_per_step, wall_ms)  # host-side gaps count too
+    timed = timed_conv_steps(wl, ns.steps, ns.warmup)
+    per_step = timed["per_step"]
+    ms_per_step = _median(per_step)
+    ms_mean = max(timed["span_ms"], timed["wall_ms"]) / ns.steps  # host-side gaps count too
+    if max(per_step) > 2 * ms_per_step:
+        worst = max(range(len(per_step)), key=per_step.__getitem__)
+        print(f"bench.py: step {worst} took {per_step[worst]:.3f} ms against a median of {ms_per_step:.3f} ms "
+              f"(per-kernel brackets of that step: " + ", ".join(f"{k} {v[worst]:.3f}" for k, v in timed["per_kernel"].items()) + ")",
+              file=sys.stderr)
     value = flop_step / (ms_per_step * 1e-3) / 1e12
 
-    # ---- per-kernel figures (HIP events around repeated launches of one operator)
-    geom = wl["geom"]
-    x_aug = halo_assemble(wl["x"], wl["strips_fwd"], geom)
+    # ---- per-kernel figures: the three convolution launches of the timed steps (the small weight
+    # re-layout and reduction launches that belong to each are inside its bracket), median over the
+    # steps; the roofline entry is the DOMINANT one: the longest
+    x_aug = timed["buf"]["x_aug"]
     it = max(5, ns.steps)
-    # the three convolution launches of the timed steps (the small weight re-layout and
-    # reduction launches that belong to each are inside its bracket); the roofline entry is
-    # the DOMINANT one: the longest
-    ms_kernel = {k: sum(a.elapsed_time(b) for a, b in v) / len(v) for k, v in kernel_events.items()}
+    ms_kernel = {k: _median(v) for k, v in timed["per_kernel"].items()}
     ms_fwd = ms_kernel["fwd"]
     dominant = max(ms_kernel, key=ms_kernel.get)
     tf = lambda ms: flop_one / (ms * 1e-3) / 1e12  # noqa: E731
@@ -627,15 +853,24 @@ def main() -> int:
         "frac": tf(ms_kernel[dominant]) / PEAK_BF16_TFLOPS,
         "traffic": CONV_TRAFFIC_BYTES[dominant],
     }
-    extra = {f"conv_{k}_in_step": {"ms": v, "tflops": tf(v), "frac_mfma_peak": tf(v) / PEAK_BF16_TFLOPS}
+    extra = {f"conv_{k}_in_step": {"ms": v, "ms_mean": sum(timed["per_kernel"][k]) / ns.steps, "ms_max": max(timed["per_kernel"][k]),
+                                   "tflops": tf(v), "frac_mfma_peak": tf(v) / PEAK_BF16_TFLOPS}
              for k, v in ms_kernel.items()}
-    if not ns.no_extras:
+    del timed
+    if "conv2" in groups:
         extra.update(conv2_extras(wl, x_aug, it, flop_one, flop_step, ms_fwd))
+    del x_aug
+    if "attention" in groups:
         extra.update(attention_figures(dev, max(10, it)))
+    if "conv3d" in groups:
         extra.update(conv3d_figures(dev, it))
+    if "swin" in groups:
         extra.update(swin_figures(dev, it))
+    if "groupnorm" in groups:
         extra.update(groupnorm_figures(dev, it))
+    if "projection" in groups:
         extra.update(projection_figures(dev, it))
+    if "attention-wide" in groups:
         extra.update(attention_wide_figures(dev, it))
 
     line = {
@@ -646,6 +881,10 @@ def main() -> int:
         "steps": ns.steps,
         "warmup": ns.warmup,
         "ms_per_step": ms_per_step,
+        "ms_per_step_stat": "median of the timed steps' HIP-event brackets",
+        "ms_per_step_mean": ms_mean,
+        "ms_per_step_max": max(per_step),
+        "ms_per_step_min": min(per_step),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

@@ -27,7 +27,7 @@ from typing import Any, Protocol
 import torch
 
 from . import _lib
-from .halo import HaloGeometry, halo_assemble, halo_fold, halo_fold_border_, halo_pack, new_strips
+from .halo import HaloGeometry, halo_assemble, halo_fold, halo_fold_border_, halo_pack, new_strips, strip_table
 
 # --------------------------------------------------------------------------- #
 # local primitives
@@ -73,11 +73,26 @@ def _out_spatial(in_spatial, kernel, stride, padding, dilation) -> tuple:
     return tuple(out)
 
 
-def _workspace(desc: _lib.ConvDesc, op: int, dtype: torch.dtype, device) -> tuple[torch.Tensor | None, int]:
+def _workspace(desc: _lib.ConvDesc, op: int, dtype: torch.dtype, device, given: torch.Tensor | None = None
+               ) -> tuple[torch.Tensor | None, int]:
+    """The workspace of one launch: ``given`` when the caller brought one (checked for size), else a new one."""
     nbytes = int(_lib.load().jg_conv_workspace_bytes(desc, op, _lib.dtype_code(dtype)))
     if nbytes == 0:
         return None, 0
+    if given is not None:
+        if given.device != torch.device(device) or not given.is_contiguous() or given.numel() * given.element_size() < nbytes:
+            raise ValueError(f"workspace: needs {nbytes} contiguous bytes on {device}")
+        return given, nbytes
     return torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes
+
+
+def _out_tensor(out: torch.Tensor | None, shape, dtype: torch.dtype, device, what: str) -> torch.Tensor:
+    """``out`` when given (shape, dtype and layout checked), else a new tensor."""
+    if out is None:
+        return torch.empty(shape, dtype=dtype, device=device)
+    if tuple(out.shape) != tuple(shape) or out.dtype != dtype or out.device != torch.device(device) or not out.is_contiguous():
+        raise ValueError(f"{what}: `out` must be a contiguous {dtype} tensor of shape {tuple(shape)} on {device}")
+    return out
 
 
 def _check_args(x_like, w, groups, padding):
@@ -358,9 +373,33 @@ def _stuffed(g: torch.Tensor, dense_sp, stride) -> torch.Tensor:
     return up
 
 
-def conv_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1) -> torch.Tensor:
-    """``F.conv{1,2,3}d(x, w, b, stride, padding, dilation, groups)`` on the HIP kernels."""
+def _single_launch(dtype, c_in, weight_shape, stride, padding, dilation, groups) -> bool:
+    """True where conv_nd / conv_nd_weight hand the tensors to the C entry point as they are (no route that
+    re-shapes the layer, copies channel slices or lays out patches first)."""
+    n = len(weight_shape) - 2
+    kernel = tuple(int(k) for k in weight_shape[2:])
+    stride, padding, dilation = _tup(stride, n, "stride"), _tup(padding, n, "padding"), _tup(dilation, n, "dilation")
+    if groups != 1:
+        return not _per_group_ok(groups, int(weight_shape[1]), int(weight_shape[0]) // groups, n)
+    if _dense_stride_ok(kernel, stride, dilation, padding) or _prepad(kernel, stride, padding, dilation) is not None:
+        return False
+    if _dilated_ok(kernel, stride, padding, dilation) or _big_kernel_ok(kernel, stride, dilation):
+        return False
+    if _embed3(kernel, stride, dilation) is not None:
+        return False
+    return not _patch_gemm_ok(dtype, c_in, int(weight_shape[0]), kernel, stride, padding, dilation)
+
+
+def conv_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1, out=None, workspace=None) -> torch.Tensor:
+    """``F.conv{1,2,3}d(x, w, b, stride, padding, dilation, groups)`` on the HIP kernels.
+
+    ``out`` / ``workspace`` (the result tensor and ``jg_conv_workspace_bytes`` bytes of scratch) let a caller
+    that runs the same layer again and again bring its own buffers, so that the call allocates nothing; they
+    are honoured where the layer runs as one launch on the given tensors and refused on the routes that
+    re-shape the layer first."""
     _lib.require_gpu(x, w, b)
+    if (out is not None or workspace is not None) and not _single_launch(x.dtype, x.shape[1], w.shape, stride, padding, dilation, groups):
+        raise NotImplementedError("conv_nd: `out` / `workspace` are taken only where the layer is one launch on the given tensors")
     n = _check_args(x, w, groups, padding)
     if x.dim() != n + 2:
         raise ValueError(f"expected a batched (N, C, *spatial) input with {n} spatial axes, got {tuple(x.shape)}")
@@ -401,9 +440,9 @@ def conv_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1) -> torch
     if plain and _patch_gemm_ok(x.dtype, x.shape[1], w.shape[0], w.shape[2:], stride, padding, dilation):
         y_tok = _proj_nt(_patchify(x, w.shape[2:], out_sp), w.reshape(w.shape[0], -1), b)
         return y_tok.reshape(x.shape[0], *out_sp, w.shape[0]).permute(0, n + 1, *range(1, n + 1)).contiguous()
-    y = torch.empty((x.shape[0], w.shape[0], *out_sp), dtype=x.dtype, device=x.device)
+    y = _out_tensor(out, (x.shape[0], w.shape[0], *out_sp), x.dtype, x.device, "conv_nd")
     desc = _desc(x.shape[0], x.shape[1], w.shape[0], x.shape[2:], w.shape[2:], stride, padding, dilation, groups)
-    ws, nbytes = _workspace(desc, 0, x.dtype, x.device)
+    ws, nbytes = _workspace(desc, 0, x.dtype, x.device, workspace)
     rc = _lib.load().jg_conv_fwd(
         _lib.ptr(y), _lib.ptr(x), _lib.ptr(w), _lib.ptr(b), desc, _lib.dtype_code(x.dtype), _lib.ptr(ws), nbytes,
         _lib.stream_ptr(x.device),
@@ -565,7 +604,8 @@ def conv_nd_weight_framed(x_frame, x_tile, geom: HaloGeometry, weight_shape, g, 
     return (gw, gb) if with_bias_grad else gw
 
 
-def conv_nd_input_fold(geom: HaloGeometry, w, g, *, stride=1, padding=0, dilation=1, groups=1, present=None):
+def conv_nd_input_fold(geom: HaloGeometry, w, g, *, stride=1, padding=0, dilation=1, groups=1, present=None,
+                       out=None, workspace=None):
     """Input gradient of the convolution on the halo-padded tile, written to its owners.
 
     Equivalent to ``conv_nd_input`` on the padded shape followed by
@@ -574,7 +614,8 @@ def conv_nd_input_fold(geom: HaloGeometry, w, g, *, stride=1, padding=0, dilatio
     cell and ``send[offset]`` is the halo block owned by that neighbour (only the
     offsets in ``present``, all by default). ``halo_fold_border_`` finishes the fold
     once the neighbours' blocks have arrived. Returns ``None`` where only the
-    unfused kernels cover the problem.
+    unfused kernels cover the problem. ``out = (gx, send)`` of an earlier call with the same
+    arguments and ``workspace`` are written again instead of new tensors.
     """
     _lib.require_gpu(w, g)
     n = _check_args(g, w, groups, padding)
@@ -595,11 +636,18 @@ def conv_nd_input_fold(geom: HaloGeometry, w, g, *, stride=1, padding=0, dilatio
             f"(expected {(batch, w.shape[0], *out_sp)})"
         )
     desc = _desc(batch, c_in, w.shape[0], padded, w.shape[2:], stride, padding, dilation, groups)
-    ws, nbytes = _workspace(desc, 1, g.dtype, g.device)
+    ws, nbytes = _workspace(desc, 1, g.dtype, g.device, workspace)
     lead = (batch, c_in)
     offs = geom.offsets() if present is None else [tuple(o) for o in present]
-    send, tab = new_strips(geom, "pack_bwd", lead, offs, g.dtype, g.device)
-    gx = torch.empty(lead + geom.size, dtype=g.dtype, device=g.device)
+    if out is None:
+        send, tab = new_strips(geom, "pack_bwd", lead, offs, g.dtype, g.device)
+        gx = torch.empty(lead + geom.size, dtype=g.dtype, device=g.device)
+    else:
+        gx, send = out
+        gx = _out_tensor(gx, lead + geom.size, g.dtype, g.device, "conv_nd_input_fold")
+        if set(send) != set(offs):
+            raise ValueError("conv_nd_input_fold: `out` holds strips for other offsets than `present`")
+        tab = strip_table(send, geom, "pack_bwd", lead, g)
     rc = _lib.load().jg_conv_dgrad_fold(
         _lib.ptr(gx), tab, _lib.ptr(w), _lib.ptr(g), desc, geom.c_geom(batch * c_in), _lib.dtype_code(g.dtype),
         _lib.ptr(ws), nbytes, _lib.stream_ptr(g.device),
@@ -610,15 +658,20 @@ def conv_nd_input_fold(geom: HaloGeometry, w, g, *, stride=1, padding=0, dilatio
     return gx, send
 
 
-def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, groups=1, with_bias_grad=False):
+def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, groups=1, with_bias_grad=False,
+                   out=None, workspace=None):
     """``torch.nn.grad.conv{1,2,3}d_weight(x, weight_shape, g, ...)`` on the HIP kernels.
 
     ``with_bias_grad=True`` returns ``(gw, gb)`` with ``gb = g.sum`` over batch and pixels
     (config.py:117-120), from the same pass over ``g`` where the MFMA kernel covers the shape.
+    ``out`` (``gw``, or ``(gw, gb)`` with the bias gradient) and ``workspace`` as for :func:`conv_nd`.
     """
     _lib.require_gpu(x, g)
     weight_shape = tuple(int(v) for v in weight_shape)
     n = len(weight_shape) - 2
+    if (out is not None or workspace is not None) and not _single_launch(x.dtype, x.shape[1], weight_shape, stride, padding, dilation, groups):
+        raise NotImplementedError("conv_nd_weight: `out` / `workspace` are taken only where the layer is one launch on the given tensors")
+    out_w, out_b = (out if with_bias_grad else (out, None)) if out is not None else (None, None)
     if isinstance(padding, str):
         raise NotImplementedError(f"string padding ({padding!r}) is not supported; pass per-axis integers")
     if not isinstance(groups, int) or groups < 1 or weight_shape[0] % groups:
@@ -696,12 +749,12 @@ def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, group
                 gb.zero_()
         gw = gw2.reshape(weight_shape)
         return (gw, gb) if with_bias_grad else gw
-    gw = torch.empty(weight_shape, dtype=x.dtype, device=x.device)
+    gw = _out_tensor(out_w, weight_shape, x.dtype, x.device, "conv_nd_weight")
     desc = _desc(x.shape[0], x.shape[1], weight_shape[0], x.shape[2:], weight_shape[2:], stride, padding, dilation, groups)
-    ws, nbytes = _workspace(desc, 2, x.dtype, x.device)
+    ws, nbytes = _workspace(desc, 2, x.dtype, x.device, workspace)
     if with_bias_grad:
         # one pass over g for both gradients where the MFMA kernel covers the shape
-        gb = torch.empty(weight_shape[0], dtype=x.dtype, device=x.device)
+        gb = _out_tensor(out_b, (weight_shape[0],), x.dtype, x.device, "conv_nd_weight (bias gradient)")
         rc = _lib.load().jg_conv_wgrad_bias(
             _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(x), _lib.ptr(g), desc, _lib.dtype_code(x.dtype), _lib.ptr(ws), nbytes,
             _lib.stream_ptr(x.device),
@@ -715,7 +768,8 @@ def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, group
     )
     _lib.check(rc, "jg_conv_wgrad")
     if with_bias_grad:
-        return gw, sum_grad_bias(g, n)
+        gb_sep = sum_grad_bias(g, n)
+        return gw, (gb_sep if out_b is None else out_b.copy_(gb_sep))
     return gw
 
 

@@ -335,12 +335,26 @@ def new_strips(geom: "HaloGeometry", verb: str, lead: tuple, offs: Sequence, dty
     return out, tab
 
 
+def strip_table(strips: Mapping[Offset, torch.Tensor], geom: "HaloGeometry", verb: str, lead: tuple, like: torch.Tensor) -> VoidP27:
+    """The pointer table for strips that exist already (what :func:`new_strips` returned on an earlier
+    call), each checked against the shape the geometry gives it."""
+    tab = VoidP27()
+    for o, t in strips.items():
+        want = tuple(lead) + geom.strip_extent(o, verb)
+        if tuple(t.shape) != want or t.dtype != like.dtype or t.device != like.device or not t.is_contiguous():
+            raise ValueError(f"strip {o}: expected a contiguous {like.dtype} tensor of shape {want} on {like.device}")
+        if t.numel():
+            tab[slot(o)] = t.data_ptr()
+    return tab
+
+
 def halo_pack(
     src: torch.Tensor,
     geom: HaloGeometry,
     *,
     from_padded: bool,
     present: Sequence[Offset] | None = None,
+    out: Mapping[Offset, torch.Tensor] | None = None,
 ) -> dict:
     """Cut the strips this rank sends, keyed by the neighbour's offset.
 
@@ -348,7 +362,8 @@ def halo_pack(
     neighbours need for their halos (forward). ``from_padded=True``: ``src`` is a
     padded tensor (the dgrad of the padded tile) and strips are its halo blocks,
     owned by the neighbours (backward). ``present`` limits the offsets to the
-    neighbours that exist.
+    neighbours that exist. ``out``: the strips of an earlier call with the same
+    arguments, filled again instead of new ones.
     """
     _lib.require_gpu(src)
     spatial = geom.padded if from_padded else geom.size
@@ -356,7 +371,12 @@ def halo_pack(
     lead = tuple(src.shape[: -geom.n_spatial])
     verb = "pack_bwd" if from_padded else "pack_fwd"
     offs = geom.offsets() if present is None else [tuple(o) for o in present]
-    out, tab = new_strips(geom, verb, lead, offs, src.dtype, src.device)
+    if out is None:
+        out, tab = new_strips(geom, verb, lead, offs, src.dtype, src.device)
+    else:
+        if set(out) != set(tuple(o) for o in offs):
+            raise ValueError("halo_pack: `out` holds strips for other offsets than `present`")
+        tab = strip_table(out, geom, verb, lead, src)
     # forward: the blocks are sized by the neighbours' halos of this tile
     cg = (geom if from_padded else geom.theirs()).c_geom(planes)
     rc = _lib.load().jg_halo_pack_3d(
@@ -441,4 +461,5 @@ __all__ = [
     "new_strips",
     "needed_input_span",
     "slot",
+    "strip_table",
 ]

@@ -34,7 +34,36 @@ def _nt(out, a, w, bias, rows, n_out, k_in, a_heads, out_heads, dims) -> None:
     _lib.check(rc, "jg_proj_nt")
 
 
-_remember_casts = True
+_remember_casts = False
+
+
+def remember_casts(on: bool = True) -> bool:
+    """Switch the remembering of parameter casts on or off for the process; returns the previous setting.
+
+    Off (the default), every forward casts the fp32 parameters to the compute dtype anew and every
+    backward transposes the saved cast: always right. On, the copies are kept on the parameter and reused
+    until the parameter changes, which saves a dozen small launches per Swin block step. A change is
+    recognised by the tensor's version counter (every in-place operation on the parameter itself, an
+    optimizer step included, bumps it) and by its storage address, device and dtype. A write through
+    ``param.data`` (``p.data.normal_()``, ``dist.broadcast(p.data, ...)``, an EMA swap that copies into
+    ``p.data``) bumps no counter and keeps the address: after such a write call :func:`invalidate_casts`
+    on the module or parameter, or leave remembering off."""
+    global _remember_casts
+    before, _remember_casts = _remember_casts, bool(on)
+    return before
+
+
+def invalidate_casts(*targets) -> None:
+    """Drop the remembered casts of the given parameters / tensors or of every parameter and buffer of the
+    given modules (after a write through ``.data``, which the version counter does not see)."""
+    for t in targets:
+        if isinstance(t, torch.nn.Module):
+            invalidate_casts(*t.parameters(), *t.buffers())
+        elif isinstance(t, torch.Tensor) and getattr(t, "_jg_casts", None) is not None:
+            try:
+                del t._jg_casts
+            except AttributeError:
+                pass
 
 
 @contextlib.contextmanager
@@ -49,12 +78,15 @@ def fresh_casts():
         _remember_casts = before
 
 
+def _cast_key(t: torch.Tensor) -> tuple:
+    return (t._version, t.data_ptr(), t.device, t.dtype, tuple(t.shape), tuple(t.stride()))
+
+
 def _cast_cached(t: torch.Tensor | None, dtype: torch.dtype, transposed: bool = False) -> torch.Tensor | None:
-    """``t`` in ``dtype``, contiguous (optionally its transpose), remembered on the tensor until
-    its next in-place update: under autocast the parameters are fp32 and every forward and
-    backward would otherwise launch a cast (and the input gradient a transpose copy) per layer.
-    The tensor's version counter, which every in-place update (an optimizer step) bumps,
-    invalidates the copies."""
+    """``t`` in ``dtype``, contiguous (optionally its transpose). With :func:`remember_casts` on, the copy is
+    kept on the tensor until its version counter, storage address, device, dtype or layout changes: under
+    autocast the parameters are fp32 and every forward and backward would otherwise launch a cast (and the
+    input gradient a transpose copy) per layer."""
     if t is None:
         return None
     if not transposed and t.dtype == dtype and t.is_contiguous():
@@ -64,8 +96,9 @@ def _cast_cached(t: torch.Tensor | None, dtype: torch.dtype, transposed: bool = 
         return (src.t() if transposed else src).to(dtype).contiguous()
     key = (dtype, transposed)
     cache = getattr(t, "_jg_casts", None)
-    if cache is None or cache[0] != t._version:
-        cache = (t._version, {})
+    stamp = _cast_key(t)
+    if cache is None or cache[0] != stamp:
+        cache = (stamp, {})
         try:
             t._jg_casts = cache
         except AttributeError:  # a tensor subclass without a __dict__: no cache
@@ -79,10 +112,10 @@ def _cast_cached(t: torch.Tensor | None, dtype: torch.dtype, transposed: bool = 
 
 
 def _transposed(ctx, w: torch.Tensor) -> torch.Tensor:
-    """The transposed weight of the input-gradient GEMM: the cached copy of the parameter when
-    the parameter is still the one the forward saw, else a transpose of the saved cast."""
+    """The transposed weight of the input-gradient GEMM: the remembered copy of the parameter when casts
+    are remembered and the parameter is still the one the forward saw, else a transpose of the saved cast."""
     ref = getattr(ctx, "weight_ref", None)
-    if ref is not None and ref._version == ctx.weight_version:
+    if _remember_casts and ref is not None and ref._version == ctx.weight_version:
         return _cast_cached(ref, w.dtype, transposed=True)
     return w.t().contiguous()
 
@@ -319,7 +352,7 @@ class _GeluMlp(torch.autograd.Function):
 
         def transposed(i, wc):
             ref, version = ctx.refs[i]
-            return _cast_cached(ref, wc.dtype, transposed=True) if ref._version == version else wc.t().contiguous()
+            return _cast_cached(ref, wc.dtype, transposed=True) if _remember_casts and ref._version == version else wc.t().contiguous()
 
         gw2, gb2 = _tn(g, act, rows, n_out, hid, False, False, (1, 1, 1, 1), dt_b2 is not None,
                        _grad_dtype(g.dtype, (dt_w2, dt_b2)))
@@ -356,4 +389,4 @@ def heads_projection(out: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor
     return _HeadsProjection.apply(out, weight, bias)
 
 
-__all__ = ["gelu_mlp", "heads_projection", "linear", "mlp_fusable", "qkv_projection"]
+__all__ = ["gelu_mlp", "heads_projection", "invalidate_casts", "linear", "mlp_fusable", "qkv_projection", "remember_casts"]
