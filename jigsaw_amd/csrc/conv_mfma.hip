@@ -281,7 +281,15 @@ __device__ inline void store_f32(const void* base, uint32_t lane_off, float v) {
 
 // F16: the 16-bit tensors hold fp16 instead of bf16 (v_mfma_f32_32x32x16_f16; everything else moves
 // 16-bit values without looking at them, the epilogue converts by out_kind).
-template <int MT, bool EVEN, bool FOLD, bool FRAMED, bool F16 = false>  // MT = produced channels per workgroup: 32 or 64
+// PX: the MFMA operands are exchanged, D[pixel][channel] instead of D[channel][pixel]: an accumulator lane
+// then owns ONE produced channel and 16 pixels, 8 consecutive ones per lane half and register octet, so that
+// a lane's results are whole 16-byte pieces of an output row and leave straight from the registers. The rows
+// of the pixel operand are dealt to the pixels with bits 2 and 3 of the row number exchanged (row 8j + 4h + t
+// of the result lies in lane half h, register 4j + t; pixel 16 (j / 2) + 8 h + 4 (j % 2) + t goes there).
+// Used where every row segment of the result is made of whole, aligned 16-byte pieces.
+__device__ __forceinline__ int px_of_row(int m) { return (m & 0x13) | ((m & 4) << 1) | ((m & 8) >> 1); }
+
+template <int MT, bool EVEN, bool FOLD, bool FRAMED, bool F16 = false, bool PX = false>  // MT = produced channels per workgroup: 32 or 64
 __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips, FwdParams p) {
   constexpr int CB = MT / 32;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -580,7 +588,7 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
   };
   auto compute_kw = [&](int buf, int wstep, int kw, int wstep_next) {  // wstep: the stage's step inside its weight group
     const u32x4* in = lds_in + buf * STAGE_SLOTS + kg * (IN_ROWS * ROW_SLOTS) + wrow0 * ROW_SLOTS;
-    const int col0 = wcol0 + ln + p.lead;  // the tile's pixel 0 sits `lead` slots into the staged row
+    const int col0 = wcol0 + (PX ? px_of_row(ln) : ln) + p.lead;  // the tile's pixel 0 sits `lead` slots into the staged row
     const u32x4* inb = in + in_slot(col0 + kw);
     if (kw == 0) {
       if (a_step != wstep) {  // wave-uniform: the first stage, after a tile without work, after a weight reload
@@ -605,9 +613,14 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
         if (r >= 0 && r < WROWS) {
 #pragma unroll
           for (int cb = 0; cb < CB; ++cb)
-            if (F16)
+            if (F16 && PX)
+              acc[cb][r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, b),
+                                                                  __builtin_bit_cast(f16x8, a[kh][cb]), acc[cb][r], 0, 0, 0);
+            else if (F16)
               acc[cb][r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[kh][cb]),
                                                                   __builtin_bit_cast(f16x8, b), acc[cb][r], 0, 0, 0);
+            else if (PX)
+              acc[cb][r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, a[kh][cb], acc[cb][r], 0, 0, 0);
             else
               acc[cb][r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kh][cb], b, acc[cb][r], 0, 0, 0);
         }
@@ -631,6 +644,17 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
   // Accumulator lane (ln, kg), register i of block cb: produced channel
   // cb*32 + 8*(i/4) + 4*kg + i%4, pixel column wcol0 + ln.
   auto init_acc = [&]() {
+    if (PX) {  // a lane owns one channel per block
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) {
+        const float bv = lds_bias[cb * 32 + ln];
+#pragma unroll
+        for (int r = 0; r < WROWS; ++r)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[cb][r][i] = bv;
+      }
+      return;
+    }
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
@@ -683,6 +707,60 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     for (int q = 0; q < MT / 16; ++q) piece[q] = *reinterpret_cast<const u32x4*>(scratch + (q * 64 + lane) * 16);
 #pragma unroll
     for (int q = 0; q < MT / 16; ++q) store_16_bytes(ytile + (size_t)q * 16 * chan_bytes, voff, piece[q]);
+  };
+
+  // PX layout: lane (ln, kg) holds channel cb * 32 + ln; registers 8 J .. 8 J + 7 hold the pixels
+  // wcol0 + 16 J + 8 kg + (0 .. 7) of the wavefront's row: one 16-byte piece of 16-bit results.
+  auto piece_16bit = [&](int cb, int r, int J) {
+    u32x4 v;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      f32x2 v2 = {acc[cb][r][8 * J + 2 * d], acc[cb][r][8 * J + 2 * d + 1]};
+      v[d] = F16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, f16x2))
+                 : __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
+    }
+    return v;
+  };
+  // A row of the wavefront (32 pixels x MT channels of 16-bit results) goes through LDS once, as 16-byte
+  // pieces both ways: lane (channel ln, half kg) writes its pieces 2 J + kg of channels cb * 32 + ln, then
+  // lane l reads piece l % 4 of channel 16 q + l / 4, so that four neighbouring lanes store 64 contiguous
+  // bytes of one channel row. A channel's four pieces sit in one 64-byte LDS row, at slot piece ^ (channel / 4 % 4):
+  // the 16 lanes of a write (consecutive channels, one piece) and of a read (four channels, all pieces)
+  // then each cover all 64 banks once. `scratch`: 64 * MT bytes of LDS of this wavefront.
+  auto epilogue_px = [&](const TileCoord& tc, int free_buf) {
+    const int tw0 = tc.tw * TW + p.org_w;
+    const size_t chan_bytes = 2 * ochan;
+    unsigned char* scratch = reinterpret_cast<unsigned char*>(lds_in + free_buf * STAGE_SLOTS) + wave * (STAGE_BYTES / WAVES);
+    // wave-uniform base: the tile's first column in produced channel mt * MT, row 0 (it may lie before
+    // the row where the tile grid starts left of the tensor; such pieces are not stored)
+    char* ytile = reinterpret_cast<char*>(p.y) +
+                  2 * ((ptrdiff_t)(((size_t)tc.n * p.M + (size_t)mt * MT) * ochan + (size_t)tc.od * plane_o) + (ptrdiff_t)tw0);
+    const int m_left = p.M - mt * MT;
+    const int l4 = lane >> 2, pc = lane & 3;  // reading side: channel 16 q + l4, piece pc
+    const int px = tw0 + wcol0 + 8 * pc;
+    const bool px_ok = px >= 0 && px + 8 <= p.Wout;
+    const uint32_t lane_off = (uint32_t)(l4 * chan_bytes) + 2u * (uint32_t)(wcol0 + 8 * pc);
+    unsigned char* wr = scratch + ln * 64;
+    const unsigned char* rd = scratch + l4 * 64 + ((pc ^ ((l4 >> 2) & 3)) << 4);
+    const int wsw = (ln >> 2) & 3;
+#pragma unroll
+    for (int r = 0; r < WROWS; ++r) {
+      const int oh = tc.th * TH + wrow0 + r;
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int J = 0; J < 2; ++J)
+          *reinterpret_cast<u32x4*>(wr + cb * 32 * 64 + (((2 * J + kg) ^ wsw) << 4)) = piece_16bit(cb, r, J);
+      u32x4 piece[MT / 16];
+#pragma unroll
+      for (int q = 0; q < MT / 16; ++q) piece[q] = *reinterpret_cast<const u32x4*>(rd + q * 16 * 64);
+      if (oh < p.Hout) {
+        const uint32_t row_off = lane_off + 2u * (uint32_t)oh * (uint32_t)p.Wout;
+#pragma unroll
+        for (int q = 0; q < MT / 16; ++q)
+          if (px_ok && q * 16 + l4 < m_left) store_16_bytes(ytile + (size_t)q * 16 * chan_bytes, row_off, piece[q]);
+      }
+    }
   };
 
   auto epilogue_rows = [&](const TileCoord& tc, auto ragged, int free_buf) {
@@ -750,7 +828,8 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     }
   };
   auto epilogue = [&](const TileCoord& tc, int free_buf) {
-    if ((mt + 1) * MT <= p.M) epilogue_rows(tc, std::false_type{}, free_buf);
+    if (PX) epilogue_px(tc, free_buf);
+    else if ((mt + 1) * MT <= p.M) epilogue_rows(tc, std::false_type{}, free_buf);
     else epilogue_rows(tc, std::true_type{}, free_buf);
   };
 
@@ -895,7 +974,8 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
         compute_kw(buf, wstep, 0, wstep_next);
         compute_kw(buf, wstep, 1, wstep_next);
       }
-      if (c16 == 0 && ti > 0) __syncthreads();  // the buffer written next was the last epilogue's scratch
+      // the buffer written next was the last epilogue's scratch
+      if (c16 == 0 && ti > 0) __syncthreads();
       if (q + 1 < stages) store_stage(buf ^ 1, q + 1);  // other buffer: no hazard with this stage's reads
       if (q + 2 < stages) issue_stage();
       if (live) compute_kw(buf, wstep, 2, wstep_next);
@@ -1106,6 +1186,19 @@ int launch_conv(const Launch& L, void* ws, size_t ws_bytes, hipStream_t s, const
   } else if (L.xt != nullptr) {
     if (MT == 64) kern = even ? &conv3x3_mfma_kernel<64, true, false, true> : &conv3x3_mfma_kernel<64, false, false, true>;
     else kern = even ? &conv3x3_mfma_kernel<32, true, false, true> : &conv3x3_mfma_kernel<32, false, false, true>;
+  } else if (wide_rows && (reinterpret_cast<uintptr_t>(L.y) & 15) == 0) {
+    // every row segment of the result is whole, aligned 16-byte pieces: results leave from the registers
+    if (L.f16) {
+      if (MT == 64)
+        kern = even ? &conv3x3_mfma_kernel<64, true, false, false, true, true> : &conv3x3_mfma_kernel<64, false, false, false, true, true>;
+      else
+        kern = even ? &conv3x3_mfma_kernel<32, true, false, false, true, true> : &conv3x3_mfma_kernel<32, false, false, false, true, true>;
+    } else {
+      if (MT == 64)
+        kern = even ? &conv3x3_mfma_kernel<64, true, false, false, false, true> : &conv3x3_mfma_kernel<64, false, false, false, false, true>;
+      else
+        kern = even ? &conv3x3_mfma_kernel<32, true, false, false, false, true> : &conv3x3_mfma_kernel<32, false, false, false, false, true>;
+    }
   } else if (L.f16) {
     if (MT == 64)
       kern = even ? &conv3x3_mfma_kernel<64, true, false, false, true> : &conv3x3_mfma_kernel<64, false, false, false, true>;
