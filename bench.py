@@ -688,7 +688,8 @@ def profile_ring(reps: int = 3) -> None:
     dout = torch.randn(b, h, n, d, device=dev, generator=g).bfloat16()
     for _ in range(reps):
         out, l = ja.ring_forward(q, ks, vs, d**-0.5)
-        ja.ring_backward(dout, q, out, l, ks, vs, d**-0.5)
+        ja.ring_backward(dout, q, out, l, ks, vs, d**-0.5)  # one pass over the four chunks
+        ja.core_backward(dout, q, ks[0], vs[0], out, l, d**-0.5)  # one chunk by itself, for comparison
     torch.cuda.synchronize()
 
 

@@ -519,6 +519,19 @@ int jg_attn_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q,
                 const float* bias, int64_t bias_period, float* dbias, int dtype,
                 void* workspace, size_t workspace_bytes, void* stream);
 
+/* The backward loop of one rank's ring over n_chunks RESIDENT chunks in one call
+ * (_functional/backward.py:176-277 with the chunks the forward saved: step s takes chunk s):
+ * k[c], v[c] (batch, sk, d) are chunk c, dk[c], dv[c] receive this rank's partial for it (what
+ * jg_attn_bwd returns for that chunk), dq the sum of the per-chunk dq, accumulated in fp32 and
+ * rounded once (the reference adds the steps in q's dtype, backward.py:184, 269). k, v, dk, dv are
+ * HOST arrays of n_chunks device pointers, read before the call returns. No bias.
+ * Covered: bf16, d = 64, sq and sk multiples of 128, 1 <= n_chunks <= 16; JG_ERR_UNSUPPORTED
+ * otherwise (call jg_attn_bwd per chunk and add the dq). workspace as for jg_attn_bwd. */
+int jg_attn_bwd_chunks(void* dq, void* const* dk, void* const* dv, const void* dout, const void* q,
+                       const void* const* k, const void* const* v, int64_t n_chunks, const void* out,
+                       const float* lse, int64_t batch, int64_t sq, int64_t sk, int64_t d, float scale,
+                       int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Windowed attention of a Swin block on the token grid itself (examples/swin.py:129-170:
  * F.scaled_dot_product_attention over (B, nW, heads, 64, 32) windows with attn_mask = the
  * relative-position bias, index of examples/swin.py:99-104, plus the shift mask of 107-126).

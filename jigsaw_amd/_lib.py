@@ -214,6 +214,11 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
          c_int64, c_int64, c_float, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_size_t, c_void_p],
     ),
+    "jg_attn_bwd_chunks": (
+        c_int,
+        [c_void_p, POINTER(c_void_p), POINTER(c_void_p), c_void_p, c_void_p, POINTER(c_void_p), POINTER(c_void_p), c_int64,
+         c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_void_p, c_size_t, c_void_p],
+    ),
     "jg_attn_swin_fwd": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,

@@ -18,6 +18,7 @@ Host-side mirror of
 
 from __future__ import annotations
 
+import ctypes
 import math
 from collections.abc import Sequence
 
@@ -343,13 +344,60 @@ def ring_forward(q, k_chunks: Sequence[torch.Tensor], v_chunks: Sequence[torch.T
     return out.to(q.dtype), lse
 
 
+_MAX_CHUNKS_PER_CALL = 16
+
+
+def backward_chunks(dout, q, out, lse, k_chunks, v_chunks, scale):
+    """``(dq, [dk_j], [dv_j])`` over resident chunks in ONE pass (``jg_attn_bwd_chunks``): the dQ
+    kernel walks every chunk with dQ in its registers (one launch, one rounding), the dK/dV kernel
+    takes the chunk as a grid dimension. ``None`` where that entry point does not cover the call
+    (anything but bf16 at head size 64 with lengths that are multiples of 128, up to 16 chunks of
+    one shape)."""
+    P = len(k_chunks)
+    if not 1 <= P <= _MAX_CHUNKS_PER_CALL or len(v_chunks) != P:
+        return None
+    if q.dtype != torch.bfloat16 or q.shape[-1] != 64 or q.shape[-2] % 128 or k_chunks[0].shape[-2] % 128:
+        return None
+    if any(t.shape != k_chunks[0].shape or t.dtype != q.dtype or t.device != q.device for t in (*k_chunks, *v_chunks)):
+        return None
+    if k_chunks[0].shape[:-2] != q.shape[:-2] or not q.is_cuda:
+        return None
+    _lib.require_gpu(dout, q, out, lse)
+    dout, out, q = dout.to(q.dtype).contiguous(), out.to(q.dtype).contiguous(), q.contiguous()
+    lse = lse.to(torch.float32).contiguous()
+    ks = [t.contiguous() for t in k_chunks]
+    vs = [t.contiguous() for t in v_chunks]
+    batch, sq, d = _flat(q)
+    sk = int(ks[0].shape[-2])
+    dq = torch.empty_like(q)
+    # one allocation for all partials: chunk j's dK / dV are views of it
+    dkv = torch.empty((2, P) + tuple(ks[0].shape), dtype=q.dtype, device=q.device)
+    dks, dvs = list(dkv[0].unbind(0)), list(dkv[1].unbind(0))
+    lib = _lib.load()
+    nbytes = int(lib.jg_attn_bwd_workspace_bytes(batch, sq, sk, d))
+    ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=q.device)
+    arr = lambda ts: (ctypes.c_void_p * P)(*(t.data_ptr() for t in ts))  # noqa: E731
+    rc = lib.jg_attn_bwd_chunks(
+        _lib.ptr(dq), arr(dks), arr(dvs), _lib.ptr(dout), _lib.ptr(q), arr(ks), arr(vs), P, _lib.ptr(out), _lib.ptr(lse),
+        batch, sq, sk, d, float(scale), _lib.dtype_code(q.dtype), _lib.ptr(ws), nbytes, _lib.stream_ptr(q.device),
+    )
+    if rc == -2:
+        return None
+    _lib.check(rc, "jg_attn_bwd_chunks")
+    return dq, dks, dvs
+
+
 def ring_backward(dout, q, out, lse, k_chunks, v_chunks, scale):
     """``(dq, [dk_j], [dv_j])``: this rank's contribution to every chunk's gradient.
 
     ``dq`` accumulates over the chunks (backward.py:184, 269; here in fp32, cast to
     ``q.dtype`` at the end — the reference accumulates in ``q.dtype``); the sum of
-    dK/dV over the ranks that attended a chunk is the caller's collective."""
+    dK/dV over the ranks that attended a chunk is the caller's collective. Chunks that are all
+    resident go through one pass (:func:`backward_chunks`) where it covers them."""
     core = q.dtype
+    one_pass = backward_chunks(dout, q, out, lse, [t.to(core) for t in k_chunks], [t.to(core) for t in v_chunks], scale)
+    if one_pass is not None:
+        return one_pass
     dout, out = dout.to(core), out.to(core)
     dq = torch.zeros(q.shape, device=q.device, dtype=torch.float32)
     dks, dvs = [], []
@@ -483,6 +531,7 @@ def swin_grid_attention(q, k, v, table, side, grid):
 __all__ = [
     "attend_step_",
     "backward",
+    "backward_chunks",
     "core_backward",
     "core_forward",
     "forward",

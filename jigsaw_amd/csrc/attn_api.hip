@@ -23,6 +23,9 @@ size_t attn_mfma_bwd_workspace(long long batch, int sq, int sk);
 int attn_mfma_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q, const void* k,
                   const void* v, const void* out, const float* lse, long long batch, int sq,
                   int sk, float scale, void* ws, hipStream_t s);
+int attn_mfma_bwd_chunks(void* dq, void* const* dk, void* const* dv, const void* dout, const void* q,
+                         const void* const* k, const void* const* v, int nchunks, const void* out, const float* lse,
+                         long long batch, int sq, int sk, float scale, void* ws, hipStream_t s);
 bool attn_wide_supported(long long batch, int sq, int sk, int d, int dtype, bool has_bias);
 int attn_wide_fwd(void* out, float* lse, const void* q, const void* k, const void* v, long long batch,
                   int sq, int sk, int d, int dtype, float scale, float* out_acc, float* lse_acc,
@@ -152,4 +155,25 @@ extern "C" int jg_attn_bwd(void* dq, void* dk, void* dv, const void* dout, const
   return jg::attn_generic_bwd(dq, dk, dv, static_cast<float*>(workspace), dbias, dout, q, k, v, out,
                               lse, batch, (int)sq, (int)sk, (int)d, scale, bias, bias_period, dtype,
                               s);
+}
+
+extern "C" int jg_attn_bwd_chunks(void* dq, void* const* dk, void* const* dv, const void* dout, const void* q,
+                                  const void* const* k, const void* const* v, int64_t n_chunks, const void* out,
+                                  const float* lse, int64_t batch, int64_t sq, int64_t sk, int64_t d, float scale,
+                                  int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  const char* who = "jg_attn_bwd_chunks";
+  int rc = check_shape(who, batch, sq, sk, d, scale, dtype);
+  if (rc) return rc;
+  JG_REQUIRE(n_chunks >= 1, "%s: n_chunks must be at least 1", who);
+  JG_REQUIRE(dq && dk && dv && dout && q && k && v && out && lse, "%s: NULL pointer", who);
+  if (n_chunks > 16 || !jg::attn_mfma_bwd_supported(batch, (int)sq, (int)sk, (int)d, dtype, false))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "%s: bf16, d = 64, sq and sk multiples of 128 and at most 16 chunks", who);
+  for (int64_t c = 0; c < n_chunks; ++c)
+    JG_REQUIRE(k[c] && v[c] && dk[c] && dv[c], "%s: NULL pointer for chunk %lld", who, (long long)c);
+  if (batch == 0 || sq == 0) return JG_OK;
+  if (workspace == nullptr || workspace_bytes < jg_attn_bwd_workspace_bytes(batch, sq, sk, d))
+    JG_FAIL(JG_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", who, workspace_bytes,
+            jg_attn_bwd_workspace_bytes(batch, sq, sk, d));
+  return jg::attn_mfma_bwd_chunks(dq, dk, dv, dout, q, k, v, (int)n_chunks, out, lse, batch, (int)sq, (int)sk, scale,
+                                  workspace, static_cast<hipStream_t>(stream));
 }

@@ -28,6 +28,12 @@
 //   ds_read_b64_tr_b16 (within 16 lanes, lane i receives element i % 4 of the 8 bytes
 //   that lanes i / 4 + 4 j point at, j = 0..3), two reads of 4 consecutive rows each.
 //
+//   Several resident chunks in one pass (the ring backward from saved chunks,
+//   jigsaw/modules/attention/_functional/backward.py:176-277): the dQ kernel walks the key tiles of
+//   every chunk in turn with dQ in its registers (one launch, one rounding), and the chunk is a
+//   third grid dimension of the dK/dV kernel. The chunk pointers travel in the kernel-argument
+//   segment (first parameter), where a wavefront reads entry c with scalar loads.
+//
 // Reference behaviour restated here:
 //   jigsaw/modules/attention/_functional/cores/math.py:125-149
 #include "jg_common.h"
@@ -121,29 +127,52 @@ __device__ __forceinline__ bf16x8 pack8(const float* e) {
 struct BlockOf {
   long long bh;
   int blk;
+  int chunk;
 };
+// gridDim = (row blocks, batch entries, chunks). The flat order is (batch entry, chunk, block), so the
+// workgroups of one XCD's range stream the Q / dO (or K / V) of the same few batch entries.
 __device__ __forceinline__ BlockOf block_of() {
-  const unsigned nblk = gridDim.x, total = gridDim.x * gridDim.y;
-  unsigned id = blockIdx.y * gridDim.x + blockIdx.x;
+  const unsigned nblk = gridDim.x, nch = gridDim.z, total = gridDim.x * gridDim.y * gridDim.z;
+  unsigned id = (blockIdx.y * nch + blockIdx.z) * nblk + blockIdx.x;
   if ((total & 7u) == 0) id = (id & 7u) * (total >> 3) + (id >> 3);
   BlockOf b;
-  b.bh = id / nblk;
   b.blk = (int)(id % nblk);
+  id /= nblk;
+  b.chunk = (int)(id % nch);
+  b.bh = id / nch;
   return b;
+}
+
+constexpr int MAX_CHUNKS = 16;
+// Chunk c: k[c], v[c] (batch, sk, 64) and where its gradients go. FIRST kernel parameter: entry c is
+// read from the kernel-argument segment by its offset (a by-value struct indexed with a run-time
+// value would otherwise be copied to private memory lane by lane).
+struct ChunkTable {
+  const uint16_t* k[MAX_CHUNKS];
+  const uint16_t* v[MAX_CHUNKS];
+  uint16_t* dk[MAX_CHUNKS];
+  uint16_t* dv[MAX_CHUNKS];
+};
+__device__ __forceinline__ const char* chunk_entry(int which, int c) {  // which: 0 k, 1 v, 2 dk, 3 dv; c wave-uniform
+#if defined(__HIP_DEVICE_COMPILE__)
+  const char* const* kt = (const char* const*)__builtin_amdgcn_kernarg_segment_ptr();
+  return kt[which * MAX_CHUNKS + c];
+#else
+  (void)which; (void)c;
+  return nullptr;
+#endif
 }
 
 struct BwdArgs {
   const uint16_t* dout;
   const uint16_t* q;
-  const uint16_t* k;
-  const uint16_t* v;
   const uint16_t* out;
   const float* lse;
   float* delta;     // (batch, sq) workspace
   uint16_t* dq;
-  uint16_t* dk;
-  uint16_t* dv;
-  int sq, sk;
+  int sq, sk;       // sk: keys per chunk
+  int nchunks;
+  long long batch;
   float scale;
 };
 
@@ -158,7 +187,7 @@ constexpr int DQ_LDS = 2 * DQ_HALF;         // 131072 (and at least 4 x 32 x 64 
 #define JG_GROUP_MFMA 0x008
 #define JG_GROUP_DS_READ 0x100
 
-__global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
+__global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(ChunkTable chunks, BwdArgs p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -167,16 +196,21 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
   const BlockOf where = block_of();
   const long long b = where.bh;
   const int q0 = where.blk * BR + qb * 32;
+  // every chunk is cut in two key halves (one per wavefront group); a half's tiles of all chunks
+  // form one stream of ntiles tiles
   const int khalf = p.sk >> 1;
-  const int ntiles = khalf / BT;
+  const int tiles_per_chunk = khalf / BT;
+  const int ntiles = tiles_per_chunk * p.nchunks;
   const float c2 = p.scale * LOG2E;
   const long long qi = b * p.sq + q0 + ln;
 
   unsigned char* lds = smem + ks * DQ_HALF;
   // this wavefront moves rows 16 qb .. 16 qb + 15 of the K tile and of the V tile of its half
   const int ks_u = __builtin_amdgcn_readfirstlane(ks), qb_u = __builtin_amdgcn_readfirstlane(qb);
-  const char* kdma = reinterpret_cast<const char*>(p.k + (b * p.sk + (long long)ks_u * khalf) * D) + 16 * qb_u * ROWB;
-  const char* vdma = reinterpret_cast<const char*>(p.v + (b * p.sk + (long long)ks_u * khalf) * D) + 16 * qb_u * ROWB;
+  const long long half_off = 2 * ((b * p.sk + (long long)ks_u * khalf) * D) + 16 * qb_u * ROWB;  // bytes into a chunk
+  int ld_chunk = 0, ld_tile = 0;  // the load cursor: tiles are requested in stream order
+  const char* kdma = chunk_entry(0, 0) + half_off;
+  const char* vdma = chunk_entry(1, 0) + half_off;
   const uint32_t dma_off = dma_lane_offset(lane);
   const uint32_t lds_dma = lds_address(smem) + (uint32_t)(ks_u * DQ_HALF + 16 * qb_u * ROWB);
   const int tr_off[2] = {tr_lane_offset(lane, 0), tr_lane_offset(lane, 1)};
@@ -186,13 +220,19 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(BwdArgs p) {
   for (int c = 0; c < 4; ++c) row_off[c] = ln * ROWB + (((2 * c + kg) ^ (ln & 7)) << 4);
 
   // K and V of tile t straight into its buffer (free since the barrier that ended the tile before)
-  auto issue_loads = [&](int t) {
-    const long long off = (long long)t * NAT;
+  auto issue_loads = [&](int t) {  // called with t = 0, 1, 2, ... in turn
+    const long long off = (long long)ld_tile * NAT;
     const uint32_t dst = lds_dma + (uint32_t)((t & (NBUF - 1)) * DQ_BUF);
     dma_1k(kdma + off, dma_off, dst);
     dma_1k(kdma + off + 8 * ROWB, dma_off, dst + 8 * ROWB);
     dma_1k(vdma + off, dma_off, dst + NAT);
     dma_1k(vdma + off + 8 * ROWB, dma_off, dst + NAT + 8 * ROWB);
+    if (++ld_tile == tiles_per_chunk && ld_chunk + 1 < p.nchunks) {
+      ld_tile = 0;
+      ++ld_chunk;
+      kdma = chunk_entry(0, ld_chunk) + half_off;
+      vdma = chunk_entry(1, ld_chunk) + half_off;
+    }
   };
   auto tiles_landed = [&]() {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's transfers have landed
@@ -359,7 +399,7 @@ constexpr int DKV_SHARE = BT / DKV_KB;                // rows of a streamed tile
 static_assert(DKV_LDS >= DKV_KB * 64 * 64 * 4, "the hand-over of the partial dK / dV reuses the tile buffers");
 static_assert(64 * DKV_KB >= 2 * BT, "one thread of a half per statistic");
 
-__global__ __launch_bounds__(DKV_THREADS, 8 / (2 * DKV_KB) >= 2 ? 2 : 1) void attn_bwd_dkv_kernel(BwdArgs p) {
+__global__ __launch_bounds__(DKV_THREADS, 8 / (2 * DKV_KB) >= 2 ? 2 : 1) void attn_bwd_dkv_kernel(ChunkTable chunks, BwdArgs p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -411,8 +451,8 @@ __global__ __launch_bounds__(DKV_THREADS, 8 / (2 * DKV_KB) >= 2 ? 2 : 1) void at
 
   bf16x8 kf[4], vf[4];
   {
-    const uint16_t* krow = p.k + ki * D + 8 * kg;
-    const uint16_t* vrow = p.v + ki * D + 8 * kg;
+    const uint16_t* krow = reinterpret_cast<const uint16_t*>(chunk_entry(0, where.chunk)) + ki * D + 8 * kg;
+    const uint16_t* vrow = reinterpret_cast<const uint16_t*>(chunk_entry(1, where.chunk)) + ki * D + 8 * kg;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       kf[c] = lds_frag(reinterpret_cast<const unsigned char*>(krow + 16 * c));
@@ -512,6 +552,8 @@ __global__ __launch_bounds__(DKV_THREADS, 8 / (2 * DKV_KB) >= 2 ? 2 : 1) void at
   }
   __syncthreads();
   if (qs == 1) return;
+  uint16_t* dk_out = reinterpret_cast<uint16_t*>(const_cast<char*>(chunk_entry(2, where.chunk)));
+  uint16_t* dv_out = reinterpret_cast<uint16_t*>(const_cast<char*>(chunk_entry(3, where.chunk)));
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
@@ -523,8 +565,8 @@ __global__ __launch_bounds__(DKV_THREADS, 8 / (2 * DKV_KB) >= 2 ? 2 : 1) void at
         c[e] = dv[nb][4 * j + e] + xo[(32 + nb * 16 + 4 * j + e) * 64 + lane];
       }
       const int col = nb * 32 + 8 * j + 4 * kg;
-      *reinterpret_cast<bf16x4*>(p.dk + ki * D + col) = __builtin_convertvector(a, bf16x4);
-      *reinterpret_cast<bf16x4*>(p.dv + ki * D + col) = __builtin_convertvector(c, bf16x4);
+      *reinterpret_cast<bf16x4*>(dk_out + ki * D + col) = __builtin_convertvector(a, bf16x4);
+      *reinterpret_cast<bf16x4*>(dv_out + ki * D + col) = __builtin_convertvector(c, bf16x4);
     }
 }
 
@@ -541,22 +583,32 @@ size_t attn_mfma_bwd_workspace(long long batch, int sq, int) {
   return (size_t)batch * sq * sizeof(float);
 }
 
-int attn_mfma_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q, const void* k,
-                  const void* v, const void* out, const float* lse, long long batch, int sq,
-                  int sk, float scale, void* ws, hipStream_t s) {
+// The ring backward over `nchunks` resident chunks: k[c], v[c] in, dk[c], dv[c] out, dq = the sum over
+// the chunks, rounded once. nchunks = 1 is the plain backward of one chunk.
+int attn_mfma_bwd_chunks(void* dq, void* const* dk, void* const* dv, const void* dout, const void* q,
+                         const void* const* k, const void* const* v, int nchunks, const void* out, const float* lse,
+                         long long batch, int sq, int sk, float scale, void* ws, hipStream_t s) {
+  if (nchunks < 1 || nchunks > MAX_CHUNKS)
+    JG_FAIL(JG_ERR_UNSUPPORTED, "jg_attn_bwd_chunks: 1 to %d chunks a call, got %d", MAX_CHUNKS, nchunks);
+  ChunkTable tab;
+  for (int c = 0; c < MAX_CHUNKS; ++c) {
+    const int u = c < nchunks ? c : 0;
+    tab.k[c] = static_cast<const uint16_t*>(k[u]);
+    tab.v[c] = static_cast<const uint16_t*>(v[u]);
+    tab.dk[c] = static_cast<uint16_t*>(dk[u]);
+    tab.dv[c] = static_cast<uint16_t*>(dv[u]);
+  }
   BwdArgs a;
   a.dout = static_cast<const uint16_t*>(dout);
   a.q = static_cast<const uint16_t*>(q);
-  a.k = static_cast<const uint16_t*>(k);
-  a.v = static_cast<const uint16_t*>(v);
   a.out = static_cast<const uint16_t*>(out);
   a.lse = lse;
   a.delta = static_cast<float*>(ws);
   a.dq = static_cast<uint16_t*>(dq);
-  a.dk = static_cast<uint16_t*>(dk);
-  a.dv = static_cast<uint16_t*>(dv);
   a.sq = sq;
   a.sk = sk;
+  a.nchunks = nchunks;
+  a.batch = batch;
   a.scale = scale;
   static bool attr_set = false;
   if (!attr_set) {
@@ -568,11 +620,17 @@ int attn_mfma_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q,
       JG_FAIL(JG_ERR_LAUNCH, "jg_attn_bwd: cannot reserve LDS");
     attr_set = true;
   }
-  attn_bwd_dq_kernel<<<dim3((unsigned)(sq / BR), (unsigned)batch, 1), THREADS, DQ_LDS, s>>>(a);
+  attn_bwd_dq_kernel<<<dim3((unsigned)(sq / BR), (unsigned)batch, 1), THREADS, DQ_LDS, s>>>(tab, a);
   JG_CHECK_LAUNCH("jg_attn_bwd(dq)");
-  attn_bwd_dkv_kernel<<<dim3((unsigned)(sk / DKV_ROWS), (unsigned)batch, 1), DKV_THREADS, DKV_LDS, s>>>(a);
+  attn_bwd_dkv_kernel<<<dim3((unsigned)(sk / DKV_ROWS), (unsigned)batch, (unsigned)nchunks), DKV_THREADS, DKV_LDS, s>>>(tab, a);
   JG_CHECK_LAUNCH("jg_attn_bwd(dkv)");
   return JG_OK;
+}
+
+int attn_mfma_bwd(void* dq, void* dk, void* dv, const void* dout, const void* q, const void* k,
+                  const void* v, const void* out, const float* lse, long long batch, int sq,
+                  int sk, float scale, void* ws, hipStream_t s) {
+  return attn_mfma_bwd_chunks(dq, &dk, &dv, dout, q, &k, &v, 1, out, lse, batch, sq, sk, scale, ws, s);
 }
 
 }  // namespace jg

@@ -948,6 +948,7 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     issue_loads();
     cursor_advance();
   };
+  const bool stage_early = __builtin_amdgcn_readfirstlane(wave) == 4 || __builtin_amdgcn_readfirstlane(wave) == 5;
   int buf = 0;
   cursor_enter(0);
   issue_stage();
@@ -970,14 +971,25 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
         __syncthreads();
       }
       const int wstep_next = wstep + 1 == p.wc16 ? 0 : wstep + 1;
+      // Wavefronts 4 and 5 hold staging tasks like wavefronts 0..3 and share SIMD 0 and 1 with two of them.
+      // They stage at the head of the stage, while their SIMD's other wavefront multiplies, and that one
+      // stages later, while they multiply; done at the same point, the two leave the matrix core idle.
+      // (Not in a tile's first stage: the buffer is the last epilogue's scratch until the barrier below.)
+      const bool stage_now = stage_early && !(c16 == 0 && ti > 0);
+      if (stage_now) {
+        if (q + 1 < stages) store_stage(buf ^ 1, q + 1);
+        if (q + 2 < stages) issue_stage();
+      }
       if (live) {
         compute_kw(buf, wstep, 0, wstep_next);
         compute_kw(buf, wstep, 1, wstep_next);
       }
       // the buffer written next was the last epilogue's scratch
       if (c16 == 0 && ti > 0) __syncthreads();
-      if (q + 1 < stages) store_stage(buf ^ 1, q + 1);  // other buffer: no hazard with this stage's reads
-      if (q + 2 < stages) issue_stage();
+      if (!stage_now) {
+        if (q + 1 < stages) store_stage(buf ^ 1, q + 1);  // other buffer: no hazard with this stage's reads
+        if (q + 2 < stages) issue_stage();
+      }
       if (live) compute_kw(buf, wstep, 2, wstep_next);
       __syncthreads();
       buf ^= 1;

@@ -54,7 +54,7 @@ from typing import Any
 
 import torch
 
-from .attention import attend_step_, core_backward
+from .attention import attend_step_, backward_chunks, core_backward
 
 HopFn = Callable[..., "tuple[torch.Tensor, Any]"]
 
@@ -203,6 +203,18 @@ class RingSeat:
         if self.save_scope == "global":
             if len(saved) != P:
                 raise ValueError(f"expected the {P} chunks the forward saved, got {len(saved)}")
+            # every chunk is resident: one pass over all of them where the kernels cover it
+            one_pass = backward_chunks(dout, q, out, lse, [c[0].to(core) for c in saved], [c[1].to(core) for c in saved], scale)
+            if one_pass is not None:
+                dq_all, dks, dvs = one_pass
+                dk_own = dv_own = None
+                for s in range(P):
+                    dk_j, dv_j = dks[s], dvs[s]
+                    if self._reduce is not None:
+                        dk_j, dv_j = self._reduce(dk_j, dv_j, s)
+                    if s == self.rank:
+                        dk_own, dv_own = dk_j, dv_j
+                return dq_all, dk_own, dv_own
             dk_own = dv_own = None
             for s, (ks, vs) in enumerate(saved):
                 dq_j, dk_j, dv_j = core_backward(dout, q, ks.to(core), vs.to(core), out, lse, scale)

@@ -323,6 +323,48 @@ def test_config4_backward_shape_properties(dev):
         assert rel_l2(dks[j][:, :, keys], want_dk) < 2e-2, f"dk chunk {j}: {rel_l2(dks[j][:, :, keys], want_dk):.3e}"
 
 
+@pytest.mark.parametrize("b,h,n,nk,P", [(1, 2, 256, 128, 3), (2, 3, 128, 384, 1), (1, 8, 512, 256, 5), (1, 1, 128, 128, 16)])
+def test_backward_over_resident_chunks_in_one_pass(b, h, n, nk, P, dev):
+    """``backward_chunks`` (one dQ launch over all chunks, the chunk as a grid dimension of the dK/dV
+    kernel): dK / dV of every chunk have the bits of the per-chunk ``core_backward`` (same kernel, same
+    arithmetic per chunk), dQ is the fp32 sum of the chunks rounded once, checked against fp64
+    (backward.py:176-277 visits chunk s at step s and adds the steps' dq)."""
+    torch.manual_seed(11)
+    d = 64
+    scale = d**-0.5
+    q = (torch.randn(b, h, n, d, device=dev) / 4).bfloat16()
+    ks = [torch.randn(b, h, nk, d, device=dev).bfloat16() for _ in range(P)]
+    vs = [torch.randn(b, h, nk, d, device=dev).bfloat16() for _ in range(P)]
+    dout = torch.randn(b, h, n, d, device=dev).bfloat16()
+    out, lse = ja.ring_forward(q, ks, vs, scale, rank=0)
+    res = ja.backward_chunks(dout, q, out, lse, ks, vs, scale)
+    assert res is not None, "bf16 at head size 64 with lengths in multiples of 128 is what the one-pass kernels cover"
+    dq, dks, dvs = res
+    want_dq = torch.zeros(q.shape, dtype=torch.float64)
+    for j in range(P):
+        dq_j, dk_j, dv_j = ja.core_backward(dout, q, ks[j], vs[j], out, lse, scale)
+        assert torch.equal(dks[j], dk_j) and torch.equal(dvs[j], dv_j), f"chunk {j}"
+        ref = oa.core_backward(dout.double().cpu(), q.double().cpu(), ks[j].double().cpu(), vs[j].double().cpu(),
+                                        out.double().cpu(), lse.double().cpu(), scale)
+        want_dq += ref[0]
+        assert rel_l2(dk_j, ref[1]) < 2e-2 and rel_l2(dv_j, ref[2]) < 2e-2
+    assert rel_l2(dq, want_dq) < 2e-2, f"dq {rel_l2(dq, want_dq):.3e}"
+    # and through ring_backward, which takes this route by itself
+    dq2, dks2, dvs2 = ja.ring_backward(dout, q, out, lse, ks, vs, scale)
+    assert torch.equal(dq2, dq) and all(torch.equal(a, c) for a, c in zip(dks2, dks))
+
+
+def test_backward_over_chunks_declines_what_it_does_not_cover(dev):
+    q = torch.randn(1, 1, 128, 64, device=dev)
+    k = [torch.randn(1, 1, 128, 64, device=dev)]
+    assert ja.backward_chunks(q, q, q, q[..., 0], k, k, 0.125) is None  # fp32
+    qb = q.bfloat16()
+    kb = [torch.randn(1, 1, 96, 64, device=dev).bfloat16()]
+    assert ja.backward_chunks(qb, qb, qb, q[..., 0], kb, kb, 0.125) is None  # 96 keys
+    many = [torch.randn(1, 1, 128, 64, device=dev).bfloat16() for _ in range(17)]
+    assert ja.backward_chunks(qb, qb, qb, q[..., 0], many, many, 0.125) is None  # more chunks than a call takes
+
+
 def test_window_attention_with_bias_and_mask(dev):
     """Swin-style windows: (B, nW, heads, N, d) with a (nW, heads, N, N) bias that
     holds -inf entries (shift mask), forward and backward incl. the bias gradient."""
