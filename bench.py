@@ -254,10 +254,36 @@ def attention_figures(dev, iters: int) -> dict:
     ms_ln = time_gpu(lambda: jl.partial_stats(x), iters)
     # the same statistics on a shard that fills the chip (2 ** 18 rows of the same local width), over six
     # different 134 MB tensors in turn: one alone would stay in the 256 MB last-level cache and the
-    # figure would not be an HBM rate
-    xls = [torch.randn(1 << 18, 256, device=dev, generator=g).bfloat16() for _ in range(6)]
+    # figure would not be an HBM rate. The C entry points are called on buffers made once, so that the
+    # host's share of such short kernels (two allocations a call) stays out of the figure.
+    from jigsaw_amd import _lib
+
+    lib = _lib.load()
+    big_rows, cols = 1 << 18, 256
+    xls = [torch.randn(big_rows, cols, device=dev, generator=g).bfloat16() for _ in range(6)]
+    mean_b, var_b = torch.empty(big_rows, device=dev), torch.empty(big_rows, device=dev)
+    bf16 = _lib.dtype_code(torch.bfloat16)
     turn = itertools.count()
-    ms_ln_big = time_gpu(lambda: jl.partial_stats(xls[next(turn) % len(xls)]), max(iters, 2 * len(xls)), warmup=len(xls))
+
+    def stats_fwd():
+        t = xls[next(turn) % len(xls)]
+        _lib.check(lib.jg_ln_partial_fwd(_lib.ptr(mean_b), _lib.ptr(var_b), _lib.ptr(t), big_rows, cols, bf16,
+                                         _lib.stream_ptr(dev)), "jg_ln_partial_fwd")
+
+    ms_ln_big = time_gpu(stats_fwd, max(iters, 2 * len(xls)), warmup=len(xls))
+    # the backward's partial sums over g and x_hat (two tensors read, column partials for the weight / bias gradient)
+    w_ln = torch.ones(cols, device=dev, dtype=torch.bfloat16)
+    gw_b, gb_b = torch.empty(cols, device=dev), torch.empty(cols, device=dev)
+    ws_bytes = int(lib.jg_ln_bwd_workspace_bytes(big_rows, cols))
+    ws_ln = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+
+    def stats_bwd():
+        i = next(turn) % (len(xls) // 2)
+        _lib.check(lib.jg_ln_partial_bwd(_lib.ptr(mean_b), _lib.ptr(var_b), _lib.ptr(gw_b), _lib.ptr(gb_b), _lib.ptr(xls[2 * i]),
+                                         _lib.ptr(xls[2 * i + 1]), _lib.ptr(w_ln), big_rows, cols, bf16, _lib.ptr(ws_ln), ws_bytes,
+                                         _lib.stream_ptr(dev)), "jg_ln_partial_bwd")
+
+    ms_ln_bwd = time_gpu(stats_bwd, max(iters, 2 * len(xls)), warmup=len(xls))
     del xls
     # the separate LSE merge (what a step runs when its core cannot fuse it): fp32 accumulator read and
     # written, the step's bf16 output read; at the step's size and at 16 x the heads
@@ -291,6 +317,9 @@ def attention_figures(dev, iters: int) -> dict:
         "ln_partial_stats": {"ms": ms_ln, "GBps": x.numel() * 2 / (ms_ln * 1e-3) / 1e9, "bytes": x.numel() * 2},
         "ln_partial_stats_262144_rows": {"ms": ms_ln_big, "GBps": (1 << 18) * 256 * 2 / (ms_ln_big * 1e-3) / 1e9,
                                          "bytes": (1 << 18) * 256 * 2, "frac_hbm_peak": (1 << 18) * 256 * 2 / (ms_ln_big * 1e-3) / 1e9 / PEAK_HBM_GBPS},
+        "ln_partial_bwd_262144_rows_with_column_reduction": {
+            "ms": ms_ln_bwd, "GBps": 2 * (1 << 18) * 256 * 2 / (ms_ln_bwd * 1e-3) / 1e9, "bytes": 2 * (1 << 18) * 256 * 2,
+            "frac_hbm_peak": 2 * (1 << 18) * 256 * 2 / (ms_ln_bwd * 1e-3) / 1e9 / PEAK_HBM_GBPS},
     }
 
 

@@ -352,21 +352,58 @@ __device__ __forceinline__ void store8(typename Elem<DT>::T* p, const float in[k
   }
 }
 
-// sum over the G lanes (a power of two) that share a row
-__device__ __forceinline__ float group_sum(float v, int G) {
-  for (int o = G >> 1; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-  return v;
+// Sum over the G lanes (a power of two) that share a row, left in every one of them: the butterfly
+// v += v[lane ^ o] for o = 1, 2, 4, ..., G / 2, without a trip through the LDS crossbar. Inside a row of
+// 16 lanes the partner comes through DPP operands (for o = 4 and 8 the mirror partner holds the bits of the
+// lane ^ o partner, because every lane of a finished group holds the same sum); rows of 16 and halves of 32
+// change places with the swap instructions. The swaps are written in assembly with their wait states: the
+// builtin was seen to be folded into "a + a" when both of its operands hold the same value.
+template <int CTRL>
+__device__ __forceinline__ float dpp_partner(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
 }
-// N such sums at once: the N shuffles of a step do not wait for each other
+__device__ __forceinline__ float add_row_partner(float v) {  // v[lane] + v[lane ^ 16]
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return a + b;
+}
+__device__ __forceinline__ float add_half_partner(float v) {  // v[lane] + v[lane ^ 32]
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return a + b;
+}
+// N such sums at once: the N instructions of a step do not wait for each other
 template <int N>
 __device__ __forceinline__ void group_sums(float (&v)[N], int G) {
-  for (int o = G >> 1; o > 0; o >>= 1) {
-    float t[N];
+  if (G > 1) {
 #pragma unroll
-    for (int i = 0; i < N; ++i) t[i] = __shfl_xor(v[i], o, kWave);
-#pragma unroll
-    for (int i = 0; i < N; ++i) v[i] += t[i];
+    for (int i = 0; i < N; ++i) v[i] += dpp_partner<0xB1>(v[i]);  // quad_perm [1, 0, 3, 2]
   }
+  if (G > 2) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] += dpp_partner<0x4E>(v[i]);  // quad_perm [2, 3, 0, 1]
+  }
+  if (G > 4) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] += dpp_partner<0x141>(v[i]);  // row_half_mirror
+  }
+  if (G > 8) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] += dpp_partner<0x140>(v[i]);  // row_mirror
+  }
+  if (G > 16) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = add_row_partner(v[i]);
+  }
+  if (G > 32) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = add_half_partner(v[i]);
+  }
+}
+__device__ __forceinline__ float group_sum(float v, int G) {
+  float one[1] = {v};
+  group_sums<1>(one, G);
+  return one[0];
 }
 
 // w (and b) of the columns a lane owns, as 16-byte loads
@@ -393,11 +430,12 @@ __global__ __launch_bounds__(kThreads) void ln_plain_fwd_kernel(
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
   const float inv = 1.0f / (float)cols;
-  const long long stride = (long long)gridDim.x * kWavesPerBlock * rpw;
+  // a wavefront's U row sets of a round lie behind each other in memory (U * rpw consecutive rows)
+  const long long stride = rpw, round_stride = (long long)gridDim.x * kWavesPerBlock * rpw * U;
   float wv[CH][kPlainVec], bv[CH][kPlainVec];
   load_params<CH>(wv, w, G, sl, cols);
   load_params<CH>(bv, b, G, sl, cols);
-  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows; r0 += stride * U) {
+  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw * U; r0 < rows; r0 += round_stride) {
     float v[U][CH][kPlainVec], m[U], rs[U];
     bool live[U];
 #pragma unroll
@@ -479,7 +517,8 @@ __global__ __launch_bounds__(kThreads) void ln_plain_bwd_kernel(
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
   const float inv = 1.0f / (float)cols;
-  const long long stride = (long long)gridDim.x * kWavesPerBlock * rpw;
+  // a wavefront's U row sets of a round lie behind each other in memory (U * rpw consecutive rows)
+  const long long stride = rpw, round_stride = (long long)gridDim.x * kWavesPerBlock * rpw * U;
   float wv[CH][kPlainVec], agw[CH][kPlainVec], agb[CH][kPlainVec];
   load_params<CH>(wv, w, G, sl, cols);
 #pragma unroll
@@ -489,7 +528,7 @@ __global__ __launch_bounds__(kThreads) void ln_plain_bwd_kernel(
       agw[k][i] = 0.0f;
       agb[k][i] = 0.0f;
     }
-  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows; r0 += stride * U) {
+  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw * U; r0 < rows; r0 += round_stride) {
     float gv[U][CH][kPlainVec], xh[U][CH][kPlainVec], m[U], rs[U], s1[U], s2[U], s12[2 * U];
     bool live[U];
 #pragma unroll
@@ -626,6 +665,32 @@ __device__ __forceinline__ void load8_or_zero(const typename Elem<DT>::T* base, 
   for (int i = 0; i < kPlainVec; ++i) out[i] = ok ? out[i] : 0.0f;
 }
 
+// 8 columns as they lie in memory (16 or 32 bytes), converted later: a kernel can then request the rows of its
+// next round before it turns to the arithmetic of the current one, and the loads stay in the air meanwhile.
+template <int DT>
+struct Raw8 {
+  typedef typename Elem<DT>::T T;
+  static constexpr int PER = 16 / sizeof(T);
+  struct alignas(16) Pack { T v[PER]; };
+  Pack p[kPlainVec / PER];
+};
+template <int DT>
+__device__ __forceinline__ void load8_raw(const typename Elem<DT>::T* base, long long r, long long rows, int c, int cols,
+                                          Raw8<DT>& out) {
+  typedef typename Raw8<DT>::Pack Pack;
+  // always an address inside the tensor (row and column clamped): no branch around the load
+  const typename Elem<DT>::T* p = base + (r < rows ? r : rows - 1) * cols + (c < cols ? c : 0);
+#pragma unroll
+  for (int h = 0; h < kPlainVec / Raw8<DT>::PER; ++h) out.p[h] = *reinterpret_cast<const Pack*>(p + h * Raw8<DT>::PER);
+}
+template <int DT>
+__device__ __forceinline__ void unpack8(const Raw8<DT>& in, bool ok, float out[kPlainVec]) {
+#pragma unroll
+  for (int h = 0; h < kPlainVec / Raw8<DT>::PER; ++h)
+#pragma unroll
+    for (int i = 0; i < Raw8<DT>::PER; ++i) out[h * Raw8<DT>::PER + i] = ok ? Elem<DT>::up(in.p[h].v[i]) : 0.0f;
+}
+
 template <int DT, int CH, int U>
 __global__ __launch_bounds__(kThreads) void ln_partial_fwd_rows_kernel(
     float* __restrict__ mean, float* __restrict__ var, const typename Elem<DT>::T* __restrict__ x,
@@ -633,20 +698,29 @@ __global__ __launch_bounds__(kThreads) void ln_partial_fwd_rows_kernel(
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
   const float inv = 1.0f / (float)cols;
-  const long long stride = (long long)gridDim.x * kWavesPerBlock * rpw;
-  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows; r0 += stride * U) {
+  // a wavefront's U row sets of a round lie behind each other in memory (U * rpw consecutive rows)
+  const long long stride = rpw;
+  const long long round_stride = (long long)gridDim.x * kWavesPerBlock * rpw * U;
+  long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw * U;
+  Raw8<DT> raw[U][CH];
+  auto request = [&](long long first) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int k = 0; k < CH; ++k) load8_raw<DT>(x, first + u * stride + sub, rows, (k * G + sl) * kPlainVec, cols, raw[u][k]);
+  };
+  if (r0 < rows) request(r0);
+  for (; r0 < rows; r0 += round_stride) {
     float v[U][CH][kPlainVec], m[U], qs[U];
     bool live[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const long long r = r0 + u * stride + sub;
-      live[u] = r < rows;
+      live[u] = r0 + u * stride + sub < rows;
 #pragma unroll
-      for (int k = 0; k < CH; ++k) {
-        const int c = (k * G + sl) * kPlainVec;
-        load8_or_zero<DT>(x, r, rows, c, cols, v[u][k]);
-      }
+      for (int k = 0; k < CH; ++k) unpack8<DT>(raw[u][k], live[u] && (k * G + sl) * kPlainVec < cols, v[u][k]);
     }
+    // the rows of the next round are on their way during the sums and shuffles of this one
+    if (r0 + round_stride < rows) request(r0 + round_stride);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       float s = 0.0f;
@@ -696,11 +770,12 @@ __global__ __launch_bounds__(kThreads) void ln_apply_rows_kernel(
     long long rows, int cols, float eps, int G) {
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
-  const long long stride = (long long)gridDim.x * kWavesPerBlock * rpw;
+  // a wavefront's U row sets of a round lie behind each other in memory (U * rpw consecutive rows)
+  const long long stride = rpw, round_stride = (long long)gridDim.x * kWavesPerBlock * rpw * U;
   float wv[CH][kPlainVec], bv[CH][kPlainVec];
   load_params_of<ODT, CH>(wv, w, G, sl, cols);
   load_params_of<ODT, CH>(bv, b, G, sl, cols);
-  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows; r0 += stride * U) {
+  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw * U; r0 < rows; r0 += round_stride) {
     float v[U][CH][kPlainVec], m[U], sd[U];
     bool live[U];
 #pragma unroll
@@ -742,15 +817,19 @@ __global__ __launch_bounds__(kThreads) void ln_apply_rows_kernel(
 }
 
 // The column partials leave the kernel as those of ln_partial_bwd_kernel do: part[blk][which][col].
-template <int DT, int CH, int U>
-__global__ __launch_bounds__(kThreads) void ln_partial_bwd_rows_kernel(
+// WAVES wavefronts a block (the number of blocks, and with it of partial rows, is bounded by the workspace
+// contract, so more wavefronts per block is how more rows are in flight per CU); a wavefront's U row sets of
+// a round lie behind each other in memory. Dynamic LDS: WAVES * 2 * cols floats.
+template <int DT, int CH, int U, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void ln_partial_bwd_rows_kernel(
     float* __restrict__ mean_gxn, float* __restrict__ dot, float* __restrict__ part,
     const typename Elem<DT>::T* __restrict__ g, const typename Elem<DT>::T* __restrict__ x_hat,
     const typename Elem<DT>::T* __restrict__ w, long long rows, int cols, int G, bool want_cols) {
+  extern __shared__ __attribute__((aligned(16))) float red[];  // [WAVES][2][cols]
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
   const float inv = 1.0f / (float)cols;
-  const long long stride = (long long)gridDim.x * kWavesPerBlock * rpw;
+  const long long round_stride = (long long)gridDim.x * WAVES * rpw * U;
   float wv[CH][kPlainVec], agw[CH][kPlainVec], agb[CH][kPlainVec];
   load_params_of<DT, CH>(wv, w, G, sl, cols);
 #pragma unroll
@@ -760,12 +839,12 @@ __global__ __launch_bounds__(kThreads) void ln_partial_bwd_rows_kernel(
       agw[k][i] = 0.0f;
       agb[k][i] = 0.0f;
     }
-  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows; r0 += stride * U) {
+  for (long long r0 = ((long long)blockIdx.x * WAVES + wave) * rpw * U; r0 < rows; r0 += round_stride) {
     float gv[U][CH][kPlainVec], xh[U][CH][kPlainVec], s12[2 * U];
     bool live[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const long long r = r0 + u * stride + sub;
+      const long long r = r0 + u * rpw + sub;
       live[u] = r < rows;
 #pragma unroll
       for (int k = 0; k < CH; ++k) {
@@ -795,7 +874,7 @@ __global__ __launch_bounds__(kThreads) void ln_partial_bwd_rows_kernel(
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       if (live[u] && sl == 0) {
-        const long long r = r0 + u * stride + sub;
+        const long long r = r0 + u * rpw + sub;
         mean_gxn[r] = s12[u] * inv;
         dot[r] = s12[U + u];
       }
@@ -811,23 +890,25 @@ __global__ __launch_bounds__(kThreads) void ln_partial_bwd_rows_kernel(
         agw[k][i] += __shfl_xor(agw[k][i], o, kWave);
         agb[k][i] += __shfl_xor(agb[k][i], o, kWave);
       }
-  __shared__ float red[kWavesPerBlock][2][kPlainChunks * kWave * kPlainVec];
   if (sub == 0) {
 #pragma unroll
     for (int k = 0; k < CH; ++k)
 #pragma unroll
       for (int i = 0; i < kPlainVec; ++i) {
-        red[wave][0][(k * G + sl) * kPlainVec + i] = agw[k][i];
-        red[wave][1][(k * G + sl) * kPlainVec + i] = agb[k][i];
+        const int c = (k * G + sl) * kPlainVec + i;
+        if (c < cols) {
+          red[(wave * 2 + 0) * cols + c] = agw[k][i];
+          red[(wave * 2 + 1) * cols + c] = agb[k][i];
+        }
       }
   }
   __syncthreads();
-  for (int c = threadIdx.x; c < cols; c += kThreads) {
+  for (int c = threadIdx.x; c < cols; c += WAVES * kWave) {
     float a = 0.0f, b2 = 0.0f;
 #pragma unroll
-    for (int wv2 = 0; wv2 < kWavesPerBlock; ++wv2) {
-      a += red[wv2][0][c];
-      b2 += red[wv2][1][c];
+    for (int wv2 = 0; wv2 < WAVES; ++wv2) {
+      a += red[(wv2 * 2 + 0) * cols + c];
+      b2 += red[(wv2 * 2 + 1) * cols + c];
     }
     part[((long long)blockIdx.x * 2 + 0) * cols + c] = a;
     part[((long long)blockIdx.x * 2 + 1) * cols + c] = b2;
@@ -842,10 +923,11 @@ __global__ __launch_bounds__(kThreads) void ln_bwd_apply_rows_kernel(
     long long rows, int cols, float inv_n, int G) {
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int sl = lane & (G - 1), sub = lane / G, rpw = kWave / G;
-  const long long stride = (long long)gridDim.x * kWavesPerBlock * rpw;
+  // a wavefront's U row sets of a round lie behind each other in memory (U * rpw consecutive rows)
+  const long long stride = rpw, round_stride = (long long)gridDim.x * kWavesPerBlock * rpw * U;
   float wv[CH][kPlainVec];
   load_params_of<DT, CH>(wv, w, G, sl, cols);
-  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw; r0 < rows; r0 += stride * U) {
+  for (long long r0 = ((long long)blockIdx.x * kWavesPerBlock + wave) * rpw * U; r0 < rows; r0 += round_stride) {
     float gv[U][CH][kPlainVec], xh[U][CH][kPlainVec], m[U], dn[U], sd[U];
     bool live[U];
 #pragma unroll
@@ -898,7 +980,7 @@ int plain_chunks(long long cols) {
 bool plain_ok(long long cols) { return cols >= kPlainVec && cols % kPlainVec == 0 && plain_chunks(cols) <= kPlainChunks; }
 int plain_blocks(long long rows, long long cols, int most = 1024) {
   const int rpw = kWave / plain_group(cols);
-  long long b = (rows + (long long)kWavesPerBlock * rpw - 1) / ((long long)kWavesPerBlock * rpw);
+  long long b = (rows + (long long)kWavesPerBlock * rpw - 1) / ((long long)kWavesPerBlock * rpw);  // one row set a wavefront
   if (b > most) b = most;
   if (b < 1) b = 1;
   return (int)b;
@@ -969,7 +1051,7 @@ extern "C" int jg_ln_partial_fwd(float* mean, float* var, const void* x, int64_t
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool v = vec_aligned(x, cols, x_dtype);
   const bool in_regs = plain_ok(cols) && aligned16(x);
-  const int G = in_regs ? plain_group(cols) : 0, blocks = in_regs ? plain_blocks(rows, cols, 2048) : 0;
+  const int G = in_regs ? plain_group(cols) : 0, blocks = in_regs ? plain_blocks(rows, cols, 8192) : 0;
 #define JG_GO(DT)                                                                                  \
   if (in_regs)                                                                                     \
     with_row_shape<4>(cols, [&](auto ch, auto u) {                                                 \
@@ -1048,12 +1130,16 @@ static int launch_partial_bwd(float* mean_gxn, float* dot, float* part, const vo
                               bool want_cols, hipStream_t s, int* blocks_used) {
   typedef typename Elem<DT>::T T;
   if (plain_ok(cols) && aligned16(g) && aligned16(x_hat) && aligned16(w)) {
-    const int G = plain_group(cols), blocks = plain_blocks(rows, cols);  // never more than bwd_blocks(rows)
+    const int G = plain_group(cols);
+    const int rpw = kWave / G;
+    long long nb = (rows + (long long)kWavesPerBlock * rpw - 1) / ((long long)kWavesPerBlock * rpw);
+    const int blocks = (int)(nb > 1024 ? 1024 : nb);  // never more than bwd_blocks(rows)
     *blocks_used = blocks;
+    const size_t lds = (size_t)kWavesPerBlock * 2 * cols * sizeof(float);
     with_row_shape<2>(cols, [&](auto ch, auto u) {
-      ln_partial_bwd_rows_kernel<DT, decltype(ch)::value, decltype(u)::value><<<blocks, kThreads, 0, s>>>(
-          mean_gxn, dot, part, static_cast<const T*>(g), static_cast<const T*>(x_hat), static_cast<const T*>(w),
-          rows, (int)cols, G, want_cols);
+      ln_partial_bwd_rows_kernel<DT, decltype(ch)::value, decltype(u)::value, kWavesPerBlock>
+          <<<blocks, kThreads, lds, s>>>(mean_gxn, dot, part, static_cast<const T*>(g), static_cast<const T*>(x_hat),
+                                         static_cast<const T*>(w), rows, (int)cols, G, want_cols);
     });
     return JG_OK;
   }
