@@ -142,6 +142,32 @@ int jg_halo_fold_2d(void* gx, const void* gx_aug, const void* const strips[9],
 int jg_halo_fold_border_3d(void* gx, const void* const strips[27],
                            const jg_halo_geom* geom, int dtype, void* stream);
 
+/* Halo exchange along ONE split axis for need spans of any shape - spans that leave out rows
+ * the rank owns, or that reach ranks which are not adjacent (the fused entry points above cover
+ * spans that hold the owned rows and reach one tile to either side at most). A tensor is seen as
+ * (outer, rows, inner) around the axis; a segment is `count` rows [src_start, +count) of `src`
+ * (outer, src_rows, inner) that belong at rows [dst_start, +count) of the destination.
+ * jg_halo_axis_gather: dst (outer, dst_rows, inner) = zero, then every segment copied in (bytes
+ * untouched; a later segment overwrites an earlier one): the need span from the own tile and the
+ * peers' parts (x_need = zeros; x_need[off : off + cnt] = part, _conv/halo.py:112-114, 134-154),
+ * or, with one segment, the contiguous part cut for a peer (:140-147, 222-226).
+ * jg_halo_axis_scatter_add: dst = 0, then dst[dst_start : +count] += segment for the segments IN
+ * THE ORDER GIVEN, each sum rounded to `dtype` (g_local = zeros; g_local[...] += recv[peer] for
+ * peer = 0 .. G-1, _conv/halo.py:207, 247-249): bit-identical to the reference's loop.
+ * At most JG_HALO_AXIS_MAX_SEGMENTS segments a call (JG_ERR_BAD_ARG beyond). */
+#define JG_HALO_AXIS_MAX_SEGMENTS 16
+typedef struct jg_axis_segment {
+  const void* src;
+  int64_t src_rows;
+  int64_t src_start;
+  int64_t dst_start;
+  int64_t count;
+} jg_axis_segment;
+int jg_halo_axis_gather(void* dst, int64_t outer, int64_t dst_rows, int64_t inner,
+                        const jg_axis_segment* segs, int n_segs, int elem_size, void* stream);
+int jg_halo_axis_scatter_add(void* dst, int64_t outer, int64_t dst_rows, int64_t inner,
+                             const jg_axis_segment* segs, int n_segs, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------- *
  * DistributedRoll (pure copies; HBM-bound)
  * ------------------------------------------------------------------------- */

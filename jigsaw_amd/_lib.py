@@ -41,6 +41,18 @@ class HaloGeom(ctypes.Structure):
     ]
 
 
+class AxisSegment(ctypes.Structure):
+    """``jg_axis_segment`` of include/jigsaw_hip.h."""
+
+    _fields_ = [
+        ("src", ctypes.c_void_p),
+        ("src_rows", ctypes.c_int64),
+        ("src_start", ctypes.c_int64),
+        ("dst_start", ctypes.c_int64),
+        ("count", ctypes.c_int64),
+    ]
+
+
 class ConvDesc(ctypes.Structure):
     """``jg_conv_desc`` of ``include/jigsaw_hip.h``."""
 
@@ -85,6 +97,8 @@ SIGNATURES: dict[str, tuple] = {
         c_int,
         [c_void_p, c_void_p, POINTER(c_void_p), c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     ),
+    "jg_halo_axis_gather": (c_int, [c_void_p, c_int64, c_int64, c_int64, POINTER(AxisSegment), c_int, c_int, c_void_p]),
+    "jg_halo_axis_scatter_add": (c_int, [c_void_p, c_int64, c_int64, c_int64, POINTER(AxisSegment), c_int, c_int, c_void_p]),
     "jg_roll": (c_int, [c_void_p, c_void_p, c_int, POINTER(c_int64), POINTER(c_int64), c_int, c_void_p]),
     "jg_roll_pack": (c_int, [c_void_p, c_void_p, c_int, POINTER(c_int64), c_int, c_int64, c_int, c_void_p]),
     "jg_roll_pack_fused": (

@@ -27,7 +27,8 @@ from typing import Any, Protocol
 import torch
 
 from . import _lib
-from .halo import HaloGeometry, halo_assemble, halo_fold, halo_fold_border_, halo_pack, new_strips, strip_table
+from .halo import (HaloGeometry, halo_assemble, halo_fold, halo_fold_border_, halo_gather_axis, halo_pack,
+                   halo_scatter_add_axis, new_strips, spans_fit_the_strips, strip_table)
 
 # --------------------------------------------------------------------------- #
 # local primitives
@@ -825,6 +826,13 @@ class HaloExchange(Protocol):
 
     def backward(self, send: dict) -> dict: ...
 
+    def along_axis(self, axis: int, send: list, backward: bool) -> list:
+        """The exchange of ONE split axis for need spans the strips do not cover
+        (``exchange_along_axis``, _common/halo.py:7-63): ``send[p]`` is the part cut for rank ``p`` of
+        that axis' group (``None``: nothing, and always for the rank itself); returns what the peers cut
+        for this rank, by peer. Only called where ``halo.spans_fit_the_strips`` says no."""
+        ...
+
 
 def _mesh_position(spatial_groups) -> tuple[tuple, tuple]:
     sizes = tuple(1 if g is None else int(g.size()) for g in spatial_groups)
@@ -881,11 +889,22 @@ def conv_halo_nway(x, w, b, stride, padding, dilation, spatial_groups, channel_g
     n = config.n_spatial
     ranks, sizes = _mesh_position(spatial_groups)
     x = x.contiguous()
+    kwargs = {"stride": stride, "padding": _local_padding(padding, sizes), "dilation": dilation, "groups": int(getattr(config, "groups_local", 1))}
+    if not spans_fit_the_strips(x.shape[-n:], w.shape[-n:], stride, padding, dilation, sizes):
+        # need spans that leave out owned rows or reach past the adjacent rank: one split axis at a
+        # time, first to last, every peer's overlap copied in (distributed.py:264-275, halo.py:101-156)
+        x_aug = x
+        for a in range(n):
+            if sizes[a] <= 1:
+                continue
+            x_aug = halo_gather_axis(x_aug, a - n, ranks[a], sizes[a], w.shape[a - n], stride[a], padding[a], dilation[a],
+                                     lambda send, a=a: config.halo_exchange.along_axis(a, send, False))
+        y = config.conv_fn(x_aug, w, b, **kwargs) if b is not None else config.conv_fn(x_aug, w, **kwargs)
+        return y, x_aug
     geom = HaloGeometry.for_conv(x.shape[-n:], w.shape[-n:], stride, padding, dilation, ranks, sizes)
     present = _present_offsets(geom, ranks, sizes)
     send = halo_pack(x, geom, from_padded=False, present=present) if present else {}
     recv = config.halo_exchange.forward(send) if present else {}
-    kwargs = {"stride": stride, "padding": _local_padding(padding, sizes), "dilation": dilation, "groups": int(getattr(config, "groups_local", 1))}
     bands = _frame_decision(config, x, geom, w.shape, kwargs)
     if bands is not None:
         # only the frame of the padded tile is built; the kernels read the tile itself elsewhere.
@@ -949,6 +968,16 @@ def conv_halo_nway_backward(
     done = (lambda gx: (gx, g_w, g_b)) if want_b else (lambda gx: (gx, g_w))
     if not need_x:
         return done(None)
+    if not spans_fit_the_strips(local_in_spatial, weight.shape[-n:], stride, padding, dilation, sizes):
+        # the general spans of the forward: fold one split axis at a time, last to first, the peers'
+        # parts added in rank order (distributed.py:378-389, halo.py:195-251)
+        g_x = config.conv_input_fn(x_aug.shape, weight, g, **kwargs)
+        for a in reversed(range(n)):
+            if sizes[a] <= 1:
+                continue
+            g_x = halo_scatter_add_axis(g_x, a - n, ranks[a], sizes[a], weight.shape[a - n], stride[a], padding[a], dilation[a],
+                                        local_in_spatial[a], lambda send, a=a: config.halo_exchange.along_axis(a, send, True))
+        return done(g_x)
     geom = HaloGeometry.for_conv(local_in_spatial, weight.shape[-n:], stride, padding, dilation, ranks, sizes)
     present = _present_offsets(geom, ranks, sizes)
     if getattr(config, "fused_fold", False) and config.conv_input_fn is conv_nd_input:
@@ -1115,9 +1144,10 @@ class _ConvNd(torch.autograd.Function):
         ctx.mark_non_differentiable(x_aug)
         # the same decision conv_halo_nway took: x_aug is a frame only, so the tile is kept
         ctx.framed = False
-        if getattr(config, "framed", False) and isinstance(padding, tuple):
-            n = config.n_spatial
-            ranks, sizes = _mesh_position(spatial_groups)
+        n = config.n_spatial
+        ranks, sizes = _mesh_position(spatial_groups)
+        if (getattr(config, "framed", False) and isinstance(padding, tuple)
+                and spans_fit_the_strips(x.shape[-n:], weight.shape[-n:], stride, padding, dilation, sizes)):
             geom = HaloGeometry.for_conv(x.shape[-n:], weight.shape[-n:], stride, padding, dilation, ranks, sizes)
             kwargs = {"stride": stride, "padding": _local_padding(padding, sizes), "dilation": dilation, "groups": int(getattr(config, "groups_local", 1))}
             x_c = x if x.dtype == x_aug.dtype else torch.empty(0, dtype=x_aug.dtype, device=x.device).new_empty(x.shape)

@@ -21,7 +21,7 @@ from typing import Mapping, Sequence
 import torch
 
 from . import _lib
-from ._lib import HaloGeom, VoidP27
+from ._lib import AxisSegment, HaloGeom, VoidP27
 
 Offset = tuple  # one entry in {-1, 0, 1} per spatial axis
 
@@ -450,16 +450,187 @@ def halo_fold_border_(
     return gx
 
 
+# --------------------------------------------------------------------------- #
+# Need spans of any shape, one split axis at a time: the reference's own scheme
+# (halo_gather / halo_scatter_add, _conv/halo.py:66-251, with exchange_along_axis,
+# _common/halo.py:7-63). The fused strip functions above serve spans that hold the
+# rank's own rows and reach at most one tile to either side; a span that leaves out
+# owned rows (stride 2 without padding on an odd tile) or reaches further (a kernel
+# wider than the tile) takes these.
+# --------------------------------------------------------------------------- #
+MAX_AXIS_SEGMENTS = 16
+
+
+def spans_fit_the_strips(local_in_spatial, kernel, stride, padding, dilation, group_sizes) -> bool:
+    """Whether EVERY rank's need span on every split axis holds its own rows and reaches one tile to
+    either side at most: what the one-pass strip functions need. Decided for the whole group, so
+    that all of its ranks exchange the same way. ``NotImplementedError`` for an output size the
+    group does not divide (``needed_input_span``) passes through."""
+    for a, n in enumerate(local_in_spatial):
+        G = group_sizes[a]
+        if G <= 1:
+            continue
+        for r in range(G):
+            lo, hi, _, _ = needed_input_span(r, G, n, kernel[a], stride[a], padding[a], dilation[a])
+            lo_w, hi_w = r * n - lo, hi - (r + 1) * n
+            if lo_w < 0 or hi_w < 0 or lo_w > n or hi_w > n:
+                return False
+    return True
+
+
+def span_overlap(lo: int, hi: int, peer: int, n: int, group_size: int) -> tuple[int, int]:
+    """``(first row, count)`` of the rows of ``[lo, hi)`` that rank ``peer`` owns, in global rows
+    (_conv/halo.py:134-138, 217-221: ``max(lo, peer * n, 0)`` to ``min(hi, (peer + 1) * n, G * n)``)."""
+    r0 = max(lo, peer * n, 0)
+    return r0, max(min(hi, (peer + 1) * n, group_size * n) - r0, 0)
+
+
+def _axis_view(t: torch.Tensor, axis: int) -> tuple[int, int, int]:
+    axis %= t.dim()
+    outer = 1
+    for v in t.shape[:axis]:
+        outer *= int(v)
+    inner = 1
+    for v in t.shape[axis + 1:]:
+        inner *= int(v)
+    return outer, int(t.shape[axis]), inner
+
+
+def _segments(parts, axis: int, like: torch.Tensor, dst_rows: int, what: str):
+    """``(array, count, kept)`` for parts ``(tensor, src_start, dst_start, count)``; the tensors checked against
+    ``like`` everywhere but along ``axis``."""
+    axis %= like.dim()
+    live = [p for p in parts if p[3] > 0]
+    if len(live) > MAX_AXIS_SEGMENTS:
+        raise NotImplementedError(f"{what}: {len(live)} parts, the kernels take {MAX_AXIS_SEGMENTS} a call")
+    arr = (AxisSegment * max(len(live), 1))()
+    kept = []
+    for i, (t, src_start, dst_start, count) in enumerate(live):
+        want = list(like.shape)
+        want[axis] = t.shape[axis]
+        if list(t.shape) != want or t.dtype != like.dtype or t.device != like.device:
+            raise ValueError(f"{what}: part {i} has shape {tuple(t.shape)} / {t.dtype}, expected {tuple(want)} / {like.dtype} on {like.device}")
+        t = t.contiguous()
+        kept.append(t)
+        if src_start < 0 or src_start + count > t.shape[axis] or dst_start < 0 or dst_start + count > dst_rows:
+            raise ValueError(f"{what}: part {i} does not fit ({src_start}, {dst_start}, {count})")
+        arr[i].src, arr[i].src_rows = t.data_ptr(), int(t.shape[axis])
+        arr[i].src_start, arr[i].dst_start, arr[i].count = int(src_start), int(dst_start), int(count)
+    return arr, len(live), kept
+
+
+def axis_gather(dst_rows: int, axis: int, parts: Sequence, like: torch.Tensor) -> torch.Tensor:
+    """A tensor like ``like`` with ``dst_rows`` rows along ``axis``: zero, then every part
+    ``(tensor, src_start, dst_start, count)`` copied in (bit-exact; ``jg_halo_axis_gather``)."""
+    _lib.require_gpu(like)
+    axis %= like.dim()
+    shape = list(like.shape)
+    shape[axis] = int(dst_rows)
+    out = torch.empty(shape, dtype=like.dtype, device=like.device)
+    arr, n, kept = _segments(parts, axis, like, int(dst_rows), "axis_gather")
+    outer, _, inner = _axis_view(out, axis)
+    rc = _lib.load().jg_halo_axis_gather(_lib.ptr(out), outer, int(dst_rows), inner, arr, n, like.element_size(),
+                                         _lib.stream_ptr(like.device))
+    _lib.check(rc, "jg_halo_axis_gather")
+    del kept
+    return out
+
+
+def axis_scatter_add(dst_rows: int, axis: int, parts: Sequence, like: torch.Tensor) -> torch.Tensor:
+    """``zeros`` with ``dst_rows`` rows along ``axis``, then ``out[dst_start : +count] += part`` for the parts in the
+    order given, every sum rounded to the dtype (``jg_halo_axis_scatter_add``)."""
+    _lib.require_gpu(like)
+    axis %= like.dim()
+    shape = list(like.shape)
+    shape[axis] = int(dst_rows)
+    out = torch.empty(shape, dtype=like.dtype, device=like.device)
+    arr, n, kept = _segments(parts, axis, like, int(dst_rows), "axis_scatter_add")
+    outer, _, inner = _axis_view(out, axis)
+    rc = _lib.load().jg_halo_axis_scatter_add(_lib.ptr(out), outer, int(dst_rows), inner, arr, n, _lib.dtype_code(like.dtype),
+                                              _lib.stream_ptr(like.device))
+    _lib.check(rc, "jg_halo_axis_scatter_add")
+    del kept
+    return out
+
+
+def halo_gather_axis(x, axis, rank, group_size, kernel, stride, padding, dilation, all_to_all):
+    """The need span of ``rank`` along ``axis`` from its tile and its peers' (``halo_gather``,
+    _conv/halo.py:66-156). ``all_to_all(send)`` is the exchange of that axis' group
+    (``exchange_along_axis``, _common/halo.py:7-63): ``send[p]`` is the contiguous part cut for
+    peer ``p`` (``None`` where there is none, and for the rank itself, whose part never travels); it
+    returns the parts the peers cut for this rank, by peer."""
+    G, n = int(group_size), int(x.shape[axis])
+    spans = [needed_input_span(r, G, n, kernel, stride, padding, dilation) for r in range(G)]
+    lo, hi, need, _ = spans[rank]
+    send: list = [None] * G
+    for peer in range(G):
+        if peer == rank:
+            continue
+        r0, cnt = span_overlap(spans[peer][0], spans[peer][1], rank, n, G)  # rows of mine that peer needs
+        if cnt > 0:
+            send[peer] = axis_gather(cnt, axis, [(x, r0 - rank * n, 0, cnt)], x)
+    recv = all_to_all(send)
+    parts = []
+    for peer in range(G):
+        r0, cnt = span_overlap(lo, hi, peer, n, G)
+        if cnt <= 0:
+            continue
+        if peer == rank:
+            parts.append((x, r0 - rank * n, r0 - lo, cnt))
+        else:
+            if recv[peer] is None or recv[peer].shape[axis] != cnt:
+                raise ValueError(f"halo_gather_axis: expected {cnt} rows from peer {peer}")
+            parts.append((recv[peer], 0, r0 - lo, cnt))
+    return axis_gather(need, axis, parts, x)
+
+
+def halo_scatter_add_axis(g_need, axis, rank, group_size, kernel, stride, padding, dilation, local_in_size, all_to_all):
+    """The gradient of the rows ``rank`` owns from its own span's gradient and its peers'
+    (``halo_scatter_add``, _conv/halo.py:159-251): the parts are added in peer order 0 .. G-1, the
+    own one in its place, each sum rounded to the dtype — the bits of the reference's loop."""
+    G, n = int(group_size), int(local_in_size)
+    spans = [needed_input_span(r, G, n, kernel, stride, padding, dilation) for r in range(G)]
+    lo, hi, need, _ = spans[rank]
+    if g_need.shape[axis] != need:
+        raise ValueError(f"halo_scatter_add_axis: the span has {need} rows, the gradient {g_need.shape[axis]}")
+    send: list = [None] * G
+    for peer in range(G):
+        if peer == rank:
+            continue
+        r0, cnt = span_overlap(lo, hi, peer, n, G)  # rows of my span that peer owns
+        if cnt > 0:
+            send[peer] = axis_gather(cnt, axis, [(g_need, r0 - lo, 0, cnt)], g_need)
+    recv = all_to_all(send)
+    parts = []
+    for peer in range(G):
+        r0, cnt = span_overlap(spans[peer][0], spans[peer][1], rank, n, G)  # rows of peer's span that I own
+        if cnt <= 0:
+            continue
+        if peer == rank:
+            parts.append((g_need, r0 - lo, r0 - rank * n, cnt))
+        else:
+            if recv[peer] is None or recv[peer].shape[axis] != cnt:
+                raise ValueError(f"halo_scatter_add_axis: expected {cnt} rows from peer {peer}")
+            parts.append((recv[peer], 0, r0 - rank * n, cnt))
+    return axis_scatter_add(n, axis, parts, g_need)
+
+
 __all__ = [
     "HaloGeometry",
+    "axis_gather",
+    "axis_scatter_add",
     "halo_assemble",
     "halo_fold",
     "halo_fold_border_",
+    "halo_gather_axis",
     "halo_pack",
+    "halo_scatter_add_axis",
     "halo_widths",
     "neighbour_widths",
     "new_strips",
     "needed_input_span",
     "slot",
+    "span_overlap",
+    "spans_fit_the_strips",
     "strip_table",
 ]

@@ -77,3 +77,67 @@ def kaiming_uniform_bound(c_in, kernel, a=5 ** 0.5):
         fan_in *= k
     gain = (2.0 / (1.0 + a * a)) ** 0.5
     return (3.0 ** 0.5) * gain / fan_in ** 0.5
+
+
+class LockstepMesh:
+    """Every rank of a spatial mesh in this process, one thread each, for the exchanges that need all ranks
+    at once (``HaloExchange.along_axis``: every rank cuts parts for its peers, then every rank picks up
+    what was cut for it). ``run(fn)`` calls ``fn(coord, exchange)`` per rank and returns ``{coord: result}``;
+    an exception in one rank releases the others and is raised again. All ranks launch on the default
+    stream, so a part is read behind the kernel that cut it."""
+
+    def __init__(self, mesh_shape):
+        import threading
+
+        self.mesh = tuple(mesh_shape)
+        self.coords = list(mesh_coords(self.mesh))
+        self._barrier = threading.Barrier(len(self.coords))
+        self._box: dict = {}
+        self.calls: list = []  # (coord, axis, backward, rows sent per peer) in call order per rank
+
+    def exchange_for(self, coord):
+        mesh = self
+
+        class _Rank:
+            def forward(self, send):
+                raise AssertionError("the strip exchange is not what general spans use")
+
+            backward = forward
+
+            def along_axis(self, axis, send, backward):
+                if len(send) != mesh.mesh[axis] or send[coord[axis]] is not None:
+                    raise AssertionError("one part per peer of the axis, none for the rank itself")
+                mesh.calls.append((coord, axis, backward, [None if t is None else int(t.shape[axis - len(mesh.mesh)]) for t in send]))
+                mesh._box[(coord, axis, backward)] = send
+                mesh._barrier.wait(timeout=60)
+                recv = []
+                for p in range(mesh.mesh[axis]):
+                    peer = tuple(p if a == axis else v for a, v in enumerate(coord))
+                    recv.append(None if peer == coord else mesh._box[(peer, axis, backward)][coord[axis]])
+                mesh._barrier.wait(timeout=60)
+                return recv
+
+        return _Rank()
+
+    def run(self, fn):
+        import threading
+
+        results, errors = {}, []
+
+        def body(c):
+            try:
+                results[c] = fn(c, self.exchange_for(c))
+            except BaseException as exc:  # noqa: BLE001
+                errors.append(exc)
+                self._barrier.abort()
+
+        threads = [threading.Thread(target=body, args=(c,)) for c in self.coords]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        self._barrier.reset()
+        if errors:
+            first = [e for e in errors if not isinstance(e, threading.BrokenBarrierError)]
+            raise (first or errors)[0]
+        return results

@@ -348,6 +348,70 @@ def _run_mesh_case(case, dev, framed, autocast):
     assert rel_l2(gb_sum, Bd.grad) < tol, f"db: {rel_l2(gb_sum, Bd.grad):.3e}"
 
 
+GENERAL_SPAN_CASES = [
+    # mesh, local spatial, N, Cin, Cout, kernel, padding, dtype, stride, dilation: need spans that leave out owned
+    # rows or reach past the adjacent rank (halo.py:49-63, 134-154): one split axis at a time
+    ((2, 2), (9, 9), 2, 3, 4, (3, 3), (0, 0), torch.float32, (2, 2), (1, 1)),
+    ((3, 2), (2, 8), 1, 4, 5, (7, 3), (3, 1), torch.float32, (1, 1), (1, 1)),
+    ((4, 1), (3, 10), 2, 2, 3, (9, 3), (4, 1), torch.float32, (1, 1), (1, 1)),
+    ((3, 2), (2, 16), 1, 16, 16, (3, 3), (3, 1), torch.bfloat16, (1, 1), (3, 1)),
+    ((2, 3, 1), (4, 2, 5), 1, 2, 3, (5, 7, 3), (2, 3, 1), torch.float32, (1, 1, 1), (1, 1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", GENERAL_SPAN_CASES, ids=lambda c: "mesh" + "x".join(map(str, c[0])) + "_k" + "x".join(map(str, c[5])) + "_" + str(c[7]).split(".")[-1])
+def test_distributed_conv_with_general_spans(case, dev):
+    """``conv_halo_nway`` and ``conv_halo_nway_backward`` on every rank of the mesh (in lockstep, one thread a rank)
+    where the need spans do not fit the strip exchange: y, dx of every rank and the summed dw, db against the
+    serial conv on the gathered tensor (the parity method of test_conv2d_multi_spatial.py:73-233). The two
+    functions are called directly: the autograd engine runs every rank's backward node on its one device thread,
+    where ranks that wait for each other cannot meet."""
+    from helpers import LockstepMesh
+    from jigsaw_amd.halo import spans_fit_the_strips
+
+    mesh, n, N, cin, cout, k, p, dtype, s, d = case
+    ns = len(mesh)
+    assert not spans_fit_the_strips(n, k, s, p, d, mesh)
+    torch.manual_seed(1)
+    gshape = tuple(a * b for a, b in zip(n, mesh))
+    X = torch.randn(N, cin, *gshape).to(dtype)
+    W = ((torch.rand(cout, cin, *k) * 2 - 1) / (cin * int(torch.tensor(k).prod())) ** 0.5).to(dtype)
+    B = (torch.randn(cout) * 0.1).to(dtype)
+    Xd, Wd, Bd = X.double().requires_grad_(), W.double().requires_grad_(), B.double().requires_grad_()
+    Y = oc.forward(Xd, Wd, Bd, s, p, d)
+    G = torch.randn_like(Y).to(dtype)
+    Y.backward(G.double())
+    tiles = oh.split_global(X, mesh)
+    gtiles = oh.split_global(G, mesh)
+    lock = LockstepMesh(mesh)
+
+    def rank(c, exchange):
+        cfg = jc.HipConvNdConfig.for_rank(ns, B.to(dev), exchange)
+        groups = tuple(jc.TileGroup(mesh[a], c[a]) for a in range(ns))
+        xl, wl, bl = tiles[c].to(dev), W.to(dev), B.to(dev)
+        y, x_aug = jc.conv_halo_nway(xl, wl, bl, s, p, d, groups, None, cfg)
+        gx, gw, gb = jc.conv_halo_nway_backward(gtiles[c].to(dev), x_aug, wl, s, p, d, n, groups, None, cfg, need=(True, True, True))
+        return y.cpu(), gx.cpu(), gw.double().cpu(), gb.double().cpu()
+
+    got = lock.run(rank)
+    tol = TOL[dtype]
+    gw_sum, gb_sum = torch.zeros_like(Wd), torch.zeros_like(Bd)
+    for c in mesh_coords(mesh):
+        y, gx, gw, gb = got[c]
+        sl = (slice(None), slice(None)) + tuple(slice(c[a] * n[a], (c[a] + 1) * n[a]) for a in range(ns))
+        no = tuple(Y.shape[2 + a] // mesh[a] for a in range(ns))
+        so = (slice(None), slice(None)) + tuple(slice(c[a] * no[a], (c[a] + 1) * no[a]) for a in range(ns))
+        assert rel_l2(y, Y.detach()[so]) < tol, f"y of rank {c}: {rel_l2(y, Y.detach()[so]):.3e}"
+        assert rel_l2(gx, Xd.grad[sl]) < tol, f"dx of rank {c}: {rel_l2(gx, Xd.grad[sl]):.3e}"
+        gw_sum += gw
+        gb_sum += gb
+    assert rel_l2(gw_sum, Wd.grad) < tol and rel_l2(gb_sum, Bd.grad) < tol
+    # the exchange ran once per split axis and direction on every rank, forward first to last, backward last to first
+    per_rank = [call for call in lock.calls if call[0] == (0,) * ns]
+    split = [a for a in range(ns) if mesh[a] > 1]
+    assert [(a, b) for _, a, b, _ in per_rank] == [(a, False) for a in split] + [(a, True) for a in reversed(split)]
+
+
 def test_frame_without_its_tile_is_refused(dev):
     """A caller that keeps only ``x_aug`` (as the reference's own autograd function does)
     cannot take the weight gradient from a frame: the backward says so instead of

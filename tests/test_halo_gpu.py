@@ -188,3 +188,78 @@ def test_pack_takes_the_blocks_the_neighbours_need(size, lo, hi, from_padded, dt
             spans.append((t.data_ptr(), t.data_ptr() + t.numel() * t.element_size()))
     spans.sort()
     assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))
+
+
+# need spans the strip functions do not cover: one split axis at a time through the per-peer overlap
+# loop (halo.py:134-154, 217-249). (mesh, local spatial, kernel, stride, padding, dilation)
+GENERAL_SPANS = [
+    ((2,), (9,), (3,), (2,), (0,), (1,)),            # stride 2 without padding on an odd tile: rank 1 leaves out its last row
+    ((3,), (2,), (7,), (1,), (3,), (1,)),            # kernel wider than the tile: rows from ranks two away
+    ((4,), (3,), (9,), (1,), (4,), (1,)),            # four ranks, every rank reaches every other
+    ((2, 2), (9, 9), (3, 3), (2, 2), (0, 0), (1, 1)),
+    ((3, 2), (2, 9), (7, 3), (1, 2), (3, 0), (1, 1)),
+    ((2, 3, 1), (4, 2, 5), (5, 7, 3), (1, 1, 1), (2, 3, 1), (1, 1, 1)),
+    ((3, 2), (2, 6), (3, 3), (1, 1), (3, 1), (3, 1)),  # dilated: three taps with an extent of 7 over tiles of 2
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", GENERAL_SPANS, ids=lambda c: "mesh" + "x".join(map(str, c[0])) + "_n" + "x".join(map(str, c[1])) + "_k" + "x".join(map(str, c[2])))
+def test_general_spans_axis_by_axis_bit_exact(case, dtype, dev):
+    """Gather and scatter-add of every rank, axis by axis, against the oracle's restatement of the
+    reference's loops: the gather bit for bit (copies, -0.0 kept), the scatter-add bit for bit (the
+    peers' parts added in rank order, each sum rounded to the dtype)."""
+    from helpers import LockstepMesh
+    from jigsaw_amd.halo import halo_gather_axis, halo_scatter_add_axis, spans_fit_the_strips
+
+    mesh, n, k, s, p, d = case
+    ns = len(mesh)
+    assert not spans_fit_the_strips(n, k, s, p, d, mesh)
+    torch.manual_seed(7)
+    lead = (2, 3)
+    tiles = {c: special_values_(torch.randn(*lead, *n)).to(dtype) for c in mesh_coords(mesh)}
+    want = oh.gather_mesh(tiles, mesh, k, s, p, d)
+    grads = {c: (torch.randn(want[c].shape) * torch.exp2(torch.randint(-12, 12, want[c].shape).float())).to(dtype) for c in tiles}
+    want_back = oh.scatter_add_mesh(grads, mesh, k, s, p, d, n)
+    lock = LockstepMesh(mesh)
+
+    def rank(c, exchange):
+        cur = tiles[c].to(dev)
+        for a in range(ns):
+            if mesh[a] > 1:
+                cur = halo_gather_axis(cur, a - ns, c[a], mesh[a], k[a], s[a], p[a], d[a],
+                                       lambda send, a=a: exchange.along_axis(a, send, False))
+        g = grads[c].to(dev)
+        for a in reversed(range(ns)):
+            if mesh[a] > 1:
+                g = halo_scatter_add_axis(g, a - ns, c[a], mesh[a], k[a], s[a], p[a], d[a], n[a],
+                                          lambda send, a=a: exchange.along_axis(a, send, True))
+        return cur.cpu(), g.cpu()
+
+    got = lock.run(rank)
+    for c in tiles:
+        assert_bit_equal(got[c][0], want[c], f"gather of rank {c}")
+        assert_bit_equal(got[c][1], want_back[c], f"scatter-add of rank {c}")
+
+
+def test_axis_segment_kernels_check_their_arguments(dev):
+    from jigsaw_amd.halo import axis_gather, axis_scatter_add
+
+    x = torch.arange(24, dtype=torch.float32, device=dev).reshape(2, 4, 3)
+    out = axis_gather(6, 1, [(x, 1, 0, 2), (x, 0, 3, 1)], x)  # rows 1, 2 to the front, row 0 to row 3, rows 2, 4, 5 zero
+    want = torch.zeros(2, 6, 3)
+    want[:, 0:2] = x.cpu()[:, 1:3]
+    want[:, 3] = x.cpu()[:, 0]
+    assert torch.equal(out.cpu(), want)
+    acc = axis_scatter_add(2, 1, [(x, 0, 0, 2), (x, 2, 0, 2), (x, 1, 1, 1)], x)
+    ref = torch.zeros(2, 2, 3)
+    ref += x.cpu()[:, 0:2]
+    ref += x.cpu()[:, 2:4]
+    ref[:, 1:2] += x.cpu()[:, 1:2]
+    assert torch.equal(acc.cpu(), ref)
+    with pytest.raises(ValueError):
+        axis_gather(2, 1, [(x, 3, 0, 2)], x)  # reads past the source
+    with pytest.raises(ValueError):
+        axis_gather(2, 1, [(x[:, :, :2], 0, 0, 1)], x)  # another inner shape
+    with pytest.raises(NotImplementedError):
+        axis_gather(40, 1, [(x, 0, i, 1) for i in range(17)], x)

@@ -250,3 +250,37 @@ def test_head_sizes_the_attention_host_pads_to():
         assert ja._kernel_head_size(d, torch.float32, True) == want
         assert ja._kernel_head_size(d, torch.bfloat16, False) == want
         assert ja._kernel_head_size(d) == want
+
+
+def test_general_span_plan_against_enumeration():
+    """``spans_fit_the_strips`` and ``span_overlap`` (the host side of the axis-by-axis exchange) from first
+    principles: output block r touches input rows ``o * s - p + d * t``; the rows of that range a peer owns are
+    what it sends, and what one rank expects from a peer is what the peer cuts for it."""
+    from jigsaw_amd.halo import needed_input_span, span_overlap, spans_fit_the_strips
+
+    seen_general = seen_fit = 0
+    for G, n, k, s, p, d in itertools.product((2, 3, 4), (2, 3, 5, 9), (1, 3, 5, 7), (1, 2), (0, 1, 3), (1, 2)):
+        extent = d * (k - 1) + 1
+        if G * n + 2 * p < extent:
+            continue
+        gout = (G * n + 2 * p - extent) // s + 1
+        if gout % G:
+            with pytest.raises(NotImplementedError):
+                spans_fit_the_strips((n,), (k,), (s,), (p,), (d,), (G,))
+            continue
+        ol = gout // G
+        fits = True
+        for r in range(G):
+            touched = sorted({o * s - p + d * t for o in range(r * ol, (r + 1) * ol) for t in range(k)})
+            lo, hi, need, out_local = needed_input_span(r, G, n, k, s, p, d)
+            assert (lo, hi - 1, out_local) == (touched[0], touched[-1], ol) and need == hi - lo
+            own = range(r * n, (r + 1) * n)
+            fits &= lo <= own[0] and hi >= own[-1] + 1 and own[0] - lo <= n and hi - (own[-1] + 1) <= n
+            for peer in range(G):
+                r0, cnt = span_overlap(lo, hi, peer, n, G)
+                rows = [g for g in range(lo, hi) if peer * n <= g < (peer + 1) * n]
+                assert cnt == len(rows) and (cnt == 0 or r0 == rows[0])
+        assert spans_fit_the_strips((n,), (k,), (s,), (p,), (d,), (G,)) == fits
+        seen_general += not fits
+        seen_fit += fits
+    assert seen_general > 20 and seen_fit > 20
