@@ -308,7 +308,12 @@ def backward(grad_out, q, k, v, out, logsumexp, scale, *args, dropout_p=0.0, see
 # per-rank ring loops over local chunks
 # --------------------------------------------------------------------------- #
 def _fused_ok(q, k) -> bool:
+    """Whether one launch attends the chunk AND merges into the running accumulators: the 16-bit MFMA
+    kernels at head sizes 64 / 96 / 128 with lengths in multiples of 128, and the fp32 matrix-core
+    kernel at head sizes 32 / 64 / 128 (any lengths, 16-byte aligned tensors)."""
     d = q.shape[-1]
+    if q.dtype == torch.float32:
+        return d in (32, 64, 128) and all(t.data_ptr() % 16 == 0 for t in (q, k))
     return (
         q.dtype in (torch.bfloat16, torch.float16) and d in (64, 96, 128) and d == _width(d, q.dtype)
         and q.shape[-2] % 128 == 0 and k.shape[-2] % 128 == 0
@@ -320,7 +325,8 @@ def attend_step_(q, kj, vj, scale, out, lse):
     ``(out, lse)`` in place (``_attend_step``, forward.py:64-96). Uses the fused
     kernel when it covers the shape, the core + merge kernels otherwise."""
     kj, vj = kj.contiguous(), vj.contiguous()
-    if _fused_ok(q, kj) and out.dtype == torch.float32 and out.is_contiguous() and lse.is_contiguous():
+    if (_fused_ok(q, kj) and q.is_contiguous() and vj.data_ptr() % 16 == 0 and out.dtype == torch.float32
+            and out.is_contiguous() and lse.is_contiguous() and out.data_ptr() % 16 == 0):
         core_forward(q, kj, vj, scale, out_acc=out, lse_acc=lse, want_out=False)
         return out, lse
     out_j, l_j = core_forward(q, kj, vj, scale)

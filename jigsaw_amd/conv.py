@@ -311,6 +311,24 @@ def _big_kernel_ok(kernel, stride, dilation) -> bool:
     return any(k not in (1, 3) for k in kernel) and math.prod(b for b, _ in _tap_blocks(kernel)) <= _MAX_TAP_BLOCKS
 
 
+_MOVED_COPY_BYTES = 8 << 30  # most that the moved copies of one call may take
+
+
+def _tap_blocks_fit(dtype, batch, c_in, kernel, out_sp) -> bool:
+    """Whether the three-tap layer the tap-block route builds is one the matrix-core kernels take (their per-image
+    extent is bounded by 32-bit byte offsets: cells * 72 * element size < 2 ** 31, fp32 counted at 4 bytes) and its
+    moved copies stay below ``_MOVED_COPY_BYTES``; otherwise the layer stays on the direct kernels as it is, where
+    zero-padded taps and the copies would only cost."""
+    if dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        return False
+    es = 4 if dtype == torch.float32 else 2
+    cells = math.prod(int(o) + 2 for o in out_sp)
+    if cells * 72 * es >= 1 << 31:
+        return False
+    blocks = math.prod(b for b, _ in _tap_blocks(kernel))
+    return int(batch) * int(c_in) * blocks * cells * (2 if dtype != torch.float32 else 4) <= _MOVED_COPY_BYTES
+
+
 def _moved_copies(x: torch.Tensor, kernel, padding, out_sp) -> torch.Tensor:
     """``(N, C, *spatial) -> (N, prod(blocks) * C, *(out + 2))``: block ``(i, j, ..)`` holds the zero-padded
     input moved by ``(3 i, 3 j, ..)`` cells, cut to what a three-tap layer without padding needs."""
@@ -429,7 +447,8 @@ def conv_nd(x, w, b=None, *, stride=1, padding=0, dilation=1, groups=1, out=None
         ext_in = tuple(-(-int(i) // p) for i, p in zip(x.shape[2:], phases))
         yb = conv_nd(_to_phases(x, phases, ext_in), w, b, stride=1, padding=tuple(pp // p for pp, p in zip(padding, phases)))
         return _from_phases(yb, phases, x.shape[0], out_sp)
-    if plain and _big_kernel_ok(tuple(w.shape[2:]), stride, dilation):
+    if (plain and _big_kernel_ok(tuple(w.shape[2:]), stride, dilation)
+            and _tap_blocks_fit(x.dtype, x.shape[0], x.shape[1], w.shape[2:], _out_spatial(x.shape[2:], w.shape[2:], stride, padding, dilation))):
         out_sp = _out_spatial(x.shape[2:], w.shape[2:], stride, padding, dilation)
         return conv_nd(_moved_copies(x, w.shape[2:], padding, out_sp), _tap_block_weight(w), b, stride=1, padding=0)
     off = _embed3(tuple(w.shape[2:]), stride, dilation) if plain else None
@@ -492,7 +511,8 @@ def conv_nd_input(input_shape, w, g, *, stride=1, padding=0, dilation=1, groups=
         gxb = conv_nd_input((g.shape[0] * math.prod(phases), input_shape[1], *ext_in), w, _to_phases(g, phases, ext_out),
                             stride=1, padding=pad0)
         return _from_phases(gxb, phases, input_shape[0], input_shape[2:])
-    if plain and _big_kernel_ok(tuple(w.shape[2:]), stride, dilation) and all(p <= k - 1 for p, k in zip(padding, w.shape[2:])):
+    if (plain and _big_kernel_ok(tuple(w.shape[2:]), stride, dilation) and all(p <= k - 1 for p, k in zip(padding, w.shape[2:]))
+            and _tap_blocks_fit(g.dtype, g.shape[0], w.shape[0], w.shape[2:], input_shape[2:])):
         out_sp = _out_spatial(input_shape[2:], w.shape[2:], stride, padding, dilation)
         if tuple(g.shape) != (input_shape[0], w.shape[0], *out_sp):
             raise ValueError(f"grad_output shape {tuple(g.shape)} does not match the convolution of an input of shape {input_shape}")
@@ -710,7 +730,8 @@ def conv_nd_weight(x, weight_shape, g, *, stride=1, padding=0, dilation=1, group
         # every residue image is one more batch entry of the undilated layer: the sum over the batch is the answer
         return conv_nd_weight(_to_phases(x, phases, ext_in), weight_shape, _to_phases(g, phases, ext_out), stride=1,
                               padding=pad0, with_bias_grad=with_bias_grad)
-    if plain and _big_kernel_ok(weight_shape[2:], stride, dilation):
+    if (plain and _big_kernel_ok(weight_shape[2:], stride, dilation)
+            and _tap_blocks_fit(x.dtype, x.shape[0], x.shape[1], weight_shape[2:], _out_spatial(x.shape[2:], weight_shape[2:], stride, padding, dilation))):
         out_sp = _out_spatial(x.shape[2:], weight_shape[2:], stride, padding, dilation)
         if tuple(g.shape) != (x.shape[0], weight_shape[0], *out_sp) or x.shape[1] != weight_shape[1]:
             raise ValueError(f"grad_output {tuple(g.shape)} / input {tuple(x.shape)} do not match weight {weight_shape}")

@@ -168,6 +168,19 @@ class _WholeBlock(torch.autograd.Function):
         b, h, w, c = x.shape
         dt, eps, heads = _compute_dtype(x), block.eps, block.attn.heads
         st = [_Stage() for _ in range(8)]
+        # what each part has to differentiate: its parameters as autograd asks for them here (a frozen parameter
+        # gets no gradient kernel where the part looks at the flag); the inputs between the parts always, x itself
+        # only when it wants a gradient
+        nig = tuple(ctx.needs_input_grad) if hasattr(ctx, "needs_input_grad") else (True,) * 15
+        pad = (False,) * 6
+        st[0].needs_input_grad = (nig[0], nig[1], nig[2]) + pad
+        st[1].needs_input_grad = (True,) + pad
+        st[2].needs_input_grad = (True, nig[3], nig[4]) + pad
+        st[3].needs_input_grad = (True, nig[5]) + pad
+        st[4].needs_input_grad = (True, nig[6], nig[7]) + pad
+        st[5].needs_input_grad = (True,) + pad
+        st[6].needs_input_grad = (True, nig[8], nig[9]) + pad
+        st[7].needs_input_grad = (True, nig[10], nig[11], nig[12], nig[13], True) + pad
         roll_args = block._roll_args()
         y = _PlainLayerNormFork.forward(st[0], x, n1w, n1b, eps, dt)[0]
         if block.shift_by:
@@ -185,6 +198,12 @@ class _WholeBlock(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad):  # noqa: D102
+        if ctx.stages is None:
+            raise RuntimeError(
+                "SwinBlock (one autograd node): backward was called a second time, but the tensors the first pass "
+                "kept were released when it finished (they are not held through save_for_backward, so "
+                "retain_graph=True does not keep them). Run the forward again, or build the block with one_node=False."
+            )
         st, (b, h, w, c) = ctx.stages, ctx.grid
         gy2, gw1, gb1, gw2, gb2, over = _GeluMlp.backward(st[7], grad)
         gx1, gn2w, gn2b = _PlainLayerNormFork.backward(st[6], gy2, over)[:3]

@@ -365,6 +365,28 @@ def test_backward_over_chunks_declines_what_it_does_not_cover(dev):
     assert ja.backward_chunks(qb, qb, qb, q[..., 0], many, many, 0.125) is None  # more chunks than a call takes
 
 
+@pytest.mark.parametrize("d,n,nk", [(64, 192, 160), (32, 100, 70), (128, 64, 96)])
+def test_fp32_ring_step_takes_the_fused_merge(d, n, nk, dev):
+    """``attend_step_`` on fp32 tensors at the head sizes of the fp32 matrix-core kernel: one launch that merges in
+    its epilogue, against the core followed by the separate merge (forward.py:64-96) and the fp64 oracle."""
+    torch.manual_seed(3)
+    scale = d**-0.5
+    q = torch.randn(1, 2, n, d, device=dev)
+    ks = [torch.randn(1, 2, nk, d, device=dev) for _ in range(3)]
+    vs = [torch.randn(1, 2, nk, d, device=dev) for _ in range(3)]
+    assert ja._fused_ok(q, ks[0])
+    out = torch.zeros_like(q)
+    lse = torch.full(q.shape[:-1], float("-inf"), device=dev)
+    out2, lse2 = out.clone(), lse.clone()
+    for kj, vj in zip(ks, vs):
+        out, lse = ja.attend_step_(q, kj, vj, scale, out, lse)
+        o_j, l_j = ja.core_forward(q, kj, vj, scale)
+        out2, lse2 = ja.fused_online_softmax_merge_(out2, lse2, o_j, l_j, "bhsd")
+    want_o, want_l = oa.ring_forward(q.double().cpu(), [t.double().cpu() for t in ks], [t.double().cpu() for t in vs], scale)
+    assert rel_l2(out, want_o) < 1e-5 and rel_l2(lse, want_l) < 1e-5
+    assert rel_l2(out, out2) < 1e-6 and rel_l2(lse, lse2) < 1e-6
+
+
 def test_window_attention_with_bias_and_mask(dev):
     """Swin-style windows: (B, nW, heads, N, d) with a (nW, heads, N, N) bias that
     holds -inf entries (shift mask), forward and backward incl. the bias gradient."""

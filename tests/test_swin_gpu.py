@@ -232,3 +232,39 @@ def test_block_step_recorded_in_a_hip_graph_replays_the_eager_step(shift, dev):
             assert step.grads[k].dtype == want.dtype and torch.equal(step.grads[k], want), (rep, k)
     with pytest.raises(NotImplementedError):
         block.captured_step(x.float(), g.float())
+
+
+def test_one_node_block_with_frozen_parameters_and_a_second_backward(dev):
+    """Frozen parameters and an input without a gradient get none from the one-node block, the others keep
+    their bits; a second backward through the same graph says why it cannot run."""
+    torch.manual_seed(5)
+    n, dim = (16, 16), 128
+
+    def comm(data, buffer, direction, *, group, async_op):
+        return torch.zeros_like(buffer), None
+
+    block = js.SwinBlock(dim, 4, 8, n, (TileGroup(1, 0), TileGroup(1, 0)), comm, shift=4, device=dev)
+    x = torch.randn(2, *n, dim, device=dev).bfloat16().requires_grad_()
+    gout = torch.randn(2, *n, dim, device=dev).bfloat16()
+
+    def grads(freeze, x_grad):
+        for name, p in block.named_parameters():
+            p.requires_grad_(name not in freeze)
+            p.grad = None
+        xi = x.detach().requires_grad_(x_grad)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            y = block(xi)
+        y.backward(gout, retain_graph=True)
+        with pytest.raises(RuntimeError, match="second time"):
+            y.backward(gout)
+        return xi.grad, {k: p.grad for k, p in block.named_parameters()}
+
+    gx_all, g_all = grads((), True)
+    frozen = ("attn.qkv.weight", "norm2.bias", "mlp.0.weight", "attn.bias_table")
+    gx_some, g_some = grads(frozen, False)
+    assert gx_some is None and gx_all is not None
+    for k, g in g_some.items():
+        if k in frozen:
+            assert g is None, k
+        else:
+            assert torch.equal(g, g_all[k]), k
