@@ -189,6 +189,39 @@ def _median(v):
     return v[n // 2] if n % 2 else 0.5 * (v[n // 2 - 1] + v[n // 2])
 
 
+def ln_statistics_calls(dev, g, big_rows: int = 1 << 18, cols: int = 256):
+    """The sharded LayerNorm's two statistics passes (forward: one tensor read; backward: g and x_hat read,
+    column partials for the weight / bias gradient and their reduction) on 2 ** 18 rows of configuration 4's
+    local width, over six different 134 MB tensors in turn: one alone would stay in the 256 MB last-level
+    cache and the figure would not be an HBM rate. The C entry points are called on buffers made once, so that
+    the host's share of such short kernels (two allocations a call) stays out of the figure. Returns the two
+    callables and the number of calls after which the inputs repeat."""
+    from jigsaw_amd import _lib
+
+    lib = _lib.load()
+    xls = [torch.randn(big_rows, cols, device=dev, generator=g).bfloat16() for _ in range(6)]
+    mean_b, var_b = torch.empty(big_rows, device=dev), torch.empty(big_rows, device=dev)
+    bf16 = _lib.dtype_code(torch.bfloat16)
+    turn = itertools.count()
+    w_ln = torch.ones(cols, device=dev, dtype=torch.bfloat16)
+    gw_b, gb_b = torch.empty(cols, device=dev), torch.empty(cols, device=dev)
+    ws_bytes = int(lib.jg_ln_bwd_workspace_bytes(big_rows, cols))
+    ws_ln = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+
+    def stats_fwd():
+        t = xls[next(turn) % len(xls)]
+        _lib.check(lib.jg_ln_partial_fwd(_lib.ptr(mean_b), _lib.ptr(var_b), _lib.ptr(t), big_rows, cols, bf16,
+                                         _lib.stream_ptr(dev)), "jg_ln_partial_fwd")
+
+    def stats_bwd():
+        i = next(turn) % (len(xls) // 2)
+        _lib.check(lib.jg_ln_partial_bwd(_lib.ptr(mean_b), _lib.ptr(var_b), _lib.ptr(gw_b), _lib.ptr(gb_b), _lib.ptr(xls[2 * i]),
+                                         _lib.ptr(xls[2 * i + 1]), _lib.ptr(w_ln), big_rows, cols, bf16, _lib.ptr(ws_ln), ws_bytes,
+                                         _lib.stream_ptr(dev)), "jg_ln_partial_bwd")
+
+    return stats_fwd, stats_bwd, len(xls)
+
+
 def attention_figures(dev, iters: int) -> dict:
     """Configuration 4: one rank's ring-attention step. 8 local heads, 4096 local
     queries, one K/V chunk of 4096 keys per step (4 steps), head size 64, bf16.
@@ -252,39 +285,11 @@ def attention_figures(dev, iters: int) -> dict:
     hop_bwd["ms_no_hop"] = time_gpu(lambda: ja.ring_backward(dout, q, out, l, ks, vs, scale), iters)
     x = torch.randn(b, n, 256, device=dev, generator=g).bfloat16()
     ms_ln = time_gpu(lambda: jl.partial_stats(x), iters)
-    # the same statistics on a shard that fills the chip (2 ** 18 rows of the same local width), over six
-    # different 134 MB tensors in turn: one alone would stay in the 256 MB last-level cache and the
-    # figure would not be an HBM rate. The C entry points are called on buffers made once, so that the
-    # host's share of such short kernels (two allocations a call) stays out of the figure.
-    from jigsaw_amd import _lib
-
-    lib = _lib.load()
-    big_rows, cols = 1 << 18, 256
-    xls = [torch.randn(big_rows, cols, device=dev, generator=g).bfloat16() for _ in range(6)]
-    mean_b, var_b = torch.empty(big_rows, device=dev), torch.empty(big_rows, device=dev)
-    bf16 = _lib.dtype_code(torch.bfloat16)
-    turn = itertools.count()
-
-    def stats_fwd():
-        t = xls[next(turn) % len(xls)]
-        _lib.check(lib.jg_ln_partial_fwd(_lib.ptr(mean_b), _lib.ptr(var_b), _lib.ptr(t), big_rows, cols, bf16,
-                                         _lib.stream_ptr(dev)), "jg_ln_partial_fwd")
-
-    ms_ln_big = time_gpu(stats_fwd, max(iters, 2 * len(xls)), warmup=len(xls))
-    # the backward's partial sums over g and x_hat (two tensors read, column partials for the weight / bias gradient)
-    w_ln = torch.ones(cols, device=dev, dtype=torch.bfloat16)
-    gw_b, gb_b = torch.empty(cols, device=dev), torch.empty(cols, device=dev)
-    ws_bytes = int(lib.jg_ln_bwd_workspace_bytes(big_rows, cols))
-    ws_ln = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-
-    def stats_bwd():
-        i = next(turn) % (len(xls) // 2)
-        _lib.check(lib.jg_ln_partial_bwd(_lib.ptr(mean_b), _lib.ptr(var_b), _lib.ptr(gw_b), _lib.ptr(gb_b), _lib.ptr(xls[2 * i]),
-                                         _lib.ptr(xls[2 * i + 1]), _lib.ptr(w_ln), big_rows, cols, bf16, _lib.ptr(ws_ln), ws_bytes,
-                                         _lib.stream_ptr(dev)), "jg_ln_partial_bwd")
-
-    ms_ln_bwd = time_gpu(stats_bwd, max(iters, 2 * len(xls)), warmup=len(xls))
-    del xls
+    # the same statistics, and the backward's partial sums, on a shard that fills the chip
+    stats_fwd, stats_bwd, n_turn = ln_statistics_calls(dev, g)
+    ms_ln_big = time_gpu(stats_fwd, max(iters, 2 * n_turn), warmup=n_turn)
+    ms_ln_bwd = time_gpu(stats_bwd, max(iters, 2 * n_turn), warmup=n_turn)
+    del stats_fwd, stats_bwd
     # the separate LSE merge (what a step runs when its core cannot fuse it): fp32 accumulator read and
     # written, the step's bf16 output read; at the step's size and at 16 x the heads
     merge = {}
@@ -764,6 +769,15 @@ def profile_sharded_layernorm(reps: int = 3) -> None:
             x.grad = w.grad = b.grad = None
             jl.layer_norm(x, w, b, None).backward(gout)
         torch.cuda.synchronize()
+        del x, gout
+    # the two statistics kernels by themselves, as bench.py's figures time them (inputs in turn, read-only
+    # neighbours): in the layer above each runs right behind a kernel that leaves 268 MB of written lines behind
+    stats_fwd, stats_bwd, n_turn = ln_statistics_calls(dev, g)
+    for _ in range(2 * n_turn):
+        stats_fwd()
+    for _ in range(2 * n_turn):
+        stats_bwd()
+    torch.cuda.synchronize()
 
 
 def profile_conv3d(reps: int = 3) -> None:
