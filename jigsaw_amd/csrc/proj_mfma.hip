@@ -335,17 +335,19 @@ struct TnShape {
   static constexpr int LDS = 2 * STAGE * 16;
 };
 
-__device__ __forceinline__ float sum_bf16x8(const u32x4& v) {
-  float s = 0.0f;
+// acc + the eight bf16 values of v. Plain shifts and adds: v_dot2c_f32_bf16 against a pair of ones is a
+// quarter of the instructions and gave the right sums by itself, but wrong ones in this kernel (chains of
+// dependent dot instructions), so it is not used.
+__device__ __forceinline__ float add_bf16x8(float acc, const u32x4& v) {
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    s += __builtin_bit_cast(float, v[j] << 16);
-    s += __builtin_bit_cast(float, v[j] & 0xffff0000u);
+    acc += __builtin_bit_cast(float, v[j] << 16);
+    acc += __builtin_bit_cast(float, v[j] & 0xffff0000u);
   }
-  return s;
+  return acc;
 }
 
-template <int IM, int JN, int WM, int WN>
+template <int IM, int JN, int WM, int WN, int AHEAD>
 __global__ __launch_bounds__(64 * WM * WN) void proj_tn_kernel(TnParams p) {
   typedef TnShape<IM, JN, WM, WN> SH;
   constexpr int T = SH::T;
@@ -363,9 +365,19 @@ __global__ __launch_bounds__(64 * WM * WN) void proj_tn_kernel(TnParams p) {
   const int nst = r_last > r_first ? (int)((r_last - r_first + BR - 1) / BR) : 0;
 
   // loads: the first half of the threads fetches g, the second x; a thread owns an 8 token x 8 feature block
-  const int half = tid / T, tt = tid % T;
+  // `half` is the same for a whole wavefront (T is a multiple of 64). The operand's map is copied
+  // field by field: a reference chosen per thread (`half ? p.xm : p.gm`) made the compiler keep a
+  // pointer to the argument and re-read the fields from memory in every stage, each read followed by a
+  // wait for ALL outstanding loads, the staged ones included, which undid the lookahead below.
+  const int half = __builtin_amdgcn_readfirstlane(tid / T), tt = tid % T;
   const int jc = tt % (T / 8), ro = tt / (T / 8);
-  const Map& mp = half ? p.xm : p.gm;
+  Map mp;
+  mp.heads = half ? p.xm.heads : p.gm.heads;
+  mp.ld = half ? p.xm.ld : p.gm.ld;
+  mp.B = half ? p.xm.B : p.gm.B;
+  mp.H = half ? p.xm.H : p.gm.H;
+  mp.S = half ? p.xm.S : p.gm.S;
+  mp.D = half ? p.xm.D : p.gm.D;
   const uint16_t* src = half ? p.x : p.g;
   const int f_count = half ? p.C : p.N;
   int f = (half ? c0 : n0) + jc * 8;
@@ -378,21 +390,27 @@ __global__ __launch_bounds__(64 * WM * WN) void proj_tn_kernel(TnParams p) {
 #pragma unroll
   for (int j = 0; j < 8; ++j) bsum[j] = 0.0f;
 
-  u32x4 v[8];
-  long long r_loaded = 0;
-  const long long tok_stride = mp.heads ? mp.D : mp.ld;  // between consecutive tokens of one batch entry
-  auto load = [&](int st) {
+  // AHEAD register sets: the loads of stage st + AHEAD are issued at the head of stage st (into the set
+  // stage st was stored from), so a load has AHEAD - 1 whole stages to arrive before its registers go to
+  // LDS. With one set a workgroup moved 32 KB per memory latency: a stage's matrix instructions take a
+  // quarter of one.
+  u32x4 vs[AHEAD][8];
+  long long rl[AHEAD];
+  const uint32_t tok_stride32 = (uint32_t)(mp.heads ? mp.D : mp.ld);  // between consecutive tokens of one batch entry
+  auto load = [&](int st, u32x4 (&v)[8], long long& r_loaded) {
     // tokens r_first + st*BR + ro*8 + i, all of one batch entry (S % 8 == 0); `walk` stands at i = 0.
     // A token past the end repeats the last one (or token 0) and is zeroed on the way to LDS.
     r_loaded = r_first + (long long)st * BR + ro * 8;
     const long long left = p.rows - r_loaded;
     const int last = left >= 8 ? 7 : (left > 0 ? (int)left - 1 : 0);
     const uint16_t* b0 = src + (left > 0 ? walk.part(mp) : 0) + fpart;
+    // 32-bit element offsets inside the block of eight tokens (the host checks that 7 strides fit)
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = *reinterpret_cast<const u32x4*>(b0 + (i < last ? i : last) * tok_stride);
+    for (int i = 0; i < 8; ++i) v[i] = *reinterpret_cast<const u32x4*>(b0 + (uint32_t)(i < last ? i : last) * tok_stride32);
     walk.advance(mp, BR);
   };
-  auto store = [&](int buf) {
+  auto store = [&](int buf, u32x4 (&v)[8], long long r_loaded, bool counted) {  // counted: a stage of this split
+    const bool add_bias = want_bias && counted;
     u32x4* dst = lds + buf * SH::STAGE + half * SH::OP + ro * SH::PITCH + jc * 9;
     if (r_loaded + 8 > p.rows) {
 #pragma unroll
@@ -408,7 +426,7 @@ __global__ __launch_bounds__(64 * WM * WN) void proj_tn_kernel(TnParams p) {
       t.z = __builtin_amdgcn_perm(v[5][px >> 1], v[4][px >> 1], sel);
       t.w = __builtin_amdgcn_perm(v[7][px >> 1], v[6][px >> 1], sel);
       dst[px] = t;
-      if (want_bias) bsum[px] += sum_bf16x8(t);
+      if (add_bias) bsum[px] = add_bf16x8(bsum[px], t);
     }
   };
 
@@ -452,16 +470,33 @@ __global__ __launch_bounds__(64 * WM * WN) void proj_tn_kernel(TnParams p) {
     }
   };
 
-  if (nst > 0) {
-    load(0);
-    store(0);
-  }
+  // stage st lives in register set st % AHEAD; the loop is unrolled AHEAD times so that the sets are named at
+  // compile time. Nothing in the main loop is conditional: a load or an LDS store under a condition made the
+  // compiler merge the set's old and new values through copies, and a copy waits for the load. Loads past the
+  // split's last stage read tokens that exist (clamped in `load`) and are never multiplied.
+#pragma unroll
+  for (int a = 0; a < AHEAD; ++a) load(a, vs[a], rl[a]);
+  store(0, vs[0], rl[0], nst > 0);
   __syncthreads();
-  for (int st = 0; st < nst; ++st) {
-    if (st + 1 < nst) load(st + 1);
-    compute(st & 1);
-    if (st + 1 < nst) store((st + 1) & 1);
-    __syncthreads();
+  const int nst_main = nst - nst % AHEAD;
+  int st = 0;
+  for (; st < nst_main; st += AHEAD) {
+#pragma unroll
+    for (int a = 0; a < AHEAD; ++a) {
+      load(st + a + AHEAD, vs[a], rl[a]);
+      compute((st + a) & 1);
+      store((st + a + 1) & 1, vs[(a + 1) % AHEAD], rl[(a + 1) % AHEAD], st + a + 1 < nst);
+      __syncthreads();
+    }
+  }
+  // the last nst % AHEAD stages: their tokens are in the sets already, the first of them in LDS
+#pragma unroll
+  for (int a = 0; a < AHEAD - 1; ++a) {
+    if (st + a < nst) {  // uniform
+      compute((st + a) & 1);
+      if (st + a + 1 < nst) store((st + a + 1) & 1, vs[a + 1], rl[a + 1], true);
+      __syncthreads();
+    }
   }
 
   // register e of block (i, j): row n0 + (wn*IM + i)*32 + 8*(e/4) + 4*kg + e%4, column c0 + (wc*JN + j)*32 + ln
@@ -499,8 +534,9 @@ __global__ __launch_bounds__(64 * WM * WN) void proj_tn_kernel(TnParams p) {
 
 // out[i] (bf16) = sum over the splits of part[split][i], for the weight gradient and (blocks behind
 // it) the bias gradient in one launch. A block takes 256 consecutive outputs: 64 lanes x 4 values,
-// and its four wavefronts each add every fourth split; the four sums are then added in a fixed
-// order, so the result does not depend on scheduling.
+// and its W wavefronts (4, or 16 where there are many splits: a small weight matrix has few blocks,
+// and each of their threads would walk the splits one load after the other) each add every W-th
+// split; the W sums are then added in a fixed order, so the result does not depend on scheduling.
 struct ReduceArgs {
   void* out_w;
   const float* part_w;
@@ -512,8 +548,9 @@ struct ReduceArgs {
   int out32;  // write fp32 instead of bf16
 };
 
-__global__ __launch_bounds__(256) void proj_reduce_kernel(ReduceArgs a) {
-  __shared__ f32x4 sm[4][64];
+template <int W>
+__global__ __launch_bounds__(64 * W) void proj_reduce_kernel(ReduceArgs a) {
+  __shared__ f32x4 sm[W][64];
   const size_t blocks_w = (a.count_w + 255) / 256;
   const bool second = blockIdx.x >= blocks_w;
   void* out_any = second ? a.out_b : a.out_w;
@@ -527,9 +564,9 @@ __global__ __launch_bounds__(256) void proj_reduce_kernel(ReduceArgs a) {
   f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
   if (i0 < count) {
     if (vec) {
-      for (int k = grp; k < a.splits; k += 4) acc += *reinterpret_cast<const f32x4*>(part + (size_t)k * count + i0);
+      for (int k = grp; k < a.splits; k += W) acc += *reinterpret_cast<const f32x4*>(part + (size_t)k * count + i0);
     } else {
-      for (int k = grp; k < a.splits; k += 4)
+      for (int k = grp; k < a.splits; k += W)
 #pragma unroll
         for (int e = 0; e < 4; ++e)
           if (i0 + e < count) acc[e] += part[(size_t)k * count + i0 + e];
@@ -538,7 +575,9 @@ __global__ __launch_bounds__(256) void proj_reduce_kernel(ReduceArgs a) {
   sm[grp][q] = acc;
   __syncthreads();
   if (grp != 0 || i0 >= count) return;
-  const f32x4 t = ((sm[0][q] + sm[1][q]) + sm[2][q]) + sm[3][q];
+  f32x4 t = sm[0][q];
+#pragma unroll
+  for (int w = 1; w < W; ++w) t += sm[w][q];
   if (a.out32) {
     float* o32 = static_cast<float*>(out_any);
     if (vec) {
@@ -689,12 +728,16 @@ bool map_octets_ok(const Map& m) { return !m.heads || m.S % 8 == 0; }
 
 // Token ranges (splits) the contraction is cut into so that `tiles` tiles fill the chip; a
 // split is worth its partial tile from about 8 stages on.
-int splits_for(long long rows, int tiles, int target) {
+int splits_for(long long rows, int tiles, int target, bool small_tiles = false) {
   const long long stages = (rows + BR - 1) / BR;
   long long want = (target + tiles - 1) / tiles;
-  if (want > stages / 8) want = stages / 8;
+  // at most 64 splits, but with one to three 128-wide tiles as many as put a workgroup on every compute
+  // unit: a compute unit streams its operands at some 20 GB/s, so 64 workgroups leave three quarters of
+  // the memory system idle (128 x 128 over 65536 tokens: 23 -> 13 us, the reduction 5 -> 6 us)
+  const long long cap = !small_tiles || tiles * 64 >= 256 ? 64 : 256 / tiles;
+  if (want > stages / (cap > 64 ? 4 : 8)) want = stages / (cap > 64 ? 4 : 8);
   if (want < 1) want = 1;
-  if (want > 64) want = 64;
+  if (want > cap) want = cap;
   return (int)want;
 }
 // Tile edge of the weight-gradient kernel: 256 (half the operand traffic per MFMA, one workgroup
@@ -706,7 +749,7 @@ int tn_tile(long long rows, int n, int c) {
 }
 int tn_splits(long long rows, int n, int c) {
   const int t = tn_tile(rows, n, c);
-  return splits_for(rows, jg::cdiv(n, t) * jg::cdiv(c, t), t == 256 ? 256 : 1024);
+  return splits_for(rows, jg::cdiv(n, t) * jg::cdiv(c, t), t == 256 ? 256 : 1024, t == 128);
 }
 
 template <int IM, int JN, int WM, int WN>
@@ -714,7 +757,8 @@ int launch_tn(TnParams& p, int splits, hipStream_t s, const char* who) {
   typedef TnShape<IM, JN, WM, WN> SH;
   p.tiles_c = jg::cdiv(p.C, SH::T);
   const int tiles = jg::cdiv(p.N, SH::T) * p.tiles_c;
-  void (*kern)(TnParams) = &proj_tn_kernel<IM, JN, WM, WN>;
+  // the 128-wide tile has the registers for three sets of staged loads, the 256-wide one for one
+  void (*kern)(TnParams) = &proj_tn_kernel<IM, JN, WM, WN, (IM * JN <= 4 ? 3 : 1)>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      SH::LDS);
   if (e != hipSuccess) JG_FAIL(JG_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS", who, SH::LDS);
@@ -816,6 +860,7 @@ int jg_proj_tn(void* gw, void* gb, const void* g, const void* x, int dtype, int 
              dtype);
   const bool out32 = grad_dtype == JG_F32 && dtype != JG_F32;
   JG_REQUIRE(rows > 0 && n > 0 && c > 0, "%s: bad sizes rows=%lld n=%d c=%d", who, (long long)rows, n, c);
+  JG_REQUIRE(n < (1 << 27) && c < (1 << 27), "%s: more than 2^27 features a row (n=%d c=%d)", who, n, c);
   Map gm, xm;
   int rc = make_map(&gm, g_heads, n, rows, B, H, S, D, who, "gradient");
   if (rc) return rc;
@@ -868,7 +913,8 @@ int jg_proj_tn(void* gw, void* gb, const void* g, const void* x, int dtype, int 
   ra.splits = splits;
   ra.out32 = out32 ? 1 : 0;
   const size_t blocks = (ra.count_w + 255) / 256 + (ra.count_b + 255) / 256;
-  proj_reduce_kernel<<<(unsigned)blocks, 256, 0, s>>>(ra);
+  if (splits >= 32) proj_reduce_kernel<16><<<(unsigned)blocks, 1024, 0, s>>>(ra);
+  else proj_reduce_kernel<4><<<(unsigned)blocks, 256, 0, s>>>(ra);
   JG_CHECK_LAUNCH(who);
   return JG_OK;
 }
