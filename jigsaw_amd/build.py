@@ -37,6 +37,16 @@ HIPCC_FLAGS = [
 ]
 
 
+# Kernels whose vector instructions read or scale their matrix accumulators (softmax on the scores, the
+# running rescale, epilogues) keep the accumulators in ordinary vector registers: left to its default the
+# compiler puts them in the accumulation registers and moves them over and back with v_accvgpr_read /
+# v_accvgpr_write around every such use (64 moves per loop iteration in the wide attention forward).
+PER_FILE_FLAGS = {
+    name: ["-mllvm", "-amdgpu-mfma-vgpr-form"]
+    for name in ("attn_wide.hip", "attn_swin.hip", "attn_window.hip", "attn_f32_mfma.hip", "proj_mfma.hip")
+}
+
+
 def hipcc() -> str:
     for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
         if cand and Path(cand).exists():
@@ -60,7 +70,7 @@ def _compile(src: Path, force: bool, extra: list[str]) -> Path:
     deps = [src, *CSRC.glob("*.h"), ROOT.parent / "include" / "jigsaw_hip.h"]
     if not force and _newer(obj, deps):
         return obj
-    cmd = [hipcc(), *HIPCC_FLAGS, *extra, "-c", str(src), "-o", str(obj)]
+    cmd = [hipcc(), *HIPCC_FLAGS, *PER_FILE_FLAGS.get(src.name, []), *extra, "-c", str(src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     # hipcc's host pass does not know the packed-fp32 feature and says so; harmless.
     err = "\n".join(

@@ -123,7 +123,6 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_mfma_kernel(FwdArgs p) {
   const int lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, kg = lane >> 5;
   const int qg = wave & 1, kq = wave >> 1;
-  const int th = tid & 127;  // thread index inside the key quarter
   const BlockOf where = block_of();
   const long long b = where.bh;
   const int q0 = where.blk * BM + qg * 64;

@@ -244,6 +244,11 @@ __global__ __launch_bounds__(THREADS) void attn_wide_fwd_kernel(Args p) {
   trans_fetch<D>(rv, vb);
   tile_store_rows<D>(rk, smem);
   trans_store<D>(rv, smem + G::ROWMAJ);
+  // The fragments that came straight from memory are waited for here, once. Left to the first matrix
+  // instruction that reads them, the wait sits inside the loop, behind the tile loads every iteration has
+  // just issued, and counts those too: each iteration then waited for its own prefetch.
+#pragma unroll
+  for (int c = 0; c < G::C16; ++c) asm volatile("" : "+v"(qf[c]));
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
     const unsigned char* kt = smem + (t & 1) * BUF;
@@ -377,6 +382,11 @@ __global__ __launch_bounds__(THREADS) void attn_wide_dq_kernel(Args p) {
   tile_store_rows<D>(rk, smem);
   tile_store_rows<D>(rv, smem + G::ROWMAJ);
   trans_store<D>(rkt, smem + 2 * G::ROWMAJ);
+  // The fragments that came straight from memory are waited for here, once. Left to the first matrix
+  // instruction that reads them, the wait sits inside the loop, behind the tile loads every iteration has
+  // just issued, and counts those too: each iteration then waited for its own prefetch.
+#pragma unroll
+  for (int c = 0; c < G::C16; ++c) asm volatile("" : "+v"(qf[c]), "+v"(dof[c]));
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
     const unsigned char* kt = smem + (t & 1) * BUF;
@@ -486,6 +496,14 @@ __global__ __launch_bounds__(THREADS, (D <= 96 || MODE != 0) ? 2 : 1) void attn_
   };
   fetch(0);
   store(0);
+  // The fragments that came straight from memory are waited for here, once. Left to the first matrix
+  // instruction that reads them, the wait sits inside the loop, behind the tile loads every iteration has
+  // just issued, and counts those too: each iteration then waited for its own prefetch.
+#pragma unroll
+  for (int c = 0; c < G::C16; ++c) {
+    asm volatile("" : "+v"(kf[c]));
+    if (DK) asm volatile("" : "+v"(vf[c]));
+  }
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
     const unsigned char* qt = smem + (t & 1) * BUF;
