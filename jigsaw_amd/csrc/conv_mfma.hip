@@ -893,18 +893,23 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
         }
         return;
       }
+      // One scalar base for the tile; the channel walks in the 32-bit lane offset (the host checks that MT
+      // planes fit it): one vector add per store. A scalar base per channel cost a multiply, a 64-bit add and
+      // the reload of a spilled scalar per store, three to four instructions for each 2-byte store.
+      const uint32_t st = (uint32_t)(2 * ps), st5 = 5u * st;
 #pragma unroll
       for (int r = 0; r < WROWS; ++r) {
         const int oh = th0 + wrow0 + r - p.lo_h;
-        const uint32_t voff = (uint32_t)(2 * ((size_t)(4 * kg) * ps + (size_t)oh * p.nW + (ow - p.lo_w)));
+        uint32_t vo = (uint32_t)(2 * ((size_t)(4 * kg) * ps + (size_t)oh * p.nW + (ow - p.lo_w)));
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const int m0 = cb * 32 + 8 * (j >> 1) + 2 * (j & 1);
+          for (int j = 0; j < 8; ++j) {  // channels cb * 32 + 8 * (j / 2) + 2 * (j % 2) and the one after (+ 4 kg, in vo)
             const uint32_t bits = pk[cb][r][j];
-            store_bf16_lo(ybase + (size_t)m0 * ps * 2, voff, bits);
-            store_bf16_hi(ybase + (size_t)(m0 + 1) * ps * 2, voff, bits);
+            store_bf16_lo(ybase, vo, bits);
+            vo += st;
+            store_bf16_hi(ybase, vo, bits);
+            vo += (j & 1) ? st5 : st;
           }
       }
       return;
@@ -922,8 +927,14 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
       const int rh = oh < p.lo_h ? 0 : (oh < p.lo_h + p.nH ? 1 : 2);
       const int ch = oh - (rh == 0 ? 0 : (rh == 1 ? p.lo_h : p.lo_h + p.nH));
       const int eh = rh == 0 ? p.lo_h : (rh == 1 ? p.nH : hi_h);
-      const int slot = rd * 9 + rh * 3 + rw;
-      char* base = slot == 13 ? reinterpret_cast<char*>(p.y) : static_cast<char*>(strip_entry(slot));
+      // The row's three possible destinations (one per region across W) are read with wave-uniform indices,
+      // i.e. through the scalar cache, and chosen per lane: a per-lane index into the table is a vector load,
+      // and waiting for it also waits for every store the row before has just issued.
+      const int slot0 = __builtin_amdgcn_readfirstlane(rd * 9 + rh * 3);
+      char* const b_lo = static_cast<char*>(strip_entry(slot0));
+      char* const b_mid = slot0 + 1 == 13 ? reinterpret_cast<char*>(p.y) : static_cast<char*>(strip_entry(slot0 + 1));
+      char* const b_hi = static_cast<char*>(strip_entry(slot0 + 2));
+      char* base = rw == 0 ? b_lo : (rw == 1 ? b_mid : b_hi);
       if (base == nullptr) continue;
       const uint32_t ps = (uint32_t)ed * (uint32_t)eh * (uint32_t)ew;  // elements per plane of that destination
       char* dst = base + 2 * ((plane0 + 4 * kg) * (size_t)ps + ((size_t)cd * eh + ch) * ew + cw);
@@ -1371,6 +1382,9 @@ int mfma_dgrad_fold(void* gx, void* const strips[27], const int lo[3], const int
   const Layout lay = layout_of(g.k[0] * pad16(g.cout), g.cin);
   if (lay.mtiles * lay.MT != g.cin)
     JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_dgrad_fold(mfma): %d input channels are not a multiple of %d", g.cin, lay.MT);
+  // the epilogue addresses the MT channel planes of a tile through a 32-bit byte offset
+  if ((long long)n[0] * n[1] * n[2] * 2 * lay.MT >= (1ll << 32) || (long long)g.in[0] * g.in[1] * g.in[2] * 2 * lay.MT >= (1ll << 32))
+    JG_FAIL(JG_ERR_UNSUPPORTED, "jg_conv_dgrad_fold(mfma): %d planes of the tile do not fit a 32-bit offset", lay.MT);
   return dgrad_launch(gx, strips, lo, n, w, go, g, ws, ws_bytes, s, "jg_conv_dgrad_fold(mfma)");
 }
 
