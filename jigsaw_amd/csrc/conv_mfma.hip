@@ -797,12 +797,17 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
         const int oh = tc.th * TH + wrow0 + r;
         if (oh < p.Hout && ow >= 0 && ow < p.Wout) {
           const uint32_t voff = (uint32_t)(4 * ((size_t)(4 * kg) * ochan + (size_t)oh * p.Wout + ow));
+          // the channel's base walks by additions (a product per store costs a scalar multiply, a 64-bit add
+          // and, with the scalar registers this kernel has left, a spill reload)
+          const char* yc = ybase32;
+          const size_t cs = ochan * 4;
 #pragma unroll
           for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
               const int m0 = cb * 32 + 8 * (i >> 2) + (i & 3);
-              if (!RAGGED || m0 < m_left) store_f32(ybase32 + (size_t)m0 * ochan * 4, voff, acc[cb][r][i]);
+              if (!RAGGED || m0 < m_left) store_f32(yc, voff, acc[cb][r][i]);
+              yc += (i & 3) == 3 ? 5 * cs : cs;
             }
         }
       }
@@ -813,6 +818,8 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
       const int oh = tc.th * TH + wrow0 + r;
       if (oh < p.Hout && ow >= 0 && ow < p.Wout) {
         const uint32_t voff = (uint32_t)(2 * ((size_t)(4 * kg) * ochan + (size_t)oh * p.Wout + ow));
+        const char* yc = ybase;  // walks by additions, as above
+        const size_t cs = ochan * 2;
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
@@ -821,8 +828,10 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
             const uint32_t h2 = F16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, f16x2))
                                                 : __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
             const int m0 = cb * 32 + 8 * (i >> 2) + (i & 3);
-            if (!RAGGED || m0 < m_left) store_bf16_lo(ybase + (size_t)m0 * ochan * 2, voff, h2);
-            if (!RAGGED || m0 + 1 < m_left) store_bf16_hi(ybase + (size_t)(m0 + 1) * ochan * 2, voff, h2);
+            if (!RAGGED || m0 < m_left) store_bf16_lo(yc, voff, h2);
+            yc += cs;
+            if (!RAGGED || m0 + 1 < m_left) store_bf16_hi(yc, voff, h2);
+            yc += (i & 2) ? 5 * cs : cs;
           }
       }
     }
