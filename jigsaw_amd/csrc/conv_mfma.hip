@@ -947,15 +947,19 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
       if (base == nullptr) continue;
       const uint32_t ps = (uint32_t)ed * (uint32_t)eh * (uint32_t)ew;  // elements per plane of that destination
       char* dst = base + 2 * ((plane0 + 4 * kg) * (size_t)ps + ((size_t)cd * eh + ch) * ew + cw);
-      const uint32_t step = 2u * ps;  // bytes between produced channels (checked on the host to fit)
+      // bytes between produced channels (checked on the host to fit); the destination's plane size differs
+      // from lane to lane, so the pointer walks by additions: a product per store is a quarter-rate
+      // vector multiply
+      const uint32_t step = 2u * ps, step5 = 5u * step;
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const uint32_t m0 = (uint32_t)(cb * 32 + 8 * (j >> 1) + 2 * (j & 1));
+        for (int j = 0; j < 8; ++j) {  // channels cb * 32 + 8 * (j / 2) + 2 * (j % 2) and the one after (+ 4 kg, in dst)
           const uint32_t bits = pk[cb][r][j];
-          *reinterpret_cast<uint16_t*>(dst + m0 * step) = (uint16_t)(bits & 0xffffu);
-          *reinterpret_cast<uint16_t*>(dst + (m0 + 1) * step) = (uint16_t)(bits >> 16);
+          *reinterpret_cast<uint16_t*>(dst) = (uint16_t)(bits & 0xffffu);
+          dst += step;
+          *reinterpret_cast<uint16_t*>(dst) = (uint16_t)(bits >> 16);
+          dst += (j & 1) ? step5 : step;
         }
     }
   };
