@@ -419,6 +419,9 @@ __global__ __launch_bounds__(64 * WM * WN) void proj_tn_kernel(TnParams p) {
   u32x4 vs[AHEAD][8];
   long long rl[AHEAD];
   const uint32_t tok_stride32 = (uint32_t)(mp.heads ? mp.D : mp.ld);  // between consecutive tokens of one batch entry
+  uint32_t tok_off[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) tok_off[i] = (uint32_t)i * tok_stride32;
   auto load = [&](int st, u32x4 (&v)[8], long long& r_loaded) {
     // tokens r_first + st*BR + ro*8 + i, all of one batch entry (S % 8 == 0); `walk` stands at i = 0.
     // A token past the end repeats the last one (or token 0) and is zeroed on the way to LDS.
@@ -426,9 +429,11 @@ __global__ __launch_bounds__(64 * WM * WN) void proj_tn_kernel(TnParams p) {
     const long long left = p.rows - r_loaded;
     const int last = left >= 8 ? 7 : (left > 0 ? (int)left - 1 : 0);
     const uint16_t* b0 = src + (left > 0 ? walk.part(mp) : 0) + fpart;
-    // 32-bit element offsets inside the block of eight tokens (the host checks that 7 strides fit)
+    // 32-bit element offsets inside the block of eight tokens (the host checks that 7 strides fit): the eight
+    // products are made once; a block cut short by the end of the tensor repeats its last token
+    const uint32_t last_off = (uint32_t)last * tok_stride32;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = *reinterpret_cast<const u32x4*>(b0 + (uint32_t)(i < last ? i : last) * tok_stride32);
+    for (int i = 0; i < 8; ++i) v[i] = *reinterpret_cast<const u32x4*>(b0 + (i < last ? tok_off[i] : last_off));
     walk.advance(mp, BR);
   };
   auto store = [&](int buf, u32x4 (&v)[8], long long r_loaded, bool counted) {  // counted: a stage of this split
