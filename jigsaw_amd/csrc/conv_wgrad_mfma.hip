@@ -101,7 +101,11 @@ __device__ __forceinline__ float sum_bf16x8(const u32x4& v) {
 // 4-byte aligned tensors and an even padding across W, so that a stage's windows start on dwords and
 // the 16-byte vector loads apply, 2 = the same with an odd padding: the x window is staged from one
 // pixel earlier, where it is dword aligned again, and the fragments are built one pixel further in.
-template <int CGB, int CXB, int EVEN, bool FRAMED, bool F16 = false>
+// ALLIN: the host has checked that every window of every stage lies inside x and every stage's
+// rows inside g (a convolution without padding over a tensor that holds its halo, tiles of whole
+// stages): the kernel is built without the element-wise border path, and its stage loop loads and
+// stores without conditions.
+template <int CGB, int CXB, int EVEN, bool FRAMED, bool F16 = false, bool ALLIN = false>
 __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(WgradParams p) {
   constexpr int THREADS = wgrad_threads(CGB, CXB);
   constexpr int LEAD = EVEN == 2 ? 1 : 0;
@@ -288,9 +292,9 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
                         2 * ((ptrdiff_t)((size_t)n * p.cin_total * p.Din * plane_x) + (ptrdiff_t)id0 * (ptrdiff_t)plane_x +
                              (ptrdiff_t)ih0 * p.Win + iw0);
     // (with LEAD the window's last dword holds one pixel more than is used; it shares its dword with one that is)
-    const bool inside = EVEN != 0 && oh0 + SR <= p.Hout && ow0 + SW <= p.Wout && ih0 >= 0 &&
+    const bool inside = ALLIN || (EVEN != 0 && oh0 + SR <= p.Hout && ow0 + SW <= p.Wout && ih0 >= 0 &&
                         ih0 + 2 <= p.Hin && iw0 >= 0 && iw0 + SW + 2 + LEAD <= p.Win && id0 >= 0 &&
-                        id0 + (XC / p.Cin) <= p.Din;
+                        id0 + (XC / p.Cin) <= p.Din);
     if (FRAMED && inside) {
       // Rows and columns of the pair's window inside the own tile (wave-uniform): a chunk
       // whose depth plane is a plane of the tile comes from the tile itself, at whatever
@@ -433,7 +437,7 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
   float bsum[ROUNDS];
 #pragma unroll
   for (int rd = 0; rd < ROUNDS; ++rd) bsum[rd] = 0.0f;
-  auto store_loads = [&](const Staged& sg, bool have_g, int gbuf, int slot_a, int slot_b) {
+  auto store_loads = [&](const Staged& sg, bool have_g, int gbuf, int slot_a, int slot_b, bool counted = true) {
     const u32x4 (&v)[ROUNDS] = sg.v;
 #pragma unroll
     for (int rd = 0; rd < ROUNDS; ++rd) {
@@ -441,7 +445,7 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
       if (q < G_CHUNKS) {
         if (have_g) {
           *reinterpret_cast<u32x4*>(smem + gbuf * G_BYTES + c_lds[rd]) = v[rd];
-          if (p.bias_part != nullptr) bsum[rd] += sum_bf16x8(v[rd]);
+          if (p.bias_part != nullptr) bsum[rd] += counted ? sum_bf16x8(v[rd]) : 0.0f;
         }
       } else if (q < CHUNKS) {
         const int slot = ((x_second >> rd) & 1u) ? slot_b : slot_a;
@@ -532,32 +536,68 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
     store_loads(stg, true, 0, 2, 3);
     issue_loads(stg, c_next, false, 0);
     store_loads(stg, false, 0, 0, 1);
-    advance(c_next);
-    Cursor c_store = c_next;          // stage whose registers are stored next (st + 1)
-    if (s_begin + 1 < s_end) {
+    if constexpr (ALLIN) {
+      // The loads of a stage are issued, and the registers of the stage before stored, in EVERY
+      // stage: the cursor stops at the workgroup's last stage, which the last two stages fetch
+      // again for nothing, and what the last stage stores nobody reads. A load or a store under
+      // a condition leaves the staged registers with two possible states where the paths meet;
+      // the compiler then waits for the loads at the end of the stage that issued them (to copy
+      // the registers together) instead of where they are stored, half a stage later.
+      if (s_begin + 1 < s_end) advance(c_next);
+      Cursor c_store = c_next;          // stage whose registers are stored next (st + 1)
       issue_loads(stg, c_next, true, 1);
+      if (s_begin + 2 < s_end) advance(c_next);
+      __syncthreads();
+      for (long long st = s_begin; st < s_end; ++st) {
+        if (wave < CWAVES) compute_group(gbuf, base, 0);
+        store_loads(stg, true, gbuf ^ 1, wrap(base + 4), wrap(base + 5), st + 1 < s_end);
+        issue_loads(stg, c_next, true, 1);
+        if (st + 3 < s_end) advance(c_next);
+        if (wave < CWAVES) compute_group(gbuf, base, 1);
+        __syncthreads();
+        if (st + 1 < s_end && c_store.hp == 0) {
+          // the next stage starts a new strip: its first two x rows, on the spot
+          Staged top;
+          issue_loads(top, c_store, false, 0);
+          store_loads(top, false, 0, wrap(base + 2), wrap(base + 3));
+          // These loads have all been stored, but the tail's under a per-lane condition: where
+          // the compiler cannot see a load waited for on every path, it waits at the loop's end,
+          // and that wait takes the stage's own loads with it. vmcnt(0), said once, here:
+          __builtin_amdgcn_s_waitcnt(0x0F70);
+          __syncthreads();
+        }
+        advance(c_store);
+        base = wrap(base + 2);
+        gbuf ^= 1;
+      }
+    } else {
       advance(c_next);
-    }
-    __syncthreads();
-    for (long long st = s_begin; st < s_end; ++st) {
-      if (wave < CWAVES) compute_group(gbuf, base, 0);
-      if (st + 1 < s_end) store_loads(stg, true, gbuf ^ 1, wrap(base + 4), wrap(base + 5));
-      if (st + 2 < s_end) {
+      Cursor c_store = c_next;          // stage whose registers are stored next (st + 1)
+      if (s_begin + 1 < s_end) {
         issue_loads(stg, c_next, true, 1);
         advance(c_next);
       }
-      if (wave < CWAVES) compute_group(gbuf, base, 1);
       __syncthreads();
-      if (st + 1 < s_end && c_store.hp == 0) {
-        // the next stage starts a new strip: its first two x rows, on the spot
-        Staged top;
-        issue_loads(top, c_store, false, 0);
-        store_loads(top, false, 0, wrap(base + 2), wrap(base + 3));
+      for (long long st = s_begin; st < s_end; ++st) {
+        if (wave < CWAVES) compute_group(gbuf, base, 0);
+        if (st + 1 < s_end) store_loads(stg, true, gbuf ^ 1, wrap(base + 4), wrap(base + 5));
+        if (st + 2 < s_end) {
+          issue_loads(stg, c_next, true, 1);
+          advance(c_next);
+        }
+        if (wave < CWAVES) compute_group(gbuf, base, 1);
         __syncthreads();
+        if (st + 1 < s_end && c_store.hp == 0) {
+          // the next stage starts a new strip: its first two x rows, on the spot
+          Staged top;
+          issue_loads(top, c_store, false, 0);
+          store_loads(top, false, 0, wrap(base + 2), wrap(base + 3));
+          __syncthreads();
+        }
+        advance(c_store);
+        base = wrap(base + 2);
+        gbuf ^= 1;
       }
-      advance(c_store);
-      base = wrap(base + 2);
-      gbuf ^= 1;
     }
   }
 
@@ -726,7 +766,7 @@ bool blocks_of(const ConvGeom& g, Blocking* b) {
 int block_width(int total, int c0, int first) { return (first == 64 && total - c0 > 32) ? 64 : 32; }
 
 template <int CGB, int CXB>
-int launch(const WgradParams& p, int even, bool f16, int wgs, hipStream_t s, const char* who) {
+int launch(const WgradParams& p, int even, bool f16, bool all_inside, int wgs, hipStream_t s, const char* who) {
   constexpr int THREADS = wgrad_threads(CGB, CXB);
   const size_t lds = 2 * (size_t)(32 * CGB * G_CH) + (size_t)(32 * CXB * X_CH);
   void (*kern)(WgradParams);
@@ -735,6 +775,8 @@ int launch(const WgradParams& p, int even, bool f16, int wgs, hipStream_t s, con
                      : (even == 2 ? &wgrad3x3_mfma_kernel<CGB, CXB, 2, false, true> : &wgrad3x3_mfma_kernel<CGB, CXB, 0, false, true>);
   else if (p.xt != nullptr)
     kern = &wgrad3x3_mfma_kernel<CGB, CXB, 1, true>;  // the framed input needs the even layout (checked by the caller)
+  else if (all_inside && even == 1)
+    kern = &wgrad3x3_mfma_kernel<CGB, CXB, 1, false, false, true>;
   else
     kern = even == 1 ? &wgrad3x3_mfma_kernel<CGB, CXB, 1, false>
                      : (even == 2 ? &wgrad3x3_mfma_kernel<CGB, CXB, 2, false> : &wgrad3x3_mfma_kernel<CGB, CXB, 0, false>);
@@ -901,6 +943,10 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
       else { p.wd_first = head_slow ? SLOW : 1; p.wd_last = tail_slow ? SLOW : 1; }
     }
   }
+  // Every stage whole and every window inside x: the kernel without the border path (see ALLIN).
+  const bool all_inside = even == 1 && xt == nullptr && g.p[0] == 0 && g.p[1] == 0 && g.p[2] == 0 &&
+                          g.out[1] % SR == 0 && g.out[2] % SW == 0 && g.out[1] + 2 <= g.in[1] &&
+                          g.out[2] + 2 <= g.in[2] && g.out[0] - 1 + g.k[0] <= g.in[0];
   const int wgs = wg_count(p.total_stages);
   p.xt = static_cast<const uint16_t*>(xt);
   p.tlo_d = tlo ? tlo[0] : 0; p.tlo_h = tlo ? tlo[1] : 0; p.tlo_w = tlo ? tlo[2] : 0;
@@ -916,11 +962,11 @@ int mfma_wgrad(void* gw, void* gb, const void* x, const void* go, const ConvGeom
     p.g = static_cast<const uint16_t*>(go) + gch * g_cs;
     p.bias_part = gb_out != nullptr ? p.part + (size_t)wgs * HALVES * 9 * cob * (bl.KD * cib) : nullptr;
     int rc;
-    if (cgb == 2 && cxb == 2) rc = launch<2, 2>(p, even, f16, wgs, s, who);
-    else if (cgb == 1 && cxb == 3) rc = launch<1, 3>(p, even, f16, wgs, s, who);
-    else if (cgb == 1 && cxb == 1) rc = launch<1, 1>(p, even, f16, wgs, s, who);
-    else if (cgb == 2 && cxb == 1) rc = launch<2, 1>(p, even, f16, wgs, s, who);
-    else if (cgb == 1 && cxb == 2) rc = launch<1, 2>(p, even, f16, wgs, s, who);
+    if (cgb == 2 && cxb == 2) rc = launch<2, 2>(p, even, f16, all_inside, wgs, s, who);
+    else if (cgb == 1 && cxb == 3) rc = launch<1, 3>(p, even, f16, all_inside, wgs, s, who);
+    else if (cgb == 1 && cxb == 1) rc = launch<1, 1>(p, even, f16, all_inside, wgs, s, who);
+    else if (cgb == 2 && cxb == 1) rc = launch<2, 1>(p, even, f16, all_inside, wgs, s, who);
+    else if (cgb == 1 && cxb == 2) rc = launch<1, 2>(p, even, f16, all_inside, wgs, s, who);
     else JG_FAIL(JG_ERR_UNSUPPORTED, "%s: channel blocking (%d, %d) not built", who, cgb, cxb);
     if (rc) return rc;
     JG_CHECK_LAUNCH(who);
