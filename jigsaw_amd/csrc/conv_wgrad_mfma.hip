@@ -468,23 +468,38 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
       for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.0f;
 
   // one 16-pixel column group (cgi = 0 or 1 of this wavefront's half) of a stage whose
-  // four x rows sit in ring rows base .. base + 3 (mod RING)
-  auto compute_group = [&](int gbuf, int base, int cgi) {
+  // four x rows sit in ring rows base .. base + 3 (mod RING): first all its LDS reads
+  // (read_group), then its matrix instructions (mfma_group), so that a stage can ask for both
+  // of its groups before the first matrix instruction and meets the LDS latency once.
+  struct Frags {
+    u32x4 a[SR];
+    u32x4 d[XR];
+    uint32_t d4[XR], d5[XR];
+  };
+  auto read_group = [&](Frags& f, int gbuf, int base, int cgi) __attribute__((always_inline)) {
     const unsigned char* gb = smem + gbuf * G_BYTES + (cb * 32 + ln) * G_CH + kgp * 16;
     const unsigned char* xb = lds_x + (ib * 32 + ln) * X_CH + kgp * 16;
     const int cg = half * (SW / 16 / HALVES) + cgi;  // 16-pixel column group of this wavefront
-    bf16x8 a[SR];
 #pragma unroll
-    for (int r = 0; r < SR; ++r)
-      a[r] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(gb + r * (SW * 2) + cg * 32));
+    for (int r = 0; r < SR; ++r) f.a[r] = *reinterpret_cast<const u32x4*>(gb + r * (SW * 2) + cg * 32);
 #pragma unroll
     for (int rho = 0; rho < XR; ++rho) {
       int slot = base + rho;
       if (slot >= RING) slot -= RING;
-      u32x4 d = *reinterpret_cast<const u32x4*>(xb + slot * X_ROW + cg * 32);
-      uint32_t d4 = *reinterpret_cast<const uint32_t*>(xb + slot * X_ROW + cg * 32 + 16);
-      uint32_t d5 = 0u;
-      if (LEAD) d5 = *reinterpret_cast<const uint32_t*>(xb + slot * X_ROW + cg * 32 + 20);
+      f.d[rho] = *reinterpret_cast<const u32x4*>(xb + slot * X_ROW + cg * 32);
+      f.d4[rho] = *reinterpret_cast<const uint32_t*>(xb + slot * X_ROW + cg * 32 + 16);
+      f.d5[rho] = 0u;
+      if (LEAD) f.d5[rho] = *reinterpret_cast<const uint32_t*>(xb + slot * X_ROW + cg * 32 + 20);
+    }
+  };
+  auto mfma_group = [&](Frags& f) __attribute__((always_inline)) {
+    bf16x8 a[SR];
+#pragma unroll
+    for (int r = 0; r < SR; ++r) a[r] = __builtin_bit_cast(bf16x8, f.a[r]);
+#pragma unroll
+    for (int rho = 0; rho < XR; ++rho) {
+      u32x4 d = f.d[rho];
+      uint32_t d4 = f.d4[rho], d5 = f.d5[rho];
       // The values are made opaque so that the kw = 2 fragment below is built with register
       // moves: left alone, the compiler reads it again from LDS at a 4-byte offset, as dword
       // pairs whose 880-byte lane stride runs into 4-way bank conflicts.
@@ -521,6 +536,11 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
       }
     }
   };
+  auto compute_group = [&](int gbuf, int base, int cgi) {
+    Frags f;
+    read_group(f, gbuf, base, cgi);
+    mfma_group(f);
+  };
 
   // Stage k of this workgroup reads ring rows base_k .. base_k + 3 with base_k = 2k mod 6:
   // its first two rows are where the stage before put its new rows (base_k-1 + 2, + 3), its
@@ -548,12 +568,34 @@ __global__ __launch_bounds__(wgrad_threads(CGB, CXB)) void wgrad3x3_mfma_kernel(
       issue_loads(stg, c_next, true, 1);
       if (s_begin + 2 < s_end) advance(c_next);
       __syncthreads();
+      // Wavefronts w and w + 4 share a SIMD and would do everything at the same time: both issue
+      // matrix instructions, then both store and load while the matrix core idles (measured with
+      // the cycle counter: 1150 cycles of a 4400-cycle stage spent by the older wavefront of each
+      // SIMD waiting at the barrier for the younger one). So the two take the stage's halves in
+      // opposite order: w multiplies while w + 4 stores the registers of the next stage and
+      // issues the loads of the one after, then the other way round. What is stored goes to the
+      // g buffer and the ring rows that no wavefront reads in this stage.
+      // (With six multiplying wavefronts, two SIMDs hold a wavefront that only stages; there the
+      // split measured slower, and every wavefront stores and loads between its two groups.)
+      const bool stage_first = CWAVES == 8 && (wave & 4) != 0;
       for (long long st = s_begin; st < s_end; ++st) {
-        if (wave < CWAVES) compute_group(gbuf, base, 0);
-        store_loads(stg, true, gbuf ^ 1, wrap(base + 4), wrap(base + 5), st + 1 < s_end);
-        issue_loads(stg, c_next, true, 1);
+        Frags f0, f1;
+        if (stage_first) {
+          store_loads(stg, true, gbuf ^ 1, wrap(base + 4), wrap(base + 5), st + 1 < s_end);
+          issue_loads(stg, c_next, true, 1);
+        }
+        if (wave < CWAVES) {
+          read_group(f0, gbuf, base, 0);
+          read_group(f1, gbuf, base, 1);
+          mfma_group(f0);
+          if (CWAVES == 8) mfma_group(f1);
+        }
+        if (!stage_first) {
+          store_loads(stg, true, gbuf ^ 1, wrap(base + 4), wrap(base + 5), st + 1 < s_end);
+          issue_loads(stg, c_next, true, 1);
+        }
+        if (CWAVES != 8 && wave < CWAVES) mfma_group(f1);
         if (st + 3 < s_end) advance(c_next);
-        if (wave < CWAVES) compute_group(gbuf, base, 1);
         __syncthreads();
         if (st + 1 < s_end && c_store.hp == 0) {
           // the next stage starts a new strip: its first two x rows, on the spot
