@@ -48,6 +48,16 @@ PRIM_CASES = [
     (2, 64, 64, (150, 330), (3, 3), (1, 1), (1, 1), (1, 1)),
     (2, 32, 32, (140, 200), (3, 3), (1, 1), (0, 0), (1, 1)),
     (1, 32, 32, (5, 40, 136), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+    # weight gradient without padding over whole stages (even rows, 64-column strips), every window inside x: the
+    # kernel without the border path, whose stage loop loads and stores without conditions. One stage per
+    # workgroup, two or three (the load cursor stops at the last one), each channel blocking
+    (2, 64, 64, (4, 66), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (1, 64, 64, (1030, 66), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (2, 64, 64, (8, 130), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (1, 32, 64, (262, 130), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (2, 64, 32, (6, 66), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (1, 32, 32, (518, 66), (3, 3), (1, 1), (0, 0), (1, 1)),
+    (1, 32, 32, (5, 260, 66), (3, 3, 3), (1, 1, 1), (0, 0, 0), (1, 1, 1)),
     # channel counts beyond one group of LDS-resident weights, and produced channels that are
     # not a multiple of the 32-row MFMA tile (padded with zero weight rows, not stored)
     (1, 128, 128, (20, 70), (3, 3), (1, 1), (1, 1), (1, 1)),
