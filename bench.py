@@ -38,7 +38,7 @@ METRIC = "halo-conv fwd+bwd & ring-attn step TFLOP/s on 1 GPU; % MFMA peak; halo
 
 # HBM bytes per launch of the three convolution kernels of the step (FETCH_SIZE + WRITE_SIZE
 # from rocprofv3 --pmc, scaled by a copy kernel of known size).
-CONV_TRAFFIC_BYTES = {"fwd": 2.24e9, "dgrad_fold": 2.885e9, "wgrad_bias": 2.31e9}  # wgrad: 2.23 GB + 0.08 GB for its reduction
+CONV_TRAFFIC_BYTES = {"fwd": 2.24e9, "dgrad_fold": 2.87e9, "wgrad_bias": 2.31e9}  # wgrad: 2.23 GB + 0.08 GB for its reduction
 CONV_KERNEL_NAMES = {
     "fwd": "conv3x3_mfma_kernel (forward, config 2)",
     "dgrad_fold": "conv3x3_mfma_kernel (dgrad with the fold epilogue, config 2)",
