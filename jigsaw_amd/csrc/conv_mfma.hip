@@ -973,6 +973,11 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     cursor_advance();
   };
   const bool stage_early = __builtin_amdgcn_readfirstlane(wave) == 4 || __builtin_amdgcn_readfirstlane(wave) == 5;
+  // Does the epilogue put anything into the free stage buffer? Every epilogue but the fold's does (rows go
+  // through LDS to leave as 16-byte pieces), and the fold's does where the tile grid lies on the 16-byte grid
+  // of the unpadded gradient (the same test as in epilogue_fold; it is the same for every tile of a launch).
+  const bool epilogue_uses_lds =
+      !FOLD || ((((p.org_w - p.lo_w) & 7) == 0) && (p.nW & 7) == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0);
   int buf = 0;
   cursor_enter(0);
   issue_stage();
@@ -998,8 +1003,9 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
       // Wavefronts 4 and 5 hold staging tasks like wavefronts 0..3 and share SIMD 0 and 1 with two of them.
       // They stage at the head of the stage, while their SIMD's other wavefront multiplies, and that one
       // stages later, while they multiply; done at the same point, the two leave the matrix core idle.
-      // (Not in a tile's first stage: the buffer is the last epilogue's scratch until the barrier below.)
-      const bool stage_now = stage_early && !(c16 == 0 && ti > 0);
+      // (Not in a tile's first stage where the buffer is the last epilogue's scratch until the barrier below.)
+      const bool after_epilogue = epilogue_uses_lds && c16 == 0 && ti > 0;
+      const bool stage_now = stage_early && !after_epilogue;
       if (stage_now) {
         if (q + 1 < stages) store_stage(buf ^ 1, q + 1);
         if (q + 2 < stages) issue_stage();
@@ -1008,8 +1014,9 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
         compute_kw(buf, wstep, 0, wstep_next);
         compute_kw(buf, wstep, 1, wstep_next);
       }
-      // the buffer written next was the last epilogue's scratch
-      if (c16 == 0 && ti > 0) __syncthreads();
+      // the buffer written next was the last epilogue's scratch (the fold's 2-byte stores leave from the registers:
+      // nothing to wait for, and the wavefronts that are through with their stores do not wait for the others here)
+      if (after_epilogue) __syncthreads();
       if (!stage_now) {
         if (q + 1 < stages) store_stage(buf ^ 1, q + 1);  // other buffer: no hazard with this stage's reads
         if (q + 2 < stages) issue_stage();
