@@ -972,7 +972,13 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
     issue_loads();
     cursor_advance();
   };
-  const bool stage_early = __builtin_amdgcn_readfirstlane(wave) == 4 || __builtin_amdgcn_readfirstlane(wave) == 5;
+  // Which two stage at the head of a stage (see the stage loop) was tried all ways round, in engine cycles of
+  // configuration 2: forward 4 and 5: 1.18 M, 0 and 1: 1.12 M, 2 and 3: 1.14 M, 0 to 3: 1.15 M, 2 to 5: 1.17 M;
+  // dgrad with the fold epilogue 4 and 5: 1.455 M, 0 and 1: 1.47 M, 0 to 3: 1.48 M, nobody or 2 to 5: 1.49 M,
+  // all six: 1.59 M. (In the fold's epilogue the older wavefronts of a SIMD get their stores out first and are
+  // back in the stage loop while 4 to 7 still store.)
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const bool stage_early = FOLD ? (wave_u == 4 || wave_u == 5) : (wave_u == 0 || wave_u == 1);
   // Does the epilogue put anything into the free stage buffer? Every epilogue but the fold's does (rows go
   // through LDS to leave as 16-byte pieces), and the fold's does where the tile grid lies on the 16-byte grid
   // of the unpadded gradient (the same test as in epilogue_fold; it is the same for every tile of a launch).
@@ -1000,9 +1006,9 @@ __global__ __launch_bounds__(THREADS) void conv3x3_mfma_kernel(StripTable strips
         __syncthreads();
       }
       const int wstep_next = wstep + 1 == p.wc16 ? 0 : wstep + 1;
-      // Wavefronts 4 and 5 hold staging tasks like wavefronts 0..3 and share SIMD 0 and 1 with two of them.
-      // They stage at the head of the stage, while their SIMD's other wavefront multiplies, and that one
-      // stages later, while they multiply; done at the same point, the two leave the matrix core idle.
+      // Wavefronts 4 and 5 hold staging tasks like wavefronts 0..3 and share SIMD 0 and 1 with 0 and 1.
+      // One of each pair stages at the head of the stage, while its SIMD's other wavefront multiplies, and that
+      // one stages later, while the first multiplies; done at the same point, the two leave the matrix core idle.
       // (Not in a tile's first stage where the buffer is the last epilogue's scratch until the barrier below.)
       const bool after_epilogue = epilogue_uses_lds && c16 == 0 && ti > 0;
       const bool stage_now = stage_early && !after_epilogue;
